@@ -1,0 +1,182 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+A step is one pass of paged decode attention (split kernel + split reduce) over one batch of the
+headline decode workload: batch 32, 32 query / 8 KV heads, head_dim 128, bf16, block size 16,
+context lengths uniform in [512, 4096], block tables from a seeded permutation of a 16384-block
+pool.  Inputs are resident in HBM before the timed region; three independent KV pools are rotated so
+consecutive steps cannot be served from the 256 MB Infinity Cache.
+
+Prints one JSON line: whole-job GB/s of algorithmic bytes, the roofline of the dominant kernel
+(measured with HIP events on the launch stream) and the CPU oracle timed on a bounded sample.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+POOLS = 3
+
+
+def parse():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=300)
+    parser.add_argument("--warmup", type=int, default=30)
+    parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--keys-per-split", type=int, default=0, help="tuning override (0 = built-in choice)")
+    return parser.parse_args()
+
+
+def cpu_baseline(work, budget_s=12.0):
+    """The reference's CPU decode as written (one thread, weights re-evaluated per output dimension),
+    restated in the oracle, timed on as many leading sequences of the same workload as fit the budget."""
+    import numpy as np
+
+    import oracle
+
+    order = list(range(work.batch))
+    done_bytes, elapsed, used = 0, 0.0, 0
+    for b in order:
+        length = int(work.seq_lens[b])
+        n = (length + work.block_size - 1) // work.block_size
+        blocks = work.block_table[b, :n].astype(np.int64)
+        import torch
+
+        index = torch.from_numpy(blocks).to(work.key_cache.device)
+        kc = work.key_cache[index].float().cpu().numpy()
+        vc = work.value_cache[index].float().cpu().numpy()
+        q = work.query[b:b + 1].float().cpu().numpy()
+        table = np.arange(n, dtype=np.uint32).reshape(1, -1)
+        start = time.perf_counter()
+        oracle.paged_kv_decode_attention_f32(q, kc, vc, [length], table, batch=1, heads=work.heads,
+                                             kv_heads=work.kv_heads, head_dim=work.head_dim,
+                                             block_size=work.block_size, block_table_batch_stride=max(n, 1),
+                                             scale=work.scale, literal=True)
+        elapsed += time.perf_counter() - start
+        done_bytes += length * 2 * work.kv_heads * work.head_dim * 2 + 2 * work.heads * work.head_dim * 2
+        used += 1
+        if elapsed > budget_s:
+            break
+    return {
+        "value": done_bytes / elapsed / 1e9,
+        "unit": "GB/s",
+        "cores": 1,
+        "kind": "port",
+        "sample": f"first {used} of {work.batch} sequences of the same workload, reference loop shape "
+                  f"(single thread, {elapsed:.1f} s)",
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no cross-GPU exchange and every box here has one "
+              "GPU; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from singe_amd import _native, synthetic
+    from singe_amd.kernel import attention as A
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    if args.keys_per_split:
+        _native.lib().singe_hip_set_decode_keys_per_split(args.keys_per_split)
+
+    work = synthetic.paged_decode_workload()
+    pools = [(work.key_cache, work.value_cache)]
+    for extra in range(1, POOLS):
+        other = synthetic.paged_decode_workload(seed=synthetic.BASE_SEED + 97 * extra)
+        pools.append((other.key_cache, other.value_cache))
+        del other
+    config = A.PagedKvDecodeAttentionConfig.contiguous(work.batch, work.heads, work.kv_heads, work.head_dim,
+                                                       work.block_size, work.physical_blocks,
+                                                       work.block_table_batch_stride, work.scale)
+    lens = torch.from_numpy(work.seq_lens).cuda()
+    table = torch.from_numpy(work.block_table.view(np.int32)).cuda()
+    out = torch.empty((work.batch, work.heads, work.head_dim), device="cuda", dtype=torch.bfloat16)
+    workspace = torch.empty(config.workspace_bytes(), dtype=torch.uint8, device="cuda")
+
+    def step(i, phases=3):
+        kc, vc = pools[i % POOLS]
+        A.paged_kv_decode_attention_bf16(None, out, work.query, kc, vc, lens, table, config, workspace, phases)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    start = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - start
+    ms_per_step = seconds / args.steps * 1e3
+
+    # The dominant kernel alone (the split kernel), bracketed by events on its own stream.
+    begin = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    finish = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    for i in range(args.steps):
+        begin[i].record()
+        step(i, phases=1)
+        finish[i].record()
+        step(i, phases=2)
+    torch.cuda.synchronize()
+    kernel_ms = sorted(b.elapsed_time(f) for b, f in zip(begin, finish))
+    kernel_avg_ms = sum(kernel_ms) / len(kernel_ms)
+
+    bytes_per_step = work.algorithmic_bytes()
+    value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
+    achieved = bytes_per_step / (kernel_avg_ms * 1e-3) / 1e9
+    result = {
+        "metric": "decode attn GB/s",
+        "value": value,
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "paged decode: batch 32, 32q/8kv heads, head_dim 128, bf16, block 16, "
+                        "ctx U[512,4096], 16384-block pool (BASELINE config 2)",
+            "total_keys": work.total_keys,
+            "algorithmic_bytes": bytes_per_step,
+            "algorithmic_flops": work.algorithmic_flops(),
+            "keys_per_split": int(_native.lib().singe_hip_decode_keys_per_split(config._c())),
+            "kv_pools_rotated": POOLS,
+        },
+        "tokens_per_s": work.batch / (ms_per_step * 1e-3),
+        "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "singe_paged_decode_bf16_d128_g4_b16",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS,
+            "traffic": None,
+            "kernel_avg_us": kernel_avg_ms * 1e3,
+            "kernel_median_us": kernel_ms[len(kernel_ms) // 2] * 1e3,
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(work)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,136 @@
+/*
+ * singe_hip_attention.h: C ABI of the MI355X (gfx950) attention kernels.
+ *
+ * This is the layer a `singe-kernel-sys`-style binding links against (the reference keeps that crate
+ * as an empty placeholder: singe-kernel-sys/src/lib.rs:1-6).  Every entry point takes plain device
+ * pointers, element counts and a #[repr(C)]-compatible config struct; nothing here allocates device
+ * memory, synchronises, or owns a buffer.  Work is enqueued on the caller's HIP stream and completes
+ * asynchronously, so every call is legal during stream capture
+ * (raw kernel execution contract: singe-kernel/src/cuda/mod.rs:3-12).
+ *
+ * The kernels live in a gfx950 code object (singe_attention_gfx950.hsaco, built by hipcc --genco)
+ * that this library loads with hipModuleLoadData and launches with hipModuleLaunchKernel, in place of
+ * the reference's NVRTC -> cuModuleLoadData -> cuLaunchKernelEx path
+ * (singe/src/backend/cuda/codegen/compile.rs:43-190, singe-cuda/src/module/mod.rs:2117-2132).
+ * The HIP runtime itself is resolved with dlopen on first use, as the reference's sys crates do
+ * (singe-loader/src/lib.rs:298-322), so the library has no link-time dependency on ROCm.
+ *
+ * Return value of every int32_t function: 0 = success; a positive SingeHipStatus = a validation
+ * failure found before launch (mirrors singe-kernel/src/error.rs:12-186); a negative value =
+ * -(hipError_t) from the HIP runtime.
+ */
+#ifndef SINGE_HIP_ATTENTION_H
+#define SINGE_HIP_ATTENTION_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SINGE_HIP_API __attribute__((visibility("default")))
+
+typedef enum SingeHipStatus {
+    SINGE_HIP_OK = 0,
+    SINGE_HIP_INVALID_LENGTH = 1,        /* Error::InvalidLength: zero extent, heads % kv_heads != 0, non-finite scale */
+    SINGE_HIP_LENGTH_TOO_SHORT = 2,      /* Error::LengthTooShort { name, minimum, actual } */
+    SINGE_HIP_LENGTH_EXCEEDS_I32 = 3,    /* Error::LengthExceedsI32 */
+    SINGE_HIP_SIZE_OVERFLOW = 4,         /* Error::SizeOverflow */
+    SINGE_HIP_UNSUPPORTED_WIDTH = 5,     /* Error::UnsupportedWidth { op, width } */
+    SINGE_HIP_NULL_POINTER = 6,          /* Error::NullPointer */
+    SINGE_HIP_KERNEL_NOT_PREPARED = 7,   /* Error::KernelNotPrepared: code object missing or not loadable */
+    SINGE_HIP_UNSUPPORTED_CONFIGURATION = 8, /* Error::UnsupportedConfiguration { op, reason } */
+    SINGE_HIP_INVALID_ARGUMENT = 9,      /* singe::Error::InvalidArgument (shape / dtype rules of the singe op) */
+    SINGE_HIP_RUNTIME_UNAVAILABLE = 10   /* the HIP runtime library could not be opened */
+} SingeHipStatus;
+
+/* Details of the last non-zero status returned on the calling thread. */
+typedef struct SingeHipErrorDetail {
+    int32_t status;
+    const char* name;      /* buffer or parameter the failure is about; static string, never NULL */
+    uint64_t minimum;      /* LengthTooShort: required element count; UnsupportedWidth: the width */
+    uint64_t actual;       /* LengthTooShort: supplied element count */
+} SingeHipErrorDetail;
+SINGE_HIP_API void singe_hip_last_error(SingeHipErrorDetail* detail);
+SINGE_HIP_API const char* singe_hip_status_string(int32_t status);
+
+/* ---- code object management -------------------------------------------------------------------
+ * Replaces Context::load_module / Module::function (singe-cuda/src/context.rs:363-385,
+ * singe-cuda/src/module/mod.rs:387-410).  An image is a gfx950 code object or a clang offload bundle
+ * holding one.  Loading is per process; the module is instantiated lazily on each device that
+ * launches.  Without an explicit load the library looks for singe_attention_gfx950.hsaco next to
+ * itself.  The image bytes are copied. */
+SINGE_HIP_API int32_t singe_hip_load(const void* image, size_t bytes);
+SINGE_HIP_API int32_t singe_hip_load_file(const char* path);
+SINGE_HIP_API void singe_hip_unload(void);
+/* Resolves every kernel of the image on the current device; returns the number found through *count. */
+SINGE_HIP_API int32_t singe_hip_prepare(int32_t* count);
+
+/* ---- singe-kernel surface: paged decode ---------------------------------------------------------
+ * Mirrors PagedKvDecodeAttentionConfig (singe-kernel/src/cuda/attention/mod.rs:76-90). */
+typedef struct SingePagedKvDecodeAttentionConfig {
+    size_t batch;
+    size_t heads;
+    size_t kv_heads;
+    size_t head_dim;
+    size_t block_size;
+    size_t physical_blocks;
+    size_t block_table_batch_stride;
+    float scale;
+} SingePagedKvDecodeAttentionConfig;
+
+/* validate_paged_kv_decode_attention_config (mod.rs:2963-2985). */
+SINGE_HIP_API int32_t singe_hip_paged_kv_decode_attention_config_validate(const SingePagedKvDecodeAttentionConfig* config);
+
+/* Scratch the split-KV decode needs, in bytes: per-split partial rows [batch, heads, splits, dim] f32
+ * followed by their natural-log LSE [batch, heads, splits] f32, the layout of the reference's
+ * caller-supplied split-KV scratch (mod.rs:2456-2539).  0 on an invalid config. */
+SINGE_HIP_API size_t singe_hip_paged_kv_decode_attention_workspace_bytes(const SingePagedKvDecodeAttentionConfig* config);
+
+/* paged_kv_decode_attention_bf16 (singe-kernel/src/cuda/attention/paged.rs:210-249).
+ * out/query [batch, heads, dim] bf16; caches [physical_blocks, block_size, kv_heads, dim] bf16;
+ * actual_seq_lens [batch] i32; block_table [batch, stride] u32.  *_len are element counts and are
+ * checked as PagedKvDecodeAttentionConfig::validate_lengths does (mod.rs:711-743).
+ * workspace: device scratch of at least ..._workspace_bytes(config), 256-byte aligned; it carries no
+ * state between calls. */
+SINGE_HIP_API int32_t singe_hip_paged_kv_decode_attention_bf16(
+    void* stream,
+    uint16_t* out, size_t out_len,
+    const uint16_t* query, size_t query_len,
+    const uint16_t* key_cache, size_t key_cache_len,
+    const uint16_t* value_cache, size_t value_cache_len,
+    const int32_t* actual_seq_lens, size_t actual_seq_lens_len,
+    const uint32_t* block_table, size_t block_table_len,
+    void* workspace, size_t workspace_bytes,
+    const SingePagedKvDecodeAttentionConfig* config);
+
+/* The same operation run phase by phase, as the reference exposes its split kernel and splitk_reduce
+ * separately (singe-kernel/src/cuda/attention/fmha.rs:1038,1155): SPLIT fills the scratch with one
+ * normalised partial row and natural-log LSE per (batch, head, split); REDUCE folds the scratch into
+ * `out` (cpu/attention.rs:2157-2193).  Both bits = the call above. */
+#define SINGE_HIP_DECODE_SPLIT 1u
+#define SINGE_HIP_DECODE_REDUCE 2u
+SINGE_HIP_API int32_t singe_hip_paged_kv_decode_attention_phases_bf16(
+    void* stream,
+    uint16_t* out, size_t out_len,
+    const uint16_t* query, size_t query_len,
+    const uint16_t* key_cache, size_t key_cache_len,
+    const uint16_t* value_cache, size_t value_cache_len,
+    const int32_t* actual_seq_lens, size_t actual_seq_lens_len,
+    const uint32_t* block_table, size_t block_table_len,
+    void* workspace, size_t workspace_bytes,
+    const SingePagedKvDecodeAttentionConfig* config,
+    uint32_t phases);
+
+/* Tuning knob of the split-KV decode: keys per split (a multiple of 32, 0 = built-in choice).  The
+ * counterpart of FmhaDecodeSplitKReduceConfig::max_splits / TuningChoice::Explicit
+ * (singe-kernel/src/cuda/attention/mod.rs:2364-2380).  Changes what ..._workspace_bytes returns. */
+SINGE_HIP_API void singe_hip_set_decode_keys_per_split(uint32_t keys);
+SINGE_HIP_API uint32_t singe_hip_decode_keys_per_split(const SingePagedKvDecodeAttentionConfig* config);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* SINGE_HIP_ATTENTION_H */

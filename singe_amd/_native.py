@@ -1,0 +1,96 @@
+"""ctypes binding of libsinge_hip_attention.so.  There is no fallback: if the library or its code
+object is missing the import of any op fails loudly."""
+from __future__ import annotations
+
+import ctypes
+import os
+
+from . import error
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIBRARY_PATH = os.path.join(_HERE, "libsinge_hip_attention.so")
+CODE_OBJECT_PATH = os.path.join(_HERE, "singe_attention_gfx950.hsaco")
+
+c_size = ctypes.c_size_t
+c_void = ctypes.c_void_p
+
+
+class ErrorDetail(ctypes.Structure):
+    _fields_ = [("status", ctypes.c_int32), ("name", ctypes.c_char_p), ("minimum", ctypes.c_uint64),
+                ("actual", ctypes.c_uint64)]
+
+
+class PagedKvDecodeAttentionConfigC(ctypes.Structure):
+    _fields_ = [("batch", c_size), ("heads", c_size), ("kv_heads", c_size), ("head_dim", c_size),
+                ("block_size", c_size), ("physical_blocks", c_size), ("block_table_batch_stride", c_size),
+                ("scale", ctypes.c_float)]
+
+
+_lib = None
+
+
+def lib() -> ctypes.CDLL:
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIBRARY_PATH):
+        raise error.KernelNotPrepared(
+            f"{LIBRARY_PATH} is missing: build it with `python -m singe_amd.build` (there is no fallback path)")
+    handle = ctypes.CDLL(LIBRARY_PATH)
+    i32 = ctypes.c_int32
+    handle.singe_hip_last_error.argtypes = [ctypes.POINTER(ErrorDetail)]
+    handle.singe_hip_last_error.restype = None
+    handle.singe_hip_status_string.argtypes = [i32]
+    handle.singe_hip_status_string.restype = ctypes.c_char_p
+    handle.singe_hip_load.argtypes = [c_void, c_size]
+    handle.singe_hip_load.restype = i32
+    handle.singe_hip_load_file.argtypes = [ctypes.c_char_p]
+    handle.singe_hip_load_file.restype = i32
+    handle.singe_hip_unload.argtypes = []
+    handle.singe_hip_unload.restype = None
+    handle.singe_hip_prepare.argtypes = [ctypes.POINTER(i32)]
+    handle.singe_hip_prepare.restype = i32
+    cfg = ctypes.POINTER(PagedKvDecodeAttentionConfigC)
+    handle.singe_hip_paged_kv_decode_attention_config_validate.argtypes = [cfg]
+    handle.singe_hip_paged_kv_decode_attention_config_validate.restype = i32
+    handle.singe_hip_paged_kv_decode_attention_workspace_bytes.argtypes = [cfg]
+    handle.singe_hip_paged_kv_decode_attention_workspace_bytes.restype = c_size
+    handle.singe_hip_paged_kv_decode_attention_bf16.argtypes = [
+        c_void, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size,
+        c_void, c_size, cfg]
+    handle.singe_hip_paged_kv_decode_attention_bf16.restype = i32
+    handle.singe_hip_paged_kv_decode_attention_phases_bf16.argtypes = [
+        c_void, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size,
+        c_void, c_size, cfg, ctypes.c_uint32]
+    handle.singe_hip_paged_kv_decode_attention_phases_bf16.restype = i32
+    handle.singe_hip_set_decode_keys_per_split.argtypes = [ctypes.c_uint32]
+    handle.singe_hip_set_decode_keys_per_split.restype = None
+    handle.singe_hip_decode_keys_per_split.argtypes = [cfg]
+    handle.singe_hip_decode_keys_per_split.restype = ctypes.c_uint32
+    _lib = handle
+    return handle
+
+
+def check(status: int, op: str = "") -> None:
+    """Turns a C status into the matching exception (the `try_ffi!` of this layer)."""
+    if status == 0:
+        return
+    detail = ErrorDetail()
+    lib().singe_hip_last_error(ctypes.byref(detail))
+    name = (detail.name or b"").decode()
+    if status < 0:
+        message = (lib().singe_hip_status_string(status) or b"").decode()
+        raise error.Hip(-status, message, name or op)
+    table = {
+        1: lambda: error.InvalidLength("invalid length"),
+        2: lambda: error.LengthTooShort(name, int(detail.minimum), int(detail.actual)),
+        3: lambda: error.LengthExceedsI32("length exceeds i32"),
+        4: lambda: error.SizeOverflow("size overflow"),
+        5: lambda: error.UnsupportedWidth(name or op, int(detail.minimum)),
+        6: lambda: error.NullPointer(f"null pointer: {name}"),
+        7: lambda: error.KernelNotPrepared(f"kernel specialization has not been prepared: {name}"),
+        8: lambda: error.UnsupportedConfiguration(f"unsupported configuration for {op}: {name}"),
+        9: lambda: error.InvalidArgument(f"{op} {name}"),
+        10: lambda: error.KernelNotPrepared("the HIP runtime library could not be opened"),
+    }
+    raise table.get(status, lambda: error.Error(f"status {status}"))()

@@ -1,0 +1,54 @@
+#include "hip_runtime_loader.h"
+
+#include <dlfcn.h>
+
+#include <mutex>
+
+namespace singe_hip {
+
+namespace {
+
+HipRuntime g_runtime;
+bool g_ready = false;
+std::once_flag g_once;
+
+void* open_runtime() {
+    // A runtime the process already holds wins, so streams and pointers created through it are ours too.
+    const char* names[] = {"libamdhip64.so.7", "libamdhip64.so", "libamdhip64.so.6"};
+    for (const char* name : names)
+        if (void* handle = dlopen(name, RTLD_NOW | RTLD_NOLOAD | RTLD_GLOBAL)) return handle;
+    for (const char* name : names)
+        if (void* handle = dlopen(name, RTLD_NOW | RTLD_GLOBAL)) return handle;
+    const char* fallbacks[] = {"/opt/rocm/lib/libamdhip64.so.7", "/opt/rocm/lib/libamdhip64.so"};
+    for (const char* name : fallbacks)
+        if (void* handle = dlopen(name, RTLD_NOW | RTLD_GLOBAL)) return handle;
+    return nullptr;
+}
+
+template <class F>
+bool resolve(void* handle, const char* name, F& slot) {
+    slot = reinterpret_cast<F>(dlsym(handle, name));
+    return slot != nullptr;
+}
+
+void load() {
+    void* handle = open_runtime();
+    if (handle == nullptr) return;
+    bool ok = true;
+    ok &= resolve(handle, "hipGetDevice", g_runtime.hipGetDevice);
+    ok &= resolve(handle, "hipModuleLoadData", g_runtime.hipModuleLoadData);
+    ok &= resolve(handle, "hipModuleUnload", g_runtime.hipModuleUnload);
+    ok &= resolve(handle, "hipModuleGetFunction", g_runtime.hipModuleGetFunction);
+    ok &= resolve(handle, "hipModuleLaunchKernel", g_runtime.hipModuleLaunchKernel);
+    ok &= resolve(handle, "hipGetErrorString", g_runtime.hipGetErrorString);
+    g_ready = ok;
+}
+
+}  // namespace
+
+const HipRuntime* hip_runtime() {
+    std::call_once(g_once, load);
+    return g_ready ? &g_runtime : nullptr;
+}
+
+}  // namespace singe_hip

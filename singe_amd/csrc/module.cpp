@@ -1,0 +1,177 @@
+#include "module.h"
+
+#include <dlfcn.h>
+
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "singe_hip_attention.h"
+
+namespace singe_hip {
+
+const char* const kKernelNames[kKernelCount] = {
+    "singe_paged_decode_bf16_d128_g1_b16",  "singe_paged_decode_bf16_d128_g2_b16",
+    "singe_paged_decode_bf16_d128_g4_b16",  "singe_paged_decode_bf16_d128_g8_b16",
+    "singe_paged_decode_bf16_d128_g16_b16", "singe_paged_decode_bf16_d128_g1_any",
+    "singe_paged_decode_bf16_d128_g2_any",  "singe_paged_decode_bf16_d128_g4_any",
+    "singe_paged_decode_bf16_d128_g8_any",  "singe_paged_decode_bf16_d128_g16_any",
+    "singe_paged_decode_combine_bf16",
+};
+
+namespace {
+
+thread_local SingeHipErrorDetail t_error = {0, "", 0, 0};
+
+constexpr int kMaxDevices = 64;
+
+struct DeviceModule {
+    hipModule_t module = nullptr;
+    bool loaded = false;
+    hipFunction_t functions[kKernelCount] = {};
+};
+
+std::mutex g_mutex;                 // guards the image and the per-device tables
+std::vector<unsigned char> g_image; // copy of the code object
+DeviceModule g_devices[kMaxDevices];
+
+std::string default_image_path() {
+    Dl_info info;
+    if (dladdr(reinterpret_cast<void*>(&default_image_path), &info) == 0 || info.dli_fname == nullptr) return "";
+    std::string path(info.dli_fname);
+    size_t slash = path.rfind('/');
+    path = slash == std::string::npos ? std::string(".") : path.substr(0, slash);
+    return path + "/singe_attention_gfx950.hsaco";
+}
+
+bool read_file(const std::string& path, std::vector<unsigned char>& bytes) {
+    FILE* file = std::fopen(path.c_str(), "rb");
+    if (file == nullptr) return false;
+    std::fseek(file, 0, SEEK_END);
+    long size = std::ftell(file);
+    std::fseek(file, 0, SEEK_SET);
+    bool ok = size > 0;
+    if (ok) {
+        bytes.resize(static_cast<size_t>(size));
+        ok = std::fread(bytes.data(), 1, bytes.size(), file) == bytes.size();
+    }
+    std::fclose(file);
+    return ok;
+}
+
+void drop_modules_locked() {
+    const HipRuntime* hip = hip_runtime();
+    for (DeviceModule& device : g_devices) {
+        if (device.loaded && hip != nullptr) hip->hipModuleUnload(device.module);
+        device = DeviceModule();
+    }
+}
+
+}  // namespace
+
+int32_t fail(int32_t status, const char* name, uint64_t minimum, uint64_t actual) {
+    t_error.status = status;
+    t_error.name = name;
+    t_error.minimum = minimum;
+    t_error.actual = actual;
+    return status;
+}
+
+int32_t fail_hip(hipError_t error, const char* what) { return fail(-static_cast<int32_t>(error), what); }
+
+int32_t kernel_function(KernelId kernel, hipFunction_t* function) {
+    const HipRuntime* hip = hip_runtime();
+    if (hip == nullptr) return fail(SINGE_HIP_RUNTIME_UNAVAILABLE, "libamdhip64");
+    int device = 0;
+    if (hipError_t error = hip->hipGetDevice(&device)) return fail_hip(error, "hipGetDevice");
+    if (device < 0 || device >= kMaxDevices) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "device index");
+    std::lock_guard<std::mutex> lock(g_mutex);
+    DeviceModule& slot = g_devices[device];
+    if (!slot.loaded) {
+        if (g_image.empty() && !read_file(default_image_path(), g_image))
+            return fail(SINGE_HIP_KERNEL_NOT_PREPARED, "singe_attention_gfx950.hsaco");
+        if (hipError_t error = hip->hipModuleLoadData(&slot.module, g_image.data())) return fail_hip(error, "hipModuleLoadData");
+        slot.loaded = true;
+    }
+    if (slot.functions[kernel] == nullptr) {
+        if (hipError_t error = hip->hipModuleGetFunction(&slot.functions[kernel], slot.module, kKernelNames[kernel])) {
+            slot.functions[kernel] = nullptr;
+            return fail_hip(error, kKernelNames[kernel]);
+        }
+    }
+    *function = slot.functions[kernel];
+    return 0;
+}
+
+}  // namespace singe_hip
+
+using namespace singe_hip;
+
+extern "C" {
+
+void singe_hip_last_error(SingeHipErrorDetail* detail) {
+    if (detail != nullptr) *detail = t_error;
+}
+
+const char* singe_hip_status_string(int32_t status) {
+    switch (status) {
+        case SINGE_HIP_OK: return "ok";
+        case SINGE_HIP_INVALID_LENGTH: return "invalid length";
+        case SINGE_HIP_LENGTH_TOO_SHORT: return "length too short";
+        case SINGE_HIP_LENGTH_EXCEEDS_I32: return "length exceeds i32";
+        case SINGE_HIP_SIZE_OVERFLOW: return "size overflow";
+        case SINGE_HIP_UNSUPPORTED_WIDTH: return "unsupported width";
+        case SINGE_HIP_NULL_POINTER: return "null pointer";
+        case SINGE_HIP_KERNEL_NOT_PREPARED: return "kernel specialization has not been prepared";
+        case SINGE_HIP_UNSUPPORTED_CONFIGURATION: return "unsupported configuration";
+        case SINGE_HIP_INVALID_ARGUMENT: return "invalid argument";
+        case SINGE_HIP_RUNTIME_UNAVAILABLE: return "hip runtime unavailable";
+        default: break;
+    }
+    if (status < 0) {
+        const HipRuntime* hip = hip_runtime();
+        if (hip != nullptr) return hip->hipGetErrorString(-status);
+        return "hip error";
+    }
+    return "unknown status";
+}
+
+int32_t singe_hip_load(const void* image, size_t bytes) {
+    if (image == nullptr) return fail(SINGE_HIP_NULL_POINTER, "image");
+    if (bytes == 0) return fail(SINGE_HIP_INVALID_LENGTH, "image");
+    std::lock_guard<std::mutex> lock(g_mutex);
+    drop_modules_locked();
+    g_image.assign(static_cast<const unsigned char*>(image), static_cast<const unsigned char*>(image) + bytes);
+    return 0;
+}
+
+int32_t singe_hip_load_file(const char* path) {
+    if (path == nullptr) return fail(SINGE_HIP_NULL_POINTER, "path");
+    std::vector<unsigned char> bytes;
+    if (!read_file(path, bytes)) return fail(SINGE_HIP_KERNEL_NOT_PREPARED, "code object file");
+    std::lock_guard<std::mutex> lock(g_mutex);
+    drop_modules_locked();
+    g_image.swap(bytes);
+    return 0;
+}
+
+void singe_hip_unload(void) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    drop_modules_locked();
+    g_image.clear();
+}
+
+int32_t singe_hip_prepare(int32_t* count) {
+    int32_t found = 0;
+    for (int kernel = 0; kernel < kKernelCount; ++kernel) {
+        hipFunction_t function = nullptr;
+        if (int32_t status = kernel_function(static_cast<KernelId>(kernel), &function)) return status;
+        ++found;
+    }
+    if (count != nullptr) *count = found;
+    return 0;
+}
+
+}  // extern "C"

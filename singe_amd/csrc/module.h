@@ -1,0 +1,40 @@
+// Code-object handling: the gfx950 image, its per-device hipModule_t, and the kernel handles.
+// Stands in for the reference's Context::load_module / Module::function pair
+// (singe-cuda/src/context.rs:363-385, singe-cuda/src/module/mod.rs:387-410).
+#pragma once
+
+#include "hip_runtime_loader.h"
+
+namespace singe_hip {
+
+// Kernels of the code object, in the order of kKernelNames.
+enum KernelId : int {
+    kDecodeG1B16 = 0, kDecodeG2B16, kDecodeG4B16, kDecodeG8B16, kDecodeG16B16,
+    kDecodeG1Any, kDecodeG2Any, kDecodeG4Any, kDecodeG8Any, kDecodeG16Any,
+    kDecodeCombine,
+    kKernelCount
+};
+
+extern const char* const kKernelNames[kKernelCount];
+
+// Status of the thread's last failure (see singe_hip_last_error).
+int32_t fail(int32_t status, const char* name = "", uint64_t minimum = 0, uint64_t actual = 0);
+int32_t fail_hip(hipError_t error, const char* what);
+
+// The handle of `kernel` on the current device, loading the module there on first use.
+// Returns 0 and sets *function, or a status.
+int32_t kernel_function(KernelId kernel, hipFunction_t* function);
+
+// hipModuleLaunchKernel of a kernel that takes one argument block by value.
+template <class Args>
+int32_t launch(KernelId kernel, unsigned grid_x, unsigned grid_y, unsigned grid_z, unsigned threads,
+               hipStream_t stream, Args& args) {
+    hipFunction_t function = nullptr;
+    if (int32_t status = kernel_function(kernel, &function)) return status;
+    void* params[] = {&args};
+    hipError_t error = hip_runtime()->hipModuleLaunchKernel(function, grid_x, grid_y, grid_z, threads, 1, 1, 0,
+                                                            stream, params, nullptr);
+    return error == hipSuccess ? 0 : fail_hip(error, kKernelNames[kernel]);
+}
+
+}  // namespace singe_hip

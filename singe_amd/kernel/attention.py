@@ -1,0 +1,130 @@
+"""Host-side mirror of ``singe_kernel::cuda::attention`` for the paged / dense attention path.
+
+Same names, argument order and error behaviour as the reference's launch functions
+(singe-kernel/src/cuda/attention/paged.rs:118-420, fmha.rs:584-790) and config structs
+(mod.rs:76-108, 253-274).  Device buffers are torch tensors (a pointer plus an element count, which
+is all the reference's DeviceInput/DeviceOutput carry); ``stream`` is a ``torch.cuda.Stream`` or
+``None`` for the current one.  Every call only enqueues work.
+"""
+from __future__ import annotations
+
+import ctypes
+import math
+from dataclasses import dataclass
+
+import torch
+
+from .. import _native, error
+
+I32_MAX = 2**31 - 1
+
+
+def _stream_handle(stream) -> int:
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return int(stream.cuda_stream)
+
+
+def _ptr(tensor: torch.Tensor) -> int:
+    return int(tensor.data_ptr())
+
+
+def _require(tensor: torch.Tensor, dtype: torch.dtype, name: str) -> None:
+    if not isinstance(tensor, torch.Tensor) or not tensor.is_cuda:
+        raise error.NullPointer(f"{name} is not a device buffer")
+    if tensor.dtype != dtype:
+        raise error.InvalidArgument(f"{name} must be {dtype}, got {tensor.dtype}")
+    if not tensor.is_contiguous():
+        raise error.InvalidArgument(f"{name} must be contiguous")
+
+
+@dataclass(frozen=True)
+class PagedKvDecodeAttentionConfig:
+    """Decode attention over paged KV caches (mod.rs:76-90): one query token per batch item, caches
+    addressed through a per-batch block table, ``actual_seq_lens`` selecting each item's prefix."""
+    batch: int
+    heads: int
+    kv_heads: int
+    head_dim: int
+    block_size: int
+    physical_blocks: int
+    block_table_batch_stride: int
+    scale: float
+
+    @classmethod
+    def contiguous(cls, batch, heads, kv_heads, head_dim, block_size, physical_blocks,
+                   block_table_batch_stride, scale) -> "PagedKvDecodeAttentionConfig":
+        """mod.rs:686-709: builds the config and validates it."""
+        config = cls(batch, heads, kv_heads, head_dim, block_size, physical_blocks, block_table_batch_stride, scale)
+        config.validate()
+        return config
+
+    def validate(self) -> None:
+        """validate_paged_kv_decode_attention_config (mod.rs:2963-2985)."""
+        extents = (self.batch, self.heads, self.kv_heads, self.head_dim, self.block_size, self.physical_blocks,
+                   self.block_table_batch_stride)
+        if any(e <= 0 for e in extents) or self.heads % self.kv_heads != 0 or not math.isfinite(self.scale):
+            raise error.InvalidLength("invalid length")
+        if any(e > I32_MAX for e in extents):
+            raise error.LengthExceedsI32("length exceeds i32")
+
+    def output_len(self) -> int:
+        return self.batch * self.heads * self.head_dim
+
+    def _c(self) -> _native.PagedKvDecodeAttentionConfigC:
+        return _native.PagedKvDecodeAttentionConfigC(self.batch, self.heads, self.kv_heads, self.head_dim,
+                                                     self.block_size, self.physical_blocks,
+                                                     self.block_table_batch_stride, self.scale)
+
+    def workspace_bytes(self) -> int:
+        c = self._c()
+        return int(_native.lib().singe_hip_paged_kv_decode_attention_workspace_bytes(ctypes.byref(c)))
+
+
+class _Workspaces:
+    """One scratch buffer per device, grown on demand.  The C ABI never allocates; this host layer
+    owns the scratch the way the reference's callers own split-KV scratch (mod.rs:2456-2539)."""
+
+    def __init__(self):
+        self._buffers = {}
+
+    def get(self, device: torch.device, nbytes: int) -> torch.Tensor:
+        key = device.index if device.index is not None else torch.cuda.current_device()
+        buffer = self._buffers.get(key)
+        if buffer is None or buffer.numel() < nbytes:
+            buffer = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+            self._buffers[key] = buffer
+        return buffer
+
+
+_workspaces = _Workspaces()
+
+
+def paged_kv_decode_attention_bf16(stream, out: torch.Tensor, query: torch.Tensor, key_cache: torch.Tensor,
+                                   value_cache: torch.Tensor, actual_seq_lens: torch.Tensor,
+                                   block_table: torch.Tensor, config: PagedKvDecodeAttentionConfig,
+                                   workspace: torch.Tensor | None = None, phases: int = 3) -> None:
+    """paged_kv_decode_attention_bf16 (paged.rs:210-249).
+
+    out/query [batch, heads, dim] bf16; caches [blocks, block_size, kv_heads, dim] bf16;
+    actual_seq_lens [batch] i32; block_table [batch, stride] u32 (an int32 tensor is read as u32).
+    ``phases``: 1 = split kernel only (fills the scratch), 2 = reduce only, 3 = both (the op).
+    """
+    _require(out, torch.bfloat16, "out")
+    _require(query, torch.bfloat16, "query")
+    _require(key_cache, torch.bfloat16, "key_cache")
+    _require(value_cache, torch.bfloat16, "value_cache")
+    _require(actual_seq_lens, torch.int32, "actual_seq_lens")
+    if block_table.dtype not in (torch.int32, torch.uint32):
+        raise error.InvalidArgument(f"block_table must hold 32-bit entries, got {block_table.dtype}")
+    _require(block_table, block_table.dtype, "block_table")
+    c = config._c()
+    if workspace is None:
+        need = int(_native.lib().singe_hip_paged_kv_decode_attention_workspace_bytes(ctypes.byref(c)))
+        workspace = _workspaces.get(out.device, need)
+    status = _native.lib().singe_hip_paged_kv_decode_attention_phases_bf16(
+        _stream_handle(stream), _ptr(out), out.numel(), _ptr(query), query.numel(), _ptr(key_cache),
+        key_cache.numel(), _ptr(value_cache), value_cache.numel(), _ptr(actual_seq_lens),
+        actual_seq_lens.numel(), _ptr(block_table), block_table.numel(), _ptr(workspace),
+        workspace.numel() * workspace.element_size(), ctypes.byref(c), phases)
+    _native.check(status, "paged_kv_decode_attention_bf16")

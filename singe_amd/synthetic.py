@@ -1,0 +1,98 @@
+"""Seeded synthetic workloads of the shapes the benchmark configurations name.
+
+Integer inputs (lengths, block tables, page lists) are drawn on the host with numpy's PCG64 so tests,
+the benchmark and the CPU baseline see the same values; float tensors are drawn N(0, 1) with a torch
+generator on the requested device and rounded to the storage type.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+BASE_SEED = 0x51A6E
+
+
+@dataclass
+class PagedDecodeWorkload:
+    """Paged decode, one query token per sequence (singe-kernel surface)."""
+    batch: int
+    heads: int
+    kv_heads: int
+    head_dim: int
+    block_size: int
+    physical_blocks: int
+    block_table_batch_stride: int
+    scale: float
+    seq_lens: np.ndarray      # [batch] int32
+    block_table: np.ndarray   # [batch, stride] uint32
+    query: torch.Tensor       # [batch, heads, dim]
+    key_cache: torch.Tensor   # [blocks, block_size, kv_heads, dim]
+    value_cache: torch.Tensor
+
+    @property
+    def total_keys(self) -> int:
+        return int(self.seq_lens.astype(np.int64).sum())
+
+    def algorithmic_bytes(self, kv_element_bytes: int = 2) -> int:
+        """Every operand element read or written once: valid KV rows, Q, O, the table entries used,
+        the lengths."""
+        kv = self.total_keys * 2 * self.kv_heads * self.head_dim * kv_element_bytes
+        qo = 2 * self.batch * self.heads * self.head_dim * 2
+        used = int(np.sum((self.seq_lens.astype(np.int64) + self.block_size - 1) // self.block_size))
+        return kv + qo + used * 4 + self.batch * 4
+
+    def algorithmic_flops(self) -> int:
+        return 4 * self.heads * self.head_dim * self.total_keys
+
+
+def paged_block_table(rng: np.random.Generator, seq_lens: np.ndarray, block_size: int, physical_blocks: int,
+                      stride: int | None = None):
+    """Consecutive slices of a seeded permutation of the block pool become the rows of the table;
+    unused entries are zero."""
+    counts = (seq_lens.astype(np.int64) + block_size - 1) // block_size
+    if stride is None:
+        stride = max(int(counts.max()), 1)
+    if int(counts.sum()) > physical_blocks:
+        raise ValueError("block pool too small")
+    perm = rng.permutation(physical_blocks)
+    table = np.zeros((len(seq_lens), stride), dtype=np.uint32)
+    at = 0
+    for b, n in enumerate(counts):
+        table[b, :n] = perm[at:at + n]
+        at += int(n)
+    return table, stride
+
+
+def paged_decode_workload(*, batch=32, heads=32, kv_heads=8, head_dim=128, block_size=16, physical_blocks=16384,
+                          min_len=512, max_len=4096, seed=BASE_SEED, device="cuda", dtype=torch.bfloat16,
+                          fill="all", seq_lens=None) -> PagedDecodeWorkload:
+    """batch sequences with context lengths uniform in [min_len, max_len], block tables drawn as a
+    seeded permutation of the physical pool.  ``fill='used'`` only draws the referenced blocks (the
+    rest stay zero), which is enough for parity tests on large pools."""
+    rng = np.random.default_rng(seed)
+    if seq_lens is None:
+        seq_lens = rng.integers(min_len, max_len + 1, size=batch).astype(np.int32)
+    else:
+        seq_lens = np.asarray(seq_lens, dtype=np.int32)
+    table, stride = paged_block_table(rng, seq_lens, block_size, physical_blocks)
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed + 1)
+    query = torch.randn((batch, heads, head_dim), generator=gen, device=device, dtype=torch.float32).to(dtype)
+    shape = (physical_blocks, block_size, kv_heads, head_dim)
+    if fill == "all":
+        key_cache = torch.randn(shape, generator=gen, device=device, dtype=torch.float32).to(dtype)
+        value_cache = torch.randn(shape, generator=gen, device=device, dtype=torch.float32).to(dtype)
+    else:
+        key_cache = torch.zeros(shape, device=device, dtype=dtype)
+        value_cache = torch.zeros(shape, device=device, dtype=dtype)
+        counts = (seq_lens.astype(np.int64) + block_size - 1) // block_size
+        used = np.concatenate([table[b, :n] for b, n in enumerate(counts)]).astype(np.int64)
+        index = torch.from_numpy(used).to(device)
+        sub = (len(used), block_size, kv_heads, head_dim)
+        key_cache[index] = torch.randn(sub, generator=gen, device=device, dtype=torch.float32).to(dtype)
+        value_cache[index] = torch.randn(sub, generator=gen, device=device, dtype=torch.float32).to(dtype)
+    return PagedDecodeWorkload(batch, heads, kv_heads, head_dim, block_size, physical_blocks, stride,
+                               float(1.0 / np.sqrt(np.float32(head_dim))), seq_lens, table, query, key_cache,
+                               value_cache)

@@ -1,0 +1,198 @@
+"""Paged decode on the GPU against the CPU oracle, through the C ABI (ctypes -> libsinge_hip_attention.so
+-> hipModuleLaunchKernel).  Tolerance for bf16 outputs: max-abs 2e-2 and mean-abs 2e-3 against the
+oracle run on the same bf16-rounded inputs widened to f32; gather indices and lengths bit-exact."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from singe_amd import error, synthetic
+from singe_amd.kernel import attention as A
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_ABS = 2e-2, 2e-3
+
+
+def compact(work):
+    """The referenced blocks only, renumbered, as f32 on the host (the oracle is invariant under a
+    permutation of physical blocks, which tests/test_oracle.py pins)."""
+    counts = (work.seq_lens.astype(np.int64) + work.block_size - 1) // work.block_size
+    used = np.concatenate([work.block_table[b, :n] for b, n in enumerate(counts)] + [np.zeros(0, np.uint32)]).astype(np.int64)
+    if len(used) == 0:
+        used = np.zeros(1, dtype=np.int64)
+    remap = np.zeros(work.physical_blocks, dtype=np.uint32)
+    remap[used] = np.arange(len(used), dtype=np.uint32)
+    table = np.zeros_like(work.block_table)
+    for b, n in enumerate(counts):
+        table[b, :n] = remap[work.block_table[b, :n]]
+    index = torch.from_numpy(used).to(work.key_cache.device)
+    kc = work.key_cache[index].float().cpu().numpy()
+    vc = work.value_cache[index].float().cpu().numpy()
+    return kc, vc, table
+
+
+def run_gpu(work, keys_per_split=0):
+    A._native.lib().singe_hip_set_decode_keys_per_split(keys_per_split)
+    try:
+        config = A.PagedKvDecodeAttentionConfig.contiguous(work.batch, work.heads, work.kv_heads, work.head_dim,
+                                                           work.block_size, work.physical_blocks,
+                                                           work.block_table_batch_stride, work.scale)
+        out = torch.full((work.batch, work.heads, work.head_dim), float("nan"), device="cuda", dtype=torch.bfloat16)
+        lens = torch.from_numpy(work.seq_lens).cuda()
+        table = torch.from_numpy(work.block_table.view(np.int32)).cuda()
+        A.paged_kv_decode_attention_bf16(None, out, work.query, work.key_cache, work.value_cache, lens, table, config)
+        torch.cuda.synchronize()
+    finally:
+        A._native.lib().singe_hip_set_decode_keys_per_split(0)
+    return out.float().cpu().numpy()
+
+
+def run_oracle(work):
+    kc, vc, table = compact(work)
+    return oracle.paged_kv_decode_attention_f32(
+        work.query.float().cpu().numpy(), kc, vc, work.seq_lens, table, batch=work.batch, heads=work.heads,
+        kv_heads=work.kv_heads, head_dim=work.head_dim, block_size=work.block_size,
+        block_table_batch_stride=work.block_table_batch_stride, scale=work.scale, threads=8)
+
+
+def assert_close(got, want, label=""):
+    assert np.isfinite(got).all(), f"{label}: non-finite output"
+    gap = np.abs(got - want)
+    assert gap.max() <= MAX_ABS, f"{label}: max-abs {gap.max()}"
+    assert gap.mean() <= MEAN_ABS, f"{label}: mean-abs {gap.mean()}"
+
+
+def test_decode_headline_shape_matches_oracle():
+    # batch 32, 32 query / 8 kv heads, dim 128, block 16, context U[512, 4096], 16384-block pool
+    work = synthetic.paged_decode_workload(fill="used")
+    print(f"total keys {work.total_keys}", flush=True)
+    assert_close(run_gpu(work), run_oracle(work), "headline")
+
+
+@pytest.mark.parametrize("heads,kv_heads", [(8, 8), (8, 4), (12, 4), (8, 2), (6, 1), (8, 1), (16, 1), (24, 2)])
+def test_decode_group_sizes(heads, kv_heads):
+    lens = [0, 1, 15, 16, 17, 31, 32, 33, 100, 257, 300, 64]
+    work = synthetic.paged_decode_workload(batch=len(lens), heads=heads, kv_heads=kv_heads, physical_blocks=256,
+                                           seq_lens=lens, seed=100 + heads * 31 + kv_heads)
+    got, want = run_gpu(work), run_oracle(work)
+    assert not got[0].any()  # an empty sequence keeps a zero row (cpu/attention.rs:1213-1215)
+    assert_close(got, want, f"{heads}/{kv_heads}")
+
+
+@pytest.mark.parametrize("block_size", [1, 7, 16, 32, 48, 5])
+@pytest.mark.parametrize("keys_per_split", [0, 32, 96, 4096])
+def test_decode_block_sizes_and_splits(block_size, keys_per_split):
+    lens = [200, 1, 333, 0, 97, 160, 31, 512]
+    blocks = sum((l + block_size - 1) // block_size for l in lens) + 9
+    work = synthetic.paged_decode_workload(batch=len(lens), heads=8, kv_heads=2, block_size=block_size,
+                                           physical_blocks=blocks, seq_lens=lens, seed=7 + block_size)
+    assert_close(run_gpu(work, keys_per_split), run_oracle(work), f"block {block_size} split {keys_per_split}")
+
+
+def test_decode_table_stride_wider_than_needed_and_poisoned_tail():
+    # Entries past a sequence's blocks hold an out-of-range block id and every cache row that no key
+    # owns is NaN: a single read outside the gather set would poison the output.
+    lens = np.array([130, 16, 47, 0, 255, 1], dtype=np.int32)
+    work = synthetic.paged_decode_workload(batch=len(lens), heads=8, kv_heads=2, physical_blocks=128,
+                                           seq_lens=lens, seed=11)
+    wide = np.full((work.batch, work.block_table_batch_stride + 5), 0xFFFFFFFF, dtype=np.uint32)
+    owned = torch.zeros((work.physical_blocks, work.block_size), dtype=torch.bool)
+    for b, length in enumerate(lens):
+        n = (int(length) + 15) // 16
+        wide[b, :n] = work.block_table[b, :n]
+        for key in range(int(length)):
+            owned[int(work.block_table[b, key // 16]), key % 16] = True
+    work.block_table, work.block_table_batch_stride = wide, wide.shape[1]
+    poison = (~owned).cuda()
+    work.key_cache[poison] = float("nan")
+    work.value_cache[poison] = float("nan")
+    got = run_gpu(work)
+    clean_k, clean_v = work.key_cache.clone(), work.value_cache.clone()
+    clean_k[poison], clean_v[poison] = 0, 0
+    work.key_cache, work.value_cache = clean_k, clean_v
+    work.block_table = np.where(wide == 0xFFFFFFFF, 0, wide).astype(np.uint32)
+    assert_close(got, run_oracle(work), "poisoned tail")
+
+
+def test_decode_gather_indices_are_bit_exact():
+    # Each cache row carries its own (block, slot) in bf16-exact integers and one key per sequence
+    # dominates the softmax, so the output row IS the gathered row: its index must equal the oracle's.
+    rng = np.random.default_rng(5)
+    batch, heads, kv_heads, dim, bs, blocks = 16, 8, 2, 128, 16, 4096
+    lens = rng.integers(1, 700, size=batch).astype(np.int32)
+    lens[:3] = [1, 16, 17]
+    work = synthetic.paged_decode_workload(batch=batch, heads=heads, kv_heads=kv_heads, block_size=bs,
+                                           physical_blocks=blocks, seq_lens=lens, seed=21)
+    ident = torch.zeros((blocks, bs, kv_heads, dim), dtype=torch.float32)
+    block_id = torch.arange(blocks).view(-1, 1, 1)
+    ident[..., 0] = (block_id % 256).float()
+    ident[..., 1] = (block_id // 256).float()
+    ident[..., 2] = torch.arange(bs).view(1, -1, 1).float()
+    ident[..., 3] = torch.arange(kv_heads).view(1, 1, -1).float()
+    work.value_cache = ident.to(torch.bfloat16).cuda()
+    for which in ("first", "last", "random"):
+        target = {"first": np.zeros(batch, np.int64), "last": lens.astype(np.int64) - 1,
+                  "random": rng.integers(0, lens)}[which]
+        keys = torch.zeros((blocks, bs, kv_heads, dim), dtype=torch.float32)
+        query = torch.ones((batch, heads, dim), dtype=torch.float32)
+        for b in range(batch):
+            blk = int(work.block_table[b, target[b] // bs])
+            keys[blk, target[b] % bs] = 8.0  # score 8 * 128 * scale ~ 90 above the zero rows
+        work.key_cache, work.query = keys.to(torch.bfloat16).cuda(), query.to(torch.bfloat16).cuda()
+        got = run_gpu(work)
+        for g in range(kv_heads):
+            offsets = oracle.paged_gather_offsets(lens, work.block_table, kv_heads=kv_heads, head_dim=dim,
+                                                  block_size=bs, block_table_batch_stride=work.block_table_batch_stride,
+                                                  kv_head=g)
+            starts = np.concatenate([[0], np.cumsum(lens.astype(np.int64))])
+            for b in range(batch):
+                want = int(offsets[starts[b] + target[b]])
+                for h in range(g * (heads // kv_heads), (g + 1) * (heads // kv_heads)):
+                    row = got[b, h]
+                    seen = (((int(row[0]) + 256 * int(row[1])) * bs + int(row[2])) * kv_heads + int(row[3])) * dim
+                    assert seen == want, (which, b, h, seen, want)
+
+
+def test_decode_lengths_are_exact():
+    # Uniform scores: the row is the mean of exactly seq_len value rows.  The key right after the
+    # last one holds a huge value, the last one a distinctive one: one key too many or too few shows.
+    lens = np.array([1, 2, 16, 17, 31, 33, 255, 256, 257, 1000], dtype=np.int32)
+    work = synthetic.paged_decode_workload(batch=len(lens), heads=4, kv_heads=1, physical_blocks=512,
+                                           seq_lens=lens, seed=31)
+    work.query = torch.zeros_like(work.query)
+    values = torch.zeros_like(work.value_cache, dtype=torch.float32)
+    for b, length in enumerate(lens):
+        last = int(length) - 1
+        values[int(work.block_table[b, last // 16]), last % 16] = float(length)
+        nxt = int(length)
+        if nxt // 16 < work.block_table_batch_stride and nxt % 16 != 0:
+            values[int(work.block_table[b, nxt // 16]), nxt % 16] = 3.0e4
+    work.value_cache = values.to(torch.bfloat16).cuda()
+    got = run_gpu(work)
+    assert np.abs(got - 1.0).max() <= 2 ** -8  # mean = length / length, rounded once to bf16
+
+
+def test_decode_validation_errors_match_the_reference():
+    good = dict(batch=2, heads=8, kv_heads=2, head_dim=128, block_size=16, physical_blocks=8,
+                block_table_batch_stride=4, scale=0.1)
+    for bad in (dict(batch=0), dict(heads=7), dict(scale=float("nan")), dict(block_size=0)):
+        with pytest.raises(error.InvalidLength):
+            A.PagedKvDecodeAttentionConfig.contiguous(**{**good, **bad})
+    with pytest.raises(error.LengthExceedsI32):
+        A.PagedKvDecodeAttentionConfig.contiguous(**{**good, "physical_blocks": 2**31})
+    config = A.PagedKvDecodeAttentionConfig.contiguous(**good)
+    out = torch.zeros((2, 8, 128), device="cuda", dtype=torch.bfloat16)
+    cache = torch.zeros((8, 16, 2, 128), device="cuda", dtype=torch.bfloat16)
+    lens = torch.zeros(2, device="cuda", dtype=torch.int32)
+    table = torch.zeros((2, 4), device="cuda", dtype=torch.int32)
+    with pytest.raises(error.LengthTooShort) as caught:
+        A.paged_kv_decode_attention_bf16(None, out, out.clone(), cache[:7], cache, lens, table, config)
+    assert caught.value.minimum == 8 * 16 * 2 * 128 and caught.value.actual == 7 * 16 * 2 * 128
+    with pytest.raises(error.UnsupportedWidth):
+        A.paged_kv_decode_attention_bf16(None, out, out.clone(), cache, cache, lens, table,
+                                         A.PagedKvDecodeAttentionConfig.contiguous(**{**good, "head_dim": 96, "heads": 8}))
+    A.paged_kv_decode_attention_bf16(None, out, out.clone(), cache, cache, lens, table, config)
+    torch.cuda.synchronize()
