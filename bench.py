@@ -32,7 +32,7 @@ def parse():
     parser.add_argument("--steps", type=int, default=300)
     parser.add_argument("--warmup", type=int, default=30)
     parser.add_argument("--no-cpu-baseline", action="store_true")
-    parser.add_argument("--keys-per-split", type=int, default=0, help="tuning override (0 = built-in choice)")
+    parser.add_argument("--workers", type=int, default=0, help="tuning override (0 = built-in choice)")
     return parser.parse_args()
 
 
@@ -91,8 +91,8 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
-    if args.keys_per_split:
-        _native.lib().singe_hip_set_decode_keys_per_split(args.keys_per_split)
+    if args.workers:
+        _native.lib().singe_hip_set_decode_workers(args.workers)
 
     work = synthetic.paged_decode_workload()
     pools = [(work.key_cache, work.value_cache)]
@@ -156,14 +156,14 @@ def main():
             "total_keys": work.total_keys,
             "algorithmic_bytes": bytes_per_step,
             "algorithmic_flops": work.algorithmic_flops(),
-            "keys_per_split": int(_native.lib().singe_hip_decode_keys_per_split(config._c())),
+            "workers": int(_native.lib().singe_hip_decode_workers(config._c())),
             "kv_pools_rotated": POOLS,
         },
         "tokens_per_s": work.batch / (ms_per_step * 1e-3),
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
         "roofline": {
             "bound": "hbm",
-            "kernel": "singe_paged_decode_bf16_d128_g4_b16",
+            "kernel": "singe_paged_decode_bf16_d128_p2_b16",
             "achieved": achieved,
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",

@@ -83,9 +83,10 @@ typedef struct SingePagedKvDecodeAttentionConfig {
 /* validate_paged_kv_decode_attention_config (mod.rs:2963-2985). */
 SINGE_HIP_API int32_t singe_hip_paged_kv_decode_attention_config_validate(const SingePagedKvDecodeAttentionConfig* config);
 
-/* Scratch the split-KV decode needs, in bytes: per-split partial rows [batch, heads, splits, dim] f32
- * followed by their natural-log LSE [batch, heads, splits] f32, the layout of the reference's
- * caller-supplied split-KV scratch (mod.rs:2456-2539).  0 on an invalid config. */
+/* Scratch the split-KV decode needs, in bytes: one normalised partial row (f32) and natural-log LSE
+ * per (kv head, key range, sequence the range touches), plus the per-sequence tile prefix the reduce
+ * step reads; caller-supplied like the reference's split-KV scratch (mod.rs:2456-2539).  Depends on
+ * the device's compute-unit count.  0 on an invalid config. */
 SINGE_HIP_API size_t singe_hip_paged_kv_decode_attention_workspace_bytes(const SingePagedKvDecodeAttentionConfig* config);
 
 /* paged_kv_decode_attention_bf16 (singe-kernel/src/cuda/attention/paged.rs:210-249).
@@ -106,8 +107,8 @@ SINGE_HIP_API int32_t singe_hip_paged_kv_decode_attention_bf16(
     const SingePagedKvDecodeAttentionConfig* config);
 
 /* The same operation run phase by phase, as the reference exposes its split kernel and splitk_reduce
- * separately (singe-kernel/src/cuda/attention/fmha.rs:1038,1155): SPLIT fills the scratch with one
- * normalised partial row and natural-log LSE per (batch, head, split); REDUCE folds the scratch into
+ * separately (singe-kernel/src/cuda/attention/fmha.rs:1038,1155): SPLIT fills the scratch with the
+ * normalised partial rows and natural-log LSEs of every key range; REDUCE folds the scratch into
  * `out` (cpu/attention.rs:2157-2193).  Both bits = the call above. */
 #define SINGE_HIP_DECODE_SPLIT 1u
 #define SINGE_HIP_DECODE_REDUCE 2u
@@ -123,11 +124,12 @@ SINGE_HIP_API int32_t singe_hip_paged_kv_decode_attention_phases_bf16(
     const SingePagedKvDecodeAttentionConfig* config,
     uint32_t phases);
 
-/* Tuning knob of the split-KV decode: keys per split (a multiple of 32, 0 = built-in choice).  The
- * counterpart of FmhaDecodeSplitKReduceConfig::max_splits / TuningChoice::Explicit
+/* Tuning knob of the split-KV decode: the number of equal key ranges each kv head's keys are cut
+ * into (0 = one workgroup per compute unit).  The counterpart of
+ * FmhaDecodeSplitKReduceConfig::max_splits / TuningChoice::Explicit
  * (singe-kernel/src/cuda/attention/mod.rs:2364-2380).  Changes what ..._workspace_bytes returns. */
-SINGE_HIP_API void singe_hip_set_decode_keys_per_split(uint32_t keys);
-SINGE_HIP_API uint32_t singe_hip_decode_keys_per_split(const SingePagedKvDecodeAttentionConfig* config);
+SINGE_HIP_API void singe_hip_set_decode_workers(uint32_t workers);
+SINGE_HIP_API uint32_t singe_hip_decode_workers(const SingePagedKvDecodeAttentionConfig* config);
 
 #ifdef __cplusplus
 }

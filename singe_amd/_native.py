@@ -63,10 +63,10 @@ def lib() -> ctypes.CDLL:
         c_void, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size,
         c_void, c_size, cfg, ctypes.c_uint32]
     handle.singe_hip_paged_kv_decode_attention_phases_bf16.restype = i32
-    handle.singe_hip_set_decode_keys_per_split.argtypes = [ctypes.c_uint32]
-    handle.singe_hip_set_decode_keys_per_split.restype = None
-    handle.singe_hip_decode_keys_per_split.argtypes = [cfg]
-    handle.singe_hip_decode_keys_per_split.restype = ctypes.c_uint32
+    handle.singe_hip_set_decode_workers.argtypes = [ctypes.c_uint32]
+    handle.singe_hip_set_decode_workers.restype = None
+    handle.singe_hip_decode_workers.argtypes = [cfg]
+    handle.singe_hip_decode_workers.restype = ctypes.c_uint32
     _lib = handle
     return handle
 

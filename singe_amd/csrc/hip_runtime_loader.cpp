@@ -36,6 +36,7 @@ void load() {
     if (handle == nullptr) return;
     bool ok = true;
     ok &= resolve(handle, "hipGetDevice", g_runtime.hipGetDevice);
+    ok &= resolve(handle, "hipDeviceGetAttribute", g_runtime.hipDeviceGetAttribute);
     ok &= resolve(handle, "hipModuleLoadData", g_runtime.hipModuleLoadData);
     ok &= resolve(handle, "hipModuleUnload", g_runtime.hipModuleUnload);
     ok &= resolve(handle, "hipModuleGetFunction", g_runtime.hipModuleGetFunction);

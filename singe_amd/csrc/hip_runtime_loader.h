@@ -18,6 +18,7 @@ constexpr hipError_t hipSuccess = 0;
 
 struct HipRuntime {
     hipError_t (*hipGetDevice)(int*);
+    hipError_t (*hipDeviceGetAttribute)(int*, int, int);
     hipError_t (*hipModuleLoadData)(hipModule_t*, const void*);
     hipError_t (*hipModuleUnload)(hipModule_t);
     hipError_t (*hipModuleGetFunction)(hipFunction_t*, hipModule_t, const char*);

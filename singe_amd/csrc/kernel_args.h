@@ -11,27 +11,33 @@ struct DecodeArgs {
     const uint16_t* value_cache;
     const int32_t* actual_seq_lens; // [batch]
     const uint32_t* block_table;    // [batch, stride]
-    float* partial_out;             // [batch, heads, splits, 128]
-    float* partial_lse;             // [batch, heads, splits], natural log
+    float* partial_out;             // [work, workers + batch, heads_per_wave, 128]
+    float* partial_lse;             // [work, workers + batch, heads_per_wave], natural log
+    uint32_t* meta;                 // [0] tiles per worker, [1] total tiles, [2 + b] tiles before sequence b
+    uint32_t batch;
     uint32_t heads;
     uint32_t kv_heads;
     uint32_t block_size;
     int32_t block_shift;            // log2(block_size) when it is a power of two, else -1
     uint32_t physical_blocks;
     uint32_t block_table_batch_stride;
-    uint32_t splits;                // scratch rows per (batch, head)
-    uint32_t keys_per_split;        // multiple of 32
+    uint32_t workers;               // equal ranges the flat tile list is cut into
+    uint32_t workers_per_wg;        // ranges one workgroup walks (each by work_per_wg waves)
+    uint32_t work_per_wg;           // (kv head, head group) pairs one workgroup covers
+    uint32_t head_groups;           // waves a kv head's query heads are spread over: ceil(group / 8)
+    uint32_t heads_per_wave;        // min(group, 8): partial rows per slot
     float scale_log2e;              // scale * log2(e)
 };
 
 struct CombineArgs {
-    uint16_t* out;                  // [batch, heads, dim] bf16
-    const float* partial_out;       // [batch, heads, splits, dim]
-    const float* partial_lse;       // [batch, heads, splits]
-    const int32_t* actual_seq_lens;
+    uint16_t* out;                  // [batch, heads, 128] bf16
+    const float* partial_out;
+    const float* partial_lse;
+    const uint32_t* meta;
+    uint32_t batch;
     uint32_t heads;
-    uint32_t dim;
-    uint32_t splits;
-    uint32_t keys_per_split;
-    uint32_t reach;                 // block_table_batch_stride * block_size
+    uint32_t kv_heads;
+    uint32_t workers;
+    uint32_t head_groups;
+    uint32_t heads_per_wave;
 };

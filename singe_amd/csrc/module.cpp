@@ -13,11 +13,9 @@
 namespace singe_hip {
 
 const char* const kKernelNames[kKernelCount] = {
-    "singe_paged_decode_bf16_d128_g1_b16",  "singe_paged_decode_bf16_d128_g2_b16",
-    "singe_paged_decode_bf16_d128_g4_b16",  "singe_paged_decode_bf16_d128_g8_b16",
-    "singe_paged_decode_bf16_d128_g16_b16", "singe_paged_decode_bf16_d128_g1_any",
-    "singe_paged_decode_bf16_d128_g2_any",  "singe_paged_decode_bf16_d128_g4_any",
-    "singe_paged_decode_bf16_d128_g8_any",  "singe_paged_decode_bf16_d128_g16_any",
+    "singe_paged_decode_bf16_d128_p1_b16", "singe_paged_decode_bf16_d128_p2_b16",
+    "singe_paged_decode_bf16_d128_p4_b16", "singe_paged_decode_bf16_d128_p1_any",
+    "singe_paged_decode_bf16_d128_p2_any", "singe_paged_decode_bf16_d128_p4_any",
     "singe_paged_decode_combine_bf16",
 };
 
@@ -80,6 +78,21 @@ int32_t fail(int32_t status, const char* name, uint64_t minimum, uint64_t actual
 }
 
 int32_t fail_hip(hipError_t error, const char* what) { return fail(-static_cast<int32_t>(error), what); }
+
+unsigned compute_units() {
+    static unsigned cached[kMaxDevices] = {};
+    const HipRuntime* hip = hip_runtime();
+    int device = 0;
+    if (hip == nullptr || hip->hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return 256;
+    if (cached[device] == 0) {
+        int count = 0;
+        constexpr int kMultiprocessorCount = 63;  // hipDeviceAttributeMultiprocessorCount
+        if (hip->hipDeviceGetAttribute(&count, kMultiprocessorCount, device) != hipSuccess || count < 1 || count > 4096)
+            count = 256;
+        cached[device] = static_cast<unsigned>(count);
+    }
+    return cached[device];
+}
 
 int32_t kernel_function(KernelId kernel, hipFunction_t* function) {
     const HipRuntime* hip = hip_runtime();

@@ -9,8 +9,8 @@ namespace singe_hip {
 
 // Kernels of the code object, in the order of kKernelNames.
 enum KernelId : int {
-    kDecodeG1B16 = 0, kDecodeG2B16, kDecodeG4B16, kDecodeG8B16, kDecodeG16B16,
-    kDecodeG1Any, kDecodeG2Any, kDecodeG4Any, kDecodeG8Any, kDecodeG16Any,
+    kDecodeP1B16 = 0, kDecodeP2B16, kDecodeP4B16,
+    kDecodeP1Any, kDecodeP2Any, kDecodeP4Any,
     kDecodeCombine,
     kKernelCount
 };
@@ -25,15 +25,18 @@ int32_t fail_hip(hipError_t error, const char* what);
 // Returns 0 and sets *function, or a status.
 int32_t kernel_function(KernelId kernel, hipFunction_t* function);
 
+// Compute units of the current device (256 when the runtime does not say).
+unsigned compute_units();
+
 // hipModuleLaunchKernel of a kernel that takes one argument block by value.
 template <class Args>
 int32_t launch(KernelId kernel, unsigned grid_x, unsigned grid_y, unsigned grid_z, unsigned threads,
-               hipStream_t stream, Args& args) {
+               hipStream_t stream, Args& args, unsigned shared_bytes = 0) {
     hipFunction_t function = nullptr;
     if (int32_t status = kernel_function(kernel, &function)) return status;
     void* params[] = {&args};
-    hipError_t error = hip_runtime()->hipModuleLaunchKernel(function, grid_x, grid_y, grid_z, threads, 1, 1, 0,
-                                                            stream, params, nullptr);
+    hipError_t error = hip_runtime()->hipModuleLaunchKernel(function, grid_x, grid_y, grid_z, threads, 1, 1,
+                                                            shared_bytes, stream, params, nullptr);
     return error == hipSuccess ? 0 : fail_hip(error, kKernelNames[kernel]);
 }
 

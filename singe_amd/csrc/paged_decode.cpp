@@ -13,41 +13,51 @@ using namespace singe_hip;
 
 namespace {
 
-std::atomic<uint32_t> g_keys_per_split{0};
+std::atomic<uint32_t> g_forced_workers{0};
 
 constexpr size_t kHeadDim = 128;
+constexpr unsigned kWavesPerWorkgroup = 8;
 
-uint32_t round_up_32(uint64_t value) { return static_cast<uint32_t>((value + 31) / 32 * 32); }
-
-// Keys per split: about 4096 work units when every sequence is at full reach, so the ~2048 resident
-// waves of the chip see two rounds of equal-sized units; never below 128 keys (64 KiB of KV per unit,
-// so the 1 KiB partial row stays in the noise) and never above 4096.
-uint32_t choose_keys_per_split(const SingePagedKvDecodeAttentionConfig& c) {
-    uint32_t forced = g_keys_per_split.load(std::memory_order_relaxed);
-    if (forced != 0) return round_up_32(forced);
-    uint64_t reach = static_cast<uint64_t>(c.block_table_batch_stride) * c.block_size;
-    uint64_t keys = reach * c.batch * c.kv_heads / 4096;
-    if (keys < 128) keys = 128;
-    if (keys > 4096) keys = 4096;
-    return round_up_32(keys);
-}
-
-struct Scratch {
-    uint32_t keys_per_split;
-    uint32_t splits;
-    size_t lse_offset;  // bytes, 256-aligned
-    size_t bytes;
+// How the flat list of 32-key tiles is shared out (see paged_decode.hip).
+struct Plan {
+    uint32_t head_groups;     // waves per kv head: ceil(group / 8)
+    uint32_t heads_per_wave;  // min(group, 8)
+    uint32_t pairs;           // 1, 2 or 4 pairs of query heads per wave
+    uint32_t work;            // kv_heads * head_groups
+    uint32_t work_per_wg;     // min(work, 8)
+    uint32_t workers_per_wg;  // 8 / work_per_wg
+    uint32_t workers;         // ranges per (kv head, head group)
+    uint32_t grid_x, grid_y;
+    size_t lse_offset, out_offset, bytes;  // scratch layout, 256-byte aligned regions
 };
 
-Scratch scratch_layout(const SingePagedKvDecodeAttentionConfig& c) {
-    Scratch s;
-    s.keys_per_split = choose_keys_per_split(c);
-    uint64_t reach = static_cast<uint64_t>(c.block_table_batch_stride) * c.block_size;
-    s.splits = static_cast<uint32_t>((reach + s.keys_per_split - 1) / s.keys_per_split);
-    size_t rows = c.batch * c.heads * static_cast<size_t>(s.splits);
-    s.lse_offset = (rows * c.head_dim * sizeof(float) + 255) / 256 * 256;
-    s.bytes = s.lse_offset + (rows * sizeof(float) + 255) / 256 * 256;
-    return s;
+size_t align256(size_t bytes) { return (bytes + 255) / 256 * 256; }
+
+// One workgroup of eight waves per compute unit, so every wave of the chip gets one equal range and
+// the launch finishes in a single round.
+Plan make_plan(const SingePagedKvDecodeAttentionConfig& c) {
+    Plan p;
+    const size_t group = c.heads / c.kv_heads;
+    p.head_groups = static_cast<uint32_t>((group + 7) / 8);
+    p.heads_per_wave = static_cast<uint32_t>(group < 8 ? group : 8);
+    p.pairs = p.heads_per_wave <= 2 ? 1 : p.heads_per_wave <= 4 ? 2 : 4;
+    p.work = static_cast<uint32_t>(c.kv_heads) * p.head_groups;
+    p.work_per_wg = p.work < kWavesPerWorkgroup ? p.work : kWavesPerWorkgroup;
+    p.workers_per_wg = kWavesPerWorkgroup / p.work_per_wg;
+    p.grid_y = (p.work + p.work_per_wg - 1) / p.work_per_wg;
+    uint32_t forced = g_forced_workers.load(std::memory_order_relaxed);
+    if (forced != 0) {
+        p.grid_x = (forced + p.workers_per_wg - 1) / p.workers_per_wg;
+    } else {
+        p.grid_x = compute_units() / p.grid_y;
+        if (p.grid_x == 0) p.grid_x = 1;
+    }
+    p.workers = p.grid_x * p.workers_per_wg;
+    const size_t rows = static_cast<size_t>(p.work) * (p.workers + c.batch) * p.heads_per_wave;
+    p.lse_offset = align256((c.batch + 3) * sizeof(uint32_t));
+    p.out_offset = p.lse_offset + align256(rows * sizeof(float));
+    p.bytes = p.out_offset + align256(rows * kHeadDim * sizeof(float));
+    return p;
 }
 
 int32_t validate_config(const SingePagedKvDecodeAttentionConfig& c) {
@@ -66,11 +76,11 @@ int32_t validate_config(const SingePagedKvDecodeAttentionConfig& c) {
 
 extern "C" {
 
-void singe_hip_set_decode_keys_per_split(uint32_t keys) { g_keys_per_split.store(keys, std::memory_order_relaxed); }
+void singe_hip_set_decode_workers(uint32_t workers) { g_forced_workers.store(workers, std::memory_order_relaxed); }
 
-uint32_t singe_hip_decode_keys_per_split(const SingePagedKvDecodeAttentionConfig* config) {
+uint32_t singe_hip_decode_workers(const SingePagedKvDecodeAttentionConfig* config) {
     if (config == nullptr || validate_config(*config) != 0) return 0;
-    return choose_keys_per_split(*config);
+    return make_plan(*config).workers;
 }
 
 int32_t singe_hip_paged_kv_decode_attention_config_validate(const SingePagedKvDecodeAttentionConfig* config) {
@@ -82,7 +92,7 @@ size_t singe_hip_paged_kv_decode_attention_workspace_bytes(const SingePagedKvDec
     if (config == nullptr || validate_config(*config) != 0) return 0;
     size_t rows = 0, elements = 0;
     if (!checked_mul(config->batch, config->heads, &rows) || !checked_mul(rows, config->head_dim, &elements)) return 0;
-    return scratch_layout(*config).bytes;
+    return make_plan(*config).bytes;
 }
 
 int32_t singe_hip_paged_kv_decode_attention_bf16(
@@ -129,16 +139,14 @@ int32_t singe_hip_paged_kv_decode_attention_phases_bf16(
     // What the gfx950 kernels take (the reference's cuTile kernels take head_dim 4..64 only and return
     // UnsupportedWidth otherwise: singe-kernel/src/cuda/cutile/attention/paged.rs:799-810).
     if (c.head_dim != kHeadDim) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, "paged_kv_decode_attention_bf16", c.head_dim, 0);
-    const size_t group = c.heads / c.kv_heads;
-    if (group > 16) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "more than 16 query heads per kv head");
     uint64_t reach = static_cast<uint64_t>(c.block_table_batch_stride) * c.block_size;
     if (!fits_i32(reach)) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "block_table_batch_stride * block_size");
 
-    const Scratch scratch = scratch_layout(c);
+    const Plan plan = make_plan(c);
     if (workspace == nullptr) return fail(SINGE_HIP_NULL_POINTER, "workspace");
-    if (workspace_bytes < scratch.bytes) return fail(SINGE_HIP_LENGTH_TOO_SHORT, "workspace", scratch.bytes, workspace_bytes);
-    if (scratch.splits > 65535 || c.kv_heads > 65535 || c.batch > 65535)
-        return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "grid extent above 65535");
+    if (workspace_bytes < plan.bytes) return fail(SINGE_HIP_LENGTH_TOO_SHORT, "workspace", plan.bytes, workspace_bytes);
+    if (c.batch > 16000) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "more than 16000 sequences per call");
+    unsigned char* scratch = static_cast<unsigned char*>(workspace);
 
     DecodeArgs args;
     args.query = query;
@@ -146,8 +154,10 @@ int32_t singe_hip_paged_kv_decode_attention_phases_bf16(
     args.value_cache = value_cache;
     args.actual_seq_lens = actual_seq_lens;
     args.block_table = block_table;
-    args.partial_out = static_cast<float*>(workspace);
-    args.partial_lse = reinterpret_cast<float*>(static_cast<unsigned char*>(workspace) + scratch.lse_offset);
+    args.meta = reinterpret_cast<uint32_t*>(scratch);
+    args.partial_lse = reinterpret_cast<float*>(scratch + plan.lse_offset);
+    args.partial_out = reinterpret_cast<float*>(scratch + plan.out_offset);
+    args.batch = static_cast<uint32_t>(c.batch);
     args.heads = static_cast<uint32_t>(c.heads);
     args.kv_heads = static_cast<uint32_t>(c.kv_heads);
     args.block_size = static_cast<uint32_t>(c.block_size);
@@ -156,18 +166,19 @@ int32_t singe_hip_paged_kv_decode_attention_phases_bf16(
         if ((static_cast<size_t>(1) << shift) == c.block_size) args.block_shift = shift;
     args.physical_blocks = static_cast<uint32_t>(c.physical_blocks);
     args.block_table_batch_stride = static_cast<uint32_t>(c.block_table_batch_stride);
-    args.splits = scratch.splits;
-    args.keys_per_split = scratch.keys_per_split;
+    args.workers = plan.workers;
+    args.workers_per_wg = plan.workers_per_wg;
+    args.work_per_wg = plan.work_per_wg;
+    args.head_groups = plan.head_groups;
+    args.heads_per_wave = plan.heads_per_wave;
     args.scale_log2e = c.scale * 1.4426950408889634074f;
 
-    int padded = 1;
-    while (static_cast<size_t>(padded) < group) padded *= 2;
-    int column = padded == 1 ? 0 : padded == 2 ? 1 : padded == 4 ? 2 : padded == 8 ? 3 : 4;
+    const int column = plan.pairs == 1 ? 0 : plan.pairs == 2 ? 1 : 2;
     const bool aligned = c.block_size % 16 == 0;
-    KernelId kernel = static_cast<KernelId>((aligned ? kDecodeG1B16 : kDecodeG1Any) + column);
+    KernelId kernel = static_cast<KernelId>((aligned ? kDecodeP1B16 : kDecodeP1Any) + column);
     if (phases & SINGE_HIP_DECODE_SPLIT)
-        if (int32_t status = launch(kernel, scratch.splits, static_cast<unsigned>(c.kv_heads),
-                                    static_cast<unsigned>(c.batch), 64, stream, args))
+        if (int32_t status = launch(kernel, plan.grid_x, plan.grid_y, 1, 64 * kWavesPerWorkgroup, stream, args,
+                                    static_cast<unsigned>((c.batch + 1) * sizeof(uint32_t))))
             return status;
     if (!(phases & SINGE_HIP_DECODE_REDUCE)) return 0;
 
@@ -175,12 +186,13 @@ int32_t singe_hip_paged_kv_decode_attention_phases_bf16(
     combine.out = out;
     combine.partial_out = args.partial_out;
     combine.partial_lse = args.partial_lse;
-    combine.actual_seq_lens = actual_seq_lens;
+    combine.meta = args.meta;
+    combine.batch = args.batch;
     combine.heads = args.heads;
-    combine.dim = static_cast<uint32_t>(c.head_dim);
-    combine.splits = scratch.splits;
-    combine.keys_per_split = scratch.keys_per_split;
-    combine.reach = static_cast<uint32_t>(reach);
+    combine.kv_heads = args.kv_heads;
+    combine.workers = plan.workers;
+    combine.head_groups = plan.head_groups;
+    combine.heads_per_wave = plan.heads_per_wave;
     return launch(kDecodeCombine, static_cast<unsigned>(c.batch * c.heads), 1, 1, 128, stream, combine);
 }
 

@@ -2,43 +2,52 @@
 // (the GPU counterpart of singe-kernel/src/cpu/attention.rs:1172-1246, replacing the cuTile kernels
 // of singe-kernel/src/cuda/cutile/kernel/attention/local.rs:9349-...).
 //
-// Layouts (fixed by the reference API): query/out [batch, heads, dim]; caches
-// [blocks, block_size, kv_heads, dim]; block_table [batch, stride] u32; actual_seq_lens [batch] i32.
+// Layouts (fixed by the reference API): query/out [batch, heads, 128]; caches
+// [blocks, block_size, kv_heads, 128]; block_table [batch, stride] u32; actual_seq_lens [batch] i32.
 //
-// Decode reads every KV byte once and does ~4 flop per byte, so it is bound by HBM bandwidth.  The
-// work unit is one wave64 over (sequence, kv head, chunk of keys): the query heads that share the kv
-// head ride along as MFMA columns, so a key row is fetched once for the whole group.
+// Decode reads every KV byte once and does a few flop per byte, so it is bound by HBM bandwidth and,
+// at these sizes (tens of microseconds), by how evenly and how early the chip is filled.
 //
-//   scores   S^T[token, head] = K[token, :] . Q[head, :] on v_mfma_f32_16x16x32_bf16 (fp32 accum);
-//            the group's heads are repeated across the 16 MFMA columns so every lane ends up with the
-//            scores of "its" head for four consecutive tokens,
-//   softmax  online, base two, per lane group of 16 (four independent streams per wave, merged once
-//            at the end), so the loop needs no cross-lane reduction,
-//   values   V rows are loaded as whole 256-byte rows (16 lanes x 16 B) and folded on the VALU with
-//            the probabilities broadcast inside quads (DPP) or groups of 8/16 (ds_swizzle).
+// Work split.  The keys of all sequences form one flat list of 32-key tiles (per-sequence tile counts,
+// prefix-summed in LDS by every workgroup).  The list is cut into `workers` equal ranges; a wave is
+// one worker for one kv head, so every wave does the same amount of work in a single round and the
+// waves of a workgroup walk the same cache blocks for neighbouring kv heads at the same time (one
+// 32 KiB block is fetched by one CU in one go).  A range that crosses a sequence boundary yields one
+// partial row per sequence; partial row of (worker v, sequence b) lives in scratch slot v + b, which is
+// unique because both grow along the list.  singe_paged_decode_combine folds a sequence's slots as
+// splitk_reduce_f32 does (cpu/attention.rs:2157-2193).
 //
-// Each chunk writes a normalised partial row and its natural-log LSE into caller-supplied scratch laid
-// out [batch, heads, splits, dim] / [batch, heads, splits], the layout of the reference's split-KV
-// scratch (singe-kernel/src/cuda/attention/mod.rs:2456-2539); singe_paged_decode_combine folds them
-// as splitk_reduce_f32 does (cpu/attention.rs:2157-2193).
+// Inner loop, per 32-key tile, all on the matrix cores:
+//   scores   S^T[key, head] = K[key, :] . Q[head, :]  (v_mfma_f32_16x16x32_bf16, fp32 accumulate).  Two
+//            query heads share one MFMA, each repeated over 8 of the 16 columns.
+//   softmax  online, base two; the tile maximum is shared by the wave (two v_permlane swaps), the
+//            running sum stays per lane until the row is flushed.
+//   values   V rows are loaded as whole 256-byte rows (16 lanes x 16 B, the coalesced layout) and used
+//            as the MFMA A operand exactly as loaded: A[chunk t][(g, e)] = V[key 4g + i][8t + e].
+//            The B operand is the probability of (head, key 4g + i) placed at position e of column
+//            (head, e), zero elsewhere, so C[t][(head, e)] accumulates O[head][8t + e].  That spends
+//            7/8 of the MFMA's multiplies on zeros, which is free here, and needs no transpose of V,
+//            no bf16 unpacking and no cross-lane traffic.  Probabilities are rounded to bf16 for this
+//            product and summed unrounded, as the reference's tensor-core kernel does
+//            (singe/src/backend/cuda/kernel_plan/source/tensor_core.rs:162-183).
 #include "common.hip.h"
 #include "kernel_args.h"
 
 namespace {
 
 constexpr int kDim = 128;
-constexpr int kTile = 32;  // keys folded per loop step: two 16-key MFMA tiles
+constexpr int kTile = 32;
 
 struct KeyTile {
-    uint4 k[2][4];  // [16-key tile][32-wide dim chunk]: lane (g, t) holds key t, dims 32g + 8c .. +8
-    uint4 v[2][4];  // [16-key tile][row]: lane (g, t) holds key 4g + row, dims 8t .. 8t + 8
-    unsigned int live;  // bit (tile * 4 + row): key tile*16 + 4g + row takes part in the softmax
+    uint4 k[2][4];      // [16-key half][32-wide dim chunk c]: lane (g, t) holds key t, dims 32g + 8c .. +8
+    uint4 v[2][4];      // [16-key half][i]: lane (g, t) holds key 4g + i, dims 8t .. 8t + 8
+    unsigned int live;  // bit (half * 4 + i): key half*16 + 4g + i takes part in the softmax
 };
 
-// Element offset of (block, token-in-block, kv_head, 0) in a [blocks, block_size, kv_heads, 128] cache.
-SINGE_DEVICE size_t cache_row(unsigned int block, unsigned int token, unsigned int block_size,
+// Element offset of (block, slot, kv_head, 0) in a [blocks, block_size, kv_heads, 128] cache.
+SINGE_DEVICE size_t cache_row(unsigned int block, unsigned int slot, unsigned int block_size,
                               unsigned int kv_heads, unsigned int kv_head) {
-    return ((static_cast<size_t>(block) * block_size + token) * kv_heads + kv_head) * kDim;
+    return ((static_cast<size_t>(block) * block_size + slot) * kv_heads + kv_head) * kDim;
 }
 
 // Splits a key index into (table entry, slot in block).  Power-of-two block sizes take the shift.
@@ -52,44 +61,52 @@ SINGE_DEVICE void split_key(const DecodeArgs& a, unsigned int key, unsigned int&
     }
 }
 
-// Loads the 32 keys from `first` (a multiple of 32) of a chunk that ends at `end` > 0.  Keys at or past
-// `end`, and keys whose table entry is not a cache block, read an in-range row instead and are marked
-// dead, so nothing is read out of bounds and no dead row can carry a NaN into the weighted sum.
+// Loads the 32 keys from `first` (a multiple of 32) of a sequence of `end` > first keys.  Keys at or
+// past `end`, and keys whose table entry is not a cache block, read an in-range row instead and are
+// marked dead, so nothing is read out of bounds and no dead row can carry a NaN into the sums.
 template <bool ALIGNED16>
 SINGE_DEVICE void load_tile(KeyTile& tile, const DecodeArgs& a, const unsigned int* table_row,
                             unsigned int first, unsigned int end, unsigned int kv_head, unsigned int g,
                             unsigned int t) {
     tile.live = 0;
+    if constexpr (ALIGNED16) {
+        // block_size is a multiple of 16, so the 16 keys of a half share one table entry; a half
+        // wholly past the end re-reads the 16-key span that holds the last key.
+        unsigned int last_entry, last_slot, entry[2], slot0[2], block[2];
+        split_key(a, end - 1, last_entry, last_slot);
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
-        const unsigned int base = first + half * 16;
-        if constexpr (ALIGNED16) {
-            // block_size is a multiple of 16, so the 16 keys from `base` share one table entry; a
-            // half tile wholly past the end re-reads the 16-key span that holds the last key.
-            const unsigned int span = base < end ? base : ((end - 1) & ~15u);
-            unsigned int entry, slot0, last_entry, last_slot;
-            split_key(a, span, entry, slot0);
-            split_key(a, end - 1, last_entry, last_slot);
-            unsigned int block = table_row[entry];
-            const bool known = block < a.physical_blocks;
-            block = known ? block : 0;
+        for (int half = 0; half < 2; ++half) {
+            const unsigned int base = first + half * 16;
+            split_key(a, base < end ? base : ((end - 1) & ~15u), entry[half], slot0[half]);
+        }
+#pragma unroll
+        for (int half = 0; half < 2; ++half) block[half] = table_row[entry[half]];
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const unsigned int base = first + half * 16;
+            const bool known = block[half] < a.physical_blocks;
+            const unsigned int safe = known ? block[half] : 0;
             {
                 const bool inside = base + t < end;
-                const uint16_t* kp =
-                    a.key_cache + cache_row(block, inside ? slot0 + t : last_slot, a.block_size, a.kv_heads, kv_head) + 32 * g;
+                const uint16_t* kp = a.key_cache +
+                    cache_row(safe, inside ? slot0[half] + t : last_slot, a.block_size, a.kv_heads, kv_head) + 32 * g;
 #pragma unroll
                 for (int c = 0; c < 4; ++c) tile.k[half][c] = *reinterpret_cast<const uint4*>(kp + 8 * c);
             }
 #pragma unroll
-            for (int row = 0; row < 4; ++row) {
-                const bool inside = base + 4 * g + row < end;
-                const uint16_t* vp =
-                    a.value_cache + cache_row(block, inside ? slot0 + 4 * g + row : last_slot, a.block_size, a.kv_heads, kv_head) + 8 * t;
-                tile.v[half][row] = *reinterpret_cast<const uint4*>(vp);
-                if (inside && known) tile.live |= 1u << (half * 4 + row);
+            for (int i = 0; i < 4; ++i) {
+                const bool inside = base + 4 * g + i < end;
+                const uint16_t* vp = a.value_cache +
+                    cache_row(safe, inside ? slot0[half] + 4 * g + i : last_slot, a.block_size, a.kv_heads, kv_head) + 8 * t;
+                tile.v[half][i] = *reinterpret_cast<const uint4*>(vp);
+                if (inside && known) tile.live |= 1u << (half * 4 + i);
             }
-        } else {
-            // Any block size: every lane looks up the table entry of its own key.
+        }
+    } else {
+        // Any block size: every lane looks up the table entry of its own key.
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const unsigned int base = first + half * 16;
             {
                 const unsigned int key = base + t < end ? base + t : end - 1;
                 unsigned int entry, slot;
@@ -101,8 +118,8 @@ SINGE_DEVICE void load_tile(KeyTile& tile, const DecodeArgs& a, const unsigned i
                 for (int c = 0; c < 4; ++c) tile.k[half][c] = *reinterpret_cast<const uint4*>(kp + 8 * c);
             }
 #pragma unroll
-            for (int row = 0; row < 4; ++row) {
-                const unsigned int wanted = base + 4 * g + row;
+            for (int i = 0; i < 4; ++i) {
+                const unsigned int wanted = base + 4 * g + i;
                 const bool inside = wanted < end;
                 unsigned int entry, slot;
                 split_key(a, inside ? wanted : end - 1, entry, slot);
@@ -110,192 +127,295 @@ SINGE_DEVICE void load_tile(KeyTile& tile, const DecodeArgs& a, const unsigned i
                 const bool known = block < a.physical_blocks;
                 block = known ? block : 0;
                 const uint16_t* vp = a.value_cache + cache_row(block, slot, a.block_size, a.kv_heads, kv_head) + 8 * t;
-                tile.v[half][row] = *reinterpret_cast<const uint4*>(vp);
-                if (inside && known) tile.live |= 1u << (half * 4 + row);
+                tile.v[half][i] = *reinterpret_cast<const uint4*>(vp);
+                if (inside && known) tile.live |= 1u << (half * 4 + i);
             }
         }
     }
 }
 
-// GROUPS = query heads per kv head rounded up to a power of two (1, 2, 4, 8, 16).
-template <int GROUPS, bool ALIGNED16>
-SINGE_DEVICE void paged_decode_body(const DecodeArgs& a) {
-    const unsigned int lane = threadIdx.x;
+// v_permlane16_swap / v_permlane32_swap of a value with a copy of itself: `kept` keeps its even rows
+// (its low half for 32) and takes the neighbour's, `taken` the other way round, so kept (op) taken
+// combines a lane with its partner 16 (32) lanes away.  Written as inline assembly because the
+// compiler's builtin returns the first result twice; the s_nop covers the VALU-write hazard the
+// compiler would otherwise pad.
+template <int ROWS>
+SINGE_DEVICE void swap_with_self(float value, float& kept, float& taken) {
+    kept = value;
+    taken = value;
+    if constexpr (ROWS == 16)
+        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(kept), "+v"(taken));
+    else
+        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(kept), "+v"(taken));
+}
+
+// max / sum over the four 16-lane groups of a wave: lanes l, l^16, l^32, l^48 end up equal.
+SINGE_DEVICE float across_groups_max(float value) {
+    float a, b;
+    swap_with_self<16>(value, a, b);
+    swap_with_self<32>(fmaxf(a, b), a, b);
+    return fmaxf(a, b);
+}
+
+SINGE_DEVICE float across_groups_sum(float value) {
+    float a, b;
+    swap_with_self<16>(value, a, b);
+    swap_with_self<32>(a + b, a, b);
+    return a + b;
+}
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+
+// bf16(value) in both halves of a dword (one v_cvt_pk_bf16_f32, round to nearest even).
+SINGE_DEVICE unsigned int bf16_twice(float value) {
+    f32x2_t both = {value, value};
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(both, bf16x2_t));
+}
+
+// Per-wave softmax state of one pair of query heads.
+struct PairState {
+    f32x4_t acc;        // C[t][(head, e)]: lane (g, n) holds chunks t = 4g .. 4g+3 of column n
+    float running_max;  // log2 units, equal in all lanes that hold the same head
+    float running_sum;  // of this lane's keys only
+};
+
+// PAIRS = pairs of query heads a wave carries (1, 2 or 4: up to 8 query heads per kv head).
+template <int PAIRS, bool ALIGNED16>
+SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
+    const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const unsigned int g = lane >> 4, t = lane & 15;
-    const unsigned int split = blockIdx.x, kv_head = blockIdx.y, batch = blockIdx.z;
-    const unsigned int group = a.heads / a.kv_heads;
-
     const unsigned int reach = a.block_table_batch_stride * a.block_size;
-    int raw_len = a.actual_seq_lens[batch];
-    const unsigned int seq_len = raw_len < 0 ? 0u : (static_cast<unsigned int>(raw_len) < reach ? static_cast<unsigned int>(raw_len) : reach);
-    const unsigned int first = split * a.keys_per_split;
-    if (first >= seq_len) return;
-    const unsigned int end = seq_len < first + a.keys_per_split ? seq_len : first + a.keys_per_split;
-    const unsigned int* table_row = a.block_table + static_cast<size_t>(batch) * a.block_table_batch_stride;
 
-    // Query rows as the MFMA B operand: column j of the 16 carries head j % GROUPS.
-    const unsigned int my_head = t % GROUPS;
-    bf16x8_t q[4];
-    {
-        const bool real = my_head < group;
-        const uint16_t* qp = a.query + (static_cast<size_t>(batch) * a.heads + kv_head * group + (real ? my_head : 0)) * kDim + 32 * g;
+    // Tiles per sequence, prefix-summed: prefix[b] = tiles of sequences before b.
+    if (wave == 0) {
+        unsigned int carry = 0;
+        for (unsigned int base = 0; base < a.batch; base += 64) {
+            unsigned int tiles = 0;
+            if (base + lane < a.batch) {
+                const int raw = a.actual_seq_lens[base + lane];
+                const unsigned int len = raw < 0 ? 0u : (static_cast<unsigned int>(raw) < reach ? static_cast<unsigned int>(raw) : reach);
+                tiles = (len + kTile - 1) / kTile;
+            }
+            unsigned int scan = tiles;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            uint4 bits = *reinterpret_cast<const uint4*>(qp + 8 * c);
-            if (!real) bits = make_uint4(0, 0, 0, 0);
-            q[c] = __builtin_bit_cast(bf16x8_t, bits);
+            for (int step = 1; step < 64; step *= 2) {
+                const unsigned int below = __shfl_up(scan, step, 64);
+                if (lane >= static_cast<unsigned int>(step)) scan += below;
+            }
+            if (base + lane < a.batch) prefix[base + lane + 1] = carry + scan;
+            carry += __shfl(scan, 63, 64);
+        }
+        if (lane == 0) prefix[0] = 0;
+    }
+    __syncthreads();
+    const unsigned int total = prefix[a.batch];
+    const unsigned int share = total == 0 ? 1u : (total + a.workers - 1) / a.workers;
+    if (blockIdx.x == 0 && blockIdx.y == 0) {
+        // What the combine kernel needs to find a sequence's slots.
+        for (unsigned int i = threadIdx.x; i <= a.batch; i += blockDim.x) a.meta[2 + i] = prefix[i];
+        if (threadIdx.x == 0) {
+            a.meta[0] = share;
+            a.meta[1] = total;
         }
     }
 
-    float acc[GROUPS][8];
-#pragma unroll
-    for (int h = 0; h < GROUPS; ++h)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[h][e] = 0.0f;
-    float running_max = -INFINITY;  // of this lane's head, over this lane group's keys, in log2 units
-    float running_sum = 0.0f;
+    const unsigned int lanes_of_work = a.kv_heads * a.head_groups;
+    const unsigned int work = blockIdx.y * a.work_per_wg + wave % a.work_per_wg;
+    const unsigned int sub = wave / a.work_per_wg;
+    if (work >= lanes_of_work || sub >= a.workers_per_wg) return;
+    const unsigned int worker = blockIdx.x * a.workers_per_wg + sub;
+    const unsigned int range_first = worker * share;
+    if (worker >= a.workers || range_first >= total) return;
+    const unsigned int range_end = total < range_first + share ? total : range_first + share;
 
-    KeyTile current, next;
-    load_tile<ALIGNED16>(current, a, table_row, first, end, kv_head, g, t);
-    for (unsigned int at = first; at < end; at += kTile) {
-        const bool more = at + kTile < end;
-        if (more) load_tile<ALIGNED16>(next, a, table_row, at + kTile, end, kv_head, g, t);
+    const unsigned int group = a.heads / a.kv_heads;
+    const unsigned int kv_head = work / a.head_groups;
+    const unsigned int head_in_group = (work % a.head_groups) * 8;  // first query head of this wave inside its group
+    const unsigned int wave_heads = group - head_in_group < 8 ? group - head_in_group : 8;
+    const unsigned int slots = a.workers + a.batch;
 
-        f32x4_t s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-        for (int c = 0; c < 4; ++c) {
-            s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, current.k[0][c]), q[c], s0, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, current.k[1][c]), q[c], s1, 0, 0, 0);
+    // The sequence that holds tile range_first: the last b with prefix[b] <= range_first.
+    unsigned int seq = 0;
+    {
+        unsigned int low = 0, high = a.batch;  // prefix[low] <= range_first < prefix[high]
+        while (high - low > 1) {
+            const unsigned int mid = (low + high) / 2;
+            if (prefix[mid] <= range_first) low = mid; else high = mid;
         }
-        float p[8];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            p[r] = (current.live >> r) & 1u ? s0[r] * a.scale_log2e : -INFINITY;
-            p[4 + r] = (current.live >> (4 + r)) & 1u ? s1[r] * a.scale_log2e : -INFINITY;
-        }
-        float largest = running_max;
-#pragma unroll
-        for (int r = 0; r < 8; ++r) largest = fmaxf(largest, p[r]);
-        const float base = largest == -INFINITY ? 0.0f : largest;
-        const float rescale = fast_exp2(running_max - base);
-        float total = 0.0f;
-#pragma unroll
-        for (int r = 0; r < 8; ++r) {
-            p[r] = fast_exp2(p[r] - base);
-            total += p[r];
-        }
-        running_sum = running_sum * rescale + total;
-        const bool moved = largest > running_max;
-        running_max = largest;
-        const bool any_moved = __any(moved);
+        seq = low;
+    }
 
-        static_for<GROUPS>([&](auto head) {
-            constexpr int h = decltype(head)::value;
-            if (any_moved) {
-                const float factor = group_broadcast<GROUPS, h>(rescale);
+    // One-hot placement of a probability: column n = lane % 16 carries head n / 8 at position n % 8.
+    unsigned int place[4];
 #pragma unroll
-                for (int e = 0; e < 8; ++e) acc[h][e] *= factor;
+    for (int r = 0; r < 4; ++r) place[r] = (t & 7) / 2 == static_cast<unsigned int>(r) ? ((t & 1) ? 0xffff0000u : 0x0000ffffu) : 0u;
+
+    bf16x8_t q[PAIRS][4];
+    PairState state[PAIRS];
+    auto load_query = [&](unsigned int b) {
+#pragma unroll
+        for (int hp = 0; hp < PAIRS; ++hp) {
+            const unsigned int local = 2 * hp + (t >> 3);
+            const bool real = local < wave_heads;
+            const uint16_t* qp = a.query + (static_cast<size_t>(b) * a.heads + kv_head * group + head_in_group + (real ? local : 0)) * kDim + 32 * g;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                uint4 bits = *reinterpret_cast<const uint4*>(qp + 8 * c);
+                if (!real) bits = make_uint4(0, 0, 0, 0);
+                q[hp][c] = __builtin_bit_cast(bf16x8_t, bits);
             }
+            state[hp].acc = {0.0f, 0.0f, 0.0f, 0.0f};
+            state[hp].running_max = -INFINITY;
+            state[hp].running_sum = 0.0f;
+        }
+    };
+
+    auto fold = [&](const KeyTile& tile) {
+#pragma unroll
+        for (int hp = 0; hp < PAIRS; ++hp) {
+            f32x4_t s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, tile.k[0][c]), q[hp][c], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, tile.k[1][c]), q[hp][c], s1, 0, 0, 0);
+            }
+            float p[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                p[i] = (tile.live >> i) & 1u ? s0[i] * a.scale_log2e : -INFINITY;
+                p[4 + i] = (tile.live >> (4 + i)) & 1u ? s1[i] * a.scale_log2e : -INFINITY;
+            }
+            float largest = fmaxf(fmaxf(fmaxf(p[0], p[1]), fmaxf(p[2], p[3])), fmaxf(fmaxf(p[4], p[5]), fmaxf(p[6], p[7])));
+            largest = fmaxf(across_groups_max(largest), state[hp].running_max);
+            const float base = largest == -INFINITY ? 0.0f : largest;
+            const float rescale = fast_exp2(state[hp].running_max - base);
+            float total = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                p[i] = fast_exp2(p[i] - base);
+                total += p[i];
+            }
+            state[hp].running_sum = state[hp].running_sum * rescale + total;
+            state[hp].running_max = largest;
+            f32x4_t acc = state[hp].acc;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[r] *= rescale;
 #pragma unroll
             for (int half = 0; half < 2; ++half)
 #pragma unroll
-                for (int row = 0; row < 4; ++row) {
-                    const float weight = group_broadcast<GROUPS, h>(p[half * 4 + row]);
-                    const uint4 bits = current.v[half][row];
-                    acc[h][0] = fmaf(weight, bf16_lo(bits.x), acc[h][0]);
-                    acc[h][1] = fmaf(weight, bf16_hi(bits.x), acc[h][1]);
-                    acc[h][2] = fmaf(weight, bf16_lo(bits.y), acc[h][2]);
-                    acc[h][3] = fmaf(weight, bf16_hi(bits.y), acc[h][3]);
-                    acc[h][4] = fmaf(weight, bf16_lo(bits.z), acc[h][4]);
-                    acc[h][5] = fmaf(weight, bf16_hi(bits.z), acc[h][5]);
-                    acc[h][6] = fmaf(weight, bf16_lo(bits.w), acc[h][6]);
-                    acc[h][7] = fmaf(weight, bf16_hi(bits.w), acc[h][7]);
+                for (int i = 0; i < 4; ++i) {
+                    const unsigned int both = bf16_twice(p[half * 4 + i]);
+                    const uint4 hot = make_uint4(both & place[0], both & place[1], both & place[2], both & place[3]);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, tile.v[half][i]),
+                                                                  __builtin_bit_cast(bf16x8_t, hot), acc, 0, 0, 0);
                 }
-        });
-        if (more) current = next;
-    }
+            state[hp].acc = acc;
+        }
+    };
 
-    // Merge the four lane groups' streams: lanes l, l^16, l^32, l^48 hold the same head.
-    float all_max = fmaxf(running_max, wave_xor(running_max, 16));
-    all_max = fmaxf(all_max, wave_xor(all_max, 32));
-    const float all_base = all_max == -INFINITY ? 0.0f : all_max;
-    const float weight = fast_exp2(running_max - all_base);
-    float all_sum = running_sum * weight;
-    all_sum += wave_xor(all_sum, 16);
-    all_sum += wave_xor(all_sum, 32);
-    const float inverse = all_sum > 0.0f ? 1.0f / all_sum : 0.0f;
-    const float lse = all_sum > 0.0f ? (all_max + fast_log2(all_sum)) * kLn2 : -INFINITY;
-
-    static_for<GROUPS>([&](auto head) {
-        constexpr int h = decltype(head)::value;
-        const float factor = group_broadcast<GROUPS, h>(weight);
-        const float norm = group_broadcast<GROUPS, h>(inverse);
+    // Writes the partial row of sequence b: O / sum per head, and the natural-log LSE.
+    auto flush = [&](unsigned int b) {
+        const size_t slot = static_cast<size_t>(work) * slots + worker + b;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            float value = acc[h][e] * factor;
-            value += wave_xor(value, 16);
-            value += wave_xor(value, 32);
-            acc[h][e] = value * norm;
+        for (int hp = 0; hp < PAIRS; ++hp) {
+            const float sum = across_groups_sum(state[hp].running_sum);
+            const float inverse = sum > 0.0f ? 1.0f / sum : 0.0f;
+            const unsigned int local = 2 * hp + (t >> 3);
+            if (local < wave_heads) {
+                float* row = a.partial_out + (slot * a.heads_per_wave + local) * kDim;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) row[8 * (4 * g + r) + (t & 7)] = state[hp].acc[r] * inverse;
+                if (g == 0 && (t & 7) == 0)
+                    a.partial_lse[slot * a.heads_per_wave + local] =
+                        sum > 0.0f ? (state[hp].running_max + fast_log2(sum)) * kLn2 : -INFINITY;
+            }
         }
-    });
+    };
 
-    // Lane group g stores heads g, g + 4, ...; 16 lanes x 32 B cover one 128-wide row.
-    static_for<GROUPS>([&](auto head) {
-        constexpr int h = decltype(head)::value;
-        if (h < group && (h & 3) == static_cast<int>(g)) {
-            const size_t row = (static_cast<size_t>(batch) * a.heads + kv_head * group + h) * a.splits + split;
-            float4* out = reinterpret_cast<float4*>(a.partial_out + row * kDim + 8 * t);
-            out[0] = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
-            out[1] = make_float4(acc[h][4], acc[h][5], acc[h][6], acc[h][7]);
+    // Walk the range tile by tile, prefetching the next tile while the current one is folded.
+    auto seq_len = [&](unsigned int b) {
+        const int raw = a.actual_seq_lens[b];
+        return raw < 0 ? 0u : (static_cast<unsigned int>(raw) < reach ? static_cast<unsigned int>(raw) : reach);
+    };
+    unsigned int at = range_first;  // flat tile index of the tile being folded
+    unsigned int len = seq_len(seq);
+    KeyTile ping, pong;
+    load_query(seq);
+    load_tile<ALIGNED16>(ping, a, a.block_table + static_cast<size_t>(seq) * a.block_table_batch_stride,
+                         (at - prefix[seq]) * kTile, len, kv_head, g, t);
+    auto advance = [&](KeyTile& current, KeyTile& upcoming) {
+        // Returns false when `current` was the last tile of the range.
+        const unsigned int next_at = at + 1;
+        const bool more = next_at < range_end;
+        unsigned int next_seq = seq, next_len = len;
+        if (more) {
+            while (prefix[next_seq + 1] <= next_at) ++next_seq;  // skips empty sequences
+            if (next_seq != seq) next_len = seq_len(next_seq);
+            load_tile<ALIGNED16>(upcoming, a, a.block_table + static_cast<size_t>(next_seq) * a.block_table_batch_stride,
+                                 (next_at - prefix[next_seq]) * kTile, next_len, kv_head, g, t);
         }
-    });
-    if (g == 0 && t < GROUPS && t < group) {
-        const size_t row = (static_cast<size_t>(batch) * a.heads + kv_head * group + t) * a.splits + split;
-        a.partial_lse[row] = lse;
+        fold(current);
+        if (!more || next_seq != seq) {
+            flush(seq);
+            if (more) load_query(next_seq);
+        }
+        at = next_at;
+        seq = next_seq;
+        len = next_len;
+        return more;
+    };
+    while (true) {
+        if (!advance(ping, pong)) break;
+        if (!advance(pong, ping)) break;
     }
 }
 
 }  // namespace
 
-#define SINGE_DECODE_KERNEL(GROUPS, ALIGNED, SUFFIX)                                                     \
-    extern "C" __global__ __launch_bounds__(64) void singe_paged_decode_bf16_d128_g##GROUPS##SUFFIX(      \
-        DecodeArgs args) {                                                                              \
-        paged_decode_body<GROUPS, ALIGNED>(args);                                                       \
+#define SINGE_DECODE_KERNEL(PAIRS, ALIGNED, SUFFIX)                                                       \
+    extern "C" __global__ __launch_bounds__(512) void singe_paged_decode_bf16_d128_p##PAIRS##SUFFIX(       \
+        DecodeArgs args) {                                                                               \
+        extern __shared__ unsigned int prefix[];                                                         \
+        paged_decode_body<PAIRS, ALIGNED>(args, prefix);                                                 \
     }
 
 SINGE_DECODE_KERNEL(1, true, _b16)
 SINGE_DECODE_KERNEL(2, true, _b16)
 SINGE_DECODE_KERNEL(4, true, _b16)
-SINGE_DECODE_KERNEL(8, true, _b16)
-SINGE_DECODE_KERNEL(16, true, _b16)
 SINGE_DECODE_KERNEL(1, false, _any)
 SINGE_DECODE_KERNEL(2, false, _any)
 SINGE_DECODE_KERNEL(4, false, _any)
-SINGE_DECODE_KERNEL(8, false, _any)
-SINGE_DECODE_KERNEL(16, false, _any)
 
-// Folds the per-split partial rows of one (batch, head) into the bf16 output:
+// Folds the partial rows of one (sequence, query head) into the bf16 output:
 // out = sum_s exp(lse_s - max) * partial_s / sum_s exp(lse_s - max)
-// (singe-kernel/src/cpu/attention.rs:2157-2193).  One thread per output element.
+// (singe-kernel/src/cpu/attention.rs:2157-2193).  One workgroup per row, one thread per dimension.
 extern "C" __global__ __launch_bounds__(128) void singe_paged_decode_combine_bf16(CombineArgs a) {
     const unsigned int row = blockIdx.x;  // batch * heads + head
-    const unsigned int batch = row / a.heads;
-    int raw_len = a.actual_seq_lens[batch];
-    const unsigned int seq_len = raw_len < 0 ? 0u : (static_cast<unsigned int>(raw_len) < a.reach ? static_cast<unsigned int>(raw_len) : a.reach);
-    const unsigned int used = (seq_len + a.keys_per_split - 1) / a.keys_per_split;
-    const float* lse = a.partial_lse + static_cast<size_t>(row) * a.splits;
-    float largest = -INFINITY;
-    for (unsigned int s = 0; s < used; ++s) largest = fmaxf(largest, lse[s]);
-    for (unsigned int d = threadIdx.x; d < a.dim; d += blockDim.x) {
-        float total = 0.0f, sum = 0.0f;
+    const unsigned int b = row / a.heads, head = row % a.heads;
+    const unsigned int group = a.heads / a.kv_heads;
+    const unsigned int kv_head = head / group, in_group = head % group;
+    const unsigned int work = kv_head * a.head_groups + in_group / 8, local = in_group % 8;
+    const unsigned int share = a.meta[0];
+    const unsigned int first_tile = a.meta[2 + b], end_tile = a.meta[3 + b];
+    const unsigned int d = threadIdx.x;
+    float result = 0.0f;  // a sequence with no keys keeps a zero row (cpu/attention.rs:1213-1215)
+    if (end_tile > first_tile) {
+        const unsigned int first_worker = first_tile / share, last_worker = (end_tile - 1) / share;
+        const size_t base = (static_cast<size_t>(work) * (a.workers + a.batch) + first_worker + b) * a.heads_per_wave + local;
+        const unsigned int count = last_worker - first_worker + 1;
+        float largest = -INFINITY;
+        for (unsigned int s = 0; s < count; ++s) largest = fmaxf(largest, a.partial_lse[base + static_cast<size_t>(s) * a.heads_per_wave]);
         if (largest != -INFINITY) {
-            for (unsigned int s = 0; s < used; ++s) {
-                const float weight = __expf(lse[s] - largest);
+            float total = 0.0f, sum = 0.0f;
+            for (unsigned int s = 0; s < count; ++s) {
+                const size_t at = base + static_cast<size_t>(s) * a.heads_per_wave;
+                const float weight = __expf(a.partial_lse[at] - largest);
                 total += weight;
-                sum = fmaf(weight, a.partial_out[(static_cast<size_t>(row) * a.splits + s) * a.dim + d], sum);
+                sum = fmaf(weight, a.partial_out[at * kDim + d], sum);
             }
+            result = total > 0.0f ? sum / total : 0.0f;
         }
-        // A sequence with no keys keeps a zero row (cpu/attention.rs:1213-1215).
-        a.out[static_cast<size_t>(row) * a.dim + d] = f32_to_bf16_bits(total > 0.0f ? sum / total : 0.0f);
     }
+    a.out[static_cast<size_t>(row) * kDim + d] = f32_to_bf16_bits(result);
 }

@@ -34,8 +34,8 @@ def compact(work):
     return kc, vc, table
 
 
-def run_gpu(work, keys_per_split=0):
-    A._native.lib().singe_hip_set_decode_keys_per_split(keys_per_split)
+def run_gpu(work, workers=0):
+    A._native.lib().singe_hip_set_decode_workers(workers)
     try:
         config = A.PagedKvDecodeAttentionConfig.contiguous(work.batch, work.heads, work.kv_heads, work.head_dim,
                                                            work.block_size, work.physical_blocks,
@@ -46,7 +46,7 @@ def run_gpu(work, keys_per_split=0):
         A.paged_kv_decode_attention_bf16(None, out, work.query, work.key_cache, work.value_cache, lens, table, config)
         torch.cuda.synchronize()
     finally:
-        A._native.lib().singe_hip_set_decode_keys_per_split(0)
+        A._native.lib().singe_hip_set_decode_workers(0)
     return out.float().cpu().numpy()
 
 
@@ -83,13 +83,13 @@ def test_decode_group_sizes(heads, kv_heads):
 
 
 @pytest.mark.parametrize("block_size", [1, 7, 16, 32, 48, 5])
-@pytest.mark.parametrize("keys_per_split", [0, 32, 96, 4096])
-def test_decode_block_sizes_and_splits(block_size, keys_per_split):
+@pytest.mark.parametrize("workers", [0, 1, 3, 50, 4096])
+def test_decode_block_sizes_and_splits(block_size, workers):
     lens = [200, 1, 333, 0, 97, 160, 31, 512]
     blocks = sum((l + block_size - 1) // block_size for l in lens) + 9
     work = synthetic.paged_decode_workload(batch=len(lens), heads=8, kv_heads=2, block_size=block_size,
                                            physical_blocks=blocks, seq_lens=lens, seed=7 + block_size)
-    assert_close(run_gpu(work, keys_per_split), run_oracle(work), f"block {block_size} split {keys_per_split}")
+    assert_close(run_gpu(work, workers), run_oracle(work), f"block {block_size} split {workers}")
 
 
 def test_decode_table_stride_wider_than_needed_and_poisoned_tail():
