@@ -69,5 +69,13 @@ SINGE_DEVICE unsigned int pack_bf16x2(float lo, float hi) {
     return static_cast<unsigned int>(f32_to_bf16_bits(lo)) | (static_cast<unsigned int>(f32_to_bf16_bits(hi)) << 16);
 }
 
+// 16-byte load of data that is read once: the non-temporal hint keeps it from displacing reusable
+// lines in the caches on its way through, which measurably raises streaming read bandwidth.
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+SINGE_DEVICE uint4 stream_load_16(const void* address) {
+    const u32x4_t bits = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(address));
+    return make_uint4(bits.x, bits.y, bits.z, bits.w);
+}
+
 SINGE_DEVICE float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 SINGE_DEVICE float fast_log2(float x) { return __builtin_amdgcn_logf(x); }

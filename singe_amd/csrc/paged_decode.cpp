@@ -145,7 +145,7 @@ int32_t singe_hip_paged_kv_decode_attention_phases_bf16(
     const Plan plan = make_plan(c);
     if (workspace == nullptr) return fail(SINGE_HIP_NULL_POINTER, "workspace");
     if (workspace_bytes < plan.bytes) return fail(SINGE_HIP_LENGTH_TOO_SHORT, "workspace", plan.bytes, workspace_bytes);
-    if (c.batch > 16000) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "more than 16000 sequences per call");
+    if (c.batch > 8000) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "more than 8000 sequences per call");
     unsigned char* scratch = static_cast<unsigned char*>(workspace);
 
     DecodeArgs args;
@@ -178,7 +178,7 @@ int32_t singe_hip_paged_kv_decode_attention_phases_bf16(
     KernelId kernel = static_cast<KernelId>((aligned ? kDecodeP1B16 : kDecodeP1Any) + column);
     if (phases & SINGE_HIP_DECODE_SPLIT)
         if (int32_t status = launch(kernel, plan.grid_x, plan.grid_y, 1, 64 * kWavesPerWorkgroup, stream, args,
-                                    static_cast<unsigned>((c.batch + 1) * sizeof(uint32_t))))
+                                    static_cast<unsigned>((2 * c.batch + 1) * sizeof(uint32_t))))
             return status;
     if (!(phases & SINGE_HIP_DECODE_REDUCE)) return 0;
 

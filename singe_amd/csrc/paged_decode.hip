@@ -39,7 +39,7 @@ constexpr int kDim = 128;
 constexpr int kTile = 32;
 
 struct KeyTile {
-    uint4 k[2][4];      // [16-key half][32-wide dim chunk c]: lane (g, t) holds key t, dims 32g + 8c .. +8
+    uint4 k[2][4];      // [16-key half][c]: lane (g, t) holds key t, dims 32c + 8g .. +8 (one load covers 64 B of each key)
     uint4 v[2][4];      // [16-key half][i]: lane (g, t) holds key 4g + i, dims 8t .. 8t + 8
     unsigned int live;  // bit (half * 4 + i): key half*16 + 4g + i takes part in the softmax
 };
@@ -89,16 +89,16 @@ SINGE_DEVICE void load_tile(KeyTile& tile, const DecodeArgs& a, const unsigned i
             {
                 const bool inside = base + t < end;
                 const uint16_t* kp = a.key_cache +
-                    cache_row(safe, inside ? slot0[half] + t : last_slot, a.block_size, a.kv_heads, kv_head) + 32 * g;
+                    cache_row(safe, inside ? slot0[half] + t : last_slot, a.block_size, a.kv_heads, kv_head) + 8 * g;
 #pragma unroll
-                for (int c = 0; c < 4; ++c) tile.k[half][c] = *reinterpret_cast<const uint4*>(kp + 8 * c);
+                for (int c = 0; c < 4; ++c) tile.k[half][c] = *reinterpret_cast<const uint4*>(kp + 32 * c);
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const bool inside = base + 4 * g + i < end;
                 const uint16_t* vp = a.value_cache +
                     cache_row(safe, inside ? slot0[half] + 4 * g + i : last_slot, a.block_size, a.kv_heads, kv_head) + 8 * t;
-                tile.v[half][i] = *reinterpret_cast<const uint4*>(vp);
+                tile.v[half][i] = stream_load_16(vp);
                 if (inside && known) tile.live |= 1u << (half * 4 + i);
             }
         }
@@ -113,9 +113,9 @@ SINGE_DEVICE void load_tile(KeyTile& tile, const DecodeArgs& a, const unsigned i
                 split_key(a, key, entry, slot);
                 unsigned int block = table_row[entry];
                 block = block < a.physical_blocks ? block : 0;
-                const uint16_t* kp = a.key_cache + cache_row(block, slot, a.block_size, a.kv_heads, kv_head) + 32 * g;
+                const uint16_t* kp = a.key_cache + cache_row(block, slot, a.block_size, a.kv_heads, kv_head) + 8 * g;
 #pragma unroll
-                for (int c = 0; c < 4; ++c) tile.k[half][c] = *reinterpret_cast<const uint4*>(kp + 8 * c);
+                for (int c = 0; c < 4; ++c) tile.k[half][c] = *reinterpret_cast<const uint4*>(kp + 32 * c);
             }
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
@@ -127,7 +127,7 @@ SINGE_DEVICE void load_tile(KeyTile& tile, const DecodeArgs& a, const unsigned i
                 const bool known = block < a.physical_blocks;
                 block = known ? block : 0;
                 const uint16_t* vp = a.value_cache + cache_row(block, slot, a.block_size, a.kv_heads, kv_head) + 8 * t;
-                tile.v[half][i] = *reinterpret_cast<const uint4*>(vp);
+                tile.v[half][i] = stream_load_16(vp);
                 if (inside && known) tile.live |= 1u << (half * 4 + i);
             }
         }
@@ -187,14 +187,16 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
     const unsigned int g = lane >> 4, t = lane & 15;
     const unsigned int reach = a.block_table_batch_stride * a.block_size;
 
-    // Tiles per sequence, prefix-summed: prefix[b] = tiles of sequences before b.
+    // Tiles per sequence, prefix-summed: prefix[b] = tiles of sequences before b; lengths[b] = its keys,
+    // clamped to what its table row can address.
+    unsigned int* lengths = prefix + a.batch + 1;
     if (wave == 0) {
         unsigned int carry = 0;
         for (unsigned int base = 0; base < a.batch; base += 64) {
-            unsigned int tiles = 0;
+            unsigned int tiles = 0, len = 0;
             if (base + lane < a.batch) {
                 const int raw = a.actual_seq_lens[base + lane];
-                const unsigned int len = raw < 0 ? 0u : (static_cast<unsigned int>(raw) < reach ? static_cast<unsigned int>(raw) : reach);
+                len = raw < 0 ? 0u : (static_cast<unsigned int>(raw) < reach ? static_cast<unsigned int>(raw) : reach);
                 tiles = (len + kTile - 1) / kTile;
             }
             unsigned int scan = tiles;
@@ -203,7 +205,10 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
                 const unsigned int below = __shfl_up(scan, step, 64);
                 if (lane >= static_cast<unsigned int>(step)) scan += below;
             }
-            if (base + lane < a.batch) prefix[base + lane + 1] = carry + scan;
+            if (base + lane < a.batch) {
+                prefix[base + lane + 1] = carry + scan;
+                lengths[base + lane] = len;
+            }
             carry += __shfl(scan, 63, 64);
         }
         if (lane == 0) prefix[0] = 0;
@@ -258,10 +263,10 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
         for (int hp = 0; hp < PAIRS; ++hp) {
             const unsigned int local = 2 * hp + (t >> 3);
             const bool real = local < wave_heads;
-            const uint16_t* qp = a.query + (static_cast<size_t>(b) * a.heads + kv_head * group + head_in_group + (real ? local : 0)) * kDim + 32 * g;
+            const uint16_t* qp = a.query + (static_cast<size_t>(b) * a.heads + kv_head * group + head_in_group + (real ? local : 0)) * kDim + 8 * g;
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                uint4 bits = *reinterpret_cast<const uint4*>(qp + 8 * c);
+                uint4 bits = *reinterpret_cast<const uint4*>(qp + 32 * c);
                 if (!real) bits = make_uint4(0, 0, 0, 0);
                 q[hp][c] = __builtin_bit_cast(bf16x8_t, bits);
             }
@@ -272,6 +277,17 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
     };
 
     auto fold = [&](const KeyTile& tile) {
+#ifdef SINGE_PROBE_LOADS_ONLY
+        // Measurement build only: touch every loaded register, skip the arithmetic.
+        unsigned int mix = tile.live;
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) mix ^= tile.k[half][c].x ^ tile.k[half][c].y ^ tile.k[half][c].z ^ tile.k[half][c].w ^
+                                               tile.v[half][c].x ^ tile.v[half][c].y ^ tile.v[half][c].z ^ tile.v[half][c].w;
+        state[0].running_sum += __builtin_bit_cast(float, mix & 0x3f800000u);
+        return;
+#endif
 #pragma unroll
         for (int hp = 0; hp < PAIRS; ++hp) {
             f32x4_t s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -334,10 +350,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
     };
 
     // Walk the range tile by tile, prefetching the next tile while the current one is folded.
-    auto seq_len = [&](unsigned int b) {
-        const int raw = a.actual_seq_lens[b];
-        return raw < 0 ? 0u : (static_cast<unsigned int>(raw) < reach ? static_cast<unsigned int>(raw) : reach);
-    };
+    auto seq_len = [&](unsigned int b) { return lengths[b]; };
     unsigned int at = range_first;  // flat tile index of the tile being folded
     unsigned int len = seq_len(seq);
     KeyTile ping, pong;
