@@ -131,6 +131,57 @@ SINGE_HIP_API int32_t singe_hip_paged_kv_decode_attention_phases_bf16(
 SINGE_HIP_API void singe_hip_set_decode_workers(uint32_t workers);
 SINGE_HIP_API uint32_t singe_hip_decode_workers(const SingePagedKvDecodeAttentionConfig* config);
 
+/* ---- singe-kernel surface: dense prefill ---------------------------------------------------------
+ * Mirrors FmhaPrefillConfig (singe-kernel/src/cuda/attention/mod.rs:253-274); strides in elements.
+ * FmhaPrefillConfig::contiguous (mod.rs:1602-1632) fills them for packed [batch, len, heads, dim]. */
+typedef struct SingeFmhaPrefillConfig {
+    size_t batch;
+    size_t query_len;
+    size_t key_len;
+    size_t heads;
+    size_t kv_heads;
+    size_t head_dim;
+    size_t query_batch_stride;
+    size_t key_batch_stride;
+    size_t value_batch_stride;
+    size_t output_batch_stride;
+    size_t query_sequence_stride;
+    size_t key_sequence_stride;
+    size_t value_sequence_stride;
+    size_t output_sequence_stride;
+    size_t query_head_stride;
+    size_t key_head_stride;
+    size_t value_head_stride;
+    size_t output_head_stride;
+    float scale;
+    uint8_t causal;   /* Rust bool: 0 or 1 */
+} SingeFmhaPrefillConfig;
+
+/* validate_fmha_prefill_config (mod.rs:3369-3398). */
+SINGE_HIP_API int32_t singe_hip_fmha_prefill_config_validate(const SingeFmhaPrefillConfig* config);
+
+/* fmha_prefill_bf16 (singe-kernel/src/cuda/attention/fmha.rs:744-790): out = softmax(scale * Q K^T
+ * [+ top-left causal mask]) V, query head h reading kv head h / (heads / kv_heads).
+ * Lengths are checked as FmhaPrefillConfig::validate_output_lengths does (mod.rs:1704-1756). */
+SINGE_HIP_API int32_t singe_hip_fmha_prefill_bf16(
+    void* stream,
+    uint16_t* out, size_t out_len,
+    const uint16_t* query, size_t query_len,
+    const uint16_t* key, size_t key_len,
+    const uint16_t* value, size_t value_len,
+    const SingeFmhaPrefillConfig* config);
+
+/* fmha_prefill_lse_bf16 (fmha.rs:638-690): also writes lse [batch, heads, query_len], the natural-log
+ * sum of exponentials of each row's scaled scores (cpu/attention.rs:1810-1811). */
+SINGE_HIP_API int32_t singe_hip_fmha_prefill_lse_bf16(
+    void* stream,
+    uint16_t* out, size_t out_len,
+    float* lse, size_t lse_len,
+    const uint16_t* query, size_t query_len,
+    const uint16_t* key, size_t key_len,
+    const uint16_t* value, size_t value_len,
+    const SingeFmhaPrefillConfig* config);
+
 #ifdef __cplusplus
 }
 #endif

@@ -26,6 +26,15 @@ class PagedKvDecodeAttentionConfigC(ctypes.Structure):
                 ("scale", ctypes.c_float)]
 
 
+class FmhaPrefillConfigC(ctypes.Structure):
+    _fields_ = [(name, c_size) for name in (
+        "batch", "query_len", "key_len", "heads", "kv_heads", "head_dim", "query_batch_stride",
+        "key_batch_stride", "value_batch_stride", "output_batch_stride", "query_sequence_stride",
+        "key_sequence_stride", "value_sequence_stride", "output_sequence_stride", "query_head_stride",
+        "key_head_stride", "value_head_stride", "output_head_stride")] + [("scale", ctypes.c_float),
+                                                                        ("causal", ctypes.c_uint8)]
+
+
 _lib = None
 
 
@@ -67,6 +76,15 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_set_decode_workers.restype = None
     handle.singe_hip_decode_workers.argtypes = [cfg]
     handle.singe_hip_decode_workers.restype = ctypes.c_uint32
+    fmha = ctypes.POINTER(FmhaPrefillConfigC)
+    handle.singe_hip_fmha_prefill_config_validate.argtypes = [fmha]
+    handle.singe_hip_fmha_prefill_config_validate.restype = i32
+    handle.singe_hip_fmha_prefill_bf16.argtypes = [c_void, c_void, c_size, c_void, c_size, c_void, c_size, c_void,
+                                                   c_size, fmha]
+    handle.singe_hip_fmha_prefill_bf16.restype = i32
+    handle.singe_hip_fmha_prefill_lse_bf16.argtypes = [c_void, c_void, c_size, c_void, c_size, c_void, c_size, c_void,
+                                                       c_size, c_void, c_size, fmha]
+    handle.singe_hip_fmha_prefill_lse_bf16.restype = i32
     _lib = handle
     return handle
 

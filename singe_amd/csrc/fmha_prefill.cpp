@@ -1,0 +1,143 @@
+// Host side of dense prefill: FmhaPrefillConfig validation as the reference does it
+// (singe-kernel/src/cuda/attention/mod.rs:1602-1756, 3369-3398, 3647-3677) and the launch.
+#include <cmath>
+
+#include "kernel_args.h"
+#include "module.h"
+#include "singe_hip_attention.h"
+#include "validate.h"
+
+using namespace singe_hip;
+
+namespace {
+
+int32_t validate_config(const SingeFmhaPrefillConfig& c) {
+    const size_t extents[] = {c.batch, c.query_len, c.key_len, c.heads, c.kv_heads, c.head_dim,
+                              c.query_batch_stride, c.key_batch_stride, c.value_batch_stride, c.output_batch_stride,
+                              c.query_sequence_stride, c.key_sequence_stride, c.value_sequence_stride,
+                              c.output_sequence_stride, c.query_head_stride, c.key_head_stride,
+                              c.value_head_stride, c.output_head_stride};
+    for (size_t extent : extents)
+        if (extent == 0) return fail(SINGE_HIP_INVALID_LENGTH, "config");
+    if (!std::isfinite(c.scale) || c.heads % c.kv_heads != 0) return fail(SINGE_HIP_INVALID_LENGTH, "config");
+    return 0;
+}
+
+// projected_layout_reach (mod.rs:3647-3668): elements one batch item can address.
+bool layout_reach(size_t sequence_len, size_t heads, size_t head_dim, size_t sequence_stride, size_t head_stride, size_t* out) {
+    size_t sequence_span, head_span;
+    if (sequence_len == 0 || heads == 0) return false;
+    return checked_mul(sequence_len - 1, sequence_stride, &sequence_span) && checked_mul(heads - 1, head_stride, &head_span) &&
+           checked_add(sequence_span, head_span, out) && checked_add(*out, head_dim, out);
+}
+
+// batched_reach (mod.rs:3670-3677).
+bool batched_reach(size_t batch, size_t item_len, size_t batch_stride, size_t* out) {
+    size_t span;
+    if (batch == 0) return false;
+    return checked_mul(batch - 1, batch_stride, &span) && checked_add(span, item_len, out);
+}
+
+int32_t ensure_reach(const char* name, size_t actual, size_t batch, size_t sequence_len, size_t heads, size_t head_dim,
+                     size_t batch_stride, size_t sequence_stride, size_t head_stride) {
+    size_t item = 0, need = 0;
+    if (!layout_reach(sequence_len, heads, head_dim, sequence_stride, head_stride, &item) ||
+        !batched_reach(batch, item, batch_stride, &need))
+        return fail(SINGE_HIP_SIZE_OVERFLOW, name);
+    return ensure_len_at_least(name, actual, need);
+}
+
+int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, bool with_lse,
+                const uint16_t* query, size_t query_len, const uint16_t* key, size_t key_len, const uint16_t* value,
+                size_t value_len, const SingeFmhaPrefillConfig* config) {
+    if (config == nullptr) return fail(SINGE_HIP_NULL_POINTER, "config");
+    const SingeFmhaPrefillConfig& c = *config;
+    // FmhaPrefillConfig::validate_lengths / validate_output_lengths (mod.rs:1634-1756), in their order.
+    if (int32_t status = validate_config(c)) return status;
+    if (int32_t status = ensure_reach("query", query_len, c.batch, c.query_len, c.heads, c.head_dim, c.query_batch_stride,
+                                      c.query_sequence_stride, c.query_head_stride)) return status;
+    if (int32_t status = ensure_reach("key", key_len, c.batch, c.key_len, c.kv_heads, c.head_dim, c.key_batch_stride,
+                                      c.key_sequence_stride, c.key_head_stride)) return status;
+    if (int32_t status = ensure_reach("value", value_len, c.batch, c.key_len, c.kv_heads, c.head_dim, c.value_batch_stride,
+                                      c.value_sequence_stride, c.value_head_stride)) return status;
+    if (int32_t status = ensure_reach("out", out_len, c.batch, c.query_len, c.heads, c.head_dim, c.output_batch_stride,
+                                      c.output_sequence_stride, c.output_head_stride)) return status;
+    if (with_lse) {
+        size_t rows = 0;
+        if (!checked_mul(c.batch, c.heads, &rows) || !checked_mul(rows, c.query_len, &rows)) return fail(SINGE_HIP_SIZE_OVERFLOW, "lse");
+        if (int32_t status = ensure_len_at_least("lse", lse_len, rows)) return status;
+        if (lse == nullptr) return fail(SINGE_HIP_NULL_POINTER, "lse");
+    }
+    const void* pointers[] = {out, query, key, value};
+    const char* names[] = {"out", "query", "key", "value"};
+    for (int i = 0; i < 4; ++i)
+        if (pointers[i] == nullptr) return fail(SINGE_HIP_NULL_POINTER, names[i]);
+
+    // What the gfx950 kernel takes: head_dim 128 and rows it can fetch 16 bytes at a time.
+    if (c.head_dim != 128) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, "fmha_prefill_bf16", c.head_dim, 0);
+    const size_t strides[] = {c.query_batch_stride, c.key_batch_stride, c.value_batch_stride, c.output_batch_stride,
+                              c.query_sequence_stride, c.key_sequence_stride, c.value_sequence_stride,
+                              c.output_sequence_stride, c.query_head_stride, c.key_head_stride,
+                              c.value_head_stride, c.output_head_stride};
+    for (size_t stride : strides)
+        if (stride % 8 != 0) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "strides must be multiples of 8 elements");
+    const uintptr_t addresses[] = {reinterpret_cast<uintptr_t>(out), reinterpret_cast<uintptr_t>(query),
+                                   reinterpret_cast<uintptr_t>(key), reinterpret_cast<uintptr_t>(value)};
+    for (uintptr_t address : addresses)
+        if (address % 16 != 0) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "buffers must be 16-byte aligned");
+    if (!fits_i32(c.query_len) || !fits_i32(c.key_len) || !fits_i32(c.batch) || !fits_i32(c.heads))
+        return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "config");
+
+    PrefillArgs args;
+    args.query = query;
+    args.key = key;
+    args.value = value;
+    args.out = out;
+    args.lse = with_lse ? lse : nullptr;
+    args.query_batch_stride = c.query_batch_stride;
+    args.query_sequence_stride = c.query_sequence_stride;
+    args.query_head_stride = c.query_head_stride;
+    args.key_batch_stride = c.key_batch_stride;
+    args.key_sequence_stride = c.key_sequence_stride;
+    args.key_head_stride = c.key_head_stride;
+    args.value_batch_stride = c.value_batch_stride;
+    args.value_sequence_stride = c.value_sequence_stride;
+    args.value_head_stride = c.value_head_stride;
+    args.output_batch_stride = c.output_batch_stride;
+    args.output_sequence_stride = c.output_sequence_stride;
+    args.output_head_stride = c.output_head_stride;
+    args.batch = static_cast<uint32_t>(c.batch);
+    args.query_len = static_cast<uint32_t>(c.query_len);
+    args.key_len = static_cast<uint32_t>(c.key_len);
+    args.heads = static_cast<uint32_t>(c.heads);
+    args.kv_heads = static_cast<uint32_t>(c.kv_heads);
+    args.query_tiles = static_cast<uint32_t>((c.query_len + 127) / 128);
+    args.scale_log2e = c.scale * 1.4426950408889634074f;
+    const uint64_t rows = (static_cast<uint64_t>(c.batch) * c.heads + 7) / 8 * 8;
+    const uint64_t groups = rows * args.query_tiles;
+    if (groups > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
+    return launch(c.causal ? kPrefillCausal : kPrefillFull, static_cast<unsigned>(groups), 1, 1, 256, stream, args);
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t singe_hip_fmha_prefill_config_validate(const SingeFmhaPrefillConfig* config) {
+    if (config == nullptr) return fail(SINGE_HIP_NULL_POINTER, "config");
+    return validate_config(*config);
+}
+
+int32_t singe_hip_fmha_prefill_bf16(void* stream, uint16_t* out, size_t out_len, const uint16_t* query, size_t query_len,
+                                    const uint16_t* key, size_t key_len, const uint16_t* value, size_t value_len,
+                                    const SingeFmhaPrefillConfig* config) {
+    return prefill(stream, out, out_len, nullptr, 0, false, query, query_len, key, key_len, value, value_len, config);
+}
+
+int32_t singe_hip_fmha_prefill_lse_bf16(void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len,
+                                        const uint16_t* query, size_t query_len, const uint16_t* key, size_t key_len,
+                                        const uint16_t* value, size_t value_len, const SingeFmhaPrefillConfig* config) {
+    return prefill(stream, out, out_len, lse, lse_len, true, query, query_len, key, key_len, value, value_len, config);
+}
+
+}  // extern "C"

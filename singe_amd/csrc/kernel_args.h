@@ -41,3 +41,22 @@ struct CombineArgs {
     uint32_t head_groups;
     uint32_t heads_per_wave;
 };
+
+struct PrefillArgs {
+    const uint16_t* query;          // [batch, query_len, heads, 128] bf16, element strides below
+    const uint16_t* key;            // [batch, key_len, kv_heads, 128]
+    const uint16_t* value;
+    uint16_t* out;                  // like query
+    float* lse;                     // [batch, heads, query_len] natural log, or null
+    uint64_t query_batch_stride, query_sequence_stride, query_head_stride;
+    uint64_t key_batch_stride, key_sequence_stride, key_head_stride;
+    uint64_t value_batch_stride, value_sequence_stride, value_head_stride;
+    uint64_t output_batch_stride, output_sequence_stride, output_head_stride;
+    uint32_t batch;
+    uint32_t query_len;
+    uint32_t key_len;
+    uint32_t heads;
+    uint32_t kv_heads;
+    uint32_t query_tiles;           // ceil(query_len / 128)
+    float scale_log2e;
+};

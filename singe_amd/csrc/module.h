@@ -12,6 +12,7 @@ enum KernelId : int {
     kDecodeP1B16 = 0, kDecodeP2B16, kDecodeP4B16,
     kDecodeP1Any, kDecodeP2Any, kDecodeP4Any,
     kDecodeCombine,
+    kPrefillCausal, kPrefillFull,
     kKernelCount
 };
 

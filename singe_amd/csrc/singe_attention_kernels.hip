@@ -1,3 +1,4 @@
 // The single translation unit of the gfx950 code object: hipcc --genco builds this file into
 // singe_attention_gfx950.hsaco, which the C-ABI library loads with hipModuleLoadData.
 #include "paged_decode.hip"
+#include "fmha_prefill.hip"

@@ -128,3 +128,71 @@ def paged_kv_decode_attention_bf16(stream, out: torch.Tensor, query: torch.Tenso
         actual_seq_lens.numel(), _ptr(block_table), block_table.numel(), _ptr(workspace),
         workspace.numel() * workspace.element_size(), ctypes.byref(c), phases)
     _native.check(status, "paged_kv_decode_attention_bf16")
+
+
+@dataclass(frozen=True)
+class FmhaPrefillConfig:
+    """Dense prefill attention (mod.rs:253-274): query/out [batch, query_len, heads, dim], key/value
+    [batch, key_len, kv_heads, dim], addressed through element strides; ``causal`` is top-left."""
+    batch: int
+    query_len: int
+    key_len: int
+    heads: int
+    kv_heads: int
+    head_dim: int
+    query_batch_stride: int
+    key_batch_stride: int
+    value_batch_stride: int
+    output_batch_stride: int
+    query_sequence_stride: int
+    key_sequence_stride: int
+    value_sequence_stride: int
+    output_sequence_stride: int
+    query_head_stride: int
+    key_head_stride: int
+    value_head_stride: int
+    output_head_stride: int
+    scale: float
+    causal: bool
+
+    @classmethod
+    def contiguous(cls, batch, query_len, key_len, heads, kv_heads, head_dim, scale, causal) -> "FmhaPrefillConfig":
+        """mod.rs:1602-1632: packed [batch, len, heads, dim] strides.  Like the reference, this does
+        not validate; the launch functions do."""
+        q_features, kv_features = heads * head_dim, kv_heads * head_dim
+        return cls(batch, query_len, key_len, heads, kv_heads, head_dim, query_len * q_features,
+                   key_len * kv_features, key_len * kv_features, query_len * q_features, q_features, kv_features,
+                   kv_features, q_features, head_dim, head_dim, head_dim, head_dim, scale, causal)
+
+    def _c(self) -> _native.FmhaPrefillConfigC:
+        return _native.FmhaPrefillConfigC(
+            self.batch, self.query_len, self.key_len, self.heads, self.kv_heads, self.head_dim,
+            self.query_batch_stride, self.key_batch_stride, self.value_batch_stride, self.output_batch_stride,
+            self.query_sequence_stride, self.key_sequence_stride, self.value_sequence_stride,
+            self.output_sequence_stride, self.query_head_stride, self.key_head_stride, self.value_head_stride,
+            self.output_head_stride, self.scale, 1 if self.causal else 0)
+
+
+def fmha_prefill_bf16(stream, out: torch.Tensor, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                      config: FmhaPrefillConfig) -> None:
+    """fmha_prefill_bf16 (fmha.rs:744-790)."""
+    for tensor, name in ((out, "out"), (query, "query"), (key, "key"), (value, "value")):
+        _require(tensor, torch.bfloat16, name)
+    c = config._c()
+    status = _native.lib().singe_hip_fmha_prefill_bf16(
+        _stream_handle(stream), _ptr(out), out.numel(), _ptr(query), query.numel(), _ptr(key), key.numel(),
+        _ptr(value), value.numel(), ctypes.byref(c))
+    _native.check(status, "fmha_prefill_bf16")
+
+
+def fmha_prefill_lse_bf16(stream, out: torch.Tensor, lse: torch.Tensor, query: torch.Tensor, key: torch.Tensor,
+                          value: torch.Tensor, config: FmhaPrefillConfig) -> None:
+    """fmha_prefill_lse_bf16 (fmha.rs:638-690): also writes lse [batch, heads, query_len], natural log."""
+    for tensor, name in ((out, "out"), (query, "query"), (key, "key"), (value, "value")):
+        _require(tensor, torch.bfloat16, name)
+    _require(lse, torch.float32, "lse")
+    c = config._c()
+    status = _native.lib().singe_hip_fmha_prefill_lse_bf16(
+        _stream_handle(stream), _ptr(out), out.numel(), _ptr(lse), lse.numel(), _ptr(query), query.numel(),
+        _ptr(key), key.numel(), _ptr(value), value.numel(), ctypes.byref(c))
+    _native.check(status, "fmha_prefill_lse_bf16")
