@@ -62,6 +62,12 @@ SINGE_DEVICE unsigned int pack_pair(float lo, float hi) {
     return __builtin_bit_cast(unsigned int, __builtin_convertvector(both, bf16x2v_t));
 }
 
+// How far (log2 units) a row's maximum may run ahead of the reference point its weights are scaled
+// by before the accumulators are rescaled.  Any reference point gives the same quotient; letting it lag
+// by up to 2^6 keeps weights far inside bf16/f32 range and makes the rescale of O^T rare after the
+// first tiles.
+constexpr float kMaxLag = 6.0f;
+
 template <bool CAUSAL>
 SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
     const unsigned int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -84,6 +90,10 @@ SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
     const uint16_t* v_base = a.value + batch * a.value_batch_stride + kv_head * a.value_head_stride;
 
     // Q^T as the MFMA B operand: lane (column = query, hi) holds dims 16s + 8hi .. +8 for s = 0..7.
+    // A negative scale is moved into Q (sign bits flipped) so the softmax below can take the row
+    // maximum of the raw scores and fold the positive factor into one fused multiply-add.
+    const float factor = fabsf(a.scale_log2e);
+    const unsigned int flip = a.scale_log2e < 0.0f ? 0x80008000u : 0u;
     bf16x8_t q[8];
     {
         const uint16_t* row = q_base + static_cast<size_t>(query_valid ? my_query : 0) * a.query_sequence_stride + 8 * hi;
@@ -91,6 +101,7 @@ SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
         for (int s = 0; s < 8; ++s) {
             uint4 bits = *reinterpret_cast<const uint4*>(row + 16 * s);
             if (!query_valid) bits = make_uint4(0, 0, 0, 0);
+            bits.x ^= flip; bits.y ^= flip; bits.z ^= flip; bits.w ^= flip;
             q[s] = __builtin_bit_cast(bf16x8_t, bits);
         }
     }
@@ -104,28 +115,32 @@ SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
     }
     const unsigned int tiles = (key_end + kKeyTile - 1) / kKeyTile;
 
-    uint4 stage_k[4], stage_v[4];
-    auto fetch = [&](unsigned int tile) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const unsigned int chunk = tid + 256u * i;
-            unsigned int key = tile * kKeyTile + (chunk >> 4);
-            key = key < a.key_len ? key : a.key_len - 1;  // rows past the end re-read the last key and are masked
-            const unsigned int dim = (chunk & 15u) * 8u;
-            stage_k[i] = *reinterpret_cast<const uint4*>(k_base + static_cast<size_t>(key) * a.key_sequence_stride + dim);
-            stage_v[i] = *reinterpret_cast<const uint4*>(v_base + static_cast<size_t>(key) * a.value_sequence_stride + dim);
-        }
+    const unsigned int load_row = tid >> 4, load_col = tid & 15u;  // chunk i of a thread: row + 16 i
+    // The next tile on its way from global memory to LDS: four 16-byte chunks of K and of V per thread
+    // (named registers, not arrays, so they are never given a stack slot).
+    uint4 k0, k1, k2, k3, v0, v1, v2, v3;
+    auto fetch_row = [&](unsigned int tile, unsigned int i, uint4& key_bits, uint4& value_bits) __attribute__((always_inline)) {
+        unsigned int key = tile * kKeyTile + load_row + 16u * i;
+        key = key < a.key_len ? key : a.key_len - 1;  // rows past the end re-read the last key and are masked
+        key_bits = *reinterpret_cast<const uint4*>(k_base + static_cast<size_t>(key) * a.key_sequence_stride + load_col * 8u);
+        value_bits = *reinterpret_cast<const uint4*>(v_base + static_cast<size_t>(key) * a.value_sequence_stride + load_col * 8u);
     };
-    auto stash = [&](unsigned int buffer) {
-        unsigned char* keys = lds + buffer * kStageBytes;
-        unsigned char* values = keys + kKeyStageBytes;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const unsigned int chunk = tid + 256u * i;
-            const unsigned int row = chunk >> 4, col = chunk & 15u;
-            *reinterpret_cast<uint4*>(keys + row * kKeyRowBytes + col * 16) = stage_k[i];
-            *reinterpret_cast<uint4*>(values + row * kValueRowBytes + col * 16) = stage_v[i];
-        }
+    auto fetch = [&](unsigned int tile) __attribute__((always_inline)) {
+        fetch_row(tile, 0, k0, v0);
+        fetch_row(tile, 1, k1, v1);
+        fetch_row(tile, 2, k2, v2);
+        fetch_row(tile, 3, k3, v3);
+    };
+    auto stash_row = [&](unsigned char* keys, unsigned char* values, unsigned int i, const uint4& key_bits, const uint4& value_bits) __attribute__((always_inline)) {
+        const unsigned int row = load_row + 16u * i;
+        *reinterpret_cast<uint4*>(keys + row * kKeyRowBytes + load_col * 16) = key_bits;
+        *reinterpret_cast<uint4*>(values + row * kValueRowBytes + load_col * 16) = value_bits;
+    };
+    auto stash = [&](unsigned char* keys, unsigned char* values) __attribute__((always_inline)) {
+        stash_row(keys, values, 0, k0, v0);
+        stash_row(keys, values, 1, k1, v1);
+        stash_row(keys, values, 2, k2, v2);
+        stash_row(keys, values, 3, k3, v3);
     };
 
     f32x16_t out[4];
@@ -133,11 +148,13 @@ SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
     for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int r = 0; r < 16; ++r) out[db][r] = 0.0f;
-    float running_max = -INFINITY, running_sum = 0.0f;
+    // reference = the point the weights are scaled by (scaled log2 units); it trails the true row
+    // maximum by at most kMaxLag.
+    float reference = -INFINITY, running_sum = 0.0f;
 
     if (tiles > 0) {
         fetch(0);
-        stash(0);
+        stash(lds, lds + kKeyStageBytes);
     }
     __syncthreads();
 
@@ -148,82 +165,96 @@ SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
     const unsigned int group = lane >> 4, sub = lane & 15u;
     const unsigned int value_read = (4 * hi + (sub >> 2)) * kValueRowBytes + (16 * (group & 1u) + 4 * (sub & 3u)) * 2;
 
-    for (unsigned int tile = 0; tile < tiles; ++tile) {
-        const unsigned int buffer = tile & 1u;
-        if (tile + 1 < tiles) fetch(tile + 1);
-
-        const unsigned char* keys = lds + buffer * kStageBytes;
-        const unsigned char* values = keys + kKeyStageBytes;
+    // Folds the 64 keys staged at `keys` / `values` (tile index `tile`) into the running state.
+    auto fold = [&](unsigned int tile, const unsigned char* keys, const unsigned char* values) __attribute__((always_inline)) {
         const unsigned int key0 = tile * kKeyTile;
         // A 32-key block wholly after the wave's last query contributes nothing under the causal mask.
-        const bool block_live[2] = {!CAUSAL || key0 <= first_row + 31u, !CAUSAL || key0 + 32u <= first_row + 31u};
+        const bool live0 = !CAUSAL || key0 <= first_row + 31u;
+        const bool live1 = !CAUSAL || key0 + 32u <= first_row + 31u;
+        if (!live0) return;
 
-        f32x16_t s[2];
+        f32x16_t s0, s1;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
+        for (int r = 0; r < 16; ++r) {
+            s0[r] = 0.0f;
+            s1[r] = 0.0f;
+        }
 #pragma unroll
-            for (int r = 0; r < 16; ++r) s[kb][r] = 0.0f;
-            if (block_live[kb]) {
+        for (int step = 0; step < 8; ++step) {
+            const uint4 bits = *reinterpret_cast<const uint4*>(keys + key_read + step * 32);
+            s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bits), q[step], s0, 0, 0, 0);
+        }
+        if (live1) {
 #pragma unroll
-                for (int step = 0; step < 8; ++step) {
-                    const uint4 bits = *reinterpret_cast<const uint4*>(keys + kb * 32 * kKeyRowBytes + key_read + step * 32);
-                    s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bits), q[step], s[kb], 0, 0, 0);
-                }
+            for (int step = 0; step < 8; ++step) {
+                const uint4 bits = *reinterpret_cast<const uint4*>(keys + 32 * kKeyRowBytes + key_read + step * 32);
+                s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bits), q[step], s1, 0, 0, 0);
             }
         }
 
-        // Mask what the query may not see: keys after it (causal) and keys past the end of the tensor.
+        // Hide what the query may not see: keys after it (causal), keys past the end of the tensor,
+        // and the second block when it is wholly hidden.  Only tiles on an edge pay for this.
         const bool edge = (CAUSAL && key0 + kKeyTile - 1 > first_row) || key0 + kKeyTile > a.key_len;
-        float largest = -INFINITY;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+        if (edge) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                float value = s[kb][r] * a.scale_log2e;
-                if (edge) {
-                    const unsigned int key = key0 + 32 * kb + 8 * (r >> 2) + 4 * hi + (r & 3);
-                    if ((CAUSAL && key > my_query) || key >= a.key_len) value = -INFINITY;
-                }
-                if (!block_live[kb]) value = -INFINITY;
-                s[kb][r] = value;
-                largest = fmaxf(largest, value);
+                const unsigned int key = key0 + 8 * (r >> 2) + 4 * hi + (r & 3);
+                if ((CAUSAL && key > my_query) || key >= a.key_len) s0[r] = -INFINITY;
+                if ((CAUSAL && key + 32 > my_query) || key + 32 >= a.key_len || !live1) s1[r] = -INFINITY;
             }
-        largest = fmaxf(swap32_max(largest), running_max);
-        const float base = largest == -INFINITY ? 0.0f : largest;
-        const float rescale = fast_exp2(running_max - base);
-        float total = 0.0f;
+        }
+
+        float largest = fmaxf(s0[0], s1[0]);
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float p = fast_exp2(s[kb][r] - base);
-                s[kb][r] = p;
-                total += p;
-            }
-        running_sum = running_sum * rescale + total;
-        const bool moved = largest > running_max;
-        running_max = largest;
-        if (__any(moved)) {
+        for (int r = 1; r < 16; ++r) largest = fmaxf(largest, fmaxf(s0[r], s1[r]));
+        largest = swap32_max(largest) * factor;  // both lanes of a query agree from here on
+        if (__any(largest > reference + kMaxLag || (reference == -INFINITY && largest != -INFINITY))) {
+            const float moved = fmaxf(reference, largest);
+            const float base = moved == -INFINITY ? 0.0f : moved;
+            const float rescale = fast_exp2(reference - base);
+            running_sum *= rescale;
 #pragma unroll
             for (int db = 0; db < 4; ++db)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) out[db][r] *= rescale;
+            reference = moved;
         }
-
-        // O^T += V^T . P^T, 16 keys per MFMA: registers 8j .. 8j+7 of block kb are keys
-        // 32kb + 16j + {0..3, 8..11} + 4hi, which is what the two transposing reads fetch.
+        const float shift = reference == -INFINITY ? 0.0f : -reference;
+        float total = 0.0f;
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-            if (!block_live[kb]) continue;
+        for (int r = 0; r < 16; ++r) {
+            s0[r] = fast_exp2(fmaf(s0[r], factor, shift));
+            s1[r] = fast_exp2(fmaf(s1[r], factor, shift));
+            total += s0[r] + s1[r];
+        }
+        running_sum += total;
+
+        // O^T += V^T . P^T, 16 keys per MFMA: registers 8j .. 8j+7 of a block are keys
+        // 16j + {0..3, 8..11} + 4hi of it, which is what the two transposing reads fetch.
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const uint4 weights = make_uint4(pack_pair(s0[8 * j + 0], s0[8 * j + 1]), pack_pair(s0[8 * j + 2], s0[8 * j + 3]),
+                                             pack_pair(s0[8 * j + 4], s0[8 * j + 5]), pack_pair(s0[8 * j + 6], s0[8 * j + 7]));
+            const unsigned char* rows = values + (16 * j) * kValueRowBytes + value_read;
+#pragma unroll
+            for (int db = 0; db < 4; ++db) {
+                const v4i16_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4i16_t __attribute__((address_space(3)))*)(rows + db * 64));
+                const v4i16_t high = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+                    (v4i16_t __attribute__((address_space(3)))*)(rows + 8 * kValueRowBytes + db * 64));
+                const v8i16_t both = __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7);
+                out[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, both),
+                                                                  __builtin_bit_cast(bf16x8_t, weights), out[db], 0, 0, 0);
+            }
+        }
+        if (live1) {
 #pragma unroll
             for (int j = 0; j < 2; ++j) {
-                const uint4 weights = make_uint4(pack_pair(s[kb][8 * j + 0], s[kb][8 * j + 1]), pack_pair(s[kb][8 * j + 2], s[kb][8 * j + 3]),
-                                                 pack_pair(s[kb][8 * j + 4], s[kb][8 * j + 5]), pack_pair(s[kb][8 * j + 6], s[kb][8 * j + 7]));
-                const unsigned char* rows = values + (32 * kb + 16 * j) * kValueRowBytes + value_read;
+                const uint4 weights = make_uint4(pack_pair(s1[8 * j + 0], s1[8 * j + 1]), pack_pair(s1[8 * j + 2], s1[8 * j + 3]),
+                                                 pack_pair(s1[8 * j + 4], s1[8 * j + 5]), pack_pair(s1[8 * j + 6], s1[8 * j + 7]));
+                const unsigned char* rows = values + (32 + 16 * j) * kValueRowBytes + value_read;
 #pragma unroll
                 for (int db = 0; db < 4; ++db) {
-                    const v4i16_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                        (v4i16_t __attribute__((address_space(3)))*)(rows + db * 64));
+                    const v4i16_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4i16_t __attribute__((address_space(3)))*)(rows + db * 64));
                     const v4i16_t high = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
                         (v4i16_t __attribute__((address_space(3)))*)(rows + 8 * kValueRowBytes + db * 64));
                     const v8i16_t both = __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -232,8 +263,21 @@ SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
                 }
             }
         }
+    };
 
-        if (tile + 1 < tiles) stash(buffer ^ 1u);
+    unsigned char* const keys0 = lds;
+    unsigned char* const values0 = lds + kKeyStageBytes;
+    unsigned char* const keys1 = lds + kStageBytes;
+    unsigned char* const values1 = lds + kStageBytes + kKeyStageBytes;
+    for (unsigned int tile = 0; tile < tiles; tile += 2) {
+        if (tile + 1 < tiles) fetch(tile + 1);
+        fold(tile, keys0, values0);
+        if (tile + 1 < tiles) stash(keys1, values1);
+        __syncthreads();
+        if (tile + 1 >= tiles) break;
+        if (tile + 2 < tiles) fetch(tile + 2);
+        fold(tile + 1, keys1, values1);
+        if (tile + 2 < tiles) stash(keys0, values0);
         __syncthreads();
     }
 
@@ -254,7 +298,7 @@ SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
             }
         if (a.lse != nullptr && hi == 0)
             a.lse[(static_cast<size_t>(batch) * a.heads + head) * a.query_len + my_query] =
-                sum > 0.0f ? (running_max + fast_log2(sum)) * kLn2 : -INFINITY;
+                sum > 0.0f ? (reference + fast_log2(sum)) * kLn2 : -INFINITY;
     }
 }
 

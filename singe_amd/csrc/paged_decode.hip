@@ -258,7 +258,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
 
     bf16x8_t q[PAIRS][4];
     PairState state[PAIRS];
-    auto load_query = [&](unsigned int b) {
+    auto load_query = [&](unsigned int b) __attribute__((always_inline)) {
 #pragma unroll
         for (int hp = 0; hp < PAIRS; ++hp) {
             const unsigned int local = 2 * hp + (t >> 3);
@@ -276,7 +276,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
         }
     };
 
-    auto fold = [&](const KeyTile& tile) {
+    auto fold = [&](const KeyTile& tile) __attribute__((always_inline)) {
 #ifdef SINGE_PROBE_LOADS_ONLY
         // Measurement build only: touch every loaded register, skip the arithmetic.
         unsigned int mix = tile.live;
@@ -331,7 +331,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
     };
 
     // Writes the partial row of sequence b: O / sum per head, and the natural-log LSE.
-    auto flush = [&](unsigned int b) {
+    auto flush = [&](unsigned int b) __attribute__((always_inline)) {
         const size_t slot = static_cast<size_t>(work) * slots + worker + b;
 #pragma unroll
         for (int hp = 0; hp < PAIRS; ++hp) {
@@ -350,14 +350,14 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
     };
 
     // Walk the range tile by tile, prefetching the next tile while the current one is folded.
-    auto seq_len = [&](unsigned int b) { return lengths[b]; };
+    auto seq_len = [&](unsigned int b) __attribute__((always_inline)) { return lengths[b]; };
     unsigned int at = range_first;  // flat tile index of the tile being folded
     unsigned int len = seq_len(seq);
     KeyTile ping, pong;
     load_query(seq);
     load_tile<ALIGNED16>(ping, a, a.block_table + static_cast<size_t>(seq) * a.block_table_batch_stride,
                          (at - prefix[seq]) * kTile, len, kv_head, g, t);
-    auto advance = [&](KeyTile& current, KeyTile& upcoming) {
+    auto advance = [&](KeyTile& current, KeyTile& upcoming) __attribute__((always_inline)) {
         // Returns false when `current` was the last tile of the range.
         const unsigned int next_at = at + 1;
         const bool more = next_at < range_end;
