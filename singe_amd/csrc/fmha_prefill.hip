@@ -173,23 +173,31 @@ SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
         const bool live1 = !CAUSAL || key0 + 32u <= first_row + 31u;
         if (!live0) return;
 
+        // Scores.  All eight K operands of a block are read before its MFMA chain starts, and the reads
+        // of the second block are issued while the first chain runs, so the matrix core never waits on
+        // a single LDS round trip.
         f32x16_t s0, s1;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             s0[r] = 0.0f;
             s1[r] = 0.0f;
         }
+        uint4 ka[8], kb[8];
 #pragma unroll
-        for (int step = 0; step < 8; ++step) {
-            const uint4 bits = *reinterpret_cast<const uint4*>(keys + key_read + step * 32);
-            s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bits), q[step], s0, 0, 0, 0);
-        }
+        for (int step = 0; step < 8; ++step) ka[step] = *reinterpret_cast<const uint4*>(keys + key_read + step * 32);
         if (live1) {
 #pragma unroll
             for (int step = 0; step < 8; ++step) {
-                const uint4 bits = *reinterpret_cast<const uint4*>(keys + 32 * kKeyRowBytes + key_read + step * 32);
-                s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, bits), q[step], s1, 0, 0, 0);
+                kb[step] = *reinterpret_cast<const uint4*>(keys + 32 * kKeyRowBytes + key_read + step * 32);
+                s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, ka[step]), q[step], s0, 0, 0, 0);
             }
+#pragma unroll
+            for (int step = 0; step < 8; ++step)
+                s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kb[step]), q[step], s1, 0, 0, 0);
+        } else {
+#pragma unroll
+            for (int step = 0; step < 8; ++step)
+                s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, ka[step]), q[step], s0, 0, 0, 0);
         }
 
         // Hide what the query may not see: keys after it (causal), keys past the end of the tensor,
