@@ -8,7 +8,9 @@ pool.  Inputs are resident in HBM before the timed region; three independent KV 
 consecutive steps cannot be served from the 256 MB Infinity Cache.
 
 Prints one JSON line: whole-job GB/s of algorithmic bytes, the roofline of the dominant kernel
-(measured with HIP events on the launch stream) and the CPU oracle timed on a bounded sample.
+(measured with HIP events on the launch stream) and the CPU oracle timed on a bounded sample.  The
+same line carries, under "prefill", the causal flash-attention prefill measurement (TFLOP/s against
+the dense bf16 MFMA peak).
 """
 from __future__ import annotations
 
@@ -23,6 +25,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
 POOLS = 3
 
 
@@ -32,6 +35,8 @@ def parse():
     parser.add_argument("--steps", type=int, default=300)
     parser.add_argument("--warmup", type=int, default=30)
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement")
+    parser.add_argument("--prefill-steps", type=int, default=40)
     parser.add_argument("--workers", type=int, default=0, help="tuning override (0 = built-in choice)")
     return parser.parse_args()
 
@@ -73,6 +78,59 @@ def cpu_baseline(work, budget_s=12.0):
         "kind": "port",
         "sample": f"first {used} of {work.batch} sequences of the same workload, reference loop shape "
                   f"(single thread, {elapsed:.1f} s)",
+    }
+
+
+def prefill_section(steps):
+    """Causal flash-attention prefill, batch 4, seq 4096, 32 heads, head_dim 128, bf16 (BASELINE
+    config 3): average kernel time from HIP events around back-to-back launches."""
+    import torch
+
+    from singe_amd.kernel import attention as A
+
+    batch, seq, heads, dim = 4, 4096, 32, 128
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x51A6E + 3)
+    q, k, v = (torch.randn((batch, seq, heads, dim), generator=gen, device="cuda").to(torch.bfloat16) for _ in range(3))
+    out = torch.empty_like(q)
+    config = A.FmhaPrefillConfig.contiguous(batch, seq, seq, heads, heads, dim, float(dim) ** -0.5, True)
+    for _ in range(5):
+        A.fmha_prefill_bf16(None, out, q, k, v, config)
+    torch.cuda.synchronize()
+    group = 5
+    groups = max(steps // group, 4)
+    begin = [torch.cuda.Event(enable_timing=True) for _ in range(groups)]
+    finish = [torch.cuda.Event(enable_timing=True) for _ in range(groups)]
+    for j in range(groups):
+        begin[j].record()
+        for _ in range(group):
+            A.fmha_prefill_bf16(None, out, q, k, v, config)
+        finish[j].record()
+    torch.cuda.synchronize()
+    ms = sorted(b.elapsed_time(f) / group for b, f in zip(begin, finish))
+    avg = sum(ms) / len(ms)
+    flops = 4 * dim * batch * heads * (seq * (seq + 1) // 2)
+    tflops = flops / (avg * 1e-3) / 1e12
+    return {
+        "workload": "causal flash prefill: batch 4, seq 4096, 32 heads (MHA), head_dim 128, bf16 in/out, "
+                    "fp32 softmax/accumulate (BASELINE config 3)",
+        "value": tflops,
+        "unit": "TFLOP/s",
+        "tokens_per_s": batch * seq / (avg * 1e-3),
+        "ms_per_step": avg,
+        "algorithmic_flops": flops,
+        "pct_bf16_mfma_peak": 100.0 * tflops / MFMA_BF16_PEAK_TFLOPS,
+        "roofline": {
+            "bound": "mfma",
+            "kernel": "singe_fmha_prefill_bf16_d128_causal",
+            "achieved": tflops,
+            "peak": MFMA_BF16_PEAK_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
+            "traffic": None,
+            "kernel_avg_us": avg * 1e3,
+            "kernel_median_us": ms[len(ms) // 2] * 1e3,
+        },
     }
 
 
@@ -167,7 +225,7 @@ def main():
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
         "roofline": {
             "bound": "hbm",
-            "kernel": "singe_paged_decode_bf16_d128_p2_b16",
+            "kernel": "singe_paged_decode_bf16_d128_g1_b16",
             "achieved": achieved,
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
@@ -179,6 +237,10 @@ def main():
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(work)
+    if not args.no_prefill:
+        del pools, workspace
+        torch.cuda.empty_cache()
+        result["prefill"] = prefill_section(args.prefill_steps)
     print(json.dumps(result), flush=True)
 
 

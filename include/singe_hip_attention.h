@@ -124,6 +124,33 @@ SINGE_HIP_API int32_t singe_hip_paged_kv_decode_attention_phases_bf16(
     const SingePagedKvDecodeAttentionConfig* config,
     uint32_t phases);
 
+/* The same decode over an fp8 e4m3 KV cache: caches hold one code per element, key_scales and
+ * value_scales [physical_blocks, kv_heads] f32 hold one scale per (block, kv head).  The kernel
+ * widens the cache in registers: every element is read as bf16_rne(f8e4m3_value(code) * scale)
+ * (singe-kernel/src/cpu/quantization.rs:245-280 for value * scale), i.e. exactly what the bf16 entry
+ * point computes on the dequantised cache.  The reference has no entry point of this kind; the
+ * argument order follows the bf16 one with the scales after the caches.  `phases` as above. */
+SINGE_HIP_API int32_t singe_hip_paged_kv_decode_attention_f8e4m3kv_bf16(
+    void* stream,
+    uint16_t* out, size_t out_len,
+    const uint16_t* query, size_t query_len,
+    const uint8_t* key_cache, size_t key_cache_len,
+    const uint8_t* value_cache, size_t value_cache_len,
+    const float* key_scales, size_t key_scales_len,
+    const float* value_scales, size_t value_scales_len,
+    const int32_t* actual_seq_lens, size_t actual_seq_lens_len,
+    const uint32_t* block_table, size_t block_table_len,
+    void* workspace, size_t workspace_bytes,
+    const SingePagedKvDecodeAttentionConfig* config,
+    uint32_t phases);
+
+/* Numerical policy, the counterpart of NumericalPolicy { precision: Full | Relaxed }
+ * (singe/src/graph/numerics/mod.rs:6-49).  Full (0, the default): fp8 elements are rounded to bf16
+ * after scaling, one by one.  Relaxed (non-zero): fp8 codes are widened exactly and the block scale is
+ * applied once per key to its score / probability, which is cheaper and not bit-identical. */
+SINGE_HIP_API void singe_hip_set_relaxed_numerics(int32_t relaxed);
+SINGE_HIP_API int32_t singe_hip_relaxed_numerics(void);
+
 /* Tuning knob of the split-KV decode: the number of equal key ranges each kv head's keys are cut
  * into (0 = one workgroup per compute unit).  The counterpart of
  * FmhaDecodeSplitKReduceConfig::max_splits / TuningChoice::Explicit

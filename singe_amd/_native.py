@@ -72,6 +72,14 @@ def lib() -> ctypes.CDLL:
         c_void, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size,
         c_void, c_size, cfg, ctypes.c_uint32]
     handle.singe_hip_paged_kv_decode_attention_phases_bf16.restype = i32
+    handle.singe_hip_paged_kv_decode_attention_f8e4m3kv_bf16.argtypes = [
+        c_void, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size,
+        c_void, c_size, c_void, c_size, c_void, c_size, cfg, ctypes.c_uint32]
+    handle.singe_hip_paged_kv_decode_attention_f8e4m3kv_bf16.restype = i32
+    handle.singe_hip_set_relaxed_numerics.argtypes = [i32]
+    handle.singe_hip_set_relaxed_numerics.restype = None
+    handle.singe_hip_relaxed_numerics.argtypes = []
+    handle.singe_hip_relaxed_numerics.restype = i32
     handle.singe_hip_set_decode_workers.argtypes = [ctypes.c_uint32]
     handle.singe_hip_set_decode_workers.restype = None
     handle.singe_hip_decode_workers.argtypes = [cfg]

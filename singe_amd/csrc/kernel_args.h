@@ -7,8 +7,10 @@
 
 struct DecodeArgs {
     const uint16_t* query;          // [batch, heads, 128] bf16
-    const uint16_t* key_cache;      // [blocks, block_size, kv_heads, 128] bf16
-    const uint16_t* value_cache;
+    const void* key_cache;          // [blocks, block_size, kv_heads, 128] bf16, or fp8 e4m3 codes
+    const void* value_cache;
+    const float* key_scales;        // fp8 caches: [blocks, kv_heads] f32, else unused
+    const float* value_scales;
     const int32_t* actual_seq_lens; // [batch]
     const uint32_t* block_table;    // [batch, stride]
     float* partial_out;             // [work, workers + batch, heads_per_wave, 128]

@@ -13,9 +13,12 @@
 namespace singe_hip {
 
 const char* const kKernelNames[kKernelCount] = {
-    "singe_paged_decode_bf16_d128_p1_b16", "singe_paged_decode_bf16_d128_p2_b16",
-    "singe_paged_decode_bf16_d128_p4_b16", "singe_paged_decode_bf16_d128_p1_any",
-    "singe_paged_decode_bf16_d128_p2_any", "singe_paged_decode_bf16_d128_p4_any",
+    "singe_paged_decode_bf16_d128_g1_b16", "singe_paged_decode_bf16_d128_g2_b16",
+    "singe_paged_decode_bf16_d128_g1_any", "singe_paged_decode_bf16_d128_g2_any",
+    "singe_paged_decode_f8kv_d128_g1_b16", "singe_paged_decode_f8kv_d128_g2_b16",
+    "singe_paged_decode_f8kv_d128_g1_any", "singe_paged_decode_f8kv_d128_g2_any",
+    "singe_paged_decode_f8kv_relaxed_d128_g1_b16", "singe_paged_decode_f8kv_relaxed_d128_g2_b16",
+    "singe_paged_decode_f8kv_relaxed_d128_g1_any", "singe_paged_decode_f8kv_relaxed_d128_g2_any",
     "singe_paged_decode_combine_bf16",
     "singe_fmha_prefill_bf16_d128_causal", "singe_fmha_prefill_bf16_d128_full",
 };

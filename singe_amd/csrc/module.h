@@ -9,9 +9,11 @@ namespace singe_hip {
 
 // Kernels of the code object, in the order of kKernelNames.
 enum KernelId : int {
-    kDecodeP1B16 = 0, kDecodeP2B16, kDecodeP4B16,
-    kDecodeP1Any, kDecodeP2Any, kDecodeP4Any,
-    kDecodeCombine,
+    // paged decode: index = base + 2 * (block size not a multiple of 16) + (two head groups per wave)
+    kDecodeBf16 = 0,
+    kDecodeF8 = 4,
+    kDecodeF8Relaxed = 8,
+    kDecodeCombine = 12,
     kPrefillCausal, kPrefillFull,
     kKernelCount
 };

@@ -14,6 +14,14 @@ using namespace singe_hip;
 namespace {
 
 std::atomic<uint32_t> g_forced_workers{0};
+std::atomic<bool> g_relaxed{false};
+
+int32_t decode(void* stream, uint16_t* out, size_t out_len, const uint16_t* query, size_t query_len,
+               const void* key_cache, size_t key_cache_len, const void* value_cache, size_t value_cache_len,
+               const float* key_scales, size_t key_scales_len, const float* value_scales, size_t value_scales_len,
+               bool fp8, const int32_t* actual_seq_lens, size_t actual_seq_lens_len, const uint32_t* block_table,
+               size_t block_table_len, void* workspace, size_t workspace_bytes,
+               const SingePagedKvDecodeAttentionConfig* config, uint32_t phases);
 
 constexpr size_t kHeadDim = 128;
 constexpr unsigned kWavesPerWorkgroup = 8;
@@ -22,7 +30,7 @@ constexpr unsigned kWavesPerWorkgroup = 8;
 struct Plan {
     uint32_t head_groups;     // waves per kv head: ceil(group / 8)
     uint32_t heads_per_wave;  // min(group, 8)
-    uint32_t pairs;           // 1, 2 or 4 pairs of query heads per wave
+    uint32_t groups;          // 1 or 2 groups of four query heads per wave
     uint32_t work;            // kv_heads * head_groups
     uint32_t work_per_wg;     // min(work, 8)
     uint32_t workers_per_wg;  // 8 / work_per_wg
@@ -40,7 +48,7 @@ Plan make_plan(const SingePagedKvDecodeAttentionConfig& c) {
     const size_t group = c.heads / c.kv_heads;
     p.head_groups = static_cast<uint32_t>((group + 7) / 8);
     p.heads_per_wave = static_cast<uint32_t>(group < 8 ? group : 8);
-    p.pairs = p.heads_per_wave <= 2 ? 1 : p.heads_per_wave <= 4 ? 2 : 4;
+    p.groups = p.heads_per_wave <= 4 ? 1 : 2;
     p.work = static_cast<uint32_t>(c.kv_heads) * p.head_groups;
     p.work_per_wg = p.work < kWavesPerWorkgroup ? p.work : kWavesPerWorkgroup;
     p.workers_per_wg = kWavesPerWorkgroup / p.work_per_wg;
@@ -113,6 +121,34 @@ int32_t singe_hip_paged_kv_decode_attention_phases_bf16(
     const int32_t* actual_seq_lens, size_t actual_seq_lens_len, const uint32_t* block_table,
     size_t block_table_len, void* workspace, size_t workspace_bytes,
     const SingePagedKvDecodeAttentionConfig* config, uint32_t phases) {
+    return decode(stream, out, out_len, query, query_len, key_cache, key_cache_len, value_cache, value_cache_len,
+                  nullptr, 0, nullptr, 0, false, actual_seq_lens, actual_seq_lens_len, block_table, block_table_len,
+                  workspace, workspace_bytes, config, phases);
+}
+
+int32_t singe_hip_paged_kv_decode_attention_f8e4m3kv_bf16(
+    void* stream, uint16_t* out, size_t out_len, const uint16_t* query, size_t query_len,
+    const uint8_t* key_cache, size_t key_cache_len, const uint8_t* value_cache, size_t value_cache_len,
+    const float* key_scales, size_t key_scales_len, const float* value_scales, size_t value_scales_len,
+    const int32_t* actual_seq_lens, size_t actual_seq_lens_len, const uint32_t* block_table,
+    size_t block_table_len, void* workspace, size_t workspace_bytes,
+    const SingePagedKvDecodeAttentionConfig* config, uint32_t phases) {
+    return decode(stream, out, out_len, query, query_len, key_cache, key_cache_len, value_cache, value_cache_len,
+                  key_scales, key_scales_len, value_scales, value_scales_len, true, actual_seq_lens,
+                  actual_seq_lens_len, block_table, block_table_len, workspace, workspace_bytes, config, phases);
+}
+
+}  // extern "C"
+
+namespace {
+
+int32_t decode(
+    void* stream, uint16_t* out, size_t out_len, const uint16_t* query, size_t query_len,
+    const void* key_cache, size_t key_cache_len, const void* value_cache, size_t value_cache_len,
+    const float* key_scales, size_t key_scales_len, const float* value_scales, size_t value_scales_len, bool fp8,
+    const int32_t* actual_seq_lens, size_t actual_seq_lens_len, const uint32_t* block_table,
+    size_t block_table_len, void* workspace, size_t workspace_bytes,
+    const SingePagedKvDecodeAttentionConfig* config, uint32_t phases) {
     if (config == nullptr) return fail(SINGE_HIP_NULL_POINTER, "config");
     const SingePagedKvDecodeAttentionConfig& c = *config;
     // PagedKvDecodeAttentionConfig::validate_lengths (mod.rs:711-743), in its order.
@@ -130,6 +166,14 @@ int32_t singe_hip_paged_kv_decode_attention_phases_bf16(
     if (int32_t status = ensure_len_at_least("actual_seq_lens", actual_seq_lens_len, c.batch)) return status;
     if (!checked_mul(c.batch, c.block_table_batch_stride, &table_len)) return fail(SINGE_HIP_SIZE_OVERFLOW, "block_table");
     if (int32_t status = ensure_len_at_least("block_table", block_table_len, table_len)) return status;
+    if (fp8) {
+        size_t scales = 0;
+        if (!checked_mul(c.physical_blocks, c.kv_heads, &scales)) return fail(SINGE_HIP_SIZE_OVERFLOW, "scales");
+        if (int32_t status = ensure_len_at_least("key_scales", key_scales_len, scales)) return status;
+        if (int32_t status = ensure_len_at_least("value_scales", value_scales_len, scales)) return status;
+        if (key_scales == nullptr) return fail(SINGE_HIP_NULL_POINTER, "key_scales");
+        if (value_scales == nullptr) return fail(SINGE_HIP_NULL_POINTER, "value_scales");
+    }
     // A DevicePointer is never null (singe-kernel/src/cuda/interop.rs:5-31).
     const void* pointers[] = {out, query, key_cache, value_cache, actual_seq_lens, block_table};
     const char* names[] = {"out", "query", "key_cache", "value_cache", "actual_seq_lens", "block_table"};
@@ -152,6 +196,8 @@ int32_t singe_hip_paged_kv_decode_attention_phases_bf16(
     args.query = query;
     args.key_cache = key_cache;
     args.value_cache = value_cache;
+    args.key_scales = key_scales;
+    args.value_scales = value_scales;
     args.actual_seq_lens = actual_seq_lens;
     args.block_table = block_table;
     args.meta = reinterpret_cast<uint32_t*>(scratch);
@@ -173,9 +219,9 @@ int32_t singe_hip_paged_kv_decode_attention_phases_bf16(
     args.heads_per_wave = plan.heads_per_wave;
     args.scale_log2e = c.scale * 1.4426950408889634074f;
 
-    const int column = plan.pairs == 1 ? 0 : plan.pairs == 2 ? 1 : 2;
     const bool aligned = c.block_size % 16 == 0;
-    KernelId kernel = static_cast<KernelId>((aligned ? kDecodeP1B16 : kDecodeP1Any) + column);
+    const int family = !fp8 ? kDecodeBf16 : (g_relaxed.load(std::memory_order_relaxed) ? kDecodeF8Relaxed : kDecodeF8);
+    KernelId kernel = static_cast<KernelId>(family + (aligned ? 0 : 2) + (plan.groups == 2 ? 1 : 0));
     if (phases & SINGE_HIP_DECODE_SPLIT)
         if (int32_t status = launch(kernel, plan.grid_x, plan.grid_y, 1, 64 * kWavesPerWorkgroup, stream, args,
                                     static_cast<unsigned>((2 * c.batch + 1) * sizeof(uint32_t))))
@@ -195,5 +241,12 @@ int32_t singe_hip_paged_kv_decode_attention_phases_bf16(
     combine.heads_per_wave = plan.heads_per_wave;
     return launch(kDecodeCombine, static_cast<unsigned>(c.batch * c.heads), 1, 1, 128, stream, combine);
 }
+
+}  // namespace
+
+extern "C" {
+
+void singe_hip_set_relaxed_numerics(int32_t relaxed) { g_relaxed.store(relaxed != 0, std::memory_order_relaxed); }
+int32_t singe_hip_relaxed_numerics(void) { return g_relaxed.load(std::memory_order_relaxed) ? 1 : 0; }
 
 }  // extern "C"

@@ -2,8 +2,9 @@
 // (the GPU counterpart of singe-kernel/src/cpu/attention.rs:1172-1246, replacing the cuTile kernels
 // of singe-kernel/src/cuda/cutile/kernel/attention/local.rs:9349-...).
 //
-// Layouts (fixed by the reference API): query/out [batch, heads, 128]; caches
-// [blocks, block_size, kv_heads, 128]; block_table [batch, stride] u32; actual_seq_lens [batch] i32.
+// Layouts (fixed by the reference API): query/out [batch, heads, 128] bf16; caches
+// [blocks, block_size, kv_heads, 128], bf16 or fp8 e4m3 with one f32 scale per (block, kv head);
+// block_table [batch, stride] u32; actual_seq_lens [batch] i32.
 //
 // Decode reads every KV byte once and does a few flop per byte, so it is bound by HBM bandwidth and,
 // at these sizes (tens of microseconds), by how evenly and how early the chip is filled.
@@ -18,18 +19,23 @@
 // splitk_reduce_f32 does (cpu/attention.rs:2157-2193).
 //
 // Inner loop, per 32-key tile, all on the matrix cores:
-//   scores   S^T[key, head] = K[key, :] . Q[head, :]  (v_mfma_f32_16x16x32_bf16, fp32 accumulate).  Two
-//            query heads share one MFMA, each repeated over 8 of the 16 columns.
+//   scores   S^T[key, head] = K[key, :] . Q[head, :]  (v_mfma_f32_16x16x32_bf16, fp32 accumulate).  Four
+//            query heads share one MFMA, each repeated over 4 of the 16 columns.
 //   softmax  online, base two; the tile maximum is shared by the wave (two v_permlane swaps), the
 //            running sum stays per lane until the row is flushed.
-//   values   V rows are loaded as whole 256-byte rows (16 lanes x 16 B, the coalesced layout) and used
-//            as the MFMA A operand exactly as loaded: A[chunk t][(g, e)] = V[key 4g + i][8t + e].
-//            The B operand is the probability of (head, key 4g + i) placed at position e of column
-//            (head, e), zero elsewhere, so C[t][(head, e)] accumulates O[head][8t + e].  That spends
-//            7/8 of the MFMA's multiplies on zeros, which is free here, and needs no transpose of V,
-//            no bf16 unpacking and no cross-lane traffic.  Probabilities are rounded to bf16 for this
-//            product and summed unrounded, as the reference's tensor-core kernel does
-//            (singe/src/backend/cuda/kernel_plan/source/tensor_core.rs:162-183).
+//   values   V rows are loaded as whole rows (16 lanes x 16 B, the coalesced layout) and used as the
+//            MFMA A operand exactly as loaded: for v_mfma_f32_16x16x16_bf16, A[chunk t][(g, e)] =
+//            V[key 4g + i][8t + 4half + e].  The B operand is the probability of (head, key 4g + i)
+//            placed at position e of column (head, e), zero elsewhere, so C[t][(head, e)] accumulates
+//            O[head][8t + 4half + e].  That spends 3/4 of the MFMA's multiplies on zeros, which is free
+//            here, and needs no transpose of V, no unpacking and no cross-lane traffic.  Probabilities
+//            are rounded to bf16 for this product and summed unrounded, as the reference's tensor-core
+//            kernel does (singe/src/backend/cuda/kernel_plan/source/tensor_core.rs:162-183).
+//
+// fp8 caches are widened to bf16 in registers on their way into the MFMA operands.  In the exact mode
+// every element becomes bf16_rne(f8e4m3_value(code) * scale) first (the value the CPU path reads after
+// dequantising the cache); in the relaxed mode the codes are widened exactly and the block's scale is
+// applied to the 32 scores / probabilities of the tile instead, which saves one multiply per element.
 #include "common.hip.h"
 #include "kernel_args.h"
 
@@ -38,10 +44,21 @@ namespace {
 constexpr int kDim = 128;
 constexpr int kTile = 32;
 
-struct KeyTile {
-    uint4 k[2][4];      // [16-key half][c]: lane (g, t) holds key t, dims 32c + 8g .. +8 (one load covers 64 B of each key)
+// One 32-key tile in registers, bf16 cache.
+struct KeyTileBf16 {
+    uint4 k[2][4];      // [16-key half][c]: lane (g, t) holds key t, dims 32c + 8g .. +8
     uint4 v[2][4];      // [16-key half][i]: lane (g, t) holds key 4g + i, dims 8t .. 8t + 8
     unsigned int live;  // bit (half * 4 + i): key half*16 + 4g + i takes part in the softmax
+};
+
+// One 32-key tile in registers, fp8 cache: the same keys and dims per lane, one byte per element.
+struct KeyTileFp8 {
+    uint4 k[2][2];        // lane (g, t): key t, dims 32g + 16x .. +16
+    uint2 v[2][4];        // lane (g, t): key 4g + i, dims 8t .. 8t + 8
+    float key_scale[2];   // scale of this lane's key t (exact mode)
+    float row_key_scale[2][4];    // scale of key 4g + i (relaxed mode: applied to its score)
+    float row_value_scale[2][4];  // scale of key 4g + i's values
+    unsigned int live;
 };
 
 // Element offset of (block, slot, kv_head, 0) in a [blocks, block_size, kv_heads, 128] cache.
@@ -61,76 +78,110 @@ SINGE_DEVICE void split_key(const DecodeArgs& a, unsigned int key, unsigned int&
     }
 }
 
-// Loads the 32 keys from `first` (a multiple of 32) of a sequence of `end` > first keys.  Keys at or
-// past `end`, and keys whose table entry is not a cache block, read an in-range row instead and are
-// marked dead, so nothing is read out of bounds and no dead row can carry a NaN into the sums.
+// Where the keys of one 16-key half live: the cache row of this lane's K key (t) and of its four V
+// keys (4g + i), whether each V key is live, and the blocks they came from (for fp8 scales).  Keys
+// at or past `end`, and keys whose table entry is not a cache block, resolve to an in-range row and
+// are dead, so nothing is read out of bounds and no dead row can carry a NaN into the sums.
+struct HalfRows {
+    size_t key_row;
+    size_t value_row[4];
+    unsigned int key_block;
+    unsigned int value_block[4];
+    unsigned int live;  // bit i
+};
+
 template <bool ALIGNED16>
-SINGE_DEVICE void load_tile(KeyTile& tile, const DecodeArgs& a, const unsigned int* table_row,
+SINGE_DEVICE HalfRows locate_half(const DecodeArgs& a, const unsigned int* table_row, unsigned int base,
+                                  unsigned int end, unsigned int kv_head, unsigned int g, unsigned int t) {
+    HalfRows rows;
+    rows.live = 0;
+    if constexpr (ALIGNED16) {
+        // block_size is a multiple of 16, so the 16 keys share one table entry; a half wholly past
+        // the end re-reads the 16-key span that holds the last key.
+        unsigned int last_entry, last_slot, entry, slot0;
+        split_key(a, end - 1, last_entry, last_slot);
+        split_key(a, base < end ? base : ((end - 1) & ~15u), entry, slot0);
+        const unsigned int block = table_row[entry];
+        const bool known = block < a.physical_blocks;
+        const unsigned int safe = known ? block : 0;
+        rows.key_block = safe;
+        rows.key_row = cache_row(safe, base + t < end ? slot0 + t : last_slot, a.block_size, a.kv_heads, kv_head);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const bool inside = base + 4 * g + i < end;
+            rows.value_block[i] = safe;
+            rows.value_row[i] = cache_row(safe, inside ? slot0 + 4 * g + i : last_slot, a.block_size, a.kv_heads, kv_head);
+            if (inside && known) rows.live |= 1u << i;
+        }
+    } else {
+        // Any block size: every lane looks up the table entry of its own keys.
+        {
+            unsigned int entry, slot;
+            split_key(a, base + t < end ? base + t : end - 1, entry, slot);
+            unsigned int block = table_row[entry];
+            block = block < a.physical_blocks ? block : 0;
+            rows.key_block = block;
+            rows.key_row = cache_row(block, slot, a.block_size, a.kv_heads, kv_head);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const unsigned int wanted = base + 4 * g + i;
+            const bool inside = wanted < end;
+            unsigned int entry, slot;
+            split_key(a, inside ? wanted : end - 1, entry, slot);
+            unsigned int block = table_row[entry];
+            const bool known = block < a.physical_blocks;
+            block = known ? block : 0;
+            rows.value_block[i] = block;
+            rows.value_row[i] = cache_row(block, slot, a.block_size, a.kv_heads, kv_head);
+            if (inside && known) rows.live |= 1u << i;
+        }
+    }
+    return rows;
+}
+
+// Loads the 32 keys from `first` (a multiple of 32) of a sequence of `end` > first keys.
+template <bool ALIGNED16>
+SINGE_DEVICE void load_tile(KeyTileBf16& tile, const DecodeArgs& a, const unsigned int* table_row,
                             unsigned int first, unsigned int end, unsigned int kv_head, unsigned int g,
                             unsigned int t) {
     tile.live = 0;
-    if constexpr (ALIGNED16) {
-        // block_size is a multiple of 16, so the 16 keys of a half share one table entry; a half
-        // wholly past the end re-reads the 16-key span that holds the last key.
-        unsigned int last_entry, last_slot, entry[2], slot0[2], block[2];
-        split_key(a, end - 1, last_entry, last_slot);
+    const uint16_t* key_cache = static_cast<const uint16_t*>(a.key_cache);
+    const uint16_t* value_cache = static_cast<const uint16_t*>(a.value_cache);
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            const unsigned int base = first + half * 16;
-            split_key(a, base < end ? base : ((end - 1) & ~15u), entry[half], slot0[half]);
+    for (int half = 0; half < 2; ++half) {
+        const HalfRows rows = locate_half<ALIGNED16>(a, table_row, first + half * 16, end, kv_head, g, t);
+        const uint16_t* kp = key_cache + rows.key_row + 8 * g;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) tile.k[half][c] = *reinterpret_cast<const uint4*>(kp + 32 * c);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) tile.v[half][i] = stream_load_16(value_cache + rows.value_row[i] + 8 * t);
+        tile.live |= rows.live << (half * 4);
+    }
+}
+
+template <bool ALIGNED16>
+SINGE_DEVICE void load_tile(KeyTileFp8& tile, const DecodeArgs& a, const unsigned int* table_row,
+                            unsigned int first, unsigned int end, unsigned int kv_head, unsigned int g,
+                            unsigned int t) {
+    tile.live = 0;
+    const uint8_t* key_cache = static_cast<const uint8_t*>(a.key_cache);
+    const uint8_t* value_cache = static_cast<const uint8_t*>(a.value_cache);
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        const HalfRows rows = locate_half<ALIGNED16>(a, table_row, first + half * 16, end, kv_head, g, t);
+        const uint8_t* kp = key_cache + rows.key_row + 32 * g;
+        tile.k[half][0] = *reinterpret_cast<const uint4*>(kp);
+        tile.k[half][1] = *reinterpret_cast<const uint4*>(kp + 16);
+        tile.key_scale[half] = a.key_scales[static_cast<size_t>(rows.key_block) * a.kv_heads + kv_head];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            tile.v[half][i] = *reinterpret_cast<const uint2*>(value_cache + rows.value_row[i] + 8 * t);
+            const size_t at = static_cast<size_t>(rows.value_block[i]) * a.kv_heads + kv_head;
+            tile.row_key_scale[half][i] = a.key_scales[at];
+            tile.row_value_scale[half][i] = a.value_scales[at];
         }
-#pragma unroll
-        for (int half = 0; half < 2; ++half) block[half] = table_row[entry[half]];
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            const unsigned int base = first + half * 16;
-            const bool known = block[half] < a.physical_blocks;
-            const unsigned int safe = known ? block[half] : 0;
-            {
-                const bool inside = base + t < end;
-                const uint16_t* kp = a.key_cache +
-                    cache_row(safe, inside ? slot0[half] + t : last_slot, a.block_size, a.kv_heads, kv_head) + 8 * g;
-#pragma unroll
-                for (int c = 0; c < 4; ++c) tile.k[half][c] = *reinterpret_cast<const uint4*>(kp + 32 * c);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const bool inside = base + 4 * g + i < end;
-                const uint16_t* vp = a.value_cache +
-                    cache_row(safe, inside ? slot0[half] + 4 * g + i : last_slot, a.block_size, a.kv_heads, kv_head) + 8 * t;
-                tile.v[half][i] = stream_load_16(vp);
-                if (inside && known) tile.live |= 1u << (half * 4 + i);
-            }
-        }
-    } else {
-        // Any block size: every lane looks up the table entry of its own key.
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-            const unsigned int base = first + half * 16;
-            {
-                const unsigned int key = base + t < end ? base + t : end - 1;
-                unsigned int entry, slot;
-                split_key(a, key, entry, slot);
-                unsigned int block = table_row[entry];
-                block = block < a.physical_blocks ? block : 0;
-                const uint16_t* kp = a.key_cache + cache_row(block, slot, a.block_size, a.kv_heads, kv_head) + 8 * g;
-#pragma unroll
-                for (int c = 0; c < 4; ++c) tile.k[half][c] = *reinterpret_cast<const uint4*>(kp + 32 * c);
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const unsigned int wanted = base + 4 * g + i;
-                const bool inside = wanted < end;
-                unsigned int entry, slot;
-                split_key(a, inside ? wanted : end - 1, entry, slot);
-                unsigned int block = table_row[entry];
-                const bool known = block < a.physical_blocks;
-                block = known ? block : 0;
-                const uint16_t* vp = a.value_cache + cache_row(block, slot, a.block_size, a.kv_heads, kv_head) + 8 * t;
-                tile.v[half][i] = stream_load_16(vp);
-                if (inside && known) tile.live |= 1u << (half * 4 + i);
-            }
-        }
+        tile.live |= rows.live << (half * 4);
     }
 }
 
@@ -166,23 +217,35 @@ SINGE_DEVICE float across_groups_sum(float value) {
 
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
+typedef short i16x4_t __attribute__((ext_vector_type(4)));
 
-// bf16(value) in both halves of a dword (one v_cvt_pk_bf16_f32, round to nearest even).
-SINGE_DEVICE unsigned int bf16_twice(float value) {
-    f32x2_t both = {value, value};
+SINGE_DEVICE unsigned int bf16_pair(float lo, float hi) {
+    f32x2_t both = {lo, hi};
     return __builtin_bit_cast(unsigned int, __builtin_convertvector(both, bf16x2_t));
 }
 
-// Per-wave softmax state of one pair of query heads.
-struct PairState {
-    f32x4_t acc;        // C[t][(head, e)]: lane (g, n) holds chunks t = 4g .. 4g+3 of column n
+// bf16(value) in both halves of a dword (one v_cvt_pk_bf16_f32, round to nearest even).
+SINGE_DEVICE unsigned int bf16_twice(float value) { return bf16_pair(value, value); }
+
+// Eight fp8 e4m3 codes -> eight bf16 values bf16_rne(value(code) * scale); scale 1 widens exactly.
+SINGE_DEVICE uint4 widen_fp8x8(unsigned int low, unsigned int high, float scale) {
+    const f32x2_t a = __builtin_amdgcn_cvt_pk_f32_fp8(low, false), b = __builtin_amdgcn_cvt_pk_f32_fp8(low, true);
+    const f32x2_t c = __builtin_amdgcn_cvt_pk_f32_fp8(high, false), d = __builtin_amdgcn_cvt_pk_f32_fp8(high, true);
+    return make_uint4(bf16_pair(a[0] * scale, a[1] * scale), bf16_pair(b[0] * scale, b[1] * scale),
+                      bf16_pair(c[0] * scale, c[1] * scale), bf16_pair(d[0] * scale, d[1] * scale));
+}
+
+// Per-wave softmax state of one group of four query heads.
+struct GroupState {
+    f32x4_t acc[2];     // [dims 8t..8t+3 | 8t+4..8t+7]: C[t][(head, e)], lane (g, n) holds chunks t = 4g .. 4g+3
     float running_max;  // log2 units, equal in all lanes that hold the same head
     float running_sum;  // of this lane's keys only
 };
 
-// PAIRS = pairs of query heads a wave carries (1, 2 or 4: up to 8 query heads per kv head).
-template <int PAIRS, bool ALIGNED16>
+// GROUPS = groups of four query heads a wave carries (1 or 2: up to 8 query heads per kv head).
+template <int GROUPS, bool ALIGNED16, bool FP8, bool EXACT>
 SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
+    using Tile = typename std::conditional<FP8, KeyTileFp8, KeyTileBf16>::type;
     const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const unsigned int g = lane >> 4, t = lane & 15;
     const unsigned int reach = a.block_table_batch_stride * a.block_size;
@@ -251,82 +314,111 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
         seq = low;
     }
 
-    // One-hot placement of a probability: column n = lane % 16 carries head n / 8 at position n % 8.
-    unsigned int place[4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) place[r] = (t & 7) / 2 == static_cast<unsigned int>(r) ? ((t & 1) ? 0xffff0000u : 0x0000ffffu) : 0u;
+    // One-hot placement of a probability: column n = lane % 16 carries head n / 4 at position n % 4.
+    const unsigned int place0 = (t & 2) ? 0u : ((t & 1) ? 0xffff0000u : 0x0000ffffu);
+    const unsigned int place1 = (t & 2) ? ((t & 1) ? 0xffff0000u : 0x0000ffffu) : 0u;
+    // Dims a lane feeds into score MFMA c: bf16 rows are fetched as 32c + 8g (64 contiguous bytes
+    // of each key per load), fp8 rows as 32g + 8c (32 contiguous bytes per lane).
+    const unsigned int dim_lane = FP8 ? 32 * g : 8 * g, dim_step = FP8 ? 8 : 32;
 
-    bf16x8_t q[PAIRS][4];
-    PairState state[PAIRS];
+    bf16x8_t q[GROUPS][4];
+    GroupState state[GROUPS];
     auto load_query = [&](unsigned int b) __attribute__((always_inline)) {
 #pragma unroll
-        for (int hp = 0; hp < PAIRS; ++hp) {
-            const unsigned int local = 2 * hp + (t >> 3);
+        for (int hg = 0; hg < GROUPS; ++hg) {
+            const unsigned int local = 4 * hg + (t >> 2);
             const bool real = local < wave_heads;
-            const uint16_t* qp = a.query + (static_cast<size_t>(b) * a.heads + kv_head * group + head_in_group + (real ? local : 0)) * kDim + 8 * g;
+            const uint16_t* qp = a.query + (static_cast<size_t>(b) * a.heads + kv_head * group + head_in_group + (real ? local : 0)) * kDim + dim_lane;
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                uint4 bits = *reinterpret_cast<const uint4*>(qp + 32 * c);
+                uint4 bits = *reinterpret_cast<const uint4*>(qp + dim_step * c);
                 if (!real) bits = make_uint4(0, 0, 0, 0);
-                q[hp][c] = __builtin_bit_cast(bf16x8_t, bits);
+                q[hg][c] = __builtin_bit_cast(bf16x8_t, bits);
             }
-            state[hp].acc = {0.0f, 0.0f, 0.0f, 0.0f};
-            state[hp].running_max = -INFINITY;
-            state[hp].running_sum = 0.0f;
+            state[hg].acc[0] = {0.0f, 0.0f, 0.0f, 0.0f};
+            state[hg].acc[1] = {0.0f, 0.0f, 0.0f, 0.0f};
+            state[hg].running_max = -INFINITY;
+            state[hg].running_sum = 0.0f;
         }
     };
 
-    auto fold = [&](const KeyTile& tile) __attribute__((always_inline)) {
-#ifdef SINGE_PROBE_LOADS_ONLY
-        // Measurement build only: touch every loaded register, skip the arithmetic.
-        unsigned int mix = tile.live;
+    auto fold = [&](const Tile& tile) __attribute__((always_inline)) {
+        // Operands as bf16: K per (half, c), V per (half, i).
+        uint4 keys[2][4], values[2][4];
+        if constexpr (FP8) {
 #pragma unroll
-        for (int half = 0; half < 2; ++half)
+            for (int half = 0; half < 2; ++half) {
+                const float ks = EXACT ? tile.key_scale[half] : 1.0f;
+                keys[half][0] = widen_fp8x8(tile.k[half][0].x, tile.k[half][0].y, ks);
+                keys[half][1] = widen_fp8x8(tile.k[half][0].z, tile.k[half][0].w, ks);
+                keys[half][2] = widen_fp8x8(tile.k[half][1].x, tile.k[half][1].y, ks);
+                keys[half][3] = widen_fp8x8(tile.k[half][1].z, tile.k[half][1].w, ks);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) mix ^= tile.k[half][c].x ^ tile.k[half][c].y ^ tile.k[half][c].z ^ tile.k[half][c].w ^
-                                               tile.v[half][c].x ^ tile.v[half][c].y ^ tile.v[half][c].z ^ tile.v[half][c].w;
-        state[0].running_sum += __builtin_bit_cast(float, mix & 0x3f800000u);
-        return;
-#endif
+                for (int i = 0; i < 4; ++i)
+                    values[half][i] = widen_fp8x8(tile.v[half][i].x, tile.v[half][i].y, EXACT ? tile.row_value_scale[half][i] : 1.0f);
+            }
+        } else {
 #pragma unroll
-        for (int hp = 0; hp < PAIRS; ++hp) {
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    keys[half][c] = tile.k[half][c];
+                    values[half][c] = tile.v[half][c];
+                }
+        }
+#pragma unroll
+        for (int hg = 0; hg < GROUPS; ++hg) {
             f32x4_t s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
-                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, tile.k[0][c]), q[hp][c], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, tile.k[1][c]), q[hp][c], s1, 0, 0, 0);
+                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, keys[0][c]), q[hg][c], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, keys[1][c]), q[hg][c], s1, 0, 0, 0);
             }
             float p[8];
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                p[i] = (tile.live >> i) & 1u ? s0[i] * a.scale_log2e : -INFINITY;
-                p[4 + i] = (tile.live >> (4 + i)) & 1u ? s1[i] * a.scale_log2e : -INFINITY;
+                float first = s0[i] * a.scale_log2e, second = s1[i] * a.scale_log2e;
+                if constexpr (FP8 && !EXACT) {
+                    first *= tile.row_key_scale[0][i];
+                    second *= tile.row_key_scale[1][i];
+                }
+                p[i] = (tile.live >> i) & 1u ? first : -INFINITY;
+                p[4 + i] = (tile.live >> (4 + i)) & 1u ? second : -INFINITY;
             }
             float largest = fmaxf(fmaxf(fmaxf(p[0], p[1]), fmaxf(p[2], p[3])), fmaxf(fmaxf(p[4], p[5]), fmaxf(p[6], p[7])));
-            largest = fmaxf(across_groups_max(largest), state[hp].running_max);
+            largest = fmaxf(across_groups_max(largest), state[hg].running_max);
             const float base = largest == -INFINITY ? 0.0f : largest;
-            const float rescale = fast_exp2(state[hp].running_max - base);
+            const float rescale = fast_exp2(state[hg].running_max - base);
             float total = 0.0f;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 p[i] = fast_exp2(p[i] - base);
                 total += p[i];
             }
-            state[hp].running_sum = state[hp].running_sum * rescale + total;
-            state[hp].running_max = largest;
-            f32x4_t acc = state[hp].acc;
+            state[hg].running_sum = state[hg].running_sum * rescale + total;
+            state[hg].running_max = largest;
+            f32x4_t low = state[hg].acc[0], high = state[hg].acc[1];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) acc[r] *= rescale;
+            for (int r = 0; r < 4; ++r) {
+                low[r] *= rescale;
+                high[r] *= rescale;
+            }
 #pragma unroll
             for (int half = 0; half < 2; ++half)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const unsigned int both = bf16_twice(p[half * 4 + i]);
-                    const uint4 hot = make_uint4(both & place[0], both & place[1], both & place[2], both & place[3]);
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, tile.v[half][i]),
-                                                                  __builtin_bit_cast(bf16x8_t, hot), acc, 0, 0, 0);
+                    float weight = p[half * 4 + i];
+                    if constexpr (FP8 && !EXACT) weight *= tile.row_value_scale[half][i];
+                    const unsigned int both = bf16_twice(weight);
+                    const uint2 hot = make_uint2(both & place0, both & place1);
+                    const uint4 row = values[half][i];
+                    low = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(i16x4_t, make_uint2(row.x, row.y)),
+                                                                   __builtin_bit_cast(i16x4_t, hot), low, 0, 0, 0);
+                    high = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(i16x4_t, make_uint2(row.z, row.w)),
+                                                                    __builtin_bit_cast(i16x4_t, hot), high, 0, 0, 0);
                 }
-            state[hp].acc = acc;
+            state[hg].acc[0] = low;
+            state[hg].acc[1] = high;
         }
     };
 
@@ -334,17 +426,20 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
     auto flush = [&](unsigned int b) __attribute__((always_inline)) {
         const size_t slot = static_cast<size_t>(work) * slots + worker + b;
 #pragma unroll
-        for (int hp = 0; hp < PAIRS; ++hp) {
-            const float sum = across_groups_sum(state[hp].running_sum);
+        for (int hg = 0; hg < GROUPS; ++hg) {
+            const float sum = across_groups_sum(state[hg].running_sum);
             const float inverse = sum > 0.0f ? 1.0f / sum : 0.0f;
-            const unsigned int local = 2 * hp + (t >> 3);
+            const unsigned int local = 4 * hg + (t >> 2);
             if (local < wave_heads) {
                 float* row = a.partial_out + (slot * a.heads_per_wave + local) * kDim;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) row[8 * (4 * g + r) + (t & 7)] = state[hp].acc[r] * inverse;
-                if (g == 0 && (t & 7) == 0)
+                for (int r = 0; r < 4; ++r) {
+                    row[8 * (4 * g + r) + (t & 3)] = state[hg].acc[0][r] * inverse;
+                    row[8 * (4 * g + r) + 4 + (t & 3)] = state[hg].acc[1][r] * inverse;
+                }
+                if (g == 0 && (t & 3) == 0)
                     a.partial_lse[slot * a.heads_per_wave + local] =
-                        sum > 0.0f ? (state[hp].running_max + fast_log2(sum)) * kLn2 : -INFINITY;
+                        sum > 0.0f ? (state[hg].running_max + fast_log2(sum)) * kLn2 : -INFINITY;
             }
         }
     };
@@ -353,11 +448,11 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
     auto seq_len = [&](unsigned int b) __attribute__((always_inline)) { return lengths[b]; };
     unsigned int at = range_first;  // flat tile index of the tile being folded
     unsigned int len = seq_len(seq);
-    KeyTile ping, pong;
+    Tile ping, pong;
     load_query(seq);
     load_tile<ALIGNED16>(ping, a, a.block_table + static_cast<size_t>(seq) * a.block_table_batch_stride,
                          (at - prefix[seq]) * kTile, len, kv_head, g, t);
-    auto advance = [&](KeyTile& current, KeyTile& upcoming) __attribute__((always_inline)) {
+    auto advance = [&](Tile& current, Tile& upcoming) __attribute__((always_inline)) {
         // Returns false when `current` was the last tile of the range.
         const unsigned int next_at = at + 1;
         const bool more = next_at < range_end;
@@ -386,19 +481,24 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
 
 }  // namespace
 
-#define SINGE_DECODE_KERNEL(PAIRS, ALIGNED, SUFFIX)                                                       \
-    extern "C" __global__ __launch_bounds__(512) void singe_paged_decode_bf16_d128_p##PAIRS##SUFFIX(       \
-        DecodeArgs args) {                                                                               \
-        extern __shared__ unsigned int prefix[];                                                         \
-        paged_decode_body<PAIRS, ALIGNED>(args, prefix);                                                 \
+#define SINGE_DECODE_KERNEL(NAME, GROUPS, ALIGNED, FP8, EXACT)                                  \
+    extern "C" __global__ __launch_bounds__(512) void NAME(DecodeArgs args) {                    \
+        extern __shared__ unsigned int prefix[];                                                \
+        paged_decode_body<GROUPS, ALIGNED, FP8, EXACT>(args, prefix);                           \
     }
 
-SINGE_DECODE_KERNEL(1, true, _b16)
-SINGE_DECODE_KERNEL(2, true, _b16)
-SINGE_DECODE_KERNEL(4, true, _b16)
-SINGE_DECODE_KERNEL(1, false, _any)
-SINGE_DECODE_KERNEL(2, false, _any)
-SINGE_DECODE_KERNEL(4, false, _any)
+SINGE_DECODE_KERNEL(singe_paged_decode_bf16_d128_g1_b16, 1, true, false, true)
+SINGE_DECODE_KERNEL(singe_paged_decode_bf16_d128_g2_b16, 2, true, false, true)
+SINGE_DECODE_KERNEL(singe_paged_decode_bf16_d128_g1_any, 1, false, false, true)
+SINGE_DECODE_KERNEL(singe_paged_decode_bf16_d128_g2_any, 2, false, false, true)
+SINGE_DECODE_KERNEL(singe_paged_decode_f8kv_d128_g1_b16, 1, true, true, true)
+SINGE_DECODE_KERNEL(singe_paged_decode_f8kv_d128_g2_b16, 2, true, true, true)
+SINGE_DECODE_KERNEL(singe_paged_decode_f8kv_d128_g1_any, 1, false, true, true)
+SINGE_DECODE_KERNEL(singe_paged_decode_f8kv_d128_g2_any, 2, false, true, true)
+SINGE_DECODE_KERNEL(singe_paged_decode_f8kv_relaxed_d128_g1_b16, 1, true, true, false)
+SINGE_DECODE_KERNEL(singe_paged_decode_f8kv_relaxed_d128_g2_b16, 2, true, true, false)
+SINGE_DECODE_KERNEL(singe_paged_decode_f8kv_relaxed_d128_g1_any, 1, false, true, false)
+SINGE_DECODE_KERNEL(singe_paged_decode_f8kv_relaxed_d128_g2_any, 2, false, true, false)
 
 // Folds the partial rows of one (sequence, query head) into the bf16 output:
 // out = sum_s exp(lse_s - max) * partial_s / sum_s exp(lse_s - max)

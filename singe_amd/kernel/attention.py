@@ -130,6 +130,44 @@ def paged_kv_decode_attention_bf16(stream, out: torch.Tensor, query: torch.Tenso
     _native.check(status, "paged_kv_decode_attention_bf16")
 
 
+def paged_kv_decode_attention_f8e4m3kv_bf16(stream, out: torch.Tensor, query: torch.Tensor, key_cache: torch.Tensor,
+                                            value_cache: torch.Tensor, key_scales: torch.Tensor,
+                                            value_scales: torch.Tensor, actual_seq_lens: torch.Tensor,
+                                            block_table: torch.Tensor, config: PagedKvDecodeAttentionConfig,
+                                            workspace: torch.Tensor | None = None, phases: int = 3) -> None:
+    """Paged decode over an fp8 e4m3 KV cache (uint8 codes, or torch.float8_e4m3fn) with one f32 scale
+    per (block, kv head); same result as paged_kv_decode_attention_bf16 on the cache dequantised to
+    bf16_rne(f8e4m3_value(code) * scale).  No counterpart in the reference's launch API."""
+    _require(out, torch.bfloat16, "out")
+    _require(query, torch.bfloat16, "query")
+    for tensor, name in ((key_cache, "key_cache"), (value_cache, "value_cache")):
+        if tensor.dtype not in (torch.uint8, torch.float8_e4m3fn):
+            raise error.InvalidArgument(f"{name} must hold fp8 e4m3 codes, got {tensor.dtype}")
+        _require(tensor, tensor.dtype, name)
+    _require(key_scales, torch.float32, "key_scales")
+    _require(value_scales, torch.float32, "value_scales")
+    _require(actual_seq_lens, torch.int32, "actual_seq_lens")
+    if block_table.dtype not in (torch.int32, torch.uint32):
+        raise error.InvalidArgument(f"block_table must hold 32-bit entries, got {block_table.dtype}")
+    _require(block_table, block_table.dtype, "block_table")
+    c = config._c()
+    if workspace is None:
+        need = int(_native.lib().singe_hip_paged_kv_decode_attention_workspace_bytes(ctypes.byref(c)))
+        workspace = _workspaces.get(out.device, need)
+    status = _native.lib().singe_hip_paged_kv_decode_attention_f8e4m3kv_bf16(
+        _stream_handle(stream), _ptr(out), out.numel(), _ptr(query), query.numel(), _ptr(key_cache),
+        key_cache.numel(), _ptr(value_cache), value_cache.numel(), _ptr(key_scales), key_scales.numel(),
+        _ptr(value_scales), value_scales.numel(), _ptr(actual_seq_lens), actual_seq_lens.numel(),
+        _ptr(block_table), block_table.numel(), _ptr(workspace), workspace.numel() * workspace.element_size(),
+        ctypes.byref(c), phases)
+    _native.check(status, "paged_kv_decode_attention_f8e4m3kv_bf16")
+
+
+def set_relaxed_numerics(relaxed: bool) -> None:
+    """NumericalPolicy precision: Full (False, default) or Relaxed (True)."""
+    _native.lib().singe_hip_set_relaxed_numerics(1 if relaxed else 0)
+
+
 @dataclass(frozen=True)
 class FmhaPrefillConfig:
     """Dense prefill attention (mod.rs:253-274): query/out [batch, query_len, heads, dim], key/value

@@ -96,3 +96,51 @@ def paged_decode_workload(*, batch=32, heads=32, kv_heads=8, head_dim=128, block
     return PagedDecodeWorkload(batch, heads, kv_heads, head_dim, block_size, physical_blocks, stride,
                                float(1.0 / np.sqrt(np.float32(head_dim))), seq_lens, table, query, key_cache,
                                value_cache)
+
+
+@dataclass
+class PagedDecodeFp8Workload(PagedDecodeWorkload):
+    """Paged decode over an fp8 e4m3 KV cache: key_cache/value_cache hold codes (uint8),
+    key_scales/value_scales [blocks, kv_heads] f32 hold one scale per (block, kv head)."""
+    key_scales: torch.Tensor = None
+    value_scales: torch.Tensor = None
+
+
+def quantize_fp8_blocks(values: torch.Tensor):
+    """[blocks, block_size, kv_heads, dim] f32 -> (codes uint8, scales [blocks, kv_heads] f32) with
+    scale = max |x| over the (block, kv head) tile / 448 and code = e4m3(x / scale), round to nearest
+    even (torch's float8_e4m3fn cast, the conversion the reference's encode table is taken from:
+    singe-codegen/src/interpret/tests.rs:274-312)."""
+    peak = values.abs().amax(dim=(1, 3))
+    scales = torch.where(peak > 0, peak / 448.0, torch.ones_like(peak)).to(torch.float32)
+    codes = (values / scales[:, None, :, None]).to(torch.float8_e4m3fn).view(torch.uint8)
+    return codes, scales
+
+
+def paged_decode_fp8_workload(*, batch=64, heads=64, kv_heads=8, head_dim=128, block_size=16,
+                              physical_blocks=131072, min_len=32768, max_len=32768, seed=BASE_SEED + 5,
+                              device="cuda", seq_lens=None, chunk_blocks=8192) -> PagedDecodeFp8Workload:
+    """Long-context decode with an fp8 KV cache (values ~ N(0, 1) before quantisation)."""
+    rng = np.random.default_rng(seed)
+    if seq_lens is None:
+        seq_lens = rng.integers(min_len, max_len + 1, size=batch).astype(np.int32)
+    else:
+        seq_lens = np.asarray(seq_lens, dtype=np.int32)
+    table, stride = paged_block_table(rng, seq_lens, block_size, physical_blocks)
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed + 1)
+    query = torch.randn((batch, heads, head_dim), generator=gen, device=device, dtype=torch.float32).to(torch.bfloat16)
+    shape = (physical_blocks, block_size, kv_heads, head_dim)
+    caches, scales = [], []
+    for _ in range(2):
+        codes = torch.empty(shape, device=device, dtype=torch.uint8)
+        scale = torch.empty((physical_blocks, kv_heads), device=device, dtype=torch.float32)
+        for first in range(0, physical_blocks, chunk_blocks):
+            count = min(chunk_blocks, physical_blocks - first)
+            source = torch.randn((count, block_size, kv_heads, head_dim), generator=gen, device=device, dtype=torch.float32)
+            codes[first:first + count], scale[first:first + count] = quantize_fp8_blocks(source)
+        caches.append(codes)
+        scales.append(scale)
+    return PagedDecodeFp8Workload(batch, heads, kv_heads, head_dim, block_size, physical_blocks, stride,
+                                  float(1.0 / np.sqrt(np.float32(head_dim))), seq_lens, table, query, caches[0],
+                                  caches[1], scales[0], scales[1])
