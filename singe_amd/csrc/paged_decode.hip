@@ -83,6 +83,7 @@ SINGE_DEVICE void split_key(const DecodeArgs& a, unsigned int key, unsigned int&
 // at or past `end`, and keys whose table entry is not a cache block, resolve to an in-range row and
 // are dead, so nothing is read out of bounds and no dead row can carry a NaN into the sums.
 struct HalfRows {
+    unsigned int cache_lane;  // lane of the entry cache that holds this half's block (aligned path)
     size_t key_row;
     size_t value_row[4];
     unsigned int key_block;
@@ -90,9 +91,38 @@ struct HalfRows {
     unsigned int live;  // bit i
 };
 
+// 64 consecutive block-table entries of one sequence, one per lane, fetched with a single vector
+// load (plus, for fp8 caches, the two scales of each block).  Tiles then pick their entry out of a
+// register with v_readlane instead of paying a dependent scalar-load round trip per 16 keys.
+struct EntryCache {
+    unsigned int sequence = 0xffffffffu;
+    unsigned int first_entry = 0;
+    unsigned int blocks = 0;      // lane l: table[sequence][first_entry + l]
+    float key_scales = 0.0f;      // lane l: scale of that block for this wave's kv head
+    float value_scales = 0.0f;
+};
+
+template <bool FP8>
+SINGE_DEVICE void fill_entries(EntryCache& cache, const DecodeArgs& a, unsigned int sequence, unsigned int first_entry,
+                               unsigned int kv_head, unsigned int lane) {
+    cache.sequence = sequence;
+    cache.first_entry = first_entry;
+    const unsigned int index = first_entry + lane;
+    unsigned int block = 0xffffffffu;
+    if (index < a.block_table_batch_stride)
+        block = a.block_table[static_cast<size_t>(sequence) * a.block_table_batch_stride + index];
+    cache.blocks = block;
+    if constexpr (FP8) {
+        const size_t at = static_cast<size_t>(block < a.physical_blocks ? block : 0) * a.kv_heads + kv_head;
+        cache.key_scales = a.key_scales[at];
+        cache.value_scales = a.value_scales[at];
+    }
+}
+
 template <bool ALIGNED16>
-SINGE_DEVICE HalfRows locate_half(const DecodeArgs& a, const unsigned int* table_row, unsigned int base,
-                                  unsigned int end, unsigned int kv_head, unsigned int g, unsigned int t) {
+SINGE_DEVICE HalfRows locate_half(const DecodeArgs& a, const unsigned int* table_row, const EntryCache& cache,
+                                  unsigned int base, unsigned int end, unsigned int kv_head, unsigned int g,
+                                  unsigned int t) {
     HalfRows rows;
     rows.live = 0;
     if constexpr (ALIGNED16) {
@@ -101,7 +131,8 @@ SINGE_DEVICE HalfRows locate_half(const DecodeArgs& a, const unsigned int* table
         unsigned int last_entry, last_slot, entry, slot0;
         split_key(a, end - 1, last_entry, last_slot);
         split_key(a, base < end ? base : ((end - 1) & ~15u), entry, slot0);
-        const unsigned int block = table_row[entry];
+        rows.cache_lane = entry - cache.first_entry;
+        const unsigned int block = __builtin_amdgcn_readlane(cache.blocks, rows.cache_lane);
         const bool known = block < a.physical_blocks;
         const unsigned int safe = known ? block : 0;
         rows.key_block = safe;
@@ -142,7 +173,7 @@ SINGE_DEVICE HalfRows locate_half(const DecodeArgs& a, const unsigned int* table
 
 // Loads the 32 keys from `first` (a multiple of 32) of a sequence of `end` > first keys.
 template <bool ALIGNED16>
-SINGE_DEVICE void load_tile(KeyTileBf16& tile, const DecodeArgs& a, const unsigned int* table_row,
+SINGE_DEVICE void load_tile(KeyTileBf16& tile, const DecodeArgs& a, const unsigned int* table_row, const EntryCache& cache,
                             unsigned int first, unsigned int end, unsigned int kv_head, unsigned int g,
                             unsigned int t) {
     tile.live = 0;
@@ -150,7 +181,7 @@ SINGE_DEVICE void load_tile(KeyTileBf16& tile, const DecodeArgs& a, const unsign
     const uint16_t* value_cache = static_cast<const uint16_t*>(a.value_cache);
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
-        const HalfRows rows = locate_half<ALIGNED16>(a, table_row, first + half * 16, end, kv_head, g, t);
+        const HalfRows rows = locate_half<ALIGNED16>(a, table_row, cache, first + half * 16, end, kv_head, g, t);
         const uint16_t* kp = key_cache + rows.key_row + 8 * g;
 #pragma unroll
         for (int c = 0; c < 4; ++c) tile.k[half][c] = *reinterpret_cast<const uint4*>(kp + 32 * c);
@@ -161,7 +192,7 @@ SINGE_DEVICE void load_tile(KeyTileBf16& tile, const DecodeArgs& a, const unsign
 }
 
 template <bool ALIGNED16>
-SINGE_DEVICE void load_tile(KeyTileFp8& tile, const DecodeArgs& a, const unsigned int* table_row,
+SINGE_DEVICE void load_tile(KeyTileFp8& tile, const DecodeArgs& a, const unsigned int* table_row, const EntryCache& cache,
                             unsigned int first, unsigned int end, unsigned int kv_head, unsigned int g,
                             unsigned int t) {
     tile.live = 0;
@@ -169,17 +200,30 @@ SINGE_DEVICE void load_tile(KeyTileFp8& tile, const DecodeArgs& a, const unsigne
     const uint8_t* value_cache = static_cast<const uint8_t*>(a.value_cache);
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
-        const HalfRows rows = locate_half<ALIGNED16>(a, table_row, first + half * 16, end, kv_head, g, t);
+        const HalfRows rows = locate_half<ALIGNED16>(a, table_row, cache, first + half * 16, end, kv_head, g, t);
         const uint8_t* kp = key_cache + rows.key_row + 32 * g;
         tile.k[half][0] = *reinterpret_cast<const uint4*>(kp);
         tile.k[half][1] = *reinterpret_cast<const uint4*>(kp + 16);
-        tile.key_scale[half] = a.key_scales[static_cast<size_t>(rows.key_block) * a.kv_heads + kv_head];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            tile.v[half][i] = *reinterpret_cast<const uint2*>(value_cache + rows.value_row[i] + 8 * t);
-            const size_t at = static_cast<size_t>(rows.value_block[i]) * a.kv_heads + kv_head;
-            tile.row_key_scale[half][i] = a.key_scales[at];
-            tile.row_value_scale[half][i] = a.value_scales[at];
+        for (int i = 0; i < 4; ++i) tile.v[half][i] = *reinterpret_cast<const uint2*>(value_cache + rows.value_row[i] + 8 * t);
+        if constexpr (ALIGNED16) {
+            // One block per half: its two scales come out of the entry cache.
+            const float ks = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, cache.key_scales), rows.cache_lane));
+            const float vs = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, cache.value_scales), rows.cache_lane));
+            tile.key_scale[half] = ks;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                tile.row_key_scale[half][i] = ks;
+                tile.row_value_scale[half][i] = vs;
+            }
+        } else {
+            tile.key_scale[half] = a.key_scales[static_cast<size_t>(rows.key_block) * a.kv_heads + kv_head];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const size_t at = static_cast<size_t>(rows.value_block[i]) * a.kv_heads + kv_head;
+                tile.row_key_scale[half][i] = a.key_scales[at];
+                tile.row_value_scale[half][i] = a.value_scales[at];
+            }
         }
         tile.live |= rows.live << (half * 4);
     }
@@ -246,6 +290,7 @@ struct GroupState {
 template <int GROUPS, bool ALIGNED16, bool FP8, bool EXACT>
 SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
     using Tile = typename std::conditional<FP8, KeyTileFp8, KeyTileBf16>::type;
+    constexpr int DEPTH = FP8 ? 3 : 2;  // an fp8 tile is half the bytes, so one more is kept in flight
     const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const unsigned int g = lane >> 4, t = lane & 15;
     const unsigned int reach = a.block_table_batch_stride * a.block_size;
@@ -343,83 +388,86 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
     };
 
     auto fold = [&](const Tile& tile) __attribute__((always_inline)) {
-        // Operands as bf16: K per (half, c), V per (half, i).
-        uint4 keys[2][4], values[2][4];
-        if constexpr (FP8) {
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                const float ks = EXACT ? tile.key_scale[half] : 1.0f;
-                keys[half][0] = widen_fp8x8(tile.k[half][0].x, tile.k[half][0].y, ks);
-                keys[half][1] = widen_fp8x8(tile.k[half][0].z, tile.k[half][0].w, ks);
-                keys[half][2] = widen_fp8x8(tile.k[half][1].x, tile.k[half][1].y, ks);
-                keys[half][3] = widen_fp8x8(tile.k[half][1].z, tile.k[half][1].w, ks);
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    values[half][i] = widen_fp8x8(tile.v[half][i].x, tile.v[half][i].y, EXACT ? tile.row_value_scale[half][i] : 1.0f);
-            }
-        } else {
-#pragma unroll
-            for (int half = 0; half < 2; ++half)
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    keys[half][c] = tile.k[half][c];
-                    values[half][c] = tile.v[half][c];
-                }
-        }
+        // Scores of every head group.  fp8 operands are widened right where they are used, so only
+        // one widened K chunk and one widened V row are alive at a time.
+        f32x4_t s0[GROUPS], s1[GROUPS];
 #pragma unroll
         for (int hg = 0; hg < GROUPS; ++hg) {
-            f32x4_t s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
+            s0[hg] = {0.0f, 0.0f, 0.0f, 0.0f};
+            s1[hg] = {0.0f, 0.0f, 0.0f, 0.0f};
+        }
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, keys[0][c]), q[hg][c], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, keys[1][c]), q[hg][c], s1, 0, 0, 0);
+        for (int c = 0; c < 4; ++c) {
+            uint4 first, second;
+            if constexpr (FP8) {
+                const uint4 a0 = tile.k[0][c >> 1], a1 = tile.k[1][c >> 1];
+                first = (c & 1) ? widen_fp8x8(a0.z, a0.w, EXACT ? tile.key_scale[0] : 1.0f)
+                                : widen_fp8x8(a0.x, a0.y, EXACT ? tile.key_scale[0] : 1.0f);
+                second = (c & 1) ? widen_fp8x8(a1.z, a1.w, EXACT ? tile.key_scale[1] : 1.0f)
+                                 : widen_fp8x8(a1.x, a1.y, EXACT ? tile.key_scale[1] : 1.0f);
+            } else {
+                first = tile.k[0][c];
+                second = tile.k[1][c];
             }
-            float p[8];
+#pragma unroll
+            for (int hg = 0; hg < GROUPS; ++hg) {
+                s0[hg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, first), q[hg][c], s0[hg], 0, 0, 0);
+                s1[hg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, second), q[hg][c], s1[hg], 0, 0, 0);
+            }
+        }
+        float p[GROUPS][8];
+#pragma unroll
+        for (int hg = 0; hg < GROUPS; ++hg) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                float first = s0[i] * a.scale_log2e, second = s1[i] * a.scale_log2e;
+                float first = s0[hg][i] * a.scale_log2e, second = s1[hg][i] * a.scale_log2e;
                 if constexpr (FP8 && !EXACT) {
                     first *= tile.row_key_scale[0][i];
                     second *= tile.row_key_scale[1][i];
                 }
-                p[i] = (tile.live >> i) & 1u ? first : -INFINITY;
-                p[4 + i] = (tile.live >> (4 + i)) & 1u ? second : -INFINITY;
+                p[hg][i] = (tile.live >> i) & 1u ? first : -INFINITY;
+                p[hg][4 + i] = (tile.live >> (4 + i)) & 1u ? second : -INFINITY;
             }
-            float largest = fmaxf(fmaxf(fmaxf(p[0], p[1]), fmaxf(p[2], p[3])), fmaxf(fmaxf(p[4], p[5]), fmaxf(p[6], p[7])));
+            float largest = fmaxf(fmaxf(fmaxf(p[hg][0], p[hg][1]), fmaxf(p[hg][2], p[hg][3])),
+                                  fmaxf(fmaxf(p[hg][4], p[hg][5]), fmaxf(p[hg][6], p[hg][7])));
             largest = fmaxf(across_groups_max(largest), state[hg].running_max);
             const float base = largest == -INFINITY ? 0.0f : largest;
             const float rescale = fast_exp2(state[hg].running_max - base);
             float total = 0.0f;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                p[i] = fast_exp2(p[i] - base);
-                total += p[i];
+                p[hg][i] = fast_exp2(p[hg][i] - base);
+                total += p[hg][i];
             }
             state[hg].running_sum = state[hg].running_sum * rescale + total;
             state[hg].running_max = largest;
-            f32x4_t low = state[hg].acc[0], high = state[hg].acc[1];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                low[r] *= rescale;
-                high[r] *= rescale;
+                state[hg].acc[0][r] *= rescale;
+                state[hg].acc[1][r] *= rescale;
             }
+        }
 #pragma unroll
-            for (int half = 0; half < 2; ++half)
+        for (int half = 0; half < 2; ++half)
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    float weight = p[half * 4 + i];
+            for (int i = 0; i < 4; ++i) {
+                uint4 row;
+                if constexpr (FP8)
+                    row = widen_fp8x8(tile.v[half][i].x, tile.v[half][i].y, EXACT ? tile.row_value_scale[half][i] : 1.0f);
+                else
+                    row = tile.v[half][i];
+#pragma unroll
+                for (int hg = 0; hg < GROUPS; ++hg) {
+                    float weight = p[hg][half * 4 + i];
                     if constexpr (FP8 && !EXACT) weight *= tile.row_value_scale[half][i];
                     const unsigned int both = bf16_twice(weight);
                     const uint2 hot = make_uint2(both & place0, both & place1);
-                    const uint4 row = values[half][i];
-                    low = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(i16x4_t, make_uint2(row.x, row.y)),
-                                                                   __builtin_bit_cast(i16x4_t, hot), low, 0, 0, 0);
-                    high = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(i16x4_t, make_uint2(row.z, row.w)),
-                                                                    __builtin_bit_cast(i16x4_t, hot), high, 0, 0, 0);
+                    state[hg].acc[0] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
+                        __builtin_bit_cast(i16x4_t, make_uint2(row.x, row.y)), __builtin_bit_cast(i16x4_t, hot), state[hg].acc[0], 0, 0, 0);
+                    state[hg].acc[1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
+                        __builtin_bit_cast(i16x4_t, make_uint2(row.z, row.w)), __builtin_bit_cast(i16x4_t, hot), state[hg].acc[1], 0, 0, 0);
                 }
-            state[hg].acc[0] = low;
-            state[hg].acc[1] = high;
-        }
+            }
     };
 
     // Writes the partial row of sequence b: O / sum per head, and the natural-log LSE.
@@ -444,38 +492,66 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
         }
     };
 
-    // Walk the range tile by tile, prefetching the next tile while the current one is folded.
-    auto seq_len = [&](unsigned int b) __attribute__((always_inline)) { return lengths[b]; };
-    unsigned int at = range_first;  // flat tile index of the tile being folded
-    unsigned int len = seq_len(seq);
-    Tile ping, pong;
-    load_query(seq);
-    load_tile<ALIGNED16>(ping, a, a.block_table + static_cast<size_t>(seq) * a.block_table_batch_stride,
-                         (at - prefix[seq]) * kTile, len, kv_head, g, t);
-    auto advance = [&](Tile& current, Tile& upcoming) __attribute__((always_inline)) {
-        // Returns false when `current` was the last tile of the range.
+    // Walk the range tile by tile with DEPTH tiles in registers: each buffer is refilled, with the tile
+    // DEPTH ahead, right after it has been folded, so DEPTH - 1 tiles are always on their way.
+    unsigned int at = range_first;                       // flat index of the tile being folded
+    unsigned int load_at = range_first, load_seq = seq;  // and of the next tile to fetch
+    EntryCache entries;
+    auto issue = [&](Tile& buffer) __attribute__((always_inline)) {
+        if (load_at >= range_end) return;
+        while (prefix[load_seq + 1] <= load_at) ++load_seq;  // skips empty sequences
+        const unsigned int first_key = (load_at - prefix[load_seq]) * kTile, end = lengths[load_seq];
+        if constexpr (ALIGNED16) {
+            // Entries this tile reads: those of its first key and of its last live key (a half past
+            // the end re-reads the last key's entry).
+            unsigned int low, high, slot;
+            split_key(a, first_key, low, slot);
+            split_key(a, (first_key + kTile <= end ? first_key + kTile : end) - 1, high, slot);
+            if (entries.sequence != load_seq || low < entries.first_entry || high >= entries.first_entry + 64)
+                fill_entries<FP8>(entries, a, load_seq, low, kv_head, lane);
+        }
+        load_tile<ALIGNED16>(buffer, a, a.block_table + static_cast<size_t>(load_seq) * a.block_table_batch_stride, entries,
+                             first_key, end, kv_head, g, t);
+        ++load_at;
+    };
+    auto consume = [&](const Tile& buffer) __attribute__((always_inline)) {
+        // Returns false when this was the last tile of the range.
+        fold(buffer);
         const unsigned int next_at = at + 1;
         const bool more = next_at < range_end;
-        unsigned int next_seq = seq, next_len = len;
-        if (more) {
-            while (prefix[next_seq + 1] <= next_at) ++next_seq;  // skips empty sequences
-            if (next_seq != seq) next_len = seq_len(next_seq);
-            load_tile<ALIGNED16>(upcoming, a, a.block_table + static_cast<size_t>(next_seq) * a.block_table_batch_stride,
-                                 (next_at - prefix[next_seq]) * kTile, next_len, kv_head, g, t);
-        }
-        fold(current);
+        unsigned int next_seq = seq;
+        if (more)
+            while (prefix[next_seq + 1] <= next_at) ++next_seq;
         if (!more || next_seq != seq) {
             flush(seq);
             if (more) load_query(next_seq);
         }
         at = next_at;
         seq = next_seq;
-        len = next_len;
         return more;
     };
-    while (true) {
-        if (!advance(ping, pong)) break;
-        if (!advance(pong, ping)) break;
+    load_query(seq);
+    Tile first, second;
+    issue(first);
+    issue(second);
+    if constexpr (DEPTH == 3) {
+        Tile third;
+        issue(third);
+        while (true) {
+            if (!consume(first)) break;
+            issue(first);
+            if (!consume(second)) break;
+            issue(second);
+            if (!consume(third)) break;
+            issue(third);
+        }
+    } else {
+        while (true) {
+            if (!consume(first)) break;
+            issue(first);
+            if (!consume(second)) break;
+            issue(second);
+        }
     }
 }
 
