@@ -209,6 +209,44 @@ SINGE_HIP_API int32_t singe_hip_fmha_prefill_lse_bf16(
     const uint16_t* value, size_t value_len,
     const SingeFmhaPrefillConfig* config);
 
+/* f32 forms for any head_dim up to 256 (fmha_prefill_f32 / fmha_prefill_lse_f32: fmha.rs:48-190).
+ * The f32 correctness anchor: dense causal [1, 8, 512, 64] attention in [batch, heads, len, dim]
+ * order is this call with batch stride heads*len*dim, head stride len*dim, sequence stride dim. */
+SINGE_HIP_API int32_t singe_hip_fmha_prefill_f32(
+    void* stream,
+    float* out, size_t out_len,
+    const float* query, size_t query_len,
+    const float* key, size_t key_len,
+    const float* value, size_t value_len,
+    const SingeFmhaPrefillConfig* config);
+SINGE_HIP_API int32_t singe_hip_fmha_prefill_lse_f32(
+    void* stream,
+    float* out, size_t out_len,
+    float* lse, size_t lse_len,
+    const float* query, size_t query_len,
+    const float* key, size_t key_len,
+    const float* value, size_t value_len,
+    const SingeFmhaPrefillConfig* config);
+
+/* Mirrors SoftcappedWindowAttentionConfig (mod.rs:292-296); Option<f32> soft_cap is the pair
+ * (has_soft_cap, soft_cap).  window_size 0 = no window, otherwise keys more than window_size away
+ * from the query on either side are hidden (cpu/attention.rs:1864-1869). */
+typedef struct SingeSoftcappedWindowAttentionConfig {
+    SingeFmhaPrefillConfig attention;
+    size_t window_size;
+    uint8_t has_soft_cap;
+    float soft_cap;
+} SingeSoftcappedWindowAttentionConfig;
+
+/* softcapped_window_attention_f32 (fmha.rs:245-290; CPU form cpu/attention.rs:1835-1925). */
+SINGE_HIP_API int32_t singe_hip_softcapped_window_attention_f32(
+    void* stream,
+    float* out, size_t out_len,
+    const float* query, size_t query_len,
+    const float* key, size_t key_len,
+    const float* value, size_t value_len,
+    const SingeSoftcappedWindowAttentionConfig* config);
+
 #ifdef __cplusplus
 }
 #endif

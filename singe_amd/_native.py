@@ -35,6 +35,11 @@ class FmhaPrefillConfigC(ctypes.Structure):
                                                                         ("causal", ctypes.c_uint8)]
 
 
+class SoftcappedWindowAttentionConfigC(ctypes.Structure):
+    _fields_ = [("attention", FmhaPrefillConfigC), ("window_size", c_size), ("has_soft_cap", ctypes.c_uint8),
+                ("soft_cap", ctypes.c_float)]
+
+
 _lib = None
 
 
@@ -93,6 +98,16 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_fmha_prefill_lse_bf16.argtypes = [c_void, c_void, c_size, c_void, c_size, c_void, c_size, c_void,
                                                        c_size, c_void, c_size, fmha]
     handle.singe_hip_fmha_prefill_lse_bf16.restype = i32
+    handle.singe_hip_fmha_prefill_f32.argtypes = [c_void, c_void, c_size, c_void, c_size, c_void, c_size, c_void,
+                                                  c_size, fmha]
+    handle.singe_hip_fmha_prefill_f32.restype = i32
+    handle.singe_hip_fmha_prefill_lse_f32.argtypes = [c_void, c_void, c_size, c_void, c_size, c_void, c_size, c_void,
+                                                      c_size, c_void, c_size, fmha]
+    handle.singe_hip_fmha_prefill_lse_f32.restype = i32
+    handle.singe_hip_softcapped_window_attention_f32.argtypes = [
+        c_void, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size,
+        ctypes.POINTER(SoftcappedWindowAttentionConfigC)]
+    handle.singe_hip_softcapped_window_attention_f32.restype = i32
     _lib = handle
     return handle
 

@@ -77,5 +77,11 @@ SINGE_DEVICE uint4 stream_load_16(const void* address) {
     return make_uint4(bits.x, bits.y, bits.z, bits.w);
 }
 
+typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+SINGE_DEVICE uint2 stream_load_8(const void* address) {
+    const u32x2_t bits = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t*>(address));
+    return make_uint2(bits.x, bits.y);
+}
+
 SINGE_DEVICE float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 SINGE_DEVICE float fast_log2(float x) { return __builtin_amdgcn_logf(x); }

@@ -47,12 +47,11 @@ int32_t ensure_reach(const char* name, size_t actual, size_t batch, size_t seque
     return ensure_len_at_least(name, actual, need);
 }
 
-int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, bool with_lse,
-                const uint16_t* query, size_t query_len, const uint16_t* key, size_t key_len, const uint16_t* value,
-                size_t value_len, const SingeFmhaPrefillConfig* config) {
-    if (config == nullptr) return fail(SINGE_HIP_NULL_POINTER, "config");
-    const SingeFmhaPrefillConfig& c = *config;
-    // FmhaPrefillConfig::validate_lengths / validate_output_lengths (mod.rs:1634-1756), in their order.
+// FmhaPrefillConfig::validate_lengths / validate_output_lengths (mod.rs:1634-1756), in their order,
+// then the null checks every DevicePointer implies.
+int32_t validate_call(const SingeFmhaPrefillConfig& c, const void* out, size_t out_len, const void* lse, size_t lse_len,
+                      bool with_lse, const void* query, size_t query_len, const void* key, size_t key_len,
+                      const void* value, size_t value_len) {
     if (int32_t status = validate_config(c)) return status;
     if (int32_t status = ensure_reach("query", query_len, c.batch, c.query_len, c.heads, c.head_dim, c.query_batch_stride,
                                       c.query_sequence_stride, c.query_head_stride)) return status;
@@ -72,6 +71,66 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
     const char* names[] = {"out", "query", "key", "value"};
     for (int i = 0; i < 4; ++i)
         if (pointers[i] == nullptr) return fail(SINGE_HIP_NULL_POINTER, names[i]);
+    if (!fits_i32(c.query_len) || !fits_i32(c.key_len) || !fits_i32(c.batch) || !fits_i32(c.heads))
+        return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "config");
+    return 0;
+}
+
+int32_t prefill_f32(void* stream, float* out, size_t out_len, float* lse, size_t lse_len, bool with_lse, const float* query,
+                    size_t query_len, const float* key, size_t key_len, const float* value, size_t value_len,
+                    const SingeFmhaPrefillConfig* config, size_t window_size, bool has_soft_cap, float soft_cap,
+                    const char* op) {
+    if (config == nullptr) return fail(SINGE_HIP_NULL_POINTER, "config");
+    const SingeFmhaPrefillConfig& c = *config;
+    if (int32_t status = validate_call(c, out, out_len, lse, lse_len, with_lse, query, query_len, key, key_len, value, value_len))
+        return status;
+    if (c.head_dim > 256) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, op, c.head_dim, 0);
+    if (!fits_i32(window_size)) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "window_size");
+    if (has_soft_cap && !(std::isfinite(soft_cap) && soft_cap != 0.0f)) return fail(SINGE_HIP_INVALID_LENGTH, "soft_cap");
+    PrefillF32Args args;
+    args.query = query;
+    args.key = key;
+    args.value = value;
+    args.out = out;
+    args.lse = with_lse ? lse : nullptr;
+    args.query_batch_stride = c.query_batch_stride;
+    args.query_sequence_stride = c.query_sequence_stride;
+    args.query_head_stride = c.query_head_stride;
+    args.key_batch_stride = c.key_batch_stride;
+    args.key_sequence_stride = c.key_sequence_stride;
+    args.key_head_stride = c.key_head_stride;
+    args.value_batch_stride = c.value_batch_stride;
+    args.value_sequence_stride = c.value_sequence_stride;
+    args.value_head_stride = c.value_head_stride;
+    args.output_batch_stride = c.output_batch_stride;
+    args.output_sequence_stride = c.output_sequence_stride;
+    args.output_head_stride = c.output_head_stride;
+    args.batch = static_cast<uint32_t>(c.batch);
+    args.query_len = static_cast<uint32_t>(c.query_len);
+    args.key_len = static_cast<uint32_t>(c.key_len);
+    args.heads = static_cast<uint32_t>(c.heads);
+    args.kv_heads = static_cast<uint32_t>(c.kv_heads);
+    args.head_dim = static_cast<uint32_t>(c.head_dim);
+    args.causal = c.causal ? 1u : 0u;
+    args.window_size = static_cast<uint32_t>(window_size);
+    args.has_soft_cap = has_soft_cap ? 1u : 0u;
+    args.soft_cap = soft_cap;
+    args.scale = c.scale;
+    const uint64_t rows = static_cast<uint64_t>(c.batch) * c.heads * c.query_len;
+    const uint64_t groups = (rows + 3) / 4;
+    if (groups > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
+    const KernelId kernel = c.head_dim <= 32 ? kPrefillF32D32 : c.head_dim <= 64 ? kPrefillF32D64
+                            : c.head_dim <= 128 ? kPrefillF32D128 : kPrefillF32D256;
+    return launch(kernel, static_cast<unsigned>(groups), 1, 1, 256, stream, args);
+}
+
+int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, bool with_lse,
+                const uint16_t* query, size_t query_len, const uint16_t* key, size_t key_len, const uint16_t* value,
+                size_t value_len, const SingeFmhaPrefillConfig* config) {
+    if (config == nullptr) return fail(SINGE_HIP_NULL_POINTER, "config");
+    const SingeFmhaPrefillConfig& c = *config;
+    if (int32_t status = validate_call(c, out, out_len, lse, lse_len, with_lse, query, query_len, key, key_len, value, value_len))
+        return status;
 
     // What the gfx950 kernel takes: head_dim 128 and rows it can fetch 16 bytes at a time.
     if (c.head_dim != 128) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, "fmha_prefill_bf16", c.head_dim, 0);
@@ -85,9 +144,6 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
                                    reinterpret_cast<uintptr_t>(key), reinterpret_cast<uintptr_t>(value)};
     for (uintptr_t address : addresses)
         if (address % 16 != 0) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "buffers must be 16-byte aligned");
-    if (!fits_i32(c.query_len) || !fits_i32(c.key_len) || !fits_i32(c.batch) || !fits_i32(c.heads))
-        return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "config");
-
     PrefillArgs args;
     args.query = query;
     args.key = key;
@@ -126,6 +182,29 @@ extern "C" {
 int32_t singe_hip_fmha_prefill_config_validate(const SingeFmhaPrefillConfig* config) {
     if (config == nullptr) return fail(SINGE_HIP_NULL_POINTER, "config");
     return validate_config(*config);
+}
+
+int32_t singe_hip_fmha_prefill_f32(void* stream, float* out, size_t out_len, const float* query, size_t query_len,
+                                   const float* key, size_t key_len, const float* value, size_t value_len,
+                                   const SingeFmhaPrefillConfig* config) {
+    return prefill_f32(stream, out, out_len, nullptr, 0, false, query, query_len, key, key_len, value, value_len, config, 0,
+                       false, 0.0f, "fmha_prefill_f32");
+}
+
+int32_t singe_hip_fmha_prefill_lse_f32(void* stream, float* out, size_t out_len, float* lse, size_t lse_len,
+                                       const float* query, size_t query_len, const float* key, size_t key_len,
+                                       const float* value, size_t value_len, const SingeFmhaPrefillConfig* config) {
+    return prefill_f32(stream, out, out_len, lse, lse_len, true, query, query_len, key, key_len, value, value_len, config, 0,
+                       false, 0.0f, "fmha_prefill_lse_f32");
+}
+
+int32_t singe_hip_softcapped_window_attention_f32(void* stream, float* out, size_t out_len, const float* query,
+                                                  size_t query_len, const float* key, size_t key_len, const float* value,
+                                                  size_t value_len, const SingeSoftcappedWindowAttentionConfig* config) {
+    if (config == nullptr) return fail(SINGE_HIP_NULL_POINTER, "config");
+    return prefill_f32(stream, out, out_len, nullptr, 0, false, query, query_len, key, key_len, value, value_len,
+                       &config->attention, config->window_size, config->has_soft_cap != 0, config->soft_cap,
+                       "softcapped_window_attention_f32");
 }
 
 int32_t singe_hip_fmha_prefill_bf16(void* stream, uint16_t* out, size_t out_len, const uint16_t* query, size_t query_len,

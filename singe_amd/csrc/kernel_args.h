@@ -62,3 +62,26 @@ struct PrefillArgs {
     uint32_t query_tiles;           // ceil(query_len / 128)
     float scale_log2e;
 };
+
+struct PrefillF32Args {
+    const float* query;             // [batch, query_len, heads, dim] through the strides below
+    const float* key;
+    const float* value;
+    float* out;
+    float* lse;                     // [batch, heads, query_len] natural log, or null
+    uint64_t query_batch_stride, query_sequence_stride, query_head_stride;
+    uint64_t key_batch_stride, key_sequence_stride, key_head_stride;
+    uint64_t value_batch_stride, value_sequence_stride, value_head_stride;
+    uint64_t output_batch_stride, output_sequence_stride, output_head_stride;
+    uint32_t batch;
+    uint32_t query_len;
+    uint32_t key_len;
+    uint32_t heads;
+    uint32_t kv_heads;
+    uint32_t head_dim;
+    uint32_t causal;
+    uint32_t window_size;           // 0 = no window
+    uint32_t has_soft_cap;
+    float soft_cap;
+    float scale;
+};

@@ -15,6 +15,7 @@ enum KernelId : int {
     kDecodeF8Relaxed = 8,
     kDecodeCombine = 12,
     kPrefillCausal, kPrefillFull,
+    kPrefillF32D32, kPrefillF32D64, kPrefillF32D128, kPrefillF32D256,
     kKernelCount
 };
 

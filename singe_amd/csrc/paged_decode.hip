@@ -205,7 +205,7 @@ SINGE_DEVICE void load_tile(KeyTileFp8& tile, const DecodeArgs& a, const unsigne
         tile.k[half][0] = *reinterpret_cast<const uint4*>(kp);
         tile.k[half][1] = *reinterpret_cast<const uint4*>(kp + 16);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) tile.v[half][i] = *reinterpret_cast<const uint2*>(value_cache + rows.value_row[i] + 8 * t);
+        for (int i = 0; i < 4; ++i) tile.v[half][i] = stream_load_8(value_cache + rows.value_row[i] + 8 * t);
         if constexpr (ALIGNED16) {
             // One block per half: its two scales come out of the entry cache.
             const float ks = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, cache.key_scales), rows.cache_lane));

@@ -2,3 +2,4 @@
 // singe_attention_gfx950.hsaco, which the C-ABI library loads with hipModuleLoadData.
 #include "paged_decode.hip"
 #include "fmha_prefill.hip"
+#include "fmha_prefill_f32.hip"

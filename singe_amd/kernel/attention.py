@@ -234,3 +234,59 @@ def fmha_prefill_lse_bf16(stream, out: torch.Tensor, lse: torch.Tensor, query: t
         _stream_handle(stream), _ptr(out), out.numel(), _ptr(lse), lse.numel(), _ptr(query), query.numel(),
         _ptr(key), key.numel(), _ptr(value), value.numel(), ctypes.byref(c))
     _native.check(status, "fmha_prefill_lse_bf16")
+
+
+def fmha_prefill_f32(stream, out: torch.Tensor, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                     config: FmhaPrefillConfig) -> None:
+    """fmha_prefill_f32 (fmha.rs:146-190): any head_dim up to 256, any strides."""
+    for tensor, name in ((out, "out"), (query, "query"), (key, "key"), (value, "value")):
+        _require(tensor, torch.float32, name)
+    c = config._c()
+    status = _native.lib().singe_hip_fmha_prefill_f32(
+        _stream_handle(stream), _ptr(out), out.numel(), _ptr(query), query.numel(), _ptr(key), key.numel(),
+        _ptr(value), value.numel(), ctypes.byref(c))
+    _native.check(status, "fmha_prefill_f32")
+
+
+def fmha_prefill_lse_f32(stream, out: torch.Tensor, lse: torch.Tensor, query: torch.Tensor, key: torch.Tensor,
+                         value: torch.Tensor, config: FmhaPrefillConfig) -> None:
+    """fmha_prefill_lse_f32 (fmha.rs:48-95)."""
+    for tensor, name in ((out, "out"), (lse, "lse"), (query, "query"), (key, "key"), (value, "value")):
+        _require(tensor, torch.float32, name)
+    c = config._c()
+    status = _native.lib().singe_hip_fmha_prefill_lse_f32(
+        _stream_handle(stream), _ptr(out), out.numel(), _ptr(lse), lse.numel(), _ptr(query), query.numel(),
+        _ptr(key), key.numel(), _ptr(value), value.numel(), ctypes.byref(c))
+    _native.check(status, "fmha_prefill_lse_f32")
+
+
+@dataclass(frozen=True)
+class SoftcappedWindowAttentionConfig:
+    """mod.rs:292-296: dense attention with an optional symmetric window and tanh soft cap."""
+    attention: FmhaPrefillConfig
+    window_size: int = 0
+    soft_cap: float | None = None
+
+
+def softcapped_window_attention_f32(stream, out: torch.Tensor, query: torch.Tensor, key: torch.Tensor,
+                                    value: torch.Tensor, config: SoftcappedWindowAttentionConfig) -> None:
+    """softcapped_window_attention_f32 (fmha.rs:245-290)."""
+    for tensor, name in ((out, "out"), (query, "query"), (key, "key"), (value, "value")):
+        _require(tensor, torch.float32, name)
+    c = _native.SoftcappedWindowAttentionConfigC(config.attention._c(), config.window_size,
+                                                 1 if config.soft_cap is not None else 0,
+                                                 config.soft_cap if config.soft_cap is not None else 0.0)
+    status = _native.lib().singe_hip_softcapped_window_attention_f32(
+        _stream_handle(stream), _ptr(out), out.numel(), _ptr(query), query.numel(), _ptr(key), key.numel(),
+        _ptr(value), value.numel(), ctypes.byref(c))
+    _native.check(status, "softcapped_window_attention_f32")
+
+
+def bhsd_config(batch, heads, kv_heads, query_len, key_len, head_dim, scale, causal) -> FmhaPrefillConfig:
+    """FmhaPrefillConfig strides for tensors stored [batch, heads, len, dim] (the order of the CPU
+    softcapped_window_attention_f32 and of singe's scaled_dot_product_attention)."""
+    return FmhaPrefillConfig(batch, query_len, key_len, heads, kv_heads, head_dim,
+                             heads * query_len * head_dim, kv_heads * key_len * head_dim, kv_heads * key_len * head_dim,
+                             heads * query_len * head_dim, head_dim, head_dim, head_dim, head_dim,
+                             query_len * head_dim, key_len * head_dim, key_len * head_dim, query_len * head_dim,
+                             scale, causal)
