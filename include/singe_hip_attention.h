@@ -247,6 +247,56 @@ SINGE_HIP_API int32_t singe_hip_softcapped_window_attention_f32(
     const float* value, size_t value_len,
     const SingeSoftcappedWindowAttentionConfig* config);
 
+/* ---- singe surface: paged attention in FlashInfer form ---------------------------------------------
+ * Operation::PagedAttention (singe/src/tensor/neural.rs:409-457): ragged queries [tokens, heads, dim]
+ * over caches [cache_pages, page_size, kv_heads, dim]; sequence b holds queries
+ * query_offsets[b] .. query_offsets[b+1] and the keys of pages pages[page_offsets[b] .. page_offsets[b+1]],
+ * all full but the last, which holds last_page_lengths[b].  Queries are a sequence's last tokens
+ * (bottom-right causal).  The extents the reference bakes into the generated source are runtime values
+ * here; the attributes are ScaledDotProductAttentionAttributes
+ * (singe/src/backend/registry/attributes/mod.rs:288-303) with each Option as a (has_, value) pair. */
+#define SINGE_HIP_INDEX_I32 0
+#define SINGE_HIP_INDEX_I64 1
+typedef struct SingePagedAttentionProblem {
+    int64_t tokens;        /* query_rows.shape[0] */
+    int64_t heads;
+    int64_t kv_heads;
+    int64_t head_dim;
+    int64_t page_size;     /* cache.shape[1] */
+    int64_t sequences;     /* last_page_lengths.len */
+    int64_t cache_pages;   /* cache.shape[0] */
+    int64_t page_table;    /* pages.len */
+    int32_t index_type;    /* SINGE_HIP_INDEX_I32 or _I64, for all four index operands */
+    uint8_t causal;
+    uint8_t has_scale;     /* Option<f32> scale, default 1 / sqrt(head_dim) */
+    uint8_t has_window;    /* Option<i64> window: key j is hidden from position i when j + window <= i */
+    uint8_t has_softcap;   /* Option<f32> softcap: softcap * tanh(score / softcap) on the scaled scores */
+    float scale;
+    float softcap;
+    int64_t window;
+} SingePagedAttentionProblem;
+
+/* The kernel artifact "singe_paged_attention" (kernel_plan/source/paged_attention.rs:544-868), with
+ * its ABI order: inputs, outputs, status (paged_attention.rs:687-715).  output [tokens, heads, dim]
+ * bf16; lse [tokens, heads] f32, base two, -inf for a row that sees no key (may be null: the fused
+ * variants do not read it).  status: device u32, zeroed by the caller, set to 1
+ * (STATUS_INDEX_OUT_OF_BOUNDS: singe/src/backend/kernel_lowering/mod.rs:40-61) by the first paging
+ * value found outside its buffers; may be null (it is while a stream is being captured:
+ * kernel_plan/mod.rs:176-197), and nothing is ever read through a bad value. */
+SINGE_HIP_API int32_t singe_hip_paged_attention_bf16(
+    void* stream,
+    const uint16_t* query_rows,
+    const uint16_t* key_cache,
+    const uint16_t* value_cache,
+    const void* query_offsets,
+    const void* page_offsets,
+    const void* pages,
+    const void* last_page_lengths,
+    uint16_t* output,
+    float* lse,
+    uint32_t* status,
+    const SingePagedAttentionProblem* problem);
+
 #ifdef __cplusplus
 }
 #endif

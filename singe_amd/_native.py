@@ -40,6 +40,15 @@ class SoftcappedWindowAttentionConfigC(ctypes.Structure):
                 ("soft_cap", ctypes.c_float)]
 
 
+class PagedAttentionProblemC(ctypes.Structure):
+    _fields_ = [("tokens", ctypes.c_int64), ("heads", ctypes.c_int64), ("kv_heads", ctypes.c_int64),
+                ("head_dim", ctypes.c_int64), ("page_size", ctypes.c_int64), ("sequences", ctypes.c_int64),
+                ("cache_pages", ctypes.c_int64), ("page_table", ctypes.c_int64), ("index_type", ctypes.c_int32),
+                ("causal", ctypes.c_uint8), ("has_scale", ctypes.c_uint8), ("has_window", ctypes.c_uint8),
+                ("has_softcap", ctypes.c_uint8), ("scale", ctypes.c_float), ("softcap", ctypes.c_float),
+                ("window", ctypes.c_int64)]
+
+
 _lib = None
 
 
@@ -108,6 +117,8 @@ def lib() -> ctypes.CDLL:
         c_void, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size,
         ctypes.POINTER(SoftcappedWindowAttentionConfigC)]
     handle.singe_hip_softcapped_window_attention_f32.restype = i32
+    handle.singe_hip_paged_attention_bf16.argtypes = [c_void] * 11 + [ctypes.POINTER(PagedAttentionProblemC)]
+    handle.singe_hip_paged_attention_bf16.restype = i32
     _lib = handle
     return handle
 

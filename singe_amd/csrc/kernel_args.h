@@ -85,3 +85,29 @@ struct PrefillF32Args {
     float soft_cap;
     float scale;
 };
+
+struct PagedAttentionArgs {
+    const uint16_t* query_rows;     // [tokens, heads, 128] bf16
+    const uint16_t* key_cache;      // [cache_pages, page_size, kv_heads, 128] bf16
+    const uint16_t* value_cache;
+    const void* query_offsets;      // [sequences + 1] i32 or i64
+    const void* page_offsets;       // [sequences + 1]
+    const void* pages;              // [page_table]
+    const void* last_page_lengths;  // [sequences]
+    uint16_t* output;               // [tokens, heads, 128] bf16
+    float* lse;                     // [tokens, heads] base two, or null
+    uint32_t* status;               // first writer wins, may be null
+    int64_t window;                 // keys a query sees before itself, itself included; -1 = no window
+    uint32_t tokens;
+    uint32_t heads;
+    uint32_t kv_heads;
+    uint32_t page_size;
+    uint32_t sequences;
+    uint32_t cache_pages;
+    uint32_t page_table;
+    uint32_t row_tiles;             // ceil(groups * tokens / 128): row tiles per (sequence, kv head)
+    uint32_t causal;
+    float scale_log2e;              // scale * log2(e)
+    float softcap_scale;            // scale / cap
+    float softcap_log2e;            // cap * log2(e)
+};

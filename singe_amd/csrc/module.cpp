@@ -22,6 +22,8 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_decode_combine_bf16",
     "singe_fmha_prefill_bf16_d128_causal", "singe_fmha_prefill_bf16_d128_full",
     "singe_fmha_prefill_f32_d32", "singe_fmha_prefill_f32_d64", "singe_fmha_prefill_f32_d128", "singe_fmha_prefill_f32_d256",
+    "singe_paged_attention_bf16_d128_i32", "singe_paged_attention_bf16_d128_i64",
+    "singe_paged_attention_bf16_d128_softcap_i32", "singe_paged_attention_bf16_d128_softcap_i64",
 };
 
 namespace {

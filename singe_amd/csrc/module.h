@@ -16,6 +16,7 @@ enum KernelId : int {
     kDecodeCombine = 12,
     kPrefillCausal, kPrefillFull,
     kPrefillF32D32, kPrefillF32D64, kPrefillF32D128, kPrefillF32D256,
+    kPagedAttentionI32, kPagedAttentionI64, kPagedAttentionSoftcapI32, kPagedAttentionSoftcapI64,
     kKernelCount
 };
 

@@ -1,0 +1,77 @@
+// Host side of the paged attention op: the shape rules of spec::paged_attention_problem
+// (singe/src/backend/spec/neural/attention.rs:337-367, 408-438) and the launch, with the kernel's
+// arguments in the order of the reference artifact's ABI
+// (singe/src/backend/cuda/kernel_plan/source/paged_attention.rs:687-715).
+#include <cmath>
+
+#include "kernel_args.h"
+#include "module.h"
+#include "singe_hip_attention.h"
+#include "validate.h"
+
+using namespace singe_hip;
+
+extern "C" int32_t singe_hip_paged_attention_bf16(void* stream, const uint16_t* query_rows, const uint16_t* key_cache,
+                                                  const uint16_t* value_cache, const void* query_offsets,
+                                                  const void* page_offsets, const void* pages,
+                                                  const void* last_page_lengths, uint16_t* output, float* lse,
+                                                  uint32_t* status, const SingePagedAttentionProblem* problem) {
+    if (problem == nullptr) return fail(SINGE_HIP_NULL_POINTER, "problem");
+    const SingePagedAttentionProblem& p = *problem;
+    // paged_attention_problem: key_dim == head_dim (one field here), kv_heads > 0 dividing heads, page_size > 0.
+    if (p.tokens < 0 || p.heads <= 0 || p.kv_heads <= 0 || p.heads % p.kv_heads != 0 || p.page_size <= 0 || p.head_dim <= 0 ||
+        p.sequences < 0 || p.cache_pages < 0 || p.page_table < 0)
+        return fail(SINGE_HIP_INVALID_ARGUMENT, "heads, head dimension, or page size");
+    if (p.index_type != SINGE_HIP_INDEX_I32 && p.index_type != SINGE_HIP_INDEX_I64)
+        return fail(SINGE_HIP_INVALID_ARGUMENT, "index type");
+    if (p.has_scale && !std::isfinite(p.scale)) return fail(SINGE_HIP_INVALID_ARGUMENT, "scale");
+    if (p.has_softcap && !(std::isfinite(p.softcap) && p.softcap != 0.0f)) return fail(SINGE_HIP_INVALID_ARGUMENT, "softcap");
+    if (p.has_window && p.window < 0) return fail(SINGE_HIP_INVALID_ARGUMENT, "window");
+    const int64_t extents[] = {p.tokens, p.heads, p.kv_heads, p.page_size, p.sequences, p.cache_pages, p.page_table};
+    for (int64_t extent : extents)
+        if (!fits_i32(static_cast<uint64_t>(extent))) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "problem");
+    // The tensor-core kernel takes head dimensions that are multiples of 16 up to 128
+    // (paged_attention.rs:586-592); this build covers 128, the general kernel is not part of it.
+    if (p.head_dim != 128) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, "paged_attention", static_cast<uint64_t>(p.head_dim), 0);
+    if (p.tokens == 0 || p.sequences == 0) return 0;  // nothing to attend
+    const void* pointers[] = {query_rows, key_cache, value_cache, query_offsets, page_offsets, last_page_lengths, output};
+    const char* names[] = {"query_rows", "key_cache", "value_cache", "query_offsets", "page_offsets", "last_page_lengths", "output"};
+    for (int i = 0; i < 7; ++i)
+        if (pointers[i] == nullptr) return fail(SINGE_HIP_NULL_POINTER, names[i]);
+    if (pages == nullptr && p.page_table > 0) return fail(SINGE_HIP_NULL_POINTER, "pages");
+
+    const uint64_t groups = static_cast<uint64_t>(p.heads / p.kv_heads);
+    PagedAttentionArgs args;
+    args.query_rows = query_rows;
+    args.key_cache = key_cache;
+    args.value_cache = value_cache;
+    args.query_offsets = query_offsets;
+    args.page_offsets = page_offsets;
+    args.pages = pages;
+    args.last_page_lengths = last_page_lengths;
+    args.output = output;
+    args.lse = lse;
+    args.status = status;
+    args.window = p.has_window ? p.window : -1;
+    args.tokens = static_cast<uint32_t>(p.tokens);
+    args.heads = static_cast<uint32_t>(p.heads);
+    args.kv_heads = static_cast<uint32_t>(p.kv_heads);
+    args.page_size = static_cast<uint32_t>(p.page_size);
+    args.sequences = static_cast<uint32_t>(p.sequences);
+    args.cache_pages = static_cast<uint32_t>(p.cache_pages);
+    args.page_table = static_cast<uint32_t>(p.page_table);
+    args.row_tiles = static_cast<uint32_t>((groups * static_cast<uint64_t>(p.tokens) + 127) / 128);
+    args.causal = p.causal ? 1u : 0u;
+    const float scale = p.has_scale ? p.scale : 1.0f / std::sqrt(static_cast<float>(p.head_dim));
+    constexpr float kLog2e = 1.4426950408889634074f;
+    args.scale_log2e = scale * kLog2e;
+    args.softcap_scale = p.has_softcap ? scale / p.softcap : 0.0f;
+    args.softcap_log2e = p.has_softcap ? p.softcap * kLog2e : 0.0f;
+    const uint64_t units = (static_cast<uint64_t>(p.sequences) * p.kv_heads + 7) / 8 * 8;
+    const uint64_t blocks = units * args.row_tiles;
+    if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
+    const bool wide = p.index_type == SINGE_HIP_INDEX_I64;
+    const KernelId kernel = p.has_softcap ? (wide ? kPagedAttentionSoftcapI64 : kPagedAttentionSoftcapI32)
+                                          : (wide ? kPagedAttentionI64 : kPagedAttentionI32);
+    return launch(kernel, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+}

@@ -3,3 +3,4 @@
 #include "paged_decode.hip"
 #include "fmha_prefill.hip"
 #include "fmha_prefill_f32.hip"
+#include "paged_attention.hip"

@@ -1,0 +1,133 @@
+"""The singe paged-attention op (FlashInfer form, bottom-right causal) on the GPU against the CPU oracle
+(attend_paged restated), through the C ABI.  bf16 outputs within max-abs 2e-2 / mean-abs 2e-3, base-two
+LSE within 2e-3; the paging error contract bit for bit."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from singe_amd import error, neural
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS, MEAN_ABS, LSE_ABS = 2e-2, 2e-3, 2e-3
+
+
+def layout(sequences, page_size, extra_pages=3):
+    query_offsets, page_offsets, last, needed = [0], [0], [], 0
+    for queries, keys in sequences:
+        query_offsets.append(query_offsets[-1] + queries)
+        pages = (keys + page_size - 1) // page_size
+        needed += pages
+        page_offsets.append(needed)
+        last.append(0 if keys == 0 else keys - (pages - 1) * page_size)
+    page_count = needed + extra_pages
+    table = [(p * 7 + 2) % page_count for p in range(needed)] if np.gcd(7, page_count) == 1 else \
+        list(np.random.default_rng(page_count).permutation(page_count)[:needed])
+    return query_offsets, page_offsets, table, last, page_count
+
+
+def run_case(sequences, heads, kv_heads, page_size, options, index_dtype=torch.int32, seed=0, dim=128):
+    query_offsets, page_offsets, table, last, page_count = layout(sequences, page_size)
+    tokens = query_offsets[-1]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+    q = torch.randn((tokens, heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
+    kc = torch.randn((page_count, page_size, kv_heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
+    vc = torch.randn((page_count, page_size, kv_heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
+    index = lambda values: torch.tensor(values, dtype=index_dtype, device="cuda")
+    paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
+    out, lse = neural.paged_attention(q, kc, vc, paging, options)
+    torch.cuda.synchronize()
+    status, want, want_lse = oracle.paged_attention_f32(
+        q.float().cpu().numpy(), kc.float().cpu().numpy(), vc.float().cpu().numpy(), query_offsets, page_offsets, table,
+        last, scale=options.scale, causal=options.causal, window=options.window, softcap=options.softcap, threads=8)
+    assert status == 0
+    got, got_lse = out.float().cpu().numpy(), lse.cpu().numpy()
+    assert np.isfinite(got).all()
+    gap = np.abs(got - want)
+    assert gap.max() <= MAX_ABS, gap.max()
+    assert gap.mean() <= MEAN_ABS, gap.mean()
+    empty = np.isneginf(want_lse)
+    assert np.array_equal(np.isneginf(got_lse), empty)
+    assert not got[empty].any()
+    assert np.abs(got_lse[~empty] - want_lse[~empty]).max(initial=0.0) <= LSE_ABS
+
+
+OPTIONS = [neural.AttentionOptions(), neural.AttentionOptions(causal=True),
+           neural.AttentionOptions(causal=True, window=16, softcap=30.0),
+           neural.AttentionOptions(causal=True, window=100), neural.AttentionOptions(scale=0.05, softcap=5.0)]
+
+
+@pytest.mark.parametrize("options", OPTIONS)
+@pytest.mark.parametrize("heads,kv_heads,page_size", [(8, 2, 1), (8, 1, 16), (4, 4, 7), (64, 8, 16)])
+def test_ragged_sequences_match_oracle(heads, kv_heads, page_size, options):
+    # decode, full prefill, chunked prefill, no keys (kernel_plan/source/tests.rs:830-889), plus more
+    # queries than keys, where the CPU path's saturating position applies
+    sequences = [(1, 150), (70, 70), (20, 90), (3, 0), (9, 4), (130, 300)]
+    run_case(sequences, heads, kv_heads, page_size, options, seed=heads + page_size)
+
+
+def test_int64_indices_and_chunked_prefill_shape():
+    # one sequence of the chunked-prefill shape: 512 new queries over a cached prefix, 64 query / 8 kv heads
+    run_case([(512, 1536 + 512), (512, 1024 + 512)], 64, 8, 16, neural.AttentionOptions(causal=True),
+             index_dtype=torch.int64, seed=4)
+
+
+TOKENS, HEADS, DIM, SLOTS, PAGES = 2, 2, 128, 4, 2
+VALID = dict(query_offsets=[0, 2], page_offsets=[0, 1], pages=[0], last_page_lengths=[2])
+INVALID = [dict(query_offsets=[0, 3]), dict(query_offsets=[-1, 2]), dict(query_offsets=[2, 0]), dict(page_offsets=[0, 2]),
+           dict(page_offsets=[-1, 1]), dict(pages=[PAGES]), dict(pages=[-1]), dict(last_page_lengths=[SLOTS + 1]),
+           dict(last_page_lengths=[-1])]
+
+
+def attend(paging_values, dtype=torch.int64):
+    # singe/tests/nn/paged_attention.rs:96-127 (head_dim 128 here: the width this build's kernel takes)
+    q = torch.zeros((TOKENS, HEADS, DIM), device="cuda", dtype=torch.bfloat16)
+    cache = torch.zeros((PAGES, SLOTS, HEADS, DIM), device="cuda", dtype=torch.bfloat16)
+    values = {**VALID, **paging_values}
+    index = lambda v: torch.tensor(v, dtype=dtype, device="cuda")
+    paging = neural.Paging(index(values["query_offsets"]), index(values["page_offsets"]), index(values["pages"]),
+                           index(values["last_page_lengths"]))
+    return neural.paged_attention(q, cache, cache, paging, neural.AttentionOptions(causal=True))
+
+
+@pytest.mark.parametrize("dtype", [torch.int32, torch.int64])
+def test_paging_values_outside_their_buffers_are_refused(dtype):
+    # singe/tests/nn/paged_attention.rs:24-73, 141-186
+    attend({}, dtype)
+    for bad in INVALID:
+        with pytest.raises(error.IndexOutOfBounds):
+            attend(bad, dtype)
+        attend({}, dtype)  # the next valid launch succeeds
+    attend(dict(last_page_lengths=[SLOTS]), dtype)
+    attend(dict(query_offsets=[0, 0], page_offsets=[0, 0], pages=[PAGES + 7], last_page_lengths=[-1]), dtype)
+    for bad in INVALID:
+        assert oracle.check_paged_values(**{**VALID, **bad}, tokens=TOKENS, cache_pages=PAGES, page_size=SLOTS) == 1
+
+
+def test_paged_equals_dense_prefill():
+    # paged == dense invariant (singe/tests/nn/cross_attention.rs:120-198): one sequence whose queries
+    # are all of its tokens is plain causal attention over the gathered keys.
+    from singe_amd.kernel import attention as A
+
+    length, heads, kv_heads, page_size, dim = 300, 8, 2, 16, 128
+    query_offsets, page_offsets, table, last, page_count = layout([(length, length)], page_size)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(12)
+    q = torch.randn((length, heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
+    kc = torch.randn((page_count, page_size, kv_heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
+    vc = torch.randn((page_count, page_size, kv_heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
+    index = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
+    out, lse = neural.paged_attention(q, kc, vc, neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last)),
+                                      neural.AttentionOptions(causal=True))
+    rows = torch.tensor([table[k // page_size] * page_size + k % page_size for k in range(length)], device="cuda")
+    k_dense = kc.view(-1, kv_heads, dim)[rows].unsqueeze(0).contiguous()
+    v_dense = vc.view(-1, kv_heads, dim)[rows].unsqueeze(0).contiguous()
+    dense = torch.empty((1, length, heads, dim), device="cuda", dtype=torch.bfloat16)
+    dense_lse = torch.empty((1, heads, length), device="cuda")
+    A.fmha_prefill_lse_bf16(None, dense, dense_lse, q.unsqueeze(0).contiguous(), k_dense, v_dense,
+                            A.FmhaPrefillConfig.contiguous(1, length, length, heads, kv_heads, dim, dim ** -0.5, True))
+    torch.cuda.synchronize()
+    assert (out.float() - dense[0].float()).abs().max().item() <= 2 ** -6
+    assert (lse - dense_lse[0].T / np.log(2.0)).abs().max().item() <= 2e-3
