@@ -1,0 +1,121 @@
+"""No-GPU checks of the C-ABI library and the host layer: the library loads, exports every symbol the
+header declares, and every validation that the reference performs before a launch returns the same
+error without touching a device."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from singe_amd import _native, error
+from singe_amd.kernel import attention as A
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "singe_hip_attention.h")).read()
+    return sorted(set(re.findall(r"SINGE_HIP_API[^;(]*?\b(singe_hip_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _native.lib()
+    names = declared_symbols()
+    assert len(names) >= 20
+    for name in names:
+        assert hasattr(lib, name), name
+
+
+def test_code_object_is_built_and_names_every_kernel():
+    assert os.path.exists(_native.CODE_OBJECT_PATH)
+    image = open(_native.CODE_OBJECT_PATH, "rb").read()
+    for kernel in (b"singe_paged_decode_bf16_d128_g1_b16", b"singe_paged_decode_f8kv_d128_g2_b16",
+                   b"singe_paged_decode_combine_bf16", b"singe_fmha_prefill_bf16_d128_causal",
+                   b"singe_fmha_prefill_f32_d64", b"singe_paged_attention_bf16_d128_i64"):
+        assert kernel in image, kernel
+
+
+def test_status_strings():
+    lib = _native.lib()
+    assert lib.singe_hip_status_string(0) == b"ok"
+    assert lib.singe_hip_status_string(1) == b"invalid length"
+    assert lib.singe_hip_status_string(2) == b"length too short"
+
+
+GOOD = dict(batch=2, heads=8, kv_heads=2, head_dim=128, block_size=16, physical_blocks=8,
+            block_table_batch_stride=4, scale=0.1)
+
+
+def decode_status(config, lens=None, pointers=None):
+    lens = lens or dict(out=2 * 8 * 128, query=2 * 8 * 128, key=8 * 16 * 2 * 128, value=8 * 16 * 2 * 128, seq=2, table=8)
+    fake = 0x1000
+    p = pointers or {}
+    return _native.lib().singe_hip_paged_kv_decode_attention_bf16(
+        None, p.get("out", fake), lens["out"], p.get("query", fake), lens["query"], p.get("key", fake), lens["key"],
+        p.get("value", fake), lens["value"], p.get("seq", fake), lens["seq"], p.get("table", fake), lens["table"],
+        p.get("workspace", fake), 1 << 30, ctypes.byref(config))
+
+
+def test_decode_validation_order_and_codes():
+    # validate_paged_kv_decode_attention_config, then validate_lengths (mod.rs:711-743, 2963-2985)
+    for bad in (dict(batch=0), dict(heads=7), dict(scale=float("inf")), dict(physical_blocks=0)):
+        with pytest.raises(error.InvalidLength):
+            A.PagedKvDecodeAttentionConfig.contiguous(**{**GOOD, **bad})
+        c = A.PagedKvDecodeAttentionConfig(**{**GOOD, **bad})._c()
+        assert decode_status(c) == 1
+    with pytest.raises(error.LengthExceedsI32):
+        A.PagedKvDecodeAttentionConfig.contiguous(**{**GOOD, "batch": 2**31})
+    assert decode_status(A.PagedKvDecodeAttentionConfig(**{**GOOD, "batch": 2**31})._c()) == 3
+    c = A.PagedKvDecodeAttentionConfig.contiguous(**GOOD)._c()
+    full = dict(out=2 * 8 * 128, query=2 * 8 * 128, key=8 * 16 * 2 * 128, value=8 * 16 * 2 * 128, seq=2, table=8)
+    for name in full:
+        status = decode_status(c, {**full, name: full[name] - 1})
+        assert status == 2, name
+        detail = _native.ErrorDetail()
+        _native.lib().singe_hip_last_error(ctypes.byref(detail))
+        assert detail.minimum == full[name] and detail.actual == full[name] - 1
+    assert decode_status(c, pointers=dict(query=None)) == 6
+    assert decode_status(A.PagedKvDecodeAttentionConfig(**{**GOOD, "head_dim": 64})._c()) == 5
+    with pytest.raises(error.UnsupportedWidth):
+        _native.check(5, "paged_kv_decode_attention_bf16")
+
+
+def test_decode_workspace_query_needs_no_device():
+    c = A.PagedKvDecodeAttentionConfig.contiguous(**GOOD)
+    assert c.workspace_bytes() > 0
+    assert _native.lib().singe_hip_paged_kv_decode_attention_workspace_bytes(None) == 0
+
+
+def test_fmha_config_validation():
+    good = A.FmhaPrefillConfig.contiguous(1, 64, 64, 4, 2, 128, 0.1, True)
+    lib = _native.lib()
+    assert lib.singe_hip_fmha_prefill_config_validate(ctypes.byref(good._c())) == 0
+    from dataclasses import replace
+    for bad in (replace(good, key_len=0), replace(good, kv_heads=3), replace(good, scale=float("nan")),
+                replace(good, query_head_stride=0)):
+        assert lib.singe_hip_fmha_prefill_config_validate(ctypes.byref(bad._c())) == 1
+    # validate_lengths: a buffer shorter than the strides can reach
+    fake = 0x1000
+    need = 64 * 4 * 128
+    status = lib.singe_hip_fmha_prefill_bf16(None, fake, need, fake, need - 1, fake, 64 * 2 * 128, fake, 64 * 2 * 128,
+                                             ctypes.byref(good._c()))
+    assert status == 2
+    assert lib.singe_hip_fmha_prefill_bf16(None, fake, need, fake, need, None, 64 * 2 * 128, fake, 64 * 2 * 128,
+                                           ctypes.byref(good._c())) == 6
+
+
+def test_paged_attention_problem_validation():
+    lib = _native.lib()
+    fake = 0x1000
+    def call(**changes):
+        fields = dict(tokens=2, heads=2, kv_heads=2, head_dim=128, page_size=4, sequences=1, cache_pages=2, page_table=1,
+                      index_type=1, causal=1, has_scale=0, has_window=0, has_softcap=0, scale=0.0, softcap=0.0, window=0)
+        fields.update(changes)
+        problem = _native.PagedAttentionProblemC(*fields.values())
+        return lib.singe_hip_paged_attention_bf16(None, *([fake] * 10), ctypes.byref(problem))
+    assert call(kv_heads=0) == 9
+    assert call(heads=3) == 9
+    assert call(page_size=0) == 9
+    assert call(index_type=7) == 9
+    assert call(head_dim=64) == 5
+    assert call(tokens=0) == 0  # nothing to attend, nothing launched
