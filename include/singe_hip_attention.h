@@ -158,6 +158,45 @@ SINGE_HIP_API int32_t singe_hip_relaxed_numerics(void);
 SINGE_HIP_API void singe_hip_set_decode_workers(uint32_t workers);
 SINGE_HIP_API uint32_t singe_hip_decode_workers(const SingePagedKvDecodeAttentionConfig* config);
 
+/* ---- singe-kernel surface: paged prefill ----------------------------------------------------------
+ * Mirrors PagedKvPrefillAttentionConfig (singe-kernel/src/cuda/attention/mod.rs:92-108). */
+typedef struct SingePagedKvPrefillAttentionConfig {
+    size_t batch;
+    size_t total_query_tokens;
+    size_t heads;
+    size_t kv_heads;
+    size_t head_dim;
+    size_t block_size;
+    size_t physical_blocks;
+    size_t block_table_batch_stride;
+    uint8_t causal;   /* Rust bool: 0 or 1 */
+    float scale;
+} SingePagedKvPrefillAttentionConfig;
+
+/* validate_paged_kv_prefill_attention_config (mod.rs:2987-3011). */
+SINGE_HIP_API int32_t singe_hip_paged_kv_prefill_attention_config_validate(const SingePagedKvPrefillAttentionConfig* config);
+
+/* paged_kv_prefill_attention_bf16 (singe-kernel/src/cuda/attention/paged.rs:370-420; CPU form
+ * cpu/attention.rs:1248-1341).  query/out [total_query_tokens, heads, dim] bf16, packed over the batch:
+ * sequence b holds tokens actual_seq_offsets[b] .. + actual_seq_lens_q[b] and reads the first
+ * actual_seq_lens_kv[b] keys of the blocks in row b of block_table [batch, stride] u32.  Causal hides
+ * key index > query index (queries align with the FIRST keys).  lse [total_query_tokens, heads] f32,
+ * natural log, -1e20 for a row that sees no key.  Rows of tokens no sequence covers are not written.
+ * A sequence whose offsets or lengths would address outside the buffers is skipped.  Lengths are
+ * checked as PagedKvPrefillAttentionConfig::validate_lengths does (mod.rs:786-818). */
+SINGE_HIP_API int32_t singe_hip_paged_kv_prefill_attention_bf16(
+    void* stream,
+    uint16_t* out, size_t out_len,
+    float* lse, size_t lse_len,
+    const uint16_t* query, size_t query_len,
+    const uint16_t* key_cache, size_t key_cache_len,
+    const uint16_t* value_cache, size_t value_cache_len,
+    const int32_t* actual_seq_lens_q, size_t actual_seq_lens_q_len,
+    const int32_t* actual_seq_lens_kv, size_t actual_seq_lens_kv_len,
+    const int32_t* actual_seq_offsets, size_t actual_seq_offsets_len,
+    const uint32_t* block_table, size_t block_table_len,
+    const SingePagedKvPrefillAttentionConfig* config);
+
 /* ---- singe-kernel surface: dense prefill ---------------------------------------------------------
  * Mirrors FmhaPrefillConfig (singe-kernel/src/cuda/attention/mod.rs:253-274); strides in elements.
  * FmhaPrefillConfig::contiguous (mod.rs:1602-1632) fills them for packed [batch, len, heads, dim]. */

@@ -26,6 +26,12 @@ class PagedKvDecodeAttentionConfigC(ctypes.Structure):
                 ("scale", ctypes.c_float)]
 
 
+class PagedKvPrefillAttentionConfigC(ctypes.Structure):
+    _fields_ = [("batch", c_size), ("total_query_tokens", c_size), ("heads", c_size), ("kv_heads", c_size),
+                ("head_dim", c_size), ("block_size", c_size), ("physical_blocks", c_size),
+                ("block_table_batch_stride", c_size), ("causal", ctypes.c_uint8), ("scale", ctypes.c_float)]
+
+
 class FmhaPrefillConfigC(ctypes.Structure):
     _fields_ = [(name, c_size) for name in (
         "batch", "query_len", "key_len", "heads", "kv_heads", "head_dim", "query_batch_stride",
@@ -98,6 +104,11 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_set_decode_workers.restype = None
     handle.singe_hip_decode_workers.argtypes = [cfg]
     handle.singe_hip_decode_workers.restype = ctypes.c_uint32
+    paged_prefill = ctypes.POINTER(PagedKvPrefillAttentionConfigC)
+    handle.singe_hip_paged_kv_prefill_attention_config_validate.argtypes = [paged_prefill]
+    handle.singe_hip_paged_kv_prefill_attention_config_validate.restype = i32
+    handle.singe_hip_paged_kv_prefill_attention_bf16.argtypes = [c_void] + [c_void, c_size] * 9 + [paged_prefill]
+    handle.singe_hip_paged_kv_prefill_attention_bf16.restype = i32
     fmha = ctypes.POINTER(FmhaPrefillConfigC)
     handle.singe_hip_fmha_prefill_config_validate.argtypes = [fmha]
     handle.singe_hip_fmha_prefill_config_validate.restype = i32

@@ -90,10 +90,11 @@ struct PagedAttentionArgs {
     const uint16_t* query_rows;     // [tokens, heads, 128] bf16
     const uint16_t* key_cache;      // [cache_pages, page_size, kv_heads, 128] bf16
     const uint16_t* value_cache;
-    const void* query_offsets;      // [sequences + 1] i32 or i64
+    const void* query_offsets;      // [sequences + 1] i32 or i64; block-table form: [sequences] i32 starts
     const void* page_offsets;       // [sequences + 1]
     const void* pages;              // [page_table]
-    const void* last_page_lengths;  // [sequences]
+    const void* last_page_lengths;  // [sequences]; block-table form: the key lengths
+    const void* query_lengths;      // block-table form only: [sequences] i32
     uint16_t* output;               // [tokens, heads, 128] bf16
     float* lse;                     // [tokens, heads] base two, or null
     uint32_t* status;               // first writer wins, may be null
@@ -104,7 +105,7 @@ struct PagedAttentionArgs {
     uint32_t page_size;
     uint32_t sequences;
     uint32_t cache_pages;
-    uint32_t page_table;
+    uint32_t page_table;            // entries of `pages`; block-table form: entries per table row
     uint32_t row_tiles;             // ceil(groups * tokens / 128): row tiles per (sequence, kv head)
     uint32_t causal;
     float scale_log2e;              // scale * log2(e)

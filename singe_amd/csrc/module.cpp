@@ -24,6 +24,7 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_fmha_prefill_f32_d32", "singe_fmha_prefill_f32_d64", "singe_fmha_prefill_f32_d128", "singe_fmha_prefill_f32_d256",
     "singe_paged_attention_bf16_d128_i32", "singe_paged_attention_bf16_d128_i64",
     "singe_paged_attention_bf16_d128_softcap_i32", "singe_paged_attention_bf16_d128_softcap_i64",
+    "singe_paged_kv_prefill_bf16_d128",
 };
 
 namespace {

@@ -17,6 +17,7 @@ enum KernelId : int {
     kPrefillCausal, kPrefillFull,
     kPrefillF32D32, kPrefillF32D64, kPrefillF32D128, kPrefillF32D256,
     kPagedAttentionI32, kPagedAttentionI64, kPagedAttentionSoftcapI32, kPagedAttentionSoftcapI64,
+    kPagedKvPrefill,
     kKernelCount
 };
 

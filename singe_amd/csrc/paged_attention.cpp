@@ -49,6 +49,7 @@ extern "C" int32_t singe_hip_paged_attention_bf16(void* stream, const uint16_t* 
     args.page_offsets = page_offsets;
     args.pages = pages;
     args.last_page_lengths = last_page_lengths;
+    args.query_lengths = nullptr;
     args.output = output;
     args.lse = lse;
     args.status = status;
@@ -74,4 +75,81 @@ extern "C" int32_t singe_hip_paged_attention_bf16(void* stream, const uint16_t* 
     const KernelId kernel = p.has_softcap ? (wide ? kPagedAttentionSoftcapI64 : kPagedAttentionSoftcapI32)
                                           : (wide ? kPagedAttentionI64 : kPagedAttentionI32);
     return launch(kernel, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+}
+
+// validate_paged_kv_prefill_attention_config (singe-kernel/src/cuda/attention/mod.rs:2987-3011).
+extern "C" int32_t singe_hip_paged_kv_prefill_attention_config_validate(const SingePagedKvPrefillAttentionConfig* config) {
+    if (config == nullptr) return fail(SINGE_HIP_NULL_POINTER, "config");
+    const SingePagedKvPrefillAttentionConfig& c = *config;
+    if (c.batch == 0 || c.total_query_tokens == 0 || c.heads == 0 || c.kv_heads == 0 || c.head_dim == 0 || c.block_size == 0 ||
+        c.physical_blocks == 0 || c.block_table_batch_stride == 0 || c.heads % c.kv_heads != 0 || !std::isfinite(c.scale))
+        return fail(SINGE_HIP_INVALID_LENGTH, "config");
+    const size_t extents[] = {c.batch, c.total_query_tokens, c.heads, c.kv_heads, c.head_dim, c.block_size, c.physical_blocks,
+                              c.block_table_batch_stride};
+    for (size_t extent : extents)
+        if (!fits_i32(extent)) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "config");
+    return 0;
+}
+
+// paged_kv_prefill_attention_bf16 (singe-kernel/src/cuda/attention/paged.rs:370-420); lengths checked
+// in the order of PagedKvPrefillAttentionConfig::validate_lengths (mod.rs:786-818).
+extern "C" int32_t singe_hip_paged_kv_prefill_attention_bf16(
+    void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, const uint16_t* query, size_t query_len,
+    const uint16_t* key_cache, size_t key_cache_len, const uint16_t* value_cache, size_t value_cache_len,
+    const int32_t* actual_seq_lens_q, size_t actual_seq_lens_q_len, const int32_t* actual_seq_lens_kv,
+    size_t actual_seq_lens_kv_len, const int32_t* actual_seq_offsets, size_t actual_seq_offsets_len,
+    const uint32_t* block_table, size_t block_table_len, const SingePagedKvPrefillAttentionConfig* config) {
+    if (int32_t status = singe_hip_paged_kv_prefill_attention_config_validate(config)) return status;
+    const SingePagedKvPrefillAttentionConfig& c = *config;
+    size_t output_len = 0, lse_needed = 0, block_len = 0, cache_len = 0, table_len = 0;
+    if (!checked_mul(c.total_query_tokens, c.heads, &lse_needed) || !checked_mul(lse_needed, c.head_dim, &output_len) ||
+        !checked_mul(c.block_size, c.kv_heads, &block_len) || !checked_mul(block_len, c.head_dim, &block_len) ||
+        !checked_mul(c.physical_blocks, block_len, &cache_len) || !checked_mul(c.batch, c.block_table_batch_stride, &table_len))
+        return fail(SINGE_HIP_SIZE_OVERFLOW, "config");
+    if (int32_t s = ensure_len_at_least("out", out_len, output_len)) return s;
+    if (int32_t s = ensure_len_at_least("lse", lse_len, lse_needed)) return s;
+    if (int32_t s = ensure_len_at_least("query", query_len, output_len)) return s;
+    if (int32_t s = ensure_len_at_least("key_cache", key_cache_len, cache_len)) return s;
+    if (int32_t s = ensure_len_at_least("value_cache", value_cache_len, cache_len)) return s;
+    if (int32_t s = ensure_len_at_least("actual_seq_lens_q", actual_seq_lens_q_len, c.batch)) return s;
+    if (int32_t s = ensure_len_at_least("actual_seq_lens_kv", actual_seq_lens_kv_len, c.batch)) return s;
+    if (int32_t s = ensure_len_at_least("actual_seq_offsets", actual_seq_offsets_len, c.batch)) return s;
+    if (int32_t s = ensure_len_at_least("block_table", block_table_len, table_len)) return s;
+    if (c.head_dim != 128) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, "paged_kv_prefill_attention_bf16", c.head_dim, 0);
+    const void* pointers[] = {out, lse, query, key_cache, value_cache, actual_seq_lens_q, actual_seq_lens_kv, actual_seq_offsets, block_table};
+    const char* names[] = {"out", "lse", "query", "key_cache", "value_cache", "actual_seq_lens_q", "actual_seq_lens_kv",
+                           "actual_seq_offsets", "block_table"};
+    for (int i = 0; i < 9; ++i)
+        if (pointers[i] == nullptr) return fail(SINGE_HIP_NULL_POINTER, names[i]);
+
+    const uint64_t groups = c.heads / c.kv_heads;
+    PagedAttentionArgs args;
+    args.query_rows = query;
+    args.key_cache = key_cache;
+    args.value_cache = value_cache;
+    args.query_offsets = actual_seq_offsets;
+    args.page_offsets = nullptr;
+    args.pages = block_table;
+    args.last_page_lengths = actual_seq_lens_kv;
+    args.query_lengths = actual_seq_lens_q;
+    args.output = out;
+    args.lse = lse;
+    args.status = nullptr;
+    args.window = -1;
+    args.tokens = static_cast<uint32_t>(c.total_query_tokens);
+    args.heads = static_cast<uint32_t>(c.heads);
+    args.kv_heads = static_cast<uint32_t>(c.kv_heads);
+    args.page_size = static_cast<uint32_t>(c.block_size);
+    args.sequences = static_cast<uint32_t>(c.batch);
+    args.cache_pages = static_cast<uint32_t>(c.physical_blocks);
+    args.page_table = static_cast<uint32_t>(c.block_table_batch_stride);
+    args.row_tiles = static_cast<uint32_t>((groups * static_cast<uint64_t>(c.total_query_tokens) + 127) / 128);
+    args.causal = c.causal ? 1u : 0u;
+    args.scale_log2e = c.scale * 1.4426950408889634074f;
+    args.softcap_scale = 0.0f;
+    args.softcap_log2e = 0.0f;
+    const uint64_t units = (static_cast<uint64_t>(c.batch) * c.kv_heads + 7) / 8 * 8;
+    const uint64_t blocks = units * args.row_tiles;
+    if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
+    return launch(kPagedKvPrefill, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
 }

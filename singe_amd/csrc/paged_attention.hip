@@ -16,6 +16,11 @@
 // their sequence's rows return at once.  Keys are gathered page by page into the same padded LDS tiles
 // as the dense kernel and folded by the shared core (prefill_core.hip.h).
 //
+// The same body also serves paged_kv_prefill_attention of the singe-kernel surface
+// (singe-kernel/src/cpu/attention.rs:1248-1341): paging as a [batch, stride] block table with per-sequence
+// query offsets, query lengths and key lengths, queries aligned with a sequence's FIRST keys, and a
+// natural-log lse that is -1e20 for a row without keys.
+//
 // Paging values come from device memory, so they are checked here: a value that would address outside
 // the queries, the page table or the cache sets the status word to 1 (first writer wins; the word may
 // be null) and nothing is read through it (paged_attention.rs:41-54, 210-262, 739-755).
@@ -26,15 +31,27 @@ namespace {
 
 using namespace prefill;
 
-template <bool WIDE>
+// How the paging arrives: FlashInfer CSR vectors of i32 or i64, or the block table of the
+// singe-kernel surface (u32 table rows, i32 per-sequence query offsets and lengths).
+enum : int { kCsrI32 = 0, kCsrI64 = 1, kTable = 2 };
+
+template <int FORM>
 SINGE_DEVICE long long read_index(const void* values, size_t at) {
-    if constexpr (WIDE)
+    if constexpr (FORM == kCsrI64)
         return static_cast<const long long*>(values)[at];
     else
         return static_cast<long long>(static_cast<const int*>(values)[at]);
 }
 
-template <bool SOFTCAP, bool WIDE>
+template <int FORM>
+SINGE_DEVICE unsigned long long read_page(const void* pages, size_t at) {
+    if constexpr (FORM == kTable)
+        return static_cast<const unsigned int*>(pages)[at];
+    else
+        return static_cast<unsigned long long>(read_index<FORM>(pages, at));  // negative ids wrap above any cache
+}
+
+template <bool SOFTCAP, int FORM>
 SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned char* lds) {
     const unsigned int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const unsigned int column = lane & 31, hi = lane >> 5;
@@ -49,25 +66,44 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
 
     // The sequence's paging values, refused when any would address outside the kernel's buffers
     // (paged_attention.rs:210-238; the CPU check is spec/neural/attention.rs:372-406).
-    const long long query_start = read_index<WIDE>(a.query_offsets, sequence);
-    const long long query_end = read_index<WIDE>(a.query_offsets, sequence + 1);
-    const long long page_start = read_index<WIDE>(a.page_offsets, sequence);
-    const long long page_end = read_index<WIDE>(a.page_offsets, sequence + 1);
-    const long long last_length = read_index<WIDE>(a.last_page_lengths, sequence);
-    if (query_start < 0 || query_end < query_start || query_end > static_cast<long long>(a.tokens) || page_start < 0 ||
-        page_end < page_start || page_end > static_cast<long long>(a.page_table) ||
-        (page_end > page_start && (last_length < 0 || last_length > static_cast<long long>(a.page_size)))) {
-        if (tid == 0) report_index_error(a.status);
-        return;
+    long long query_start, query_count, page_start, key_count;
+    if constexpr (FORM == kTable) {
+        // Block-table form (singe-kernel/src/cpu/attention.rs:1272-1276): offsets, query and key
+        // lengths per sequence; row `sequence` of the table holds its blocks.
+        query_start = read_index<FORM>(a.query_offsets, sequence);
+        query_count = read_index<FORM>(a.query_lengths, sequence);
+        key_count = read_index<FORM>(a.last_page_lengths, sequence);
+        page_start = static_cast<long long>(sequence) * a.page_table;
+        if (query_start < 0 || query_count < 0 || query_start + query_count > static_cast<long long>(a.tokens) || key_count < 0 ||
+            key_count > static_cast<long long>(a.page_table) * a.page_size) {
+            if (tid == 0) report_index_error(a.status);
+            return;
+        }
+    } else {
+        query_start = read_index<FORM>(a.query_offsets, sequence);
+        const long long query_end = read_index<FORM>(a.query_offsets, sequence + 1);
+        page_start = read_index<FORM>(a.page_offsets, sequence);
+        const long long page_end = read_index<FORM>(a.page_offsets, sequence + 1);
+        const long long last_length = read_index<FORM>(a.last_page_lengths, sequence);
+        if (query_start < 0 || query_end < query_start || query_end > static_cast<long long>(a.tokens) || page_start < 0 ||
+            page_end < page_start || page_end > static_cast<long long>(a.page_table) ||
+            (page_end > page_start && (last_length < 0 || last_length > static_cast<long long>(a.page_size)))) {
+            if (tid == 0) report_index_error(a.status);
+            return;
+        }
+        query_count = query_end - query_start;
+        const long long page_count = page_end - page_start;
+        key_count = page_count == 0 ? 0 : (page_count - 1) * a.page_size + last_length;
     }
-    const unsigned int queries = static_cast<unsigned int>(query_end - query_start);
+    const unsigned int queries = static_cast<unsigned int>(query_count);
     const unsigned int packed = queries * groups;
     if (first_row >= packed) return;
-    const unsigned int page_count = static_cast<unsigned int>(page_end - page_start);
-    const unsigned int keys = page_count == 0 ? 0u : (page_count - 1u) * a.page_size + static_cast<unsigned int>(last_length);
+    const unsigned int keys = static_cast<unsigned int>(key_count);
 
-    // Key position of packed row r: max(keys - queries + r / groups, 0).
+    // Key position of packed row r: max(keys - queries + r / groups, 0); the block-table form aligns
+    // queries with the FIRST keys instead (key > query index is hidden, cpu/attention.rs:1283).
     auto position_of = [&](unsigned int row) __attribute__((always_inline)) {
+        if constexpr (FORM == kTable) return row / groups;
         const long long position = static_cast<long long>(keys) - static_cast<long long>(queries) + row / groups;
         return position < 0 ? 0u : static_cast<unsigned int>(position);
     };
@@ -122,7 +158,7 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     auto lookup_row = [&](unsigned int tile, unsigned int i, unsigned long long& page) __attribute__((always_inline)) {
         const unsigned int key = tile * kKeyTile + load_row + 16u * i;
         page = 0;
-        if (key < keys) page = static_cast<unsigned long long>(read_index<WIDE>(a.pages, static_cast<size_t>(page_start) + key / a.page_size));
+        if (key < keys) page = read_page<FORM>(a.pages, static_cast<size_t>(page_start) + key / a.page_size);
     };
     auto lookup = [&](unsigned int tile) __attribute__((always_inline)) {
         lookup_row(tile, 0, page0);
@@ -231,19 +267,27 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
                 packed_bits.y = pack_pair(state.out[db][4 * quad + 2] * inverse, state.out[db][4 * quad + 3] * inverse);
                 *reinterpret_cast<uint2*>(row + 32 * db + 8 * quad + 4 * hi) = packed_bits;
             }
-        if (a.lse != nullptr && hi == 0) a.lse[flat] = sum > 0.0f ? state.reference + fast_log2(sum) : -INFINITY;
+        if (a.lse != nullptr && hi == 0) {
+            const float lse2 = state.reference + fast_log2(sum);
+            if constexpr (FORM == kTable)  // natural log, -1e20 for a row without keys (cpu/attention.rs:1304-1317)
+                a.lse[flat] = sum > 0.0f ? lse2 * 0.69314718055994530942f : -1.0e20f;
+            else
+                a.lse[flat] = sum > 0.0f ? lse2 : -INFINITY;
+        }
     }
 }
 
 }  // namespace
 
-#define SINGE_PAGED_ATTENTION_KERNEL(NAME, SOFTCAP, WIDE)                                              \
+#define SINGE_PAGED_ATTENTION_KERNEL(NAME, SOFTCAP, FORM)                                              \
     extern "C" __global__ __launch_bounds__(256, 2) void NAME(PagedAttentionArgs args) {                \
         __shared__ __attribute__((aligned(16))) unsigned char paged_lds[2 * prefill::kStageBytes];     \
-        paged_attention_body<SOFTCAP, WIDE>(args, paged_lds);                                          \
+        paged_attention_body<SOFTCAP, FORM>(args, paged_lds);                                          \
     }
 
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i32, false, false)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i64, false, true)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i32, true, false)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i64, true, true)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i32, false, kCsrI32)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i64, false, kCsrI64)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i32, true, kCsrI32)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i64, true, kCsrI64)
+// paged_kv_prefill_attention_bf16 of the singe-kernel surface: same gather, block-table paging.
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_bf16_d128, false, kTable)

@@ -169,6 +169,83 @@ def set_relaxed_numerics(relaxed: bool) -> None:
 
 
 @dataclass(frozen=True)
+class PagedKvPrefillAttentionConfig:
+    """Prefill attention over paged KV caches (mod.rs:92-108): query tokens packed across the batch and
+    indexed by sequence offsets, K/V cache tokens addressed through a block table."""
+    batch: int
+    total_query_tokens: int
+    heads: int
+    kv_heads: int
+    head_dim: int
+    block_size: int
+    physical_blocks: int
+    block_table_batch_stride: int
+    causal: bool
+    scale: float
+
+    @classmethod
+    def contiguous(cls, batch, total_query_tokens, heads, kv_heads, head_dim, block_size, physical_blocks,
+                   block_table_batch_stride, causal, scale) -> "PagedKvPrefillAttentionConfig":
+        """mod.rs:746-773: builds the config and validates it."""
+        config = cls(batch, total_query_tokens, heads, kv_heads, head_dim, block_size, physical_blocks,
+                     block_table_batch_stride, bool(causal), scale)
+        config.validate()
+        return config
+
+    def validate(self) -> None:
+        """validate_paged_kv_prefill_attention_config (mod.rs:2987-3011)."""
+        extents = (self.batch, self.total_query_tokens, self.heads, self.kv_heads, self.head_dim, self.block_size,
+                   self.physical_blocks, self.block_table_batch_stride)
+        if any(e <= 0 for e in extents) or self.heads % self.kv_heads != 0 or not math.isfinite(self.scale):
+            raise error.InvalidLength("invalid length")
+        if any(e > I32_MAX for e in extents):
+            raise error.LengthExceedsI32("length exceeds i32")
+
+    def output_len(self) -> int:
+        return self.total_query_tokens * self.heads * self.head_dim
+
+    def lse_len(self) -> int:
+        return self.total_query_tokens * self.heads
+
+    def _c(self) -> _native.PagedKvPrefillAttentionConfigC:
+        return _native.PagedKvPrefillAttentionConfigC(self.batch, self.total_query_tokens, self.heads, self.kv_heads,
+                                                      self.head_dim, self.block_size, self.physical_blocks,
+                                                      self.block_table_batch_stride, 1 if self.causal else 0,
+                                                      self.scale)
+
+
+def paged_kv_prefill_attention_bf16(stream, out: torch.Tensor, lse: torch.Tensor, query: torch.Tensor,
+                                    key_cache: torch.Tensor, value_cache: torch.Tensor,
+                                    actual_seq_lens_q: torch.Tensor, actual_seq_lens_kv: torch.Tensor,
+                                    actual_seq_offsets: torch.Tensor, block_table: torch.Tensor,
+                                    config: PagedKvPrefillAttentionConfig) -> None:
+    """paged_kv_prefill_attention_bf16 (paged.rs:370-420).
+
+    out/query [total_query_tokens, heads, dim] bf16; lse [total_query_tokens, heads] f32 (natural log,
+    -1e20 for a row without keys); caches [blocks, block_size, kv_heads, dim] bf16; the three per-sequence
+    vectors [batch] i32; block_table [batch, stride] u32.  Causal hides key index > query index.
+    """
+    _require(out, torch.bfloat16, "out")
+    _require(lse, torch.float32, "lse")
+    _require(query, torch.bfloat16, "query")
+    _require(key_cache, torch.bfloat16, "key_cache")
+    _require(value_cache, torch.bfloat16, "value_cache")
+    _require(actual_seq_lens_q, torch.int32, "actual_seq_lens_q")
+    _require(actual_seq_lens_kv, torch.int32, "actual_seq_lens_kv")
+    _require(actual_seq_offsets, torch.int32, "actual_seq_offsets")
+    if block_table.dtype not in (torch.int32, torch.uint32):
+        raise error.InvalidArgument(f"block_table must hold 32-bit entries, got {block_table.dtype}")
+    _require(block_table, block_table.dtype, "block_table")
+    c = config._c()
+    status = _native.lib().singe_hip_paged_kv_prefill_attention_bf16(
+        _stream_handle(stream), _ptr(out), out.numel(), _ptr(lse), lse.numel(), _ptr(query), query.numel(),
+        _ptr(key_cache), key_cache.numel(), _ptr(value_cache), value_cache.numel(), _ptr(actual_seq_lens_q),
+        actual_seq_lens_q.numel(), _ptr(actual_seq_lens_kv), actual_seq_lens_kv.numel(), _ptr(actual_seq_offsets),
+        actual_seq_offsets.numel(), _ptr(block_table), block_table.numel(), ctypes.byref(c))
+    _native.check(status, "paged_kv_prefill_attention_bf16")
+
+
+@dataclass(frozen=True)
 class FmhaPrefillConfig:
     """Dense prefill attention (mod.rs:253-274): query/out [batch, query_len, heads, dim], key/value
     [batch, key_len, kv_heads, dim], addressed through element strides; ``causal`` is top-left."""
