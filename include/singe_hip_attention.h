@@ -336,6 +336,109 @@ SINGE_HIP_API int32_t singe_hip_paged_attention_bf16(
     uint32_t* status,
     const SingePagedAttentionProblem* problem);
 
+/* The same op for f32 and f16 tensors, and (through the bf16 entry point above) for bf16 at head
+ * dimensions other than 128, up to 256: the general kernel, one wave per (token, head) row, f32
+ * arithmetic whatever the storage type (kernel_plan/source/paged_general.rs:73-247; CPU form
+ * singe/src/backend/cpu/normalization/attention.rs:297-330, 424-538). */
+SINGE_HIP_API int32_t singe_hip_paged_attention_f32(
+    void* stream,
+    const float* query_rows,
+    const float* key_cache,
+    const float* value_cache,
+    const void* query_offsets,
+    const void* page_offsets,
+    const void* pages,
+    const void* last_page_lengths,
+    float* output,
+    float* lse,
+    uint32_t* status,
+    const SingePagedAttentionProblem* problem);
+SINGE_HIP_API int32_t singe_hip_paged_attention_f16(
+    void* stream,
+    const uint16_t* query_rows,
+    const uint16_t* key_cache,
+    const uint16_t* value_cache,
+    const void* query_offsets,
+    const void* page_offsets,
+    const void* pages,
+    const void* last_page_lengths,
+    uint16_t* output,
+    float* lse,
+    uint32_t* status,
+    const SingePagedAttentionProblem* problem);
+
+/* ---- singe surface: dense scaled-dot-product attention ----------------------------------------------
+ * Operation::ScaledDotProductAttention (singe/src/tensor/neural.rs:92-190; CPU form
+ * singe/src/backend/cpu/normalization/attention.rs:191-276; shape rules spec/neural/attention.rs:209-290):
+ * query [batch, heads, query_len, head_dim], key [batch, kv_heads, key_len, head_dim], value
+ * [batch, kv_heads, key_len, value_dim], output [batch, heads, query_len, value_dim], all contiguous and
+ * of one element type; query head h reads kv head h / (heads / kv_heads).  Causal hides key > query
+ * (top-left), window hides key + window <= query, softcap caps the scaled scores, then `mask` (element
+ * type of the query, read through mask_strides over (batch, head, query, key), 0 = broadcast) adds to
+ * them; `sinks` [heads] joins each row's softmax without weighing a value; `key_lengths` [batch] i32
+ * hides the keys past each batch's count (a count of zero gives zeros).  mask, sinks and key_lengths may
+ * be null.  head_dim and value_dim up to 256. */
+#define SINGE_HIP_F32 0
+#define SINGE_HIP_BF16 1
+#define SINGE_HIP_F16 2
+typedef struct SingeAttentionProblem {
+    int64_t batch;
+    int64_t heads;
+    int64_t kv_heads;
+    int64_t query_len;
+    int64_t key_len;
+    int64_t head_dim;
+    int64_t value_dim;
+    int64_t mask_strides[4];
+    int32_t data_type;     /* SINGE_HIP_F32, _BF16 or _F16 */
+    uint8_t causal;
+    uint8_t has_scale;
+    uint8_t has_window;
+    uint8_t has_softcap;
+    float scale;
+    float softcap;
+    int64_t window;
+} SingeAttentionProblem;
+
+SINGE_HIP_API int32_t singe_hip_scaled_dot_product_attention(
+    void* stream,
+    const void* query,
+    const void* key,
+    const void* value,
+    const void* mask,
+    const void* sinks,
+    const int32_t* key_lengths,
+    void* output,
+    const SingeAttentionProblem* problem);
+
+/* ---- singe-kernel surface: split-KV reduce -----------------------------------------------------------
+ * Mirrors SplitKReduceConfig (singe-kernel/src/cuda/attention/mod.rs:385-398); strides in elements.
+ * SplitKReduceConfig::contiguous (mod.rs:2312-2328) fills them for attn [batch, heads, splits, dim],
+ * lse [batch, heads, splits], out [batch, heads, dim]. */
+typedef struct SingeSplitKReduceConfig {
+    size_t batch;
+    size_t heads;
+    size_t splits;
+    size_t head_dim;
+    size_t attn_batch_stride;
+    size_t attn_head_stride;
+    size_t attn_split_stride;
+    size_t lse_batch_stride;
+    size_t lse_head_stride;
+    size_t output_batch_stride;
+    size_t output_head_stride;
+} SingeSplitKReduceConfig;
+
+/* splitk_reduce_f32 (singe-kernel/src/cuda/attention/fmha.rs:1038-1067; CPU form
+ * cpu/attention.rs:2157-2193): out = sum_s exp(lse_s - max) * attn_s / sum_s exp(lse_s - max), natural
+ * log.  Lengths are checked as SplitKReduceConfig::validate_lengths does (mod.rs:2330-2361). */
+SINGE_HIP_API int32_t singe_hip_splitk_reduce_f32(
+    void* stream,
+    float* out, size_t out_len,
+    const float* attn_splitk, size_t attn_splitk_len,
+    const float* lse_splitk, size_t lse_splitk_len,
+    const SingeSplitKReduceConfig* config);
+
 #ifdef __cplusplus
 }
 #endif

@@ -55,6 +55,23 @@ class PagedAttentionProblemC(ctypes.Structure):
                 ("window", ctypes.c_int64)]
 
 
+class AttentionProblemC(ctypes.Structure):
+    _fields_ = [("batch", ctypes.c_int64), ("heads", ctypes.c_int64), ("kv_heads", ctypes.c_int64),
+                ("query_len", ctypes.c_int64), ("key_len", ctypes.c_int64), ("head_dim", ctypes.c_int64),
+                ("value_dim", ctypes.c_int64), ("mask_strides", ctypes.c_int64 * 4), ("data_type", ctypes.c_int32),
+                ("causal", ctypes.c_uint8), ("has_scale", ctypes.c_uint8), ("has_window", ctypes.c_uint8),
+                ("has_softcap", ctypes.c_uint8), ("scale", ctypes.c_float), ("softcap", ctypes.c_float),
+                ("window", ctypes.c_int64)]
+
+
+class SplitKReduceConfigC(ctypes.Structure):
+    _fields_ = [(name, c_size) for name in (
+        "batch", "heads", "splits", "head_dim", "attn_batch_stride", "attn_head_stride", "attn_split_stride",
+        "lse_batch_stride", "lse_head_stride", "output_batch_stride", "output_head_stride")]
+
+
+DATA_TYPE_F32, DATA_TYPE_BF16, DATA_TYPE_F16 = 0, 1, 2
+
 _lib = None
 
 
@@ -130,6 +147,15 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_softcapped_window_attention_f32.restype = i32
     handle.singe_hip_paged_attention_bf16.argtypes = [c_void] * 11 + [ctypes.POINTER(PagedAttentionProblemC)]
     handle.singe_hip_paged_attention_bf16.restype = i32
+    handle.singe_hip_paged_attention_f32.argtypes = [c_void] * 11 + [ctypes.POINTER(PagedAttentionProblemC)]
+    handle.singe_hip_paged_attention_f32.restype = i32
+    handle.singe_hip_paged_attention_f16.argtypes = [c_void] * 11 + [ctypes.POINTER(PagedAttentionProblemC)]
+    handle.singe_hip_paged_attention_f16.restype = i32
+    handle.singe_hip_scaled_dot_product_attention.argtypes = [c_void] * 8 + [ctypes.POINTER(AttentionProblemC)]
+    handle.singe_hip_scaled_dot_product_attention.restype = i32
+    handle.singe_hip_splitk_reduce_f32.argtypes = [c_void, c_void, c_size, c_void, c_size, c_void, c_size,
+                                                   ctypes.POINTER(SplitKReduceConfigC)]
+    handle.singe_hip_splitk_reduce_f32.restype = i32
     _lib = handle
     return handle
 

@@ -1,0 +1,194 @@
+// Host side of the kernels that take any element type and head dimension: the dense
+// scaled-dot-product attention of the singe crate (shape rules of spec::attention_problem,
+// singe/src/backend/spec/neural/attention.rs:209-290), the general paged attention
+// (singe/src/backend/cuda/kernel_plan/source/paged_general.rs:73-247) and splitk_reduce_f32
+// (singe-kernel/src/cuda/attention/fmha.rs:1038-1067).
+#include <cmath>
+
+#include "kernel_args.h"
+#include "module.h"
+#include "singe_hip_attention.h"
+#include "validate.h"
+
+using namespace singe_hip;
+
+namespace {
+
+// Kernel of a family for (element, widest dimension): families are laid out element-major with
+// the 64 / 128 / 256 variants consecutive.
+int32_t pick(KernelId base, int32_t data_type, uint64_t widest, const char* op, KernelId* kernel) {
+    if (data_type != SINGE_HIP_F32 && data_type != SINGE_HIP_BF16 && data_type != SINGE_HIP_F16)
+        return fail(SINGE_HIP_INVALID_ARGUMENT, "data type");
+    if (widest > 256) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, op, 0, widest);
+    const int width = widest <= 64 ? 0 : widest <= 128 ? 1 : 2;
+    *kernel = static_cast<KernelId>(base + 3 * data_type + width);
+    return 0;
+}
+
+bool span_reach(size_t count, size_t stride, size_t* total) {  // *total += (count - 1) * stride
+    size_t span = 0;
+    return count > 0 && checked_mul(count - 1, stride, &span) && checked_add(*total, span, total);
+}
+
+}  // namespace
+
+namespace singe_hip {
+
+// Shared with the bf16 entry point, which hands head dimensions other than 128 to this kernel.
+int32_t paged_attention_general(int32_t data_type, void* stream, const void* query_rows, const void* key_cache,
+                                const void* value_cache, const void* query_offsets, const void* page_offsets,
+                                const void* pages, const void* last_page_lengths, void* output, float* lse, uint32_t* status,
+                                const SingePagedAttentionProblem& p, float scale) {
+    KernelId kernel;
+    if (int32_t s = pick(kPagedGeneral, data_type, static_cast<uint64_t>(p.head_dim), "paged_attention", &kernel)) return s;
+    GeneralPagedArgs args;
+    args.query_rows = query_rows;
+    args.key_cache = key_cache;
+    args.value_cache = value_cache;
+    args.query_offsets = query_offsets;
+    args.page_offsets = page_offsets;
+    args.pages = pages;
+    args.last_page_lengths = last_page_lengths;
+    args.output = output;
+    args.lse = lse;
+    args.status = status;
+    args.window = p.has_window ? p.window : -1;
+    args.tokens = static_cast<uint32_t>(p.tokens);
+    args.heads = static_cast<uint32_t>(p.heads);
+    args.kv_heads = static_cast<uint32_t>(p.kv_heads);
+    args.head_dim = static_cast<uint32_t>(p.head_dim);
+    args.page_size = static_cast<uint32_t>(p.page_size);
+    args.sequences = static_cast<uint32_t>(p.sequences);
+    args.cache_pages = static_cast<uint32_t>(p.cache_pages);
+    args.page_table = static_cast<uint32_t>(p.page_table);
+    const uint64_t row_blocks = (static_cast<uint64_t>(p.tokens) * p.heads + 3) / 4;
+    args.row_blocks = static_cast<uint32_t>(row_blocks);
+    args.causal = p.causal ? 1u : 0u;
+    args.has_softcap = p.has_softcap ? 1u : 0u;
+    args.wide_index = p.index_type == SINGE_HIP_INDEX_I64 ? 1u : 0u;
+    args.scale = scale;
+    args.softcap = p.has_softcap ? p.softcap : 0.0f;
+    const uint64_t blocks = row_blocks * static_cast<uint64_t>(p.sequences);
+    if (blocks > 0x7fffffffull || row_blocks > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
+    return launch(kernel, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+}
+
+}  // namespace singe_hip
+
+extern "C" int32_t singe_hip_scaled_dot_product_attention(void* stream, const void* query, const void* key, const void* value,
+                                                          const void* mask, const void* sinks, const int32_t* key_lengths,
+                                                          void* output, const SingeAttentionProblem* problem) {
+    if (problem == nullptr) return fail(SINGE_HIP_NULL_POINTER, "problem");
+    const SingeAttentionProblem& p = *problem;
+    // attention_problem: batch, heads, query length and value dimension may be zero; head dimension and
+    // key length may not; the key heads divide the query heads.
+    if (p.batch < 0 || p.heads < 0 || p.query_len < 0 || p.value_dim < 0 || p.head_dim <= 0 || p.key_len <= 0 || p.kv_heads <= 0 ||
+        p.heads % p.kv_heads != 0)
+        return fail(SINGE_HIP_INVALID_ARGUMENT, "attention shape");
+    if (p.has_scale && !std::isfinite(p.scale)) return fail(SINGE_HIP_INVALID_ARGUMENT, "scale");
+    if (p.has_softcap && !(std::isfinite(p.softcap) && p.softcap != 0.0f)) return fail(SINGE_HIP_INVALID_ARGUMENT, "softcap");
+    if (p.has_window && p.window < 0) return fail(SINGE_HIP_INVALID_ARGUMENT, "window");
+    const int64_t extents[] = {p.batch, p.heads, p.kv_heads, p.query_len, p.key_len, p.head_dim, p.value_dim};
+    for (int64_t extent : extents)
+        if (!fits_i32(static_cast<uint64_t>(extent))) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "problem");
+    for (int64_t stride : p.mask_strides)
+        if (stride < 0) return fail(SINGE_HIP_INVALID_ARGUMENT, "mask stride");
+    const uint64_t rows = static_cast<uint64_t>(p.batch) * p.heads * p.query_len;
+    if (rows == 0 || p.value_dim == 0) return 0;
+    if (query == nullptr) return fail(SINGE_HIP_NULL_POINTER, "query");
+    if (key == nullptr) return fail(SINGE_HIP_NULL_POINTER, "key");
+    if (value == nullptr) return fail(SINGE_HIP_NULL_POINTER, "value");
+    if (output == nullptr) return fail(SINGE_HIP_NULL_POINTER, "output");
+    const float scale = p.has_scale ? p.scale : 1.0f / std::sqrt(static_cast<float>(p.head_dim));
+
+    // bf16 at head dimension 128 with no mask, sinks, key lengths, window or cap is what the MFMA
+    // flash kernel computes, reading [batch, heads, len, dim] through its strides.
+    if (p.data_type == SINGE_HIP_BF16 && p.head_dim == 128 && p.value_dim == 128 && mask == nullptr && sinks == nullptr &&
+        key_lengths == nullptr && !p.has_window && !p.has_softcap) {
+        SingeFmhaPrefillConfig c;
+        c.batch = p.batch, c.query_len = p.query_len, c.key_len = p.key_len, c.heads = p.heads, c.kv_heads = p.kv_heads, c.head_dim = 128;
+        c.query_batch_stride = c.output_batch_stride = static_cast<size_t>(p.heads) * p.query_len * 128;
+        c.key_batch_stride = c.value_batch_stride = static_cast<size_t>(p.kv_heads) * p.key_len * 128;
+        c.query_sequence_stride = c.key_sequence_stride = c.value_sequence_stride = c.output_sequence_stride = 128;
+        c.query_head_stride = c.output_head_stride = static_cast<size_t>(p.query_len) * 128;
+        c.key_head_stride = c.value_head_stride = static_cast<size_t>(p.key_len) * 128;
+        c.scale = scale, c.causal = p.causal ? 1 : 0;
+        const size_t q_len = static_cast<size_t>(rows) * 128, kv_len = static_cast<size_t>(p.batch) * p.kv_heads * p.key_len * 128;
+        return singe_hip_fmha_prefill_bf16(stream, static_cast<uint16_t*>(output), q_len, static_cast<const uint16_t*>(query), q_len,
+                                           static_cast<const uint16_t*>(key), kv_len, static_cast<const uint16_t*>(value), kv_len, &c);
+    }
+
+    KernelId kernel;
+    const uint64_t widest = static_cast<uint64_t>(p.head_dim > p.value_dim ? p.head_dim : p.value_dim);
+    if (int32_t s = pick(kDenseGeneral, p.data_type, widest, "scaled_dot_product_attention", &kernel)) return s;
+    GeneralAttentionArgs args;
+    args.query = query;
+    args.key = key;
+    args.value = value;
+    args.mask = mask;
+    args.sinks = sinks;
+    args.key_lengths = key_lengths;
+    args.out = output;
+    for (int i = 0; i < 4; ++i) args.mask_strides[i] = static_cast<uint64_t>(p.mask_strides[i]);
+    args.window = p.has_window ? p.window : -1;
+    args.batch = static_cast<uint32_t>(p.batch);
+    args.heads = static_cast<uint32_t>(p.heads);
+    args.kv_heads = static_cast<uint32_t>(p.kv_heads);
+    args.query_len = static_cast<uint32_t>(p.query_len);
+    args.key_len = static_cast<uint32_t>(p.key_len);
+    args.head_dim = static_cast<uint32_t>(p.head_dim);
+    args.value_dim = static_cast<uint32_t>(p.value_dim);
+    args.causal = p.causal ? 1u : 0u;
+    args.has_softcap = p.has_softcap ? 1u : 0u;
+    args.scale = scale;
+    args.softcap = p.has_softcap ? p.softcap : 0.0f;
+    const uint64_t blocks = (rows + 3) / 4;
+    if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
+    return launch(kernel, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+}
+
+// validate_splitk_reduce_config (singe-kernel/src/cuda/attention/mod.rs:3557-3573) and
+// SplitKReduceConfig::validate_lengths (mod.rs:2330-2361).
+extern "C" int32_t singe_hip_splitk_reduce_f32(void* stream, float* out, size_t out_len, const float* attn_splitk,
+                                               size_t attn_splitk_len, const float* lse_splitk, size_t lse_splitk_len,
+                                               const SingeSplitKReduceConfig* config) {
+    if (config == nullptr) return fail(SINGE_HIP_NULL_POINTER, "config");
+    const SingeSplitKReduceConfig& c = *config;
+    if (c.batch == 0 || c.heads == 0 || c.splits == 0 || c.head_dim == 0 || c.attn_batch_stride == 0 || c.attn_head_stride == 0 ||
+        c.attn_split_stride == 0 || c.lse_batch_stride == 0 || c.lse_head_stride == 0 || c.output_batch_stride == 0 ||
+        c.output_head_stride == 0)
+        return fail(SINGE_HIP_INVALID_LENGTH, "config");
+    size_t attn_reach = c.head_dim, lse_reach = c.splits, out_reach = c.head_dim;
+    if (!span_reach(c.heads, c.attn_head_stride, &attn_reach) || !span_reach(c.splits, c.attn_split_stride, &attn_reach) ||
+        !span_reach(c.batch, c.attn_batch_stride, &attn_reach) || !span_reach(c.heads, c.lse_head_stride, &lse_reach) ||
+        !span_reach(c.batch, c.lse_batch_stride, &lse_reach) || !span_reach(c.heads, c.output_head_stride, &out_reach) ||
+        !span_reach(c.batch, c.output_batch_stride, &out_reach))
+        return fail(SINGE_HIP_SIZE_OVERFLOW, "config");
+    if (int32_t s = ensure_len_at_least("attn_splitk", attn_splitk_len, attn_reach)) return s;
+    if (int32_t s = ensure_len_at_least("lse_splitk", lse_splitk_len, lse_reach)) return s;
+    if (int32_t s = ensure_len_at_least("out", out_len, out_reach)) return s;
+    const size_t extents[] = {c.batch, c.heads, c.splits, c.head_dim};
+    for (size_t extent : extents)
+        if (!fits_i32(extent)) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "config");
+    if (out == nullptr) return fail(SINGE_HIP_NULL_POINTER, "out");
+    if (attn_splitk == nullptr) return fail(SINGE_HIP_NULL_POINTER, "attn_splitk");
+    if (lse_splitk == nullptr) return fail(SINGE_HIP_NULL_POINTER, "lse_splitk");
+    SplitKReduceArgs args;
+    args.out = out;
+    args.attn = attn_splitk;
+    args.lse = lse_splitk;
+    args.attn_batch_stride = c.attn_batch_stride;
+    args.attn_head_stride = c.attn_head_stride;
+    args.attn_split_stride = c.attn_split_stride;
+    args.lse_batch_stride = c.lse_batch_stride;
+    args.lse_head_stride = c.lse_head_stride;
+    args.output_batch_stride = c.output_batch_stride;
+    args.output_head_stride = c.output_head_stride;
+    args.batch = static_cast<uint32_t>(c.batch);
+    args.heads = static_cast<uint32_t>(c.heads);
+    args.splits = static_cast<uint32_t>(c.splits);
+    args.head_dim = static_cast<uint32_t>(c.head_dim);
+    const uint64_t blocks = (static_cast<uint64_t>(c.batch) * c.heads + 3) / 4;
+    if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
+    return launch(kSplitKReduce, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+}

@@ -1,0 +1,232 @@
+// Attention for any element type (f32, bf16, f16) and any head dimension up to 256: the fallback the
+// tensor-core kernels do not cover, the gfx950 counterpart of the reference's warp-per-row kernels
+// (singe/src/backend/cuda/kernel_plan/source/paged_general.rs:73-247) and of the CPU paths
+// singe/src/backend/cpu/normalization/attention.rs:191-276 (dense: causal, window, softcap, additive mask,
+// sinks, key lengths) and :424-538 (paged, FlashInfer form).
+//
+// One wave64 per query row.  Lanes take keys 64 apart; a lane's score is the same left-to-right fma chain
+// over the head dimension as the CPU path, in f32 whatever the storage type (the CPU path widens bf16/f16
+// to f32 first: attention.rs:63-69, 297-330); its softmax is online in natural base with expf, and the 64
+// per-lane partial rows are merged once at the end.
+#include "common.hip.h"
+#include "kernel_args.h"
+#include "paging.hip.h"
+
+namespace general {
+
+template <uint32_t ELEMENT>
+struct Element;
+template <>
+struct Element<kElementF32> {
+    typedef float type;
+    static SINGE_DEVICE float load(const type* at) { return *at; }
+    static SINGE_DEVICE void store(type* at, float value) { *at = value; }
+};
+template <>
+struct Element<kElementBf16> {
+    typedef unsigned short type;
+    static SINGE_DEVICE float load(const type* at) { return __builtin_bit_cast(float, static_cast<unsigned int>(*at) << 16); }
+    static SINGE_DEVICE void store(type* at, float value) { *at = f32_to_bf16_bits(value); }
+};
+template <>
+struct Element<kElementF16> {
+    typedef _Float16 type;
+    static SINGE_DEVICE float load(const type* at) { return static_cast<float>(*at); }
+    static SINGE_DEVICE void store(type* at, float value) { *at = static_cast<_Float16>(value); }  // round to nearest even
+};
+
+// Per-lane running state over the keys a lane has seen.
+template <int DMAX>
+struct LaneState {
+    float acc[DMAX];
+    float largest;
+    float total;
+};
+
+template <int DMAX>
+SINGE_DEVICE void reset(LaneState<DMAX>& state) {
+#pragma unroll
+    for (int d = 0; d < DMAX; ++d) state.acc[d] = 0.0f;
+    state.largest = -INFINITY;
+    state.total = 0.0f;
+}
+
+// Folds one key into a lane's state.  A score of -inf (a masked key) weighs nothing.
+template <class E, int DMAX>
+SINGE_DEVICE void fold_key(LaneState<DMAX>& state, const float* q_row, const typename E::type* k_row,
+                           const typename E::type* v_row, unsigned int dim, unsigned int value_dim, float scale,
+                           bool has_softcap, float softcap, float additive) {
+    float score = 0.0f;
+    if (k_row != nullptr)
+        for (unsigned int d = 0; d < dim; ++d) score = fmaf(q_row[d], E::load(k_row + d), score);
+    score *= scale;
+    if (has_softcap) score = tanhf(score / softcap) * softcap;
+    score += additive;
+    if (score == -INFINITY) return;
+    const float moved = fmaxf(state.largest, score);
+    const float rescale = expf(state.largest - moved);  // exp(-inf) = 0 on the first key
+    const float weight = expf(score - moved);
+    state.total = state.total * rescale + weight;
+    state.largest = moved;
+#pragma unroll
+    for (int d = 0; d < DMAX; ++d)
+        if (static_cast<unsigned int>(d) < value_dim)
+            state.acc[d] = fmaf(weight, v_row != nullptr ? E::load(v_row + d) : 0.0f, state.acc[d] * rescale);
+}
+
+// Merges the 64 lanes and writes the row.  `sink` joins the softmax without weighing a value
+// (attention.rs:255-262); pass -inf for none.  Returns max + ln(sum) of the row, -inf when it saw nothing.
+template <class E, int DMAX>
+SINGE_DEVICE float finish_row(const LaneState<DMAX>& state, typename E::type* out, unsigned int value_dim, unsigned int lane,
+                              float sink) {
+    float row_max = state.largest;
+#pragma unroll
+    for (int step = 32; step >= 1; step >>= 1) row_max = fmaxf(row_max, __shfl_xor(row_max, step, 64));
+    row_max = fmaxf(row_max, sink);
+    const float mine = state.largest == -INFINITY ? 0.0f : expf(state.largest - row_max);
+    float row_sum = state.total * mine;
+#pragma unroll
+    for (int step = 32; step >= 1; step >>= 1) row_sum += __shfl_xor(row_sum, step, 64);
+    if (sink != -INFINITY) row_sum += expf(sink - row_max);
+    const float inverse = row_sum > 0.0f ? 1.0f / row_sum : 0.0f;
+#pragma unroll
+    for (int d = 0; d < DMAX; ++d) {
+        if (static_cast<unsigned int>(d) < value_dim) {
+            float value = state.acc[d] * mine;
+#pragma unroll
+            for (int step = 32; step >= 1; step >>= 1) value += __shfl_xor(value, step, 64);
+            // A row that sees no key stays zero (attention.rs:503-515; a key count of zero gives zeros).
+            if (lane == (d & 63)) E::store(out + d, value * inverse);
+        }
+    }
+    return row_sum > 0.0f ? row_max + logf(row_sum) : -INFINITY;
+}
+
+template <uint32_t ELEMENT, int DMAX>
+SINGE_DEVICE void dense_body(const GeneralAttentionArgs& a, float* lds) {
+    typedef Element<ELEMENT> E;
+    typedef typename E::type T;
+    const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const unsigned long long row = static_cast<unsigned long long>(blockIdx.x) * 4 + wave;
+    const unsigned long long rows = static_cast<unsigned long long>(a.batch) * a.heads * a.query_len;
+    if (row >= rows) return;
+    const unsigned int query = static_cast<unsigned int>(row % a.query_len);
+    const unsigned int head = static_cast<unsigned int>((row / a.query_len) % a.heads);
+    const unsigned int batch = static_cast<unsigned int>(row / (static_cast<unsigned long long>(a.query_len) * a.heads));
+    const unsigned int kv_head = head / (a.heads / a.kv_heads);
+    const size_t kv_unit = static_cast<size_t>(batch) * a.kv_heads + kv_head;
+    const T* q = static_cast<const T*>(a.query) + row * a.head_dim;
+    const T* k = static_cast<const T*>(a.key) + kv_unit * a.key_len * a.head_dim;
+    const T* v = static_cast<const T*>(a.value) + kv_unit * a.key_len * a.value_dim;
+    const T* mask = a.mask == nullptr ? nullptr
+                                      : static_cast<const T*>(a.mask) + batch * a.mask_strides[0] + head * a.mask_strides[1] +
+                                            query * a.mask_strides[2];
+
+    float* q_row = lds + wave * DMAX;
+    for (unsigned int d = lane; d < a.head_dim; d += 64) q_row[d] = E::load(q + d);
+    __builtin_amdgcn_wave_barrier();
+
+    // Keys the row may see (attention.rs:225-246): top-left causal, per-batch key count, and the
+    // window's `key + window <= query` rule.
+    unsigned int first = 0, end = a.key_len;
+    if (a.causal && query + 1 < end) end = query + 1;
+    if (a.key_lengths != nullptr) {
+        const int length = a.key_lengths[batch];
+        const unsigned int bound = length > 0 ? static_cast<unsigned int>(length) : 0u;
+        if (bound < end) end = bound;
+    }
+    if (a.window >= 0) {
+        const unsigned long long window = static_cast<unsigned long long>(a.window);
+        if (static_cast<unsigned long long>(query) + 1 > window) first = static_cast<unsigned int>(query + 1 - window);
+    }
+
+    LaneState<DMAX> state;
+    reset(state);
+    for (unsigned int key = first + lane; key < end; key += 64) {
+        const float additive = mask != nullptr ? E::load(mask + key * a.mask_strides[3]) : 0.0f;
+        fold_key<E, DMAX>(state, q_row, k + static_cast<size_t>(key) * a.head_dim, v + static_cast<size_t>(key) * a.value_dim,
+                          a.head_dim, a.value_dim, a.scale, a.has_softcap != 0, a.softcap, additive);
+    }
+    const float sink = a.sinks != nullptr ? E::load(static_cast<const T*>(a.sinks) + head) : -INFINITY;
+    finish_row<E, DMAX>(state, static_cast<T*>(a.out) + row * a.value_dim, a.value_dim, lane, sink);
+}
+
+template <uint32_t ELEMENT, int DMAX, int FORM>
+SINGE_DEVICE void paged_rows(const GeneralPagedArgs& a, float* lds) {
+    typedef Element<ELEMENT> E;
+    typedef typename E::type T;
+    const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const unsigned int sequence = blockIdx.x / a.row_blocks;
+    const unsigned int local_row = (blockIdx.x % a.row_blocks) * 4 + wave;  // (query, head) of the sequence
+    const SequenceSpan span = load_span<FORM>(sequence, a.query_offsets, a.page_offsets, a.last_page_lengths, nullptr, a.tokens,
+                                              a.page_table, a.page_size);
+    if (!span.valid) {
+        if (threadIdx.x == 0) report_index_error(a.status);
+        return;
+    }
+    if (local_row >= span.queries * a.heads) return;
+    const unsigned int query = local_row / a.heads, head = local_row % a.heads;
+    const unsigned int kv_head = head / (a.heads / a.kv_heads);
+    const size_t flat = (static_cast<size_t>(span.query_start) + query) * a.heads + head;
+    const T* q = static_cast<const T*>(a.query_rows) + flat * a.head_dim;
+
+    float* q_row = lds + wave * DMAX;
+    for (unsigned int d = lane; d < a.head_dim; d += 64) q_row[d] = E::load(q + d);
+    __builtin_amdgcn_wave_barrier();
+
+    // Bottom-right alignment with the CPU path's saturating position (attention.rs:482-488).
+    const long long raw = static_cast<long long>(span.keys) - static_cast<long long>(span.queries) + query;
+    const unsigned int position = raw < 0 ? 0u : static_cast<unsigned int>(raw);
+    unsigned int first = 0, end = span.keys;
+    if (a.causal && position + 1 < end) end = position + 1;
+    if (a.window >= 0) {
+        const unsigned long long window = static_cast<unsigned long long>(a.window);
+        if (static_cast<unsigned long long>(position) + 1 > window) first = static_cast<unsigned int>(position + 1 - window);
+    }
+
+    LaneState<DMAX> state;
+    reset(state);
+    const T* key_cache = static_cast<const T*>(a.key_cache);
+    const T* value_cache = static_cast<const T*>(a.value_cache);
+    for (unsigned int key = first + lane; key < end; key += 64) {
+        const unsigned long long page = read_page<FORM>(a.pages, static_cast<size_t>(span.page_start) + key / a.page_size);
+        const bool valid = page < static_cast<unsigned long long>(a.cache_pages);
+        if (!valid) report_index_error(a.status);
+        // A key behind a bad page id is read as zeros; the status word tells the caller.
+        const size_t offset = ((page * a.page_size + key % a.page_size) * a.kv_heads + kv_head) * a.head_dim;
+        fold_key<E, DMAX>(state, q_row, valid ? key_cache + offset : nullptr, valid ? value_cache + offset : nullptr, a.head_dim,
+                          a.head_dim, a.scale, a.has_softcap != 0, a.softcap, 0.0f);
+    }
+    const float lse = finish_row<E, DMAX>(state, static_cast<T*>(a.output) + flat * a.head_dim, a.head_dim, lane, -INFINITY);
+    if (a.lse != nullptr && lane == 0) a.lse[flat] = lse * kLog2e;  // base two; -inf stays -inf
+}
+
+template <uint32_t ELEMENT, int DMAX>
+SINGE_DEVICE void paged_body(const GeneralPagedArgs& a, float* lds) {
+    if (a.wide_index)
+        paged_rows<ELEMENT, DMAX, kCsrI64>(a, lds);
+    else
+        paged_rows<ELEMENT, DMAX, kCsrI32>(a, lds);
+}
+
+}  // namespace general
+
+#define SINGE_GENERAL_KERNELS(TAG, ELEMENT, DMAX)                                                                            \
+    extern "C" __global__ __launch_bounds__(256) void singe_attention_general_##TAG##_d##DMAX(GeneralAttentionArgs args) {   \
+        __shared__ float rows[4 * DMAX];                                                                                     \
+        general::dense_body<ELEMENT, DMAX>(args, rows);                                                                      \
+    }                                                                                                                        \
+    extern "C" __global__ __launch_bounds__(256) void singe_paged_attention_general_##TAG##_d##DMAX(GeneralPagedArgs args) { \
+        __shared__ float rows[4 * DMAX];                                                                                     \
+        general::paged_body<ELEMENT, DMAX>(args, rows);                                                                      \
+    }
+
+SINGE_GENERAL_KERNELS(f32, kElementF32, 64)
+SINGE_GENERAL_KERNELS(f32, kElementF32, 128)
+SINGE_GENERAL_KERNELS(f32, kElementF32, 256)
+SINGE_GENERAL_KERNELS(bf16, kElementBf16, 64)
+SINGE_GENERAL_KERNELS(bf16, kElementBf16, 128)
+SINGE_GENERAL_KERNELS(bf16, kElementBf16, 256)
+SINGE_GENERAL_KERNELS(f16, kElementF16, 64)
+SINGE_GENERAL_KERNELS(f16, kElementF16, 128)
+SINGE_GENERAL_KERNELS(f16, kElementF16, 256)

@@ -112,3 +112,53 @@ struct PagedAttentionArgs {
     float softcap_scale;            // scale / cap
     float softcap_log2e;            // cap * log2(e)
 };
+
+// singe_splitk_reduce_f32: strides in elements.
+struct SplitKReduceArgs {
+    float* out;         // [batch, heads, dim]
+    const float* attn;  // [batch, heads, splits, dim]
+    const float* lse;   // [batch, heads, splits] natural log
+    uint64_t attn_batch_stride, attn_head_stride, attn_split_stride;
+    uint64_t lse_batch_stride, lse_head_stride;
+    uint64_t output_batch_stride, output_head_stride;
+    uint32_t batch, heads, splits, head_dim;
+};
+
+// Element types of the general (any head dimension) kernels.
+enum SingeElement : uint32_t { kElementF32 = 0, kElementBf16 = 1, kElementF16 = 2 };
+
+// singe_attention_general_*: dense attention over [batch, heads, len, dim] tensors with every option
+// of ScaledDotProductAttentionAttributes.
+struct GeneralAttentionArgs {
+    const void* query;              // [batch, heads, query_len, head_dim]
+    const void* key;                // [batch, kv_heads, key_len, head_dim]
+    const void* value;              // [batch, kv_heads, key_len, value_dim]
+    const void* mask;               // additive, element type of the query, strides below; or null
+    const void* sinks;              // [heads], element type of the query; or null
+    const int32_t* key_lengths;     // [batch]; or null
+    void* out;                      // [batch, heads, query_len, value_dim]
+    uint64_t mask_strides[4];       // over (batch, head, query, key); 0 broadcasts
+    int64_t window;                 // -1 = none
+    uint32_t batch, heads, kv_heads, query_len, key_len, head_dim, value_dim;
+    uint32_t causal, has_softcap;
+    float scale, softcap;
+};
+
+// singe_paged_attention_general_*: the FlashInfer-form paged op for any element type and head dimension.
+struct GeneralPagedArgs {
+    const void* query_rows;         // [tokens, heads, head_dim]
+    const void* key_cache;          // [cache_pages, page_size, kv_heads, head_dim]
+    const void* value_cache;
+    const void* query_offsets;
+    const void* page_offsets;
+    const void* pages;
+    const void* last_page_lengths;
+    void* output;                   // [tokens, heads, head_dim]
+    float* lse;                     // [tokens, heads] base two, or null
+    uint32_t* status;
+    int64_t window;
+    uint32_t tokens, heads, kv_heads, head_dim, page_size, sequences, cache_pages, page_table;
+    uint32_t row_blocks;            // workgroups (4 rows each) per sequence
+    uint32_t causal, has_softcap, wide_index;
+    float scale, softcap;
+};

@@ -18,7 +18,11 @@ enum KernelId : int {
     kPrefillF32D32, kPrefillF32D64, kPrefillF32D128, kPrefillF32D256,
     kPagedAttentionI32, kPagedAttentionI64, kPagedAttentionSoftcapI32, kPagedAttentionSoftcapI64,
     kPagedKvPrefill,
-    kKernelCount
+    kSplitKReduce,
+    // general kernels: index = base + 3 * element (f32, bf16, f16) + width (64, 128, 256)
+    kDenseGeneral,
+    kPagedGeneral = kDenseGeneral + 9,
+    kKernelCount = kPagedGeneral + 9
 };
 
 extern const char* const kKernelNames[kKernelCount];

@@ -11,11 +11,19 @@
 
 using namespace singe_hip;
 
-extern "C" int32_t singe_hip_paged_attention_bf16(void* stream, const uint16_t* query_rows, const uint16_t* key_cache,
-                                                  const uint16_t* value_cache, const void* query_offsets,
-                                                  const void* page_offsets, const void* pages,
-                                                  const void* last_page_lengths, uint16_t* output, float* lse,
-                                                  uint32_t* status, const SingePagedAttentionProblem* problem) {
+namespace singe_hip {
+int32_t paged_attention_general(int32_t data_type, void* stream, const void* query_rows, const void* key_cache,
+                                const void* value_cache, const void* query_offsets, const void* page_offsets,
+                                const void* pages, const void* last_page_lengths, void* output, float* lse, uint32_t* status,
+                                const SingePagedAttentionProblem& p, float scale);
+}
+
+namespace {
+
+int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_any, const void* key_cache_any,
+                        const void* value_cache_any, const void* query_offsets, const void* page_offsets, const void* pages,
+                        const void* last_page_lengths, void* output_any, float* lse, uint32_t* status,
+                        const SingePagedAttentionProblem* problem) {
     if (problem == nullptr) return fail(SINGE_HIP_NULL_POINTER, "problem");
     const SingePagedAttentionProblem& p = *problem;
     // paged_attention_problem: key_dim == head_dim (one field here), kv_heads > 0 dividing heads, page_size > 0.
@@ -30,15 +38,24 @@ extern "C" int32_t singe_hip_paged_attention_bf16(void* stream, const uint16_t* 
     const int64_t extents[] = {p.tokens, p.heads, p.kv_heads, p.page_size, p.sequences, p.cache_pages, p.page_table};
     for (int64_t extent : extents)
         if (!fits_i32(static_cast<uint64_t>(extent))) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "problem");
-    // The tensor-core kernel takes head dimensions that are multiples of 16 up to 128
-    // (paged_attention.rs:586-592); this build covers 128, the general kernel is not part of it.
-    if (p.head_dim != 128) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, "paged_attention", static_cast<uint64_t>(p.head_dim), 0);
+    if (!fits_i32(static_cast<uint64_t>(p.head_dim))) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "problem");
     if (p.tokens == 0 || p.sequences == 0) return 0;  // nothing to attend
-    const void* pointers[] = {query_rows, key_cache, value_cache, query_offsets, page_offsets, last_page_lengths, output};
+    const void* pointers[] = {query_rows_any, key_cache_any, value_cache_any, query_offsets, page_offsets, last_page_lengths, output_any};
     const char* names[] = {"query_rows", "key_cache", "value_cache", "query_offsets", "page_offsets", "last_page_lengths", "output"};
     for (int i = 0; i < 7; ++i)
         if (pointers[i] == nullptr) return fail(SINGE_HIP_NULL_POINTER, names[i]);
     if (pages == nullptr && p.page_table > 0) return fail(SINGE_HIP_NULL_POINTER, "pages");
+    const float scale = p.has_scale ? p.scale : 1.0f / std::sqrt(static_cast<float>(p.head_dim));
+    // The tensor-core kernel covers bf16 at head dimension 128 (the reference's takes f16/bf16 at
+    // multiples of 16 up to 128: paged_attention.rs:586-592); everything else goes to the general one
+    // (paged_general.rs:73-247).
+    if (data_type != SINGE_HIP_BF16 || p.head_dim != 128)
+        return paged_attention_general(data_type, stream, query_rows_any, key_cache_any, value_cache_any, query_offsets,
+                                       page_offsets, pages, last_page_lengths, output_any, lse, status, p, scale);
+    const uint16_t* query_rows = static_cast<const uint16_t*>(query_rows_any);
+    const uint16_t* key_cache = static_cast<const uint16_t*>(key_cache_any);
+    const uint16_t* value_cache = static_cast<const uint16_t*>(value_cache_any);
+    uint16_t* output = static_cast<uint16_t*>(output_any);
 
     const uint64_t groups = static_cast<uint64_t>(p.heads / p.kv_heads);
     PagedAttentionArgs args;
@@ -63,7 +80,6 @@ extern "C" int32_t singe_hip_paged_attention_bf16(void* stream, const uint16_t* 
     args.page_table = static_cast<uint32_t>(p.page_table);
     args.row_tiles = static_cast<uint32_t>((groups * static_cast<uint64_t>(p.tokens) + 127) / 128);
     args.causal = p.causal ? 1u : 0u;
-    const float scale = p.has_scale ? p.scale : 1.0f / std::sqrt(static_cast<float>(p.head_dim));
     constexpr float kLog2e = 1.4426950408889634074f;
     args.scale_log2e = scale * kLog2e;
     args.softcap_scale = p.has_softcap ? scale / p.softcap : 0.0f;
@@ -75,6 +91,33 @@ extern "C" int32_t singe_hip_paged_attention_bf16(void* stream, const uint16_t* 
     const KernelId kernel = p.has_softcap ? (wide ? kPagedAttentionSoftcapI64 : kPagedAttentionSoftcapI32)
                                           : (wide ? kPagedAttentionI64 : kPagedAttentionI32);
     return launch(kernel, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+}
+
+}  // namespace
+
+extern "C" int32_t singe_hip_paged_attention_bf16(void* stream, const uint16_t* query_rows, const uint16_t* key_cache,
+                                                  const uint16_t* value_cache, const void* query_offsets,
+                                                  const void* page_offsets, const void* pages,
+                                                  const void* last_page_lengths, uint16_t* output, float* lse,
+                                                  uint32_t* status, const SingePagedAttentionProblem* problem) {
+    return paged_attention(SINGE_HIP_BF16, stream, query_rows, key_cache, value_cache, query_offsets, page_offsets, pages,
+                           last_page_lengths, output, lse, status, problem);
+}
+
+extern "C" int32_t singe_hip_paged_attention_f32(void* stream, const float* query_rows, const float* key_cache,
+                                                 const float* value_cache, const void* query_offsets, const void* page_offsets,
+                                                 const void* pages, const void* last_page_lengths, float* output, float* lse,
+                                                 uint32_t* status, const SingePagedAttentionProblem* problem) {
+    return paged_attention(SINGE_HIP_F32, stream, query_rows, key_cache, value_cache, query_offsets, page_offsets, pages,
+                           last_page_lengths, output, lse, status, problem);
+}
+
+extern "C" int32_t singe_hip_paged_attention_f16(void* stream, const uint16_t* query_rows, const uint16_t* key_cache,
+                                                 const uint16_t* value_cache, const void* query_offsets, const void* page_offsets,
+                                                 const void* pages, const void* last_page_lengths, uint16_t* output, float* lse,
+                                                 uint32_t* status, const SingePagedAttentionProblem* problem) {
+    return paged_attention(SINGE_HIP_F16, stream, query_rows, key_cache, value_cache, query_offsets, page_offsets, pages,
+                           last_page_lengths, output, lse, status, problem);
 }
 
 // validate_paged_kv_prefill_attention_config (singe-kernel/src/cuda/attention/mod.rs:2987-3011).

@@ -25,31 +25,12 @@
 // the queries, the page table or the cache sets the status word to 1 (first writer wins; the word may
 // be null) and nothing is read through it (paged_attention.rs:41-54, 210-262, 739-755).
 #include "kernel_args.h"
+#include "paging.hip.h"
 #include "prefill_core.hip.h"
 
 namespace {
 
 using namespace prefill;
-
-// How the paging arrives: FlashInfer CSR vectors of i32 or i64, or the block table of the
-// singe-kernel surface (u32 table rows, i32 per-sequence query offsets and lengths).
-enum : int { kCsrI32 = 0, kCsrI64 = 1, kTable = 2 };
-
-template <int FORM>
-SINGE_DEVICE long long read_index(const void* values, size_t at) {
-    if constexpr (FORM == kCsrI64)
-        return static_cast<const long long*>(values)[at];
-    else
-        return static_cast<long long>(static_cast<const int*>(values)[at]);
-}
-
-template <int FORM>
-SINGE_DEVICE unsigned long long read_page(const void* pages, size_t at) {
-    if constexpr (FORM == kTable)
-        return static_cast<const unsigned int*>(pages)[at];
-    else
-        return static_cast<unsigned long long>(read_index<FORM>(pages, at));  // negative ids wrap above any cache
-}
 
 template <bool SOFTCAP, int FORM>
 SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned char* lds) {
@@ -64,41 +45,17 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     const unsigned int sequence = unit / a.kv_heads, kv_head = unit % a.kv_heads;
     const unsigned int first_row = (within % a.row_tiles) * kQueryTile;
 
-    // The sequence's paging values, refused when any would address outside the kernel's buffers
-    // (paged_attention.rs:210-238; the CPU check is spec/neural/attention.rs:372-406).
-    long long query_start, query_count, page_start, key_count;
-    if constexpr (FORM == kTable) {
-        // Block-table form (singe-kernel/src/cpu/attention.rs:1272-1276): offsets, query and key
-        // lengths per sequence; row `sequence` of the table holds its blocks.
-        query_start = read_index<FORM>(a.query_offsets, sequence);
-        query_count = read_index<FORM>(a.query_lengths, sequence);
-        key_count = read_index<FORM>(a.last_page_lengths, sequence);
-        page_start = static_cast<long long>(sequence) * a.page_table;
-        if (query_start < 0 || query_count < 0 || query_start + query_count > static_cast<long long>(a.tokens) || key_count < 0 ||
-            key_count > static_cast<long long>(a.page_table) * a.page_size) {
-            if (tid == 0) report_index_error(a.status);
-            return;
-        }
-    } else {
-        query_start = read_index<FORM>(a.query_offsets, sequence);
-        const long long query_end = read_index<FORM>(a.query_offsets, sequence + 1);
-        page_start = read_index<FORM>(a.page_offsets, sequence);
-        const long long page_end = read_index<FORM>(a.page_offsets, sequence + 1);
-        const long long last_length = read_index<FORM>(a.last_page_lengths, sequence);
-        if (query_start < 0 || query_end < query_start || query_end > static_cast<long long>(a.tokens) || page_start < 0 ||
-            page_end < page_start || page_end > static_cast<long long>(a.page_table) ||
-            (page_end > page_start && (last_length < 0 || last_length > static_cast<long long>(a.page_size)))) {
-            if (tid == 0) report_index_error(a.status);
-            return;
-        }
-        query_count = query_end - query_start;
-        const long long page_count = page_end - page_start;
-        key_count = page_count == 0 ? 0 : (page_count - 1) * a.page_size + last_length;
+    // The sequence's paging values, refused when any would address outside the kernel's buffers.
+    const SequenceSpan span = load_span<FORM>(sequence, a.query_offsets, a.page_offsets, a.last_page_lengths, a.query_lengths,
+                                              a.tokens, a.page_table, a.page_size);
+    if (!span.valid) {
+        if (tid == 0) report_index_error(a.status);
+        return;
     }
-    const unsigned int queries = static_cast<unsigned int>(query_count);
+    const long long query_start = span.query_start, page_start = span.page_start;
+    const unsigned int queries = span.queries, keys = span.keys;
     const unsigned int packed = queries * groups;
     if (first_row >= packed) return;
-    const unsigned int keys = static_cast<unsigned int>(key_count);
 
     // Key position of packed row r: max(keys - queries + r / groups, 0); the block-table form aligns
     // queries with the FIRST keys instead (key > query index is hidden, cpu/attention.rs:1283).

@@ -1,0 +1,67 @@
+// Reading and checking one sequence's paging values on the device, shared by the paged kernels.
+// Paging arrives as FlashInfer CSR vectors of i32 or i64 (singe/src/tensor/neural.rs:409-457), or as the
+// block table of the singe-kernel surface: u32 table rows plus i32 per-sequence query offsets, query
+// lengths and key lengths (singe-kernel/src/cpu/attention.rs:1248-1276).
+#pragma once
+
+#include "common.hip.h"
+
+enum : int { kCsrI32 = 0, kCsrI64 = 1, kTable = 2 };
+
+template <int FORM>
+SINGE_DEVICE long long read_index(const void* values, size_t at) {
+    if constexpr (FORM == kCsrI64)
+        return static_cast<const long long*>(values)[at];
+    else
+        return static_cast<long long>(static_cast<const int*>(values)[at]);
+}
+
+template <int FORM>
+SINGE_DEVICE unsigned long long read_page(const void* pages, size_t at) {
+    if constexpr (FORM == kTable)
+        return static_cast<const unsigned int*>(pages)[at];
+    else
+        return static_cast<unsigned long long>(read_index<FORM>(pages, at));  // negative ids wrap above any cache
+}
+
+struct SequenceSpan {
+    long long query_start;  // first token of the sequence in the packed queries
+    long long page_start;   // first entry of the sequence in `pages`
+    unsigned int queries;
+    unsigned int keys;
+    bool valid;             // false: some value would address outside the queries or the page table
+};
+
+// The checks of paged_attention.rs:210-238 (CPU: spec/neural/attention.rs:372-406): offsets monotone
+// inside [0, tokens] / [0, page_table], last_page_length in [0, page_size] unless the sequence has no
+// pages.  keys = (page_count - 1) * page_size + last_page_length (paged_attention.rs:256).
+template <int FORM>
+SINGE_DEVICE SequenceSpan load_span(unsigned int sequence, const void* query_offsets, const void* page_offsets,
+                                    const void* last_page_lengths, const void* query_lengths, unsigned int tokens,
+                                    unsigned int page_table, unsigned int page_size) {
+    SequenceSpan span;
+    long long query_count, key_count;
+    if constexpr (FORM == kTable) {
+        span.query_start = read_index<FORM>(query_offsets, sequence);
+        query_count = read_index<FORM>(query_lengths, sequence);
+        key_count = read_index<FORM>(last_page_lengths, sequence);
+        span.page_start = static_cast<long long>(sequence) * page_table;
+        span.valid = !(span.query_start < 0 || query_count < 0 || span.query_start + query_count > static_cast<long long>(tokens) ||
+                       key_count < 0 || key_count > static_cast<long long>(page_table) * page_size);
+    } else {
+        span.query_start = read_index<FORM>(query_offsets, sequence);
+        const long long query_end = read_index<FORM>(query_offsets, sequence + 1);
+        span.page_start = read_index<FORM>(page_offsets, sequence);
+        const long long page_end = read_index<FORM>(page_offsets, sequence + 1);
+        const long long last_length = read_index<FORM>(last_page_lengths, sequence);
+        span.valid = !(span.query_start < 0 || query_end < span.query_start || query_end > static_cast<long long>(tokens) ||
+                       span.page_start < 0 || page_end < span.page_start || page_end > static_cast<long long>(page_table) ||
+                       (page_end > span.page_start && (last_length < 0 || last_length > static_cast<long long>(page_size))));
+        query_count = query_end - span.query_start;
+        const long long page_count = page_end - span.page_start;
+        key_count = page_count == 0 ? 0 : (page_count - 1) * page_size + last_length;
+    }
+    span.queries = span.valid ? static_cast<unsigned int>(query_count) : 0u;
+    span.keys = span.valid ? static_cast<unsigned int>(key_count) : 0u;
+    return span;
+}

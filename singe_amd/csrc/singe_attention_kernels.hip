@@ -4,3 +4,5 @@
 #include "fmha_prefill.hip"
 #include "fmha_prefill_f32.hip"
 #include "paged_attention.hip"
+#include "splitk_reduce.hip"
+#include "general_attention.hip"

@@ -19,6 +19,10 @@ class LengthTooShort(Error):
         self.name, self.minimum, self.actual = name, minimum, actual
 
 
+class LengthMismatch(Error):
+    """Two extents that must agree differ (Error::LengthMismatch)."""
+
+
 class LengthExceedsI32(Error):
     """A dimension cannot fit the native signed 32-bit interface (Error::LengthExceedsI32)."""
 

@@ -367,3 +367,43 @@ def bhsd_config(batch, heads, kv_heads, query_len, key_len, head_dim, scale, cau
                              heads * query_len * head_dim, head_dim, head_dim, head_dim, head_dim,
                              query_len * head_dim, key_len * head_dim, key_len * head_dim, query_len * head_dim,
                              scale, causal)
+
+
+@dataclass(frozen=True)
+class SplitKReduceConfig:
+    """SplitKReduceConfig (mod.rs:385-398): strides in elements."""
+    batch: int
+    heads: int
+    splits: int
+    head_dim: int
+    attn_batch_stride: int
+    attn_head_stride: int
+    attn_split_stride: int
+    lse_batch_stride: int
+    lse_head_stride: int
+    output_batch_stride: int
+    output_head_stride: int
+
+    @classmethod
+    def contiguous(cls, batch, heads, splits, head_dim) -> "SplitKReduceConfig":
+        """mod.rs:2312-2328: attn [batch, heads, splits, dim], lse [batch, heads, splits], out [batch, heads, dim]."""
+        return cls(batch, heads, splits, head_dim, heads * splits * head_dim, splits * head_dim, head_dim,
+                   heads * splits, splits, heads * head_dim, head_dim)
+
+    def _c(self) -> _native.SplitKReduceConfigC:
+        return _native.SplitKReduceConfigC(self.batch, self.heads, self.splits, self.head_dim, self.attn_batch_stride,
+                                           self.attn_head_stride, self.attn_split_stride, self.lse_batch_stride,
+                                           self.lse_head_stride, self.output_batch_stride, self.output_head_stride)
+
+
+def splitk_reduce_f32(stream, out: torch.Tensor, attn_splitk: torch.Tensor, lse_splitk: torch.Tensor,
+                      config: SplitKReduceConfig) -> None:
+    """splitk_reduce_f32 (fmha.rs:1038-1067): folds per-split partial rows and natural-log LSEs."""
+    _require(out, torch.float32, "out")
+    _require(attn_splitk, torch.float32, "attn_splitk")
+    _require(lse_splitk, torch.float32, "lse_splitk")
+    c = config._c()
+    status = _native.lib().singe_hip_splitk_reduce_f32(_stream_handle(stream), _ptr(out), out.numel(), _ptr(attn_splitk),
+                                                       attn_splitk.numel(), _ptr(lse_splitk), lse_splitk.numel(),
+                                                       ctypes.byref(c))
+    _native.check(status, "splitk_reduce_f32")

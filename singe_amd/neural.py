@@ -1,7 +1,8 @@
 """Host-side mirror of the ``singe`` crate's attention ops on tensors
-(singe/src/tensor/neural.rs:25-32, 409-457): ``AttentionOptions``, ``Paging`` and
-``paged_attention``, which attends ragged queries over a paged key/value cache as FlashInfer batches
-decode and prefill, and returns the output and each row's base-two log-sum-exp."""
+(singe/src/tensor/neural.rs:25-32, 92-175, 409-457): ``AttentionOptions``, the dense
+``scaled_dot_product_attention`` / ``attend`` / ``attend_padded``, and ``Paging`` with ``paged_attention``,
+which attends ragged queries over a paged key/value cache as FlashInfer batches decode and prefill, and
+returns the output and each row's base-two log-sum-exp."""
 from __future__ import annotations
 
 import ctypes
@@ -64,19 +65,103 @@ def _problem(query, key_cache, value_cache, paging: Paging, options: AttentionOp
         options.softcap if options.softcap is not None else 0.0, options.window if options.window is not None else 0)
 
 
+_DATA_TYPES = {torch.float32: _native.DATA_TYPE_F32, torch.bfloat16: _native.DATA_TYPE_BF16,
+               torch.float16: _native.DATA_TYPE_F16}
+
+
+def scaled_dot_product_attention(query, key, value, scale: float | None = None, causal: bool = False, *, stream=None):
+    """Tensor::scaled_dot_product_attention (tensor/neural.rs:92-110)."""
+    return _attend_all(query, key, value, None, None, None, AttentionOptions(scale=scale, causal=causal), stream)
+
+
+def attend(query, key, value, mask=None, sinks=None, options: AttentionOptions = AttentionOptions(), *, stream=None):
+    """Tensor::attend (tensor/neural.rs:112-124): a ``mask`` broadcast to the scores' [B, H, L, S] adds to
+    them after any cap (a Boolean mask lets the keys where it holds take part and hides the others);
+    ``sinks``, one logit per query head, join each row's softmax without weighing a value."""
+    return _attend_all(query, key, value, mask, sinks, None, options, stream)
+
+
+def attend_padded(query, key, value, key_lengths, options: AttentionOptions = AttentionOptions(), *, stream=None):
+    """Tensor::attend_padded (tensor/neural.rs:126-137): batch b attends to its first key_lengths[b] keys
+    ([B] int32); a batch of no keys gives zeros."""
+    return _attend_all(query, key, value, None, None, key_lengths, options, stream)
+
+
+def _attend_all(query, key, value, mask, sinks, key_lengths, options, stream):
+    """attend_all (tensor/neural.rs:139-175) with the shape rules of spec::attention_problem
+    (singe/src/backend/spec/neural/attention.rs:209-290)."""
+    for tensor, name in ((query, "query"), (key, "key"), (value, "value")):
+        if tensor.dim() != 4:
+            raise error.InvalidArgument(f"scaled dot-product attention {name} rank")
+        if not tensor.is_cuda or tensor.dtype != query.dtype or not tensor.is_contiguous():
+            raise error.InvalidArgument(f"scaled dot-product attention {name} must be a contiguous device tensor of the query's type")
+    if query.dtype not in _DATA_TYPES:
+        raise error.InvalidArgument(f"scaled dot-product attention data type {query.dtype}")
+    batch, heads, query_len, head_dim = query.shape
+    key_batch, kv_heads, key_len, key_dim = key.shape
+    value_batch, value_heads, value_len, value_dim = value.shape
+    if head_dim <= 0 or key_len <= 0:
+        raise error.InvalidArgument("scaled dot-product attention head dimension and key length must be positive")
+    if batch != key_batch or batch != value_batch:
+        raise error.LengthMismatch("scaled dot-product attention batch")
+    if kv_heads == 0 or heads % kv_heads != 0:
+        raise error.InvalidArgument("scaled dot-product attention key heads must divide the query heads")
+    if kv_heads != value_heads or head_dim != key_dim or key_len != value_len:
+        raise error.LengthMismatch("scaled dot-product attention key and value shapes")
+    strides = [0, 0, 0, 0]
+    if mask is not None:
+        if mask.dtype == torch.bool:
+            mask = torch.where(mask, 0.0, float("-inf")).to(query.dtype)
+        else:
+            mask = mask.to(query.dtype)
+        if mask.dim() > 4:
+            raise error.InvalidArgument("scaled dot-product attention mask rank")
+        shape = (1,) * (4 - mask.dim()) + tuple(mask.shape)
+        target = (batch, heads, query_len, key_len)
+        if any(have not in (1, want) for have, want in zip(shape, target)):
+            raise error.InvalidArgument("scaled dot-product attention mask does not broadcast to the scores")
+        mask = mask.contiguous().reshape(shape)
+        strides = [0 if have == 1 else stride for have, stride in zip(shape, mask.stride())]
+    if sinks is not None:
+        if sinks.numel() != heads:
+            raise error.InvalidArgument("scaled dot-product attention sinks must hold one logit per query head")
+        sinks = sinks.to(query.dtype).contiguous()
+    if key_lengths is not None:
+        if key_lengths.dtype != torch.int32 or key_lengths.numel() != batch:
+            raise error.InvalidArgument("scaled dot-product attention key lengths must be [batch] int32")
+        key_lengths = key_lengths.contiguous()
+    problem = _native.AttentionProblemC(
+        batch, heads, kv_heads, query_len, key_len, head_dim, value_dim, (ctypes.c_int64 * 4)(*strides),
+        _DATA_TYPES[query.dtype], 1 if options.causal else 0, 1 if options.scale is not None else 0,
+        1 if options.window is not None else 0, 1 if options.softcap is not None else 0,
+        options.scale if options.scale is not None else 0.0, options.softcap if options.softcap is not None else 0.0,
+        options.window if options.window is not None else 0)
+    output = torch.empty((batch, heads, query_len, value_dim), device=query.device, dtype=query.dtype)
+    handle = int((stream or torch.cuda.current_stream()).cuda_stream)
+    pointer = lambda tensor: tensor.data_ptr() if tensor is not None else None
+    code = _native.lib().singe_hip_scaled_dot_product_attention(
+        handle, query.data_ptr(), key.data_ptr(), value.data_ptr(), pointer(mask), pointer(sinks), pointer(key_lengths),
+        output.data_ptr(), ctypes.byref(problem))
+    _native.check(code, "scaled_dot_product_attention")
+    return output
+
+
 def paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor, paging: Paging,
                     options: AttentionOptions = AttentionOptions(), *, stream=None, status: torch.Tensor | None = None,
                     check: bool = True):
-    """Tensor::paged_attention (tensor/neural.rs:420-457) for bf16 tensors on the GPU.
+    """Tensor::paged_attention (tensor/neural.rs:420-457) for bf16, f16 or f32 tensors on the GPU; bf16 at
+    head dimension 128 runs on the matrix cores, everything else on the general kernel.
 
-    Returns (output [tokens, heads, dim] bf16, lse [tokens, heads] f32 base two).  Like the reference's
+    Returns (output [tokens, heads, dim] of the query's type, lse [tokens, heads] f32 base two).  Like the reference's
     eager launch (kernel_plan/mod.rs:156-251) it zeroes a status word, launches, and reads the word
     back: a paging value outside its buffers raises IndexOutOfBounds.  ``check=False`` skips the
     read-back (and the synchronisation it implies); pass ``status`` to inspect the word yourself.
     """
     for tensor, name in ((query, "query"), (key_cache, "key_cache"), (value_cache, "value_cache")):
-        if not tensor.is_cuda or tensor.dtype != torch.bfloat16 or not tensor.is_contiguous():
-            raise error.InvalidArgument(f"paged attention {name} must be a contiguous bf16 device tensor")
+        if not tensor.is_cuda or tensor.dtype != query.dtype or not tensor.is_contiguous():
+            raise error.InvalidArgument(f"paged attention {name} must be a contiguous device tensor of the query's type")
+    if query.dtype not in _DATA_TYPES:
+        raise error.InvalidArgument(f"paged attention data type {query.dtype}")
     for tensor in (paging.query_offsets, paging.page_offsets, paging.pages, paging.last_page_lengths):
         if not tensor.is_cuda or not tensor.is_contiguous():
             raise error.InvalidArgument("paged attention index tensors must be contiguous device tensors")
@@ -86,7 +171,10 @@ def paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: t
     if status is None:
         status = torch.zeros(1, device=query.device, dtype=torch.int32)
     handle = int((stream or torch.cuda.current_stream()).cuda_stream)
-    code = _native.lib().singe_hip_paged_attention_bf16(
+    entry = {torch.bfloat16: _native.lib().singe_hip_paged_attention_bf16,
+             torch.float32: _native.lib().singe_hip_paged_attention_f32,
+             torch.float16: _native.lib().singe_hip_paged_attention_f16}[query.dtype]
+    code = entry(
         handle, query.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), paging.query_offsets.data_ptr(),
         paging.page_offsets.data_ptr(), paging.pages.data_ptr(), paging.last_page_lengths.data_ptr(),
         output.data_ptr(), lse.data_ptr(), status.data_ptr(), ctypes.byref(problem))

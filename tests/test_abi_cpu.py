@@ -117,5 +117,48 @@ def test_paged_attention_problem_validation():
     assert call(heads=3) == 9
     assert call(page_size=0) == 9
     assert call(index_type=7) == 9
-    assert call(head_dim=64) == 5
+    assert call(head_dim=300) == 5  # beyond the general kernel's 256
+    detail = _native.ErrorDetail()
+    lib.singe_hip_last_error(ctypes.byref(detail))
+    assert detail.actual == 300
     assert call(tokens=0) == 0  # nothing to attend, nothing launched
+
+
+def test_paged_kv_prefill_config_validation_mirrors_reference_cases():
+    """singe-kernel/src/cuda/attention/tests.rs:349-375."""
+    lib = _native.lib()
+    good = _native.PagedKvPrefillAttentionConfigC(2, 7, 4, 2, 8, 3, 5, 4, 1, 0.5)
+    assert lib.singe_hip_paged_kv_prefill_attention_config_validate(ctypes.byref(good)) == 0
+    bad_heads = _native.PagedKvPrefillAttentionConfigC(2, 7, 3, 2, 8, 3, 5, 4, 1, 0.5)
+    assert lib.singe_hip_paged_kv_prefill_attention_config_validate(ctypes.byref(bad_heads)) == 1
+    fake = 0x1000
+    status = lib.singe_hip_paged_kv_prefill_attention_bf16(None, fake, 224, fake, 27, fake, 224, fake, 240, fake, 240, fake, 2,
+                                                           fake, 2, fake, 2, fake, 8, ctypes.byref(good))
+    assert status == 2
+    detail = _native.ErrorDetail()
+    lib.singe_hip_last_error(ctypes.byref(detail))
+    assert detail.name == b"lse" and detail.minimum == 28 and detail.actual == 27
+
+
+def test_dense_problem_and_splitk_validation():
+    lib = _native.lib()
+    fake = 0x1000
+    def dense(**changes):
+        fields = dict(batch=1, heads=4, kv_heads=2, query_len=3, key_len=5, head_dim=64, value_dim=64,
+                      mask_strides=(ctypes.c_int64 * 4)(0, 0, 0, 0), data_type=0, causal=0, has_scale=0, has_window=0,
+                      has_softcap=0, scale=0.0, softcap=0.0, window=0)
+        fields.update(changes)
+        problem = _native.AttentionProblemC(*fields.values())
+        return lib.singe_hip_scaled_dot_product_attention(None, fake, fake, fake, None, None, None, fake, ctypes.byref(problem))
+    assert dense(kv_heads=3) == 9
+    assert dense(key_len=0) == 9
+    assert dense(head_dim=0) == 9
+    assert dense(data_type=5) == 9
+    assert dense(head_dim=257) == 5
+    assert dense(query_len=0) == 0  # an empty output, nothing launched
+    assert dense(has_softcap=1, softcap=0.0) == 9
+    config = _native.SplitKReduceConfigC(1, 2, 5, 8, 80, 40, 8, 10, 5, 16, 8)
+    assert lib.singe_hip_splitk_reduce_f32(None, fake, 16, fake, 80, fake, 10, ctypes.byref(config)) != 2
+    assert lib.singe_hip_splitk_reduce_f32(None, fake, 16, fake, 79, fake, 10, ctypes.byref(config)) == 2
+    zero = _native.SplitKReduceConfigC(1, 2, 0, 8, 80, 40, 8, 10, 5, 16, 8)
+    assert lib.singe_hip_splitk_reduce_f32(None, fake, 16, fake, 80, fake, 10, ctypes.byref(zero)) == 1
