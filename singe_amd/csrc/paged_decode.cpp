@@ -239,7 +239,7 @@ int32_t decode(
     combine.workers = plan.workers;
     combine.head_groups = plan.head_groups;
     combine.heads_per_wave = plan.heads_per_wave;
-    return launch(kDecodeCombine, static_cast<unsigned>(c.batch * c.heads), 1, 1, 128, stream, combine);
+    return launch(kDecodeCombine, static_cast<unsigned>((c.batch * c.heads + 3) / 4), 1, 1, 256, stream, combine);
 }
 
 }  // namespace

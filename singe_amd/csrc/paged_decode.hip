@@ -578,33 +578,65 @@ SINGE_DECODE_KERNEL(singe_paged_decode_f8kv_relaxed_d128_g2_any, 2, false, true,
 
 // Folds the partial rows of one (sequence, query head) into the bf16 output:
 // out = sum_s exp(lse_s - max) * partial_s / sum_s exp(lse_s - max)
-// (singe-kernel/src/cpu/attention.rs:2157-2193).  One workgroup per row, one thread per dimension.
-extern "C" __global__ __launch_bounds__(128) void singe_paged_decode_combine_bf16(CombineArgs a) {
-    const unsigned int row = blockIdx.x;  // batch * heads + head
+// (singe-kernel/src/cpu/attention.rs:2157-2193).  One wave per row.  The kernel is a chain of dependent
+// memory round trips, so it is written to need few of them: lane s fetches the log-sum-exp of slot s
+// (one trip for up to 64 slots), and the slots' rows are fetched sixteen at a time, two dims per lane.
+extern "C" __global__ __launch_bounds__(256) void singe_paged_decode_combine_bf16(CombineArgs a) {
+    const unsigned int lane = threadIdx.x & 63;
+    const unsigned int row = blockIdx.x * 4 + (threadIdx.x >> 6);  // batch * heads + head
+    if (row >= a.batch * a.heads) return;
     const unsigned int b = row / a.heads, head = row % a.heads;
     const unsigned int group = a.heads / a.kv_heads;
     const unsigned int kv_head = head / group, in_group = head % group;
     const unsigned int work = kv_head * a.head_groups + in_group / 8, local = in_group % 8;
     const unsigned int share = a.meta[0];
     const unsigned int first_tile = a.meta[2 + b], end_tile = a.meta[3 + b];
-    const unsigned int d = threadIdx.x;
-    float result = 0.0f;  // a sequence with no keys keeps a zero row (cpu/attention.rs:1213-1215)
+    float low = 0.0f, high = 0.0f;  // a sequence with no keys keeps a zero row (cpu/attention.rs:1213-1215)
     if (end_tile > first_tile) {
         const unsigned int first_worker = first_tile / share, last_worker = (end_tile - 1) / share;
         const size_t base = (static_cast<size_t>(work) * (a.workers + a.batch) + first_worker + b) * a.heads_per_wave + local;
         const unsigned int count = last_worker - first_worker + 1;
-        float largest = -INFINITY;
-        for (unsigned int s = 0; s < count; ++s) largest = fmaxf(largest, a.partial_lse[base + static_cast<size_t>(s) * a.heads_per_wave]);
-        if (largest != -INFINITY) {
-            float total = 0.0f, sum = 0.0f;
-            for (unsigned int s = 0; s < count; ++s) {
-                const size_t at = base + static_cast<size_t>(s) * a.heads_per_wave;
-                const float weight = __expf(a.partial_lse[at] - largest);
-                total += weight;
-                sum = fmaf(weight, a.partial_out[at * kDim + d], sum);
+        float best = -INFINITY, total = 0.0f;
+        for (unsigned int chunk = 0; chunk < count; chunk += 64) {
+            const unsigned int n = count - chunk < 64 ? count - chunk : 64;
+            const size_t chunk_base = base + static_cast<size_t>(chunk) * a.heads_per_wave;
+            const float mine = lane < n ? a.partial_lse[chunk_base + static_cast<size_t>(lane) * a.heads_per_wave] : -INFINITY;
+            float largest = mine;
+#pragma unroll
+            for (int step = 32; step >= 1; step >>= 1) largest = fmaxf(largest, __shfl_xor(largest, step, 64));
+            largest = fmaxf(largest, best);
+            if (largest == -INFINITY) continue;  // nothing but empty slots so far
+            const float rescale = __expf(best - largest);
+            const float weight = __expf(mine - largest);  // 0 for lanes past n
+            float weights = weight;
+#pragma unroll
+            for (int step = 32; step >= 1; step >>= 1) weights += __shfl_xor(weights, step, 64);
+            total = total * rescale + weights;
+            low *= rescale;
+            high *= rescale;
+            best = largest;
+            for (unsigned int first = 0; first < n; first += 16) {
+                float2 rows[16];
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    rows[j] = make_float2(0.0f, 0.0f);
+                    if (first + j < n)
+                        rows[j] = *reinterpret_cast<const float2*>(a.partial_out + (chunk_base + static_cast<size_t>(first + j) * a.heads_per_wave) * kDim + 2 * lane);
+                }
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    const float w = __shfl(weight, static_cast<int>(first) + j, 64);
+                    if (first + j < n) {
+                        low = fmaf(w, rows[j].x, low);
+                        high = fmaf(w, rows[j].y, high);
+                    }
+                }
             }
-            result = total > 0.0f ? sum / total : 0.0f;
+        }
+        if (total > 0.0f) {
+            low /= total;
+            high /= total;
         }
     }
-    a.out[static_cast<size_t>(row) * kDim + d] = f32_to_bf16_bits(result);
+    *reinterpret_cast<unsigned int*>(a.out + static_cast<size_t>(row) * kDim + 2 * lane) = pack_bf16x2(low, high);
 }

@@ -196,3 +196,37 @@ def test_decode_validation_errors_match_the_reference():
                                          A.PagedKvDecodeAttentionConfig.contiguous(**{**good, "head_dim": 96, "heads": 8}))
     A.paged_kv_decode_attention_bf16(None, out, out.clone(), cache, cache, lens, table, config)
     torch.cuda.synchronize()
+
+
+def test_decode_phases_and_scratch_reuse():
+    """The one-call form and the split + reduce phases run apart give the same rows, also on repeated
+    calls of different shapes that share one caller-owned scratch buffer, which carries no state."""
+    shapes = [dict(batch=12, heads=16, kv_heads=4, seq_lens=[0, 700, 33, 1, 2048, 16, 90, 513, 64, 300, 5, 1000]),
+              dict(batch=3, heads=8, kv_heads=8, seq_lens=[4000, 0, 129]),
+              dict(batch=40, heads=8, kv_heads=2, seq_lens=list(range(1, 400, 10)))]
+    works = [synthetic.paged_decode_workload(physical_blocks=1024, seed=900 + i, **shape) for i, shape in enumerate(shapes)]
+    configs = [A.PagedKvDecodeAttentionConfig.contiguous(w.batch, w.heads, w.kv_heads, w.head_dim, w.block_size,
+                                                         w.physical_blocks, w.block_table_batch_stride, w.scale) for w in works]
+    size = max(c.workspace_bytes() for c in configs)
+    scratch = torch.randint(1, 255, (size,), dtype=torch.uint8, device="cuda")  # dirty on purpose
+    for _ in range(2):
+        for work, config in zip(works, configs):
+            want = run_oracle(work)
+            lens = torch.from_numpy(work.seq_lens).cuda()
+            table = torch.from_numpy(work.block_table.view(np.int32)).cuda()
+            both = torch.full((work.batch, work.heads, work.head_dim), float("nan"), device="cuda", dtype=torch.bfloat16)
+            A.paged_kv_decode_attention_bf16(None, both, work.query, work.key_cache, work.value_cache, lens, table, config, scratch)
+            apart = torch.full_like(both, float("nan"))
+            A.paged_kv_decode_attention_bf16(None, apart, work.query, work.key_cache, work.value_cache, lens, table, config, scratch, 1)
+            A.paged_kv_decode_attention_bf16(None, apart, work.query, work.key_cache, work.value_cache, lens, table, config, scratch, 2)
+            torch.cuda.synchronize()
+            assert_close(both.float().cpu().numpy(), want, "both phases")
+            assert torch.equal(both.view(torch.int16), apart.view(torch.int16))
+
+
+def test_decode_one_long_sequence_spans_more_than_64_ranges():
+    """A single sequence cut into more key ranges than a wave has lanes: the reduce walks its slots in
+    chunks."""
+    work = synthetic.paged_decode_workload(batch=1, heads=8, kv_heads=8, physical_blocks=640, seq_lens=[10000], seed=77)
+    assert_close(run_gpu(work), run_oracle(work), "one long sequence")
+    assert_close(run_gpu(work, workers=200), run_oracle(work), "one long sequence, 200 ranges")
