@@ -144,6 +144,11 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
                                    reinterpret_cast<uintptr_t>(key), reinterpret_cast<uintptr_t>(value)};
     for (uintptr_t address : addresses)
         if (address % 16 != 0) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "buffers must be 16-byte aligned");
+    // The kernel addresses the keys of one (batch, head) slice with 32-bit byte offsets.
+    const size_t widest = c.key_sequence_stride > c.value_sequence_stride ? c.key_sequence_stride : c.value_sequence_stride;
+    size_t slice_bytes = 0;
+    if (!checked_mul(c.key_len, widest, &slice_bytes) || !checked_mul(slice_bytes, 2, &slice_bytes) || slice_bytes > 0xffffffffull)
+        return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "key_len * sequence stride beyond 4 GiB");
     PrefillArgs args;
     args.query = query;
     args.key = key;

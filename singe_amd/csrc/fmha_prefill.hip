@@ -9,9 +9,9 @@
 // The per-tile arithmetic (transposed products on v_mfma_f32_32x32x16_bf16, online softmax, transposing
 // LDS reads for V) is the shared core in prefill_core.hip.h.
 //
-// Grid: one workgroup per (batch, head, 128-row query tile).  Workgroup i lands on XCD i % 8, so ids
-// are laid out to keep the query tiles of one head on one XCD (its K/V then stay in that XCD's L2),
-// heaviest (last) query tiles first so the causal triangle drains evenly.
+// Grid: one workgroup per (batch, head, 128-row query tile).  Workgroup i lands on XCD i % 8, so a
+// (batch, head) is pinned to an XCD (its K/V then stay in that XCD's L2); within an XCD the workgroups
+// run the heaviest (last) query tiles of every head first, so the causal triangle drains evenly.
 #include "kernel_args.h"
 #include "prefill_core.hip.h"
 
@@ -21,14 +21,18 @@ using namespace prefill;
 
 template <bool CAUSAL>
 SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
-    const unsigned int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const unsigned int tid = threadIdx.x, lane = tid & 63;
+    // The wave index is the same in all lanes; saying so keeps everything derived from it (which keys
+    // are live, whether a tile is on the mask's edge) in scalar registers and scalar branches.
+    const unsigned int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const unsigned int column = lane & 31, hi = lane >> 5;
 
     // Workgroup id -> (batch * heads + head, query tile): see the header comment.
     const unsigned int xcd = blockIdx.x & 7u, within = blockIdx.x >> 3;
-    const unsigned int bh = (within / a.query_tiles) * 8u + xcd;
+    const unsigned int per_xcd = (a.batch * a.heads + 7u) / 8u;
+    const unsigned int bh = (within % per_xcd) * 8u + xcd;
     if (bh >= a.batch * a.heads) return;
-    const unsigned int query_tile = a.query_tiles - 1u - within % a.query_tiles;
+    const unsigned int query_tile = a.query_tiles - 1u - within / per_xcd;
     const unsigned int batch = bh / a.heads, head = bh % a.heads;
     const unsigned int kv_head = head / (a.heads / a.kv_heads);
 
@@ -70,11 +74,17 @@ SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
     // The next tile on its way from global memory to LDS: four 16-byte chunks of K and of V per thread
     // (named registers, not arrays, so they are never given a stack slot).
     uint4 k0, k1, k2, k3, v0, v1, v2, v3;
+    // Offsets inside one (batch, head) slice fit 32 bits (checked by the host), so a load is a uniform
+    // base plus a 32-bit lane offset.
+    const unsigned int key_stride_bytes = static_cast<unsigned int>(a.key_sequence_stride) * 2u;
+    const unsigned int value_stride_bytes = static_cast<unsigned int>(a.value_sequence_stride) * 2u;
+    const unsigned char* const k_bytes = reinterpret_cast<const unsigned char*>(k_base);
+    const unsigned char* const v_bytes = reinterpret_cast<const unsigned char*>(v_base);
     auto fetch_row = [&](unsigned int tile, unsigned int i, uint4& key_bits, uint4& value_bits) __attribute__((always_inline)) {
         unsigned int key = tile * kKeyTile + load_row + 16u * i;
         key = key < a.key_len ? key : a.key_len - 1;  // rows past the end re-read the last key and are masked
-        key_bits = *reinterpret_cast<const uint4*>(k_base + static_cast<size_t>(key) * a.key_sequence_stride + load_col * 8u);
-        value_bits = *reinterpret_cast<const uint4*>(v_base + static_cast<size_t>(key) * a.value_sequence_stride + load_col * 8u);
+        key_bits = *reinterpret_cast<const uint4*>(k_bytes + (key * key_stride_bytes + load_col * 16u));
+        value_bits = *reinterpret_cast<const uint4*>(v_bytes + (key * value_stride_bytes + load_col * 16u));
     };
     auto fetch = [&](unsigned int tile) __attribute__((always_inline)) {
         fetch_row(tile, 0, k0, v0);

@@ -47,6 +47,14 @@ SINGE_DEVICE float swap32_sum(float value) {
     return kept + taken;
 }
 
+// max(a, b, c) in one instruction.  The scores come straight out of the matrix core and are never
+// signalling NaNs, so the canonicalising copies the compiler puts in front of fmaxf are not needed.
+SINGE_DEVICE float max3(float a, float b, float c) {
+    float result;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(result) : "v"(a), "v"(b), "v"(c));
+    return result;
+}
+
 SINGE_DEVICE unsigned int pack_pair(float lo, float hi) {
     f32x2v_t both = {lo, hi};
     return __builtin_bit_cast(unsigned int, __builtin_convertvector(both, bf16x2v_t));
@@ -84,21 +92,16 @@ SINGE_DEVICE unsigned int value_read_offset(unsigned int lane) {
     return (4 * hi + (sub >> 2)) * kValueRowBytes + (16 * (group & 1u) + 4 * (sub & 3u)) * 2;
 }
 
-// Folds the 64 keys staged at `keys` / `values` into `state`.
-//   factor     scale * log2(e) (positive; a negative scale is moved into Q by the caller)
-//   live1      false when the second 32-key block is wholly hidden from this wave
-//   edge       true when some score of this tile must be hidden; then hidden(block, key_in_block)
-//              says which (key_in_block = 8(r / 4) + 4hi + (r % 4) for accumulator register r)
-//   SOFTCAP    scores become cap * tanh(score * scale / cap) before the softmax
-//              (singe/src/backend/cuda/kernel_plan/source/tensor_core.rs:49-54)
-template <bool SOFTCAP, class Hidden>
-SINGE_DEVICE void fold_staged_keys(RowState& state, const bf16x8_t (&q)[8], const unsigned char* keys,
-                                   const unsigned char* values, unsigned int key_read, unsigned int value_read,
-                                   unsigned int hi, float factor, bool live1, bool edge, Hidden&& hidden,
-                                   float cap_scale = 0.0f, float cap_log2e = 0.0f) {
-    // Scores.  All eight K operands of a block are read before its MFMA chain starts, and the reads
-    // of the second block are issued while the first chain runs, so the matrix core never waits on
-    // a single LDS round trip.
+// Scores of a wave's 32 queries against the 64 keys staged at `keys`: S^T blocks s0 (keys 0..31) and s1
+// (keys 32..63; left at zero when live1 is false).  All eight K operands of a block are read before its
+// MFMA chain starts and the two blocks' chains alternate, so no MFMA waits on an LDS round trip or on the
+// MFMA issued just before it.  The products run on while the caller does other work.
+struct Scores {
+    f32x16_t s0, s1;
+};
+
+SINGE_DEVICE void score_staged_keys(Scores& scores, const bf16x8_t (&q)[8], const unsigned char* keys, unsigned int key_read,
+                                    bool live1) {
     f32x16_t s0, s1;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -110,19 +113,34 @@ SINGE_DEVICE void fold_staged_keys(RowState& state, const bf16x8_t (&q)[8], cons
     for (int step = 0; step < 8; ++step) ka[step] = *reinterpret_cast<const uint4*>(keys + key_read + step * 32);
     if (live1) {
 #pragma unroll
-        for (int step = 0; step < 8; ++step) {
-            kb[step] = *reinterpret_cast<const uint4*>(keys + 32 * kKeyRowBytes + key_read + step * 32);
-            s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, ka[step]), q[step], s0, 0, 0, 0);
-        }
+        for (int step = 0; step < 8; ++step) kb[step] = *reinterpret_cast<const uint4*>(keys + 32 * kKeyRowBytes + key_read + step * 32);
 #pragma unroll
-        for (int step = 0; step < 8; ++step)
+        for (int step = 0; step < 8; ++step) {
+            s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, ka[step]), q[step], s0, 0, 0, 0);
             s1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, kb[step]), q[step], s1, 0, 0, 0);
+        }
     } else {
 #pragma unroll
         for (int step = 0; step < 8; ++step)
             s0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, ka[step]), q[step], s0, 0, 0, 0);
     }
+    scores.s0 = s0;
+    scores.s1 = s1;
+}
 
+// Folds the scores of a staged tile, whose values sit at `values`, into `state`.
+//   factor     scale * log2(e) (positive; a negative scale is moved into Q by the caller)
+//   live1      false when the second 32-key block is wholly hidden from this wave
+//   edge       true when some score of this tile must be hidden; then hidden(block, key_in_block)
+//              says which (key_in_block = 8(r / 4) + 4hi + (r % 4) for accumulator register r)
+//   SOFTCAP    scores become cap * tanh(score * scale / cap) before the softmax
+//              (singe/src/backend/cuda/kernel_plan/source/tensor_core.rs:49-54)
+template <bool SOFTCAP, class Hidden>
+SINGE_DEVICE void fold_scores(RowState& state, Scores& scores, const unsigned char* values, unsigned int value_read,
+                              unsigned int hi, float factor, bool live1, bool edge, Hidden&& hidden, float cap_scale = 0.0f,
+                              float cap_log2e = 0.0f) {
+    f32x16_t& s0 = scores.s0;
+    f32x16_t& s1 = scores.s1;
     if constexpr (SOFTCAP) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -140,10 +158,14 @@ SINGE_DEVICE void fold_staged_keys(RowState& state, const bf16x8_t (&q)[8], cons
         }
     }
 
-    float largest = fmaxf(s0[0], s1[0]);
+    float largest = max3(s0[0], s1[0], s0[1]), other = max3(s1[1], s0[2], s1[2]);
 #pragma unroll
-    for (int r = 1; r < 16; ++r) largest = fmaxf(largest, fmaxf(s0[r], s1[r]));
-    largest = swap32_max(largest) * factor;  // both lanes of a query agree from here on
+    for (int r = 3; r < 15; r += 2) {
+        largest = max3(largest, s0[r], s1[r]);
+        other = max3(other, s0[r + 1], s1[r + 1]);
+    }
+    largest = max3(largest, s0[15], s1[15]);
+    largest = swap32_max(fmaxf(largest, other)) * factor;  // both lanes of a query agree from here on
     if (__any(largest > state.reference + kMaxLag || (state.reference == -INFINITY && largest != -INFINITY))) {
         const float moved = fmaxf(state.reference, largest);
         const float base = moved == -INFINITY ? 0.0f : moved;
@@ -166,39 +188,50 @@ SINGE_DEVICE void fold_staged_keys(RowState& state, const bf16x8_t (&q)[8], cons
     state.running_sum += total;
 
     // O^T += V^T . P^T, 16 keys per MFMA: registers 8j .. 8j+7 of a block are keys
-    // 16j + {0..3, 8..11} + 4hi of it, which is what the two transposing reads fetch.
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        const uint4 weights = make_uint4(pack_pair(s0[8 * j + 0], s0[8 * j + 1]), pack_pair(s0[8 * j + 2], s0[8 * j + 3]),
-                                         pack_pair(s0[8 * j + 4], s0[8 * j + 5]), pack_pair(s0[8 * j + 6], s0[8 * j + 7]));
-        const unsigned char* rows = values + (16 * j) * kValueRowBytes + value_read;
+    // 16j + {0..3, 8..11} + 4hi of it, which is what the two transposing reads fetch.  The V^T operands
+    // of the next 16 keys are read while the matrix core works on the current ones.
+    typedef v4i16_t __attribute__((address_space(3))) * lds_v4_t;
+    auto read_group = [&](int group, v8i16_t (&operand)[4]) __attribute__((always_inline)) {
+        const unsigned char* rows = values + (16 * group) * kValueRowBytes + value_read;
 #pragma unroll
         for (int db = 0; db < 4; ++db) {
-            const v4i16_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4i16_t __attribute__((address_space(3)))*)(rows + db * 64));
-            const v4i16_t high = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                (v4i16_t __attribute__((address_space(3)))*)(rows + 8 * kValueRowBytes + db * 64));
-            const v8i16_t both = __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7);
-            state.out[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, both),
+            const v4i16_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(rows + db * 64));
+            const v4i16_t high = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(rows + 8 * kValueRowBytes + db * 64));
+            operand[db] = __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+    };
+    auto weights_of = [&](const f32x16_t& s, int j) __attribute__((always_inline)) {
+        return make_uint4(pack_pair(s[8 * j + 0], s[8 * j + 1]), pack_pair(s[8 * j + 2], s[8 * j + 3]),
+                          pack_pair(s[8 * j + 4], s[8 * j + 5]), pack_pair(s[8 * j + 6], s[8 * j + 7]));
+    };
+    auto multiply = [&](const v8i16_t (&operand)[4], const uint4& weights) __attribute__((always_inline)) {
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+            state.out[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, operand[db]),
                                                               __builtin_bit_cast(bf16x8_t, weights), state.out[db], 0, 0, 0);
-        }
-    }
+    };
+    v8i16_t even[4], odd[4];
+    read_group(0, even);
+    read_group(1, odd);
+    multiply(even, weights_of(s0, 0));
+    if (live1) read_group(2, even);
+    multiply(odd, weights_of(s0, 1));
     if (live1) {
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const uint4 weights = make_uint4(pack_pair(s1[8 * j + 0], s1[8 * j + 1]), pack_pair(s1[8 * j + 2], s1[8 * j + 3]),
-                                             pack_pair(s1[8 * j + 4], s1[8 * j + 5]), pack_pair(s1[8 * j + 6], s1[8 * j + 7]));
-            const unsigned char* rows = values + (32 + 16 * j) * kValueRowBytes + value_read;
-#pragma unroll
-            for (int db = 0; db < 4; ++db) {
-                const v4i16_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((v4i16_t __attribute__((address_space(3)))*)(rows + db * 64));
-                const v4i16_t high = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                    (v4i16_t __attribute__((address_space(3)))*)(rows + 8 * kValueRowBytes + db * 64));
-                const v8i16_t both = __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7);
-                state.out[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, both),
-                                                                  __builtin_bit_cast(bf16x8_t, weights), state.out[db], 0, 0, 0);
-            }
-        }
+        read_group(3, odd);
+        multiply(even, weights_of(s1, 0));
+        multiply(odd, weights_of(s1, 1));
     }
+}
+
+// Scores and fold in one go.
+template <bool SOFTCAP, class Hidden>
+SINGE_DEVICE void fold_staged_keys(RowState& state, const bf16x8_t (&q)[8], const unsigned char* keys,
+                                   const unsigned char* values, unsigned int key_read, unsigned int value_read,
+                                   unsigned int hi, float factor, bool live1, bool edge, Hidden&& hidden,
+                                   float cap_scale = 0.0f, float cap_log2e = 0.0f) {
+    Scores scores;
+    score_staged_keys(scores, q, keys, key_read, live1);
+    fold_scores<SOFTCAP>(state, scores, values, value_read, hi, factor, live1, edge, hidden, cap_scale, cap_log2e);
 }
 
 }  // namespace prefill
