@@ -5,25 +5,31 @@
 // strides from FmhaPrefillConfig; lse [batch, heads, query_len], natural log.
 //
 // A workgroup of four waves owns 128 query rows of one (batch, head); each wave owns 32 of them and
-// walks the key axis in tiles of 64 keys staged in LDS (double buffered, one barrier per tile).
-// The per-tile arithmetic (transposed products on v_mfma_f32_32x32x16_bf16, online softmax, transposing
-// LDS reads for V) is the shared core in prefill_core.hip.h.
+// walks the key axis in blocks of 32 keys.  Tiles of 64 keys go from global memory straight into LDS
+// (three K stages, two V stages, one barrier per tile): while tile t is worked on, K of tile t + 2 and V of
+// tile t + 1 are on their way, so every load has a whole tile's arithmetic to land and no register holds
+// data in transit.  The score products of a block are woven into the exponentials of the block before it
+// (prefill_blocks.hip.h), which keeps the matrix core fed while the vector unit works.
 //
 // Grid: one workgroup per (batch, head, 128-row query tile).  Workgroup i lands on XCD i % 8, so a
 // (batch, head) is pinned to an XCD (its K/V then stay in that XCD's L2); within an XCD the workgroups
 // run the heaviest (last) query tiles of every head first, so the causal triangle drains evenly.
 #include "kernel_args.h"
-#include "prefill_core.hip.h"
+#include "prefill_blocks.hip.h"
 
 namespace {
 
 using namespace prefill;
 
+constexpr int kKeyStages = 3, kValueStages = 2;
+constexpr int kValueBase = kKeyStages * kTileBytes;
+constexpr int kDenseLdsBytes = (kKeyStages + kValueStages) * kTileBytes;
+
 template <bool CAUSAL>
 SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
     const unsigned int tid = threadIdx.x, lane = tid & 63;
-    // The wave index is the same in all lanes; saying so keeps everything derived from it (which keys
-    // are live, whether a tile is on the mask's edge) in scalar registers and scalar branches.
+    // The wave index is the same in all lanes; saying so keeps everything derived from it (which blocks
+    // are live, whether a block is on the mask's edge, LDS bases) in scalar registers and scalar branches.
     const unsigned int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const unsigned int column = lane & 31, hi = lane >> 5;
 
@@ -41,8 +47,8 @@ SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
     const bool query_valid = my_query < a.query_len;
 
     const uint16_t* q_base = a.query + batch * a.query_batch_stride + head * a.query_head_stride;
-    const uint16_t* k_base = a.key + batch * a.key_batch_stride + kv_head * a.key_head_stride;
-    const uint16_t* v_base = a.value + batch * a.value_batch_stride + kv_head * a.value_head_stride;
+    const unsigned char* const k_bytes = reinterpret_cast<const unsigned char*>(a.key + batch * a.key_batch_stride + kv_head * a.key_head_stride);
+    const unsigned char* const v_bytes = reinterpret_cast<const unsigned char*>(a.value + batch * a.value_batch_stride + kv_head * a.value_head_stride);
 
     // Q^T as the MFMA B operand: lane (column = query, hi) holds dims 16s + 8hi .. +8 for s = 0..7.
     // A negative scale is moved into Q (sign bits flipped) so the softmax can take the row maximum of
@@ -61,89 +67,121 @@ SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
         }
     }
 
-    // Keys this workgroup must visit, and its share of the tile loads: 1024 16-byte chunks per
-    // operand per tile, four per thread.
+    // Keys this workgroup must visit, and the blocks of them this wave folds: under the causal mask a
+    // block wholly after the wave's last query contributes nothing.
     unsigned int key_end = a.key_len;
     if (CAUSAL) {
         const unsigned int reach = query_tile * kQueryTile + kQueryTile;
         key_end = key_end < reach ? key_end : reach;
     }
     const unsigned int tiles = (key_end + kKeyTile - 1) / kKeyTile;
+    unsigned int wave_blocks = (key_end + 31u) / 32u;
+    if (CAUSAL) {
+        const unsigned int seen = (first_row + 31u) / 32u + 1u;
+        wave_blocks = wave_blocks < seen ? wave_blocks : seen;
+    }
 
-    const unsigned int load_row = tid >> 4, load_col = tid & 15u;  // chunk i of a thread: row + 16 i
-    // The next tile on its way from global memory to LDS: four 16-byte chunks of K and of V per thread
-    // (named registers, not arrays, so they are never given a stack slot).
-    uint4 k0, k1, k2, k3, v0, v1, v2, v3;
-    // Offsets inside one (batch, head) slice fit 32 bits (checked by the host), so a load is a uniform
-    // base plus a 32-bit lane offset.
+    // A tile load is 1024 16-byte chunks per operand: instruction i of wave w fills rows 16 i + 4 w .. + 3
+    // (1 KiB of LDS starting at a wave-uniform address), lane l the chunk position l % 16 of row
+    // 16 i + 4 w + l / 16, fetched from the chunk the row's permutation puts there.  Offsets inside one
+    // (batch, head) slice fit 32 bits (checked by the host).
     const unsigned int key_stride_bytes = static_cast<unsigned int>(a.key_sequence_stride) * 2u;
     const unsigned int value_stride_bytes = static_cast<unsigned int>(a.value_sequence_stride) * 2u;
-    const unsigned char* const k_bytes = reinterpret_cast<const unsigned char*>(k_base);
-    const unsigned char* const v_bytes = reinterpret_cast<const unsigned char*>(v_base);
-    auto fetch_row = [&](unsigned int tile, unsigned int i, uint4& key_bits, uint4& value_bits) __attribute__((always_inline)) {
-        unsigned int key = tile * kKeyTile + load_row + 16u * i;
-        key = key < a.key_len ? key : a.key_len - 1;  // rows past the end re-read the last key and are masked
-        key_bits = *reinterpret_cast<const uint4*>(k_bytes + (key * key_stride_bytes + load_col * 16u));
-        value_bits = *reinterpret_cast<const uint4*>(v_bytes + (key * value_stride_bytes + load_col * 16u));
+    const unsigned int load_row = 4u * wave + (lane >> 4), position = lane & 15u;
+    const unsigned int key_chunk = (position ^ (load_row & 15u)) * 16u, value_chunk = (position ^ (4u * (load_row & 3u))) * 16u;
+    auto load_keys = [&](unsigned int tile, unsigned int stage) __attribute__((always_inline)) {
+#pragma unroll
+        for (unsigned int i = 0; i < 4; ++i) {
+            unsigned int key = tile * kKeyTile + 16u * i + load_row;
+            key = key < a.key_len ? key : a.key_len - 1;  // rows past the end re-read the last key and are masked
+            __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(k_bytes + (key * key_stride_bytes + key_chunk)),
+                                             (lds_words_t)(lds + stage * kTileBytes + (16u * i + 4u * wave) * kRowBytes), 16, 0, 0);
+        }
     };
-    auto fetch = [&](unsigned int tile) __attribute__((always_inline)) {
-        fetch_row(tile, 0, k0, v0);
-        fetch_row(tile, 1, k1, v1);
-        fetch_row(tile, 2, k2, v2);
-        fetch_row(tile, 3, k3, v3);
-    };
-    auto stash_row = [&](unsigned char* keys, unsigned char* values, unsigned int i, const uint4& key_bits, const uint4& value_bits) __attribute__((always_inline)) {
-        const unsigned int row = load_row + 16u * i;
-        *reinterpret_cast<uint4*>(keys + row * kKeyRowBytes + load_col * 16) = key_bits;
-        *reinterpret_cast<uint4*>(values + row * kValueRowBytes + load_col * 16) = value_bits;
-    };
-    auto stash = [&](unsigned char* keys, unsigned char* values) __attribute__((always_inline)) {
-        stash_row(keys, values, 0, k0, v0);
-        stash_row(keys, values, 1, k1, v1);
-        stash_row(keys, values, 2, k2, v2);
-        stash_row(keys, values, 3, k3, v3);
+    auto load_values = [&](unsigned int tile, unsigned int stage) __attribute__((always_inline)) {
+#pragma unroll
+        for (unsigned int i = 0; i < 4; ++i) {
+            unsigned int key = tile * kKeyTile + 16u * i + load_row;
+            key = key < a.key_len ? key : a.key_len - 1;
+            __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(v_bytes + (key * value_stride_bytes + value_chunk)),
+                                             (lds_words_t)(lds + kValueBase + stage * kTileBytes + (16u * i + 4u * wave) * kRowBytes), 16, 0, 0);
+        }
     };
 
     RowState state;
     reset(state);
+    const ReadOffsets offsets = read_offsets(lane);
 
     if (tiles > 0) {
-        fetch(0);
-        stash(lds, lds + kKeyStageBytes);
+        load_keys(0, 0);
+        load_values(0, 0);
     }
+    if (tiles > 1) load_keys(1, 1);
     __syncthreads();
 
-    const unsigned int key_read = key_read_offset(lane), value_read = value_read_offset(lane);
-
-    // Folds the 64 keys staged at `keys` / `values` (tile index `tile`) into the running state.
-    auto fold = [&](unsigned int tile, const unsigned char* keys, const unsigned char* values) __attribute__((always_inline)) {
-        const unsigned int key0 = tile * kKeyTile;
-        // A 32-key block wholly after the wave's last query contributes nothing under the causal mask.
-        const bool live0 = !CAUSAL || key0 <= first_row + 31u;
-        const bool live1 = !CAUSAL || key0 + 32u <= first_row + 31u;
-        if (!live0) return;
-        // Keys after the query (causal) and keys past the end of the tensor are hidden.
-        const bool edge = (CAUSAL && key0 + kKeyTile - 1 > first_row) || key0 + kKeyTile > a.key_len;
-        fold_staged_keys<false>(state, q, keys, values, key_read, value_read, hi, factor, live1, edge,
-                                [&](unsigned int block, unsigned int key_in_block) {
-                                    const unsigned int key = key0 + 32 * block + key_in_block;
-                                    return (CAUSAL && key > my_query) || key >= a.key_len;
-                                });
+    // Folds block `block` (scores in `s`, values at `values`) with the mask's edges applied.
+    auto fold = [&](unsigned int block, f32x16_t& s, const unsigned char* values) __attribute__((always_inline)) {
+        const unsigned int key0 = block * 32u;
+        const bool edge = (CAUSAL && key0 + 31u > first_row) || key0 + 32u > a.key_len;
+        const float shift = begin_block(state, s, hi, factor, edge, [&](unsigned int key_in_block) {
+            const unsigned int key = key0 + key_in_block;
+            return (CAUSAL && key > my_query) || key >= a.key_len;
+        });
+        finish_block<false>(state, s, factor, shift, values, offsets, s, q, values);
     };
 
-    unsigned char* const keys0 = lds;
-    unsigned char* const values0 = lds + kKeyStageBytes;
-    unsigned char* const keys1 = lds + kStageBytes;
-    unsigned char* const values1 = lds + kStageBytes + kKeyStageBytes;
-    for (unsigned int tile = 0; tile < tiles; tile += 2) {
-        if (tile + 1 < tiles) fetch(tile + 1);
-        fold(tile, keys0, values0);
-        if (tile + 1 < tiles) stash(keys1, values1);
+    // One block ahead: while block b is folded, the scores of block b + 1 are computed; `scores` holds
+    // those of the block that is folded next.
+    f32x16_t scores;
+    if (wave_blocks > 0) score_block(scores, q, lds, offsets);
+    unsigned int key_stage = 0, value_stage = 0;  // tile % 3, tile % 2
+    // Starts the loads of a tile's iteration and names the stages it works on.  Everyone left the stages
+    // that held K of tile - 1 and V of tile - 1 at the last barrier.
+    const unsigned char *keys, *next_keys, *values;
+    auto enter = [&](unsigned int tile) __attribute__((always_inline)) {
+        const unsigned int next_key_stage = key_stage + 1 == kKeyStages ? 0 : key_stage + 1;
+        const unsigned int spare_key_stage = next_key_stage + 1 == kKeyStages ? 0 : next_key_stage + 1;
+        if (tile + 2 < tiles) load_keys(tile + 2, spare_key_stage);
+        if (tile + 1 < tiles) load_values(tile + 1, value_stage ^ 1u);
+        keys = lds + key_stage * kTileBytes;
+        next_keys = lds + next_key_stage * kTileBytes;
+        values = lds + kValueBase + value_stage * kTileBytes;
+        key_stage = next_key_stage;
+        value_stage ^= 1u;
+    };
+
+    // Tiles with no mask to apply and another block to come after them: straight-line code.  They come
+    // first for every wave (the mask's edge and the end of the keys are the last tiles a wave works on).
+    unsigned int interior_tiles = wave_blocks > 2 ? (wave_blocks - 1) / 2 : 0;  // tiles t with 2 t + 2 < wave_blocks
+    if (CAUSAL) {
+        const unsigned int unmasked = (first_row + 1) / kKeyTile;  // tiles t with 64 t + 63 <= first_row
+        interior_tiles = interior_tiles < unmasked ? interior_tiles : unmasked;
+    }
+    {
+        const unsigned int whole = a.key_len / kKeyTile;  // tiles t with 64 t + 64 <= key_len
+        interior_tiles = interior_tiles < whole ? interior_tiles : whole;
+    }
+    unsigned int tile = 0;
+    for (; tile < interior_tiles; ++tile) {
+        enter(tile);
+        const float shift_even = begin_block(state, scores, hi, factor, false, [](unsigned int) { return false; });
+        finish_block<true>(state, scores, factor, shift_even, values, offsets, scores, q, keys + kBlockBytes);
+        __builtin_amdgcn_sched_barrier(0);  // keeps the second block's operand reads out of the first block's registers
+        const float shift_odd = begin_block(state, scores, hi, factor, false, [](unsigned int) { return false; });
+        finish_block<true>(state, scores, factor, shift_odd, values + kBlockBytes, offsets, scores, q, next_keys);
         __syncthreads();
-        if (tile + 1 >= tiles) break;
-        if (tile + 2 < tiles) fetch(tile + 2);
-        fold(tile + 1, keys1, values1);
-        if (tile + 2 < tiles) stash(keys0, values0);
+    }
+    // Tiles on the mask's edge and the last ones (and, for waves that have run out of blocks, the
+    // workgroup's remaining loads and barriers): the same steps one after the other.
+    for (; tile < tiles; ++tile) {
+        enter(tile);
+        const unsigned int block = 2u * tile;
+        if (block < wave_blocks) fold(block, scores, values);
+        if (block + 1 < wave_blocks) {
+            score_block(scores, q, keys + kBlockBytes, offsets);
+            fold(block + 1, scores, values + kBlockBytes);
+        }
+        if (block + 2 < wave_blocks) score_block(scores, q, next_keys, offsets);
         __syncthreads();
     }
 
@@ -171,11 +209,11 @@ SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
 }  // namespace
 
 extern "C" __global__ __launch_bounds__(256, 2) void singe_fmha_prefill_bf16_d128_causal(PrefillArgs args) {
-    __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[2 * prefill::kStageBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char prefill_lds[kDenseLdsBytes];
     fmha_prefill_body<true>(args, prefill_lds);
 }
 
 extern "C" __global__ __launch_bounds__(256, 2) void singe_fmha_prefill_bf16_d128_full(PrefillArgs args) {
-    __shared__ __attribute__((aligned(16))) unsigned char prefill_lds[2 * prefill::kStageBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char prefill_lds[kDenseLdsBytes];
     fmha_prefill_body<false>(args, prefill_lds);
 }

@@ -1,0 +1,153 @@
+// Block-pipelined core of the dense bf16 flash-attention prefill kernel: one wave folds blocks of 32 keys
+// into the running softmax state of its 32 query rows, with the score products of the next block issued
+// before the softmax of the current one so the matrix core and the vector unit work at the same time.
+// Everything is kept transposed so the softmax weights never leave registers (see prefill_core.hip.h for
+// the register layouts, which this file shares):
+//
+//   S^T[key, query] = K . Q^T      v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = the wave's Q^T;
+//   O^T[dim, query] += V^T . P^T   A = V^T through ds_read_b64_tr_b16, B = P^T packed from the S^T registers.
+//
+// Tiles of 64 keys reach LDS straight from global memory (global_load_lds_dwordx4: lane l of a wave puts
+// its 16 bytes at the wave's LDS base + 16 l, whatever global address it read), so rows are stored
+// unpadded, 256 bytes each, and bank conflicts are avoided by permuting the sixteen 16-byte chunks of a
+// row instead: K keeps chunk c of row r at position c ^ (r & 15), V at position c ^ 4 (r & 3).  The
+// permutation is applied on the global side (which chunk a lane fetches) and undone by the read offsets.
+#pragma once
+
+#include "prefill_core.hip.h"
+
+namespace prefill {
+
+constexpr int kRowBytes = 256;                       // one key's 128 bf16
+constexpr int kTileBytes = kKeyTile * kRowBytes;     // 64 keys of K or of V
+constexpr int kBlockBytes = 32 * kRowBytes;
+
+typedef unsigned int __attribute__((address_space(3))) * lds_words_t;
+
+// Per-lane LDS read offsets inside a 32-key block, kept as a base and the bits the row's permutation
+// flips so that each read's offset costs one xor-add instead of a register.
+struct ReadOffsets {
+    unsigned int key_base, key_flip;      // K operand of step s: key_base + ((32 s) ^ key_flip)
+    unsigned int value_base, value_flip;  // V^T operand of dim block db: value_base + ((64 db) ^ value_flip)
+    SINGE_DEVICE unsigned int key(unsigned int step) const { return ((32u * step) ^ key_flip) + key_base; }
+    SINGE_DEVICE unsigned int value(unsigned int db) const { return ((64u * db) ^ value_flip) + value_base; }
+};
+
+// K: row lane % 32, chunk (2 s + hi) ^ (row & 15), 16 bytes per chunk.  V^T: keys 4 hi + (sub >> 2) of a
+// 16-key group (add 8 rows for its high half), chunk (4 db + 2 (group & 1) + ((sub & 3) >> 1)) ^ 4 (row & 3),
+// 8 bytes at 8 (sub & 1) inside it.
+SINGE_DEVICE ReadOffsets read_offsets(unsigned int lane) {
+    ReadOffsets offsets;
+    const unsigned int hi = lane >> 5, row = lane & 31u;
+    offsets.key_base = row * kRowBytes;
+    offsets.key_flip = ((lane & 15u) ^ hi) * 16u;
+    const unsigned int group = lane >> 4, sub = lane & 15u, row_in_quad = sub >> 2;
+    offsets.value_base = (4u * hi + row_in_quad) * kRowBytes + (2u * (group & 1u) + ((sub & 3u) >> 1)) * 16u + 8u * (sub & 1u);
+    offsets.value_flip = 64u * row_in_quad;
+    return offsets;
+}
+
+// Scores of the wave's 32 queries against the 32 keys of the block at `keys` (LDS byte address of the
+// block's first row).  The products run on while the caller does other work.
+SINGE_DEVICE void score_block(f32x16_t& scores, const bf16x8_t (&q)[8], const unsigned char* keys, const ReadOffsets& offsets) {
+    f32x16_t s;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s[r] = 0.0f;
+    uint4 operand[8];
+#pragma unroll
+    for (int step = 0; step < 8; ++step) operand[step] = *reinterpret_cast<const uint4*>(keys + offsets.key(step));
+#pragma unroll
+    for (int step = 0; step < 8; ++step)
+        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, operand[step]), q[step], s, 0, 0, 0);
+    scores = s;
+}
+
+// First half of folding a 32-key block: hides what the mask hides, takes the row maxima and moves the
+// softmax reference point when a row's maximum has run too far ahead of it.  Returns the shift the
+// exponentials take (minus the reference, 0 for rows that have seen nothing).
+//   edge     true when some score of the block must be hidden; then hidden(key_in_block) says which
+//            (key_in_block = 8(r / 4) + 4hi + (r % 4) for accumulator register r)
+template <class Hidden>
+SINGE_DEVICE float begin_block(RowState& state, f32x16_t& s, unsigned int hi, float factor, bool edge, Hidden&& hidden) {
+    if (edge) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            if (hidden(8u * (r >> 2) + 4u * hi + (r & 3))) s[r] = -INFINITY;
+    }
+    float largest = max3(s[0], s[1], s[2]), other = max3(s[3], s[4], s[5]);
+    largest = max3(largest, s[6], s[7]);
+    other = max3(other, s[8], s[9]);
+    largest = max3(largest, s[10], s[11]);
+    other = max3(other, s[12], s[13]);
+    largest = max3(largest, s[14], s[15]);
+    largest = swap32_max(fmaxf(largest, other)) * factor;  // both lanes of a query agree from here on
+    if (__any(largest > state.reference + kMaxLag || (state.reference == -INFINITY && largest != -INFINITY))) {
+        const float moved = fmaxf(state.reference, largest);
+        const float base = moved == -INFINITY ? 0.0f : moved;
+        const float rescale = fast_exp2(state.reference - base);
+        state.running_sum *= rescale;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) state.out[db][r] *= rescale;
+        state.reference = moved;
+    }
+    return state.reference == -INFINITY ? 0.0f : -state.reference;
+}
+
+// Second half, free of branches so the compiler can weave its parts together: the scores `s` become
+// weights and O^T += V^T . P^T, and, when NEXT is set, the score products of the block at `next_keys` are
+// issued in between: one MFMA, then the exponentials of two registers, and so on, so the matrix core
+// computes the next block's scores while the vector unit exponentiates this one's.
+template <bool NEXT>
+SINGE_DEVICE void finish_block(RowState& state, f32x16_t& s, float factor, float shift, const unsigned char* values,
+                               const ReadOffsets& offsets, f32x16_t& next, const bf16x8_t (&q)[8], const unsigned char* next_keys) {
+    typedef v4i16_t __attribute__((address_space(3))) * lds_v4_t;
+    uint4 operand[8];
+    if constexpr (NEXT) {
+#pragma unroll
+        for (int step = 0; step < 8; ++step) operand[step] = *reinterpret_cast<const uint4*>(next_keys + offsets.key(step));
+    }
+    v8i16_t first[4], second[4];
+#pragma unroll
+    for (int db = 0; db < 4; ++db) {
+        const v4i16_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(values + offsets.value(db)));
+        const v4i16_t high = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(values + 8 * kRowBytes + offsets.value(db)));
+        first[db] = __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+    f32x16_t upcoming;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) upcoming[r] = 0.0f;
+    float total = 0.0f;
+#pragma unroll
+    for (int step = 0; step < 8; ++step) {
+        if (step == 4) {
+            // The second half of the values, fetched once half of the K operands have been used up.
+#pragma unroll
+            for (int db = 0; db < 4; ++db) {
+                const v4i16_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(values + 16 * kRowBytes + offsets.value(db)));
+                const v4i16_t high = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(values + 24 * kRowBytes + offsets.value(db)));
+                second[db] = __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7);
+            }
+        }
+        if constexpr (NEXT)
+            upcoming = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, operand[step]), q[step], upcoming, 0, 0, 0);
+        s[2 * step] = fast_exp2(fmaf(s[2 * step], factor, shift));
+        s[2 * step + 1] = fast_exp2(fmaf(s[2 * step + 1], factor, shift));
+        total += s[2 * step] + s[2 * step + 1];
+    }
+    state.running_sum += total;
+    // O^T += V^T . P^T, 16 keys per MFMA: registers 8j .. 8j+7 are keys 16j + {0..3, 8..11} + 4hi.
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint4 weights = make_uint4(pack_pair(s[8 * j + 0], s[8 * j + 1]), pack_pair(s[8 * j + 2], s[8 * j + 3]),
+                                         pack_pair(s[8 * j + 4], s[8 * j + 5]), pack_pair(s[8 * j + 6], s[8 * j + 7]));
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+            state.out[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, j == 0 ? first[db] : second[db]),
+                                                              __builtin_bit_cast(bf16x8_t, weights), state.out[db], 0, 0, 0);
+    }
+    if constexpr (NEXT) next = upcoming;
+}
+
+}  // namespace prefill
