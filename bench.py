@@ -24,6 +24,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
+# HBM bytes per launch of the decode split kernel at the headline workload, from rocprofv3 --pmc runs of
+# this script: FETCH_SIZE 145768 x 2 KiB (the counter's unit, calibrated on a copy of known size) +
+# WRITE_SIZE 4552 KiB.  Reported only for that kernel, workload and tuning.
+DECODE_TRAFFIC_BYTES = (145768 * 2 + 4552) * 1024
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 POOLS = 3
@@ -36,6 +40,7 @@ def parse():
     parser.add_argument("--warmup", type=int, default=30)
     parser.add_argument("--no-cpu-baseline", action="store_true")
     parser.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement")
+    parser.add_argument("--no-extras", action="store_true", help="skip the chunked-prefill and fp8-decode measurements")
     parser.add_argument("--prefill-steps", type=int, default=40)
     parser.add_argument("--workers", type=int, default=0, help="tuning override (0 = built-in choice)")
     return parser.parse_args()
@@ -131,6 +136,115 @@ def prefill_section(steps):
             "kernel_avg_us": avg * 1e3,
             "kernel_median_us": ms[len(ms) // 2] * 1e3,
         },
+    }
+
+
+def time_launches(launch, steps, group):
+    """Average milliseconds per launch from HIP events on the current stream around groups of
+    back-to-back launches; returns (average, median)."""
+    import torch
+
+    groups = max(steps // group, 4)
+    begin = [torch.cuda.Event(enable_timing=True) for _ in range(groups)]
+    finish = [torch.cuda.Event(enable_timing=True) for _ in range(groups)]
+    for j in range(groups):
+        begin[j].record()
+        for _ in range(group):
+            launch()
+        finish[j].record()
+    torch.cuda.synchronize()
+    ms = sorted(b.elapsed_time(f) / group for b, f in zip(begin, finish))
+    return sum(ms) / len(ms), ms[len(ms) // 2]
+
+
+def chunked_prefill_section(steps):
+    """Chunked paged prefill: 8 sequences, 512 new tokens each on prefixes U[1024, 16384], 64 query /
+    8 KV heads, head_dim 128, page 16, bf16 (BASELINE config 4), through the paged attention op."""
+    import ctypes
+
+    import numpy as np
+    import torch
+
+    from singe_amd import _native, neural, synthetic
+
+    work = synthetic.chunked_prefill_workload()
+    index = lambda values: torch.from_numpy(np.asarray(values, dtype=np.int32)).cuda()
+    paging = neural.Paging(index(work.query_offsets), index(work.page_offsets), index(work.pages), index(work.last_page_lengths))
+    options = neural.AttentionOptions(causal=True)
+    problem = neural._problem(work.query, work.key_cache, work.value_cache, paging, options)
+    out = torch.empty_like(work.query)
+    lse = torch.empty(work.query.shape[:2], device="cuda", dtype=torch.float32)
+    status = torch.zeros(1, device="cuda", dtype=torch.int32)
+    handle = int(torch.cuda.current_stream().cuda_stream)
+
+    def launch():
+        code = _native.lib().singe_hip_paged_attention_bf16(
+            handle, work.query.data_ptr(), work.key_cache.data_ptr(), work.value_cache.data_ptr(),
+            paging.query_offsets.data_ptr(), paging.page_offsets.data_ptr(), paging.pages.data_ptr(),
+            paging.last_page_lengths.data_ptr(), out.data_ptr(), lse.data_ptr(), status.data_ptr(), ctypes.byref(problem))
+        _native.check(code, "paged_attention")
+
+    for _ in range(3):
+        launch()
+    torch.cuda.synchronize()
+    avg, median = time_launches(launch, steps, 4)
+    assert int(status.item()) == 0
+    flops = work.algorithmic_flops()
+    tflops = flops / (avg * 1e-3) / 1e12
+    return {
+        "workload": "chunked paged prefill: 8 sequences x 512 new tokens on prefixes U[1024,16384], 64q/8kv heads, "
+                    "head_dim 128, page 16, bf16 (BASELINE config 4)",
+        "value": tflops,
+        "unit": "TFLOP/s",
+        "tokens_per_s": work.sequences * work.new_tokens / (avg * 1e-3),
+        "ms_per_step": avg,
+        "algorithmic_flops": flops,
+        "roofline": {"bound": "mfma", "kernel": "singe_paged_attention_bf16_d128_i32", "achieved": tflops,
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
+                     "traffic": None, "kernel_avg_us": avg * 1e3, "kernel_median_us": median * 1e3},
+    }
+
+
+def fp8_decode_section(steps):
+    """Long-context decode over an fp8 e4m3 KV cache: batch 64, 64 query / 8 KV heads, head_dim 128,
+    context 32768, block 16, one f32 scale per (block, kv head) (BASELINE config 5); exact numerics."""
+    import numpy as np
+    import torch
+
+    from singe_amd import synthetic
+    from singe_amd.kernel import attention as A
+
+    work = synthetic.paged_decode_fp8_workload()
+    config = A.PagedKvDecodeAttentionConfig.contiguous(work.batch, work.heads, work.kv_heads, work.head_dim,
+                                                       work.block_size, work.physical_blocks,
+                                                       work.block_table_batch_stride, work.scale)
+    lens = torch.from_numpy(work.seq_lens).cuda()
+    table = torch.from_numpy(work.block_table.view(np.int32)).cuda()
+    out = torch.empty((work.batch, work.heads, work.head_dim), device="cuda", dtype=torch.bfloat16)
+    workspace = torch.empty(config.workspace_bytes(), dtype=torch.uint8, device="cuda")
+
+    def launch():
+        A.paged_kv_decode_attention_f8e4m3kv_bf16(None, out, work.query, work.key_cache, work.value_cache, work.key_scales,
+                                                  work.value_scales, lens, table, config, workspace)
+
+    for _ in range(3):
+        launch()
+    torch.cuda.synchronize()
+    avg, median = time_launches(launch, steps, 2)
+    used_blocks = int(np.sum((work.seq_lens.astype(np.int64) + work.block_size - 1) // work.block_size))
+    nbytes = work.algorithmic_bytes(1) + 2 * used_blocks * work.kv_heads * 4  # + the scales of the used blocks
+    gbps = nbytes / (avg * 1e-3) / 1e9
+    return {
+        "workload": "paged decode, fp8 e4m3 KV: batch 64, 64q/8kv heads, head_dim 128, ctx 32768, block 16, "
+                    "f32 scale per (block, kv head) (BASELINE config 5); split + reduce kernels",
+        "value": gbps,
+        "unit": "GB/s",
+        "tokens_per_s": work.batch / (avg * 1e-3),
+        "ms_per_step": avg,
+        "algorithmic_bytes": nbytes,
+        "roofline": {"bound": "hbm", "kernel": "singe_paged_decode_f8kv_d128_g2_b16", "achieved": gbps, "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": None, "step_avg_us": avg * 1e3,
+                     "step_median_us": median * 1e3},
     }
 
 
@@ -230,7 +344,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": None,
+            "traffic": DECODE_TRAFFIC_BYTES if not args.workers else None,
             "kernel_avg_us": kernel_avg_ms * 1e3,
             "kernel_median_us": kernel_ms[len(kernel_ms) // 2] * 1e3,
         },
@@ -241,6 +355,15 @@ def main():
         del pools, workspace
         torch.cuda.empty_cache()
         result["prefill"] = prefill_section(args.prefill_steps)
+    if not args.no_extras:
+        try:
+            del pools, workspace
+        except NameError:
+            pass
+        torch.cuda.empty_cache()
+        result["chunked_prefill"] = chunked_prefill_section(20)
+        torch.cuda.empty_cache()
+        result["fp8_decode"] = fp8_decode_section(10)
     print(json.dumps(result), flush=True)
 
 

@@ -144,3 +144,53 @@ def paged_decode_fp8_workload(*, batch=64, heads=64, kv_heads=8, head_dim=128, b
     return PagedDecodeFp8Workload(batch, heads, kv_heads, head_dim, block_size, physical_blocks, stride,
                                   float(1.0 / np.sqrt(np.float32(head_dim))), seq_lens, table, query, caches[0],
                                   caches[1], scales[0], scales[1])
+
+
+@dataclass
+class ChunkedPrefillWorkload:
+    """Chunked paged prefill in FlashInfer form: each sequence appends `new_tokens` queries to a cached
+    prefix (singe surface, bottom-right causal)."""
+    sequences: int
+    new_tokens: int
+    heads: int
+    kv_heads: int
+    head_dim: int
+    page_size: int
+    prefix: np.ndarray             # [sequences] int64
+    query_offsets: np.ndarray      # [sequences + 1]
+    page_offsets: np.ndarray       # [sequences + 1]
+    pages: np.ndarray              # [sum pages]
+    last_page_lengths: np.ndarray  # [sequences]
+    query: torch.Tensor            # [sequences * new_tokens, heads, dim]
+    key_cache: torch.Tensor        # [pool, page_size, kv_heads, dim]
+    value_cache: torch.Tensor
+
+    def algorithmic_flops(self) -> int:
+        """4 * dim flops per unmasked (query row, key) pair: a query at offset i of a chunk sees
+        prefix + i + 1 keys."""
+        new = self.new_tokens
+        pairs = self.heads * sum(int(new * p + new * (new + 1) // 2) for p in self.prefix)
+        return 4 * self.head_dim * pairs
+
+
+def chunked_prefill_workload(*, sequences=8, new_tokens=512, heads=64, kv_heads=8, head_dim=128, page_size=16,
+                             pool_pages=16384, min_prefix=1024, max_prefix=16384, seed=BASE_SEED + 4,
+                             device="cuda", dtype=torch.bfloat16) -> ChunkedPrefillWorkload:
+    rng = np.random.default_rng(seed)
+    prefix = rng.integers(min_prefix, max_prefix + 1, size=sequences).astype(np.int64)
+    keys = prefix + new_tokens
+    counts = (keys + page_size - 1) // page_size
+    if int(counts.sum()) > pool_pages:
+        raise ValueError("page pool too small")
+    pages = rng.permutation(pool_pages)[: int(counts.sum())].astype(np.int64)
+    query_offsets = np.arange(sequences + 1, dtype=np.int64) * new_tokens
+    page_offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
+    last = keys - (counts - 1) * page_size
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed + 1)
+    query = torch.randn((sequences * new_tokens, heads, head_dim), generator=gen, device=device, dtype=torch.float32).to(dtype)
+    shape = (pool_pages, page_size, kv_heads, head_dim)
+    key_cache = torch.randn(shape, generator=gen, device=device, dtype=torch.float32).to(dtype)
+    value_cache = torch.randn(shape, generator=gen, device=device, dtype=torch.float32).to(dtype)
+    return ChunkedPrefillWorkload(sequences, new_tokens, heads, kv_heads, head_dim, page_size, prefix, query_offsets,
+                                  page_offsets, pages, last, query, key_cache, value_cache)
