@@ -11,9 +11,10 @@
 // data in transit.  The score products of a block are woven into the exponentials of the block before it
 // (prefill_blocks.hip.h), which keeps the matrix core fed while the vector unit works.
 //
-// Grid: one workgroup per (batch, head, 128-row query tile).  Workgroup i lands on XCD i % 8, so a
-// (batch, head) is pinned to an XCD (its K/V then stay in that XCD's L2); within an XCD the workgroups
-// run the heaviest (last) query tiles of every head first, so the causal triangle drains evenly.
+// Grid: one workgroup per (batch, head, pair of 128-row query tiles): tile i from the end and tile i from
+// the start, so under the causal mask every workgroup has the same amount of work.  Workgroup i lands on
+// XCD i % 8; ids are laid out so the workgroups of one (batch, head) are neighbours on one XCD and walk
+// its keys side by side, which keeps its K/V in that XCD's L2.
 #include "kernel_args.h"
 #include "prefill_blocks.hip.h"
 
@@ -25,20 +26,15 @@ constexpr int kKeyStages = 3, kValueStages = 2;
 constexpr int kValueBase = kKeyStages * kTileBytes;
 constexpr int kDenseLdsBytes = (kKeyStages + kValueStages) * kTileBytes;
 
+// One 128-row query tile of (batch, head) pair `bh`.
 template <bool CAUSAL>
-SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
+SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, unsigned int bh, unsigned int query_tile) {
     const unsigned int tid = threadIdx.x, lane = tid & 63;
     // The wave index is the same in all lanes; saying so keeps everything derived from it (which blocks
     // are live, whether a block is on the mask's edge, LDS bases) in scalar registers and scalar branches.
     const unsigned int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const unsigned int column = lane & 31, hi = lane >> 5;
 
-    // Workgroup id -> (batch * heads + head, query tile): see the header comment.
-    const unsigned int xcd = blockIdx.x & 7u, within = blockIdx.x >> 3;
-    const unsigned int per_xcd = (a.batch * a.heads + 7u) / 8u;
-    const unsigned int bh = (within % per_xcd) * 8u + xcd;
-    if (bh >= a.batch * a.heads) return;
-    const unsigned int query_tile = a.query_tiles - 1u - within / per_xcd;
     const unsigned int batch = bh / a.heads, head = bh % a.heads;
     const unsigned int kv_head = head / (a.heads / a.kv_heads);
 
@@ -204,6 +200,18 @@ SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
             a.lse[(static_cast<size_t>(batch) * a.heads + head) * a.query_len + my_query] =
                 sum > 0.0f ? (state.reference + fast_log2(sum)) * kLn2 : -INFINITY;
     }
+}
+
+// Workgroup id -> (batch * heads + head, pair of query tiles): see the header comment.
+template <bool CAUSAL>
+SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
+    const unsigned int xcd = blockIdx.x & 7u, within = blockIdx.x >> 3;
+    const unsigned int pairs = (a.query_tiles + 1u) / 2u;
+    const unsigned int bh = (within / pairs) * 8u + xcd;
+    if (bh >= a.batch * a.heads) return;
+    const unsigned int light = within % pairs, heavy = a.query_tiles - 1u - light;
+    fmha_prefill_tile<CAUSAL>(a, lds, bh, heavy);
+    if (light != heavy) fmha_prefill_tile<CAUSAL>(a, lds, bh, light);
 }
 
 }  // namespace
