@@ -439,6 +439,82 @@ SINGE_HIP_API int32_t singe_hip_splitk_reduce_f32(
     const float* lse_splitk, size_t lse_splitk_len,
     const SingeSplitKReduceConfig* config);
 
+/* ---- singe surface: the steps either side of paged attention ------------------------------------------
+ * The fused rotate-and-append kernel "rotary_cache_write"
+ * (singe/src/backend/cuda/kernel_plan/source/rotary_cache.rs:249-427): rotates query [tokens, query_heads,
+ * dim] into query_out, rotates key [tokens, cache_heads, dim] into key_cache[page_index[t], slot_index[t]]
+ * and copies value [tokens, cache_heads, dim] into value_cache at the same cell; caches are
+ * [cache_pages, page_slots, cache_heads, dim] and only the selected cells are written.  Half-split pairs
+ * (p, p + dim / 2) turn by the angles cos / sin [tokens, dim / 2] (of table_type): first = a cos - b sin,
+ * second = b cos + a sin, after an optional RMS normalisation (scale = rsqrt(mean(x^2) + eps), times an
+ * optional weight [dim]; rotary_cache.rs:92-185).  A negative page or slot counts from the end; one still
+ * outside its extent sets *status to 1 and leaves the caches alone for that token (rotary_cache.rs:376-385).
+ * Operands in the order of the reference kernel's ABI (rotary_cache.rs:52-66, 268-293); query, query_out
+ * and the weights may be null (query_heads 0 when attention rotates its own query). */
+typedef struct SingeRotaryCacheProblem {
+    int64_t tokens;
+    int64_t query_heads;
+    int64_t cache_heads;
+    int64_t head_dim;
+    int64_t cache_pages;
+    int64_t page_slots;
+    int32_t data_type;    /* SINGE_HIP_F32, _BF16 or _F16: queries, keys, values, weights, caches */
+    int32_t table_type;   /* cos and sin */
+    int32_t index_type;   /* SINGE_HIP_INDEX_I32 or _I64: page_index and slot_index */
+    uint8_t has_query_norm;
+    uint8_t has_key_norm;
+    float query_eps;
+    float key_eps;
+} SingeRotaryCacheProblem;
+
+SINGE_HIP_API int32_t singe_hip_rotary_cache_write(
+    void* stream,
+    const void* query,
+    const void* key,
+    const void* value,
+    const void* cos,
+    const void* sin,
+    const void* page_index,
+    const void* slot_index,
+    const void* query_weight,
+    const void* key_weight,
+    void* query_out,
+    void* key_cache,
+    void* value_cache,
+    uint32_t* status,
+    const SingeRotaryCacheProblem* problem);
+
+/* The kernel "paged_cudnn_indices" (kernel_plan/source/paged_attention.rs:325-398): FlashInfer CSR paging
+ * -> block-table paging.  Writes packed_offsets [sequences + 1] (first element of each sequence's queries:
+ * token offset * row_elements), query_lengths and key_lengths [sequences], and page_table
+ * [sequences, width] (a sequence's pages, zero-padded; width is the widest row the caller allows, pages past
+ * it are dropped).  Offsets are clamped into [0, tokens] and made monotone, so everything written stays
+ * inside its buffer whatever the input holds; a sequence or page id that the attention kernels would refuse
+ * sets *status to 1 and gets zero keys / a zero entry. */
+typedef struct SingePagingIndicesProblem {
+    int64_t sequences;
+    int64_t tokens;
+    int64_t page_count;     /* pages.len */
+    int64_t page_size;
+    int64_t cache_pages;
+    int64_t width;          /* page_table row length */
+    int64_t row_elements;   /* elements of one query token: heads * dim */
+    int32_t index_type;
+} SingePagingIndicesProblem;
+
+SINGE_HIP_API int32_t singe_hip_paging_indices(
+    void* stream,
+    const void* query_offsets,
+    const void* page_offsets,
+    const void* pages,
+    const void* last_page_lengths,
+    int32_t* packed_offsets,
+    int32_t* query_lengths,
+    int32_t* key_lengths,
+    int32_t* page_table,
+    uint32_t* status,
+    const SingePagingIndicesProblem* problem);
+
 #ifdef __cplusplus
 }
 #endif

@@ -298,3 +298,63 @@ def paged_slots(page_offsets, pages, last_page_lengths, *, page_size):
     lib().oracle_paged_slots(_ptr(slots), _ptr(counts), _ptr(po), _ptr(pg), _ptr(lp), _c_size(len(lp)),
                              _c_size(page_size))
     return slots, counts
+
+
+def rotary_embedding_f32(values, cos, sin):
+    """singe/src/backend/cpu/normalization/attention.rs:132-188: values [..., sequence, head_dim], cos/sin
+    [sequence, rotary_pairs]; interleaved pairs."""
+    values, cos, sin = _f32(values), _f32(cos), _f32(sin)
+    sequence, pairs = cos.shape
+    head_dim = values.shape[-1]
+    out = np.empty_like(values)
+    lib().oracle_rotary_embedding_f32(_ptr(out), _ptr(values), _ptr(cos), _ptr(sin), _c_size(values.size // head_dim),
+                                      _c_size(sequence), _c_size(head_dim), _c_size(pairs))
+    return out
+
+
+def rotary_cache_write_f32(query, key, value, cos, sin, pages, slots, key_cache, value_cache, *, query_norm=None,
+                           key_norm=None):
+    """The fused rotate-and-append step (singe/src/backend/cuda/kernel_plan/source/rotary_cache.rs:249-427).
+    query [T, H, D] or None, key/value [T, G, D], cos/sin [T, D/2], caches [P, S, G, D] (copied, then the
+    selected cells written); a norm is (eps, weight or None).  Returns (status, query_out, key_cache,
+    value_cache)."""
+    key, value, cos, sin = _f32(key), _f32(value), _f32(cos), _f32(sin)
+    key_cache, value_cache = _f32(key_cache).copy(), _f32(value_cache).copy()
+    tokens, cache_heads, head_dim = key.shape
+    cache_pages, page_slots = key_cache.shape[:2]
+    query_heads = 0 if query is None else query.shape[1]
+    query_a = None if query is None else _f32(query)
+    query_out = None if query is None else np.zeros_like(query_a)
+    pg = np.ascontiguousarray(pages, dtype=np.int64)
+    sl = np.ascontiguousarray(slots, dtype=np.int64)
+    def norm(spec):
+        if spec is None:
+            return 0, 0.0, None
+        eps, weight = spec
+        return 1, float(eps), (None if weight is None else _f32(weight))
+    qn, qe, qw = norm(query_norm)
+    kn, ke, kw = norm(key_norm)
+    status = lib().oracle_rotary_cache_write_f32(
+        _ptr(query_out), _ptr(key_cache), _ptr(value_cache), _ptr(query_a), _ptr(key), _ptr(value), _ptr(cos), _ptr(sin),
+        _ptr(pg), _ptr(sl), _c_size(tokens), _c_size(query_heads), _c_size(cache_heads), _c_size(head_dim),
+        _c_size(cache_pages), _c_size(page_slots), _c_int(qn), _c_float(qe), _ptr(qw), _c_int(kn), _c_float(ke), _ptr(kw))
+    return int(status), query_out, key_cache, value_cache
+
+
+def paging_indices(query_offsets, page_offsets, pages, last_page_lengths, *, tokens, page_size, cache_pages, width,
+                   row_elements):
+    """CSR paging -> block-table paging (kernel_plan/source/paged_attention.rs:325-398).  Returns (status,
+    packed_offsets, query_lengths, key_lengths, page_table [sequences, width])."""
+    qo = np.ascontiguousarray(query_offsets, dtype=np.int64)
+    po = np.ascontiguousarray(page_offsets, dtype=np.int64)
+    pg = np.ascontiguousarray(pages, dtype=np.int64)
+    lp = np.ascontiguousarray(last_page_lengths, dtype=np.int64)
+    sequences = len(lp)
+    packed = np.zeros(sequences + 1, dtype=np.int32)
+    query_lengths = np.zeros(sequences, dtype=np.int32)
+    key_lengths = np.zeros(sequences, dtype=np.int32)
+    table = np.zeros((sequences, width), dtype=np.int32)
+    status = lib().oracle_paging_indices(_ptr(packed), _ptr(query_lengths), _ptr(key_lengths), _ptr(table), _ptr(qo), _ptr(po),
+                                         _ptr(pg), _ptr(lp), _c_size(sequences), _c_i64(tokens), _c_i64(len(pg)),
+                                         _c_i64(page_size), _c_i64(cache_pages), _c_size(width), _c_i64(row_elements))
+    return int(status), packed, query_lengths, key_lengths, table

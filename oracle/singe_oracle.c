@@ -640,6 +640,147 @@ ORACLE_API size_t oracle_paged_slots(uint64_t *slots, uint64_t *key_counts, cons
     return at;
 }
 
+/* ---- rotation and cache append ---------------------------------------------- */
+
+/* singe/src/backend/cpu/normalization/attention.rs:132-188  rotary_embedding
+ * (f32): rows of head_dim values; row r sits at position r % sequence and
+ * rotates its leading `rotary_pairs` INTERLEAVED pairs (2p, 2p+1) by the
+ * angles cos/sin [sequence, rotary_pairs]; the rest of the row is copied. */
+ORACLE_API void oracle_rotary_embedding_f32(float *out, const float *input, const float *cos_table,
+                                            const float *sin_table, size_t rows, size_t sequence,
+                                            size_t head_dim, size_t rotary_pairs) {
+    memcpy(out, input, rows * head_dim * sizeof(float));
+    for (size_t row = 0; row < rows; ++row) {
+        const float *token = input + row * head_dim;
+        float *o = out + row * head_dim;
+        size_t position = row % sequence * rotary_pairs;
+        for (size_t pair = 0; pair < rotary_pairs; ++pair) {
+            float c = cos_table[position + pair], s = sin_table[position + pair];
+            float even = token[2 * pair], odd = token[2 * pair + 1];
+            o[2 * pair] = fmaf(odd, -s, even * c);
+            o[2 * pair + 1] = fmaf(even, s, odd * c);
+        }
+    }
+}
+
+/* One head of the fused rotation kernel
+ * (singe/src/backend/cuda/kernel_plan/source/rotary_cache.rs:92-185): an
+ * optional RMS normalisation, scale = rsqrt(mean(x^2) + eps) times an
+ * optional weight per element, then HALF-SPLIT pairs (p, p + dim/2):
+ * first = a cos - b sin, second = b cos + a sin, angles [dim/2] of the token. */
+static void rotate_head(float *out, const float *x, const float *c, const float *s, size_t dim,
+                        int has_norm, float eps, const float *weight) {
+    size_t half = dim / 2;
+    float scale = 1.0f;
+    if (has_norm) {
+        float squares = 0.0f;
+        for (size_t pair = 0; pair < half; ++pair)
+            squares += x[pair] * x[pair] + x[pair + half] * x[pair + half];
+        scale = 1.0f / sqrtf(squares / (float)dim + eps);
+    }
+    for (size_t pair = 0; pair < half; ++pair) {
+        float a = x[pair], b = x[pair + half];
+        if (has_norm) {
+            a = a * scale;
+            b = b * scale;
+            if (weight) {
+                a = a * weight[pair];
+                b = b * weight[pair + half];
+            }
+        }
+        out[pair] = a * c[pair] - b * s[pair];
+        out[pair + half] = b * c[pair] + a * s[pair];
+    }
+}
+
+/* The fused step before attention, as the reference's kernel runs it
+ * (rotary_cache.rs:249-427): rotates queries [T, H, D] into query_out, rotates
+ * keys [T, G, D] into key_cache[page[t], slot[t], :, :] and copies values
+ * [T, G, D] into value_cache at the same cell; caches are [P, S, G, D] and
+ * only the selected cells are written.  A negative page or slot counts from
+ * the end (rotary_cache.rs:376-381); one still outside its extent makes the
+ * token's cache writes vanish and the status 1.  query may be NULL (H = 0).
+ * Returns the status. */
+ORACLE_API int oracle_rotary_cache_write_f32(float *query_out, float *key_cache, float *value_cache,
+                                             const float *query, const float *key, const float *value,
+                                             const float *cos_table, const float *sin_table,
+                                             const int64_t *pages, const int64_t *slots, size_t tokens,
+                                             size_t query_heads, size_t cache_heads, size_t head_dim,
+                                             size_t cache_pages, size_t page_slots, int has_query_norm,
+                                             float query_eps, const float *query_weight,
+                                             int has_key_norm, float key_eps, const float *key_weight) {
+    int status = 0;
+    size_t half = head_dim / 2;
+    for (size_t t = 0; t < tokens; ++t) {
+        const float *c = cos_table + t * half, *s = sin_table + t * half;
+        for (size_t h = 0; query && h < query_heads; ++h)
+            rotate_head(query_out + (t * query_heads + h) * head_dim, query + (t * query_heads + h) * head_dim,
+                        c, s, head_dim, has_query_norm, query_eps, query_weight);
+        int64_t page = pages[t], slot = slots[t];
+        if (page < 0) page += (int64_t)cache_pages;
+        if (slot < 0) slot += (int64_t)page_slots;
+        if (page < 0 || page >= (int64_t)cache_pages || slot < 0 || slot >= (int64_t)page_slots) {
+            status = 1;
+            continue;
+        }
+        size_t cell = ((size_t)page * page_slots + (size_t)slot) * cache_heads;
+        for (size_t g = 0; g < cache_heads; ++g) {
+            rotate_head(key_cache + (cell + g) * head_dim, key + (t * cache_heads + g) * head_dim, c, s,
+                        head_dim, has_key_norm, key_eps, key_weight);
+            memcpy(value_cache + (cell + g) * head_dim, value + (t * cache_heads + g) * head_dim,
+                   head_dim * sizeof(float));
+        }
+    }
+    return status;
+}
+
+/* The conversion from CSR paging to block-table paging as the reference's
+ * kernel does it (kernel_plan/source/paged_attention.rs:325-398): packed
+ * offsets from the query offsets clamped into [0, tokens] and made monotone,
+ * query lengths, key lengths ((pages - 1) * page_size + last length, 0 for a
+ * sequence the bounds check refuses), and the page table [sequences, width],
+ * zero-padded, a refused page id left at zero.  Returns the status. */
+ORACLE_API int oracle_paging_indices(int32_t *packed_offsets, int32_t *query_lengths, int32_t *key_lengths,
+                                     int32_t *page_table, const int64_t *query_offsets,
+                                     const int64_t *page_offsets, const int64_t *pages,
+                                     const int64_t *last_page_lengths, size_t sequences, int64_t tokens,
+                                     int64_t page_count, int64_t page_size, int64_t cache_pages, size_t width,
+                                     int64_t row_elements) {
+    int status = 0;
+    memset(page_table, 0, sequences * width * sizeof(int32_t));
+    /* prefix[i] = max over j <= i of the clamped offsets: sequence s starts at
+     * prefix[s] and ends at prefix[s + 1] (paged_attention.rs:366-381). */
+    int64_t running = 0, start = 0;
+    for (size_t i = 0; i <= sequences; ++i) {
+        int64_t offset = query_offsets[i];
+        offset = offset < 0 ? 0 : (offset > tokens ? tokens : offset);
+        if (offset > running) running = offset;
+        if (i > 0) query_lengths[i - 1] = (int32_t)(running - start);
+        packed_offsets[i] = (int32_t)(running * row_elements);
+        start = running;
+    }
+    for (size_t s = 0; s < sequences; ++s) {
+        key_lengths[s] = 0;
+        int64_t qs = query_offsets[s], qe = query_offsets[s + 1], ps = page_offsets[s], pe = page_offsets[s + 1];
+        int64_t last = last_page_lengths[s];
+        if (qs < 0 || qe < qs || qe > tokens || ps < 0 || pe < ps || pe > page_count ||
+            (pe > ps && (last < 0 || last > page_size))) {
+            status = 1;
+            continue;
+        }
+        key_lengths[s] = (int32_t)(pe > ps ? (pe - ps - 1) * page_size + last : 0);
+        for (size_t entry = 0; entry < width && ps + (int64_t)entry < pe; ++entry) {
+            int64_t page = pages[ps + (int64_t)entry];
+            if (page < 0 || page >= cache_pages) {
+                status = 1;
+                continue;
+            }
+            page_table[s * width + entry] = (int32_t)page;
+        }
+    }
+    return status;
+}
+
 /* ---- fp8 KV cache --------------------------------------------------------- */
 
 /* Dequantises an fp8-e4m3 cache [blocks, block_size, kv_heads, dim] with one

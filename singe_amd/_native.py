@@ -70,6 +70,20 @@ class SplitKReduceConfigC(ctypes.Structure):
         "lse_batch_stride", "lse_head_stride", "output_batch_stride", "output_head_stride")]
 
 
+class RotaryCacheProblemC(ctypes.Structure):
+    _fields_ = [("tokens", ctypes.c_int64), ("query_heads", ctypes.c_int64), ("cache_heads", ctypes.c_int64),
+                ("head_dim", ctypes.c_int64), ("cache_pages", ctypes.c_int64), ("page_slots", ctypes.c_int64),
+                ("data_type", ctypes.c_int32), ("table_type", ctypes.c_int32), ("index_type", ctypes.c_int32),
+                ("has_query_norm", ctypes.c_uint8), ("has_key_norm", ctypes.c_uint8), ("query_eps", ctypes.c_float),
+                ("key_eps", ctypes.c_float)]
+
+
+class PagingIndicesProblemC(ctypes.Structure):
+    _fields_ = [("sequences", ctypes.c_int64), ("tokens", ctypes.c_int64), ("page_count", ctypes.c_int64),
+                ("page_size", ctypes.c_int64), ("cache_pages", ctypes.c_int64), ("width", ctypes.c_int64),
+                ("row_elements", ctypes.c_int64), ("index_type", ctypes.c_int32)]
+
+
 DATA_TYPE_F32, DATA_TYPE_BF16, DATA_TYPE_F16 = 0, 1, 2
 
 _lib = None
@@ -156,6 +170,10 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_splitk_reduce_f32.argtypes = [c_void, c_void, c_size, c_void, c_size, c_void, c_size,
                                                    ctypes.POINTER(SplitKReduceConfigC)]
     handle.singe_hip_splitk_reduce_f32.restype = i32
+    handle.singe_hip_rotary_cache_write.argtypes = [c_void] * 14 + [ctypes.POINTER(RotaryCacheProblemC)]
+    handle.singe_hip_rotary_cache_write.restype = i32
+    handle.singe_hip_paging_indices.argtypes = [c_void] * 10 + [ctypes.POINTER(PagingIndicesProblemC)]
+    handle.singe_hip_paging_indices.restype = i32
     _lib = handle
     return handle
 

@@ -1,0 +1,176 @@
+// The steps either side of paged attention in a decode layer:
+//
+//  * singe_rotary_cache_write_*: rotates queries and keys and appends keys and values to the paged cache in
+//    one launch, the gfx950 counterpart of the reference's rotary_cache_write kernel
+//    (singe/src/backend/cuda/kernel_plan/source/rotary_cache.rs:249-427): query [T, H, D], key / value
+//    [T, G, D], angles cos / sin [T, D / 2], one (page, slot) per token, caches [P, S, G, D]; half-split
+//    pairs (p, p + D / 2): first = a cos - b sin, second = b cos + a sin, after an optional RMS
+//    normalisation with an optional per-element weight (rotary_cache.rs:92-185).
+//  * singe_paging_indices: turns FlashInfer CSR paging (query offsets, page offsets, pages, last page
+//    lengths) into per-sequence packed offsets, query lengths, key lengths and a dense page table
+//    [sequences, width], the form block-table kernels read (kernel_plan/source/paged_attention.rs:325-398).
+//
+// Both are bound by memory traffic and small; sixteen lanes take one head.
+#include "common.hip.h"
+#include "kernel_args.h"
+#include "paging.hip.h"
+
+namespace cache_ops {
+
+template <uint32_t ELEMENT>
+struct Element;
+template <>
+struct Element<kElementF32> {
+    typedef float type;
+    static SINGE_DEVICE float load(const type* at) { return *at; }
+    static SINGE_DEVICE void store(type* at, float value) { *at = value; }
+};
+template <>
+struct Element<kElementBf16> {
+    typedef unsigned short type;
+    static SINGE_DEVICE float load(const type* at) { return __builtin_bit_cast(float, static_cast<unsigned int>(*at) << 16); }
+    static SINGE_DEVICE void store(type* at, float value) { *at = f32_to_bf16_bits(value); }
+};
+template <>
+struct Element<kElementF16> {
+    typedef _Float16 type;
+    static SINGE_DEVICE float load(const type* at) { return static_cast<float>(*at); }
+    static SINGE_DEVICE void store(type* at, float value) { *at = static_cast<_Float16>(value); }
+};
+
+SINGE_DEVICE float table_value(const void* table, uint32_t table_type, size_t at) {
+    if (table_type == kElementF32) return static_cast<const float*>(table)[at];
+    if (table_type == kElementBf16) return Element<kElementBf16>::load(static_cast<const unsigned short*>(table) + at);
+    return Element<kElementF16>::load(static_cast<const _Float16*>(table) + at);
+}
+
+// Rotates one head: sixteen lanes, lane `part` takes pairs part, part + 16, ...
+template <class E>
+SINGE_DEVICE void rotate_head(typename E::type* to, const typename E::type* from, const RotaryCacheArgs& a, size_t token,
+                              unsigned int part, bool has_norm, float eps, const void* weight) {
+    const unsigned int half = a.head_dim / 2;
+    float scale = 1.0f;
+    if (has_norm) {
+        float squares = 0.0f;
+        for (unsigned int pair = part; pair < half; pair += 16) {
+            const float first = E::load(from + pair), second = E::load(from + pair + half);
+            squares += first * first + second * second;
+        }
+#pragma unroll
+        for (int step = 1; step < 16; step <<= 1) squares += __shfl_xor(squares, step, 16);
+        scale = rsqrtf(squares / static_cast<float>(a.head_dim) + eps);
+    }
+    for (unsigned int pair = part; pair < half; pair += 16) {
+        float first = E::load(from + pair), second = E::load(from + pair + half);
+        if (has_norm) {
+            first *= scale;
+            second *= scale;
+            if (weight != nullptr) {
+                first *= E::load(static_cast<const typename E::type*>(weight) + pair);
+                second *= E::load(static_cast<const typename E::type*>(weight) + pair + half);
+            }
+        }
+        const float cosine = table_value(a.cos, a.table_type, token * half + pair);
+        const float sine = table_value(a.sin, a.table_type, token * half + pair);
+        E::store(to + pair, first * cosine - second * sine);
+        E::store(to + pair + half, second * cosine + first * sine);
+    }
+}
+
+template <uint32_t ELEMENT>
+SINGE_DEVICE void rotary_cache_write_body(const RotaryCacheArgs& a) {
+    typedef Element<ELEMENT> E;
+    typedef typename E::type T;
+    const unsigned int part = threadIdx.x & 15u;
+    const unsigned long long item = static_cast<unsigned long long>(blockIdx.x) * (blockDim.x / 16) + (threadIdx.x >> 4);
+    const unsigned int total_heads = a.query_heads + 2 * a.cache_heads;
+    if (item >= static_cast<unsigned long long>(a.tokens) * total_heads) return;
+    const size_t token = static_cast<size_t>(item / total_heads);
+    const unsigned int local = static_cast<unsigned int>(item % total_heads);
+    if (local < a.query_heads) {
+        const size_t at = (token * a.query_heads + local) * a.head_dim;
+        rotate_head<E>(static_cast<T*>(a.query_out) + at, static_cast<const T*>(a.query) + at, a, token, part, a.has_query_norm != 0,
+                       a.query_eps, a.query_weight);
+        return;
+    }
+    // Where the token goes: a negative page or slot counts from the end (rotary_cache.rs:376-381).
+    long long page = a.wide_index ? static_cast<const long long*>(a.pages)[token] : static_cast<const int*>(a.pages)[token];
+    long long slot = a.wide_index ? static_cast<const long long*>(a.slots)[token] : static_cast<const int*>(a.slots)[token];
+    if (page < 0) page += a.cache_pages;
+    if (slot < 0) slot += a.page_slots;
+    if (page < 0 || page >= static_cast<long long>(a.cache_pages) || slot < 0 || slot >= static_cast<long long>(a.page_slots)) {
+        if (part == 0) report_index_error(a.status);
+        return;
+    }
+    const size_t cell = (static_cast<size_t>(page) * a.page_slots + static_cast<size_t>(slot)) * a.cache_heads;
+    if (local < a.query_heads + a.cache_heads) {
+        const unsigned int head = local - a.query_heads;
+        rotate_head<E>(static_cast<T*>(a.key_cache) + (cell + head) * a.head_dim,
+                       static_cast<const T*>(a.key) + (token * a.cache_heads + head) * a.head_dim, a, token, part, a.has_key_norm != 0,
+                       a.key_eps, a.key_weight);
+        return;
+    }
+    const unsigned int head = local - a.query_heads - a.cache_heads;
+    const T* from = static_cast<const T*>(a.value) + (token * a.cache_heads + head) * a.head_dim;
+    T* to = static_cast<T*>(a.value_cache) + (cell + head) * a.head_dim;
+    for (unsigned int dim = part; dim < a.head_dim; dim += 16) to[dim] = from[dim];
+}
+
+template <bool WIDE>
+SINGE_DEVICE void paging_indices_body(const PagingIndicesArgs& a) {
+    constexpr int FORM = WIDE ? kCsrI64 : kCsrI32;
+    const unsigned long long index = static_cast<unsigned long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    if (index >= static_cast<unsigned long long>(a.sequences) * a.width) return;
+    const unsigned int sequence = static_cast<unsigned int>(index / a.width), entry = static_cast<unsigned int>(index % a.width);
+    a.page_table[index] = 0;
+    if (entry == 0) {
+        // Offsets clamped into [0, tokens] and made monotone, so what is written stays inside every buffer
+        // whatever the input holds (paged_attention.rs:366-378).
+        long long running = 0, sequence_start = 0;
+        for (unsigned int other = 0; other <= sequence + 1; ++other) {
+            long long offset = read_index<FORM>(a.query_offsets, other);
+            offset = offset < 0 ? 0 : (offset > static_cast<long long>(a.tokens) ? static_cast<long long>(a.tokens) : offset);
+            if (offset > running) running = offset;
+            if (other == sequence) sequence_start = running;
+        }
+        a.packed_offsets[sequence] = static_cast<int>(sequence_start * a.row_elements);
+        if (sequence + 1 == a.sequences) a.packed_offsets[sequence + 1] = static_cast<int>(running * a.row_elements);
+        a.query_lengths[sequence] = static_cast<int>(running - sequence_start);
+        a.key_lengths[sequence] = 0;
+    }
+    const SequenceSpan span = load_span<FORM>(sequence, a.query_offsets, a.page_offsets, a.last_page_lengths, nullptr, a.tokens,
+                                              a.page_count, a.page_size);
+    if (!span.valid) {
+        report_index_error(a.status);
+        return;
+    }
+    if (entry == 0) a.key_lengths[sequence] = static_cast<int>(span.keys);
+    const long long page_end = read_index<FORM>(a.page_offsets, sequence + 1);
+    const long long table_entry = span.page_start + entry;
+    if (table_entry < page_end) {
+        const long long page = read_index<FORM>(a.pages, static_cast<size_t>(table_entry));
+        if (page < 0 || page >= static_cast<long long>(a.cache_pages)) {
+            report_index_error(a.status);
+            return;
+        }
+        a.page_table[index] = static_cast<int>(page);
+    }
+}
+
+}  // namespace cache_ops
+
+extern "C" __global__ __launch_bounds__(256) void singe_rotary_cache_write_f32(RotaryCacheArgs args) {
+    cache_ops::rotary_cache_write_body<kElementF32>(args);
+}
+extern "C" __global__ __launch_bounds__(256) void singe_rotary_cache_write_bf16(RotaryCacheArgs args) {
+    cache_ops::rotary_cache_write_body<kElementBf16>(args);
+}
+extern "C" __global__ __launch_bounds__(256) void singe_rotary_cache_write_f16(RotaryCacheArgs args) {
+    cache_ops::rotary_cache_write_body<kElementF16>(args);
+}
+extern "C" __global__ __launch_bounds__(256) void singe_paging_indices_i32(PagingIndicesArgs args) {
+    cache_ops::paging_indices_body<false>(args);
+}
+extern "C" __global__ __launch_bounds__(256) void singe_paging_indices_i64(PagingIndicesArgs args) {
+    cache_ops::paging_indices_body<true>(args);
+}

@@ -162,3 +162,40 @@ struct GeneralPagedArgs {
     uint32_t causal, has_softcap, wide_index;
     float scale, softcap;
 };
+
+// singe_rotary_cache_write_*: contiguous operands of one element type; angles may be f32.
+struct RotaryCacheArgs {
+    const void* query;          // [tokens, query_heads, dim] or null when query_heads is 0
+    const void* key;            // [tokens, cache_heads, dim]
+    const void* value;          // [tokens, cache_heads, dim]
+    const void* cos;            // [tokens, dim / 2]
+    const void* sin;
+    const void* pages;          // [tokens] i32 or i64
+    const void* slots;
+    const void* query_weight;   // [dim] or null
+    const void* key_weight;
+    void* query_out;            // [tokens, query_heads, dim]
+    void* key_cache;            // [cache_pages, page_slots, cache_heads, dim]
+    void* value_cache;
+    uint32_t* status;
+    uint32_t tokens, query_heads, cache_heads, head_dim, cache_pages, page_slots;
+    uint32_t table_type;        // element type of cos / sin
+    uint32_t wide_index;
+    uint32_t has_query_norm, has_key_norm;
+    float query_eps, key_eps;
+};
+
+// singe_paging_indices_*: FlashInfer CSR paging -> block-table paging.
+struct PagingIndicesArgs {
+    const void* query_offsets;      // [sequences + 1]
+    const void* page_offsets;       // [sequences + 1]
+    const void* pages;              // [page_count]
+    const void* last_page_lengths;  // [sequences]
+    int32_t* packed_offsets;        // [sequences + 1]: first element of each sequence's queries
+    int32_t* query_lengths;         // [sequences]
+    int32_t* key_lengths;           // [sequences]
+    int32_t* page_table;            // [sequences, width]
+    uint32_t* status;
+    uint32_t sequences, tokens, page_count, page_size, cache_pages, width;
+    uint64_t row_elements;          // elements of one query token: heads * dim
+};

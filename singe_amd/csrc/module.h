@@ -19,6 +19,8 @@ enum KernelId : int {
     kPagedAttentionI32, kPagedAttentionI64, kPagedAttentionSoftcapI32, kPagedAttentionSoftcapI64,
     kPagedKvPrefill,
     kSplitKReduce,
+    kRotaryCacheF32, kRotaryCacheBf16, kRotaryCacheF16,
+    kPagingIndicesI32, kPagingIndicesI64,
     // general kernels: index = base + 3 * element (f32, bf16, f16) + width (64, 128, 256)
     kDenseGeneral,
     kPagedGeneral = kDenseGeneral + 9,

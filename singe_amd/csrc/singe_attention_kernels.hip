@@ -6,3 +6,4 @@
 #include "paged_attention.hip"
 #include "splitk_reduce.hip"
 #include "general_attention.hip"
+#include "cache_ops.hip"

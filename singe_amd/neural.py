@@ -182,3 +182,94 @@ def paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: t
     if check and int(status.item()) == STATUS_INDEX_OUT_OF_BOUNDS:
         raise error.IndexOutOfBounds("paged attention paging value outside its buffers")
     return output, lse
+
+
+@dataclass(frozen=True)
+class RotationNorm:
+    """The RMS normalisation a rotation applies first (rotary_cache.rs:25-30)."""
+    eps: float
+    weight: torch.Tensor | None = None
+
+
+def rotary_cache_write(query, key, value, cos, sin, pages, slots, key_cache, value_cache, *,
+                       query_norm: RotationNorm | None = None, key_norm: RotationNorm | None = None, stream=None,
+                       status: torch.Tensor | None = None, check: bool = True):
+    """The step before paged attention in a decode layer, as one kernel
+    (singe/src/backend/cuda/kernel_plan/source/rotary_cache.rs:249-427): rotates ``query`` [T, H, D] (or None)
+    and ``key`` [T, G, D] by the angles ``cos`` / ``sin`` [T, D/2] (half-split pairs), and writes the rotated
+    keys and ``value`` [T, G, D] into the caches [P, S, G, D] at (pages[t], slots[t]), in place.  Returns the
+    rotated queries (None without a query).  A page or slot outside the cache raises IndexOutOfBounds."""
+    tensors = [(key, "key"), (value, "value"), (key_cache, "key_cache"), (value_cache, "value_cache")]
+    if query is not None:
+        tensors.append((query, "query"))
+    for tensor, name in tensors:
+        if not tensor.is_cuda or tensor.dtype != key.dtype or not tensor.is_contiguous():
+            raise error.InvalidArgument(f"rotary cache {name} must be a contiguous device tensor of the key's type")
+    if key.dtype not in _DATA_TYPES or cos.dtype not in _DATA_TYPES or sin.dtype != cos.dtype:
+        raise error.InvalidArgument("rotary cache data type")
+    tokens, cache_heads, head_dim = key.shape
+    if value.shape != key.shape or key_cache.shape != value_cache.shape or key_cache.dim() != 4:
+        raise error.InvalidArgument("rotary cache value or cache shape")
+    cache_pages, page_slots = key_cache.shape[:2]
+    if tuple(key_cache.shape[2:]) != (cache_heads, head_dim):
+        raise error.InvalidArgument("rotary cache heads or head dimension")
+    cos, sin = cos.contiguous(), sin.contiguous()
+    if cos.numel() != tokens * (head_dim // 2) or sin.numel() != cos.numel():
+        raise error.InvalidArgument("rotary cache angles must be [tokens, 1, head_dim / 2]")
+    if pages.dtype != slots.dtype or pages.dtype not in (torch.int32, torch.int64) or pages.numel() != tokens or slots.numel() != tokens:
+        raise error.InvalidArgument("rotary cache pages and slots must be [tokens] of one integer type")
+    query_heads = 0 if query is None else query.shape[1]
+    query_out = None if query is None else torch.empty_like(query)
+    weights = []
+    for norm in (query_norm, key_norm):
+        weight = None if norm is None or norm.weight is None else norm.weight.to(key.dtype).contiguous()
+        if weight is not None and weight.numel() != head_dim:
+            raise error.InvalidArgument("rotary cache norm weight must hold head_dim values")
+        weights.append(weight)
+    problem = _native.RotaryCacheProblemC(
+        tokens, query_heads, cache_heads, head_dim, cache_pages, page_slots, _DATA_TYPES[key.dtype], _DATA_TYPES[cos.dtype],
+        1 if pages.dtype == torch.int64 else 0, 1 if query_norm is not None else 0, 1 if key_norm is not None else 0,
+        query_norm.eps if query_norm is not None else 0.0, key_norm.eps if key_norm is not None else 0.0)
+    if status is None:
+        status = torch.zeros(1, device=key.device, dtype=torch.int32)
+    pointer = lambda tensor: tensor.data_ptr() if tensor is not None else None
+    handle = int((stream or torch.cuda.current_stream()).cuda_stream)
+    code = _native.lib().singe_hip_rotary_cache_write(
+        handle, pointer(query), key.data_ptr(), value.data_ptr(), cos.data_ptr(), sin.data_ptr(), pages.contiguous().data_ptr(),
+        slots.contiguous().data_ptr(), pointer(weights[0]), pointer(weights[1]), pointer(query_out), key_cache.data_ptr(),
+        value_cache.data_ptr(), status.data_ptr(), ctypes.byref(problem))
+    _native.check(code, "rotary_cache_write")
+    if check and int(status.item()) == STATUS_INDEX_OUT_OF_BOUNDS:
+        raise error.IndexOutOfBounds("rotary cache page or slot outside the cache")
+    return query_out
+
+
+def paging_indices(paging: Paging, *, tokens: int, page_size: int, cache_pages: int, width: int, row_elements: int,
+                   stream=None, status: torch.Tensor | None = None, check: bool = True):
+    """FlashInfer CSR paging -> block-table paging, on the device
+    (singe/src/backend/cuda/kernel_plan/source/paged_attention.rs:325-398).  Returns int32 tensors
+    (packed_offsets [sequences + 1], query_lengths [sequences], key_lengths [sequences],
+    page_table [sequences, width])."""
+    indices = (paging.query_offsets, paging.page_offsets, paging.pages, paging.last_page_lengths)
+    kinds = {t.dtype for t in indices}
+    if len(kinds) != 1 or not kinds <= {torch.int32, torch.int64}:
+        raise error.InvalidArgument("paging index tensors must share one integer type")
+    sequences = paging.last_page_lengths.numel()
+    device = paging.pages.device
+    packed = torch.zeros(sequences + 1, device=device, dtype=torch.int32)
+    query_lengths = torch.zeros(sequences, device=device, dtype=torch.int32)
+    key_lengths = torch.zeros(sequences, device=device, dtype=torch.int32)
+    table = torch.zeros((sequences, width), device=device, dtype=torch.int32)
+    if status is None:
+        status = torch.zeros(1, device=device, dtype=torch.int32)
+    problem = _native.PagingIndicesProblemC(sequences, tokens, paging.pages.numel(), page_size, cache_pages, width, row_elements,
+                                            1 if paging.pages.dtype == torch.int64 else 0)
+    handle = int((stream or torch.cuda.current_stream()).cuda_stream)
+    code = _native.lib().singe_hip_paging_indices(
+        handle, paging.query_offsets.data_ptr(), paging.page_offsets.data_ptr(), paging.pages.data_ptr(),
+        paging.last_page_lengths.data_ptr(), packed.data_ptr(), query_lengths.data_ptr(), key_lengths.data_ptr(), table.data_ptr(),
+        status.data_ptr(), ctypes.byref(problem))
+    _native.check(code, "paging_indices")
+    if check and int(status.item()) == STATUS_INDEX_OUT_OF_BOUNDS:
+        raise error.IndexOutOfBounds("paging value outside its buffers")
+    return packed, query_lengths, key_lengths, table

@@ -507,3 +507,89 @@ def test_fp8_cache_dequantises_to_bf16_values():
     table = oracle.f8e4m3_table()
     want = torch.from_numpy(table[codes] * scales[:, None, :, None]).to(torch.bfloat16).float().numpy()
     assert np.array_equal(got, want)
+
+
+# ---- rotation, cache append and the paging bridge ---------------------------------------------------
+
+def test_rotary_embedding_closed_forms():
+    """Angle 0 is the identity, a quarter turn maps (even, odd) to (-odd, even), rotation keeps each
+    pair's length, and positions repeat with the sequence length (cpu/normalization/attention.rs:172-185)."""
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((2, 3, 5, 8)).astype(np.float32)
+    pairs = 3  # the last pair of each row is not rotated
+    zeros, ones = np.zeros((5, pairs), np.float32), np.ones((5, pairs), np.float32)
+    assert np.array_equal(oracle.rotary_embedding_f32(x, ones, zeros), x)
+    quarter = oracle.rotary_embedding_f32(x, zeros, ones)
+    assert np.array_equal(quarter[..., 0:6:2], -x[..., 1:6:2]) and np.array_equal(quarter[..., 1:6:2], x[..., 0:6:2])
+    assert np.array_equal(quarter[..., 6:], x[..., 6:])
+    angle = rng.uniform(0, 6.28, (5, pairs)).astype(np.float32)
+    turned = oracle.rotary_embedding_f32(x, np.cos(angle), np.sin(angle))
+    lengths = lambda v: v[..., 0:6:2] ** 2 + v[..., 1:6:2] ** 2
+    assert np.allclose(lengths(turned), lengths(x), rtol=1e-5)
+    want = x[..., 0:6:2] * np.cos(angle) - x[..., 1:6:2] * np.sin(angle)  # position = row % sequence
+    assert np.allclose(turned[..., 0:6:2], want, atol=1e-6)
+
+
+def test_rotary_cache_write_closed_forms():
+    """Half-split pairs, cells chosen by (page, slot), untouched cells kept, negative indices counted from the
+    end, an index outside the cache reported and skipped (rotary_cache.rs:92-185, 367-400)."""
+    rng = np.random.default_rng(5)
+    tokens, heads, groups, dim, pages, slots = 4, 3, 2, 8, 3, 4
+    q = rng.standard_normal((tokens, heads, dim)).astype(np.float32)
+    k = rng.standard_normal((tokens, groups, dim)).astype(np.float32)
+    v = rng.standard_normal((tokens, groups, dim)).astype(np.float32)
+    kc = rng.standard_normal((pages, slots, groups, dim)).astype(np.float32)
+    vc = rng.standard_normal((pages, slots, groups, dim)).astype(np.float32)
+    angle = rng.uniform(0, 6.28, (tokens, dim // 2)).astype(np.float32)
+    page_index, slot_index = [2, 0, -1, 1], [1, 3, -4, 2]
+    status, q_out, kc_out, vc_out = oracle.rotary_cache_write_f32(q, k, v, np.cos(angle), np.sin(angle), page_index, slot_index, kc, vc)
+    assert status == 0
+    half = dim // 2
+    want = np.concatenate([q[..., :half] * np.cos(angle)[:, None] - q[..., half:] * np.sin(angle)[:, None],
+                           q[..., half:] * np.cos(angle)[:, None] + q[..., :half] * np.sin(angle)[:, None]], axis=-1)
+    assert np.allclose(q_out, want, atol=1e-6)
+    cells = [(2, 1), (0, 3), (2, 0), (1, 2)]  # -1 -> page 2, -4 -> slot 0
+    touched = np.zeros((pages, slots), bool)
+    for t, (p, s) in enumerate(cells):
+        touched[p, s] = True
+        assert np.array_equal(vc_out[p, s], v[t])
+        assert np.allclose(np.linalg.norm(kc_out[p, s], axis=-1), np.linalg.norm(k[t], axis=-1), rtol=1e-5)
+    assert np.array_equal(kc_out[~touched], kc[~touched]) and np.array_equal(vc_out[~touched], vc[~touched])
+    # identity angles + RMS norm with a weight: x / rms(x) * w
+    weight = rng.standard_normal(dim).astype(np.float32)
+    ones, zeros = np.ones((tokens, half), np.float32), np.zeros((tokens, half), np.float32)
+    _, q_norm, _, _ = oracle.rotary_cache_write_f32(q, k, v, ones, zeros, page_index, slot_index, kc, vc, query_norm=(1e-6, weight))
+    rms = np.sqrt((q.astype(np.float64) ** 2).mean(-1, keepdims=True) + 1e-6)
+    assert np.allclose(q_norm, q / rms * weight, atol=1e-5)
+    # out of range: reported, that token's cells untouched, the others written
+    status, _, kc_bad, _ = oracle.rotary_cache_write_f32(q, k, v, ones, zeros, [2, 3, -1, 1], slot_index, kc, vc)
+    assert status == 1 and np.array_equal(kc_bad[0, 3], kc[0, 3]) and np.array_equal(kc_bad[2, 1], k[0])
+
+
+def test_paging_indices_against_brute_force():
+    """The FlashInfer index set of the reference's generator (conformance.py:1570-1582) and its shuffle
+    recipe (kernel_plan/source/tests.rs:853-889) through the CSR -> table conversion."""
+    status, packed, qlen, klen, table = oracle.paging_indices([0, 1, 6, 9], [0, 3, 5, 5], [4, 0, 6, 2, 5], [2, 3, 0], tokens=9,
+                                                              page_size=4, cache_pages=7, width=4, row_elements=32)
+    assert status == 0
+    assert packed.tolist() == [0, 32, 192, 288] and qlen.tolist() == [1, 5, 3] and klen.tolist() == [10, 7, 0]
+    assert table.tolist() == [[4, 0, 6, 0], [2, 5, 0, 0], [0, 0, 0, 0]]
+    for page_size in (1, 16, 7):
+        sequences = [(1, 150), (70, 70), (20, 90), (3, 0)]
+        qo, po, last = [0], [0], []
+        for queries, keys in sequences:
+            qo.append(qo[-1] + queries)
+            n = -(-keys // page_size)
+            po.append(po[-1] + n)
+            last.append(0 if keys == 0 else keys - (n - 1) * page_size)
+        count = po[-1]
+        pages = [(p * 7 + 2) % count for p in range(count)]
+        width = max(b - a for a, b in zip(po, po[1:]))
+        status, packed, qlen, klen, table = oracle.paging_indices(qo, po, pages, last, tokens=qo[-1], page_size=page_size,
+                                                                  cache_pages=count, width=width, row_elements=1)
+        assert status == 0 and klen.tolist() == [k for _, k in sequences] and qlen.tolist() == [q for q, _ in sequences]
+        for s, (a, b) in enumerate(zip(po, po[1:])):
+            assert table[s, :b - a].tolist() == pages[a:b] and not table[s, b - a:].any()
+    # the reference's invalid tuples are refused here too
+    assert oracle.paging_indices([0, 1, 3], [0, 2, 3], [1, 0, 3], [2, 1], tokens=3, page_size=4, cache_pages=3, width=2, row_elements=1)[0] == 1
+    assert oracle.paging_indices([0, 2, 1], [0, 2, 3], [1, 0, 2], [2, 1], tokens=3, page_size=4, cache_pages=3, width=2, row_elements=1)[0] == 1
