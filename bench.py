@@ -242,7 +242,7 @@ def fp8_decode_section(steps):
         "tokens_per_s": work.batch / (avg * 1e-3),
         "ms_per_step": avg,
         "algorithmic_bytes": nbytes,
-        "roofline": {"bound": "hbm", "kernel": "singe_paged_decode_f8kv_d128_g2_b16", "achieved": gbps, "peak": HBM_PEAK_GBPS,
+        "roofline": {"bound": "hbm", "kernel": "singe_paged_decode_f8kv_wide_d128_b16", "achieved": gbps, "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": None, "step_avg_us": avg * 1e3,
                      "step_median_us": median * 1e3},
     }

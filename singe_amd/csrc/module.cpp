@@ -15,11 +15,9 @@ namespace singe_hip {
 const char* const kKernelNames[kKernelCount] = {
     "singe_paged_decode_bf16_d128_g1_b16", "singe_paged_decode_bf16_d128_g2_b16",
     "singe_paged_decode_bf16_d128_g1_any", "singe_paged_decode_bf16_d128_g2_any",
-    "singe_paged_decode_f8kv_d128_g1_b16", "singe_paged_decode_f8kv_d128_g2_b16",
-    "singe_paged_decode_f8kv_d128_g1_any", "singe_paged_decode_f8kv_d128_g2_any",
-    "singe_paged_decode_f8kv_relaxed_d128_g1_b16", "singe_paged_decode_f8kv_relaxed_d128_g2_b16",
-    "singe_paged_decode_f8kv_relaxed_d128_g1_any", "singe_paged_decode_f8kv_relaxed_d128_g2_any",
     "singe_paged_decode_combine_bf16",
+    "singe_paged_decode_f8kv_wide_d128_b16", "singe_paged_decode_f8kv_wide_d128_any",
+    "singe_paged_decode_f8kv_wide_relaxed_d128_b16", "singe_paged_decode_f8kv_wide_relaxed_d128_any",
     "singe_fmha_prefill_bf16_d128_causal", "singe_fmha_prefill_bf16_d128_full",
     "singe_fmha_prefill_f32_d32", "singe_fmha_prefill_f32_d64", "singe_fmha_prefill_f32_d128", "singe_fmha_prefill_f32_d256",
     "singe_paged_attention_bf16_d128_i32", "singe_paged_attention_bf16_d128_i64",

@@ -9,11 +9,11 @@ namespace singe_hip {
 
 // Kernels of the code object, in the order of kKernelNames.
 enum KernelId : int {
-    // paged decode: index = base + 2 * (block size not a multiple of 16) + (two head groups per wave)
+    // bf16 paged decode: index = 2 * (block size not a multiple of 16) + (two head groups per wave)
     kDecodeBf16 = 0,
-    kDecodeF8 = 4,
-    kDecodeF8Relaxed = 8,
-    kDecodeCombine = 12,
+    kDecodeCombine = 4,
+    // fp8 decode, dense form: + (block size not a multiple of 16) + 2 * relaxed
+    kDecodeF8Wide, kDecodeF8WideAny, kDecodeF8WideRelaxed, kDecodeF8WideRelaxedAny,
     kPrefillCausal, kPrefillFull,
     kPrefillF32D32, kPrefillF32D64, kPrefillF32D128, kPrefillF32D256,
     kPagedAttentionI32, kPagedAttentionI64, kPagedAttentionSoftcapI32, kPagedAttentionSoftcapI64,

@@ -220,8 +220,9 @@ int32_t decode(
     args.scale_log2e = c.scale * 1.4426950408889634074f;
 
     const bool aligned = c.block_size % 16 == 0;
-    const int family = !fp8 ? kDecodeBf16 : (g_relaxed.load(std::memory_order_relaxed) ? kDecodeF8Relaxed : kDecodeF8);
-    KernelId kernel = static_cast<KernelId>(family + (aligned ? 0 : 2) + (plan.groups == 2 ? 1 : 0));
+    // bf16 caches take the one-hot form, fp8 caches the dense form (see paged_decode.hip).
+    const KernelId kernel = fp8 ? static_cast<KernelId>(kDecodeF8Wide + (aligned ? 0 : 1) + (g_relaxed.load(std::memory_order_relaxed) ? 2 : 0))
+                                : static_cast<KernelId>(kDecodeBf16 + (aligned ? 0 : 2) + (plan.groups == 2 ? 1 : 0));
     if (phases & SINGE_HIP_DECODE_SPLIT)
         if (int32_t status = launch(kernel, plan.grid_x, plan.grid_y, 1, 64 * kWavesPerWorkgroup, stream, args,
                                     static_cast<unsigned>((2 * c.batch + 1) * sizeof(uint32_t))))

@@ -35,7 +35,9 @@
 // fp8 caches are widened to bf16 in registers on their way into the MFMA operands.  In the exact mode
 // every element becomes bf16_rne(f8e4m3_value(code) * scale) first (the value the CPU path reads after
 // dequantising the cache); in the relaxed mode the codes are widened exactly and the block's scale is
-// applied to the 32 scores / probabilities of the tile instead, which saves one multiply per element.
+// applied to the 32 scores / probabilities of the tile instead, which saves the multiply and half of the
+// conversions.  They take a different inner loop (WIDE below): an fp8 cache halves the bytes per key, so
+// the one-hot form's spare multiplies and repeated exponentials are no longer free.
 #include "common.hip.h"
 #include "kernel_args.h"
 
@@ -271,12 +273,23 @@ SINGE_DEVICE unsigned int bf16_pair(float lo, float hi) {
 // bf16(value) in both halves of a dword (one v_cvt_pk_bf16_f32, round to nearest even).
 SINGE_DEVICE unsigned int bf16_twice(float value) { return bf16_pair(value, value); }
 
-// Eight fp8 e4m3 codes -> eight bf16 values bf16_rne(value(code) * scale); scale 1 widens exactly.
+// Eight fp8 e4m3 codes -> eight bf16 values.  EXACT: bf16_rne(value(code) * scale), the value the CPU path
+// reads after dequantising the cache.  Otherwise the codes are widened as they are (every e4m3 value is a
+// bf16 value), which v_cvt_scalef32_pk_bf16_fp8 does for two codes at a time; its scale operand only
+// carries a power of two, so it cannot stand in for the multiply above.
+template <bool EXACT>
 SINGE_DEVICE uint4 widen_fp8x8(unsigned int low, unsigned int high, float scale) {
-    const f32x2_t a = __builtin_amdgcn_cvt_pk_f32_fp8(low, false), b = __builtin_amdgcn_cvt_pk_f32_fp8(low, true);
-    const f32x2_t c = __builtin_amdgcn_cvt_pk_f32_fp8(high, false), d = __builtin_amdgcn_cvt_pk_f32_fp8(high, true);
-    return make_uint4(bf16_pair(a[0] * scale, a[1] * scale), bf16_pair(b[0] * scale, b[1] * scale),
-                      bf16_pair(c[0] * scale, c[1] * scale), bf16_pair(d[0] * scale, d[1] * scale));
+    if constexpr (EXACT) {
+        const f32x2_t a = __builtin_amdgcn_cvt_pk_f32_fp8(low, false), b = __builtin_amdgcn_cvt_pk_f32_fp8(low, true);
+        const f32x2_t c = __builtin_amdgcn_cvt_pk_f32_fp8(high, false), d = __builtin_amdgcn_cvt_pk_f32_fp8(high, true);
+        return make_uint4(bf16_pair(a[0] * scale, a[1] * scale), bf16_pair(b[0] * scale, b[1] * scale),
+                          bf16_pair(c[0] * scale, c[1] * scale), bf16_pair(d[0] * scale, d[1] * scale));
+    } else {
+        return make_uint4(__builtin_bit_cast(unsigned int, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(low, 1.0f, false)),
+                          __builtin_bit_cast(unsigned int, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(low, 1.0f, true)),
+                          __builtin_bit_cast(unsigned int, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(high, 1.0f, false)),
+                          __builtin_bit_cast(unsigned int, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(high, 1.0f, true)));
+    }
 }
 
 // Per-wave softmax state of one group of four query heads.
@@ -286,9 +299,21 @@ struct GroupState {
     float running_sum;  // of this lane's keys only
 };
 
+// Rows of a wave's private V staging buffer in LDS (WIDE): 256 bytes of bf16 plus 16 bytes of padding, so
+// the sixteen rows a transposing read touches fall into all banks twice over, which is the best 512
+// bytes can do.
+constexpr int kStagedRowBytes = 272;
+constexpr int kStagedTileBytes = kTile * kStagedRowBytes;
+
 // GROUPS = groups of four query heads a wave carries (1 or 2: up to 8 query heads per kv head).
-template <int GROUPS, bool ALIGNED16, bool FP8, bool EXACT>
-SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
+// WIDE (fp8 caches): the query heads of the kv head sit in the sixteen columns of one MFMA, each once, and
+// the values take the dense route: widened V rows are staged in a private LDS buffer and read back
+// transposed (ds_read_b64_tr_b16) as the A operand of v_mfma_f32_16x16x32_bf16, O^T[dim, head] += V^T . P^T.
+// That is a third of the matrix instructions and half the exponentials of the one-hot form, which matters
+// where the byte rate of an fp8 cache leaves the vector and matrix units little time per byte.
+template <int GROUPS, bool ALIGNED16, bool FP8, bool EXACT, bool WIDE = false>
+SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, unsigned char* staging = nullptr) {
+    static_assert(WIDE == FP8 && (!WIDE || GROUPS == 1), "fp8 caches take the wide form, bf16 caches the one-hot form");
     using Tile = typename std::conditional<FP8, KeyTileFp8, KeyTileBf16>::type;
     constexpr int DEPTH = FP8 ? 3 : 2;  // an fp8 tile is half the bytes, so one more is kept in flight
     const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -368,7 +393,26 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
 
     bf16x8_t q[GROUPS][4];
     GroupState state[GROUPS];
+    // WIDE: column t of the score MFMAs is query head t of the wave; acc[db][r] is O^T[16 db + 4 g + r][head t].
+    f32x4_t wide_acc[WIDE ? 8 : 1];
+    float wide_max = -INFINITY, wide_sum = 0.0f;
+    unsigned char* const staged = WIDE ? staging + wave * kStagedTileBytes : nullptr;
     auto load_query = [&](unsigned int b) __attribute__((always_inline)) {
+        if constexpr (WIDE) {
+            const bool real = t < wave_heads;
+            const uint16_t* qp = a.query + (static_cast<size_t>(b) * a.heads + kv_head * group + head_in_group + (real ? t : 0)) * kDim + dim_lane;
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                uint4 bits = *reinterpret_cast<const uint4*>(qp + dim_step * c);
+                if (!real) bits = make_uint4(0, 0, 0, 0);
+                q[0][c] = __builtin_bit_cast(bf16x8_t, bits);
+            }
+#pragma unroll
+            for (int db = 0; db < 8; ++db) wide_acc[db] = {0.0f, 0.0f, 0.0f, 0.0f};
+            wide_max = -INFINITY;
+            wide_sum = 0.0f;
+            return;
+        }
 #pragma unroll
         for (int hg = 0; hg < GROUPS; ++hg) {
             const unsigned int local = 4 * hg + (t >> 2);
@@ -387,7 +431,78 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
         }
     };
 
+    auto fold_wide = [&](const Tile& tile) __attribute__((always_inline)) {
+        if constexpr (WIDE) {
+            // Values first: widened rows go to the staging buffer while the scores are computed.  Lane (g, t)
+            // holds key 16 half + 4 g + i, dims 8 t .. 8 t + 7.
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint4 row = widen_fp8x8<EXACT>(tile.v[half][i].x, tile.v[half][i].y, EXACT ? tile.row_value_scale[half][i] : 1.0f);
+                    *reinterpret_cast<uint4*>(staged + (16 * half + 4 * g + i) * kStagedRowBytes + 16 * t) = row;
+                }
+            // Scores S^T[key 16 half + row][head]: row = lane % 16 of the A operand is key t of the half.
+            f32x4_t s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint4 a0 = tile.k[0][c >> 1], a1 = tile.k[1][c >> 1];
+                const uint4 first = (c & 1) ? widen_fp8x8<EXACT>(a0.z, a0.w, EXACT ? tile.key_scale[0] : 1.0f)
+                                            : widen_fp8x8<EXACT>(a0.x, a0.y, EXACT ? tile.key_scale[0] : 1.0f);
+                const uint4 second = (c & 1) ? widen_fp8x8<EXACT>(a1.z, a1.w, EXACT ? tile.key_scale[1] : 1.0f)
+                                             : widen_fp8x8<EXACT>(a1.x, a1.y, EXACT ? tile.key_scale[1] : 1.0f);
+                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, first), q[0][c], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, second), q[0][c], s1, 0, 0, 0);
+            }
+            // Lane (g, t) now holds head t against keys 16 half + 4 g + i.
+            float p[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float first = s0[i] * a.scale_log2e, second = s1[i] * a.scale_log2e;
+                if constexpr (!EXACT) {
+                    first *= tile.row_key_scale[0][i];
+                    second *= tile.row_key_scale[1][i];
+                }
+                p[i] = (tile.live >> i) & 1u ? first : -INFINITY;
+                p[4 + i] = (tile.live >> (4 + i)) & 1u ? second : -INFINITY;
+            }
+            float largest = fmaxf(fmaxf(fmaxf(p[0], p[1]), fmaxf(p[2], p[3])), fmaxf(fmaxf(p[4], p[5]), fmaxf(p[6], p[7])));
+            largest = fmaxf(across_groups_max(largest), wide_max);
+            const float base = largest == -INFINITY ? 0.0f : largest;
+            const float rescale = fast_exp2(wide_max - base);
+            float total = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                p[i] = fast_exp2(p[i] - base);
+                total += p[i];
+                if constexpr (!EXACT) p[i] *= tile.row_value_scale[i >> 2][i & 3];
+            }
+            wide_sum = wide_sum * rescale + total;
+            wide_max = largest;
+            const uint4 weights = make_uint4(bf16_pair(p[0], p[1]), bf16_pair(p[2], p[3]), bf16_pair(p[4], p[5]), bf16_pair(p[6], p[7]));
+            // O^T[dim, head] += V^T . P^T: k-slots 8 g + j of the MFMA are keys 4 g + j (j < 4) and
+            // 16 + 4 g + j - 4, which is how the two transposing reads of a 16-lane group deliver them.
+            typedef short v4i16_t __attribute__((ext_vector_type(4)));
+            typedef short v8i16_t __attribute__((ext_vector_type(8)));
+            typedef v4i16_t __attribute__((address_space(3))) * lds_v4_t;
+            const unsigned char* patch = staged + (4 * g + (t >> 2)) * kStagedRowBytes + 8 * (t & 3);
+#pragma unroll
+            for (int db = 0; db < 8; ++db) {
+                const v4i16_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(patch + 32 * db));
+                const v4i16_t high = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(patch + 16 * kStagedRowBytes + 32 * db));
+                const v8i16_t both = __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) wide_acc[db][r] *= rescale;
+                wide_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, both), __builtin_bit_cast(bf16x8_t, weights),
+                                                                  wide_acc[db], 0, 0, 0);
+            }
+        }
+    };
     auto fold = [&](const Tile& tile) __attribute__((always_inline)) {
+        if constexpr (WIDE) {
+            fold_wide(tile);
+            return;
+        }
         // Scores of every head group.  fp8 operands are widened right where they are used, so only
         // one widened K chunk and one widened V row are alive at a time.
         f32x4_t s0[GROUPS], s1[GROUPS];
@@ -399,13 +514,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             uint4 first, second;
-            if constexpr (FP8) {
-                const uint4 a0 = tile.k[0][c >> 1], a1 = tile.k[1][c >> 1];
-                first = (c & 1) ? widen_fp8x8(a0.z, a0.w, EXACT ? tile.key_scale[0] : 1.0f)
-                                : widen_fp8x8(a0.x, a0.y, EXACT ? tile.key_scale[0] : 1.0f);
-                second = (c & 1) ? widen_fp8x8(a1.z, a1.w, EXACT ? tile.key_scale[1] : 1.0f)
-                                 : widen_fp8x8(a1.x, a1.y, EXACT ? tile.key_scale[1] : 1.0f);
-            } else {
+            if constexpr (!FP8) {
                 first = tile.k[0][c];
                 second = tile.k[1][c];
             }
@@ -420,11 +529,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
         for (int hg = 0; hg < GROUPS; ++hg) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                float first = s0[hg][i] * a.scale_log2e, second = s1[hg][i] * a.scale_log2e;
-                if constexpr (FP8 && !EXACT) {
-                    first *= tile.row_key_scale[0][i];
-                    second *= tile.row_key_scale[1][i];
-                }
+                const float first = s0[hg][i] * a.scale_log2e, second = s1[hg][i] * a.scale_log2e;
                 p[hg][i] = (tile.live >> i) & 1u ? first : -INFINITY;
                 p[hg][4 + i] = (tile.live >> (4 + i)) & 1u ? second : -INFINITY;
             }
@@ -452,15 +557,10 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 uint4 row;
-                if constexpr (FP8)
-                    row = widen_fp8x8(tile.v[half][i].x, tile.v[half][i].y, EXACT ? tile.row_value_scale[half][i] : 1.0f);
-                else
-                    row = tile.v[half][i];
+                if constexpr (!FP8) row = tile.v[half][i];
 #pragma unroll
                 for (int hg = 0; hg < GROUPS; ++hg) {
-                    float weight = p[hg][half * 4 + i];
-                    if constexpr (FP8 && !EXACT) weight *= tile.row_value_scale[half][i];
-                    const unsigned int both = bf16_twice(weight);
+                    const unsigned int both = bf16_twice(p[hg][half * 4 + i]);
                     const uint2 hot = make_uint2(both & place0, both & place1);
                     state[hg].acc[0] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
                         __builtin_bit_cast(i16x4_t, make_uint2(row.x, row.y)), __builtin_bit_cast(i16x4_t, hot), state[hg].acc[0], 0, 0, 0);
@@ -473,6 +573,19 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix) {
     // Writes the partial row of sequence b: O / sum per head, and the natural-log LSE.
     auto flush = [&](unsigned int b) __attribute__((always_inline)) {
         const size_t slot = static_cast<size_t>(work) * slots + worker + b;
+        if constexpr (WIDE) {
+            const float sum = across_groups_sum(wide_sum);
+            const float inverse = sum > 0.0f ? 1.0f / sum : 0.0f;
+            if (t < wave_heads) {
+                float* row = a.partial_out + (slot * a.heads_per_wave + t) * kDim;
+#pragma unroll
+                for (int db = 0; db < 8; ++db)
+                    *reinterpret_cast<float4*>(row + 16 * db + 4 * g) = make_float4(wide_acc[db][0] * inverse, wide_acc[db][1] * inverse,
+                                                                                    wide_acc[db][2] * inverse, wide_acc[db][3] * inverse);
+                if (g == 0) a.partial_lse[slot * a.heads_per_wave + t] = sum > 0.0f ? (wide_max + fast_log2(sum)) * kLn2 : -INFINITY;
+            }
+            return;
+        }
 #pragma unroll
         for (int hg = 0; hg < GROUPS; ++hg) {
             const float sum = across_groups_sum(state[hg].running_sum);
@@ -567,14 +680,18 @@ SINGE_DECODE_KERNEL(singe_paged_decode_bf16_d128_g1_b16, 1, true, false, true)
 SINGE_DECODE_KERNEL(singe_paged_decode_bf16_d128_g2_b16, 2, true, false, true)
 SINGE_DECODE_KERNEL(singe_paged_decode_bf16_d128_g1_any, 1, false, false, true)
 SINGE_DECODE_KERNEL(singe_paged_decode_bf16_d128_g2_any, 2, false, false, true)
-SINGE_DECODE_KERNEL(singe_paged_decode_f8kv_d128_g1_b16, 1, true, true, true)
-SINGE_DECODE_KERNEL(singe_paged_decode_f8kv_d128_g2_b16, 2, true, true, true)
-SINGE_DECODE_KERNEL(singe_paged_decode_f8kv_d128_g1_any, 1, false, true, true)
-SINGE_DECODE_KERNEL(singe_paged_decode_f8kv_d128_g2_any, 2, false, true, true)
-SINGE_DECODE_KERNEL(singe_paged_decode_f8kv_relaxed_d128_g1_b16, 1, true, true, false)
-SINGE_DECODE_KERNEL(singe_paged_decode_f8kv_relaxed_d128_g2_b16, 2, true, true, false)
-SINGE_DECODE_KERNEL(singe_paged_decode_f8kv_relaxed_d128_g1_any, 1, false, true, false)
-SINGE_DECODE_KERNEL(singe_paged_decode_f8kv_relaxed_d128_g2_any, 2, false, true, false)
+
+#define SINGE_DECODE_WIDE_KERNEL(NAME, ALIGNED, EXACT)                                          \
+    extern "C" __global__ __launch_bounds__(512) void NAME(DecodeArgs args) {                    \
+        extern __shared__ unsigned int prefix[];                                                \
+        __shared__ __attribute__((aligned(16))) unsigned char staging[8 * kStagedTileBytes];    \
+        paged_decode_body<1, ALIGNED, true, EXACT, true>(args, prefix, staging);                \
+    }
+
+SINGE_DECODE_WIDE_KERNEL(singe_paged_decode_f8kv_wide_d128_b16, true, true)
+SINGE_DECODE_WIDE_KERNEL(singe_paged_decode_f8kv_wide_d128_any, false, true)
+SINGE_DECODE_WIDE_KERNEL(singe_paged_decode_f8kv_wide_relaxed_d128_b16, true, false)
+SINGE_DECODE_WIDE_KERNEL(singe_paged_decode_f8kv_wide_relaxed_d128_any, false, false)
 
 // Folds the partial rows of one (sequence, query head) into the bf16 output:
 // out = sum_s exp(lse_s - max) * partial_s / sum_s exp(lse_s - max)

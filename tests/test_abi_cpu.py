@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
 def test_code_object_is_built_and_names_every_kernel():
     assert os.path.exists(_native.CODE_OBJECT_PATH)
     image = open(_native.CODE_OBJECT_PATH, "rb").read()
-    for kernel in (b"singe_paged_decode_bf16_d128_g1_b16", b"singe_paged_decode_f8kv_d128_g2_b16",
+    for kernel in (b"singe_paged_decode_bf16_d128_g1_b16", b"singe_paged_decode_f8kv_wide_d128_b16",
                    b"singe_paged_decode_combine_bf16", b"singe_fmha_prefill_bf16_d128_causal",
                    b"singe_fmha_prefill_f32_d64", b"singe_paged_attention_bf16_d128_i64"):
         assert kernel in image, kernel
