@@ -28,6 +28,8 @@ if ROOT not in sys.path:
 # this script: FETCH_SIZE 145768 x 2 KiB (the counter's unit, calibrated on a copy of known size) +
 # WRITE_SIZE 4552 KiB.  Reported only for that kernel, workload and tuning.
 DECODE_TRAFFIC_BYTES = (145768 * 2 + 4552) * 1024
+# The same for the dense prefill kernel at batch 4 x seq 4096 x 32 heads: FETCH_SIZE 301283, WRITE_SIZE 131377.
+PREFILL_TRAFFIC_BYTES = (301283 * 2 + 131377) * 1024
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 POOLS = 3
@@ -132,7 +134,7 @@ def prefill_section(steps):
             "peak": MFMA_BF16_PEAK_TFLOPS,
             "unit": "TFLOP/s",
             "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
-            "traffic": None,
+            "traffic": PREFILL_TRAFFIC_BYTES,
             "kernel_avg_us": avg * 1e3,
             "kernel_median_us": ms[len(ms) // 2] * 1e3,
         },
