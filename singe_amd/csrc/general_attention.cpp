@@ -19,7 +19,7 @@ namespace {
 int32_t pick(KernelId base, int32_t data_type, uint64_t widest, const char* op, KernelId* kernel) {
     if (data_type != SINGE_HIP_F32 && data_type != SINGE_HIP_BF16 && data_type != SINGE_HIP_F16)
         return fail(SINGE_HIP_INVALID_ARGUMENT, "data type");
-    if (widest > 256) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, op, 0, widest);
+    if (widest > 256) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, op, widest, 0);
     const int width = widest <= 64 ? 0 : widest <= 128 ? 1 : 2;
     *kernel = static_cast<KernelId>(base + 3 * data_type + width);
     return 0;

@@ -120,7 +120,7 @@ def test_paged_attention_problem_validation():
     assert call(head_dim=300) == 5  # beyond the general kernel's 256
     detail = _native.ErrorDetail()
     lib.singe_hip_last_error(ctypes.byref(detail))
-    assert detail.actual == 300
+    assert detail.minimum == 300  # the refused width
     assert call(tokens=0) == 0  # nothing to attend, nothing launched
 
 
