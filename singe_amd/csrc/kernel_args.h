@@ -108,6 +108,7 @@ struct PagedAttentionArgs {
     uint32_t page_table;            // entries of `pages`; block-table form: entries per table row
     uint32_t row_tiles;             // ceil(groups * tokens / 128): row tiles per (sequence, kv head)
     uint32_t causal;
+    int32_t page_shift;             // log2(page_size) when it is a power of two, else -1
     float scale_log2e;              // scale * log2(e)
     float softcap_scale;            // scale / cap
     float softcap_log2e;            // cap * log2(e)

@@ -39,6 +39,8 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
     for (int64_t extent : extents)
         if (!fits_i32(static_cast<uint64_t>(extent))) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "problem");
     if (!fits_i32(static_cast<uint64_t>(p.head_dim))) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "problem");
+    if (static_cast<uint64_t>(p.page_size) * static_cast<uint64_t>(p.kv_heads) * static_cast<uint64_t>(p.head_dim) > 0xffffffffull)
+        return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "a cache page beyond 4 Gi elements");
     if (p.tokens == 0 || p.sequences == 0) return 0;  // nothing to attend
     const void* pointers[] = {query_rows_any, key_cache_any, value_cache_any, query_offsets, page_offsets, last_page_lengths, output_any};
     const char* names[] = {"query_rows", "key_cache", "value_cache", "query_offsets", "page_offsets", "last_page_lengths", "output"};
@@ -80,6 +82,9 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
     args.page_table = static_cast<uint32_t>(p.page_table);
     args.row_tiles = static_cast<uint32_t>((groups * static_cast<uint64_t>(p.tokens) + 127) / 128);
     args.causal = p.causal ? 1u : 0u;
+    args.page_shift = -1;
+    for (int shift = 0; shift < 31; ++shift)
+        if ((int64_t{1} << shift) == p.page_size) args.page_shift = shift;
     constexpr float kLog2e = 1.4426950408889634074f;
     args.scale_log2e = scale * kLog2e;
     args.softcap_scale = p.has_softcap ? scale / p.softcap : 0.0f;
@@ -159,6 +164,7 @@ extern "C" int32_t singe_hip_paged_kv_prefill_attention_bf16(
     if (int32_t s = ensure_len_at_least("actual_seq_offsets", actual_seq_offsets_len, c.batch)) return s;
     if (int32_t s = ensure_len_at_least("block_table", block_table_len, table_len)) return s;
     if (c.head_dim != 128) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, "paged_kv_prefill_attention_bf16", c.head_dim, 0);
+    if (block_len > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "a cache block beyond 4 Gi elements");
     const void* pointers[] = {out, lse, query, key_cache, value_cache, actual_seq_lens_q, actual_seq_lens_kv, actual_seq_offsets, block_table};
     const char* names[] = {"out", "lse", "query", "key_cache", "value_cache", "actual_seq_lens_q", "actual_seq_lens_kv",
                            "actual_seq_offsets", "block_table"};
@@ -188,6 +194,9 @@ extern "C" int32_t singe_hip_paged_kv_prefill_attention_bf16(
     args.page_table = static_cast<uint32_t>(c.block_table_batch_stride);
     args.row_tiles = static_cast<uint32_t>((groups * static_cast<uint64_t>(c.total_query_tokens) + 127) / 128);
     args.causal = c.causal ? 1u : 0u;
+    args.page_shift = -1;
+    for (int shift = 0; shift < 31; ++shift)
+        if ((size_t{1} << shift) == c.block_size) args.page_shift = shift;
     args.scale_log2e = c.scale * 1.4426950408889634074f;
     args.softcap_scale = 0.0f;
     args.softcap_log2e = 0.0f;

@@ -110,12 +110,31 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     // The page of each row is looked up one tile ahead of the row itself, so the gather never waits on
     // two dependent round trips.
     const unsigned int load_row = tid >> 4, load_col = tid & 15u;
+    const unsigned int page_elements = a.page_size * a.kv_heads * kHeadDim;  // fits 32 bits (checked by the host)
+    // When the page size divides the tile (1, 2, ..., 64 keys) a thread's rows sit at the same slots of
+    // their pages in every tile and a tile covers a whole number of pages, so only the page ids change from
+    // tile to tile; other page sizes divide per row.
+    const bool regular = a.page_shift >= 0 && a.page_size <= static_cast<unsigned int>(kKeyTile);
+    const unsigned int pages_per_tile = regular ? static_cast<unsigned int>(kKeyTile) >> a.page_shift : 0u;
+    auto slot_of = [&](unsigned int key) __attribute__((always_inline)) { return regular ? key & (a.page_size - 1u) : key % a.page_size; };
+    auto entry_of = [&](unsigned int key) __attribute__((always_inline)) { return regular ? key >> a.page_shift : key / a.page_size; };
+    unsigned int row_offset0 = 0, row_offset1 = 0, row_offset2 = 0, row_offset3 = 0;  // (slot * kv_heads + kv_head) * 128 + column
+    if (regular) {
+        row_offset0 = (slot_of(load_row) * a.kv_heads + kv_head) * kHeadDim + load_col * 8u;
+        row_offset1 = (slot_of(load_row + 16u) * a.kv_heads + kv_head) * kHeadDim + load_col * 8u;
+        row_offset2 = (slot_of(load_row + 32u) * a.kv_heads + kv_head) * kHeadDim + load_col * 8u;
+        row_offset3 = (slot_of(load_row + 48u) * a.kv_heads + kv_head) * kHeadDim + load_col * 8u;
+    }
     uint4 k0, k1, k2, k3, v0, v1, v2, v3;
     unsigned long long page0, page1, page2, page3;  // of the rows of the tile that is fetched next
     auto lookup_row = [&](unsigned int tile, unsigned int i, unsigned long long& page) __attribute__((always_inline)) {
         const unsigned int key = tile * kKeyTile + load_row + 16u * i;
         page = 0;
-        if (key < keys) page = read_page<FORM>(a.pages, static_cast<size_t>(page_start) + key / a.page_size);
+        if (key < keys) {
+            // The tile's first table entry is the same for every lane; the row adds a small offset.
+            const size_t tile_entry = static_cast<size_t>(page_start) + (regular ? tile * pages_per_tile : 0u);
+            page = read_page<FORM>(a.pages, tile_entry + (regular ? entry_of(load_row + 16u * i) : entry_of(key)));
+        }
     };
     auto lookup = [&](unsigned int tile) __attribute__((always_inline)) {
         lookup_row(tile, 0, page0);
@@ -123,7 +142,8 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         lookup_row(tile, 2, page2);
         lookup_row(tile, 3, page3);
     };
-    auto fetch_row = [&](unsigned int tile, unsigned int i, unsigned long long page, uint4& key_bits, uint4& value_bits) __attribute__((always_inline)) {
+    auto fetch_row = [&](unsigned int tile, unsigned int i, unsigned long long page, unsigned int row_offset, uint4& key_bits,
+                         uint4& value_bits) __attribute__((always_inline)) {
         const unsigned int key = tile * kKeyTile + load_row + 16u * i;
         const bool wanted = key < keys;
         const bool valid = wanted && page < static_cast<unsigned long long>(a.cache_pages);  // negative pages wrap above it
@@ -131,16 +151,18 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         key_bits = make_uint4(0, 0, 0, 0);
         value_bits = make_uint4(0, 0, 0, 0);
         if (valid) {
-            const size_t offset = ((page * a.page_size + key % a.page_size) * a.kv_heads + kv_head) * kHeadDim + load_col * 8u;
+            if (!regular) row_offset = (slot_of(key) * a.kv_heads + kv_head) * kHeadDim + load_col * 8u;
+            // One 32 x 32 -> 64-bit multiply-add places the page; everything else is 32-bit.
+            const size_t offset = static_cast<size_t>(static_cast<unsigned int>(page)) * page_elements + row_offset;
             key_bits = *reinterpret_cast<const uint4*>(a.key_cache + offset);
             value_bits = *reinterpret_cast<const uint4*>(a.value_cache + offset);
         }
     };
     auto fetch = [&](unsigned int tile) __attribute__((always_inline)) {
-        fetch_row(tile, 0, page0, k0, v0);
-        fetch_row(tile, 1, page1, k1, v1);
-        fetch_row(tile, 2, page2, k2, v2);
-        fetch_row(tile, 3, page3, k3, v3);
+        fetch_row(tile, 0, page0, row_offset0, k0, v0);
+        fetch_row(tile, 1, page1, row_offset1, k1, v1);
+        fetch_row(tile, 2, page2, row_offset2, k2, v2);
+        fetch_row(tile, 3, page3, row_offset3, k3, v3);
     };
     auto stash_row = [&](unsigned char* keys_at, unsigned char* values_at, unsigned int i, const uint4& key_bits, const uint4& value_bits) __attribute__((always_inline)) {
         const unsigned int row = load_row + 16u * i;
