@@ -22,10 +22,6 @@ namespace {
 
 using namespace prefill;
 
-constexpr int kKeyStages = 3, kValueStages = 2;
-constexpr int kValueBase = kKeyStages * kTileBytes;
-constexpr int kDenseLdsBytes = (kKeyStages + kValueStages) * kTileBytes;
-
 // One 128-row query tile of (batch, head) pair `bh`.
 template <bool CAUSAL>
 SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, unsigned int bh, unsigned int query_tile) {
@@ -217,11 +213,11 @@ SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
 }  // namespace
 
 extern "C" __global__ __launch_bounds__(256, 2) void singe_fmha_prefill_bf16_d128_causal(PrefillArgs args) {
-    __shared__ __attribute__((aligned(1024))) unsigned char prefill_lds[kDenseLdsBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char prefill_lds[kStagedLdsBytes];
     fmha_prefill_body<true>(args, prefill_lds);
 }
 
 extern "C" __global__ __launch_bounds__(256, 2) void singe_fmha_prefill_bf16_d128_full(PrefillArgs args) {
-    __shared__ __attribute__((aligned(1024))) unsigned char prefill_lds[kDenseLdsBytes];
+    __shared__ __attribute__((aligned(1024))) unsigned char prefill_lds[kStagedLdsBytes];
     fmha_prefill_body<false>(args, prefill_lds);
 }

@@ -13,8 +13,10 @@
 // A workgroup owns 128 packed rows of one (sequence, kv head): the query heads that share the kv head,
 // a token's heads consecutive (row r = token r / groups, head r % groups), so a key tile is staged once
 // for the whole group.  The grid covers every sequence's longest possible run of rows; workgroups past
-// their sequence's rows return at once.  Keys are gathered page by page into the same padded LDS tiles
-// as the dense kernel and folded by the shared core (prefill_core.hip.h).
+// their sequence's rows return at once.  Keys are gathered row by row, each lane placing its own row in its
+// page, straight from the cache into the same permuted LDS tiles as the dense kernel (three K stages, two V
+// stages, page ids looked up three tiles ahead) and folded by the same block-pipelined core
+// (prefill_blocks.hip.h).
 //
 // The same body also serves paged_kv_prefill_attention of the singe-kernel surface
 // (singe-kernel/src/cpu/attention.rs:1248-1341): paging as a [batch, stride] block table with per-sequence
@@ -26,15 +28,18 @@
 // be null) and nothing is read through it (paged_attention.rs:41-54, 210-262, 739-755).
 #include "kernel_args.h"
 #include "paging.hip.h"
-#include "prefill_core.hip.h"
+#include "prefill_blocks.hip.h"
 
 namespace {
 
 using namespace prefill;
 
+constexpr unsigned int kNoPage = 0xFFFFFFFFu;  // a table entry outside the cache: reported, never read through
+
 template <bool SOFTCAP, int FORM>
 SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned char* lds) {
-    const unsigned int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const unsigned int tid = threadIdx.x, lane = tid & 63;
+    const unsigned int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and known to be
     const unsigned int column = lane & 31, hi = lane >> 5;
     const unsigned int groups = a.heads / a.kv_heads;
 
@@ -75,9 +80,11 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     const unsigned int wave_first_row = first_row + wave * 32u;
     const bool wave_live = wave_first_row < packed;
     const unsigned int wave_last_row = wave_live ? (wave_first_row + 31u < packed ? wave_first_row + 31u : packed - 1u) : first_row;
-    const unsigned int wave_low = position_of(wave_live ? wave_first_row : first_row), wave_high = position_of(wave_last_row);
+    const unsigned int wave_low = __builtin_amdgcn_readfirstlane(position_of(wave_live ? wave_first_row : first_row));
+    const unsigned int wave_high = __builtin_amdgcn_readfirstlane(position_of(wave_last_row));
 
-    // Keys this workgroup must visit.
+    // Keys this workgroup must visit, in tiles; and the blocks of them this wave folds: under the causal
+    // mask a block wholly after the wave's last position contributes nothing.
     const unsigned int group_last_row = first_row + kQueryTile - 1 < packed ? first_row + kQueryTile - 1 : packed - 1u;
     unsigned int key_end = keys;
     if (causal) {
@@ -89,7 +96,17 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         const unsigned int low = position_of(first_row) + 1u;  // keys below low - window are hidden from every row
         first_tile = low > window ? (low - window) / kKeyTile : 0u;
     }
-    const unsigned int end_tile = (key_end + kKeyTile - 1) / kKeyTile;
+    first_tile = __builtin_amdgcn_readfirstlane(first_tile);
+    const unsigned int tiles = __builtin_amdgcn_readfirstlane((key_end + kKeyTile - 1) / kKeyTile);
+    unsigned int wave_blocks = 0;
+    if (wave_live) {
+        wave_blocks = (key_end + 31u) / 32u;
+        if (causal) {
+            const unsigned int seen = wave_high / 32u + 1u;
+            wave_blocks = wave_blocks < seen ? wave_blocks : seen;
+        }
+    }
+    wave_blocks = __builtin_amdgcn_readfirstlane(wave_blocks);
 
     // Q^T as the MFMA B operand; a negative scale moves into Q (see fmha_prefill.hip).
     const float factor = SOFTCAP ? 1.0f : fabsf(a.scale_log2e);
@@ -106,128 +123,161 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         }
     }
 
-    // Tile loads: 1024 16-byte chunks per operand per tile, four per thread (rows load_row + 16 i).
-    // The page of each row is looked up one tile ahead of the row itself, so the gather never waits on
-    // two dependent round trips.
-    const unsigned int load_row = tid >> 4, load_col = tid & 15u;
-    const unsigned int page_elements = a.page_size * a.kv_heads * kHeadDim;  // fits 32 bits (checked by the host)
-    // When the page size divides the tile (1, 2, ..., 64 keys) a thread's rows sit at the same slots of
-    // their pages in every tile and a tile covers a whole number of pages, so only the page ids change from
-    // tile to tile; other page sizes divide per row.
-    const bool regular = a.page_shift >= 0 && a.page_size <= static_cast<unsigned int>(kKeyTile);
-    const unsigned int pages_per_tile = regular ? static_cast<unsigned int>(kKeyTile) >> a.page_shift : 0u;
-    auto slot_of = [&](unsigned int key) __attribute__((always_inline)) { return regular ? key & (a.page_size - 1u) : key % a.page_size; };
-    auto entry_of = [&](unsigned int key) __attribute__((always_inline)) { return regular ? key >> a.page_shift : key / a.page_size; };
-    unsigned int row_offset0 = 0, row_offset1 = 0, row_offset2 = 0, row_offset3 = 0;  // (slot * kv_heads + kv_head) * 128 + column
-    if (regular) {
-        row_offset0 = (slot_of(load_row) * a.kv_heads + kv_head) * kHeadDim + load_col * 8u;
-        row_offset1 = (slot_of(load_row + 16u) * a.kv_heads + kv_head) * kHeadDim + load_col * 8u;
-        row_offset2 = (slot_of(load_row + 32u) * a.kv_heads + kv_head) * kHeadDim + load_col * 8u;
-        row_offset3 = (slot_of(load_row + 48u) * a.kv_heads + kv_head) * kHeadDim + load_col * 8u;
-    }
-    uint4 k0, k1, k2, k3, v0, v1, v2, v3;
-    unsigned long long page0, page1, page2, page3;  // of the rows of the tile that is fetched next
-    auto lookup_row = [&](unsigned int tile, unsigned int i, unsigned long long& page) __attribute__((always_inline)) {
-        const unsigned int key = tile * kKeyTile + load_row + 16u * i;
-        page = 0;
-        if (key < keys) {
-            // The tile's first table entry is the same for every lane; the row adds a small offset.
-            const size_t tile_entry = static_cast<size_t>(page_start) + (regular ? tile * pages_per_tile : 0u);
-            page = read_page<FORM>(a.pages, tile_entry + (regular ? entry_of(load_row + 16u * i) : entry_of(key)));
+    // A tile load is 1024 16-byte chunks per operand: instruction i of wave w fills rows 16 i + 4 w .. + 3,
+    // lane l the chunk position l % 16 of row 16 i + 4 w + l / 16, fetched from the chunk the row's
+    // permutation puts there (prefill_blocks.hip.h).  A row is key (tile, row) of the sequence, found in page
+    // pages[page_start + key / page_size] at slot key % page_size; rows past the sequence's last key re-read
+    // that key and are masked, so nothing the sequence does not own reaches LDS.  Page ids are looked up
+    // three tiles ahead and checked then; K is loaded two tiles ahead and V one, from the same ids.
+    const unsigned int load_row = 4u * wave + (lane >> 4), chunk_position = lane & 15u;
+    const unsigned int key_chunk = (chunk_position ^ (load_row & 15u)) * 16u, value_chunk = (chunk_position ^ (4u * (load_row & 3u))) * 16u;
+    const size_t page_bytes = static_cast<size_t>(a.page_size) * a.kv_heads * kRowBytes;
+    const unsigned int head_bytes = kv_head * kRowBytes, slot_bytes = a.kv_heads * kRowBytes;
+    const unsigned char* const key_bytes = reinterpret_cast<const unsigned char*>(a.key_cache);
+    const unsigned char* const value_bytes = reinterpret_cast<const unsigned char*>(a.value_cache);
+    const bool shifted = a.page_shift >= 0;
+    struct Pages {
+        unsigned int id[4];
+    };
+    struct RawPages {
+        RawPage<FORM> value[4];  // as loaded: nothing computes on them until they are checked, a tile later
+    };
+    auto key_of = [&](unsigned int tile, unsigned int i) __attribute__((always_inline)) {
+        const unsigned int key = tile * kKeyTile + 16u * i + load_row;
+        return key < keys ? key : keys - 1u;
+    };
+    auto lookup = [&](unsigned int tile, RawPages& raw) __attribute__((always_inline)) {
+#pragma unroll
+        for (unsigned int i = 0; i < 4; ++i) {
+            const unsigned int key = key_of(tile, i);
+            const unsigned int entry = shifted ? key >> a.page_shift : key / a.page_size;
+            raw.value[i] = read_raw_page<FORM>(a.pages, static_cast<size_t>(page_start) + entry);
         }
     };
-    auto lookup = [&](unsigned int tile) __attribute__((always_inline)) {
-        lookup_row(tile, 0, page0);
-        lookup_row(tile, 1, page1);
-        lookup_row(tile, 2, page2);
-        lookup_row(tile, 3, page3);
-    };
-    auto fetch_row = [&](unsigned int tile, unsigned int i, unsigned long long page, unsigned int row_offset, uint4& key_bits,
-                         uint4& value_bits) __attribute__((always_inline)) {
-        const unsigned int key = tile * kKeyTile + load_row + 16u * i;
-        const bool wanted = key < keys;
-        const bool valid = wanted && page < static_cast<unsigned long long>(a.cache_pages);  // negative pages wrap above it
-        if (wanted && !valid) report_index_error(a.status);
-        key_bits = make_uint4(0, 0, 0, 0);
-        value_bits = make_uint4(0, 0, 0, 0);
-        if (valid) {
-            if (!regular) row_offset = (slot_of(key) * a.kv_heads + kv_head) * kHeadDim + load_col * 8u;
-            // One 32 x 32 -> 64-bit multiply-add places the page; everything else is 32-bit.
-            const size_t offset = static_cast<size_t>(static_cast<unsigned int>(page)) * page_elements + row_offset;
-            key_bits = *reinterpret_cast<const uint4*>(a.key_cache + offset);
-            value_bits = *reinterpret_cast<const uint4*>(a.value_cache + offset);
+    auto check = [&](const RawPages& raw, Pages& pages) __attribute__((always_inline)) {
+#pragma unroll
+        for (unsigned int i = 0; i < 4; ++i) {
+            const unsigned long long page = static_cast<unsigned long long>(raw.value[i]);  // negative ids wrap above any cache
+            const bool valid = page < static_cast<unsigned long long>(a.cache_pages);
+            if (!valid) report_index_error(a.status);
+            pages.id[i] = valid ? static_cast<unsigned int>(page) : kNoPage;
         }
     };
-    auto fetch = [&](unsigned int tile) __attribute__((always_inline)) {
-        fetch_row(tile, 0, page0, row_offset0, k0, v0);
-        fetch_row(tile, 1, page1, row_offset1, k1, v1);
-        fetch_row(tile, 2, page2, row_offset2, k2, v2);
-        fetch_row(tile, 3, page3, row_offset3, k3, v3);
+    auto load = [&](const unsigned char* cache, unsigned int chunk, unsigned int tile, const Pages& pages, unsigned char* stage) __attribute__((always_inline)) {
+#pragma unroll
+        for (unsigned int i = 0; i < 4; ++i) {
+            const unsigned int key = key_of(tile, i);
+            const unsigned int slot = shifted ? key & (a.page_size - 1u) : key % a.page_size;
+            const size_t offset = pages.id[i] * page_bytes + (slot * slot_bytes + head_bytes + chunk);
+            if (pages.id[i] != kNoPage)
+                __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(cache + offset),
+                                                 (lds_words_t)(stage + (16u * i + 4u * wave) * kRowBytes), 16, 0, 0);
+        }
     };
-    auto stash_row = [&](unsigned char* keys_at, unsigned char* values_at, unsigned int i, const uint4& key_bits, const uint4& value_bits) __attribute__((always_inline)) {
-        const unsigned int row = load_row + 16u * i;
-        *reinterpret_cast<uint4*>(keys_at + row * kKeyRowBytes + load_col * 16) = key_bits;
-        *reinterpret_cast<uint4*>(values_at + row * kValueRowBytes + load_col * 16) = value_bits;
+    auto load_keys = [&](unsigned int tile, const Pages& pages, unsigned int stage) __attribute__((always_inline)) {
+        load(key_bytes, key_chunk, tile, pages, lds + stage * kTileBytes);
     };
-    auto stash = [&](unsigned char* keys_at, unsigned char* values_at) __attribute__((always_inline)) {
-        stash_row(keys_at, values_at, 0, k0, v0);
-        stash_row(keys_at, values_at, 1, k1, v1);
-        stash_row(keys_at, values_at, 2, k2, v2);
-        stash_row(keys_at, values_at, 3, k3, v3);
+    auto load_values = [&](unsigned int tile, const Pages& pages, unsigned int stage) __attribute__((always_inline)) {
+        load(value_bytes, value_chunk, tile, pages, lds + kValueBase + stage * kTileBytes);
     };
 
     RowState state;
     reset(state);
-    const unsigned int key_read = key_read_offset(lane), value_read = value_read_offset(lane);
+    const ReadOffsets offsets = read_offsets(lane);
 
-    auto fold = [&](unsigned int tile, const unsigned char* keys_at, const unsigned char* values_at) __attribute__((always_inline)) {
-        const unsigned int key0 = tile * kKeyTile;
-        // A 32-key block is dead for the wave when every row's mask hides all of it.
-        auto block_live = [&](unsigned int base) __attribute__((always_inline)) {
-            if (!wave_live || base >= keys) return false;
-            if (causal && base > wave_high) return false;
-            if (windowed && base + 31u + window <= wave_low) return false;
-            return true;
-        };
-        const bool live0 = block_live(key0), live1 = block_live(key0 + 32u);
-        if (!live0 && !live1) return;
-        const bool edge = !live0 || (causal && key0 + kKeyTile - 1 > wave_low) || key0 + kKeyTile > keys || windowed;
-        fold_staged_keys<SOFTCAP>(state, q, keys_at, values_at, key_read, value_read, hi, factor, live1, edge,
-                                  [&](unsigned int block, unsigned int key_in_block) {
-                                      const unsigned int key = key0 + 32 * block + key_in_block;
-                                      return (block == 0 && !live0) || key >= keys || (causal && key > my_position) ||
-                                             (windowed && key + window <= my_position);
-                                  },
-                                  fabsf(a.softcap_scale), a.softcap_log2e);
-    };
-
-    unsigned char* const keys0 = lds;
-    unsigned char* const values0 = lds + kKeyStageBytes;
-    unsigned char* const keys1 = lds + kStageBytes;
-    unsigned char* const values1 = lds + kStageBytes + kKeyStageBytes;
-    if (first_tile < end_tile) {
-        lookup(first_tile);
-        fetch(first_tile);
-        if (first_tile + 1 < end_tile) lookup(first_tile + 1);
-        stash(keys0, values0);
+    Pages behind = {}, ahead = {};  // of tile + 1 and tile + 2 at the top of tile's iteration
+    RawPages fresh = {};            // of tile + 3, on their way during it
+    if (first_tile < tiles) {
+        RawPages raw_first = {}, raw_behind = {}, raw_ahead = {};
+        lookup(first_tile, raw_first);
+        if (first_tile + 1 < tiles) lookup(first_tile + 1, raw_behind);
+        if (first_tile + 2 < tiles) lookup(first_tile + 2, raw_ahead);
+        Pages first;
+        check(raw_first, first);
+        if (first_tile + 1 < tiles) check(raw_behind, behind);
+        if (first_tile + 2 < tiles) check(raw_ahead, ahead);
+        load_keys(first_tile, first, 0);
+        load_values(first_tile, first, 0);
+        if (first_tile + 1 < tiles) load_keys(first_tile + 1, behind, 1);
     }
     __syncthreads();
-    for (unsigned int tile = first_tile; tile < end_tile; tile += 2) {
-        if (tile + 1 < end_tile) {
-            fetch(tile + 1);
-            if (tile + 2 < end_tile) lookup(tile + 2);
+
+    // Folds block `block` (scores in `s`, values at `values`) with the masks' edges applied.
+    auto fold = [&](unsigned int block, f32x16_t& s, const unsigned char* values) __attribute__((always_inline)) {
+        const unsigned int key0 = block * 32u;
+        if constexpr (SOFTCAP) {
+            // Scores become cap * tanh(score * scale / cap) before the softmax
+            // (singe/src/backend/cuda/kernel_plan/source/tensor_core.rs:49-54).
+            const float cap_scale = fabsf(a.softcap_scale);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[r] = tanhf(s[r] * cap_scale) * a.softcap_log2e;
         }
-        fold(tile, keys0, values0);
-        if (tile + 1 < end_tile) stash(keys1, values1);
+        const bool edge = (causal && key0 + 31u > wave_low) || key0 + 32u > keys || windowed;
+        const float shift = begin_block(state, s, hi, factor, edge, [&](unsigned int key_in_block) {
+            const unsigned int key = key0 + key_in_block;
+            return key >= keys || (causal && key > my_position) || (windowed && key + window <= my_position);
+        });
+        finish_block<false>(state, s, factor, shift, values, offsets, s, q, values);
+    };
+
+    // One block ahead, as in the dense kernel: `scores` holds those of the block that is folded next.
+    f32x16_t scores;
+    if (2u * first_tile < wave_blocks) score_block(scores, q, lds, offsets);
+    unsigned int key_stage = 0, value_stage = 0;
+    const unsigned char *keys_at, *next_keys, *values_at;
+    auto enter = [&](unsigned int tile) __attribute__((always_inline)) {
+        const unsigned int next_key_stage = key_stage + 1 == kKeyStages ? 0 : key_stage + 1;
+        const unsigned int spare_key_stage = next_key_stage + 1 == kKeyStages ? 0 : next_key_stage + 1;
+        if (tile + 3 < tiles) lookup(tile + 3, fresh);
+        if (tile + 2 < tiles) load_keys(tile + 2, ahead, spare_key_stage);
+        if (tile + 1 < tiles) load_values(tile + 1, behind, value_stage ^ 1u);
+        keys_at = lds + key_stage * kTileBytes;
+        next_keys = lds + next_key_stage * kTileBytes;
+        values_at = lds + kValueBase + value_stage * kTileBytes;
+        key_stage = next_key_stage;
+        value_stage ^= 1u;
+    };
+    // Ends a tile's iteration: the ids looked up at its start have had the whole tile to arrive.
+    auto leave = [&](unsigned int tile) __attribute__((always_inline)) {
+        __builtin_amdgcn_sched_barrier(0);
+        behind = ahead;
+        if (tile + 3 < tiles) check(fresh, ahead);
         __syncthreads();
-        if (tile + 1 >= end_tile) break;
-        if (tile + 2 < end_tile) {
-            fetch(tile + 2);
-            if (tile + 3 < end_tile) lookup(tile + 3);
+    };
+
+    // Tiles no mask touches for this wave, with another block to come after them: straight-line code.
+    unsigned int interior_end = first_tile;
+    if (!SOFTCAP && !windowed) {
+        interior_end = wave_blocks > 2 ? (wave_blocks - 1) / 2 : 0;  // tiles t with 2 t + 2 < wave_blocks
+        if (causal) {
+            const unsigned int unmasked = (wave_low + 1) / kKeyTile;  // tiles t with 64 t + 63 <= wave_low
+            interior_end = interior_end < unmasked ? interior_end : unmasked;
         }
-        fold(tile + 1, keys1, values1);
-        if (tile + 2 < end_tile) stash(keys0, values0);
-        __syncthreads();
+        const unsigned int whole = keys / kKeyTile;  // tiles t with 64 t + 64 <= keys
+        interior_end = interior_end < whole ? interior_end : whole;
+    }
+    unsigned int tile = first_tile;
+    for (; tile < interior_end; ++tile) {
+        enter(tile);
+        const float shift_even = begin_block(state, scores, hi, factor, false, [](unsigned int) { return false; });
+        finish_block<true>(state, scores, factor, shift_even, values_at, offsets, scores, q, keys_at + kBlockBytes);
+        __builtin_amdgcn_sched_barrier(0);
+        const float shift_odd = begin_block(state, scores, hi, factor, false, [](unsigned int) { return false; });
+        finish_block<true>(state, scores, factor, shift_odd, values_at + kBlockBytes, offsets, scores, q, next_keys);
+        leave(tile);
+    }
+    // Tiles on a mask's edge and the last ones (and, for waves that have run out of blocks, the workgroup's
+    // remaining loads and barriers): the same steps one after the other.
+    for (; tile < tiles; ++tile) {
+        enter(tile);
+        const unsigned int block = 2u * tile;
+        if (block < wave_blocks) fold(block, scores, values_at);
+        if (block + 1 < wave_blocks) {
+            score_block(scores, q, keys_at + kBlockBytes, offsets);
+            fold(block + 1, scores, values_at + kBlockBytes);
+        }
+        if (block + 2 < wave_blocks) score_block(scores, q, next_keys, offsets);
+        leave(tile);
     }
 
     // Normalise and store; a row that sees no key stays zero and has a log-sum-exp of -inf
@@ -258,10 +308,10 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
 
 }  // namespace
 
-#define SINGE_PAGED_ATTENTION_KERNEL(NAME, SOFTCAP, FORM)                                              \
-    extern "C" __global__ __launch_bounds__(256, 2) void NAME(PagedAttentionArgs args) {                \
-        __shared__ __attribute__((aligned(16))) unsigned char paged_lds[2 * prefill::kStageBytes];     \
-        paged_attention_body<SOFTCAP, FORM>(args, paged_lds);                                          \
+#define SINGE_PAGED_ATTENTION_KERNEL(NAME, SOFTCAP, FORM)                                                  \
+    extern "C" __global__ __launch_bounds__(256, 2) void NAME(PagedAttentionArgs args) {                    \
+        __shared__ __attribute__((aligned(1024))) unsigned char paged_lds[prefill::kStagedLdsBytes];        \
+        paged_attention_body<SOFTCAP, FORM>(args, paged_lds);                                              \
     }
 
 SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i32, false, kCsrI32)

@@ -24,6 +24,19 @@ SINGE_DEVICE unsigned long long read_page(const void* pages, size_t at) {
         return static_cast<unsigned long long>(read_index<FORM>(pages, at));  // negative ids wrap above any cache
 }
 
+// A page id as it sits in memory, and the load of one with no arithmetic on the result (a consumer that
+// wants to keep the load in flight widens it later: static_cast<unsigned long long> sign-extends the CSR
+// forms, so negative ids wrap above any cache, and zero-extends a block table's u32).
+template <int FORM> struct RawPageType { typedef int type; };
+template <> struct RawPageType<kCsrI64> { typedef long long type; };
+template <> struct RawPageType<kTable> { typedef unsigned int type; };
+template <int FORM> using RawPage = typename RawPageType<FORM>::type;
+
+template <int FORM>
+SINGE_DEVICE RawPage<FORM> read_raw_page(const void* pages, size_t at) {
+    return static_cast<const RawPage<FORM>*>(pages)[at];
+}
+
 struct SequenceSpan {
     long long query_start;  // first token of the sequence in the packed queries
     long long page_start;   // first entry of the sequence in `pages`

@@ -21,6 +21,10 @@ namespace prefill {
 constexpr int kRowBytes = 256;                       // one key's 128 bf16
 constexpr int kTileBytes = kKeyTile * kRowBytes;     // 64 keys of K or of V
 constexpr int kBlockBytes = 32 * kRowBytes;
+// LDS of a workgroup: three stages of K and two of V, so K can be loaded two tiles ahead and V one.
+constexpr int kKeyStages = 3, kValueStages = 2;
+constexpr int kValueBase = kKeyStages * kTileBytes;
+constexpr int kStagedLdsBytes = (kKeyStages + kValueStages) * kTileBytes;
 
 typedef unsigned int __attribute__((address_space(3))) * lds_words_t;
 
