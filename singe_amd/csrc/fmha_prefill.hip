@@ -81,23 +81,39 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     const unsigned int value_stride_bytes = static_cast<unsigned int>(a.value_sequence_stride) * 2u;
     const unsigned int load_row = 4u * wave + (lane >> 4), position = lane & 15u;
     const unsigned int key_chunk = (position ^ (load_row & 15u)) * 16u, value_chunk = (position ^ (4u * (load_row & 3u))) * 16u;
-    auto load_keys = [&](unsigned int tile, unsigned int stage) __attribute__((always_inline)) {
+    // A tile that lies wholly inside the keys is addressed as a scalar base (tile and instruction) plus a
+    // per-lane offset that never changes, so its loads cost no vector arithmetic; the last, partial tile
+    // clamps each row (rows past the end re-read the last key and are masked).
+    const unsigned int key_lane = load_row * key_stride_bytes + key_chunk, value_lane = load_row * value_stride_bytes + value_chunk;
+    auto load_tile = [&](const unsigned char* rows, unsigned int stride_bytes, unsigned int lane_offset, unsigned int chunk,
+                         unsigned int tile, unsigned char* stage) __attribute__((always_inline)) {
+        if (tile * kKeyTile + kKeyTile <= a.key_len) {
+            const unsigned char* base = rows + static_cast<size_t>(tile * kKeyTile) * stride_bytes;
+            asm("" : "+s"(base));  // a scalar the compiler cannot fold the lane's part into
 #pragma unroll
-        for (unsigned int i = 0; i < 4; ++i) {
-            unsigned int key = tile * kKeyTile + 16u * i + load_row;
-            key = key < a.key_len ? key : a.key_len - 1;  // rows past the end re-read the last key and are masked
-            __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(k_bytes + (key * key_stride_bytes + key_chunk)),
-                                             (lds_words_t)(lds + stage * kTileBytes + (16u * i + 4u * wave) * kRowBytes), 16, 0, 0);
+            for (unsigned int i = 0; i < 4; ++i) {
+                // The offset is pinned to this spot as a 32-bit value: hoisted and widened, it would take the
+                // load out of its scalar-base form and cost a 64-bit add per lane.
+                unsigned int offset = lane_offset + 16u * i * stride_bytes;
+                asm volatile("" : "+v"(offset));
+                __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(base + offset),
+                                                 (lds_words_t)(stage + (16u * i + 4u * wave) * kRowBytes), 16, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (unsigned int i = 0; i < 4; ++i) {
+                unsigned int key = tile * kKeyTile + 16u * i + load_row;
+                key = key < a.key_len ? key : a.key_len - 1;
+                __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(rows + (key * stride_bytes + chunk)),
+                                                 (lds_words_t)(stage + (16u * i + 4u * wave) * kRowBytes), 16, 0, 0);
+            }
         }
     };
-    auto load_values = [&](unsigned int tile, unsigned int stage) __attribute__((always_inline)) {
-#pragma unroll
-        for (unsigned int i = 0; i < 4; ++i) {
-            unsigned int key = tile * kKeyTile + 16u * i + load_row;
-            key = key < a.key_len ? key : a.key_len - 1;
-            __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(v_bytes + (key * value_stride_bytes + value_chunk)),
-                                             (lds_words_t)(lds + kValueBase + stage * kTileBytes + (16u * i + 4u * wave) * kRowBytes), 16, 0, 0);
-        }
+    auto load_keys = [&](unsigned int tile, unsigned char* stage) __attribute__((always_inline)) {
+        load_tile(k_bytes, key_stride_bytes, key_lane, key_chunk, tile, stage);
+    };
+    auto load_values = [&](unsigned int tile, unsigned char* stage) __attribute__((always_inline)) {
+        load_tile(v_bytes, value_stride_bytes, value_lane, value_chunk, tile, stage);
     };
 
     RowState state;
@@ -105,10 +121,11 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     const ReadOffsets offsets = read_offsets(lane);
 
     if (tiles > 0) {
-        load_keys(0, 0);
-        load_values(0, 0);
+        load_keys(0, lds);
+        load_values(0, lds + kValueBase);
     }
-    if (tiles > 1) load_keys(1, 1);
+    if (tiles > 1) load_keys(1, lds + kTileBytes);
+    loads_landed();
     __syncthreads();
 
     // Folds block `block` (scores in `s`, values at `values`) with the mask's edges applied.
@@ -127,19 +144,25 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     f32x16_t scores;
     if (wave_blocks > 0) score_block(scores, q, lds, offsets);
     unsigned int key_stage = 0, value_stage = 0;  // tile % 3, tile % 2
-    // Starts the loads of a tile's iteration and names the stages it works on.  Everyone left the stages
-    // that held K of tile - 1 and V of tile - 1 at the last barrier.
-    const unsigned char *keys, *next_keys, *values;
-    auto enter = [&](unsigned int tile) __attribute__((always_inline)) {
+    // Names the stages a tile's iteration works on and loads into.  Everyone left the stages that held K of
+    // tile - 1 and V of tile - 1 at the last barrier.
+    auto enter = [&]() __attribute__((always_inline)) {
         const unsigned int next_key_stage = key_stage + 1 == kKeyStages ? 0 : key_stage + 1;
         const unsigned int spare_key_stage = next_key_stage + 1 == kKeyStages ? 0 : next_key_stage + 1;
-        if (tile + 2 < tiles) load_keys(tile + 2, spare_key_stage);
-        if (tile + 1 < tiles) load_values(tile + 1, value_stage ^ 1u);
-        keys = lds + key_stage * kTileBytes;
-        next_keys = lds + next_key_stage * kTileBytes;
-        values = lds + kValueBase + value_stage * kTileBytes;
+        TileStages stages;
+        stages.keys = lds + key_stage * kTileBytes;
+        stages.next_keys = lds + next_key_stage * kTileBytes;
+        stages.values = lds + kValueBase + value_stage * kTileBytes;
+        stages.key_dest = lds + spare_key_stage * kTileBytes;
+        stages.value_dest = lds + kValueBase + (value_stage ^ 1u) * kTileBytes;
         key_stage = next_key_stage;
         value_stage ^= 1u;
+        return stages;
+    };
+    // Hands the stages on: this wave's loads have landed, and everyone has finished reading.
+    auto leave = [&]() __attribute__((always_inline)) {
+        loads_landed();
+        __syncthreads();
     };
 
     // Tiles with no mask to apply and another block to come after them: straight-line code.  They come
@@ -154,27 +177,23 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
         interior_tiles = interior_tiles < whole ? interior_tiles : whole;
     }
     unsigned int tile = 0;
+    auto issue = [&](unsigned char* key_dest, unsigned char* value_dest) __attribute__((always_inline)) {
+        if (tile + 2 < tiles) load_keys(tile + 2, key_dest);
+        if (tile + 1 < tiles) load_values(tile + 1, value_dest);
+    };
     for (; tile < interior_tiles; ++tile) {
-        enter(tile);
-        const float shift_even = begin_block(state, scores, hi, factor, false, [](unsigned int) { return false; });
-        finish_block<true>(state, scores, factor, shift_even, values, offsets, scores, q, keys + kBlockBytes);
-        __builtin_amdgcn_sched_barrier(0);  // keeps the second block's operand reads out of the first block's registers
-        const float shift_odd = begin_block(state, scores, hi, factor, false, [](unsigned int) { return false; });
-        finish_block<true>(state, scores, factor, shift_odd, values + kBlockBytes, offsets, scores, q, next_keys);
-        __syncthreads();
+        const TileStages stages = enter();
+        fold_interior_tile(state, scores, q, offsets, hi, factor, stages.keys, stages.next_keys, stages.values, stages.key_dest,
+                           stages.value_dest, issue);
+        leave();
     }
     // Tiles on the mask's edge and the last ones (and, for waves that have run out of blocks, the
-    // workgroup's remaining loads and barriers): the same steps one after the other.
+    // workgroup's remaining loads and barriers).
     for (; tile < tiles; ++tile) {
-        enter(tile);
-        const unsigned int block = 2u * tile;
-        if (block < wave_blocks) fold(block, scores, values);
-        if (block + 1 < wave_blocks) {
-            score_block(scores, q, keys + kBlockBytes, offsets);
-            fold(block + 1, scores, values + kBlockBytes);
-        }
-        if (block + 2 < wave_blocks) score_block(scores, q, next_keys, offsets);
-        __syncthreads();
+        const TileStages stages = enter();
+        fold_edge_tile(scores, q, offsets, 2u * tile, wave_blocks, stages.keys, stages.next_keys, stages.values, stages.key_dest,
+                       stages.value_dest, issue, fold);
+        leave();
     }
 
     // Normalise and store.  Lane (query, hi) holds dims 32db + 8(r / 4) + 4hi + (r % 4).

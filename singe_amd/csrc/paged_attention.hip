@@ -44,11 +44,27 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     const unsigned int groups = a.heads / a.kv_heads;
 
     // Workgroup i runs on XCD i % 8: the row tiles of one (sequence, kv head) share an XCD and its L2.
+    // Within an XCD the order is band by band of 32 row tiles: every unit's tiles 0 .. 31 (a unit's side by
+    // side, walking its keys together), then every unit's tiles 32 .. 63, and so on, so the workgroups past
+    // a sequence's rows, which return at once, mostly come after those with work instead of between them.
+    constexpr unsigned int kBand = 32;
     const unsigned int xcd = blockIdx.x & 7u, within = blockIdx.x >> 3;
-    const unsigned int unit = (within / a.row_tiles) * 8u + xcd;
+    const unsigned int units_per_xcd = (a.sequences * a.kv_heads + 7u) / 8u;
+    const unsigned int full_bands = a.row_tiles / kBand, band = within / (units_per_xcd * kBand);
+    unsigned int local_unit, row_tile;
+    if (band < full_bands) {
+        const unsigned int rest = within % (units_per_xcd * kBand);
+        local_unit = rest / kBand;
+        row_tile = band * kBand + rest % kBand;
+    } else {
+        const unsigned int rest = within - full_bands * units_per_xcd * kBand, tail = a.row_tiles - full_bands * kBand;
+        local_unit = rest / tail;
+        row_tile = full_bands * kBand + rest % tail;
+    }
+    const unsigned int unit = local_unit * 8u + xcd;
     if (unit >= a.sequences * a.kv_heads) return;
     const unsigned int sequence = unit / a.kv_heads, kv_head = unit % a.kv_heads;
-    const unsigned int first_row = (within % a.row_tiles) * kQueryTile;
+    const unsigned int first_row = row_tile * kQueryTile;
 
     // The sequence's paging values, refused when any would address outside the kernel's buffers.
     const SequenceSpan span = load_span<FORM>(sequence, a.query_offsets, a.page_offsets, a.last_page_lengths, a.query_lengths,

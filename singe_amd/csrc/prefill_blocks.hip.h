@@ -154,4 +154,52 @@ SINGE_DEVICE void finish_block(RowState& state, f32x16_t& s, float factor, float
     if constexpr (NEXT) next = upcoming;
 }
 
+// The stages of a tile's iteration, as the tile functions below take them.  The functions' pointer
+// parameters are __restrict__ and that is what they are for: once inlined, every LDS read in them is known
+// not to touch the stages the iteration's direct-to-LDS loads write, so the compiler does not make the
+// first read after those loads wait for them to land (without that knowledge it must, and each tile would
+// stall for a round trip to memory).  The caller waits for the loads itself, with loads_landed(), before
+// the barrier that hands the stages on.
+struct TileStages {
+    const unsigned char* keys;       // K of this tile
+    const unsigned char* next_keys;  // K of the next tile, landed before the last barrier
+    const unsigned char* values;     // V of this tile
+    unsigned char* key_dest;         // where K of the tile after next goes
+    unsigned char* value_dest;       // where V of the next tile goes
+};
+
+// All of this wave's outstanding loads from global memory, those to LDS included, have completed.
+SINGE_DEVICE void loads_landed() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0), other counters left alone
+
+// A tile no mask touches, with another block to come after it: issue(key_dest, value_dest) starts the
+// iteration's loads, then both blocks are folded while the scores of the block after each are computed.
+template <class Issue>
+SINGE_DEVICE void fold_interior_tile(RowState& state, f32x16_t& scores, const bf16x8_t (&q)[8], const ReadOffsets& offsets,
+                                     unsigned int hi, float factor, const unsigned char* __restrict__ keys,
+                                     const unsigned char* __restrict__ next_keys, const unsigned char* __restrict__ values,
+                                     unsigned char* __restrict__ key_dest, unsigned char* __restrict__ value_dest, Issue&& issue) {
+    issue(key_dest, value_dest);
+    const float shift_even = begin_block(state, scores, hi, factor, false, [](unsigned int) { return false; });
+    finish_block<true>(state, scores, factor, shift_even, values, offsets, scores, q, keys + kBlockBytes);
+    __builtin_amdgcn_sched_barrier(0);  // keeps the second block's operand reads out of the first block's registers
+    const float shift_odd = begin_block(state, scores, hi, factor, false, [](unsigned int) { return false; });
+    finish_block<true>(state, scores, factor, shift_odd, values + kBlockBytes, offsets, scores, q, next_keys);
+}
+
+// Any other tile: the same steps one after the other, each only if the wave still has that block;
+// fold(block, scores, values) applies the masks and folds one block.
+template <class Issue, class Fold>
+SINGE_DEVICE void fold_edge_tile(f32x16_t& scores, const bf16x8_t (&q)[8], const ReadOffsets& offsets, unsigned int block,
+                                 unsigned int wave_blocks, const unsigned char* __restrict__ keys,
+                                 const unsigned char* __restrict__ next_keys, const unsigned char* __restrict__ values,
+                                 unsigned char* __restrict__ key_dest, unsigned char* __restrict__ value_dest, Issue&& issue, Fold&& fold) {
+    issue(key_dest, value_dest);
+    if (block < wave_blocks) fold(block, scores, values);
+    if (block + 1 < wave_blocks) {
+        score_block(scores, q, keys + kBlockBytes, offsets);
+        fold(block + 1, scores, values + kBlockBytes);
+    }
+    if (block + 2 < wave_blocks) score_block(scores, q, next_keys, offsets);
+}
+
 }  // namespace prefill
