@@ -190,11 +190,11 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
                                                  (lds_words_t)(stage + (16u * i + 4u * wave) * kRowBytes), 16, 0, 0);
         }
     };
-    auto load_keys = [&](unsigned int tile, const Pages& pages, unsigned int stage) __attribute__((always_inline)) {
-        load(key_bytes, key_chunk, tile, pages, lds + stage * kTileBytes);
+    auto load_keys = [&](unsigned int tile, const Pages& pages, unsigned char* stage) __attribute__((always_inline)) {
+        load(key_bytes, key_chunk, tile, pages, stage);
     };
-    auto load_values = [&](unsigned int tile, const Pages& pages, unsigned int stage) __attribute__((always_inline)) {
-        load(value_bytes, value_chunk, tile, pages, lds + kValueBase + stage * kTileBytes);
+    auto load_values = [&](unsigned int tile, const Pages& pages, unsigned char* stage) __attribute__((always_inline)) {
+        load(value_bytes, value_chunk, tile, pages, stage);
     };
 
     RowState state;
@@ -212,10 +212,11 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         check(raw_first, first);
         if (first_tile + 1 < tiles) check(raw_behind, behind);
         if (first_tile + 2 < tiles) check(raw_ahead, ahead);
-        load_keys(first_tile, first, 0);
-        load_values(first_tile, first, 0);
-        if (first_tile + 1 < tiles) load_keys(first_tile + 1, behind, 1);
+        load_keys(first_tile, first, lds);
+        load_values(first_tile, first, lds + kValueBase);
+        if (first_tile + 1 < tiles) load_keys(first_tile + 1, behind, lds + kTileBytes);
     }
+    loads_landed();
     __syncthreads();
 
     // Folds block `block` (scores in `s`, values at `values`) with the masks' edges applied.
@@ -240,24 +241,34 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     f32x16_t scores;
     if (2u * first_tile < wave_blocks) score_block(scores, q, lds, offsets);
     unsigned int key_stage = 0, value_stage = 0;
-    const unsigned char *keys_at, *next_keys, *values_at;
-    auto enter = [&](unsigned int tile) __attribute__((always_inline)) {
+    // Names the stages a tile's iteration works on and loads into.
+    auto enter = [&]() __attribute__((always_inline)) {
         const unsigned int next_key_stage = key_stage + 1 == kKeyStages ? 0 : key_stage + 1;
         const unsigned int spare_key_stage = next_key_stage + 1 == kKeyStages ? 0 : next_key_stage + 1;
-        if (tile + 3 < tiles) lookup(tile + 3, fresh);
-        if (tile + 2 < tiles) load_keys(tile + 2, ahead, spare_key_stage);
-        if (tile + 1 < tiles) load_values(tile + 1, behind, value_stage ^ 1u);
-        keys_at = lds + key_stage * kTileBytes;
-        next_keys = lds + next_key_stage * kTileBytes;
-        values_at = lds + kValueBase + value_stage * kTileBytes;
+        TileStages stages;
+        stages.keys = lds + key_stage * kTileBytes;
+        stages.next_keys = lds + next_key_stage * kTileBytes;
+        stages.values = lds + kValueBase + value_stage * kTileBytes;
+        stages.key_dest = lds + spare_key_stage * kTileBytes;
+        stages.value_dest = lds + kValueBase + (value_stage ^ 1u) * kTileBytes;
         key_stage = next_key_stage;
         value_stage ^= 1u;
+        return stages;
     };
-    // Ends a tile's iteration: the ids looked up at its start have had the whole tile to arrive.
-    auto leave = [&](unsigned int tile) __attribute__((always_inline)) {
+    unsigned int tile = first_tile;
+    // Starts a tile's loads: ids for tile + 3, K of tile + 2, V of tile + 1.
+    auto issue = [&](unsigned char* key_dest, unsigned char* value_dest) __attribute__((always_inline)) {
+        if (tile + 3 < tiles) lookup(tile + 3, fresh);
+        if (tile + 2 < tiles) load_keys(tile + 2, ahead, key_dest);
+        if (tile + 1 < tiles) load_values(tile + 1, behind, value_dest);
+    };
+    // Ends a tile's iteration: the ids looked up at its start have had the whole tile to arrive, this wave's
+    // loads have landed, and the barrier hands the stages on.
+    auto leave = [&]() __attribute__((always_inline)) {
         __builtin_amdgcn_sched_barrier(0);
         behind = ahead;
         if (tile + 3 < tiles) check(fresh, ahead);
+        loads_landed();
         __syncthreads();
     };
 
@@ -272,28 +283,19 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         const unsigned int whole = keys / kKeyTile;  // tiles t with 64 t + 64 <= keys
         interior_end = interior_end < whole ? interior_end : whole;
     }
-    unsigned int tile = first_tile;
     for (; tile < interior_end; ++tile) {
-        enter(tile);
-        const float shift_even = begin_block(state, scores, hi, factor, false, [](unsigned int) { return false; });
-        finish_block<true>(state, scores, factor, shift_even, values_at, offsets, scores, q, keys_at + kBlockBytes);
-        __builtin_amdgcn_sched_barrier(0);
-        const float shift_odd = begin_block(state, scores, hi, factor, false, [](unsigned int) { return false; });
-        finish_block<true>(state, scores, factor, shift_odd, values_at + kBlockBytes, offsets, scores, q, next_keys);
-        leave(tile);
+        const TileStages stages = enter();
+        fold_interior_tile(state, scores, q, offsets, hi, factor, stages.keys, stages.next_keys, stages.values, stages.key_dest,
+                           stages.value_dest, issue);
+        leave();
     }
     // Tiles on a mask's edge and the last ones (and, for waves that have run out of blocks, the workgroup's
-    // remaining loads and barriers): the same steps one after the other.
+    // remaining loads and barriers).
     for (; tile < tiles; ++tile) {
-        enter(tile);
-        const unsigned int block = 2u * tile;
-        if (block < wave_blocks) fold(block, scores, values_at);
-        if (block + 1 < wave_blocks) {
-            score_block(scores, q, keys_at + kBlockBytes, offsets);
-            fold(block + 1, scores, values_at + kBlockBytes);
-        }
-        if (block + 2 < wave_blocks) score_block(scores, q, next_keys, offsets);
-        leave(tile);
+        const TileStages stages = enter();
+        fold_edge_tile(scores, q, offsets, 2u * tile, wave_blocks, stages.keys, stages.next_keys, stages.values, stages.key_dest,
+                       stages.value_dest, issue, fold);
+        leave();
     }
 
     // Normalise and store; a row that sees no key stays zero and has a log-sum-exp of -inf
