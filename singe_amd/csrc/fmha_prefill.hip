@@ -22,6 +22,10 @@ namespace {
 
 using namespace prefill;
 
+// Whether the interior tiles read their K operands a block ahead (prefill_blocks.hip.h): measured, it gains
+// nothing here (the other wave of the SIMD already covers the reads' latency) and costs 30 registers.
+constexpr bool kDenseOperandsAhead = false;
+
 // One 128-row query tile of (batch, head) pair `bh`.
 template <bool CAUSAL>
 SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, unsigned int bh, unsigned int query_tile) {
@@ -177,13 +181,15 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
         interior_tiles = interior_tiles < whole ? interior_tiles : whole;
     }
     unsigned int tile = 0;
+    uint4 operand[8];
+    if (kDenseOperandsAhead && interior_tiles > 0) read_key_operands(operand, lds + kBlockBytes, offsets);
     auto issue = [&](unsigned char* key_dest, unsigned char* value_dest) __attribute__((always_inline)) {
         if (tile + 2 < tiles) load_keys(tile + 2, key_dest);
         if (tile + 1 < tiles) load_values(tile + 1, value_dest);
     };
     for (; tile < interior_tiles; ++tile) {
         const TileStages stages = enter();
-        fold_interior_tile(state, scores, q, offsets, hi, factor, stages.keys, stages.next_keys, stages.values, stages.key_dest,
+        fold_interior_tile<kDenseOperandsAhead>(state, scores, operand, q, offsets, hi, factor, stages.keys, stages.next_keys, stages.values, stages.key_dest,
                            stages.value_dest, issue);
         leave();
     }

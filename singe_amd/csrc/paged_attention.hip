@@ -34,6 +34,9 @@ namespace {
 
 using namespace prefill;
 
+// Whether the interior tiles read their K operands a block ahead (prefill_blocks.hip.h).
+constexpr bool kPagedOperandsAhead = true;
+
 constexpr unsigned int kNoPage = 0xFFFFFFFFu;  // a table entry outside the cache: reported, never read through
 
 template <bool SOFTCAP, int FORM>
@@ -283,9 +286,11 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         const unsigned int whole = keys / kKeyTile;  // tiles t with 64 t + 64 <= keys
         interior_end = interior_end < whole ? interior_end : whole;
     }
+    uint4 operand[8];
+    if (kPagedOperandsAhead && tile < interior_end) read_key_operands(operand, lds + kBlockBytes, offsets);
     for (; tile < interior_end; ++tile) {
         const TileStages stages = enter();
-        fold_interior_tile(state, scores, q, offsets, hi, factor, stages.keys, stages.next_keys, stages.values, stages.key_dest,
+        fold_interior_tile<kPagedOperandsAhead>(state, scores, operand, q, offsets, hi, factor, stages.keys, stages.next_keys, stages.values, stages.key_dest,
                            stages.value_dest, issue);
         leave();
     }

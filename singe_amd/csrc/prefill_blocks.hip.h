@@ -103,12 +103,16 @@ SINGE_DEVICE float begin_block(RowState& state, f32x16_t& s, unsigned int hi, fl
 // weights and O^T += V^T . P^T, and, when NEXT is set, the score products of the block at `next_keys` are
 // issued in between: one MFMA, then the exponentials of two registers, and so on, so the matrix core
 // computes the next block's scores while the vector unit exponentiates this one's.
-template <bool NEXT>
+//   AHEAD       the K operands travel between calls in `operand`: on entry those of the block whose scores
+//               are computed here (`next_keys` is not read), on return those of the block at `after_keys`, each
+//               read as soon as the product that used its register has been issued, a whole block before
+//               its use.  Otherwise the operands are read from `next_keys` at the start of the call.
+template <bool NEXT, bool AHEAD = false>
 SINGE_DEVICE void finish_block(RowState& state, f32x16_t& s, float factor, float shift, const unsigned char* values,
-                               const ReadOffsets& offsets, f32x16_t& next, const bf16x8_t (&q)[8], const unsigned char* next_keys) {
+                               const ReadOffsets& offsets, f32x16_t& next, const bf16x8_t (&q)[8], const unsigned char* next_keys,
+                               uint4 (&operand)[8], const unsigned char* after_keys) {
     typedef v4i16_t __attribute__((address_space(3))) * lds_v4_t;
-    uint4 operand[8];
-    if constexpr (NEXT) {
+    if constexpr (NEXT && !AHEAD) {
 #pragma unroll
         for (int step = 0; step < 8; ++step) operand[step] = *reinterpret_cast<const uint4*>(next_keys + offsets.key(step));
     }
@@ -134,8 +138,10 @@ SINGE_DEVICE void finish_block(RowState& state, f32x16_t& s, float factor, float
                 second[db] = __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7);
             }
         }
-        if constexpr (NEXT)
+        if constexpr (NEXT) {
             upcoming = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, operand[step]), q[step], upcoming, 0, 0, 0);
+            if constexpr (AHEAD) operand[step] = *reinterpret_cast<const uint4*>(after_keys + offsets.key(step));
+        }
         s[2 * step] = fast_exp2(fmaf(s[2 * step], factor, shift));
         s[2 * step + 1] = fast_exp2(fmaf(s[2 * step + 1], factor, shift));
         total += s[2 * step] + s[2 * step + 1];
@@ -152,6 +158,13 @@ SINGE_DEVICE void finish_block(RowState& state, f32x16_t& s, float factor, float
                                                               __builtin_bit_cast(bf16x8_t, weights), state.out[db], 0, 0, 0);
     }
     if constexpr (NEXT) next = upcoming;
+}
+
+template <bool NEXT>
+SINGE_DEVICE void finish_block(RowState& state, f32x16_t& s, float factor, float shift, const unsigned char* values,
+                               const ReadOffsets& offsets, f32x16_t& next, const bf16x8_t (&q)[8], const unsigned char* next_keys) {
+    uint4 operand[8];
+    finish_block<NEXT, false>(state, s, factor, shift, values, offsets, next, q, next_keys, operand, next_keys);
 }
 
 // The stages of a tile's iteration, as the tile functions below take them.  The functions' pointer
@@ -173,17 +186,26 @@ SINGE_DEVICE void loads_landed() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmc
 
 // A tile no mask touches, with another block to come after it: issue(key_dest, value_dest) starts the
 // iteration's loads, then both blocks are folded while the scores of the block after each are computed.
-template <class Issue>
-SINGE_DEVICE void fold_interior_tile(RowState& state, f32x16_t& scores, const bf16x8_t (&q)[8], const ReadOffsets& offsets,
-                                     unsigned int hi, float factor, const unsigned char* __restrict__ keys,
+// With AHEAD the K operands of those products are read a block early and carried in `operand`: those of the
+// tile's second block on entry (read_key_operands before the first tile), of the next tile's on return.
+template <bool AHEAD, class Issue>
+SINGE_DEVICE void fold_interior_tile(RowState& state, f32x16_t& scores, uint4 (&operand)[8], const bf16x8_t (&q)[8],
+                                     const ReadOffsets& offsets, unsigned int hi, float factor, const unsigned char* __restrict__ keys,
                                      const unsigned char* __restrict__ next_keys, const unsigned char* __restrict__ values,
                                      unsigned char* __restrict__ key_dest, unsigned char* __restrict__ value_dest, Issue&& issue) {
     issue(key_dest, value_dest);
     const float shift_even = begin_block(state, scores, hi, factor, false, [](unsigned int) { return false; });
-    finish_block<true>(state, scores, factor, shift_even, values, offsets, scores, q, keys + kBlockBytes);
+    finish_block<true, AHEAD>(state, scores, factor, shift_even, values, offsets, scores, q, keys + kBlockBytes, operand, next_keys);
     __builtin_amdgcn_sched_barrier(0);  // keeps the second block's operand reads out of the first block's registers
     const float shift_odd = begin_block(state, scores, hi, factor, false, [](unsigned int) { return false; });
-    finish_block<true>(state, scores, factor, shift_odd, values + kBlockBytes, offsets, scores, q, next_keys);
+    finish_block<true, AHEAD>(state, scores, factor, shift_odd, values + kBlockBytes, offsets, scores, q, next_keys, operand,
+                              next_keys + kBlockBytes);
+}
+
+// The K operands of the block at `keys`.
+SINGE_DEVICE void read_key_operands(uint4 (&operand)[8], const unsigned char* keys, const ReadOffsets& offsets) {
+#pragma unroll
+    for (int step = 0; step < 8; ++step) operand[step] = *reinterpret_cast<const uint4*>(keys + offsets.key(step));
 }
 
 // Any other tile: the same steps one after the other, each only if the wave still has that block;
