@@ -16,8 +16,10 @@ enum KernelId : int {
     kDecodeF8Wide, kDecodeF8WideAny, kDecodeF8WideRelaxed, kDecodeF8WideRelaxedAny,
     kPrefillCausal, kPrefillFull,
     kPrefillF32D32, kPrefillF32D64, kPrefillF32D128, kPrefillF32D256,
+    // paged attention: + 4 when the page size is a power of two of at least 16 keys
     kPagedAttentionI32, kPagedAttentionI64, kPagedAttentionSoftcapI32, kPagedAttentionSoftcapI64,
-    kPagedKvPrefill,
+    kPagedAttentionI32P16, kPagedAttentionI64P16, kPagedAttentionSoftcapI32P16, kPagedAttentionSoftcapI64P16,
+    kPagedKvPrefill, kPagedKvPrefillP16,
     kSplitKReduce,
     kRotaryCacheF32, kRotaryCacheBf16, kRotaryCacheF16,
     kPagingIndicesI32, kPagingIndicesI64,

@@ -93,9 +93,10 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
     const uint64_t blocks = units * args.row_tiles;
     if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
     const bool wide = p.index_type == SINGE_HIP_INDEX_I64;
-    const KernelId kernel = p.has_softcap ? (wide ? kPagedAttentionSoftcapI64 : kPagedAttentionSoftcapI32)
-                                          : (wide ? kPagedAttentionI64 : kPagedAttentionI32);
-    return launch(kernel, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+    const int kernel = (p.has_softcap ? (wide ? kPagedAttentionSoftcapI64 : kPagedAttentionSoftcapI32)
+                                      : (wide ? kPagedAttentionI64 : kPagedAttentionI32)) +
+                       (args.page_shift >= 4 ? 4 : 0);
+    return launch(static_cast<KernelId>(kernel), static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
 }
 
 }  // namespace
@@ -203,5 +204,5 @@ extern "C" int32_t singe_hip_paged_kv_prefill_attention_bf16(
     const uint64_t units = (static_cast<uint64_t>(c.batch) * c.kv_heads + 7) / 8 * 8;
     const uint64_t blocks = units * args.row_tiles;
     if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
-    return launch(kPagedKvPrefill, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+    return launch(args.page_shift >= 4 ? kPagedKvPrefillP16 : kPagedKvPrefill, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
 }

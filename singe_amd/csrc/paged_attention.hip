@@ -39,7 +39,7 @@ constexpr bool kPagedOperandsAhead = true;
 
 constexpr unsigned int kNoPage = 0xFFFFFFFFu;  // a table entry outside the cache: reported, never read through
 
-template <bool SOFTCAP, int FORM>
+template <bool SOFTCAP, int FORM, bool GROUPED>
 SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned char* lds) {
     const unsigned int tid = threadIdx.x, lane = tid & 63;
     const unsigned int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and known to be
@@ -77,7 +77,7 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         return;
     }
     const long long query_start = span.query_start, page_start = span.page_start;
-    const unsigned int queries = span.queries, keys = span.keys;
+    const unsigned int queries = __builtin_amdgcn_readfirstlane(span.queries), keys = __builtin_amdgcn_readfirstlane(span.keys);
     const unsigned int packed = queries * groups;
     if (first_row >= packed) return;
 
@@ -148,6 +148,12 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     // pages[page_start + key / page_size] at slot key % page_size; rows past the sequence's last key re-read
     // that key and are masked, so nothing the sequence does not own reaches LDS.  Page ids are looked up
     // three tiles ahead and checked then; K is loaded two tiles ahead and V one, from the same ids.
+    //
+    // GROUPED (the page size is 16, 32, 64, ... keys): the sixteen rows of an instruction, keys 16-aligned, sit
+    // in one page, so its id is one scalar load, checked and multiplied on the scalar unit, and a load's
+    // address is a scalar base (page, the group's first slot, the kv head) plus a per-lane offset that never
+    // changes (row in the group, chunk): no vector arithmetic per load.  Otherwise each lane looks up and
+    // places its own row.
     const unsigned int load_row = 4u * wave + (lane >> 4), chunk_position = lane & 15u;
     const unsigned int key_chunk = (chunk_position ^ (load_row & 15u)) * 16u, value_chunk = (chunk_position ^ (4u * (load_row & 3u))) * 16u;
     const size_t page_bytes = static_cast<size_t>(a.page_size) * a.kv_heads * kRowBytes;
@@ -155,6 +161,7 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     const unsigned char* const key_bytes = reinterpret_cast<const unsigned char*>(a.key_cache);
     const unsigned char* const value_bytes = reinterpret_cast<const unsigned char*>(a.value_cache);
     const bool shifted = a.page_shift >= 0;
+    const unsigned int last_group = (keys - 1u) & ~15u;  // first key of the sixteen that hold the last one (keys > 0 where used)
     struct Pages {
         unsigned int id[4];
     };
@@ -165,12 +172,21 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         const unsigned int key = tile * kKeyTile + 16u * i + load_row;
         return key < keys ? key : keys - 1u;
     };
+    // GROUPED: first key of the group instruction i of a tile reads: its own, or the last group of the sequence.
+    auto group_of = [&](unsigned int tile, unsigned int i) __attribute__((always_inline)) {
+        const unsigned int first = tile * kKeyTile + 16u * i;
+        return first < last_group ? first : last_group;
+    };
     auto lookup = [&](unsigned int tile, RawPages& raw) __attribute__((always_inline)) {
 #pragma unroll
         for (unsigned int i = 0; i < 4; ++i) {
-            const unsigned int key = key_of(tile, i);
-            const unsigned int entry = shifted ? key >> a.page_shift : key / a.page_size;
-            raw.value[i] = read_raw_page<FORM>(a.pages, static_cast<size_t>(page_start) + entry);
+            if constexpr (GROUPED) {
+                raw.value[i] = read_raw_page_uniform<FORM>(a.pages, static_cast<size_t>(page_start) + (group_of(tile, i) >> a.page_shift));
+            } else {
+                const unsigned int key = key_of(tile, i);
+                const unsigned int entry = shifted ? key >> a.page_shift : key / a.page_size;
+                raw.value[i] = read_raw_page<FORM>(a.pages, static_cast<size_t>(page_start) + entry);
+            }
         }
     };
     auto check = [&](const RawPages& raw, Pages& pages) __attribute__((always_inline)) {
@@ -182,22 +198,41 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
             pages.id[i] = valid ? static_cast<unsigned int>(page) : kNoPage;
         }
     };
-    auto load = [&](const unsigned char* cache, unsigned int chunk, unsigned int tile, const Pages& pages, unsigned char* stage) __attribute__((always_inline)) {
+    const unsigned int key_lane = load_row * slot_bytes + key_chunk, value_lane = load_row * slot_bytes + value_chunk;
+    auto load = [&](const unsigned char* cache, unsigned int chunk, unsigned int lane_offset, unsigned int tile, const Pages& pages,
+                    unsigned char* stage) __attribute__((always_inline)) {
 #pragma unroll
         for (unsigned int i = 0; i < 4; ++i) {
-            const unsigned int key = key_of(tile, i);
-            const unsigned int slot = shifted ? key & (a.page_size - 1u) : key % a.page_size;
-            const size_t offset = pages.id[i] * page_bytes + (slot * slot_bytes + head_bytes + chunk);
-            if (pages.id[i] != kNoPage)
-                __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(cache + offset),
+            if constexpr (GROUPED) {
+                if (pages.id[i] == kNoPage) continue;
+                const unsigned int first = tile * kKeyTile + 16u * i, group = group_of(tile, i);
+                const unsigned char* base = cache + (pages.id[i] * page_bytes + ((group & (a.page_size - 1u)) * slot_bytes + head_bytes));
+                unsigned int offset = lane_offset;
+                if (first + 15u >= keys) {  // the group holds the sequence's last key, or lies past it
+                    const unsigned int last = keys - 1u - group;
+                    offset = (load_row < last ? load_row : last) * slot_bytes + chunk;
+                }
+                // Both pinned as they are (a scalar, a 32-bit per-lane offset) so the load keeps its
+                // scalar-base form (see fmha_prefill.hip).
+                asm("" : "+s"(base));
+                asm volatile("" : "+v"(offset));
+                __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(base + offset),
                                                  (lds_words_t)(stage + (16u * i + 4u * wave) * kRowBytes), 16, 0, 0);
+            } else {
+                const unsigned int key = key_of(tile, i);
+                const unsigned int slot = shifted ? key & (a.page_size - 1u) : key % a.page_size;
+                const size_t offset = pages.id[i] * page_bytes + (slot * slot_bytes + head_bytes + chunk);
+                if (pages.id[i] != kNoPage)
+                    __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(cache + offset),
+                                                     (lds_words_t)(stage + (16u * i + 4u * wave) * kRowBytes), 16, 0, 0);
+            }
         }
     };
     auto load_keys = [&](unsigned int tile, const Pages& pages, unsigned char* stage) __attribute__((always_inline)) {
-        load(key_bytes, key_chunk, tile, pages, stage);
+        load(key_bytes, key_chunk, key_lane, tile, pages, stage);
     };
     auto load_values = [&](unsigned int tile, const Pages& pages, unsigned char* stage) __attribute__((always_inline)) {
-        load(value_bytes, value_chunk, tile, pages, stage);
+        load(value_bytes, value_chunk, value_lane, tile, pages, stage);
     };
 
     RowState state;
@@ -331,15 +366,21 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
 
 }  // namespace
 
-#define SINGE_PAGED_ATTENTION_KERNEL(NAME, SOFTCAP, FORM)                                                  \
+#define SINGE_PAGED_ATTENTION_KERNEL(NAME, SOFTCAP, FORM, GROUPED)                                         \
     extern "C" __global__ __launch_bounds__(256, 2) void NAME(PagedAttentionArgs args) {                    \
         __shared__ __attribute__((aligned(1024))) unsigned char paged_lds[prefill::kStagedLdsBytes];        \
-        paged_attention_body<SOFTCAP, FORM>(args, paged_lds);                                              \
+        paged_attention_body<SOFTCAP, FORM, GROUPED>(args, paged_lds);                                     \
     }
 
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i32, false, kCsrI32)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i64, false, kCsrI64)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i32, true, kCsrI32)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i64, true, kCsrI64)
+// _p16: the page size is a power of two of at least 16 keys (page ids on the scalar unit).
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i32, false, kCsrI32, false)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i64, false, kCsrI64, false)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i32, true, kCsrI32, false)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i64, true, kCsrI64, false)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i32_p16, false, kCsrI32, true)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i64_p16, false, kCsrI64, true)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i32_p16, true, kCsrI32, true)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i64_p16, true, kCsrI64, true)
 // paged_kv_prefill_attention_bf16 of the singe-kernel surface: same gather, block-table paging.
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_bf16_d128, false, kTable)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_bf16_d128, false, kTable, false)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_bf16_d128_p16, false, kTable, true)

@@ -37,6 +37,14 @@ SINGE_DEVICE RawPage<FORM> read_raw_page(const void* pages, size_t at) {
     return static_cast<const RawPage<FORM>*>(pages)[at];
 }
 
+// The same load from an address every lane shares, through the constant address space (paging vectors are
+// not written while a kernel that reads them runs), which lets it run on the scalar unit.
+template <int FORM>
+SINGE_DEVICE RawPage<FORM> read_raw_page_uniform(const void* pages, size_t at) {
+    typedef const RawPage<FORM> __attribute__((address_space(4))) * constant_pages_t;
+    return ((constant_pages_t)pages)[at];
+}
+
 struct SequenceSpan {
     long long query_start;  // first token of the sequence in the packed queries
     long long page_start;   // first entry of the sequence in `pages`
