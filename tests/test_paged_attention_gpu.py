@@ -60,7 +60,8 @@ OPTIONS = [neural.AttentionOptions(), neural.AttentionOptions(causal=True),
 
 
 @pytest.mark.parametrize("options", OPTIONS)
-@pytest.mark.parametrize("heads,kv_heads,page_size", [(8, 2, 1), (8, 1, 16), (4, 4, 7), (64, 8, 16)])
+@pytest.mark.parametrize("heads,kv_heads,page_size", [(8, 2, 1), (8, 1, 16), (4, 4, 7), (64, 8, 16), (8, 2, 8), (8, 2, 32),
+                                                      (4, 1, 64), (8, 2, 128), (6, 3, 48)])
 def test_ragged_sequences_match_oracle(heads, kv_heads, page_size, options):
     # decode, full prefill, chunked prefill, no keys (kernel_plan/source/tests.rs:830-889), plus more
     # queries than keys, where the CPU path's saturating position applies
@@ -72,6 +73,24 @@ def test_int64_indices_and_chunked_prefill_shape():
     # one sequence of the chunked-prefill shape: 512 new queries over a cached prefix, 64 query / 8 kv heads
     run_case([(512, 1536 + 512), (512, 1024 + 512)], 64, 8, 16, neural.AttentionOptions(causal=True),
              index_dtype=torch.int64, seed=4)
+
+
+def test_a_bad_page_in_a_large_page_table_is_refused_and_the_rest_is_right():
+    """Page sizes of 16 keys and more look their pages up on the scalar unit: the same error contract."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(8)
+    q = torch.randn((40, 4, 128), generator=gen, device="cuda").to(torch.bfloat16)
+    cache = torch.randn((6, 32, 2, 128), generator=gen, device="cuda").to(torch.bfloat16)
+    index = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
+    good = neural.Paging(index([0, 20, 40]), index([0, 3, 5]), index([4, 1, 0, 2, 5]), index([7, 32]))
+    want, _ = neural.paged_attention(q, cache, cache, good, neural.AttentionOptions(causal=True))
+    bad = neural.Paging(index([0, 20, 40]), index([0, 3, 5]), index([4, 1, 0, 2, 6]), index([7, 32]))  # page 6 of 6
+    status = torch.zeros(1, dtype=torch.int32, device="cuda")
+    got, _ = neural.paged_attention(q, cache, cache, bad, neural.AttentionOptions(causal=True), status=status, check=False)
+    assert status.item() == 1
+    assert torch.equal(got[:20], want[:20])  # the sequence with good pages is untouched by its neighbour's error
+    with pytest.raises(error.IndexOutOfBounds):
+        neural.paged_attention(q, cache, cache, bad, neural.AttentionOptions(causal=True))
 
 
 TOKENS, HEADS, DIM, SLOTS, PAGES = 2, 2, 128, 4, 2

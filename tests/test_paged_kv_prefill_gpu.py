@@ -86,6 +86,8 @@ def run_case(sequences, heads, kv_heads, block_size, causal, seed=0, gap_tokens=
     dict(sequences=[(130, 130), (1, 1), (33, 200), (64, 10)], heads=8, kv_heads=2, block_size=16),
     dict(sequences=[(300, 257)], heads=2, kv_heads=2, block_size=7),
     dict(sequences=[(70, 70), (0, 12), (9, 0), (20, 90)], heads=16, kv_heads=2, block_size=16, gap_tokens=2),
+    dict(sequences=[(100, 300), (7, 33), (64, 64)], heads=8, kv_heads=2, block_size=32),
+    dict(sequences=[(40, 200), (129, 129)], heads=4, kv_heads=1, block_size=128),
 ])
 def test_matches_oracle(case, causal):
     run_case(causal=causal, seed=11, **case)
