@@ -27,9 +27,9 @@ if ROOT not in sys.path:
 # HBM bytes per launch of the decode split kernel at the headline workload, from rocprofv3 --pmc runs of
 # this script: FETCH_SIZE 145768 x 2 KiB (the counter's unit, calibrated on a copy of known size) +
 # WRITE_SIZE 4552 KiB.  Reported only for that kernel, workload and tuning.
-DECODE_TRAFFIC_BYTES = (145768 * 2 + 4552) * 1024
+DECODE_TRAFFIC_BYTES = (145766 * 2 + 4552) * 1024
 # The same for the dense prefill kernel at batch 4 x seq 4096 x 32 heads: FETCH_SIZE 301283, WRITE_SIZE 131377.
-PREFILL_TRAFFIC_BYTES = (301283 * 2 + 131377) * 1024
+PREFILL_TRAFFIC_BYTES = (311083 * 2 + 132590) * 1024
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 POOLS = 3
@@ -201,7 +201,7 @@ def chunked_prefill_section(steps):
         "tokens_per_s": work.sequences * work.new_tokens / (avg * 1e-3),
         "ms_per_step": avg,
         "algorithmic_flops": flops,
-        "roofline": {"bound": "mfma", "kernel": "singe_paged_attention_bf16_d128_i32", "achieved": tflops,
+        "roofline": {"bound": "mfma", "kernel": "singe_paged_attention_bf16_d128_i32_p16", "achieved": tflops,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": None, "kernel_avg_us": avg * 1e3, "kernel_median_us": median * 1e3},
     }
