@@ -336,6 +336,42 @@ SINGE_HIP_API int32_t singe_hip_paged_attention_bf16(
     uint32_t* status,
     const SingePagedAttentionProblem* problem);
 
+/* The same op over a query the kernel normalises and rotates itself, the counterpart of
+ * KernelPlanner::rotary_paged_attention (singe/src/backend/cuda/kernel_plan/source/paged_attention.rs:533-542,
+ * query stage :881-977; operand order :687-715: the attention's inputs, the output, then cos, sin and the
+ * norm's weight, then the status word).  `query_rows` holds the query BEFORE its rotation; cos and sin are
+ * [tokens, head_dim / 2] of `table_type` (the angles of each token, shared by its heads); pairs are half-split,
+ * (p, p + head_dim / 2): first = a cos - b sin, second = b cos + a sin, after an optional RMS norm over the head
+ * dimension (x * rsqrt(mean(x^2) + eps)) times an optional weight [head_dim] of the query's type; the rotated
+ * query is rounded to the query's type before the products, as the reference rounds what it stages.
+ * bf16 at head dimension 128 without a softcap; other shapes return SINGE_HIP_UNSUPPORTED_WIDTH or
+ * SINGE_HIP_UNSUPPORTED_CONFIGURATION and take singe_hip_rotary_cache_write followed by
+ * singe_hip_paged_attention_*, as the reference plans them apart (compiled/plan/group.rs:94-98).
+ * `lse` may be null (the reference's fused kernel keeps it in scratch). */
+typedef struct SingeQueryRotation {
+    int32_t table_type;   /* SINGE_HIP_F32, SINGE_HIP_BF16 or SINGE_HIP_F16 */
+    uint8_t has_norm;
+    float eps;
+} SingeQueryRotation;
+
+SINGE_HIP_API int32_t singe_hip_rotary_paged_attention_bf16(
+    void* stream,
+    const uint16_t* query_rows,
+    const uint16_t* key_cache,
+    const uint16_t* value_cache,
+    const void* query_offsets,
+    const void* page_offsets,
+    const void* pages,
+    const void* last_page_lengths,
+    const void* cos,
+    const void* sin,
+    const uint16_t* query_weight,
+    uint16_t* output,
+    float* lse,
+    uint32_t* status,
+    const SingePagedAttentionProblem* problem,
+    const SingeQueryRotation* rotation);
+
 /* The same op for f32 and f16 tensors, and (through the bf16 entry point above) for bf16 at head
  * dimensions other than 128, up to 256: the general kernel, one wave per (token, head) row, f32
  * arithmetic whatever the storage type (kernel_plan/source/paged_general.rs:73-247; CPU form

@@ -70,6 +70,10 @@ class SplitKReduceConfigC(ctypes.Structure):
         "lse_batch_stride", "lse_head_stride", "output_batch_stride", "output_head_stride")]
 
 
+class QueryRotationC(ctypes.Structure):
+    _fields_ = [("table_type", ctypes.c_int32), ("has_norm", ctypes.c_uint8), ("eps", ctypes.c_float)]
+
+
 class RotaryCacheProblemC(ctypes.Structure):
     _fields_ = [("tokens", ctypes.c_int64), ("query_heads", ctypes.c_int64), ("cache_heads", ctypes.c_int64),
                 ("head_dim", ctypes.c_int64), ("cache_pages", ctypes.c_int64), ("page_slots", ctypes.c_int64),
@@ -161,6 +165,9 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_softcapped_window_attention_f32.restype = i32
     handle.singe_hip_paged_attention_bf16.argtypes = [c_void] * 11 + [ctypes.POINTER(PagedAttentionProblemC)]
     handle.singe_hip_paged_attention_bf16.restype = i32
+    handle.singe_hip_rotary_paged_attention_bf16.argtypes = [c_void] * 14 + [ctypes.POINTER(PagedAttentionProblemC),
+                                                                             ctypes.POINTER(QueryRotationC)]
+    handle.singe_hip_rotary_paged_attention_bf16.restype = i32
     handle.singe_hip_paged_attention_f32.argtypes = [c_void] * 11 + [ctypes.POINTER(PagedAttentionProblemC)]
     handle.singe_hip_paged_attention_f32.restype = i32
     handle.singe_hip_paged_attention_f16.argtypes = [c_void] * 11 + [ctypes.POINTER(PagedAttentionProblemC)]

@@ -112,6 +112,13 @@ struct PagedAttentionArgs {
     float scale_log2e;              // scale * log2(e)
     float softcap_scale;            // scale / cap
     float softcap_log2e;            // cap * log2(e)
+    // Kernels that rotate their query themselves (rotary_paged_attention):
+    const void* cos = nullptr;                // [tokens, 64] of table_type
+    const void* sin = nullptr;
+    const uint16_t* query_weight = nullptr;   // [128] bf16, or null
+    uint32_t table_type = 0;                  // SingeElement of cos and sin
+    uint32_t has_query_norm = 0;              // RMS norm over the head dimension before the rotation
+    float query_eps = 0.0f;
 };
 
 // singe_splitk_reduce_f32: strides in elements.

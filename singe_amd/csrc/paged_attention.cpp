@@ -20,12 +20,33 @@ int32_t paged_attention_general(int32_t data_type, void* stream, const void* que
 
 namespace {
 
+// What rotary_paged_attention adds to the operands: the angle tables, the norm's weight and its attributes.
+struct Rotation {
+    const void* cos;
+    const void* sin;
+    const void* weight;
+    const SingeQueryRotation* attributes;
+};
+
 int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_any, const void* key_cache_any,
                         const void* value_cache_any, const void* query_offsets, const void* page_offsets, const void* pages,
                         const void* last_page_lengths, void* output_any, float* lse, uint32_t* status,
-                        const SingePagedAttentionProblem* problem) {
+                        const SingePagedAttentionProblem* problem, const Rotation* rotation = nullptr) {
     if (problem == nullptr) return fail(SINGE_HIP_NULL_POINTER, "problem");
     const SingePagedAttentionProblem& p = *problem;
+    if (rotation != nullptr) {
+        if (rotation->attributes == nullptr) return fail(SINGE_HIP_NULL_POINTER, "rotation");
+        const int32_t table = rotation->attributes->table_type;
+        if (table != SINGE_HIP_F32 && table != SINGE_HIP_BF16 && table != SINGE_HIP_F16)
+            return fail(SINGE_HIP_INVALID_ARGUMENT, "angle table type");
+        if (rotation->attributes->has_norm && !std::isfinite(rotation->attributes->eps)) return fail(SINGE_HIP_INVALID_ARGUMENT, "eps");
+        // The fused form exists for the tensor-core kernel alone and without softcap here; the reference
+        // plans the rotation and the attention apart for the rest (compiled/plan/group.rs:94-98), and so
+        // does a caller of this library (singe_hip_rotary_cache_write, then singe_hip_paged_attention_*).
+        if (data_type != SINGE_HIP_BF16 || p.head_dim != 128)
+            return fail(SINGE_HIP_UNSUPPORTED_WIDTH, "rotary_paged_attention", static_cast<uint64_t>(p.head_dim));
+        if (p.has_softcap) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "rotary paged attention with a softcap");
+    }
     // paged_attention_problem: key_dim == head_dim (one field here), kv_heads > 0 dividing heads, page_size > 0.
     if (p.tokens < 0 || p.heads <= 0 || p.kv_heads <= 0 || p.heads % p.kv_heads != 0 || p.page_size <= 0 || p.head_dim <= 0 ||
         p.sequences < 0 || p.cache_pages < 0 || p.page_table < 0)
@@ -47,6 +68,7 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
     for (int i = 0; i < 7; ++i)
         if (pointers[i] == nullptr) return fail(SINGE_HIP_NULL_POINTER, names[i]);
     if (pages == nullptr && p.page_table > 0) return fail(SINGE_HIP_NULL_POINTER, "pages");
+    if (rotation != nullptr && (rotation->cos == nullptr || rotation->sin == nullptr)) return fail(SINGE_HIP_NULL_POINTER, "cos or sin");
     const float scale = p.has_scale ? p.scale : 1.0f / std::sqrt(static_cast<float>(p.head_dim));
     // The tensor-core kernel covers bf16 at head dimension 128 (the reference's takes f16/bf16 at
     // multiples of 16 up to 128: paged_attention.rs:586-592); everything else goes to the general one
@@ -93,6 +115,16 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
     const uint64_t blocks = units * args.row_tiles;
     if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
     const bool wide = p.index_type == SINGE_HIP_INDEX_I64;
+    if (rotation != nullptr) {
+        args.cos = rotation->cos;
+        args.sin = rotation->sin;
+        args.query_weight = rotation->attributes->has_norm ? static_cast<const uint16_t*>(rotation->weight) : nullptr;
+        args.table_type = static_cast<uint32_t>(rotation->attributes->table_type);
+        args.has_query_norm = rotation->attributes->has_norm ? 1u : 0u;
+        args.query_eps = rotation->attributes->eps;
+        const int rotary = kRotaryPagedAttention + (wide ? 1 : 0) + (args.page_shift >= 4 ? 2 : 0);
+        return launch(static_cast<KernelId>(rotary), static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+    }
     const int kernel = (p.has_softcap ? (wide ? kPagedAttentionSoftcapI64 : kPagedAttentionSoftcapI32)
                                       : (wide ? kPagedAttentionI64 : kPagedAttentionI32)) +
                        (args.page_shift >= 4 ? 4 : 0);
@@ -100,6 +132,18 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
 }
 
 }  // namespace
+
+extern "C" int32_t singe_hip_rotary_paged_attention_bf16(void* stream, const uint16_t* query_rows, const uint16_t* key_cache,
+                                                         const uint16_t* value_cache, const void* query_offsets,
+                                                         const void* page_offsets, const void* pages,
+                                                         const void* last_page_lengths, const void* cos, const void* sin,
+                                                         const uint16_t* query_weight, uint16_t* output, float* lse,
+                                                         uint32_t* status, const SingePagedAttentionProblem* problem,
+                                                         const SingeQueryRotation* rotation) {
+    const Rotation operands = {cos, sin, query_weight, rotation};
+    return paged_attention(SINGE_HIP_BF16, stream, query_rows, key_cache, value_cache, query_offsets, page_offsets, pages,
+                           last_page_lengths, output, lse, status, problem, &operands);
+}
 
 extern "C" int32_t singe_hip_paged_attention_bf16(void* stream, const uint16_t* query_rows, const uint16_t* key_cache,
                                                   const uint16_t* value_cache, const void* query_offsets,

@@ -37,9 +37,16 @@ using namespace prefill;
 // Whether the interior tiles read their K operands a block ahead (prefill_blocks.hip.h).
 constexpr bool kPagedOperandsAhead = true;
 
+// One value of an angle table of f32, bf16 or f16 (SingeElement).
+SINGE_DEVICE float table_value(const void* table, uint32_t table_type, size_t at) {
+    if (table_type == kElementF32) return static_cast<const float*>(table)[at];
+    if (table_type == kElementBf16) return __builtin_bit_cast(float, static_cast<unsigned int>(static_cast<const unsigned short*>(table)[at]) << 16);
+    return static_cast<float>(static_cast<const _Float16*>(table)[at]);
+}
+
 constexpr unsigned int kNoPage = 0xFFFFFFFFu;  // a table entry outside the cache: reported, never read through
 
-template <bool SOFTCAP, int FORM, bool GROUPED>
+template <bool SOFTCAP, int FORM, bool GROUPED, bool ROTATE = false>
 SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned char* lds) {
     const unsigned int tid = threadIdx.x, lane = tid & 63;
     const unsigned int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and known to be
@@ -133,12 +140,69 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     bf16x8_t q[8];
     {
         const uint16_t* row = a.query_rows + ((static_cast<size_t>(query_start) + my_token) * a.heads + kv_head * groups + my_head) * kHeadDim + 8 * hi;
+        uint4 bits[8];
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
-            uint4 bits = *reinterpret_cast<const uint4*>(row + 16 * s);
-            if (!row_valid) bits = make_uint4(0, 0, 0, 0);
-            bits.x ^= flip; bits.y ^= flip; bits.z ^= flip; bits.w ^= flip;
-            q[s] = __builtin_bit_cast(bf16x8_t, bits);
+            bits[s] = *reinterpret_cast<const uint4*>(row + 16 * s);
+            if (!row_valid) bits[s] = make_uint4(0, 0, 0, 0);
+        }
+        if constexpr (ROTATE) {
+            // The query arrives before its rotation (paged_attention.rs:881-977): an optional RMS norm over
+            // the head dimension with an optional weight, then half-split pairs (p, p + 64) turned by the
+            // token's angles, first = a cos - b sin, second = b cos + a sin, rounded to bf16 as the
+            // reference rounds what it stores in its tile.  A lane holds both halves of its pairs (dims
+            // 16 s + 8 hi + j and the same + 64); the other half of the row's squares is one swap away.
+            auto wide = [](unsigned int pair, int upper) __attribute__((always_inline)) {
+                return __builtin_bit_cast(float, upper ? pair & 0xffff0000u : pair << 16);
+            };
+            float scale = 1.0f;
+            if (a.has_query_norm != 0) {
+                float squares = 0.0f;
+#pragma unroll
+                for (int s = 0; s < 8; ++s) {
+                    const unsigned int words[4] = {bits[s].x, bits[s].y, bits[s].z, bits[s].w};
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) squares += wide(words[w], 0) * wide(words[w], 0) + wide(words[w], 1) * wide(words[w], 1);
+                }
+                squares = swap32_sum(squares);
+                scale = rsqrtf(squares / static_cast<float>(kHeadDim) + a.query_eps);
+            }
+            const size_t token = static_cast<size_t>(query_start) + my_token;
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                unsigned int first_words[4] = {bits[s].x, bits[s].y, bits[s].z, bits[s].w};
+                unsigned int second_words[4] = {bits[s + 4].x, bits[s + 4].y, bits[s + 4].z, bits[s + 4].w};
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    float rotated_first[2], rotated_second[2];
+#pragma unroll
+                    for (int upper = 0; upper < 2; ++upper) {
+                        const unsigned int pair = 16u * s + 8u * hi + 2u * w + upper;
+                        float first = wide(first_words[w], upper), second = wide(second_words[w], upper);
+                        if (a.has_query_norm != 0) {
+                            first *= scale;
+                            second *= scale;
+                            if (a.query_weight != nullptr) {
+                                first *= __builtin_bit_cast(float, static_cast<unsigned int>(a.query_weight[pair]) << 16);
+                                second *= __builtin_bit_cast(float, static_cast<unsigned int>(a.query_weight[pair + 64]) << 16);
+                            }
+                        }
+                        const float cosine = table_value(a.cos, a.table_type, token * 64 + pair);
+                        const float sine = table_value(a.sin, a.table_type, token * 64 + pair);
+                        rotated_first[upper] = first * cosine - second * sine;
+                        rotated_second[upper] = second * cosine + first * sine;
+                    }
+                    first_words[w] = row_valid ? pack_pair(rotated_first[0], rotated_first[1]) : 0u;
+                    second_words[w] = row_valid ? pack_pair(rotated_second[0], rotated_second[1]) : 0u;
+                }
+                bits[s] = make_uint4(first_words[0], first_words[1], first_words[2], first_words[3]);
+                bits[s + 4] = make_uint4(second_words[0], second_words[1], second_words[2], second_words[3]);
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < 8; ++s) {
+            bits[s].x ^= flip; bits[s].y ^= flip; bits[s].z ^= flip; bits[s].w ^= flip;
+            q[s] = __builtin_bit_cast(bf16x8_t, bits[s]);
         }
     }
 
@@ -366,21 +430,26 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
 
 }  // namespace
 
-#define SINGE_PAGED_ATTENTION_KERNEL(NAME, SOFTCAP, FORM, GROUPED)                                         \
+#define SINGE_PAGED_ATTENTION_KERNEL(NAME, SOFTCAP, FORM, GROUPED, ROTATE)                                 \
     extern "C" __global__ __launch_bounds__(256, 2) void NAME(PagedAttentionArgs args) {                    \
         __shared__ __attribute__((aligned(1024))) unsigned char paged_lds[prefill::kStagedLdsBytes];        \
-        paged_attention_body<SOFTCAP, FORM, GROUPED>(args, paged_lds);                                     \
+        paged_attention_body<SOFTCAP, FORM, GROUPED, ROTATE>(args, paged_lds);                             \
     }
 
 // _p16: the page size is a power of two of at least 16 keys (page ids on the scalar unit).
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i32, false, kCsrI32, false)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i64, false, kCsrI64, false)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i32, true, kCsrI32, false)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i64, true, kCsrI64, false)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i32_p16, false, kCsrI32, true)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i64_p16, false, kCsrI64, true)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i32_p16, true, kCsrI32, true)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i64_p16, true, kCsrI64, true)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i32, false, kCsrI32, false, false)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i64, false, kCsrI64, false, false)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i32, true, kCsrI32, false, false)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i64, true, kCsrI64, false, false)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i32_p16, false, kCsrI32, true, false)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i64_p16, false, kCsrI64, true, false)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i32_p16, true, kCsrI32, true, false)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i64_p16, true, kCsrI64, true, false)
 // paged_kv_prefill_attention_bf16 of the singe-kernel surface: same gather, block-table paging.
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_bf16_d128, false, kTable, false)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_bf16_d128_p16, false, kTable, true)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_bf16_d128, false, kTable, false, false)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_bf16_d128_p16, false, kTable, true, false)
+// rotary_paged_attention: the query is normalised and rotated on its way into the registers.
+SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i32, false, kCsrI32, false, true)
+SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i64, false, kCsrI64, false, true)
+SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i32_p16, false, kCsrI32, true, true)
+SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i64_p16, false, kCsrI64, true, true)

@@ -184,6 +184,52 @@ def paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: t
     return output, lse
 
 
+def rotary_paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor, paging: Paging,
+                           cos: torch.Tensor, sin: torch.Tensor, options: AttentionOptions = AttentionOptions(), *,
+                           query_norm: "RotationNorm | None" = None, stream=None, status: torch.Tensor | None = None,
+                           check: bool = True):
+    """Paged attention over a query the kernel normalises and rotates itself, the reference's fused
+    rotary_paged_attention (singe/src/backend/cuda/kernel_plan/source/paged_attention.rs:533-542, 881-977):
+    ``query`` [tokens, heads, 128] bf16 before its rotation, ``cos`` / ``sin`` [tokens, 1, 64] (or [tokens, 64]) of
+    f32, bf16 or f16, the same pairs and norm as ``rotary_cache_write``.  Returns (output, lse) like
+    ``paged_attention``.  Other types and head dimensions raise UnsupportedWidth: rotate with
+    ``rotary_cache_write`` and attend with ``paged_attention``, as the reference plans them apart."""
+    for tensor, name in ((query, "query"), (key_cache, "key_cache"), (value_cache, "value_cache")):
+        if not tensor.is_cuda or tensor.dtype != query.dtype or not tensor.is_contiguous():
+            raise error.InvalidArgument(f"paged attention {name} must be a contiguous device tensor of the query's type")
+    if query.dtype != torch.bfloat16:
+        raise error.UnsupportedWidth("rotary_paged_attention takes bf16")
+    for tensor in (paging.query_offsets, paging.page_offsets, paging.pages, paging.last_page_lengths):
+        if not tensor.is_cuda or not tensor.is_contiguous():
+            raise error.InvalidArgument("paged attention index tensors must be contiguous device tensors")
+    if cos.dtype not in _DATA_TYPES or sin.dtype != cos.dtype or not cos.is_cuda or not sin.is_cuda:
+        raise error.InvalidArgument("rotary paged attention angle tables")
+    cos, sin = cos.contiguous(), sin.contiguous()
+    tokens, _, head_dim = query.shape
+    if cos.numel() != tokens * (head_dim // 2) or sin.numel() != cos.numel():
+        raise error.InvalidArgument("rotary paged attention angles must be [tokens, 1, head_dim / 2]")
+    weight = None if query_norm is None or query_norm.weight is None else query_norm.weight.to(query.dtype).contiguous()
+    if weight is not None and weight.numel() != head_dim:
+        raise error.InvalidArgument("rotary paged attention norm weight must hold head_dim values")
+    problem = _problem(query, key_cache, value_cache, paging, options)
+    rotation = _native.QueryRotationC(_DATA_TYPES[cos.dtype], 1 if query_norm is not None else 0,
+                                      query_norm.eps if query_norm is not None else 0.0)
+    output = torch.zeros_like(query)
+    lse = torch.full(query.shape[:2], float("-inf"), device=query.device, dtype=torch.float32)
+    if status is None:
+        status = torch.zeros(1, device=query.device, dtype=torch.int32)
+    handle = int((stream or torch.cuda.current_stream()).cuda_stream)
+    code = _native.lib().singe_hip_rotary_paged_attention_bf16(
+        handle, query.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), paging.query_offsets.data_ptr(),
+        paging.page_offsets.data_ptr(), paging.pages.data_ptr(), paging.last_page_lengths.data_ptr(), cos.data_ptr(), sin.data_ptr(),
+        None if weight is None else weight.data_ptr(), output.data_ptr(), lse.data_ptr(), status.data_ptr(), ctypes.byref(problem),
+        ctypes.byref(rotation))
+    _native.check(code, "rotary_paged_attention")
+    if check and int(status.item()) == STATUS_INDEX_OUT_OF_BOUNDS:
+        raise error.IndexOutOfBounds("paged attention paging value outside its buffers")
+    return output, lse
+
+
 @dataclass(frozen=True)
 class RotationNorm:
     """The RMS normalisation a rotation applies first (rotary_cache.rs:25-30)."""

@@ -31,7 +31,8 @@ def test_code_object_is_built_and_names_every_kernel():
     image = open(_native.CODE_OBJECT_PATH, "rb").read()
     for kernel in (b"singe_paged_decode_bf16_d128_g1_b16", b"singe_paged_decode_f8kv_wide_d128_b16",
                    b"singe_paged_decode_combine_bf16", b"singe_fmha_prefill_bf16_d128_causal",
-                   b"singe_fmha_prefill_f32_d64", b"singe_paged_attention_bf16_d128_i64"):
+                   b"singe_fmha_prefill_f32_d64", b"singe_paged_attention_bf16_d128_i64", b"singe_paged_attention_bf16_d128_i32_p16",
+                   b"singe_paged_kv_prefill_bf16_d128_p16", b"singe_rotary_paged_attention_bf16_d128_i64_p16"):
         assert kernel in image, kernel
 
 
@@ -122,6 +123,25 @@ def test_paged_attention_problem_validation():
     lib.singe_hip_last_error(ctypes.byref(detail))
     assert detail.minimum == 300  # the refused width
     assert call(tokens=0) == 0  # nothing to attend, nothing launched
+
+
+def test_rotary_paged_attention_validation():
+    lib = _native.lib()
+    fake = 0x1000
+    def call(rotation, cos=fake, **changes):
+        fields = dict(tokens=2, heads=2, kv_heads=2, head_dim=128, page_size=4, sequences=1, cache_pages=2, page_table=1,
+                      index_type=1, causal=1, has_scale=0, has_window=0, has_softcap=0, scale=0.0, softcap=0.0, window=0)
+        fields.update(changes)
+        problem = _native.PagedAttentionProblemC(*fields.values())
+        return lib.singe_hip_rotary_paged_attention_bf16(None, *([fake] * 7), cos, fake, None, fake, None, None, ctypes.byref(problem),
+                                                         None if rotation is None else ctypes.byref(rotation))
+    good = _native.QueryRotationC(0, 1, 1e-5)
+    assert call(None) == 6                                       # no rotation attributes
+    assert call(_native.QueryRotationC(7, 0, 0.0)) == 9          # unknown table type
+    assert call(good, head_dim=64) == 5                          # the fused form takes head dimension 128
+    assert call(good, has_softcap=1, softcap=5.0) == 8
+    assert call(good, cos=None) == 6
+    assert call(good, tokens=0) == 0
 
 
 def test_paged_kv_prefill_config_validation_mirrors_reference_cases():
