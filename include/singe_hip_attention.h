@@ -475,6 +475,49 @@ SINGE_HIP_API int32_t singe_hip_splitk_reduce_f32(
     const float* lse_splitk, size_t lse_splitk_len,
     const SingeSplitKReduceConfig* config);
 
+/* ---- latent (MLA) attention over paged caches --------------------------------------------------------
+ * Tensor::paged_mla_attention / Operation::PagedMlaAttention (singe/src/backend/spec/neural/attention.rs:453-497;
+ * CPU singe/src/backend/cpu/normalization/attention.rs:540-679; kernel plan
+ * singe/src/backend/cuda/kernel_plan/source/mla.rs, operands in its ABI order :219-230, status word :260).
+ * Every head of a token attends over one shared latent cache [cache_pages, page_size, latent_dim], whose rows
+ * are the keys, with a positional part [cache_pages, page_size, position_dim] beside them, and the values:
+ * score = (q_latent . c_latent + q_positional . c_positional) * scale, scale = 1 / sqrt(latent_dim +
+ * position_dim) unless given; output [tokens, heads, latent_dim] of the operands' type; lse [tokens, heads] f32
+ * base two, -inf for a row without keys (may be null).  Paging, causal alignment and the status word are those
+ * of singe_hip_paged_attention_*.  All operands contiguous, one element type; latent_dim <= 512 and
+ * position_dim <= 128 (SINGE_HIP_UNSUPPORTED_WIDTH beyond).  A vector-unit kernel, one wave per (token, head)
+ * row: it gives the op on this device, not the matrix-core throughput of the reference's plan. */
+typedef struct SingePagedMlaAttentionProblem {
+    int64_t tokens;
+    int64_t heads;
+    int64_t latent_dim;
+    int64_t position_dim;
+    int64_t page_size;
+    int64_t sequences;
+    int64_t cache_pages;
+    int64_t page_table;    /* entries of `pages` */
+    int32_t data_type;     /* SINGE_HIP_F32, _BF16 or _F16 */
+    int32_t index_type;    /* SINGE_HIP_INDEX_I32 or _I64 */
+    uint8_t causal;
+    uint8_t has_scale;
+    float scale;
+} SingePagedMlaAttentionProblem;
+
+SINGE_HIP_API int32_t singe_hip_paged_mla_attention(
+    void* stream,
+    const void* latent_queries,
+    const void* positional_queries,
+    const void* latent_cache,
+    const void* positional_cache,
+    const void* query_offsets,
+    const void* page_offsets,
+    const void* pages,
+    const void* last_page_lengths,
+    void* output,
+    float* lse,
+    uint32_t* status,
+    const SingePagedMlaAttentionProblem* problem);
+
 /* ---- singe surface: the steps either side of paged attention ------------------------------------------
  * The fused rotate-and-append kernel "rotary_cache_write"
  * (singe/src/backend/cuda/kernel_plan/source/rotary_cache.rs:249-427): rotates query [tokens, query_heads,

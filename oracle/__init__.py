@@ -48,6 +48,7 @@ def lib() -> ctypes.CDLL:
         _lib.oracle_f8e4m3_encode.argtypes = [ctypes.c_double]
         _lib.oracle_check_paged_values.restype = _c_int
         _lib.oracle_paged_attention_f32.restype = _c_int
+        _lib.oracle_paged_mla_attention.restype = _c_int
         _lib.oracle_paged_slots.restype = _c_size
         _lib.oracle_max_threads.restype = _c_int
     return _lib
@@ -282,6 +283,30 @@ def paged_attention_f32(query, key_cache, value_cache, query_offsets, page_offse
         _c_size(kv_heads), _c_size(head_dim), _c_size(page_size), _c_size(cache_pages), _c_float(scale),
         _c_int(bool(causal)), _c_i64(-1 if window is None else int(window)),
         _c_int(softcap is not None), _c_float(softcap if softcap is not None else 0.0), _c_int(threads))
+    return int(status), out, lse
+
+
+def paged_mla_attention(query, query_positions, latent_cache, position_cache, query_offsets, page_offsets, pages,
+                        last_page_lengths, *, scale=None, causal=False, threads=1):
+    """singe/src/backend/cpu/normalization/attention.rs:540-679 (f64 compute).  query [T, H, L], query_positions
+    [T, H, R], latent_cache [P, S, L], position_cache [P, S, R].  Returns (status, out [T, H, L] f32, lse [T, H]
+    base two); status 1 = index out of bounds."""
+    query, query_positions = _f32(query), _f32(query_positions)
+    latent_cache, position_cache = _f32(latent_cache), _f32(position_cache)
+    tokens, heads, latent = query.shape
+    positional = query_positions.shape[2]
+    cache_pages, page_size, _ = latent_cache.shape
+    qo = np.ascontiguousarray(query_offsets, dtype=np.int64)
+    po = np.ascontiguousarray(page_offsets, dtype=np.int64)
+    pg = np.ascontiguousarray(pages, dtype=np.int64)
+    lp = np.ascontiguousarray(last_page_lengths, dtype=np.int64)
+    out = np.zeros((tokens, heads, latent), dtype=np.float32)
+    lse = np.full((tokens, heads), -np.inf, dtype=np.float32)
+    status = lib().oracle_paged_mla_attention(
+        _ptr(out), _ptr(lse), _ptr(query), _ptr(query_positions), _ptr(latent_cache), _ptr(position_cache), _ptr(qo), _ptr(po),
+        _ptr(pg), _ptr(lp), _c_size(len(lp)), _c_size(len(pg)), _c_size(tokens), _c_size(heads), _c_size(latent),
+        _c_size(positional), _c_size(page_size), _c_size(cache_pages), _c_int(scale is not None),
+        _c_float(scale if scale is not None else 0.0), _c_int(bool(causal)), _c_int(threads))
     return int(status), out, lse
 
 

@@ -25,7 +25,7 @@
  *
  * Parity pinning: the reference holds no numeric fixture for
  * paged_kv_decode_attention_f32, paged_kv_prefill_attention_f32,
- * fmha_prefill_lse_f32 or attend_paged, and the Rust original cannot be
+ * fmha_prefill_lse_f32, attend_paged or paged_mla_attention, and the Rust original cannot be
  * compiled in this image, so their last-ulp f32 outputs are pinned only by
  * construction plus closed forms and invariants (see tests/test_oracle.py);
  * everything integer (gather offsets, lengths, the paging error contract),
@@ -613,6 +613,73 @@ ORACLE_API int oracle_paged_attention_f32(
                 for (size_t d = 0; d < head_dim; ++d) o[d] = fmaf(w, v[d], o[d]);
             }
             free(weights);
+        }
+    }
+    return 0;
+}
+
+/* Latent attention over paged caches (singe/src/backend/cpu/normalization/attention.rs:540-679): every head
+ * of a token attends over one shared latent cache [pages, page_size, latent], whose rows are the keys, with a
+ * positional part [pages, page_size, positional] beside them, and the values.  In f64 as the reference
+ * computes it: score = (q_latent . c_latent + q_positional . c_positional) * scale, weights = exp(score -
+ * largest) / total, out = sum weights * c_latent; lse = (largest + ln total) / ln 2 as f32, -inf where a row
+ * sees no key (:648-658).  Queries are the sequence's last tokens (:620-621).  `out` is f64 -> f32 (the caller
+ * rounds to the queries' type as the reference's cast does, :675).  Returns 1 without touching the outputs
+ * when the paging values fail oracle_check_paged_values (:589-594). */
+ORACLE_API int oracle_paged_mla_attention(
+    float *out, float *lse, const float *query, const float *query_positions, const float *latent_cache,
+    const float *position_cache, const int64_t *query_offsets, const int64_t *page_offsets, const int64_t *pages,
+    const int64_t *last_page_lengths, size_t sequences, size_t table, size_t tokens, size_t heads, size_t latent,
+    size_t positional, size_t page_size, size_t cache_pages, int has_scale, float scale_value, int causal, int threads) {
+    if (oracle_check_paged_values(query_offsets, page_offsets, pages, last_page_lengths, sequences,
+                                  (int64_t)table, (int64_t)tokens, (int64_t)cache_pages, (int64_t)page_size))
+        return 1;
+    const double ln2 = 0.693147180559945309417232121458176568; /* std::f64::consts::LN_2 */
+    const double scale = has_scale ? (double)scale_value : 1.0 / sqrt((double)(latent + positional));
+    for (size_t i = 0; i < tokens * heads * latent; ++i) out[i] = 0.0f;
+    for (size_t i = 0; i < tokens * heads; ++i) lse[i] = -INFINITY;
+    for (size_t s = 0; s < sequences; ++s) {
+        size_t first_query = (size_t)query_offsets[s], end_query = (size_t)query_offsets[s + 1];
+        const int64_t *sequence_pages = pages + page_offsets[s];
+        size_t page_count = (size_t)(page_offsets[s + 1] - page_offsets[s]);
+        size_t keys = page_count == 0 ? 0 : (page_count - 1) * page_size + (size_t)last_page_lengths[s];
+        size_t queries = end_query > first_query ? end_query - first_query : 0;
+        long rows = (long)(queries * heads);
+#pragma omp parallel for schedule(dynamic, 4) num_threads(thread_count(threads))
+        for (long row_index = 0; row_index < rows; ++row_index) {
+            size_t token = first_query + (size_t)row_index / heads, head = (size_t)row_index % heads;
+            size_t reach = keys + token - first_query;
+            size_t position = reach > queries ? reach - queries : 0;
+            size_t end = causal ? (keys < position + 1 ? keys : position + 1) : keys;
+            if (end == 0) continue;
+            size_t row = token * heads + head;
+            const float *latent_query = query + row * latent;
+            const float *position_query = query_positions + row * positional;
+            double *scores = (double *)malloc(end * sizeof(double));
+            double largest = -INFINITY;
+            for (size_t key = 0; key < end; ++key) {
+                size_t slot = (size_t)sequence_pages[key / page_size] * page_size + key % page_size;
+                double first = 0.0, second = 0.0;
+                for (size_t d = 0; d < latent; ++d) first += (double)latent_query[d] * (double)latent_cache[slot * latent + d];
+                for (size_t d = 0; d < positional; ++d) second += (double)position_query[d] * (double)position_cache[slot * positional + d];
+                scores[key] = (first + second) * scale;
+                if (scores[key] > largest) largest = scores[key];
+            }
+            double total = 0.0;
+            for (size_t key = 0; key < end; ++key) {
+                scores[key] = exp(scores[key] - largest);
+                total += scores[key];
+            }
+            lse[row] = (float)((largest + log(total)) / ln2);
+            double *sum = (double *)calloc(latent, sizeof(double));
+            for (size_t key = 0; key < end; ++key) {
+                size_t slot = (size_t)sequence_pages[key / page_size] * page_size + key % page_size;
+                double weight = scores[key] / total;
+                for (size_t d = 0; d < latent; ++d) sum[d] += weight * (double)latent_cache[slot * latent + d];
+            }
+            for (size_t d = 0; d < latent; ++d) out[row * latent + d] = (float)sum[d];
+            free(sum);
+            free(scores);
         }
     }
     return 0;

@@ -70,6 +70,14 @@ class SplitKReduceConfigC(ctypes.Structure):
         "lse_batch_stride", "lse_head_stride", "output_batch_stride", "output_head_stride")]
 
 
+class PagedMlaAttentionProblemC(ctypes.Structure):
+    _fields_ = [("tokens", ctypes.c_int64), ("heads", ctypes.c_int64), ("latent_dim", ctypes.c_int64),
+                ("position_dim", ctypes.c_int64), ("page_size", ctypes.c_int64), ("sequences", ctypes.c_int64),
+                ("cache_pages", ctypes.c_int64), ("page_table", ctypes.c_int64), ("data_type", ctypes.c_int32),
+                ("index_type", ctypes.c_int32), ("causal", ctypes.c_uint8), ("has_scale", ctypes.c_uint8),
+                ("scale", ctypes.c_float)]
+
+
 class QueryRotationC(ctypes.Structure):
     _fields_ = [("table_type", ctypes.c_int32), ("has_norm", ctypes.c_uint8), ("eps", ctypes.c_float)]
 
@@ -168,6 +176,8 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_rotary_paged_attention_bf16.argtypes = [c_void] * 14 + [ctypes.POINTER(PagedAttentionProblemC),
                                                                              ctypes.POINTER(QueryRotationC)]
     handle.singe_hip_rotary_paged_attention_bf16.restype = i32
+    handle.singe_hip_paged_mla_attention.argtypes = [c_void] * 12 + [ctypes.POINTER(PagedMlaAttentionProblemC)]
+    handle.singe_hip_paged_mla_attention.restype = i32
     handle.singe_hip_paged_attention_f32.argtypes = [c_void] * 11 + [ctypes.POINTER(PagedAttentionProblemC)]
     handle.singe_hip_paged_attention_f32.restype = i32
     handle.singe_hip_paged_attention_f16.argtypes = [c_void] * 11 + [ctypes.POINTER(PagedAttentionProblemC)]

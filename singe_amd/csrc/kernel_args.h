@@ -171,6 +171,25 @@ struct GeneralPagedArgs {
     float scale, softcap;
 };
 
+// singe_paged_mla_attention_general_*: contiguous operands of one element type.
+struct LatentAttentionArgs {
+    const void* latent_queries;      // [tokens, heads, latent_dim]
+    const void* positional_queries;  // [tokens, heads, position_dim]
+    const void* latent_cache;        // [cache_pages, page_size, latent_dim]
+    const void* positional_cache;    // [cache_pages, page_size, position_dim]
+    const void* query_offsets;
+    const void* page_offsets;
+    const void* pages;
+    const void* last_page_lengths;
+    void* output;                    // [tokens, heads, latent_dim]
+    float* lse;                      // [tokens, heads] base two, or null
+    uint32_t* status;
+    uint32_t tokens, heads, latent_dim, position_dim, page_size, sequences, cache_pages, page_table;
+    uint32_t row_blocks;             // workgroups (4 rows each) per sequence
+    uint32_t causal, wide_index;
+    float scale;
+};
+
 // singe_rotary_cache_write_*: contiguous operands of one element type; angles may be f32.
 struct RotaryCacheArgs {
     const void* query;          // [tokens, query_heads, dim] or null when query_heads is 0

@@ -25,6 +25,8 @@ enum KernelId : int {
     kSplitKReduce,
     kRotaryCacheF32, kRotaryCacheBf16, kRotaryCacheF16,
     kPagingIndicesI32, kPagingIndicesI64,
+    // latent (MLA) attention: + element (f32, bf16, f16)
+    kLatentGeneral, kLatentGeneralBf16, kLatentGeneralF16,
     // general kernels: index = base + 3 * element (f32, bf16, f16) + width (64, 128, 256)
     kDenseGeneral,
     kPagedGeneral = kDenseGeneral + 9,

@@ -6,4 +6,5 @@
 #include "paged_attention.hip"
 #include "splitk_reduce.hip"
 #include "general_attention.hip"
+#include "latent_attention.hip"
 #include "cache_ops.hip"

@@ -184,6 +184,57 @@ def paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: t
     return output, lse
 
 
+def paged_mla_attention(query: torch.Tensor, query_positions: torch.Tensor, latent_cache: torch.Tensor,
+                        position_cache: torch.Tensor, paging: Paging, options: AttentionOptions = AttentionOptions(), *,
+                        stream=None, status: torch.Tensor | None = None, check: bool = True):
+    """Tensor::paged_mla_attention (singe/src/backend/spec/neural/attention.rs:453-497, CPU
+    normalization/attention.rs:540-679): latent attention over paged caches.  ``query`` [tokens, heads, latent],
+    ``query_positions`` [tokens, heads, positional], ``latent_cache`` [pages, page_size, latent], ``position_cache``
+    [pages, page_size, positional], f32 / bf16 / f16.  Only ``causal`` and ``scale`` of the options apply.  Returns
+    (output [tokens, heads, latent] of the query's type, lse [tokens, heads] f32 base two)."""
+    if options.window is not None or options.softcap is not None:
+        raise error.InvalidArgument("paged mla attention takes a scale and a causal mask only")
+    operands = ((query, "query"), (query_positions, "query_positions"), (latent_cache, "latent_cache"), (position_cache, "position_cache"))
+    for tensor, name in operands:
+        if not tensor.is_cuda or tensor.dtype != query.dtype or not tensor.is_contiguous() or tensor.dim() != 3:
+            raise error.InvalidArgument(f"paged mla attention {name} must be a contiguous rank-3 device tensor of the query's type")
+    if query.dtype not in _DATA_TYPES:
+        raise error.InvalidArgument(f"paged mla attention data type {query.dtype}")
+    tokens, heads, latent = query.shape
+    pages, page_size, cached_latent = latent_cache.shape
+    positional = query_positions.shape[2]
+    if (tuple(query_positions.shape[:2]) != (tokens, heads) or tuple(position_cache.shape[:2]) != (pages, page_size)
+            or cached_latent != latent or position_cache.shape[2] != positional or page_size <= 0 or latent <= 0):
+        raise error.InvalidArgument("paged mla attention query or cache shapes")
+    indices = (paging.query_offsets, paging.page_offsets, paging.pages, paging.last_page_lengths)
+    kinds = {t.dtype for t in indices}
+    if len(kinds) != 1 or not kinds <= {torch.int32, torch.int64}:
+        raise error.InvalidArgument("paging index tensors must share one integer type")
+    for tensor in indices:
+        if not tensor.is_cuda or not tensor.is_contiguous():
+            raise error.InvalidArgument("paged attention index tensors must be contiguous device tensors")
+    sequences = paging.last_page_lengths.numel()
+    if paging.query_offsets.numel() != sequences + 1 or paging.page_offsets.numel() != sequences + 1:
+        raise error.InvalidArgument("paging offsets must hold one more entry than there are sequences")
+    problem = _native.PagedMlaAttentionProblemC(
+        tokens, heads, latent, positional, page_size, sequences, pages, paging.pages.numel(), _DATA_TYPES[query.dtype],
+        1 if paging.pages.dtype == torch.int64 else 0, 1 if options.causal else 0, 1 if options.scale is not None else 0,
+        options.scale if options.scale is not None else 0.0)
+    output = torch.zeros_like(query)
+    lse = torch.full((tokens, heads), float("-inf"), device=query.device, dtype=torch.float32)
+    if status is None:
+        status = torch.zeros(1, device=query.device, dtype=torch.int32)
+    handle = int((stream or torch.cuda.current_stream()).cuda_stream)
+    code = _native.lib().singe_hip_paged_mla_attention(
+        handle, query.data_ptr(), query_positions.data_ptr(), latent_cache.data_ptr(), position_cache.data_ptr(),
+        paging.query_offsets.data_ptr(), paging.page_offsets.data_ptr(), paging.pages.data_ptr(), paging.last_page_lengths.data_ptr(),
+        output.data_ptr(), lse.data_ptr(), status.data_ptr(), ctypes.byref(problem))
+    _native.check(code, "paged_mla_attention")
+    if check and int(status.item()) == STATUS_INDEX_OUT_OF_BOUNDS:
+        raise error.IndexOutOfBounds("paged mla attention paging value outside its buffers")
+    return output, lse
+
+
 def rotary_paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor, paging: Paging,
                            cos: torch.Tensor, sin: torch.Tensor, options: AttentionOptions = AttentionOptions(), *,
                            query_norm: "RotationNorm | None" = None, stream=None, status: torch.Tensor | None = None,

@@ -144,6 +144,22 @@ def test_rotary_paged_attention_validation():
     assert call(good, tokens=0) == 0
 
 
+def test_paged_mla_attention_validation():
+    lib = _native.lib()
+    fake = 0x1000
+    def call(**changes):
+        fields = dict(tokens=2, heads=2, latent_dim=32, position_dim=8, page_size=4, sequences=1, cache_pages=2, page_table=1,
+                      data_type=1, index_type=0, causal=1, has_scale=0, scale=0.0)
+        fields.update(changes)
+        problem = _native.PagedMlaAttentionProblemC(*fields.values())
+        return lib.singe_hip_paged_mla_attention(None, *([fake] * 9), None, None, ctypes.byref(problem))
+    assert call(page_size=0) == 9 and call(latent_dim=0) == 9      # paged_mla_attention_problem's own refusals
+    assert call(data_type=4) == 9 and call(index_type=3) == 9
+    assert call(has_scale=1, scale=float("nan")) == 9
+    assert call(latent_dim=576) == 5 and call(position_dim=160) == 5
+    assert call(tokens=0) == 0
+
+
 def test_paged_kv_prefill_config_validation_mirrors_reference_cases():
     """singe-kernel/src/cuda/attention/tests.rs:349-375."""
     lib = _native.lib()

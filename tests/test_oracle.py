@@ -593,3 +593,45 @@ def test_paging_indices_against_brute_force():
     # the reference's invalid tuples are refused here too
     assert oracle.paging_indices([0, 1, 3], [0, 2, 3], [1, 0, 3], [2, 1], tokens=3, page_size=4, cache_pages=3, width=2, row_elements=1)[0] == 1
     assert oracle.paging_indices([0, 2, 1], [0, 2, 3], [1, 0, 2], [2, 1], tokens=3, page_size=4, cache_pages=3, width=2, row_elements=1)[0] == 1
+
+
+def test_paged_mla_attention_against_a_float64_restatement_and_closed_forms():
+    """The latent-attention oracle has no numeric fixture in the reference: it is pinned by an independent numpy
+    float64 restatement (a dropped positional term, a wrong slot or a wrong causal end fails it), by single-key rows
+    (out == that latent row, lse == score / ln 2) and by the paging error contract."""
+    gen = np.random.default_rng(5)
+    tokens, heads, latent, positional, pages, slots = 7, 3, 24, 8, 9, 4
+    q = gen.standard_normal((tokens, heads, latent)).astype(np.float32)
+    qp = gen.standard_normal((tokens, heads, positional)).astype(np.float32)
+    lc = gen.standard_normal((pages, slots, latent)).astype(np.float32)
+    pc = gen.standard_normal((pages, slots, positional)).astype(np.float32)
+    qo, po, table, last = [0, 3, 4, 7], [0, 3, 3, 7], [8, 0, 3, 5, 1, 2, 6], [2, 0, 1]
+    for causal in (False, True):
+        status, out, lse = oracle.paged_mla_attention(q, qp, lc, pc, qo, po, table, last, causal=causal, scale=None if causal else 0.3)
+        assert status == 0
+        scale = 1.0 / np.sqrt(latent + positional) if causal else 0.3
+        for s in range(3):
+            own = table[po[s]:po[s + 1]]
+            keys = 0 if not own else (len(own) - 1) * slots + last[s]
+            rows = np.concatenate([lc[p] for p in own])[:keys].astype(np.float64) if own else np.zeros((0, latent))
+            tails = np.concatenate([pc[p] for p in own])[:keys].astype(np.float64) if own else np.zeros((0, positional))
+            count = qo[s + 1] - qo[s]
+            for t in range(qo[s], qo[s + 1]):
+                position = max(keys + (t - qo[s]) - count, 0)
+                end = min(keys, position + 1) if causal else keys
+                for h in range(heads):
+                    if end == 0:
+                        assert not out[t, h].any() and np.isneginf(lse[t, h])
+                        continue
+                    scores = (rows[:end] @ q[t, h].astype(np.float64) + tails[:end] @ qp[t, h].astype(np.float64)) * scale
+                    weights = np.exp(scores - scores.max())
+                    assert np.allclose(out[t, h], (weights / weights.sum()) @ rows[:end], atol=2e-6)
+                    assert abs(lse[t, h] - (scores.max() + np.log(weights.sum())) / np.log(2.0)) < 1e-5
+    # A single key: the output is its latent row, the LSE its score in base two.
+    status, out, lse = oracle.paged_mla_attention(q[:1], qp[:1], lc, pc, [0, 1], [0, 1], [4], [1], scale=0.5)
+    assert status == 0 and np.array_equal(out[0, 0], lc[4, 0])
+    score = (np.dot(q[0, 0].astype(np.float64), lc[4, 0]) + np.dot(qp[0, 0].astype(np.float64), pc[4, 0])) * 0.5
+    assert abs(lse[0, 0] - score / np.log(2.0)) < 1e-5
+    # The paging error contract is the op's (spec/neural/attention.rs:372-406).
+    assert oracle.paged_mla_attention(q[:1], qp[:1], lc, pc, [0, 1], [0, 1], [pages], [1])[0] == 1
+    assert oracle.paged_mla_attention(q[:1], qp[:1], lc, pc, [0, 2], [0, 1], [0], [1])[0] == 1

@@ -1,0 +1,112 @@
+"""Latent (MLA) attention over paged caches on the GPU against the CPU oracle (paged_mla_attention restated, f64),
+through the C ABI.  Inputs, shapes and tolerances are those of the reference's own device-against-CPU test
+(singe/src/backend/cuda/kernel_plan/source/tests.rs:1191-1316): values ((index * 37 + seed * 11) % 41) / 40 - 0.5,
+scale 0.07, output within 0.02 (bf16) / 0.003 (f16), LSE within 1e-3 relative; f32 within 1e-4 here."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from singe_amd import error, neural
+
+pytestmark = pytest.mark.gpu
+
+
+def values(shape, seed):
+    count = int(np.prod(shape))
+    index = np.arange(count, dtype=np.int64)
+    return (((index * 37 + seed * 11) % 41).astype(np.float32) / 40.0 - 0.5).reshape(shape)
+
+
+BATCHES = [
+    [(1, 150), (9, 9), (5, 70), (2, 0)],   # decode over a long cache, a whole prefill, a chunk, a sequence with no keys
+    [(1, 2000), (2, 1500)],                # few long sequences
+    [(1, 300), (1, 40), (1, 0)],           # decoding alone
+]
+TOLERANCE = {torch.bfloat16: 0.02, torch.float16: 0.003, torch.float32: 1e-4}
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("heads,latent,positional,page_size", [(16, 512, 64, 1), (8, 128, 32, 5)])
+@pytest.mark.parametrize("sequences", BATCHES)
+def test_matches_the_cpu_over_ragged_sequences(sequences, heads, latent, positional, page_size, causal, dtype):
+    query_offsets, page_offsets, last, needed = [0], [0], [], 0
+    for queries, keys in sequences:
+        query_offsets.append(query_offsets[-1] + queries)
+        pages = (keys + page_size - 1) // page_size
+        needed += pages
+        page_offsets.append(needed)
+        last.append(0 if keys == 0 else keys - (pages - 1) * page_size)
+    page_count = needed + 3
+    table = [(page * 7 + 2) % page_count for page in range(needed)]
+    tokens = query_offsets[-1]
+    host = [values((tokens, heads, latent), 1), values((tokens, heads, positional), 2), values((page_count, page_size, latent), 3),
+            values((page_count, page_size, positional), 4)]
+    device = [torch.tensor(array).to(dtype).cuda() for array in host]
+    rounded = [tensor.float().cpu().numpy() for tensor in device]
+    index = lambda entries: torch.tensor(entries, dtype=torch.int32, device="cuda")
+    paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
+    out, lse = neural.paged_mla_attention(*device, paging, neural.AttentionOptions(causal=causal, scale=0.07))
+    torch.cuda.synchronize()
+    status, want, want_lse = oracle.paged_mla_attention(*rounded, query_offsets, page_offsets, table, last, scale=0.07, causal=causal,
+                                                        threads=8)
+    assert status == 0
+    got, got_lse = out.float().cpu().numpy(), lse.cpu().numpy()
+    assert np.abs(got - want).max() <= TOLERANCE[dtype]
+    empty = np.isneginf(want_lse)
+    assert np.array_equal(np.isneginf(got_lse), empty) and not got[empty].any()
+    assert (np.abs(got_lse[~empty] - want_lse[~empty]) <= 1e-3 * np.maximum(np.abs(want_lse[~empty]), 1.0)).all()
+
+
+def test_default_scale_counts_the_whole_key_width_and_int64_indices():
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(1)
+    rand = lambda *shape: torch.randn(shape, generator=gen, device="cuda").to(torch.bfloat16)
+    q, qp, lc, pc = rand(7, 4, 192), rand(7, 4, 24), rand(9, 4, 192), rand(9, 4, 24)
+    index = lambda entries: torch.tensor(entries, dtype=torch.int64, device="cuda")
+    qo, po, table, last = [0, 3, 7], [0, 4, 7], [8, 0, 3, 5, 1, 2, 6], [2, 4]
+    out, lse = neural.paged_mla_attention(q, qp, lc, pc, neural.Paging(index(qo), index(po), index(table), index(last)),
+                                          neural.AttentionOptions(causal=True))
+    host = lambda tensor: tensor.float().cpu().numpy()
+    status, want, want_lse = oracle.paged_mla_attention(host(q), host(qp), host(lc), host(pc), qo, po, table, last, causal=True)
+    assert status == 0
+    assert np.abs(host(out) - want).max() <= 0.02 and np.abs(lse.cpu().numpy() - want_lse).max() <= 2e-3
+
+
+TOKENS, HEADS, LATENT, POSITIONAL, SLOTS, PAGES = 2, 2, 32, 8, 4, 2
+VALID = dict(query_offsets=[0, 2], page_offsets=[0, 1], pages=[0], last_page_lengths=[2])
+INVALID = [dict(query_offsets=[0, 3]), dict(query_offsets=[-1, 2]), dict(query_offsets=[2, 0]), dict(page_offsets=[0, 2]),
+           dict(page_offsets=[-1, 1]), dict(pages=[PAGES]), dict(pages=[-1]), dict(last_page_lengths=[SLOTS + 1]),
+           dict(last_page_lengths=[-1])]
+
+
+def attend_mla(paging_values, dtype):
+    # singe/tests/nn/paged_attention.rs:127-161
+    q = torch.zeros((TOKENS, HEADS, LATENT), device="cuda", dtype=torch.bfloat16)
+    qp = torch.zeros((TOKENS, HEADS, POSITIONAL), device="cuda", dtype=torch.bfloat16)
+    lc = torch.zeros((PAGES, SLOTS, LATENT), device="cuda", dtype=torch.bfloat16)
+    pc = torch.zeros((PAGES, SLOTS, POSITIONAL), device="cuda", dtype=torch.bfloat16)
+    entries = {**VALID, **paging_values}
+    index = lambda v: torch.tensor(v, dtype=dtype, device="cuda")
+    paging = neural.Paging(index(entries["query_offsets"]), index(entries["page_offsets"]), index(entries["pages"]),
+                           index(entries["last_page_lengths"]))
+    return neural.paged_mla_attention(q, qp, lc, pc, paging, neural.AttentionOptions(causal=True))
+
+
+@pytest.mark.parametrize("dtype", [torch.int32, torch.int64])
+def test_paging_values_outside_their_buffers_are_refused(dtype):
+    attend_mla({}, dtype)
+    for bad in INVALID:
+        with pytest.raises(error.IndexOutOfBounds):
+            attend_mla(bad, dtype)
+
+
+def test_shapes_the_op_does_not_take():
+    zeros = lambda *shape: torch.zeros(shape, device="cuda", dtype=torch.bfloat16)
+    index = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
+    paging = neural.Paging(index([0, 2]), index([0, 1]), index([0]), index([2]))
+    with pytest.raises(error.InvalidArgument):   # positional cache of another width
+        neural.paged_mla_attention(zeros(2, 2, 32), zeros(2, 2, 8), zeros(2, 4, 32), zeros(2, 4, 16), paging)
+    with pytest.raises(error.UnsupportedWidth):  # beyond the widths this kernel holds
+        neural.paged_mla_attention(zeros(2, 2, 576), zeros(2, 2, 8), zeros(2, 4, 576), zeros(2, 4, 8), paging)
