@@ -336,6 +336,35 @@ SINGE_HIP_API int32_t singe_hip_paged_attention_bf16(
     uint32_t* status,
     const SingePagedAttentionProblem* problem);
 
+/* The same op with scratch for key splits.  With few query rows (decoding, short chunks) one workgroup per
+ * (sequence, kv head, 128 packed rows) cannot fill the chip and the longest sequence sets the time; given
+ * scratch, the keys of a row tile are shared out over several workgroups, each leaving a normalised f32
+ * partial and its log-sum-exp, and a second kernel merges them (the scheme of the reference's own split
+ * kernels, which declare such scratch in their plan: kernel_plan/source/mla.rs:232-241, 497-560).
+ * singe_hip_paged_attention_scratch_bytes says how much this problem wants (0: it would not split);
+ * with a null or smaller buffer the call runs unsplit, exactly as singe_hip_paged_attention_bf16.  The scratch
+ * holds nothing between calls; calls that share it must not overlap.  Results equal the unsplit ones up to
+ * the order of summation.  singe_hip_set_paged_attention_splits fixes the number of shares (0 = chosen by
+ * problem size, the default), the counterpart of TuningChoice::Explicit
+ * (singe-kernel/src/cuda/attention/mod.rs:2364-2380); it changes what ..._scratch_bytes returns. */
+SINGE_HIP_API size_t singe_hip_paged_attention_scratch_bytes(const SingePagedAttentionProblem* problem);
+SINGE_HIP_API void singe_hip_set_paged_attention_splits(uint32_t splits);
+SINGE_HIP_API int32_t singe_hip_paged_attention_scratch_bf16(
+    void* stream,
+    const uint16_t* query_rows,
+    const uint16_t* key_cache,
+    const uint16_t* value_cache,
+    const void* query_offsets,
+    const void* page_offsets,
+    const void* pages,
+    const void* last_page_lengths,
+    uint16_t* output,
+    float* lse,
+    uint32_t* status,
+    void* scratch,
+    size_t scratch_bytes,
+    const SingePagedAttentionProblem* problem);
+
 /* The same op over a query the kernel normalises and rotates itself, the counterpart of
  * KernelPlanner::rotary_paged_attention (singe/src/backend/cuda/kernel_plan/source/paged_attention.rs:533-542,
  * query stage :881-977; operand order :687-715: the attention's inputs, the output, then cos, sin and the

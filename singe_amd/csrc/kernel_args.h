@@ -112,6 +112,11 @@ struct PagedAttentionArgs {
     float scale_log2e;              // scale * log2(e)
     float softcap_scale;            // scale / cap
     float softcap_log2e;            // cap * log2(e)
+    // Key splits (1 = none): workgroup (unit, row tile, split) folds its share of the tiles and leaves a
+    // normalised f32 partial and its base-two log-sum-exp for singe_paged_attention_combine_bf16.
+    uint32_t splits = 1;
+    float* partial_out = nullptr;   // [splits, tokens * heads, 128]
+    float* partial_lse = nullptr;   // [splits, tokens * heads]
     // Kernels that rotate their query themselves (rotary_paged_attention):
     const void* cos = nullptr;                // [tokens, 64] of table_type
     const void* sin = nullptr;

@@ -20,6 +20,7 @@ enum KernelId : int {
     kPagedAttentionI32, kPagedAttentionI64, kPagedAttentionSoftcapI32, kPagedAttentionSoftcapI64,
     kPagedAttentionI32P16, kPagedAttentionI64P16, kPagedAttentionSoftcapI32P16, kPagedAttentionSoftcapI64P16,
     kPagedKvPrefill, kPagedKvPrefillP16,
+    kPagedAttentionCombineI32, kPagedAttentionCombineI64,
     // fused query rotation: + (i64 indices) + 2 * (page size a power of two of at least 16 keys)
     kRotaryPagedAttention, kRotaryPagedAttentionI64, kRotaryPagedAttentionP16, kRotaryPagedAttentionI64P16,
     kSplitKReduce,

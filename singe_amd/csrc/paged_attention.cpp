@@ -28,10 +28,39 @@ struct Rotation {
     const SingeQueryRotation* attributes;
 };
 
+// Scratch for key splits: what singe_hip_paged_attention_scratch_bytes asked for, or nothing.
+struct Scratch {
+    void* memory;
+    size_t bytes;
+};
+
+// 0 = chosen by problem size (singe_hip_set_paged_attention_splits).
+uint32_t g_paged_attention_splits = 0;
+
+// Key splits for a problem: enough workgroups to fill the compute units four times over, when the query rows
+// alone do not (decoding, short chunks); one (no split) for other element types and head dimensions.
+uint32_t paged_attention_splits(const SingePagedAttentionProblem& p) {
+    if (p.head_dim != 128 || p.tokens <= 0 || p.sequences <= 0 || p.kv_heads <= 0 || p.heads <= 0) return 1;
+    if (g_paged_attention_splits != 0) return g_paged_attention_splits;
+    const uint64_t groups = static_cast<uint64_t>(p.heads / p.kv_heads);
+    const uint64_t row_tiles = (groups * static_cast<uint64_t>(p.tokens) + 127) / 128;
+    const uint64_t workgroups = static_cast<uint64_t>(p.sequences) * p.kv_heads * row_tiles;
+    const uint64_t wanted = 4ull * compute_units();
+    if (workgroups >= wanted) return 1;
+    const uint64_t splits = wanted / workgroups;
+    return static_cast<uint32_t>(splits > 16 ? 16 : splits < 1 ? 1 : splits);
+}
+
+size_t scratch_bytes_for(const SingePagedAttentionProblem& p, uint32_t splits) {
+    if (splits <= 1) return 0;
+    return static_cast<size_t>(splits) * static_cast<size_t>(p.tokens) * static_cast<size_t>(p.heads) * (128 + 1) * sizeof(float);
+}
+
 int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_any, const void* key_cache_any,
                         const void* value_cache_any, const void* query_offsets, const void* page_offsets, const void* pages,
                         const void* last_page_lengths, void* output_any, float* lse, uint32_t* status,
-                        const SingePagedAttentionProblem* problem, const Rotation* rotation = nullptr) {
+                        const SingePagedAttentionProblem* problem, const Rotation* rotation = nullptr,
+                        const Scratch* scratch = nullptr) {
     if (problem == nullptr) return fail(SINGE_HIP_NULL_POINTER, "problem");
     const SingePagedAttentionProblem& p = *problem;
     if (rotation != nullptr) {
@@ -115,6 +144,21 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
     const uint64_t blocks = units * args.row_tiles;
     if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
     const bool wide = p.index_type == SINGE_HIP_INDEX_I64;
+    // Key splits, when the caller lent scratch for them: the attention kernel leaves partials, a second
+    // kernel merges them.  Without scratch (or with too little) the keys of a row tile stay in one workgroup.
+    uint32_t splits = scratch != nullptr && scratch->memory != nullptr ? paged_attention_splits(p) : 1;
+    if (splits > 1 && scratch->bytes < scratch_bytes_for(p, splits)) splits = 1;
+    if (splits > 1 && blocks * splits > 0x7fffffffull) splits = 1;
+    args.splits = splits;
+    if (splits > 1) {
+        args.partial_out = static_cast<float*>(scratch->memory);
+        args.partial_lse = args.partial_out + static_cast<size_t>(splits) * p.tokens * p.heads * 128;
+    }
+    const unsigned grid = static_cast<unsigned>(blocks * splits);
+    auto finish = [&](int32_t launched) -> int32_t {
+        if (launched != 0 || splits == 1) return launched;
+        return launch(wide ? kPagedAttentionCombineI64 : kPagedAttentionCombineI32, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+    };
     if (rotation != nullptr) {
         args.cos = rotation->cos;
         args.sin = rotation->sin;
@@ -123,15 +167,33 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
         args.has_query_norm = rotation->attributes->has_norm ? 1u : 0u;
         args.query_eps = rotation->attributes->eps;
         const int rotary = kRotaryPagedAttention + (wide ? 1 : 0) + (args.page_shift >= 4 ? 2 : 0);
-        return launch(static_cast<KernelId>(rotary), static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+        return finish(launch(static_cast<KernelId>(rotary), grid, 1, 1, 256, stream, args));
     }
     const int kernel = (p.has_softcap ? (wide ? kPagedAttentionSoftcapI64 : kPagedAttentionSoftcapI32)
                                       : (wide ? kPagedAttentionI64 : kPagedAttentionI32)) +
                        (args.page_shift >= 4 ? 4 : 0);
-    return launch(static_cast<KernelId>(kernel), static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+    return finish(launch(static_cast<KernelId>(kernel), grid, 1, 1, 256, stream, args));
 }
 
 }  // namespace
+
+extern "C" void singe_hip_set_paged_attention_splits(uint32_t splits) { g_paged_attention_splits = splits > 64 ? 64 : splits; }
+
+extern "C" size_t singe_hip_paged_attention_scratch_bytes(const SingePagedAttentionProblem* problem) {
+    if (problem == nullptr) return 0;
+    return scratch_bytes_for(*problem, paged_attention_splits(*problem));
+}
+
+extern "C" int32_t singe_hip_paged_attention_scratch_bf16(void* stream, const uint16_t* query_rows, const uint16_t* key_cache,
+                                                          const uint16_t* value_cache, const void* query_offsets,
+                                                          const void* page_offsets, const void* pages,
+                                                          const void* last_page_lengths, uint16_t* output, float* lse,
+                                                          uint32_t* status, void* scratch, size_t scratch_bytes,
+                                                          const SingePagedAttentionProblem* problem) {
+    const Scratch lent = {scratch, scratch_bytes};
+    return paged_attention(SINGE_HIP_BF16, stream, query_rows, key_cache, value_cache, query_offsets, page_offsets, pages,
+                           last_page_lengths, output, lse, status, problem, nullptr, &lent);
+}
 
 extern "C" int32_t singe_hip_rotary_paged_attention_bf16(void* stream, const uint16_t* query_rows, const uint16_t* key_cache,
                                                          const uint16_t* value_cache, const void* query_offsets,

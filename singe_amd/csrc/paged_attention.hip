@@ -46,22 +46,21 @@ SINGE_DEVICE float table_value(const void* table, uint32_t table_type, size_t at
 
 constexpr unsigned int kNoPage = 0xFFFFFFFFu;  // a table entry outside the cache: reported, never read through
 
-template <bool SOFTCAP, int FORM, bool GROUPED, bool ROTATE = false>
-SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned char* lds) {
-    const unsigned int tid = threadIdx.x, lane = tid & 63;
-    const unsigned int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and known to be
-    const unsigned int column = lane & 31, hi = lane >> 5;
-    const unsigned int groups = a.heads / a.kv_heads;
-
-    // Workgroup i runs on XCD i % 8: the row tiles of one (sequence, kv head) share an XCD and its L2.
-    // Within an XCD the order is band by band of 32 row tiles: every unit's tiles 0 .. 31 (a unit's side by
-    // side, walking its keys together), then every unit's tiles 32 .. 63, and so on, so the workgroups past
-    // a sequence's rows, which return at once, mostly come after those with work instead of between them.
+// Workgroup id -> (unit = sequence * kv_heads + kv head, row tile, key split); false for ids past the units.
+// Workgroup i runs on XCD i % 8: the row tiles of one (sequence, kv head) share an XCD and its L2.  Within an XCD
+// the order is band by band of 32 row tiles: every unit's tiles 0 .. 31 (a unit's side by side, walking its
+// keys together), then every unit's tiles 32 .. 63, and so on, so the workgroups past a sequence's rows,
+// which return at once, mostly come after those with work instead of between them.  The splits of one
+// (unit, row tile) are neighbours.
+SINGE_DEVICE bool locate(const PagedAttentionArgs& a, unsigned int& unit, unsigned int& row_tile, unsigned int& split) {
     constexpr unsigned int kBand = 32;
-    const unsigned int xcd = blockIdx.x & 7u, within = blockIdx.x >> 3;
+    const unsigned int xcd = blockIdx.x & 7u;
+    unsigned int within = blockIdx.x >> 3;
+    split = within % a.splits;
+    within /= a.splits;
     const unsigned int units_per_xcd = (a.sequences * a.kv_heads + 7u) / 8u;
     const unsigned int full_bands = a.row_tiles / kBand, band = within / (units_per_xcd * kBand);
-    unsigned int local_unit, row_tile;
+    unsigned int local_unit;
     if (band < full_bands) {
         const unsigned int rest = within % (units_per_xcd * kBand);
         local_unit = rest / kBand;
@@ -71,8 +70,19 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         local_unit = rest / tail;
         row_tile = full_bands * kBand + rest % tail;
     }
-    const unsigned int unit = local_unit * 8u + xcd;
-    if (unit >= a.sequences * a.kv_heads) return;
+    unit = local_unit * 8u + xcd;
+    return unit < a.sequences * a.kv_heads;
+}
+
+template <bool SOFTCAP, int FORM, bool GROUPED, bool ROTATE = false>
+SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned char* lds) {
+    const unsigned int tid = threadIdx.x, lane = tid & 63;
+    const unsigned int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and known to be
+    const unsigned int column = lane & 31, hi = lane >> 5;
+    const unsigned int groups = a.heads / a.kv_heads;
+
+    unsigned int unit, row_tile, split;
+    if (!locate(a, unit, row_tile, split)) return;
     const unsigned int sequence = unit / a.kv_heads, kv_head = unit % a.kv_heads;
     const unsigned int first_row = row_tile * kQueryTile;
 
@@ -122,8 +132,15 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         const unsigned int low = position_of(first_row) + 1u;  // keys below low - window are hidden from every row
         first_tile = low > window ? (low - window) / kKeyTile : 0u;
     }
+    unsigned int tiles = (key_end + kKeyTile - 1) / kKeyTile;
+    if (a.splits > 1) {
+        // This workgroup's share of the tiles; a share may be empty.
+        const unsigned int share = tiles > first_tile ? (tiles - first_tile + a.splits - 1) / a.splits : 0u;
+        first_tile += split * share;
+        tiles = tiles < first_tile + share ? tiles : first_tile + share;
+    }
     first_tile = __builtin_amdgcn_readfirstlane(first_tile);
-    const unsigned int tiles = __builtin_amdgcn_readfirstlane((key_end + kKeyTile - 1) / kKeyTile);
+    tiles = __builtin_amdgcn_readfirstlane(tiles);
     unsigned int wave_blocks = 0;
     if (wave_live) {
         wave_blocks = (key_end + 31u) / 32u;
@@ -131,6 +148,7 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
             const unsigned int seen = wave_high / 32u + 1u;
             wave_blocks = wave_blocks < seen ? wave_blocks : seen;
         }
+        wave_blocks = wave_blocks < 2u * tiles ? wave_blocks : 2u * tiles;  // a share ends with its last tile
     }
     wave_blocks = __builtin_amdgcn_readfirstlane(wave_blocks);
 
@@ -406,7 +424,19 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     // (paged_attention.rs:811-821, attention.rs:503-515).
     const float sum = swap32_sum(state.running_sum);
     const float inverse = sum > 0.0f ? 1.0f / sum : 0.0f;
-    if (row_valid) {
+    if (row_valid && a.splits > 1) {
+        const size_t flat = (static_cast<size_t>(query_start) + my_token) * a.heads + kv_head * groups + my_head;
+        const size_t slot = static_cast<size_t>(split) * a.tokens * a.heads + flat;
+        float* row = a.partial_out + slot * kHeadDim;
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int quad = 0; quad < 4; ++quad)
+                *reinterpret_cast<float4*>(row + 32 * db + 8 * quad + 4 * hi) =
+                    make_float4(state.out[db][4 * quad + 0] * inverse, state.out[db][4 * quad + 1] * inverse,
+                                state.out[db][4 * quad + 2] * inverse, state.out[db][4 * quad + 3] * inverse);
+        if (hi == 0) a.partial_lse[slot] = sum > 0.0f ? state.reference + fast_log2(sum) : -INFINITY;
+    } else if (row_valid) {
         const size_t flat = (static_cast<size_t>(query_start) + my_token) * a.heads + kv_head * groups + my_head;
         uint16_t* row = a.output + flat * kHeadDim;
 #pragma unroll
@@ -428,7 +458,73 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     }
 }
 
+// Merges the key splits of every row of a (unit, row tile): each share's output weighs 2^(lse - largest) over
+// the sum of those (the merge of the reference's own split kernels, kernel_plan/source/mla.rs:497-560), the row's
+// log-sum-exp is largest + log2 of that sum.  One thread per (row, 64 dims); launched with splits = 1 so the
+// workgroup ids map as in the attention kernel, the number of shares in `shares`.
+template <int FORM>
+SINGE_DEVICE void combine_body(const PagedAttentionArgs& a, unsigned int shares) {
+    unsigned int unit, row_tile, split;
+    if (!locate(a, unit, row_tile, split)) return;
+    const unsigned int sequence = unit / a.kv_heads, kv_head = unit % a.kv_heads, groups = a.heads / a.kv_heads;
+    const SequenceSpan span = load_span<FORM>(sequence, a.query_offsets, a.page_offsets, a.last_page_lengths, a.query_lengths,
+                                              a.tokens, a.page_table, a.page_size);
+    if (!span.valid) return;  // reported by the attention kernel
+    const unsigned int row = row_tile * kQueryTile + (threadIdx.x >> 1), half = threadIdx.x & 1u;
+    if (row >= span.queries * groups) return;
+    const size_t flat = (static_cast<size_t>(span.query_start) + row / groups) * a.heads + kv_head * groups + row % groups;
+    const size_t rows_total = static_cast<size_t>(a.tokens) * a.heads;
+    float largest = -INFINITY;
+    for (unsigned int s = 0; s < shares; ++s) largest = fmaxf(largest, a.partial_lse[s * rows_total + flat]);
+    float total = 0.0f;
+    float merged[64];
+#pragma unroll
+    for (int d = 0; d < 64; ++d) merged[d] = 0.0f;
+    if (largest != -INFINITY) {
+        for (unsigned int s = 0; s < shares; ++s) {
+            const float lse = a.partial_lse[s * rows_total + flat];
+            if (lse == -INFINITY) continue;  // an empty share: its output was never meant to be read
+            const float weight = fast_exp2(lse - largest);
+            total += weight;
+            const float4* from = reinterpret_cast<const float4*>(a.partial_out + (s * rows_total + flat) * kHeadDim + 64 * half);
+#pragma unroll
+            for (int c = 0; c < 16; ++c) {
+                const float4 part = from[c];
+                merged[4 * c + 0] = fmaf(weight, part.x, merged[4 * c + 0]);
+                merged[4 * c + 1] = fmaf(weight, part.y, merged[4 * c + 1]);
+                merged[4 * c + 2] = fmaf(weight, part.z, merged[4 * c + 2]);
+                merged[4 * c + 3] = fmaf(weight, part.w, merged[4 * c + 3]);
+            }
+        }
+    }
+    const float inverse = total > 0.0f ? 1.0f / total : 0.0f;
+    uint16_t* out = a.output + flat * kHeadDim + 64 * half;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        uint4 packed_bits;
+        packed_bits.x = pack_pair(merged[8 * c + 0] * inverse, merged[8 * c + 1] * inverse);
+        packed_bits.y = pack_pair(merged[8 * c + 2] * inverse, merged[8 * c + 3] * inverse);
+        packed_bits.z = pack_pair(merged[8 * c + 4] * inverse, merged[8 * c + 5] * inverse);
+        packed_bits.w = pack_pair(merged[8 * c + 6] * inverse, merged[8 * c + 7] * inverse);
+        reinterpret_cast<uint4*>(out)[c] = packed_bits;
+    }
+    if (a.lse != nullptr && half == 0) a.lse[flat] = total > 0.0f ? largest + fast_log2(total) : -INFINITY;
+}
+
 }  // namespace
+
+// The merge of key splits: the same argument block as the attention kernel, whose `splits` counts the shares
+// here while workgroup ids map as without splits.
+extern "C" __global__ __launch_bounds__(256) void singe_paged_attention_combine_bf16_i32(PagedAttentionArgs args) {
+    const unsigned int shares = args.splits;
+    args.splits = 1;
+    combine_body<kCsrI32>(args, shares);
+}
+extern "C" __global__ __launch_bounds__(256) void singe_paged_attention_combine_bf16_i64(PagedAttentionArgs args) {
+    const unsigned int shares = args.splits;
+    args.splits = 1;
+    combine_body<kCsrI64>(args, shares);
+}
 
 #define SINGE_PAGED_ATTENTION_KERNEL(NAME, SOFTCAP, FORM, GROUPED, ROTATE)                                 \
     extern "C" __global__ __launch_bounds__(256, 2) void NAME(PagedAttentionArgs args) {                    \

@@ -146,9 +146,21 @@ def _attend_all(query, key, value, mask, sinks, key_lengths, options, stream):
     return output
 
 
+_scratch: dict = {}
+
+
+def _scratch_for(device, nbytes: int) -> torch.Tensor:
+    """A per-device buffer that grows to the largest request (the launch scratch a runtime would own)."""
+    held = _scratch.get(device)
+    if held is None or held.numel() < nbytes:
+        held = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
+        _scratch[device] = held
+    return held
+
+
 def paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor, paging: Paging,
                     options: AttentionOptions = AttentionOptions(), *, stream=None, status: torch.Tensor | None = None,
-                    check: bool = True):
+                    check: bool = True, scratch: "torch.Tensor | bool" = True):
     """Tensor::paged_attention (tensor/neural.rs:420-457) for bf16, f16 or f32 tensors on the GPU; bf16 at
     head dimension 128 runs on the matrix cores, everything else on the general kernel.
 
@@ -174,10 +186,23 @@ def paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: t
     entry = {torch.bfloat16: _native.lib().singe_hip_paged_attention_bf16,
              torch.float32: _native.lib().singe_hip_paged_attention_f32,
              torch.float16: _native.lib().singe_hip_paged_attention_f16}[query.dtype]
-    code = entry(
-        handle, query.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), paging.query_offsets.data_ptr(),
-        paging.page_offsets.data_ptr(), paging.pages.data_ptr(), paging.last_page_lengths.data_ptr(),
-        output.data_ptr(), lse.data_ptr(), status.data_ptr(), ctypes.byref(problem))
+    # bf16 calls with few query rows (decoding) share a row tile's keys out over several workgroups, given
+    # scratch: ``scratch`` is a uint8 device tensor, True for this module's own per-device buffer (calls on
+    # different streams must then not overlap), or False for none.
+    wanted = 0
+    if query.dtype == torch.bfloat16 and scratch is not False:
+        wanted = int(_native.lib().singe_hip_paged_attention_scratch_bytes(ctypes.byref(problem)))
+    if wanted > 0:
+        lent = _scratch_for(query.device, wanted) if scratch is True else scratch
+        code = _native.lib().singe_hip_paged_attention_scratch_bf16(
+            handle, query.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), paging.query_offsets.data_ptr(),
+            paging.page_offsets.data_ptr(), paging.pages.data_ptr(), paging.last_page_lengths.data_ptr(),
+            output.data_ptr(), lse.data_ptr(), status.data_ptr(), lent.data_ptr(), lent.numel(), ctypes.byref(problem))
+    else:
+        code = entry(
+            handle, query.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), paging.query_offsets.data_ptr(),
+            paging.page_offsets.data_ptr(), paging.pages.data_ptr(), paging.last_page_lengths.data_ptr(),
+            output.data_ptr(), lse.data_ptr(), status.data_ptr(), ctypes.byref(problem))
     _native.check(code, "paged_attention")
     if check and int(status.item()) == STATUS_INDEX_OUT_OF_BOUNDS:
         raise error.IndexOutOfBounds("paged attention paging value outside its buffers")

@@ -144,6 +144,22 @@ def test_rotary_paged_attention_validation():
     assert call(good, tokens=0) == 0
 
 
+def test_paged_attention_scratch_query_needs_no_device():
+    lib = _native.lib()
+    def wanted(**changes):
+        fields = dict(tokens=32, heads=32, kv_heads=8, head_dim=128, page_size=16, sequences=32, cache_pages=100, page_table=100,
+                      index_type=0, causal=1, has_scale=0, has_window=0, has_softcap=0, scale=0.0, softcap=0.0, window=0)
+        fields.update(changes)
+        return lib.singe_hip_paged_attention_scratch_bytes(ctypes.byref(_native.PagedAttentionProblemC(*fields.values())))
+    lib.singe_hip_set_paged_attention_splits(4)
+    try:
+        assert wanted() == 4 * 32 * 32 * 129 * 4     # shares x rows x (128 values + a log-sum-exp) of f32
+        assert wanted(head_dim=64) == 0               # the general kernel does not split
+    finally:
+        lib.singe_hip_set_paged_attention_splits(0)
+    assert lib.singe_hip_paged_attention_scratch_bytes(None) == 0
+
+
 def test_paged_mla_attention_validation():
     lib = _native.lib()
     fake = 0x1000

@@ -150,3 +150,37 @@ def test_paged_equals_dense_prefill():
     torch.cuda.synchronize()
     assert (out.float() - dense[0].float()).abs().max().item() <= 2 ** -6
     assert (lse - dense_lse[0].T / np.log(2.0)).abs().max().item() <= 2e-3
+
+
+@pytest.mark.parametrize("splits", [2, 3, 7, 16, 64])
+@pytest.mark.parametrize("options", [neural.AttentionOptions(causal=True), neural.AttentionOptions(),
+                                     neural.AttentionOptions(causal=True, window=100, softcap=20.0)])
+def test_key_splits_match_oracle(splits, options):
+    """With scratch lent, a row tile's keys are shared out over workgroups and merged by a second kernel: decode rows
+    over long and short caches, a chunk, a sequence without keys, more shares than a sequence has tiles."""
+    from singe_amd import _native
+    _native.lib().singe_hip_set_paged_attention_splits(splits)
+    try:
+        run_case([(1, 1500), (1, 40), (5, 700), (2, 0), (1, 65), (130, 300)], 8, 2, 16, options, seed=splits)
+        run_case([(1, 333), (3, 64)], 8, 1, 7, options, index_dtype=torch.int64, seed=splits + 1)
+    finally:
+        _native.lib().singe_hip_set_paged_attention_splits(0)
+
+
+def test_decode_shaped_calls_split_on_their_own_and_agree_with_the_unsplit_kernel():
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(21)
+    lens = [4096, 512, 1000, 2047, 16, 3000, 1, 777]
+    pages_of = [(n + 15) // 16 for n in lens]
+    page_count = sum(pages_of) + 5
+    q = torch.randn((len(lens), 32, 128), generator=gen, device="cuda").to(torch.bfloat16)
+    kc = torch.randn((page_count, 16, 8, 128), generator=gen, device="cuda").to(torch.bfloat16)
+    vc = torch.randn((page_count, 16, 8, 128), generator=gen, device="cuda").to(torch.bfloat16)
+    index = lambda values: torch.tensor(values, dtype=torch.int32, device="cuda")
+    table = np.random.default_rng(3).permutation(page_count)[:sum(pages_of)]
+    paging = neural.Paging(index(list(range(len(lens) + 1))), index(np.concatenate([[0], np.cumsum(pages_of)])), index(table),
+                           index([n - (p - 1) * 16 for n, p in zip(lens, pages_of)]))
+    apart, apart_lse = neural.paged_attention(q, kc, vc, paging, neural.AttentionOptions(causal=True), scratch=False)
+    split, split_lse = neural.paged_attention(q, kc, vc, paging, neural.AttentionOptions(causal=True))
+    assert (apart.float() - split.float()).abs().max().item() <= 4e-3
+    assert (apart_lse - split_lse).abs().max().item() <= 1e-3
