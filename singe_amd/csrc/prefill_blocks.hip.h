@@ -84,7 +84,7 @@ SINGE_DEVICE float begin_block(RowState& state, f32x16_t& s, unsigned int hi, fl
     largest = max3(largest, s[10], s[11]);
     other = max3(other, s[12], s[13]);
     largest = max3(largest, s[14], s[15]);
-    largest = swap32_max(fmaxf(largest, other)) * factor;  // both lanes of a query agree from here on
+    largest = swap32_max(max2(largest, other)) * factor;  // both lanes of a query agree from here on
     if (__any(largest > state.reference + kMaxLag || (state.reference == -INFINITY && largest != -INFINITY))) {
         const float moved = fmaxf(state.reference, largest);
         const float base = moved == -INFINITY ? 0.0f : moved;

@@ -32,10 +32,19 @@ typedef short v8i16_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2v_t __attribute__((ext_vector_type(2)));
 typedef float f32x2v_t __attribute__((ext_vector_type(2)));
 
+// max(a, b) in one instruction, without the canonicalising copies the compiler puts in front of fmaxf when
+// it cannot see where the operands come from (here: out of inline assembly); for values that are never
+// signalling NaNs.
+SINGE_DEVICE float max2(float a, float b) {
+    float result;
+    asm("v_max_f32 %0, %1, %2" : "=v"(result) : "v"(a), "v"(b));
+    return result;
+}
+
 SINGE_DEVICE float swap32_max(float value) {
     float kept = value, taken = value;
     asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(kept), "+v"(taken));
-    return fmaxf(kept, taken);
+    return max2(kept, taken);
 }
 
 SINGE_DEVICE float swap32_sum(float value) {
