@@ -89,8 +89,8 @@ def cpu_baseline(work, budget_s=12.0):
 
 
 def prefill_section(steps):
-    """Causal flash-attention prefill, batch 4, seq 4096, 32 heads, head_dim 128, bf16 (BASELINE
-    config 3): average kernel time from HIP events around back-to-back launches."""
+    """Causal flash-attention prefill, batch 4, seq 4096, 32 heads, head_dim 128, bf16 (the
+    third benchmark configuration): average kernel time from HIP events around back-to-back launches."""
     import torch
 
     from singe_amd.kernel import attention as A
@@ -161,7 +161,7 @@ def time_launches(launch, steps, group):
 
 def chunked_prefill_section(steps):
     """Chunked paged prefill: 8 sequences, 512 new tokens each on prefixes U[1024, 16384], 64 query /
-    8 KV heads, head_dim 128, page 16, bf16 (BASELINE config 4), through the paged attention op."""
+    8 KV heads, head_dim 128, page 16, bf16 (the fourth benchmark configuration), through the paged attention op."""
     import ctypes
 
     import numpy as np
@@ -209,7 +209,7 @@ def chunked_prefill_section(steps):
 
 def fp8_decode_section(steps):
     """Long-context decode over an fp8 e4m3 KV cache: batch 64, 64 query / 8 KV heads, head_dim 128,
-    context 32768, block 16, one f32 scale per (block, kv head) (BASELINE config 5); exact numerics."""
+    context 32768, block 16, one f32 scale per (block, kv head) (the fifth benchmark configuration); exact numerics."""
     import numpy as np
     import torch
 
