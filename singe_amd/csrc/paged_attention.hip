@@ -460,8 +460,8 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
 
 // Merges the key splits of every row of a (unit, row tile): each share's output weighs 2^(lse - largest) over
 // the sum of those (the merge of the reference's own split kernels, kernel_plan/source/mla.rs:497-560), the row's
-// log-sum-exp is largest + log2 of that sum.  One thread per (row, 64 dims); launched with splits = 1 so the
-// workgroup ids map as in the attention kernel, the number of shares in `shares`.
+// log-sum-exp is largest + log2 of that sum.  Workgroup ids map as in the attention kernel without splits; `shares`
+// (at most 64) is the number of shares.
 template <int FORM>
 SINGE_DEVICE void combine_body(const PagedAttentionArgs& a, unsigned int shares) {
     unsigned int unit, row_tile, split;
@@ -470,45 +470,33 @@ SINGE_DEVICE void combine_body(const PagedAttentionArgs& a, unsigned int shares)
     const SequenceSpan span = load_span<FORM>(sequence, a.query_offsets, a.page_offsets, a.last_page_lengths, a.query_lengths,
                                               a.tokens, a.page_table, a.page_size);
     if (!span.valid) return;  // reported by the attention kernel
-    const unsigned int row = row_tile * kQueryTile + (threadIdx.x >> 1), half = threadIdx.x & 1u;
-    if (row >= span.queries * groups) return;
-    const size_t flat = (static_cast<size_t>(span.query_start) + row / groups) * a.heads + kv_head * groups + row % groups;
+    // A wave per row, rows of the tile four apart; a lane takes two of the 128 values.
+    const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    const unsigned int packed = span.queries * groups;
     const size_t rows_total = static_cast<size_t>(a.tokens) * a.heads;
-    float largest = -INFINITY;
-    for (unsigned int s = 0; s < shares; ++s) largest = fmaxf(largest, a.partial_lse[s * rows_total + flat]);
-    float total = 0.0f;
-    float merged[64];
+    for (unsigned int row = row_tile * kQueryTile + wave; row < packed && row < (row_tile + 1u) * kQueryTile; row += 4u) {
+        const size_t flat = (static_cast<size_t>(span.query_start) + row / groups) * a.heads + kv_head * groups + row % groups;
+        // The shares' log-sum-exps, one per lane (at most 64 shares), and their largest.
+        const float mine = lane < shares ? a.partial_lse[lane * rows_total + flat] : -INFINITY;
+        float largest = mine;
 #pragma unroll
-    for (int d = 0; d < 64; ++d) merged[d] = 0.0f;
-    if (largest != -INFINITY) {
+        for (int step = 32; step > 0; step >>= 1) largest = fmaxf(largest, __shfl_xor(largest, step, 64));
+        const float weight = mine == -INFINITY ? 0.0f : fast_exp2(mine - largest);  // an empty share weighs nothing
+        float total = weight;
+#pragma unroll
+        for (int step = 32; step > 0; step >>= 1) total += __shfl_xor(total, step, 64);
+        float2 merged = make_float2(0.0f, 0.0f);
         for (unsigned int s = 0; s < shares; ++s) {
-            const float lse = a.partial_lse[s * rows_total + flat];
-            if (lse == -INFINITY) continue;  // an empty share: its output was never meant to be read
-            const float weight = fast_exp2(lse - largest);
-            total += weight;
-            const float4* from = reinterpret_cast<const float4*>(a.partial_out + (s * rows_total + flat) * kHeadDim + 64 * half);
-#pragma unroll
-            for (int c = 0; c < 16; ++c) {
-                const float4 part = from[c];
-                merged[4 * c + 0] = fmaf(weight, part.x, merged[4 * c + 0]);
-                merged[4 * c + 1] = fmaf(weight, part.y, merged[4 * c + 1]);
-                merged[4 * c + 2] = fmaf(weight, part.z, merged[4 * c + 2]);
-                merged[4 * c + 3] = fmaf(weight, part.w, merged[4 * c + 3]);
-            }
+            const float w = __shfl(weight, s, 64);
+            if (w == 0.0f) continue;  // its output was never meant to be read
+            const float2 part = *reinterpret_cast<const float2*>(a.partial_out + (s * rows_total + flat) * kHeadDim + 2u * lane);
+            merged.x = fmaf(w, part.x, merged.x);
+            merged.y = fmaf(w, part.y, merged.y);
         }
+        const float inverse = total > 0.0f ? 1.0f / total : 0.0f;
+        reinterpret_cast<unsigned int*>(a.output + flat * kHeadDim)[lane] = pack_pair(merged.x * inverse, merged.y * inverse);
+        if (a.lse != nullptr && lane == 0) a.lse[flat] = total > 0.0f ? largest + fast_log2(total) : -INFINITY;
     }
-    const float inverse = total > 0.0f ? 1.0f / total : 0.0f;
-    uint16_t* out = a.output + flat * kHeadDim + 64 * half;
-#pragma unroll
-    for (int c = 0; c < 8; ++c) {
-        uint4 packed_bits;
-        packed_bits.x = pack_pair(merged[8 * c + 0] * inverse, merged[8 * c + 1] * inverse);
-        packed_bits.y = pack_pair(merged[8 * c + 2] * inverse, merged[8 * c + 3] * inverse);
-        packed_bits.z = pack_pair(merged[8 * c + 4] * inverse, merged[8 * c + 5] * inverse);
-        packed_bits.w = pack_pair(merged[8 * c + 6] * inverse, merged[8 * c + 7] * inverse);
-        reinterpret_cast<uint4*>(out)[c] = packed_bits;
-    }
-    if (a.lse != nullptr && half == 0) a.lse[flat] = total > 0.0f ? largest + fast_log2(total) : -INFINITY;
 }
 
 }  // namespace
