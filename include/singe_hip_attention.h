@@ -248,6 +248,24 @@ SINGE_HIP_API int32_t singe_hip_fmha_prefill_lse_bf16(
     const uint16_t* value, size_t value_len,
     const SingeFmhaPrefillConfig* config);
 
+/* fmha_prefill_f16 / fmha_prefill_lse_f16 (fmha.rs, the f16 twins of the two calls above): the same kernels on
+ * v_mfma_f32_32x32x16_f16; operands and outputs are IEEE half bit patterns. */
+SINGE_HIP_API int32_t singe_hip_fmha_prefill_f16(
+    void* stream,
+    uint16_t* out, size_t out_len,
+    const uint16_t* query, size_t query_len,
+    const uint16_t* key, size_t key_len,
+    const uint16_t* value, size_t value_len,
+    const SingeFmhaPrefillConfig* config);
+SINGE_HIP_API int32_t singe_hip_fmha_prefill_lse_f16(
+    void* stream,
+    uint16_t* out, size_t out_len,
+    float* lse, size_t lse_len,
+    const uint16_t* query, size_t query_len,
+    const uint16_t* key, size_t key_len,
+    const uint16_t* value, size_t value_len,
+    const SingeFmhaPrefillConfig* config);
+
 /* f32 forms for any head_dim up to 256 (fmha_prefill_f32 / fmha_prefill_lse_f32: fmha.rs:48-190).
  * The f32 correctness anchor: dense causal [1, 8, 512, 64] attention in [batch, heads, len, dim]
  * order is this call with batch stride heads*len*dim, head stride len*dim, sequence stride dim. */
@@ -350,6 +368,22 @@ SINGE_HIP_API int32_t singe_hip_paged_attention_bf16(
 SINGE_HIP_API size_t singe_hip_paged_attention_scratch_bytes(const SingePagedAttentionProblem* problem);
 SINGE_HIP_API void singe_hip_set_paged_attention_splits(uint32_t splits);
 SINGE_HIP_API int32_t singe_hip_paged_attention_scratch_bf16(
+    void* stream,
+    const uint16_t* query_rows,
+    const uint16_t* key_cache,
+    const uint16_t* value_cache,
+    const void* query_offsets,
+    const void* page_offsets,
+    const void* pages,
+    const void* last_page_lengths,
+    uint16_t* output,
+    float* lse,
+    uint32_t* status,
+    void* scratch,
+    size_t scratch_bytes,
+    const SingePagedAttentionProblem* problem);
+
+SINGE_HIP_API int32_t singe_hip_paged_attention_scratch_f16(
     void* stream,
     const uint16_t* query_rows,
     const uint16_t* key_cache,

@@ -161,6 +161,12 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_fmha_prefill_lse_bf16.argtypes = [c_void, c_void, c_size, c_void, c_size, c_void, c_size, c_void,
                                                        c_size, c_void, c_size, fmha]
     handle.singe_hip_fmha_prefill_lse_bf16.restype = i32
+    handle.singe_hip_fmha_prefill_f16.argtypes = handle.singe_hip_fmha_prefill_bf16.argtypes
+    handle.singe_hip_fmha_prefill_f16.restype = i32
+    handle.singe_hip_fmha_prefill_lse_f16.argtypes = handle.singe_hip_fmha_prefill_lse_bf16.argtypes
+    handle.singe_hip_fmha_prefill_lse_f16.restype = i32
+    handle.singe_hip_paged_attention_scratch_f16.argtypes = [c_void] * 12 + [ctypes.c_size_t, ctypes.POINTER(PagedAttentionProblemC)]
+    handle.singe_hip_paged_attention_scratch_f16.restype = i32
     handle.singe_hip_fmha_prefill_f32.argtypes = [c_void, c_void, c_size, c_void, c_size, c_void, c_size, c_void,
                                                   c_size, fmha]
     handle.singe_hip_fmha_prefill_f32.restype = i32

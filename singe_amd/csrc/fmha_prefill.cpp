@@ -126,14 +126,14 @@ int32_t prefill_f32(void* stream, float* out, size_t out_len, float* lse, size_t
 
 int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, bool with_lse,
                 const uint16_t* query, size_t query_len, const uint16_t* key, size_t key_len, const uint16_t* value,
-                size_t value_len, const SingeFmhaPrefillConfig* config) {
+                size_t value_len, const SingeFmhaPrefillConfig* config, bool f16 = false) {
     if (config == nullptr) return fail(SINGE_HIP_NULL_POINTER, "config");
     const SingeFmhaPrefillConfig& c = *config;
     if (int32_t status = validate_call(c, out, out_len, lse, lse_len, with_lse, query, query_len, key, key_len, value, value_len))
         return status;
 
     // What the gfx950 kernel takes: head_dim 128 and rows it can fetch 16 bytes at a time.
-    if (c.head_dim != 128) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, "fmha_prefill_bf16", c.head_dim, 0);
+    if (c.head_dim != 128) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, f16 ? "fmha_prefill_f16" : "fmha_prefill_bf16", c.head_dim, 0);
     const size_t strides[] = {c.query_batch_stride, c.key_batch_stride, c.value_batch_stride, c.output_batch_stride,
                               c.query_sequence_stride, c.key_sequence_stride, c.value_sequence_stride,
                               c.output_sequence_stride, c.query_head_stride, c.key_head_stride,
@@ -177,7 +177,8 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
     const uint64_t rows = (static_cast<uint64_t>(c.batch) * c.heads + 7) / 8 * 8;
     const uint64_t groups = rows * ((args.query_tiles + 1) / 2);  // a workgroup takes a pair of query tiles
     if (groups > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
-    return launch(c.causal ? kPrefillCausal : kPrefillFull, static_cast<unsigned>(groups), 1, 1, 256, stream, args);
+    const KernelId kernel = f16 ? (c.causal ? kPrefillCausalF16 : kPrefillFullF16) : (c.causal ? kPrefillCausal : kPrefillFull);
+    return launch(kernel, static_cast<unsigned>(groups), 1, 1, 256, stream, args);
 }
 
 }  // namespace
@@ -222,6 +223,19 @@ int32_t singe_hip_fmha_prefill_lse_bf16(void* stream, uint16_t* out, size_t out_
                                         const uint16_t* query, size_t query_len, const uint16_t* key, size_t key_len,
                                         const uint16_t* value, size_t value_len, const SingeFmhaPrefillConfig* config) {
     return prefill(stream, out, out_len, lse, lse_len, true, query, query_len, key, key_len, value, value_len, config);
+}
+
+// fmha_prefill_f16 / fmha_prefill_lse_f16 (fmha.rs): the same kernels on f16 operands.
+int32_t singe_hip_fmha_prefill_f16(void* stream, uint16_t* out, size_t out_len, const uint16_t* query, size_t query_len,
+                                   const uint16_t* key, size_t key_len, const uint16_t* value, size_t value_len,
+                                   const SingeFmhaPrefillConfig* config) {
+    return prefill(stream, out, out_len, nullptr, 0, false, query, query_len, key, key_len, value, value_len, config, true);
+}
+
+int32_t singe_hip_fmha_prefill_lse_f16(void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len,
+                                       const uint16_t* query, size_t query_len, const uint16_t* key, size_t key_len,
+                                       const uint16_t* value, size_t value_len, const SingeFmhaPrefillConfig* config) {
+    return prefill(stream, out, out_len, lse, lse_len, true, query, query_len, key, key_len, value, value_len, config, true);
 }
 
 }  // extern "C"

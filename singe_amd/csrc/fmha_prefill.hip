@@ -27,7 +27,7 @@ using namespace prefill;
 constexpr bool kDenseOperandsAhead = false;
 
 // One 128-row query tile of (batch, head) pair `bh`.
-template <bool CAUSAL>
+template <bool CAUSAL, class Half>
 SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, unsigned int bh, unsigned int query_tile) {
     const unsigned int tid = threadIdx.x, lane = tid & 63;
     // The wave index is the same in all lanes; saying so keeps everything derived from it (which blocks
@@ -51,7 +51,8 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     // the raw scores and fold the positive factor into one fused multiply-add.
     const float factor = fabsf(a.scale_log2e);
     const unsigned int flip = a.scale_log2e < 0.0f ? 0x80008000u : 0u;
-    bf16x8_t q[8];
+    const Half half{};
+    uint4 q[8];
     {
         const uint16_t* row = q_base + static_cast<size_t>(query_valid ? my_query : 0) * a.query_sequence_stride + 8 * hi;
 #pragma unroll
@@ -59,7 +60,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
             uint4 bits = *reinterpret_cast<const uint4*>(row + 16 * s);
             if (!query_valid) bits = make_uint4(0, 0, 0, 0);
             bits.x ^= flip; bits.y ^= flip; bits.z ^= flip; bits.w ^= flip;
-            q[s] = __builtin_bit_cast(bf16x8_t, bits);
+            q[s] = bits;
         }
     }
 
@@ -140,13 +141,13 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
             const unsigned int key = key0 + key_in_block;
             return (CAUSAL && key > my_query) || key >= a.key_len;
         });
-        finish_block<false>(state, s, factor, shift, values, offsets, s, q, values);
+        finish_block<false>(half, state, s, factor, shift, values, offsets, s, q, values);
     };
 
     // One block ahead: while block b is folded, the scores of block b + 1 are computed; `scores` holds
     // those of the block that is folded next.
     f32x16_t scores;
-    if (wave_blocks > 0) score_block(scores, q, lds, offsets);
+    if (wave_blocks > 0) score_block(half, scores, q, lds, offsets);
     unsigned int key_stage = 0, value_stage = 0;  // tile % 3, tile % 2
     // Names the stages a tile's iteration works on and loads into.  Everyone left the stages that held K of
     // tile - 1 and V of tile - 1 at the last barrier.
@@ -189,7 +190,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     };
     for (; tile < interior_tiles; ++tile) {
         const TileStages stages = enter();
-        fold_interior_tile<kDenseOperandsAhead>(state, scores, operand, q, offsets, hi, factor, stages.keys, stages.next_keys, stages.values, stages.key_dest,
+        fold_interior_tile<kDenseOperandsAhead>(half, state, scores, operand, q, offsets, hi, factor, stages.keys, stages.next_keys, stages.values, stages.key_dest,
                            stages.value_dest, issue);
         leave();
     }
@@ -197,7 +198,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     // workgroup's remaining loads and barriers).
     for (; tile < tiles; ++tile) {
         const TileStages stages = enter();
-        fold_edge_tile(scores, q, offsets, 2u * tile, wave_blocks, stages.keys, stages.next_keys, stages.values, stages.key_dest,
+        fold_edge_tile(half, scores, q, offsets, 2u * tile, wave_blocks, stages.keys, stages.next_keys, stages.values, stages.key_dest,
                        stages.value_dest, issue, fold);
         leave();
     }
@@ -213,8 +214,8 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
 #pragma unroll
             for (int quad = 0; quad < 4; ++quad) {
                 uint2 packed;
-                packed.x = pack_pair(state.out[db][4 * quad + 0] * inverse, state.out[db][4 * quad + 1] * inverse);
-                packed.y = pack_pair(state.out[db][4 * quad + 2] * inverse, state.out[db][4 * quad + 3] * inverse);
+                packed.x = pack_pair(half, state.out[db][4 * quad + 0] * inverse, state.out[db][4 * quad + 1] * inverse);
+                packed.y = pack_pair(half, state.out[db][4 * quad + 2] * inverse, state.out[db][4 * quad + 3] * inverse);
                 *reinterpret_cast<uint2*>(row + 32 * db + 8 * quad + 4 * hi) = packed;
             }
         if (a.lse != nullptr && hi == 0)
@@ -224,25 +225,26 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
 }
 
 // Workgroup id -> (batch * heads + head, pair of query tiles): see the header comment.
-template <bool CAUSAL>
+template <bool CAUSAL, class Half>
 SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
     const unsigned int xcd = blockIdx.x & 7u, within = blockIdx.x >> 3;
     const unsigned int pairs = (a.query_tiles + 1u) / 2u;
     const unsigned int bh = (within / pairs) * 8u + xcd;
     if (bh >= a.batch * a.heads) return;
     const unsigned int light = within % pairs, heavy = a.query_tiles - 1u - light;
-    fmha_prefill_tile<CAUSAL>(a, lds, bh, heavy);
-    if (light != heavy) fmha_prefill_tile<CAUSAL>(a, lds, bh, light);
+    fmha_prefill_tile<CAUSAL, Half>(a, lds, bh, heavy);
+    if (light != heavy) fmha_prefill_tile<CAUSAL, Half>(a, lds, bh, light);
 }
 
 }  // namespace
 
-extern "C" __global__ __launch_bounds__(256, 2) void singe_fmha_prefill_bf16_d128_causal(PrefillArgs args) {
-    __shared__ __attribute__((aligned(1024))) unsigned char prefill_lds[kStagedLdsBytes];
-    fmha_prefill_body<true>(args, prefill_lds);
-}
+#define SINGE_FMHA_PREFILL_KERNEL(NAME, CAUSAL, HALF)                                              \
+    extern "C" __global__ __launch_bounds__(256, 2) void NAME(PrefillArgs args) {                    \
+        __shared__ __attribute__((aligned(1024))) unsigned char prefill_lds[kStagedLdsBytes];        \
+        fmha_prefill_body<CAUSAL, prefill::HALF>(args, prefill_lds);                                \
+    }
 
-extern "C" __global__ __launch_bounds__(256, 2) void singe_fmha_prefill_bf16_d128_full(PrefillArgs args) {
-    __shared__ __attribute__((aligned(1024))) unsigned char prefill_lds[kStagedLdsBytes];
-    fmha_prefill_body<false>(args, prefill_lds);
-}
+SINGE_FMHA_PREFILL_KERNEL(singe_fmha_prefill_bf16_d128_causal, true, Bf16)
+SINGE_FMHA_PREFILL_KERNEL(singe_fmha_prefill_bf16_d128_full, false, Bf16)
+SINGE_FMHA_PREFILL_KERNEL(singe_fmha_prefill_f16_d128_causal, true, F16)
+SINGE_FMHA_PREFILL_KERNEL(singe_fmha_prefill_f16_d128_full, false, F16)

@@ -14,15 +14,17 @@ enum KernelId : int {
     kDecodeCombine = 4,
     // fp8 decode, dense form: + (block size not a multiple of 16) + 2 * relaxed
     kDecodeF8Wide, kDecodeF8WideAny, kDecodeF8WideRelaxed, kDecodeF8WideRelaxedAny,
-    kPrefillCausal, kPrefillFull,
+    kPrefillCausal, kPrefillFull, kPrefillCausalF16, kPrefillFullF16,
     kPrefillF32D32, kPrefillF32D64, kPrefillF32D128, kPrefillF32D256,
     // paged attention: + 4 when the page size is a power of two of at least 16 keys
     kPagedAttentionI32, kPagedAttentionI64, kPagedAttentionSoftcapI32, kPagedAttentionSoftcapI64,
     kPagedAttentionI32P16, kPagedAttentionI64P16, kPagedAttentionSoftcapI32P16, kPagedAttentionSoftcapI64P16,
     kPagedKvPrefill, kPagedKvPrefillP16,
-    kPagedAttentionCombineI32, kPagedAttentionCombineI64,
+    kPagedAttentionCombineI32, kPagedAttentionCombineI64, kPagedAttentionCombineF16I32, kPagedAttentionCombineF16I64,
+    // f16 paged attention: same order as the eight bf16 kernels from kPagedAttentionI32
+    kPagedAttentionF16,
     // fused query rotation: + (i64 indices) + 2 * (page size a power of two of at least 16 keys)
-    kRotaryPagedAttention, kRotaryPagedAttentionI64, kRotaryPagedAttentionP16, kRotaryPagedAttentionI64P16,
+    kRotaryPagedAttention = kPagedAttentionF16 + 8, kRotaryPagedAttentionI64, kRotaryPagedAttentionP16, kRotaryPagedAttentionI64P16,
     kSplitKReduce,
     kRotaryCacheF32, kRotaryCacheBf16, kRotaryCacheF16,
     kPagingIndicesI32, kPagingIndicesI64,

@@ -99,10 +99,11 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
     if (pages == nullptr && p.page_table > 0) return fail(SINGE_HIP_NULL_POINTER, "pages");
     if (rotation != nullptr && (rotation->cos == nullptr || rotation->sin == nullptr)) return fail(SINGE_HIP_NULL_POINTER, "cos or sin");
     const float scale = p.has_scale ? p.scale : 1.0f / std::sqrt(static_cast<float>(p.head_dim));
-    // The tensor-core kernel covers bf16 at head dimension 128 (the reference's takes f16/bf16 at
+    // The tensor-core kernel covers bf16 and f16 at head dimension 128 (the reference's takes f16/bf16 at
     // multiples of 16 up to 128: paged_attention.rs:586-592); everything else goes to the general one
     // (paged_general.rs:73-247).
-    if (data_type != SINGE_HIP_BF16 || p.head_dim != 128)
+    const bool f16 = data_type == SINGE_HIP_F16;
+    if ((data_type != SINGE_HIP_BF16 && !f16) || p.head_dim != 128)
         return paged_attention_general(data_type, stream, query_rows_any, key_cache_any, value_cache_any, query_offsets,
                                        page_offsets, pages, last_page_lengths, output_any, lse, status, p, scale);
     const uint16_t* query_rows = static_cast<const uint16_t*>(query_rows_any);
@@ -157,7 +158,8 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
     const unsigned grid = static_cast<unsigned>(blocks * splits);
     auto finish = [&](int32_t launched) -> int32_t {
         if (launched != 0 || splits == 1) return launched;
-        return launch(wide ? kPagedAttentionCombineI64 : kPagedAttentionCombineI32, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+        const int combine = (f16 ? kPagedAttentionCombineF16I32 : kPagedAttentionCombineI32) + (wide ? 1 : 0);
+        return launch(static_cast<KernelId>(combine), static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
     };
     if (rotation != nullptr) {
         args.cos = rotation->cos;
@@ -169,8 +171,7 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
         const int rotary = kRotaryPagedAttention + (wide ? 1 : 0) + (args.page_shift >= 4 ? 2 : 0);
         return finish(launch(static_cast<KernelId>(rotary), grid, 1, 1, 256, stream, args));
     }
-    const int kernel = (p.has_softcap ? (wide ? kPagedAttentionSoftcapI64 : kPagedAttentionSoftcapI32)
-                                      : (wide ? kPagedAttentionI64 : kPagedAttentionI32)) +
+    const int kernel = (f16 ? kPagedAttentionF16 : kPagedAttentionI32) + (p.has_softcap ? 2 : 0) + (wide ? 1 : 0) +
                        (args.page_shift >= 4 ? 4 : 0);
     return finish(launch(static_cast<KernelId>(kernel), grid, 1, 1, 256, stream, args));
 }
@@ -192,6 +193,17 @@ extern "C" int32_t singe_hip_paged_attention_scratch_bf16(void* stream, const ui
                                                           const SingePagedAttentionProblem* problem) {
     const Scratch lent = {scratch, scratch_bytes};
     return paged_attention(SINGE_HIP_BF16, stream, query_rows, key_cache, value_cache, query_offsets, page_offsets, pages,
+                           last_page_lengths, output, lse, status, problem, nullptr, &lent);
+}
+
+extern "C" int32_t singe_hip_paged_attention_scratch_f16(void* stream, const uint16_t* query_rows, const uint16_t* key_cache,
+                                                         const uint16_t* value_cache, const void* query_offsets,
+                                                         const void* page_offsets, const void* pages,
+                                                         const void* last_page_lengths, uint16_t* output, float* lse,
+                                                         uint32_t* status, void* scratch, size_t scratch_bytes,
+                                                         const SingePagedAttentionProblem* problem) {
+    const Scratch lent = {scratch, scratch_bytes};
+    return paged_attention(SINGE_HIP_F16, stream, query_rows, key_cache, value_cache, query_offsets, page_offsets, pages,
                            last_page_lengths, output, lse, status, problem, nullptr, &lent);
 }
 

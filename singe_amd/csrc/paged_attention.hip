@@ -74,7 +74,7 @@ SINGE_DEVICE bool locate(const PagedAttentionArgs& a, unsigned int& unit, unsign
     return unit < a.sequences * a.kv_heads;
 }
 
-template <bool SOFTCAP, int FORM, bool GROUPED, bool ROTATE = false>
+template <bool SOFTCAP, int FORM, bool GROUPED, bool ROTATE, class Half>
 SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned char* lds) {
     const unsigned int tid = threadIdx.x, lane = tid & 63;
     const unsigned int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform, and known to be
@@ -155,7 +155,9 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     // Q^T as the MFMA B operand; a negative scale moves into Q (see fmha_prefill.hip).
     const float factor = SOFTCAP ? 1.0f : fabsf(a.scale_log2e);
     const unsigned int flip = (SOFTCAP ? a.softcap_scale : a.scale_log2e) < 0.0f ? 0x80008000u : 0u;
-    bf16x8_t q[8];
+    static_assert(!ROTATE || std::is_same<Half, Bf16>::value, "the fused rotation reads bf16 queries");
+    const Half half{};
+    uint4 q[8];
     {
         const uint16_t* row = a.query_rows + ((static_cast<size_t>(query_start) + my_token) * a.heads + kv_head * groups + my_head) * kHeadDim + 8 * hi;
         uint4 bits[8];
@@ -220,7 +222,7 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
 #pragma unroll
         for (int s = 0; s < 8; ++s) {
             bits[s].x ^= flip; bits[s].y ^= flip; bits[s].z ^= flip; bits[s].w ^= flip;
-            q[s] = __builtin_bit_cast(bf16x8_t, bits[s]);
+            q[s] = bits[s];
         }
     }
 
@@ -354,12 +356,12 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
             const unsigned int key = key0 + key_in_block;
             return key >= keys || (causal && key > my_position) || (windowed && key + window <= my_position);
         });
-        finish_block<false>(state, s, factor, shift, values, offsets, s, q, values);
+        finish_block<false>(half, state, s, factor, shift, values, offsets, s, q, values);
     };
 
     // One block ahead, as in the dense kernel: `scores` holds those of the block that is folded next.
     f32x16_t scores;
-    if (2u * first_tile < wave_blocks) score_block(scores, q, lds, offsets);
+    if (2u * first_tile < wave_blocks) score_block(half, scores, q, lds, offsets);
     unsigned int key_stage = 0, value_stage = 0;
     // Names the stages a tile's iteration works on and loads into.
     auto enter = [&]() __attribute__((always_inline)) {
@@ -407,7 +409,7 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     if (kPagedOperandsAhead && tile < interior_end) read_key_operands(operand, lds + kBlockBytes, offsets);
     for (; tile < interior_end; ++tile) {
         const TileStages stages = enter();
-        fold_interior_tile<kPagedOperandsAhead>(state, scores, operand, q, offsets, hi, factor, stages.keys, stages.next_keys, stages.values, stages.key_dest,
+        fold_interior_tile<kPagedOperandsAhead>(half, state, scores, operand, q, offsets, hi, factor, stages.keys, stages.next_keys, stages.values, stages.key_dest,
                            stages.value_dest, issue);
         leave();
     }
@@ -415,7 +417,7 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     // remaining loads and barriers).
     for (; tile < tiles; ++tile) {
         const TileStages stages = enter();
-        fold_edge_tile(scores, q, offsets, 2u * tile, wave_blocks, stages.keys, stages.next_keys, stages.values, stages.key_dest,
+        fold_edge_tile(half, scores, q, offsets, 2u * tile, wave_blocks, stages.keys, stages.next_keys, stages.values, stages.key_dest,
                        stages.value_dest, issue, fold);
         leave();
     }
@@ -444,8 +446,8 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
 #pragma unroll
             for (int quad = 0; quad < 4; ++quad) {
                 uint2 packed_bits;
-                packed_bits.x = pack_pair(state.out[db][4 * quad + 0] * inverse, state.out[db][4 * quad + 1] * inverse);
-                packed_bits.y = pack_pair(state.out[db][4 * quad + 2] * inverse, state.out[db][4 * quad + 3] * inverse);
+                packed_bits.x = pack_pair(half, state.out[db][4 * quad + 0] * inverse, state.out[db][4 * quad + 1] * inverse);
+                packed_bits.y = pack_pair(half, state.out[db][4 * quad + 2] * inverse, state.out[db][4 * quad + 3] * inverse);
                 *reinterpret_cast<uint2*>(row + 32 * db + 8 * quad + 4 * hi) = packed_bits;
             }
         if (a.lse != nullptr && hi == 0) {
@@ -462,7 +464,7 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
 // the sum of those (the merge of the reference's own split kernels, kernel_plan/source/mla.rs:497-560), the row's
 // log-sum-exp is largest + log2 of that sum.  Workgroup ids map as in the attention kernel without splits; `shares`
 // (at most 64) is the number of shares.
-template <int FORM>
+template <int FORM, class Half>
 SINGE_DEVICE void combine_body(const PagedAttentionArgs& a, unsigned int shares) {
     unsigned int unit, row_tile, split;
     if (!locate(a, unit, row_tile, split)) return;
@@ -494,7 +496,7 @@ SINGE_DEVICE void combine_body(const PagedAttentionArgs& a, unsigned int shares)
             merged.y = fmaf(w, part.y, merged.y);
         }
         const float inverse = total > 0.0f ? 1.0f / total : 0.0f;
-        reinterpret_cast<unsigned int*>(a.output + flat * kHeadDim)[lane] = pack_pair(merged.x * inverse, merged.y * inverse);
+        reinterpret_cast<unsigned int*>(a.output + flat * kHeadDim)[lane] = pack_pair(Half{}, merged.x * inverse, merged.y * inverse);
         if (a.lse != nullptr && lane == 0) a.lse[flat] = total > 0.0f ? largest + fast_log2(total) : -INFINITY;
     }
 }
@@ -503,37 +505,47 @@ SINGE_DEVICE void combine_body(const PagedAttentionArgs& a, unsigned int shares)
 
 // The merge of key splits: the same argument block as the attention kernel, whose `splits` counts the shares
 // here while workgroup ids map as without splits.
-extern "C" __global__ __launch_bounds__(256) void singe_paged_attention_combine_bf16_i32(PagedAttentionArgs args) {
-    const unsigned int shares = args.splits;
-    args.splits = 1;
-    combine_body<kCsrI32>(args, shares);
-}
-extern "C" __global__ __launch_bounds__(256) void singe_paged_attention_combine_bf16_i64(PagedAttentionArgs args) {
-    const unsigned int shares = args.splits;
-    args.splits = 1;
-    combine_body<kCsrI64>(args, shares);
-}
+#define SINGE_PAGED_COMBINE_KERNEL(NAME, FORM, HALF)                                         \
+    extern "C" __global__ __launch_bounds__(256) void NAME(PagedAttentionArgs args) {        \
+        const unsigned int shares = args.splits;                                             \
+        args.splits = 1;                                                                     \
+        combine_body<FORM, prefill::HALF>(args, shares);                                     \
+    }
 
-#define SINGE_PAGED_ATTENTION_KERNEL(NAME, SOFTCAP, FORM, GROUPED, ROTATE)                                 \
+SINGE_PAGED_COMBINE_KERNEL(singe_paged_attention_combine_bf16_i32, kCsrI32, Bf16)
+SINGE_PAGED_COMBINE_KERNEL(singe_paged_attention_combine_bf16_i64, kCsrI64, Bf16)
+SINGE_PAGED_COMBINE_KERNEL(singe_paged_attention_combine_f16_i32, kCsrI32, F16)
+SINGE_PAGED_COMBINE_KERNEL(singe_paged_attention_combine_f16_i64, kCsrI64, F16)
+
+#define SINGE_PAGED_ATTENTION_KERNEL(NAME, SOFTCAP, FORM, GROUPED, ROTATE, HALF)                           \
     extern "C" __global__ __launch_bounds__(256, 2) void NAME(PagedAttentionArgs args) {                    \
         __shared__ __attribute__((aligned(1024))) unsigned char paged_lds[prefill::kStagedLdsBytes];        \
-        paged_attention_body<SOFTCAP, FORM, GROUPED, ROTATE>(args, paged_lds);                             \
+        paged_attention_body<SOFTCAP, FORM, GROUPED, ROTATE, prefill::HALF>(args, paged_lds);              \
     }
 
 // _p16: the page size is a power of two of at least 16 keys (page ids on the scalar unit).
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i32, false, kCsrI32, false, false)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i64, false, kCsrI64, false, false)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i32, true, kCsrI32, false, false)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i64, true, kCsrI64, false, false)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i32_p16, false, kCsrI32, true, false)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i64_p16, false, kCsrI64, true, false)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i32_p16, true, kCsrI32, true, false)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i64_p16, true, kCsrI64, true, false)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i32, false, kCsrI32, false, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i64, false, kCsrI64, false, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i32, true, kCsrI32, false, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i64, true, kCsrI64, false, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i32_p16, false, kCsrI32, true, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i64_p16, false, kCsrI64, true, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i32_p16, true, kCsrI32, true, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i64_p16, true, kCsrI64, true, false, Bf16)
 // paged_kv_prefill_attention_bf16 of the singe-kernel surface: same gather, block-table paging.
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_bf16_d128, false, kTable, false, false)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_bf16_d128_p16, false, kTable, true, false)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_bf16_d128, false, kTable, false, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_bf16_d128_p16, false, kTable, true, false, Bf16)
 // rotary_paged_attention: the query is normalised and rotated on its way into the registers.
-SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i32, false, kCsrI32, false, true)
-SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i64, false, kCsrI64, false, true)
-SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i32_p16, false, kCsrI32, true, true)
-SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i64_p16, false, kCsrI64, true, true)
+SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i32, false, kCsrI32, false, true, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i64, false, kCsrI64, false, true, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i32_p16, false, kCsrI32, true, true, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i64_p16, false, kCsrI64, true, true, Bf16)
+// f16 operands: the same kernels on v_mfma_f32_32x32x16_f16.
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_f16_d128_i32, false, kCsrI32, false, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_f16_d128_i64, false, kCsrI64, false, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_f16_d128_softcap_i32, true, kCsrI32, false, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_f16_d128_softcap_i64, true, kCsrI64, false, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_f16_d128_i32_p16, false, kCsrI32, true, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_f16_d128_i64_p16, false, kCsrI64, true, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_f16_d128_softcap_i32_p16, true, kCsrI32, true, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_f16_d128_softcap_i64_p16, true, kCsrI64, true, false, F16)

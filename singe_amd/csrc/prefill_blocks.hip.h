@@ -4,7 +4,7 @@
 // Everything is kept transposed so the softmax weights never leave registers (see prefill_core.hip.h for
 // the register layouts, which this file shares):
 //
-//   S^T[key, query] = K . Q^T      v_mfma_f32_32x32x16_bf16, A = K rows from LDS, B = the wave's Q^T;
+//   S^T[key, query] = K . Q^T      v_mfma_f32_32x32x16_bf16 (or _f16), A = K rows from LDS, B = the wave's Q^T;
 //   O^T[dim, query] += V^T . P^T   A = V^T through ds_read_b64_tr_b16, B = P^T packed from the S^T registers.
 //
 // Tiles of 64 keys reach LDS straight from global memory (global_load_lds_dwordx4: lane l of a wave puts
@@ -53,7 +53,8 @@ SINGE_DEVICE ReadOffsets read_offsets(unsigned int lane) {
 
 // Scores of the wave's 32 queries against the 32 keys of the block at `keys` (LDS byte address of the
 // block's first row).  The products run on while the caller does other work.
-SINGE_DEVICE void score_block(f32x16_t& scores, const bf16x8_t (&q)[8], const unsigned char* keys, const ReadOffsets& offsets) {
+template <class Half>
+SINGE_DEVICE void score_block(Half half, f32x16_t& scores, const uint4 (&q)[8], const unsigned char* keys, const ReadOffsets& offsets) {
     f32x16_t s;
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = 0.0f;
@@ -62,7 +63,7 @@ SINGE_DEVICE void score_block(f32x16_t& scores, const bf16x8_t (&q)[8], const un
     for (int step = 0; step < 8; ++step) operand[step] = *reinterpret_cast<const uint4*>(keys + offsets.key(step));
 #pragma unroll
     for (int step = 0; step < 8; ++step)
-        s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, operand[step]), q[step], s, 0, 0, 0);
+        s = mma(half, operand[step], q[step], s);
     scores = s;
 }
 
@@ -107,9 +108,9 @@ SINGE_DEVICE float begin_block(RowState& state, f32x16_t& s, unsigned int hi, fl
 //               are computed here (`next_keys` is not read), on return those of the block at `after_keys`, each
 //               read as soon as the product that used its register has been issued, a whole block before
 //               its use.  Otherwise the operands are read from `next_keys` at the start of the call.
-template <bool NEXT, bool AHEAD = false>
-SINGE_DEVICE void finish_block(RowState& state, f32x16_t& s, float factor, float shift, const unsigned char* values,
-                               const ReadOffsets& offsets, f32x16_t& next, const bf16x8_t (&q)[8], const unsigned char* next_keys,
+template <bool NEXT, bool AHEAD = false, class Half>
+SINGE_DEVICE void finish_block(Half half, RowState& state, f32x16_t& s, float factor, float shift, const unsigned char* values,
+                               const ReadOffsets& offsets, f32x16_t& next, const uint4 (&q)[8], const unsigned char* next_keys,
                                uint4 (&operand)[8], const unsigned char* after_keys) {
     typedef v4i16_t __attribute__((address_space(3))) * lds_v4_t;
     if constexpr (NEXT && !AHEAD) {
@@ -139,7 +140,7 @@ SINGE_DEVICE void finish_block(RowState& state, f32x16_t& s, float factor, float
             }
         }
         if constexpr (NEXT) {
-            upcoming = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, operand[step]), q[step], upcoming, 0, 0, 0);
+            upcoming = mma(half, operand[step], q[step], upcoming);
             if constexpr (AHEAD) operand[step] = *reinterpret_cast<const uint4*>(after_keys + offsets.key(step));
         }
         s[2 * step] = fast_exp2(fmaf(s[2 * step], factor, shift));
@@ -150,21 +151,20 @@ SINGE_DEVICE void finish_block(RowState& state, f32x16_t& s, float factor, float
     // O^T += V^T . P^T, 16 keys per MFMA: registers 8j .. 8j+7 are keys 16j + {0..3, 8..11} + 4hi.
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        const uint4 weights = make_uint4(pack_pair(s[8 * j + 0], s[8 * j + 1]), pack_pair(s[8 * j + 2], s[8 * j + 3]),
-                                         pack_pair(s[8 * j + 4], s[8 * j + 5]), pack_pair(s[8 * j + 6], s[8 * j + 7]));
+        const uint4 weights = make_uint4(pack_pair(half, s[8 * j + 0], s[8 * j + 1]), pack_pair(half, s[8 * j + 2], s[8 * j + 3]),
+                                         pack_pair(half, s[8 * j + 4], s[8 * j + 5]), pack_pair(half, s[8 * j + 6], s[8 * j + 7]));
 #pragma unroll
         for (int db = 0; db < 4; ++db)
-            state.out[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, j == 0 ? first[db] : second[db]),
-                                                              __builtin_bit_cast(bf16x8_t, weights), state.out[db], 0, 0, 0);
+            state.out[db] = mma(half, __builtin_bit_cast(uint4, j == 0 ? first[db] : second[db]), weights, state.out[db]);
     }
     if constexpr (NEXT) next = upcoming;
 }
 
-template <bool NEXT>
-SINGE_DEVICE void finish_block(RowState& state, f32x16_t& s, float factor, float shift, const unsigned char* values,
-                               const ReadOffsets& offsets, f32x16_t& next, const bf16x8_t (&q)[8], const unsigned char* next_keys) {
+template <bool NEXT, class Half>
+SINGE_DEVICE void finish_block(Half half, RowState& state, f32x16_t& s, float factor, float shift, const unsigned char* values,
+                               const ReadOffsets& offsets, f32x16_t& next, const uint4 (&q)[8], const unsigned char* next_keys) {
     uint4 operand[8];
-    finish_block<NEXT, false>(state, s, factor, shift, values, offsets, next, q, next_keys, operand, next_keys);
+    finish_block<NEXT, false>(half, state, s, factor, shift, values, offsets, next, q, next_keys, operand, next_keys);
 }
 
 // The stages of a tile's iteration, as the tile functions below take them.  The functions' pointer
@@ -188,17 +188,17 @@ SINGE_DEVICE void loads_landed() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmc
 // iteration's loads, then both blocks are folded while the scores of the block after each are computed.
 // With AHEAD the K operands of those products are read a block early and carried in `operand`: those of the
 // tile's second block on entry (read_key_operands before the first tile), of the next tile's on return.
-template <bool AHEAD, class Issue>
-SINGE_DEVICE void fold_interior_tile(RowState& state, f32x16_t& scores, uint4 (&operand)[8], const bf16x8_t (&q)[8],
+template <bool AHEAD, class Half, class Issue>
+SINGE_DEVICE void fold_interior_tile(Half half, RowState& state, f32x16_t& scores, uint4 (&operand)[8], const uint4 (&q)[8],
                                      const ReadOffsets& offsets, unsigned int hi, float factor, const unsigned char* __restrict__ keys,
                                      const unsigned char* __restrict__ next_keys, const unsigned char* __restrict__ values,
                                      unsigned char* __restrict__ key_dest, unsigned char* __restrict__ value_dest, Issue&& issue) {
     issue(key_dest, value_dest);
     const float shift_even = begin_block(state, scores, hi, factor, false, [](unsigned int) { return false; });
-    finish_block<true, AHEAD>(state, scores, factor, shift_even, values, offsets, scores, q, keys + kBlockBytes, operand, next_keys);
+    finish_block<true, AHEAD>(half, state, scores, factor, shift_even, values, offsets, scores, q, keys + kBlockBytes, operand, next_keys);
     __builtin_amdgcn_sched_barrier(0);  // keeps the second block's operand reads out of the first block's registers
     const float shift_odd = begin_block(state, scores, hi, factor, false, [](unsigned int) { return false; });
-    finish_block<true, AHEAD>(state, scores, factor, shift_odd, values + kBlockBytes, offsets, scores, q, next_keys, operand,
+    finish_block<true, AHEAD>(half, state, scores, factor, shift_odd, values + kBlockBytes, offsets, scores, q, next_keys, operand,
                               next_keys + kBlockBytes);
 }
 
@@ -210,18 +210,18 @@ SINGE_DEVICE void read_key_operands(uint4 (&operand)[8], const unsigned char* ke
 
 // Any other tile: the same steps one after the other, each only if the wave still has that block;
 // fold(block, scores, values) applies the masks and folds one block.
-template <class Issue, class Fold>
-SINGE_DEVICE void fold_edge_tile(f32x16_t& scores, const bf16x8_t (&q)[8], const ReadOffsets& offsets, unsigned int block,
+template <class Half, class Issue, class Fold>
+SINGE_DEVICE void fold_edge_tile(Half half, f32x16_t& scores, const uint4 (&q)[8], const ReadOffsets& offsets, unsigned int block,
                                  unsigned int wave_blocks, const unsigned char* __restrict__ keys,
                                  const unsigned char* __restrict__ next_keys, const unsigned char* __restrict__ values,
                                  unsigned char* __restrict__ key_dest, unsigned char* __restrict__ value_dest, Issue&& issue, Fold&& fold) {
     issue(key_dest, value_dest);
     if (block < wave_blocks) fold(block, scores, values);
     if (block + 1 < wave_blocks) {
-        score_block(scores, q, keys + kBlockBytes, offsets);
+        score_block(half, scores, q, keys + kBlockBytes, offsets);
         fold(block + 1, scores, values + kBlockBytes);
     }
-    if (block + 2 < wave_blocks) score_block(scores, q, next_keys, offsets);
+    if (block + 2 < wave_blocks) score_block(half, scores, q, next_keys, offsets);
 }
 
 }  // namespace prefill

@@ -61,9 +61,31 @@ SINGE_DEVICE float max3(float a, float b, float c) {
     return result;
 }
 
-SINGE_DEVICE unsigned int pack_pair(float lo, float hi) {
+// The 16-bit storage type of Q, K, V, P and the output: a tag the functions below are overloaded on.  The
+// operands travel as bit patterns (uint4 = eight halves); only the product and the rounding differ.
+struct Bf16 {};
+struct F16 {};
+
+typedef _Float16 f16x2v_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8v_t __attribute__((ext_vector_type(8)));
+
+// Two f32 values rounded to nearest even and packed, low half first.
+SINGE_DEVICE unsigned int pack_pair(Bf16, float lo, float hi) {
     f32x2v_t both = {lo, hi};
     return __builtin_bit_cast(unsigned int, __builtin_convertvector(both, bf16x2v_t));
+}
+SINGE_DEVICE unsigned int pack_pair(F16, float lo, float hi) {
+    f32x2v_t both = {lo, hi};
+    return __builtin_bit_cast(unsigned int, __builtin_convertvector(both, f16x2v_t));
+}
+SINGE_DEVICE unsigned int pack_pair(float lo, float hi) { return pack_pair(Bf16{}, lo, hi); }
+
+// D = A . B + C on the matrix core: 32 x 32 outputs, sixteen values of the contracted index per lane pair.
+SINGE_DEVICE f32x16_t mma(Bf16, uint4 a, uint4 b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+SINGE_DEVICE f32x16_t mma(F16, uint4 a, uint4 b, f32x16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8v_t, a), __builtin_bit_cast(f16x8v_t, b), c, 0, 0, 0);
 }
 
 // How far (log2 units) a row's maximum may run ahead of the reference point its weights are scaled

@@ -313,6 +313,31 @@ def fmha_prefill_lse_bf16(stream, out: torch.Tensor, lse: torch.Tensor, query: t
     _native.check(status, "fmha_prefill_lse_bf16")
 
 
+def fmha_prefill_f16(stream, out: torch.Tensor, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                     config: FmhaPrefillConfig) -> None:
+    """fmha_prefill_f16 (fmha.rs:692-742)."""
+    for tensor, name in ((out, "out"), (query, "query"), (key, "key"), (value, "value")):
+        _require(tensor, torch.float16, name)
+    c = config._c()
+    status = _native.lib().singe_hip_fmha_prefill_f16(
+        _stream_handle(stream), _ptr(out), out.numel(), _ptr(query), query.numel(), _ptr(key), key.numel(),
+        _ptr(value), value.numel(), ctypes.byref(c))
+    _native.check(status, "fmha_prefill_f16")
+
+
+def fmha_prefill_lse_f16(stream, out: torch.Tensor, lse: torch.Tensor, query: torch.Tensor, key: torch.Tensor,
+                         value: torch.Tensor, config: FmhaPrefillConfig) -> None:
+    """fmha_prefill_lse_f16 (fmha.rs:584-636): also writes lse [batch, heads, query_len], natural log."""
+    for tensor, name in ((out, "out"), (query, "query"), (key, "key"), (value, "value")):
+        _require(tensor, torch.float16, name)
+    _require(lse, torch.float32, "lse")
+    c = config._c()
+    status = _native.lib().singe_hip_fmha_prefill_lse_f16(
+        _stream_handle(stream), _ptr(out), out.numel(), _ptr(lse), lse.numel(), _ptr(query), query.numel(),
+        _ptr(key), key.numel(), _ptr(value), value.numel(), ctypes.byref(c))
+    _native.check(status, "fmha_prefill_lse_f16")
+
+
 def fmha_prefill_f32(stream, out: torch.Tensor, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
                      config: FmhaPrefillConfig) -> None:
     """fmha_prefill_f32 (fmha.rs:146-190): any head_dim up to 256, any strides."""

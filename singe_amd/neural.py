@@ -190,11 +190,13 @@ def paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: t
     # scratch: ``scratch`` is a uint8 device tensor, True for this module's own per-device buffer (calls on
     # different streams must then not overlap), or False for none.
     wanted = 0
-    if query.dtype == torch.bfloat16 and scratch is not False:
+    if query.dtype in (torch.bfloat16, torch.float16) and scratch is not False:
         wanted = int(_native.lib().singe_hip_paged_attention_scratch_bytes(ctypes.byref(problem)))
     if wanted > 0:
         lent = _scratch_for(query.device, wanted) if scratch is True else scratch
-        code = _native.lib().singe_hip_paged_attention_scratch_bf16(
+        with_scratch = (_native.lib().singe_hip_paged_attention_scratch_bf16 if query.dtype == torch.bfloat16
+                        else _native.lib().singe_hip_paged_attention_scratch_f16)
+        code = with_scratch(
             handle, query.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), paging.query_offsets.data_ptr(),
             paging.page_offsets.data_ptr(), paging.pages.data_ptr(), paging.last_page_lengths.data_ptr(),
             output.data_ptr(), lse.data_ptr(), status.data_ptr(), lent.data_ptr(), lent.numel(), ctypes.byref(problem))
