@@ -42,7 +42,11 @@ typedef enum SingeHipStatus {
     SINGE_HIP_KERNEL_NOT_PREPARED = 7,   /* Error::KernelNotPrepared: code object missing or not loadable */
     SINGE_HIP_UNSUPPORTED_CONFIGURATION = 8, /* Error::UnsupportedConfiguration { op, reason } */
     SINGE_HIP_INVALID_ARGUMENT = 9,      /* singe::Error::InvalidArgument (shape / dtype rules of the singe op) */
-    SINGE_HIP_RUNTIME_UNAVAILABLE = 10   /* the HIP runtime library could not be opened */
+    SINGE_HIP_RUNTIME_UNAVAILABLE = 10,  /* the HIP runtime library could not be opened */
+    SINGE_HIP_TUNE_CACHE_MISS = 11,      /* Error::TuneCacheMiss { op }: TuningChoice::Cached without a cached entry */
+    SINGE_HIP_AUTOTUNE_DURING_CAPTURE = 12, /* Error::AutotuneDuringCapture { op } */
+    SINGE_HIP_NO_TUNE_CANDIDATES = 13,   /* Error::NoTuneCandidates { op } */
+    SINGE_HIP_NO_SUCCESSFUL_TUNE_CANDIDATES = 14 /* Error::NoSuccessfulTuneCandidates { op } */
 } SingeHipStatus;
 
 /* Details of the last non-zero status returned on the calling thread. */
@@ -537,6 +541,127 @@ SINGE_HIP_API int32_t singe_hip_splitk_reduce_f32(
     const float* attn_splitk, size_t attn_splitk_len,
     const float* lse_splitk, size_t lse_splitk_len,
     const SingeSplitKReduceConfig* config);
+
+/* ---- dense f32 decode with split keys -----------------------------------------------------------------
+ * The reference's split-KV convention (singe-kernel/src/cuda/attention/fmha.rs:1074-1250): a split kernel
+ * writes one normalised partial output and one natural-log LSE per (batch, head, split) into scratch the
+ * caller supplies, and splitk_reduce_f32 (above) combines them.  query / out [batch, heads, dim], key / value
+ * [batch, key_len, kv_heads, dim], all f32, through element strides.  head_dim 4, 8, 16, 32, 64 (the reference's
+ * set, cutile/attention/splitk.rs:124-139) and 128, 256; other widths give SINGE_HIP_UNSUPPORTED_WIDTH. */
+
+/* Mirrors FmhaDecodeConfig (mod.rs:366-383); FmhaDecodeConfig::contiguous (mod.rs:2233-2261) fills the strides. */
+typedef struct SingeFmhaDecodeConfig {
+    size_t batch;
+    size_t key_len;
+    size_t heads;
+    size_t kv_heads;
+    size_t head_dim;
+    size_t query_batch_stride;
+    size_t key_batch_stride;
+    size_t value_batch_stride;
+    size_t output_batch_stride;
+    size_t query_head_stride;
+    size_t key_sequence_stride;
+    size_t value_sequence_stride;
+    size_t output_head_stride;
+    size_t key_head_stride;
+    size_t value_head_stride;
+    float scale;
+} SingeFmhaDecodeConfig;
+
+/* Mirrors FmhaDecodeSplitKConfig (mod.rs:401-423; contiguous form mod.rs:2662-2697): split s covers keys
+ * s * kv_len_per_split .. + kv_len_per_split, clipped to key_len. */
+typedef struct SingeFmhaDecodeSplitKConfig {
+    size_t batch;
+    size_t key_len;
+    size_t heads;
+    size_t kv_heads;
+    size_t splits;
+    size_t kv_len_per_split;
+    size_t head_dim;
+    size_t query_batch_stride;
+    size_t key_batch_stride;
+    size_t value_batch_stride;
+    size_t output_batch_stride;
+    size_t query_head_stride;
+    size_t key_sequence_stride;
+    size_t value_sequence_stride;
+    size_t output_head_stride;
+    size_t output_split_stride;
+    size_t key_head_stride;
+    size_t value_head_stride;
+    size_t lse_batch_stride;
+    size_t lse_head_stride;
+    float scale;
+} SingeFmhaDecodeSplitKConfig;
+
+/* fmha_decode_splitk_f32 (fmha.rs:1074-1118; kernel cutile/kernel/attention/local.rs:6127-6272): out[b, h, s, :]
+ * is the softmax-weighted mean of the slice's values (zeros for an empty slice), lse[b, h, s] = max + ln(sum)
+ * (-1e20 for an empty slice).  Lengths are checked as FmhaDecodeSplitKConfig::validate_lengths does
+ * (mod.rs:2699-2760). */
+SINGE_HIP_API int32_t singe_hip_fmha_decode_splitk_f32(
+    void* stream,
+    float* out, size_t out_len,
+    float* lse, size_t lse_len,
+    const float* query, size_t query_len,
+    const float* key, size_t key_len,
+    const float* value, size_t value_len,
+    const SingeFmhaDecodeSplitKConfig* config);
+
+/* TuningChoice<AttentionSplitKTuning> (singe-kernel/src/cuda/autotune.rs:77-89) and TuneOptions (:34-71,
+ * defaults warmup 1, repeats 5, no candidate limit; zero repeats count as one). */
+typedef enum SingeHipTuningChoice {
+    SINGE_HIP_TUNING_DEFAULT = 0,  /* min(max_splits, key_len) splits */
+    SINGE_HIP_TUNING_EXPLICIT = 1, /* explicit_splits; must be 1 .. min(max_splits, key_len) */
+    SINGE_HIP_TUNING_CACHED = 2,   /* the cached winner, SINGE_HIP_TUNE_CACHE_MISS without one */
+    SINGE_HIP_TUNING_TUNE = 3,     /* time the candidates on a cache miss, store and use the winner */
+    SINGE_HIP_TUNING_RETUNE = 4    /* always time again */
+} SingeHipTuningChoice;
+
+typedef struct SingeHipTuneOptions {
+    size_t warmup;
+    size_t repeats;
+    size_t max_candidates;
+} SingeHipTuneOptions;
+
+/* Mirrors FmhaDecodeSplitKReduceConfig (mod.rs:452-458). */
+typedef struct SingeFmhaDecodeSplitKReduceConfig {
+    SingeFmhaDecodeConfig decode;
+    size_t max_splits;
+    int32_t tuning;                /* SingeHipTuningChoice */
+    size_t explicit_splits;        /* SINGE_HIP_TUNING_EXPLICIT */
+    SingeHipTuneOptions options;   /* SINGE_HIP_TUNING_TUNE / RETUNE */
+} SingeFmhaDecodeSplitKReduceConfig;
+
+/* fmha_decode_splitk_reduce_f32 (fmha.rs:1155-1250): the split kernel into the caller's scratch, then the
+ * reduce.  attn_scratch holds at least batch * heads * min(max_splits, key_len) * head_dim elements laid out
+ * [batch, heads, splits, dim] for the split count in use, lse_scratch batch * heads * min(max_splits, key_len)
+ * laid out [batch, heads, splits] (mod.rs:2456-2539).  Timing candidates synchronises the stream's events and is
+ * refused while the stream is being captured (SINGE_HIP_AUTOTUNE_DURING_CAPTURE), also when the cache would
+ * have answered, as in the reference (fmha.rs:1203-1207); winners are cached per process and device, keyed
+ * by (batch, key_len, heads, kv_heads, head_dim, max_splits), and the winner is launched once more so `out`
+ * holds its result. */
+SINGE_HIP_API int32_t singe_hip_fmha_decode_splitk_reduce_f32(
+    void* stream,
+    float* out, size_t out_len,
+    float* attn_scratch, size_t attn_scratch_len,
+    float* lse_scratch, size_t lse_scratch_len,
+    const float* query, size_t query_len,
+    const float* key, size_t key_len,
+    const float* value, size_t value_len,
+    const SingeFmhaDecodeSplitKReduceConfig* config);
+
+/* attention_splitk_candidates (mod.rs:2364-2380): {1, 2, 4, 8, 16, 32, 64} up to min(max_splits, key_len), and
+ * that bound itself.  Writes at most `capacity` of them to `splits` (which may be NULL) and their number to
+ * `count`. */
+SINGE_HIP_API int32_t singe_hip_attention_splitk_candidates(
+    const SingeFmhaDecodeSplitKReduceConfig* config, size_t* splits, size_t capacity, size_t* count);
+
+/* The cached winner for this problem on the current device, 0 when there is none (autotune::cache().get,
+ * mod.rs:2432-2441); and MemoryTuneCache::clear. */
+SINGE_HIP_API int32_t singe_hip_fmha_decode_splitk_reduce_tuned_splits(
+    const SingeFmhaDecodeSplitKReduceConfig* config, size_t* splits);
+SINGE_HIP_API void singe_hip_clear_tune_cache(void);
 
 /* ---- latent (MLA) attention over paged caches --------------------------------------------------------
  * Tensor::paged_mla_attention / Operation::PagedMlaAttention (singe/src/backend/spec/neural/attention.rs:453-497;

@@ -222,6 +222,20 @@ def splitk_reduce_f32(attn, lse, *, batch, heads, splits, head_dim):
     return out.reshape(batch, heads, head_dim)
 
 
+def fmha_decode_splitk_f32(query, key, value, *, splits, kv_len_per_split, scale):
+    """singe-kernel/src/cuda/cutile/kernel/attention/local.rs:6127-6272.  query [B,H,D], key / value [B,S,G,D];
+    returns (out [B,H,splits,D], lse [B,H,splits] natural log)."""
+    query, key, value = _f32(query), _f32(key), _f32(value)
+    batch, heads, head_dim = query.shape
+    _, key_len, kv_heads, _ = key.shape
+    out = np.empty((batch, heads, splits, head_dim), dtype=np.float32)
+    lse = np.empty((batch, heads, splits), dtype=np.float32)
+    lib().oracle_fmha_decode_splitk_f32(_ptr(out), _ptr(lse), _ptr(query), _ptr(key), _ptr(value), _c_size(batch),
+                                        _c_size(key_len), _c_size(heads), _c_size(kv_heads), _c_size(splits),
+                                        _c_size(kv_len_per_split), _c_size(head_dim), ctypes.c_float(scale))
+    return out, lse
+
+
 # ---- singe surface --------------------------------------------------------------
 
 def scaled_dot_product_attention_f32(query, key, value, *, scale=None, causal=False, window=None,

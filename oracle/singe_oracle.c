@@ -466,6 +466,54 @@ ORACLE_API void oracle_splitk_reduce_f32(float *out, const float *attn, const fl
         }
 }
 
+/* singe-kernel/src/cuda/cutile/kernel/attention/local.rs:6127-6272  fmha_decode_splitk_f32 (the reference has
+ * no CPU form of this function; this restates its kernel, one output element at a time as the kernel does).
+ * query [batch, heads, dim], key / value [batch, key_len, kv_heads, dim], contiguous; split s covers keys
+ * s * per_split .. + per_split, clipped to key_len.  Two passes like the kernel: the maximum (starting from
+ * -1e20, strictly greater wins), then weights expf(score - max); score = (sum_d q_d * k_d) * scale with a
+ * multiply and an add per term.  out [batch, heads, splits, dim] = sum / denom, or 0 when denom is 0;
+ * lse [batch, heads, splits] = max + logf(denom), or -1e20 when denom is 0. */
+ORACLE_API void oracle_fmha_decode_splitk_f32(float *out, float *lse, const float *query, const float *key,
+                                              const float *value, size_t batch, size_t key_len, size_t heads,
+                                              size_t kv_heads, size_t splits, size_t per_split, size_t head_dim,
+                                              float scale) {
+    size_t group = heads / kv_heads;
+    for (size_t b = 0; b < batch; ++b)
+        for (size_t head = 0; head < heads; ++head)
+            for (size_t split = 0; split < splits; ++split) {
+                const float *q = query + (b * heads + head) * head_dim;
+                size_t kv_head = head / group, start = split * per_split;
+                float largest = -1.0e20f;
+                for (size_t offset = 0; offset < per_split; ++offset) {
+                    size_t k = start + offset;
+                    if (k >= key_len) continue;
+                    const float *row = key + ((b * key_len + k) * kv_heads + kv_head) * head_dim;
+                    float score = 0.0f;
+                    for (size_t d = 0; d < head_dim; ++d) score = score + q[d] * row[d];
+                    score = score * scale;
+                    if (score > largest) largest = score;
+                }
+                float denom = 0.0f;
+                float *o = out + ((b * heads + head) * splits + split) * head_dim;
+                for (size_t d = 0; d < head_dim; ++d) o[d] = 0.0f;
+                for (size_t offset = 0; offset < per_split; ++offset) {
+                    size_t k = start + offset;
+                    if (k >= key_len) continue;
+                    const float *row = key + ((b * key_len + k) * kv_heads + kv_head) * head_dim;
+                    const float *v = value + ((b * key_len + k) * kv_heads + kv_head) * head_dim;
+                    float score = 0.0f;
+                    for (size_t d = 0; d < head_dim; ++d) score = score + q[d] * row[d];
+                    score = score * scale;
+                    float weight = expf(score - largest);
+                    denom = denom + weight;
+                    for (size_t d = 0; d < head_dim; ++d) o[d] = o[d] + weight * v[d];
+                }
+                int has_keys = denom > 0.0f;
+                for (size_t d = 0; d < head_dim; ++d) o[d] = has_keys ? o[d] / denom : 0.0f;
+                lse[(b * heads + head) * splits + split] = has_keys ? largest + logf(denom) : -1.0e20f;
+            }
+}
+
 /* ---- singe: dense scaled-dot-product attention ----------------------------- */
 
 /* singe/src/backend/cpu/normalization/attention.rs:191-276

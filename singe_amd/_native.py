@@ -70,6 +70,32 @@ class SplitKReduceConfigC(ctypes.Structure):
         "lse_batch_stride", "lse_head_stride", "output_batch_stride", "output_head_stride")]
 
 
+_DECODE_FIELDS = ("batch", "key_len", "heads", "kv_heads", "head_dim", "query_batch_stride", "key_batch_stride",
+                  "value_batch_stride", "output_batch_stride", "query_head_stride", "key_sequence_stride",
+                  "value_sequence_stride", "output_head_stride", "key_head_stride", "value_head_stride")
+
+
+class FmhaDecodeConfigC(ctypes.Structure):
+    _fields_ = [(name, c_size) for name in _DECODE_FIELDS] + [("scale", ctypes.c_float)]
+
+
+class FmhaDecodeSplitKConfigC(ctypes.Structure):
+    _fields_ = [(name, c_size) for name in (
+        "batch", "key_len", "heads", "kv_heads", "splits", "kv_len_per_split", "head_dim", "query_batch_stride",
+        "key_batch_stride", "value_batch_stride", "output_batch_stride", "query_head_stride", "key_sequence_stride",
+        "value_sequence_stride", "output_head_stride", "output_split_stride", "key_head_stride", "value_head_stride",
+        "lse_batch_stride", "lse_head_stride")] + [("scale", ctypes.c_float)]
+
+
+class TuneOptionsC(ctypes.Structure):
+    _fields_ = [("warmup", c_size), ("repeats", c_size), ("max_candidates", c_size)]
+
+
+class FmhaDecodeSplitKReduceConfigC(ctypes.Structure):
+    _fields_ = [("decode", FmhaDecodeConfigC), ("max_splits", c_size), ("tuning", ctypes.c_int32),
+                ("explicit_splits", c_size), ("options", TuneOptionsC)]
+
+
 class PagedMlaAttentionProblemC(ctypes.Structure):
     _fields_ = [("tokens", ctypes.c_int64), ("heads", ctypes.c_int64), ("latent_dim", ctypes.c_int64),
                 ("position_dim", ctypes.c_int64), ("page_size", ctypes.c_int64), ("sequences", ctypes.c_int64),
@@ -199,6 +225,19 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_splitk_reduce_f32.argtypes = [c_void, c_void, c_size, c_void, c_size, c_void, c_size,
                                                    ctypes.POINTER(SplitKReduceConfigC)]
     handle.singe_hip_splitk_reduce_f32.restype = i32
+    split = ctypes.POINTER(FmhaDecodeSplitKConfigC)
+    split_reduce = ctypes.POINTER(FmhaDecodeSplitKReduceConfigC)
+    handle.singe_hip_fmha_decode_splitk_f32.argtypes = [c_void] + [c_void, c_size] * 5 + [split]
+    handle.singe_hip_fmha_decode_splitk_f32.restype = i32
+    handle.singe_hip_fmha_decode_splitk_reduce_f32.argtypes = [c_void] + [c_void, c_size] * 6 + [split_reduce]
+    handle.singe_hip_fmha_decode_splitk_reduce_f32.restype = i32
+    handle.singe_hip_attention_splitk_candidates.argtypes = [split_reduce, ctypes.POINTER(c_size), c_size,
+                                                             ctypes.POINTER(c_size)]
+    handle.singe_hip_attention_splitk_candidates.restype = i32
+    handle.singe_hip_fmha_decode_splitk_reduce_tuned_splits.argtypes = [split_reduce, ctypes.POINTER(c_size)]
+    handle.singe_hip_fmha_decode_splitk_reduce_tuned_splits.restype = i32
+    handle.singe_hip_clear_tune_cache.argtypes = []
+    handle.singe_hip_clear_tune_cache.restype = None
     handle.singe_hip_rotary_cache_write.argtypes = [c_void] * 14 + [ctypes.POINTER(RotaryCacheProblemC)]
     handle.singe_hip_rotary_cache_write.restype = i32
     handle.singe_hip_paging_indices.argtypes = [c_void] * 10 + [ctypes.POINTER(PagingIndicesProblemC)]
@@ -228,5 +267,9 @@ def check(status: int, op: str = "") -> None:
         8: lambda: error.UnsupportedConfiguration(f"unsupported configuration for {op}: {name}"),
         9: lambda: error.InvalidArgument(f"{op} {name}"),
         10: lambda: error.KernelNotPrepared("the HIP runtime library could not be opened"),
+        11: lambda: error.TuneCacheMiss(f"tune cache miss for {name or op}"),
+        12: lambda: error.AutotuneDuringCapture(f"autotune during stream capture for {name or op}"),
+        13: lambda: error.NoTuneCandidates(f"no tune candidates for {name or op}"),
+        14: lambda: error.NoTuneCandidates(f"no tune candidate completed for {name or op}"),
     }
     raise table.get(status, lambda: error.Error(f"status {status}"))()

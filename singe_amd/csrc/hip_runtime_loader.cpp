@@ -42,6 +42,12 @@ void load() {
     ok &= resolve(handle, "hipModuleGetFunction", g_runtime.hipModuleGetFunction);
     ok &= resolve(handle, "hipModuleLaunchKernel", g_runtime.hipModuleLaunchKernel);
     ok &= resolve(handle, "hipGetErrorString", g_runtime.hipGetErrorString);
+    ok &= resolve(handle, "hipEventCreate", g_runtime.hipEventCreate);
+    ok &= resolve(handle, "hipEventDestroy", g_runtime.hipEventDestroy);
+    ok &= resolve(handle, "hipEventRecord", g_runtime.hipEventRecord);
+    ok &= resolve(handle, "hipEventSynchronize", g_runtime.hipEventSynchronize);
+    ok &= resolve(handle, "hipEventElapsedTime", g_runtime.hipEventElapsedTime);
+    ok &= resolve(handle, "hipStreamIsCapturing", g_runtime.hipStreamIsCapturing);
     g_ready = ok;
 }
 

@@ -25,6 +25,13 @@ struct HipRuntime {
     hipError_t (*hipModuleLaunchKernel)(hipFunction_t, unsigned, unsigned, unsigned, unsigned, unsigned, unsigned,
                                         unsigned, hipStream_t, void**, void**);
     const char* (*hipGetErrorString)(hipError_t);
+    // Timing and capture queries, for the one entry point that tunes itself.
+    hipError_t (*hipEventCreate)(void**);
+    hipError_t (*hipEventDestroy)(void*);
+    hipError_t (*hipEventRecord)(void*, hipStream_t);
+    hipError_t (*hipEventSynchronize)(void*);
+    hipError_t (*hipEventElapsedTime)(float*, void*, void*);
+    hipError_t (*hipStreamIsCapturing)(hipStream_t, int*);
 };
 
 // Returns the resolved table, or nullptr when no HIP runtime can be opened.

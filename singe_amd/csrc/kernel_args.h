@@ -137,6 +137,21 @@ struct SplitKReduceArgs {
     uint32_t batch, heads, splits, head_dim;
 };
 
+// singe_fmha_decode_splitk_f32_d*: one query per (batch, head) over a slice of the keys.
+struct FmhaDecodeSplitKArgs {
+    float* out;          // [batch, heads, splits, dim] through the strides below
+    float* lse;          // [batch, heads, splits] natural log
+    const float* query;  // [batch, heads, dim]
+    const float* key;    // [batch, key_len, kv_heads, dim]
+    const float* value;
+    uint64_t query_batch_stride, key_batch_stride, value_batch_stride, output_batch_stride;
+    uint64_t query_head_stride, key_sequence_stride, value_sequence_stride, output_head_stride, output_split_stride;
+    uint64_t key_head_stride, value_head_stride, lse_batch_stride, lse_head_stride;
+    uint32_t batch, key_len, heads, kv_heads, splits, kv_len_per_split;
+    uint32_t aligned;    // every row of query, key and value starts on a 16-byte boundary
+    float scale;
+};
+
 // Element types of the general (any head dimension) kernels.
 enum SingeElement : uint32_t { kElementF32 = 0, kElementBf16 = 1, kElementF16 = 2 };
 

@@ -35,6 +35,9 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_rotary_paged_attention_bf16_d128_i32", "singe_rotary_paged_attention_bf16_d128_i64",
     "singe_rotary_paged_attention_bf16_d128_i32_p16", "singe_rotary_paged_attention_bf16_d128_i64_p16",
     "singe_splitk_reduce_f32",
+    "singe_fmha_decode_splitk_f32_d4", "singe_fmha_decode_splitk_f32_d8", "singe_fmha_decode_splitk_f32_d16",
+    "singe_fmha_decode_splitk_f32_d32", "singe_fmha_decode_splitk_f32_d64", "singe_fmha_decode_splitk_f32_d128",
+    "singe_fmha_decode_splitk_f32_d256",
     "singe_rotary_cache_write_f32", "singe_rotary_cache_write_bf16", "singe_rotary_cache_write_f16",
     "singe_paging_indices_i32", "singe_paging_indices_i64",
     "singe_paged_mla_attention_general_f32", "singe_paged_mla_attention_general_bf16", "singe_paged_mla_attention_general_f16",
@@ -168,6 +171,10 @@ const char* singe_hip_status_string(int32_t status) {
         case SINGE_HIP_UNSUPPORTED_CONFIGURATION: return "unsupported configuration";
         case SINGE_HIP_INVALID_ARGUMENT: return "invalid argument";
         case SINGE_HIP_RUNTIME_UNAVAILABLE: return "hip runtime unavailable";
+        case SINGE_HIP_TUNE_CACHE_MISS: return "tune cache miss";
+        case SINGE_HIP_AUTOTUNE_DURING_CAPTURE: return "autotune during stream capture";
+        case SINGE_HIP_NO_TUNE_CANDIDATES: return "no tune candidates";
+        case SINGE_HIP_NO_SUCCESSFUL_TUNE_CANDIDATES: return "no tune candidate completed";
         default: break;
     }
     if (status < 0) {

@@ -26,6 +26,8 @@ enum KernelId : int {
     // fused query rotation: + (i64 indices) + 2 * (page size a power of two of at least 16 keys)
     kRotaryPagedAttention = kPagedAttentionF16 + 8, kRotaryPagedAttentionI64, kRotaryPagedAttentionP16, kRotaryPagedAttentionI64P16,
     kSplitKReduce,
+    // dense f32 split-KV decode: + head dimension (4, 8, 16, 32, 64, 128, 256)
+    kFmhaDecodeSplitK, kFmhaDecodeSplitKLast = kFmhaDecodeSplitK + 6,
     kRotaryCacheF32, kRotaryCacheBf16, kRotaryCacheF16,
     kPagingIndicesI32, kPagingIndicesI64,
     // latent (MLA) attention: + element (f32, bf16, f16)

@@ -59,6 +59,18 @@ class IndexOutOfBounds(Error):
     """A paging value addresses outside its buffers (singe::Error::IndexOutOfBounds)."""
 
 
+class TuneCacheMiss(Error):
+    """TuningChoice::Cached found no cached entry (Error::TuneCacheMiss)."""
+
+
+class AutotuneDuringCapture(Error):
+    """Candidates cannot be timed while the stream is being captured (Error::AutotuneDuringCapture)."""
+
+
+class NoTuneCandidates(Error):
+    """No candidate is left to time, or none completed (Error::NoTuneCandidates / NoSuccessfulTuneCandidates)."""
+
+
 class Hip(Error):
     """A HIP runtime call failed (the counterpart of Error::Cuda)."""
 

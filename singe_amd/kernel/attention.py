@@ -432,3 +432,228 @@ def splitk_reduce_f32(stream, out: torch.Tensor, attn_splitk: torch.Tensor, lse_
                                                        attn_splitk.numel(), _ptr(lse_splitk), lse_splitk.numel(),
                                                        ctypes.byref(c))
     _native.check(status, "splitk_reduce_f32")
+
+
+@dataclass(frozen=True)
+class FmhaDecodeConfig:
+    """FmhaDecodeConfig (mod.rs:366-383): one query per (batch, head); query / out [batch, heads, dim], key /
+    value [batch, key_len, kv_heads, dim]; strides in elements."""
+    batch: int
+    key_len: int
+    heads: int
+    kv_heads: int
+    head_dim: int
+    query_batch_stride: int
+    key_batch_stride: int
+    value_batch_stride: int
+    output_batch_stride: int
+    query_head_stride: int
+    key_sequence_stride: int
+    value_sequence_stride: int
+    output_head_stride: int
+    key_head_stride: int
+    value_head_stride: int
+    scale: float
+
+    @classmethod
+    def contiguous(cls, batch, key_len, heads, kv_heads, head_dim, scale) -> "FmhaDecodeConfig":
+        """mod.rs:2233-2261."""
+        q_features, kv_features = heads * head_dim, kv_heads * head_dim
+        return cls(batch, key_len, heads, kv_heads, head_dim, q_features, key_len * kv_features, key_len * kv_features,
+                   q_features, head_dim, kv_features, kv_features, head_dim, head_dim, head_dim, scale)
+
+    def _c(self) -> _native.FmhaDecodeConfigC:
+        return _native.FmhaDecodeConfigC(*(getattr(self, name) for name in _native._DECODE_FIELDS), self.scale)
+
+
+@dataclass(frozen=True)
+class FmhaDecodeSplitKConfig:
+    """FmhaDecodeSplitKConfig (mod.rs:401-423): the decode layout plus the split count, the keys per split and
+    where each split's partial output and LSE go."""
+    batch: int
+    key_len: int
+    heads: int
+    kv_heads: int
+    splits: int
+    kv_len_per_split: int
+    head_dim: int
+    query_batch_stride: int
+    key_batch_stride: int
+    value_batch_stride: int
+    output_batch_stride: int
+    query_head_stride: int
+    key_sequence_stride: int
+    value_sequence_stride: int
+    output_head_stride: int
+    output_split_stride: int
+    key_head_stride: int
+    value_head_stride: int
+    lse_batch_stride: int
+    lse_head_stride: int
+    scale: float
+
+    @classmethod
+    def contiguous(cls, batch, key_len, heads, kv_heads, splits, kv_len_per_split, head_dim, scale) -> "FmhaDecodeSplitKConfig":
+        """mod.rs:2662-2697: out [batch, heads, splits, dim], lse [batch, heads, splits]."""
+        q_features, kv_features, split_values = heads * head_dim, kv_heads * head_dim, splits * head_dim
+        return cls(batch, key_len, heads, kv_heads, splits, kv_len_per_split, head_dim, q_features,
+                   key_len * kv_features, key_len * kv_features, heads * split_values, head_dim, kv_features,
+                   kv_features, split_values, head_dim, head_dim, head_dim, heads * splits, splits, scale)
+
+    def _c(self) -> _native.FmhaDecodeSplitKConfigC:
+        names = [name for name, _ in _native.FmhaDecodeSplitKConfigC._fields_]
+        return _native.FmhaDecodeSplitKConfigC(*(getattr(self, name) for name in names))
+
+
+def fmha_decode_splitk_f32(stream, out: torch.Tensor, lse: torch.Tensor, query: torch.Tensor, key: torch.Tensor,
+                           value: torch.Tensor, config: FmhaDecodeSplitKConfig) -> None:
+    """fmha_decode_splitk_f32 (fmha.rs:1074-1118): per split a normalised partial output and a natural-log LSE
+    (zeros and -1e20 for a split without keys)."""
+    for tensor, name in ((out, "out"), (lse, "lse"), (query, "query"), (key, "key"), (value, "value")):
+        _require(tensor, torch.float32, name)
+    c = config._c()
+    status = _native.lib().singe_hip_fmha_decode_splitk_f32(
+        _stream_handle(stream), _ptr(out), out.numel(), _ptr(lse), lse.numel(), _ptr(query), query.numel(), _ptr(key),
+        key.numel(), _ptr(value), value.numel(), ctypes.byref(c))
+    _native.check(status, "fmha_decode_splitk_f32")
+
+
+@dataclass(frozen=True)
+class AttentionSplitKTuning:
+    """AttentionSplitKTuning (mod.rs:442-450)."""
+    splits: int
+
+    @classmethod
+    def create(cls, splits: int) -> "AttentionSplitKTuning":
+        return cls(splits)
+
+
+@dataclass(frozen=True)
+class TuneOptions:
+    """TuneOptions (singe-kernel/src/cuda/autotune.rs:34-71): zero repeats count as one."""
+    warmup: int = 1
+    repeats: int = 5
+    max_candidates: int = 2**64 - 1
+
+    @classmethod
+    def create(cls, warmup: int, repeats: int, max_candidates: int) -> "TuneOptions":
+        return cls(warmup, repeats, max_candidates)
+
+
+@dataclass(frozen=True)
+class TuningChoice:
+    """TuningChoice<T> (autotune.rs:77-89): ``kind`` is one of the class constants; ``value`` the explicit
+    tuning or the options of Tune / Retune."""
+    kind: int = 0
+    value: object = None
+
+    DEFAULT, EXPLICIT, CACHED, TUNE, RETUNE = range(5)
+
+    @classmethod
+    def Default(cls) -> "TuningChoice":
+        return cls(cls.DEFAULT)
+
+    @classmethod
+    def Explicit(cls, tuning: AttentionSplitKTuning) -> "TuningChoice":
+        return cls(cls.EXPLICIT, tuning)
+
+    @classmethod
+    def Cached(cls) -> "TuningChoice":
+        return cls(cls.CACHED)
+
+    @classmethod
+    def Tune(cls, options: TuneOptions) -> "TuningChoice":
+        return cls(cls.TUNE, options)
+
+    @classmethod
+    def Retune(cls, options: TuneOptions) -> "TuningChoice":
+        return cls(cls.RETUNE, options)
+
+
+@dataclass(frozen=True)
+class FmhaDecodeSplitKReduceConfig:
+    """FmhaDecodeSplitKReduceConfig (mod.rs:452-505)."""
+    decode: FmhaDecodeConfig
+    max_splits: int
+    tuning: TuningChoice = TuningChoice()
+
+    @classmethod
+    def contiguous(cls, batch, key_len, heads, kv_heads, head_dim, max_splits, scale) -> "FmhaDecodeSplitKReduceConfig":
+        """mod.rs:461-478: validates, unlike the other ``contiguous`` builders
+        (validate_fmha_decode_splitk_reduce_config, mod.rs:2554-2560)."""
+        decode = FmhaDecodeConfig.contiguous(batch, key_len, heads, kv_heads, head_dim, scale)
+        extents = [getattr(decode, name) for name in _native._DECODE_FIELDS]
+        if any(extent == 0 for extent in extents) or not math.isfinite(scale) or heads % kv_heads != 0 or max_splits == 0:
+            raise error.InvalidLength("invalid length")
+        return cls(decode, max_splits)
+
+    def with_tuning(self, tuning: TuningChoice) -> "FmhaDecodeSplitKReduceConfig":
+        return FmhaDecodeSplitKReduceConfig(self.decode, self.max_splits, tuning)
+
+    def explicit_tuning(self, tuning: AttentionSplitKTuning) -> "FmhaDecodeSplitKReduceConfig":
+        return self.with_tuning(TuningChoice.Explicit(tuning))
+
+    def cached_tuning(self) -> "FmhaDecodeSplitKReduceConfig":
+        return self.with_tuning(TuningChoice.Cached())
+
+    def tune(self, options: TuneOptions) -> "FmhaDecodeSplitKReduceConfig":
+        return self.with_tuning(TuningChoice.Tune(options))
+
+    def retune(self, options: TuneOptions) -> "FmhaDecodeSplitKReduceConfig":
+        return self.with_tuning(TuningChoice.Retune(options))
+
+    def _c(self) -> _native.FmhaDecodeSplitKReduceConfigC:
+        explicit = self.tuning.value.splits if self.tuning.kind == TuningChoice.EXPLICIT else 0
+        options = self.tuning.value if self.tuning.kind in (TuningChoice.TUNE, TuningChoice.RETUNE) else TuneOptions()
+        return _native.FmhaDecodeSplitKReduceConfigC(
+            self.decode._c(), self.max_splits, self.tuning.kind, explicit,
+            _native.TuneOptionsC(options.warmup, options.repeats, min(options.max_candidates, 2**64 - 1)))
+
+
+def attention_splitk_candidates(config: FmhaDecodeSplitKReduceConfig) -> list:
+    """attention_splitk_candidates (mod.rs:2364-2380): the split counts tuning tries."""
+    c = config._c()
+    found = (_native.c_size * 16)()
+    count = _native.c_size(0)
+    _native.check(_native.lib().singe_hip_attention_splitk_candidates(ctypes.byref(c), found, 16, ctypes.byref(count)),
+                  "attention_splitk_candidates")
+    return [AttentionSplitKTuning(int(found[i])) for i in range(min(int(count.value), 16))]
+
+
+def fmha_decode_splitk_reduce_f32(stream, out: torch.Tensor, attn_scratch: torch.Tensor, lse_scratch: torch.Tensor,
+                                  query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                                  config: FmhaDecodeSplitKReduceConfig) -> None:
+    """fmha_decode_splitk_reduce_f32 (fmha.rs:1155-1250): the split kernel into the caller's scratch, then the
+    reduce, with the split count the config's TuningChoice asks for."""
+    for tensor, name in ((out, "out"), (attn_scratch, "attn_scratch"), (lse_scratch, "lse_scratch"), (query, "query"),
+                         (key, "key"), (value, "value")):
+        _require(tensor, torch.float32, name)
+    c = config._c()
+    status = _native.lib().singe_hip_fmha_decode_splitk_reduce_f32(
+        _stream_handle(stream), _ptr(out), out.numel(), _ptr(attn_scratch), attn_scratch.numel(), _ptr(lse_scratch),
+        lse_scratch.numel(), _ptr(query), query.numel(), _ptr(key), key.numel(), _ptr(value), value.numel(),
+        ctypes.byref(c))
+    _native.check(status, "fmha_decode_splitk_reduce_f32")
+
+
+def tune_fmha_decode_splitk_reduce_f32(stream, out: torch.Tensor, attn_scratch: torch.Tensor, lse_scratch: torch.Tensor,
+                                       query: torch.Tensor, key: torch.Tensor, value: torch.Tensor,
+                                       config: FmhaDecodeSplitKReduceConfig, options: TuneOptions) -> AttentionSplitKTuning:
+    """tune_fmha_decode_splitk_reduce_f32 (fmha.rs:1257-1313): times the candidates again, caches the winner and
+    returns it; ``out`` holds the winner's result."""
+    fmha_decode_splitk_reduce_f32(stream, out, attn_scratch, lse_scratch, query, key, value, config.retune(options))
+    return cached_fmha_decode_splitk_reduce_tuning(config)
+
+
+def cached_fmha_decode_splitk_reduce_tuning(config: FmhaDecodeSplitKReduceConfig):
+    """The cached winner for this problem on the current device, or None."""
+    c = config._c()
+    splits = _native.c_size(0)
+    _native.check(_native.lib().singe_hip_fmha_decode_splitk_reduce_tuned_splits(ctypes.byref(c), ctypes.byref(splits)),
+                  "fmha_decode_splitk_reduce_f32")
+    return AttentionSplitKTuning(int(splits.value)) if splits.value else None
+
+
+def clear_tune_cache() -> None:
+    """MemoryTuneCache::clear."""
+    _native.lib().singe_hip_clear_tune_cache()
