@@ -25,9 +25,11 @@
  *
  * Parity pinning: the reference holds no numeric fixture for
  * paged_kv_decode_attention_f32, paged_kv_prefill_attention_f32,
- * fmha_prefill_lse_f32, attend_paged or paged_mla_attention, and the Rust original cannot be
- * compiled in this image, so their last-ulp f32 outputs are pinned only by
- * construction plus closed forms and invariants (see tests/test_oracle.py);
+ * fmha_prefill_lse_f32, attend_paged, paged_mla_attention or fmha_decode_splitk_f32 (which
+ * has no CPU form in the reference at all: its restatement follows the GPU kernel), and the
+ * Rust original cannot be compiled in this image, so their last-ulp f32 outputs are "parity
+ * unpinned": pinned only by construction plus closed forms and invariants (see
+ * tests/test_oracle.py and tests/test_fmha_decode_splitk_cpu.py);
  * everything integer (gather offsets, lengths, the paging error contract),
  * the GQA head map, the causal direction, the fp8 and bf16 codecs are pinned
  * against the reference's own test vectors.
