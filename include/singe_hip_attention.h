@@ -542,6 +542,43 @@ SINGE_HIP_API int32_t singe_hip_splitk_reduce_f32(
     const float* lse_splitk, size_t lse_splitk_len,
     const SingeSplitKReduceConfig* config);
 
+/* ---- f32 forms of the two block-table ops -------------------------------------------------------------
+ * paged_kv_decode_attention_f32 and paged_kv_prefill_attention_f32 (singe-kernel/src/cuda/attention/paged.rs; CPU
+ * forms singe-kernel/src/cpu/attention.rs:1172-1246, 1248-1341), same operands, config structs and length checks
+ * as the bf16 entry points above, f32 throughout.  head_dim 4, 8, 16, 32, 64 (the reference's set for these
+ * kernels, cutile/attention/paged.rs:799-810) and 128, 256.  Vector-unit kernels: accuracy anchors at 1e-4, HBM
+ * bound for decode, not the matrix-core path.  A sequence length beyond what its table row can name is cut
+ * there and a table entry beyond the cache is read as the last block (the reference checks neither).
+ * Decode splits the keys of each (sequence, kv head) over workgroups and combines with the split-KV reduce;
+ * its scratch is caller-supplied: ..._f32_workspace_bytes(config), 16-byte aligned, no state between calls.
+ * Prefill writes every token row: zeros and an LSE of 0 for a token no sequence covers (what the CPU form's
+ * zero-filled outputs hold there), zeros and -1e20 for a covered row without visible keys. */
+SINGE_HIP_API size_t singe_hip_paged_kv_decode_attention_f32_workspace_bytes(const SingePagedKvDecodeAttentionConfig* config);
+
+SINGE_HIP_API int32_t singe_hip_paged_kv_decode_attention_f32(
+    void* stream,
+    float* out, size_t out_len,
+    const float* query, size_t query_len,
+    const float* key_cache, size_t key_cache_len,
+    const float* value_cache, size_t value_cache_len,
+    const int32_t* actual_seq_lens, size_t actual_seq_lens_len,
+    const uint32_t* block_table, size_t block_table_len,
+    void* workspace, size_t workspace_bytes,
+    const SingePagedKvDecodeAttentionConfig* config);
+
+SINGE_HIP_API int32_t singe_hip_paged_kv_prefill_attention_f32(
+    void* stream,
+    float* out, size_t out_len,
+    float* lse, size_t lse_len,
+    const float* query, size_t query_len,
+    const float* key_cache, size_t key_cache_len,
+    const float* value_cache, size_t value_cache_len,
+    const int32_t* actual_seq_lens_q, size_t actual_seq_lens_q_len,
+    const int32_t* actual_seq_lens_kv, size_t actual_seq_lens_kv_len,
+    const int32_t* actual_seq_offsets, size_t actual_seq_offsets_len,
+    const uint32_t* block_table, size_t block_table_len,
+    const SingePagedKvPrefillAttentionConfig* config);
+
 /* ---- dense f32 decode with split keys -----------------------------------------------------------------
  * The reference's split-KV convention (singe-kernel/src/cuda/attention/fmha.rs:1074-1250): a split kernel
  * writes one normalised partial output and one natural-log LSE per (batch, head, split) into scratch the

@@ -225,6 +225,12 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_splitk_reduce_f32.argtypes = [c_void, c_void, c_size, c_void, c_size, c_void, c_size,
                                                    ctypes.POINTER(SplitKReduceConfigC)]
     handle.singe_hip_splitk_reduce_f32.restype = i32
+    handle.singe_hip_paged_kv_decode_attention_f32_workspace_bytes.argtypes = [cfg]
+    handle.singe_hip_paged_kv_decode_attention_f32_workspace_bytes.restype = ctypes.c_size_t
+    handle.singe_hip_paged_kv_decode_attention_f32.argtypes = [c_void] + [c_void, c_size] * 7 + [cfg]
+    handle.singe_hip_paged_kv_decode_attention_f32.restype = i32
+    handle.singe_hip_paged_kv_prefill_attention_f32.argtypes = [c_void] + [c_void, c_size] * 9 + [paged_prefill]
+    handle.singe_hip_paged_kv_prefill_attention_f32.restype = i32
     split = ctypes.POINTER(FmhaDecodeSplitKConfigC)
     split_reduce = ctypes.POINTER(FmhaDecodeSplitKReduceConfigC)
     handle.singe_hip_fmha_decode_splitk_f32.argtypes = [c_void] + [c_void, c_size] * 5 + [split]

@@ -25,7 +25,7 @@ HIPCC_FLAGS = [
     "-Wall", "-Wno-unused-function",
 ]
 HOST_SOURCES = ["hip_runtime_loader.cpp", "module.cpp", "paged_decode.cpp", "fmha_prefill.cpp", "paged_attention.cpp",
-                "general_attention.cpp", "fmha_decode.cpp", "latent_attention.cpp", "cache_ops.cpp"]
+                "general_attention.cpp", "fmha_decode.cpp", "paged_rows_f32.cpp", "latent_attention.cpp", "cache_ops.cpp"]
 
 
 def _run(cmd):

@@ -15,6 +15,10 @@
 // 64 / LANES keys per step, the dot products finish with log2(LANES) cross-lane adds, and each set of lanes
 // keeps its own running softmax state, merged across lane sets and waves once at the end.  Query heads are
 // taken four at a time to bound registers (a group of more than four re-reads the slice from L2).
+//
+// The same loop serves the f32 forms of the two block-table ops, paged_kv_decode_attention_f32 and
+// paged_kv_prefill_attention_f32 (singe-kernel/src/cpu/attention.rs:1172-1341; launch API
+// singe-kernel/src/cuda/attention/paged.rs): only where the rows come from and where the result goes differ.
 #include "common.hip.h"
 #include "kernel_args.h"
 
@@ -51,30 +55,25 @@ SINGE_DEVICE void merge(DecodeState<VEC>& mine, float other_largest, float other
     mine.largest = largest;
 }
 
-template <int LANES, int VEC, bool ALIGNED>
-SINGE_DEVICE void fmha_decode_splitk_body(const FmhaDecodeSplitKArgs& a, float* lds) {
+// The loop all three kernels of this file share.  `rows` says what the workgroup works on:
+//   rows.groups, rows.begin, rows.end          query heads that share the key rows, and the keys to fold
+//   rows.query(head_in_group)                  that head's dims
+//   rows.key(k), rows.value(k)                 row k of the group's KV head
+//   rows.store(head_in_group, part, total)     takes the finished state; called by the LANES lanes that hold the dims
+template <int LANES, int VEC, bool ALIGNED, class Rows>
+SINGE_DEVICE void fold_rows(const Rows& rows, float scale, float* lds) {
     constexpr int kDim = LANES * 4 * VEC, kKeysPerWave = 64 / LANES;
     const unsigned int lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const unsigned int part = lane % LANES, set = lane / LANES;  // which dims of a key, which key of the wave's step
-    const unsigned int groups = a.heads / a.kv_heads;
-    unsigned int unit = blockIdx.x;
-    const unsigned int split = unit % a.splits;
-    unit /= a.splits;
-    const unsigned int kv_head = unit % a.kv_heads, batch = unit / a.kv_heads;
-    const unsigned long long first = static_cast<unsigned long long>(split) * a.kv_len_per_split;
-    const unsigned int begin = first < a.key_len ? static_cast<unsigned int>(first) : a.key_len;
-    const unsigned int end = first + a.kv_len_per_split < a.key_len ? static_cast<unsigned int>(first + a.kv_len_per_split) : a.key_len;
-    const float* keys = a.key + batch * a.key_batch_stride + kv_head * a.key_head_stride + part * (4 * VEC);
-    const float* values = a.value + batch * a.value_batch_stride + kv_head * a.value_head_stride + part * (4 * VEC);
+    const unsigned int begin = rows.begin, end = rows.end;
 
-    for (unsigned int pass = 0; pass < groups; pass += kDecodeHeadsPerPass) {
-        const unsigned int live = groups - pass < kDecodeHeadsPerPass ? groups - pass : kDecodeHeadsPerPass;
+    for (unsigned int pass = 0; pass < rows.groups; pass += kDecodeHeadsPerPass) {
+        const unsigned int live = rows.groups - pass < kDecodeHeadsPerPass ? rows.groups - pass : kDecodeHeadsPerPass;
         float4 q[kDecodeHeadsPerPass][VEC];
         DecodeState<VEC> state[kDecodeHeadsPerPass];
 #pragma unroll
         for (int g = 0; g < kDecodeHeadsPerPass; ++g) {
-            const unsigned int head = kv_head * groups + pass + (g < static_cast<int>(live) ? g : 0);
-            const float* row = a.query + batch * a.query_batch_stride + head * a.query_head_stride + part * (4 * VEC);
+            const float* row = rows.query(pass + (g < static_cast<int>(live) ? g : 0)) + part * (4 * VEC);
 #pragma unroll
             for (int v = 0; v < VEC; ++v) {
                 q[g][v] = load4<ALIGNED>(row + 4 * v);
@@ -87,11 +86,13 @@ SINGE_DEVICE void fmha_decode_splitk_body(const FmhaDecodeSplitKArgs& a, float* 
             const unsigned int key = base + set;
             const bool valid = key < end;
             const unsigned int row = valid ? key : end - 1;
+            const float* key_row = rows.key(row) + part * (4 * VEC);
+            const float* value_row = rows.value(row) + part * (4 * VEC);
             float4 k[VEC], v[VEC];
 #pragma unroll
             for (int i = 0; i < VEC; ++i) {
-                k[i] = load4<ALIGNED>(keys + row * a.key_sequence_stride + 4 * i);
-                v[i] = load4<ALIGNED>(values + row * a.value_sequence_stride + 4 * i);
+                k[i] = load4<ALIGNED>(key_row + 4 * i);
+                v[i] = load4<ALIGNED>(value_row + 4 * i);
             }
 #pragma unroll
             for (int g = 0; g < kDecodeHeadsPerPass; ++g) {
@@ -105,7 +106,7 @@ SINGE_DEVICE void fmha_decode_splitk_body(const FmhaDecodeSplitKArgs& a, float* 
                 }
 #pragma unroll
                 for (int step = 1; step < LANES; step *= 2) score += wave_xor(score, step);
-                score *= a.scale;
+                score *= scale;
                 if (valid) {
                     DecodeState<VEC>& s = state[g];
                     const float largest = fmaxf(s.largest, score);
@@ -153,14 +154,13 @@ SINGE_DEVICE void fmha_decode_splitk_body(const FmhaDecodeSplitKArgs& a, float* 
         __syncthreads();
         // Wave g of the workgroup finishes head g of the pass: lane `part` of its first set holds the dims.
         if (wave < live && set == 0) {
-            const unsigned int g = wave;
             DecodeState<VEC> total;
             total.largest = kEmptySliceLse;
             total.sum = 0.0f;
 #pragma unroll
             for (int i = 0; i < VEC; ++i) total.acc[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             for (unsigned int w = 0; w < 4; ++w) {
-                const float* slot = lds + (w * kDecodeHeadsPerPass + g) * kSlot;
+                const float* slot = lds + (w * kDecodeHeadsPerPass + wave) * kSlot;
                 float4 other_acc[VEC];
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) {
@@ -169,38 +169,177 @@ SINGE_DEVICE void fmha_decode_splitk_body(const FmhaDecodeSplitKArgs& a, float* 
                 }
                 merge(total, slot[0], slot[1], other_acc);
             }
-            const unsigned int head = kv_head * groups + pass + g;
-            const bool has_keys = total.sum > 0.0f;
-            const float inverse = has_keys ? 1.0f / total.sum : 0.0f;
-            float* out = a.out + batch * a.output_batch_stride + head * a.output_head_stride + split * a.output_split_stride + part * (4 * VEC);
-#pragma unroll
-            for (int i = 0; i < VEC; ++i) {
-                out[4 * i + 0] = total.acc[i].x * inverse;
-                out[4 * i + 1] = total.acc[i].y * inverse;
-                out[4 * i + 2] = total.acc[i].z * inverse;
-                out[4 * i + 3] = total.acc[i].w * inverse;
-            }
-            if (part == 0)
-                a.lse[batch * a.lse_batch_stride + head * a.lse_head_stride + split] =
-                    has_keys ? total.largest + __logf(total.sum) : kEmptySliceLse;
+            rows.store(pass + wave, part, total);
         }
         __syncthreads();
     }
 }
 
+// out[0 .. 4 VEC) = acc / sum (zeros for a row that saw no key), and what the row's LSE is.
+template <int VEC>
+SINGE_DEVICE float finish(float* out, const DecodeState<VEC>& total) {
+    const bool has_keys = total.sum > 0.0f;
+    const float inverse = has_keys ? 1.0f / total.sum : 0.0f;
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+        out[4 * i + 0] = total.acc[i].x * inverse;
+        out[4 * i + 1] = total.acc[i].y * inverse;
+        out[4 * i + 2] = total.acc[i].z * inverse;
+        out[4 * i + 3] = total.acc[i].w * inverse;
+    }
+    return has_keys ? total.largest + __logf(total.sum) : kEmptySliceLse;
+}
+
+// fmha_decode_splitk_f32: workgroup = (batch, kv head, split) of dense [batch, key_len, kv_heads, dim] keys.
+template <int VEC>
+struct DenseSplitRows {
+    const FmhaDecodeSplitKArgs& a;
+    unsigned int groups, begin, end, batch, kv_head, split;
+    SINGE_DEVICE explicit DenseSplitRows(const FmhaDecodeSplitKArgs& args) : a(args) {
+        groups = a.heads / a.kv_heads;
+        unsigned int unit = blockIdx.x;
+        split = unit % a.splits;
+        unit /= a.splits;
+        kv_head = unit % a.kv_heads;
+        batch = unit / a.kv_heads;
+        const unsigned long long first = static_cast<unsigned long long>(split) * a.kv_len_per_split;
+        begin = first < a.key_len ? static_cast<unsigned int>(first) : a.key_len;
+        end = first + a.kv_len_per_split < a.key_len ? static_cast<unsigned int>(first + a.kv_len_per_split) : a.key_len;
+    }
+    SINGE_DEVICE const float* query(unsigned int g) const {
+        return a.query + batch * a.query_batch_stride + (kv_head * groups + g) * a.query_head_stride;
+    }
+    SINGE_DEVICE const float* key(unsigned int k) const {
+        return a.key + batch * a.key_batch_stride + kv_head * a.key_head_stride + k * a.key_sequence_stride;
+    }
+    SINGE_DEVICE const float* value(unsigned int k) const {
+        return a.value + batch * a.value_batch_stride + kv_head * a.value_head_stride + k * a.value_sequence_stride;
+    }
+    SINGE_DEVICE void store(unsigned int g, unsigned int part, const DecodeState<VEC>& total) const {
+        const unsigned int head = kv_head * groups + g;
+        const float lse = finish(a.out + batch * a.output_batch_stride + head * a.output_head_stride + split * a.output_split_stride +
+                                     part * (4 * VEC), total);
+        if (part == 0) a.lse[batch * a.lse_batch_stride + head * a.lse_head_stride + split] = lse;
+    }
+};
+
+// The two paged forms read rows [block, slot, kv head, dim] through a block table
+// (block = table[sequence * stride + key / block_size], slot = key % block_size: cpu/attention.rs:1196-1206).
+// A table entry past the cache is clamped to its last block: the reference does not check it, and a wild
+// entry must not become a wild address here; nor must a length the table has no entries for.
+struct PagedCaches {
+    const PagedRowsF32Args& a;
+    unsigned int sequence, kv_head, dim;
+    // Keys one row of the table can name; a sequence length beyond it is cut there (the host checks that the
+    // product fits 32 bits).
+    SINGE_DEVICE unsigned int capacity() const { return a.block_table_batch_stride * a.block_size; }
+    SINGE_DEVICE size_t row(unsigned int k) const {
+        unsigned int block = a.block_table[static_cast<size_t>(sequence) * a.block_table_batch_stride + k / a.block_size];
+        block = block < a.physical_blocks ? block : a.physical_blocks - 1;
+        return ((static_cast<size_t>(block) * a.block_size + k % a.block_size) * a.kv_heads + kv_head) * dim;
+    }
+};
+
+// paged_kv_decode_attention_f32 (cpu/attention.rs:1172-1246), split over the keys: workgroup = (sequence, kv head,
+// split); split s of a sequence of L keys covers ceil(L / splits) of them.  Partials in the layout
+// splitk_reduce_f32 takes: out [batch, heads, splits, dim], lse [batch, heads, splits].
+template <int VEC>
+struct PagedDecodeRows {
+    const PagedRowsF32Args& a;
+    PagedCaches caches;
+    unsigned int groups, begin, end, split;
+    SINGE_DEVICE PagedDecodeRows(const PagedRowsF32Args& args, unsigned int dim) : a(args), caches{args, 0, 0, dim} {
+        groups = a.heads / a.kv_heads;
+        unsigned int unit = blockIdx.x;
+        split = unit % a.splits;
+        unit /= a.splits;
+        caches.kv_head = unit % a.kv_heads;
+        caches.sequence = unit / a.kv_heads;
+        const int length = a.seq_lens_kv[caches.sequence];
+        unsigned int keys = length > 0 ? static_cast<unsigned int>(length) : 0u;
+        keys = keys < caches.capacity() ? keys : caches.capacity();
+        const unsigned int per = (keys + a.splits - 1) / a.splits;
+        begin = split * per < keys ? split * per : keys;
+        end = begin + per < keys ? begin + per : keys;
+    }
+    SINGE_DEVICE const float* query(unsigned int g) const {
+        return a.query + (static_cast<size_t>(caches.sequence) * a.heads + caches.kv_head * groups + g) * caches.dim;
+    }
+    SINGE_DEVICE const float* key(unsigned int k) const { return a.key_cache + caches.row(k); }
+    SINGE_DEVICE const float* value(unsigned int k) const { return a.value_cache + caches.row(k); }
+    SINGE_DEVICE void store(unsigned int g, unsigned int part, const DecodeState<VEC>& total) const {
+        const size_t row = (static_cast<size_t>(caches.sequence) * a.heads + caches.kv_head * groups + g) * a.splits + split;
+        const float lse = finish(a.out + row * caches.dim + part * (4 * VEC), total);
+        if (part == 0) a.lse[row] = lse;
+    }
+};
+
+// paged_kv_prefill_attention_f32 (cpu/attention.rs:1248-1341): workgroup = (token, kv head).  Token t belongs to
+// the last sequence b with offsets[b] <= t < offsets[b] + len_q[b] (the reference walks the sequences in order,
+// so a later one overwrites); query i of a sequence sees keys 0 .. min(i + 1, len_kv) under the causal mask, all
+// len_kv without.  A token of no sequence gets zeros and an LSE of 0, a row without keys zeros and -1e20.
+template <int VEC>
+struct PagedPrefillRows {
+    const PagedRowsF32Args& a;
+    PagedCaches caches;
+    unsigned int groups, begin, end, token;
+    bool owned;
+    SINGE_DEVICE PagedPrefillRows(const PagedRowsF32Args& args, unsigned int dim) : a(args), caches{args, 0, 0, dim} {
+        groups = a.heads / a.kv_heads;
+        token = blockIdx.x / a.kv_heads;
+        caches.kv_head = blockIdx.x % a.kv_heads;
+        owned = false;
+        begin = end = 0;
+        for (unsigned int b = 0; b < a.batch; ++b) {
+            const int offset = a.seq_offsets[b], queries = a.seq_lens_q[b];
+            if (offset < 0 || queries <= 0 || static_cast<int>(token) < offset || static_cast<long long>(token) >= static_cast<long long>(offset) + queries) continue;
+            owned = true;
+            caches.sequence = b;
+            const int length = a.seq_lens_kv[b];
+            unsigned int keys = length > 0 ? static_cast<unsigned int>(length) : 0u;
+            keys = keys < caches.capacity() ? keys : caches.capacity();
+            const unsigned int index = token - static_cast<unsigned int>(offset);
+            end = a.causal && index + 1 < keys ? index + 1 : keys;
+        }
+    }
+    SINGE_DEVICE const float* query(unsigned int g) const {
+        return a.query + (static_cast<size_t>(token) * a.heads + caches.kv_head * groups + g) * caches.dim;
+    }
+    SINGE_DEVICE const float* key(unsigned int k) const { return a.key_cache + caches.row(k); }
+    SINGE_DEVICE const float* value(unsigned int k) const { return a.value_cache + caches.row(k); }
+    SINGE_DEVICE void store(unsigned int g, unsigned int part, const DecodeState<VEC>& total) const {
+        const size_t row = static_cast<size_t>(token) * a.heads + caches.kv_head * groups + g;
+        const float lse = finish(a.out + row * caches.dim + part * (4 * VEC), total);
+        if (part == 0) a.lse[row] = owned ? lse : 0.0f;
+    }
+};
+
 }  // namespace
 
-#define SINGE_FMHA_DECODE_SPLITK_KERNEL(DIM, LANES, VEC)                                                                   \
-    extern "C" __global__ __launch_bounds__(256) void singe_fmha_decode_splitk_f32_d##DIM(FmhaDecodeSplitKArgs args) {     \
-        __shared__ float lds[4 * kDecodeHeadsPerPass * (2 + DIM)];                                                         \
-        if (args.aligned) fmha_decode_splitk_body<LANES, VEC, true>(args, lds);                                            \
-        else fmha_decode_splitk_body<LANES, VEC, false>(args, lds);                                                        \
+#define SINGE_F32_ROW_KERNELS(DIM, LANES, VEC)                                                                               \
+    extern "C" __global__ __launch_bounds__(256) void singe_fmha_decode_splitk_f32_d##DIM(FmhaDecodeSplitKArgs args) {       \
+        __shared__ float lds[4 * kDecodeHeadsPerPass * (2 + DIM)];                                                           \
+        const DenseSplitRows<VEC> rows(args);                                                                                \
+        if (args.aligned) fold_rows<LANES, VEC, true>(rows, args.scale, lds);                                                \
+        else fold_rows<LANES, VEC, false>(rows, args.scale, lds);                                                            \
+    }                                                                                                                        \
+    extern "C" __global__ __launch_bounds__(256) void singe_paged_kv_decode_splitk_f32_d##DIM(PagedRowsF32Args args) {       \
+        __shared__ float lds[4 * kDecodeHeadsPerPass * (2 + DIM)];                                                           \
+        const PagedDecodeRows<VEC> rows(args, DIM);                                                                          \
+        if (args.aligned) fold_rows<LANES, VEC, true>(rows, args.scale, lds);                                                \
+        else fold_rows<LANES, VEC, false>(rows, args.scale, lds);                                                            \
+    }                                                                                                                        \
+    extern "C" __global__ __launch_bounds__(256) void singe_paged_kv_prefill_f32_d##DIM(PagedRowsF32Args args) {             \
+        __shared__ float lds[4 * kDecodeHeadsPerPass * (2 + DIM)];                                                           \
+        const PagedPrefillRows<VEC> rows(args, DIM);                                                                         \
+        if (args.aligned) fold_rows<LANES, VEC, true>(rows, args.scale, lds);                                                \
+        else fold_rows<LANES, VEC, false>(rows, args.scale, lds);                                                            \
     }
 
-SINGE_FMHA_DECODE_SPLITK_KERNEL(4, 1, 1)
-SINGE_FMHA_DECODE_SPLITK_KERNEL(8, 2, 1)
-SINGE_FMHA_DECODE_SPLITK_KERNEL(16, 4, 1)
-SINGE_FMHA_DECODE_SPLITK_KERNEL(32, 8, 1)
-SINGE_FMHA_DECODE_SPLITK_KERNEL(64, 16, 1)
-SINGE_FMHA_DECODE_SPLITK_KERNEL(128, 16, 2)
-SINGE_FMHA_DECODE_SPLITK_KERNEL(256, 16, 4)
+SINGE_F32_ROW_KERNELS(4, 1, 1)
+SINGE_F32_ROW_KERNELS(8, 2, 1)
+SINGE_F32_ROW_KERNELS(16, 4, 1)
+SINGE_F32_ROW_KERNELS(32, 8, 1)
+SINGE_F32_ROW_KERNELS(64, 16, 1)
+SINGE_F32_ROW_KERNELS(128, 16, 2)
+SINGE_F32_ROW_KERNELS(256, 16, 4)

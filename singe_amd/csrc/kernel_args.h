@@ -152,6 +152,25 @@ struct FmhaDecodeSplitKArgs {
     float scale;
 };
 
+// singe_paged_kv_decode_splitk_f32_d* and singe_paged_kv_prefill_f32_d*: f32 rows over block-table caches
+// [blocks, block_size, kv_heads, dim].
+struct PagedRowsF32Args {
+    float* out;                  // decode: partials [batch, heads, splits, dim]; prefill: [tokens, heads, dim]
+    float* lse;                  // decode: [batch, heads, splits]; prefill: [tokens, heads]; natural log
+    const float* query;          // decode: [batch, heads, dim]; prefill: [tokens, heads, dim]
+    const float* key_cache;
+    const float* value_cache;
+    const int32_t* seq_lens_q;   // prefill only
+    const int32_t* seq_lens_kv;
+    const int32_t* seq_offsets;  // prefill only
+    const uint32_t* block_table;
+    uint32_t batch, heads, kv_heads, block_size, block_table_batch_stride, physical_blocks;
+    uint32_t splits;             // decode only
+    uint32_t causal;             // prefill only
+    uint32_t aligned;            // every row of the query and the caches starts on a 16-byte boundary
+    float scale;
+};
+
 // Element types of the general (any head dimension) kernels.
 enum SingeElement : uint32_t { kElementF32 = 0, kElementBf16 = 1, kElementF16 = 2 };
 

@@ -28,6 +28,9 @@ enum KernelId : int {
     kSplitKReduce,
     // dense f32 split-KV decode: + head dimension (4, 8, 16, 32, 64, 128, 256)
     kFmhaDecodeSplitK, kFmhaDecodeSplitKLast = kFmhaDecodeSplitK + 6,
+    // f32 block-table decode (split over keys) and prefill, same seven head dimensions each
+    kPagedKvDecodeSplitKF32, kPagedKvDecodeSplitKF32Last = kPagedKvDecodeSplitKF32 + 6,
+    kPagedKvPrefillF32, kPagedKvPrefillF32Last = kPagedKvPrefillF32 + 6,
     kRotaryCacheF32, kRotaryCacheBf16, kRotaryCacheF16,
     kPagingIndicesI32, kPagingIndicesI64,
     // latent (MLA) attention: + element (f32, bf16, f16)

@@ -214,3 +214,36 @@ def test_dense_problem_and_splitk_validation():
     assert lib.singe_hip_splitk_reduce_f32(None, fake, 16, fake, 79, fake, 10, ctypes.byref(config)) == 2
     zero = _native.SplitKReduceConfigC(1, 2, 0, 8, 80, 40, 8, 10, 5, 16, 8)
     assert lib.singe_hip_splitk_reduce_f32(None, fake, 16, fake, 80, fake, 10, ctypes.byref(zero)) == 1
+
+
+def test_f32_block_table_ops_validate_like_the_bf16_ones():
+    lib = _native.lib()
+    fake = 0x1000
+    config = _native.PagedKvDecodeAttentionConfigC(**GOOD)
+    lens = dict(out=2 * 8 * 128, query=2 * 8 * 128, key=8 * 16 * 2 * 128, value=8 * 16 * 2 * 128, seq=2, table=8)
+    def decode(config=config, workspace=fake, workspace_bytes=1 << 30, **short):
+        n = dict(lens, **short)
+        return lib.singe_hip_paged_kv_decode_attention_f32(None, fake, n["out"], fake, n["query"], fake, n["key"], fake, n["value"],
+                                                           fake, n["seq"], fake, n["table"], workspace, workspace_bytes, ctypes.byref(config))
+    need = lib.singe_hip_paged_kv_decode_attention_f32_workspace_bytes(ctypes.byref(config))
+    assert need == 2 * 8 * 64 * 129 * 4
+    for name in ("out", "query", "key", "value", "seq", "table"):
+        assert decode(**{name: lens[name] - 1}) == 2, name
+    assert decode(workspace=None) == 6
+    assert decode(workspace_bytes=need - 1) == 2
+    assert decode(config=_native.PagedKvDecodeAttentionConfigC(**dict(GOOD, kv_heads=3))) == 1
+    assert decode(config=_native.PagedKvDecodeAttentionConfigC(**dict(GOOD, head_dim=48)), out=1 << 20, query=1 << 20) == 5
+    assert lib.singe_hip_paged_kv_decode_attention_f32_workspace_bytes(
+        ctypes.byref(_native.PagedKvDecodeAttentionConfigC(**dict(GOOD, batch=0)))) == 0
+    prefill = A.PagedKvPrefillAttentionConfig(2, 10, 4, 2, 64, 16, 8, 4, True, 0.1)._c()
+    sizes = [10 * 4 * 64, 10 * 4, 10 * 4 * 64, 8 * 16 * 2 * 64, 8 * 16 * 2 * 64, 2, 2, 2, 8]
+    def run(sizes, pointer=fake):
+        flat = []
+        for n in sizes:
+            flat += [pointer, n]
+        return lib.singe_hip_paged_kv_prefill_attention_f32(None, *flat, ctypes.byref(prefill))
+    for index in range(9):
+        short = list(sizes)
+        short[index] -= 1
+        assert run(short) == 2, index
+    assert run(sizes, pointer=None) == 6
