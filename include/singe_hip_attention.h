@@ -201,6 +201,20 @@ SINGE_HIP_API int32_t singe_hip_paged_kv_prefill_attention_bf16(
     const uint32_t* block_table, size_t block_table_len,
     const SingePagedKvPrefillAttentionConfig* config);
 
+/* paged_kv_prefill_attention_f16 (paged.rs): the same kernel on f16 operands (v_mfma_f32_32x32x16_f16). */
+SINGE_HIP_API int32_t singe_hip_paged_kv_prefill_attention_f16(
+    void* stream,
+    uint16_t* out, size_t out_len,
+    float* lse, size_t lse_len,
+    const uint16_t* query, size_t query_len,
+    const uint16_t* key_cache, size_t key_cache_len,
+    const uint16_t* value_cache, size_t value_cache_len,
+    const int32_t* actual_seq_lens_q, size_t actual_seq_lens_q_len,
+    const int32_t* actual_seq_lens_kv, size_t actual_seq_lens_kv_len,
+    const int32_t* actual_seq_offsets, size_t actual_seq_offsets_len,
+    const uint32_t* block_table, size_t block_table_len,
+    const SingePagedKvPrefillAttentionConfig* config);
+
 /* ---- singe-kernel surface: dense prefill ---------------------------------------------------------
  * Mirrors FmhaPrefillConfig (singe-kernel/src/cuda/attention/mod.rs:253-274); strides in elements.
  * FmhaPrefillConfig::contiguous (mod.rs:1602-1632) fills them for packed [batch, len, heads, dim]. */

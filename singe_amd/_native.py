@@ -178,6 +178,8 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_paged_kv_prefill_attention_config_validate.restype = i32
     handle.singe_hip_paged_kv_prefill_attention_bf16.argtypes = [c_void] + [c_void, c_size] * 9 + [paged_prefill]
     handle.singe_hip_paged_kv_prefill_attention_bf16.restype = i32
+    handle.singe_hip_paged_kv_prefill_attention_f16.argtypes = [c_void] + [c_void, c_size] * 9 + [paged_prefill]
+    handle.singe_hip_paged_kv_prefill_attention_f16.restype = i32
     fmha = ctypes.POINTER(FmhaPrefillConfigC)
     handle.singe_hip_fmha_prefill_config_validate.argtypes = [fmha]
     handle.singe_hip_fmha_prefill_config_validate.restype = i32

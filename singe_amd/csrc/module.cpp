@@ -26,6 +26,7 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_attention_bf16_d128_i32_p16", "singe_paged_attention_bf16_d128_i64_p16",
     "singe_paged_attention_bf16_d128_softcap_i32_p16", "singe_paged_attention_bf16_d128_softcap_i64_p16",
     "singe_paged_kv_prefill_bf16_d128", "singe_paged_kv_prefill_bf16_d128_p16",
+    "singe_paged_kv_prefill_f16_d128", "singe_paged_kv_prefill_f16_d128_p16",
     "singe_paged_attention_combine_bf16_i32", "singe_paged_attention_combine_bf16_i64",
     "singe_paged_attention_combine_f16_i32", "singe_paged_attention_combine_f16_i64",
     "singe_paged_attention_f16_d128_i32", "singe_paged_attention_f16_d128_i64",

@@ -19,7 +19,7 @@ enum KernelId : int {
     // paged attention: + 4 when the page size is a power of two of at least 16 keys
     kPagedAttentionI32, kPagedAttentionI64, kPagedAttentionSoftcapI32, kPagedAttentionSoftcapI64,
     kPagedAttentionI32P16, kPagedAttentionI64P16, kPagedAttentionSoftcapI32P16, kPagedAttentionSoftcapI64P16,
-    kPagedKvPrefill, kPagedKvPrefillP16,
+    kPagedKvPrefill, kPagedKvPrefillP16, kPagedKvPrefillF16, kPagedKvPrefillF16P16,
     kPagedAttentionCombineI32, kPagedAttentionCombineI64, kPagedAttentionCombineF16I32, kPagedAttentionCombineF16I64,
     // f16 paged attention: same order as the eight bf16 kernels from kPagedAttentionI32
     kPagedAttentionF16,

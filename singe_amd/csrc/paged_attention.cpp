@@ -260,8 +260,41 @@ extern "C" int32_t singe_hip_paged_kv_prefill_attention_config_validate(const Si
 
 // paged_kv_prefill_attention_bf16 (singe-kernel/src/cuda/attention/paged.rs:370-420); lengths checked
 // in the order of PagedKvPrefillAttentionConfig::validate_lengths (mod.rs:786-818).
+namespace {
+int32_t paged_kv_prefill(
+    bool f16, void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, const uint16_t* query, size_t query_len,
+    const uint16_t* key_cache, size_t key_cache_len, const uint16_t* value_cache, size_t value_cache_len,
+    const int32_t* actual_seq_lens_q, size_t actual_seq_lens_q_len, const int32_t* actual_seq_lens_kv,
+    size_t actual_seq_lens_kv_len, const int32_t* actual_seq_offsets, size_t actual_seq_offsets_len,
+    const uint32_t* block_table, size_t block_table_len, const SingePagedKvPrefillAttentionConfig* config);
+}  // namespace
+
 extern "C" int32_t singe_hip_paged_kv_prefill_attention_bf16(
     void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, const uint16_t* query, size_t query_len,
+    const uint16_t* key_cache, size_t key_cache_len, const uint16_t* value_cache, size_t value_cache_len,
+    const int32_t* actual_seq_lens_q, size_t actual_seq_lens_q_len, const int32_t* actual_seq_lens_kv,
+    size_t actual_seq_lens_kv_len, const int32_t* actual_seq_offsets, size_t actual_seq_offsets_len,
+    const uint32_t* block_table, size_t block_table_len, const SingePagedKvPrefillAttentionConfig* config) {
+    return paged_kv_prefill(false, stream, out, out_len, lse, lse_len, query, query_len, key_cache, key_cache_len, value_cache,
+                            value_cache_len, actual_seq_lens_q, actual_seq_lens_q_len, actual_seq_lens_kv, actual_seq_lens_kv_len,
+                            actual_seq_offsets, actual_seq_offsets_len, block_table, block_table_len, config);
+}
+
+// paged_kv_prefill_attention_f16: the same kernel on f16 operands.
+extern "C" int32_t singe_hip_paged_kv_prefill_attention_f16(
+    void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, const uint16_t* query, size_t query_len,
+    const uint16_t* key_cache, size_t key_cache_len, const uint16_t* value_cache, size_t value_cache_len,
+    const int32_t* actual_seq_lens_q, size_t actual_seq_lens_q_len, const int32_t* actual_seq_lens_kv,
+    size_t actual_seq_lens_kv_len, const int32_t* actual_seq_offsets, size_t actual_seq_offsets_len,
+    const uint32_t* block_table, size_t block_table_len, const SingePagedKvPrefillAttentionConfig* config) {
+    return paged_kv_prefill(true, stream, out, out_len, lse, lse_len, query, query_len, key_cache, key_cache_len, value_cache,
+                            value_cache_len, actual_seq_lens_q, actual_seq_lens_q_len, actual_seq_lens_kv, actual_seq_lens_kv_len,
+                            actual_seq_offsets, actual_seq_offsets_len, block_table, block_table_len, config);
+}
+
+namespace {
+int32_t paged_kv_prefill(
+    bool f16, void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, const uint16_t* query, size_t query_len,
     const uint16_t* key_cache, size_t key_cache_len, const uint16_t* value_cache, size_t value_cache_len,
     const int32_t* actual_seq_lens_q, size_t actual_seq_lens_q_len, const int32_t* actual_seq_lens_kv,
     size_t actual_seq_lens_kv_len, const int32_t* actual_seq_offsets, size_t actual_seq_offsets_len,
@@ -282,7 +315,8 @@ extern "C" int32_t singe_hip_paged_kv_prefill_attention_bf16(
     if (int32_t s = ensure_len_at_least("actual_seq_lens_kv", actual_seq_lens_kv_len, c.batch)) return s;
     if (int32_t s = ensure_len_at_least("actual_seq_offsets", actual_seq_offsets_len, c.batch)) return s;
     if (int32_t s = ensure_len_at_least("block_table", block_table_len, table_len)) return s;
-    if (c.head_dim != 128) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, "paged_kv_prefill_attention_bf16", c.head_dim, 0);
+    if (c.head_dim != 128)
+        return fail(SINGE_HIP_UNSUPPORTED_WIDTH, f16 ? "paged_kv_prefill_attention_f16" : "paged_kv_prefill_attention_bf16", c.head_dim, 0);
     if (block_len > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "a cache block beyond 4 Gi elements");
     const void* pointers[] = {out, lse, query, key_cache, value_cache, actual_seq_lens_q, actual_seq_lens_kv, actual_seq_offsets, block_table};
     const char* names[] = {"out", "lse", "query", "key_cache", "value_cache", "actual_seq_lens_q", "actual_seq_lens_kv",
@@ -322,5 +356,7 @@ extern "C" int32_t singe_hip_paged_kv_prefill_attention_bf16(
     const uint64_t units = (static_cast<uint64_t>(c.batch) * c.kv_heads + 7) / 8 * 8;
     const uint64_t blocks = units * args.row_tiles;
     if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
-    return launch(args.page_shift >= 4 ? kPagedKvPrefillP16 : kPagedKvPrefill, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+    const int kernel = (f16 ? kPagedKvPrefillF16 : kPagedKvPrefill) + (args.page_shift >= 4 ? 1 : 0);
+    return launch(static_cast<KernelId>(kernel), static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
 }
+}  // namespace

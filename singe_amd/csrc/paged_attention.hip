@@ -535,6 +535,8 @@ SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i64_p16, tr
 // paged_kv_prefill_attention_bf16 of the singe-kernel surface: same gather, block-table paging.
 SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_bf16_d128, false, kTable, false, false, Bf16)
 SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_bf16_d128_p16, false, kTable, true, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_f16_d128, false, kTable, false, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_f16_d128_p16, false, kTable, true, false, F16)
 // rotary_paged_attention: the query is normalised and rotated on its way into the registers.
 SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i32, false, kCsrI32, false, true, Bf16)
 SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i64, false, kCsrI64, false, true, Bf16)

@@ -245,6 +245,37 @@ def paged_kv_prefill_attention_bf16(stream, out: torch.Tensor, lse: torch.Tensor
     _native.check(status, "paged_kv_prefill_attention_bf16")
 
 
+def paged_kv_prefill_attention_f16(stream, out: torch.Tensor, lse: torch.Tensor, query: torch.Tensor,
+                                    key_cache: torch.Tensor, value_cache: torch.Tensor,
+                                    actual_seq_lens_q: torch.Tensor, actual_seq_lens_kv: torch.Tensor,
+                                    actual_seq_offsets: torch.Tensor, block_table: torch.Tensor,
+                                    config: PagedKvPrefillAttentionConfig) -> None:
+    """paged_kv_prefill_attention_f16 (paged.rs): the bf16 op on f16 operands.
+
+    out/query [total_query_tokens, heads, dim] f16; lse [total_query_tokens, heads] f32 (natural log,
+    -1e20 for a row without keys); caches [blocks, block_size, kv_heads, dim] f16; the three per-sequence
+    vectors [batch] i32; block_table [batch, stride] u32.  Causal hides key index > query index.
+    """
+    _require(out, torch.float16, "out")
+    _require(lse, torch.float32, "lse")
+    _require(query, torch.float16, "query")
+    _require(key_cache, torch.float16, "key_cache")
+    _require(value_cache, torch.float16, "value_cache")
+    _require(actual_seq_lens_q, torch.int32, "actual_seq_lens_q")
+    _require(actual_seq_lens_kv, torch.int32, "actual_seq_lens_kv")
+    _require(actual_seq_offsets, torch.int32, "actual_seq_offsets")
+    if block_table.dtype not in (torch.int32, torch.uint32):
+        raise error.InvalidArgument(f"block_table must hold 32-bit entries, got {block_table.dtype}")
+    _require(block_table, block_table.dtype, "block_table")
+    c = config._c()
+    status = _native.lib().singe_hip_paged_kv_prefill_attention_f16(
+        _stream_handle(stream), _ptr(out), out.numel(), _ptr(lse), lse.numel(), _ptr(query), query.numel(),
+        _ptr(key_cache), key_cache.numel(), _ptr(value_cache), value_cache.numel(), _ptr(actual_seq_lens_q),
+        actual_seq_lens_q.numel(), _ptr(actual_seq_lens_kv), actual_seq_lens_kv.numel(), _ptr(actual_seq_offsets),
+        actual_seq_offsets.numel(), _ptr(block_table), block_table.numel(), ctypes.byref(c))
+    _native.check(status, "paged_kv_prefill_attention_f16")
+
+
 @dataclass(frozen=True)
 class FmhaPrefillConfig:
     """Dense prefill attention (mod.rs:253-274): query/out [batch, query_len, heads, dim], key/value

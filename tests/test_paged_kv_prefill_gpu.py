@@ -44,16 +44,18 @@ def build(sequences, heads, kv_heads, block_size, seed, gap_tokens=0, extra_bloc
     return lens_q, lens_kv, np.array(offsets, dtype=np.int32), table, stride, blocks, total, query, kc, vc
 
 
-def run_case(sequences, heads, kv_heads, block_size, causal, seed=0, gap_tokens=0, scale=None):
+def run_case(sequences, heads, kv_heads, block_size, causal, seed=0, gap_tokens=0, scale=None, dtype=torch.bfloat16):
     lens_q, lens_kv, offsets, table, stride, blocks, total, query, kc, vc = build(sequences, heads, kv_heads, block_size,
                                                                                 seed, gap_tokens)
+    query, kc, vc = query.to(dtype), kc.to(dtype), vc.to(dtype)
     scale = DIM ** -0.5 if scale is None else scale
     config = A.PagedKvPrefillAttentionConfig.contiguous(len(sequences), total, heads, kv_heads, DIM, block_size, blocks,
                                                         stride, causal, scale)
     sentinel = 7.0
-    out = torch.full((total, heads, DIM), sentinel, device="cuda", dtype=torch.bfloat16)
+    out = torch.full((total, heads, DIM), sentinel, device="cuda", dtype=dtype)
     lse = torch.full((total, heads), sentinel, device="cuda", dtype=torch.float32)
-    A.paged_kv_prefill_attention_bf16(None, out, lse, query, kc, vc, torch.from_numpy(lens_q).cuda(),
+    op = A.paged_kv_prefill_attention_bf16 if dtype == torch.bfloat16 else A.paged_kv_prefill_attention_f16
+    op(None, out, lse, query, kc, vc, torch.from_numpy(lens_q).cuda(),
                                       torch.from_numpy(lens_kv).cuda(), torch.from_numpy(offsets).cuda(),
                                       torch.from_numpy(table.view(np.int32)).cuda(), config)
     torch.cuda.synchronize()
@@ -72,8 +74,11 @@ def run_case(sequences, heads, kv_heads, block_size, causal, seed=0, gap_tokens=
         return
     assert np.isfinite(got).all()
     gap = np.abs(got - want)
-    assert gap.max() <= MAX_ABS, gap.max()
-    assert gap.mean() <= MEAN_ABS, gap.mean()
+    # f16 carries three more mantissa bits than bf16: the reference's own bounds are 0.03 and 0.005
+    # (kernel_plan/source/tests.rs:549-553); the same ratio is applied to the bf16 bounds here.
+    tighter = 1.0 if dtype == torch.bfloat16 else 1.0 / 6.0
+    assert gap.max() <= MAX_ABS * tighter, gap.max()
+    assert gap.mean() <= MEAN_ABS * tighter, gap.mean()
     empty = want_lse == np.float32(-1.0e20)
     assert np.array_equal(got_lse == np.float32(-1.0e20), empty)
     assert not got[empty].any()
@@ -91,6 +96,16 @@ def run_case(sequences, heads, kv_heads, block_size, causal, seed=0, gap_tokens=
 ])
 def test_matches_oracle(case, causal):
     run_case(causal=causal, seed=11, **case)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("case", [
+    dict(sequences=[(130, 130), (1, 1), (33, 200), (64, 10)], heads=8, kv_heads=2, block_size=16),
+    dict(sequences=[(300, 257)], heads=2, kv_heads=2, block_size=7),
+    dict(sequences=[(70, 70), (0, 12), (9, 0), (20, 90)], heads=16, kv_heads=2, block_size=16, gap_tokens=2),
+])
+def test_f16_matches_oracle(case, causal):
+    run_case(causal=causal, seed=12, dtype=torch.float16, **case)
 
 
 def test_more_queries_than_keys_causal_and_full():
