@@ -110,6 +110,19 @@ SINGE_HIP_API int32_t singe_hip_paged_kv_decode_attention_bf16(
     void* workspace, size_t workspace_bytes,
     const SingePagedKvDecodeAttentionConfig* config);
 
+/* paged_kv_decode_attention_f16 (paged.rs): the same kernels on f16 operands (v_mfma_f32_16x16x32_f16); same
+ * workspace size and rules. */
+SINGE_HIP_API int32_t singe_hip_paged_kv_decode_attention_f16(
+    void* stream,
+    uint16_t* out, size_t out_len,
+    const uint16_t* query, size_t query_len,
+    const uint16_t* key_cache, size_t key_cache_len,
+    const uint16_t* value_cache, size_t value_cache_len,
+    const int32_t* actual_seq_lens, size_t actual_seq_lens_len,
+    const uint32_t* block_table, size_t block_table_len,
+    void* workspace, size_t workspace_bytes,
+    const SingePagedKvDecodeAttentionConfig* config);
+
 /* The same operation run phase by phase, as the reference exposes its split kernel and splitk_reduce
  * separately (singe-kernel/src/cuda/attention/fmha.rs:1038,1155): SPLIT fills the scratch with the
  * normalised partial rows and natural-log LSEs of every key range; REDUCE folds the scratch into

@@ -16,6 +16,9 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_decode_bf16_d128_g1_b16", "singe_paged_decode_bf16_d128_g2_b16",
     "singe_paged_decode_bf16_d128_g1_any", "singe_paged_decode_bf16_d128_g2_any",
     "singe_paged_decode_combine_bf16",
+    "singe_paged_decode_f16_d128_g1_b16", "singe_paged_decode_f16_d128_g2_b16",
+    "singe_paged_decode_f16_d128_g1_any", "singe_paged_decode_f16_d128_g2_any",
+    "singe_paged_decode_combine_f16",
     "singe_paged_decode_f8kv_wide_d128_b16", "singe_paged_decode_f8kv_wide_d128_any",
     "singe_paged_decode_f8kv_wide_relaxed_d128_b16", "singe_paged_decode_f8kv_wide_relaxed_d128_any",
     "singe_fmha_prefill_bf16_d128_causal", "singe_fmha_prefill_bf16_d128_full",

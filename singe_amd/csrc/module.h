@@ -12,6 +12,8 @@ enum KernelId : int {
     // bf16 paged decode: index = 2 * (block size not a multiple of 16) + (two head groups per wave)
     kDecodeBf16 = 0,
     kDecodeCombine = 4,
+    // f16 paged decode: the four bf16 forms in the same order, then their combine
+    kDecodeF16, kDecodeF16Combine = kDecodeF16 + 4,
     // fp8 decode, dense form: + (block size not a multiple of 16) + 2 * relaxed
     kDecodeF8Wide, kDecodeF8WideAny, kDecodeF8WideRelaxed, kDecodeF8WideRelaxedAny,
     kPrefillCausal, kPrefillFull, kPrefillCausalF16, kPrefillFullF16,

@@ -21,7 +21,7 @@ int32_t decode(void* stream, uint16_t* out, size_t out_len, const uint16_t* quer
                const float* key_scales, size_t key_scales_len, const float* value_scales, size_t value_scales_len,
                bool fp8, const int32_t* actual_seq_lens, size_t actual_seq_lens_len, const uint32_t* block_table,
                size_t block_table_len, void* workspace, size_t workspace_bytes,
-               const SingePagedKvDecodeAttentionConfig* config, uint32_t phases);
+               const SingePagedKvDecodeAttentionConfig* config, uint32_t phases, bool f16 = false);
 
 constexpr size_t kHeadDim = 128;
 constexpr unsigned kWavesPerWorkgroup = 8;
@@ -126,6 +126,18 @@ int32_t singe_hip_paged_kv_decode_attention_phases_bf16(
                   workspace, workspace_bytes, config, phases);
 }
 
+// paged_kv_decode_attention_f16 (singe-kernel/src/cuda/attention/paged.rs): the bf16 kernels on f16 operands.
+int32_t singe_hip_paged_kv_decode_attention_f16(
+    void* stream, uint16_t* out, size_t out_len, const uint16_t* query, size_t query_len,
+    const uint16_t* key_cache, size_t key_cache_len, const uint16_t* value_cache, size_t value_cache_len,
+    const int32_t* actual_seq_lens, size_t actual_seq_lens_len, const uint32_t* block_table,
+    size_t block_table_len, void* workspace, size_t workspace_bytes,
+    const SingePagedKvDecodeAttentionConfig* config) {
+    return decode(stream, out, out_len, query, query_len, key_cache, key_cache_len, value_cache, value_cache_len,
+                  nullptr, 0, nullptr, 0, false, actual_seq_lens, actual_seq_lens_len, block_table, block_table_len,
+                  workspace, workspace_bytes, config, SINGE_HIP_DECODE_SPLIT | SINGE_HIP_DECODE_REDUCE, true);
+}
+
 int32_t singe_hip_paged_kv_decode_attention_f8e4m3kv_bf16(
     void* stream, uint16_t* out, size_t out_len, const uint16_t* query, size_t query_len,
     const uint8_t* key_cache, size_t key_cache_len, const uint8_t* value_cache, size_t value_cache_len,
@@ -148,7 +160,7 @@ int32_t decode(
     const float* key_scales, size_t key_scales_len, const float* value_scales, size_t value_scales_len, bool fp8,
     const int32_t* actual_seq_lens, size_t actual_seq_lens_len, const uint32_t* block_table,
     size_t block_table_len, void* workspace, size_t workspace_bytes,
-    const SingePagedKvDecodeAttentionConfig* config, uint32_t phases) {
+    const SingePagedKvDecodeAttentionConfig* config, uint32_t phases, bool f16) {
     if (config == nullptr) return fail(SINGE_HIP_NULL_POINTER, "config");
     const SingePagedKvDecodeAttentionConfig& c = *config;
     // PagedKvDecodeAttentionConfig::validate_lengths (mod.rs:711-743), in its order.
@@ -182,7 +194,8 @@ int32_t decode(
 
     // What the gfx950 kernels take (the reference's cuTile kernels take head_dim 4..64 only and return
     // UnsupportedWidth otherwise: singe-kernel/src/cuda/cutile/attention/paged.rs:799-810).
-    if (c.head_dim != kHeadDim) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, "paged_kv_decode_attention_bf16", c.head_dim, 0);
+    if (c.head_dim != kHeadDim)
+        return fail(SINGE_HIP_UNSUPPORTED_WIDTH, f16 ? "paged_kv_decode_attention_f16" : "paged_kv_decode_attention_bf16", c.head_dim, 0);
     uint64_t reach = static_cast<uint64_t>(c.block_table_batch_stride) * c.block_size;
     if (!fits_i32(reach)) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "block_table_batch_stride * block_size");
 
@@ -222,7 +235,7 @@ int32_t decode(
     const bool aligned = c.block_size % 16 == 0;
     // bf16 caches take the one-hot form, fp8 caches the dense form (see paged_decode.hip).
     const KernelId kernel = fp8 ? static_cast<KernelId>(kDecodeF8Wide + (aligned ? 0 : 1) + (g_relaxed.load(std::memory_order_relaxed) ? 2 : 0))
-                                : static_cast<KernelId>(kDecodeBf16 + (aligned ? 0 : 2) + (plan.groups == 2 ? 1 : 0));
+                                : static_cast<KernelId>((f16 ? kDecodeF16 : kDecodeBf16) + (aligned ? 0 : 2) + (plan.groups == 2 ? 1 : 0));
     if (phases & SINGE_HIP_DECODE_SPLIT)
         if (int32_t status = launch(kernel, plan.grid_x, plan.grid_y, 1, 64 * kWavesPerWorkgroup, stream, args,
                                     static_cast<unsigned>((2 * c.batch + 1) * sizeof(uint32_t))))
@@ -240,7 +253,7 @@ int32_t decode(
     combine.workers = plan.workers;
     combine.head_groups = plan.head_groups;
     combine.heads_per_wave = plan.heads_per_wave;
-    return launch(kDecodeCombine, static_cast<unsigned>((c.batch * c.heads + 3) / 4), 1, 1, 256, stream, combine);
+    return launch(f16 ? kDecodeF16Combine : kDecodeCombine, static_cast<unsigned>((c.batch * c.heads + 3) / 4), 1, 1, 256, stream, combine);
 }
 
 }  // namespace

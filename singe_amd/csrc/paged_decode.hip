@@ -273,6 +273,38 @@ SINGE_DEVICE unsigned int bf16_pair(float lo, float hi) {
 // bf16(value) in both halves of a dword (one v_cvt_pk_bf16_f32, round to nearest even).
 SINGE_DEVICE unsigned int bf16_twice(float value) { return bf16_pair(value, value); }
 
+// The same value rounded to the cache's 16-bit type in both halves of a dword, and the two MFMA shapes, for bf16
+// (the default) or f16 operands.
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+
+template <bool F16>
+SINGE_DEVICE unsigned int half_twice(float value) {
+    if constexpr (F16) {
+        const f32x2_t both = {value, value};
+        return __builtin_bit_cast(unsigned int, __builtin_convertvector(both, f16x2_t));
+    } else {
+        return bf16_twice(value);
+    }
+}
+
+template <bool F16>
+SINGE_DEVICE f32x4_t score_mma(uint4 keys, bf16x8_t query, f32x4_t acc) {
+    if constexpr (F16)
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8_t, keys), __builtin_bit_cast(f16x8_t, query), acc, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, keys), query, acc, 0, 0, 0);
+}
+
+template <bool F16>
+SINGE_DEVICE f32x4_t value_mma(uint2 values, uint2 weights, f32x4_t acc) {
+    if constexpr (F16)
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4_t, values), __builtin_bit_cast(f16x4_t, weights), acc, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(i16x4_t, values), __builtin_bit_cast(i16x4_t, weights), acc, 0, 0, 0);
+}
+
 // Eight fp8 e4m3 codes -> eight bf16 values.  EXACT: bf16_rne(value(code) * scale), the value the CPU path
 // reads after dequantising the cache.  Otherwise the codes are widened as they are (every e4m3 value is a
 // bf16 value), which v_cvt_scalef32_pk_bf16_fp8 does for two codes at a time; its scale operand only
@@ -311,7 +343,7 @@ constexpr int kStagedTileBytes = kTile * kStagedRowBytes;
 // transposed (ds_read_b64_tr_b16) as the A operand of v_mfma_f32_16x16x32_bf16, O^T[dim, head] += V^T . P^T.
 // That is a third of the matrix instructions and half the exponentials of the one-hot form, which matters
 // where the byte rate of an fp8 cache leaves the vector and matrix units little time per byte.
-template <int GROUPS, bool ALIGNED16, bool FP8, bool EXACT, bool WIDE = false>
+template <int GROUPS, bool ALIGNED16, bool FP8, bool EXACT, bool WIDE = false, bool F16 = false>
 SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, unsigned char* staging = nullptr) {
     static_assert(WIDE == FP8 && (!WIDE || GROUPS == 1), "fp8 caches take the wide form, bf16 caches the one-hot form");
     using Tile = typename std::conditional<FP8, KeyTileFp8, KeyTileBf16>::type;
@@ -520,8 +552,8 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
             }
 #pragma unroll
             for (int hg = 0; hg < GROUPS; ++hg) {
-                s0[hg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, first), q[hg][c], s0[hg], 0, 0, 0);
-                s1[hg] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, second), q[hg][c], s1[hg], 0, 0, 0);
+                s0[hg] = score_mma<F16>(first, q[hg][c], s0[hg]);
+                s1[hg] = score_mma<F16>(second, q[hg][c], s1[hg]);
             }
         }
         float p[GROUPS][8];
@@ -560,12 +592,10 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
                 if constexpr (!FP8) row = tile.v[half][i];
 #pragma unroll
                 for (int hg = 0; hg < GROUPS; ++hg) {
-                    const unsigned int both = bf16_twice(p[hg][half * 4 + i]);
+                    const unsigned int both = half_twice<F16>(p[hg][half * 4 + i]);
                     const uint2 hot = make_uint2(both & place0, both & place1);
-                    state[hg].acc[0] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
-                        __builtin_bit_cast(i16x4_t, make_uint2(row.x, row.y)), __builtin_bit_cast(i16x4_t, hot), state[hg].acc[0], 0, 0, 0);
-                    state[hg].acc[1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(
-                        __builtin_bit_cast(i16x4_t, make_uint2(row.z, row.w)), __builtin_bit_cast(i16x4_t, hot), state[hg].acc[1], 0, 0, 0);
+                    state[hg].acc[0] = value_mma<F16>(make_uint2(row.x, row.y), hot, state[hg].acc[0]);
+                    state[hg].acc[1] = value_mma<F16>(make_uint2(row.z, row.w), hot, state[hg].acc[1]);
                 }
             }
     };
@@ -681,6 +711,18 @@ SINGE_DECODE_KERNEL(singe_paged_decode_bf16_d128_g2_b16, 2, true, false, true)
 SINGE_DECODE_KERNEL(singe_paged_decode_bf16_d128_g1_any, 1, false, false, true)
 SINGE_DECODE_KERNEL(singe_paged_decode_bf16_d128_g2_any, 2, false, false, true)
 
+// paged_kv_decode_attention_f16: the same kernels on f16 operands.
+#define SINGE_DECODE_F16_KERNEL(NAME, GROUPS, ALIGNED)                                          \
+    extern "C" __global__ __launch_bounds__(512) void NAME(DecodeArgs args) {                    \
+        extern __shared__ unsigned int prefix[];                                                \
+        paged_decode_body<GROUPS, ALIGNED, false, true, false, true>(args, prefix);             \
+    }
+
+SINGE_DECODE_F16_KERNEL(singe_paged_decode_f16_d128_g1_b16, 1, true)
+SINGE_DECODE_F16_KERNEL(singe_paged_decode_f16_d128_g2_b16, 2, true)
+SINGE_DECODE_F16_KERNEL(singe_paged_decode_f16_d128_g1_any, 1, false)
+SINGE_DECODE_F16_KERNEL(singe_paged_decode_f16_d128_g2_any, 2, false)
+
 #define SINGE_DECODE_WIDE_KERNEL(NAME, ALIGNED, EXACT)                                          \
     extern "C" __global__ __launch_bounds__(512) void NAME(DecodeArgs args) {                    \
         extern __shared__ unsigned int prefix[];                                                \
@@ -698,7 +740,8 @@ SINGE_DECODE_WIDE_KERNEL(singe_paged_decode_f8kv_wide_relaxed_d128_any, false, f
 // (singe-kernel/src/cpu/attention.rs:2157-2193).  One wave per row.  The kernel is a chain of dependent
 // memory round trips, so it is written to need few of them: lane s fetches the log-sum-exp of slot s
 // (one trip for up to 64 slots), and the slots' rows are fetched sixteen at a time, two dims per lane.
-extern "C" __global__ __launch_bounds__(256) void singe_paged_decode_combine_bf16(CombineArgs a) {
+template <bool F16>
+SINGE_DEVICE void paged_decode_combine_body(const CombineArgs& a) {
     const unsigned int lane = threadIdx.x & 63;
     const unsigned int row = blockIdx.x * 4 + (threadIdx.x >> 6);  // batch * heads + head
     if (row >= a.batch * a.heads) return;
@@ -755,5 +798,15 @@ extern "C" __global__ __launch_bounds__(256) void singe_paged_decode_combine_bf1
             high /= total;
         }
     }
-    *reinterpret_cast<unsigned int*>(a.out + static_cast<size_t>(row) * kDim + 2 * lane) = pack_bf16x2(low, high);
+    unsigned int packed;
+    if constexpr (F16) {
+        const f32x2_t both = {low, high};
+        packed = __builtin_bit_cast(unsigned int, __builtin_convertvector(both, f16x2_t));
+    } else {
+        packed = pack_bf16x2(low, high);
+    }
+    *reinterpret_cast<unsigned int*>(a.out + static_cast<size_t>(row) * kDim + 2 * lane) = packed;
 }
+
+extern "C" __global__ __launch_bounds__(256) void singe_paged_decode_combine_bf16(CombineArgs a) { paged_decode_combine_body<false>(a); }
+extern "C" __global__ __launch_bounds__(256) void singe_paged_decode_combine_f16(CombineArgs a) { paged_decode_combine_body<true>(a); }

@@ -732,3 +732,24 @@ def paged_kv_prefill_attention_f32(stream, out: torch.Tensor, lse: torch.Tensor,
         actual_seq_lens_q.numel(), _ptr(actual_seq_lens_kv), actual_seq_lens_kv.numel(), _ptr(actual_seq_offsets),
         actual_seq_offsets.numel(), _ptr(block_table), block_table.numel(), ctypes.byref(c))
     _native.check(status, "paged_kv_prefill_attention_f32")
+
+
+def paged_kv_decode_attention_f16(stream, out: torch.Tensor, query: torch.Tensor, key_cache: torch.Tensor,
+                                  value_cache: torch.Tensor, actual_seq_lens: torch.Tensor, block_table: torch.Tensor,
+                                  config: PagedKvDecodeAttentionConfig, workspace: torch.Tensor | None = None) -> None:
+    """paged_kv_decode_attention_f16 (paged.rs): the bf16 op on f16 operands, same scratch."""
+    for tensor, name in ((out, "out"), (query, "query"), (key_cache, "key_cache"), (value_cache, "value_cache")):
+        _require(tensor, torch.float16, name)
+    _require(actual_seq_lens, torch.int32, "actual_seq_lens")
+    if block_table.dtype not in (torch.int32, torch.uint32):
+        raise error.InvalidArgument(f"block_table must hold 32-bit entries, got {block_table.dtype}")
+    _require(block_table, block_table.dtype, "block_table")
+    c = config._c()
+    if workspace is None:
+        need = int(_native.lib().singe_hip_paged_kv_decode_attention_workspace_bytes(ctypes.byref(c)))
+        workspace = _workspaces.get(out.device, need)
+    status = _native.lib().singe_hip_paged_kv_decode_attention_f16(
+        _stream_handle(stream), _ptr(out), out.numel(), _ptr(query), query.numel(), _ptr(key_cache), key_cache.numel(),
+        _ptr(value_cache), value_cache.numel(), _ptr(actual_seq_lens), actual_seq_lens.numel(), _ptr(block_table),
+        block_table.numel(), _ptr(workspace), workspace.numel() * workspace.element_size(), ctypes.byref(c))
+    _native.check(status, "paged_kv_decode_attention_f16")

@@ -34,9 +34,19 @@ def compact(work):
     return kc, vc, table
 
 
-def run_gpu(work, workers=0):
+def run_gpu(work, workers=0, dtype=torch.bfloat16):
     A._native.lib().singe_hip_set_decode_workers(workers)
     try:
+        if dtype == torch.float16:
+            config = A.PagedKvDecodeAttentionConfig.contiguous(work.batch, work.heads, work.kv_heads, work.head_dim,
+                                                               work.block_size, work.physical_blocks,
+                                                               work.block_table_batch_stride, work.scale)
+            out = torch.full((work.batch, work.heads, work.head_dim), float("nan"), device="cuda", dtype=dtype)
+            A.paged_kv_decode_attention_f16(None, out, work.query.to(dtype), work.key_cache.to(dtype), work.value_cache.to(dtype),
+                                            torch.from_numpy(work.seq_lens).cuda(),
+                                            torch.from_numpy(work.block_table.view(np.int32)).cuda(), config)
+            torch.cuda.synchronize()
+            return out.float().cpu().numpy()
         config = A.PagedKvDecodeAttentionConfig.contiguous(work.batch, work.heads, work.kv_heads, work.head_dim,
                                                            work.block_size, work.physical_blocks,
                                                            work.block_table_batch_stride, work.scale)
@@ -230,3 +240,26 @@ def test_decode_one_long_sequence_spans_more_than_64_ranges():
     work = synthetic.paged_decode_workload(batch=1, heads=8, kv_heads=8, physical_blocks=640, seq_lens=[10000], seed=77)
     assert_close(run_gpu(work), run_oracle(work), "one long sequence")
     assert_close(run_gpu(work, workers=200), run_oracle(work), "one long sequence, 200 ranges")
+
+
+@pytest.mark.parametrize("heads,kv_heads,block_size", [(8, 2, 16), (8, 8, 16), (16, 1, 16), (12, 4, 7), (32, 8, 32)])
+def test_f16_decode_matches_oracle(heads, kv_heads, block_size):
+    # bf16 values are f16 values here (N(0,1) magnitudes), so the same inputs and the same oracle serve both; the
+    # f16 bounds are the bf16 ones scaled as the reference scales its own (0.03 -> 0.005, tests.rs:549-553)
+    lens = [0, 1, 15, 16, 17, 100, 257, 1300, 64]
+    blocks = sum((l + block_size - 1) // block_size for l in lens) + 5
+    work = synthetic.paged_decode_workload(batch=len(lens), heads=heads, kv_heads=kv_heads, block_size=block_size,
+                                           physical_blocks=blocks, seq_lens=lens, seed=200 + heads)
+    got, want = run_gpu(work, dtype=torch.float16), run_oracle(work)
+    assert not got[0].any()
+    gap = np.abs(got - want)
+    assert gap.max() <= MAX_ABS / 6 and gap.mean() <= MEAN_ABS / 6, (gap.max(), gap.mean())
+    # and the f16 kernel against the bf16 one on the same values: they differ by the weights' rounding only
+    assert np.abs(got - run_gpu(work)).max() <= MAX_ABS
+
+
+def test_f16_decode_headline_shape():
+    work = synthetic.paged_decode_workload(fill="used")
+    got, want = run_gpu(work, dtype=torch.float16), run_oracle(work)
+    gap = np.abs(got - want)
+    assert gap.max() <= MAX_ABS / 6 and gap.mean() <= MEAN_ABS / 6, (gap.max(), gap.mean())
