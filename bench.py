@@ -10,7 +10,8 @@ consecutive steps cannot be served from the 256 MB Infinity Cache.
 Prints one JSON line: whole-job GB/s of algorithmic bytes, the roofline of the dominant kernel
 (measured with HIP events on the launch stream) and the CPU oracle timed on a bounded sample.  The
 same line carries, under "prefill", the causal flash-attention prefill measurement (TFLOP/s against
-the dense bf16 MFMA peak).
+the dense bf16 MFMA peak), and under "chunked_prefill", "fp8_decode" and "dense_f32" the other three
+benchmark configurations.
 """
 from __future__ import annotations
 
@@ -207,6 +208,40 @@ def chunked_prefill_section(steps):
     }
 
 
+def dense_f32_section(steps):
+    """The first benchmark configuration, the f32 accuracy anchor: causal dense attention, batch 1, 8 heads,
+    512 x 512, head_dim 64, scale 1/8, tensors [batch, heads, len, dim].  Far too small for a roofline: the
+    figure is microseconds per launch."""
+    import torch
+
+    from singe_amd.kernel import attention as A
+
+    batch, heads, seq, dim = 1, 8, 512, 64
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x51A6E + 1)
+    q, k, v = (torch.randn((batch, heads, seq, dim), generator=gen, device="cuda") for _ in range(3))
+    out = torch.empty_like(q)
+    config = A.SoftcappedWindowAttentionConfig(A.bhsd_config(batch, heads, heads, seq, seq, dim, 0.125, True), 0, None)
+
+    def launch():
+        A.softcapped_window_attention_f32(None, out, q, k, v, config)
+
+    for _ in range(5):
+        launch()
+    torch.cuda.synchronize()
+    avg, median = time_launches(launch, steps, 10)
+    return {
+        "workload": "causal dense attention f32: batch 1, 8 heads, 512 x 512, head_dim 64, scale 0.125, BHSD "
+                    "(BASELINE config 1, the accuracy anchor)",
+        "value": avg * 1e3,
+        "unit": "us",
+        "us_per_step_median": median * 1e3,
+        "algorithmic_flops": 4 * dim * heads * (seq * (seq + 1) // 2),
+        "algorithmic_bytes": 4 * batch * heads * seq * dim * 4,
+        "kernel": "singe_fmha_prefill_rows_f32_d64",
+    }
+
+
 def fp8_decode_section(steps):
     """Long-context decode over an fp8 e4m3 KV cache: batch 64, 64 query / 8 KV heads, head_dim 128,
     context 32768, block 16, one f32 scale per (block, kv head) (the fifth benchmark configuration); exact numerics."""
@@ -366,6 +401,8 @@ def main():
         result["chunked_prefill"] = chunked_prefill_section(20)
         torch.cuda.empty_cache()
         result["fp8_decode"] = fp8_decode_section(10)
+        torch.cuda.empty_cache()
+        result["dense_f32"] = dense_f32_section(100)
     print(json.dumps(result), flush=True)
 
 

@@ -16,7 +16,8 @@
 // keeps its own running softmax state, merged across lane sets and waves once at the end.  Query heads are
 // taken four at a time to bound registers (a group of more than four re-reads the slice from L2).
 //
-// The same loop serves the f32 forms of the two block-table ops, paged_kv_decode_attention_f32 and
+// The same loop serves the dense f32 prefill ops at these head dimensions (fmha_prefill_f32, fmha_prefill_lse_f32,
+// softcapped_window_attention_f32) and the f32 forms of the two block-table ops, paged_kv_decode_attention_f32 and
 // paged_kv_prefill_attention_f32 (singe-kernel/src/cpu/attention.rs:1172-1341; launch API
 // singe-kernel/src/cuda/attention/paged.rs): only where the rows come from and where the result goes differ.
 #include "common.hip.h"
@@ -59,6 +60,7 @@ SINGE_DEVICE void merge(DecodeState<VEC>& mine, float other_largest, float other
 //   rows.groups, rows.begin, rows.end          query heads that share the key rows, and the keys to fold
 //   rows.query(head_in_group)                  that head's dims
 //   rows.key(k), rows.value(k)                 row k of the group's KV head
+//   rows.shape(score)                          what the scaled score becomes (a soft cap, or itself)
 //   rows.store(head_in_group, part, total)     takes the finished state; called by the LANES lanes that hold the dims
 template <int LANES, int VEC, bool ALIGNED, class Rows>
 SINGE_DEVICE void fold_rows(const Rows& rows, float scale, float* lds) {
@@ -96,6 +98,7 @@ SINGE_DEVICE void fold_rows(const Rows& rows, float scale, float* lds) {
             }
 #pragma unroll
             for (int g = 0; g < kDecodeHeadsPerPass; ++g) {
+                if (g >= static_cast<int>(live)) break;  // the same in every lane of the workgroup
                 float score = 0.0f;
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) {
@@ -106,7 +109,7 @@ SINGE_DEVICE void fold_rows(const Rows& rows, float scale, float* lds) {
                 }
 #pragma unroll
                 for (int step = 1; step < LANES; step *= 2) score += wave_xor(score, step);
-                score *= scale;
+                score = rows.shape(score * scale);
                 if (valid) {
                     DecodeState<VEC>& s = state[g];
                     const float largest = fmaxf(s.largest, score);
@@ -215,11 +218,57 @@ struct DenseSplitRows {
     SINGE_DEVICE const float* value(unsigned int k) const {
         return a.value + batch * a.value_batch_stride + kv_head * a.value_head_stride + k * a.value_sequence_stride;
     }
+    SINGE_DEVICE float shape(float score) const { return score; }
     SINGE_DEVICE void store(unsigned int g, unsigned int part, const DecodeState<VEC>& total) const {
         const unsigned int head = kv_head * groups + g;
         const float lse = finish(a.out + batch * a.output_batch_stride + head * a.output_head_stride + split * a.output_split_stride +
                                      part * (4 * VEC), total);
         if (part == 0) a.lse[batch * a.lse_batch_stride + head * a.lse_head_stride + split] = lse;
+    }
+};
+
+// fmha_prefill_f32 / fmha_prefill_lse_f32 / softcapped_window_attention_f32 (cpu/attention.rs:1758-1925):
+// workgroup = (batch, query, kv head) of dense tensors addressed through element strides.  Top-left causal
+// hides key > query; a window hides keys more than window_size away on either side (cpu/attention.rs:1860-1869).
+template <int VEC>
+struct DensePrefillRows {
+    const PrefillF32Args& a;
+    unsigned int groups, begin, end, batch, query_index, kv_head;
+    SINGE_DEVICE explicit DensePrefillRows(const PrefillF32Args& args) : a(args) {
+        groups = a.heads / a.kv_heads;
+        unsigned int unit = blockIdx.x;
+        kv_head = unit % a.kv_heads;
+        unit /= a.kv_heads;
+        query_index = unit % a.query_len;
+        batch = unit / a.query_len;
+        begin = 0;
+        end = a.key_len;
+        if (a.causal && query_index + 1 < end) end = query_index + 1;
+        if (a.window_size > 0) {
+            if (query_index > a.window_size) begin = query_index - a.window_size;
+            const unsigned long long last = static_cast<unsigned long long>(query_index) + a.window_size + 1;
+            if (last < end) end = static_cast<unsigned int>(last);
+        }
+        if (begin > end) begin = end;
+    }
+    SINGE_DEVICE const float* query(unsigned int g) const {
+        return a.query + batch * a.query_batch_stride + static_cast<size_t>(query_index) * a.query_sequence_stride +
+               (kv_head * groups + g) * a.query_head_stride;
+    }
+    SINGE_DEVICE const float* key(unsigned int k) const {
+        return a.key + batch * a.key_batch_stride + kv_head * a.key_head_stride + static_cast<size_t>(k) * a.key_sequence_stride;
+    }
+    SINGE_DEVICE const float* value(unsigned int k) const {
+        return a.value + batch * a.value_batch_stride + kv_head * a.value_head_stride + static_cast<size_t>(k) * a.value_sequence_stride;
+    }
+    SINGE_DEVICE float shape(float score) const { return a.has_soft_cap ? tanhf(score / a.soft_cap) * a.soft_cap : score; }
+    SINGE_DEVICE void store(unsigned int g, unsigned int part, const DecodeState<VEC>& total) const {
+        const unsigned int head = kv_head * groups + g;
+        const float lse = finish(a.out + batch * a.output_batch_stride + static_cast<size_t>(query_index) * a.output_sequence_stride +
+                                     head * a.output_head_stride + part * (4 * VEC), total);
+        // A row that sees no key (a window wholly past the keys) stays zero; its LSE is ln 0.
+        if (a.lse != nullptr && part == 0)
+            a.lse[(static_cast<size_t>(batch) * a.heads + head) * a.query_len + query_index] = total.sum > 0.0f ? lse : -INFINITY;
     }
 };
 
@@ -267,6 +316,7 @@ struct PagedDecodeRows {
     }
     SINGE_DEVICE const float* key(unsigned int k) const { return a.key_cache + caches.row(k); }
     SINGE_DEVICE const float* value(unsigned int k) const { return a.value_cache + caches.row(k); }
+    SINGE_DEVICE float shape(float score) const { return score; }
     SINGE_DEVICE void store(unsigned int g, unsigned int part, const DecodeState<VEC>& total) const {
         const size_t row = (static_cast<size_t>(caches.sequence) * a.heads + caches.kv_head * groups + g) * a.splits + split;
         const float lse = finish(a.out + row * caches.dim + part * (4 * VEC), total);
@@ -307,6 +357,7 @@ struct PagedPrefillRows {
     }
     SINGE_DEVICE const float* key(unsigned int k) const { return a.key_cache + caches.row(k); }
     SINGE_DEVICE const float* value(unsigned int k) const { return a.value_cache + caches.row(k); }
+    SINGE_DEVICE float shape(float score) const { return score; }
     SINGE_DEVICE void store(unsigned int g, unsigned int part, const DecodeState<VEC>& total) const {
         const size_t row = static_cast<size_t>(token) * a.heads + caches.kv_head * groups + g;
         const float lse = finish(a.out + row * caches.dim + part * (4 * VEC), total);
@@ -320,6 +371,12 @@ struct PagedPrefillRows {
     extern "C" __global__ __launch_bounds__(256) void singe_fmha_decode_splitk_f32_d##DIM(FmhaDecodeSplitKArgs args) {       \
         __shared__ float lds[4 * kDecodeHeadsPerPass * (2 + DIM)];                                                           \
         const DenseSplitRows<VEC> rows(args);                                                                                \
+        if (args.aligned) fold_rows<LANES, VEC, true>(rows, args.scale, lds);                                                \
+        else fold_rows<LANES, VEC, false>(rows, args.scale, lds);                                                            \
+    }                                                                                                                        \
+    extern "C" __global__ __launch_bounds__(256) void singe_fmha_prefill_rows_f32_d##DIM(PrefillF32Args args) {              \
+        __shared__ float lds[4 * kDecodeHeadsPerPass * (2 + DIM)];                                                           \
+        const DensePrefillRows<VEC> rows(args);                                                                              \
         if (args.aligned) fold_rows<LANES, VEC, true>(rows, args.scale, lds);                                                \
         else fold_rows<LANES, VEC, false>(rows, args.scale, lds);                                                            \
     }                                                                                                                        \

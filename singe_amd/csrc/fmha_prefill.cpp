@@ -116,6 +116,21 @@ int32_t prefill_f32(void* stream, float* out, size_t out_len, float* lse, size_t
     args.has_soft_cap = has_soft_cap ? 1u : 0u;
     args.soft_cap = soft_cap;
     args.scale = c.scale;
+    // Head dimensions that are powers of two from 4 to 256 take the row kernel (a workgroup per (batch, query, kv
+    // head), several keys per wave step); the rest the one-wave-per-row kernel below.
+    const size_t widths[] = {4, 8, 16, 32, 64, 128, 256};
+    for (int index = 0; index < 7; ++index) {
+        if (c.head_dim != widths[index]) continue;
+        const size_t strides[] = {c.query_batch_stride, c.query_sequence_stride, c.query_head_stride, c.key_batch_stride,
+                                  c.key_sequence_stride, c.key_head_stride, c.value_batch_stride, c.value_sequence_stride,
+                                  c.value_head_stride};
+        bool aligned = ((reinterpret_cast<uintptr_t>(query) | reinterpret_cast<uintptr_t>(key) | reinterpret_cast<uintptr_t>(value)) & 15u) == 0;
+        for (size_t stride : strides) aligned = aligned && stride % 4 == 0;
+        args.aligned = aligned ? 1u : 0u;
+        const uint64_t units = static_cast<uint64_t>(c.batch) * c.query_len * c.kv_heads;
+        if (units > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
+        return launch(static_cast<KernelId>(kPrefillRowsF32 + index), static_cast<unsigned>(units), 1, 1, 256, stream, args);
+    }
     const uint64_t rows = static_cast<uint64_t>(c.batch) * c.heads * c.query_len;
     const uint64_t groups = (rows + 3) / 4;
     if (groups > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");

@@ -84,6 +84,7 @@ struct PrefillF32Args {
     uint32_t has_soft_cap;
     float soft_cap;
     float scale;
+    uint32_t aligned = 0;           // row kernels: every row of query, key and value starts on a 16-byte boundary
 };
 
 struct PagedAttentionArgs {

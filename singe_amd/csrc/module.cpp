@@ -48,6 +48,9 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_kv_prefill_f32_d4", "singe_paged_kv_prefill_f32_d8", "singe_paged_kv_prefill_f32_d16",
     "singe_paged_kv_prefill_f32_d32", "singe_paged_kv_prefill_f32_d64", "singe_paged_kv_prefill_f32_d128",
     "singe_paged_kv_prefill_f32_d256",
+    "singe_fmha_prefill_rows_f32_d4", "singe_fmha_prefill_rows_f32_d8", "singe_fmha_prefill_rows_f32_d16",
+    "singe_fmha_prefill_rows_f32_d32", "singe_fmha_prefill_rows_f32_d64", "singe_fmha_prefill_rows_f32_d128",
+    "singe_fmha_prefill_rows_f32_d256",
     "singe_rotary_cache_write_f32", "singe_rotary_cache_write_bf16", "singe_rotary_cache_write_f16",
     "singe_paging_indices_i32", "singe_paging_indices_i64",
     "singe_paged_mla_attention_general_f32", "singe_paged_mla_attention_general_bf16", "singe_paged_mla_attention_general_f16",

@@ -33,6 +33,7 @@ enum KernelId : int {
     // f32 block-table decode (split over keys) and prefill, same seven head dimensions each
     kPagedKvDecodeSplitKF32, kPagedKvDecodeSplitKF32Last = kPagedKvDecodeSplitKF32 + 6,
     kPagedKvPrefillF32, kPagedKvPrefillF32Last = kPagedKvPrefillF32 + 6,
+    kPrefillRowsF32, kPrefillRowsF32Last = kPrefillRowsF32 + 6,
     kRotaryCacheF32, kRotaryCacheBf16, kRotaryCacheF16,
     kPagingIndicesI32, kPagingIndicesI64,
     // latent (MLA) attention: + element (f32, bf16, f16)
