@@ -187,13 +187,14 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
     args.key_len = static_cast<uint32_t>(c.key_len);
     args.heads = static_cast<uint32_t>(c.heads);
     args.kv_heads = static_cast<uint32_t>(c.kv_heads);
-    args.query_tiles = static_cast<uint32_t>((c.query_len + 127) / 128);
+    constexpr size_t kTileRows = 32 * kDensePrefillWaves;
+    args.query_tiles = static_cast<uint32_t>((c.query_len + kTileRows - 1) / kTileRows);
     args.scale_log2e = c.scale * 1.4426950408889634074f;
     const uint64_t rows = (static_cast<uint64_t>(c.batch) * c.heads + 7) / 8 * 8;
     const uint64_t groups = rows * ((args.query_tiles + 1) / 2);  // a workgroup takes a pair of query tiles
     if (groups > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
     const KernelId kernel = f16 ? (c.causal ? kPrefillCausalF16 : kPrefillFullF16) : (c.causal ? kPrefillCausal : kPrefillFull);
-    return launch(kernel, static_cast<unsigned>(groups), 1, 1, 256, stream, args);
+    return launch(kernel, static_cast<unsigned>(groups), 1, 1, 64 * kDensePrefillWaves, stream, args);
 }
 
 }  // namespace

@@ -4,7 +4,7 @@
 // query/out [batch, query_len, heads, 128], key/value [batch, key_len, kv_heads, 128] with element
 // strides from FmhaPrefillConfig; lse [batch, heads, query_len], natural log.
 //
-// A workgroup of four waves owns 128 query rows of one (batch, head); each wave owns 32 of them and
+// A workgroup of kDensePrefillWaves (four) waves owns 32 query rows per wave of one (batch, head); each wave
 // walks the key axis in blocks of 32 keys.  Tiles of 64 keys go from global memory straight into LDS
 // (three K stages, two V stages, one barrier per tile): while tile t is worked on, K of tile t + 2 and V of
 // tile t + 1 are on their way, so every load has a whole tile's arithmetic to land and no register holds
@@ -25,10 +25,15 @@ using namespace prefill;
 // Whether the interior tiles read their K operands a block ahead (prefill_blocks.hip.h): measured, it gains
 // nothing here (the other wave of the SIMD already covers the reads' latency) and costs 30 registers.
 constexpr bool kDenseOperandsAhead = false;
+// Waves of a workgroup, 32 query rows each: the K and V tiles a workgroup loads serve all of them.
+constexpr int kDenseWaves = kDensePrefillWaves;
 
 // One 128-row query tile of (batch, head) pair `bh`.
-template <bool CAUSAL, class Half>
+template <bool CAUSAL, class Half, int WAVES>
 SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, unsigned int bh, unsigned int query_tile) {
+    constexpr unsigned int kRows = 32u * WAVES;        // query rows of the workgroup
+    constexpr unsigned int kLoadRows = 4u * WAVES;     // key rows one load instruction of every wave brings in
+    constexpr unsigned int kLoads = kKeyTile / kLoadRows;
     const unsigned int tid = threadIdx.x, lane = tid & 63;
     // The wave index is the same in all lanes; saying so keeps everything derived from it (which blocks
     // are live, whether a block is on the mask's edge, LDS bases) in scalar registers and scalar branches.
@@ -38,7 +43,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     const unsigned int batch = bh / a.heads, head = bh % a.heads;
     const unsigned int kv_head = head / (a.heads / a.kv_heads);
 
-    const unsigned int first_row = query_tile * kQueryTile + wave * 32u;  // of this wave
+    const unsigned int first_row = query_tile * kRows + wave * 32u;  // of this wave
     const unsigned int my_query = first_row + column;
     const bool query_valid = my_query < a.query_len;
 
@@ -68,7 +73,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     // block wholly after the wave's last query contributes nothing.
     unsigned int key_end = a.key_len;
     if (CAUSAL) {
-        const unsigned int reach = query_tile * kQueryTile + kQueryTile;
+        const unsigned int reach = query_tile * kRows + kRows;
         key_end = key_end < reach ? key_end : reach;
     }
     const unsigned int tiles = (key_end + kKeyTile - 1) / kKeyTile;
@@ -96,21 +101,21 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
             const unsigned char* base = rows + static_cast<size_t>(tile * kKeyTile) * stride_bytes;
             asm("" : "+s"(base));  // a scalar the compiler cannot fold the lane's part into
 #pragma unroll
-            for (unsigned int i = 0; i < 4; ++i) {
+            for (unsigned int i = 0; i < kLoads; ++i) {
                 // The offset is pinned to this spot as a 32-bit value: hoisted and widened, it would take the
                 // load out of its scalar-base form and cost a 64-bit add per lane.
-                unsigned int offset = lane_offset + 16u * i * stride_bytes;
+                unsigned int offset = lane_offset + kLoadRows * i * stride_bytes;
                 asm volatile("" : "+v"(offset));
                 __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(base + offset),
-                                                 (lds_words_t)(stage + (16u * i + 4u * wave) * kRowBytes), 16, 0, 0);
+                                                 (lds_words_t)(stage + (kLoadRows * i + 4u * wave) * kRowBytes), 16, 0, 0);
             }
         } else {
 #pragma unroll
-            for (unsigned int i = 0; i < 4; ++i) {
-                unsigned int key = tile * kKeyTile + 16u * i + load_row;
+            for (unsigned int i = 0; i < kLoads; ++i) {
+                unsigned int key = tile * kKeyTile + kLoadRows * i + load_row;
                 key = key < a.key_len ? key : a.key_len - 1;
                 __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(rows + (key * stride_bytes + chunk)),
-                                                 (lds_words_t)(stage + (16u * i + 4u * wave) * kRowBytes), 16, 0, 0);
+                                                 (lds_words_t)(stage + (kLoadRows * i + 4u * wave) * kRowBytes), 16, 0, 0);
             }
         }
     };
@@ -225,23 +230,23 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
 }
 
 // Workgroup id -> (batch * heads + head, pair of query tiles): see the header comment.
-template <bool CAUSAL, class Half>
+template <bool CAUSAL, class Half, int WAVES>
 SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
     const unsigned int xcd = blockIdx.x & 7u, within = blockIdx.x >> 3;
     const unsigned int pairs = (a.query_tiles + 1u) / 2u;
     const unsigned int bh = (within / pairs) * 8u + xcd;
     if (bh >= a.batch * a.heads) return;
     const unsigned int light = within % pairs, heavy = a.query_tiles - 1u - light;
-    fmha_prefill_tile<CAUSAL, Half>(a, lds, bh, heavy);
-    if (light != heavy) fmha_prefill_tile<CAUSAL, Half>(a, lds, bh, light);
+    fmha_prefill_tile<CAUSAL, Half, WAVES>(a, lds, bh, heavy);
+    if (light != heavy) fmha_prefill_tile<CAUSAL, Half, WAVES>(a, lds, bh, light);
 }
 
 }  // namespace
 
 #define SINGE_FMHA_PREFILL_KERNEL(NAME, CAUSAL, HALF)                                              \
-    extern "C" __global__ __launch_bounds__(256, 2) void NAME(PrefillArgs args) {                    \
+    extern "C" __global__ __launch_bounds__(64 * kDenseWaves, 8 / kDenseWaves) void NAME(PrefillArgs args) { \
         __shared__ __attribute__((aligned(1024))) unsigned char prefill_lds[kStagedLdsBytes];        \
-        fmha_prefill_body<CAUSAL, prefill::HALF>(args, prefill_lds);                                \
+        fmha_prefill_body<CAUSAL, prefill::HALF, kDenseWaves>(args, prefill_lds);                   \
     }
 
 SINGE_FMHA_PREFILL_KERNEL(singe_fmha_prefill_bf16_d128_causal, true, Bf16)

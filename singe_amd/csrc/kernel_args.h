@@ -44,6 +44,11 @@ struct CombineArgs {
     uint32_t heads_per_wave;
 };
 
+// Waves of a dense prefill workgroup (singe_fmha_prefill_*_d128_*), 32 query rows each: host and kernel agree on
+// it through this constant.  4 (two workgroups per compute unit) and 8 (one, whose K and V tiles serve 256 rows)
+// both pass the tests and measure the same; 4 is what the committed profiles were taken with.
+constexpr int kDensePrefillWaves = 4;
+
 struct PrefillArgs {
     const uint16_t* query;          // [batch, query_len, heads, 128] bf16, element strides below
     const uint16_t* key;            // [batch, key_len, kv_heads, 128]
