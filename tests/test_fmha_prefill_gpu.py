@@ -111,3 +111,30 @@ def test_prefill_validation_errors():
         A.fmha_prefill_bf16(None, out, q, k[:, :63].contiguous(), v, good)
     with pytest.raises(error.UnsupportedWidth):
         A.fmha_prefill_bf16(None, out, q, k, v, A.FmhaPrefillConfig.contiguous(1, 64, 64, 4, 2, 64, 0.1, True))
+
+
+@pytest.mark.parametrize("magnitude,causal", [(8.0, True), (8.0, False), (30.0, True), (0.01, True)])
+def test_scores_that_keep_outrunning_the_reference_point(magnitude, causal):
+    # Scores grow steadily along the keys (by far more than the lag the running maximum is allowed), so every
+    # block moves the softmax reference point and rescales the output; small magnitudes give a flat softmax.
+    batch, seq, heads, kv_heads = 1, 700, 4, 2
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(int(magnitude * 100) + int(causal))
+    q = (torch.randn((batch, seq, heads, 128), generator=gen, device="cuda") * magnitude).to(torch.bfloat16)
+    k = (torch.randn((batch, seq, kv_heads, 128), generator=gen, device="cuda") * magnitude).to(torch.bfloat16)
+    v = torch.randn((batch, seq, kv_heads, 128), generator=gen, device="cuda").to(torch.bfloat16)
+    k[:, :, :, 0] += torch.linspace(0, 40 * magnitude, seq, device="cuda").to(torch.bfloat16)[None, :, None]
+    q[:, :, :, 0] = magnitude
+    scale = float(1.0 / np.sqrt(np.float32(128)))
+    config = A.FmhaPrefillConfig.contiguous(batch, seq, seq, heads, kv_heads, 128, scale, causal)
+    out = torch.full_like(q, float("nan"))
+    lse = torch.full((batch, heads, seq), float("nan"), device="cuda", dtype=torch.float32)
+    A.fmha_prefill_lse_bf16(None, out, lse, q, k, v, config)
+    want, want_lse = oracle.fmha_prefill_lse_f32(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), batch=batch,
+                                                 query_len=seq, key_len=seq, heads=heads, kv_heads=kv_heads, head_dim=128,
+                                                 scale=scale, causal=causal, threads=8)
+    got = out.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    gap = np.abs(got - want)
+    assert gap.max() <= 2e-2 and gap.mean() <= 2e-3, (gap.max(), gap.mean())
+    assert (np.abs(lse.cpu().numpy() - want_lse) / np.maximum(1.0, np.abs(want_lse))).max() <= 1e-5
