@@ -263,3 +263,14 @@ def test_f16_decode_headline_shape():
     got, want = run_gpu(work, dtype=torch.float16), run_oracle(work)
     gap = np.abs(got - want)
     assert gap.max() <= MAX_ABS / 6 and gap.mean() <= MEAN_ABS / 6, (gap.max(), gap.mean())
+
+
+@pytest.mark.parametrize("magnitude", [20.0, 0.01])
+def test_decode_peaked_and_flat_softmax(magnitude):
+    # Queries twenty times larger give scores of standard deviation twenty (one or two keys carry a row and the
+    # running maximum keeps jumping); a hundred times smaller give a flat average of the values.
+    lens = [700, 33, 1024, 5]
+    work = synthetic.paged_decode_workload(batch=len(lens), heads=8, kv_heads=2, physical_blocks=160, seq_lens=lens, seed=77)
+    work.query.mul_(magnitude)
+    got, want = run_gpu(work), run_oracle(work)
+    assert_close(got, want, f"magnitude {magnitude}")
