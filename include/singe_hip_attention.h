@@ -703,7 +703,7 @@ typedef struct SingeFmhaDecodeSplitKReduceConfig {
  * laid out [batch, heads, splits] (mod.rs:2456-2539).  Timing candidates synchronises the stream's events and is
  * refused while the stream is being captured (SINGE_HIP_AUTOTUNE_DURING_CAPTURE), also when the cache would
  * have answered, as in the reference (fmha.rs:1203-1207); winners are cached per process and device, keyed
- * by (batch, key_len, heads, kv_heads, head_dim, max_splits), and the winner is launched once more so `out`
+ * by the extents, max_splits and the strides (TuneProblemKey::AttentionSplitK, mod.rs:2394-2413), and the winner is launched once more so `out`
  * holds its result. */
 SINGE_HIP_API int32_t singe_hip_fmha_decode_splitk_reduce_f32(
     void* stream,

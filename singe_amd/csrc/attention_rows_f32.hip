@@ -1,5 +1,6 @@
-// Dense f32 decode attention over a slice of the keys: the gfx950 counterpart of fmha_decode_splitk_f32
-// (kernel singe-kernel/src/cuda/cutile/kernel/attention/local.rs:6127-6272, launch API
+// f32 attention rows on the vector unit: one loop, four ops.  Its first form is dense decode over a slice of the
+// keys, the gfx950 counterpart of fmha_decode_splitk_f32 (kernel
+// singe-kernel/src/cuda/cutile/kernel/attention/local.rs:6127-6272, launch API
 // singe-kernel/src/cuda/attention/fmha.rs:1074-1118), the first half of the reference's split-KV convention
 // (fmha_decode_splitk_reduce_f32, fmha.rs:1155-1250); splitk_reduce.hip is the second half.
 //

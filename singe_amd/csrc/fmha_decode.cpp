@@ -7,7 +7,7 @@
 #include <limits>
 #include <map>
 #include <mutex>
-#include <tuple>
+#include <array>
 #include <vector>
 
 #include "kernel_args.h"
@@ -221,8 +221,9 @@ std::vector<size_t> candidates(const SingeFmhaDecodeSplitKReduceConfig& c) {
     return splits;
 }
 
-// The tune cache: what TuneProblemKey::AttentionSplitK holds (mod.rs:2382-2415) plus the device.
-using TuneKey = std::tuple<int, size_t, size_t, size_t, size_t, size_t, size_t>;
+// The tune cache: the device and what TuneProblemKey::AttentionSplitK holds (mod.rs:2382-2415): the extents,
+// max_splits and the ten strides.
+using TuneKey = std::array<size_t, 17>;
 std::mutex g_tune_mutex;
 std::map<TuneKey, size_t> g_tuned;
 
@@ -231,7 +232,9 @@ bool tune_key(const SingeFmhaDecodeSplitKReduceConfig& c, TuneKey* key) {
     int device = 0;
     if (hip == nullptr || hip->hipGetDevice(&device) != hipSuccess) return false;
     const SingeFmhaDecodeConfig& d = c.decode;
-    *key = TuneKey(device, d.batch, d.key_len, d.heads, d.kv_heads, d.head_dim, c.max_splits);
+    *key = TuneKey{static_cast<size_t>(device), d.batch, d.key_len, d.heads, d.kv_heads, d.head_dim, c.max_splits,
+                   d.query_batch_stride, d.key_batch_stride, d.value_batch_stride, d.output_batch_stride, d.query_head_stride,
+                   d.key_sequence_stride, d.value_sequence_stride, d.output_head_stride, d.key_head_stride, d.value_head_stride};
     return true;
 }
 

@@ -2,7 +2,7 @@
 // paged_kv_prefill_attention_f32 (singe-kernel/src/cuda/attention/paged.rs; CPU forms
 // singe-kernel/src/cpu/attention.rs:1172-1341), validated as the bf16 entry points are
 // (PagedKvDecodeAttentionConfig::validate_lengths, mod.rs:711-743; PagedKvPrefillAttentionConfig::validate_lengths,
-// mod.rs:786-818) and run on the vector-unit row kernels of fmha_decode.hip.
+// mod.rs:786-818) and run on the vector-unit row kernels of attention_rows_f32.hip.
 #include <algorithm>
 #include <cmath>
 

@@ -5,7 +5,7 @@
 #include "fmha_prefill_f32.hip"
 #include "paged_attention.hip"
 #include "splitk_reduce.hip"
-#include "fmha_decode.hip"
+#include "attention_rows_f32.hip"
 #include "general_attention.hip"
 #include "latent_attention.hip"
 #include "cache_ops.hip"
