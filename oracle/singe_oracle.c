@@ -29,7 +29,8 @@
  * has no CPU form in the reference at all: its restatement follows the GPU kernel), and the
  * Rust original cannot be compiled in this image, so their last-ulp f32 outputs are "parity
  * unpinned": pinned only by construction plus closed forms and invariants (see
- * tests/test_oracle.py and tests/test_fmha_decode_splitk_cpu.py);
+ * tests/test_oracle.py and tests/test_fmha_decode_splitk_cpu.py) and, to 3e-6, by the
+ * answers of a library routine kept as fixtures (tests/test_golden_fixtures.py);
  * everything integer (gather offsets, lengths, the paging error contract),
  * the GQA head map, the causal direction, the fp8 and bf16 codecs are pinned
  * against the reference's own test vectors.
