@@ -41,6 +41,14 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     const unsigned int column = lane & 31, hi = lane >> 5;
 
     const unsigned int batch = bh / a.heads, head = bh % a.heads;
+    // Keys that take part: all of them, or the batch entry's own count (singe/src/backend/cpu/normalization/attention.rs:191-276, key_lengths).
+    unsigned int key_len = a.key_len;
+    if (a.key_lengths != nullptr) {
+        const int own = a.key_lengths[batch];
+        const unsigned int bound = own > 0 ? static_cast<unsigned int>(own) : 0u;
+        key_len = bound < key_len ? bound : key_len;
+    }
+    key_len = __builtin_amdgcn_readfirstlane(key_len);
     const unsigned int kv_head = head / (a.heads / a.kv_heads);
 
     const unsigned int first_row = query_tile * kRows + wave * 32u;  // of this wave
@@ -71,7 +79,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
 
     // Keys this workgroup must visit, and the blocks of them this wave folds: under the causal mask a
     // block wholly after the wave's last query contributes nothing.
-    unsigned int key_end = a.key_len;
+    unsigned int key_end = key_len;
     if (CAUSAL) {
         const unsigned int reach = query_tile * kRows + kRows;
         key_end = key_end < reach ? key_end : reach;
@@ -97,7 +105,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     const unsigned int key_lane = load_row * key_stride_bytes + key_chunk, value_lane = load_row * value_stride_bytes + value_chunk;
     auto load_tile = [&](const unsigned char* rows, unsigned int stride_bytes, unsigned int lane_offset, unsigned int chunk,
                          unsigned int tile, unsigned char* stage) __attribute__((always_inline)) {
-        if (tile * kKeyTile + kKeyTile <= a.key_len) {
+        if (tile * kKeyTile + kKeyTile <= key_len) {
             const unsigned char* base = rows + static_cast<size_t>(tile * kKeyTile) * stride_bytes;
             asm("" : "+s"(base));  // a scalar the compiler cannot fold the lane's part into
 #pragma unroll
@@ -113,7 +121,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
 #pragma unroll
             for (unsigned int i = 0; i < kLoads; ++i) {
                 unsigned int key = tile * kKeyTile + kLoadRows * i + load_row;
-                key = key < a.key_len ? key : a.key_len - 1;
+                key = key < key_len ? key : key_len - 1;
                 __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(rows + (key * stride_bytes + chunk)),
                                                  (lds_words_t)(stage + (kLoadRows * i + 4u * wave) * kRowBytes), 16, 0, 0);
             }
@@ -128,6 +136,16 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
 
     RowState state;
     reset(state);
+    if (a.sinks != nullptr) {
+        // The head's sink: a score that is always there and weighs no value.  The row starts with it as its reference
+        // point and a sum of one (held by one of the row's two lanes).
+        const uint16_t bits = a.sinks[head];
+        float sink;
+        if constexpr (std::is_same_v<Half, F16>) sink = static_cast<float>(__builtin_bit_cast(_Float16, bits));
+        else sink = __builtin_bit_cast(float, static_cast<unsigned int>(bits) << 16);
+        state.reference = sink * kLog2e;
+        state.running_sum = hi == 0 && state.reference != -INFINITY ? 1.0f : 0.0f;
+    }
     const ReadOffsets offsets = read_offsets(lane);
 
     if (tiles > 0) {
@@ -141,10 +159,10 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     // Folds block `block` (scores in `s`, values at `values`) with the mask's edges applied.
     auto fold = [&](unsigned int block, f32x16_t& s, const unsigned char* values) __attribute__((always_inline)) {
         const unsigned int key0 = block * 32u;
-        const bool edge = (CAUSAL && key0 + 31u > first_row) || key0 + 32u > a.key_len;
+        const bool edge = (CAUSAL && key0 + 31u > first_row) || key0 + 32u > key_len;
         const float shift = begin_block(state, s, hi, factor, edge, [&](unsigned int key_in_block) {
             const unsigned int key = key0 + key_in_block;
-            return (CAUSAL && key > my_query) || key >= a.key_len;
+            return (CAUSAL && key > my_query) || key >= key_len;
         });
         finish_block<false>(half, state, s, factor, shift, values, offsets, s, q, values);
     };
@@ -183,7 +201,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
         interior_tiles = interior_tiles < unmasked ? interior_tiles : unmasked;
     }
     {
-        const unsigned int whole = a.key_len / kKeyTile;  // tiles t with 64 t + 64 <= key_len
+        const unsigned int whole = key_len / kKeyTile;  // tiles t with 64 t + 64 <= key_len
         interior_tiles = interior_tiles < whole ? interior_tiles : whole;
     }
     unsigned int tile = 0;

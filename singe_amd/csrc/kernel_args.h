@@ -66,6 +66,11 @@ struct PrefillArgs {
     uint32_t kv_heads;
     uint32_t query_tiles;           // ceil(query_len / 128)
     float scale_log2e;
+    // The two options of the dense op this kernel takes (null when absent): one logit per query head that joins
+    // every row's softmax without a value, in the element type of the query; and the number of keys of each batch
+    // entry that take part (the rest are hidden).
+    const uint16_t* sinks = nullptr;
+    const int32_t* key_lengths = nullptr;
 };
 
 struct PrefillF32Args {

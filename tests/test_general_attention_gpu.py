@@ -117,6 +117,40 @@ def test_dense_bf16_at_128_takes_the_matrix_core_kernel_and_matches():
         close(host(out), want, torch.bfloat16)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [False, True])
+def test_dense_at_128_with_sinks_and_key_lengths_on_the_matrix_core_kernel(dtype, causal):
+    # Sinks and key lengths stay on the flash kernel at head dimension 128; a mask, a window or a cap do not.
+    batch, heads, kv_heads, query_len, key_len = 3, 8, 2, 150, 333
+    q, k, v = tensors((batch, heads, query_len, 128), (batch, kv_heads, key_len, 128), (batch, kv_heads, key_len, 128), dtype, 17)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(9)
+    sinks = (torch.randn((heads,), generator=gen, device="cuda") * 3).to(dtype)
+    sinks[1] = float("-inf")  # a sink that never counts
+    sinks[2] = 30.0           # a sink that takes nearly all of every row
+    options = neural.AttentionOptions(causal=causal)
+    out = neural.attend(q, k, v, None, sinks, options)
+    want = oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), causal=causal, sinks=host(sinks), threads=8)
+    close(host(out), want, dtype)
+    lengths = torch.tensor([0, 77, 400], dtype=torch.int32, device="cuda")
+    out = neural.attend_padded(q, k, v, lengths, options)
+    want = oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), causal=causal, key_lengths=[0, 77, 400], threads=8)
+    close(host(out), want, dtype)
+    assert not host(out)[0].any()
+    # Both at once, through the C ABI's nullable operands.
+    import ctypes
+    from singe_amd import _native
+    problem = _native.AttentionProblemC(batch, heads, kv_heads, query_len, key_len, 128, 128, (ctypes.c_int64 * 4)(0, 0, 0, 0),
+                                        {torch.bfloat16: 1, torch.float16: 2}[dtype], int(causal), 0, 0, 0, 0.0, 0.0, 0)
+    both = torch.empty_like(q)
+    status = _native.lib().singe_hip_scaled_dot_product_attention(None, q.data_ptr(), k.data_ptr(), v.data_ptr(), None, sinks.data_ptr(),
+                                                                  lengths.data_ptr(), both.data_ptr(), ctypes.byref(problem))
+    assert status == 0
+    want = oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), causal=causal, sinks=host(sinks), key_lengths=[0, 77, 400],
+                                                   threads=8)
+    close(host(both), want, dtype)
+
+
 def test_dense_shape_rules():
     q, k, v = tensors((1, 4, 8, 32), (1, 3, 8, 32), (1, 3, 8, 32), torch.float32, 1)
     with pytest.raises(error.InvalidArgument):
