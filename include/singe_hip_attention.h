@@ -507,9 +507,10 @@ SINGE_HIP_API int32_t singe_hip_paged_attention_f16(
  * type of the query, read through mask_strides over (batch, head, query, key), 0 = broadcast) adds to
  * them; `sinks` [heads] joins each row's softmax without weighing a value; `key_lengths` [batch] i32
  * hides the keys past each batch's count (a count of zero gives zeros).  mask, sinks and key_lengths may
- * be null.  head_dim and value_dim up to 256.  bf16 and f16 at head_dim = value_dim = 128 without a mask, a
- * window or a cap (sinks and key_lengths allowed) run on the matrix-core flash kernel of fmha_prefill_*; every
- * other combination on the vector-unit kernel. */
+ * be null.  head_dim and value_dim up to 256.  bf16 and f16 at head_dim = value_dim = 128 run on the matrix-core
+ * flash kernel of fmha_prefill_* with every option (a mask, a window or a cap take its block-by-block masked path);
+ * other widths and f32 on the vector-unit kernel.  A row whose every key is hidden gives zeros (the CPU form
+ * divides zero by zero there). */
 #define SINGE_HIP_F32 0
 #define SINGE_HIP_BF16 1
 #define SINGE_HIP_F16 2

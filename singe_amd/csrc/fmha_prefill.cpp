@@ -141,8 +141,7 @@ int32_t prefill_f32(void* stream, float* out, size_t out_len, float* lse, size_t
 
 int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, bool with_lse,
                 const uint16_t* query, size_t query_len, const uint16_t* key, size_t key_len, const uint16_t* value,
-                size_t value_len, const SingeFmhaPrefillConfig* config, bool f16 = false, const uint16_t* sinks = nullptr,
-                const int32_t* key_lengths = nullptr) {
+                size_t value_len, const SingeFmhaPrefillConfig* config, bool f16 = false, const DenseOptions& options = DenseOptions()) {
     if (config == nullptr) return fail(SINGE_HIP_NULL_POINTER, "config");
     const SingeFmhaPrefillConfig& c = *config;
     if (int32_t status = validate_call(c, out, out_len, lse, lse_len, with_lse, query, query_len, key, key_len, value, value_len))
@@ -191,12 +190,20 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
     constexpr size_t kTileRows = 32 * kDensePrefillWaves;
     args.query_tiles = static_cast<uint32_t>((c.query_len + kTileRows - 1) / kTileRows);
     args.scale_log2e = c.scale * 1.4426950408889634074f;
-    args.sinks = sinks;
-    args.key_lengths = key_lengths;
+    args.sinks = options.sinks;
+    args.key_lengths = options.key_lengths;
+    const bool with_options = options.mask != nullptr || options.window >= 0 || options.softcap != 0.0f;
+    args.mask = options.mask;
+    for (int i = 0; i < 4; ++i) args.mask_strides[i] = options.mask_strides[i];
+    args.window = options.window;
+    if (options.softcap != 0.0f) {
+        args.cap_scale = std::fabs(c.scale / options.softcap);
+        args.cap_log2e = std::fabs(options.softcap) * 1.4426950408889634074f;
+    }
     const uint64_t rows = (static_cast<uint64_t>(c.batch) * c.heads + 7) / 8 * 8;
     const uint64_t groups = rows * ((args.query_tiles + 1) / 2);  // a workgroup takes a pair of query tiles
     if (groups > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
-    const KernelId kernel = f16 ? (c.causal ? kPrefillCausalF16 : kPrefillFullF16) : (c.causal ? kPrefillCausal : kPrefillFull);
+    const KernelId kernel = static_cast<KernelId>((f16 ? kPrefillCausalF16 : kPrefillCausal) + (c.causal ? 0 : 1) + (with_options ? 4 : 0));
     return launch(kernel, static_cast<unsigned>(groups), 1, 1, 64 * kDensePrefillWaves, stream, args);
 }
 
@@ -204,13 +211,12 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
 
 namespace singe_hip {
 
-// The dense op's way into the matrix-core kernel: the public entry points' checks and launch, plus the op's two
-// options the kernel takes (general_attention.cpp).
+// The dense op's way into the matrix-core kernel: the public entry points' checks and launch, plus the op's options
+// (general_attention.cpp).
 int32_t dense_prefill_with_options(void* stream, bool f16, uint16_t* out, size_t out_len, const uint16_t* query, size_t query_len,
                                    const uint16_t* key, size_t key_len, const uint16_t* value, size_t value_len,
-                                   const SingeFmhaPrefillConfig* config, const uint16_t* sinks, const int32_t* key_lengths) {
-    return prefill(stream, out, out_len, nullptr, 0, false, query, query_len, key, key_len, value, value_len, config, f16, sinks,
-                   key_lengths);
+                                   const SingeFmhaPrefillConfig* config, const DenseOptions& options) {
+    return prefill(stream, out, out_len, nullptr, 0, false, query, query_len, key, key_len, value, value_len, config, f16, options);
 }
 
 }  // namespace singe_hip

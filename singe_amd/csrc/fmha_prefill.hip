@@ -29,7 +29,9 @@ constexpr bool kDenseOperandsAhead = false;
 constexpr int kDenseWaves = kDensePrefillWaves;
 
 // One 128-row query tile of (batch, head) pair `bh`.
-template <bool CAUSAL, class Half, int WAVES>
+// OPTIONS: the dense op's additive mask, window and score cap, applied block by block to the scaled scores; every
+// tile then takes the masked path.
+template <bool CAUSAL, class Half, int WAVES, bool OPTIONS>
 SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, unsigned int bh, unsigned int query_tile) {
     constexpr unsigned int kRows = 32u * WAVES;        // query rows of the workgroup
     constexpr unsigned int kLoadRows = 4u * WAVES;     // key rows one load instruction of every wave brings in
@@ -159,6 +161,38 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     // Folds block `block` (scores in `s`, values at `values`) with the mask's edges applied.
     auto fold = [&](unsigned int block, f32x16_t& s, const unsigned char* values) __attribute__((always_inline)) {
         const unsigned int key0 = block * 32u;
+        if constexpr (OPTIONS) {
+            // Scores in their final units (base-two logits): scaled, capped (singe/src/backend/cpu/normalization/
+            // attention.rs:255-262: the cap, then the mask), the mask added.  Register r of lane (query, hi) is key
+            // key0 + 8 (r / 4) + 4 hi + (r % 4).
+            const bool capped = a.cap_log2e != 0.0f;
+            const float to_units = capped ? a.cap_scale : factor;
+            const uint16_t* mask_row = nullptr;
+            if (a.mask != nullptr)
+                mask_row = a.mask + batch * a.mask_strides[0] + head * a.mask_strides[1] + static_cast<size_t>(query_valid ? my_query : 0) * a.mask_strides[2];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                float x = s[r] * to_units;
+                if (capped) x = tanhf(x) * a.cap_log2e;
+                if (mask_row != nullptr) {
+                    const unsigned int key = key0 + 8u * (r >> 2) + 4u * hi + (r & 3);
+                    const uint16_t bits = mask_row[static_cast<size_t>(key < key_len ? key : 0) * a.mask_strides[3]];
+                    float extra;
+                    if constexpr (std::is_same_v<Half, F16>) extra = static_cast<float>(__builtin_bit_cast(_Float16, bits));
+                    else extra = __builtin_bit_cast(float, static_cast<unsigned int>(bits) << 16);
+                    x += extra * kLog2e;
+                }
+                s[r] = x;
+            }
+            const bool windowed = a.window >= 0;
+            const unsigned long long window = windowed ? static_cast<unsigned long long>(a.window) : 0ull;
+            const float shift = begin_block(state, s, hi, 1.0f, true, [&](unsigned int key_in_block) {
+                const unsigned int key = key0 + key_in_block;
+                return (CAUSAL && key > my_query) || key >= key_len || (windowed && key + window <= my_query);
+            });
+            finish_block<false>(half, state, s, 1.0f, shift, values, offsets, s, q, values);
+            return;
+        }
         const bool edge = (CAUSAL && key0 + 31u > first_row) || key0 + 32u > key_len;
         const float shift = begin_block(state, s, hi, factor, edge, [&](unsigned int key_in_block) {
             const unsigned int key = key0 + key_in_block;
@@ -204,6 +238,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
         const unsigned int whole = key_len / kKeyTile;  // tiles t with 64 t + 64 <= key_len
         interior_tiles = interior_tiles < whole ? interior_tiles : whole;
     }
+    if (OPTIONS) interior_tiles = 0;
     unsigned int tile = 0;
     uint4 operand[8];
     if (kDenseOperandsAhead && interior_tiles > 0) read_key_operands(operand, lds + kBlockBytes, offsets);
@@ -248,15 +283,15 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
 }
 
 // Workgroup id -> (batch * heads + head, pair of query tiles): see the header comment.
-template <bool CAUSAL, class Half, int WAVES>
+template <bool CAUSAL, class Half, int WAVES, bool OPTIONS = false>
 SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
     const unsigned int xcd = blockIdx.x & 7u, within = blockIdx.x >> 3;
     const unsigned int pairs = (a.query_tiles + 1u) / 2u;
     const unsigned int bh = (within / pairs) * 8u + xcd;
     if (bh >= a.batch * a.heads) return;
     const unsigned int light = within % pairs, heavy = a.query_tiles - 1u - light;
-    fmha_prefill_tile<CAUSAL, Half, WAVES>(a, lds, bh, heavy);
-    if (light != heavy) fmha_prefill_tile<CAUSAL, Half, WAVES>(a, lds, bh, light);
+    fmha_prefill_tile<CAUSAL, Half, WAVES, OPTIONS>(a, lds, bh, heavy);
+    if (light != heavy) fmha_prefill_tile<CAUSAL, Half, WAVES, OPTIONS>(a, lds, bh, light);
 }
 
 }  // namespace
@@ -267,6 +302,16 @@ SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
         fmha_prefill_body<CAUSAL, prefill::HALF, kDenseWaves>(args, prefill_lds);                   \
     }
 
+#define SINGE_FMHA_PREFILL_OPTIONS_KERNEL(NAME, CAUSAL, HALF)                                      \
+    extern "C" __global__ __launch_bounds__(64 * kDenseWaves, 8 / kDenseWaves) void NAME(PrefillArgs args) { \
+        __shared__ __attribute__((aligned(1024))) unsigned char prefill_lds[kStagedLdsBytes];        \
+        fmha_prefill_body<CAUSAL, prefill::HALF, kDenseWaves, true>(args, prefill_lds);             \
+    }
+
+SINGE_FMHA_PREFILL_OPTIONS_KERNEL(singe_fmha_prefill_bf16_d128_causal_options, true, Bf16)
+SINGE_FMHA_PREFILL_OPTIONS_KERNEL(singe_fmha_prefill_bf16_d128_full_options, false, Bf16)
+SINGE_FMHA_PREFILL_OPTIONS_KERNEL(singe_fmha_prefill_f16_d128_causal_options, true, F16)
+SINGE_FMHA_PREFILL_OPTIONS_KERNEL(singe_fmha_prefill_f16_d128_full_options, false, F16)
 SINGE_FMHA_PREFILL_KERNEL(singe_fmha_prefill_bf16_d128_causal, true, Bf16)
 SINGE_FMHA_PREFILL_KERNEL(singe_fmha_prefill_bf16_d128_full, false, Bf16)
 SINGE_FMHA_PREFILL_KERNEL(singe_fmha_prefill_f16_d128_causal, true, F16)

@@ -101,10 +101,9 @@ extern "C" int32_t singe_hip_scaled_dot_product_attention(void* stream, const vo
     if (output == nullptr) return fail(SINGE_HIP_NULL_POINTER, "output");
     const float scale = p.has_scale ? p.scale : 1.0f / std::sqrt(static_cast<float>(p.head_dim));
 
-    // bf16 and f16 at head dimension 128 with no mask, window or cap are what the MFMA flash kernel computes,
-    // sinks and key lengths included, reading [batch, heads, len, dim] through its strides.
-    if ((p.data_type == SINGE_HIP_BF16 || p.data_type == SINGE_HIP_F16) && p.head_dim == 128 && p.value_dim == 128 && mask == nullptr &&
-        !p.has_window && !p.has_softcap) {
+    // bf16 and f16 at head dimension 128 are what the MFMA flash kernel computes, every option included, reading
+    // [batch, heads, len, dim] through its strides.
+    if ((p.data_type == SINGE_HIP_BF16 || p.data_type == SINGE_HIP_F16) && p.head_dim == 128 && p.value_dim == 128) {
         SingeFmhaPrefillConfig c;
         c.batch = p.batch, c.query_len = p.query_len, c.key_len = p.key_len, c.heads = p.heads, c.kv_heads = p.kv_heads, c.head_dim = 128;
         c.query_batch_stride = c.output_batch_stride = static_cast<size_t>(p.heads) * p.query_len * 128;
@@ -114,9 +113,16 @@ extern "C" int32_t singe_hip_scaled_dot_product_attention(void* stream, const vo
         c.key_head_stride = c.value_head_stride = static_cast<size_t>(p.key_len) * 128;
         c.scale = scale, c.causal = p.causal ? 1 : 0;
         const size_t q_len = static_cast<size_t>(rows) * 128, kv_len = static_cast<size_t>(p.batch) * p.kv_heads * p.key_len * 128;
+        DenseOptions options;
+        options.sinks = static_cast<const uint16_t*>(sinks);
+        options.key_lengths = key_lengths;
+        options.mask = static_cast<const uint16_t*>(mask);
+        for (int i = 0; i < 4; ++i) options.mask_strides[i] = static_cast<uint64_t>(p.mask_strides[i]);
+        options.window = p.has_window ? p.window : -1;
+        options.softcap = p.has_softcap ? p.softcap : 0.0f;
         return dense_prefill_with_options(stream, p.data_type == SINGE_HIP_F16, static_cast<uint16_t*>(output), q_len,
                                           static_cast<const uint16_t*>(query), q_len, static_cast<const uint16_t*>(key), kv_len,
-                                          static_cast<const uint16_t*>(value), kv_len, &c, static_cast<const uint16_t*>(sinks), key_lengths);
+                                          static_cast<const uint16_t*>(value), kv_len, &c, options);
     }
 
     KernelId kernel;

@@ -71,6 +71,14 @@ struct PrefillArgs {
     // entry that take part (the rest are hidden).
     const uint16_t* sinks = nullptr;
     const int32_t* key_lengths = nullptr;
+    // The *_options kernels only: an additive mask in the element type of the query, read through element strides
+    // over (batch, head, query, key) with 0 for a broadcast axis (null when absent); a window that hides
+    // key + window <= query (negative when absent); a cap on the scaled scores, cap * tanh(score / cap)
+    // (cap_scale = |scale / cap|, cap_log2e = |cap| * log2(e); both 0 when absent).
+    const uint16_t* mask = nullptr;
+    uint64_t mask_strides[4] = {0, 0, 0, 0};
+    long long window = -1;
+    float cap_scale = 0.0f, cap_log2e = 0.0f;
 };
 
 struct PrefillF32Args {

@@ -23,6 +23,8 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_decode_f8kv_wide_relaxed_d128_b16", "singe_paged_decode_f8kv_wide_relaxed_d128_any",
     "singe_fmha_prefill_bf16_d128_causal", "singe_fmha_prefill_bf16_d128_full",
     "singe_fmha_prefill_f16_d128_causal", "singe_fmha_prefill_f16_d128_full",
+    "singe_fmha_prefill_bf16_d128_causal_options", "singe_fmha_prefill_bf16_d128_full_options",
+    "singe_fmha_prefill_f16_d128_causal_options", "singe_fmha_prefill_f16_d128_full_options",
     "singe_fmha_prefill_f32_d32", "singe_fmha_prefill_f32_d64", "singe_fmha_prefill_f32_d128", "singe_fmha_prefill_f32_d256",
     "singe_paged_attention_bf16_d128_i32", "singe_paged_attention_bf16_d128_i64",
     "singe_paged_attention_bf16_d128_softcap_i32", "singe_paged_attention_bf16_d128_softcap_i64",

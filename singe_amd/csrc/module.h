@@ -17,6 +17,8 @@ enum KernelId : int {
     // fp8 decode, dense form: + (block size not a multiple of 16) + 2 * relaxed
     kDecodeF8Wide, kDecodeF8WideAny, kDecodeF8WideRelaxed, kDecodeF8WideRelaxedAny,
     kPrefillCausal, kPrefillFull, kPrefillCausalF16, kPrefillFullF16,
+    // the same four with the dense op's mask, window and cap
+    kPrefillCausalOptions, kPrefillFullOptions, kPrefillCausalOptionsF16, kPrefillFullOptionsF16,
     kPrefillF32D32, kPrefillF32D64, kPrefillF32D128, kPrefillF32D256,
     // paged attention: + 4 when the page size is a power of two of at least 16 keys
     kPagedAttentionI32, kPagedAttentionI64, kPagedAttentionSoftcapI32, kPagedAttentionSoftcapI64,

@@ -21,9 +21,18 @@ inline int32_t ensure_len_at_least(const char* name, size_t actual, size_t minim
     return 0;
 }
 
-// fmha_prefill.cpp: the bf16 / f16 matrix-core prefill with the dense op's sinks and key lengths (either may be null).
+// fmha_prefill.cpp: the bf16 / f16 matrix-core prefill with the options of the dense op.  sinks [heads] and mask are
+// in the element type of the query; any pointer may be null, window negative and softcap 0 when absent.
+struct DenseOptions {
+    const uint16_t* sinks = nullptr;
+    const int32_t* key_lengths = nullptr;
+    const uint16_t* mask = nullptr;
+    uint64_t mask_strides[4] = {0, 0, 0, 0};
+    long long window = -1;
+    float softcap = 0.0f;
+};
 int32_t dense_prefill_with_options(void* stream, bool f16, uint16_t* out, size_t out_len, const uint16_t* query, size_t query_len,
                                    const uint16_t* key, size_t key_len, const uint16_t* value, size_t value_len,
-                                   const SingeFmhaPrefillConfig* config, const uint16_t* sinks, const int32_t* key_lengths);
+                                   const SingeFmhaPrefillConfig* config, const DenseOptions& options);
 
 }  // namespace singe_hip

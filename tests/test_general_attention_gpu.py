@@ -151,6 +151,55 @@ def test_dense_at_128_with_sinks_and_key_lengths_on_the_matrix_core_kernel(dtype
     close(host(both), want, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("options", [dict(window=40), dict(causal=True, window=7), dict(softcap=3.0), dict(softcap=-2.0, causal=True),
+                                     dict(causal=True, window=100, softcap=5.0, scale=-0.05), dict(window=0)])
+def test_dense_at_128_with_window_and_cap_on_the_matrix_core_kernel(dtype, options):
+    batch, heads, kv_heads, query_len, key_len = 2, 4, 2, 200, 333
+    q, k, v = tensors((batch, heads, query_len, 128), (batch, kv_heads, key_len, 128), (batch, kv_heads, key_len, 128), dtype, 19)
+    out = neural.attend(q, k, v, options=neural.AttentionOptions(**options))
+    want = oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), threads=8, **options)
+    close(host(out), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_dense_at_128_with_masks_on_the_matrix_core_kernel(dtype):
+    batch, heads, kv_heads, query_len, key_len = 2, 4, 2, 150, 201
+    q, k, v = tensors((batch, heads, query_len, 128), (batch, kv_heads, key_len, 128), (batch, kv_heads, key_len, 128), dtype, 23)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(3)
+    sinks = torch.randn((heads,), generator=gen, device="cuda").to(dtype)
+    lengths = torch.tensor([170, 500], dtype=torch.int32, device="cuda")
+    # broadcast over batch and heads, with hidden keys and one row hidden but for its last keys
+    mask = torch.randn((query_len, key_len), generator=gen, device="cuda").to(dtype)
+    mask[:, 3] = float("-inf")
+    mask[7, :190] = float("-inf")
+    out = neural.attend(q, k, v, mask, sinks, neural.AttentionOptions(softcap=10.0))
+    want = oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), softcap=10.0, mask=host(mask), sinks=host(sinks), threads=8)
+    close(host(out), want, dtype)
+    # per batch and head, causal and windowed; one row has every key hidden: the CPU form divides zero by zero
+    # there (NaN), the kernel writes zeros like every other row without keys
+    full = torch.randn((batch, heads, query_len, key_len), generator=gen, device="cuda").to(dtype)
+    full[1, 2, 5, :] = float("-inf")
+    out = neural.attend(q, k, v, full, None, neural.AttentionOptions(causal=True, window=64))
+    want = oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), causal=True, window=64, mask=host(full), threads=8)
+    assert np.isnan(want[1, 2, 5]).all() and not host(out)[1, 2, 5].any()
+    want[1, 2, 5] = 0.0
+    close(host(out), want, dtype)
+    # broadcast over queries ([batch, 1, 1, key]) and a Boolean mask over [heads, query, key]
+    padding = torch.zeros((batch, 1, 1, key_len), device="cuda", dtype=dtype)
+    padding[0, ..., 120:] = float("-inf")
+    out = neural.attend(q, k, v, padding)
+    want = oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), mask=host(padding), threads=8)
+    close(host(out), want, dtype)
+    keep = torch.rand((heads, query_len, key_len), generator=gen, device="cuda") > 0.3
+    keep[..., 0] = True
+    out = neural.attend(q, k, v, keep, sinks)
+    want = oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), mask=np.where(keep.cpu().numpy(), 0.0, -np.inf).astype(np.float32),
+                                                   sinks=host(sinks), threads=8)
+    close(host(out), want, dtype)
+
+
 def test_dense_shape_rules():
     q, k, v = tensors((1, 4, 8, 32), (1, 3, 8, 32), (1, 3, 8, 32), torch.float32, 1)
     with pytest.raises(error.InvalidArgument):

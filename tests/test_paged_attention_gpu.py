@@ -69,6 +69,14 @@ def test_ragged_sequences_match_oracle(heads, kv_heads, page_size, options):
     run_case(sequences, heads, kv_heads, page_size, options, seed=heads + page_size)
 
 
+@pytest.mark.parametrize("options", [neural.AttentionOptions(causal=True, softcap=-4.0), neural.AttentionOptions(scale=-0.06, softcap=5.0),
+                                     neural.AttentionOptions(scale=-0.06, softcap=-5.0, causal=True, window=50)])
+@pytest.mark.parametrize("heads,kv_heads,page_size", [(8, 2, 16), (4, 4, 7)])
+def test_negative_caps_and_scales(heads, kv_heads, page_size, options):
+    # cap * tanh(score / cap) does not care about the sign of the cap; a negative scale turns the scores round
+    run_case([(1, 150), (70, 70), (20, 90)], heads, kv_heads, page_size, options, seed=heads)
+
+
 def test_int64_indices_and_chunked_prefill_shape():
     # one sequence of the chunked-prefill shape: 512 new queries over a cached prefix, 64 query / 8 kv heads
     run_case([(512, 1536 + 512), (512, 1024 + 512)], 64, 8, 16, neural.AttentionOptions(causal=True),
