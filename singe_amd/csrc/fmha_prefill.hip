@@ -150,11 +150,20 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     }
     const ReadOffsets offsets = read_offsets(lane);
 
-    if (tiles > 0) {
-        load_keys(0, lds);
-        load_values(0, lds + kValueBase);
+    // The first tile any row of the workgroup can see: 0, or with a window the tile of the first key the
+    // workgroup's first row still sees (later rows see later keys).
+    unsigned int first_tile = 0;
+    if (OPTIONS && a.window >= 0) {
+        const unsigned long long low = static_cast<unsigned long long>(query_tile) * kRows + 1u;
+        const unsigned long long window = static_cast<unsigned long long>(a.window);
+        if (low > window) first_tile = static_cast<unsigned int>((low - window) / kKeyTile);
+        first_tile = first_tile < tiles ? first_tile : tiles;
     }
-    if (tiles > 1) load_keys(1, lds + kTileBytes);
+    if (first_tile < tiles) {
+        load_keys(first_tile, lds);
+        load_values(first_tile, lds + kValueBase);
+    }
+    if (first_tile + 1 < tiles) load_keys(first_tile + 1, lds + kTileBytes);
     loads_landed();
     __syncthreads();
 
@@ -204,7 +213,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     // One block ahead: while block b is folded, the scores of block b + 1 are computed; `scores` holds
     // those of the block that is folded next.
     f32x16_t scores;
-    if (wave_blocks > 0) score_block(half, scores, q, lds, offsets);
+    if (2u * first_tile < wave_blocks) score_block(half, scores, q, lds, offsets);
     unsigned int key_stage = 0, value_stage = 0;  // tile % 3, tile % 2
     // Names the stages a tile's iteration works on and loads into.  Everyone left the stages that held K of
     // tile - 1 and V of tile - 1 at the last barrier.
@@ -239,7 +248,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
         interior_tiles = interior_tiles < whole ? interior_tiles : whole;
     }
     if (OPTIONS) interior_tiles = 0;
-    unsigned int tile = 0;
+    unsigned int tile = first_tile;
     uint4 operand[8];
     if (kDenseOperandsAhead && interior_tiles > 0) read_key_operands(operand, lds + kBlockBytes, offsets);
     auto issue = [&](unsigned char* key_dest, unsigned char* value_dest) __attribute__((always_inline)) {
