@@ -85,3 +85,6 @@ SINGE_DEVICE uint2 stream_load_8(const void* address) {
 
 SINGE_DEVICE float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 SINGE_DEVICE float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+// tanh(x) = 1 - 2 / (e^(2x) + 1): one exponential and one reciprocal; exact at both infinities, absolute error
+// about 1e-7 near zero (the subtraction), which a capped score multiplies by the cap.
+SINGE_DEVICE float fast_tanh(float x) { return 1.0f - 2.0f * __builtin_amdgcn_rcpf(fast_exp2(x * (2.0f * kLog2e)) + 1.0f); }

@@ -182,7 +182,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 float x = s[r] * to_units;
-                if (capped) x = tanhf(x) * a.cap_log2e;
+                if (capped) x = fast_tanh(x) * a.cap_log2e;
                 if (mask_row != nullptr) {
                     const unsigned int key = key0 + 8u * (r >> 2) + 4u * hi + (r & 3);
                     const uint16_t bits = mask_row[static_cast<size_t>(key < key_len ? key : 0) * a.mask_strides[3]];

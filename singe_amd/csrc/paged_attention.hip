@@ -349,7 +349,7 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
             // (singe/src/backend/cuda/kernel_plan/source/tensor_core.rs:49-54).
             const float cap_scale = fabsf(a.softcap_scale);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) s[r] = tanhf(s[r] * cap_scale) * a.softcap_log2e;
+            for (int r = 0; r < 16; ++r) s[r] = fast_tanh(s[r] * cap_scale) * a.softcap_log2e;
         }
         const bool edge = (causal && key0 + 31u > wave_low) || key0 + 32u > keys || windowed;
         const float shift = begin_block(state, s, hi, factor, edge, [&](unsigned int key_in_block) {
