@@ -195,6 +195,10 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
     const bool with_options = options.mask != nullptr || options.window >= 0 || options.softcap != 0.0f;
     args.mask = options.mask;
     for (int i = 0; i < 4; ++i) args.mask_strides[i] = options.mask_strides[i];
+    args.mask_packed = options.mask != nullptr && options.mask_strides[3] == 1 && options.mask_strides[0] % 4 == 0 &&
+                               options.mask_strides[1] % 4 == 0 && options.mask_strides[2] % 4 == 0 &&
+                               (reinterpret_cast<uintptr_t>(options.mask) & 7u) == 0
+                           ? 1u : 0u;
     args.window = options.window;
     if (options.softcap != 0.0f) {
         args.cap_scale = std::fabs(c.scale / options.softcap);

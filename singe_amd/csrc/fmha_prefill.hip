@@ -179,16 +179,34 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
             const uint16_t* mask_row = nullptr;
             if (a.mask != nullptr)
                 mask_row = a.mask + batch * a.mask_strides[0] + head * a.mask_strides[1] + static_cast<size_t>(query_valid ? my_query : 0) * a.mask_strides[2];
+            // The lane's keys come in four runs of four; a run inside the keys is one 8-byte load when the host found
+            // every mask row to start on an 8-byte boundary with its keys side by side.
+            uint16_t mask_bits[16];
+            if (mask_row != nullptr) {
+#pragma unroll
+                for (int run = 0; run < 4; ++run) {
+                    const unsigned int key = key0 + 8u * run + 4u * hi;
+                    if (a.mask_packed && key + 3u < key_len) {
+                        const uint2 four = *reinterpret_cast<const uint2*>(mask_row + key);
+                        mask_bits[4 * run + 0] = static_cast<uint16_t>(four.x);
+                        mask_bits[4 * run + 1] = static_cast<uint16_t>(four.x >> 16);
+                        mask_bits[4 * run + 2] = static_cast<uint16_t>(four.y);
+                        mask_bits[4 * run + 3] = static_cast<uint16_t>(four.y >> 16);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            mask_bits[4 * run + i] = mask_row[static_cast<size_t>(key + i < key_len ? key + i : 0) * a.mask_strides[3]];
+                    }
+                }
+            }
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 float x = s[r] * to_units;
                 if (capped) x = fast_tanh(x) * a.cap_log2e;
                 if (mask_row != nullptr) {
-                    const unsigned int key = key0 + 8u * (r >> 2) + 4u * hi + (r & 3);
-                    const uint16_t bits = mask_row[static_cast<size_t>(key < key_len ? key : 0) * a.mask_strides[3]];
                     float extra;
-                    if constexpr (std::is_same_v<Half, F16>) extra = static_cast<float>(__builtin_bit_cast(_Float16, bits));
-                    else extra = __builtin_bit_cast(float, static_cast<unsigned int>(bits) << 16);
+                    if constexpr (std::is_same_v<Half, F16>) extra = static_cast<float>(__builtin_bit_cast(_Float16, mask_bits[r]));
+                    else extra = __builtin_bit_cast(float, static_cast<unsigned int>(mask_bits[r]) << 16);
                     x += extra * kLog2e;
                 }
                 s[r] = x;

@@ -77,6 +77,7 @@ struct PrefillArgs {
     // (cap_scale = |scale / cap|, cap_log2e = |cap| * log2(e); both 0 when absent).
     const uint16_t* mask = nullptr;
     uint64_t mask_strides[4] = {0, 0, 0, 0};
+    uint32_t mask_packed = 0;  // key stride 1, the other strides multiples of 4, the mask on an 8-byte boundary
     long long window = -1;
     float cap_scale = 0.0f, cap_log2e = 0.0f;
 };
