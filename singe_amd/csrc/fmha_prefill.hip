@@ -265,7 +265,10 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
         const unsigned int whole = key_len / kKeyTile;  // tiles t with 64 t + 64 <= key_len
         interior_tiles = interior_tiles < whole ? interior_tiles : whole;
     }
-    if (OPTIONS) interior_tiles = 0;
+    // With options, only a cap alone leaves the unmasked tiles their straight-line path (the cap is applied to each
+    // block's scores before they are folded); a mask or a window send every tile down the masked one.
+    const bool cap_only = OPTIONS && a.mask == nullptr && a.window < 0 && a.cap_log2e != 0.0f;
+    if (OPTIONS && !cap_only) interior_tiles = 0;
     unsigned int tile = first_tile;
     uint4 operand[8];
     if (kDenseOperandsAhead && interior_tiles > 0) read_key_operands(operand, lds + kBlockBytes, offsets);
@@ -273,6 +276,18 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
         if (tile + 2 < tiles) load_keys(tile + 2, key_dest);
         if (tile + 1 < tiles) load_values(tile + 1, value_dest);
     };
+    if constexpr (OPTIONS) {
+        const float cap_scale = a.cap_scale, cap_log2e = a.cap_log2e;
+        for (; tile < interior_tiles; ++tile) {
+            const TileStages stages = enter();
+            fold_interior_tile<kDenseOperandsAhead>(half, state, scores, operand, q, offsets, hi, 1.0f, stages.keys, stages.next_keys, stages.values,
+                                                    stages.key_dest, stages.value_dest, issue, [&](f32x16_t& s) {
+#pragma unroll
+                                                        for (int r = 0; r < 16; ++r) s[r] = fast_tanh(s[r] * cap_scale) * cap_log2e;
+                                                    });
+            leave();
+        }
+    }
     for (; tile < interior_tiles; ++tile) {
         const TileStages stages = enter();
         fold_interior_tile<kDenseOperandsAhead>(half, state, scores, operand, q, offsets, hi, factor, stages.keys, stages.next_keys, stages.values, stages.key_dest,

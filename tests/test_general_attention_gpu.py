@@ -162,6 +162,30 @@ def test_dense_at_128_with_window_and_cap_on_the_matrix_core_kernel(dtype, optio
     close(host(out), want, dtype)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_dense_at_128_cap_alone_with_sinks_and_key_lengths(causal):
+    """A cap without mask or window keeps the straight-line tiles of the matrix-core kernel; sinks and
+    per-batch key lengths ride along."""
+    batch, heads, kv_heads, query_len, key_len = 2, 4, 2, 520, 700
+    dtype = torch.bfloat16
+    q, k, v = tensors((batch, heads, query_len, 128), (batch, kv_heads, key_len, 128), (batch, kv_heads, key_len, 128), dtype, 29)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(5)
+    sinks = torch.randn((heads,), generator=gen, device="cuda").to(dtype)
+    lengths = torch.tensor([333, 700], dtype=torch.int32, device="cuda")
+    import ctypes
+    from singe_amd import _native
+    problem = _native.AttentionProblemC(batch, heads, kv_heads, query_len, key_len, 128, 128, (ctypes.c_int64 * 4)(0, 0, 0, 0), 1,
+                                        int(causal), 0, 0, 1, 0.0, 4.0, 0)
+    out = torch.empty_like(q)
+    status = _native.lib().singe_hip_scaled_dot_product_attention(None, q.data_ptr(), k.data_ptr(), v.data_ptr(), None, sinks.data_ptr(),
+                                                                  lengths.data_ptr(), out.data_ptr(), ctypes.byref(problem))
+    assert status == 0
+    want = oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), causal=causal, softcap=4.0, sinks=host(sinks),
+                                                   key_lengths=[333, 700], threads=8)
+    close(host(out), want, dtype)
+
+
 @pytest.mark.parametrize("key_len", [201, 204])  # mask rows off and on an 8-byte boundary (the packed loads)
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_dense_at_128_with_masks_on_the_matrix_core_kernel(dtype, key_len):
