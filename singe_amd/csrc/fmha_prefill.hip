@@ -265,27 +265,49 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
         const unsigned int whole = key_len / kKeyTile;  // tiles t with 64 t + 64 <= key_len
         interior_tiles = interior_tiles < whole ? interior_tiles : whole;
     }
-    // With options, only a cap alone leaves the unmasked tiles their straight-line path (the cap is applied to each
-    // block's scores before they are folded); a mask or a window send every tile down the masked one.
-    const bool cap_only = OPTIONS && a.mask == nullptr && a.window < 0 && a.cap_log2e != 0.0f;
-    if (OPTIONS && !cap_only) interior_tiles = 0;
+    // With options, a cap and a window leave the unmasked tiles their straight-line path (the cap is applied to each
+    // block's scores before they are folded; the tiles that reach back past the window of the wave's last row come
+    // first and take the masked path); an additive mask sends every tile down the masked one.
+    unsigned int inner_begin = first_tile;
+    if (OPTIONS) {
+        if (a.mask != nullptr) interior_tiles = 0;
+        if (a.window >= 0) {
+            // Tile t lies inside every row's window when 64 t + window > first_row + 31.
+            const unsigned long long past = static_cast<unsigned long long>(first_row) + 32u, window = static_cast<unsigned long long>(a.window);
+            if (past > window) {
+                const unsigned long long whole = (past - window + kKeyTile - 1) / kKeyTile;
+                inner_begin = whole < tiles ? static_cast<unsigned int>(whole) : tiles;
+            }
+            inner_begin = inner_begin > first_tile ? inner_begin : first_tile;
+        }
+    }
     unsigned int tile = first_tile;
     uint4 operand[8];
-    if (kDenseOperandsAhead && interior_tiles > 0) read_key_operands(operand, lds + kBlockBytes, offsets);
     auto issue = [&](unsigned char* key_dest, unsigned char* value_dest) __attribute__((always_inline)) {
         if (tile + 2 < tiles) load_keys(tile + 2, key_dest);
         if (tile + 1 < tiles) load_values(tile + 1, value_dest);
     };
     if constexpr (OPTIONS) {
-        const float cap_scale = a.cap_scale, cap_log2e = a.cap_log2e;
-        for (; tile < interior_tiles; ++tile) {
+        for (; tile < inner_begin && tile < interior_tiles; ++tile) {
             const TileStages stages = enter();
-            fold_interior_tile<kDenseOperandsAhead>(half, state, scores, operand, q, offsets, hi, 1.0f, stages.keys, stages.next_keys, stages.values,
-                                                    stages.key_dest, stages.value_dest, issue, [&](f32x16_t& s) {
-#pragma unroll
-                                                        for (int r = 0; r < 16; ++r) s[r] = fast_tanh(s[r] * cap_scale) * cap_log2e;
-                                                    });
+            fold_edge_tile(half, scores, q, offsets, 2u * tile, wave_blocks, stages.keys, stages.next_keys, stages.values, stages.key_dest,
+                           stages.value_dest, issue, fold);
             leave();
+        }
+    }
+    if (kDenseOperandsAhead && tile < interior_tiles) read_key_operands(operand, lds + key_stage * kTileBytes + kBlockBytes, offsets);
+    if constexpr (OPTIONS) {
+        if (a.cap_log2e != 0.0f) {
+            const float cap_scale = a.cap_scale, cap_log2e = a.cap_log2e;
+            for (; tile < interior_tiles; ++tile) {
+                const TileStages stages = enter();
+                fold_interior_tile<kDenseOperandsAhead>(half, state, scores, operand, q, offsets, hi, 1.0f, stages.keys, stages.next_keys, stages.values,
+                                                        stages.key_dest, stages.value_dest, issue, [&](f32x16_t& s) {
+#pragma unroll
+                                                            for (int r = 0; r < 16; ++r) s[r] = fast_tanh(s[r] * cap_scale) * cap_log2e;
+                                                        });
+                leave();
+            }
         }
     }
     for (; tile < interior_tiles; ++tile) {

@@ -162,6 +162,19 @@ def test_dense_at_128_with_window_and_cap_on_the_matrix_core_kernel(dtype, optio
     close(host(out), want, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("options", [dict(causal=True, window=300), dict(causal=True, window=129, softcap=6.0), dict(window=200),
+                                     dict(causal=True, window=64), dict(causal=True, window=1000)])
+def test_dense_at_128_long_windows(dtype, options):
+    """Rows long enough that a wave meets all three kinds of tile: reaching back past the window, wholly
+    inside it, and on the causal edge."""
+    batch, heads, kv_heads, query_len, key_len = 1, 4, 2, 900, 900
+    q, k, v = tensors((batch, heads, query_len, 128), (batch, kv_heads, key_len, 128), (batch, kv_heads, key_len, 128), dtype, 31)
+    out = neural.attend(q, k, v, options=neural.AttentionOptions(**options))
+    want = oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), threads=8, **options)
+    close(host(out), want, dtype)
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_dense_at_128_cap_alone_with_sinks_and_key_lengths(causal):
     """A cap without mask or window keeps the straight-line tiles of the matrix-core kernel; sinks and
