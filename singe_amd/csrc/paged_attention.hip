@@ -394,23 +394,45 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         __syncthreads();
     };
 
-    // Tiles no mask touches for this wave, with another block to come after them: straight-line code.
-    unsigned int interior_end = first_tile;
-    if (!SOFTCAP && !windowed) {
-        interior_end = wave_blocks > 2 ? (wave_blocks - 1) / 2 : 0;  // tiles t with 2 t + 2 < wave_blocks
-        if (causal) {
-            const unsigned int unmasked = (wave_low + 1) / kKeyTile;  // tiles t with 64 t + 63 <= wave_low
-            interior_end = interior_end < unmasked ? interior_end : unmasked;
-        }
+    // Tiles no mask touches for this wave, with another block to come after them: straight-line code.  With a
+    // window, the tiles that reach back past the window of the wave's last row come before them and take the
+    // masked path; a cap is applied to each block's scores before they are folded.
+    unsigned int interior_end = wave_blocks > 2 ? (wave_blocks - 1) / 2 : 0;  // tiles t with 2 t + 2 < wave_blocks
+    if (causal) {
+        const unsigned int unmasked = (wave_low + 1) / kKeyTile;  // tiles t with 64 t + 63 <= wave_low
+        interior_end = interior_end < unmasked ? interior_end : unmasked;
+    }
+    {
         const unsigned int whole = keys / kKeyTile;  // tiles t with 64 t + 64 <= keys
         interior_end = interior_end < whole ? interior_end : whole;
     }
+    unsigned int interior_begin = first_tile;
+    if (windowed && wave_high + 1u > window) {
+        // Tile t lies inside every row's window when 64 t + window > wave_high.
+        const unsigned int inside = (wave_high + 1u - window + kKeyTile - 1) / kKeyTile;
+        interior_begin = inside > first_tile ? inside : first_tile;
+    }
     uint4 operand[8];
-    if (kPagedOperandsAhead && tile < interior_end) read_key_operands(operand, lds + kBlockBytes, offsets);
+    for (; tile < interior_begin && tile < interior_end; ++tile) {
+        const TileStages stages = enter();
+        fold_edge_tile(half, scores, q, offsets, 2u * tile, wave_blocks, stages.keys, stages.next_keys, stages.values, stages.key_dest,
+                       stages.value_dest, issue, fold);
+        leave();
+    }
+    if (kPagedOperandsAhead && tile < interior_end) read_key_operands(operand, lds + key_stage * kTileBytes + kBlockBytes, offsets);
     for (; tile < interior_end; ++tile) {
         const TileStages stages = enter();
-        fold_interior_tile<kPagedOperandsAhead>(half, state, scores, operand, q, offsets, hi, factor, stages.keys, stages.next_keys, stages.values, stages.key_dest,
-                           stages.value_dest, issue);
+        if constexpr (SOFTCAP) {
+            const float cap_scale = fabsf(a.softcap_scale), cap_log2e = a.softcap_log2e;
+            fold_interior_tile<kPagedOperandsAhead>(half, state, scores, operand, q, offsets, hi, factor, stages.keys, stages.next_keys, stages.values,
+                                                    stages.key_dest, stages.value_dest, issue, [&](f32x16_t& s) {
+#pragma unroll
+                                                        for (int r = 0; r < 16; ++r) s[r] = fast_tanh(s[r] * cap_scale) * cap_log2e;
+                                                    });
+        } else {
+            fold_interior_tile<kPagedOperandsAhead>(half, state, scores, operand, q, offsets, hi, factor, stages.keys, stages.next_keys, stages.values,
+                                                    stages.key_dest, stages.value_dest, issue);
+        }
         leave();
     }
     // Tiles on a mask's edge and the last ones (and, for waves that have run out of blocks, the workgroup's

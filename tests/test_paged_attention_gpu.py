@@ -77,6 +77,16 @@ def test_negative_caps_and_scales(heads, kv_heads, page_size, options):
     run_case([(1, 150), (70, 70), (20, 90)], heads, kv_heads, page_size, options, seed=heads)
 
 
+@pytest.mark.parametrize("options", [neural.AttentionOptions(causal=True, window=300), neural.AttentionOptions(causal=True, window=200, softcap=8.0),
+                                     neural.AttentionOptions(causal=True, window=64), neural.AttentionOptions(causal=True, softcap=6.0),
+                                     neural.AttentionOptions(window=500), neural.AttentionOptions(softcap=3.0, scale=-0.05)])
+@pytest.mark.parametrize("heads,kv_heads,page_size", [(8, 2, 16), (4, 4, 16), (16, 1, 5)])
+def test_long_windows_and_caps(heads, kv_heads, page_size, options):
+    """Sequences long enough that a wave meets tiles reaching back past the window, tiles wholly inside it (which,
+    like the capped ones, take the straight-line path) and tiles on the causal edge."""
+    run_case([(300, 1100), (700, 700), (1, 1300), (40, 64)], heads, kv_heads, page_size, options, seed=heads + 3)
+
+
 def test_int64_indices_and_chunked_prefill_shape():
     # one sequence of the chunked-prefill shape: 512 new queries over a cached prefix, 64 query / 8 kv heads
     run_case([(512, 1536 + 512), (512, 1024 + 512)], 64, 8, 16, neural.AttentionOptions(causal=True),
