@@ -267,7 +267,8 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     }
     // With options, a cap and a window leave the unmasked tiles their straight-line path (the cap is applied to each
     // block's scores before they are folded; the tiles that reach back past the window of the wave's last row come
-    // first and take the masked path); an additive mask sends every tile down the masked one.
+    // first and take the masked path); an additive mask sends every tile down the masked one (its words held a tile
+    // ahead in registers made the straight-line tiles spill, and the reloads wait for the K and V loads in flight).
     unsigned int inner_begin = first_tile;
     if (OPTIONS) {
         if (a.mask != nullptr) interior_tiles = 0;
@@ -302,7 +303,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
             for (; tile < interior_tiles; ++tile) {
                 const TileStages stages = enter();
                 fold_interior_tile<kDenseOperandsAhead>(half, state, scores, operand, q, offsets, hi, 1.0f, stages.keys, stages.next_keys, stages.values,
-                                                        stages.key_dest, stages.value_dest, issue, [&](f32x16_t& s) {
+                                                        stages.key_dest, stages.value_dest, issue, [&](f32x16_t& s, unsigned int) {
 #pragma unroll
                                                             for (int r = 0; r < 16; ++r) s[r] = fast_tanh(s[r] * cap_scale) * cap_log2e;
                                                         });

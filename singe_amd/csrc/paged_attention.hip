@@ -425,7 +425,7 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         if constexpr (SOFTCAP) {
             const float cap_scale = fabsf(a.softcap_scale), cap_log2e = a.softcap_log2e;
             fold_interior_tile<kPagedOperandsAhead>(half, state, scores, operand, q, offsets, hi, factor, stages.keys, stages.next_keys, stages.values,
-                                                    stages.key_dest, stages.value_dest, issue, [&](f32x16_t& s) {
+                                                    stages.key_dest, stages.value_dest, issue, [&](f32x16_t& s, unsigned int) {
 #pragma unroll
                                                         for (int r = 0; r < 16; ++r) s[r] = fast_tanh(s[r] * cap_scale) * cap_log2e;
                                                     });

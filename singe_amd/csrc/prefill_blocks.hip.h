@@ -188,8 +188,9 @@ SINGE_DEVICE void loads_landed() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmc
 // iteration's loads, then both blocks are folded while the scores of the block after each are computed.
 // With AHEAD the K operands of those products are read a block early and carried in `operand`: those of the
 // tile's second block on entry (read_key_operands before the first tile), of the next tile's on return.
-//   shape(scores)   turns a block's raw scores into what the softmax takes (a score cap) before they are folded;
-//                   the caller then passes the factor that is left to apply (1 when shape did the scaling).
+//   shape(scores, which)   turns the raw scores of the tile's first (which = 0) or second block into what the softmax
+//                          takes (a score cap, an added mask) before they are folded; the caller then passes the
+//                          factor that is left to apply (1 when shape did the scaling).
 template <bool AHEAD, class Half, class Issue, class Shape>
 SINGE_DEVICE void fold_interior_tile(Half half, RowState& state, f32x16_t& scores, uint4 (&operand)[8], const uint4 (&q)[8],
                                      const ReadOffsets& offsets, unsigned int hi, float factor, const unsigned char* __restrict__ keys,
@@ -197,11 +198,11 @@ SINGE_DEVICE void fold_interior_tile(Half half, RowState& state, f32x16_t& score
                                      unsigned char* __restrict__ key_dest, unsigned char* __restrict__ value_dest, Issue&& issue,
                                      Shape&& shape) {
     issue(key_dest, value_dest);
-    shape(scores);
+    shape(scores, 0u);
     const float shift_even = begin_block(state, scores, hi, factor, false, [](unsigned int) { return false; });
     finish_block<true, AHEAD>(half, state, scores, factor, shift_even, values, offsets, scores, q, keys + kBlockBytes, operand, next_keys);
     __builtin_amdgcn_sched_barrier(0);  // keeps the second block's operand reads out of the first block's registers
-    shape(scores);
+    shape(scores, 1u);
     const float shift_odd = begin_block(state, scores, hi, factor, false, [](unsigned int) { return false; });
     finish_block<true, AHEAD>(half, state, scores, factor, shift_odd, values + kBlockBytes, offsets, scores, q, next_keys, operand,
                               next_keys + kBlockBytes);
@@ -213,7 +214,7 @@ SINGE_DEVICE void fold_interior_tile(Half half, RowState& state, f32x16_t& score
                                      const unsigned char* __restrict__ next_keys, const unsigned char* __restrict__ values,
                                      unsigned char* __restrict__ key_dest, unsigned char* __restrict__ value_dest, Issue&& issue) {
     fold_interior_tile<AHEAD>(half, state, scores, operand, q, offsets, hi, factor, keys, next_keys, values, key_dest, value_dest, issue,
-                              [](f32x16_t&) {});
+                              [](f32x16_t&, unsigned int) {});
 }
 
 // The K operands of the block at `keys`.
