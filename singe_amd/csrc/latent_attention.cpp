@@ -61,7 +61,11 @@ extern "C" int32_t singe_hip_paged_mla_attention(void* stream, const void* laten
     args.sequences = static_cast<uint32_t>(p.sequences);
     args.cache_pages = static_cast<uint32_t>(p.cache_pages);
     args.page_table = static_cast<uint32_t>(p.page_table);
-    const uint64_t row_blocks = (static_cast<uint64_t>(p.tokens) * p.heads + 3) / 4;
+    // Latent width 512 with positional width 64 in a 16-bit type runs on the matrix cores, 128 (token, head) rows of
+    // a sequence to a workgroup; every other shape on the vector unit, 4 rows to a workgroup.
+    const bool tiles = p.data_type != SINGE_HIP_F32 && p.latent_dim == 512 && p.position_dim == 64;
+    const uint64_t rows_per_block = tiles ? 128 : 4;
+    const uint64_t row_blocks = (static_cast<uint64_t>(p.tokens) * p.heads + rows_per_block - 1) / rows_per_block;
     args.row_blocks = static_cast<uint32_t>(row_blocks);
     args.causal = p.causal ? 1u : 0u;
     args.wide_index = p.index_type == SINGE_HIP_INDEX_I64 ? 1u : 0u;
@@ -69,6 +73,8 @@ extern "C" int32_t singe_hip_paged_mla_attention(void* stream, const void* laten
     args.scale = p.has_scale ? p.scale : static_cast<float>(1.0 / std::sqrt(static_cast<double>(p.latent_dim + p.position_dim)));
     const uint64_t blocks = row_blocks * static_cast<uint64_t>(p.sequences);
     if (blocks > 0x7fffffffull || row_blocks > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
+    if (tiles)
+        return launch(p.data_type == SINGE_HIP_BF16 ? kLatentTilesBf16 : kLatentTilesF16, static_cast<unsigned>(blocks), 1, 1, 512, stream, args);
     const int kernel = kLatentGeneral + (p.data_type == SINGE_HIP_F32 ? 0 : p.data_type == SINGE_HIP_BF16 ? 1 : 2);
     return launch(static_cast<KernelId>(kernel), static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
 }

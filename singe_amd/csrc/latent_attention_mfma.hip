@@ -1,0 +1,362 @@
+// Latent attention over paged caches on the matrix cores: bf16 or f16, latent width 512, positional width 64
+// (DeepSeek's absorbed MLA).  The same op as latent_attention.hip (CPU: singe/src/backend/cpu/normalization/
+// attention.rs:540-679; kernel plan: singe/src/backend/cuda/kernel_plan/source/mla.rs), for the one shape that
+// matters in practice; every other shape stays on the vector-unit kernel.
+//
+// Every head of a token attends over the same cache rows, so the rows of a sequence, (query, head) pairs in
+// query-major order, are tiled 128 to a workgroup and the cache is read once per tile of rows instead of once
+// per head.  A workgroup is eight waves; wave w owns rows 16 w .. 16 w + 15 of the tile for the whole of the
+// keys.  Keys come in tiles of 32, straight from global memory into LDS (global_load_lds_dwordx4), one tile
+// ahead of the one being worked on; all eight waves read every tile.
+//
+//   S^T[key, row] = C[key, :] . Q[row, :]   v_mfma_f32_16x16x32: A = cache rows from LDS (ds_read_b128),
+//                                           B = the wave's Q^T, 18 steps of 32 dims (16 latent, 2 positional)
+//                                           held in registers; two products of 16 keys each.
+//   O^T[dim, row] += C^T[dim, key] . P^T    A = the latent part of the same LDS rows, transposed on the way
+//                                           out by ds_read_b64_tr_b16; B = the weights, packed from the score
+//                                           registers with no lane traffic: lane (row, g) holds keys
+//                                           4 g .. 4 g + 3 of either 16-key half, which is what the A operand's
+//                                           lane group g is made to read.  32 products of 16 dims.
+//
+// LDS rows are unpadded (the direct loads write 1 KiB runs); bank conflicts are kept down by permuting the 16-byte
+// chunks of a row, on the global side of the load and again in the read offsets: latent chunk c of key k sits at
+// c ^ f(k), f(k) = ((k & 7) << 1) | ((k >> 3) & 1), which spreads the 16 keys of a score operand over all banks
+// and the 8 keys of half a transposed read too; positional chunk c (of 8) sits at c ^ (k & 7).
+#include "common.hip.h"
+#include "kernel_args.h"
+#include "paging.hip.h"
+#include "prefill_core.hip.h"
+
+namespace latent_mfma {
+
+using prefill::Bf16;
+using prefill::F16;
+using prefill::kMaxLag;
+using prefill::pack_pair;
+using prefill::v4i16_t;
+
+constexpr int kLatent = 512, kPositional = 64;
+constexpr int kWaves = 8, kRows = 16 * kWaves;  // rows of a workgroup
+constexpr int kKeys = 32;                      // keys per tile
+constexpr int kLatentRowBytes = kLatent * 2, kPositionalRowBytes = kPositional * 2;
+constexpr int kLatentTileBytes = kKeys * kLatentRowBytes;          // 32 KiB
+constexpr int kPositionalTileBytes = kKeys * kPositionalRowBytes;  // 4 KiB
+constexpr int kStageBytes = kLatentTileBytes + kPositionalTileBytes;
+// The first steps of Q^T live in LDS, one 16-byte slot per (step, lane) that only its own lane touches, to leave the
+// wave registers for the operands in flight.
+constexpr int kParkedSteps = 10;
+constexpr int kParkedBytes = kParkedSteps * 1024 * kWaves;
+constexpr int kLdsBytes = 2 * kStageBytes + kParkedBytes;
+constexpr int kLatentSteps = kLatent / 32, kSteps = (kLatent + kPositional) / 32;
+constexpr int kDimBlocks = kLatent / 16;
+
+typedef unsigned int __attribute__((address_space(3))) * lds_words_t;
+typedef v4i16_t __attribute__((address_space(3))) * lds_v4_t;
+
+SINGE_DEVICE f32x4_t mma(Bf16, uint4 a, uint4 b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+SINGE_DEVICE f32x4_t mma(F16, uint4 a, uint4 b, f32x4_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(prefill::f16x8v_t, a), __builtin_bit_cast(prefill::f16x8v_t, b), c, 0, 0, 0);
+}
+
+// One direct-to-LDS load: every active lane's 16 bytes at `source` go to the wave's `dest` + 16 * lane.  Written as
+// text so that the compiler keeps counting its own LDS reads and loads as usual (it makes every LDS read after the
+// built-in form wait for all of them, and the first one for the load itself); the kernel waits for these loads with
+// vmcnt(0) before the barrier that hands a stage on.
+SINGE_DEVICE void load_to_lds(const unsigned char* source, unsigned char* dest) {
+    const unsigned int base = __builtin_amdgcn_readfirstlane(static_cast<unsigned int>(reinterpret_cast<__UINTPTR_TYPE__>((lds_words_t)dest)));
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(source) : "memory");
+}
+
+// Where the chunk permutation of a latent row puts things: see the header comment.
+SINGE_DEVICE unsigned int chunk_flip(unsigned int key) { return ((key & 7u) << 1) | ((key >> 3) & 1u); }
+
+// What a wave needs to know of the keys it loads for one tile: its four latent rows (wave-uniform) and, for waves
+// 0-3, each lane's positional row.
+template <int FORM>
+struct TilePages {
+    RawPage<FORM> latent[4];
+    RawPage<FORM> positional;
+};
+
+template <class Half, int FORM>
+SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* lds) {
+    const unsigned int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
+    const unsigned int column = lane & 15u, g = lane >> 4;  // row of the wave, lane group
+    // Row tiles are the slow index of the grid: the first tiles of all sequences, the ones a decode step has, are
+    // neighbours and spread over the chip.
+    const unsigned int sequence = blockIdx.x % a.sequences, row_tile = blockIdx.x / a.sequences;
+    const SequenceSpan span = load_span<FORM>(sequence, a.query_offsets, a.page_offsets, a.last_page_lengths, nullptr, a.tokens,
+                                              a.page_table, a.page_size);
+    if (!span.valid) {
+        if (threadIdx.x == 0) report_index_error(a.status);
+        return;
+    }
+    const unsigned long long rows = static_cast<unsigned long long>(span.queries) * a.heads;
+    const unsigned long long first_row = static_cast<unsigned long long>(row_tile) * kRows;
+    if (first_row >= rows) return;
+    const unsigned int keys = span.keys;
+
+    // Queries are the sequence's last tokens, with the CPU path's saturating position (attention.rs:619-627).
+    auto position_of = [&](unsigned long long row) __attribute__((always_inline)) {
+        const long long raw = static_cast<long long>(keys) - static_cast<long long>(span.queries) + static_cast<long long>(row / a.heads);
+        return raw < 0 ? 0u : static_cast<unsigned int>(raw);
+    };
+    const unsigned long long my_row = first_row + 16u * wave + column;
+    const bool row_valid = my_row < rows;
+    const unsigned long long safe_row = row_valid ? my_row : first_row;
+    const size_t flat = (static_cast<size_t>(span.query_start) + safe_row / a.heads) * a.heads + safe_row % a.heads;
+    const unsigned int my_position = position_of(safe_row);
+    const bool causal = a.causal != 0;
+
+    // Keys the workgroup visits, and how far this wave's rows see.
+    const unsigned long long group_last = first_row + kRows - 1 < rows ? first_row + kRows - 1 : rows - 1;
+    unsigned int key_end = keys;
+    if (causal) {
+        const unsigned int reach = position_of(group_last) + 1u;
+        key_end = key_end < reach ? key_end : reach;
+    }
+    const unsigned int tiles = (key_end + kKeys - 1) / kKeys;
+    const unsigned long long wave_first = first_row + 16u * wave;
+    const bool wave_live = wave_first < rows;
+    const unsigned long long wave_last = wave_first + 15u < rows ? wave_first + 15u : rows - 1;
+    unsigned int wave_end = 0;  // keys before this take part for some row of the wave
+    if (wave_live) {
+        wave_end = keys;
+        if (causal) {
+            const unsigned int reach = position_of(wave_last) + 1u;
+            wave_end = wave_end < reach ? wave_end : reach;
+        }
+    }
+    wave_end = __builtin_amdgcn_readfirstlane(wave_end);
+    const unsigned int wave_low = __builtin_amdgcn_readfirstlane(wave_live ? position_of(wave_first) : 0u);
+
+    // Q^T: lane (row, g) holds dims 32 s + 8 g .. + 8 of its row for every step s.
+    const Half half{};
+    uint4 q[kSteps - kParkedSteps];  // steps kParkedSteps and up
+    unsigned char* parked = lds + 2 * kStageBytes + wave * (kParkedSteps * 1024) + 16u * lane;
+    {
+        const unsigned char* latent_row = static_cast<const unsigned char*>(a.latent_queries) + flat * kLatentRowBytes + 16u * g;
+        const unsigned char* positional_row = static_cast<const unsigned char*>(a.positional_queries) + flat * kPositionalRowBytes + 16u * g;
+#pragma unroll
+        for (int s = 0; s < kSteps; ++s) {
+            uint4 bits = s < kLatentSteps ? *reinterpret_cast<const uint4*>(latent_row + 64 * s)
+                                          : *reinterpret_cast<const uint4*>(positional_row + 64 * (s - kLatentSteps));
+            if (!row_valid) bits = make_uint4(0, 0, 0, 0);
+            if (s < kParkedSteps)
+                *reinterpret_cast<uint4*>(parked + 1024 * s) = bits;
+            else
+                q[s - kParkedSteps] = bits;
+        }
+    }
+
+    // Loading a tile: wave w brings latent rows w, w + 8, w + 16, w + 24 (one 1 KiB instruction each) and, for
+    // w < 4, the positional parts of rows 8 w .. 8 w + 7 (lane l: row 8 w + l / 8, chunk position l % 8).
+    const unsigned char* latent_cache = static_cast<const unsigned char*>(a.latent_cache);
+    const unsigned char* positional_cache = static_cast<const unsigned char*>(a.positional_cache);
+    const unsigned int positional_row = 8u * wave + (lane >> 3);
+    auto key_of = [&](unsigned int tile, unsigned int row) __attribute__((always_inline)) {
+        const unsigned int key = tile * kKeys + row;
+        return key < keys ? key : keys - 1u;  // rows past the end re-read the last key and are masked
+    };
+    auto lookup = [&](unsigned int tile) __attribute__((always_inline)) {
+        TilePages<FORM> pages;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            pages.latent[i] = read_raw_page_uniform<FORM>(a.pages, static_cast<size_t>(span.page_start) + key_of(tile, wave + 8u * i) / a.page_size);
+        pages.positional = 0;
+        if (wave < 4) pages.positional = read_raw_page<FORM>(a.pages, static_cast<size_t>(span.page_start) + key_of(tile, positional_row) / a.page_size);
+        return pages;
+    };
+    // A key behind a bad page id is read as zeros; the status word tells the caller.
+    auto issue = [&](unsigned int tile, const TilePages<FORM>& pages, unsigned char* __restrict__ stage) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const unsigned int row = wave + 8u * i;
+            const unsigned long long page = static_cast<unsigned long long>(pages.latent[i]);
+            unsigned char* dest = stage + row * kLatentRowBytes;
+            if (page < static_cast<unsigned long long>(a.cache_pages)) {
+                const size_t slot = static_cast<size_t>(page) * a.page_size + key_of(tile, row) % a.page_size;
+                const unsigned char* source = latent_cache + slot * kLatentRowBytes + 16u * (lane ^ chunk_flip(row & 15u));
+                load_to_lds(source, dest);
+            } else {
+                if (lane == 0) report_index_error(a.status);
+                *reinterpret_cast<uint4*>(dest + 16u * lane) = make_uint4(0, 0, 0, 0);
+            }
+        }
+        if (wave < 4) {
+            const unsigned long long page = static_cast<unsigned long long>(pages.positional);
+            unsigned char* dest = stage + kLatentTileBytes + 8u * wave * kPositionalRowBytes;
+            if (page < static_cast<unsigned long long>(a.cache_pages)) {
+                const size_t slot = static_cast<size_t>(page) * a.page_size + key_of(tile, positional_row) % a.page_size;
+                const unsigned char* source = positional_cache + slot * kPositionalRowBytes + 16u * ((lane & 7u) ^ (positional_row & 7u));
+                load_to_lds(source, dest);
+            } else {
+                report_index_error(a.status);
+                *reinterpret_cast<uint4*>(dest + 16u * lane) = make_uint4(0, 0, 0, 0);
+            }
+        }
+    };
+
+    // Read offsets.  Score operand of step s, 16-key half t: row 16 t + column, chunk (4 s + g) ^ flip.  Transposed
+    // operand of dim block db: rows 4 g + column / 4 (and 16 more), chunk (2 db + (column & 3) / 2) ^ flip, the
+    // low or high 8 bytes of it by column & 1.  A flip touches the low four bits of a chunk index only, so the
+    // offsets repeat every 256 bytes of a row: four registers serve the score operands, eight the transposed ones,
+    // and the rest of an address is an immediate.
+    unsigned int score_at[4], positional_at[2], value_at[8];
+    {
+        const unsigned int score_row = column * kLatentRowBytes, score_flip = chunk_flip(column);
+#pragma unroll
+        for (unsigned int i = 0; i < 4; ++i) score_at[i] = score_row + 16u * ((4u * i + g) ^ score_flip);
+        const unsigned int positional_row_at = kLatentTileBytes + column * kPositionalRowBytes, positional_flip = column & 7u;
+#pragma unroll
+        for (unsigned int i = 0; i < 2; ++i) positional_at[i] = positional_row_at + 16u * ((4u * i + g) ^ positional_flip);
+        const unsigned int value_key = 4u * g + (column >> 2);
+        const unsigned int value_row = value_key * kLatentRowBytes + 8u * (column & 1u);
+        const unsigned int value_flip = chunk_flip(value_key), value_chunk = (column & 3u) >> 1;
+#pragma unroll
+        for (unsigned int i = 0; i < 8; ++i) value_at[i] = value_row + 16u * ((2u * i + value_chunk) ^ value_flip);
+    }
+
+    f32x4_t out[kDimBlocks];  // lane (row, g): dims 16 db + 4 g + r of its row
+#pragma unroll
+    for (int db = 0; db < kDimBlocks; ++db) out[db] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
+    float reference = -INFINITY, running_sum = 0.0f;  // the sum of this lane's keys only
+    const float scale_log2e = a.scale * kLog2e;
+
+    auto fold = [&](unsigned int tile, const unsigned char* __restrict__ stage) __attribute__((always_inline)) {
+        const unsigned int key0 = tile * kKeys;
+        f32x4_t s[2] = {f32x4_t{0.0f, 0.0f, 0.0f, 0.0f}, f32x4_t{0.0f, 0.0f, 0.0f, 0.0f}};
+        // The operands of a step are read a step before its products (two sets taking turns), and the order is
+        // pinned: left to itself the compiler, short of registers, reads each operand right before its use and the
+        // matrix core waits out every LDS round trip.
+        uint4 operand[2][2], parked_q[2];
+        auto read_step = [&](int step, int slot) __attribute__((always_inline)) {
+            const unsigned char* at = step < kLatentSteps ? stage + score_at[step & 3] + 256 * (step >> 2) : stage + positional_at[step & 1];
+            const int half_stride = step < kLatentSteps ? 16 * kLatentRowBytes : 16 * kPositionalRowBytes;
+            operand[slot][0] = *reinterpret_cast<const uint4*>(at);
+            operand[slot][1] = *reinterpret_cast<const uint4*>(at + half_stride);
+            if (step < kParkedSteps) parked_q[slot] = *reinterpret_cast<const uint4*>(parked + 1024 * step);
+        };
+        read_step(0, 0);
+#pragma unroll
+        for (int step = 0; step < kSteps; ++step) {
+            if (step + 1 < kSteps) read_step(step + 1, (step + 1) % 2);
+            __builtin_amdgcn_sched_barrier(0);
+            const uint4 mine = step < kParkedSteps ? parked_q[step % 2] : q[step < kParkedSteps ? 0 : step - kParkedSteps];
+            s[0] = mma(half, operand[step % 2][0], mine, s[0]);
+            s[1] = mma(half, operand[step % 2][1], mine, s[1]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // Register r of half t is key key0 + 16 t + 4 g + r against the lane's row.
+        float x[8];
+        const bool edge = key0 + kKeys > keys || (causal && key0 + kKeys - 1u > wave_low);
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                float value = s[t][r] * scale_log2e;
+                if (edge) {
+                    const unsigned int key = key0 + 16u * t + 4u * g + r;
+                    if (key >= keys || (causal && key > my_position)) value = -INFINITY;
+                }
+                x[4 * t + r] = value;
+            }
+        float largest = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
+        largest = fmaxf(largest, __shfl_xor(largest, 16, 64));
+        largest = fmaxf(largest, __shfl_xor(largest, 32, 64));  // the four lanes of a row agree from here on
+        if (__any(largest > reference + kMaxLag || (reference == -INFINITY && largest != -INFINITY))) {
+            const float moved = fmaxf(reference, largest);
+            const float base = moved == -INFINITY ? 0.0f : moved;
+            const float rescale = fast_exp2(reference - base);
+            running_sum *= rescale;
+#pragma unroll
+            for (int db = 0; db < kDimBlocks; ++db)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) out[db][r] *= rescale;
+            reference = moved;
+        }
+        const float shift = reference == -INFINITY ? 0.0f : -reference;
+        float p[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            p[i] = fast_exp2(x[i] + shift);
+            running_sum += p[i];
+        }
+        // The weights, rounded as the value product takes them: slots 8 g .. 8 g + 3 are keys 4 g .. 4 g + 3, slots
+        // 8 g + 4 .. 8 g + 7 keys 16 + 4 g .. 16 + 4 g + 3.
+        const uint4 weights = make_uint4(pack_pair(half, p[0], p[1]), pack_pair(half, p[2], p[3]), pack_pair(half, p[4], p[5]),
+                                         pack_pair(half, p[6], p[7]));
+        // The transposed operands likewise, two dim blocks ahead (a ring of three).
+        v4i16_t low[3], high[3];
+        auto read_block = [&](int db, int slot) __attribute__((always_inline)) {
+            const unsigned char* at = stage + value_at[db & 7] + 256 * (db >> 3);
+            low[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(at));
+            high[slot] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(at + 16 * kLatentRowBytes));
+        };
+        read_block(0, 0);
+        read_block(1, 1);
+#pragma unroll
+        for (int db = 0; db < kDimBlocks; ++db) {
+            if (db + 2 < kDimBlocks) read_block(db + 2, (db + 2) % 3);
+            __builtin_amdgcn_sched_barrier(0);
+            const prefill::v8i16_t both = __builtin_shufflevector(low[db % 3], high[db % 3], 0, 1, 2, 3, 4, 5, 6, 7);
+            out[db] = mma(half, __builtin_bit_cast(uint4, both), weights, out[db]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    if (tiles > 0) {
+        TilePages<FORM> pages = lookup(0);
+        issue(0, pages, lds);
+        if (tiles > 1) pages = lookup(1);
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __syncthreads();
+        for (unsigned int tile = 0; tile < tiles; ++tile) {
+            unsigned char* stage = lds + (tile & 1u) * kStageBytes;
+            unsigned char* other = lds + ((tile & 1u) ^ 1u) * kStageBytes;
+            if (tile + 1 < tiles) issue(tile + 1, pages, other);
+            if (tile + 2 < tiles) pages = lookup(tile + 2);
+            if (tile * kKeys < wave_end) fold(tile, stage);
+            __builtin_amdgcn_s_waitcnt(0x0F70);  // this wave's loads have landed
+            __syncthreads();                     // and everyone has finished reading
+        }
+    }
+
+    // Normalise and store; a row that sees no key stays zero and has a log-sum-exp of -inf.
+    float sum = running_sum;
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
+    const float inverse = sum > 0.0f ? 1.0f / sum : 0.0f;
+    if (row_valid) {
+        unsigned char* row = static_cast<unsigned char*>(a.output) + flat * kLatentRowBytes + 8u * g;
+#pragma unroll
+        for (int db = 0; db < kDimBlocks; ++db) {
+            uint2 packed;
+            packed.x = pack_pair(half, out[db][0] * inverse, out[db][1] * inverse);
+            packed.y = pack_pair(half, out[db][2] * inverse, out[db][3] * inverse);
+            *reinterpret_cast<uint2*>(row + 32 * db) = packed;
+        }
+        if (a.lse != nullptr && g == 0) a.lse[flat] = sum > 0.0f ? reference + fast_log2(sum) : -INFINITY;
+    }
+}
+
+template <class Half>
+SINGE_DEVICE void latent_tile_body(const LatentAttentionArgs& a, unsigned char* lds) {
+    if (a.wide_index)
+        latent_tile_rows<Half, kCsrI64>(a, lds);
+    else
+        latent_tile_rows<Half, kCsrI32>(a, lds);
+}
+
+}  // namespace latent_mfma
+
+#define SINGE_LATENT_MFMA_KERNEL(NAME, HALF)                                                              \
+    extern "C" __global__ __launch_bounds__(64 * latent_mfma::kWaves, 2) void NAME(LatentAttentionArgs args) { \
+        __shared__ __attribute__((aligned(1024))) unsigned char latent_lds[latent_mfma::kLdsBytes];         \
+        latent_mfma::latent_tile_body<prefill::HALF>(args, latent_lds);                                    \
+    }
+
+SINGE_LATENT_MFMA_KERNEL(singe_paged_mla_attention_bf16_l512_p64, Bf16)
+SINGE_LATENT_MFMA_KERNEL(singe_paged_mla_attention_f16_l512_p64, F16)

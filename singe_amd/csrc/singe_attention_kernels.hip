@@ -8,4 +8,5 @@
 #include "attention_rows_f32.hip"
 #include "general_attention.hip"
 #include "latent_attention.hip"
+#include "latent_attention_mfma.hip"
 #include "cache_ops.hip"

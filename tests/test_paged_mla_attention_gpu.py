@@ -59,6 +59,44 @@ def test_matches_the_cpu_over_ragged_sequences(sequences, heads, latent, positio
     assert (np.abs(got_lse[~empty] - want_lse[~empty]) <= 1e-3 * np.maximum(np.abs(want_lse[~empty]), 1.0)).all()
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("heads,page_size,index_dtype", [(128, 16, torch.int32), (24, 5, torch.int64), (1, 64, torch.int32), (40, 1, torch.int32)])
+def test_matrix_core_shape_on_random_data(heads, page_size, index_dtype, causal, dtype):
+    """Latent width 512 with positional width 64 runs on the matrix cores, 128 (token, head) rows to a workgroup:
+    head counts that fill a workgroup exactly, leave waves empty, or let one wave's rows span several tokens;
+    decode rows, chunks, whole prefills, more queries than keys, a sequence without keys."""
+    sequences = [(1, 700), (37, 37), (20, 333), (3, 0), (9, 4), (1, 65)]
+    query_offsets, page_offsets, last, needed = [0], [0], [], 0
+    for queries, keys in sequences:
+        query_offsets.append(query_offsets[-1] + queries)
+        pages = (keys + page_size - 1) // page_size
+        needed += pages
+        page_offsets.append(needed)
+        last.append(0 if keys == 0 else keys - (pages - 1) * page_size)
+    page_count = needed + 2
+    rng = np.random.default_rng(heads + page_size)
+    table = [int(page) for page in rng.permutation(page_count)[:needed]]
+    tokens = query_offsets[-1]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(heads)
+    rand = lambda *shape: torch.randn(shape, generator=gen, device="cuda").to(dtype)
+    device = [rand(tokens, heads, 512), rand(tokens, heads, 64), rand(page_count, page_size, 512), rand(page_count, page_size, 64)]
+    index = lambda entries: torch.tensor(entries, dtype=index_dtype, device="cuda")
+    paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
+    out, lse = neural.paged_mla_attention(*device, paging, neural.AttentionOptions(causal=causal))
+    torch.cuda.synchronize()
+    status, want, want_lse = oracle.paged_mla_attention(*[tensor.float().cpu().numpy() for tensor in device], query_offsets, page_offsets, table,
+                                                        last, causal=causal, threads=8)
+    assert status == 0
+    got, got_lse = out.float().cpu().numpy(), lse.cpu().numpy()
+    gap = np.abs(got - want)
+    assert gap.max() <= 2e-2 and gap.mean() <= 2e-3, (gap.max(), gap.mean())
+    empty = np.isneginf(want_lse)
+    assert np.array_equal(np.isneginf(got_lse), empty) and not got[empty].any()
+    assert np.abs(got_lse[~empty] - want_lse[~empty]).max() <= 5e-3
+
+
 def test_default_scale_counts_the_whole_key_width_and_int64_indices():
     gen = torch.Generator(device="cuda")
     gen.manual_seed(1)
