@@ -740,8 +740,9 @@ SINGE_HIP_API void singe_hip_clear_tune_cache(void);
  * position_dim) unless given; output [tokens, heads, latent_dim] of the operands' type; lse [tokens, heads] f32
  * base two, -inf for a row without keys (may be null).  Paging, causal alignment and the status word are those
  * of singe_hip_paged_attention_*.  All operands contiguous, one element type; latent_dim <= 512 and
- * position_dim <= 128 (SINGE_HIP_UNSUPPORTED_WIDTH beyond).  A vector-unit kernel, one wave per (token, head)
- * row: it gives the op on this device, not the matrix-core throughput of the reference's plan. */
+ * position_dim <= 128 (SINGE_HIP_UNSUPPORTED_WIDTH beyond).  bf16 and f16 at latent_dim 512 with position_dim 64
+ * run on the matrix cores, 128 (token, head) rows of a sequence to a workgroup that share every cache tile; every
+ * other shape on a vector-unit kernel, one wave per (token, head) row. */
 typedef struct SingePagedMlaAttentionProblem {
     int64_t tokens;
     int64_t heads;
@@ -771,6 +772,35 @@ SINGE_HIP_API int32_t singe_hip_paged_mla_attention(
     void* output,
     float* lse,
     uint32_t* status,
+    const SingePagedMlaAttentionProblem* problem);
+
+/* The same op with scratch for key splits, for the shapes on the matrix cores.  A decode step or a short chunk has
+ * one workgroup per 128 rows of a sequence, too few to fill the chip; given scratch, the keys of a row tile are
+ * shared out over several workgroups, each leaving a normalised f32 partial and its base-two log-sum-exp, and a
+ * second kernel merges them (the reference's plan declares such scratch and merges the same way:
+ * kernel_plan/source/mla.rs:232-241, 497-560).  singe_hip_paged_mla_attention_scratch_bytes says how much this
+ * problem wants (0: it would not split); with a null or smaller buffer the call runs unsplit, exactly as
+ * singe_hip_paged_mla_attention.  The scratch, 16-byte aligned, holds nothing between calls; calls that share it
+ * must not overlap.  Results equal the unsplit ones up to the order of summation.
+ * singe_hip_set_paged_mla_attention_splits fixes the number of shares (0 = chosen by problem size, the default; at
+ * most 64); it changes what ..._scratch_bytes returns. */
+SINGE_HIP_API size_t singe_hip_paged_mla_attention_scratch_bytes(const SingePagedMlaAttentionProblem* problem);
+SINGE_HIP_API void singe_hip_set_paged_mla_attention_splits(uint32_t splits);
+SINGE_HIP_API int32_t singe_hip_paged_mla_attention_scratch(
+    void* stream,
+    const void* latent_queries,
+    const void* positional_queries,
+    const void* latent_cache,
+    const void* positional_cache,
+    const void* query_offsets,
+    const void* page_offsets,
+    const void* pages,
+    const void* last_page_lengths,
+    void* output,
+    float* lse,
+    uint32_t* status,
+    void* scratch,
+    size_t scratch_bytes,
     const SingePagedMlaAttentionProblem* problem);
 
 /* ---- singe surface: the steps either side of paged attention ------------------------------------------

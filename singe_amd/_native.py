@@ -220,6 +220,12 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_set_paged_attention_splits.restype = None
     handle.singe_hip_paged_mla_attention.argtypes = [c_void] * 12 + [ctypes.POINTER(PagedMlaAttentionProblemC)]
     handle.singe_hip_paged_mla_attention.restype = i32
+    handle.singe_hip_paged_mla_attention_scratch.argtypes = [c_void] * 13 + [c_size, ctypes.POINTER(PagedMlaAttentionProblemC)]
+    handle.singe_hip_paged_mla_attention_scratch.restype = i32
+    handle.singe_hip_paged_mla_attention_scratch_bytes.argtypes = [ctypes.POINTER(PagedMlaAttentionProblemC)]
+    handle.singe_hip_paged_mla_attention_scratch_bytes.restype = ctypes.c_size_t
+    handle.singe_hip_set_paged_mla_attention_splits.argtypes = [ctypes.c_uint32]
+    handle.singe_hip_set_paged_mla_attention_splits.restype = None
     handle.singe_hip_paged_attention_f32.argtypes = [c_void] * 11 + [ctypes.POINTER(PagedAttentionProblemC)]
     handle.singe_hip_paged_attention_f32.restype = i32
     handle.singe_hip_paged_attention_f16.argtypes = [c_void] * 11 + [ctypes.POINTER(PagedAttentionProblemC)]

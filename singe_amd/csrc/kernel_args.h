@@ -244,9 +244,15 @@ struct LatentAttentionArgs {
     float* lse;                      // [tokens, heads] base two, or null
     uint32_t* status;
     uint32_t tokens, heads, latent_dim, position_dim, page_size, sequences, cache_pages, page_table;
-    uint32_t row_blocks;             // workgroups (4 rows each) per sequence
+    uint32_t row_blocks;             // workgroups per sequence (4 rows each; 128 each on the matrix-core kernel)
     uint32_t causal, wide_index;
     float scale;
+    // Matrix-core kernel with key splits (splits > 1): each of a row tile's `splits` workgroups leaves its rows
+    // normalised in partial_out [splits, tokens, heads, latent_dim] with a base-two log-sum-exp in partial_lse
+    // [splits, tokens, heads] (-inf and zeros for a share without keys); singe_paged_mla_attention_combine_* merges.
+    uint32_t splits;
+    float* partial_out;
+    float* partial_lse;
 };
 
 // singe_rotary_cache_write_*: contiguous operands of one element type; angles may be f32.

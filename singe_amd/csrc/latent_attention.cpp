@@ -2,6 +2,7 @@
 // (singe/src/backend/spec/neural/attention.rs:453-497) and the launch, with the kernel's arguments in the order of
 // the reference artifact's ABI (singe/src/backend/cuda/kernel_plan/source/mla.rs:219-230, 260).
 #include <cmath>
+#include <cstdint>
 
 #include "kernel_args.h"
 #include "module.h"
@@ -10,11 +11,40 @@
 
 using namespace singe_hip;
 
-extern "C" int32_t singe_hip_paged_mla_attention(void* stream, const void* latent_queries, const void* positional_queries,
-                                                 const void* latent_cache, const void* positional_cache,
-                                                 const void* query_offsets, const void* page_offsets, const void* pages,
-                                                 const void* last_page_lengths, void* output, float* lse, uint32_t* status,
-                                                 const SingePagedMlaAttentionProblem* problem) {
+namespace {
+
+// Whether the problem runs on the matrix-core kernel (latent width 512, positional width 64, a 16-bit type).
+bool on_matrix_cores(const SingePagedMlaAttentionProblem& p) {
+    return p.data_type != SINGE_HIP_F32 && p.latent_dim == 512 && p.position_dim == 64;
+}
+
+// Key splits for a problem: the row tiles of a decode step or a short chunk (one workgroup each, one workgroup to a
+// compute unit) leave most of the chip idle, so each tile's keys are shared out until there is about one workgroup
+// per compute unit.  The count of live tiles is not known on the host (it depends on the offsets on the device):
+// every sequence has at least one, and together they hold at least tokens * heads / 128.
+// 0 = chosen by problem size (singe_hip_set_paged_mla_attention_splits).
+uint32_t g_latent_splits = 0;
+
+uint32_t latent_splits(const SingePagedMlaAttentionProblem& p) {
+    if (!on_matrix_cores(p) || p.tokens <= 0 || p.heads <= 0 || p.sequences <= 0) return 1;
+    if (g_latent_splits != 0) return g_latent_splits;
+    const uint64_t packed = (static_cast<uint64_t>(p.tokens) * p.heads + 127) / 128;
+    const uint64_t workgroups = packed > static_cast<uint64_t>(p.sequences) ? packed : static_cast<uint64_t>(p.sequences);
+    const uint64_t wanted = compute_units();
+    if (workgroups >= wanted) return 1;
+    const uint64_t splits = wanted / workgroups;
+    return static_cast<uint32_t>(splits > 16 ? 16 : splits < 1 ? 1 : splits);
+}
+
+size_t latent_scratch_bytes(const SingePagedMlaAttentionProblem& p, uint32_t splits) {
+    if (splits <= 1) return 0;
+    return static_cast<size_t>(splits) * static_cast<size_t>(p.tokens) * static_cast<size_t>(p.heads) * (512 + 1) * sizeof(float);
+}
+
+int32_t paged_mla_attention(void* stream, const void* latent_queries, const void* positional_queries, const void* latent_cache,
+                            const void* positional_cache, const void* query_offsets, const void* page_offsets, const void* pages,
+                            const void* last_page_lengths, void* output, float* lse, uint32_t* status, void* scratch,
+                            size_t scratch_bytes, const SingePagedMlaAttentionProblem* problem) {
     if (problem == nullptr) return fail(SINGE_HIP_NULL_POINTER, "problem");
     const SingePagedMlaAttentionProblem& p = *problem;
     // paged_mla_attention_problem: a page holds at least one key and the latent width is positive; the
@@ -63,7 +93,7 @@ extern "C" int32_t singe_hip_paged_mla_attention(void* stream, const void* laten
     args.page_table = static_cast<uint32_t>(p.page_table);
     // Latent width 512 with positional width 64 in a 16-bit type runs on the matrix cores, 128 (token, head) rows of
     // a sequence to a workgroup; every other shape on the vector unit, 4 rows to a workgroup.
-    const bool tiles = p.data_type != SINGE_HIP_F32 && p.latent_dim == 512 && p.position_dim == 64;
+    const bool tiles = on_matrix_cores(p);
     const uint64_t rows_per_block = tiles ? 128 : 4;
     const uint64_t row_blocks = (static_cast<uint64_t>(p.tokens) * p.heads + rows_per_block - 1) / rows_per_block;
     args.row_blocks = static_cast<uint32_t>(row_blocks);
@@ -71,10 +101,57 @@ extern "C" int32_t singe_hip_paged_mla_attention(void* stream, const void* laten
     args.wide_index = p.index_type == SINGE_HIP_INDEX_I64 ? 1u : 0u;
     // The default scale counts the whole key width (attention.rs:603-606).
     args.scale = p.has_scale ? p.scale : static_cast<float>(1.0 / std::sqrt(static_cast<double>(p.latent_dim + p.position_dim)));
-    const uint64_t blocks = row_blocks * static_cast<uint64_t>(p.sequences);
+    // The matrix-core kernel's units: a sequence owns one per 128 of its rows, at least one; the vector-unit kernel
+    // takes the upper bound for every sequence.
+    const uint64_t blocks = tiles ? row_blocks + static_cast<uint64_t>(p.sequences) : row_blocks * static_cast<uint64_t>(p.sequences);
     if (blocks > 0x7fffffffull || row_blocks > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
-    if (tiles)
-        return launch(p.data_type == SINGE_HIP_BF16 ? kLatentTilesBf16 : kLatentTilesF16, static_cast<unsigned>(blocks), 1, 1, 512, stream, args);
+    args.splits = 1;
+    args.partial_out = nullptr;
+    args.partial_lse = nullptr;
+    if (tiles) {
+        // Key splits, when the caller lent scratch for them: the attention kernel leaves partials, a second kernel
+        // merges them.
+        uint32_t splits = scratch != nullptr ? latent_splits(p) : 1;
+        if (splits > 1 && (scratch_bytes < latent_scratch_bytes(p, splits) || blocks * splits > 0x7fffffffull)) splits = 1;
+        if (splits > 1) {
+            if (reinterpret_cast<uintptr_t>(scratch) % 16 != 0) return fail(SINGE_HIP_INVALID_ARGUMENT, "scratch alignment");
+            args.splits = splits;
+            args.partial_out = static_cast<float*>(scratch);
+            args.partial_lse = args.partial_out + static_cast<size_t>(splits) * p.tokens * p.heads * 512;
+        }
+        const bool bf16 = p.data_type == SINGE_HIP_BF16;
+        const int32_t launched = launch(bf16 ? kLatentTilesBf16 : kLatentTilesF16, static_cast<unsigned>(blocks * splits), 1, 1, 512, stream, args);
+        if (launched != 0 || splits == 1) return launched;
+        return launch(bf16 ? kLatentCombineBf16 : kLatentCombineF16, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+    }
     const int kernel = kLatentGeneral + (p.data_type == SINGE_HIP_F32 ? 0 : p.data_type == SINGE_HIP_BF16 ? 1 : 2);
     return launch(static_cast<KernelId>(kernel), static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+}
+
+}  // namespace
+
+extern "C" int32_t singe_hip_paged_mla_attention(void* stream, const void* latent_queries, const void* positional_queries,
+                                                 const void* latent_cache, const void* positional_cache,
+                                                 const void* query_offsets, const void* page_offsets, const void* pages,
+                                                 const void* last_page_lengths, void* output, float* lse, uint32_t* status,
+                                                 const SingePagedMlaAttentionProblem* problem) {
+    return paged_mla_attention(stream, latent_queries, positional_queries, latent_cache, positional_cache, query_offsets, page_offsets,
+                               pages, last_page_lengths, output, lse, status, nullptr, 0, problem);
+}
+
+extern "C" void singe_hip_set_paged_mla_attention_splits(uint32_t splits) { g_latent_splits = splits > 64 ? 64 : splits; }
+
+extern "C" size_t singe_hip_paged_mla_attention_scratch_bytes(const SingePagedMlaAttentionProblem* problem) {
+    if (problem == nullptr) return 0;
+    return latent_scratch_bytes(*problem, latent_splits(*problem));
+}
+
+extern "C" int32_t singe_hip_paged_mla_attention_scratch(void* stream, const void* latent_queries, const void* positional_queries,
+                                                         const void* latent_cache, const void* positional_cache,
+                                                         const void* query_offsets, const void* page_offsets, const void* pages,
+                                                         const void* last_page_lengths, void* output, float* lse, uint32_t* status,
+                                                         void* scratch, size_t scratch_bytes,
+                                                         const SingePagedMlaAttentionProblem* problem) {
+    return paged_mla_attention(stream, latent_queries, positional_queries, latent_cache, positional_cache, query_offsets, page_offsets,
+                               pages, last_page_lengths, output, lse, status, scratch, scratch_bytes, problem);
 }

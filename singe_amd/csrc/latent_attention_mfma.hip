@@ -77,6 +77,42 @@ SINGE_DEVICE unsigned int chunk_flip(unsigned int key) {
     return (pair << 1) | ((key >> 3) & 1u);
 }
 
+// Workgroup units map to (sequence, row tile) in sequence order: sequence s owns max(1, ceil(rows_s / 128)) units (one
+// even without rows, so that its paging values are checked), which every wave finds for itself by a prefix sum over
+// the query offsets, 64 sequences at a time.  Returns false for a unit past the last sequence's.
+template <int FORM>
+SINGE_DEVICE bool find_unit(const LatentAttentionArgs& a, unsigned int unit, unsigned int& sequence, unsigned int& row_tile) {
+    const unsigned int lane = threadIdx.x & 63u;
+    unsigned int base = 0;
+    for (unsigned int first = 0; first < a.sequences; first += 64u) {
+        const unsigned int s = first + lane;
+        unsigned int mine = 0;
+        if (s < a.sequences) {
+            long long count = read_index<FORM>(a.query_offsets, s + 1) - read_index<FORM>(a.query_offsets, s);
+            count = count < 0 ? 0 : count > static_cast<long long>(a.tokens) ? static_cast<long long>(a.tokens) : count;
+            const unsigned long long tiles = (static_cast<unsigned long long>(count) * a.heads + kRows - 1) / kRows;
+            mine = tiles == 0 ? 1u : static_cast<unsigned int>(tiles);
+        }
+        unsigned int through = mine;  // inclusive prefix sum over the wave
+#pragma unroll
+        for (int step = 1; step < 64; step <<= 1) {
+            const unsigned int below = __shfl_up(through, step, 64);
+            if (lane >= static_cast<unsigned int>(step)) through += below;
+        }
+        const unsigned int total = __shfl(through, 63, 64);
+        if (unit < base + total) {
+            const unsigned long long holds = __ballot(unit < base + through);  // first lane whose range reaches the unit
+            const unsigned int owner = static_cast<unsigned int>(__builtin_ctzll(holds));
+            const unsigned int owner_through = __shfl(through, owner, 64), owner_mine = __shfl(mine, owner, 64);
+            sequence = first + owner;
+            row_tile = unit - (base + owner_through - owner_mine);
+            return true;
+        }
+        base += total;
+    }
+    return false;
+}
+
 // What a wave needs to know of the keys it loads for one tile: its four latent rows (wave-uniform) and, for waves
 // 0-3, each lane's positional row.
 template <int FORM>
@@ -89,9 +125,12 @@ template <class Half, int FORM>
 SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* lds) {
     const unsigned int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
     const unsigned int column = lane & 15u, g = lane >> 4;  // row of the wave, lane group
-    // Row tiles are the slow index of the grid: the first tiles of all sequences, the ones a decode step has, are
-    // neighbours and spread over the chip.
-    const unsigned int sequence = blockIdx.x % a.sequences, row_tile = blockIdx.x / a.sequences;
+    const unsigned int splits = a.splits > 1 ? a.splits : 1u;
+    const unsigned int split = blockIdx.x % splits, unit = blockIdx.x / splits;
+    unsigned int sequence, row_tile;
+    if (!find_unit<FORM>(a, unit, sequence, row_tile)) return;
+    sequence = __builtin_amdgcn_readfirstlane(sequence);
+    row_tile = __builtin_amdgcn_readfirstlane(row_tile);
     const SequenceSpan span = load_span<FORM>(sequence, a.query_offsets, a.page_offsets, a.last_page_lengths, nullptr, a.tokens,
                                               a.page_table, a.page_size);
     if (!span.valid) {
@@ -122,7 +161,13 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
         const unsigned int reach = position_of(group_last) + 1u;
         key_end = key_end < reach ? key_end : reach;
     }
-    const unsigned int tiles = (key_end + kKeys - 1) / kKeys;
+    // With key splits this workgroup takes one share of the tiles; a share may be empty.
+    unsigned int first_tile = 0, tiles = (key_end + kKeys - 1) / kKeys;
+    if (splits > 1) {
+        const unsigned int share = (tiles + splits - 1) / splits;
+        first_tile = split * share;
+        tiles = tiles < first_tile + share ? tiles : first_tile + share;
+    }
     const unsigned long long wave_first = first_row + 16u * wave;
     const bool wave_live = wave_first < rows;
     const unsigned long long wave_last = wave_first + 15u < rows ? wave_first + 15u : rows - 1;
@@ -312,13 +357,13 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
         }
     };
 
-    if (tiles > 0) {
-        TilePages<FORM> pages = lookup(0);
-        issue(0, pages, lds);
-        if (tiles > 1) pages = lookup(1);
+    if (first_tile < tiles) {
+        TilePages<FORM> pages = lookup(first_tile);
+        issue(first_tile, pages, lds + (first_tile & 1u) * kStageBytes);
+        if (first_tile + 1 < tiles) pages = lookup(first_tile + 1);
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
-        for (unsigned int tile = 0; tile < tiles; ++tile) {
+        for (unsigned int tile = first_tile; tile < tiles; ++tile) {
             unsigned char* stage = lds + (tile & 1u) * kStageBytes;
             unsigned char* other = lds + ((tile & 1u) ^ 1u) * kStageBytes;
             if (tile + 1 < tiles) issue(tile + 1, pages, other);
@@ -334,7 +379,15 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
     sum += __shfl_xor(sum, 16, 64);
     sum += __shfl_xor(sum, 32, 64);
     const float inverse = sum > 0.0f ? 1.0f / sum : 0.0f;
-    if (row_valid) {
+    if (row_valid && splits > 1) {
+        const size_t slot = static_cast<size_t>(split) * a.tokens * a.heads + flat;
+        float* row = a.partial_out + slot * kLatent + 4u * g;
+#pragma unroll
+        for (int db = 0; db < kDimBlocks; ++db)
+            *reinterpret_cast<float4*>(row + 16 * db) =
+                make_float4(out[db][0] * inverse, out[db][1] * inverse, out[db][2] * inverse, out[db][3] * inverse);
+        if (g == 0) a.partial_lse[slot] = sum > 0.0f ? reference + fast_log2(sum) : -INFINITY;
+    } else if (row_valid) {
         unsigned char* row = static_cast<unsigned char*>(a.output) + flat * kLatentRowBytes + 8u * g;
 #pragma unroll
         for (int db = 0; db < kDimBlocks; ++db) {
@@ -344,6 +397,52 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
             *reinterpret_cast<uint2*>(row + 32 * db) = packed;
         }
         if (a.lse != nullptr && g == 0) a.lse[flat] = sum > 0.0f ? reference + fast_log2(sum) : -INFINITY;
+    }
+}
+
+// Merges the shares of a row: out = sum_s 2^(lse_s - m) o_s / sum_s 2^(lse_s - m), lse = m + log2 of that sum
+// (the merge of the reference's own split kernels, kernel_plan/source/mla.rs:497-560).  One wave per (token, head)
+// row at a time, lane l dims 8 l .. 8 l + 7; a row whose shares are all empty stays zero with a log-sum-exp of -inf.
+template <class Half, int FORM>
+SINGE_DEVICE void latent_combine_rows(const LatentAttentionArgs& a) {
+    const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    // Workgroups map to (sequence, row tile) as in the attention kernel, so only rows that kernel wrote are read.
+    unsigned int sequence, row_tile;
+    if (!find_unit<FORM>(a, blockIdx.x, sequence, row_tile)) return;
+    const SequenceSpan span = load_span<FORM>(sequence, a.query_offsets, a.page_offsets, a.last_page_lengths, nullptr, a.tokens,
+                                              a.page_table, a.page_size);
+    if (!span.valid) return;  // the attention kernel has reported it
+    const unsigned long long rows = static_cast<unsigned long long>(span.queries) * a.heads;
+    const size_t rows_total = static_cast<size_t>(a.tokens) * a.heads;
+    const unsigned long long tile_end = static_cast<unsigned long long>(row_tile + 1u) * kRows;
+    for (unsigned long long local = static_cast<unsigned long long>(row_tile) * kRows + wave; local < rows && local < tile_end; local += 4u) {
+        const size_t row = (static_cast<size_t>(span.query_start) + local / a.heads) * a.heads + local % a.heads;
+        float largest = -INFINITY;
+        for (unsigned int s = 0; s < a.splits; ++s) largest = fmaxf(largest, a.partial_lse[s * rows_total + row]);
+        float total = 0.0f, acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+        if (largest != -INFINITY) {
+            for (unsigned int s = 0; s < a.splits; ++s) {
+                const float mine = a.partial_lse[s * rows_total + row];
+                if (mine == -INFINITY) continue;  // an empty share weighs nothing
+                const float weight = fast_exp2(mine - largest);
+                const float* part = a.partial_out + (s * rows_total + row) * kLatent + 8u * lane;
+                const float4 low = *reinterpret_cast<const float4*>(part), high = *reinterpret_cast<const float4*>(part + 4);
+                total += weight;
+                acc[0] = fmaf(weight, low.x, acc[0]); acc[1] = fmaf(weight, low.y, acc[1]);
+                acc[2] = fmaf(weight, low.z, acc[2]); acc[3] = fmaf(weight, low.w, acc[3]);
+                acc[4] = fmaf(weight, high.x, acc[4]); acc[5] = fmaf(weight, high.y, acc[5]);
+                acc[6] = fmaf(weight, high.z, acc[6]); acc[7] = fmaf(weight, high.w, acc[7]);
+            }
+        }
+        const float inverse = total > 0.0f ? 1.0f / total : 0.0f;
+        const Half half{};
+        uint4 packed;
+        packed.x = pack_pair(half, acc[0] * inverse, acc[1] * inverse);
+        packed.y = pack_pair(half, acc[2] * inverse, acc[3] * inverse);
+        packed.z = pack_pair(half, acc[4] * inverse, acc[5] * inverse);
+        packed.w = pack_pair(half, acc[6] * inverse, acc[7] * inverse);
+        *reinterpret_cast<uint4*>(static_cast<unsigned char*>(a.output) + row * kLatentRowBytes + 16u * lane) = packed;
+        if (a.lse != nullptr && lane == 0) a.lse[row] = total > 0.0f ? largest + fast_log2(total) : -INFINITY;
     }
 }
 
@@ -363,5 +462,15 @@ SINGE_DEVICE void latent_tile_body(const LatentAttentionArgs& a, unsigned char* 
         latent_mfma::latent_tile_body<prefill::HALF>(args, latent_lds);                                    \
     }
 
+#define SINGE_LATENT_COMBINE_KERNEL(NAME, HALF)                                                  \
+    extern "C" __global__ __launch_bounds__(256) void NAME(LatentAttentionArgs args) {          \
+        if (args.wide_index)                                                                    \
+            latent_mfma::latent_combine_rows<prefill::HALF, kCsrI64>(args);                     \
+        else                                                                                    \
+            latent_mfma::latent_combine_rows<prefill::HALF, kCsrI32>(args);                     \
+    }
+
+SINGE_LATENT_COMBINE_KERNEL(singe_paged_mla_attention_combine_bf16, Bf16)
+SINGE_LATENT_COMBINE_KERNEL(singe_paged_mla_attention_combine_f16, F16)
 SINGE_LATENT_MFMA_KERNEL(singe_paged_mla_attention_bf16_l512_p64, Bf16)
 SINGE_LATENT_MFMA_KERNEL(singe_paged_mla_attention_f16_l512_p64, F16)

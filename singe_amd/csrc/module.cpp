@@ -57,6 +57,7 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paging_indices_i32", "singe_paging_indices_i64",
     "singe_paged_mla_attention_general_f32", "singe_paged_mla_attention_general_bf16", "singe_paged_mla_attention_general_f16",
     "singe_paged_mla_attention_bf16_l512_p64", "singe_paged_mla_attention_f16_l512_p64",
+    "singe_paged_mla_attention_combine_bf16", "singe_paged_mla_attention_combine_f16",
     "singe_attention_general_f32_d64", "singe_attention_general_f32_d128", "singe_attention_general_f32_d256",
     "singe_attention_general_bf16_d64", "singe_attention_general_bf16_d128", "singe_attention_general_bf16_d256",
     "singe_attention_general_f16_d64", "singe_attention_general_f16_d128", "singe_attention_general_f16_d256",

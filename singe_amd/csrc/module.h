@@ -41,7 +41,7 @@ enum KernelId : int {
     // latent (MLA) attention: + element (f32, bf16, f16)
     kLatentGeneral, kLatentGeneralBf16, kLatentGeneralF16,
     // the same at latent width 512, positional width 64 on the matrix cores
-    kLatentTilesBf16, kLatentTilesF16,
+    kLatentTilesBf16, kLatentTilesF16, kLatentCombineBf16, kLatentCombineF16,
     // general kernels: index = base + 3 * element (f32, bf16, f16) + width (64, 128, 256)
     kDenseGeneral,
     kPagedGeneral = kDenseGeneral + 9,

@@ -213,12 +213,15 @@ def paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: t
 
 def paged_mla_attention(query: torch.Tensor, query_positions: torch.Tensor, latent_cache: torch.Tensor,
                         position_cache: torch.Tensor, paging: Paging, options: AttentionOptions = AttentionOptions(), *,
-                        stream=None, status: torch.Tensor | None = None, check: bool = True):
+                        stream=None, status: torch.Tensor | None = None, check: bool = True,
+                        scratch: "torch.Tensor | bool" = True):
     """Tensor::paged_mla_attention (singe/src/backend/spec/neural/attention.rs:453-497, CPU
     normalization/attention.rs:540-679): latent attention over paged caches.  ``query`` [tokens, heads, latent],
     ``query_positions`` [tokens, heads, positional], ``latent_cache`` [pages, page_size, latent], ``position_cache``
     [pages, page_size, positional], f32 / bf16 / f16.  Only ``causal`` and ``scale`` of the options apply.  Returns
-    (output [tokens, heads, latent] of the query's type, lse [tokens, heads] f32 base two)."""
+    (output [tokens, heads, latent] of the query's type, lse [tokens, heads] f32 base two).  ``scratch`` as for
+    paged_attention: with few rows (decoding) the matrix-core kernel shares a row tile's keys out over several
+    workgroups, given a uint8 device tensor, or True for this module's own per-device buffer; False for none."""
     if options.window is not None or options.softcap is not None:
         raise error.InvalidArgument("paged mla attention takes a scale and a causal mask only")
     operands = ((query, "query"), (query_positions, "query_positions"), (latent_cache, "latent_cache"), (position_cache, "position_cache"))
@@ -252,10 +255,18 @@ def paged_mla_attention(query: torch.Tensor, query_positions: torch.Tensor, late
     if status is None:
         status = torch.zeros(1, device=query.device, dtype=torch.int32)
     handle = int((stream or torch.cuda.current_stream()).cuda_stream)
-    code = _native.lib().singe_hip_paged_mla_attention(
-        handle, query.data_ptr(), query_positions.data_ptr(), latent_cache.data_ptr(), position_cache.data_ptr(),
-        paging.query_offsets.data_ptr(), paging.page_offsets.data_ptr(), paging.pages.data_ptr(), paging.last_page_lengths.data_ptr(),
-        output.data_ptr(), lse.data_ptr(), status.data_ptr(), ctypes.byref(problem))
+    wanted = 0 if scratch is False else int(_native.lib().singe_hip_paged_mla_attention_scratch_bytes(ctypes.byref(problem)))
+    if wanted > 0:
+        lent = _scratch_for(query.device, wanted) if scratch is True else scratch
+        code = _native.lib().singe_hip_paged_mla_attention_scratch(
+            handle, query.data_ptr(), query_positions.data_ptr(), latent_cache.data_ptr(), position_cache.data_ptr(),
+            paging.query_offsets.data_ptr(), paging.page_offsets.data_ptr(), paging.pages.data_ptr(), paging.last_page_lengths.data_ptr(),
+            output.data_ptr(), lse.data_ptr(), status.data_ptr(), lent.data_ptr(), lent.numel(), ctypes.byref(problem))
+    else:
+        code = _native.lib().singe_hip_paged_mla_attention(
+            handle, query.data_ptr(), query_positions.data_ptr(), latent_cache.data_ptr(), position_cache.data_ptr(),
+            paging.query_offsets.data_ptr(), paging.page_offsets.data_ptr(), paging.pages.data_ptr(), paging.last_page_lengths.data_ptr(),
+            output.data_ptr(), lse.data_ptr(), status.data_ptr(), ctypes.byref(problem))
     _native.check(code, "paged_mla_attention")
     if check and int(status.item()) == STATUS_INDEX_OUT_OF_BOUNDS:
         raise error.IndexOutOfBounds("paged mla attention paging value outside its buffers")

@@ -97,6 +97,51 @@ def test_matrix_core_shape_on_random_data(heads, page_size, index_dtype, causal,
     assert np.abs(got_lse[~empty] - want_lse[~empty]).max() <= 5e-3
 
 
+@pytest.mark.parametrize("splits", [2, 3, 16, 64])
+@pytest.mark.parametrize("causal", [False, True])
+def test_key_splits_match_the_cpu_and_the_unsplit_kernel(splits, causal):
+    """With scratch lent, a row tile's keys are shared out over workgroups and merged by a second kernel: decode rows
+    over long and short caches, a chunk, a sequence without keys, more shares than a sequence has tiles."""
+    import ctypes
+    from singe_amd import _native
+    sequences, heads, page_size = [(1, 1500), (1, 40), (5, 700), (2, 0), (1, 65), (3, 300)], 24, 16
+    query_offsets, page_offsets, last, needed = [0], [0], [], 0
+    for queries, keys in sequences:
+        query_offsets.append(query_offsets[-1] + queries)
+        pages = (keys + page_size - 1) // page_size
+        needed += pages
+        page_offsets.append(needed)
+        last.append(0 if keys == 0 else keys - (pages - 1) * page_size)
+    rng = np.random.default_rng(splits)
+    table = [int(page) for page in rng.permutation(needed + 2)[:needed]]
+    tokens = query_offsets[-1]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(splits)
+    rand = lambda *shape: torch.randn(shape, generator=gen, device="cuda").to(torch.bfloat16)
+    device = [rand(tokens, heads, 512), rand(tokens, heads, 64), rand(needed + 2, page_size, 512), rand(needed + 2, page_size, 64)]
+    index = lambda entries: torch.tensor(entries, dtype=torch.int32, device="cuda")
+    paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
+    options = neural.AttentionOptions(causal=causal)
+    whole, whole_lse = neural.paged_mla_attention(*device, paging, options, scratch=False)
+    _native.lib().singe_hip_set_paged_mla_attention_splits(splits)
+    try:
+        out, lse = neural.paged_mla_attention(*device, paging, options)
+    finally:
+        _native.lib().singe_hip_set_paged_mla_attention_splits(0)
+    torch.cuda.synchronize()
+    status, want, want_lse = oracle.paged_mla_attention(*[tensor.float().cpu().numpy() for tensor in device], query_offsets, page_offsets, table,
+                                                        last, causal=causal, threads=8)
+    assert status == 0
+    got, got_lse = out.float().cpu().numpy(), lse.cpu().numpy()
+    gap = np.abs(got - want)
+    assert gap.max() <= 2e-2 and gap.mean() <= 2e-3, (gap.max(), gap.mean())
+    empty = np.isneginf(want_lse)
+    assert np.array_equal(np.isneginf(got_lse), empty) and not got[empty].any()
+    assert np.abs(got_lse[~empty] - want_lse[~empty]).max() <= 5e-3
+    assert (out.float() - whole.float()).abs().max().item() <= 2e-2
+    assert np.abs(got_lse[~empty] - whole_lse.cpu().numpy()[~empty]).max() <= 2e-3
+
+
 def test_default_scale_counts_the_whole_key_width_and_int64_indices():
     gen = torch.Generator(device="cuda")
     gen.manual_seed(1)
