@@ -10,8 +10,8 @@ consecutive steps cannot be served from the 256 MB Infinity Cache.
 Prints one JSON line: whole-job GB/s of algorithmic bytes, the roofline of the dominant kernel
 (measured with HIP events on the launch stream) and the CPU oracle timed on a bounded sample.  The
 same line carries, under "prefill", the causal flash-attention prefill measurement (TFLOP/s against
-the dense bf16 MFMA peak), and under "chunked_prefill", "fp8_decode" and "dense_f32" the other three
-benchmark configurations.
+the dense bf16 MFMA peak), under "chunked_prefill", "fp8_decode" and "dense_f32" the other three
+benchmark configurations, and under "latent" latent (MLA) attention over paged caches (decode and chunked prefill).
 """
 from __future__ import annotations
 
@@ -221,6 +221,66 @@ def chunked_prefill_section(steps):
     }
 
 
+def latent_section(steps):
+    """Latent (MLA) attention over paged caches at DeepSeek's widths (latent 512, positional 64, 128 heads, bf16,
+    page 64), beside the benchmark's configurations: a decode step (256 sequences of 4096 keys; every head reads
+    the same 1152 bytes per key, so the step is priced against HBM and the matrix cores both) and a chunked
+    prefill (8 x 512 new tokens on 8192 keys, priced against the dense bf16 MFMA peak).  Synthetic N(0,1) data."""
+    import numpy as np
+    import torch
+
+    from singe_amd import neural
+
+    def case(sequences, heads=128, page=64):
+        query_offsets, page_offsets, last, table, pages = [0], [0], [], [], 0
+        for queries, keys in sequences:
+            query_offsets.append(query_offsets[-1] + queries)
+            count = (keys + page - 1) // page
+            page_offsets.append(page_offsets[-1] + count)
+            last.append(keys - (count - 1) * page)
+            table += list(range(pages, pages + count))
+            pages += count
+        order = np.random.default_rng(7).permutation(pages)
+        table = [int(order[entry]) for entry in table]
+        gen = torch.Generator(device="cuda")
+        gen.manual_seed(11)
+        rand = lambda *shape: torch.randn(shape, generator=gen, device="cuda").to(torch.bfloat16)
+        tokens = query_offsets[-1]
+        operands = (rand(tokens, heads, 512), rand(tokens, heads, 64), rand(pages, page, 512), rand(pages, page, 64))
+        index = lambda values: torch.tensor(values, dtype=torch.int32, device="cuda")
+        paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
+        options = neural.AttentionOptions(causal=True)
+        launch = lambda: neural.paged_mla_attention(*operands, paging, options, check=False)
+        for _ in range(2):
+            launch()
+        torch.cuda.synchronize()
+        avg, median = time_launches(launch, steps, 2)
+        pairs = sum(sum(min(keys, max(keys - queries + i, 0) + 1) for i in range(queries)) for queries, keys in sequences)
+        flops = pairs * heads * (576 + 512) * 2
+        cache_bytes = sum(keys for _, keys in sequences) * 1152 + tokens * heads * (576 + 512) * 2
+        return avg, median, flops, cache_bytes
+
+    avg, median, flops, cache_bytes = case([(1, 4096)] * 256)
+    gbps, tflops = cache_bytes / (avg * 1e-3) / 1e9, flops / (avg * 1e-3) / 1e12
+    decode = {
+        "workload": "latent attention decode: 256 sequences x 4096 keys, 128 heads, latent 512 + positional 64, page 64, bf16",
+        "value": gbps, "unit": "GB/s", "tflops": tflops, "ms_per_step": avg, "ms_per_step_median": median,
+        "algorithmic_bytes": cache_bytes, "algorithmic_flops": flops,
+        "roofline": {"bound": "hbm", "kernel": "singe_paged_mla_attention_bf16_l512_p64", "achieved": gbps, "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": None, "mfma_frac": tflops / MFMA_BF16_PEAK_TFLOPS},
+    }
+    avg, median, flops, cache_bytes = case([(512, 8192)] * 8)
+    tflops = flops / (avg * 1e-3) / 1e12
+    chunked = {
+        "workload": "latent attention chunked prefill: 8 sequences x 512 new tokens on 8192 keys, 128 heads, latent 512 + "
+                    "positional 64, page 64, bf16",
+        "value": tflops, "unit": "TFLOP/s", "ms_per_step": avg, "ms_per_step_median": median, "algorithmic_flops": flops,
+        "roofline": {"bound": "mfma", "kernel": "singe_paged_mla_attention_bf16_l512_p64", "achieved": tflops,
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None},
+    }
+    return {"decode": decode, "chunked_prefill": chunked}
+
+
 def dense_f32_section(steps):
     """The first benchmark configuration, the f32 accuracy anchor: causal dense attention, batch 1, 8 heads,
     512 x 512, head_dim 64, scale 1/8, tensors [batch, heads, len, dim].  Far too small for a roofline: the
@@ -416,6 +476,8 @@ def main():
         result["fp8_decode"] = fp8_decode_section(10)
         torch.cuda.empty_cache()
         result["dense_f32"] = dense_f32_section(100)
+        torch.cuda.empty_cache()
+        result["latent"] = latent_section(8)
     print(json.dumps(result), flush=True)
 
 
