@@ -142,6 +142,29 @@ def test_key_splits_match_the_cpu_and_the_unsplit_kernel(splits, causal):
     assert np.abs(got_lse[~empty] - whole_lse.cpu().numpy()[~empty]).max() <= 2e-3
 
 
+@pytest.mark.parametrize("bad_page", [-1, 9])
+def test_matrix_core_kernel_reports_a_bad_page_and_leaves_other_sequences_right(bad_page):
+    """A page id outside the cache sets the status word (its keys are read as zeros); the other sequence's rows are
+    what they are without it."""
+    heads, page_size, pages = 16, 16, 9
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(5)
+    rand = lambda *shape: torch.randn(shape, generator=gen, device="cuda").to(torch.bfloat16)
+    device = [rand(3, heads, 512), rand(3, heads, 64), rand(pages, page_size, 512), rand(pages, page_size, 64)]
+    index = lambda entries: torch.tensor(entries, dtype=torch.int32, device="cuda")
+    good = neural.Paging(index([0, 1, 3]), index([0, 4, 8]), index([8, 0, 3, 5, 1, 2, 6, 7]), index([10, 16]))
+    bad = neural.Paging(index([0, 1, 3]), index([0, 4, 8]), index([8, 0, 3, 5, 1, bad_page, 6, 7]), index([10, 16]))
+    want, want_lse = neural.paged_mla_attention(*device, good, neural.AttentionOptions(causal=True))
+    with pytest.raises(error.IndexOutOfBounds):
+        neural.paged_mla_attention(*device, bad, neural.AttentionOptions(causal=True))
+    status = torch.zeros(1, device="cuda", dtype=torch.int32)
+    out, lse = neural.paged_mla_attention(*device, bad, neural.AttentionOptions(causal=True), status=status, check=False)
+    torch.cuda.synchronize()
+    assert int(status.item()) == 1
+    assert torch.equal(out[:1], want[:1]) and torch.equal(lse[:1], want_lse[:1])
+    assert torch.isfinite(out.float()).all()
+
+
 def test_default_scale_counts_the_whole_key_width_and_int64_indices():
     gen = torch.Generator(device="cuda")
     gen.manual_seed(1)
