@@ -251,6 +251,7 @@ struct LatentAttentionArgs {
     // normalised in partial_out [splits, tokens, heads, latent_dim] with a base-two log-sum-exp in partial_lse
     // [splits, tokens, heads] (-inf and zeros for a share without keys); singe_paged_mla_attention_combine_* merges.
     uint32_t splits;
+    int32_t page_shift;              // log2(page_size) when that is a power of two, else -1 (matrix-core kernel)
     float* partial_out;
     float* partial_lse;
 };

@@ -106,6 +106,9 @@ int32_t paged_mla_attention(void* stream, const void* latent_queries, const void
     const uint64_t blocks = tiles ? row_blocks + static_cast<uint64_t>(p.sequences) : row_blocks * static_cast<uint64_t>(p.sequences);
     if (blocks > 0x7fffffffull || row_blocks > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
     args.splits = 1;
+    args.page_shift = -1;
+    for (int shift = 0; shift < 31; ++shift)
+        if (p.page_size == (int64_t{1} << shift)) args.page_shift = shift;
     args.partial_out = nullptr;
     args.partial_lse = nullptr;
     if (tiles) {

@@ -210,13 +210,19 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
         const unsigned int key = tile * kKeys + row;
         return key < keys ? key : keys - 1u;  // rows past the end re-read the last key and are masked
     };
+    // A key's entry in the sequence's pages and its place in the page; a power-of-two page size takes the shift.
+    const int page_shift = a.page_shift;
+    auto entry_of = [&](unsigned int key) __attribute__((always_inline)) { return page_shift >= 0 ? key >> page_shift : key / a.page_size; };
+    auto place_of = [&](unsigned int key) __attribute__((always_inline)) {
+        return page_shift >= 0 ? key & (a.page_size - 1u) : key % a.page_size;
+    };
     auto lookup = [&](unsigned int tile) __attribute__((always_inline)) {
         TilePages<FORM> pages;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-            pages.latent[i] = read_raw_page_uniform<FORM>(a.pages, static_cast<size_t>(span.page_start) + key_of(tile, wave + 8u * i) / a.page_size);
+            pages.latent[i] = read_raw_page_uniform<FORM>(a.pages, static_cast<size_t>(span.page_start) + entry_of(key_of(tile, wave + 8u * i)));
         pages.positional = 0;
-        if (wave < 4) pages.positional = read_raw_page<FORM>(a.pages, static_cast<size_t>(span.page_start) + key_of(tile, positional_row) / a.page_size);
+        if (wave < 4) pages.positional = read_raw_page<FORM>(a.pages, static_cast<size_t>(span.page_start) + entry_of(key_of(tile, positional_row)));
         return pages;
     };
     // A key behind a bad page id is read as zeros; the status word tells the caller.
@@ -227,7 +233,7 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
             const unsigned long long page = static_cast<unsigned long long>(pages.latent[i]);
             unsigned char* dest = stage + row * kLatentRowBytes;
             if (page < static_cast<unsigned long long>(a.cache_pages)) {
-                const size_t slot = static_cast<size_t>(page) * a.page_size + key_of(tile, row) % a.page_size;
+                const size_t slot = static_cast<size_t>(page) * a.page_size + place_of(key_of(tile, row));
                 const unsigned char* source = latent_cache + slot * kLatentRowBytes + 16u * (lane ^ chunk_flip(row & 15u));
                 load_to_lds(source, dest);
             } else {
@@ -239,7 +245,7 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
             const unsigned long long page = static_cast<unsigned long long>(pages.positional);
             unsigned char* dest = stage + kLatentTileBytes + 8u * wave * kPositionalRowBytes;
             if (page < static_cast<unsigned long long>(a.cache_pages)) {
-                const size_t slot = static_cast<size_t>(page) * a.page_size + key_of(tile, positional_row) % a.page_size;
+                const size_t slot = static_cast<size_t>(page) * a.page_size + place_of(key_of(tile, positional_row));
                 const unsigned char* source = positional_cache + slot * kPositionalRowBytes + 16u * ((lane & 7u) ^ (positional_row & 7u));
                 load_to_lds(source, dest);
             } else {
@@ -314,8 +320,7 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
                 x[4 * t + r] = value;
             }
         float largest = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
-        largest = fmaxf(largest, __shfl_xor(largest, 16, 64));
-        largest = fmaxf(largest, __shfl_xor(largest, 32, 64));  // the four lanes of a row agree from here on
+        largest = across_groups_max(largest);  // the four lanes of a row agree from here on
         if (__any(largest > reference + kMaxLag || (reference == -INFINITY && largest != -INFINITY))) {
             const float moved = fmaxf(reference, largest);
             const float base = moved == -INFINITY ? 0.0f : moved;
@@ -375,9 +380,7 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
     }
 
     // Normalise and store; a row that sees no key stays zero and has a log-sum-exp of -inf.
-    float sum = running_sum;
-    sum += __shfl_xor(sum, 16, 64);
-    sum += __shfl_xor(sum, 32, 64);
+    const float sum = across_groups_sum(running_sum);
     const float inverse = sum > 0.0f ? 1.0f / sum : 0.0f;
     if (row_valid && splits > 1) {
         const size_t slot = static_cast<size_t>(split) * a.tokens * a.heads + flat;

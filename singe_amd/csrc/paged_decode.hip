@@ -231,36 +231,6 @@ SINGE_DEVICE void load_tile(KeyTileFp8& tile, const DecodeArgs& a, const unsigne
     }
 }
 
-// v_permlane16_swap / v_permlane32_swap of a value with a copy of itself: `kept` keeps its even rows
-// (its low half for 32) and takes the neighbour's, `taken` the other way round, so kept (op) taken
-// combines a lane with its partner 16 (32) lanes away.  Written as inline assembly because the
-// compiler's builtin returns the first result twice; the s_nop covers the VALU-write hazard the
-// compiler would otherwise pad.
-template <int ROWS>
-SINGE_DEVICE void swap_with_self(float value, float& kept, float& taken) {
-    kept = value;
-    taken = value;
-    if constexpr (ROWS == 16)
-        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(kept), "+v"(taken));
-    else
-        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(kept), "+v"(taken));
-}
-
-// max / sum over the four 16-lane groups of a wave: lanes l, l^16, l^32, l^48 end up equal.
-SINGE_DEVICE float across_groups_max(float value) {
-    float a, b;
-    swap_with_self<16>(value, a, b);
-    swap_with_self<32>(fmaxf(a, b), a, b);
-    return fmaxf(a, b);
-}
-
-SINGE_DEVICE float across_groups_sum(float value) {
-    float a, b;
-    swap_with_self<16>(value, a, b);
-    swap_with_self<32>(a + b, a, b);
-    return a + b;
-}
-
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
 typedef short i16x4_t __attribute__((ext_vector_type(4)));
