@@ -226,9 +226,12 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
         return pages;
     };
     // A key behind a bad page id is read as zeros; the status word tells the caller.
-    auto issue = [&](unsigned int tile, const TilePages<FORM>& pages, unsigned char* __restrict__ stage) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
+    // In pieces, so that a tile's iteration can spread them between its first score products: piece 0-3 one latent
+    // row each, piece 4 the positional parts.
+    auto issue_piece = [&](int piece, unsigned int tile, const TilePages<FORM>& pages, unsigned char* __restrict__ stage)
+                           __attribute__((always_inline)) {
+        if (piece < 4) {
+            const int i = piece;
             const unsigned int row = wave + 8u * i;
             const unsigned long long page = static_cast<unsigned long long>(pages.latent[i]);
             unsigned char* dest = stage + row * kLatentRowBytes;
@@ -240,8 +243,7 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
                 if (lane == 0) report_index_error(a.status);
                 *reinterpret_cast<uint4*>(dest + 16u * lane) = make_uint4(0, 0, 0, 0);
             }
-        }
-        if (wave < 4) {
+        } else if (wave < 4) {
             const unsigned long long page = static_cast<unsigned long long>(pages.positional);
             unsigned char* dest = stage + kLatentTileBytes + 8u * wave * kPositionalRowBytes;
             if (page < static_cast<unsigned long long>(a.cache_pages)) {
@@ -253,6 +255,11 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
                 *reinterpret_cast<uint4*>(dest + 16u * lane) = make_uint4(0, 0, 0, 0);
             }
         }
+    };
+
+    auto issue = [&](unsigned int tile, const TilePages<FORM>& pages, unsigned char* __restrict__ stage) __attribute__((always_inline)) {
+#pragma unroll
+        for (int piece = 0; piece < 5; ++piece) issue_piece(piece, tile, pages, stage);
     };
 
     // Read offsets.  Score operand of step s, 16-key half t: row 16 t + column, chunk (4 s + g) ^ flip.  Transposed
@@ -281,7 +288,7 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
     float reference = -INFINITY, running_sum = 0.0f;  // the sum of this lane's keys only
     const float scale_log2e = a.scale * kLog2e;
 
-    auto fold = [&](unsigned int tile, const unsigned char* __restrict__ stage) __attribute__((always_inline)) {
+    auto fold = [&](unsigned int tile, const unsigned char* __restrict__ stage, auto&& between) __attribute__((always_inline)) {
         const unsigned int key0 = tile * kKeys;
         f32x4_t s[2] = {f32x4_t{0.0f, 0.0f, 0.0f, 0.0f}, f32x4_t{0.0f, 0.0f, 0.0f, 0.0f}};
         // The operands of a step are read a step before its products (two sets taking turns), and the order is
@@ -303,6 +310,7 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
             const uint4 mine = step < kParkedSteps ? parked_q[step % 2] : q[step < kParkedSteps ? 0 : step - kParkedSteps];
             s[0] = mma(half, operand[step % 2][0], mine, s[0]);
             s[1] = mma(half, operand[step % 2][1], mine, s[1]);
+            between(step);  // the caller's paging arithmetic and loads, while the products run
             __builtin_amdgcn_sched_barrier(0);
         }
         // Register r of half t is key key0 + 16 t + 4 g + r against the lane's row.
@@ -371,9 +379,21 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
         for (unsigned int tile = first_tile; tile < tiles; ++tile) {
             unsigned char* stage = lds + (tile & 1u) * kStageBytes;
             unsigned char* other = lds + ((tile & 1u) ^ 1u) * kStageBytes;
-            if (tile + 1 < tiles) issue(tile + 1, pages, other);
-            if (tile + 2 < tiles) pages = lookup(tile + 2);
-            if (tile * kKeys < wave_end) fold(tile, stage);
+            // The next tile's loads go out one piece after each of the first score steps, the page ids of the tile
+            // after it once those have been used: address arithmetic in the shadow of the products.
+            auto between = [&](int step) __attribute__((always_inline)) {
+                if (step < 5) {
+                    if (tile + 1 < tiles) issue_piece(step, tile + 1, pages, other);
+                } else if (step == 6) {
+                    if (tile + 2 < tiles) pages = lookup(tile + 2);
+                }
+            };
+            if (tile * kKeys < wave_end) {
+                fold(tile, stage, between);
+            } else {
+#pragma unroll
+                for (int step = 0; step < 7; ++step) between(step);
+            }
             __builtin_amdgcn_s_waitcnt(0x0F70);  // this wave's loads have landed
             __syncthreads();                     // and everyone has finished reading
         }
