@@ -31,6 +31,10 @@ if ROOT not in sys.path:
 DECODE_TRAFFIC_BYTES = (145766 * 2 + 4552) * 1024
 # The same for the dense prefill kernel at batch 4 x seq 4096 x 32 heads: FETCH_SIZE 301283, WRITE_SIZE 131377.
 PREFILL_TRAFFIC_BYTES = (311083 * 2 + 132590) * 1024
+# The same for the latent attention kernel at its two workloads (--only-latent under rocprofv3 --pmc): decode
+# FETCH_SIZE 608520, WRITE_SIZE 33047; chunked prefill FETCH_SIZE 1376200, WRITE_SIZE 526390.
+LATENT_DECODE_TRAFFIC_BYTES = (608520 * 2 + 33047) * 1024
+LATENT_CHUNKED_TRAFFIC_BYTES = (1376200 * 2 + 526390) * 1024
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 POOLS = 3
@@ -46,6 +50,8 @@ def parse():
     parser.add_argument("--no-extras", action="store_true", help="skip the chunked-prefill and fp8-decode measurements")
     parser.add_argument("--prefill-steps", type=int, default=40)
     parser.add_argument("--workers", type=int, default=0, help="tuning override (0 = built-in choice)")
+    parser.add_argument("--only-latent", action="store_true",
+                        help="run the latent attention section alone and print it (for counter runs of its kernel)")
     return parser.parse_args()
 
 
@@ -267,7 +273,8 @@ def latent_section(steps):
         "value": gbps, "unit": "GB/s", "tflops": tflops, "ms_per_step": avg, "ms_per_step_median": median,
         "algorithmic_bytes": cache_bytes, "algorithmic_flops": flops,
         "roofline": {"bound": "hbm", "kernel": "singe_paged_mla_attention_bf16_l512_p64", "achieved": gbps, "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": None, "mfma_frac": tflops / MFMA_BF16_PEAK_TFLOPS},
+                     "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": LATENT_DECODE_TRAFFIC_BYTES,
+                     "mfma_frac": tflops / MFMA_BF16_PEAK_TFLOPS},
     }
     avg, median, flops, cache_bytes = case([(512, 8192)] * 8)
     tflops = flops / (avg * 1e-3) / 1e12
@@ -276,7 +283,8 @@ def latent_section(steps):
                     "positional 64, page 64, bf16",
         "value": tflops, "unit": "TFLOP/s", "ms_per_step": avg, "ms_per_step_median": median, "algorithmic_flops": flops,
         "roofline": {"bound": "mfma", "kernel": "singe_paged_mla_attention_bf16_l512_p64", "achieved": tflops,
-                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS, "traffic": None},
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
+                     "traffic": LATENT_CHUNKED_TRAFFIC_BYTES},
     }
     return {"decode": decode, "chunked_prefill": chunked}
 
@@ -373,6 +381,9 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
+    if args.only_latent:
+        print(json.dumps({"latent": latent_section(4)}), flush=True)
+        return
     if args.workers:
         _native.lib().singe_hip_set_decode_workers(args.workers)
 
