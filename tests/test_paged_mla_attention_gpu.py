@@ -97,9 +97,10 @@ def test_matrix_core_shape_on_random_data(heads, page_size, index_dtype, causal,
     assert np.abs(got_lse[~empty] - want_lse[~empty]).max() <= 5e-3
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("splits", [2, 3, 16, 64])
 @pytest.mark.parametrize("causal", [False, True])
-def test_key_splits_match_the_cpu_and_the_unsplit_kernel(splits, causal):
+def test_key_splits_match_the_cpu_and_the_unsplit_kernel(splits, causal, dtype):
     """With scratch lent, a row tile's keys are shared out over workgroups and merged by a second kernel: decode rows
     over long and short caches, a chunk, a sequence without keys, more shares than a sequence has tiles."""
     import ctypes
@@ -117,7 +118,7 @@ def test_key_splits_match_the_cpu_and_the_unsplit_kernel(splits, causal):
     tokens = query_offsets[-1]
     gen = torch.Generator(device="cuda")
     gen.manual_seed(splits)
-    rand = lambda *shape: torch.randn(shape, generator=gen, device="cuda").to(torch.bfloat16)
+    rand = lambda *shape: torch.randn(shape, generator=gen, device="cuda").to(dtype)
     device = [rand(tokens, heads, 512), rand(tokens, heads, 64), rand(needed + 2, page_size, 512), rand(needed + 2, page_size, 64)]
     index = lambda entries: torch.tensor(entries, dtype=torch.int32, device="cuda")
     paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
