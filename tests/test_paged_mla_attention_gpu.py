@@ -166,6 +166,45 @@ def test_matrix_core_kernel_reports_a_bad_page_and_leaves_other_sequences_right(
     assert torch.isfinite(out.float()).all()
 
 
+def test_decode_at_full_size_splits_on_its_own_and_agrees_with_the_unsplit_kernel_and_a_torch_reference():
+    """64 sequences of 2048 to 4096 keys, 128 heads: too large for the CPU oracle in a test, so the split and unsplit
+    kernels are held to each other and to a plain torch f32 evaluation of the same rows on the device."""
+    import ctypes
+    heads, page_size = 128, 64
+    rng = np.random.default_rng(3)
+    lengths = [int(n) for n in rng.integers(2048, 4097, size=64)]
+    query_offsets, page_offsets, last, needed = list(range(65)), [0], [], 0
+    for keys in lengths:
+        pages = (keys + page_size - 1) // page_size
+        needed += pages
+        page_offsets.append(needed)
+        last.append(keys - (pages - 1) * page_size)
+    table = [int(page) for page in rng.permutation(needed)]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(13)
+    rand = lambda *shape: torch.randn(shape, generator=gen, device="cuda").to(torch.bfloat16)
+    q, qp, lc, pc = rand(64, heads, 512), rand(64, heads, 64), rand(needed, page_size, 512), rand(needed, page_size, 64)
+    index = lambda entries: torch.tensor(entries, dtype=torch.int32, device="cuda")
+    paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
+    options = neural.AttentionOptions(causal=True)
+    whole, whole_lse = neural.paged_mla_attention(q, qp, lc, pc, paging, options, scratch=False)
+    out, lse = neural.paged_mla_attention(q, qp, lc, pc, paging, options)  # 64 workgroups for 256 compute units: it splits
+    assert (out.float() - whole.float()).abs().max().item() <= 1e-2
+    assert (lse - whole_lse).abs().max().item() <= 1e-3
+    scale = 1.0 / np.sqrt(576.0)
+    for sequence in (0, 31, 63):
+        pages = torch.tensor(table[page_offsets[sequence]:page_offsets[sequence + 1]], device="cuda")
+        keys = lengths[sequence]
+        latent = lc[pages].reshape(-1, 512)[:keys].float()
+        positional = pc[pages].reshape(-1, 64)[:keys].float()
+        scores = (q[sequence].float() @ latent.T + qp[sequence].float() @ positional.T) * scale
+        want = torch.softmax(scores, dim=-1) @ latent
+        gap = (out[sequence].float() - want).abs()
+        assert gap.max().item() <= 2e-2 and gap.mean().item() <= 2e-3
+        want_lse = torch.logsumexp(scores, dim=-1) / np.log(2.0)
+        assert (lse[sequence] - want_lse).abs().max().item() <= 5e-3
+
+
 def test_default_scale_counts_the_whole_key_width_and_int64_indices():
     gen = torch.Generator(device="cuda")
     gen.manual_seed(1)
