@@ -123,6 +123,26 @@ SINGE_HIP_API int32_t singe_hip_paged_kv_decode_attention_f16(
     void* workspace, size_t workspace_bytes,
     const SingePagedKvDecodeAttentionConfig* config);
 
+/* The bf16 decode above for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference: its split-KV scratch is always the
+ * caller's.  Same kernels, same results bit for bit, but the scratch is a fixed array of
+ * SINGE_HIP_STATIC_SCRATCH_BYTES in device memory that the library's device image carries (each GPU the library
+ * runs on holds it until the process ends); the call allocates and frees nothing.  A config whose scratch
+ * (..._workspace_bytes) exceeds that returns SINGE_HIP_LENGTH_TOO_SHORT naming "static scratch" (minimum = bytes
+ * needed, actual = the fixed size).  The array's address is resolved on the first call on a device (or by
+ * singe_hip_prepare), which must not run under stream capture.  All calls on a GPU share the one array, which keeps
+ * the last call's contents (the kernels need none of it cleared): calls that overlap on one GPU race. */
+#define SINGE_HIP_STATIC_SCRATCH_BYTES (16u << 20)
+SINGE_HIP_API int32_t singe_hip_paged_kv_decode_attention_no_alloc_bf16(
+    void* stream,
+    uint16_t* out, size_t out_len,
+    const uint16_t* query, size_t query_len,
+    const uint16_t* key_cache, size_t key_cache_len,
+    const uint16_t* value_cache, size_t value_cache_len,
+    const int32_t* actual_seq_lens, size_t actual_seq_lens_len,
+    const uint32_t* block_table, size_t block_table_len,
+    const SingePagedKvDecodeAttentionConfig* config);
+
 /* The same operation run phase by phase, as the reference exposes its split kernel and splitk_reduce
  * separately (singe-kernel/src/cuda/attention/fmha.rs:1038,1155): SPLIT fills the scratch with the
  * normalised partial rows and natural-log LSEs of every key range; REDUCE folds the scratch into

@@ -157,6 +157,9 @@ def lib() -> ctypes.CDLL:
         c_void, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size,
         c_void, c_size, cfg]
     handle.singe_hip_paged_kv_decode_attention_bf16.restype = i32
+    handle.singe_hip_paged_kv_decode_attention_no_alloc_bf16.argtypes = [
+        c_void, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size, c_void, c_size, cfg]
+    handle.singe_hip_paged_kv_decode_attention_no_alloc_bf16.restype = i32
     handle.singe_hip_paged_kv_decode_attention_f16.argtypes = handle.singe_hip_paged_kv_decode_attention_bf16.argtypes
     handle.singe_hip_paged_kv_decode_attention_f16.restype = i32
     handle.singe_hip_paged_kv_decode_attention_phases_bf16.argtypes = [

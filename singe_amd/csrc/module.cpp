@@ -9,6 +9,7 @@
 #include <vector>
 
 #include "singe_hip_attention.h"
+#include "static_scratch.h"
 
 namespace singe_hip {
 
@@ -234,6 +235,10 @@ int32_t singe_hip_prepare(int32_t* count) {
         if (int32_t status = kernel_function(static_cast<KernelId>(kernel), &function)) return status;
         ++found;
     }
+    // The fixed scratch of the entry points that allocate nothing: resolve its address on this device now.
+    void* scratch = nullptr;
+    size_t scratch_bytes = 0;
+    if (int status = static_scratch(&scratch, &scratch_bytes)) return fail(status, "hipGetSymbolAddress(static scratch)");
     if (count != nullptr) *count = found;
     return 0;
 }

@@ -7,6 +7,7 @@
 #include "kernel_args.h"
 #include "module.h"
 #include "singe_hip_attention.h"
+#include "static_scratch.h"
 #include "validate.h"
 
 using namespace singe_hip;
@@ -124,6 +125,25 @@ int32_t singe_hip_paged_kv_decode_attention_phases_bf16(
     return decode(stream, out, out_len, query, query_len, key_cache, key_cache_len, value_cache, value_cache_len,
                   nullptr, 0, nullptr, 0, false, actual_seq_lens, actual_seq_lens_len, block_table, block_table_len,
                   workspace, workspace_bytes, config, phases);
+}
+
+// The bf16 decode on the library's fixed device scratch: allocates nothing (no counterpart in the reference).
+int32_t singe_hip_paged_kv_decode_attention_no_alloc_bf16(
+    void* stream, uint16_t* out, size_t out_len, const uint16_t* query, size_t query_len,
+    const uint16_t* key_cache, size_t key_cache_len, const uint16_t* value_cache, size_t value_cache_len,
+    const int32_t* actual_seq_lens, size_t actual_seq_lens_len, const uint32_t* block_table,
+    size_t block_table_len, const SingePagedKvDecodeAttentionConfig* config) {
+    if (config == nullptr) return fail(SINGE_HIP_NULL_POINTER, "config");
+    if (int32_t status = validate_config(*config)) return status;
+    const size_t need = make_plan(*config).bytes;
+    if (need > SINGE_HIP_STATIC_SCRATCH_BYTES)
+        return fail(SINGE_HIP_LENGTH_TOO_SHORT, "static scratch", need, SINGE_HIP_STATIC_SCRATCH_BYTES);
+    void* scratch = nullptr;
+    size_t scratch_bytes = 0;
+    if (int status = static_scratch(&scratch, &scratch_bytes)) return fail(status, "hipGetSymbolAddress(static scratch)");
+    return decode(stream, out, out_len, query, query_len, key_cache, key_cache_len, value_cache, value_cache_len,
+                  nullptr, 0, nullptr, 0, false, actual_seq_lens, actual_seq_lens_len, block_table, block_table_len,
+                  scratch, scratch_bytes, config, SINGE_HIP_DECODE_SPLIT | SINGE_HIP_DECODE_REDUCE);
 }
 
 // paged_kv_decode_attention_f16 (singe-kernel/src/cuda/attention/paged.rs): the bf16 kernels on f16 operands.

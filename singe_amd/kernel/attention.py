@@ -130,6 +130,31 @@ def paged_kv_decode_attention_bf16(stream, out: torch.Tensor, query: torch.Tenso
     _native.check(status, "paged_kv_decode_attention_bf16")
 
 
+STATIC_SCRATCH_BYTES = 16 << 20
+
+
+def paged_kv_decode_attention_no_alloc_bf16(stream, out: torch.Tensor, query: torch.Tensor, key_cache: torch.Tensor,
+                                            value_cache: torch.Tensor, actual_seq_lens: torch.Tensor,
+                                            block_table: torch.Tensor, config: PagedKvDecodeAttentionConfig) -> None:
+    """paged_kv_decode_attention_bf16 on the library's fixed device scratch (STATIC_SCRATCH_BYTES per GPU): neither
+    this wrapper nor the library allocates, for callers that cannot (graph capture, serving loops).  Calls that
+    overlap on one GPU share the scratch and race.  No counterpart in the reference."""
+    _require(out, torch.bfloat16, "out")
+    _require(query, torch.bfloat16, "query")
+    _require(key_cache, torch.bfloat16, "key_cache")
+    _require(value_cache, torch.bfloat16, "value_cache")
+    _require(actual_seq_lens, torch.int32, "actual_seq_lens")
+    if block_table.dtype not in (torch.int32, torch.uint32):
+        raise error.InvalidArgument(f"block_table must hold 32-bit entries, got {block_table.dtype}")
+    _require(block_table, block_table.dtype, "block_table")
+    c = config._c()
+    status = _native.lib().singe_hip_paged_kv_decode_attention_no_alloc_bf16(
+        _stream_handle(stream), _ptr(out), out.numel(), _ptr(query), query.numel(), _ptr(key_cache),
+        key_cache.numel(), _ptr(value_cache), value_cache.numel(), _ptr(actual_seq_lens),
+        actual_seq_lens.numel(), _ptr(block_table), block_table.numel(), ctypes.byref(c))
+    _native.check(status, "paged_kv_decode_attention_no_alloc_bf16")
+
+
 def paged_kv_decode_attention_f8e4m3kv_bf16(stream, out: torch.Tensor, query: torch.Tensor, key_cache: torch.Tensor,
                                             value_cache: torch.Tensor, key_scales: torch.Tensor,
                                             value_scales: torch.Tensor, actual_seq_lens: torch.Tensor,
