@@ -8,7 +8,7 @@
  * asynchronously, so every call is legal during stream capture
  * (raw kernel execution contract: singe-kernel/src/cuda/mod.rs:3-12).
  *
- * The kernels live in a gfx950 code object (singe_attention_gfx950.hsaco, built by hipcc --genco)
+ * The kernels live in a gfx950 code object built in parts (singe_attention_gfx950.<part>.hsaco, hipcc --genco)
  * that this library loads with hipModuleLoadData and launches with hipModuleLaunchKernel, in place of
  * the reference's NVRTC -> cuModuleLoadData -> cuLaunchKernelEx path
  * (singe/src/backend/cuda/codegen/compile.rs:43-190, singe-cuda/src/module/mod.rs:2117-2132).
@@ -63,13 +63,20 @@ SINGE_HIP_API const char* singe_hip_status_string(int32_t status);
  * Replaces Context::load_module / Module::function (singe-cuda/src/context.rs:363-385,
  * singe-cuda/src/module/mod.rs:387-410).  An image is a gfx950 code object or a clang offload bundle
  * holding one.  Loading is per process; the module is instantiated lazily on each device that
- * launches.  Without an explicit load the library looks for singe_attention_gfx950.hsaco next to
- * itself.  The image bytes are copied. */
+ * launches.  Without an explicit load the library looks for the parts, singe_attention_gfx950.<part>.hsaco,
+ * next to itself and loads a part when a kernel of it is first launched; an image handed to singe_hip_load holds
+ * every kernel.  The image bytes are copied.  Launches read their kernel handle without a lock once it has been
+ * resolved on their device (the first launch of a kernel there, or singe_hip_prepare, takes a mutex), so load and
+ * unload must not run while another thread launches. */
 SINGE_HIP_API int32_t singe_hip_load(const void* image, size_t bytes);
 SINGE_HIP_API int32_t singe_hip_load_file(const char* path);
 SINGE_HIP_API void singe_hip_unload(void);
 /* Resolves every kernel of the image on the current device; returns the number found through *count. */
 SINGE_HIP_API int32_t singe_hip_prepare(int32_t* count);
+/* The kernels the library launches, as profilers report them (the reference names its artifacts the same way,
+ * singe/src/backend/cuda/kernel_plan/source/mod.rs:841-853), and the part of the code object each one is loaded from
+ * (singe_attention_gfx950.<part>.hsaco).  index from 0; SINGE_HIP_INVALID_ARGUMENT past the last kernel. */
+SINGE_HIP_API int32_t singe_hip_kernel(int32_t index, const char** name, const char** part);
 
 /* ---- singe-kernel surface: paged decode ---------------------------------------------------------
  * Mirrors PagedKvDecodeAttentionConfig (singe-kernel/src/cuda/attention/mod.rs:76-90). */

@@ -9,7 +9,10 @@ from . import error
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIBRARY_PATH = os.path.join(_HERE, "libsinge_hip_attention.so")
-CODE_OBJECT_PATH = os.path.join(_HERE, "singe_attention_gfx950.hsaco")
+CODE_OBJECT_PARTS = ("paged_decode", "fmha_prefill", "fmha_prefill_f32", "paged_attention", "splitk_reduce",
+                     "attention_rows_f32", "cache_ops", "latent_attention", "latent_attention_mfma",
+                     "general_attention_f32", "general_attention_bf16", "general_attention_f16")
+CODE_OBJECT_PATHS = [os.path.join(_HERE, f"singe_attention_gfx950.{part}.hsaco") for part in CODE_OBJECT_PARTS]
 
 c_size = ctypes.c_size_t
 c_void = ctypes.c_void_p
@@ -146,6 +149,8 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_load_file.restype = i32
     handle.singe_hip_unload.argtypes = []
     handle.singe_hip_unload.restype = None
+    handle.singe_hip_kernel.argtypes = [i32, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(ctypes.c_char_p)]
+    handle.singe_hip_kernel.restype = i32
     handle.singe_hip_prepare.argtypes = [ctypes.POINTER(i32)]
     handle.singe_hip_prepare.restype = i32
     cfg = ctypes.POINTER(PagedKvDecodeAttentionConfigC)

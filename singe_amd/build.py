@@ -1,22 +1,26 @@
-"""Builds the two native artefacts in-tree:
+"""Builds the native artefacts in-tree:
 
-* ``singe_attention_gfx950.hsaco``: the gfx950 code object (hipcc --genco), and
+* ``singe_attention_gfx950.<part>.hsaco``: the gfx950 code object, one part per kernel source (hipcc --genco), built
+  side by side, and
 * ``libsinge_hip_attention.so``: the C-ABI launcher (plain g++; it resolves the HIP runtime with dlopen, and
   links it only for the one hipcc-built unit that holds the fixed device scratch).
 
-Run as ``python -m singe_amd.build``.  hipcc cross-compiles, so no GPU is needed.
+Run as ``python -m singe_amd.build`` (everything) or ``python -m singe_amd.build --changed`` (only the parts whose
+sources changed since they were last built).  hipcc cross-compiles, so no GPU is needed.
 """
 from __future__ import annotations
 
+import hashlib
 import os
+import re
 import shutil
 import subprocess
 import sys
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
-CODE_OBJECT = os.path.join(HERE, "singe_attention_gfx950.hsaco")
 LIBRARY = os.path.join(HERE, "libsinge_hip_attention.so")
 STATIC_SCRATCH_OBJECT = os.path.join(HERE, "csrc", "static_scratch.o")
 
@@ -26,8 +30,31 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",
 ]
+# (part name, source file, extra flags), in the order of kPartNames in csrc/module.cpp.
+PARTS = [
+    ("paged_decode", "paged_decode.hip", []),
+    ("fmha_prefill", "fmha_prefill.hip", []),
+    ("fmha_prefill_f32", "fmha_prefill_f32.hip", []),
+    ("paged_attention", "paged_attention.hip", []),
+    ("splitk_reduce", "splitk_reduce.hip", []),
+    ("attention_rows_f32", "attention_rows_f32.hip", []),
+    ("cache_ops", "cache_ops.hip", []),
+    ("latent_attention", "latent_attention.hip", []),
+    ("latent_attention_mfma", "latent_attention_mfma.hip", []),
+    ("general_attention_f32", "general_attention.hip", ["-DSINGE_GENERAL_ELEMENT=0"]),
+    ("general_attention_bf16", "general_attention.hip", ["-DSINGE_GENERAL_ELEMENT=1"]),
+    ("general_attention_f16", "general_attention.hip", ["-DSINGE_GENERAL_ELEMENT=2"]),
+]
 HOST_SOURCES = ["hip_runtime_loader.cpp", "module.cpp", "paged_decode.cpp", "fmha_prefill.cpp", "paged_attention.cpp",
                 "general_attention.cpp", "fmha_decode.cpp", "paged_rows_f32.cpp", "latent_attention.cpp", "cache_ops.cpp"]
+JOBS = 8
+
+
+def code_object(part: str) -> str:
+    return os.path.join(HERE, f"singe_attention_gfx950.{part}.hsaco")
+
+
+CODE_OBJECTS = [code_object(part) for part, _, _ in PARTS]
 
 
 def _run(cmd):
@@ -42,10 +69,40 @@ def hipcc() -> str:
     return found
 
 
-def build_code_object(extra_flags=()) -> str:
-    source = os.path.join(CSRC, "singe_attention_kernels.hip")
-    _run([hipcc(), *HIPCC_FLAGS, *extra_flags, "-I", CSRC, source, "-o", CODE_OBJECT])
-    return CODE_OBJECT
+def _closure(source: str, seen=None) -> list:
+    """The source and every header of this directory it includes, directly or not."""
+    seen = seen if seen is not None else []
+    path = os.path.join(CSRC, source)
+    if path in seen or not os.path.exists(path):
+        return seen
+    seen.append(path)
+    for name in re.findall(r'#include "([^"]+)"', open(path).read()):
+        _closure(name, seen)
+    return seen
+
+
+def _fingerprint(source: str, flags) -> str:
+    digest = hashlib.sha256(" ".join([*HIPCC_FLAGS, *flags]).encode())
+    for path in sorted(_closure(source)):
+        digest.update(open(path, "rb").read())
+    return digest.hexdigest()
+
+
+def build_part(part: str, source: str, flags, only_changed: bool = False) -> str:
+    target, stamp = code_object(part), code_object(part) + ".stamp"
+    fingerprint = _fingerprint(source, flags)
+    if only_changed and os.path.exists(target) and os.path.exists(stamp) and open(stamp).read() == fingerprint:
+        return target
+    _run([hipcc(), *HIPCC_FLAGS, *flags, "-I", CSRC, os.path.join(CSRC, source), "-o", target])
+    with open(stamp, "w") as handle:
+        handle.write(fingerprint)
+    return target
+
+
+def build_code_object(only_changed: bool = False, parts=None) -> list:
+    wanted = [entry for entry in PARTS if parts is None or entry[0] in parts]
+    with ThreadPoolExecutor(max_workers=JOBS) as pool:
+        return list(pool.map(lambda entry: build_part(*entry, only_changed=only_changed), wanted))
 
 
 def rocm_lib_dir() -> str:
@@ -72,11 +129,11 @@ def build_library() -> str:
     return LIBRARY
 
 
-def build() -> None:
-    build_code_object()
+def build(only_changed: bool = False) -> None:
+    build_code_object(only_changed=only_changed)
     build_library()
 
 
 if __name__ == "__main__":
-    build()
+    build(only_changed="--changed" in sys.argv[1:])
     sys.exit(0)

@@ -221,12 +221,21 @@ SINGE_DEVICE void paged_body(const GeneralPagedArgs& a, float* lds) {
         general::paged_body<ELEMENT, DMAX>(args, rows);                                                                      \
     }
 
+// The build compiles this file once per element type (SINGE_GENERAL_ELEMENT = 0 f32, 1 bf16, 2 f16), each into its
+// own part of the code object.
+#ifndef SINGE_GENERAL_ELEMENT
+#error "define SINGE_GENERAL_ELEMENT: 0 (f32), 1 (bf16) or 2 (f16)"
+#endif
+#if SINGE_GENERAL_ELEMENT == 0
 SINGE_GENERAL_KERNELS(f32, kElementF32, 64)
 SINGE_GENERAL_KERNELS(f32, kElementF32, 128)
 SINGE_GENERAL_KERNELS(f32, kElementF32, 256)
+#elif SINGE_GENERAL_ELEMENT == 1
 SINGE_GENERAL_KERNELS(bf16, kElementBf16, 64)
 SINGE_GENERAL_KERNELS(bf16, kElementBf16, 128)
 SINGE_GENERAL_KERNELS(bf16, kElementBf16, 256)
+#else
 SINGE_GENERAL_KERNELS(f16, kElementF16, 64)
 SINGE_GENERAL_KERNELS(f16, kElementF16, 128)
 SINGE_GENERAL_KERNELS(f16, kElementF16, 256)
+#endif

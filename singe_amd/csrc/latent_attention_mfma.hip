@@ -68,7 +68,11 @@ SINGE_DEVICE f32x4_t mma(F16, uint4 a, uint4 b, f32x4_t c) {
 // vmcnt(0) before the barrier that hands a stage on.
 SINGE_DEVICE void load_to_lds(const unsigned char* source, unsigned char* dest) {
     const unsigned int base = __builtin_amdgcn_readfirstlane(static_cast<unsigned int>(reinterpret_cast<__UINTPTR_TYPE__>((lds_words_t)dest)));
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(base), "v"(source) : "memory");
+    // M0 carries the LDS base of the load; it is read when the load issues, so the statement puts back what M0 held
+    // and the compiler's own uses of M0 around it are not disturbed.
+    unsigned int kept;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
+                 : "=&s"(kept) : "s"(base), "v"(source) : "memory");
 }
 
 // Where the chunk permutation of a latent row puts things: see the header comment.

@@ -2,6 +2,7 @@
 
 #include <dlfcn.h>
 
+#include <atomic>
 #include <cstdio>
 #include <cstring>
 #include <mutex>
@@ -67,29 +68,68 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_attention_general_f16_d64", "singe_paged_attention_general_f16_d128", "singe_paged_attention_general_f16_d256",
 };
 
+// The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
+// the parts it launches from): singe_attention_gfx950.<part>.hsaco next to the library.  kKernelNames is grouped by
+// part; kPartRuns gives the part of each run of consecutive kernels.
+const char* const kPartNames[kPartCount] = {
+    "paged_decode", "fmha_prefill", "fmha_prefill_f32", "paged_attention", "splitk_reduce", "attention_rows_f32",
+    "cache_ops", "latent_attention", "latent_attention_mfma", "general_attention_f32", "general_attention_bf16",
+    "general_attention_f16",
+};
+
+namespace {
+
+struct PartRun {
+    int part, kernels;
+};
+constexpr PartRun kPartRuns[] = {
+    {0, 14}, {1, 8}, {2, 4}, {3, 28}, {4, 1}, {5, 28}, {6, 5}, {7, 3}, {8, 4},
+    {9, 3}, {10, 3}, {11, 3},  // dense general kernels: f32, bf16, f16
+    {9, 3}, {10, 3}, {11, 3},  // paged general kernels
+};
+constexpr int runs_total() {
+    int total = 0;
+    for (const PartRun& run : kPartRuns) total += run.kernels;
+    return total;
+}
+static_assert(runs_total() == kKernelCount, "every kernel belongs to one part");
+
+}  // namespace
+
+int kernel_part(int kernel) {
+    for (const PartRun& run : kPartRuns) {
+        if (kernel < run.kernels) return run.part;
+        kernel -= run.kernels;
+    }
+    return 0;
+}
+
 namespace {
 
 thread_local SingeHipErrorDetail t_error = {0, "", 0, 0};
 
 constexpr int kMaxDevices = 64;
 
+// A device's kernel handles are published one by one as they are first asked for; a launch reads its handle
+// without a lock and takes the mutex only when the handle is not there yet.
 struct DeviceModule {
-    hipModule_t module = nullptr;
-    bool loaded = false;
-    hipFunction_t functions[kKernelCount] = {};
+    hipModule_t modules[kPartCount] = {};
+    bool loaded[kPartCount] = {};
+    std::atomic<hipFunction_t> functions[kKernelCount] = {};
 };
 
-std::mutex g_mutex;                 // guards the image and the per-device tables
-std::vector<unsigned char> g_image; // copy of the code object
+std::mutex g_mutex;                               // guards the images, module loading and the publishing of handles
+std::vector<unsigned char> g_images[kPartCount];  // copies of the code object's parts
+bool g_single_image = false;                      // an image handed to singe_hip_load holds every kernel (in slot 0)
 DeviceModule g_devices[kMaxDevices];
 
-std::string default_image_path() {
+std::string default_image_path(int part) {
     Dl_info info;
     if (dladdr(reinterpret_cast<void*>(&default_image_path), &info) == 0 || info.dli_fname == nullptr) return "";
     std::string path(info.dli_fname);
     size_t slash = path.rfind('/');
     path = slash == std::string::npos ? std::string(".") : path.substr(0, slash);
-    return path + "/singe_attention_gfx950.hsaco";
+    return path + "/singe_attention_gfx950." + kPartNames[part] + ".hsaco";
 }
 
 bool read_file(const std::string& path, std::vector<unsigned char>& bytes) {
@@ -110,8 +150,12 @@ bool read_file(const std::string& path, std::vector<unsigned char>& bytes) {
 void drop_modules_locked() {
     const HipRuntime* hip = hip_runtime();
     for (DeviceModule& device : g_devices) {
-        if (device.loaded && hip != nullptr) hip->hipModuleUnload(device.module);
-        device = DeviceModule();
+        for (std::atomic<hipFunction_t>& function : device.functions) function.store(nullptr, std::memory_order_release);
+        for (int part = 0; part < kPartCount; ++part) {
+            if (device.loaded[part] && hip != nullptr) hip->hipModuleUnload(device.modules[part]);
+            device.modules[part] = nullptr;
+            device.loaded[part] = false;
+        }
     }
 }
 
@@ -148,21 +192,25 @@ int32_t kernel_function(KernelId kernel, hipFunction_t* function) {
     int device = 0;
     if (hipError_t error = hip->hipGetDevice(&device)) return fail_hip(error, "hipGetDevice");
     if (device < 0 || device >= kMaxDevices) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "device index");
-    std::lock_guard<std::mutex> lock(g_mutex);
     DeviceModule& slot = g_devices[device];
-    if (!slot.loaded) {
-        if (g_image.empty() && !read_file(default_image_path(), g_image))
-            return fail(SINGE_HIP_KERNEL_NOT_PREPARED, "singe_attention_gfx950.hsaco");
-        if (hipError_t error = hip->hipModuleLoadData(&slot.module, g_image.data())) return fail_hip(error, "hipModuleLoadData");
-        slot.loaded = true;
+    if (hipFunction_t published = slot.functions[kernel].load(std::memory_order_acquire)) {
+        *function = published;
+        return 0;
     }
-    if (slot.functions[kernel] == nullptr) {
-        if (hipError_t error = hip->hipModuleGetFunction(&slot.functions[kernel], slot.module, kKernelNames[kernel])) {
-            slot.functions[kernel] = nullptr;
-            return fail_hip(error, kKernelNames[kernel]);
-        }
+    std::lock_guard<std::mutex> lock(g_mutex);
+    const int part = g_single_image ? 0 : kernel_part(kernel);
+    if (!slot.loaded[part]) {
+        if (g_images[part].empty() && !read_file(default_image_path(part), g_images[part]))
+            return fail(SINGE_HIP_KERNEL_NOT_PREPARED, kPartNames[part]);
+        if (hipError_t error = hip->hipModuleLoadData(&slot.modules[part], g_images[part].data())) return fail_hip(error, "hipModuleLoadData");
+        slot.loaded[part] = true;
     }
-    *function = slot.functions[kernel];
+    hipFunction_t found = slot.functions[kernel].load(std::memory_order_relaxed);
+    if (found == nullptr) {
+        if (hipError_t error = hip->hipModuleGetFunction(&found, slot.modules[part], kKernelNames[kernel])) return fail_hip(error, kKernelNames[kernel]);
+        slot.functions[kernel].store(found, std::memory_order_release);
+    }
+    *function = found;
     return 0;
 }
 
@@ -208,7 +256,9 @@ int32_t singe_hip_load(const void* image, size_t bytes) {
     if (bytes == 0) return fail(SINGE_HIP_INVALID_LENGTH, "image");
     std::lock_guard<std::mutex> lock(g_mutex);
     drop_modules_locked();
-    g_image.assign(static_cast<const unsigned char*>(image), static_cast<const unsigned char*>(image) + bytes);
+    for (std::vector<unsigned char>& held : g_images) held.clear();
+    g_images[0].assign(static_cast<const unsigned char*>(image), static_cast<const unsigned char*>(image) + bytes);
+    g_single_image = true;
     return 0;
 }
 
@@ -218,14 +268,24 @@ int32_t singe_hip_load_file(const char* path) {
     if (!read_file(path, bytes)) return fail(SINGE_HIP_KERNEL_NOT_PREPARED, "code object file");
     std::lock_guard<std::mutex> lock(g_mutex);
     drop_modules_locked();
-    g_image.swap(bytes);
+    for (std::vector<unsigned char>& held : g_images) held.clear();
+    g_images[0].swap(bytes);
+    g_single_image = true;
     return 0;
 }
 
 void singe_hip_unload(void) {
     std::lock_guard<std::mutex> lock(g_mutex);
     drop_modules_locked();
-    g_image.clear();
+    for (std::vector<unsigned char>& held : g_images) held.clear();
+    g_single_image = false;
+}
+
+int32_t singe_hip_kernel(int32_t index, const char** name, const char** part) {
+    if (index < 0 || index >= kKernelCount) return fail(SINGE_HIP_INVALID_ARGUMENT, "kernel index");
+    if (name != nullptr) *name = kKernelNames[index];
+    if (part != nullptr) *part = kPartNames[kernel_part(index)];
+    return 0;
 }
 
 int32_t singe_hip_prepare(int32_t* count) {

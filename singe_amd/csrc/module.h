@@ -50,6 +50,11 @@ enum KernelId : int {
 
 extern const char* const kKernelNames[kKernelCount];
 
+// Parts of the code object (one file each) and the part a kernel lives in.
+constexpr int kPartCount = 12;
+extern const char* const kPartNames[kPartCount];
+int kernel_part(int kernel);
+
 // Status of the thread's last failure (see singe_hip_last_error).
 int32_t fail(int32_t status, const char* name = "", uint64_t minimum = 0, uint64_t actual = 0);
 int32_t fail_hip(hipError_t error, const char* what);

@@ -9,7 +9,7 @@
 // overlap on one GPU race.
 #include <hip/hip_runtime.h>
 
-#include <mutex>
+#include <atomic>
 
 #include "static_scratch.h"
 
@@ -23,8 +23,7 @@ __global__ void singe_static_scratch_probe(unsigned int* seen) {
 }
 
 constexpr int kMaxDevices = 64;
-std::mutex g_mutex;
-void* g_address[kMaxDevices] = {};
+std::atomic<void*> g_address[kMaxDevices] = {};
 
 }  // namespace
 
@@ -34,14 +33,14 @@ int static_scratch(void** pointer, size_t* bytes) {
     int device = 0;
     if (hipError_t error = hipGetDevice(&device)) return -static_cast<int>(error);
     if (device < 0 || device >= kMaxDevices) return -static_cast<int>(hipErrorInvalidDevice);
-    std::lock_guard<std::mutex> lock(g_mutex);
-    if (g_address[device] == nullptr) {
-        void* address = nullptr;
+    void* address = g_address[device].load(std::memory_order_acquire);
+    if (address == nullptr) {
+        // Two threads that get here together resolve the same address.
         if (hipError_t error = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch))) return -static_cast<int>(error);
         if (address == nullptr) return -static_cast<int>(hipErrorInvalidSymbol);
-        g_address[device] = address;
+        g_address[device].store(address, std::memory_order_release);
     }
-    *pointer = g_address[device];
+    *pointer = address;
     *bytes = SINGE_HIP_STATIC_SCRATCH_BYTES;
     return 0;
 }

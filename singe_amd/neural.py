@@ -6,6 +6,7 @@ returns the output and each row's base-two log-sum-exp."""
 from __future__ import annotations
 
 import ctypes
+import functools
 from dataclasses import dataclass
 
 import torch
@@ -13,6 +14,20 @@ import torch
 from . import _native, error
 
 STATUS_INDEX_OUT_OF_BOUNDS = 1  # singe/src/backend/kernel_lowering/mod.rs:40-61
+
+
+def _on_stream(op):
+    """Runs ``op`` with its ``stream=`` argument as torch's current stream, so everything the op does besides its
+    own launch (allocating and filling the outputs and the status word, converting a mask, reading the status
+    word back) is ordered on the stream the kernel runs on, as the reference keeps one kernel stream per device
+    for its launches and their buffers (kernel_plan/mod.rs:156-232)."""
+    @functools.wraps(op)
+    def ordered(*args, stream=None, **kwargs):
+        if stream is None or stream == torch.cuda.current_stream(stream.device):
+            return op(*args, stream=stream, **kwargs)
+        with torch.cuda.stream(stream):
+            return op(*args, stream=stream, **kwargs)
+    return ordered
 
 
 @dataclass(frozen=True)
@@ -88,6 +103,11 @@ def attend_padded(query, key, value, key_lengths, options: AttentionOptions = At
 
 
 def _attend_all(query, key, value, mask, sinks, key_lengths, options, stream):
+    return _attend_all_ordered(query, key, value, mask, sinks, key_lengths, options, stream=stream)
+
+
+@_on_stream
+def _attend_all_ordered(query, key, value, mask, sinks, key_lengths, options, *, stream=None):
     """attend_all (tensor/neural.rs:139-175) with the shape rules of spec::attention_problem
     (singe/src/backend/spec/neural/attention.rs:209-290)."""
     for tensor, name in ((query, "query"), (key, "key"), (value, "value")):
@@ -158,6 +178,7 @@ def _scratch_for(device, nbytes: int) -> torch.Tensor:
     return held
 
 
+@_on_stream
 def paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor, paging: Paging,
                     options: AttentionOptions = AttentionOptions(), *, stream=None, status: torch.Tensor | None = None,
                     check: bool = True, scratch: "torch.Tensor | bool" = True):
@@ -211,6 +232,7 @@ def paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: t
     return output, lse
 
 
+@_on_stream
 def paged_mla_attention(query: torch.Tensor, query_positions: torch.Tensor, latent_cache: torch.Tensor,
                         position_cache: torch.Tensor, paging: Paging, options: AttentionOptions = AttentionOptions(), *,
                         stream=None, status: torch.Tensor | None = None, check: bool = True,
@@ -273,6 +295,7 @@ def paged_mla_attention(query: torch.Tensor, query_positions: torch.Tensor, late
     return output, lse
 
 
+@_on_stream
 def rotary_paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: torch.Tensor, paging: Paging,
                            cos: torch.Tensor, sin: torch.Tensor, options: AttentionOptions = AttentionOptions(), *,
                            query_norm: "RotationNorm | None" = None, stream=None, status: torch.Tensor | None = None,
@@ -326,6 +349,7 @@ class RotationNorm:
     weight: torch.Tensor | None = None
 
 
+@_on_stream
 def rotary_cache_write(query, key, value, cos, sin, pages, slots, key_cache, value_cache, *,
                        query_norm: RotationNorm | None = None, key_norm: RotationNorm | None = None, stream=None,
                        status: torch.Tensor | None = None, check: bool = True):
@@ -379,6 +403,7 @@ def rotary_cache_write(query, key, value, cos, sin, pages, slots, key_cache, val
     return query_out
 
 
+@_on_stream
 def paging_indices(paging: Paging, *, tokens: int, page_size: int, cache_pages: int, width: int, row_elements: int,
                    stream=None, status: torch.Tensor | None = None, check: bool = True):
     """FlashInfer CSR paging -> block-table paging, on the device

@@ -26,14 +26,24 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, name), name
 
 
-def test_code_object_is_built_and_names_every_kernel():
-    assert os.path.exists(_native.CODE_OBJECT_PATH)
-    image = open(_native.CODE_OBJECT_PATH, "rb").read()
+def test_code_object_is_built_and_every_part_names_its_kernels():
+    images = {}
+    for part, path in zip(_native.CODE_OBJECT_PARTS, _native.CODE_OBJECT_PATHS):
+        assert os.path.exists(path), path
+        images[part] = open(path, "rb").read()
+    lib, names = _native.lib(), []
+    name, part = ctypes.c_char_p(), ctypes.c_char_p()
+    index = 0
+    while lib.singe_hip_kernel(index, ctypes.byref(name), ctypes.byref(part)) == 0:
+        assert name.value in images[part.value.decode()], (name.value, part.value)
+        names.append(name.value)
+        index += 1
+    assert len(names) == len(set(names)) >= 113
     for kernel in (b"singe_paged_decode_bf16_d128_g1_b16", b"singe_paged_decode_f8kv_wide_d128_b16",
                    b"singe_paged_decode_combine_bf16", b"singe_fmha_prefill_bf16_d128_causal",
                    b"singe_fmha_prefill_f32_d64", b"singe_paged_attention_bf16_d128_i64", b"singe_paged_attention_bf16_d128_i32_p16",
                    b"singe_paged_kv_prefill_bf16_d128_p16", b"singe_rotary_paged_attention_bf16_d128_i64_p16"):
-        assert kernel in image, kernel
+        assert kernel in names, kernel
 
 
 def test_status_strings():

@@ -202,3 +202,29 @@ def test_decode_shaped_calls_split_on_their_own_and_agree_with_the_unsplit_kerne
     split, split_lse = neural.paged_attention(q, kc, vc, paging, neural.AttentionOptions(causal=True))
     assert (apart.float() - split.float()).abs().max().item() <= 4e-3
     assert (apart_lse - split_lse).abs().max().item() <= 1e-3
+
+
+def test_a_stream_that_is_not_torchs_current_one_orders_the_fills_and_the_status_word():
+    """The wrapper fills the output, the log-sum-exp and the status word and reads the word back: all of it has to
+    run on the stream the kernel is launched on, also when that is not torch's current stream.  The current stream
+    is kept busy meanwhile, so work queued on it by mistake would land after the kernel's."""
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(9)
+    q = torch.randn((40, 4, 128), generator=gen, device="cuda").to(torch.bfloat16)
+    cache = torch.randn((6, 32, 2, 128), generator=gen, device="cuda").to(torch.bfloat16)
+    index = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
+    good = neural.Paging(index([0, 20, 40]), index([0, 3, 5]), index([4, 1, 0, 2, 5]), index([7, 32]))
+    bad = neural.Paging(index([0, 20, 40]), index([0, 3, 5]), index([4, 1, 0, 2, 6]), index([7, 32]))
+    want, want_lse = neural.paged_attention(q, cache, cache, good, neural.AttentionOptions(causal=True))
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    busy = torch.randn((4096, 4096), device="cuda")
+    for _ in range(3):
+        for _ in range(20):
+            busy = busy @ busy * 1e-3  # the current stream stays busy while the side stream works
+        got, got_lse = neural.paged_attention(q, cache, cache, good, neural.AttentionOptions(causal=True), stream=side)
+        side.synchronize()
+        assert torch.equal(got, want) and torch.equal(got_lse, want_lse)
+        with pytest.raises(error.IndexOutOfBounds):
+            neural.paged_attention(q, cache, cache, bad, neural.AttentionOptions(causal=True), stream=side)
+    torch.cuda.synchronize()
