@@ -7,11 +7,18 @@ context lengths uniform in [512, 4096], block tables from a seeded permutation o
 pool.  Inputs are resident in HBM before the timed region; three independent KV pools are rotated so
 consecutive steps cannot be served from the 256 MB Infinity Cache.
 
-Prints one JSON line: whole-job GB/s of algorithmic bytes, the roofline of the dominant kernel
-(measured with HIP events on the launch stream) and the CPU oracle timed on a bounded sample.  The
-same line carries, under "prefill", the causal flash-attention prefill measurement (TFLOP/s against
-the dense bf16 MFMA peak), under "chunked_prefill", "fp8_decode" and "dense_f32" the other three
-benchmark configurations, and under "latent" latent (MLA) attention over paged caches (decode and chunked prefill).
+Prints one JSON line: whole-job GB/s of algorithmic bytes over exactly --steps steps after --warmup
+steps, the roofline of the dominant kernel and the CPU oracle timed on a bounded sample.  The same line
+carries one object per further benchmark configuration ("prefill", "chunked_prefill", "fp8_decode",
+"dense_f32"), "latent" (MLA attention over paged caches), "head_dim_64" (the matrix-core kernels at the
+reference's other head dimension) and "mfma_ceiling" (what the matrix cores sustain on a register-only loop
+of the prefill kernels' product, on zeros and on the benchmark's kind of data).
+
+How every kernel figure is taken, whatever --steps says: at least 300 ms of warm-up launches, then at
+least 30 samples, each a pair of HIP events on the launch stream around a small group of back-to-back
+launches; mean, median and the quartiles are reported (the reference times its kernels the same way:
+singe-testing/src/bench.rs:11-13, singe/src/backend/cuda/kernel_tuning/measure/mod.rs:34-53).
+`--only SECTION` runs one section alone and prints it, for rocprofv3 runs of its kernel.
 """
 from __future__ import annotations
 
@@ -25,19 +32,39 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-# HBM bytes per launch of the decode split kernel at the headline workload, from rocprofv3 --pmc runs of
-# this script: FETCH_SIZE 145768 x 2 KiB (the counter's unit, calibrated on a copy of known size) +
-# WRITE_SIZE 4552 KiB.  Reported only for that kernel, workload and tuning.
-DECODE_TRAFFIC_BYTES = (145766 * 2 + 4552) * 1024
-# The same for the dense prefill kernel at batch 4 x seq 4096 x 32 heads: FETCH_SIZE 301283, WRITE_SIZE 131377.
-PREFILL_TRAFFIC_BYTES = (311083 * 2 + 132590) * 1024
-# The same for the latent attention kernel at its two workloads (--only-latent under rocprofv3 --pmc): decode
-# FETCH_SIZE 608520, WRITE_SIZE 33047; chunked prefill FETCH_SIZE 1376200, WRITE_SIZE 526390.
-LATENT_DECODE_TRAFFIC_BYTES = (608520 * 2 + 33047) * 1024
-LATENT_CHUNKED_TRAFFIC_BYTES = (1376200 * 2 + 526390) * 1024
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 POOLS = 3
+WARMUP_SECONDS = 0.3
+MIN_SAMPLES = 30
+
+# HBM bytes per launch from rocprofv3 --pmc runs of `bench.py --only SECTION` (FETCH_SIZE, then WRITE_SIZE, each in
+# a run of its own).  Both counters were calibrated in the same runs on torch's f32 -> bf16 copy of 2^28 elements
+# (1 GiB read, 512 MiB written): FETCH_SIZE counts units of 2 KiB, WRITE_SIZE units of 1 KiB.  The figures belong
+# to the kernel, workload and tuning named, are not re-measured by the run that prints them, and are listed with the
+# profile summary they come from.
+FETCH_UNIT_BYTES, WRITE_UNIT_BYTES = 2048, 1024
+COUNTER_TRAFFIC = {
+    "decode": {"kernel": "singe_paged_decode_bf16_d128_g1_b16", "FETCH_SIZE": 145766, "WRITE_SIZE": 4552,
+               "source": "profiles/paged_decode_and_prefill_hbm_traffic.md"},
+    "prefill": {"kernel": "singe_fmha_prefill_bf16_d128_causal", "FETCH_SIZE": 311083, "WRITE_SIZE": 132590,
+                "source": "profiles/paged_decode_and_prefill_hbm_traffic.md"},
+    "latent_decode": {"kernel": "singe_paged_mla_attention_bf16_l512_p64", "FETCH_SIZE": 608520, "WRITE_SIZE": 33047,
+                      "source": "profiles/paged_mla_attention_latent_kernel_stats.md"},
+    "latent_chunked_prefill": {"kernel": "singe_paged_mla_attention_bf16_l512_p64", "FETCH_SIZE": 1376200,
+                               "WRITE_SIZE": 526390, "source": "profiles/paged_mla_attention_latent_kernel_stats.md"},
+}
+
+
+def traffic(key):
+    """(bytes per launch, where the counters were read) or (None, None) when no counter run covers the kernel."""
+    entry = COUNTER_TRAFFIC.get(key)
+    if entry is None:
+        return None, None
+    return entry["FETCH_SIZE"] * FETCH_UNIT_BYTES + entry["WRITE_SIZE"] * WRITE_UNIT_BYTES, entry["source"]
+
+
+SECTIONS = ("decode", "prefill", "chunked_prefill", "fp8_decode", "dense_f32", "latent", "head_dim_64", "mfma_ceiling")
 
 
 def parse():
@@ -46,140 +73,256 @@ def parse():
     parser.add_argument("--steps", type=int, default=300)
     parser.add_argument("--warmup", type=int, default=30)
     parser.add_argument("--no-cpu-baseline", action="store_true")
-    parser.add_argument("--no-prefill", action="store_true", help="skip the prefill measurement")
-    parser.add_argument("--no-extras", action="store_true", help="skip the chunked-prefill and fp8-decode measurements")
-    parser.add_argument("--prefill-steps", type=int, default=40)
-    parser.add_argument("--workers", type=int, default=0, help="tuning override (0 = built-in choice)")
-    parser.add_argument("--only-latent", action="store_true",
-                        help="run the latent attention section alone and print it (for counter runs of its kernel)")
+    parser.add_argument("--no-extras", action="store_true", help="the headline decode section only")
+    parser.add_argument("--workers", type=int, default=0, help="decode tuning override (0 = built-in choice)")
+    parser.add_argument("--only", choices=SECTIONS, default=None,
+                        help="run one section alone and print it (for profiler and counter runs of its kernel)")
+    parser.add_argument("--few", action="store_true", help="with --only: a handful of launches, no warm-up (counter runs)")
     return parser.parse_args()
 
 
-def cpu_baseline(work, budget_s=12.0):
-    """The reference's CPU decode as written (one thread, weights re-evaluated per output dimension),
-    restated in the oracle, timed on as many leading sequences of the same workload as fit the budget."""
-    import numpy as np
-
-    import oracle
-
-    order = list(range(work.batch))
-    done_bytes, elapsed, used = 0, 0.0, 0
-    cores = min(os.cpu_count() or 1, 16)
-    parallel = 0.0
-    for b in order:
-        length = int(work.seq_lens[b])
-        n = (length + work.block_size - 1) // work.block_size
-        blocks = work.block_table[b, :n].astype(np.int64)
-        import torch
-
-        index = torch.from_numpy(blocks).to(work.key_cache.device)
-        kc = work.key_cache[index].float().cpu().numpy()
-        vc = work.value_cache[index].float().cpu().numpy()
-        q = work.query[b:b + 1].float().cpu().numpy()
-        table = np.arange(n, dtype=np.uint32).reshape(1, -1)
-        start = time.perf_counter()
-        oracle.paged_kv_decode_attention_f32(q, kc, vc, [length], table, batch=1, heads=work.heads,
-                                             kv_heads=work.kv_heads, head_dim=work.head_dim,
-                                             block_size=work.block_size, block_table_batch_stride=max(n, 1),
-                                             scale=work.scale, literal=True)
-        elapsed += time.perf_counter() - start
-        # The same sequence with its independent head rows on every host core and the weight of a (row, key)
-        # pair evaluated once: the way the reference's dense op spreads rows over threads
-        # (singe/src/backend/cpu/normalization/attention.rs:219-223); bit-identical outputs.
-        start = time.perf_counter()
-        oracle.paged_kv_decode_attention_f32(q, kc, vc, [length], table, batch=1, heads=work.heads,
-                                             kv_heads=work.kv_heads, head_dim=work.head_dim,
-                                             block_size=work.block_size, block_table_batch_stride=max(n, 1),
-                                             scale=work.scale, threads=cores)
-        parallel += time.perf_counter() - start
-        done_bytes += length * 2 * work.kv_heads * work.head_dim * 2 + 2 * work.heads * work.head_dim * 2
-        used += 1
-        if elapsed > budget_s:
-            break
-    return {
-        "value": done_bytes / elapsed / 1e9,
-        "unit": "GB/s",
-        "cores": 1,
-        "kind": "port",
-        "sample": f"first {used} of {work.batch} sequences of the same workload, reference loop shape "
-                  f"(single thread, {elapsed:.1f} s)",
-        "row_parallel": {"value": done_bytes / parallel / 1e9, "unit": "GB/s", "cores": cores,
-                         "sample": f"the same sequences, head rows over {cores} threads, weights hoisted ({parallel:.2f} s)"},
-    }
+FEW = False
 
 
-def prefill_section(steps):
-    """Causal flash-attention prefill, batch 4, seq 4096, 32 heads, head_dim 128, bf16 (the
-    third benchmark configuration): average kernel time from HIP events around back-to-back launches."""
+def measure(launch, group):
+    """Per-launch time of `launch` in milliseconds: warm-up for WARMUP_SECONDS, then MIN_SAMPLES samples, each a pair of
+    HIP events on torch's current stream (the stream every launch here goes to) around `group` back-to-back launches."""
     import torch
 
-    from singe_amd.kernel import attention as A
-
-    batch, seq, heads, dim = 4, 4096, 32, 128
-    gen = torch.Generator(device="cuda")
-    gen.manual_seed(0x51A6E + 3)
-    q, k, v = (torch.randn((batch, seq, heads, dim), generator=gen, device="cuda").to(torch.bfloat16) for _ in range(3))
-    out = torch.empty_like(q)
-    config = A.FmhaPrefillConfig.contiguous(batch, seq, seq, heads, heads, dim, float(dim) ** -0.5, True)
-    for _ in range(5):
-        A.fmha_prefill_bf16(None, out, q, k, v, config)
-    torch.cuda.synchronize()
-    group = 5
-    groups = max(steps // group, 4)
-    begin = [torch.cuda.Event(enable_timing=True) for _ in range(groups)]
-    finish = [torch.cuda.Event(enable_timing=True) for _ in range(groups)]
-    for j in range(groups):
-        begin[j].record()
-        for _ in range(group):
-            A.fmha_prefill_bf16(None, out, q, k, v, config)
-        finish[j].record()
-    torch.cuda.synchronize()
-    ms = sorted(b.elapsed_time(f) / group for b, f in zip(begin, finish))
-    avg = sum(ms) / len(ms)
-    flops = 4 * dim * batch * heads * (seq * (seq + 1) // 2)
-    tflops = flops / (avg * 1e-3) / 1e12
-    return {
-        "workload": "causal flash prefill: batch 4, seq 4096, 32 heads (MHA), head_dim 128, bf16 in/out, "
-                    "fp32 softmax/accumulate (BASELINE config 3)",
-        "value": tflops,
-        "unit": "TFLOP/s",
-        "tokens_per_s": batch * seq / (avg * 1e-3),
-        "ms_per_step": avg,
-        "algorithmic_flops": flops,
-        "pct_bf16_mfma_peak": 100.0 * tflops / MFMA_BF16_PEAK_TFLOPS,
-        "roofline": {
-            "bound": "mfma",
-            "kernel": "singe_fmha_prefill_bf16_d128_causal",
-            "achieved": tflops,
-            "peak": MFMA_BF16_PEAK_TFLOPS,
-            "unit": "TFLOP/s",
-            "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
-            "traffic": PREFILL_TRAFFIC_BYTES,
-            "kernel_avg_us": avg * 1e3,
-            "kernel_median_us": ms[len(ms) // 2] * 1e3,
-        },
-    }
-
-
-def time_launches(launch, steps, group):
-    """Average milliseconds per launch from HIP events on the current stream around groups of
-    back-to-back launches; returns (average, median)."""
-    import torch
-
-    groups = max(steps // group, 4)
-    begin = [torch.cuda.Event(enable_timing=True) for _ in range(groups)]
-    finish = [torch.cuda.Event(enable_timing=True) for _ in range(groups)]
-    for j in range(groups):
+    samples = 3 if FEW else MIN_SAMPLES
+    if not FEW:
+        started = time.perf_counter()
+        while time.perf_counter() - started < WARMUP_SECONDS:
+            for _ in range(group):
+                launch()
+            torch.cuda.synchronize()
+    begin = [torch.cuda.Event(enable_timing=True) for _ in range(samples)]
+    finish = [torch.cuda.Event(enable_timing=True) for _ in range(samples)]
+    for j in range(samples):
         begin[j].record()
         for _ in range(group):
             launch()
         finish[j].record()
     torch.cuda.synchronize()
     ms = sorted(b.elapsed_time(f) / group for b, f in zip(begin, finish))
-    return sum(ms) / len(ms), ms[len(ms) // 2]
+    quartile = lambda q: ms[min(len(ms) - 1, int(round(q * (len(ms) - 1))))]
+    return {"mean_ms": sum(ms) / len(ms), "median_ms": quartile(0.5), "p25_ms": quartile(0.25), "p75_ms": quartile(0.75),
+            "iqr_ms": quartile(0.75) - quartile(0.25), "min_ms": ms[0], "samples": len(ms), "launches_per_sample": group}
 
 
-def chunked_prefill_section(steps):
+def timing_fields(stats):
+    return {"kernel_avg_us": stats["mean_ms"] * 1e3, "kernel_median_us": stats["median_ms"] * 1e3,
+            "kernel_p25_us": stats["p25_ms"] * 1e3, "kernel_p75_us": stats["p75_ms"] * 1e3,
+            "kernel_iqr_us": stats["iqr_ms"] * 1e3, "samples": stats["samples"],
+            "launches_per_sample": stats["launches_per_sample"]}
+
+
+def host_description():
+    model = "unknown"
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                model = line.split(":", 1)[1].strip()
+                break
+    except OSError:
+        pass
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    return {"cpu_model": model, "nproc": os.cpu_count() or 1, "usable_cores": usable}
+
+
+def cpu_threads():
+    return min(host_description()["usable_cores"], 16)
+
+
+# ---- CPU baselines: the oracle (a C restatement of the reference's CPU functions) on a bounded sample -------------
+
+def decode_cpu_baseline(work, budget_s=12.0, fp8=False):
+    """The reference's CPU decode as written (one thread, weights re-evaluated per output dimension,
+    singe-kernel/src/cpu/attention.rs:1172-1246), restated in the oracle, timed on as many leading sequences of the
+    same workload as fit the budget; then the same sequences with the head rows over the host's cores and the
+    weight of a (row, key) pair evaluated once, the way the reference's dense op spreads rows over threads
+    (singe/src/backend/cpu/normalization/attention.rs:219-223); bit-identical outputs.  With an fp8 cache the
+    oracle reads the cache dequantised to bf16_rne(value(code) * scale), one KV head of it."""
+    import numpy as np
+    import torch
+
+    import oracle
+
+    done_bytes, elapsed, used, parallel = 0, 0.0, 0, 0.0
+    cores = cpu_threads()
+    kv_heads = 1 if fp8 else work.kv_heads
+    heads = work.heads // work.kv_heads * kv_heads
+    for b in range(work.batch):
+        length = int(work.seq_lens[b])
+        n = (length + work.block_size - 1) // work.block_size
+        index = torch.from_numpy(work.block_table[b, :n].astype(np.int64)).to(work.key_cache.device)
+        if fp8:
+            widen = lambda codes, scales: (codes[index][:, :, :1].view(torch.float8_e4m3fn).float()
+                                           * scales[index][:, None, :1, None]).to(torch.bfloat16).float().cpu().numpy()
+            kc, vc = widen(work.key_cache, work.key_scales), widen(work.value_cache, work.value_scales)
+        else:
+            kc, vc = work.key_cache[index].float().cpu().numpy(), work.value_cache[index].float().cpu().numpy()
+        q = work.query[b:b + 1, :heads].float().cpu().numpy()
+        table = np.arange(n, dtype=np.uint32).reshape(1, -1)
+        shape = dict(batch=1, heads=heads, kv_heads=kv_heads, head_dim=work.head_dim, block_size=work.block_size,
+                     block_table_batch_stride=max(n, 1), scale=work.scale)
+        start = time.perf_counter()
+        oracle.paged_kv_decode_attention_f32(q, kc, vc, [length], table, literal=True, **shape)
+        elapsed += time.perf_counter() - start
+        start = time.perf_counter()
+        oracle.paged_kv_decode_attention_f32(q, kc, vc, [length], table, threads=cores, **shape)
+        parallel += time.perf_counter() - start
+        element = 1 if fp8 else 2
+        done_bytes += length * 2 * kv_heads * work.head_dim * element + 2 * heads * work.head_dim * 2
+        if fp8:
+            done_bytes += 2 * n * kv_heads * 4
+        used += 1
+        if elapsed > budget_s:
+            break
+    what = f"first {used} of {work.batch} sequences" + (", one of its 8 KV heads (8 query heads)" if fp8 else "")
+    return {
+        "value": done_bytes / elapsed / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+        "sample": f"{what} of the same workload, reference loop shape (single thread, {elapsed:.1f} s); bytes counted "
+                  f"as for the GPU figure",
+        "row_parallel": {"value": done_bytes / parallel / 1e9, "unit": "GB/s", "cores": cores,
+                         "sample": f"the same sequences, head rows over {cores} threads, weights hoisted ({parallel:.2f} s)"},
+        "host": host_description(),
+    }
+
+
+def prefill_cpu_baseline(q, k, v, scale):
+    """fmha_prefill_lse_f32 (singe-kernel/src/cpu/attention.rs:1758-1833) on one (batch, head) of the workload: rows
+    1792..2303 as written (one thread, the weight re-evaluated per output dimension), extrapolated to the whole
+    problem by the exact count of (query, key) pairs; then every row of two heads over the host's cores with the
+    weights hoisted."""
+    import numpy as np
+
+    import oracle
+
+    batch, seq, heads, dim = q.shape
+    one = lambda t, h: np.ascontiguousarray(t[0, :, h:h + 1, :].float().cpu().numpy()[None])
+    first, count = 1792, 512
+    start = time.perf_counter()
+    oracle.fmha_prefill_lse_f32_literal(one(q, 0), one(k, 0), one(v, 0), batch=1, query_len=seq, key_len=seq, heads=1,
+                                        kv_heads=1, head_dim=dim, scale=scale, causal=True, row_first=first, row_count=count)
+    elapsed = time.perf_counter() - start
+    pairs = sum(r + 1 for r in range(first, first + count))
+    cores = cpu_threads()
+    two = lambda t: np.ascontiguousarray(t[0, :, 0:2, :].float().cpu().numpy()[None])
+    start = time.perf_counter()
+    oracle.fmha_prefill_lse_f32(two(q), two(k), two(v), batch=1, query_len=seq, key_len=seq, heads=2, kv_heads=2,
+                                head_dim=dim, scale=scale, causal=True, threads=cores)
+    parallel = time.perf_counter() - start
+    parallel_pairs = 2 * seq * (seq + 1) // 2
+    return {
+        "value": 4 * dim * pairs / elapsed / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+        "sample": f"rows {first}..{first + count - 1} of one (batch, head): {pairs} of the problem's "
+                  f"{batch * heads * seq * (seq + 1) // 2} (query, key) pairs, reference loop shape (single thread, {elapsed:.1f} s)",
+        "row_parallel": {"value": 4 * dim * parallel_pairs / parallel / 1e12, "unit": "TFLOP/s", "cores": cores,
+                         "sample": f"all rows of two heads of one batch ({parallel_pairs} pairs), rows over {cores} threads, "
+                                   f"weights hoisted ({parallel:.2f} s)"},
+        "host": host_description(),
+    }
+
+
+def chunked_prefill_cpu_baseline(work):
+    """attend_paged (singe/src/backend/cpu/normalization/attention.rs:424-538, serial in the reference) on the last 64
+    new tokens of the first sequence over its whole prefix, one KV head (8 query heads): single thread, then the same
+    rows over the host's cores."""
+    import numpy as np
+    import torch
+
+    import oracle
+
+    group = work.heads // work.kv_heads
+    first, last = int(work.page_offsets[0]), int(work.page_offsets[1])
+    index = torch.from_numpy(np.asarray(work.pages[first:last], dtype=np.int64)).to(work.key_cache.device)
+    kc = work.key_cache[index][:, :, :1].float().cpu().numpy()
+    vc = work.value_cache[index][:, :, :1].float().cpu().numpy()
+    tokens = 64
+    end = int(work.query_offsets[1])
+    q = work.query[end - tokens:end, :group].float().cpu().numpy()
+    keys = int(work.prefix[0]) + work.new_tokens
+    paging = dict(query_offsets=[0, tokens], page_offsets=[0, last - first], pages=list(range(last - first)),
+                  last_page_lengths=[int(work.last_page_lengths[0])])
+    pairs = group * sum(keys - tokens + i + 1 for i in range(tokens))
+    results = []
+    for threads in (1, cpu_threads()):
+        start = time.perf_counter()
+        status, _, _ = oracle.paged_attention_f32(q, kc, vc, paging["query_offsets"], paging["page_offsets"], paging["pages"],
+                                                  paging["last_page_lengths"], causal=True, threads=threads)
+        results.append(time.perf_counter() - start)
+        assert status == 0
+    total_pairs = work.algorithmic_flops() // (4 * work.head_dim)
+    return {
+        "value": 4 * work.head_dim * pairs / results[0] / 1e12, "unit": "TFLOP/s", "cores": 1, "kind": "port",
+        "sample": f"last {tokens} new tokens of sequence 0 over its {keys} keys, one KV head ({group} query heads): {pairs} of "
+                  f"the problem's {total_pairs} (query, key) pairs, single thread ({results[0]:.1f} s)",
+        "row_parallel": {"value": 4 * work.head_dim * pairs / results[1] / 1e12, "unit": "TFLOP/s", "cores": cpu_threads(),
+                         "sample": f"the same rows over {cpu_threads()} threads ({results[1]:.2f} s)"},
+        "host": host_description(),
+    }
+
+
+def dense_f32_cpu_baseline(q, k, v):
+    """softcapped_window_attention_f32 (singe-kernel/src/cpu/attention.rs:1835-1925) on the whole first configuration:
+    single thread, then rows over the host's cores (weights hoisted in both; the outputs are bit-identical to the
+    reference loop's)."""
+    import oracle
+
+    batch, heads, seq, dim = q.shape
+    operands = [t.cpu().numpy() for t in (q, k, v)]
+    times = []
+    for threads in (1, cpu_threads()):
+        start = time.perf_counter()
+        oracle.softcapped_window_attention_f32(*operands, batch=batch, query_len=seq, key_len=seq, heads=heads, kv_heads=heads,
+                                               head_dim=dim, scale=0.125, causal=True, threads=threads)
+        times.append(time.perf_counter() - start)
+    return {"value": times[0] * 1e6, "unit": "us", "cores": 1, "kind": "port",
+            "sample": "the whole configuration, single thread, weights hoisted",
+            "row_parallel": {"value": times[1] * 1e6, "unit": "us", "cores": cpu_threads(), "sample": "rows over the host's cores"},
+            "host": host_description()}
+
+
+# ---- GPU sections ----------------------------------------------------------------------------------------------------
+
+def prefill_section(with_cpu=True, dim=128, key="prefill"):
+    """Causal flash-attention prefill, batch 4, seq 4096, 32 heads, bf16 (the third benchmark configuration at
+    head_dim 128)."""
+    import torch
+
+    from singe_amd.kernel import attention as A
+
+    batch, seq, heads = 4, 4096, 32
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x51A6E + 3)
+    q, k, v = (torch.randn((batch, seq, heads, dim), generator=gen, device="cuda").to(torch.bfloat16) for _ in range(3))
+    out = torch.empty_like(q)
+    scale = float(dim) ** -0.5
+    config = A.FmhaPrefillConfig.contiguous(batch, seq, seq, heads, heads, dim, scale, True)
+    stats = measure(lambda: A.fmha_prefill_bf16(None, out, q, k, v, config), 5)
+    flops = 4 * dim * batch * heads * (seq * (seq + 1) // 2)
+    tflops = flops / (stats["mean_ms"] * 1e-3) / 1e12
+    nbytes, source = traffic(key)
+    result = {
+        "workload": f"causal flash prefill: batch 4, seq 4096, 32 heads (MHA), head_dim {dim}, bf16 in/out, "
+                    "fp32 softmax/accumulate" + (" (BASELINE config 3)" if dim == 128 else ""),
+        "value": tflops, "unit": "TFLOP/s", "tokens_per_s": batch * seq / (stats["mean_ms"] * 1e-3),
+        "ms_per_step": stats["mean_ms"], "ms_per_step_median": stats["median_ms"], "algorithmic_flops": flops,
+        "pct_bf16_mfma_peak": 100.0 * tflops / MFMA_BF16_PEAK_TFLOPS,
+        "roofline": {"bound": "mfma", "kernel": f"singe_fmha_prefill_bf16_d{dim}_causal", "achieved": tflops,
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
+                     "traffic": nbytes, "traffic_source": source, **timing_fields(stats)},
+    }
+    if with_cpu:
+        result["cpu_baseline"] = prefill_cpu_baseline(q, k, v, scale)
+    return result
+
+
+def chunked_prefill_section(with_cpu=True):
     """Chunked paged prefill: 8 sequences, 512 new tokens each on prefixes U[1024, 16384], 64 query /
     8 KV heads, head_dim 128, page 16, bf16 (the fourth benchmark configuration), through the paged attention op."""
     import ctypes
@@ -198,36 +341,45 @@ def chunked_prefill_section(steps):
     lse = torch.empty(work.query.shape[:2], device="cuda", dtype=torch.float32)
     status = torch.zeros(1, device="cuda", dtype=torch.int32)
     handle = int(torch.cuda.current_stream().cuda_stream)
+    scratch_bytes = int(_native.lib().singe_hip_paged_attention_scratch_bytes(ctypes.byref(problem)))
+    scratch = torch.empty(max(scratch_bytes, 1), device="cuda", dtype=torch.uint8)
 
     def launch():
-        code = _native.lib().singe_hip_paged_attention_bf16(
-            handle, work.query.data_ptr(), work.key_cache.data_ptr(), work.value_cache.data_ptr(),
-            paging.query_offsets.data_ptr(), paging.page_offsets.data_ptr(), paging.pages.data_ptr(),
-            paging.last_page_lengths.data_ptr(), out.data_ptr(), lse.data_ptr(), status.data_ptr(), ctypes.byref(problem))
+        if scratch_bytes:
+            code = _native.lib().singe_hip_paged_attention_scratch_bf16(
+                handle, work.query.data_ptr(), work.key_cache.data_ptr(), work.value_cache.data_ptr(),
+                paging.query_offsets.data_ptr(), paging.page_offsets.data_ptr(), paging.pages.data_ptr(),
+                paging.last_page_lengths.data_ptr(), out.data_ptr(), lse.data_ptr(), status.data_ptr(), scratch.data_ptr(),
+                scratch.numel(), ctypes.byref(problem))
+        else:
+            code = _native.lib().singe_hip_paged_attention_bf16(
+                handle, work.query.data_ptr(), work.key_cache.data_ptr(), work.value_cache.data_ptr(),
+                paging.query_offsets.data_ptr(), paging.page_offsets.data_ptr(), paging.pages.data_ptr(),
+                paging.last_page_lengths.data_ptr(), out.data_ptr(), lse.data_ptr(), status.data_ptr(), ctypes.byref(problem))
         _native.check(code, "paged_attention")
 
-    for _ in range(3):
-        launch()
-    torch.cuda.synchronize()
-    avg, median = time_launches(launch, steps, 4)
+    stats = measure(launch, 4)
     assert int(status.item()) == 0
     flops = work.algorithmic_flops()
-    tflops = flops / (avg * 1e-3) / 1e12
-    return {
+    tflops = flops / (stats["mean_ms"] * 1e-3) / 1e12
+    nbytes, source = traffic("chunked_prefill")
+    result = {
         "workload": "chunked paged prefill: 8 sequences x 512 new tokens on prefixes U[1024,16384], 64q/8kv heads, "
-                    "head_dim 128, page 16, bf16 (BASELINE config 4)",
-        "value": tflops,
-        "unit": "TFLOP/s",
-        "tokens_per_s": work.sequences * work.new_tokens / (avg * 1e-3),
-        "ms_per_step": avg,
-        "algorithmic_flops": flops,
+                    "head_dim 128, page 16, bf16 (BASELINE config 4); whole op (the attention kernel and, where the op "
+                    "shares keys out, its merge)",
+        "value": tflops, "unit": "TFLOP/s", "tokens_per_s": work.sequences * work.new_tokens / (stats["mean_ms"] * 1e-3),
+        "ms_per_step": stats["mean_ms"], "ms_per_step_median": stats["median_ms"], "algorithmic_flops": flops,
+        "key_splits_scratch_bytes": scratch_bytes,
         "roofline": {"bound": "mfma", "kernel": "singe_paged_attention_bf16_d128_i32_p16", "achieved": tflops,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": None, "kernel_avg_us": avg * 1e3, "kernel_median_us": median * 1e3},
+                     "traffic": nbytes, "traffic_source": source, **timing_fields(stats)},
     }
+    if with_cpu:
+        result["cpu_baseline"] = chunked_prefill_cpu_baseline(work)
+    return result
 
 
-def latent_section(steps):
+def latent_section():
     """Latent (MLA) attention over paged caches at DeepSeek's widths (latent 512, positional 64, 128 heads, bf16,
     page 64), beside the benchmark's configurations: a decode step (256 sequences of 4096 keys; every head reads
     the same 1152 bytes per key, so the step is priced against HBM and the matrix cores both) and a chunked
@@ -237,7 +389,7 @@ def latent_section(steps):
 
     from singe_amd import neural
 
-    def case(sequences, heads=128, page=64):
+    def case(sequences, group, heads=128, page=64):
         query_offsets, page_offsets, last, table, pages = [0], [0], [], [], 0
         for queries, keys in sequences:
             query_offsets.append(query_offsets[-1] + queries)
@@ -256,40 +408,39 @@ def latent_section(steps):
         index = lambda values: torch.tensor(values, dtype=torch.int32, device="cuda")
         paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
         options = neural.AttentionOptions(causal=True)
-        launch = lambda: neural.paged_mla_attention(*operands, paging, options, check=False)
-        for _ in range(2):
-            launch()
-        torch.cuda.synchronize()
-        avg, median = time_launches(launch, steps, 2)
+        stats = measure(lambda: neural.paged_mla_attention(*operands, paging, options, check=False), group)
         pairs = sum(sum(min(keys, max(keys - queries + i, 0) + 1) for i in range(queries)) for queries, keys in sequences)
         flops = pairs * heads * (576 + 512) * 2
         cache_bytes = sum(keys for _, keys in sequences) * 1152 + tokens * heads * (576 + 512) * 2
-        return avg, median, flops, cache_bytes
+        return stats, flops, cache_bytes
 
-    avg, median, flops, cache_bytes = case([(1, 4096)] * 256)
-    gbps, tflops = cache_bytes / (avg * 1e-3) / 1e9, flops / (avg * 1e-3) / 1e12
+    stats, flops, cache_bytes = case([(1, 4096)] * 256, 4)
+    gbps, tflops = cache_bytes / (stats["mean_ms"] * 1e-3) / 1e9, flops / (stats["mean_ms"] * 1e-3) / 1e12
+    nbytes, source = traffic("latent_decode")
     decode = {
         "workload": "latent attention decode: 256 sequences x 4096 keys, 128 heads, latent 512 + positional 64, page 64, bf16",
-        "value": gbps, "unit": "GB/s", "tflops": tflops, "ms_per_step": avg, "ms_per_step_median": median,
+        "value": gbps, "unit": "GB/s", "tflops": tflops, "ms_per_step": stats["mean_ms"], "ms_per_step_median": stats["median_ms"],
         "algorithmic_bytes": cache_bytes, "algorithmic_flops": flops,
         "roofline": {"bound": "hbm", "kernel": "singe_paged_mla_attention_bf16_l512_p64", "achieved": gbps, "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": LATENT_DECODE_TRAFFIC_BYTES,
-                     "mfma_frac": tflops / MFMA_BF16_PEAK_TFLOPS},
+                     "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": nbytes, "traffic_source": source,
+                     "mfma_frac": tflops / MFMA_BF16_PEAK_TFLOPS, **timing_fields(stats)},
     }
-    avg, median, flops, cache_bytes = case([(512, 8192)] * 8)
-    tflops = flops / (avg * 1e-3) / 1e12
+    stats, flops, cache_bytes = case([(512, 8192)] * 8, 1)
+    tflops = flops / (stats["mean_ms"] * 1e-3) / 1e12
+    nbytes, source = traffic("latent_chunked_prefill")
     chunked = {
         "workload": "latent attention chunked prefill: 8 sequences x 512 new tokens on 8192 keys, 128 heads, latent 512 + "
                     "positional 64, page 64, bf16",
-        "value": tflops, "unit": "TFLOP/s", "ms_per_step": avg, "ms_per_step_median": median, "algorithmic_flops": flops,
+        "value": tflops, "unit": "TFLOP/s", "ms_per_step": stats["mean_ms"], "ms_per_step_median": stats["median_ms"],
+        "algorithmic_flops": flops,
         "roofline": {"bound": "mfma", "kernel": "singe_paged_mla_attention_bf16_l512_p64", "achieved": tflops,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": LATENT_CHUNKED_TRAFFIC_BYTES},
+                     "traffic": nbytes, "traffic_source": source, **timing_fields(stats)},
     }
     return {"decode": decode, "chunked_prefill": chunked}
 
 
-def dense_f32_section(steps):
+def dense_f32_section(with_cpu=True):
     """The first benchmark configuration, the f32 accuracy anchor: causal dense attention, batch 1, 8 heads,
     512 x 512, head_dim 64, scale 1/8, tensors [batch, heads, len, dim].  Far too small for a roofline: the
     figure is microseconds per launch."""
@@ -303,27 +454,20 @@ def dense_f32_section(steps):
     q, k, v = (torch.randn((batch, heads, seq, dim), generator=gen, device="cuda") for _ in range(3))
     out = torch.empty_like(q)
     config = A.SoftcappedWindowAttentionConfig(A.bhsd_config(batch, heads, heads, seq, seq, dim, 0.125, True), 0, None)
-
-    def launch():
-        A.softcapped_window_attention_f32(None, out, q, k, v, config)
-
-    for _ in range(5):
-        launch()
-    torch.cuda.synchronize()
-    avg, median = time_launches(launch, steps, 10)
-    return {
+    stats = measure(lambda: A.softcapped_window_attention_f32(None, out, q, k, v, config), 10)
+    result = {
         "workload": "causal dense attention f32: batch 1, 8 heads, 512 x 512, head_dim 64, scale 0.125, BHSD "
                     "(BASELINE config 1, the accuracy anchor)",
-        "value": avg * 1e3,
-        "unit": "us",
-        "us_per_step_median": median * 1e3,
-        "algorithmic_flops": 4 * dim * heads * (seq * (seq + 1) // 2),
-        "algorithmic_bytes": 4 * batch * heads * seq * dim * 4,
-        "kernel": "singe_fmha_prefill_rows_f32_d64",
+        "value": stats["mean_ms"] * 1e3, "unit": "us", "us_per_step_median": stats["median_ms"] * 1e3,
+        "algorithmic_flops": 4 * dim * heads * (seq * (seq + 1) // 2), "algorithmic_bytes": 4 * batch * heads * seq * dim * 4,
+        "kernel": "singe_fmha_prefill_rows_f32_d64", **timing_fields(stats),
     }
+    if with_cpu:
+        result["cpu_baseline"] = dense_f32_cpu_baseline(q, k, v)
+    return result
 
 
-def fp8_decode_section(steps):
+def fp8_decode_section(with_cpu=True):
     """Long-context decode over an fp8 e4m3 KV cache: batch 64, 64 query / 8 KV heads, head_dim 128,
     context 32768, block 16, one f32 scale per (block, kv head) (the fifth benchmark configuration); exact numerics."""
     import numpy as np
@@ -341,52 +485,102 @@ def fp8_decode_section(steps):
     out = torch.empty((work.batch, work.heads, work.head_dim), device="cuda", dtype=torch.bfloat16)
     workspace = torch.empty(config.workspace_bytes(), dtype=torch.uint8, device="cuda")
 
-    def launch():
+    def launch(phases=3):
         A.paged_kv_decode_attention_f8e4m3kv_bf16(None, out, work.query, work.key_cache, work.value_cache, work.key_scales,
-                                                  work.value_scales, lens, table, config, workspace)
+                                                  work.value_scales, lens, table, config, workspace, phases)
 
-    for _ in range(3):
-        launch()
-    torch.cuda.synchronize()
-    avg, median = time_launches(launch, steps, 2)
+    step = measure(launch, 2)
+    kernel = measure(lambda: launch(1), 2)
     used_blocks = int(np.sum((work.seq_lens.astype(np.int64) + work.block_size - 1) // work.block_size))
     nbytes = work.algorithmic_bytes(1) + 2 * used_blocks * work.kv_heads * 4  # + the scales of the used blocks
-    gbps = nbytes / (avg * 1e-3) / 1e9
-    return {
+    gbps = nbytes / (step["mean_ms"] * 1e-3) / 1e9
+    achieved = nbytes / (kernel["mean_ms"] * 1e-3) / 1e9
+    counted, source = traffic("fp8_decode")
+    result = {
         "workload": "paged decode, fp8 e4m3 KV: batch 64, 64q/8kv heads, head_dim 128, ctx 32768, block 16, "
                     "f32 scale per (block, kv head) (BASELINE config 5); split + reduce kernels",
-        "value": gbps,
-        "unit": "GB/s",
-        "tokens_per_s": work.batch / (avg * 1e-3),
-        "ms_per_step": avg,
-        "algorithmic_bytes": nbytes,
-        "roofline": {"bound": "hbm", "kernel": "singe_paged_decode_f8kv_wide_d128_b16", "achieved": gbps, "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": None, "step_avg_us": avg * 1e3,
-                     "step_median_us": median * 1e3},
+        "value": gbps, "unit": "GB/s", "tokens_per_s": work.batch / (step["mean_ms"] * 1e-3),
+        "ms_per_step": step["mean_ms"], "ms_per_step_median": step["median_ms"], "step_iqr_us": step["iqr_ms"] * 1e3,
+        "pct_hbm_peak": 100.0 * gbps / HBM_PEAK_GBPS, "algorithmic_bytes": nbytes,
+        "roofline": {"bound": "hbm", "kernel": "singe_paged_decode_f8kv_wide_d128_b16", "achieved": achieved, "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": counted, "traffic_source": source,
+                     **timing_fields(kernel)},
     }
+    if with_cpu:
+        result["cpu_baseline"] = decode_cpu_baseline(work, budget_s=2.0, fp8=True)
+    return result
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: this path has no cross-GPU exchange and every box here has one "
-              "GPU; run with --gpus 1", file=sys.stderr)
-        sys.exit(2)
+def head_dim_64_section():
+    """The matrix-core kernels at head_dim 64, the other head dimension of the reference's own tests
+    (singe/src/backend/cuda/kernel_plan/source/tests.rs:830-966): the third configuration's prefill and the second
+    configuration's decode at that width."""
+    import numpy as np
+    import torch
 
+    from singe_amd import synthetic
+    from singe_amd.kernel import attention as A
+
+    prefill = prefill_section(with_cpu=False, dim=64, key="prefill_d64")
+    work = synthetic.paged_decode_workload(head_dim=64)
+    config = A.PagedKvDecodeAttentionConfig.contiguous(work.batch, work.heads, work.kv_heads, work.head_dim,
+                                                       work.block_size, work.physical_blocks,
+                                                       work.block_table_batch_stride, work.scale)
+    lens = torch.from_numpy(work.seq_lens).cuda()
+    table = torch.from_numpy(work.block_table.view(np.int32)).cuda()
+    out = torch.empty((work.batch, work.heads, work.head_dim), device="cuda", dtype=torch.bfloat16)
+    workspace = torch.empty(config.workspace_bytes(), dtype=torch.uint8, device="cuda")
+    stats = measure(lambda: A.paged_kv_decode_attention_bf16(None, out, work.query, work.key_cache, work.value_cache, lens, table,
+                                                             config, workspace), 6)
+    nbytes = work.algorithmic_bytes()
+    gbps = nbytes / (stats["mean_ms"] * 1e-3) / 1e9
+    decode = {"workload": "paged decode: batch 32, 32q/8kv heads, head_dim 64, bf16, block 16, ctx U[512,4096]; split + reduce",
+              "value": gbps, "unit": "GB/s", "ms_per_step": stats["mean_ms"], "algorithmic_bytes": nbytes,
+              "pct_hbm_peak": 100.0 * gbps / HBM_PEAK_GBPS, **timing_fields(stats)}
+    return {"prefill": prefill, "decode": decode}
+
+
+def mfma_ceiling_section():
+    """What the matrix cores sustain with nothing else in the way: 512 workgroups of four waves, each wave a
+    register-only loop of the prefill kernels' product (v_mfma_f32_32x32x16_bf16), on all-zero operands and on
+    N(0, 1) operands from the same generator as the benchmark's tensors.  The clock under such a loop is set by
+    power, and power by the operands' bits, so the second figure is the ceiling a prefill kernel has on data like
+    the benchmark's."""
+    import torch
+
+    from singe_amd import _native
+
+    workgroups, iterations = 512, 4000
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x51A6E + 9)
+    operands = {"zeros": torch.zeros(1 << 22, device="cuda", dtype=torch.bfloat16),
+                "normal": torch.randn(1 << 22, generator=gen, device="cuda").to(torch.bfloat16)}
+    out = torch.empty(workgroups * 256, device="cuda", dtype=torch.float32)
+    handle = int(torch.cuda.current_stream().cuda_stream)
+    flops = workgroups * 4 * iterations * 32 * 32768
+    result = {"kernel": "singe_mfma_ceiling_bf16", "workgroups": workgroups, "iterations": iterations, "flops_per_launch": flops,
+              "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s"}
+    for name, data in operands.items():
+        def launch():
+            _native.check(_native.lib().singe_hip_mfma_ceiling(handle, data.data_ptr(), data.numel() * 2, out.data_ptr(),
+                                                               out.numel(), workgroups, iterations, 0), "mfma_ceiling")
+        stats = measure(launch, 1)
+        tflops = flops / (stats["mean_ms"] * 1e-3) / 1e12
+        result[name] = {"value": tflops, "frac_of_peak": tflops / MFMA_BF16_PEAK_TFLOPS, **timing_fields(stats)}
+    return result
+
+
+def decode_section(args, with_cpu):
+    """The headline: --warmup untimed steps, exactly --steps timed steps between two synchronisations, then the split
+    kernel alone under HIP events."""
     import numpy as np
     import torch
 
     from singe_amd import _native, synthetic
     from singe_amd.kernel import attention as A
 
-    assert torch.cuda.is_available(), "bench.py needs a GPU"
-    torch.cuda.set_device(0)
-    if args.only_latent:
-        print(json.dumps({"latent": latent_section(4)}), flush=True)
-        return
     if args.workers:
         _native.lib().singe_hip_set_decode_workers(args.workers)
-
     work = synthetic.paged_decode_workload()
     pools = [(work.key_cache, work.value_cache)]
     for extra in range(1, POOLS):
@@ -400,95 +594,90 @@ def main():
     table = torch.from_numpy(work.block_table.view(np.int32)).cuda()
     out = torch.empty((work.batch, work.heads, work.head_dim), device="cuda", dtype=torch.bfloat16)
     workspace = torch.empty(config.workspace_bytes(), dtype=torch.uint8, device="cuda")
+    counter = [0]
 
-    def step(i, phases=3):
-        kc, vc = pools[i % POOLS]
+    def step(phases=3):
+        kc, vc = pools[counter[0] % POOLS]
+        counter[0] += 1
         A.paged_kv_decode_attention_bf16(None, out, work.query, kc, vc, lens, table, config, workspace, phases)
 
-    for i in range(args.warmup):
-        step(i)
+    for _ in range(args.warmup):
+        step()
     torch.cuda.synchronize()
     start = time.perf_counter()
-    for i in range(args.steps):
-        step(i)
+    for _ in range(args.steps):
+        step()
     torch.cuda.synchronize()
     seconds = time.perf_counter() - start
     ms_per_step = seconds / args.steps * 1e3
 
-    # The dominant kernel alone (the split kernel): HIP events on its own stream around groups of
-    # back-to-back launches (one per KV pool in turn), so the cost of recording an event is spread
-    # over the group instead of being charged to one ~50 us launch.
-    group = 6
-    groups = max(args.steps // group, 5)
-    begin = [torch.cuda.Event(enable_timing=True) for _ in range(groups)]
-    finish = [torch.cuda.Event(enable_timing=True) for _ in range(groups)]
-    for j in range(groups):
-        begin[j].record()
-        for i in range(group):
-            step(j * group + i, phases=1)
-        finish[j].record()
-    torch.cuda.synchronize()
-    kernel_ms = sorted(b.elapsed_time(f) / group for b, f in zip(begin, finish))
-    kernel_avg_ms = sum(kernel_ms) / len(kernel_ms)
-
+    whole = measure(step, 6)               # the op under events: split + reduce
+    kernel = measure(lambda: step(1), 6)   # the dominant kernel alone
     bytes_per_step = work.algorithmic_bytes()
     value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
-    achieved = bytes_per_step / (kernel_avg_ms * 1e-3) / 1e9
+    achieved = bytes_per_step / (kernel["mean_ms"] * 1e-3) / 1e9
+    counted, source = traffic("decode") if not args.workers else (None, None)
     result = {
-        "metric": "decode attn GB/s",
-        "value": value,
-        "unit": "GB/s",
-        "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "bf16",
+        "metric": "decode attn GB/s", "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {
             "workload": "paged decode: batch 32, 32q/8kv heads, head_dim 128, bf16, block 16, "
                         "ctx U[512,4096], 16384-block pool (BASELINE config 2)",
-            "total_keys": work.total_keys,
-            "algorithmic_bytes": bytes_per_step,
-            "algorithmic_flops": work.algorithmic_flops(),
-            "workers": int(_native.lib().singe_hip_decode_workers(config._c())),
-            "kv_pools_rotated": POOLS,
+            "total_keys": work.total_keys, "algorithmic_bytes": bytes_per_step, "algorithmic_flops": work.algorithmic_flops(),
+            "workers": int(_native.lib().singe_hip_decode_workers(config._c())), "kv_pools_rotated": POOLS,
         },
         "tokens_per_s": work.batch / (ms_per_step * 1e-3),
         "pct_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
-        "roofline": {
-            "bound": "hbm",
-            "kernel": "singe_paged_decode_bf16_d128_g1_b16",
-            "achieved": achieved,
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": DECODE_TRAFFIC_BYTES if not args.workers else None,
-            "kernel_avg_us": kernel_avg_ms * 1e3,
-            "kernel_median_us": kernel_ms[len(kernel_ms) // 2] * 1e3,
-        },
+        "step_under_events": {"mean_us": whole["mean_ms"] * 1e3, "median_us": whole["median_ms"] * 1e3,
+                              "p25_us": whole["p25_ms"] * 1e3, "p75_us": whole["p75_ms"] * 1e3, "samples": whole["samples"],
+                              "pct_hbm_peak": 100.0 * bytes_per_step / (whole["mean_ms"] * 1e-3) / 1e9 / HBM_PEAK_GBPS},
+        "roofline": {"bound": "hbm", "kernel": "singe_paged_decode_bf16_d128_g1_b16", "achieved": achieved, "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": counted, "traffic_source": source,
+                     **timing_fields(kernel)},
     }
-    if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(work)
-    if not args.no_prefill:
-        del pools, workspace
+    if with_cpu:
+        result["cpu_baseline"] = decode_cpu_baseline(work)
+    return result
+
+
+def main():
+    global FEW
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no cross-GPU exchange and every box here has one "
+              "GPU; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    with_cpu = not args.no_cpu_baseline
+    FEW = bool(args.few and args.only)
+    sections = {
+        "prefill": lambda: prefill_section(with_cpu), "chunked_prefill": lambda: chunked_prefill_section(with_cpu),
+        "fp8_decode": lambda: fp8_decode_section(with_cpu), "dense_f32": lambda: dense_f32_section(with_cpu),
+        "latent": latent_section, "head_dim_64": head_dim_64_section, "mfma_ceiling": mfma_ceiling_section,
+    }
+    if args.only and args.only != "decode":
+        print(json.dumps({args.only: sections[args.only]()}), flush=True)
+        return
+    result = decode_section(args, with_cpu)
+    if args.only == "decode" or args.no_extras:
+        print(json.dumps(result), flush=True)
+        return
+    from singe_amd import error
+
+    for name, run in sections.items():
         torch.cuda.empty_cache()
-        result["prefill"] = prefill_section(args.prefill_steps)
-    if not args.no_extras:
         try:
-            del pools, workspace
-        except NameError:
-            pass
-        torch.cuda.empty_cache()
-        result["chunked_prefill"] = chunked_prefill_section(20)
-        torch.cuda.empty_cache()
-        result["fp8_decode"] = fp8_decode_section(10)
-        torch.cuda.empty_cache()
-        result["dense_f32"] = dense_f32_section(100)
-        torch.cuda.empty_cache()
-        result["latent"] = latent_section(8)
+            result[name] = run()
+        except error.UnsupportedWidth as refused:  # a width this build has no kernel for is said, not hidden
+            result[name] = {"unsupported": str(refused)}
+    ceiling = result["mfma_ceiling"]["normal"]["value"]
+    for name in ("prefill", "chunked_prefill"):
+        result[name]["roofline"]["frac_of_measured_ceiling"] = result[name]["roofline"]["achieved"] / ceiling
     print(json.dumps(result), flush=True)
 
 

@@ -906,6 +906,15 @@ SINGE_HIP_API int32_t singe_hip_paging_indices(
     uint32_t* status,
     const SingePagingIndicesProblem* problem);
 
+/* A measurement aid with no counterpart in the reference: `iterations` rounds of 32 register-only
+ * v_mfma_f32_32x32x16 products per wave (bf16, or f16 when `f16` is set), `workgroups` workgroups of four waves, on
+ * operands read once from `operands` (16-byte chunks, taken modulo the buffer).  No LDS, no softmax, no memory traffic
+ * inside the loop: the rate it reaches is the matrix cores' own ceiling on that data (the clock under such a loop is
+ * set by power, and power by the operands' bits), which the prefill kernels are priced against beside the published
+ * peak.  Flop per launch = workgroups * 4 * iterations * 32 * 32768.  `out` takes one float per lane. */
+SINGE_HIP_API int32_t singe_hip_mfma_ceiling(void* stream, const void* operands, size_t operand_bytes, float* out,
+                                             size_t out_len, uint32_t workgroups, uint32_t iterations, int32_t f16);
+
 #ifdef __cplusplus
 }
 #endif

@@ -188,6 +188,21 @@ def fmha_prefill_lse_f32(query, key, value, *, batch, query_len, key_len, heads,
     return out.reshape(batch, query_len, heads, head_dim), lse.reshape(batch, heads, query_len)
 
 
+def fmha_prefill_lse_f32_literal(query, key, value, *, batch, query_len, key_len, heads, kv_heads, head_dim,
+                                 scale, causal, row_first=0, row_count=None):
+    """fmha_prefill_lse_f32 with the reference's loop shape kept literally (cpu/attention.rs:1776-1830), on query rows
+    [row_first, row_first + row_count) of every (batch, head); the other rows stay zero."""
+    query, key, value = _f32(query), _f32(key), _f32(value)
+    out = np.empty(batch * query_len * heads * head_dim, dtype=np.float32)
+    lse = np.empty(batch * heads * query_len, dtype=np.float32)
+    count = query_len - row_first if row_count is None else row_count
+    lib().oracle_fmha_prefill_lse_f32_literal(_ptr(out), _ptr(lse), _ptr(query), _ptr(key), _ptr(value),
+                                              _c_size(batch), _c_size(query_len), _c_size(key_len),
+                                              _c_size(heads), _c_size(kv_heads), _c_size(head_dim),
+                                              _c_float(scale), _c_int(bool(causal)), _c_size(row_first), _c_size(count))
+    return out.reshape(batch, query_len, heads, head_dim), lse.reshape(batch, heads, query_len)
+
+
 def softcapped_window_attention_f32(query, key, value, *, batch, query_len, key_len, heads, kv_heads,
                                     head_dim, scale, causal, window_size=0, soft_cap=None, threads=1):
     """singe-kernel/src/cpu/attention.rs:1835-1925 (BHSD)."""

@@ -354,6 +354,57 @@ ORACLE_API void oracle_fmha_prefill_lse_f32(
     }
 }
 
+/* Same function with the reference's loop shape kept literally (cpu/attention.rs:1776-1830): one thread, the
+ * weight expf(s - max) / denom re-evaluated for every output dimension; restricted to query rows
+ * [row_first, row_first + row_count) of every (batch, head), so a benchmark can time a stated share of the rows.
+ * Rows outside the range keep out = 0 and lse = 0. */
+ORACLE_API void oracle_fmha_prefill_lse_f32_literal(
+    float *out, float *lse, const float *query, const float *key, const float *value, size_t batch,
+    size_t query_len, size_t key_len, size_t heads, size_t kv_heads, size_t head_dim, float scale,
+    int causal, size_t row_first, size_t row_count) {
+    size_t q_features = heads * head_dim, kv_features = kv_heads * head_dim;
+    size_t group = heads / kv_heads;
+    memset(out, 0, batch * query_len * q_features * sizeof(float));
+    memset(lse, 0, batch * heads * query_len * sizeof(float));
+    size_t row_end = row_first + row_count < query_len ? row_first + row_count : query_len;
+    float *scores = (float *)malloc((key_len ? key_len : 1) * sizeof(float));
+    size_t *kept = (size_t *)malloc((key_len ? key_len : 1) * sizeof(size_t));
+    for (size_t b = 0; b < batch; ++b) {
+        for (size_t head = 0; head < heads; ++head) {
+            size_t kv_head = head / group;
+            for (size_t query_index = row_first; query_index < row_end; ++query_index) {
+                size_t count = 0;
+                for (size_t key_index = 0; key_index < key_len; ++key_index) {
+                    if (causal && key_index > query_index) continue;
+                    float score = 0.0f;
+                    for (size_t d = 0; d < head_dim; ++d) {
+                        size_t qo = b * query_len * q_features + query_index * q_features + head * head_dim + d;
+                        size_t ko = b * key_len * kv_features + key_index * kv_features + kv_head * head_dim + d;
+                        score = fmaf(query[qo], key[ko], score);
+                    }
+                    kept[count] = key_index;
+                    scores[count++] = score * scale;
+                }
+                float largest = fold_max(scores, count);
+                float denom = 0.0f;
+                for (size_t j = 0; j < count; ++j) denom += expf(scores[j] - largest);
+                lse[b * heads * query_len + head * query_len + query_index] = largest + logf(denom);
+                for (size_t d = 0; d < head_dim; ++d) {
+                    float sum = 0.0f;
+                    for (size_t j = 0; j < count; ++j) {
+                        float weight = expf(scores[j] - largest) / denom;
+                        size_t vo = b * key_len * kv_features + kept[j] * kv_features + kv_head * head_dim + d;
+                        sum = fmaf(weight, value[vo], sum);
+                    }
+                    out[b * query_len * q_features + query_index * q_features + head * head_dim + d] = sum;
+                }
+            }
+        }
+    }
+    free(kept);
+    free(scores);
+}
+
 /* singe-kernel/src/cpu/attention.rs:1835-1925  softcapped_window_attention_f32.
  * query/out [batch, heads, query_len, dim] (BHSD), key/value
  * [batch, kv_heads, key_len, dim].  window_size 0 = no window; otherwise keys

@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIBRARY_PATH = os.path.join(_HERE, "libsinge_hip_attention.so")
 CODE_OBJECT_PARTS = ("paged_decode", "fmha_prefill", "fmha_prefill_f32", "paged_attention", "splitk_reduce",
                      "attention_rows_f32", "cache_ops", "latent_attention", "latent_attention_mfma",
-                     "general_attention_f32", "general_attention_bf16", "general_attention_f16")
+                     "general_attention_f32", "general_attention_bf16", "general_attention_f16", "mfma_ceiling")
 CODE_OBJECT_PATHS = [os.path.join(_HERE, f"singe_attention_gfx950.{part}.hsaco") for part in CODE_OBJECT_PARTS]
 
 c_size = ctypes.c_size_t
@@ -151,6 +151,8 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_unload.restype = None
     handle.singe_hip_kernel.argtypes = [i32, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(ctypes.c_char_p)]
     handle.singe_hip_kernel.restype = i32
+    handle.singe_hip_mfma_ceiling.argtypes = [c_void, c_void, c_size, c_void, c_size, ctypes.c_uint32, ctypes.c_uint32, i32]
+    handle.singe_hip_mfma_ceiling.restype = i32
     handle.singe_hip_prepare.argtypes = [ctypes.POINTER(i32)]
     handle.singe_hip_prepare.restype = i32
     cfg = ctypes.POINTER(PagedKvDecodeAttentionConfigC)

@@ -44,9 +44,11 @@ PARTS = [
     ("general_attention_f32", "general_attention.hip", ["-DSINGE_GENERAL_ELEMENT=0"]),
     ("general_attention_bf16", "general_attention.hip", ["-DSINGE_GENERAL_ELEMENT=1"]),
     ("general_attention_f16", "general_attention.hip", ["-DSINGE_GENERAL_ELEMENT=2"]),
+    ("mfma_ceiling", "mfma_ceiling.hip", []),
 ]
 HOST_SOURCES = ["hip_runtime_loader.cpp", "module.cpp", "paged_decode.cpp", "fmha_prefill.cpp", "paged_attention.cpp",
-                "general_attention.cpp", "fmha_decode.cpp", "paged_rows_f32.cpp", "latent_attention.cpp", "cache_ops.cpp"]
+                "general_attention.cpp", "fmha_decode.cpp", "paged_rows_f32.cpp", "latent_attention.cpp", "cache_ops.cpp",
+                "mfma_ceiling.cpp"]
 JOBS = 8
 
 

@@ -146,6 +146,14 @@ struct PagedAttentionArgs {
     float query_eps = 0.0f;
 };
 
+// singe_mfma_ceiling_*: the register-only product loop.
+struct MfmaCeilingArgs {
+    const void* operands;   // operand_chunks 16-byte chunks of bf16 / f16 data
+    float* out;             // one float per lane of the launch
+    uint64_t operand_chunks;
+    uint32_t iterations;
+};
+
 // singe_splitk_reduce_f32: strides in elements.
 struct SplitKReduceArgs {
     float* out;         // [batch, heads, dim]

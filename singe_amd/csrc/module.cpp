@@ -66,6 +66,7 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_attention_general_f32_d64", "singe_paged_attention_general_f32_d128", "singe_paged_attention_general_f32_d256",
     "singe_paged_attention_general_bf16_d64", "singe_paged_attention_general_bf16_d128", "singe_paged_attention_general_bf16_d256",
     "singe_paged_attention_general_f16_d64", "singe_paged_attention_general_f16_d128", "singe_paged_attention_general_f16_d256",
+    "singe_mfma_ceiling_bf16", "singe_mfma_ceiling_f16",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -74,7 +75,7 @@ const char* const kKernelNames[kKernelCount] = {
 const char* const kPartNames[kPartCount] = {
     "paged_decode", "fmha_prefill", "fmha_prefill_f32", "paged_attention", "splitk_reduce", "attention_rows_f32",
     "cache_ops", "latent_attention", "latent_attention_mfma", "general_attention_f32", "general_attention_bf16",
-    "general_attention_f16",
+    "general_attention_f16", "mfma_ceiling",
 };
 
 namespace {
@@ -86,6 +87,7 @@ constexpr PartRun kPartRuns[] = {
     {0, 14}, {1, 8}, {2, 4}, {3, 28}, {4, 1}, {5, 28}, {6, 5}, {7, 3}, {8, 4},
     {9, 3}, {10, 3}, {11, 3},  // dense general kernels: f32, bf16, f16
     {9, 3}, {10, 3}, {11, 3},  // paged general kernels
+    {12, 2},
 };
 constexpr int runs_total() {
     int total = 0;

@@ -45,13 +45,15 @@ enum KernelId : int {
     // general kernels: index = base + 3 * element (f32, bf16, f16) + width (64, 128, 256)
     kDenseGeneral,
     kPagedGeneral = kDenseGeneral + 9,
-    kKernelCount = kPagedGeneral + 9
+    // the register-only product loop a prefill kernel is priced against
+    kMfmaCeilingBf16 = kPagedGeneral + 9, kMfmaCeilingF16,
+    kKernelCount
 };
 
 extern const char* const kKernelNames[kKernelCount];
 
 // Parts of the code object (one file each) and the part a kernel lives in.
-constexpr int kPartCount = 12;
+constexpr int kPartCount = 13;
 extern const char* const kPartNames[kPartCount];
 int kernel_part(int kernel);
 

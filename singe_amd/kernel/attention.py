@@ -57,7 +57,19 @@ class PagedKvDecodeAttentionConfig:
         """mod.rs:686-709: builds the config and validates it."""
         config = cls(batch, heads, kv_heads, head_dim, block_size, physical_blocks, block_table_batch_stride, scale)
         config.validate()
+        config.reserve_workspace()
         return config
+
+    def reserve_workspace(self, device: "torch.device | None" = None) -> None:
+        """Sizes this module's per-device scratch for the config now, so that a decode call without a ``workspace``
+        of its own allocates nothing (the call is then enqueue-only, legal under stream capture, as the reference
+        asks of its launch functions: singe-kernel/src/cuda/mod.rs:3-12).  Without a visible GPU it does nothing."""
+        if not torch.cuda.is_available():
+            return
+        device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+        need = self.workspace_bytes()
+        if need > 0:
+            _workspaces.get(device, need)
 
     def validate(self) -> None:
         """validate_paged_kv_decode_attention_config (mod.rs:2963-2985)."""

@@ -635,3 +635,22 @@ def test_paged_mla_attention_against_a_float64_restatement_and_closed_forms():
     # The paging error contract is the op's (spec/neural/attention.rs:372-406).
     assert oracle.paged_mla_attention(q[:1], qp[:1], lc, pc, [0, 1], [0, 1], [pages], [1])[0] == 1
     assert oracle.paged_mla_attention(q[:1], qp[:1], lc, pc, [0, 2], [0, 1], [0], [1])[0] == 1
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_prefill_literal_loop_equals_the_hoisted_one_bit_for_bit(causal):
+    """The benchmark's single-thread CPU line keeps the reference's loop shape (cpu/attention.rs:1776-1830: the weight
+    re-evaluated per output dimension); it must give the bits of the restatement every parity test uses, on the rows it
+    is asked for, and leave the others alone."""
+    rng = np.random.default_rng(17)
+    batch, query_len, key_len, heads, kv_heads, dim = 2, 9, 13, 4, 2, 8
+    q = rng.standard_normal((batch, query_len, heads, dim)).astype(np.float32)
+    k = rng.standard_normal((batch, key_len, kv_heads, dim)).astype(np.float32)
+    v = rng.standard_normal((batch, key_len, kv_heads, dim)).astype(np.float32)
+    kw = dict(batch=batch, query_len=query_len, key_len=key_len, heads=heads, kv_heads=kv_heads, head_dim=dim, scale=0.3, causal=causal)
+    want, want_lse = oracle.fmha_prefill_lse_f32(q, k, v, **kw)
+    got, got_lse = oracle.fmha_prefill_lse_f32_literal(q, k, v, **kw)
+    assert np.array_equal(got, want) and np.array_equal(got_lse, want_lse)
+    part, part_lse = oracle.fmha_prefill_lse_f32_literal(q, k, v, row_first=3, row_count=4, **kw)
+    assert np.array_equal(part[:, 3:7], want[:, 3:7]) and np.array_equal(part_lse[:, :, 3:7], want_lse[:, :, 3:7])
+    assert not part[:, :3].any() and not part[:, 7:].any()
