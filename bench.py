@@ -660,6 +660,12 @@ def main():
         "fp8_decode": lambda: fp8_decode_section(with_cpu), "dense_f32": lambda: dense_f32_section(with_cpu),
         "latent": latent_section, "head_dim_64": head_dim_64_section, "mfma_ceiling": mfma_ceiling_section,
     }
+    if FEW:
+        # A copy of known size beside the kernel, for the unit of the profiler's byte counters: torch's f32 -> bf16
+        # copy of 2^28 elements reads 1 GiB and writes 512 MiB.
+        torch.empty(1 << 28, device="cuda", dtype=torch.float32).to(torch.bfloat16)
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
     if args.only and args.only != "decode":
         print(json.dumps({args.only: sections[args.only]()}), flush=True)
         return

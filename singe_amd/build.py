@@ -45,6 +45,9 @@ PARTS = [
     ("general_attention_bf16", "general_attention.hip", ["-DSINGE_GENERAL_ELEMENT=1"]),
     ("general_attention_f16", "general_attention.hip", ["-DSINGE_GENERAL_ELEMENT=2"]),
     ("mfma_ceiling", "mfma_ceiling.hip", []),
+    ("paged_decode_d64", "paged_decode.hip", ["-DSINGE_HEAD_DIM=64"]),
+    ("fmha_prefill_d64", "fmha_prefill.hip", ["-DSINGE_HEAD_DIM=64"]),
+    ("paged_attention_d64", "paged_attention.hip", ["-DSINGE_HEAD_DIM=64"]),
 ]
 HOST_SOURCES = ["hip_runtime_loader.cpp", "module.cpp", "paged_decode.cpp", "fmha_prefill.cpp", "paged_attention.cpp",
                 "general_attention.cpp", "fmha_decode.cpp", "paged_rows_f32.cpp", "latent_attention.cpp", "cache_ops.cpp",

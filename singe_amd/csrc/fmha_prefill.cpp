@@ -148,7 +148,20 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
         return status;
 
     // What the gfx950 kernel takes: head_dim 128 and rows it can fetch 16 bytes at a time.
-    if (c.head_dim != 128) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, f16 ? "fmha_prefill_f16" : "fmha_prefill_bf16", c.head_dim, 0);
+    if (c.head_dim != 128 && c.head_dim != 64) {
+        // Other head dimensions (the reference's matrix path takes 16 and 32 too: fmha.rs:752-755) run on the
+        // one-wave-per-row kernel, up to 256; without the dense op's options, which only reach here at 64 and 128.
+        DenseGeneralOperands o;
+        o.query = query, o.key = key, o.value = value, o.out = out, o.lse = with_lse ? lse : nullptr;
+        o.query_strides[0] = c.query_batch_stride, o.query_strides[1] = c.query_head_stride, o.query_strides[2] = c.query_sequence_stride;
+        o.key_strides[0] = c.key_batch_stride, o.key_strides[1] = c.key_head_stride, o.key_strides[2] = c.key_sequence_stride;
+        o.value_strides[0] = c.value_batch_stride, o.value_strides[1] = c.value_head_stride, o.value_strides[2] = c.value_sequence_stride;
+        o.out_strides[0] = c.output_batch_stride, o.out_strides[1] = c.output_head_stride, o.out_strides[2] = c.output_sequence_stride;
+        o.batch = c.batch, o.heads = c.heads, o.kv_heads = c.kv_heads, o.query_len = c.query_len, o.key_len = c.key_len;
+        o.head_dim = o.value_dim = c.head_dim;
+        o.causal = c.causal != 0, o.scale = c.scale;
+        return dense_general(f16 ? SINGE_HIP_F16 : SINGE_HIP_BF16, stream, f16 ? "fmha_prefill_f16" : "fmha_prefill_bf16", o);
+    }
     const size_t strides[] = {c.query_batch_stride, c.key_batch_stride, c.value_batch_stride, c.output_batch_stride,
                               c.query_sequence_stride, c.key_sequence_stride, c.value_sequence_stride,
                               c.output_sequence_stride, c.query_head_stride, c.key_head_stride,
@@ -208,7 +221,7 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
     const uint64_t groups = rows * ((args.query_tiles + 1) / 2);  // a workgroup takes a pair of query tiles
     if (groups > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
     const KernelId kernel = static_cast<KernelId>((f16 ? kPrefillCausalF16 : kPrefillCausal) + (c.causal ? 0 : 1) + (with_options ? 4 : 0));
-    return launch(kernel, static_cast<unsigned>(groups), 1, 1, 64 * kDensePrefillWaves, stream, args);
+    return launch(c.head_dim == 64 ? at_head_dim_64(kernel) : kernel, static_cast<unsigned>(groups), 1, 1, 64 * kDensePrefillWaves, stream, args);
 }
 
 }  // namespace

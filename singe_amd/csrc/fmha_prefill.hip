@@ -1,4 +1,4 @@
-// Dense flash-attention prefill, bf16, head_dim 128, optional top-left causal mask, grouped KV heads
+// Dense flash-attention prefill, bf16 or f16, head_dim 128 or 64 (one build each), optional top-left causal mask, grouped KV heads
 // (the GPU counterpart of singe-kernel/src/cpu/attention.rs:1758-1833 fmha_prefill_lse_f32, replacing
 // the cuTile fmha_prefill / fmha_prefill_mma kernels: singe-kernel/src/cuda/attention/fmha.rs:584-790).
 // query/out [batch, query_len, heads, 128], key/value [batch, key_len, kv_heads, 128] with element
@@ -67,11 +67,11 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     const float factor = fabsf(a.scale_log2e);
     const unsigned int flip = a.scale_log2e < 0.0f ? 0x80008000u : 0u;
     const Half half{};
-    uint4 q[8];
+    uint4 q[kSteps];
     {
         const uint16_t* row = q_base + static_cast<size_t>(query_valid ? my_query : 0) * a.query_sequence_stride + 8 * hi;
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
+        for (int s = 0; s < kSteps; ++s) {
             uint4 bits = *reinterpret_cast<const uint4*>(row + 16 * s);
             if (!query_valid) bits = make_uint4(0, 0, 0, 0);
             bits.x ^= flip; bits.y ^= flip; bits.z ^= flip; bits.w ^= flip;
@@ -101,12 +101,16 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     const unsigned int value_stride_bytes = static_cast<unsigned int>(a.value_sequence_stride) * 2u;
     const unsigned int load_row = 4u * wave + (lane >> 4), position = lane & 15u;
     const unsigned int key_chunk = (position ^ (load_row & 15u)) * 16u, value_chunk = (position ^ (4u * (load_row & 3u))) * 16u;
+    // At head_dim 64 a global row has eight chunks: the lanes whose position holds one of the other eight fetch nothing.
+    const bool key_lane_live = key_chunk < kGlobalRowBytes, value_lane_live = value_chunk < kGlobalRowBytes;
     // A tile that lies wholly inside the keys is addressed as a scalar base (tile and instruction) plus a
     // per-lane offset that never changes, so its loads cost no vector arithmetic; the last, partial tile
     // clamps each row (rows past the end re-read the last key and are masked).
     const unsigned int key_lane = load_row * key_stride_bytes + key_chunk, value_lane = load_row * value_stride_bytes + value_chunk;
     auto load_tile = [&](const unsigned char* rows, unsigned int stride_bytes, unsigned int lane_offset, unsigned int chunk,
-                         unsigned int tile, unsigned char* stage) __attribute__((always_inline)) {
+                         bool lane_live, unsigned int tile, unsigned char* stage) __attribute__((always_inline)) {
+        // (only the load itself is predicated, so that the scalar address arithmetic stays outside the branch)
+        const bool fetch = kGlobalRowBytes == kRowBytes || lane_live;
         if (tile * kKeyTile + kKeyTile <= key_len) {
             const unsigned char* base = rows + static_cast<size_t>(tile * kKeyTile) * stride_bytes;
             asm("" : "+s"(base));  // a scalar the compiler cannot fold the lane's part into
@@ -116,24 +120,26 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
                 // load out of its scalar-base form and cost a 64-bit add per lane.
                 unsigned int offset = lane_offset + kLoadRows * i * stride_bytes;
                 asm volatile("" : "+v"(offset));
-                __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(base + offset),
-                                                 (lds_words_t)(stage + (kLoadRows * i + 4u * wave) * kRowBytes), 16, 0, 0);
+                if (fetch)
+                    __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(base + offset),
+                                                     (lds_words_t)(stage + (kLoadRows * i + 4u * wave) * kRowBytes), 16, 0, 0);
             }
         } else {
 #pragma unroll
             for (unsigned int i = 0; i < kLoads; ++i) {
                 unsigned int key = tile * kKeyTile + kLoadRows * i + load_row;
                 key = key < key_len ? key : key_len - 1;
-                __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(rows + (key * stride_bytes + chunk)),
+                if (fetch)
+                    __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(rows + (key * stride_bytes + chunk)),
                                                  (lds_words_t)(stage + (kLoadRows * i + 4u * wave) * kRowBytes), 16, 0, 0);
             }
         }
     };
     auto load_keys = [&](unsigned int tile, unsigned char* stage) __attribute__((always_inline)) {
-        load_tile(k_bytes, key_stride_bytes, key_lane, key_chunk, tile, stage);
+        load_tile(k_bytes, key_stride_bytes, key_lane, key_chunk, key_lane_live, tile, stage);
     };
     auto load_values = [&](unsigned int tile, unsigned char* stage) __attribute__((always_inline)) {
-        load_tile(v_bytes, value_stride_bytes, value_lane, value_chunk, tile, stage);
+        load_tile(v_bytes, value_stride_bytes, value_lane, value_chunk, value_lane_live, tile, stage);
     };
 
     RowState state;
@@ -283,7 +289,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
         }
     }
     unsigned int tile = first_tile;
-    uint4 operand[8];
+    uint4 operand[kSteps];
     auto issue = [&](unsigned char* key_dest, unsigned char* value_dest) __attribute__((always_inline)) {
         if (tile + 2 < tiles) load_keys(tile + 2, key_dest);
         if (tile + 1 < tiles) load_values(tile + 1, value_dest);
@@ -333,7 +339,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
         uint16_t* row = a.out + batch * a.output_batch_stride + static_cast<size_t>(my_query) * a.output_sequence_stride +
                         head * a.output_head_stride;
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < kDimBlocks; ++db)
 #pragma unroll
             for (int quad = 0; quad < 4; ++quad) {
                 uint2 packed;
@@ -373,11 +379,16 @@ SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
         fmha_prefill_body<CAUSAL, prefill::HALF, kDenseWaves, true>(args, prefill_lds);             \
     }
 
-SINGE_FMHA_PREFILL_OPTIONS_KERNEL(singe_fmha_prefill_bf16_d128_causal_options, true, Bf16)
-SINGE_FMHA_PREFILL_OPTIONS_KERNEL(singe_fmha_prefill_bf16_d128_full_options, false, Bf16)
-SINGE_FMHA_PREFILL_OPTIONS_KERNEL(singe_fmha_prefill_f16_d128_causal_options, true, F16)
-SINGE_FMHA_PREFILL_OPTIONS_KERNEL(singe_fmha_prefill_f16_d128_full_options, false, F16)
-SINGE_FMHA_PREFILL_KERNEL(singe_fmha_prefill_bf16_d128_causal, true, Bf16)
-SINGE_FMHA_PREFILL_KERNEL(singe_fmha_prefill_bf16_d128_full, false, Bf16)
-SINGE_FMHA_PREFILL_KERNEL(singe_fmha_prefill_f16_d128_causal, true, F16)
-SINGE_FMHA_PREFILL_KERNEL(singe_fmha_prefill_f16_d128_full, false, F16)
+// Names carry the head dimension of the build: singe_fmha_prefill_bf16_d128_causal, ..._d64_causal.
+#define SINGE_PASTE3_(a, b, c) a##b##c
+#define SINGE_PASTE3(a, b, c) SINGE_PASTE3_(a, b, c)
+#define SINGE_PREFILL_NAME(TYPE, TAIL) SINGE_PASTE3(singe_fmha_prefill_##TYPE##_d, SINGE_HEAD_DIM, TAIL)
+
+SINGE_FMHA_PREFILL_OPTIONS_KERNEL(SINGE_PREFILL_NAME(bf16, _causal_options), true, Bf16)
+SINGE_FMHA_PREFILL_OPTIONS_KERNEL(SINGE_PREFILL_NAME(bf16, _full_options), false, Bf16)
+SINGE_FMHA_PREFILL_OPTIONS_KERNEL(SINGE_PREFILL_NAME(f16, _causal_options), true, F16)
+SINGE_FMHA_PREFILL_OPTIONS_KERNEL(SINGE_PREFILL_NAME(f16, _full_options), false, F16)
+SINGE_FMHA_PREFILL_KERNEL(SINGE_PREFILL_NAME(bf16, _causal), true, Bf16)
+SINGE_FMHA_PREFILL_KERNEL(SINGE_PREFILL_NAME(bf16, _full), false, Bf16)
+SINGE_FMHA_PREFILL_KERNEL(SINGE_PREFILL_NAME(f16, _causal), true, F16)
+SINGE_FMHA_PREFILL_KERNEL(SINGE_PREFILL_NAME(f16, _full), false, F16)

@@ -49,6 +49,7 @@ int32_t paged_attention_general(int32_t data_type, void* stream, const void* que
     args.page_offsets = page_offsets;
     args.pages = pages;
     args.last_page_lengths = last_page_lengths;
+    args.query_lengths = nullptr;
     args.output = output;
     args.lse = lse;
     args.status = status;
@@ -65,11 +66,97 @@ int32_t paged_attention_general(int32_t data_type, void* stream, const void* que
     args.row_blocks = static_cast<uint32_t>(row_blocks);
     args.causal = p.causal ? 1u : 0u;
     args.has_softcap = p.has_softcap ? 1u : 0u;
-    args.wide_index = p.index_type == SINGE_HIP_INDEX_I64 ? 1u : 0u;
+    args.form = p.index_type == SINGE_HIP_INDEX_I64 ? 1u : 0u;
     args.scale = scale;
     args.softcap = p.has_softcap ? p.softcap : 0.0f;
     const uint64_t blocks = row_blocks * static_cast<uint64_t>(p.sequences);
     if (blocks > 0x7fffffffull || row_blocks > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
+    return launch(kernel, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+}
+
+// The block-table ops of the singe-kernel surface at head dimensions the matrix-core kernels are not built for
+// (the reference's own kernels take 4 to 64 there: singe-kernel/src/cuda/cutile/attention/paged.rs:799-810), on the
+// same one-wave-per-row kernel.  Prefill: `query_offsets`, `query_lengths`, `key_lengths` [sequences] i32; decode:
+// query_lengths null, one query per sequence at row `sequence`.
+int32_t paged_table_general(int32_t data_type, void* stream, const char* op, const void* query_rows, const void* key_cache,
+                            const void* value_cache, const int32_t* query_offsets, const int32_t* query_lengths,
+                            const int32_t* key_lengths, const uint32_t* block_table, void* output, float* lse, uint64_t tokens,
+                            uint64_t sequences, uint64_t heads, uint64_t kv_heads, uint64_t head_dim, uint64_t block_size,
+                            uint64_t physical_blocks, uint64_t table_stride, bool causal, float scale) {
+    KernelId kernel;
+    if (int32_t s = pick(kPagedGeneral, data_type, head_dim, op, &kernel)) return s;
+    const bool decode = query_lengths == nullptr;
+    GeneralPagedArgs args;
+    args.query_rows = query_rows;
+    args.key_cache = key_cache;
+    args.value_cache = value_cache;
+    args.query_offsets = query_offsets;
+    args.page_offsets = nullptr;
+    args.pages = block_table;
+    args.last_page_lengths = key_lengths;
+    args.query_lengths = query_lengths;
+    args.output = output;
+    args.lse = lse;
+    args.status = nullptr;
+    args.window = -1;
+    args.tokens = static_cast<uint32_t>(tokens);
+    args.heads = static_cast<uint32_t>(heads);
+    args.kv_heads = static_cast<uint32_t>(kv_heads);
+    args.head_dim = static_cast<uint32_t>(head_dim);
+    args.page_size = static_cast<uint32_t>(block_size);
+    args.sequences = static_cast<uint32_t>(sequences);
+    args.cache_pages = static_cast<uint32_t>(physical_blocks);
+    args.page_table = static_cast<uint32_t>(table_stride);
+    // A sequence holds at most every token (prefill) or one (decode).
+    const uint64_t row_blocks = ((decode ? 1 : tokens) * heads + 3) / 4;
+    args.row_blocks = static_cast<uint32_t>(row_blocks);
+    args.causal = causal ? 1u : 0u;
+    args.has_softcap = 0;
+    args.form = decode ? 3u : 2u;
+    args.scale = scale;
+    args.softcap = 0.0f;
+    const uint64_t blocks = row_blocks * sequences;
+    if (blocks > 0x7fffffffull || row_blocks > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
+    return launch(kernel, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+}
+
+// Dense attention through element strides on the one-wave-per-row kernel: the scaled-dot-product op below, and
+// fmha_prefill[_lse] of the singe-kernel surface at head dimensions the matrix-core kernels are not built for.
+int32_t dense_general(int32_t data_type, void* stream, const char* op, const DenseGeneralOperands& o) {
+    KernelId kernel;
+    const uint64_t widest = o.head_dim > o.value_dim ? o.head_dim : o.value_dim;
+    if (int32_t s = pick(kDenseGeneral, data_type, widest, op, &kernel)) return s;
+    GeneralAttentionArgs args;
+    args.query = o.query;
+    args.key = o.key;
+    args.value = o.value;
+    args.mask = o.mask;
+    args.sinks = o.sinks;
+    args.key_lengths = o.key_lengths;
+    args.out = o.out;
+    args.lse = o.lse;
+    for (int i = 0; i < 3; ++i) {
+        args.query_strides[i] = o.query_strides[i];
+        args.key_strides[i] = o.key_strides[i];
+        args.value_strides[i] = o.value_strides[i];
+        args.out_strides[i] = o.out_strides[i];
+    }
+    for (int i = 0; i < 4; ++i) args.mask_strides[i] = o.mask_strides[i];
+    args.window = o.window;
+    args.batch = static_cast<uint32_t>(o.batch);
+    args.heads = static_cast<uint32_t>(o.heads);
+    args.kv_heads = static_cast<uint32_t>(o.kv_heads);
+    args.query_len = static_cast<uint32_t>(o.query_len);
+    args.key_len = static_cast<uint32_t>(o.key_len);
+    args.head_dim = static_cast<uint32_t>(o.head_dim);
+    args.value_dim = static_cast<uint32_t>(o.value_dim);
+    args.causal = o.causal ? 1u : 0u;
+    args.has_softcap = o.has_softcap ? 1u : 0u;
+    args.scale = o.scale;
+    args.softcap = o.softcap;
+    const uint64_t rows = o.batch * o.heads * o.query_len;
+    const uint64_t blocks = (rows + 3) / 4;
+    if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
     return launch(kernel, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
 }
 
@@ -101,18 +188,20 @@ extern "C" int32_t singe_hip_scaled_dot_product_attention(void* stream, const vo
     if (output == nullptr) return fail(SINGE_HIP_NULL_POINTER, "output");
     const float scale = p.has_scale ? p.scale : 1.0f / std::sqrt(static_cast<float>(p.head_dim));
 
-    // bf16 and f16 at head dimension 128 are what the MFMA flash kernel computes, every option included, reading
-    // [batch, heads, len, dim] through its strides.
-    if ((p.data_type == SINGE_HIP_BF16 || p.data_type == SINGE_HIP_F16) && p.head_dim == 128 && p.value_dim == 128) {
+    // bf16 and f16 at head dimensions 128 and 64 are what the MFMA flash kernels compute, every option included,
+    // reading [batch, heads, len, dim] through their strides.
+    if ((p.data_type == SINGE_HIP_BF16 || p.data_type == SINGE_HIP_F16) && (p.head_dim == 128 || p.head_dim == 64) &&
+        p.value_dim == p.head_dim) {
+        const size_t dim = static_cast<size_t>(p.head_dim);
         SingeFmhaPrefillConfig c;
-        c.batch = p.batch, c.query_len = p.query_len, c.key_len = p.key_len, c.heads = p.heads, c.kv_heads = p.kv_heads, c.head_dim = 128;
-        c.query_batch_stride = c.output_batch_stride = static_cast<size_t>(p.heads) * p.query_len * 128;
-        c.key_batch_stride = c.value_batch_stride = static_cast<size_t>(p.kv_heads) * p.key_len * 128;
-        c.query_sequence_stride = c.key_sequence_stride = c.value_sequence_stride = c.output_sequence_stride = 128;
-        c.query_head_stride = c.output_head_stride = static_cast<size_t>(p.query_len) * 128;
-        c.key_head_stride = c.value_head_stride = static_cast<size_t>(p.key_len) * 128;
+        c.batch = p.batch, c.query_len = p.query_len, c.key_len = p.key_len, c.heads = p.heads, c.kv_heads = p.kv_heads, c.head_dim = dim;
+        c.query_batch_stride = c.output_batch_stride = static_cast<size_t>(p.heads) * p.query_len * dim;
+        c.key_batch_stride = c.value_batch_stride = static_cast<size_t>(p.kv_heads) * p.key_len * dim;
+        c.query_sequence_stride = c.key_sequence_stride = c.value_sequence_stride = c.output_sequence_stride = dim;
+        c.query_head_stride = c.output_head_stride = static_cast<size_t>(p.query_len) * dim;
+        c.key_head_stride = c.value_head_stride = static_cast<size_t>(p.key_len) * dim;
         c.scale = scale, c.causal = p.causal ? 1 : 0;
-        const size_t q_len = static_cast<size_t>(rows) * 128, kv_len = static_cast<size_t>(p.batch) * p.kv_heads * p.key_len * 128;
+        const size_t q_len = static_cast<size_t>(rows) * dim, kv_len = static_cast<size_t>(p.batch) * p.kv_heads * p.key_len * dim;
         DenseOptions options;
         options.sinks = static_cast<const uint16_t*>(sinks);
         options.key_lengths = key_lengths;
@@ -125,33 +214,21 @@ extern "C" int32_t singe_hip_scaled_dot_product_attention(void* stream, const vo
                                           static_cast<const uint16_t*>(value), kv_len, &c, options);
     }
 
-    KernelId kernel;
-    const uint64_t widest = static_cast<uint64_t>(p.head_dim > p.value_dim ? p.head_dim : p.value_dim);
-    if (int32_t s = pick(kDenseGeneral, p.data_type, widest, "scaled_dot_product_attention", &kernel)) return s;
-    GeneralAttentionArgs args;
-    args.query = query;
-    args.key = key;
-    args.value = value;
-    args.mask = mask;
-    args.sinks = sinks;
-    args.key_lengths = key_lengths;
-    args.out = output;
-    for (int i = 0; i < 4; ++i) args.mask_strides[i] = static_cast<uint64_t>(p.mask_strides[i]);
-    args.window = p.has_window ? p.window : -1;
-    args.batch = static_cast<uint32_t>(p.batch);
-    args.heads = static_cast<uint32_t>(p.heads);
-    args.kv_heads = static_cast<uint32_t>(p.kv_heads);
-    args.query_len = static_cast<uint32_t>(p.query_len);
-    args.key_len = static_cast<uint32_t>(p.key_len);
-    args.head_dim = static_cast<uint32_t>(p.head_dim);
-    args.value_dim = static_cast<uint32_t>(p.value_dim);
-    args.causal = p.causal ? 1u : 0u;
-    args.has_softcap = p.has_softcap ? 1u : 0u;
-    args.scale = scale;
-    args.softcap = p.has_softcap ? p.softcap : 0.0f;
-    const uint64_t blocks = (rows + 3) / 4;
-    if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
-    return launch(kernel, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+    DenseGeneralOperands o;
+    o.query = query, o.key = key, o.value = value, o.mask = mask, o.sinks = sinks, o.key_lengths = key_lengths, o.out = output;
+    const uint64_t dim = static_cast<uint64_t>(p.head_dim), value_dim = static_cast<uint64_t>(p.value_dim);
+    const uint64_t query_len = static_cast<uint64_t>(p.query_len), key_len = static_cast<uint64_t>(p.key_len);
+    o.query_strides[0] = p.heads * query_len * dim, o.query_strides[1] = query_len * dim, o.query_strides[2] = dim;
+    o.key_strides[0] = p.kv_heads * key_len * dim, o.key_strides[1] = key_len * dim, o.key_strides[2] = dim;
+    o.value_strides[0] = p.kv_heads * key_len * value_dim, o.value_strides[1] = key_len * value_dim, o.value_strides[2] = value_dim;
+    o.out_strides[0] = p.heads * query_len * value_dim, o.out_strides[1] = query_len * value_dim, o.out_strides[2] = value_dim;
+    for (int i = 0; i < 4; ++i) o.mask_strides[i] = static_cast<uint64_t>(p.mask_strides[i]);
+    o.window = p.has_window ? p.window : -1;
+    o.batch = p.batch, o.heads = p.heads, o.kv_heads = p.kv_heads, o.query_len = query_len, o.key_len = key_len;
+    o.head_dim = dim, o.value_dim = value_dim;
+    o.causal = p.causal != 0, o.has_softcap = p.has_softcap != 0;
+    o.scale = scale, o.softcap = p.has_softcap ? p.softcap : 0.0f;
+    return dense_general(p.data_type, stream, "scaled_dot_product_attention", o);
 }
 
 // validate_splitk_reduce_config (singe-kernel/src/cuda/attention/mod.rs:3557-3573) and

@@ -114,10 +114,9 @@ SINGE_DEVICE void dense_body(const GeneralAttentionArgs& a, float* lds) {
     const unsigned int head = static_cast<unsigned int>((row / a.query_len) % a.heads);
     const unsigned int batch = static_cast<unsigned int>(row / (static_cast<unsigned long long>(a.query_len) * a.heads));
     const unsigned int kv_head = head / (a.heads / a.kv_heads);
-    const size_t kv_unit = static_cast<size_t>(batch) * a.kv_heads + kv_head;
-    const T* q = static_cast<const T*>(a.query) + row * a.head_dim;
-    const T* k = static_cast<const T*>(a.key) + kv_unit * a.key_len * a.head_dim;
-    const T* v = static_cast<const T*>(a.value) + kv_unit * a.key_len * a.value_dim;
+    const T* q = static_cast<const T*>(a.query) + batch * a.query_strides[0] + head * a.query_strides[1] + query * a.query_strides[2];
+    const T* k = static_cast<const T*>(a.key) + batch * a.key_strides[0] + kv_head * a.key_strides[1];
+    const T* v = static_cast<const T*>(a.value) + batch * a.value_strides[0] + kv_head * a.value_strides[1];
     const T* mask = a.mask == nullptr ? nullptr
                                       : static_cast<const T*>(a.mask) + batch * a.mask_strides[0] + head * a.mask_strides[1] +
                                             query * a.mask_strides[2];
@@ -144,22 +143,36 @@ SINGE_DEVICE void dense_body(const GeneralAttentionArgs& a, float* lds) {
     reset(state);
     for (unsigned int key = first + lane; key < end; key += 64) {
         const float additive = mask != nullptr ? E::load(mask + key * a.mask_strides[3]) : 0.0f;
-        fold_key<E, DMAX>(state, q_row, k + static_cast<size_t>(key) * a.head_dim, v + static_cast<size_t>(key) * a.value_dim,
+        fold_key<E, DMAX>(state, q_row, k + static_cast<size_t>(key) * a.key_strides[2], v + static_cast<size_t>(key) * a.value_strides[2],
                           a.head_dim, a.value_dim, a.scale, a.has_softcap != 0, a.softcap, additive);
     }
     const float sink = a.sinks != nullptr ? E::load(static_cast<const T*>(a.sinks) + head) : -INFINITY;
-    finish_row<E, DMAX>(state, static_cast<T*>(a.out) + row * a.value_dim, a.value_dim, lane, sink);
+    T* out = static_cast<T*>(a.out) + batch * a.out_strides[0] + head * a.out_strides[1] + query * a.out_strides[2];
+    const float lse = finish_row<E, DMAX>(state, out, a.value_dim, lane, sink);
+    if (a.lse != nullptr && lane == 0) a.lse[row] = lse;  // row = (batch * heads + head) * query_len + query
 }
 
-template <uint32_t ELEMENT, int DMAX, int FORM>
+template <uint32_t ELEMENT, int DMAX, int FORM, bool DECODE = false>
 SINGE_DEVICE void paged_rows(const GeneralPagedArgs& a, float* lds) {
     typedef Element<ELEMENT> E;
     typedef typename E::type T;
     const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const unsigned int sequence = blockIdx.x / a.row_blocks;
     const unsigned int local_row = (blockIdx.x % a.row_blocks) * 4 + wave;  // (query, head) of the sequence
-    const SequenceSpan span = load_span<FORM>(sequence, a.query_offsets, a.page_offsets, a.last_page_lengths, nullptr, a.tokens,
-                                              a.page_table, a.page_size);
+    SequenceSpan span;
+    if (DECODE) {
+        // One query per sequence, at row `sequence`; a key count is clamped to what the table row addresses.
+        const int raw = static_cast<const int*>(a.last_page_lengths)[sequence];
+        const unsigned long long reach = static_cast<unsigned long long>(a.page_table) * a.page_size;
+        span.query_start = sequence;
+        span.page_start = static_cast<long long>(sequence) * a.page_table;
+        span.queries = 1;
+        span.keys = raw < 0 ? 0u : static_cast<unsigned int>(static_cast<unsigned long long>(raw) < reach ? static_cast<unsigned long long>(raw) : reach);
+        span.valid = true;
+    } else {
+        span = load_span<FORM>(sequence, a.query_offsets, a.page_offsets, a.last_page_lengths, a.query_lengths, a.tokens, a.page_table,
+                               a.page_size);
+    }
     if (!span.valid) {
         if (threadIdx.x == 0) report_index_error(a.status);
         return;
@@ -174,8 +187,10 @@ SINGE_DEVICE void paged_rows(const GeneralPagedArgs& a, float* lds) {
     for (unsigned int d = lane; d < a.head_dim; d += 64) q_row[d] = E::load(q + d);
     __builtin_amdgcn_wave_barrier();
 
-    // Bottom-right alignment with the CPU path's saturating position (attention.rs:482-488).
-    const long long raw = static_cast<long long>(span.keys) - static_cast<long long>(span.queries) + query;
+    // Bottom-right alignment with the CPU path's saturating position (attention.rs:482-488); the block-table form
+    // aligns a sequence's queries with its first keys (cpu/attention.rs:1283).
+    const long long raw = FORM == kTable ? static_cast<long long>(query)
+                                         : static_cast<long long>(span.keys) - static_cast<long long>(span.queries) + query;
     const unsigned int position = raw < 0 ? 0u : static_cast<unsigned int>(raw);
     unsigned int first = 0, end = span.keys;
     if (a.causal && position + 1 < end) end = position + 1;
@@ -192,19 +207,27 @@ SINGE_DEVICE void paged_rows(const GeneralPagedArgs& a, float* lds) {
         const unsigned long long page = read_page<FORM>(a.pages, static_cast<size_t>(span.page_start) + key / a.page_size);
         const bool valid = page < static_cast<unsigned long long>(a.cache_pages);
         if (!valid) report_index_error(a.status);
+        if (FORM == kTable && !valid) continue;  // a table entry that is no cache block hides its keys
         // A key behind a bad page id is read as zeros; the status word tells the caller.
         const size_t offset = ((page * a.page_size + key % a.page_size) * a.kv_heads + kv_head) * a.head_dim;
         fold_key<E, DMAX>(state, q_row, valid ? key_cache + offset : nullptr, valid ? value_cache + offset : nullptr, a.head_dim,
                           a.head_dim, a.scale, a.has_softcap != 0, a.softcap, 0.0f);
     }
     const float lse = finish_row<E, DMAX>(state, static_cast<T*>(a.output) + flat * a.head_dim, a.head_dim, lane, -INFINITY);
-    if (a.lse != nullptr && lane == 0) a.lse[flat] = lse * kLog2e;  // base two; -inf stays -inf
+    if (a.lse != nullptr && lane == 0) {
+        if (FORM == kTable) a.lse[flat] = lse == -INFINITY ? -1.0e20f : lse;  // natural log (cpu/attention.rs:1304-1317)
+        else a.lse[flat] = lse * kLog2e;                                      // base two; -inf stays -inf
+    }
 }
 
 template <uint32_t ELEMENT, int DMAX>
 SINGE_DEVICE void paged_body(const GeneralPagedArgs& a, float* lds) {
-    if (a.wide_index)
+    if (a.form == 1)
         paged_rows<ELEMENT, DMAX, kCsrI64>(a, lds);
+    else if (a.form == 2)
+        paged_rows<ELEMENT, DMAX, kTable>(a, lds);
+    else if (a.form == 3)
+        paged_rows<ELEMENT, DMAX, kTable, true>(a, lds);
     else
         paged_rows<ELEMENT, DMAX, kCsrI32>(a, lds);
 }

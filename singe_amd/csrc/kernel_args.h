@@ -212,6 +212,9 @@ struct GeneralAttentionArgs {
     const void* sinks;              // [heads], element type of the query; or null
     const int32_t* key_lengths;     // [batch]; or null
     void* out;                      // [batch, heads, query_len, value_dim]
+    float* lse;                     // [batch, heads, query_len] natural log, or null
+    // Element strides over (batch, head, position) of the query, key, value and output; a row's dims are contiguous.
+    uint64_t query_strides[3], key_strides[3], value_strides[3], out_strides[3];
     uint64_t mask_strides[4];       // over (batch, head, query, key); 0 broadcasts
     int64_t window;                 // -1 = none
     uint32_t batch, heads, kv_heads, query_len, key_len, head_dim, value_dim;
@@ -219,7 +222,12 @@ struct GeneralAttentionArgs {
     float scale, softcap;
 };
 
-// singe_paged_attention_general_*: the FlashInfer-form paged op for any element type and head dimension.
+// singe_paged_attention_general_*: the paged ops for any element type and head dimension.  `form`: the FlashInfer
+// form with i32 (0) or i64 (1) paging vectors (bottom-right causal, base-two lse, -inf for an empty row), or the
+// block-table form of the singe-kernel surface (top-left causal, natural-log lse, -1e20 for an empty row): prefill (2:
+// pages = the table, query_offsets / query_lengths / last_page_lengths = per-sequence i32 offsets, query counts and
+// key counts) and decode (3: one query per sequence at row `sequence`, last_page_lengths = the key counts, clamped
+// to what a table row addresses).
 struct GeneralPagedArgs {
     const void* query_rows;         // [tokens, heads, head_dim]
     const void* key_cache;          // [cache_pages, page_size, kv_heads, head_dim]
@@ -228,13 +236,14 @@ struct GeneralPagedArgs {
     const void* page_offsets;
     const void* pages;
     const void* last_page_lengths;
+    const void* query_lengths;      // form 2 only
     void* output;                   // [tokens, heads, head_dim]
-    float* lse;                     // [tokens, heads] base two, or null
+    float* lse;                     // [tokens, heads], or null
     uint32_t* status;
     int64_t window;
     uint32_t tokens, heads, kv_heads, head_dim, page_size, sequences, cache_pages, page_table;
     uint32_t row_blocks;            // workgroups (4 rows each) per sequence
-    uint32_t causal, has_softcap, wide_index;
+    uint32_t causal, has_softcap, form;
     float scale, softcap;
 };
 

@@ -67,6 +67,29 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_attention_general_bf16_d64", "singe_paged_attention_general_bf16_d128", "singe_paged_attention_general_bf16_d256",
     "singe_paged_attention_general_f16_d64", "singe_paged_attention_general_f16_d128", "singe_paged_attention_general_f16_d256",
     "singe_mfma_ceiling_bf16", "singe_mfma_ceiling_f16",
+    "singe_paged_decode_bf16_d64_g1_b16", "singe_paged_decode_bf16_d64_g2_b16",
+    "singe_paged_decode_bf16_d64_g1_any", "singe_paged_decode_bf16_d64_g2_any",
+    "singe_paged_decode_combine_bf16_d64", "singe_paged_decode_f16_d64_g1_b16",
+    "singe_paged_decode_f16_d64_g2_b16", "singe_paged_decode_f16_d64_g1_any",
+    "singe_paged_decode_f16_d64_g2_any", "singe_paged_decode_combine_f16_d64",
+    "singe_fmha_prefill_bf16_d64_causal", "singe_fmha_prefill_bf16_d64_full",
+    "singe_fmha_prefill_f16_d64_causal", "singe_fmha_prefill_f16_d64_full",
+    "singe_fmha_prefill_bf16_d64_causal_options", "singe_fmha_prefill_bf16_d64_full_options",
+    "singe_fmha_prefill_f16_d64_causal_options", "singe_fmha_prefill_f16_d64_full_options",
+    "singe_paged_attention_bf16_d64_i32", "singe_paged_attention_bf16_d64_i64",
+    "singe_paged_attention_bf16_d64_softcap_i32", "singe_paged_attention_bf16_d64_softcap_i64",
+    "singe_paged_attention_bf16_d64_i32_p16", "singe_paged_attention_bf16_d64_i64_p16",
+    "singe_paged_attention_bf16_d64_softcap_i32_p16", "singe_paged_attention_bf16_d64_softcap_i64_p16",
+    "singe_paged_kv_prefill_bf16_d64", "singe_paged_kv_prefill_bf16_d64_p16",
+    "singe_paged_kv_prefill_f16_d64", "singe_paged_kv_prefill_f16_d64_p16",
+    "singe_paged_attention_combine_bf16_d64_i32", "singe_paged_attention_combine_bf16_d64_i64",
+    "singe_paged_attention_combine_f16_d64_i32", "singe_paged_attention_combine_f16_d64_i64",
+    "singe_paged_attention_f16_d64_i32", "singe_paged_attention_f16_d64_i64",
+    "singe_paged_attention_f16_d64_softcap_i32", "singe_paged_attention_f16_d64_softcap_i64",
+    "singe_paged_attention_f16_d64_i32_p16", "singe_paged_attention_f16_d64_i64_p16",
+    "singe_paged_attention_f16_d64_softcap_i32_p16", "singe_paged_attention_f16_d64_softcap_i64_p16",
+    "singe_rotary_paged_attention_bf16_d64_i32", "singe_rotary_paged_attention_bf16_d64_i64",
+    "singe_rotary_paged_attention_bf16_d64_i32_p16", "singe_rotary_paged_attention_bf16_d64_i64_p16",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -75,7 +98,7 @@ const char* const kKernelNames[kKernelCount] = {
 const char* const kPartNames[kPartCount] = {
     "paged_decode", "fmha_prefill", "fmha_prefill_f32", "paged_attention", "splitk_reduce", "attention_rows_f32",
     "cache_ops", "latent_attention", "latent_attention_mfma", "general_attention_f32", "general_attention_bf16",
-    "general_attention_f16", "mfma_ceiling",
+    "general_attention_f16", "mfma_ceiling", "paged_decode_d64", "fmha_prefill_d64", "paged_attention_d64",
 };
 
 namespace {
@@ -88,6 +111,7 @@ constexpr PartRun kPartRuns[] = {
     {9, 3}, {10, 3}, {11, 3},  // dense general kernels: f32, bf16, f16
     {9, 3}, {10, 3}, {11, 3},  // paged general kernels
     {12, 2},
+    {13, 10}, {14, 8}, {15, 28},  // the head_dim 64 builds
 };
 constexpr int runs_total() {
     int total = 0;

@@ -47,13 +47,24 @@ enum KernelId : int {
     kPagedGeneral = kDenseGeneral + 9,
     // the register-only product loop a prefill kernel is priced against
     kMfmaCeilingBf16 = kPagedGeneral + 9, kMfmaCeilingF16,
-    kKernelCount
+    // the matrix-core kernels built for head_dim 64, each bank in the order of its head_dim 128 forms: the ten
+    // bf16 / f16 decode kernels from kDecodeBf16, the eight dense prefill kernels from kPrefillCausal, the paged
+    // attention kernels from kPagedAttentionI32 up to kSplitKReduce
+    kDecodeD64, kPrefillD64 = kDecodeD64 + 10, kPagedD64 = kPrefillD64 + 8,
+    kKernelCount = kPagedD64 + (kSplitKReduce - kPagedAttentionI32)
 };
+
+// The head_dim 64 build of a matrix-core kernel named by its head_dim 128 id.
+inline KernelId at_head_dim_64(KernelId kernel) {
+    if (kernel < kDecodeF8Wide) return static_cast<KernelId>(kDecodeD64 + kernel);
+    if (kernel >= kPrefillCausal && kernel < kPrefillF32D32) return static_cast<KernelId>(kPrefillD64 + (kernel - kPrefillCausal));
+    return static_cast<KernelId>(kPagedD64 + (kernel - kPagedAttentionI32));
+}
 
 extern const char* const kKernelNames[kKernelCount];
 
 // Parts of the code object (one file each) and the part a kernel lives in.
-constexpr int kPartCount = 13;
+constexpr int kPartCount = 16;
 extern const char* const kPartNames[kPartCount];
 int kernel_part(int kernel);
 

@@ -40,7 +40,7 @@ uint32_t g_paged_attention_splits = 0;
 // Key splits for a problem: enough workgroups to fill the compute units four times over, when the query rows
 // alone do not (decoding, short chunks); one (no split) for other element types and head dimensions.
 uint32_t paged_attention_splits(const SingePagedAttentionProblem& p) {
-    if (p.head_dim != 128 || p.tokens <= 0 || p.sequences <= 0 || p.kv_heads <= 0 || p.heads <= 0) return 1;
+    if ((p.head_dim != 128 && p.head_dim != 64) || p.tokens <= 0 || p.sequences <= 0 || p.kv_heads <= 0 || p.heads <= 0) return 1;
     if (g_paged_attention_splits != 0) return g_paged_attention_splits;
     const uint64_t groups = static_cast<uint64_t>(p.heads / p.kv_heads);
     const uint64_t row_tiles = (groups * static_cast<uint64_t>(p.tokens) + 127) / 128;
@@ -53,7 +53,7 @@ uint32_t paged_attention_splits(const SingePagedAttentionProblem& p) {
 
 size_t scratch_bytes_for(const SingePagedAttentionProblem& p, uint32_t splits) {
     if (splits <= 1) return 0;
-    return static_cast<size_t>(splits) * static_cast<size_t>(p.tokens) * static_cast<size_t>(p.heads) * (128 + 1) * sizeof(float);
+    return static_cast<size_t>(splits) * static_cast<size_t>(p.tokens) * static_cast<size_t>(p.heads) * (static_cast<size_t>(p.head_dim) + 1) * sizeof(float);
 }
 
 int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_any, const void* key_cache_any,
@@ -72,7 +72,7 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
         // The fused form exists for the tensor-core kernel alone and without softcap here; the reference
         // plans the rotation and the attention apart for the rest (compiled/plan/group.rs:94-98), and so
         // does a caller of this library (singe_hip_rotary_cache_write, then singe_hip_paged_attention_*).
-        if (data_type != SINGE_HIP_BF16 || p.head_dim != 128)
+        if (data_type != SINGE_HIP_BF16 || (p.head_dim != 128 && p.head_dim != 64))
             return fail(SINGE_HIP_UNSUPPORTED_WIDTH, "rotary_paged_attention", static_cast<uint64_t>(p.head_dim));
         if (p.has_softcap) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "rotary paged attention with a softcap");
     }
@@ -99,11 +99,13 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
     if (pages == nullptr && p.page_table > 0) return fail(SINGE_HIP_NULL_POINTER, "pages");
     if (rotation != nullptr && (rotation->cos == nullptr || rotation->sin == nullptr)) return fail(SINGE_HIP_NULL_POINTER, "cos or sin");
     const float scale = p.has_scale ? p.scale : 1.0f / std::sqrt(static_cast<float>(p.head_dim));
-    // The tensor-core kernel covers bf16 and f16 at head dimension 128 (the reference's takes f16/bf16 at
+    // The matrix-core kernels cover bf16 and f16 at head dimensions 128 and 64 (the reference's take f16/bf16 at
     // multiples of 16 up to 128: paged_attention.rs:586-592); everything else goes to the general one
     // (paged_general.rs:73-247).
     const bool f16 = data_type == SINGE_HIP_F16;
-    if ((data_type != SINGE_HIP_BF16 && !f16) || p.head_dim != 128)
+    const bool narrow = p.head_dim == 64;  // the head_dim 64 build of the same kernels
+    auto built = [narrow](int kernel) { return narrow ? at_head_dim_64(static_cast<KernelId>(kernel)) : static_cast<KernelId>(kernel); };
+    if ((data_type != SINGE_HIP_BF16 && !f16) || (p.head_dim != 128 && !narrow))
         return paged_attention_general(data_type, stream, query_rows_any, key_cache_any, value_cache_any, query_offsets,
                                        page_offsets, pages, last_page_lengths, output_any, lse, status, p, scale);
     const uint16_t* query_rows = static_cast<const uint16_t*>(query_rows_any);
@@ -153,13 +155,13 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
     args.splits = splits;
     if (splits > 1) {
         args.partial_out = static_cast<float*>(scratch->memory);
-        args.partial_lse = args.partial_out + static_cast<size_t>(splits) * p.tokens * p.heads * 128;
+        args.partial_lse = args.partial_out + static_cast<size_t>(splits) * p.tokens * p.heads * p.head_dim;
     }
     const unsigned grid = static_cast<unsigned>(blocks * splits);
     auto finish = [&](int32_t launched) -> int32_t {
         if (launched != 0 || splits == 1) return launched;
         const int combine = (f16 ? kPagedAttentionCombineF16I32 : kPagedAttentionCombineI32) + (wide ? 1 : 0);
-        return launch(static_cast<KernelId>(combine), static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+        return launch(built(combine), static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
     };
     if (rotation != nullptr) {
         args.cos = rotation->cos;
@@ -169,11 +171,11 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
         args.has_query_norm = rotation->attributes->has_norm ? 1u : 0u;
         args.query_eps = rotation->attributes->eps;
         const int rotary = kRotaryPagedAttention + (wide ? 1 : 0) + (args.page_shift >= 4 ? 2 : 0);
-        return finish(launch(static_cast<KernelId>(rotary), grid, 1, 1, 256, stream, args));
+        return finish(launch(built(rotary), grid, 1, 1, 256, stream, args));
     }
     const int kernel = (f16 ? kPagedAttentionF16 : kPagedAttentionI32) + (p.has_softcap ? 2 : 0) + (wide ? 1 : 0) +
                        (args.page_shift >= 4 ? 4 : 0);
-    return finish(launch(static_cast<KernelId>(kernel), grid, 1, 1, 256, stream, args));
+    return finish(launch(built(kernel), grid, 1, 1, 256, stream, args));
 }
 
 }  // namespace
@@ -315,14 +317,20 @@ int32_t paged_kv_prefill(
     if (int32_t s = ensure_len_at_least("actual_seq_lens_kv", actual_seq_lens_kv_len, c.batch)) return s;
     if (int32_t s = ensure_len_at_least("actual_seq_offsets", actual_seq_offsets_len, c.batch)) return s;
     if (int32_t s = ensure_len_at_least("block_table", block_table_len, table_len)) return s;
-    if (c.head_dim != 128)
-        return fail(SINGE_HIP_UNSUPPORTED_WIDTH, f16 ? "paged_kv_prefill_attention_f16" : "paged_kv_prefill_attention_bf16", c.head_dim, 0);
     if (block_len > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "a cache block beyond 4 Gi elements");
     const void* pointers[] = {out, lse, query, key_cache, value_cache, actual_seq_lens_q, actual_seq_lens_kv, actual_seq_offsets, block_table};
     const char* names[] = {"out", "lse", "query", "key_cache", "value_cache", "actual_seq_lens_q", "actual_seq_lens_kv",
                            "actual_seq_offsets", "block_table"};
     for (int i = 0; i < 9; ++i)
         if (pointers[i] == nullptr) return fail(SINGE_HIP_NULL_POINTER, names[i]);
+    // The matrix-core kernels are built for head dimensions 128 and 64; the others (up to 256) take the
+    // one-wave-per-row kernel.
+    if (c.head_dim != 128 && c.head_dim != 64)
+        return paged_table_general(f16 ? SINGE_HIP_F16 : SINGE_HIP_BF16, stream,
+                                   f16 ? "paged_kv_prefill_attention_f16" : "paged_kv_prefill_attention_bf16", query, key_cache,
+                                   value_cache, actual_seq_offsets, actual_seq_lens_q, actual_seq_lens_kv, block_table, out, lse,
+                                   c.total_query_tokens, c.batch, c.heads, c.kv_heads, c.head_dim, c.block_size, c.physical_blocks,
+                                   c.block_table_batch_stride, c.causal != 0, c.scale);
 
     const uint64_t groups = c.heads / c.kv_heads;
     PagedAttentionArgs args;
@@ -356,7 +364,7 @@ int32_t paged_kv_prefill(
     const uint64_t units = (static_cast<uint64_t>(c.batch) * c.kv_heads + 7) / 8 * 8;
     const uint64_t blocks = units * args.row_tiles;
     if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
-    const int kernel = (f16 ? kPagedKvPrefillF16 : kPagedKvPrefill) + (args.page_shift >= 4 ? 1 : 0);
-    return launch(static_cast<KernelId>(kernel), static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+    const KernelId kernel = static_cast<KernelId>((f16 ? kPagedKvPrefillF16 : kPagedKvPrefill) + (args.page_shift >= 4 ? 1 : 0));
+    return launch(c.head_dim == 64 ? at_head_dim_64(kernel) : kernel, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
 }
 }  // namespace

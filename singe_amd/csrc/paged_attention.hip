@@ -3,7 +3,8 @@
 // (singe/src/backend/cuda/kernel_plan/source/paged_attention.rs:544-868) and of the CPU attend_paged
 // (singe/src/backend/cpu/normalization/attention.rs:424-538).
 //
-// query_rows/output [tokens, heads, 128] bf16; caches [pages, page_size, kv_heads, 128] bf16; sequence b
+// query_rows/output [tokens, heads, D] bf16 or f16; caches [pages, page_size, kv_heads, D], D = 128 or 64 (one build
+// each); sequence b
 // holds queries query_offsets[b] .. query_offsets[b+1] and the keys of pages
 // pages[page_offsets[b] .. page_offsets[b+1]], all full but the last, which holds last_page_lengths[b];
 // lse [tokens, heads] f32, base two, -inf for a row that sees no key.  Queries are a sequence's LAST
@@ -157,21 +158,21 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     const unsigned int flip = (SOFTCAP ? a.softcap_scale : a.scale_log2e) < 0.0f ? 0x80008000u : 0u;
     static_assert(!ROTATE || std::is_same<Half, Bf16>::value, "the fused rotation reads bf16 queries");
     const Half half{};
-    uint4 q[8];
+    uint4 q[kSteps];
     {
         const uint16_t* row = a.query_rows + ((static_cast<size_t>(query_start) + my_token) * a.heads + kv_head * groups + my_head) * kHeadDim + 8 * hi;
-        uint4 bits[8];
+        uint4 bits[kSteps];
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
+        for (int s = 0; s < kSteps; ++s) {
             bits[s] = *reinterpret_cast<const uint4*>(row + 16 * s);
             if (!row_valid) bits[s] = make_uint4(0, 0, 0, 0);
         }
         if constexpr (ROTATE) {
             // The query arrives before its rotation (paged_attention.rs:881-977): an optional RMS norm over
-            // the head dimension with an optional weight, then half-split pairs (p, p + 64) turned by the
+            // the head dimension with an optional weight, then half-split pairs (p, p + head_dim / 2) turned by the
             // token's angles, first = a cos - b sin, second = b cos + a sin, rounded to bf16 as the
             // reference rounds what it stores in its tile.  A lane holds both halves of its pairs (dims
-            // 16 s + 8 hi + j and the same + 64); the other half of the row's squares is one swap away.
+            // 16 s + 8 hi + j and the same + head_dim / 2); the other half of the row's squares is one swap away.
             auto wide = [](unsigned int pair, int upper) __attribute__((always_inline)) {
                 return __builtin_bit_cast(float, upper ? pair & 0xffff0000u : pair << 16);
             };
@@ -179,7 +180,7 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
             if (a.has_query_norm != 0) {
                 float squares = 0.0f;
 #pragma unroll
-                for (int s = 0; s < 8; ++s) {
+                for (int s = 0; s < kSteps; ++s) {
                     const unsigned int words[4] = {bits[s].x, bits[s].y, bits[s].z, bits[s].w};
 #pragma unroll
                     for (int w = 0; w < 4; ++w) squares += wide(words[w], 0) * wide(words[w], 0) + wide(words[w], 1) * wide(words[w], 1);
@@ -188,10 +189,11 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
                 scale = rsqrtf(squares / static_cast<float>(kHeadDim) + a.query_eps);
             }
             const size_t token = static_cast<size_t>(query_start) + my_token;
+            constexpr int kPairs = kHeadDim / 2, kHalfSteps = kSteps / 2;
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
+            for (int s = 0; s < kHalfSteps; ++s) {
                 unsigned int first_words[4] = {bits[s].x, bits[s].y, bits[s].z, bits[s].w};
-                unsigned int second_words[4] = {bits[s + 4].x, bits[s + 4].y, bits[s + 4].z, bits[s + 4].w};
+                unsigned int second_words[4] = {bits[s + kHalfSteps].x, bits[s + kHalfSteps].y, bits[s + kHalfSteps].z, bits[s + kHalfSteps].w};
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
                     float rotated_first[2], rotated_second[2];
@@ -204,11 +206,11 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
                             second *= scale;
                             if (a.query_weight != nullptr) {
                                 first *= __builtin_bit_cast(float, static_cast<unsigned int>(a.query_weight[pair]) << 16);
-                                second *= __builtin_bit_cast(float, static_cast<unsigned int>(a.query_weight[pair + 64]) << 16);
+                                second *= __builtin_bit_cast(float, static_cast<unsigned int>(a.query_weight[pair + kPairs]) << 16);
                             }
                         }
-                        const float cosine = table_value(a.cos, a.table_type, token * 64 + pair);
-                        const float sine = table_value(a.sin, a.table_type, token * 64 + pair);
+                        const float cosine = table_value(a.cos, a.table_type, token * kPairs + pair);
+                        const float sine = table_value(a.sin, a.table_type, token * kPairs + pair);
                         rotated_first[upper] = first * cosine - second * sine;
                         rotated_second[upper] = second * cosine + first * sine;
                     }
@@ -216,11 +218,11 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
                     second_words[w] = row_valid ? pack_pair(rotated_second[0], rotated_second[1]) : 0u;
                 }
                 bits[s] = make_uint4(first_words[0], first_words[1], first_words[2], first_words[3]);
-                bits[s + 4] = make_uint4(second_words[0], second_words[1], second_words[2], second_words[3]);
+                bits[s + kHalfSteps] = make_uint4(second_words[0], second_words[1], second_words[2], second_words[3]);
             }
         }
 #pragma unroll
-        for (int s = 0; s < 8; ++s) {
+        for (int s = 0; s < kSteps; ++s) {
             bits[s].x ^= flip; bits[s].y ^= flip; bits[s].z ^= flip; bits[s].w ^= flip;
             q[s] = bits[s];
         }
@@ -240,8 +242,10 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     // places its own row.
     const unsigned int load_row = 4u * wave + (lane >> 4), chunk_position = lane & 15u;
     const unsigned int key_chunk = (chunk_position ^ (load_row & 15u)) * 16u, value_chunk = (chunk_position ^ (4u * (load_row & 3u))) * 16u;
-    const size_t page_bytes = static_cast<size_t>(a.page_size) * a.kv_heads * kRowBytes;
-    const unsigned int head_bytes = kv_head * kRowBytes, slot_bytes = a.kv_heads * kRowBytes;
+    // At head_dim 64 a cache row has eight chunks: the lanes whose LDS position holds one of the other eight fetch nothing.
+    const bool key_lane_live = key_chunk < kGlobalRowBytes, value_lane_live = value_chunk < kGlobalRowBytes;
+    const size_t page_bytes = static_cast<size_t>(a.page_size) * a.kv_heads * kGlobalRowBytes;
+    const unsigned int head_bytes = kv_head * kGlobalRowBytes, slot_bytes = a.kv_heads * kGlobalRowBytes;
     const unsigned char* const key_bytes = reinterpret_cast<const unsigned char*>(a.key_cache);
     const unsigned char* const value_bytes = reinterpret_cast<const unsigned char*>(a.value_cache);
     const bool shifted = a.page_shift >= 0;
@@ -283,8 +287,10 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         }
     };
     const unsigned int key_lane = load_row * slot_bytes + key_chunk, value_lane = load_row * slot_bytes + value_chunk;
-    auto load = [&](const unsigned char* cache, unsigned int chunk, unsigned int lane_offset, unsigned int tile, const Pages& pages,
-                    unsigned char* stage) __attribute__((always_inline)) {
+    auto load = [&](const unsigned char* cache, unsigned int chunk, unsigned int lane_offset, bool lane_live, unsigned int tile,
+                    const Pages& pages, unsigned char* stage) __attribute__((always_inline)) {
+        // (only the load itself is predicated, so that the scalar address arithmetic stays outside the branch)
+        const bool fetch = kGlobalRowBytes == kRowBytes || lane_live;
 #pragma unroll
         for (unsigned int i = 0; i < 4; ++i) {
             if constexpr (GROUPED) {
@@ -300,23 +306,24 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
                 // scalar-base form (see fmha_prefill.hip).
                 asm("" : "+s"(base));
                 asm volatile("" : "+v"(offset));
-                __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(base + offset),
-                                                 (lds_words_t)(stage + (16u * i + 4u * wave) * kRowBytes), 16, 0, 0);
+                if (fetch)
+                    __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(base + offset),
+                                                     (lds_words_t)(stage + (16u * i + 4u * wave) * kRowBytes), 16, 0, 0);
             } else {
                 const unsigned int key = key_of(tile, i);
                 const unsigned int slot = shifted ? key & (a.page_size - 1u) : key % a.page_size;
                 const size_t offset = pages.id[i] * page_bytes + (slot * slot_bytes + head_bytes + chunk);
-                if (pages.id[i] != kNoPage)
+                if (pages.id[i] != kNoPage && fetch)
                     __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(cache + offset),
                                                      (lds_words_t)(stage + (16u * i + 4u * wave) * kRowBytes), 16, 0, 0);
             }
         }
     };
     auto load_keys = [&](unsigned int tile, const Pages& pages, unsigned char* stage) __attribute__((always_inline)) {
-        load(key_bytes, key_chunk, key_lane, tile, pages, stage);
+        load(key_bytes, key_chunk, key_lane, key_lane_live, tile, pages, stage);
     };
     auto load_values = [&](unsigned int tile, const Pages& pages, unsigned char* stage) __attribute__((always_inline)) {
-        load(value_bytes, value_chunk, value_lane, tile, pages, stage);
+        load(value_bytes, value_chunk, value_lane, value_lane_live, tile, pages, stage);
     };
 
     RowState state;
@@ -412,7 +419,7 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         const unsigned int inside = (wave_high + 1u - window + kKeyTile - 1) / kKeyTile;
         interior_begin = inside > first_tile ? inside : first_tile;
     }
-    uint4 operand[8];
+    uint4 operand[kSteps];
     for (; tile < interior_begin && tile < interior_end; ++tile) {
         const TileStages stages = enter();
         fold_edge_tile(half, scores, q, offsets, 2u * tile, wave_blocks, stages.keys, stages.next_keys, stages.values, stages.key_dest,
@@ -453,7 +460,7 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         const size_t slot = static_cast<size_t>(split) * a.tokens * a.heads + flat;
         float* row = a.partial_out + slot * kHeadDim;
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < kDimBlocks; ++db)
 #pragma unroll
             for (int quad = 0; quad < 4; ++quad)
                 *reinterpret_cast<float4*>(row + 32 * db + 8 * quad + 4 * hi) =
@@ -464,7 +471,7 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         const size_t flat = (static_cast<size_t>(query_start) + my_token) * a.heads + kv_head * groups + my_head;
         uint16_t* row = a.output + flat * kHeadDim;
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < kDimBlocks; ++db)
 #pragma unroll
             for (int quad = 0; quad < 4; ++quad) {
                 uint2 packed_bits;
@@ -494,7 +501,7 @@ SINGE_DEVICE void combine_body(const PagedAttentionArgs& a, unsigned int shares)
     const SequenceSpan span = load_span<FORM>(sequence, a.query_offsets, a.page_offsets, a.last_page_lengths, a.query_lengths,
                                               a.tokens, a.page_table, a.page_size);
     if (!span.valid) return;  // reported by the attention kernel
-    // A wave per row, rows of the tile four apart; a lane takes two of the 128 values.
+    // A wave per row, rows of the tile four apart; a lane takes two of the row's values (the first 32 lanes at head_dim 64).
     const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
     const unsigned int packed = span.queries * groups;
     const size_t rows_total = static_cast<size_t>(a.tokens) * a.heads;
@@ -510,15 +517,16 @@ SINGE_DEVICE void combine_body(const PagedAttentionArgs& a, unsigned int shares)
 #pragma unroll
         for (int step = 32; step > 0; step >>= 1) total += __shfl_xor(total, step, 64);
         float2 merged = make_float2(0.0f, 0.0f);
+        const bool holds_values = 2u * lane < static_cast<unsigned int>(kHeadDim);
         for (unsigned int s = 0; s < shares; ++s) {
             const float w = __shfl(weight, s, 64);
-            if (w == 0.0f) continue;  // its output was never meant to be read
+            if (w == 0.0f || !holds_values) continue;  // a share that weighs nothing was never meant to be read
             const float2 part = *reinterpret_cast<const float2*>(a.partial_out + (s * rows_total + flat) * kHeadDim + 2u * lane);
             merged.x = fmaf(w, part.x, merged.x);
             merged.y = fmaf(w, part.y, merged.y);
         }
         const float inverse = total > 0.0f ? 1.0f / total : 0.0f;
-        reinterpret_cast<unsigned int*>(a.output + flat * kHeadDim)[lane] = pack_pair(Half{}, merged.x * inverse, merged.y * inverse);
+        if (holds_values) reinterpret_cast<unsigned int*>(a.output + flat * kHeadDim)[lane] = pack_pair(Half{}, merged.x * inverse, merged.y * inverse);
         if (a.lse != nullptr && lane == 0) a.lse[flat] = total > 0.0f ? largest + fast_log2(total) : -INFINITY;
     }
 }
@@ -534,10 +542,22 @@ SINGE_DEVICE void combine_body(const PagedAttentionArgs& a, unsigned int shares)
         combine_body<FORM, prefill::HALF>(args, shares);                                     \
     }
 
+// Names carry the head dimension of the build: singe_paged_attention_bf16_d128_i32, ..._d64_i32.
+#define SINGE_PASTE4_(a, b, c, d) a##b##c##d
+#define SINGE_PASTE4(a, b, c, d) SINGE_PASTE4_(a, b, c, d)
+#define SINGE_PAGED_NAME(STEM, TAIL) SINGE_PASTE4(STEM, _d, SINGE_HEAD_DIM, TAIL)
+#if SINGE_HEAD_DIM == 128
+// (the merge kernels of the head_dim 128 build keep their first names)
 SINGE_PAGED_COMBINE_KERNEL(singe_paged_attention_combine_bf16_i32, kCsrI32, Bf16)
 SINGE_PAGED_COMBINE_KERNEL(singe_paged_attention_combine_bf16_i64, kCsrI64, Bf16)
 SINGE_PAGED_COMBINE_KERNEL(singe_paged_attention_combine_f16_i32, kCsrI32, F16)
 SINGE_PAGED_COMBINE_KERNEL(singe_paged_attention_combine_f16_i64, kCsrI64, F16)
+#else
+SINGE_PAGED_COMBINE_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_combine_bf16, _i32), kCsrI32, Bf16)
+SINGE_PAGED_COMBINE_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_combine_bf16, _i64), kCsrI64, Bf16)
+SINGE_PAGED_COMBINE_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_combine_f16, _i32), kCsrI32, F16)
+SINGE_PAGED_COMBINE_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_combine_f16, _i64), kCsrI64, F16)
+#endif
 
 #define SINGE_PAGED_ATTENTION_KERNEL(NAME, SOFTCAP, FORM, GROUPED, ROTATE, HALF)                           \
     extern "C" __global__ __launch_bounds__(256, 2) void NAME(PagedAttentionArgs args) {                    \
@@ -546,30 +566,30 @@ SINGE_PAGED_COMBINE_KERNEL(singe_paged_attention_combine_f16_i64, kCsrI64, F16)
     }
 
 // _p16: the page size is a power of two of at least 16 keys (page ids on the scalar unit).
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i32, false, kCsrI32, false, false, Bf16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i64, false, kCsrI64, false, false, Bf16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i32, true, kCsrI32, false, false, Bf16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i64, true, kCsrI64, false, false, Bf16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i32_p16, false, kCsrI32, true, false, Bf16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_i64_p16, false, kCsrI64, true, false, Bf16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i32_p16, true, kCsrI32, true, false, Bf16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_bf16_d128_softcap_i64_p16, true, kCsrI64, true, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_bf16, _i32), false, kCsrI32, false, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_bf16, _i64), false, kCsrI64, false, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_bf16, _softcap_i32), true, kCsrI32, false, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_bf16, _softcap_i64), true, kCsrI64, false, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_bf16, _i32_p16), false, kCsrI32, true, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_bf16, _i64_p16), false, kCsrI64, true, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_bf16, _softcap_i32_p16), true, kCsrI32, true, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_bf16, _softcap_i64_p16), true, kCsrI64, true, false, Bf16)
 // paged_kv_prefill_attention_bf16 of the singe-kernel surface: same gather, block-table paging.
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_bf16_d128, false, kTable, false, false, Bf16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_bf16_d128_p16, false, kTable, true, false, Bf16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_f16_d128, false, kTable, false, false, F16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_kv_prefill_f16_d128_p16, false, kTable, true, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_kv_prefill_bf16, /**/), false, kTable, false, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_kv_prefill_bf16, _p16), false, kTable, true, false, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_kv_prefill_f16, /**/), false, kTable, false, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_kv_prefill_f16, _p16), false, kTable, true, false, F16)
 // rotary_paged_attention: the query is normalised and rotated on its way into the registers.
-SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i32, false, kCsrI32, false, true, Bf16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i64, false, kCsrI64, false, true, Bf16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i32_p16, false, kCsrI32, true, true, Bf16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_rotary_paged_attention_bf16_d128_i64_p16, false, kCsrI64, true, true, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_bf16, _i32), false, kCsrI32, false, true, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_bf16, _i64), false, kCsrI64, false, true, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_bf16, _i32_p16), false, kCsrI32, true, true, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_bf16, _i64_p16), false, kCsrI64, true, true, Bf16)
 // f16 operands: the same kernels on v_mfma_f32_32x32x16_f16.
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_f16_d128_i32, false, kCsrI32, false, false, F16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_f16_d128_i64, false, kCsrI64, false, false, F16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_f16_d128_softcap_i32, true, kCsrI32, false, false, F16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_f16_d128_softcap_i64, true, kCsrI64, false, false, F16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_f16_d128_i32_p16, false, kCsrI32, true, false, F16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_f16_d128_i64_p16, false, kCsrI64, true, false, F16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_f16_d128_softcap_i32_p16, true, kCsrI32, true, false, F16)
-SINGE_PAGED_ATTENTION_KERNEL(singe_paged_attention_f16_d128_softcap_i64_p16, true, kCsrI64, true, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_f16, _i32), false, kCsrI32, false, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_f16, _i64), false, kCsrI64, false, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_f16, _softcap_i32), true, kCsrI32, false, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_f16, _softcap_i64), true, kCsrI64, false, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_f16, _i32_p16), false, kCsrI32, true, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_f16, _i64_p16), false, kCsrI64, true, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_f16, _softcap_i32_p16), true, kCsrI32, true, false, F16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_f16, _softcap_i64_p16), true, kCsrI64, true, false, F16)

@@ -24,7 +24,6 @@ int32_t decode(void* stream, uint16_t* out, size_t out_len, const uint16_t* quer
                size_t block_table_len, void* workspace, size_t workspace_bytes,
                const SingePagedKvDecodeAttentionConfig* config, uint32_t phases, bool f16 = false);
 
-constexpr size_t kHeadDim = 128;
 constexpr unsigned kWavesPerWorkgroup = 8;
 
 // How the flat list of 32-key tiles is shared out (see paged_decode.hip).
@@ -65,7 +64,7 @@ Plan make_plan(const SingePagedKvDecodeAttentionConfig& c) {
     const size_t rows = static_cast<size_t>(p.work) * (p.workers + c.batch) * p.heads_per_wave;
     p.lse_offset = align256((c.batch + 3) * sizeof(uint32_t));
     p.out_offset = p.lse_offset + align256(rows * sizeof(float));
-    p.bytes = p.out_offset + align256(rows * kHeadDim * sizeof(float));
+    p.bytes = p.out_offset + align256(rows * c.head_dim * sizeof(float));
     return p;
 }
 
@@ -214,8 +213,20 @@ int32_t decode(
 
     // What the gfx950 kernels take (the reference's cuTile kernels take head_dim 4..64 only and return
     // UnsupportedWidth otherwise: singe-kernel/src/cuda/cutile/attention/paged.rs:799-810).
-    if (c.head_dim != kHeadDim)
-        return fail(SINGE_HIP_UNSUPPORTED_WIDTH, f16 ? "paged_kv_decode_attention_f16" : "paged_kv_decode_attention_bf16", c.head_dim, 0);
+    if (fp8 && c.head_dim != 128) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, "paged_kv_decode_attention_f8e4m3kv_bf16", c.head_dim, 0);
+    // The matrix-core kernels are built for head dimensions 128 and 64; the others (the reference's own kernels
+    // take 4 to 64 here, this library up to 256) run on the one-wave-per-row kernel and need no workspace.
+    if (c.head_dim != 128 && c.head_dim != 64) {
+        if (!(phases & SINGE_HIP_DECODE_REDUCE)) return 0;  // nothing is left in the workspace at these widths
+        uint64_t reach_keys = static_cast<uint64_t>(c.block_table_batch_stride) * c.block_size;
+        if (!fits_i32(reach_keys)) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "block_table_batch_stride * block_size");
+        return paged_table_general(f16 ? SINGE_HIP_F16 : SINGE_HIP_BF16, stream,
+                                   f16 ? "paged_kv_decode_attention_f16" : "paged_kv_decode_attention_bf16", query, key_cache,
+                                   value_cache, nullptr, nullptr, actual_seq_lens, block_table, out, nullptr, c.batch, c.batch,
+                                   c.heads, c.kv_heads, c.head_dim, c.block_size, c.physical_blocks, c.block_table_batch_stride,
+                                   false, c.scale);
+    }
+    const bool narrow = c.head_dim == 64;  // the head_dim 64 build of the same kernels
     uint64_t reach = static_cast<uint64_t>(c.block_table_batch_stride) * c.block_size;
     if (!fits_i32(reach)) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "block_table_batch_stride * block_size");
 
@@ -257,7 +268,7 @@ int32_t decode(
     const KernelId kernel = fp8 ? static_cast<KernelId>(kDecodeF8Wide + (aligned ? 0 : 1) + (g_relaxed.load(std::memory_order_relaxed) ? 2 : 0))
                                 : static_cast<KernelId>((f16 ? kDecodeF16 : kDecodeBf16) + (aligned ? 0 : 2) + (plan.groups == 2 ? 1 : 0));
     if (phases & SINGE_HIP_DECODE_SPLIT)
-        if (int32_t status = launch(kernel, plan.grid_x, plan.grid_y, 1, 64 * kWavesPerWorkgroup, stream, args,
+        if (int32_t status = launch(narrow ? at_head_dim_64(kernel) : kernel, plan.grid_x, plan.grid_y, 1, 64 * kWavesPerWorkgroup, stream, args,
                                     static_cast<unsigned>((2 * c.batch + 1) * sizeof(uint32_t))))
             return status;
     if (!(phases & SINGE_HIP_DECODE_REDUCE)) return 0;
@@ -273,7 +284,8 @@ int32_t decode(
     combine.workers = plan.workers;
     combine.head_groups = plan.head_groups;
     combine.heads_per_wave = plan.heads_per_wave;
-    return launch(f16 ? kDecodeF16Combine : kDecodeCombine, static_cast<unsigned>((c.batch * c.heads + 3) / 4), 1, 1, 256, stream, combine);
+    const KernelId merge = f16 ? kDecodeF16Combine : kDecodeCombine;
+    return launch(narrow ? at_head_dim_64(merge) : merge, static_cast<unsigned>((c.batch * c.heads + 3) / 4), 1, 1, 256, stream, combine);
 }
 
 }  // namespace

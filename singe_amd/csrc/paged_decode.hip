@@ -43,7 +43,16 @@
 
 namespace {
 
-constexpr int kDim = 128;
+// The head dimension a build of these kernels is for: the source is compiled once per value (128, and 64 with
+// -DSINGE_HEAD_DIM=64, bf16 and f16 caches only), each into its own part of the code object.  At 64 the register
+// layouts below stay as they are and only their first half is live: a key's row is eight 16-byte chunks, so lanes
+// t >= 8 fetch no values and the score products run over two 32-dim steps instead of four.
+#ifndef SINGE_HEAD_DIM
+#define SINGE_HEAD_DIM 128
+#endif
+constexpr int kDim = SINGE_HEAD_DIM;
+static_assert(kDim == 64 || kDim == 128, "head dimensions the decode kernels are built for");
+constexpr int kDimSteps = kDim / 32;  // score products per 16 keys
 constexpr int kTile = 32;
 
 // One 32-key tile in registers, bf16 cache.
@@ -186,9 +195,14 @@ SINGE_DEVICE void load_tile(KeyTileBf16& tile, const DecodeArgs& a, const unsign
         const HalfRows rows = locate_half<ALIGNED16>(a, table_row, cache, first + half * 16, end, kv_head, g, t);
         const uint16_t* kp = key_cache + rows.key_row + 8 * g;
 #pragma unroll
-        for (int c = 0; c < 4; ++c) tile.k[half][c] = *reinterpret_cast<const uint4*>(kp + 32 * c);
+        for (int c = 0; c < kDimSteps; ++c) tile.k[half][c] = *reinterpret_cast<const uint4*>(kp + 32 * c);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) tile.v[half][i] = stream_load_16(value_cache + rows.value_row[i] + 8 * t);
+        for (int i = 0; i < 4; ++i) {
+            if (kDim == 128 || 8 * t < static_cast<unsigned int>(kDim))
+                tile.v[half][i] = stream_load_16(value_cache + rows.value_row[i] + 8 * t);
+            else
+                tile.v[half][i] = make_uint4(0, 0, 0, 0);
+        }
         tile.live |= rows.live << (half * 4);
     }
 }
@@ -421,7 +435,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
             const bool real = local < wave_heads;
             const uint16_t* qp = a.query + (static_cast<size_t>(b) * a.heads + kv_head * group + head_in_group + (real ? local : 0)) * kDim + dim_lane;
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
+            for (int c = 0; c < kDimSteps; ++c) {
                 uint4 bits = *reinterpret_cast<const uint4*>(qp + dim_step * c);
                 if (!real) bits = make_uint4(0, 0, 0, 0);
                 q[hg][c] = __builtin_bit_cast(bf16x8_t, bits);
@@ -514,7 +528,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
             s1[hg] = {0.0f, 0.0f, 0.0f, 0.0f};
         }
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
+        for (int c = 0; c < kDimSteps; ++c) {
             uint4 first, second;
             if constexpr (!FP8) {
                 first = tile.k[0][c];
@@ -595,8 +609,10 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
                 float* row = a.partial_out + (slot * a.heads_per_wave + local) * kDim;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    row[8 * (4 * g + r) + (t & 3)] = state[hg].acc[0][r] * inverse;
-                    row[8 * (4 * g + r) + 4 + (t & 3)] = state[hg].acc[1][r] * inverse;
+                    if (kDim == 128 || 8 * (4 * g + r) < static_cast<unsigned int>(kDim)) {
+                        row[8 * (4 * g + r) + (t & 3)] = state[hg].acc[0][r] * inverse;
+                        row[8 * (4 * g + r) + 4 + (t & 3)] = state[hg].acc[1][r] * inverse;
+                    }
                 }
                 if (g == 0 && (t & 3) == 0)
                     a.partial_lse[slot * a.heads_per_wave + local] =
@@ -670,16 +686,21 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
 
 }  // namespace
 
+// Names carry the head dimension of the build: singe_paged_decode_bf16_d128_g1_b16, ..._d64_g1_b16.
+#define SINGE_PASTE4_(a, b, c, d) a##b##c##d
+#define SINGE_PASTE4(a, b, c, d) SINGE_PASTE4_(a, b, c, d)
+#define SINGE_DECODE_NAME(STEM, TAIL) SINGE_PASTE4(STEM, _d, SINGE_HEAD_DIM, TAIL)
+
 #define SINGE_DECODE_KERNEL(NAME, GROUPS, ALIGNED, FP8, EXACT)                                  \
     extern "C" __global__ __launch_bounds__(512) void NAME(DecodeArgs args) {                    \
         extern __shared__ unsigned int prefix[];                                                \
         paged_decode_body<GROUPS, ALIGNED, FP8, EXACT>(args, prefix);                           \
     }
 
-SINGE_DECODE_KERNEL(singe_paged_decode_bf16_d128_g1_b16, 1, true, false, true)
-SINGE_DECODE_KERNEL(singe_paged_decode_bf16_d128_g2_b16, 2, true, false, true)
-SINGE_DECODE_KERNEL(singe_paged_decode_bf16_d128_g1_any, 1, false, false, true)
-SINGE_DECODE_KERNEL(singe_paged_decode_bf16_d128_g2_any, 2, false, false, true)
+SINGE_DECODE_KERNEL(SINGE_DECODE_NAME(singe_paged_decode_bf16, _g1_b16), 1, true, false, true)
+SINGE_DECODE_KERNEL(SINGE_DECODE_NAME(singe_paged_decode_bf16, _g2_b16), 2, true, false, true)
+SINGE_DECODE_KERNEL(SINGE_DECODE_NAME(singe_paged_decode_bf16, _g1_any), 1, false, false, true)
+SINGE_DECODE_KERNEL(SINGE_DECODE_NAME(singe_paged_decode_bf16, _g2_any), 2, false, false, true)
 
 // paged_kv_decode_attention_f16: the same kernels on f16 operands.
 #define SINGE_DECODE_F16_KERNEL(NAME, GROUPS, ALIGNED)                                          \
@@ -688,11 +709,12 @@ SINGE_DECODE_KERNEL(singe_paged_decode_bf16_d128_g2_any, 2, false, false, true)
         paged_decode_body<GROUPS, ALIGNED, false, true, false, true>(args, prefix);             \
     }
 
-SINGE_DECODE_F16_KERNEL(singe_paged_decode_f16_d128_g1_b16, 1, true)
-SINGE_DECODE_F16_KERNEL(singe_paged_decode_f16_d128_g2_b16, 2, true)
-SINGE_DECODE_F16_KERNEL(singe_paged_decode_f16_d128_g1_any, 1, false)
-SINGE_DECODE_F16_KERNEL(singe_paged_decode_f16_d128_g2_any, 2, false)
+SINGE_DECODE_F16_KERNEL(SINGE_DECODE_NAME(singe_paged_decode_f16, _g1_b16), 1, true)
+SINGE_DECODE_F16_KERNEL(SINGE_DECODE_NAME(singe_paged_decode_f16, _g2_b16), 2, true)
+SINGE_DECODE_F16_KERNEL(SINGE_DECODE_NAME(singe_paged_decode_f16, _g1_any), 1, false)
+SINGE_DECODE_F16_KERNEL(SINGE_DECODE_NAME(singe_paged_decode_f16, _g2_any), 2, false)
 
+#if SINGE_HEAD_DIM == 128
 #define SINGE_DECODE_WIDE_KERNEL(NAME, ALIGNED, EXACT)                                          \
     extern "C" __global__ __launch_bounds__(512) void NAME(DecodeArgs args) {                    \
         extern __shared__ unsigned int prefix[];                                                \
@@ -704,6 +726,7 @@ SINGE_DECODE_WIDE_KERNEL(singe_paged_decode_f8kv_wide_d128_b16, true, true)
 SINGE_DECODE_WIDE_KERNEL(singe_paged_decode_f8kv_wide_d128_any, false, true)
 SINGE_DECODE_WIDE_KERNEL(singe_paged_decode_f8kv_wide_relaxed_d128_b16, true, false)
 SINGE_DECODE_WIDE_KERNEL(singe_paged_decode_f8kv_wide_relaxed_d128_any, false, false)
+#endif
 
 // Folds the partial rows of one (sequence, query head) into the bf16 output:
 // out = sum_s exp(lse_s - max) * partial_s / sum_s exp(lse_s - max)
@@ -722,6 +745,7 @@ SINGE_DEVICE void paged_decode_combine_body(const CombineArgs& a) {
     const unsigned int share = a.meta[0];
     const unsigned int first_tile = a.meta[2 + b], end_tile = a.meta[3 + b];
     float low = 0.0f, high = 0.0f;  // a sequence with no keys keeps a zero row (cpu/attention.rs:1213-1215)
+    const bool holds_values = 2 * lane < static_cast<unsigned int>(kDim);  // a lane takes two of the row's values
     if (end_tile > first_tile) {
         const unsigned int first_worker = first_tile / share, last_worker = (end_tile - 1) / share;
         const size_t base = (static_cast<size_t>(work) * (a.workers + a.batch) + first_worker + b) * a.heads_per_wave + local;
@@ -750,7 +774,7 @@ SINGE_DEVICE void paged_decode_combine_body(const CombineArgs& a) {
 #pragma unroll
                 for (int j = 0; j < 16; ++j) {
                     rows[j] = make_float2(0.0f, 0.0f);
-                    if (first + j < n)
+                    if (first + j < n && holds_values)
                         rows[j] = *reinterpret_cast<const float2*>(a.partial_out + (chunk_base + static_cast<size_t>(first + j) * a.heads_per_wave) * kDim + 2 * lane);
                 }
 #pragma unroll
@@ -775,8 +799,13 @@ SINGE_DEVICE void paged_decode_combine_body(const CombineArgs& a) {
     } else {
         packed = pack_bf16x2(low, high);
     }
-    *reinterpret_cast<unsigned int*>(a.out + static_cast<size_t>(row) * kDim + 2 * lane) = packed;
+    if (holds_values) *reinterpret_cast<unsigned int*>(a.out + static_cast<size_t>(row) * kDim + 2 * lane) = packed;
 }
 
+#if SINGE_HEAD_DIM == 128
 extern "C" __global__ __launch_bounds__(256) void singe_paged_decode_combine_bf16(CombineArgs a) { paged_decode_combine_body<false>(a); }
 extern "C" __global__ __launch_bounds__(256) void singe_paged_decode_combine_f16(CombineArgs a) { paged_decode_combine_body<true>(a); }
+#else
+extern "C" __global__ __launch_bounds__(256) void SINGE_DECODE_NAME(singe_paged_decode_combine_bf16, /**/)(CombineArgs a) { paged_decode_combine_body<false>(a); }
+extern "C" __global__ __launch_bounds__(256) void SINGE_DECODE_NAME(singe_paged_decode_combine_f16, /**/)(CombineArgs a) { paged_decode_combine_body<true>(a); }
+#endif

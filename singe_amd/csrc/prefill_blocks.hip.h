@@ -18,7 +18,9 @@
 
 namespace prefill {
 
-constexpr int kRowBytes = 256;                       // one key's 128 bf16
+constexpr int kRowBytes = 256;                       // an LDS row: one key's 128 halves; at head_dim 64 its chunks 0 .. 7,
+                                                     // scattered over the sixteen positions by the same permutation
+constexpr int kGlobalRowBytes = 2 * kHeadDim;        // one key's halves in global memory
 constexpr int kTileBytes = kKeyTile * kRowBytes;     // 64 keys of K or of V
 constexpr int kBlockBytes = 32 * kRowBytes;
 // LDS of a workgroup: three stages of K and two of V, so K can be loaded two tiles ahead and V one.
@@ -54,15 +56,15 @@ SINGE_DEVICE ReadOffsets read_offsets(unsigned int lane) {
 // Scores of the wave's 32 queries against the 32 keys of the block at `keys` (LDS byte address of the
 // block's first row).  The products run on while the caller does other work.
 template <class Half>
-SINGE_DEVICE void score_block(Half half, f32x16_t& scores, const uint4 (&q)[8], const unsigned char* keys, const ReadOffsets& offsets) {
+SINGE_DEVICE void score_block(Half half, f32x16_t& scores, const uint4 (&q)[kSteps], const unsigned char* keys, const ReadOffsets& offsets) {
     f32x16_t s;
 #pragma unroll
     for (int r = 0; r < 16; ++r) s[r] = 0.0f;
-    uint4 operand[8];
+    uint4 operand[kSteps];
 #pragma unroll
-    for (int step = 0; step < 8; ++step) operand[step] = *reinterpret_cast<const uint4*>(keys + offsets.key(step));
+    for (int step = 0; step < kSteps; ++step) operand[step] = *reinterpret_cast<const uint4*>(keys + offsets.key(step));
 #pragma unroll
-    for (int step = 0; step < 8; ++step)
+    for (int step = 0; step < kSteps; ++step)
         s = mma(half, operand[step], q[step], s);
     scores = s;
 }
@@ -92,7 +94,7 @@ SINGE_DEVICE float begin_block(RowState& state, f32x16_t& s, unsigned int hi, fl
         const float rescale = fast_exp2(state.reference - base);
         state.running_sum *= rescale;
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < kDimBlocks; ++db)
 #pragma unroll
             for (int r = 0; r < 16; ++r) state.out[db][r] *= rescale;
         state.reference = moved;
@@ -110,16 +112,16 @@ SINGE_DEVICE float begin_block(RowState& state, f32x16_t& s, unsigned int hi, fl
 //               its use.  Otherwise the operands are read from `next_keys` at the start of the call.
 template <bool NEXT, bool AHEAD = false, class Half>
 SINGE_DEVICE void finish_block(Half half, RowState& state, f32x16_t& s, float factor, float shift, const unsigned char* values,
-                               const ReadOffsets& offsets, f32x16_t& next, const uint4 (&q)[8], const unsigned char* next_keys,
-                               uint4 (&operand)[8], const unsigned char* after_keys) {
+                               const ReadOffsets& offsets, f32x16_t& next, const uint4 (&q)[kSteps], const unsigned char* next_keys,
+                               uint4 (&operand)[kSteps], const unsigned char* after_keys) {
     typedef v4i16_t __attribute__((address_space(3))) * lds_v4_t;
     if constexpr (NEXT && !AHEAD) {
 #pragma unroll
-        for (int step = 0; step < 8; ++step) operand[step] = *reinterpret_cast<const uint4*>(next_keys + offsets.key(step));
+        for (int step = 0; step < kSteps; ++step) operand[step] = *reinterpret_cast<const uint4*>(next_keys + offsets.key(step));
     }
-    v8i16_t first[4], second[4];
+    v8i16_t first[kDimBlocks], second[kDimBlocks];
 #pragma unroll
-    for (int db = 0; db < 4; ++db) {
+    for (int db = 0; db < kDimBlocks; ++db) {
         const v4i16_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(values + offsets.value(db)));
         const v4i16_t high = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(values + 8 * kRowBytes + offsets.value(db)));
         first[db] = __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -133,15 +135,18 @@ SINGE_DEVICE void finish_block(Half half, RowState& state, f32x16_t& s, float fa
         if (step == 4) {
             // The second half of the values, fetched once half of the K operands have been used up.
 #pragma unroll
-            for (int db = 0; db < 4; ++db) {
+            for (int db = 0; db < kDimBlocks; ++db) {
                 const v4i16_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(values + 16 * kRowBytes + offsets.value(db)));
                 const v4i16_t high = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(values + 24 * kRowBytes + offsets.value(db)));
                 second[db] = __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7);
             }
         }
         if constexpr (NEXT) {
-            upcoming = mma(half, operand[step], q[step], upcoming);
-            if constexpr (AHEAD) operand[step] = *reinterpret_cast<const uint4*>(after_keys + offsets.key(step));
+            // Eight pairs of exponentials take the block's kSteps products between them.
+            if (step < kSteps) {
+                upcoming = mma(half, operand[step], q[step], upcoming);
+                if constexpr (AHEAD) operand[step] = *reinterpret_cast<const uint4*>(after_keys + offsets.key(step));
+            }
         }
         s[2 * step] = fast_exp2(fmaf(s[2 * step], factor, shift));
         s[2 * step + 1] = fast_exp2(fmaf(s[2 * step + 1], factor, shift));
@@ -154,7 +159,7 @@ SINGE_DEVICE void finish_block(Half half, RowState& state, f32x16_t& s, float fa
         const uint4 weights = make_uint4(pack_pair(half, s[8 * j + 0], s[8 * j + 1]), pack_pair(half, s[8 * j + 2], s[8 * j + 3]),
                                          pack_pair(half, s[8 * j + 4], s[8 * j + 5]), pack_pair(half, s[8 * j + 6], s[8 * j + 7]));
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < kDimBlocks; ++db)
             state.out[db] = mma(half, __builtin_bit_cast(uint4, j == 0 ? first[db] : second[db]), weights, state.out[db]);
     }
     if constexpr (NEXT) next = upcoming;
@@ -162,8 +167,8 @@ SINGE_DEVICE void finish_block(Half half, RowState& state, f32x16_t& s, float fa
 
 template <bool NEXT, class Half>
 SINGE_DEVICE void finish_block(Half half, RowState& state, f32x16_t& s, float factor, float shift, const unsigned char* values,
-                               const ReadOffsets& offsets, f32x16_t& next, const uint4 (&q)[8], const unsigned char* next_keys) {
-    uint4 operand[8];
+                               const ReadOffsets& offsets, f32x16_t& next, const uint4 (&q)[kSteps], const unsigned char* next_keys) {
+    uint4 operand[kSteps];
     finish_block<NEXT, false>(half, state, s, factor, shift, values, offsets, next, q, next_keys, operand, next_keys);
 }
 
@@ -192,7 +197,7 @@ SINGE_DEVICE void loads_landed() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmc
 //                          takes (a score cap, an added mask) before they are folded; the caller then passes the
 //                          factor that is left to apply (1 when shape did the scaling).
 template <bool AHEAD, class Half, class Issue, class Shape>
-SINGE_DEVICE void fold_interior_tile(Half half, RowState& state, f32x16_t& scores, uint4 (&operand)[8], const uint4 (&q)[8],
+SINGE_DEVICE void fold_interior_tile(Half half, RowState& state, f32x16_t& scores, uint4 (&operand)[kSteps], const uint4 (&q)[kSteps],
                                      const ReadOffsets& offsets, unsigned int hi, float factor, const unsigned char* __restrict__ keys,
                                      const unsigned char* __restrict__ next_keys, const unsigned char* __restrict__ values,
                                      unsigned char* __restrict__ key_dest, unsigned char* __restrict__ value_dest, Issue&& issue,
@@ -209,7 +214,7 @@ SINGE_DEVICE void fold_interior_tile(Half half, RowState& state, f32x16_t& score
 }
 
 template <bool AHEAD, class Half, class Issue>
-SINGE_DEVICE void fold_interior_tile(Half half, RowState& state, f32x16_t& scores, uint4 (&operand)[8], const uint4 (&q)[8],
+SINGE_DEVICE void fold_interior_tile(Half half, RowState& state, f32x16_t& scores, uint4 (&operand)[kSteps], const uint4 (&q)[kSteps],
                                      const ReadOffsets& offsets, unsigned int hi, float factor, const unsigned char* __restrict__ keys,
                                      const unsigned char* __restrict__ next_keys, const unsigned char* __restrict__ values,
                                      unsigned char* __restrict__ key_dest, unsigned char* __restrict__ value_dest, Issue&& issue) {
@@ -218,15 +223,15 @@ SINGE_DEVICE void fold_interior_tile(Half half, RowState& state, f32x16_t& score
 }
 
 // The K operands of the block at `keys`.
-SINGE_DEVICE void read_key_operands(uint4 (&operand)[8], const unsigned char* keys, const ReadOffsets& offsets) {
+SINGE_DEVICE void read_key_operands(uint4 (&operand)[kSteps], const unsigned char* keys, const ReadOffsets& offsets) {
 #pragma unroll
-    for (int step = 0; step < 8; ++step) operand[step] = *reinterpret_cast<const uint4*>(keys + offsets.key(step));
+    for (int step = 0; step < kSteps; ++step) operand[step] = *reinterpret_cast<const uint4*>(keys + offsets.key(step));
 }
 
 // Any other tile: the same steps one after the other, each only if the wave still has that block;
 // fold(block, scores, values) applies the masks and folds one block.
 template <class Half, class Issue, class Fold>
-SINGE_DEVICE void fold_edge_tile(Half half, f32x16_t& scores, const uint4 (&q)[8], const ReadOffsets& offsets, unsigned int block,
+SINGE_DEVICE void fold_edge_tile(Half half, f32x16_t& scores, const uint4 (&q)[kSteps], const ReadOffsets& offsets, unsigned int block,
                                  unsigned int wave_blocks, const unsigned char* __restrict__ keys,
                                  const unsigned char* __restrict__ next_keys, const unsigned char* __restrict__ values,
                                  unsigned char* __restrict__ key_dest, unsigned char* __restrict__ value_dest, Issue&& issue, Fold&& fold) {

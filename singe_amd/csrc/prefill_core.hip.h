@@ -3,7 +3,7 @@
 // weights never leave registers:
 //
 //   S^T[key, query] = K . Q^T      v_mfma_f32_32x32x16_bf16, A = K rows read from LDS (16-byte reads), B = the
-//                                  wave's Q^T, resident in 32 VGPRs for the whole kernel;
+//                                  wave's Q^T, resident in 32 VGPRs (head_dim 128) for the whole kernel;
 //   online softmax                 base two; a lane holds the scores of ONE query (its MFMA column), so
 //                                  the row maximum is in-lane max ops plus one v_permlane32_swap, and
 //                                  rescaling O^T needs no broadcast;
@@ -23,7 +23,15 @@
 
 namespace prefill {
 
-constexpr int kHeadDim = 128;
+// The head dimension a build of these kernels is for: the sources are compiled once per value (128, and 64 with
+// -DSINGE_HEAD_DIM=64), each into its own part of the code object.
+#ifndef SINGE_HEAD_DIM
+#define SINGE_HEAD_DIM 128
+#endif
+constexpr int kHeadDim = SINGE_HEAD_DIM;
+static_assert(kHeadDim == 64 || kHeadDim == 128, "head dimensions the matrix-core kernels are built for");
+constexpr int kSteps = kHeadDim / 16;      // products per 32-key block of scores: sixteen dims each
+constexpr int kDimBlocks = kHeadDim / 32;  // 32-dim blocks of O^T
 constexpr int kQueryTile = 128;       // query rows per workgroup
 constexpr int kKeyTile = 64;          // keys per LDS stage
 
@@ -97,14 +105,14 @@ constexpr float kMaxLag = 6.0f;
 // Running state of a wave's 32 query rows: lane (query = lane % 32, hi = lane / 32) holds dims
 // 32db + 8(r / 4) + 4hi + (r % 4) of its query in out[db][r].
 struct RowState {
-    f32x16_t out[4];
+    f32x16_t out[kDimBlocks];
     float reference;    // point the weights are scaled by (scaled log2 units); trails the row maximum
     float running_sum;  // of this lane's keys only
 };
 
 SINGE_DEVICE void reset(RowState& state) {
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+    for (int db = 0; db < kDimBlocks; ++db)
 #pragma unroll
         for (int r = 0; r < 16; ++r) state.out[db][r] = 0.0f;
     state.reference = -INFINITY;

@@ -35,4 +35,30 @@ int32_t dense_prefill_with_options(void* stream, bool f16, uint16_t* out, size_t
                                    const uint16_t* key, size_t key_len, const uint16_t* value, size_t value_len,
                                    const SingeFmhaPrefillConfig* config, const DenseOptions& options);
 
+// general_attention.cpp: the one-wave-per-row kernels behind entry points of other files, for head dimensions the
+// matrix-core kernels are not built for.  Block-table prefill (query_lengths given) or decode (query_lengths null).
+int32_t paged_table_general(int32_t data_type, void* stream, const char* op, const void* query_rows, const void* key_cache,
+                            const void* value_cache, const int32_t* query_offsets, const int32_t* query_lengths,
+                            const int32_t* key_lengths, const uint32_t* block_table, void* output, float* lse, uint64_t tokens,
+                            uint64_t sequences, uint64_t heads, uint64_t kv_heads, uint64_t head_dim, uint64_t block_size,
+                            uint64_t physical_blocks, uint64_t table_stride, bool causal, float scale);
+// Dense attention through element strides over (batch, head, position); lse [batch, heads, query_len] natural log.
+struct DenseGeneralOperands {
+    const void* query = nullptr;
+    const void* key = nullptr;
+    const void* value = nullptr;
+    const void* mask = nullptr;
+    const void* sinks = nullptr;
+    const int32_t* key_lengths = nullptr;
+    void* out = nullptr;
+    float* lse = nullptr;
+    uint64_t query_strides[3] = {0, 0, 0}, key_strides[3] = {0, 0, 0}, value_strides[3] = {0, 0, 0}, out_strides[3] = {0, 0, 0};
+    uint64_t mask_strides[4] = {0, 0, 0, 0};
+    long long window = -1;
+    uint64_t batch = 0, heads = 0, kv_heads = 0, query_len = 0, key_len = 0, head_dim = 0, value_dim = 0;
+    bool causal = false, has_softcap = false;
+    float scale = 1.0f, softcap = 0.0f;
+};
+int32_t dense_general(int32_t data_type, void* stream, const char* op, const DenseGeneralOperands& operands);
+
 }  // namespace singe_hip

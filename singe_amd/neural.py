@@ -183,7 +183,7 @@ def paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: t
                     options: AttentionOptions = AttentionOptions(), *, stream=None, status: torch.Tensor | None = None,
                     check: bool = True, scratch: "torch.Tensor | bool" = True):
     """Tensor::paged_attention (tensor/neural.rs:420-457) for bf16, f16 or f32 tensors on the GPU; bf16 at
-    head dimension 128 runs on the matrix cores, everything else on the general kernel.
+    head dimensions 128 and 64 runs on the matrix cores, everything else on the general kernel.
 
     Returns (output [tokens, heads, dim] of the query's type, lse [tokens, heads] f32 base two).  Like the reference's
     eager launch (kernel_plan/mod.rs:156-251) it zeroes a status word, launches, and reads the word
@@ -302,7 +302,7 @@ def rotary_paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_c
                            check: bool = True):
     """Paged attention over a query the kernel normalises and rotates itself, the reference's fused
     rotary_paged_attention (singe/src/backend/cuda/kernel_plan/source/paged_attention.rs:533-542, 881-977):
-    ``query`` [tokens, heads, 128] bf16 before its rotation, ``cos`` / ``sin`` [tokens, 1, 64] (or [tokens, 64]) of
+    ``query`` [tokens, heads, D] bf16 (D = 128 or 64) before its rotation, ``cos`` / ``sin`` [tokens, 1, D / 2] (or [tokens, D / 2]) of
     f32, bf16 or f16, the same pairs and norm as ``rotary_cache_write``.  Returns (output, lse) like
     ``paged_attention``.  Other types and head dimensions raise UnsupportedWidth: rotate with
     ``rotary_cache_write`` and attend with ``paged_attention``, as the reference plans them apart."""

@@ -86,7 +86,9 @@ def test_decode_validation_order_and_codes():
         _native.lib().singe_hip_last_error(ctypes.byref(detail))
         assert detail.minimum == full[name] and detail.actual == full[name] - 1
     assert decode_status(c, pointers=dict(query=None)) == 6
-    assert decode_status(A.PagedKvDecodeAttentionConfig(**{**GOOD, "head_dim": 64})._c()) == 5
+    big = 1 << 30  # buffers long enough for any width: head dimensions past 256 have no kernel at all
+    wide = dict(out=big, query=big, key=big, value=big, seq=2, table=8)
+    assert decode_status(A.PagedKvDecodeAttentionConfig(**{**GOOD, "head_dim": 320})._c(), wide) == 5
     with pytest.raises(error.UnsupportedWidth):
         _native.check(5, "paged_kv_decode_attention_bf16")
 
@@ -148,7 +150,7 @@ def test_rotary_paged_attention_validation():
     good = _native.QueryRotationC(0, 1, 1e-5)
     assert call(None) == 6                                       # no rotation attributes
     assert call(_native.QueryRotationC(7, 0, 0.0)) == 9          # unknown table type
-    assert call(good, head_dim=64) == 5                          # the fused form takes head dimension 128
+    assert call(good, head_dim=96) == 5                          # the fused form takes head dimensions 128 and 64
     assert call(good, has_softcap=1, softcap=5.0) == 8
     assert call(good, cos=None) == 6
     assert call(good, tokens=0) == 0
@@ -164,7 +166,8 @@ def test_paged_attention_scratch_query_needs_no_device():
     lib.singe_hip_set_paged_attention_splits(4)
     try:
         assert wanted() == 4 * 32 * 32 * 129 * 4     # shares x rows x (128 values + a log-sum-exp) of f32
-        assert wanted(head_dim=64) == 0               # the general kernel does not split
+        assert wanted(head_dim=64) == 4 * 32 * 32 * 65 * 4   # the head_dim 64 build splits the same way
+        assert wanted(head_dim=96) == 0               # the general kernel does not split
     finally:
         lib.singe_hip_set_paged_attention_splits(0)
     assert lib.singe_hip_paged_attention_scratch_bytes(None) == 0

@@ -109,8 +109,9 @@ def test_prefill_validation_errors():
         A.fmha_prefill_bf16(None, out, q, k, v, replace(good, scale=float("inf")))
     with pytest.raises(error.LengthTooShort):
         A.fmha_prefill_bf16(None, out, q, k[:, :63].contiguous(), v, good)
-    with pytest.raises(error.UnsupportedWidth):
-        A.fmha_prefill_bf16(None, out, q, k, v, A.FmhaPrefillConfig.contiguous(1, 64, 64, 4, 2, 64, 0.1, True))
+    wide = lambda heads: torch.zeros((1, 64, heads, 320), device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(error.UnsupportedWidth):  # head dimensions past 256 have no kernel
+        A.fmha_prefill_bf16(None, wide(4), wide(4), wide(2), wide(2), A.FmhaPrefillConfig.contiguous(1, 64, 64, 4, 2, 320, 0.1, True))
 
 
 @pytest.mark.parametrize("magnitude,causal", [(8.0, True), (8.0, False), (30.0, True), (0.01, True)])

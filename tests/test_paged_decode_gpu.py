@@ -201,9 +201,11 @@ def test_decode_validation_errors_match_the_reference():
     with pytest.raises(error.LengthTooShort) as caught:
         A.paged_kv_decode_attention_bf16(None, out, out.clone(), cache[:7], cache, lens, table, config)
     assert caught.value.minimum == 8 * 16 * 2 * 128 and caught.value.actual == 7 * 16 * 2 * 128
-    with pytest.raises(error.UnsupportedWidth):
-        A.paged_kv_decode_attention_bf16(None, out, out.clone(), cache, cache, lens, table,
-                                         A.PagedKvDecodeAttentionConfig.contiguous(**{**good, "head_dim": 96, "heads": 8}))
+    wide_out = torch.zeros((2, 8, 320), device="cuda", dtype=torch.bfloat16)
+    wide_cache = torch.zeros((8, 16, 2, 320), device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(error.UnsupportedWidth):  # head dimensions past 256 have no kernel
+        A.paged_kv_decode_attention_bf16(None, wide_out, wide_out.clone(), wide_cache, wide_cache, lens, table,
+                                         A.PagedKvDecodeAttentionConfig.contiguous(**{**good, "head_dim": 320, "heads": 8}))
     A.paged_kv_decode_attention_bf16(None, out, out.clone(), cache, cache, lens, table, config)
     torch.cuda.synchronize()
 

@@ -16,7 +16,7 @@ MAX_ABS, MEAN_ABS, LSE_ABS = 2e-2, 2e-3, 2e-3
 DIM = 128
 
 
-def build(sequences, heads, kv_heads, block_size, seed, gap_tokens=0, extra_blocks=5):
+def build(sequences, heads, kv_heads, block_size, seed, gap_tokens=0, extra_blocks=5, dim=DIM):
     """sequences: (query tokens, keys) pairs.  Tokens are packed in order with `gap_tokens` unowned
     rows between sequences; table rows are slices of a seeded permutation of the pool."""
     rng = np.random.default_rng(seed)
@@ -38,15 +38,16 @@ def build(sequences, heads, kv_heads, block_size, seed, gap_tokens=0, extra_bloc
         used += int(n)
     gen = torch.Generator(device="cuda")
     gen.manual_seed(seed)
-    query = torch.randn((total, heads, DIM), generator=gen, device="cuda").to(torch.bfloat16)
-    kc = torch.randn((blocks, block_size, kv_heads, DIM), generator=gen, device="cuda").to(torch.bfloat16)
-    vc = torch.randn((blocks, block_size, kv_heads, DIM), generator=gen, device="cuda").to(torch.bfloat16)
+    query = torch.randn((total, heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
+    kc = torch.randn((blocks, block_size, kv_heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
+    vc = torch.randn((blocks, block_size, kv_heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
     return lens_q, lens_kv, np.array(offsets, dtype=np.int32), table, stride, blocks, total, query, kc, vc
 
 
-def run_case(sequences, heads, kv_heads, block_size, causal, seed=0, gap_tokens=0, scale=None, dtype=torch.bfloat16):
+def run_case(sequences, heads, kv_heads, block_size, causal, seed=0, gap_tokens=0, scale=None, dtype=torch.bfloat16, dim=DIM):
+    DIM = dim
     lens_q, lens_kv, offsets, table, stride, blocks, total, query, kc, vc = build(sequences, heads, kv_heads, block_size,
-                                                                                seed, gap_tokens)
+                                                                                seed, gap_tokens, dim=dim)
     query, kc, vc = query.to(dtype), kc.to(dtype), vc.to(dtype)
     scale = DIM ** -0.5 if scale is None else scale
     config = A.PagedKvPrefillAttentionConfig.contiguous(len(sequences), total, heads, kv_heads, DIM, block_size, blocks,
@@ -127,17 +128,20 @@ def test_validation_mirrors_reference_cases():
     assert config.output_len() == 224 and config.lse_len() == 28
     with pytest.raises(error.InvalidLength):
         A.PagedKvPrefillAttentionConfig.contiguous(2, 7, 3, 2, 8, 3, 5, 4, True, 0.5)
-    # A short lse is refused before anything is launched (tests.rs:356-366); head_dim 8 itself is
-    # outside this build's bf16 kernel and reported as an unsupported width after the length checks.
+    # A short lse is refused before anything is launched (tests.rs:356-366); a head dimension past 256 has no
+    # kernel and is reported as an unsupported width after the length checks.
     bf16 = lambda n: torch.zeros(n, device="cuda", dtype=torch.bfloat16)
     i32 = lambda n: torch.zeros(n, device="cuda", dtype=torch.int32)
     with pytest.raises(error.LengthTooShort) as caught:
         A.paged_kv_prefill_attention_bf16(None, bf16(224), torch.zeros(27, device="cuda"), bf16(224), bf16(240), bf16(240),
                                           i32(2), i32(2), i32(2), i32(8), config)
     assert caught.value.name == "lse" and caught.value.minimum == 28 and caught.value.actual == 27
+    A.paged_kv_prefill_attention_bf16(None, bf16(224), torch.zeros(28, device="cuda"), bf16(224), bf16(240), bf16(240),
+                                      i32(2), i32(2), i32(2), i32(8), config)  # the reference's own shape runs
+    wide = A.PagedKvPrefillAttentionConfig.contiguous(2, 7, 4, 2, 320, 3, 5, 4, True, 0.5)
     with pytest.raises(error.UnsupportedWidth):
-        A.paged_kv_prefill_attention_bf16(None, bf16(224), torch.zeros(28, device="cuda"), bf16(224), bf16(240), bf16(240),
-                                          i32(2), i32(2), i32(2), i32(8), config)
+        A.paged_kv_prefill_attention_bf16(None, bf16(7 * 4 * 320), torch.zeros(28, device="cuda"), bf16(7 * 4 * 320),
+                                          bf16(5 * 3 * 2 * 320), bf16(5 * 3 * 2 * 320), i32(2), i32(2), i32(2), i32(8), wide)
 
 
 def test_out_of_range_sequence_is_skipped():

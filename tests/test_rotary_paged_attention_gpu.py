@@ -25,7 +25,7 @@ def bf16_round(array):
 
 def oracle_rotation(query, cos, sin, norm):
     """The query path of the rotate-and-append restatement, on a one-cell dummy cache."""
-    tokens = query.shape[0]
+    tokens, DIM = query.shape[0], query.shape[2]
     key = np.zeros((tokens, 1, DIM), dtype=np.float32)
     cache = np.zeros((1, 1, 1, DIM), dtype=np.float32)
     cells = np.zeros(tokens, dtype=np.int64)
@@ -34,7 +34,8 @@ def oracle_rotation(query, cos, sin, norm):
     return rotated
 
 
-def run_case(sequences, heads, kv_heads, page_size, table_dtype, index_dtype, norm, options, seed):
+def run_case(sequences, heads, kv_heads, page_size, table_dtype, index_dtype, norm, options, seed, dim=DIM):
+    DIM = dim
     gen = torch.Generator(device="cuda")
     gen.manual_seed(seed)
     query_offsets, page_offsets, last, table = [0], [0], [], []
@@ -104,12 +105,20 @@ def test_fused_rotation_options():
     run_case(SEQUENCES, 8, 2, 16, torch.float32, torch.int32, None, neural.AttentionOptions(), seed=4)
 
 
+@pytest.mark.parametrize("norm", [None, "weighted"])
+@pytest.mark.parametrize("heads,kv_heads,page_size,table_dtype,index_dtype", [
+    (8, 2, 16, torch.float32, torch.int32), (8, 1, 7, torch.bfloat16, torch.int64)])
+def test_fused_rotation_at_head_dim_64(heads, kv_heads, page_size, table_dtype, index_dtype, norm):
+    run_case(SEQUENCES, heads, kv_heads, page_size, table_dtype, index_dtype, norm, neural.AttentionOptions(causal=True),
+             seed=heads + page_size, dim=64)
+
+
 def test_fused_rotation_refuses_what_it_does_not_take():
-    q = torch.zeros((2, 2, 64), device="cuda", dtype=torch.bfloat16)
-    cache = torch.zeros((2, 4, 2, 64), device="cuda", dtype=torch.bfloat16)
+    q = torch.zeros((2, 2, 96), device="cuda", dtype=torch.bfloat16)
+    cache = torch.zeros((2, 4, 2, 96), device="cuda", dtype=torch.bfloat16)
     index = lambda values: torch.tensor(values, dtype=torch.int32, device="cuda")
     paging = neural.Paging(index([0, 2]), index([0, 1]), index([0]), index([2]))
-    angles = torch.zeros((2, 1, 32), device="cuda")
+    angles = torch.zeros((2, 1, 48), device="cuda")
     with pytest.raises(error.UnsupportedWidth):
         neural.rotary_paged_attention(q, cache, cache, paging, angles, angles)
     q128 = torch.zeros((2, 2, 128), device="cuda", dtype=torch.bfloat16)
