@@ -46,7 +46,8 @@ typedef enum SingeHipStatus {
     SINGE_HIP_TUNE_CACHE_MISS = 11,      /* Error::TuneCacheMiss { op }: TuningChoice::Cached without a cached entry */
     SINGE_HIP_AUTOTUNE_DURING_CAPTURE = 12, /* Error::AutotuneDuringCapture { op } */
     SINGE_HIP_NO_TUNE_CANDIDATES = 13,   /* Error::NoTuneCandidates { op } */
-    SINGE_HIP_NO_SUCCESSFUL_TUNE_CANDIDATES = 14 /* Error::NoSuccessfulTuneCandidates { op } */
+    SINGE_HIP_NO_SUCCESSFUL_TUNE_CANDIDATES = 14, /* Error::NoSuccessfulTuneCandidates { op } */
+    SINGE_HIP_STALE_RECORD = 15          /* singe::Error::StaleRecord { key }: parameters the kernels do not take */
 } SingeHipStatus;
 
 /* Details of the last non-zero status returned on the calling thread. */
@@ -510,6 +511,21 @@ SINGE_HIP_API int32_t singe_hip_paged_attention_f32(
     float* lse,
     uint32_t* status,
     const SingePagedAttentionProblem* problem);
+/* f64 tensors, computed in f64 as the CPU path and the reference's general kernel do (paged_general.rs:91-99); the
+ * log-sum-exp stays f32. */
+SINGE_HIP_API int32_t singe_hip_paged_attention_f64(
+    void* stream,
+    const double* query_rows,
+    const double* key_cache,
+    const double* value_cache,
+    const void* query_offsets,
+    const void* page_offsets,
+    const void* pages,
+    const void* last_page_lengths,
+    double* output,
+    float* lse,
+    uint32_t* status,
+    const SingePagedAttentionProblem* problem);
 SINGE_HIP_API int32_t singe_hip_paged_attention_f16(
     void* stream,
     const uint16_t* query_rows,
@@ -541,6 +557,7 @@ SINGE_HIP_API int32_t singe_hip_paged_attention_f16(
 #define SINGE_HIP_F32 0
 #define SINGE_HIP_BF16 1
 #define SINGE_HIP_F16 2
+#define SINGE_HIP_F64 3   /* the vector-unit kernels only, with f64 arithmetic (attention.rs:63-69; paged_general.rs:91-99) */
 typedef struct SingeAttentionProblem {
     int64_t batch;
     int64_t heads;
@@ -550,7 +567,7 @@ typedef struct SingeAttentionProblem {
     int64_t head_dim;
     int64_t value_dim;
     int64_t mask_strides[4];
-    int32_t data_type;     /* SINGE_HIP_F32, _BF16 or _F16 */
+    int32_t data_type;     /* SINGE_HIP_F32, _BF16, _F16 or _F64 */
     uint8_t causal;
     uint8_t has_scale;
     uint8_t has_window;
@@ -570,6 +587,66 @@ SINGE_HIP_API int32_t singe_hip_scaled_dot_product_attention(
     const int32_t* key_lengths,
     void* output,
     const SingeAttentionProblem* problem);
+
+/* The same op with scratch for key splits (the reference's fused_attention plans the same: few blocks and many keys
+ * split the keys into chunks attended separately and combined after, singe/src/backend/cuda/kernel_plan/source/
+ * attention.rs:283-292, 420-452, 588-654).  A decode-shaped call (few query rows, many keys) has one workgroup per
+ * (batch, head) and cannot fill the chip; given scratch, bf16 / f16 calls at head_dim 128 or 64 share the keys of a
+ * query tile out over several workgroups, each leaving a normalised f32 partial and its base-two log-sum-exp, and a
+ * second kernel merges them (sinks join the first share).  ..._scratch_bytes says how much the problem wants (0: it
+ * would not split, by SingeAttentionParameters.split_below_blocks and the key count); with a null or smaller buffer,
+ * and for every other type and width, the call is singe_hip_scaled_dot_product_attention.  The scratch holds nothing
+ * between calls; calls that share it must not overlap. */
+SINGE_HIP_API size_t singe_hip_scaled_dot_product_attention_scratch_bytes(const SingeAttentionProblem* problem);
+SINGE_HIP_API int32_t singe_hip_scaled_dot_product_attention_scratch(
+    void* stream,
+    const void* query,
+    const void* key,
+    const void* value,
+    const void* mask,
+    const void* sinks,
+    const int32_t* key_lengths,
+    void* output,
+    void* scratch,
+    size_t scratch_bytes,
+    const SingeAttentionProblem* problem);
+
+/* ---- singe surface: the choices the attention kernels leave open ----------------------------------------
+ * AttentionParameters (singe/src/backend/cuda/kernel_plan/source/parameters.rs:21-57), field for field.  On gfx950:
+ *   warps               4: a workgroup is four waves of 32 query rows; nothing else is built
+ *   key_tile            64: keys per LDS stage; nothing else is built
+ *   stages              1 or 2: both name the one pipeline the kernels have (LDS always holds the tiles to come:
+ *                       three stages of K, two of V), so a record tuned to either runs the same code
+ *   split_below_blocks  a launch of fewer workgroups than this splits its keys, into
+ *                       min(ceil(2 * split_below_blocks / workgroups), ceil(keys / (4 * key_tile)), 16) shares
+ *                       (attention.rs:283-292), given scratch; 0 never splits.  Default: twice the compute units
+ *   min_blocks          none, or 2: the kernels are built with two workgroups per compute unit
+ * ..._candidates lists what the kernels take on the current device, the default first, as attention_candidates does
+ * (attention.rs:113-160); ..._set installs one of them for the paged op and the dense op of this process (null: the
+ * default) and returns SINGE_HIP_STALE_RECORD for anything else, as the reference refuses a record whose parameters
+ * its kernel no longer takes (parameters.rs:245-250) instead of quietly running the default. */
+typedef struct SingeAttentionParameters {
+    size_t warps;
+    size_t key_tile;
+    size_t stages;
+    size_t split_below_blocks;
+    uint8_t has_min_blocks;   /* Option<u32> min_blocks */
+    uint32_t min_blocks;
+} SingeAttentionParameters;
+SINGE_HIP_API void singe_hip_attention_parameters_default(SingeAttentionParameters* parameters);
+SINGE_HIP_API int32_t singe_hip_attention_candidates(SingeAttentionParameters* candidates, size_t capacity, size_t* count);
+SINGE_HIP_API int32_t singe_hip_set_attention_parameters(const SingeAttentionParameters* parameters);
+SINGE_HIP_API void singe_hip_attention_parameters(SingeAttentionParameters* parameters);
+/* parameter_key (parameters.rs:221-230): the key a tuning record of the op is stored under,
+ * "kernel|<label>|<numerical policy>|<attributes>" followed by " <type><dimensions><strides>+<offset % 8>" per
+ * operand, spelled as Rust's Debug spells them, for contiguous operands at offset 0: label "paged_attention" with
+ * its seven operands, or "attention" with query, key, value (a mask, sinks and key lengths are flags of the
+ * attributes).  Writes at most capacity bytes, NUL included, and returns the length the whole key needs without it
+ * (0 on a null problem). */
+SINGE_HIP_API size_t singe_hip_paged_attention_parameter_key(const SingePagedAttentionProblem* problem, int32_t data_type,
+                                                             char* buffer, size_t capacity);
+SINGE_HIP_API size_t singe_hip_attention_parameter_key(const SingeAttentionProblem* problem, int32_t masked, int32_t sinks,
+                                                       int32_t key_lengths, char* buffer, size_t capacity);
 
 /* ---- singe-kernel surface: split-KV reduce -----------------------------------------------------------
  * Mirrors SplitKReduceConfig (singe-kernel/src/cuda/attention/mod.rs:385-398); strides in elements.

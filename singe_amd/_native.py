@@ -12,7 +12,7 @@ LIBRARY_PATH = os.path.join(_HERE, "libsinge_hip_attention.so")
 CODE_OBJECT_PARTS = ("paged_decode", "fmha_prefill", "fmha_prefill_f32", "paged_attention", "splitk_reduce",
                      "attention_rows_f32", "cache_ops", "latent_attention", "latent_attention_mfma",
                      "general_attention_f32", "general_attention_bf16", "general_attention_f16", "mfma_ceiling",
-                     "paged_decode_d64", "fmha_prefill_d64", "paged_attention_d64")
+                     "paged_decode_d64", "fmha_prefill_d64", "paged_attention_d64", "general_attention_f64")
 CODE_OBJECT_PATHS = [os.path.join(_HERE, f"singe_attention_gfx950.{part}.hsaco") for part in CODE_OBJECT_PARTS]
 
 c_size = ctypes.c_size_t
@@ -108,6 +108,11 @@ class PagedMlaAttentionProblemC(ctypes.Structure):
                 ("scale", ctypes.c_float)]
 
 
+class AttentionParametersC(ctypes.Structure):
+    _fields_ = [("warps", c_size), ("key_tile", c_size), ("stages", c_size), ("split_below_blocks", c_size),
+                ("has_min_blocks", ctypes.c_uint8), ("min_blocks", ctypes.c_uint32)]
+
+
 class QueryRotationC(ctypes.Structure):
     _fields_ = [("table_type", ctypes.c_int32), ("has_norm", ctypes.c_uint8), ("eps", ctypes.c_float)]
 
@@ -126,7 +131,7 @@ class PagingIndicesProblemC(ctypes.Structure):
                 ("row_elements", ctypes.c_int64), ("index_type", ctypes.c_int32)]
 
 
-DATA_TYPE_F32, DATA_TYPE_BF16, DATA_TYPE_F16 = 0, 1, 2
+DATA_TYPE_F32, DATA_TYPE_BF16, DATA_TYPE_F16, DATA_TYPE_F64 = 0, 1, 2, 3
 
 _lib = None
 
@@ -152,6 +157,23 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_unload.restype = None
     handle.singe_hip_kernel.argtypes = [i32, ctypes.POINTER(ctypes.c_char_p), ctypes.POINTER(ctypes.c_char_p)]
     handle.singe_hip_kernel.restype = i32
+    parameters = ctypes.POINTER(AttentionParametersC)
+    handle.singe_hip_attention_parameters_default.argtypes = [parameters]
+    handle.singe_hip_attention_parameters_default.restype = None
+    handle.singe_hip_attention_parameters.argtypes = [parameters]
+    handle.singe_hip_attention_parameters.restype = None
+    handle.singe_hip_attention_candidates.argtypes = [parameters, c_size, ctypes.POINTER(c_size)]
+    handle.singe_hip_attention_candidates.restype = i32
+    handle.singe_hip_set_attention_parameters.argtypes = [parameters]
+    handle.singe_hip_set_attention_parameters.restype = i32
+    handle.singe_hip_paged_attention_parameter_key.argtypes = [ctypes.POINTER(PagedAttentionProblemC), i32, ctypes.c_char_p, c_size]
+    handle.singe_hip_paged_attention_parameter_key.restype = c_size
+    handle.singe_hip_attention_parameter_key.argtypes = [ctypes.POINTER(AttentionProblemC), i32, i32, i32, ctypes.c_char_p, c_size]
+    handle.singe_hip_attention_parameter_key.restype = c_size
+    handle.singe_hip_scaled_dot_product_attention_scratch_bytes.argtypes = [ctypes.POINTER(AttentionProblemC)]
+    handle.singe_hip_scaled_dot_product_attention_scratch_bytes.restype = c_size
+    handle.singe_hip_scaled_dot_product_attention_scratch.argtypes = [c_void] * 8 + [c_void, c_size, ctypes.POINTER(AttentionProblemC)]
+    handle.singe_hip_scaled_dot_product_attention_scratch.restype = i32
     handle.singe_hip_mfma_ceiling.argtypes = [c_void, c_void, c_size, c_void, c_size, ctypes.c_uint32, ctypes.c_uint32, i32]
     handle.singe_hip_mfma_ceiling.restype = i32
     handle.singe_hip_prepare.argtypes = [ctypes.POINTER(i32)]
@@ -239,6 +261,8 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_set_paged_mla_attention_splits.restype = None
     handle.singe_hip_paged_attention_f32.argtypes = [c_void] * 11 + [ctypes.POINTER(PagedAttentionProblemC)]
     handle.singe_hip_paged_attention_f32.restype = i32
+    handle.singe_hip_paged_attention_f64.argtypes = [c_void] * 11 + [ctypes.POINTER(PagedAttentionProblemC)]
+    handle.singe_hip_paged_attention_f64.restype = i32
     handle.singe_hip_paged_attention_f16.argtypes = [c_void] * 11 + [ctypes.POINTER(PagedAttentionProblemC)]
     handle.singe_hip_paged_attention_f16.restype = i32
     handle.singe_hip_scaled_dot_product_attention.argtypes = [c_void] * 8 + [ctypes.POINTER(AttentionProblemC)]
@@ -298,5 +322,6 @@ def check(status: int, op: str = "") -> None:
         12: lambda: error.AutotuneDuringCapture(f"autotune during stream capture for {name or op}"),
         13: lambda: error.NoTuneCandidates(f"no tune candidates for {name or op}"),
         14: lambda: error.NoTuneCandidates(f"no tune candidate completed for {name or op}"),
+        15: lambda: error.StaleRecord(f"stale record: {name or op}"),
     }
     raise table.get(status, lambda: error.Error(f"status {status}"))()

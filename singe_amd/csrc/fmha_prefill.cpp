@@ -159,7 +159,7 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
         o.out_strides[0] = c.output_batch_stride, o.out_strides[1] = c.output_head_stride, o.out_strides[2] = c.output_sequence_stride;
         o.batch = c.batch, o.heads = c.heads, o.kv_heads = c.kv_heads, o.query_len = c.query_len, o.key_len = c.key_len;
         o.head_dim = o.value_dim = c.head_dim;
-        o.causal = c.causal != 0, o.scale = c.scale;
+        o.causal = c.causal != 0, o.scale = c.scale, o.scale_wide = c.scale;
         return dense_general(f16 ? SINGE_HIP_F16 : SINGE_HIP_BF16, stream, f16 ? "fmha_prefill_f16" : "fmha_prefill_bf16", o);
     }
     const size_t strides[] = {c.query_batch_stride, c.key_batch_stride, c.value_batch_stride, c.output_batch_stride,
@@ -218,15 +218,45 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
         args.cap_log2e = std::fabs(options.softcap) * 1.4426950408889634074f;
     }
     const uint64_t rows = (static_cast<uint64_t>(c.batch) * c.heads + 7) / 8 * 8;
-    const uint64_t groups = rows * ((args.query_tiles + 1) / 2);  // a workgroup takes a pair of query tiles
+    uint64_t groups = rows * ((args.query_tiles + 1) / 2);  // a workgroup takes a pair of query tiles
     if (groups > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
+    // Key splits, when the caller lent scratch for them and the launch is too small to fill the chip.
+    uint32_t splits = options.scratch != nullptr ? dense_prefill_splits(c) : 1;
+    if (splits > 1 && (options.scratch_bytes < dense_prefill_scratch_bytes(c, splits) || groups * splits > 0x7fffffffull)) splits = 1;
+    args.splits = splits;
+    if (splits > 1) {
+        const size_t row_count = static_cast<size_t>(c.batch) * c.heads * c.query_len;
+        args.partial_out = static_cast<float*>(options.scratch);
+        args.partial_lse = args.partial_out + static_cast<size_t>(splits) * row_count * c.head_dim;
+        groups *= splits;
+    }
+    const bool narrow = c.head_dim == 64;
     const KernelId kernel = static_cast<KernelId>((f16 ? kPrefillCausalF16 : kPrefillCausal) + (c.causal ? 0 : 1) + (with_options ? 4 : 0));
-    return launch(c.head_dim == 64 ? at_head_dim_64(kernel) : kernel, static_cast<unsigned>(groups), 1, 1, 64 * kDensePrefillWaves, stream, args);
+    if (int32_t status = launch(narrow ? at_head_dim_64(kernel) : kernel, static_cast<unsigned>(groups), 1, 1, 64 * kDensePrefillWaves, stream, args))
+        return status;
+    if (splits == 1) return 0;
+    const uint64_t merge_groups = (static_cast<uint64_t>(c.batch) * c.heads * c.query_len + 3) / 4;
+    if (merge_groups > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
+    const KernelId merge = static_cast<KernelId>((narrow ? kPrefillCombineD64 : kPrefillCombine) + (f16 ? 1 : 0));
+    return launch(merge, static_cast<unsigned>(merge_groups), 1, 1, 256, stream, args);
 }
 
 }  // namespace
 
 namespace singe_hip {
+
+uint32_t dense_prefill_splits(const SingeFmhaPrefillConfig& c) {
+    if ((c.head_dim != 128 && c.head_dim != 64) || c.batch == 0 || c.heads == 0 || c.query_len == 0) return 1;
+    constexpr size_t kTileRows = 32 * kDensePrefillWaves;
+    const uint64_t query_tiles = (c.query_len + kTileRows - 1) / kTileRows;
+    const uint64_t workgroups = static_cast<uint64_t>(c.batch) * c.heads * ((query_tiles + 1) / 2);
+    return attention_key_splits(workgroups, c.key_len);
+}
+
+size_t dense_prefill_scratch_bytes(const SingeFmhaPrefillConfig& c, uint32_t splits) {
+    if (splits <= 1) return 0;
+    return static_cast<size_t>(splits) * c.batch * c.heads * c.query_len * (c.head_dim + 1) * sizeof(float);
+}
 
 // The dense op's way into the matrix-core kernel: the public entry points' checks and launch, plus the op's options
 // (general_attention.cpp).

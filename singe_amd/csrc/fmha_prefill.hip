@@ -32,7 +32,7 @@ constexpr int kDenseWaves = kDensePrefillWaves;
 // OPTIONS: the dense op's additive mask, window and score cap, applied block by block to the scaled scores; every
 // tile then takes the masked path.
 template <bool CAUSAL, class Half, int WAVES, bool OPTIONS>
-SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, unsigned int bh, unsigned int query_tile) {
+SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, unsigned int bh, unsigned int query_tile, unsigned int split) {
     constexpr unsigned int kRows = 32u * WAVES;        // query rows of the workgroup
     constexpr unsigned int kLoadRows = 4u * WAVES;     // key rows one load instruction of every wave brings in
     constexpr unsigned int kLoads = kKeyTile / kLoadRows;
@@ -86,11 +86,28 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
         const unsigned int reach = query_tile * kRows + kRows;
         key_end = key_end < reach ? key_end : reach;
     }
-    const unsigned int tiles = (key_end + kKeyTile - 1) / kKeyTile;
+    unsigned int tiles = (key_end + kKeyTile - 1) / kKeyTile;
     unsigned int wave_blocks = (key_end + 31u) / 32u;
     if (CAUSAL) {
         const unsigned int seen = (first_row + 31u) / 32u + 1u;
         wave_blocks = wave_blocks < seen ? wave_blocks : seen;
+    }
+    // The first tile any row of the workgroup can see: 0, or with a window the tile of the first key the
+    // workgroup's first row still sees (later rows see later keys).
+    unsigned int first_tile = 0;
+    if (OPTIONS && a.window >= 0) {
+        const unsigned long long low = static_cast<unsigned long long>(query_tile) * kRows + 1u;
+        const unsigned long long window = static_cast<unsigned long long>(a.window);
+        if (low > window) first_tile = static_cast<unsigned int>((low - window) / kKeyTile);
+        first_tile = first_tile < tiles ? first_tile : tiles;
+    }
+    if (a.splits > 1) {
+        // This workgroup's share of the tiles; a share may be empty, and ends with its last tile.
+        const unsigned int share = tiles > first_tile ? (tiles - first_tile + a.splits - 1) / a.splits : 0u;
+        first_tile += split * share;
+        tiles = tiles < first_tile + share ? tiles : first_tile + share;
+        first_tile = first_tile < tiles ? first_tile : tiles;
+        wave_blocks = wave_blocks < 2u * tiles ? wave_blocks : 2u * tiles;
     }
 
     // A tile load is 1024 16-byte chunks per operand: instruction i of wave w fills rows 16 i + 4 w .. + 3
@@ -144,7 +161,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
 
     RowState state;
     reset(state);
-    if (a.sinks != nullptr) {
+    if (a.sinks != nullptr && split == 0) {
         // The head's sink: a score that is always there and weighs no value.  The row starts with it as its reference
         // point and a sum of one (held by one of the row's two lanes).
         const uint16_t bits = a.sinks[head];
@@ -156,15 +173,6 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     }
     const ReadOffsets offsets = read_offsets(lane);
 
-    // The first tile any row of the workgroup can see: 0, or with a window the tile of the first key the
-    // workgroup's first row still sees (later rows see later keys).
-    unsigned int first_tile = 0;
-    if (OPTIONS && a.window >= 0) {
-        const unsigned long long low = static_cast<unsigned long long>(query_tile) * kRows + 1u;
-        const unsigned long long window = static_cast<unsigned long long>(a.window);
-        if (low > window) first_tile = static_cast<unsigned int>((low - window) / kKeyTile);
-        first_tile = first_tile < tiles ? first_tile : tiles;
-    }
     if (first_tile < tiles) {
         load_keys(first_tile, lds);
         load_values(first_tile, lds + kValueBase);
@@ -335,7 +343,19 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     // Normalise and store.  Lane (query, hi) holds dims 32db + 8(r / 4) + 4hi + (r % 4).
     const float sum = swap32_sum(state.running_sum);
     const float inverse = sum > 0.0f ? 1.0f / sum : 0.0f;
-    if (query_valid) {
+    if (query_valid && a.splits > 1) {
+        const size_t flat = (static_cast<size_t>(batch) * a.heads + head) * a.query_len + my_query;
+        const size_t slot = static_cast<size_t>(split) * a.batch * a.heads * a.query_len + flat;
+        float* row = a.partial_out + slot * kHeadDim;
+#pragma unroll
+        for (int db = 0; db < kDimBlocks; ++db)
+#pragma unroll
+            for (int quad = 0; quad < 4; ++quad)
+                *reinterpret_cast<float4*>(row + 32 * db + 8 * quad + 4 * hi) =
+                    make_float4(state.out[db][4 * quad + 0] * inverse, state.out[db][4 * quad + 1] * inverse,
+                                state.out[db][4 * quad + 2] * inverse, state.out[db][4 * quad + 3] * inverse);
+        if (hi == 0) a.partial_lse[slot] = sum > 0.0f ? state.reference + fast_log2(sum) : -INFINITY;
+    } else if (query_valid) {
         uint16_t* row = a.out + batch * a.output_batch_stride + static_cast<size_t>(my_query) * a.output_sequence_stride +
                         head * a.output_head_stride;
 #pragma unroll
@@ -356,13 +376,51 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
 // Workgroup id -> (batch * heads + head, pair of query tiles): see the header comment.
 template <bool CAUSAL, class Half, int WAVES, bool OPTIONS = false>
 SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
-    const unsigned int xcd = blockIdx.x & 7u, within = blockIdx.x >> 3;
+    const unsigned int xcd = blockIdx.x & 7u;
+    unsigned int within = blockIdx.x >> 3;
+    const unsigned int split = within % a.splits;  // the shares of a query tile are neighbours
+    within /= a.splits;
     const unsigned int pairs = (a.query_tiles + 1u) / 2u;
     const unsigned int bh = (within / pairs) * 8u + xcd;
     if (bh >= a.batch * a.heads) return;
     const unsigned int light = within % pairs, heavy = a.query_tiles - 1u - light;
-    fmha_prefill_tile<CAUSAL, Half, WAVES, OPTIONS>(a, lds, bh, heavy);
-    if (light != heavy) fmha_prefill_tile<CAUSAL, Half, WAVES, OPTIONS>(a, lds, bh, light);
+    fmha_prefill_tile<CAUSAL, Half, WAVES, OPTIONS>(a, lds, bh, heavy, split);
+    if (light != heavy) fmha_prefill_tile<CAUSAL, Half, WAVES, OPTIONS>(a, lds, bh, light, split);
+}
+
+// Merges the key splits of a row: each share's rows weigh 2^(lse - largest) over the sum of those (the reference's
+// combine, singe/src/backend/cuda/kernel_plan/source/attention.rs:588-654).  A wave per (batch, head, query) row; a lane
+// takes two of the row's values.
+template <class Half>
+SINGE_DEVICE void fmha_prefill_combine_body(const PrefillArgs& a) {
+    const unsigned int lane = threadIdx.x & 63u;
+    const size_t rows_total = static_cast<size_t>(a.batch) * a.heads * a.query_len;
+    const size_t flat = static_cast<size_t>(blockIdx.x) * 4u + (threadIdx.x >> 6);
+    if (flat >= rows_total) return;
+    const unsigned int query = static_cast<unsigned int>(flat % a.query_len);
+    const unsigned int head = static_cast<unsigned int>((flat / a.query_len) % a.heads);
+    const unsigned int batch = static_cast<unsigned int>(flat / (static_cast<size_t>(a.query_len) * a.heads));
+    const float mine = lane < a.splits ? a.partial_lse[lane * rows_total + flat] : -INFINITY;
+    float largest = mine;
+#pragma unroll
+    for (int step = 32; step > 0; step >>= 1) largest = fmaxf(largest, __shfl_xor(largest, step, 64));
+    const float weight = mine == -INFINITY ? 0.0f : fast_exp2(mine - largest);  // an empty share weighs nothing
+    float total = weight;
+#pragma unroll
+    for (int step = 32; step > 0; step >>= 1) total += __shfl_xor(total, step, 64);
+    const bool holds_values = 2u * lane < static_cast<unsigned int>(kHeadDim);
+    float2 merged = make_float2(0.0f, 0.0f);
+    for (unsigned int s = 0; s < a.splits; ++s) {
+        const float w = __shfl(weight, s, 64);
+        if (w == 0.0f || !holds_values) continue;
+        const float2 part = *reinterpret_cast<const float2*>(a.partial_out + (s * rows_total + flat) * kHeadDim + 2u * lane);
+        merged.x = fmaf(w, part.x, merged.x);
+        merged.y = fmaf(w, part.y, merged.y);
+    }
+    const float inverse = total > 0.0f ? 1.0f / total : 0.0f;
+    uint16_t* row = a.out + batch * a.output_batch_stride + static_cast<size_t>(query) * a.output_sequence_stride + head * a.output_head_stride;
+    if (holds_values) reinterpret_cast<unsigned int*>(row)[lane] = pack_pair(Half{}, merged.x * inverse, merged.y * inverse);
+    if (a.lse != nullptr && lane == 0) a.lse[flat] = total > 0.0f ? (largest + fast_log2(total)) * kLn2 : -INFINITY;
 }
 
 }  // namespace
@@ -392,3 +450,5 @@ SINGE_FMHA_PREFILL_KERNEL(SINGE_PREFILL_NAME(bf16, _causal), true, Bf16)
 SINGE_FMHA_PREFILL_KERNEL(SINGE_PREFILL_NAME(bf16, _full), false, Bf16)
 SINGE_FMHA_PREFILL_KERNEL(SINGE_PREFILL_NAME(f16, _causal), true, F16)
 SINGE_FMHA_PREFILL_KERNEL(SINGE_PREFILL_NAME(f16, _full), false, F16)
+extern "C" __global__ __launch_bounds__(256) void SINGE_PREFILL_NAME(bf16, _combine)(PrefillArgs args) { fmha_prefill_combine_body<prefill::Bf16>(args); }
+extern "C" __global__ __launch_bounds__(256) void SINGE_PREFILL_NAME(f16, _combine)(PrefillArgs args) { fmha_prefill_combine_body<prefill::F16>(args); }

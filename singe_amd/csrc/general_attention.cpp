@@ -17,11 +17,14 @@ namespace {
 // Kernel of a family for (element, widest dimension): families are laid out element-major with
 // the 64 / 128 / 256 variants consecutive.
 int32_t pick(KernelId base, int32_t data_type, uint64_t widest, const char* op, KernelId* kernel) {
-    if (data_type != SINGE_HIP_F32 && data_type != SINGE_HIP_BF16 && data_type != SINGE_HIP_F16)
+    if (data_type != SINGE_HIP_F32 && data_type != SINGE_HIP_BF16 && data_type != SINGE_HIP_F16 && data_type != SINGE_HIP_F64)
         return fail(SINGE_HIP_INVALID_ARGUMENT, "data type");
     if (widest > 256) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, op, widest, 0);
     const int width = widest <= 64 ? 0 : widest <= 128 ? 1 : 2;
-    *kernel = static_cast<KernelId>(base + 3 * data_type + width);
+    if (data_type == SINGE_HIP_F64)  // the f64 kernels sit after the others: dense, then paged
+        *kernel = static_cast<KernelId>((base == kDenseGeneral ? kDenseGeneralF64 : kPagedGeneralF64) + width);
+    else
+        *kernel = static_cast<KernelId>(base + 3 * data_type + width);
     return 0;
 }
 
@@ -68,6 +71,7 @@ int32_t paged_attention_general(int32_t data_type, void* stream, const void* que
     args.has_softcap = p.has_softcap ? 1u : 0u;
     args.form = p.index_type == SINGE_HIP_INDEX_I64 ? 1u : 0u;
     args.scale = scale;
+    args.scale_wide = p.has_scale ? static_cast<double>(p.scale) : 1.0 / std::sqrt(static_cast<double>(p.head_dim));
     args.softcap = p.has_softcap ? p.softcap : 0.0f;
     const uint64_t blocks = row_blocks * static_cast<uint64_t>(p.sequences);
     if (blocks > 0x7fffffffull || row_blocks > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
@@ -114,6 +118,7 @@ int32_t paged_table_general(int32_t data_type, void* stream, const char* op, con
     args.has_softcap = 0;
     args.form = decode ? 3u : 2u;
     args.scale = scale;
+    args.scale_wide = scale;
     args.softcap = 0.0f;
     const uint64_t blocks = row_blocks * sequences;
     if (blocks > 0x7fffffffull || row_blocks > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
@@ -153,6 +158,7 @@ int32_t dense_general(int32_t data_type, void* stream, const char* op, const Den
     args.causal = o.causal ? 1u : 0u;
     args.has_softcap = o.has_softcap ? 1u : 0u;
     args.scale = o.scale;
+    args.scale_wide = o.scale_wide;
     args.softcap = o.softcap;
     const uint64_t rows = o.batch * o.heads * o.query_len;
     const uint64_t blocks = (rows + 3) / 4;
@@ -162,9 +168,30 @@ int32_t dense_general(int32_t data_type, void* stream, const char* op, const Den
 
 }  // namespace singe_hip
 
-extern "C" int32_t singe_hip_scaled_dot_product_attention(void* stream, const void* query, const void* key, const void* value,
-                                                          const void* mask, const void* sinks, const int32_t* key_lengths,
-                                                          void* output, const SingeAttentionProblem* problem) {
+namespace {
+
+// The config the matrix-core dense kernels read a [batch, heads, len, dim] problem through.
+SingeFmhaPrefillConfig matrix_core_config(const SingeAttentionProblem& p, float scale) {
+    const size_t dim = static_cast<size_t>(p.head_dim);
+    SingeFmhaPrefillConfig c;
+    c.batch = p.batch, c.query_len = p.query_len, c.key_len = p.key_len, c.heads = p.heads, c.kv_heads = p.kv_heads, c.head_dim = dim;
+    c.query_batch_stride = c.output_batch_stride = static_cast<size_t>(p.heads) * p.query_len * dim;
+    c.key_batch_stride = c.value_batch_stride = static_cast<size_t>(p.kv_heads) * p.key_len * dim;
+    c.query_sequence_stride = c.key_sequence_stride = c.value_sequence_stride = c.output_sequence_stride = dim;
+    c.query_head_stride = c.output_head_stride = static_cast<size_t>(p.query_len) * dim;
+    c.key_head_stride = c.value_head_stride = static_cast<size_t>(p.key_len) * dim;
+    c.scale = scale, c.causal = p.causal ? 1 : 0;
+    return c;
+}
+
+bool takes_matrix_cores(const SingeAttentionProblem& p) {
+    return (p.data_type == SINGE_HIP_BF16 || p.data_type == SINGE_HIP_F16) && (p.head_dim == 128 || p.head_dim == 64) &&
+           p.value_dim == p.head_dim;
+}
+
+int32_t scaled_dot_product_attention(void* stream, const void* query, const void* key, const void* value, const void* mask,
+                                     const void* sinks, const int32_t* key_lengths, void* output, void* scratch, size_t scratch_bytes,
+                                     const SingeAttentionProblem* problem) {
     if (problem == nullptr) return fail(SINGE_HIP_NULL_POINTER, "problem");
     const SingeAttentionProblem& p = *problem;
     // attention_problem: batch, heads, query length and value dimension may be zero; head dimension and
@@ -190,19 +217,13 @@ extern "C" int32_t singe_hip_scaled_dot_product_attention(void* stream, const vo
 
     // bf16 and f16 at head dimensions 128 and 64 are what the MFMA flash kernels compute, every option included,
     // reading [batch, heads, len, dim] through their strides.
-    if ((p.data_type == SINGE_HIP_BF16 || p.data_type == SINGE_HIP_F16) && (p.head_dim == 128 || p.head_dim == 64) &&
-        p.value_dim == p.head_dim) {
+    if (takes_matrix_cores(p)) {
         const size_t dim = static_cast<size_t>(p.head_dim);
-        SingeFmhaPrefillConfig c;
-        c.batch = p.batch, c.query_len = p.query_len, c.key_len = p.key_len, c.heads = p.heads, c.kv_heads = p.kv_heads, c.head_dim = dim;
-        c.query_batch_stride = c.output_batch_stride = static_cast<size_t>(p.heads) * p.query_len * dim;
-        c.key_batch_stride = c.value_batch_stride = static_cast<size_t>(p.kv_heads) * p.key_len * dim;
-        c.query_sequence_stride = c.key_sequence_stride = c.value_sequence_stride = c.output_sequence_stride = dim;
-        c.query_head_stride = c.output_head_stride = static_cast<size_t>(p.query_len) * dim;
-        c.key_head_stride = c.value_head_stride = static_cast<size_t>(p.key_len) * dim;
-        c.scale = scale, c.causal = p.causal ? 1 : 0;
+        SingeFmhaPrefillConfig c = matrix_core_config(p, scale);
         const size_t q_len = static_cast<size_t>(rows) * dim, kv_len = static_cast<size_t>(p.batch) * p.kv_heads * p.key_len * dim;
         DenseOptions options;
+        options.scratch = scratch;
+        options.scratch_bytes = scratch_bytes;
         options.sinks = static_cast<const uint16_t*>(sinks);
         options.key_lengths = key_lengths;
         options.mask = static_cast<const uint16_t*>(mask);
@@ -228,7 +249,31 @@ extern "C" int32_t singe_hip_scaled_dot_product_attention(void* stream, const vo
     o.head_dim = dim, o.value_dim = value_dim;
     o.causal = p.causal != 0, o.has_softcap = p.has_softcap != 0;
     o.scale = scale, o.softcap = p.has_softcap ? p.softcap : 0.0f;
+    o.scale_wide = p.has_scale ? static_cast<double>(p.scale) : 1.0 / std::sqrt(static_cast<double>(p.head_dim));
     return dense_general(p.data_type, stream, "scaled_dot_product_attention", o);
+}
+
+}  // namespace
+
+extern "C" int32_t singe_hip_scaled_dot_product_attention(void* stream, const void* query, const void* key, const void* value,
+                                                          const void* mask, const void* sinks, const int32_t* key_lengths,
+                                                          void* output, const SingeAttentionProblem* problem) {
+    return scaled_dot_product_attention(stream, query, key, value, mask, sinks, key_lengths, output, nullptr, 0, problem);
+}
+
+extern "C" int32_t singe_hip_scaled_dot_product_attention_scratch(void* stream, const void* query, const void* key, const void* value,
+                                                                  const void* mask, const void* sinks, const int32_t* key_lengths,
+                                                                  void* output, void* scratch, size_t scratch_bytes,
+                                                                  const SingeAttentionProblem* problem) {
+    return scaled_dot_product_attention(stream, query, key, value, mask, sinks, key_lengths, output, scratch, scratch_bytes, problem);
+}
+
+extern "C" size_t singe_hip_scaled_dot_product_attention_scratch_bytes(const SingeAttentionProblem* problem) {
+    if (problem == nullptr || !takes_matrix_cores(*problem) || problem->batch <= 0 || problem->heads <= 0 || problem->query_len <= 0 ||
+        problem->key_len <= 0 || problem->kv_heads <= 0)
+        return 0;
+    const SingeFmhaPrefillConfig c = matrix_core_config(*problem, 1.0f);
+    return dense_prefill_scratch_bytes(c, dense_prefill_splits(c));
 }
 
 // validate_splitk_reduce_config (singe-kernel/src/cuda/attention/mod.rs:3557-3573) and

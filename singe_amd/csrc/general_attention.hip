@@ -5,9 +5,10 @@
 // sinks, key lengths) and :424-538 (paged, FlashInfer form).
 //
 // One wave64 per query row.  Lanes take keys 64 apart; a lane's score is the same left-to-right fma chain
-// over the head dimension as the CPU path, in f32 whatever the storage type (the CPU path widens bf16/f16
-// to f32 first: attention.rs:63-69, 297-330); its softmax is online in natural base with expf, and the 64
-// per-lane partial rows are merged once at the end.
+// over the head dimension as the CPU path, in f32 for f32 / bf16 / f16 storage (the CPU path widens bf16/f16
+// to f32 first: attention.rs:63-69, 297-330) and in f64 for f64 storage (the CPU path and the reference's general
+// kernel compute f64 in f64: attention.rs:63-69, paged_general.rs:91-99); its softmax is online in natural base
+// with exp, and the 64 per-lane partial rows are merged once at the end.
 #include "common.hip.h"
 #include "kernel_args.h"
 #include "paging.hip.h"
@@ -19,93 +20,125 @@ struct Element;
 template <>
 struct Element<kElementF32> {
     typedef float type;
+    typedef float real;  // the type the arithmetic runs in
     static SINGE_DEVICE float load(const type* at) { return *at; }
     static SINGE_DEVICE void store(type* at, float value) { *at = value; }
 };
 template <>
+struct Element<kElementF64> {
+    typedef double type;
+    typedef double real;
+    static SINGE_DEVICE double load(const type* at) { return *at; }
+    static SINGE_DEVICE void store(type* at, double value) { *at = value; }
+};
+template <>
 struct Element<kElementBf16> {
     typedef unsigned short type;
+    typedef float real;
     static SINGE_DEVICE float load(const type* at) { return __builtin_bit_cast(float, static_cast<unsigned int>(*at) << 16); }
     static SINGE_DEVICE void store(type* at, float value) { *at = f32_to_bf16_bits(value); }
 };
 template <>
 struct Element<kElementF16> {
     typedef _Float16 type;
+    typedef float real;
     static SINGE_DEVICE float load(const type* at) { return static_cast<float>(*at); }
     static SINGE_DEVICE void store(type* at, float value) { *at = static_cast<_Float16>(value); }  // round to nearest even
 };
 
+// exp, log, tanh and fma in the arithmetic's own precision.
+SINGE_DEVICE float real_exp(float x) { return expf(x); }
+SINGE_DEVICE double real_exp(double x) { return exp(x); }
+SINGE_DEVICE float real_log(float x) { return logf(x); }
+SINGE_DEVICE double real_log(double x) { return log(x); }
+SINGE_DEVICE float real_tanh(float x) { return tanhf(x); }
+SINGE_DEVICE double real_tanh(double x) { return tanh(x); }
+SINGE_DEVICE float real_fma(float a, float b, float c) { return fmaf(a, b, c); }
+SINGE_DEVICE double real_fma(double a, double b, double c) { return fma(a, b, c); }
+SINGE_DEVICE float real_max(float a, float b) { return fmaxf(a, b); }
+SINGE_DEVICE double real_max(double a, double b) { return fmax(a, b); }
+
+// The scale in the arithmetic's precision (the CPU path derives its default in the tensors' type: attention.rs:82-87).
+template <class R, class Args>
+SINGE_DEVICE R own_scale(const Args& a) {
+    if constexpr (std::is_same<R, double>::value) return a.scale_wide;
+    else return a.scale;
+}
+
 // Per-lane running state over the keys a lane has seen.
-template <int DMAX>
+template <int DMAX, class R = float>
 struct LaneState {
-    float acc[DMAX];
-    float largest;
-    float total;
+    R acc[DMAX];
+    R largest;
+    R total;
 };
 
-template <int DMAX>
-SINGE_DEVICE void reset(LaneState<DMAX>& state) {
+template <int DMAX, class R>
+SINGE_DEVICE void reset(LaneState<DMAX, R>& state) {
 #pragma unroll
-    for (int d = 0; d < DMAX; ++d) state.acc[d] = 0.0f;
+    for (int d = 0; d < DMAX; ++d) state.acc[d] = 0;
     state.largest = -INFINITY;
-    state.total = 0.0f;
+    state.total = 0;
 }
 
 // Folds one key into a lane's state.  A score of -inf (a masked key) weighs nothing.
 template <class E, int DMAX>
-SINGE_DEVICE void fold_key(LaneState<DMAX>& state, const float* q_row, const typename E::type* k_row,
-                           const typename E::type* v_row, unsigned int dim, unsigned int value_dim, float scale,
-                           bool has_softcap, float softcap, float additive) {
-    float score = 0.0f;
+SINGE_DEVICE void fold_key(LaneState<DMAX, typename E::real>& state, const typename E::real* q_row, const typename E::type* k_row,
+                           const typename E::type* v_row, unsigned int dim, unsigned int value_dim, typename E::real scale,
+                           bool has_softcap, float softcap, typename E::real additive) {
+    typedef typename E::real R;
+    R score = 0;
     if (k_row != nullptr)
-        for (unsigned int d = 0; d < dim; ++d) score = fmaf(q_row[d], E::load(k_row + d), score);
+        for (unsigned int d = 0; d < dim; ++d) score = real_fma(q_row[d], static_cast<R>(E::load(k_row + d)), score);
     score *= scale;
-    if (has_softcap) score = tanhf(score / softcap) * softcap;
+    if (has_softcap) score = real_tanh(score / static_cast<R>(softcap)) * static_cast<R>(softcap);
     score += additive;
     if (score == -INFINITY) return;
-    const float moved = fmaxf(state.largest, score);
-    const float rescale = expf(state.largest - moved);  // exp(-inf) = 0 on the first key
-    const float weight = expf(score - moved);
+    const R moved = real_max(state.largest, score);
+    const R rescale = real_exp(state.largest - moved);  // exp(-inf) = 0 on the first key
+    const R weight = real_exp(score - moved);
     state.total = state.total * rescale + weight;
     state.largest = moved;
 #pragma unroll
     for (int d = 0; d < DMAX; ++d)
         if (static_cast<unsigned int>(d) < value_dim)
-            state.acc[d] = fmaf(weight, v_row != nullptr ? E::load(v_row + d) : 0.0f, state.acc[d] * rescale);
+            state.acc[d] = real_fma(weight, v_row != nullptr ? static_cast<R>(E::load(v_row + d)) : R(0), state.acc[d] * rescale);
 }
 
 // Merges the 64 lanes and writes the row.  `sink` joins the softmax without weighing a value
 // (attention.rs:255-262); pass -inf for none.  Returns max + ln(sum) of the row, -inf when it saw nothing.
 template <class E, int DMAX>
-SINGE_DEVICE float finish_row(const LaneState<DMAX>& state, typename E::type* out, unsigned int value_dim, unsigned int lane,
-                              float sink) {
-    float row_max = state.largest;
+SINGE_DEVICE typename E::real finish_row(const LaneState<DMAX, typename E::real>& state, typename E::type* out, unsigned int value_dim,
+                                         unsigned int lane, typename E::real sink) {
+    typedef typename E::real R;
+    R row_max = state.largest;
 #pragma unroll
-    for (int step = 32; step >= 1; step >>= 1) row_max = fmaxf(row_max, __shfl_xor(row_max, step, 64));
-    row_max = fmaxf(row_max, sink);
-    const float mine = state.largest == -INFINITY ? 0.0f : expf(state.largest - row_max);
-    float row_sum = state.total * mine;
+    for (int step = 32; step >= 1; step >>= 1) row_max = real_max(row_max, __shfl_xor(row_max, step, 64));
+    row_max = real_max(row_max, sink);
+    const R mine = state.largest == -INFINITY ? R(0) : real_exp(state.largest - row_max);
+    R row_sum = state.total * mine;
 #pragma unroll
     for (int step = 32; step >= 1; step >>= 1) row_sum += __shfl_xor(row_sum, step, 64);
-    if (sink != -INFINITY) row_sum += expf(sink - row_max);
-    const float inverse = row_sum > 0.0f ? 1.0f / row_sum : 0.0f;
+    if (sink != -INFINITY) row_sum += real_exp(sink - row_max);
+    const R inverse = row_sum > 0 ? R(1) / row_sum : R(0);
 #pragma unroll
     for (int d = 0; d < DMAX; ++d) {
         if (static_cast<unsigned int>(d) < value_dim) {
-            float value = state.acc[d] * mine;
+            R value = state.acc[d] * mine;
 #pragma unroll
             for (int step = 32; step >= 1; step >>= 1) value += __shfl_xor(value, step, 64);
             // A row that sees no key stays zero (attention.rs:503-515; a key count of zero gives zeros).
             if (lane == (d & 63)) E::store(out + d, value * inverse);
         }
     }
-    return row_sum > 0.0f ? row_max + logf(row_sum) : -INFINITY;
+    return row_sum > 0 ? row_max + real_log(row_sum) : R(-INFINITY);
 }
 
 template <uint32_t ELEMENT, int DMAX>
-SINGE_DEVICE void dense_body(const GeneralAttentionArgs& a, float* lds) {
+SINGE_DEVICE void dense_body(const GeneralAttentionArgs& a, typename Element<ELEMENT>::real* lds) {
     typedef Element<ELEMENT> E;
     typedef typename E::type T;
+    typedef typename E::real R;
     const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const unsigned long long row = static_cast<unsigned long long>(blockIdx.x) * 4 + wave;
     const unsigned long long rows = static_cast<unsigned long long>(a.batch) * a.heads * a.query_len;
@@ -121,7 +154,7 @@ SINGE_DEVICE void dense_body(const GeneralAttentionArgs& a, float* lds) {
                                       : static_cast<const T*>(a.mask) + batch * a.mask_strides[0] + head * a.mask_strides[1] +
                                             query * a.mask_strides[2];
 
-    float* q_row = lds + wave * DMAX;
+    R* q_row = lds + wave * DMAX;
     for (unsigned int d = lane; d < a.head_dim; d += 64) q_row[d] = E::load(q + d);
     __builtin_amdgcn_wave_barrier();
 
@@ -139,23 +172,24 @@ SINGE_DEVICE void dense_body(const GeneralAttentionArgs& a, float* lds) {
         if (static_cast<unsigned long long>(query) + 1 > window) first = static_cast<unsigned int>(query + 1 - window);
     }
 
-    LaneState<DMAX> state;
+    LaneState<DMAX, R> state;
     reset(state);
     for (unsigned int key = first + lane; key < end; key += 64) {
-        const float additive = mask != nullptr ? E::load(mask + key * a.mask_strides[3]) : 0.0f;
+        const R additive = mask != nullptr ? static_cast<R>(E::load(mask + key * a.mask_strides[3])) : R(0);
         fold_key<E, DMAX>(state, q_row, k + static_cast<size_t>(key) * a.key_strides[2], v + static_cast<size_t>(key) * a.value_strides[2],
-                          a.head_dim, a.value_dim, a.scale, a.has_softcap != 0, a.softcap, additive);
+                          a.head_dim, a.value_dim, own_scale<R>(a), a.has_softcap != 0, a.softcap, additive);
     }
-    const float sink = a.sinks != nullptr ? E::load(static_cast<const T*>(a.sinks) + head) : -INFINITY;
+    const R sink = a.sinks != nullptr ? static_cast<R>(E::load(static_cast<const T*>(a.sinks) + head)) : R(-INFINITY);
     T* out = static_cast<T*>(a.out) + batch * a.out_strides[0] + head * a.out_strides[1] + query * a.out_strides[2];
-    const float lse = finish_row<E, DMAX>(state, out, a.value_dim, lane, sink);
-    if (a.lse != nullptr && lane == 0) a.lse[row] = lse;  // row = (batch * heads + head) * query_len + query
+    const R lse = finish_row<E, DMAX>(state, out, a.value_dim, lane, sink);
+    if (a.lse != nullptr && lane == 0) a.lse[row] = static_cast<float>(lse);  // row = (batch * heads + head) * query_len + query
 }
 
 template <uint32_t ELEMENT, int DMAX, int FORM, bool DECODE = false>
-SINGE_DEVICE void paged_rows(const GeneralPagedArgs& a, float* lds) {
+SINGE_DEVICE void paged_rows(const GeneralPagedArgs& a, typename Element<ELEMENT>::real* lds) {
     typedef Element<ELEMENT> E;
     typedef typename E::type T;
+    typedef typename E::real R;
     const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const unsigned int sequence = blockIdx.x / a.row_blocks;
     const unsigned int local_row = (blockIdx.x % a.row_blocks) * 4 + wave;  // (query, head) of the sequence
@@ -183,7 +217,7 @@ SINGE_DEVICE void paged_rows(const GeneralPagedArgs& a, float* lds) {
     const size_t flat = (static_cast<size_t>(span.query_start) + query) * a.heads + head;
     const T* q = static_cast<const T*>(a.query_rows) + flat * a.head_dim;
 
-    float* q_row = lds + wave * DMAX;
+    R* q_row = lds + wave * DMAX;
     for (unsigned int d = lane; d < a.head_dim; d += 64) q_row[d] = E::load(q + d);
     __builtin_amdgcn_wave_barrier();
 
@@ -199,7 +233,7 @@ SINGE_DEVICE void paged_rows(const GeneralPagedArgs& a, float* lds) {
         if (static_cast<unsigned long long>(position) + 1 > window) first = static_cast<unsigned int>(position + 1 - window);
     }
 
-    LaneState<DMAX> state;
+    LaneState<DMAX, R> state;
     reset(state);
     const T* key_cache = static_cast<const T*>(a.key_cache);
     const T* value_cache = static_cast<const T*>(a.value_cache);
@@ -211,17 +245,17 @@ SINGE_DEVICE void paged_rows(const GeneralPagedArgs& a, float* lds) {
         // A key behind a bad page id is read as zeros; the status word tells the caller.
         const size_t offset = ((page * a.page_size + key % a.page_size) * a.kv_heads + kv_head) * a.head_dim;
         fold_key<E, DMAX>(state, q_row, valid ? key_cache + offset : nullptr, valid ? value_cache + offset : nullptr, a.head_dim,
-                          a.head_dim, a.scale, a.has_softcap != 0, a.softcap, 0.0f);
+                          a.head_dim, own_scale<R>(a), a.has_softcap != 0, a.softcap, R(0));
     }
-    const float lse = finish_row<E, DMAX>(state, static_cast<T*>(a.output) + flat * a.head_dim, a.head_dim, lane, -INFINITY);
+    const R lse = finish_row<E, DMAX>(state, static_cast<T*>(a.output) + flat * a.head_dim, a.head_dim, lane, R(-INFINITY));
     if (a.lse != nullptr && lane == 0) {
-        if (FORM == kTable) a.lse[flat] = lse == -INFINITY ? -1.0e20f : lse;  // natural log (cpu/attention.rs:1304-1317)
-        else a.lse[flat] = lse * kLog2e;                                      // base two; -inf stays -inf
+        if (FORM == kTable) a.lse[flat] = lse == -INFINITY ? -1.0e20f : static_cast<float>(lse);  // natural log (cpu/attention.rs:1304-1317)
+        else a.lse[flat] = static_cast<float>(lse * static_cast<R>(1.4426950408889634074));       // base two; -inf stays -inf
     }
 }
 
 template <uint32_t ELEMENT, int DMAX>
-SINGE_DEVICE void paged_body(const GeneralPagedArgs& a, float* lds) {
+SINGE_DEVICE void paged_body(const GeneralPagedArgs& a, typename Element<ELEMENT>::real* lds) {
     if (a.form == 1)
         paged_rows<ELEMENT, DMAX, kCsrI64>(a, lds);
     else if (a.form == 2)
@@ -236,18 +270,18 @@ SINGE_DEVICE void paged_body(const GeneralPagedArgs& a, float* lds) {
 
 #define SINGE_GENERAL_KERNELS(TAG, ELEMENT, DMAX)                                                                            \
     extern "C" __global__ __launch_bounds__(256) void singe_attention_general_##TAG##_d##DMAX(GeneralAttentionArgs args) {   \
-        __shared__ float rows[4 * DMAX];                                                                                     \
+        __shared__ general::Element<ELEMENT>::real rows[4 * DMAX];                                                           \
         general::dense_body<ELEMENT, DMAX>(args, rows);                                                                      \
     }                                                                                                                        \
     extern "C" __global__ __launch_bounds__(256) void singe_paged_attention_general_##TAG##_d##DMAX(GeneralPagedArgs args) { \
-        __shared__ float rows[4 * DMAX];                                                                                     \
+        __shared__ general::Element<ELEMENT>::real rows[4 * DMAX];                                                           \
         general::paged_body<ELEMENT, DMAX>(args, rows);                                                                      \
     }
 
 // The build compiles this file once per element type (SINGE_GENERAL_ELEMENT = 0 f32, 1 bf16, 2 f16), each into its
 // own part of the code object.
 #ifndef SINGE_GENERAL_ELEMENT
-#error "define SINGE_GENERAL_ELEMENT: 0 (f32), 1 (bf16) or 2 (f16)"
+#error "define SINGE_GENERAL_ELEMENT: 0 (f32), 1 (bf16), 2 (f16) or 3 (f64)"
 #endif
 #if SINGE_GENERAL_ELEMENT == 0
 SINGE_GENERAL_KERNELS(f32, kElementF32, 64)
@@ -257,8 +291,12 @@ SINGE_GENERAL_KERNELS(f32, kElementF32, 256)
 SINGE_GENERAL_KERNELS(bf16, kElementBf16, 64)
 SINGE_GENERAL_KERNELS(bf16, kElementBf16, 128)
 SINGE_GENERAL_KERNELS(bf16, kElementBf16, 256)
-#else
+#elif SINGE_GENERAL_ELEMENT == 2
 SINGE_GENERAL_KERNELS(f16, kElementF16, 64)
 SINGE_GENERAL_KERNELS(f16, kElementF16, 128)
 SINGE_GENERAL_KERNELS(f16, kElementF16, 256)
+#else
+SINGE_GENERAL_KERNELS(f64, kElementF64, 64)
+SINGE_GENERAL_KERNELS(f64, kElementF64, 128)
+SINGE_GENERAL_KERNELS(f64, kElementF64, 256)
 #endif

@@ -80,6 +80,13 @@ struct PrefillArgs {
     uint32_t mask_packed = 0;  // key stride 1, the other strides multiples of 4, the mask on an 8-byte boundary
     long long window = -1;
     float cap_scale = 0.0f, cap_log2e = 0.0f;
+    // Key splits (splits > 1): the key tiles of a query tile are shared out over `splits` workgroups, each leaving its
+    // rows normalised in partial_out [splits, batch * heads * query_len, head_dim] with a base-two log-sum-exp in
+    // partial_lse [splits, batch * heads * query_len] (-inf and zeros for a share that saw nothing); a sink joins the
+    // first share; singe_fmha_prefill_combine_* merges them into out and lse.
+    uint32_t splits = 1;
+    float* partial_out = nullptr;
+    float* partial_lse = nullptr;
 };
 
 struct PrefillF32Args {
@@ -200,7 +207,7 @@ struct PagedRowsF32Args {
 };
 
 // Element types of the general (any head dimension) kernels.
-enum SingeElement : uint32_t { kElementF32 = 0, kElementBf16 = 1, kElementF16 = 2 };
+enum SingeElement : uint32_t { kElementF32 = 0, kElementBf16 = 1, kElementF16 = 2, kElementF64 = 3 };
 
 // singe_attention_general_*: dense attention over [batch, heads, len, dim] tensors with every option
 // of ScaledDotProductAttentionAttributes.
@@ -220,6 +227,7 @@ struct GeneralAttentionArgs {
     uint32_t batch, heads, kv_heads, query_len, key_len, head_dim, value_dim;
     uint32_t causal, has_softcap;
     float scale, softcap;
+    double scale_wide;              // the scale for f64 tensors: the default 1 / sqrt(head_dim) is taken in f64 there
 };
 
 // singe_paged_attention_general_*: the paged ops for any element type and head dimension.  `form`: the FlashInfer
@@ -245,6 +253,7 @@ struct GeneralPagedArgs {
     uint32_t row_blocks;            // workgroups (4 rows each) per sequence
     uint32_t causal, has_softcap, form;
     float scale, softcap;
+    double scale_wide;              // the scale for f64 tensors: the default 1 / sqrt(head_dim) is taken in f64 there
 };
 
 // singe_paged_mla_attention_general_*: contiguous operands of one element type.

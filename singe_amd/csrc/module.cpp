@@ -90,6 +90,10 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_attention_f16_d64_softcap_i32_p16", "singe_paged_attention_f16_d64_softcap_i64_p16",
     "singe_rotary_paged_attention_bf16_d64_i32", "singe_rotary_paged_attention_bf16_d64_i64",
     "singe_rotary_paged_attention_bf16_d64_i32_p16", "singe_rotary_paged_attention_bf16_d64_i64_p16",
+    "singe_fmha_prefill_bf16_d128_combine", "singe_fmha_prefill_f16_d128_combine",
+    "singe_fmha_prefill_bf16_d64_combine", "singe_fmha_prefill_f16_d64_combine",
+    "singe_attention_general_f64_d64", "singe_attention_general_f64_d128", "singe_attention_general_f64_d256",
+    "singe_paged_attention_general_f64_d64", "singe_paged_attention_general_f64_d128", "singe_paged_attention_general_f64_d256",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -99,6 +103,7 @@ const char* const kPartNames[kPartCount] = {
     "paged_decode", "fmha_prefill", "fmha_prefill_f32", "paged_attention", "splitk_reduce", "attention_rows_f32",
     "cache_ops", "latent_attention", "latent_attention_mfma", "general_attention_f32", "general_attention_bf16",
     "general_attention_f16", "mfma_ceiling", "paged_decode_d64", "fmha_prefill_d64", "paged_attention_d64",
+    "general_attention_f64",
 };
 
 namespace {
@@ -112,6 +117,8 @@ constexpr PartRun kPartRuns[] = {
     {9, 3}, {10, 3}, {11, 3},  // paged general kernels
     {12, 2},
     {13, 10}, {14, 8}, {15, 28},  // the head_dim 64 builds
+    {1, 2}, {14, 2},              // the dense kernels' merges
+    {16, 6},                      // the general kernels on f64
 };
 constexpr int runs_total() {
     int total = 0;
@@ -267,6 +274,7 @@ const char* singe_hip_status_string(int32_t status) {
         case SINGE_HIP_AUTOTUNE_DURING_CAPTURE: return "autotune during stream capture";
         case SINGE_HIP_NO_TUNE_CANDIDATES: return "no tune candidates";
         case SINGE_HIP_NO_SUCCESSFUL_TUNE_CANDIDATES: return "no tune candidate completed";
+        case SINGE_HIP_STALE_RECORD: return "stale record";
         default: break;
     }
     if (status < 0) {

@@ -51,7 +51,11 @@ enum KernelId : int {
     // bf16 / f16 decode kernels from kDecodeBf16, the eight dense prefill kernels from kPrefillCausal, the paged
     // attention kernels from kPagedAttentionI32 up to kSplitKReduce
     kDecodeD64, kPrefillD64 = kDecodeD64 + 10, kPagedD64 = kPrefillD64 + 8,
-    kKernelCount = kPagedD64 + (kSplitKReduce - kPagedAttentionI32)
+    // the merge of the dense kernels' key splits: bf16, f16, then the same for head_dim 64
+    kPrefillCombine = kPagedD64 + (kSplitKReduce - kPagedAttentionI32), kPrefillCombineF16, kPrefillCombineD64, kPrefillCombineF16D64,
+    // the general kernels on f64 tensors: + width (64, 128, 256)
+    kDenseGeneralF64, kPagedGeneralF64 = kDenseGeneralF64 + 3,
+    kKernelCount = kPagedGeneralF64 + 3
 };
 
 // The head_dim 64 build of a matrix-core kernel named by its head_dim 128 id.
@@ -64,7 +68,7 @@ inline KernelId at_head_dim_64(KernelId kernel) {
 extern const char* const kKernelNames[kKernelCount];
 
 // Parts of the code object (one file each) and the part a kernel lives in.
-constexpr int kPartCount = 16;
+constexpr int kPartCount = 17;
 extern const char* const kPartNames[kPartCount];
 int kernel_part(int kernel);
 

@@ -45,10 +45,9 @@ uint32_t paged_attention_splits(const SingePagedAttentionProblem& p) {
     const uint64_t groups = static_cast<uint64_t>(p.heads / p.kv_heads);
     const uint64_t row_tiles = (groups * static_cast<uint64_t>(p.tokens) + 127) / 128;
     const uint64_t workgroups = static_cast<uint64_t>(p.sequences) * p.kv_heads * row_tiles;
-    const uint64_t wanted = 4ull * compute_units();
-    if (workgroups >= wanted) return 1;
-    const uint64_t splits = wanted / workgroups;
-    return static_cast<uint32_t>(splits > 16 ? 16 : splits < 1 ? 1 : splits);
+    // A sequence's key count lives in device memory: the most its pages can hold bounds it.
+    const uint64_t keys = static_cast<uint64_t>(p.page_table > 0 ? p.page_table : 0) * static_cast<uint64_t>(p.page_size);
+    return attention_key_splits(workgroups, keys);
 }
 
 size_t scratch_bytes_for(const SingePagedAttentionProblem& p, uint32_t splits) {
@@ -235,6 +234,14 @@ extern "C" int32_t singe_hip_paged_attention_f32(void* stream, const float* quer
                                                  const void* pages, const void* last_page_lengths, float* output, float* lse,
                                                  uint32_t* status, const SingePagedAttentionProblem* problem) {
     return paged_attention(SINGE_HIP_F32, stream, query_rows, key_cache, value_cache, query_offsets, page_offsets, pages,
+                           last_page_lengths, output, lse, status, problem);
+}
+
+extern "C" int32_t singe_hip_paged_attention_f64(void* stream, const double* query_rows, const double* key_cache,
+                                                 const double* value_cache, const void* query_offsets, const void* page_offsets,
+                                                 const void* pages, const void* last_page_lengths, double* output, float* lse,
+                                                 uint32_t* status, const SingePagedAttentionProblem* problem) {
+    return paged_attention(SINGE_HIP_F64, stream, query_rows, key_cache, value_cache, query_offsets, page_offsets, pages,
                            last_page_lengths, output, lse, status, problem);
 }
 

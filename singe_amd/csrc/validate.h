@@ -24,6 +24,9 @@ inline int32_t ensure_len_at_least(const char* name, size_t actual, size_t minim
 // fmha_prefill.cpp: the bf16 / f16 matrix-core prefill with the options of the dense op.  sinks [heads] and mask are
 // in the element type of the query; any pointer may be null, window negative and softcap 0 when absent.
 struct DenseOptions {
+    // Scratch for key splits (null: none), see singe_hip_scaled_dot_product_attention_scratch.
+    void* scratch = nullptr;
+    size_t scratch_bytes = 0;
     const uint16_t* sinks = nullptr;
     const int32_t* key_lengths = nullptr;
     const uint16_t* mask = nullptr;
@@ -34,6 +37,15 @@ struct DenseOptions {
 int32_t dense_prefill_with_options(void* stream, bool f16, uint16_t* out, size_t out_len, const uint16_t* query, size_t query_len,
                                    const uint16_t* key, size_t key_len, const uint16_t* value, size_t value_len,
                                    const SingeFmhaPrefillConfig* config, const DenseOptions& options);
+
+// fmha_prefill.cpp: the shares the matrix-core dense kernel would split this problem's keys into (1 = none) and the
+// scratch they need.
+uint32_t dense_prefill_splits(const SingeFmhaPrefillConfig& config);
+size_t dense_prefill_scratch_bytes(const SingeFmhaPrefillConfig& config, uint32_t splits);
+
+// attention_parameters.cpp: the shares a launch of `workgroups` workgroups over at most `keys` keys splits its keys
+// into under the installed AttentionParameters (1 = no split).
+uint32_t attention_key_splits(uint64_t workgroups, uint64_t keys);
 
 // general_attention.cpp: the one-wave-per-row kernels behind entry points of other files, for head dimensions the
 // matrix-core kernels are not built for.  Block-table prefill (query_lengths given) or decode (query_lengths null).
@@ -58,6 +70,7 @@ struct DenseGeneralOperands {
     uint64_t batch = 0, heads = 0, kv_heads = 0, query_len = 0, key_len = 0, head_dim = 0, value_dim = 0;
     bool causal = false, has_softcap = false;
     float scale = 1.0f, softcap = 0.0f;
+    double scale_wide = 1.0;  // for f64 tensors
 };
 int32_t dense_general(int32_t data_type, void* stream, const char* op, const DenseGeneralOperands& operands);
 

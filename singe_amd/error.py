@@ -71,6 +71,10 @@ class NoTuneCandidates(Error):
     """No candidate is left to time, or none completed (Error::NoTuneCandidates / NoSuccessfulTuneCandidates)."""
 
 
+class StaleRecord(Error):
+    """singe::Error::StaleRecord: parameters a kernel does not take (any more)."""
+
+
 class Hip(Error):
     """A HIP runtime call failed (the counterpart of Error::Cuda)."""
 

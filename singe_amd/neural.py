@@ -82,6 +82,8 @@ def _problem(query, key_cache, value_cache, paging: Paging, options: AttentionOp
 
 _DATA_TYPES = {torch.float32: _native.DATA_TYPE_F32, torch.bfloat16: _native.DATA_TYPE_BF16,
                torch.float16: _native.DATA_TYPE_F16}
+# The dense op and the paged op also take f64 (on the vector-unit kernels, in f64 arithmetic).
+_ATTENTION_TYPES = {**_DATA_TYPES, torch.float64: _native.DATA_TYPE_F64}
 
 
 def scaled_dot_product_attention(query, key, value, scale: float | None = None, causal: bool = False, *, stream=None):
@@ -115,7 +117,7 @@ def _attend_all_ordered(query, key, value, mask, sinks, key_lengths, options, *,
             raise error.InvalidArgument(f"scaled dot-product attention {name} rank")
         if not tensor.is_cuda or tensor.dtype != query.dtype or not tensor.is_contiguous():
             raise error.InvalidArgument(f"scaled dot-product attention {name} must be a contiguous device tensor of the query's type")
-    if query.dtype not in _DATA_TYPES:
+    if query.dtype not in _ATTENTION_TYPES:
         raise error.InvalidArgument(f"scaled dot-product attention data type {query.dtype}")
     batch, heads, query_len, head_dim = query.shape
     key_batch, kv_heads, key_len, key_dim = key.shape
@@ -152,18 +154,85 @@ def _attend_all_ordered(query, key, value, mask, sinks, key_lengths, options, *,
         key_lengths = key_lengths.contiguous()
     problem = _native.AttentionProblemC(
         batch, heads, kv_heads, query_len, key_len, head_dim, value_dim, (ctypes.c_int64 * 4)(*strides),
-        _DATA_TYPES[query.dtype], 1 if options.causal else 0, 1 if options.scale is not None else 0,
+        _ATTENTION_TYPES[query.dtype], 1 if options.causal else 0, 1 if options.scale is not None else 0,
         1 if options.window is not None else 0, 1 if options.softcap is not None else 0,
         options.scale if options.scale is not None else 0.0, options.softcap if options.softcap is not None else 0.0,
         options.window if options.window is not None else 0)
     output = torch.empty((batch, heads, query_len, value_dim), device=query.device, dtype=query.dtype)
     handle = int((stream or torch.cuda.current_stream()).cuda_stream)
     pointer = lambda tensor: tensor.data_ptr() if tensor is not None else None
-    code = _native.lib().singe_hip_scaled_dot_product_attention(
-        handle, query.data_ptr(), key.data_ptr(), value.data_ptr(), pointer(mask), pointer(sinks), pointer(key_lengths),
-        output.data_ptr(), ctypes.byref(problem))
+    # A decode-shaped call (few query rows, many keys) shares its keys out over several workgroups, on this module's
+    # per-device scratch (calls on different streams must then not overlap), as the reference's plan splits them
+    # (kernel_plan/source/attention.rs:283-292).
+    wanted = int(_native.lib().singe_hip_scaled_dot_product_attention_scratch_bytes(ctypes.byref(problem)))
+    if wanted > 0:
+        lent = _scratch_for(query.device, wanted)
+        code = _native.lib().singe_hip_scaled_dot_product_attention_scratch(
+            handle, query.data_ptr(), key.data_ptr(), value.data_ptr(), pointer(mask), pointer(sinks), pointer(key_lengths),
+            output.data_ptr(), lent.data_ptr(), lent.numel(), ctypes.byref(problem))
+    else:
+        code = _native.lib().singe_hip_scaled_dot_product_attention(
+            handle, query.data_ptr(), key.data_ptr(), value.data_ptr(), pointer(mask), pointer(sinks), pointer(key_lengths),
+            output.data_ptr(), ctypes.byref(problem))
     _native.check(code, "scaled_dot_product_attention")
     return output
+
+
+@dataclass(frozen=True)
+class AttentionParameters:
+    """The choices the attention kernels leave open (singe/src/backend/cuda/kernel_plan/source/parameters.rs:21-57).
+    On gfx950 `warps` is 4 and `key_tile` 64, `stages` 1 or 2 name the one pipeline the kernels have, `min_blocks` is
+    None or 2, and `split_below_blocks` is the number of workgroups below which a launch splits its keys (0 never)."""
+    warps: int = 4
+    key_tile: int = 64
+    stages: int = 1
+    split_below_blocks: int = 64
+    min_blocks: int | None = None
+
+    def _c(self) -> _native.AttentionParametersC:
+        return _native.AttentionParametersC(self.warps, self.key_tile, self.stages, self.split_below_blocks,
+                                            0 if self.min_blocks is None else 1, self.min_blocks or 0)
+
+    @classmethod
+    def _of(cls, raw: _native.AttentionParametersC) -> "AttentionParameters":
+        return cls(raw.warps, raw.key_tile, raw.stages, raw.split_below_blocks, raw.min_blocks if raw.has_min_blocks else None)
+
+
+def default_attention_parameters() -> AttentionParameters:
+    """AttentionParameters::default() of this device: split_below_blocks is twice its compute units."""
+    raw = _native.AttentionParametersC()
+    _native.lib().singe_hip_attention_parameters_default(ctypes.byref(raw))
+    return AttentionParameters._of(raw)
+
+
+def attention_candidates() -> list:
+    """attention_candidates (kernel_plan/source/attention.rs:113-160): what the kernels take, the default first."""
+    raw = (_native.AttentionParametersC * 16)()
+    count = ctypes.c_size_t(0)
+    _native.check(_native.lib().singe_hip_attention_candidates(raw, 16, ctypes.byref(count)), "attention_candidates")
+    return [AttentionParameters._of(raw[i]) for i in range(min(count.value, 16))]
+
+
+def set_attention_parameters(parameters: AttentionParameters | None) -> None:
+    """Installs the parameters a tuning record gives the paged and the dense op (None: the default); parameters the
+    kernels do not take raise StaleRecord, as the reference refuses them (parameters.rs:245-250)."""
+    code = _native.lib().singe_hip_set_attention_parameters(None if parameters is None else ctypes.byref(parameters._c()))
+    _native.check(code, "attention parameters")
+
+
+def attention_parameters() -> AttentionParameters:
+    raw = _native.AttentionParametersC()
+    _native.lib().singe_hip_attention_parameters(ctypes.byref(raw))
+    return AttentionParameters._of(raw)
+
+
+def paged_attention_parameter_key(query, key_cache, value_cache, paging: Paging, options: AttentionOptions = AttentionOptions()) -> str:
+    """parameter_key("paged_attention", ...) (parameters.rs:221-230) of contiguous operands."""
+    problem = _problem(query, key_cache, value_cache, paging, options)
+    need = int(_native.lib().singe_hip_paged_attention_parameter_key(ctypes.byref(problem), _ATTENTION_TYPES[query.dtype], None, 0))
+    buffer = ctypes.create_string_buffer(need + 1)
+    _native.lib().singe_hip_paged_attention_parameter_key(ctypes.byref(problem), _ATTENTION_TYPES[query.dtype], buffer, need + 1)
+    return buffer.value.decode()
 
 
 _scratch: dict = {}
@@ -193,7 +262,7 @@ def paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: t
     for tensor, name in ((query, "query"), (key_cache, "key_cache"), (value_cache, "value_cache")):
         if not tensor.is_cuda or tensor.dtype != query.dtype or not tensor.is_contiguous():
             raise error.InvalidArgument(f"paged attention {name} must be a contiguous device tensor of the query's type")
-    if query.dtype not in _DATA_TYPES:
+    if query.dtype not in _ATTENTION_TYPES:
         raise error.InvalidArgument(f"paged attention data type {query.dtype}")
     for tensor in (paging.query_offsets, paging.page_offsets, paging.pages, paging.last_page_lengths):
         if not tensor.is_cuda or not tensor.is_contiguous():
@@ -206,6 +275,7 @@ def paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_cache: t
     handle = int((stream or torch.cuda.current_stream()).cuda_stream)
     entry = {torch.bfloat16: _native.lib().singe_hip_paged_attention_bf16,
              torch.float32: _native.lib().singe_hip_paged_attention_f32,
+             torch.float64: _native.lib().singe_hip_paged_attention_f64,
              torch.float16: _native.lib().singe_hip_paged_attention_f16}[query.dtype]
     # bf16 calls with few query rows (decoding) share a row tile's keys out over several workgroups, given
     # scratch: ``scratch`` is a uint8 device tensor, True for this module's own per-device buffer (calls on
