@@ -11,8 +11,9 @@ Prints one JSON line: whole-job GB/s of algorithmic bytes over exactly --steps s
 steps, the roofline of the dominant kernel and the CPU oracle timed on a bounded sample.  The same line
 carries one object per further benchmark configuration ("prefill", "chunked_prefill", "fp8_decode",
 "dense_f32"), "latent" (MLA attention over paged caches), "head_dim_64" (the matrix-core kernels at the
-reference's other head dimension) and "mfma_ceiling" (what the matrix cores sustain on a register-only loop
-of the prefill kernels' product, on zeros and on the benchmark's kind of data).
+reference's other head dimension), "mfma_ceiling" (what the matrix cores sustain on a register-only loop
+of the prefill kernels' product, on zeros and on the benchmark's kind of data) and "hbm_ceiling" (what a kernel that
+only reads gets out of HBM at the decode workloads' sizes).
 
 How every kernel figure is taken, whatever --steps says: at least 300 ms of warm-up launches, then at
 least 30 samples, each a pair of HIP events on the launch stream around a small group of back-to-back
@@ -64,7 +65,8 @@ def traffic(key):
     return entry["FETCH_SIZE"] * FETCH_UNIT_BYTES + entry["WRITE_SIZE"] * WRITE_UNIT_BYTES, entry["source"]
 
 
-SECTIONS = ("decode", "prefill", "chunked_prefill", "fp8_decode", "dense_f32", "latent", "head_dim_64", "mfma_ceiling")
+SECTIONS = ("decode", "prefill", "chunked_prefill", "fp8_decode", "dense_f32", "latent", "head_dim_64", "mfma_ceiling",
+            "hbm_ceiling")
 
 
 def parse():
@@ -570,6 +572,35 @@ def mfma_ceiling_section():
     return result
 
 
+def hbm_ceiling_section():
+    """What the memory system delivers to a kernel that only reads: one workgroup of 512 lanes per compute unit (the
+    decode kernels' launch shape) streams buffers of the two decode workloads' sizes, 297 MB and 4.3 GB, once per
+    launch with non-temporal loads; three buffers are rotated as the decode section rotates its KV pools."""
+    import torch
+
+    from singe_amd import _native
+
+    workgroups = torch.cuda.get_device_properties(0).multi_processor_count
+    out = torch.empty(workgroups * 512, device="cuda", dtype=torch.int32)
+    handle = int(torch.cuda.current_stream().cuda_stream)
+    result = {"kernel": "singe_hbm_stream_read", "workgroups": workgroups, "peak": HBM_PEAK_GBPS, "unit": "GB/s"}
+    for name, nbytes, pools, group in (("decode_sized", 296_748_908 // 16 * 16, 3, 6), ("fp8_decode_sized", 4_305_977_600, 2, 2)):
+        buffers = [torch.randint(0, 255, (nbytes,), device="cuda", dtype=torch.uint8) for _ in range(pools)]
+        turn = [0]
+
+        def launch():
+            data = buffers[turn[0] % pools]
+            turn[0] += 1
+            _native.check(_native.lib().singe_hip_hbm_stream_read(handle, data.data_ptr(), nbytes, out.data_ptr(), out.numel(),
+                                                                  workgroups), "hbm_stream_read")
+        stats = measure(launch, group)
+        gbps = nbytes / (stats["mean_ms"] * 1e-3) / 1e9
+        result[name] = {"bytes": nbytes, "value": gbps, "frac_of_peak": gbps / HBM_PEAK_GBPS, **timing_fields(stats)}
+        del buffers
+        torch.cuda.empty_cache()
+    return result
+
+
 def decode_section(args, with_cpu):
     """The headline: --warmup untimed steps, exactly --steps timed steps between two synchronisations, then the split
     kernel alone under HIP events."""
@@ -659,6 +690,7 @@ def main():
         "prefill": lambda: prefill_section(with_cpu), "chunked_prefill": lambda: chunked_prefill_section(with_cpu),
         "fp8_decode": lambda: fp8_decode_section(with_cpu), "dense_f32": lambda: dense_f32_section(with_cpu),
         "latent": latent_section, "head_dim_64": head_dim_64_section, "mfma_ceiling": mfma_ceiling_section,
+        "hbm_ceiling": hbm_ceiling_section,
     }
     if FEW:
         # A copy of known size beside the kernel, for the unit of the profiler's byte counters: torch's f32 -> bf16
@@ -684,6 +716,9 @@ def main():
     ceiling = result["mfma_ceiling"]["normal"]["value"]
     for name in ("prefill", "chunked_prefill"):
         result[name]["roofline"]["frac_of_measured_ceiling"] = result[name]["roofline"]["achieved"] / ceiling
+    result["roofline"]["frac_of_measured_ceiling"] = result["roofline"]["achieved"] / result["hbm_ceiling"]["decode_sized"]["value"]
+    result["fp8_decode"]["roofline"]["frac_of_measured_ceiling"] = (result["fp8_decode"]["roofline"]["achieved"]
+                                                                    / result["hbm_ceiling"]["fp8_decode_sized"]["value"])
     print(json.dumps(result), flush=True)
 
 

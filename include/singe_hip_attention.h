@@ -989,6 +989,11 @@ SINGE_HIP_API int32_t singe_hip_paging_indices(
  * inside the loop: the rate it reaches is the matrix cores' own ceiling on that data (the clock under such a loop is
  * set by power, and power by the operands' bits), which the prefill kernels are priced against beside the published
  * peak.  Flop per launch = workgroups * 4 * iterations * 32 * 32768.  `out` takes one float per lane. */
+/* The same kind of aid for the memory-bound kernels: `workgroups` workgroups of 512 lanes stream `bytes` of `data`
+ * once with 16-byte non-temporal loads, eight in flight per lane, and do nothing else; bytes / time is the streaming
+ * read rate the decode kernels are priced against beside the published HBM peak.  `out` takes one word per lane. */
+SINGE_HIP_API int32_t singe_hip_hbm_stream_read(void* stream, const void* data, size_t bytes, uint32_t* out, size_t out_len,
+                                                uint32_t workgroups);
 SINGE_HIP_API int32_t singe_hip_mfma_ceiling(void* stream, const void* operands, size_t operand_bytes, float* out,
                                              size_t out_len, uint32_t workgroups, uint32_t iterations, int32_t f16);
 

@@ -12,7 +12,7 @@ LIBRARY_PATH = os.path.join(_HERE, "libsinge_hip_attention.so")
 CODE_OBJECT_PARTS = ("paged_decode", "fmha_prefill", "fmha_prefill_f32", "paged_attention", "splitk_reduce",
                      "attention_rows_f32", "cache_ops", "latent_attention", "latent_attention_mfma",
                      "general_attention_f32", "general_attention_bf16", "general_attention_f16", "mfma_ceiling",
-                     "paged_decode_d64", "fmha_prefill_d64", "paged_attention_d64", "general_attention_f64")
+                     "paged_decode_d64", "fmha_prefill_d64", "paged_attention_d64", "general_attention_f64", "hbm_stream")
 CODE_OBJECT_PATHS = [os.path.join(_HERE, f"singe_attention_gfx950.{part}.hsaco") for part in CODE_OBJECT_PARTS]
 
 c_size = ctypes.c_size_t
@@ -174,6 +174,8 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_scaled_dot_product_attention_scratch_bytes.restype = c_size
     handle.singe_hip_scaled_dot_product_attention_scratch.argtypes = [c_void] * 8 + [c_void, c_size, ctypes.POINTER(AttentionProblemC)]
     handle.singe_hip_scaled_dot_product_attention_scratch.restype = i32
+    handle.singe_hip_hbm_stream_read.argtypes = [c_void, c_void, c_size, c_void, c_size, ctypes.c_uint32]
+    handle.singe_hip_hbm_stream_read.restype = i32
     handle.singe_hip_mfma_ceiling.argtypes = [c_void, c_void, c_size, c_void, c_size, ctypes.c_uint32, ctypes.c_uint32, i32]
     handle.singe_hip_mfma_ceiling.restype = i32
     handle.singe_hip_prepare.argtypes = [ctypes.POINTER(i32)]

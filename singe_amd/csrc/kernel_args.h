@@ -161,6 +161,13 @@ struct MfmaCeilingArgs {
     uint32_t iterations;
 };
 
+// singe_hbm_stream_read: the plain streaming read.
+struct HbmStreamArgs {
+    const void* data;       // chunks 16-byte chunks
+    unsigned int* out;      // one word per lane of the launch
+    uint64_t chunks;
+};
+
 // singe_splitk_reduce_f32: strides in elements.
 struct SplitKReduceArgs {
     float* out;         // [batch, heads, dim]

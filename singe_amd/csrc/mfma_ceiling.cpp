@@ -6,6 +6,21 @@
 
 using namespace singe_hip;
 
+extern "C" int32_t singe_hip_hbm_stream_read(void* stream, const void* data, size_t bytes, uint32_t* out, size_t out_len,
+                                             uint32_t workgroups) {
+    if (data == nullptr) return fail(SINGE_HIP_NULL_POINTER, "data");
+    if (out == nullptr) return fail(SINGE_HIP_NULL_POINTER, "out");
+    if (workgroups == 0) return fail(SINGE_HIP_INVALID_LENGTH, "workgroups");
+    if (bytes < 16) return fail(SINGE_HIP_LENGTH_TOO_SHORT, "data", 16, bytes);
+    const size_t lanes = static_cast<size_t>(workgroups) * 512;
+    if (out_len < lanes) return fail(SINGE_HIP_LENGTH_TOO_SHORT, "out", lanes, out_len);
+    HbmStreamArgs args;
+    args.data = data;
+    args.out = out;
+    args.chunks = bytes / 16;
+    return launch(kHbmStreamRead, workgroups, 1, 1, 512, stream, args);
+}
+
 extern "C" int32_t singe_hip_mfma_ceiling(void* stream, const void* operands, size_t operand_bytes, float* out, size_t out_len,
                                           uint32_t workgroups, uint32_t iterations, int32_t f16) {
     if (operands == nullptr) return fail(SINGE_HIP_NULL_POINTER, "operands");

@@ -94,6 +94,7 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_fmha_prefill_bf16_d64_combine", "singe_fmha_prefill_f16_d64_combine",
     "singe_attention_general_f64_d64", "singe_attention_general_f64_d128", "singe_attention_general_f64_d256",
     "singe_paged_attention_general_f64_d64", "singe_paged_attention_general_f64_d128", "singe_paged_attention_general_f64_d256",
+    "singe_hbm_stream_read",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -103,7 +104,7 @@ const char* const kPartNames[kPartCount] = {
     "paged_decode", "fmha_prefill", "fmha_prefill_f32", "paged_attention", "splitk_reduce", "attention_rows_f32",
     "cache_ops", "latent_attention", "latent_attention_mfma", "general_attention_f32", "general_attention_bf16",
     "general_attention_f16", "mfma_ceiling", "paged_decode_d64", "fmha_prefill_d64", "paged_attention_d64",
-    "general_attention_f64",
+    "general_attention_f64", "hbm_stream",
 };
 
 namespace {
@@ -119,6 +120,7 @@ constexpr PartRun kPartRuns[] = {
     {13, 10}, {14, 8}, {15, 28},  // the head_dim 64 builds
     {1, 2}, {14, 2},              // the dense kernels' merges
     {16, 6},                      // the general kernels on f64
+    {17, 1},
 };
 constexpr int runs_total() {
     int total = 0;

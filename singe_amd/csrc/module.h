@@ -55,7 +55,9 @@ enum KernelId : int {
     kPrefillCombine = kPagedD64 + (kSplitKReduce - kPagedAttentionI32), kPrefillCombineF16, kPrefillCombineD64, kPrefillCombineF16D64,
     // the general kernels on f64 tensors: + width (64, 128, 256)
     kDenseGeneralF64, kPagedGeneralF64 = kDenseGeneralF64 + 3,
-    kKernelCount = kPagedGeneralF64 + 3
+    // the plain streaming read a decode kernel is priced against
+    kHbmStreamRead = kPagedGeneralF64 + 3,
+    kKernelCount
 };
 
 // The head_dim 64 build of a matrix-core kernel named by its head_dim 128 id.
@@ -68,7 +70,7 @@ inline KernelId at_head_dim_64(KernelId kernel) {
 extern const char* const kKernelNames[kKernelCount];
 
 // Parts of the code object (one file each) and the part a kernel lives in.
-constexpr int kPartCount = 17;
+constexpr int kPartCount = 18;
 extern const char* const kPartNames[kPartCount];
 int kernel_part(int kernel);
 

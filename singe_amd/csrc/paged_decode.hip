@@ -55,10 +55,12 @@ static_assert(kDim == 64 || kDim == 128, "head dimensions the decode kernels are
 constexpr int kDimSteps = kDim / 32;  // score products per 16 keys
 constexpr int kTile = 32;
 
-// One 32-key tile in registers, bf16 cache.
+// One 32-key tile in registers, bf16 cache.  K and V are fetched the same way, as whole rows (16 lanes x 16 bytes, the
+// coalesced layout: fetched in the matrix operand's layout, where neighbouring lanes read different rows, K alone
+// held the kernel to 5.6 TB/s); K is turned into its operand layout through a per-wave LDS buffer when the tile is folded.
 struct KeyTileBf16 {
-    uint4 k[2][4];      // [16-key half][c]: lane (g, t) holds key t, dims 32c + 8g .. +8
-    uint4 v[2][4];      // [16-key half][i]: lane (g, t) holds key 4g + i, dims 8t .. 8t + 8
+    uint4 k[2][4];      // [16-key half][i]: lane (g, t) holds key 4g + i, dims 8t .. 8t + 8
+    uint4 v[2][4];      // the same of the values
     unsigned int live;  // bit (half * 4 + i): key half*16 + 4g + i takes part in the softmax
 };
 
@@ -193,15 +195,15 @@ SINGE_DEVICE void load_tile(KeyTileBf16& tile, const DecodeArgs& a, const unsign
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
         const HalfRows rows = locate_half<ALIGNED16>(a, table_row, cache, first + half * 16, end, kv_head, g, t);
-        const uint16_t* kp = key_cache + rows.key_row + 8 * g;
-#pragma unroll
-        for (int c = 0; c < kDimSteps; ++c) tile.k[half][c] = *reinterpret_cast<const uint4*>(kp + 32 * c);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            if (kDim == 128 || 8 * t < static_cast<unsigned int>(kDim))
+            if (kDim == 128 || 8 * t < static_cast<unsigned int>(kDim)) {
+                tile.k[half][i] = stream_load_16(key_cache + rows.value_row[i] + 8 * t);
                 tile.v[half][i] = stream_load_16(value_cache + rows.value_row[i] + 8 * t);
-            else
+            } else {
+                tile.k[half][i] = make_uint4(0, 0, 0, 0);
                 tile.v[half][i] = make_uint4(0, 0, 0, 0);
+            }
         }
         tile.live |= rows.live << (half * 4);
     }
@@ -320,6 +322,8 @@ struct GroupState {
 // bytes can do.
 constexpr int kStagedRowBytes = 272;
 constexpr int kStagedTileBytes = kTile * kStagedRowBytes;
+// A wave's K staging buffer (bf16 / f16 caches): 32 rows of 256 bytes.
+constexpr int kKeyStagingBytes = kTile * 256;
 
 // GROUPS = groups of four query heads a wave carries (1 or 2: up to 8 query heads per kv head).
 // WIDE (fp8 caches): the query heads of the kv head sit in the sixteen columns of one MFMA, each once, and
@@ -527,12 +531,24 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
             s0[hg] = {0.0f, 0.0f, 0.0f, 0.0f};
             s1[hg] = {0.0f, 0.0f, 0.0f, 0.0f};
         }
+        if constexpr (!FP8) {
+            // K into its operand layout: rows go to the wave's LDS buffer as fetched (row = key, the sixteen 16-byte
+            // chunks of a row permuted by the row's low bits so that the sixteen rows an operand read touches fall
+            // in different banks) and come back as lane (g, t): key t, dims 32 c + 8 g .. + 8.
+#pragma unroll
+            for (int half = 0; half < 2; ++half)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (kDim == 128 || 8 * t < static_cast<unsigned int>(kDim))
+                        *reinterpret_cast<uint4*>(staging + wave * kKeyStagingBytes + (16 * half + 4 * g + i) * 256 + ((t ^ (4 * g + i)) << 4)) = tile.k[half][i];
+        }
 #pragma unroll
         for (int c = 0; c < kDimSteps; ++c) {
             uint4 first, second;
             if constexpr (!FP8) {
-                first = tile.k[0][c];
-                second = tile.k[1][c];
+                const unsigned char* row = staging + wave * kKeyStagingBytes + t * 256 + (((4 * c + g) ^ t) << 4);
+                first = *reinterpret_cast<const uint4*>(row);
+                second = *reinterpret_cast<const uint4*>(row + 16 * 256);
             }
 #pragma unroll
             for (int hg = 0; hg < GROUPS; ++hg) {
@@ -645,7 +661,15 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
     };
     auto consume = [&](const Tile& buffer) __attribute__((always_inline)) {
         // Returns false when this was the last tile of the range.
+#ifdef SINGE_PROBE_NO_FOLD
+        if constexpr (!FP8) {
+            unsigned int x = 0;
+            for (int h = 0; h < 2; ++h) for (int i = 0; i < 4; ++i) x ^= buffer.k[h][i].x ^ buffer.k[h][i].w ^ buffer.v[h][i].x ^ buffer.v[h][i].w;
+            state[0].running_sum += __builtin_bit_cast(float, x & 0x3fffffffu);
+        }
+#else
         fold(buffer);
+#endif
         const unsigned int next_at = at + 1;
         const bool more = next_at < range_end;
         unsigned int next_seq = seq;
@@ -694,7 +718,8 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
 #define SINGE_DECODE_KERNEL(NAME, GROUPS, ALIGNED, FP8, EXACT)                                  \
     extern "C" __global__ __launch_bounds__(512) void NAME(DecodeArgs args) {                    \
         extern __shared__ unsigned int prefix[];                                                \
-        paged_decode_body<GROUPS, ALIGNED, FP8, EXACT>(args, prefix);                           \
+        __shared__ __attribute__((aligned(16))) unsigned char staging[8 * kKeyStagingBytes];    \
+        paged_decode_body<GROUPS, ALIGNED, FP8, EXACT>(args, prefix, staging);                  \
     }
 
 SINGE_DECODE_KERNEL(SINGE_DECODE_NAME(singe_paged_decode_bf16, _g1_b16), 1, true, false, true)
@@ -706,7 +731,8 @@ SINGE_DECODE_KERNEL(SINGE_DECODE_NAME(singe_paged_decode_bf16, _g2_any), 2, fals
 #define SINGE_DECODE_F16_KERNEL(NAME, GROUPS, ALIGNED)                                          \
     extern "C" __global__ __launch_bounds__(512) void NAME(DecodeArgs args) {                    \
         extern __shared__ unsigned int prefix[];                                                \
-        paged_decode_body<GROUPS, ALIGNED, false, true, false, true>(args, prefix);             \
+        __shared__ __attribute__((aligned(16))) unsigned char staging[8 * kKeyStagingBytes];    \
+        paged_decode_body<GROUPS, ALIGNED, false, true, false, true>(args, prefix, staging);    \
     }
 
 SINGE_DECODE_F16_KERNEL(SINGE_DECODE_NAME(singe_paged_decode_f16, _g1_b16), 1, true)
@@ -755,6 +781,18 @@ SINGE_DEVICE void paged_decode_combine_body(const CombineArgs& a) {
             const unsigned int n = count - chunk < 64 ? count - chunk : 64;
             const size_t chunk_base = base + static_cast<size_t>(chunk) * a.heads_per_wave;
             const float mine = lane < n ? a.partial_lse[chunk_base + static_cast<size_t>(lane) * a.heads_per_wave] : -INFINITY;
+            // The first sixteen rows are asked for together with the log-sum-exps, before anything waits for those: a
+            // sequence rarely has more slots, and the kernel is a chain of memory round trips.
+            float2 rows[16];
+            auto fetch = [&](unsigned int first) __attribute__((always_inline)) {
+#pragma unroll
+                for (int j = 0; j < 16; ++j) {
+                    rows[j] = make_float2(0.0f, 0.0f);
+                    if (first + j < n && holds_values)
+                        rows[j] = *reinterpret_cast<const float2*>(a.partial_out + (chunk_base + static_cast<size_t>(first + j) * a.heads_per_wave) * kDim + 2 * lane);
+                }
+            };
+            fetch(0);
             float largest = mine;
 #pragma unroll
             for (int step = 32; step >= 1; step >>= 1) largest = fmaxf(largest, __shfl_xor(largest, step, 64));
@@ -770,13 +808,7 @@ SINGE_DEVICE void paged_decode_combine_body(const CombineArgs& a) {
             high *= rescale;
             best = largest;
             for (unsigned int first = 0; first < n; first += 16) {
-                float2 rows[16];
-#pragma unroll
-                for (int j = 0; j < 16; ++j) {
-                    rows[j] = make_float2(0.0f, 0.0f);
-                    if (first + j < n && holds_values)
-                        rows[j] = *reinterpret_cast<const float2*>(a.partial_out + (chunk_base + static_cast<size_t>(first + j) * a.heads_per_wave) * kDim + 2 * lane);
-                }
+                if (first != 0) fetch(first);
 #pragma unroll
                 for (int j = 0; j < 16; ++j) {
                     const float w = __shfl(weight, static_cast<int>(first) + j, 64);
