@@ -661,15 +661,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
     };
     auto consume = [&](const Tile& buffer) __attribute__((always_inline)) {
         // Returns false when this was the last tile of the range.
-#ifdef SINGE_PROBE_NO_FOLD
-        if constexpr (!FP8) {
-            unsigned int x = 0;
-            for (int h = 0; h < 2; ++h) for (int i = 0; i < 4; ++i) x ^= buffer.k[h][i].x ^ buffer.k[h][i].w ^ buffer.v[h][i].x ^ buffer.v[h][i].w;
-            state[0].running_sum += __builtin_bit_cast(float, x & 0x3fffffffu);
-        }
-#else
         fold(buffer);
-#endif
         const unsigned int next_at = at + 1;
         const bool more = next_at < range_end;
         unsigned int next_seq = seq;
