@@ -133,7 +133,9 @@ struct PagedAttentionArgs {
     uint32_t sequences;
     uint32_t cache_pages;
     uint32_t page_table;            // entries of `pages`; block-table form: entries per table row
-    uint32_t row_tiles;             // ceil(groups * tokens / 128): row tiles per (sequence, kv head)
+    uint32_t row_tiles;             // ceil(groups * tokens / 128): row tiles per (sequence, kv head); with `compact`,
+                                    // a bound on the row tiles of all sequences together
+    uint32_t compact = 0;           // workgroups find their (sequence, row tile) by a prefix sum over the sequences
     uint32_t causal;
     int32_t page_shift;             // log2(page_size) when it is a power of two, else -1
     float scale_log2e;              // scale * log2(e)

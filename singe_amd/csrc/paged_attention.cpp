@@ -34,6 +34,32 @@ struct Scratch {
     size_t bytes;
 };
 
+// How the grid covers the row tiles (see `locate` in paged_attention.hip).  When no sequence can have more than one
+// row tile the plain form is used: sequences x kv heads workgroups, a sequence found from the workgroup id alone.
+// Otherwise the compact form: every sequence has at least one entry, and the entries of all of them are at most
+// floor(tokens * groups / 128) + sequences.
+struct RowTileGrid {
+    uint32_t compact;
+    uint64_t row_tiles;   // the kernel argument
+    uint64_t blocks;      // workgroups without key splits
+};
+
+RowTileGrid grid_of(uint64_t tokens, uint64_t sequences, uint64_t groups, uint64_t kv_heads = 1) {
+    RowTileGrid grid;
+    const uint64_t longest = (groups * tokens + 127) / 128;
+    if (longest <= 1) {
+        grid.compact = 0;
+        grid.row_tiles = longest;
+        grid.blocks = (sequences * kv_heads + 7) / 8 * 8 * longest;
+    } else {
+        grid.compact = 1;
+        grid.row_tiles = groups * tokens / 128 + sequences;
+        const uint64_t bands = (grid.row_tiles + 31) / 32;
+        grid.blocks = (kv_heads * bands + 7) / 8 * 8 * 32;
+    }
+    return grid;
+}
+
 // 0 = chosen by problem size (singe_hip_set_paged_attention_splits).
 uint32_t g_paged_attention_splits = 0;
 
@@ -43,8 +69,7 @@ uint32_t paged_attention_splits(const SingePagedAttentionProblem& p) {
     if ((p.head_dim != 128 && p.head_dim != 64) || p.tokens <= 0 || p.sequences <= 0 || p.kv_heads <= 0 || p.heads <= 0) return 1;
     if (g_paged_attention_splits != 0) return g_paged_attention_splits;
     const uint64_t groups = static_cast<uint64_t>(p.heads / p.kv_heads);
-    const uint64_t row_tiles = (groups * static_cast<uint64_t>(p.tokens) + 127) / 128;
-    const uint64_t workgroups = static_cast<uint64_t>(p.sequences) * p.kv_heads * row_tiles;
+    const uint64_t workgroups = static_cast<uint64_t>(p.kv_heads) * grid_of(p.tokens, p.sequences, groups).row_tiles;
     // A sequence's key count lives in device memory: the most its pages can hold bounds it.
     const uint64_t keys = static_cast<uint64_t>(p.page_table > 0 ? p.page_table : 0) * static_cast<uint64_t>(p.page_size);
     return attention_key_splits(workgroups, keys);
@@ -133,7 +158,11 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
     args.sequences = static_cast<uint32_t>(p.sequences);
     args.cache_pages = static_cast<uint32_t>(p.cache_pages);
     args.page_table = static_cast<uint32_t>(p.page_table);
-    args.row_tiles = static_cast<uint32_t>((groups * static_cast<uint64_t>(p.tokens) + 127) / 128);
+    const RowTileGrid tiling = grid_of(static_cast<uint64_t>(p.tokens), static_cast<uint64_t>(p.sequences), groups,
+                                     static_cast<uint64_t>(p.kv_heads));
+    if (tiling.row_tiles > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many row tiles");
+    args.row_tiles = static_cast<uint32_t>(tiling.row_tiles);
+    args.compact = tiling.compact;
     args.causal = p.causal ? 1u : 0u;
     args.page_shift = -1;
     for (int shift = 0; shift < 31; ++shift)
@@ -142,8 +171,7 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
     args.scale_log2e = scale * kLog2e;
     args.softcap_scale = p.has_softcap ? scale / p.softcap : 0.0f;
     args.softcap_log2e = p.has_softcap ? p.softcap * kLog2e : 0.0f;
-    const uint64_t units = (static_cast<uint64_t>(p.sequences) * p.kv_heads + 7) / 8 * 8;
-    const uint64_t blocks = units * args.row_tiles;
+    const uint64_t blocks = tiling.blocks;
     if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
     const bool wide = p.index_type == SINGE_HIP_INDEX_I64;
     // Key splits, when the caller lent scratch for them: the attention kernel leaves partials, a second
@@ -360,7 +388,10 @@ int32_t paged_kv_prefill(
     args.sequences = static_cast<uint32_t>(c.batch);
     args.cache_pages = static_cast<uint32_t>(c.physical_blocks);
     args.page_table = static_cast<uint32_t>(c.block_table_batch_stride);
-    args.row_tiles = static_cast<uint32_t>((groups * static_cast<uint64_t>(c.total_query_tokens) + 127) / 128);
+    const RowTileGrid tiling = grid_of(c.total_query_tokens, c.batch, groups, c.kv_heads);
+    if (tiling.row_tiles > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many row tiles");
+    args.row_tiles = static_cast<uint32_t>(tiling.row_tiles);
+    args.compact = tiling.compact;
     args.causal = c.causal ? 1u : 0u;
     args.page_shift = -1;
     for (int shift = 0; shift < 31; ++shift)
@@ -368,8 +399,7 @@ int32_t paged_kv_prefill(
     args.scale_log2e = c.scale * 1.4426950408889634074f;
     args.softcap_scale = 0.0f;
     args.softcap_log2e = 0.0f;
-    const uint64_t units = (static_cast<uint64_t>(c.batch) * c.kv_heads + 7) / 8 * 8;
-    const uint64_t blocks = units * args.row_tiles;
+    const uint64_t blocks = tiling.blocks;
     if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
     const KernelId kernel = static_cast<KernelId>((f16 ? kPagedKvPrefillF16 : kPagedKvPrefill) + (args.page_shift >= 4 ? 1 : 0));
     return launch(c.head_dim == 64 ? at_head_dim_64(kernel) : kernel, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);

@@ -48,17 +48,64 @@ SINGE_DEVICE float table_value(const void* table, uint32_t table_type, size_t at
 constexpr unsigned int kNoPage = 0xFFFFFFFFu;  // a table entry outside the cache: reported, never read through
 
 // Workgroup id -> (unit = sequence * kv_heads + kv head, row tile, key split); false for ids past the units.
-// Workgroup i runs on XCD i % 8: the row tiles of one (sequence, kv head) share an XCD and its L2.  Within an XCD
-// the order is band by band of 32 row tiles: every unit's tiles 0 .. 31 (a unit's side by side, walking its
-// keys together), then every unit's tiles 32 .. 63, and so on, so the workgroups past a sequence's rows,
-// which return at once, mostly come after those with work instead of between them.  The splits of one
-// (unit, row tile) are neighbours.
+// Workgroup i runs on XCD i % 8: the row tiles of one (sequence, kv head) share an XCD and its L2.
+//
+// Plain form (a.compact == 0; calls where no sequence can have more than one row tile, decoding above all): the grid
+// covers every sequence's longest possible run of rows.  Within an XCD the order is band by band of 32 row tiles:
+// every unit's tiles 0 .. 31 (a unit's side by side, walking its keys together), then every unit's tiles 32 .. 63,
+// and so on.  The splits of one (unit, row tile) are neighbours.
+//
+// Compact form (a.compact != 0): the row tiles of all sequences form one list in sequence order, sequence s owning
+// max(1, ceil(queries_s * groups / 128)) of them (one even without queries, so that its paging values are checked),
+// and the grid covers a bound on the list's length instead of sequences x the longest possible sequence; a workgroup
+// finds its entry by a prefix sum over the sequences' query counts, 64 sequences at a time.  The list is cut into
+// bands of 32 entries; (band, kv head) pairs go round the XCDs, so a band's tiles for one kv head are neighbours on
+// one XCD and walk their keys side by side.
+template <int FORM>
 SINGE_DEVICE bool locate(const PagedAttentionArgs& a, unsigned int& unit, unsigned int& row_tile, unsigned int& split) {
     constexpr unsigned int kBand = 32;
     const unsigned int xcd = blockIdx.x & 7u;
     unsigned int within = blockIdx.x >> 3;
     split = within % a.splits;
     within /= a.splits;
+    if (a.compact != 0) {
+        const unsigned int bands = (a.row_tiles + kBand - 1) / kBand;
+        const unsigned int pair = xcd + 8u * (within / kBand);
+        if (pair >= a.kv_heads * bands) return false;
+        const unsigned int kv_head = pair % a.kv_heads, entry = (pair / a.kv_heads) * kBand + within % kBand;
+        if (entry >= a.row_tiles) return false;
+        const unsigned int lane = threadIdx.x & 63u, groups = a.heads / a.kv_heads;
+        unsigned int base = 0;
+        for (unsigned int first = 0; first < a.sequences; first += 64u) {
+            const unsigned int s = first + lane;
+            unsigned int mine = 0;
+            if (s < a.sequences) {
+                long long count;
+                if constexpr (FORM == kTable) count = read_index<FORM>(a.query_lengths, s);
+                else count = read_index<FORM>(a.query_offsets, s + 1) - read_index<FORM>(a.query_offsets, s);
+                count = count < 0 ? 0 : count > static_cast<long long>(a.tokens) ? static_cast<long long>(a.tokens) : count;
+                const unsigned long long tiles = (static_cast<unsigned long long>(count) * groups + kQueryTile - 1) / kQueryTile;
+                mine = tiles == 0 ? 1u : static_cast<unsigned int>(tiles);
+            }
+            unsigned int through = mine;  // inclusive prefix sum over the wave
+#pragma unroll
+            for (int step = 1; step < 64; step <<= 1) {
+                const unsigned int below = __shfl_up(through, step, 64);
+                if (lane >= static_cast<unsigned int>(step)) through += below;
+            }
+            const unsigned int total = __shfl(through, 63, 64);
+            if (entry < base + total) {
+                const unsigned long long holds = __ballot(entry < base + through);  // first lane whose range reaches the entry
+                const unsigned int owner = static_cast<unsigned int>(__builtin_ctzll(holds));
+                const unsigned int owner_through = __shfl(through, owner, 64), owner_mine = __shfl(mine, owner, 64);
+                unit = (first + owner) * a.kv_heads + kv_head;
+                row_tile = entry - (base + owner_through - owner_mine);
+                return true;
+            }
+            base += total;
+        }
+        return false;
+    }
     const unsigned int units_per_xcd = (a.sequences * a.kv_heads + 7u) / 8u;
     const unsigned int full_bands = a.row_tiles / kBand, band = within / (units_per_xcd * kBand);
     unsigned int local_unit;
@@ -83,7 +130,9 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     const unsigned int groups = a.heads / a.kv_heads;
 
     unsigned int unit, row_tile, split;
-    if (!locate(a, unit, row_tile, split)) return;
+    if (!locate<FORM>(a, unit, row_tile, split)) return;
+    unit = __builtin_amdgcn_readfirstlane(unit);  // the same in every lane, and known to the compiler to be
+    row_tile = __builtin_amdgcn_readfirstlane(row_tile);
     const unsigned int sequence = unit / a.kv_heads, kv_head = unit % a.kv_heads;
     const unsigned int first_row = row_tile * kQueryTile;
 
@@ -496,7 +545,7 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
 template <int FORM, class Half>
 SINGE_DEVICE void combine_body(const PagedAttentionArgs& a, unsigned int shares) {
     unsigned int unit, row_tile, split;
-    if (!locate(a, unit, row_tile, split)) return;
+    if (!locate<FORM>(a, unit, row_tile, split)) return;
     const unsigned int sequence = unit / a.kv_heads, kv_head = unit % a.kv_heads, groups = a.heads / a.kv_heads;
     const SequenceSpan span = load_span<FORM>(sequence, a.query_offsets, a.page_offsets, a.last_page_lengths, a.query_lengths,
                                               a.tokens, a.page_table, a.page_size);

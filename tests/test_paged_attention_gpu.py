@@ -6,7 +6,7 @@ import pytest
 import torch
 
 import oracle
-from singe_amd import error, neural
+from singe_amd import _native, error, neural
 
 pytestmark = pytest.mark.gpu
 
@@ -67,6 +67,25 @@ def test_ragged_sequences_match_oracle(heads, kv_heads, page_size, options):
     # queries than keys, where the CPU path's saturating position applies
     sequences = [(1, 150), (70, 70), (20, 90), (3, 0), (9, 4), (130, 300)]
     run_case(sequences, heads, kv_heads, page_size, options, seed=heads + page_size)
+
+
+@pytest.mark.parametrize("index_dtype", [torch.int32, torch.int64])
+@pytest.mark.parametrize("heads,kv_heads,page_size,splits", [(8, 2, 16, 0), (4, 4, 16, 0), (16, 1, 8, 3)])
+def test_many_ragged_sequences_find_their_row_tiles(heads, kv_heads, page_size, splits, index_dtype):
+    # more sequences than one wave's prefix sum covers (64), some without queries, some without keys, query
+    # counts from under one row tile to several
+    rng = np.random.default_rng(heads * 31 + page_size)
+    sequences = []
+    for s in range(150):
+        queries = int(rng.choice([0, 1, 1, 2, 5, 17, 31, 32, 33, 64, 100, 129, 200]))
+        keys = 0 if s % 23 == 7 else queries + int(rng.integers(0, 120))
+        sequences.append((queries, keys))
+    _native.lib().singe_hip_set_paged_attention_splits(splits)
+    try:
+        run_case(sequences, heads, kv_heads, page_size, neural.AttentionOptions(causal=True), index_dtype=index_dtype, seed=heads)
+        run_case(sequences[:70], heads, kv_heads, page_size, neural.AttentionOptions(window=40, causal=True), index_dtype=index_dtype, seed=3)
+    finally:
+        _native.lib().singe_hip_set_paged_attention_splits(0)
 
 
 @pytest.mark.parametrize("options", [neural.AttentionOptions(causal=True, softcap=-4.0), neural.AttentionOptions(scale=-0.06, softcap=5.0),
