@@ -289,6 +289,7 @@ struct LatentAttentionArgs {
     int32_t page_shift;              // log2(page_size) when that is a power of two, else -1 (matrix-core kernel)
     float* partial_out;
     float* partial_lse;
+    uint32_t unit_band;              // matrix-core kernel: neighbouring units (row tiles) that go to one XCD together
 };
 
 // singe_rotary_cache_write_*: contiguous operands of one element type; angles may be f32.

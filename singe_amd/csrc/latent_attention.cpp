@@ -111,6 +111,7 @@ int32_t paged_mla_attention(void* stream, const void* latent_queries, const void
         if (p.page_size == (int64_t{1} << shift)) args.page_shift = shift;
     args.partial_out = nullptr;
     args.partial_lse = nullptr;
+    args.unit_band = 1;
     if (tiles) {
         // Key splits, when the caller lent scratch for them: the attention kernel leaves partials, a second kernel
         // merges them.
@@ -122,8 +123,14 @@ int32_t paged_mla_attention(void* stream, const void* latent_queries, const void
             args.partial_out = static_cast<float*>(scratch);
             args.partial_lse = args.partial_out + static_cast<size_t>(splits) * p.tokens * p.heads * 512;
         }
+        // Units go to the XCDs in bands of neighbours (see the kernel): as wide as leaves every XCD something to do,
+        // 32 (an XCD's compute units, each of which holds one workgroup) at most.  The grid covers whole rounds of eight bands.
+        const uint64_t band = blocks >= 256 ? 32 : (blocks + 7) / 8;
+        const uint64_t rounds = (blocks + 8 * band - 1) / (8 * band);
+        args.unit_band = static_cast<uint32_t>(band);
+        if (rounds * 8 * band * splits > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
         const bool bf16 = p.data_type == SINGE_HIP_BF16;
-        const int32_t launched = launch(bf16 ? kLatentTilesBf16 : kLatentTilesF16, static_cast<unsigned>(blocks * splits), 1, 1, 512, stream, args);
+        const int32_t launched = launch(bf16 ? kLatentTilesBf16 : kLatentTilesF16, static_cast<unsigned>(rounds * 8 * band * splits), 1, 1, 512, stream, args);
         if (launched != 0 || splits == 1) return launched;
         return launch(bf16 ? kLatentCombineBf16 : kLatentCombineF16, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
     }

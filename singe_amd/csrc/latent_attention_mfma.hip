@@ -130,7 +130,18 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
     const unsigned int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
     const unsigned int column = lane & 15u, g = lane >> 4;  // row of the wave, lane group
     const unsigned int splits = a.splits > 1 ? a.splits : 1u;
-    const unsigned int split = blockIdx.x % splits, unit = blockIdx.x / splits;
+    // Workgroup i runs on XCD i % 8.  Units (row tiles, in sequence order) are dealt to the XCDs in bands of
+    // a.unit_band neighbours, so that the workgroups an XCD runs side by side are row tiles of the same sequence
+    // walking the same keys, and the cache rows one of them brings into the XCD's L2 serve the others.  The splits
+    // of a unit are neighbours.
+    unsigned int split, unit;
+    {
+        const unsigned int xcd = blockIdx.x & 7u;
+        unsigned int within = blockIdx.x >> 3;
+        split = within % splits;
+        within /= splits;
+        unit = ((within / a.unit_band) * 8u + xcd) * a.unit_band + within % a.unit_band;
+    }
     unsigned int sequence, row_tile;
     if (!find_unit<FORM>(a, unit, sequence, row_tile)) return;
     sequence = __builtin_amdgcn_readfirstlane(sequence);
