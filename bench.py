@@ -46,14 +46,18 @@ MIN_SAMPLES = 30
 # profile summary they come from.
 FETCH_UNIT_BYTES, WRITE_UNIT_BYTES = 2048, 1024
 COUNTER_TRAFFIC = {
-    "decode": {"kernel": "singe_paged_decode_bf16_d128_g1_b16", "FETCH_SIZE": 145766, "WRITE_SIZE": 4552,
-               "source": "profiles/paged_decode_and_prefill_hbm_traffic.md"},
-    "prefill": {"kernel": "singe_fmha_prefill_bf16_d128_causal", "FETCH_SIZE": 311083, "WRITE_SIZE": 132590,
-                "source": "profiles/paged_decode_and_prefill_hbm_traffic.md"},
-    "latent_decode": {"kernel": "singe_paged_mla_attention_bf16_l512_p64", "FETCH_SIZE": 608520, "WRITE_SIZE": 33047,
-                      "source": "profiles/paged_mla_attention_latent_kernel_stats.md"},
-    "latent_chunked_prefill": {"kernel": "singe_paged_mla_attention_bf16_l512_p64", "FETCH_SIZE": 1376200,
-                               "WRITE_SIZE": 526390, "source": "profiles/paged_mla_attention_latent_kernel_stats.md"},
+    "decode": {"kernel": "singe_paged_decode_bf16_d128_g1_b16", "FETCH_SIZE": 145725, "WRITE_SIZE": 4550,
+               "source": "profiles/hbm_traffic_counters.md"},
+    "prefill": {"kernel": "singe_fmha_prefill_bf16_d128_causal", "FETCH_SIZE": 319301, "WRITE_SIZE": 131415,
+                "source": "profiles/hbm_traffic_counters.md"},
+    "chunked_prefill": {"kernel": "singe_paged_attention_bf16_d128_i32_p16", "FETCH_SIZE": 183449, "WRITE_SIZE": 66568,
+                        "source": "profiles/hbm_traffic_counters.md"},
+    "fp8_decode": {"kernel": "singe_paged_decode_f8kv_wide_d128_b16", "FETCH_SIZE": 2129880, "WRITE_SIZE": 8256,
+                   "source": "profiles/hbm_traffic_counters.md"},
+    "latent_decode": {"kernel": "singe_paged_mla_attention_bf16_l512_p64", "FETCH_SIZE": 608523, "WRITE_SIZE": 32997,
+                      "source": "profiles/hbm_traffic_counters.md"},
+    "latent_chunked_prefill": {"kernel": "singe_paged_mla_attention_bf16_l512_p64", "FETCH_SIZE": 869183,
+                               "WRITE_SIZE": 526765, "source": "profiles/hbm_traffic_counters.md"},
 }
 
 
@@ -371,7 +375,7 @@ def chunked_prefill_section(with_cpu=True):
                     "shares keys out, its merge)",
         "value": tflops, "unit": "TFLOP/s", "tokens_per_s": work.sequences * work.new_tokens / (stats["mean_ms"] * 1e-3),
         "ms_per_step": stats["mean_ms"], "ms_per_step_median": stats["median_ms"], "algorithmic_flops": flops,
-        "key_splits_scratch_bytes": scratch_bytes,
+        "algorithmic_bytes": work.algorithmic_bytes(), "key_splits_scratch_bytes": scratch_bytes,
         "roofline": {"bound": "mfma", "kernel": "singe_paged_attention_bf16_d128_i32_p16", "achieved": tflops,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": nbytes, "traffic_source": source, **timing_fields(stats)},

@@ -172,6 +172,16 @@ class ChunkedPrefillWorkload:
         pairs = self.heads * sum(int(new * p + new * (new + 1) // 2) for p in self.prefix)
         return 4 * self.head_dim * pairs
 
+    def algorithmic_bytes(self) -> int:
+        """Every operand element once: the keys and values of prefix + new tokens per sequence, the queries, the
+        outputs, one f32 log-sum-exp per (token, head), the paging vectors (i32)."""
+        tokens = self.sequences * self.new_tokens
+        keys = int(sum(int(p) + self.new_tokens for p in self.prefix))
+        cache = 2 * keys * self.kv_heads * self.head_dim * 2
+        rows = 2 * tokens * self.heads * self.head_dim * 2 + tokens * self.heads * 4
+        paging = 4 * (len(self.query_offsets) + len(self.page_offsets) + len(self.pages) + len(self.last_page_lengths))
+        return cache + rows + paging
+
 
 def chunked_prefill_workload(*, sequences=8, new_tokens=512, heads=64, kv_heads=8, head_dim=128, page_size=16,
                              pool_pages=16384, min_prefix=1024, max_prefix=16384, seed=BASE_SEED + 4,
