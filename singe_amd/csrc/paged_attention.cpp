@@ -69,7 +69,9 @@ uint32_t paged_attention_splits(const SingePagedAttentionProblem& p) {
     if ((p.head_dim != 128 && p.head_dim != 64) || p.tokens <= 0 || p.sequences <= 0 || p.kv_heads <= 0 || p.heads <= 0) return 1;
     if (g_paged_attention_splits != 0) return g_paged_attention_splits;
     const uint64_t groups = static_cast<uint64_t>(p.heads / p.kv_heads);
-    const uint64_t workgroups = static_cast<uint64_t>(p.kv_heads) * grid_of(p.tokens, p.sequences, groups).row_tiles;
+    // Workgroups of the unsplit grid that can have work: the list of row tiles, or one per sequence, for every kv head.
+    const RowTileGrid tiling = grid_of(static_cast<uint64_t>(p.tokens), static_cast<uint64_t>(p.sequences), groups);
+    const uint64_t workgroups = static_cast<uint64_t>(p.kv_heads) * (tiling.compact ? tiling.row_tiles : tiling.row_tiles * static_cast<uint64_t>(p.sequences));
     // A sequence's key count lives in device memory: the most its pages can hold bounds it.
     const uint64_t keys = static_cast<uint64_t>(p.page_table > 0 ? p.page_table : 0) * static_cast<uint64_t>(p.page_size);
     return attention_key_splits(workgroups, keys);
