@@ -73,7 +73,8 @@ int32_t paged_attention_general(int32_t data_type, void* stream, const void* que
     args.scale = scale;
     args.scale_wide = p.has_scale ? static_cast<double>(p.scale) : 1.0 / std::sqrt(static_cast<double>(p.head_dim));
     args.softcap = p.has_softcap ? p.softcap : 0.0f;
-    const uint64_t blocks = row_blocks * static_cast<uint64_t>(p.sequences);
+    // Four rows to a workgroup, at least one workgroup to a sequence: a bound on the list the kernel walks.
+    const uint64_t blocks = static_cast<uint64_t>(p.tokens) * p.heads / 4 + static_cast<uint64_t>(p.sequences);
     if (blocks > 0x7fffffffull || row_blocks > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
     return launch(kernel, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
 }
@@ -120,7 +121,9 @@ int32_t paged_table_general(int32_t data_type, void* stream, const char* op, con
     args.scale = scale;
     args.scale_wide = scale;
     args.softcap = 0.0f;
-    const uint64_t blocks = row_blocks * sequences;
+    // Decoding: ceil(heads / 4) workgroups to a sequence.  Prefill: four rows to a workgroup, at least one workgroup
+    // to a sequence, a bound on the list the kernel walks.
+    const uint64_t blocks = decode ? row_blocks * sequences : tokens * heads / 4 + sequences;
     if (blocks > 0x7fffffffull || row_blocks > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
     return launch(kernel, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
 }

@@ -191,8 +191,19 @@ SINGE_DEVICE void paged_rows(const GeneralPagedArgs& a, typename Element<ELEMENT
     typedef typename E::type T;
     typedef typename E::real R;
     const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const unsigned int sequence = blockIdx.x / a.row_blocks;
-    const unsigned int local_row = (blockIdx.x % a.row_blocks) * 4 + wave;  // (query, head) of the sequence
+    // Decoding, every sequence has `heads` rows and a.row_blocks workgroups; otherwise the workgroups of all
+    // sequences form one list in sequence order (find_row_unit), which the grid covers without a workgroup for
+    // every row a sequence might have had.
+    unsigned int sequence, block;
+    if (DECODE) {
+        sequence = blockIdx.x / a.row_blocks;
+        block = blockIdx.x % a.row_blocks;
+    } else {
+        if (!find_row_unit<FORM>(a.query_offsets, a.query_lengths, a.sequences, a.tokens, a.heads, 4u, blockIdx.x, sequence, block)) return;
+        sequence = __builtin_amdgcn_readfirstlane(sequence);
+        block = __builtin_amdgcn_readfirstlane(block);
+    }
+    const unsigned int local_row = block * 4 + wave;  // (query, head) of the sequence
     SequenceSpan span;
     if (DECODE) {
         // One query per sequence, at row `sequence`; a key count is clamped to what the table row addresses.

@@ -101,9 +101,8 @@ int32_t paged_mla_attention(void* stream, const void* latent_queries, const void
     args.wide_index = p.index_type == SINGE_HIP_INDEX_I64 ? 1u : 0u;
     // The default scale counts the whole key width (attention.rs:603-606).
     args.scale = p.has_scale ? p.scale : static_cast<float>(1.0 / std::sqrt(static_cast<double>(p.latent_dim + p.position_dim)));
-    // The matrix-core kernel's units: a sequence owns one per 128 of its rows, at least one; the vector-unit kernel
-    // takes the upper bound for every sequence.
-    const uint64_t blocks = tiles ? row_blocks + static_cast<uint64_t>(p.sequences) : row_blocks * static_cast<uint64_t>(p.sequences);
+    // Either kernel's units: a sequence owns one per 128 (matrix cores) or 4 (vector unit) of its rows, at least one.
+    const uint64_t blocks = row_blocks + static_cast<uint64_t>(p.sequences);
     if (blocks > 0x7fffffffull || row_blocks > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
     args.splits = 1;
     args.page_shift = -1;

@@ -52,8 +52,12 @@ SINGE_DEVICE void latent_rows(const LatentAttentionArgs& a, float* lds) {
     typedef Element<ELEMENT> E;
     typedef typename E::type T;
     const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const unsigned int sequence = blockIdx.x / a.row_blocks;
-    const unsigned int local_row = (blockIdx.x % a.row_blocks) * 4 + wave;  // (query, head) of the sequence
+    // The workgroups of all sequences form one list in sequence order (find_row_unit), four rows each.
+    unsigned int sequence, block;
+    if (!find_row_unit<FORM>(a.query_offsets, nullptr, a.sequences, a.tokens, a.heads, 4u, blockIdx.x, sequence, block)) return;
+    sequence = __builtin_amdgcn_readfirstlane(sequence);
+    block = __builtin_amdgcn_readfirstlane(block);
+    const unsigned int local_row = block * 4 + wave;  // (query, head) of the sequence
     const SequenceSpan span = load_span<FORM>(sequence, a.query_offsets, a.page_offsets, a.last_page_lengths, nullptr, a.tokens,
                                               a.page_table, a.page_size);
     if (!span.valid) {

@@ -86,3 +86,46 @@ SINGE_DEVICE SequenceSpan load_span(unsigned int sequence, const void* query_off
     span.keys = span.valid ? static_cast<unsigned int>(key_count) : 0u;
     return span;
 }
+
+// Workgroup units in sequence order: sequence s owns max(1, ceil(rows_s * heads / rows_per_unit)) of them (one even
+// without rows, so that its paging values are checked), rows_s being its query count (from the offsets, or from
+// `query_lengths` in the block-table form; counts that make no sense are held to [0, tokens] and their sequence's
+// checks report them).  Every wave finds the owner of `unit` for itself by a prefix sum over the sequences, 64 at a
+// time; false for a unit past the last sequence's.  A grid of tokens * heads / rows_per_unit + sequences units
+// covers them all.
+template <int FORM>
+SINGE_DEVICE bool find_row_unit(const void* query_offsets, const void* query_lengths, unsigned int sequences, unsigned int tokens,
+                                unsigned int heads, unsigned int rows_per_unit, unsigned int unit, unsigned int& sequence,
+                                unsigned int& unit_of_sequence) {
+    const unsigned int lane = threadIdx.x & 63u;
+    unsigned int base = 0;
+    for (unsigned int first = 0; first < sequences; first += 64u) {
+        const unsigned int s = first + lane;
+        unsigned int mine = 0;
+        if (s < sequences) {
+            long long count;
+            if constexpr (FORM == kTable) count = read_index<FORM>(query_lengths, s);
+            else count = read_index<FORM>(query_offsets, s + 1) - read_index<FORM>(query_offsets, s);
+            count = count < 0 ? 0 : count > static_cast<long long>(tokens) ? static_cast<long long>(tokens) : count;
+            const unsigned long long units = (static_cast<unsigned long long>(count) * heads + rows_per_unit - 1) / rows_per_unit;
+            mine = units == 0 ? 1u : static_cast<unsigned int>(units);
+        }
+        unsigned int through = mine;  // inclusive prefix sum over the wave
+#pragma unroll
+        for (int step = 1; step < 64; step <<= 1) {
+            const unsigned int below = __shfl_up(through, step, 64);
+            if (lane >= static_cast<unsigned int>(step)) through += below;
+        }
+        const unsigned int total = __shfl(through, 63, 64);
+        if (unit < base + total) {
+            const unsigned long long holds = __ballot(unit < base + through);  // first lane whose range reaches the unit
+            const unsigned int owner = static_cast<unsigned int>(__builtin_ctzll(holds));
+            const unsigned int owner_through = __shfl(through, owner, 64), owner_mine = __shfl(mine, owner, 64);
+            sequence = first + owner;
+            unit_of_sequence = unit - (base + owner_through - owner_mine);
+            return true;
+        }
+        base += total;
+    }
+    return false;
+}

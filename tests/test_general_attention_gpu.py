@@ -292,6 +292,30 @@ def test_general_paged(dtype, dim, options, index_dtype):
     assert np.abs(got_lse[~empty] - want_lse[~empty]).max(initial=0.0) <= 2e-3
 
 
+@pytest.mark.parametrize("dtype,dim,index_dtype", [(torch.float32, 64, torch.int32), (torch.bfloat16, 48, torch.int64)])
+def test_general_paged_finds_the_rows_of_many_ragged_sequences(dtype, dim, index_dtype):
+    # more sequences than one wave's prefix sum covers (64), some without queries, some without keys
+    rng = np.random.default_rng(dim)
+    sequences = []
+    for s in range(150):
+        queries = int(rng.choice([0, 1, 1, 2, 3, 5, 9, 17]))
+        sequences.append((queries, 0 if s % 19 == 3 else queries + int(rng.integers(0, 40))))
+    heads, kv_heads, page_size = 6, 2, 5
+    query_offsets, page_offsets, table, last, page_count = paged_layout(sequences, page_size)
+    q, kc, vc = tensors((query_offsets[-1], heads, dim), (page_count, page_size, kv_heads, dim), (page_count, page_size, kv_heads, dim),
+                        dtype, 9)
+    index = lambda values: torch.tensor(values, dtype=index_dtype, device="cuda")
+    paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
+    out, lse = neural.paged_attention(q, kc, vc, paging, neural.AttentionOptions(causal=True))
+    status, want, want_lse = oracle.paged_attention_f32(host(q), host(kc), host(vc), query_offsets, page_offsets, table, last,
+                                                        threads=8, causal=True)
+    assert status == 0
+    close(host(out), want, dtype)
+    empty = np.isneginf(want_lse)
+    assert np.array_equal(np.isneginf(lse.cpu().numpy()), empty)
+    assert np.abs(lse.cpu().numpy()[~empty] - want_lse[~empty]).max(initial=0.0) <= 2e-3
+
+
 VALID = dict(query_offsets=[0, 1, 3], page_offsets=[0, 2, 3], pages=[1, 0, 2], last=[2, 1])
 INVALID = [
     dict(pages=[1, 0, 3]), dict(pages=[1, -1, 2]), dict(last=[2, 5]), dict(last=[-1, 1]), dict(query_offsets=[0, 2, 1]),

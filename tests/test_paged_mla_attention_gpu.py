@@ -18,7 +18,9 @@ def values(shape, seed):
     return (((index * 37 + seed * 11) % 41).astype(np.float32) / 40.0 - 0.5).reshape(shape)
 
 
+MANY = [(int(q), 0 if s % 17 == 5 else int(q) + s % 23) for s, q in enumerate(np.random.default_rng(2).choice([0, 1, 1, 2, 3, 7], size=100))]
 BATCHES = [
+    MANY,                                  # more sequences than one wave's prefix sum covers, some without queries or keys
     [(1, 150), (9, 9), (5, 70), (2, 0)],   # decode over a long cache, a whole prefill, a chunk, a sequence with no keys
     [(1, 2000), (2, 1500)],                # few long sequences
     [(1, 300), (1, 40), (1, 0)],           # decoding alone
