@@ -109,6 +109,19 @@ def test_f16_matches_oracle(case, causal):
     run_case(causal=causal, seed=12, dtype=torch.float16, **case)
 
 
+@pytest.mark.parametrize("dtype,dim", [(torch.bfloat16, 128), (torch.bfloat16, 64), (torch.float16, 96)])
+def test_many_ragged_sequences_find_their_row_tiles(dtype, dim):
+    # more sequences than one wave's prefix sum covers (64), query counts from none to several 128-row tiles,
+    # unowned rows between sequences; 96 takes the one-wave-per-row kernel's list of workgroups
+    rng = np.random.default_rng(dim)
+    sequences = []
+    for s in range(130):
+        queries = int(rng.choice([0, 1, 2, 7, 31, 32, 33, 70, 150]))
+        sequences.append((queries, 0 if s % 29 == 4 else queries + int(rng.integers(0, 90))))
+    run_case(sequences, 8, 2, 16, True, seed=dim, gap_tokens=1, dtype=dtype, dim=dim)
+    run_case(sequences[:70], 4, 4, 7, False, seed=dim + 1, dtype=dtype, dim=dim)
+
+
 def test_more_queries_than_keys_causal_and_full():
     """Queries past the last key see every key when causal (key <= query index) and when not."""
     run_case([(48, 5)], 4, 1, 4, True, seed=3)
