@@ -520,7 +520,8 @@ def fp8_decode_section(with_cpu=True):
 def head_dim_64_section():
     """The matrix-core kernels at head_dim 64, the other head dimension of the reference's own tests
     (singe/src/backend/cuda/kernel_plan/source/tests.rs:830-966): the third configuration's prefill and the second
-    configuration's decode at that width."""
+    configuration's decode at that width; and the prefill at head_dim 96 and 32, which the dense and paged kernels are
+    built for as well."""
     import numpy as np
     import torch
 
@@ -543,7 +544,9 @@ def head_dim_64_section():
     decode = {"workload": "paged decode: batch 32, 32q/8kv heads, head_dim 64, bf16, block 16, ctx U[512,4096]; split + reduce",
               "value": gbps, "unit": "GB/s", "ms_per_step": stats["mean_ms"], "algorithmic_bytes": nbytes,
               "pct_hbm_peak": 100.0 * gbps / HBM_PEAK_GBPS, **timing_fields(stats)}
-    return {"prefill": prefill, "decode": decode}
+    # The dense prefill at the other widths the matrix-core kernels are built for.
+    others = {f"prefill_d{dim}": prefill_section(with_cpu=False, dim=dim, key=f"prefill_d{dim}") for dim in (96, 32)}
+    return {"prefill": prefill, "decode": decode, **others}
 
 
 def mfma_ceiling_section():

@@ -50,6 +50,10 @@ PARTS = [
     ("paged_attention_d64", "paged_attention.hip", ["-DSINGE_HEAD_DIM=64"]),
     ("general_attention_f64", "general_attention.hip", ["-DSINGE_GENERAL_ELEMENT=3"]),
     ("hbm_stream", "hbm_stream.hip", []),
+    ("fmha_prefill_d32", "fmha_prefill.hip", ["-DSINGE_HEAD_DIM=32"]),
+    ("paged_attention_d32", "paged_attention.hip", ["-DSINGE_HEAD_DIM=32"]),
+    ("fmha_prefill_d96", "fmha_prefill.hip", ["-DSINGE_HEAD_DIM=96"]),
+    ("paged_attention_d96", "paged_attention.hip", ["-DSINGE_HEAD_DIM=96"]),
 ]
 HOST_SOURCES = ["hip_runtime_loader.cpp", "module.cpp", "paged_decode.cpp", "fmha_prefill.cpp", "paged_attention.cpp",
                 "general_attention.cpp", "fmha_decode.cpp", "paged_rows_f32.cpp", "latent_attention.cpp", "cache_ops.cpp",

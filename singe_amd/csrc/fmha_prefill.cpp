@@ -148,7 +148,7 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
         return status;
 
     // What the gfx950 kernel takes: head_dim 128 and rows it can fetch 16 bytes at a time.
-    if (c.head_dim != 128 && c.head_dim != 64) {
+    if (!has_matrix_core_build(static_cast<long long>(c.head_dim))) {
         // Other head dimensions (the reference's matrix path takes 16 and 32 too: fmha.rs:752-755) run on the
         // one-wave-per-row kernel, up to 256; without the dense op's options, which only reach here at 64 and 128.
         DenseGeneralOperands o;
@@ -230,14 +230,14 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
         args.partial_lse = args.partial_out + static_cast<size_t>(splits) * row_count * c.head_dim;
         groups *= splits;
     }
-    const bool narrow = c.head_dim == 64;
+    const long long head_dim = static_cast<long long>(c.head_dim);
     const KernelId kernel = static_cast<KernelId>((f16 ? kPrefillCausalF16 : kPrefillCausal) + (c.causal ? 0 : 1) + (with_options ? 4 : 0));
-    if (int32_t status = launch(narrow ? at_head_dim_64(kernel) : kernel, static_cast<unsigned>(groups), 1, 1, 64 * kDensePrefillWaves, stream, args))
+    if (int32_t status = launch(at_head_dim(kernel, head_dim), static_cast<unsigned>(groups), 1, 1, 64 * kDensePrefillWaves, stream, args))
         return status;
     if (splits == 1) return 0;
     const uint64_t merge_groups = (static_cast<uint64_t>(c.batch) * c.heads * c.query_len + 3) / 4;
     if (merge_groups > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
-    const KernelId merge = static_cast<KernelId>((narrow ? kPrefillCombineD64 : kPrefillCombine) + (f16 ? 1 : 0));
+    const KernelId merge = static_cast<KernelId>(prefill_combine_at(head_dim) + (f16 ? 1 : 0));
     return launch(merge, static_cast<unsigned>(merge_groups), 1, 1, 256, stream, args);
 }
 
@@ -246,7 +246,7 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
 namespace singe_hip {
 
 uint32_t dense_prefill_splits(const SingeFmhaPrefillConfig& c) {
-    if ((c.head_dim != 128 && c.head_dim != 64) || c.batch == 0 || c.heads == 0 || c.query_len == 0) return 1;
+    if (!has_matrix_core_build(static_cast<long long>(c.head_dim)) || c.batch == 0 || c.heads == 0 || c.query_len == 0) return 1;
     constexpr size_t kTileRows = 32 * kDensePrefillWaves;
     const uint64_t query_tiles = (c.query_len + kTileRows - 1) / kTileRows;
     const uint64_t workgroups = static_cast<uint64_t>(c.batch) * c.heads * ((query_tiles + 1) / 2);

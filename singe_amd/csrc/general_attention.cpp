@@ -188,7 +188,7 @@ SingeFmhaPrefillConfig matrix_core_config(const SingeAttentionProblem& p, float 
 }
 
 bool takes_matrix_cores(const SingeAttentionProblem& p) {
-    return (p.data_type == SINGE_HIP_BF16 || p.data_type == SINGE_HIP_F16) && (p.head_dim == 128 || p.head_dim == 64) &&
+    return (p.data_type == SINGE_HIP_BF16 || p.data_type == SINGE_HIP_F16) && has_matrix_core_build(p.head_dim) &&
            p.value_dim == p.head_dim;
 }
 

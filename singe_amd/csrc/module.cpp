@@ -95,6 +95,44 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_attention_general_f64_d64", "singe_attention_general_f64_d128", "singe_attention_general_f64_d256",
     "singe_paged_attention_general_f64_d64", "singe_paged_attention_general_f64_d128", "singe_paged_attention_general_f64_d256",
     "singe_hbm_stream_read",
+    "singe_fmha_prefill_bf16_d32_causal", "singe_fmha_prefill_bf16_d32_full",
+    "singe_fmha_prefill_f16_d32_causal", "singe_fmha_prefill_f16_d32_full",
+    "singe_fmha_prefill_bf16_d32_causal_options", "singe_fmha_prefill_bf16_d32_full_options",
+    "singe_fmha_prefill_f16_d32_causal_options", "singe_fmha_prefill_f16_d32_full_options",
+    "singe_fmha_prefill_bf16_d32_combine", "singe_fmha_prefill_f16_d32_combine",
+    "singe_paged_attention_bf16_d32_i32", "singe_paged_attention_bf16_d32_i64",
+    "singe_paged_attention_bf16_d32_softcap_i32", "singe_paged_attention_bf16_d32_softcap_i64",
+    "singe_paged_attention_bf16_d32_i32_p16", "singe_paged_attention_bf16_d32_i64_p16",
+    "singe_paged_attention_bf16_d32_softcap_i32_p16", "singe_paged_attention_bf16_d32_softcap_i64_p16",
+    "singe_paged_kv_prefill_bf16_d32", "singe_paged_kv_prefill_bf16_d32_p16",
+    "singe_paged_kv_prefill_f16_d32", "singe_paged_kv_prefill_f16_d32_p16",
+    "singe_paged_attention_combine_bf16_d32_i32", "singe_paged_attention_combine_bf16_d32_i64",
+    "singe_paged_attention_combine_f16_d32_i32", "singe_paged_attention_combine_f16_d32_i64",
+    "singe_paged_attention_f16_d32_i32", "singe_paged_attention_f16_d32_i64",
+    "singe_paged_attention_f16_d32_softcap_i32", "singe_paged_attention_f16_d32_softcap_i64",
+    "singe_paged_attention_f16_d32_i32_p16", "singe_paged_attention_f16_d32_i64_p16",
+    "singe_paged_attention_f16_d32_softcap_i32_p16", "singe_paged_attention_f16_d32_softcap_i64_p16",
+    "singe_rotary_paged_attention_bf16_d32_i32", "singe_rotary_paged_attention_bf16_d32_i64",
+    "singe_rotary_paged_attention_bf16_d32_i32_p16", "singe_rotary_paged_attention_bf16_d32_i64_p16",
+    "singe_fmha_prefill_bf16_d96_causal", "singe_fmha_prefill_bf16_d96_full",
+    "singe_fmha_prefill_f16_d96_causal", "singe_fmha_prefill_f16_d96_full",
+    "singe_fmha_prefill_bf16_d96_causal_options", "singe_fmha_prefill_bf16_d96_full_options",
+    "singe_fmha_prefill_f16_d96_causal_options", "singe_fmha_prefill_f16_d96_full_options",
+    "singe_fmha_prefill_bf16_d96_combine", "singe_fmha_prefill_f16_d96_combine",
+    "singe_paged_attention_bf16_d96_i32", "singe_paged_attention_bf16_d96_i64",
+    "singe_paged_attention_bf16_d96_softcap_i32", "singe_paged_attention_bf16_d96_softcap_i64",
+    "singe_paged_attention_bf16_d96_i32_p16", "singe_paged_attention_bf16_d96_i64_p16",
+    "singe_paged_attention_bf16_d96_softcap_i32_p16", "singe_paged_attention_bf16_d96_softcap_i64_p16",
+    "singe_paged_kv_prefill_bf16_d96", "singe_paged_kv_prefill_bf16_d96_p16",
+    "singe_paged_kv_prefill_f16_d96", "singe_paged_kv_prefill_f16_d96_p16",
+    "singe_paged_attention_combine_bf16_d96_i32", "singe_paged_attention_combine_bf16_d96_i64",
+    "singe_paged_attention_combine_f16_d96_i32", "singe_paged_attention_combine_f16_d96_i64",
+    "singe_paged_attention_f16_d96_i32", "singe_paged_attention_f16_d96_i64",
+    "singe_paged_attention_f16_d96_softcap_i32", "singe_paged_attention_f16_d96_softcap_i64",
+    "singe_paged_attention_f16_d96_i32_p16", "singe_paged_attention_f16_d96_i64_p16",
+    "singe_paged_attention_f16_d96_softcap_i32_p16", "singe_paged_attention_f16_d96_softcap_i64_p16",
+    "singe_rotary_paged_attention_bf16_d96_i32", "singe_rotary_paged_attention_bf16_d96_i64",
+    "singe_rotary_paged_attention_bf16_d96_i32_p16", "singe_rotary_paged_attention_bf16_d96_i64_p16",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -104,7 +142,7 @@ const char* const kPartNames[kPartCount] = {
     "paged_decode", "fmha_prefill", "fmha_prefill_f32", "paged_attention", "splitk_reduce", "attention_rows_f32",
     "cache_ops", "latent_attention", "latent_attention_mfma", "general_attention_f32", "general_attention_bf16",
     "general_attention_f16", "mfma_ceiling", "paged_decode_d64", "fmha_prefill_d64", "paged_attention_d64",
-    "general_attention_f64", "hbm_stream",
+    "general_attention_f64", "hbm_stream", "fmha_prefill_d32", "paged_attention_d32", "fmha_prefill_d96", "paged_attention_d96",
 };
 
 namespace {
@@ -121,6 +159,8 @@ constexpr PartRun kPartRuns[] = {
     {1, 2}, {14, 2},              // the dense kernels' merges
     {16, 6},                      // the general kernels on f64
     {17, 1},
+    {18, 10}, {19, 28},           // the head_dim 32 builds: dense kernels with their merges, paged kernels
+    {20, 10}, {21, 28},           // the head_dim 96 builds
 };
 constexpr int runs_total() {
     int total = 0;

@@ -57,7 +57,11 @@ enum KernelId : int {
     kDenseGeneralF64, kPagedGeneralF64 = kDenseGeneralF64 + 3,
     // the plain streaming read a decode kernel is priced against
     kHbmStreamRead = kPagedGeneralF64 + 3,
-    kKernelCount
+    // the dense prefill and paged attention kernels built for head_dim 32 and for 96, each bank in the order of
+    // its head_dim 128 forms (eight dense kernels, their two merges, the paged kernels up to kSplitKReduce)
+    kPrefillD32, kPrefillCombineD32 = kPrefillD32 + 8, kPagedD32 = kPrefillCombineD32 + 2,
+    kPrefillD96 = kPagedD32 + (kSplitKReduce - kPagedAttentionI32), kPrefillCombineD96 = kPrefillD96 + 8, kPagedD96 = kPrefillCombineD96 + 2,
+    kKernelCount = kPagedD96 + (kSplitKReduce - kPagedAttentionI32)
 };
 
 // The head_dim 64 build of a matrix-core kernel named by its head_dim 128 id.
@@ -67,10 +71,27 @@ inline KernelId at_head_dim_64(KernelId kernel) {
     return static_cast<KernelId>(kPagedD64 + (kernel - kPagedAttentionI32));
 }
 
+// Whether the dense prefill and paged attention kernels have a matrix-core build for a head dimension.
+inline bool has_matrix_core_build(long long head_dim) { return head_dim == 128 || head_dim == 96 || head_dim == 64 || head_dim == 32; }
+
+// That build of a dense prefill or paged attention kernel named by its head_dim 128 id (decode kernels: 64 only).
+inline KernelId at_head_dim(KernelId kernel, long long head_dim) {
+    if (head_dim == 128) return kernel;
+    if (head_dim == 64) return at_head_dim_64(kernel);
+    const bool dense = kernel >= kPrefillCausal && kernel < kPrefillF32D32;
+    if (head_dim == 32) return static_cast<KernelId>(dense ? kPrefillD32 + (kernel - kPrefillCausal) : kPagedD32 + (kernel - kPagedAttentionI32));
+    return static_cast<KernelId>(dense ? kPrefillD96 + (kernel - kPrefillCausal) : kPagedD96 + (kernel - kPagedAttentionI32));
+}
+
+// The merge kernel of the dense kernels' key splits for a head dimension (+ 1 for f16).
+inline KernelId prefill_combine_at(long long head_dim) {
+    return head_dim == 128 ? kPrefillCombine : head_dim == 64 ? kPrefillCombineD64 : head_dim == 32 ? kPrefillCombineD32 : kPrefillCombineD96;
+}
+
 extern const char* const kKernelNames[kKernelCount];
 
 // Parts of the code object (one file each) and the part a kernel lives in.
-constexpr int kPartCount = 18;
+constexpr int kPartCount = 22;
 extern const char* const kPartNames[kPartCount];
 int kernel_part(int kernel);
 

@@ -66,7 +66,7 @@ uint32_t g_paged_attention_splits = 0;
 // Key splits for a problem: enough workgroups to fill the compute units four times over, when the query rows
 // alone do not (decoding, short chunks); one (no split) for other element types and head dimensions.
 uint32_t paged_attention_splits(const SingePagedAttentionProblem& p) {
-    if ((p.head_dim != 128 && p.head_dim != 64) || p.tokens <= 0 || p.sequences <= 0 || p.kv_heads <= 0 || p.heads <= 0) return 1;
+    if (!has_matrix_core_build(p.head_dim) || p.tokens <= 0 || p.sequences <= 0 || p.kv_heads <= 0 || p.heads <= 0) return 1;
     if (g_paged_attention_splits != 0) return g_paged_attention_splits;
     const uint64_t groups = static_cast<uint64_t>(p.heads / p.kv_heads);
     // Workgroups of the unsplit grid that can have work: the list of row tiles, or one per sequence, for every kv head.
@@ -98,7 +98,7 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
         // The fused form exists for the tensor-core kernel alone and without softcap here; the reference
         // plans the rotation and the attention apart for the rest (compiled/plan/group.rs:94-98), and so
         // does a caller of this library (singe_hip_rotary_cache_write, then singe_hip_paged_attention_*).
-        if (data_type != SINGE_HIP_BF16 || (p.head_dim != 128 && p.head_dim != 64))
+        if (data_type != SINGE_HIP_BF16 || !has_matrix_core_build(p.head_dim))
             return fail(SINGE_HIP_UNSUPPORTED_WIDTH, "rotary_paged_attention", static_cast<uint64_t>(p.head_dim));
         if (p.has_softcap) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "rotary paged attention with a softcap");
     }
@@ -129,9 +129,9 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
     // multiples of 16 up to 128: paged_attention.rs:586-592); everything else goes to the general one
     // (paged_general.rs:73-247).
     const bool f16 = data_type == SINGE_HIP_F16;
-    const bool narrow = p.head_dim == 64;  // the head_dim 64 build of the same kernels
-    auto built = [narrow](int kernel) { return narrow ? at_head_dim_64(static_cast<KernelId>(kernel)) : static_cast<KernelId>(kernel); };
-    if ((data_type != SINGE_HIP_BF16 && !f16) || (p.head_dim != 128 && !narrow))
+    const long long head_dim = p.head_dim;  // the build of the kernels for it
+    auto built = [head_dim](int kernel) { return at_head_dim(static_cast<KernelId>(kernel), head_dim); };
+    if ((data_type != SINGE_HIP_BF16 && !f16) || !has_matrix_core_build(head_dim))
         return paged_attention_general(data_type, stream, query_rows_any, key_cache_any, value_cache_any, query_offsets,
                                        page_offsets, pages, last_page_lengths, output_any, lse, status, p, scale);
     const uint16_t* query_rows = static_cast<const uint16_t*>(query_rows_any);
@@ -362,7 +362,7 @@ int32_t paged_kv_prefill(
         if (pointers[i] == nullptr) return fail(SINGE_HIP_NULL_POINTER, names[i]);
     // The matrix-core kernels are built for head dimensions 128 and 64; the others (up to 256) take the
     // one-wave-per-row kernel.
-    if (c.head_dim != 128 && c.head_dim != 64)
+    if (!has_matrix_core_build(static_cast<long long>(c.head_dim)))
         return paged_table_general(f16 ? SINGE_HIP_F16 : SINGE_HIP_BF16, stream,
                                    f16 ? "paged_kv_prefill_attention_f16" : "paged_kv_prefill_attention_bf16", query, key_cache,
                                    value_cache, actual_seq_offsets, actual_seq_lens_q, actual_seq_lens_kv, block_table, out, lse,
@@ -404,6 +404,6 @@ int32_t paged_kv_prefill(
     const uint64_t blocks = tiling.blocks;
     if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
     const KernelId kernel = static_cast<KernelId>((f16 ? kPagedKvPrefillF16 : kPagedKvPrefill) + (args.page_shift >= 4 ? 1 : 0));
-    return launch(c.head_dim == 64 ? at_head_dim_64(kernel) : kernel, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+    return launch(at_head_dim(kernel, static_cast<long long>(c.head_dim)), static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
 }
 }  // namespace

@@ -108,17 +108,18 @@ def test_fused_rotation_options():
 @pytest.mark.parametrize("norm", [None, "weighted"])
 @pytest.mark.parametrize("heads,kv_heads,page_size,table_dtype,index_dtype", [
     (8, 2, 16, torch.float32, torch.int32), (8, 1, 7, torch.bfloat16, torch.int64)])
-def test_fused_rotation_at_head_dim_64(heads, kv_heads, page_size, table_dtype, index_dtype, norm):
+@pytest.mark.parametrize("dim", [64, 32, 96])
+def test_fused_rotation_at_other_head_dims(heads, kv_heads, page_size, table_dtype, index_dtype, norm, dim):
     run_case(SEQUENCES, heads, kv_heads, page_size, table_dtype, index_dtype, norm, neural.AttentionOptions(causal=True),
-             seed=heads + page_size, dim=64)
+             seed=heads + page_size, dim=dim)
 
 
 def test_fused_rotation_refuses_what_it_does_not_take():
-    q = torch.zeros((2, 2, 96), device="cuda", dtype=torch.bfloat16)
-    cache = torch.zeros((2, 4, 2, 96), device="cuda", dtype=torch.bfloat16)
+    q = torch.zeros((2, 2, 80), device="cuda", dtype=torch.bfloat16)
+    cache = torch.zeros((2, 4, 2, 80), device="cuda", dtype=torch.bfloat16)
     index = lambda values: torch.tensor(values, dtype=torch.int32, device="cuda")
     paging = neural.Paging(index([0, 2]), index([0, 1]), index([0]), index([2]))
-    angles = torch.zeros((2, 1, 48), device="cuda")
+    angles = torch.zeros((2, 1, 40), device="cuda")
     with pytest.raises(error.UnsupportedWidth):
         neural.rotary_paged_attention(q, cache, cache, paging, angles, angles)
     q128 = torch.zeros((2, 2, 128), device="cuda", dtype=torch.bfloat16)
