@@ -351,7 +351,8 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
         for (int db = 0; db < kDimBlocks; ++db)
 #pragma unroll
             for (int quad = 0; quad < 4; ++quad)
-                *reinterpret_cast<float4*>(row + 32 * db + 8 * quad + 4 * hi) =
+                if (32 * db + 8 * quad < kHeadDim)
+                    *reinterpret_cast<float4*>(row + 32 * db + 8 * quad + 4 * hi) =
                     make_float4(state.out[db][4 * quad + 0] * inverse, state.out[db][4 * quad + 1] * inverse,
                                 state.out[db][4 * quad + 2] * inverse, state.out[db][4 * quad + 3] * inverse);
         if (hi == 0) a.partial_lse[slot] = sum > 0.0f ? state.reference + fast_log2(sum) : -INFINITY;
@@ -362,6 +363,7 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
         for (int db = 0; db < kDimBlocks; ++db)
 #pragma unroll
             for (int quad = 0; quad < 4; ++quad) {
+                if (32 * db + 8 * quad >= kHeadDim) continue;
                 uint2 packed;
                 packed.x = pack_pair(half, state.out[db][4 * quad + 0] * inverse, state.out[db][4 * quad + 1] * inverse);
                 packed.y = pack_pair(half, state.out[db][4 * quad + 2] * inverse, state.out[db][4 * quad + 3] * inverse);

@@ -133,6 +133,82 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_attention_f16_d96_softcap_i32_p16", "singe_paged_attention_f16_d96_softcap_i64_p16",
     "singe_rotary_paged_attention_bf16_d96_i32", "singe_rotary_paged_attention_bf16_d96_i64",
     "singe_rotary_paged_attention_bf16_d96_i32_p16", "singe_rotary_paged_attention_bf16_d96_i64_p16",
+    "singe_fmha_prefill_bf16_d16_causal", "singe_fmha_prefill_bf16_d16_full",
+    "singe_fmha_prefill_f16_d16_causal", "singe_fmha_prefill_f16_d16_full",
+    "singe_fmha_prefill_bf16_d16_causal_options", "singe_fmha_prefill_bf16_d16_full_options",
+    "singe_fmha_prefill_f16_d16_causal_options", "singe_fmha_prefill_f16_d16_full_options",
+    "singe_fmha_prefill_bf16_d16_combine", "singe_fmha_prefill_f16_d16_combine",
+    "singe_paged_attention_bf16_d16_i32", "singe_paged_attention_bf16_d16_i64",
+    "singe_paged_attention_bf16_d16_softcap_i32", "singe_paged_attention_bf16_d16_softcap_i64",
+    "singe_paged_attention_bf16_d16_i32_p16", "singe_paged_attention_bf16_d16_i64_p16",
+    "singe_paged_attention_bf16_d16_softcap_i32_p16", "singe_paged_attention_bf16_d16_softcap_i64_p16",
+    "singe_paged_kv_prefill_bf16_d16", "singe_paged_kv_prefill_bf16_d16_p16",
+    "singe_paged_kv_prefill_f16_d16", "singe_paged_kv_prefill_f16_d16_p16",
+    "singe_paged_attention_combine_bf16_d16_i32", "singe_paged_attention_combine_bf16_d16_i64",
+    "singe_paged_attention_combine_f16_d16_i32", "singe_paged_attention_combine_f16_d16_i64",
+    "singe_paged_attention_f16_d16_i32", "singe_paged_attention_f16_d16_i64",
+    "singe_paged_attention_f16_d16_softcap_i32", "singe_paged_attention_f16_d16_softcap_i64",
+    "singe_paged_attention_f16_d16_i32_p16", "singe_paged_attention_f16_d16_i64_p16",
+    "singe_paged_attention_f16_d16_softcap_i32_p16", "singe_paged_attention_f16_d16_softcap_i64_p16",
+    "singe_rotary_paged_attention_bf16_d16_i32", "singe_rotary_paged_attention_bf16_d16_i64",
+    "singe_rotary_paged_attention_bf16_d16_i32_p16", "singe_rotary_paged_attention_bf16_d16_i64_p16",
+    "singe_fmha_prefill_bf16_d48_causal", "singe_fmha_prefill_bf16_d48_full",
+    "singe_fmha_prefill_f16_d48_causal", "singe_fmha_prefill_f16_d48_full",
+    "singe_fmha_prefill_bf16_d48_causal_options", "singe_fmha_prefill_bf16_d48_full_options",
+    "singe_fmha_prefill_f16_d48_causal_options", "singe_fmha_prefill_f16_d48_full_options",
+    "singe_fmha_prefill_bf16_d48_combine", "singe_fmha_prefill_f16_d48_combine",
+    "singe_paged_attention_bf16_d48_i32", "singe_paged_attention_bf16_d48_i64",
+    "singe_paged_attention_bf16_d48_softcap_i32", "singe_paged_attention_bf16_d48_softcap_i64",
+    "singe_paged_attention_bf16_d48_i32_p16", "singe_paged_attention_bf16_d48_i64_p16",
+    "singe_paged_attention_bf16_d48_softcap_i32_p16", "singe_paged_attention_bf16_d48_softcap_i64_p16",
+    "singe_paged_kv_prefill_bf16_d48", "singe_paged_kv_prefill_bf16_d48_p16",
+    "singe_paged_kv_prefill_f16_d48", "singe_paged_kv_prefill_f16_d48_p16",
+    "singe_paged_attention_combine_bf16_d48_i32", "singe_paged_attention_combine_bf16_d48_i64",
+    "singe_paged_attention_combine_f16_d48_i32", "singe_paged_attention_combine_f16_d48_i64",
+    "singe_paged_attention_f16_d48_i32", "singe_paged_attention_f16_d48_i64",
+    "singe_paged_attention_f16_d48_softcap_i32", "singe_paged_attention_f16_d48_softcap_i64",
+    "singe_paged_attention_f16_d48_i32_p16", "singe_paged_attention_f16_d48_i64_p16",
+    "singe_paged_attention_f16_d48_softcap_i32_p16", "singe_paged_attention_f16_d48_softcap_i64_p16",
+    "singe_rotary_paged_attention_bf16_d48_i32", "singe_rotary_paged_attention_bf16_d48_i64",
+    "singe_rotary_paged_attention_bf16_d48_i32_p16", "singe_rotary_paged_attention_bf16_d48_i64_p16",
+    "singe_fmha_prefill_bf16_d80_causal", "singe_fmha_prefill_bf16_d80_full",
+    "singe_fmha_prefill_f16_d80_causal", "singe_fmha_prefill_f16_d80_full",
+    "singe_fmha_prefill_bf16_d80_causal_options", "singe_fmha_prefill_bf16_d80_full_options",
+    "singe_fmha_prefill_f16_d80_causal_options", "singe_fmha_prefill_f16_d80_full_options",
+    "singe_fmha_prefill_bf16_d80_combine", "singe_fmha_prefill_f16_d80_combine",
+    "singe_paged_attention_bf16_d80_i32", "singe_paged_attention_bf16_d80_i64",
+    "singe_paged_attention_bf16_d80_softcap_i32", "singe_paged_attention_bf16_d80_softcap_i64",
+    "singe_paged_attention_bf16_d80_i32_p16", "singe_paged_attention_bf16_d80_i64_p16",
+    "singe_paged_attention_bf16_d80_softcap_i32_p16", "singe_paged_attention_bf16_d80_softcap_i64_p16",
+    "singe_paged_kv_prefill_bf16_d80", "singe_paged_kv_prefill_bf16_d80_p16",
+    "singe_paged_kv_prefill_f16_d80", "singe_paged_kv_prefill_f16_d80_p16",
+    "singe_paged_attention_combine_bf16_d80_i32", "singe_paged_attention_combine_bf16_d80_i64",
+    "singe_paged_attention_combine_f16_d80_i32", "singe_paged_attention_combine_f16_d80_i64",
+    "singe_paged_attention_f16_d80_i32", "singe_paged_attention_f16_d80_i64",
+    "singe_paged_attention_f16_d80_softcap_i32", "singe_paged_attention_f16_d80_softcap_i64",
+    "singe_paged_attention_f16_d80_i32_p16", "singe_paged_attention_f16_d80_i64_p16",
+    "singe_paged_attention_f16_d80_softcap_i32_p16", "singe_paged_attention_f16_d80_softcap_i64_p16",
+    "singe_rotary_paged_attention_bf16_d80_i32", "singe_rotary_paged_attention_bf16_d80_i64",
+    "singe_rotary_paged_attention_bf16_d80_i32_p16", "singe_rotary_paged_attention_bf16_d80_i64_p16",
+    "singe_fmha_prefill_bf16_d112_causal", "singe_fmha_prefill_bf16_d112_full",
+    "singe_fmha_prefill_f16_d112_causal", "singe_fmha_prefill_f16_d112_full",
+    "singe_fmha_prefill_bf16_d112_causal_options", "singe_fmha_prefill_bf16_d112_full_options",
+    "singe_fmha_prefill_f16_d112_causal_options", "singe_fmha_prefill_f16_d112_full_options",
+    "singe_fmha_prefill_bf16_d112_combine", "singe_fmha_prefill_f16_d112_combine",
+    "singe_paged_attention_bf16_d112_i32", "singe_paged_attention_bf16_d112_i64",
+    "singe_paged_attention_bf16_d112_softcap_i32", "singe_paged_attention_bf16_d112_softcap_i64",
+    "singe_paged_attention_bf16_d112_i32_p16", "singe_paged_attention_bf16_d112_i64_p16",
+    "singe_paged_attention_bf16_d112_softcap_i32_p16", "singe_paged_attention_bf16_d112_softcap_i64_p16",
+    "singe_paged_kv_prefill_bf16_d112", "singe_paged_kv_prefill_bf16_d112_p16",
+    "singe_paged_kv_prefill_f16_d112", "singe_paged_kv_prefill_f16_d112_p16",
+    "singe_paged_attention_combine_bf16_d112_i32", "singe_paged_attention_combine_bf16_d112_i64",
+    "singe_paged_attention_combine_f16_d112_i32", "singe_paged_attention_combine_f16_d112_i64",
+    "singe_paged_attention_f16_d112_i32", "singe_paged_attention_f16_d112_i64",
+    "singe_paged_attention_f16_d112_softcap_i32", "singe_paged_attention_f16_d112_softcap_i64",
+    "singe_paged_attention_f16_d112_i32_p16", "singe_paged_attention_f16_d112_i64_p16",
+    "singe_paged_attention_f16_d112_softcap_i32_p16", "singe_paged_attention_f16_d112_softcap_i64_p16",
+    "singe_rotary_paged_attention_bf16_d112_i32", "singe_rotary_paged_attention_bf16_d112_i64",
+    "singe_rotary_paged_attention_bf16_d112_i32_p16", "singe_rotary_paged_attention_bf16_d112_i64_p16",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -143,6 +219,8 @@ const char* const kPartNames[kPartCount] = {
     "cache_ops", "latent_attention", "latent_attention_mfma", "general_attention_f32", "general_attention_bf16",
     "general_attention_f16", "mfma_ceiling", "paged_decode_d64", "fmha_prefill_d64", "paged_attention_d64",
     "general_attention_f64", "hbm_stream", "fmha_prefill_d32", "paged_attention_d32", "fmha_prefill_d96", "paged_attention_d96",
+    "fmha_prefill_d16", "paged_attention_d16", "fmha_prefill_d48", "paged_attention_d48", "fmha_prefill_d80", "paged_attention_d80",
+    "fmha_prefill_d112", "paged_attention_d112",
 };
 
 namespace {
@@ -161,6 +239,7 @@ constexpr PartRun kPartRuns[] = {
     {17, 1},
     {18, 10}, {19, 28},           // the head_dim 32 builds: dense kernels with their merges, paged kernels
     {20, 10}, {21, 28},           // the head_dim 96 builds
+    {22, 10}, {23, 28}, {24, 10}, {25, 28}, {26, 10}, {27, 28}, {28, 10}, {29, 28},  // and those for 16, 48, 80, 112
 };
 constexpr int runs_total() {
     int total = 0;

@@ -57,11 +57,11 @@ enum KernelId : int {
     kDenseGeneralF64, kPagedGeneralF64 = kDenseGeneralF64 + 3,
     // the plain streaming read a decode kernel is priced against
     kHbmStreamRead = kPagedGeneralF64 + 3,
-    // the dense prefill and paged attention kernels built for head_dim 32 and for 96, each bank in the order of
-    // its head_dim 128 forms (eight dense kernels, their two merges, the paged kernels up to kSplitKReduce)
-    kPrefillD32, kPrefillCombineD32 = kPrefillD32 + 8, kPagedD32 = kPrefillCombineD32 + 2,
-    kPrefillD96 = kPagedD32 + (kSplitKReduce - kPagedAttentionI32), kPrefillCombineD96 = kPrefillD96 + 8, kPagedD96 = kPrefillCombineD96 + 2,
-    kKernelCount = kPagedD96 + (kSplitKReduce - kPagedAttentionI32)
+    // the dense prefill and paged attention kernels built for the other multiples of 16 (32, 96, 16, 48, 80, 112, in
+    // that order), each bank in the order of its head_dim 128 forms: eight dense kernels, their two merges, the
+    // paged kernels up to kSplitKReduce
+    kOtherHeadDims,
+    kKernelCount = kOtherHeadDims + 6 * (10 + (kSplitKReduce - kPagedAttentionI32))
 };
 
 // The head_dim 64 build of a matrix-core kernel named by its head_dim 128 id.
@@ -72,26 +72,34 @@ inline KernelId at_head_dim_64(KernelId kernel) {
 }
 
 // Whether the dense prefill and paged attention kernels have a matrix-core build for a head dimension.
-inline bool has_matrix_core_build(long long head_dim) { return head_dim == 128 || head_dim == 96 || head_dim == 64 || head_dim == 32; }
+inline bool has_matrix_core_build(long long head_dim) { return head_dim >= 16 && head_dim <= 128 && head_dim % 16 == 0; }
+
+// The bank of the builds for a head dimension other than 128 and 64.
+inline int other_head_dim_bank(long long head_dim) {
+    const int order = head_dim == 32 ? 0 : head_dim == 96 ? 1 : head_dim == 16 ? 2 : head_dim == 48 ? 3 : head_dim == 80 ? 4 : 5;
+    return kOtherHeadDims + order * (10 + (kSplitKReduce - kPagedAttentionI32));
+}
 
 // That build of a dense prefill or paged attention kernel named by its head_dim 128 id (decode kernels: 64 only).
 inline KernelId at_head_dim(KernelId kernel, long long head_dim) {
     if (head_dim == 128) return kernel;
     if (head_dim == 64) return at_head_dim_64(kernel);
     const bool dense = kernel >= kPrefillCausal && kernel < kPrefillF32D32;
-    if (head_dim == 32) return static_cast<KernelId>(dense ? kPrefillD32 + (kernel - kPrefillCausal) : kPagedD32 + (kernel - kPagedAttentionI32));
-    return static_cast<KernelId>(dense ? kPrefillD96 + (kernel - kPrefillCausal) : kPagedD96 + (kernel - kPagedAttentionI32));
+    const int bank = other_head_dim_bank(head_dim);
+    return static_cast<KernelId>(dense ? bank + (kernel - kPrefillCausal) : bank + 10 + (kernel - kPagedAttentionI32));
 }
 
 // The merge kernel of the dense kernels' key splits for a head dimension (+ 1 for f16).
 inline KernelId prefill_combine_at(long long head_dim) {
-    return head_dim == 128 ? kPrefillCombine : head_dim == 64 ? kPrefillCombineD64 : head_dim == 32 ? kPrefillCombineD32 : kPrefillCombineD96;
+    if (head_dim == 128) return kPrefillCombine;
+    if (head_dim == 64) return kPrefillCombineD64;
+    return static_cast<KernelId>(other_head_dim_bank(head_dim) + 8);
 }
 
 extern const char* const kKernelNames[kKernelCount];
 
 // Parts of the code object (one file each) and the part a kernel lives in.
-constexpr int kPartCount = 22;
+constexpr int kPartCount = 30;
 extern const char* const kPartNames[kPartCount];
 int kernel_part(int kernel);
 

@@ -98,7 +98,7 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
         // The fused form exists for the tensor-core kernel alone and without softcap here; the reference
         // plans the rotation and the attention apart for the rest (compiled/plan/group.rs:94-98), and so
         // does a caller of this library (singe_hip_rotary_cache_write, then singe_hip_paged_attention_*).
-        if (data_type != SINGE_HIP_BF16 || !has_matrix_core_build(p.head_dim))
+        if (data_type != SINGE_HIP_BF16 || !has_matrix_core_build(p.head_dim) || p.head_dim % 32 != 0)  // pairs are whole steps apart
             return fail(SINGE_HIP_UNSUPPORTED_WIDTH, "rotary_paged_attention", static_cast<uint64_t>(p.head_dim));
         if (p.has_softcap) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "rotary paged attention with a softcap");
     }

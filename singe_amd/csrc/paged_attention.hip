@@ -238,6 +238,8 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
                 scale = rsqrtf(squares / static_cast<float>(kHeadDim) + a.query_eps);
             }
             const size_t token = static_cast<size_t>(query_start) + my_token;
+            // (Pairs are dims i and i + head_dim / 2, whole steps apart at multiples of 32; the launcher sends the other
+            // head dimensions to the two-step form.)
             constexpr int kPairs = kHeadDim / 2, kHalfSteps = kSteps / 2;
 #pragma unroll
             for (int s = 0; s < kHalfSteps; ++s) {
@@ -512,7 +514,8 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         for (int db = 0; db < kDimBlocks; ++db)
 #pragma unroll
             for (int quad = 0; quad < 4; ++quad)
-                *reinterpret_cast<float4*>(row + 32 * db + 8 * quad + 4 * hi) =
+                if (32 * db + 8 * quad < kHeadDim)
+                    *reinterpret_cast<float4*>(row + 32 * db + 8 * quad + 4 * hi) =
                     make_float4(state.out[db][4 * quad + 0] * inverse, state.out[db][4 * quad + 1] * inverse,
                                 state.out[db][4 * quad + 2] * inverse, state.out[db][4 * quad + 3] * inverse);
         if (hi == 0) a.partial_lse[slot] = sum > 0.0f ? state.reference + fast_log2(sum) : -INFINITY;
@@ -523,6 +526,7 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         for (int db = 0; db < kDimBlocks; ++db)
 #pragma unroll
             for (int quad = 0; quad < 4; ++quad) {
+                if (32 * db + 8 * quad >= kHeadDim) continue;
                 uint2 packed_bits;
                 packed_bits.x = pack_pair(half, state.out[db][4 * quad + 0] * inverse, state.out[db][4 * quad + 1] * inverse);
                 packed_bits.y = pack_pair(half, state.out[db][4 * quad + 2] * inverse, state.out[db][4 * quad + 3] * inverse);

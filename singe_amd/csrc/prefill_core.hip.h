@@ -23,15 +23,17 @@
 
 namespace prefill {
 
-// The head dimension a build of these kernels is for: the sources are compiled once per value (128, and 32, 64, 96
-// with -DSINGE_HEAD_DIM=...), each into its own part of the code object.
+// The head dimension a build of these kernels is for: the sources are compiled once per value (128, and the other
+// multiples of 16 with -DSINGE_HEAD_DIM=...), each into its own part of the code object.
 #ifndef SINGE_HEAD_DIM
 #define SINGE_HEAD_DIM 128
 #endif
 constexpr int kHeadDim = SINGE_HEAD_DIM;
-static_assert(kHeadDim % 32 == 0 && kHeadDim >= 32 && kHeadDim <= 128, "head dimensions the matrix-core kernels are built for");
+static_assert(kHeadDim % 16 == 0 && kHeadDim >= 16 && kHeadDim <= 128, "head dimensions the matrix-core kernels are built for");
 constexpr int kSteps = kHeadDim / 16;      // products per 32-key block of scores: sixteen dims each
-constexpr int kDimBlocks = kHeadDim / 32;  // 32-dim blocks of O^T
+constexpr int kDimBlocks = (kHeadDim + 31) / 32;  // 32-dim blocks of O^T; at an odd multiple of 16 the last one is half
+                                                 // real: its other sixteen dims multiply whatever the LDS rows hold past
+                                                 // a key's last chunk, stay in registers of their own and are never stored
 constexpr int kQueryTile = 128;       // query rows per workgroup
 constexpr int kKeyTile = 64;          // keys per LDS stage
 

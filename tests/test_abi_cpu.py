@@ -151,6 +151,7 @@ def test_rotary_paged_attention_validation():
     assert call(None) == 6                                       # no rotation attributes
     assert call(_native.QueryRotationC(7, 0, 0.0)) == 9          # unknown table type
     assert call(good, head_dim=80) == 5                          # the fused form takes head dimensions 32, 64, 96 and 128
+    assert call(good, head_dim=72) == 5
     assert call(good, has_softcap=1, softcap=5.0) == 8
     assert call(good, cos=None) == 6
     assert call(good, tokens=0) == 0
@@ -167,8 +168,9 @@ def test_paged_attention_scratch_query_needs_no_device():
     try:
         assert wanted() == 4 * 32 * 32 * 129 * 4     # shares x rows x (128 values + a log-sum-exp) of f32
         assert wanted(head_dim=64) == 4 * 32 * 32 * 65 * 4   # the head_dim 64 build splits the same way
-        assert wanted(head_dim=96) == 4 * 32 * 32 * 97 * 4   # so do the builds for 96 and 32
-        assert wanted(head_dim=80) == 0               # the general kernel does not split
+        assert wanted(head_dim=96) == 4 * 32 * 32 * 97 * 4   # so do the builds for the other multiples of 16
+        assert wanted(head_dim=80) == 4 * 32 * 32 * 81 * 4
+        assert wanted(head_dim=72) == 0               # the general kernel does not split
     finally:
         lib.singe_hip_set_paged_attention_splits(0)
     assert lib.singe_hip_paged_attention_scratch_bytes(None) == 0

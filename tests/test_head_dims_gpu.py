@@ -4,8 +4,9 @@ The reference's own kernels take head_dim 4 to 64 for block-table decode
 (singe-kernel/src/cuda/cutile/attention/paged.rs:799-810), 16 / 32 / 64 / 128 for the dense prefill's matrix path
 (singe-kernel/src/cuda/attention/fmha.rs:752-755) and every multiple of 16 up to 128 for the tensor-core paged and dense
 kernels (singe/src/backend/cuda/kernel_plan/source/paged_attention.rs:586-592); two of the three shapes of its own
-paged test are head_dim 64 (kernel_plan/source/tests.rs:830-966).  Here head_dim 32, 64 and 96 run on builds of the
-matrix-core kernels for those widths (decode: 64 only), the other widths on the one-wave-per-row kernels.  Tolerances as at head_dim 128: bf16 max-abs
+paged test are head_dim 64 (kernel_plan/source/tests.rs:830-966).  Here every multiple of 16 up to 128 runs on a build
+of the matrix-core dense and paged kernels for that width (decode: 64 and 128), the other widths on the
+one-wave-per-row kernels.  Tolerances as at head_dim 128: bf16 max-abs
 2e-2 / mean-abs 2e-3, log-sum-exp 2e-3."""
 import numpy as np
 import pytest
@@ -25,7 +26,8 @@ pytestmark = pytest.mark.gpu
 @pytest.mark.parametrize("options", paged.OPTIONS)
 @pytest.mark.parametrize("heads,kv_heads,dim,page_size", [(8, 2, 64, 1), (4, 4, 64, 7), (8, 1, 64, 16), (64, 8, 64, 16), (6, 3, 64, 48),
                                                           (8, 2, 32, 1), (4, 4, 32, 7), (16, 2, 32, 16), (8, 2, 96, 1), (4, 4, 96, 7),
-                                                          (16, 2, 96, 16), (6, 3, 96, 48)])
+                                                          (16, 2, 96, 16), (6, 3, 96, 48), (8, 2, 16, 1), (8, 2, 16, 16), (4, 4, 48, 7),
+                                                          (16, 2, 48, 16), (8, 2, 80, 16), (6, 3, 80, 5), (8, 2, 112, 16), (4, 1, 112, 3)])
 def test_paged_attention_at_the_matrix_core_head_dims_matches_oracle(heads, kv_heads, dim, page_size, options):
     # the reference's recipe: decode, full prefill, chunked prefill, no keys (tests.rs:830-889), plus more queries than keys
     sequences = [(1, 150), (70, 70), (20, 90), (3, 0), (9, 4), (130, 300)]
@@ -38,7 +40,7 @@ def test_paged_attention_at_other_head_dims_matches_oracle(dim, options):
     paged.run_case([(1, 150), (70, 70), (20, 90), (3, 0)], 8, 2, 16, options, seed=dim, dim=dim)
 
 
-@pytest.mark.parametrize("dim", [64, 32, 96])
+@pytest.mark.parametrize("dim", [64, 32, 96, 16, 48, 80, 112])
 @pytest.mark.parametrize("splits", [2, 7, 16])
 def test_paged_attention_key_splits_at_other_head_dims(splits, dim):
     _native.lib().singe_hip_set_paged_attention_splits(splits)
@@ -51,7 +53,7 @@ def test_paged_attention_key_splits_at_other_head_dims(splits, dim):
 
 
 @pytest.mark.parametrize("causal", [True, False])
-@pytest.mark.parametrize("dim", [16, 32, 64, 96, 80])
+@pytest.mark.parametrize("dim", [16, 32, 48, 64, 80, 96, 112, 72])
 @pytest.mark.parametrize("batch,query_len,key_len,heads,kv_heads", [
     (1, 128, 128, 1, 1), (2, 256, 256, 4, 2), (1, 100, 100, 3, 1), (1, 1, 1, 1, 1), (1, 33, 97, 2, 1), (1, 300, 129, 2, 2),
     (1, 640, 1000, 4, 1),
@@ -78,7 +80,7 @@ def test_dense_prefill_f16_at_head_dim_64():
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("dim", [16, 32, 64, 96])
+@pytest.mark.parametrize("dim", [16, 32, 48, 64, 80, 96, 112, 40])
 @pytest.mark.parametrize("causal", [True, False])
 def test_block_table_prefill_at_other_head_dims(dim, causal, dtype):
     table_prefill.run_case([(130, 130), (1, 1), (33, 200), (64, 10)], 8, 2, 16, causal, seed=dim, dtype=dtype, dim=dim)
