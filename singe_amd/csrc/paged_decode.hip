@@ -54,6 +54,7 @@ constexpr int kDim = SINGE_HEAD_DIM;
 static_assert(kDim == 64 || kDim == 128, "head dimensions the decode kernels are built for");
 constexpr int kDimSteps = kDim / 32;  // score products per 16 keys
 constexpr int kTile = 32;
+constexpr float kReferenceLag = 6.0f;  // doublings a softmax reference point may lag the largest score seen
 
 // One 32-key tile in registers, bf16 cache.  K and V are fetched the same way, as whole rows (16 lanes x 16 bytes, the
 // coalesced layout: fetched in the matrix operand's layout, where neighbouring lanes read different rows, K alone
@@ -487,9 +488,21 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
                 p[4 + i] = (tile.live >> (4 + i)) & 1u ? second : -INFINITY;
             }
             float largest = fmaxf(fmaxf(fmaxf(p[0], p[1]), fmaxf(p[2], p[3])), fmaxf(fmaxf(p[4], p[5]), fmaxf(p[6], p[7])));
-            largest = fmaxf(across_groups_max(largest), wide_max);
-            const float base = largest == -INFINITY ? 0.0f : largest;
-            const float rescale = fast_exp2(wide_max - base);
+            largest = across_groups_max(largest);
+            // The reference point of a head may lag its largest score by kReferenceLag doublings: the weights then
+            // reach 2^kReferenceLag at most, and the 32 accumulator registers are rescaled on the few tiles where some
+            // head's scores outgrow that, not on every tile.
+            if (__any(largest > wide_max + kReferenceLag || (wide_max == -INFINITY && largest != -INFINITY))) {
+                const float moved = fmaxf(wide_max, largest);
+                const float rescale = fast_exp2(wide_max - (moved == -INFINITY ? 0.0f : moved));
+                wide_sum *= rescale;
+#pragma unroll
+                for (int db = 0; db < 8; ++db)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) wide_acc[db][r] *= rescale;
+                wide_max = moved;
+            }
+            const float base = wide_max == -INFINITY ? 0.0f : wide_max;
             float total = 0.0f;
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
@@ -497,8 +510,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
                 total += p[i];
                 if constexpr (!EXACT) p[i] *= tile.row_value_scale[i >> 2][i & 3];
             }
-            wide_sum = wide_sum * rescale + total;
-            wide_max = largest;
+            wide_sum += total;
             const uint4 weights = make_uint4(bf16_pair(p[0], p[1]), bf16_pair(p[2], p[3]), bf16_pair(p[4], p[5]), bf16_pair(p[6], p[7]));
             // O^T[dim, head] += V^T . P^T: k-slots 8 g + j of the MFMA are keys 4 g + j (j < 4) and
             // 16 + 4 g + j - 4, which is how the two transposing reads of a 16-lane group deliver them.
@@ -511,8 +523,6 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
                 const v4i16_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(patch + 32 * db));
                 const v4i16_t high = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(patch + 16 * kStagedRowBytes + 32 * db));
                 const v8i16_t both = __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) wide_acc[db][r] *= rescale;
                 wide_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, both), __builtin_bit_cast(bf16x8_t, weights),
                                                                   wide_acc[db], 0, 0, 0);
             }
