@@ -36,6 +36,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 POOLS = 3
+DECODE_BYTES = 305_940_888  # algorithmic bytes of the headline decode workload (its lengths sum to 74 560 keys)
 WARMUP_SECONDS = 0.3
 MIN_SAMPLES = 30
 
@@ -46,18 +47,18 @@ MIN_SAMPLES = 30
 # profile summary they come from.
 FETCH_UNIT_BYTES, WRITE_UNIT_BYTES = 2048, 1024
 COUNTER_TRAFFIC = {
-    "decode": {"kernel": "singe_paged_decode_bf16_d128_g1_b16", "FETCH_SIZE": 145725, "WRITE_SIZE": 4550,
+    "decode": {"kernel": "singe_paged_decode_bf16_d128_g1_b16", "FETCH_SIZE": 150137, "WRITE_SIZE": 4238,
                "source": "profiles/hbm_traffic_counters.md"},
-    "prefill": {"kernel": "singe_fmha_prefill_bf16_d128_causal", "FETCH_SIZE": 319301, "WRITE_SIZE": 131415,
+    "prefill": {"kernel": "singe_fmha_prefill_bf16_d128_causal", "FETCH_SIZE": 318579, "WRITE_SIZE": 131440,
                 "source": "profiles/hbm_traffic_counters.md"},
-    "chunked_prefill": {"kernel": "singe_paged_attention_bf16_d128_i32_p16", "FETCH_SIZE": 183449, "WRITE_SIZE": 66568,
+    "chunked_prefill": {"kernel": "singe_paged_attention_bf16_d128_i32_p16", "FETCH_SIZE": 182479, "WRITE_SIZE": 66566,
                         "source": "profiles/hbm_traffic_counters.md"},
-    "fp8_decode": {"kernel": "singe_paged_decode_f8kv_wide_d128_b16", "FETCH_SIZE": 2129880, "WRITE_SIZE": 8256,
+    "fp8_decode": {"kernel": "singe_paged_decode_f8kv_wide_d128_b16", "FETCH_SIZE": 2129860, "WRITE_SIZE": 8256,
                    "source": "profiles/hbm_traffic_counters.md"},
-    "latent_decode": {"kernel": "singe_paged_mla_attention_bf16_l512_p64", "FETCH_SIZE": 608523, "WRITE_SIZE": 32997,
+    "latent_decode": {"kernel": "singe_paged_mla_attention_bf16_l512_p64", "FETCH_SIZE": 608523, "WRITE_SIZE": 32999,
                       "source": "profiles/hbm_traffic_counters.md"},
-    "latent_chunked_prefill": {"kernel": "singe_paged_mla_attention_bf16_l512_p64", "FETCH_SIZE": 869183,
-                               "WRITE_SIZE": 526765, "source": "profiles/hbm_traffic_counters.md"},
+    "latent_chunked_prefill": {"kernel": "singe_paged_mla_attention_bf16_l512_p64", "FETCH_SIZE": 868387,
+                               "WRITE_SIZE": 526766, "source": "profiles/hbm_traffic_counters.md"},
 }
 
 
@@ -302,10 +303,11 @@ def prefill_section(with_cpu=True, dim=128, key="prefill"):
 
     from singe_amd.kernel import attention as A
 
+    from singe_amd import synthetic
+
     batch, seq, heads = 4, 4096, 32
-    gen = torch.Generator(device="cuda")
-    gen.manual_seed(0x51A6E + 3)
-    q, k, v = (torch.randn((batch, seq, heads, dim), generator=gen, device="cuda").to(torch.bfloat16) for _ in range(3))
+    q, k, v = (synthetic.portable_normal(f"{key}.{tensor}", (batch, seq, heads, dim), torch.bfloat16)
+               for tensor in ("query", "key", "value"))
     out = torch.empty_like(q)
     scale = float(dim) ** -0.5
     config = A.FmhaPrefillConfig.contiguous(batch, seq, seq, heads, heads, dim, scale, True)
@@ -338,7 +340,7 @@ def chunked_prefill_section(with_cpu=True):
 
     from singe_amd import _native, neural, synthetic
 
-    work = synthetic.chunked_prefill_workload()
+    work = synthetic.chunked_prefill_workload(portable=True)
     index = lambda values: torch.from_numpy(np.asarray(values, dtype=np.int32)).cuda()
     paging = neural.Paging(index(work.query_offsets), index(work.page_offsets), index(work.pages), index(work.last_page_lengths))
     options = neural.AttentionOptions(causal=True)
@@ -393,7 +395,7 @@ def latent_section():
     import numpy as np
     import torch
 
-    from singe_amd import neural
+    from singe_amd import neural, synthetic
 
     def case(sequences, group, heads=128, page=64):
         query_offsets, page_offsets, last, table, pages = [0], [0], [], [], 0
@@ -404,13 +406,13 @@ def latent_section():
             last.append(keys - (count - 1) * page)
             table += list(range(pages, pages + count))
             pages += count
-        order = np.random.default_rng(7).permutation(pages)
+        source = synthetic._PortableSource(synthetic.BASE_SEED, "cuda", f"latent_{len(sequences)}x{sequences[0][0]}")
+        order = source.permutation("pages", pages)
         table = [int(order[entry]) for entry in table]
-        gen = torch.Generator(device="cuda")
-        gen.manual_seed(11)
-        rand = lambda *shape: torch.randn(shape, generator=gen, device="cuda").to(torch.bfloat16)
         tokens = query_offsets[-1]
-        operands = (rand(tokens, heads, 512), rand(tokens, heads, 64), rand(pages, page, 512), rand(pages, page, 64))
+        operands = tuple(source.normal(tensor, shape).to(torch.bfloat16) for tensor, shape in (
+            ("latent_queries", (tokens, heads, 512)), ("positional_queries", (tokens, heads, 64)),
+            ("latent_cache", (pages, page, 512)), ("positional_cache", (pages, page, 64))))
         index = lambda values: torch.tensor(values, dtype=torch.int32, device="cuda")
         paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
         options = neural.AttentionOptions(causal=True)
@@ -454,10 +456,10 @@ def dense_f32_section(with_cpu=True):
 
     from singe_amd.kernel import attention as A
 
+    from singe_amd import synthetic
+
     batch, heads, seq, dim = 1, 8, 512, 64
-    gen = torch.Generator(device="cuda")
-    gen.manual_seed(0x51A6E + 1)
-    q, k, v = (torch.randn((batch, heads, seq, dim), generator=gen, device="cuda") for _ in range(3))
+    q, k, v = (synthetic.portable_normal(f"dense_f32.{tensor}", (batch, heads, seq, dim)) for tensor in ("query", "key", "value"))
     out = torch.empty_like(q)
     config = A.SoftcappedWindowAttentionConfig(A.bhsd_config(batch, heads, heads, seq, seq, dim, 0.125, True), 0, None)
     stats = measure(lambda: A.softcapped_window_attention_f32(None, out, q, k, v, config), 10)
@@ -482,7 +484,7 @@ def fp8_decode_section(with_cpu=True):
     from singe_amd import synthetic
     from singe_amd.kernel import attention as A
 
-    work = synthetic.paged_decode_fp8_workload()
+    work = synthetic.paged_decode_fp8_workload(portable=True)
     config = A.PagedKvDecodeAttentionConfig.contiguous(work.batch, work.heads, work.kv_heads, work.head_dim,
                                                        work.block_size, work.physical_blocks,
                                                        work.block_table_batch_stride, work.scale)
@@ -529,7 +531,7 @@ def head_dim_64_section():
     from singe_amd.kernel import attention as A
 
     prefill = prefill_section(with_cpu=False, dim=64, key="prefill_d64")
-    work = synthetic.paged_decode_workload(head_dim=64)
+    work = synthetic.paged_decode_workload(head_dim=64, portable=True, name="paged_decode_d64")
     config = A.PagedKvDecodeAttentionConfig.contiguous(work.batch, work.heads, work.kv_heads, work.head_dim,
                                                        work.block_size, work.physical_blocks,
                                                        work.block_table_batch_stride, work.scale)
@@ -560,10 +562,10 @@ def mfma_ceiling_section():
     from singe_amd import _native
 
     workgroups, iterations = 512, 4000
-    gen = torch.Generator(device="cuda")
-    gen.manual_seed(0x51A6E + 9)
+    from singe_amd import synthetic
+
     operands = {"zeros": torch.zeros(1 << 22, device="cuda", dtype=torch.bfloat16),
-                "normal": torch.randn(1 << 22, generator=gen, device="cuda").to(torch.bfloat16)}
+                "normal": synthetic.portable_normal("mfma_ceiling.operands", (1 << 22,), torch.bfloat16)}
     out = torch.empty(workgroups * 256, device="cuda", dtype=torch.float32)
     handle = int(torch.cuda.current_stream().cuda_stream)
     flops = workgroups * 4 * iterations * 32 * 32768
@@ -581,7 +583,7 @@ def mfma_ceiling_section():
 
 def hbm_ceiling_section():
     """What the memory system delivers to a kernel that only reads: one workgroup of 512 lanes per compute unit (the
-    decode kernels' launch shape) streams buffers of the two decode workloads' sizes, 297 MB and 4.3 GB, once per
+    decode kernels' launch shape) streams buffers of the two decode workloads' sizes, 306 MB and 4.3 GB, once per
     launch with non-temporal loads; three buffers are rotated as the decode section rotates its KV pools."""
     import torch
 
@@ -591,7 +593,7 @@ def hbm_ceiling_section():
     out = torch.empty(workgroups * 512, device="cuda", dtype=torch.int32)
     handle = int(torch.cuda.current_stream().cuda_stream)
     result = {"kernel": "singe_hbm_stream_read", "workgroups": workgroups, "peak": HBM_PEAK_GBPS, "unit": "GB/s"}
-    for name, nbytes, pools, group in (("decode_sized", 296_748_908 // 16 * 16, 3, 6), ("fp8_decode_sized", 4_305_977_600, 2, 2)):
+    for name, nbytes, pools, group in (("decode_sized", DECODE_BYTES // 16 * 16, 3, 6), ("fp8_decode_sized", 4_305_977_600, 2, 2)):
         buffers = [torch.randint(0, 255, (nbytes,), device="cuda", dtype=torch.uint8) for _ in range(pools)]
         turn = [0]
 
@@ -619,10 +621,10 @@ def decode_section(args, with_cpu):
 
     if args.workers:
         _native.lib().singe_hip_set_decode_workers(args.workers)
-    work = synthetic.paged_decode_workload()
+    work = synthetic.paged_decode_workload(portable=True)
     pools = [(work.key_cache, work.value_cache)]
     for extra in range(1, POOLS):
-        other = synthetic.paged_decode_workload(seed=synthetic.BASE_SEED + 97 * extra)
+        other = synthetic.paged_decode_workload(portable=True, name=f"paged_decode_pool{extra}")
         pools.append((other.key_cache, other.value_cache))
         del other
     config = A.PagedKvDecodeAttentionConfig.contiguous(work.batch, work.heads, work.kv_heads, work.head_dim,
@@ -659,13 +661,14 @@ def decode_section(args, with_cpu):
     whole = measure(step, 6)               # the op under events: split + reduce
     kernel = measure(lambda: step(1), 6)   # the dominant kernel alone
     bytes_per_step = work.algorithmic_bytes()
+    assert bytes_per_step == DECODE_BYTES, (bytes_per_step, DECODE_BYTES)
     value = bytes_per_step / (ms_per_step * 1e-3) / 1e9
     achieved = bytes_per_step / (kernel["mean_ms"] * 1e-3) / 1e9
     counted, source = traffic("decode") if not args.workers else (None, None)
     result = {
         "metric": "decode attn GB/s", "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "warmup_steps_run": warm_steps, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
-        "data": "synthetic",
+        "data": "synthetic (splitmix64 counter streams, Box-Muller N(0,1), base seed 0x51A6E; singe_amd/synthetic.py portable=True)",
         "config": {
             "workload": "paged decode: batch 32, 32q/8kv heads, head_dim 128, bf16, block 16, "
                         "ctx U[512,4096], 16384-block pool (BASELINE config 2)",

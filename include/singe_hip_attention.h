@@ -997,6 +997,20 @@ SINGE_HIP_API int32_t singe_hip_hbm_stream_read(void* stream, const void* data, 
 SINGE_HIP_API int32_t singe_hip_mfma_ceiling(void* stream, const void* operands, size_t operand_bytes, float* out,
                                              size_t out_len, uint32_t workgroups, uint32_t iterations, int32_t f16);
 
+/* Seeded benchmark inputs made on the host, the same for every caller whatever its language (no counterpart among the
+ * reference's attention launchers; the stream is the splitmix64 sequence of its plan search,
+ * singe/src/backend/cuda/tuning/plan.rs:527-543, read as a counter).  Word i of a stream is
+ * mix(seed + (i + 1) * 0x9E3779B97F4A7C15).  Normal values: word i gives elements 2 i and 2 i + 1 by Box-Muller on
+ * u1 = ((word >> 40) + 1) / 2^24 and u2 = ((word >> 16) & 0xFFFFFF) / 2^24, computed in double and rounded to float.
+ * Integers: low + ((word >> 32) * span >> 32), span < 2^32.  Permutation: Fisher-Yates from the back, step k drawing
+ * from [0, count - 1 - k] with word k.  A tensor's seed is base_seed ^ FNV-1a-64(name).  Host memory only. */
+SINGE_HIP_API uint64_t singe_hip_synthetic_seed(uint64_t base_seed, const char* tensor_name);
+SINGE_HIP_API uint64_t singe_hip_synthetic_word(uint64_t seed, uint64_t index);
+SINGE_HIP_API void singe_hip_synthetic_normal_f32(uint64_t seed, uint64_t first_element, float* out, size_t count, uint32_t threads);
+SINGE_HIP_API void singe_hip_synthetic_integers(uint64_t seed, uint64_t first_index, int64_t low, uint64_t span, int64_t* out,
+                                                size_t count);
+SINGE_HIP_API void singe_hip_synthetic_permutation(uint64_t seed, int64_t* out, size_t count);
+
 #ifdef __cplusplus
 }
 #endif

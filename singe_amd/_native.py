@@ -181,6 +181,17 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_hbm_stream_read.restype = i32
     handle.singe_hip_mfma_ceiling.argtypes = [c_void, c_void, c_size, c_void, c_size, ctypes.c_uint32, ctypes.c_uint32, i32]
     handle.singe_hip_mfma_ceiling.restype = i32
+    u64 = ctypes.c_uint64
+    handle.singe_hip_synthetic_seed.argtypes = [u64, ctypes.c_char_p]
+    handle.singe_hip_synthetic_seed.restype = u64
+    handle.singe_hip_synthetic_word.argtypes = [u64, u64]
+    handle.singe_hip_synthetic_word.restype = u64
+    handle.singe_hip_synthetic_normal_f32.argtypes = [u64, u64, c_void, c_size, ctypes.c_uint32]
+    handle.singe_hip_synthetic_normal_f32.restype = None
+    handle.singe_hip_synthetic_integers.argtypes = [u64, u64, ctypes.c_int64, u64, c_void, c_size]
+    handle.singe_hip_synthetic_integers.restype = None
+    handle.singe_hip_synthetic_permutation.argtypes = [u64, c_void, c_size]
+    handle.singe_hip_synthetic_permutation.restype = None
     handle.singe_hip_prepare.argtypes = [ctypes.POINTER(i32)]
     handle.singe_hip_prepare.restype = i32
     cfg = ctypes.POINTER(PagedKvDecodeAttentionConfigC)
