@@ -136,6 +136,7 @@ struct PagedAttentionArgs {
     uint32_t row_tiles;             // ceil(groups * tokens / 128): row tiles per (sequence, kv head); with `compact`,
                                     // a bound on the row tiles of all sequences together
     uint32_t compact = 0;           // workgroups find their (sequence, row tile) by a prefix sum over the sequences
+    uint32_t longest_first = 0;     // with `compact` and at most 64 sequences: the list takes the sequences longest first
     uint32_t causal;
     int32_t page_shift;             // log2(page_size) when it is a power of two, else -1
     float scale_log2e;              // scale * log2(e)

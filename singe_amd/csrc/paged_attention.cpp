@@ -40,6 +40,7 @@ struct Scratch {
 // floor(tokens * groups / 128) + sequences.
 struct RowTileGrid {
     uint32_t compact;
+    uint32_t longest_first;  // the compact list takes the sequences longest first (see `locate`)
     uint64_t row_tiles;   // the kernel argument
     uint64_t blocks;      // workgroups without key splits
 };
@@ -47,6 +48,7 @@ struct RowTileGrid {
 RowTileGrid grid_of(uint64_t tokens, uint64_t sequences, uint64_t groups, uint64_t kv_heads = 1) {
     RowTileGrid grid;
     const uint64_t longest = (groups * tokens + 127) / 128;
+    grid.longest_first = 0;
     if (longest <= 1) {
         grid.compact = 0;
         grid.row_tiles = longest;
@@ -54,6 +56,9 @@ RowTileGrid grid_of(uint64_t tokens, uint64_t sequences, uint64_t groups, uint64
     } else {
         grid.compact = 1;
         grid.row_tiles = groups * tokens / 128 + sequences;
+        // Longest sequences first where sequences have row tiles to spare (chunks of a prefill): their workgroups run
+        // for hundreds of microseconds and the order decides how full the chip's last round is.
+        grid.longest_first = sequences <= 64 && groups * tokens / 128 >= 2 * sequences ? 1u : 0u;
         const uint64_t bands = (grid.row_tiles + 31) / 32;
         grid.blocks = (kv_heads * bands + 7) / 8 * 8 * 32;
     }
@@ -165,6 +170,7 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
     if (tiling.row_tiles > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many row tiles");
     args.row_tiles = static_cast<uint32_t>(tiling.row_tiles);
     args.compact = tiling.compact;
+    args.longest_first = tiling.longest_first;
     args.causal = p.causal ? 1u : 0u;
     args.page_shift = -1;
     for (int shift = 0; shift < 31; ++shift)
@@ -394,6 +400,7 @@ int32_t paged_kv_prefill(
     if (tiling.row_tiles > 0xffffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many row tiles");
     args.row_tiles = static_cast<uint32_t>(tiling.row_tiles);
     args.compact = tiling.compact;
+    args.longest_first = tiling.longest_first;
     args.causal = c.causal ? 1u : 0u;
     args.page_shift = -1;
     for (int shift = 0; shift < 31; ++shift)

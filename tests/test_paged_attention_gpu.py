@@ -88,6 +88,25 @@ def test_many_ragged_sequences_find_their_row_tiles(heads, kv_heads, page_size, 
         _native.lib().singe_hip_set_paged_attention_splits(0)
 
 
+@pytest.mark.parametrize("index_dtype", [torch.int32, torch.int64])
+@pytest.mark.parametrize("heads,kv_heads,page_size,splits", [(8, 2, 16, 0), (16, 1, 8, 2), (4, 4, 3, 0)])
+def test_up_to_64_sequences_with_tiles_to_spare_are_taken_longest_first(heads, kv_heads, page_size, splits, index_dtype):
+    # few sequences with several row tiles each: the grid lists them by pages held, longest first, ties by index;
+    # equal lengths, sequences without queries or without keys, and one much longer than the rest
+    groups = heads // kv_heads
+    base = 128 // groups  # queries of one row tile
+    sequences = [(3 * base, 700), (3 * base, 700), (0, 300), (5 * base + 1, 5 * base + 1), (2 * base, 0), (base, 2000),
+                 (4 * base, 700), (1, 64), (6 * base, 1100), (2 * base + 7, 333)]
+    assert sum(q for q, _ in sequences) * groups // 128 >= 2 * len(sequences)
+    _native.lib().singe_hip_set_paged_attention_splits(splits)
+    try:
+        run_case(sequences, heads, kv_heads, page_size, neural.AttentionOptions(causal=True), index_dtype=index_dtype, seed=heads + 9)
+        run_case(sequences[::-1], heads, kv_heads, page_size, neural.AttentionOptions(causal=True, window=90), index_dtype=index_dtype, seed=2)
+        run_case(sequences * 6, heads, kv_heads, page_size, neural.AttentionOptions(causal=True), index_dtype=index_dtype, seed=5)  # 60 of them
+    finally:
+        _native.lib().singe_hip_set_paged_attention_splits(0)
+
+
 @pytest.mark.parametrize("options", [neural.AttentionOptions(causal=True, softcap=-4.0), neural.AttentionOptions(scale=-0.06, softcap=5.0),
                                      neural.AttentionOptions(scale=-0.06, softcap=-5.0, causal=True, window=50)])
 @pytest.mark.parametrize("heads,kv_heads,page_size", [(8, 2, 16), (4, 4, 7)])
