@@ -46,7 +46,7 @@ constexpr int kPositionalTileBytes = kKeys * kPositionalRowBytes;  // 4 KiB
 constexpr int kStageBytes = kLatentTileBytes + kPositionalTileBytes;
 // The first steps of Q^T live in LDS, one 16-byte slot per (step, lane) that only its own lane touches, to leave the
 // wave registers for the operands in flight.
-constexpr int kParkedSteps = 10;
+constexpr int kParkedSteps = 8;
 constexpr int kParkedBytes = kParkedSteps * 1024 * kWaves;
 constexpr int kLdsBytes = 2 * kStageBytes + kParkedBytes;
 constexpr int kLatentSteps = kLatent / 32, kSteps = (kLatent + kPositional) / 32;
@@ -73,6 +73,20 @@ SINGE_DEVICE void load_to_lds(const unsigned char* source, unsigned char* dest) 
     unsigned int kept;
     asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0"
                  : "=&s"(kept) : "s"(base), "v"(source) : "memory");
+}
+
+// The same with the address in two parts, a base every lane shares (kept in scalar registers) and a 32-bit offset per
+// lane: a wave-uniform row costs no 64-bit address per lane, in registers or in arithmetic.
+SINGE_DEVICE void load_to_lds(const unsigned char* shared_base, unsigned int lane_offset, unsigned char* dest) {
+    const unsigned int base = __builtin_amdgcn_readfirstlane(static_cast<unsigned int>(reinterpret_cast<__UINTPTR_TYPE__>((lds_words_t)dest)));
+    const unsigned long long bits = reinterpret_cast<unsigned long long>(shared_base);
+    // (the built-in returns an int: through unsigned int first, or a low word with its top bit set would fill the high word)
+    const unsigned int low_word = __builtin_amdgcn_readfirstlane(static_cast<unsigned int>(bits));
+    const unsigned int high_word = __builtin_amdgcn_readfirstlane(static_cast<unsigned int>(bits >> 32));
+    const unsigned long long scalar = static_cast<unsigned long long>(low_word) | (static_cast<unsigned long long>(high_word) << 32);
+    unsigned int kept;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b32 m0, %0"
+                 : "=&s"(kept) : "s"(base), "v"(lane_offset), "s"(scalar) : "memory");
 }
 
 // Where the chunk permutation of a latent row puts things: see the header comment.
@@ -243,6 +257,9 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
     // A key behind a bad page id is read as zeros; the status word tells the caller.
     // In pieces, so that a tile's iteration can spread them between its first score products: piece 0-3 one latent
     // row each, piece 4 the positional parts.
+    const unsigned int positional_chunk = 16u * ((lane & 7u) ^ (positional_row & 7u));
+    // Rows w and w + 16 of a tile permute their chunks alike, and so do w + 8 and w + 24.
+    const unsigned int lane_chunk[2] = {16u * (lane ^ chunk_flip(wave & 15u)), 16u * (lane ^ chunk_flip((wave + 8u) & 15u))};
     auto issue_piece = [&](int piece, unsigned int tile, const TilePages<FORM>& pages, unsigned char* __restrict__ stage)
                            __attribute__((always_inline)) {
         if (piece < 4) {
@@ -252,8 +269,7 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
             unsigned char* dest = stage + row * kLatentRowBytes;
             if (page < static_cast<unsigned long long>(a.cache_pages)) {
                 const size_t slot = static_cast<size_t>(page) * a.page_size + place_of(key_of(tile, row));
-                const unsigned char* source = latent_cache + slot * kLatentRowBytes + 16u * (lane ^ chunk_flip(row & 15u));
-                load_to_lds(source, dest);
+                load_to_lds(latent_cache + slot * kLatentRowBytes, lane_chunk[i & 1], dest);
             } else {
                 if (lane == 0) report_index_error(a.status);
                 *reinterpret_cast<uint4*>(dest + 16u * lane) = make_uint4(0, 0, 0, 0);
@@ -263,7 +279,11 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
             unsigned char* dest = stage + kLatentTileBytes + 8u * wave * kPositionalRowBytes;
             if (page < static_cast<unsigned long long>(a.cache_pages)) {
                 const size_t slot = static_cast<size_t>(page) * a.page_size + place_of(key_of(tile, positional_row));
-                const unsigned char* source = positional_cache + slot * kPositionalRowBytes + 16u * ((lane & 7u) ^ (positional_row & 7u));
+                // (the lane's chunk is made opaque here: added to the cache's address ahead of the loop it would be a
+                // 64-bit value per lane to keep)
+                unsigned int chunk = positional_chunk;
+                asm volatile("" : "+v"(chunk));
+                const unsigned char* source = positional_cache + (slot * kPositionalRowBytes + chunk);
                 load_to_lds(source, dest);
             } else {
                 report_index_error(a.status);
