@@ -11,7 +11,7 @@ Prints one JSON line: whole-job GB/s of algorithmic bytes over exactly --steps s
 steps, the roofline of the dominant kernel and the CPU oracle timed on a bounded sample.  The same line
 carries one object per further benchmark configuration ("prefill", "chunked_prefill", "fp8_decode",
 "dense_f32"), "latent" (MLA attention over paged caches), "head_dim_64" (the matrix-core kernels at the
-reference's other head dimension), "mfma_ceiling" (what the matrix cores sustain on a register-only loop
+reference's other head dimensions, and the headline decode at eight and sixteen query heads per KV head), "mfma_ceiling" (what the matrix cores sustain on a register-only loop
 of the prefill kernels' product, on zeros and on the benchmark's kind of data) and "hbm_ceiling" (what a kernel that
 only reads gets out of HBM at the decode workloads' sizes).
 
@@ -546,8 +546,34 @@ def head_dim_64_section():
     decode = {"workload": "paged decode: batch 32, 32q/8kv heads, head_dim 64, bf16, block 16, ctx U[512,4096]; split + reduce",
               "value": gbps, "unit": "GB/s", "ms_per_step": stats["mean_ms"], "algorithmic_bytes": nbytes,
               "pct_hbm_peak": 100.0 * gbps / HBM_PEAK_GBPS, **timing_fields(stats)}
+    del work, out, workspace
+    torch.cuda.empty_cache()
     # The dense prefill at the other widths the matrix-core kernels are built for.
     others = {f"prefill_d{dim}": prefill_section(with_cpu=False, dim=dim, key=f"prefill_d{dim}") for dim in (96, 32)}
+    # The headline decode at eight and sixteen query heads per KV head (head_dim 128): the dense form of the decode
+    # kernel, every query head a column of one product.
+    for heads in (64, 128):
+        work = synthetic.paged_decode_workload(heads=heads, portable=True, name=f"paged_decode_h{heads}")
+        config = A.PagedKvDecodeAttentionConfig.contiguous(work.batch, work.heads, work.kv_heads, work.head_dim,
+                                                           work.block_size, work.physical_blocks,
+                                                           work.block_table_batch_stride, work.scale)
+        lens = torch.from_numpy(work.seq_lens).cuda()
+        table = torch.from_numpy(work.block_table.view(np.int32)).cuda()
+        out = torch.empty((work.batch, work.heads, work.head_dim), device="cuda", dtype=torch.bfloat16)
+        workspace = torch.empty(config.workspace_bytes(), dtype=torch.uint8, device="cuda")
+        step = lambda phases=3: A.paged_kv_decode_attention_bf16(None, out, work.query, work.key_cache, work.value_cache, lens,
+                                                                 table, config, workspace, phases)
+        whole, kernel = measure(step, 6), measure(lambda: step(1), 6)
+        nbytes = work.algorithmic_bytes()
+        rate = lambda stats: nbytes / (stats["mean_ms"] * 1e-3) / 1e9
+        others[f"decode_{heads // 8}_heads_per_kv_head"] = {
+            "workload": f"paged decode: batch 32, {heads}q/8kv heads, head_dim 128, bf16, block 16, ctx U[512,4096]; split + reduce",
+            "value": rate(whole), "unit": "GB/s", "ms_per_step": whole["mean_ms"], "algorithmic_bytes": nbytes,
+            "pct_hbm_peak": 100.0 * rate(whole) / HBM_PEAK_GBPS,
+            "roofline": {"bound": "hbm", "kernel": "singe_paged_decode_bf16_wide_d128_b16", "achieved": rate(kernel), "peak": HBM_PEAK_GBPS,
+                         "unit": "GB/s", "frac": rate(kernel) / HBM_PEAK_GBPS, **timing_fields(kernel)}}
+        del work, out, workspace
+        torch.cuda.empty_cache()
     return {"prefill": prefill, "decode": decode, **others}
 
 

@@ -209,6 +209,8 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_attention_f16_d112_softcap_i32_p16", "singe_paged_attention_f16_d112_softcap_i64_p16",
     "singe_rotary_paged_attention_bf16_d112_i32", "singe_rotary_paged_attention_bf16_d112_i64",
     "singe_rotary_paged_attention_bf16_d112_i32_p16", "singe_rotary_paged_attention_bf16_d112_i64_p16",
+    "singe_paged_decode_bf16_wide_d128_b16", "singe_paged_decode_bf16_wide_d128_any",
+    "singe_paged_decode_f16_wide_d128_b16", "singe_paged_decode_f16_wide_d128_any",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -240,6 +242,7 @@ constexpr PartRun kPartRuns[] = {
     {18, 10}, {19, 28},           // the head_dim 32 builds: dense kernels with their merges, paged kernels
     {20, 10}, {21, 28},           // the head_dim 96 builds
     {22, 10}, {23, 28}, {24, 10}, {25, 28}, {26, 10}, {27, 28}, {28, 10}, {29, 28},  // and those for 16, 48, 80, 112
+    {0, 4},                       // the wide decode kernels for bf16 / f16 caches
 };
 constexpr int runs_total() {
     int total = 0;

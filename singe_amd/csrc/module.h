@@ -61,7 +61,10 @@ enum KernelId : int {
     // that order), each bank in the order of its head_dim 128 forms: eight dense kernels, their two merges, the
     // paged kernels up to kSplitKReduce
     kOtherHeadDims,
-    kKernelCount = kOtherHeadDims + 6 * (10 + (kSplitKReduce - kPagedAttentionI32))
+    // bf16 / f16 paged decode at head_dim 128 with five to eight query heads per kv head, dense form:
+    // + (block size not a multiple of 16) + 2 * f16
+    kDecodeWide = kOtherHeadDims + 6 * (10 + (kSplitKReduce - kPagedAttentionI32)),
+    kKernelCount = kDecodeWide + 4
 };
 
 // The head_dim 64 build of a matrix-core kernel named by its head_dim 128 id.

@@ -26,10 +26,11 @@ int32_t decode(void* stream, uint16_t* out, size_t out_len, const uint16_t* quer
 
 constexpr unsigned kWavesPerWorkgroup = 8;
 
-// How the flat list of 32-key tiles is shared out (see paged_decode.hip).
+// How the flat list of 32-key tiles is shared out (see paged_decode.hip).  `span` is the most query heads a wave
+// carries: 8 (the one-hot form, and the dense form of fp8 caches), or 16 (the dense form of bf16 / f16 caches).
 struct Plan {
-    uint32_t head_groups;     // waves per kv head: ceil(group / 8)
-    uint32_t heads_per_wave;  // min(group, 8)
+    uint32_t head_groups;     // waves per kv head: ceil(group / span)
+    uint32_t heads_per_wave;  // min(group, span)
     uint32_t groups;          // 1 or 2 groups of four query heads per wave
     uint32_t work;            // kv_heads * head_groups
     uint32_t work_per_wg;     // min(work, 8)
@@ -43,11 +44,11 @@ size_t align256(size_t bytes) { return (bytes + 255) / 256 * 256; }
 
 // One workgroup of eight waves per compute unit, so every wave of the chip gets one equal range and
 // the launch finishes in a single round.
-Plan make_plan(const SingePagedKvDecodeAttentionConfig& c) {
+Plan make_plan(const SingePagedKvDecodeAttentionConfig& c, size_t span = 8) {
     Plan p;
     const size_t group = c.heads / c.kv_heads;
-    p.head_groups = static_cast<uint32_t>((group + 7) / 8);
-    p.heads_per_wave = static_cast<uint32_t>(group < 8 ? group : 8);
+    p.head_groups = static_cast<uint32_t>((group + span - 1) / span);
+    p.heads_per_wave = static_cast<uint32_t>(group < span ? group : span);
     p.groups = p.heads_per_wave <= 4 ? 1 : 2;
     p.work = static_cast<uint32_t>(c.kv_heads) * p.head_groups;
     p.work_per_wg = p.work < kWavesPerWorkgroup ? p.work : kWavesPerWorkgroup;
@@ -66,6 +67,13 @@ Plan make_plan(const SingePagedKvDecodeAttentionConfig& c) {
     p.out_offset = p.lse_offset + align256(rows * sizeof(float));
     p.bytes = p.out_offset + align256(rows * c.head_dim * sizeof(float));
     return p;
+}
+
+// What singe_hip_paged_kv_decode_attention_workspace_bytes asks for: the config does not say the cache's type, so
+// enough for either form.
+size_t workspace_need(const SingePagedKvDecodeAttentionConfig& c) {
+    const size_t narrow = make_plan(c, 8).bytes, wide = make_plan(c, 16).bytes;
+    return narrow > wide ? narrow : wide;
 }
 
 int32_t validate_config(const SingePagedKvDecodeAttentionConfig& c) {
@@ -100,7 +108,7 @@ size_t singe_hip_paged_kv_decode_attention_workspace_bytes(const SingePagedKvDec
     if (config == nullptr || validate_config(*config) != 0) return 0;
     size_t rows = 0, elements = 0;
     if (!checked_mul(config->batch, config->heads, &rows) || !checked_mul(rows, config->head_dim, &elements)) return 0;
-    return make_plan(*config).bytes;
+    return workspace_need(*config);
 }
 
 int32_t singe_hip_paged_kv_decode_attention_bf16(
@@ -134,7 +142,7 @@ int32_t singe_hip_paged_kv_decode_attention_no_alloc_bf16(
     size_t block_table_len, const SingePagedKvDecodeAttentionConfig* config) {
     if (config == nullptr) return fail(SINGE_HIP_NULL_POINTER, "config");
     if (int32_t status = validate_config(*config)) return status;
-    const size_t need = make_plan(*config).bytes;
+    const size_t need = workspace_need(*config);
     if (need > SINGE_HIP_STATIC_SCRATCH_BYTES)
         return fail(SINGE_HIP_LENGTH_TOO_SHORT, "static scratch", need, SINGE_HIP_STATIC_SCRATCH_BYTES);
     void* scratch = nullptr;
@@ -230,7 +238,13 @@ int32_t decode(
     uint64_t reach = static_cast<uint64_t>(c.block_table_batch_stride) * c.block_size;
     if (!fits_i32(reach)) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "block_table_batch_stride * block_size");
 
-    const Plan plan = make_plan(c);
+    // bf16 caches take the one-hot form, fp8 caches the dense form (see paged_decode.hip); and so do bf16 / f16
+    // caches with more than four query heads per kv head at head_dim 128, where the one-hot form would carry two
+    // groups per wave, as long as the batch's prefix sums fit beside that form's 132 KiB of staging in LDS.
+    const unsigned prefix_bytes = static_cast<unsigned>((2 * c.batch + 1) * sizeof(uint32_t));
+    constexpr unsigned kWideStagingBytes = 135168, kLdsBytes = 160 * 1024;
+    const bool wide = !fp8 && !narrow && c.heads / c.kv_heads > 4 && kWideStagingBytes + prefix_bytes <= kLdsBytes;
+    const Plan plan = make_plan(c, wide || fp8 ? 16 : 8);  // (the dense form of fp8 caches has its Q^T in registers and no such limit)
     if (workspace == nullptr) return fail(SINGE_HIP_NULL_POINTER, "workspace");
     if (workspace_bytes < plan.bytes) return fail(SINGE_HIP_LENGTH_TOO_SHORT, "workspace", plan.bytes, workspace_bytes);
     if (c.batch > 8000) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "more than 8000 sequences per call");
@@ -264,12 +278,12 @@ int32_t decode(
     args.scale_log2e = c.scale * 1.4426950408889634074f;
 
     const bool aligned = c.block_size % 16 == 0;
-    // bf16 caches take the one-hot form, fp8 caches the dense form (see paged_decode.hip).
-    const KernelId kernel = fp8 ? static_cast<KernelId>(kDecodeF8Wide + (aligned ? 0 : 1) + (g_relaxed.load(std::memory_order_relaxed) ? 2 : 0))
-                                : static_cast<KernelId>((f16 ? kDecodeF16 : kDecodeBf16) + (aligned ? 0 : 2) + (plan.groups == 2 ? 1 : 0));
+    const KernelId kernel = fp8    ? static_cast<KernelId>(kDecodeF8Wide + (aligned ? 0 : 1) + (g_relaxed.load(std::memory_order_relaxed) ? 2 : 0))
+                            : wide ? static_cast<KernelId>(kDecodeWide + (aligned ? 0 : 1) + (f16 ? 2 : 0))
+                                   : static_cast<KernelId>((f16 ? kDecodeF16 : kDecodeBf16) + (aligned ? 0 : 2) + (plan.groups == 2 ? 1 : 0));
     if (phases & SINGE_HIP_DECODE_SPLIT)
         if (int32_t status = launch(narrow ? at_head_dim_64(kernel) : kernel, plan.grid_x, plan.grid_y, 1, 64 * kWavesPerWorkgroup, stream, args,
-                                    static_cast<unsigned>((2 * c.batch + 1) * sizeof(uint32_t))))
+                                    prefix_bytes))
             return status;
     if (!(phases & SINGE_HIP_DECODE_REDUCE)) return 0;
 

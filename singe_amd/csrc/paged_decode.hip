@@ -276,6 +276,17 @@ SINGE_DEVICE unsigned int half_twice(float value) {
     }
 }
 
+// Two values rounded to the cache's 16-bit type, low half first.
+template <bool F16>
+SINGE_DEVICE unsigned int half_pair(float lo, float hi) {
+    if constexpr (F16) {
+        const f32x2_t both = {lo, hi};
+        return __builtin_bit_cast(unsigned int, __builtin_convertvector(both, f16x2_t));
+    } else {
+        return bf16_pair(lo, hi);
+    }
+}
+
 template <bool F16>
 SINGE_DEVICE f32x4_t score_mma(uint4 keys, bf16x8_t query, f32x4_t acc) {
     if constexpr (F16)
@@ -327,14 +338,19 @@ constexpr int kStagedTileBytes = kTile * kStagedRowBytes;
 constexpr int kKeyStagingBytes = kTile * 256;
 
 // GROUPS = groups of four query heads a wave carries (1 or 2: up to 8 query heads per kv head).
-// WIDE (fp8 caches): the query heads of the kv head sit in the sixteen columns of one MFMA, each once, and
-// the values take the dense route: widened V rows are staged in a private LDS buffer and read back
-// transposed (ds_read_b64_tr_b16) as the A operand of v_mfma_f32_16x16x32_bf16, O^T[dim, head] += V^T . P^T.
-// That is a third of the matrix instructions and half the exponentials of the one-hot form, which matters
-// where the byte rate of an fp8 cache leaves the vector and matrix units little time per byte.
+// WIDE (fp8 caches, and bf16 / f16 caches with more than four query heads per kv head): the query heads of the kv
+// head sit in the sixteen columns of one MFMA, each once, and the values take the dense route: V rows (widened, for
+// fp8) are staged in a private LDS buffer and read back transposed (ds_read_b64_tr_b16) as the A operand of
+// v_mfma_f32_16x16x32, O^T[dim, head] += V^T . P^T.  That is a third of the matrix instructions and half the
+// exponentials of the one-hot form with two groups, which matters where the byte rate of an fp8 cache leaves the vector
+// and matrix units little time per byte, and where eight query heads share a kv head (the one-hot form with two
+// groups runs out of registers there and reached 55 % of the HBM peak where one group reaches 74 %).  With bf16 / f16
+// caches the wave's Q^T lives in LDS too (four kilobytes, read twice per tile): two 64-register tiles, the 32
+// accumulators and Q^T would not fit the wave's registers together.
 template <int GROUPS, bool ALIGNED16, bool FP8, bool EXACT, bool WIDE = false, bool F16 = false>
 SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, unsigned char* staging = nullptr) {
-    static_assert(WIDE == FP8 && (!WIDE || GROUPS == 1), "fp8 caches take the wide form, bf16 caches the one-hot form");
+    static_assert((!FP8 || WIDE) && (!WIDE || GROUPS == 1), "fp8 caches take the wide form; the wide form carries one group");
+    constexpr bool kQueryInLds = WIDE && !FP8;
     using Tile = typename std::conditional<FP8, KeyTileFp8, KeyTileBf16>::type;
     constexpr int DEPTH = FP8 ? 3 : 2;  // an fp8 tile is half the bytes, so one more is kept in flight
     const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -390,8 +406,8 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
 
     const unsigned int group = a.heads / a.kv_heads;
     const unsigned int kv_head = work / a.head_groups;
-    const unsigned int head_in_group = (work % a.head_groups) * 8;  // first query head of this wave inside its group
-    const unsigned int wave_heads = group - head_in_group < 8 ? group - head_in_group : 8;
+    const unsigned int head_in_group = (work % a.head_groups) * a.heads_per_wave;  // first query head of this wave inside its group
+    const unsigned int wave_heads = group - head_in_group < a.heads_per_wave ? group - head_in_group : a.heads_per_wave;
     const unsigned int slots = a.workers + a.batch;
 
     // The sequence that holds tile range_first: the last b with prefix[b] <= range_first.
@@ -418,6 +434,11 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
     f32x4_t wide_acc[WIDE ? 8 : 1];
     float wide_max = -INFINITY, wide_sum = 0.0f;
     unsigned char* const staged = WIDE ? staging + wave * kStagedTileBytes : nullptr;
+    // K's way into its operand layout (bf16 / f16 caches): behind the eight value buffers in the wide form, and the
+    // waves' Q^T behind those.
+    // (the wide form takes K through in two halves of sixteen keys, a buffer of half the size)
+    unsigned char* const key_staging = WIDE ? staging + 8 * kStagedTileBytes + wave * (kKeyStagingBytes / 2) : staging + wave * kKeyStagingBytes;
+    unsigned char* const query_slot = staging + 8 * (kStagedTileBytes + kKeyStagingBytes / 2) + wave * 4096 + 16 * lane;
     auto load_query = [&](unsigned int b) __attribute__((always_inline)) {
         if constexpr (WIDE) {
             const bool real = t < wave_heads;
@@ -426,7 +447,8 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
             for (int c = 0; c < 4; ++c) {
                 uint4 bits = *reinterpret_cast<const uint4*>(qp + dim_step * c);
                 if (!real) bits = make_uint4(0, 0, 0, 0);
-                q[0][c] = __builtin_bit_cast(bf16x8_t, bits);
+                if constexpr (kQueryInLds) *reinterpret_cast<uint4*>(query_slot + 1024 * c) = bits;  // a slot only this lane touches
+                else q[0][c] = __builtin_bit_cast(bf16x8_t, bits);
             }
 #pragma unroll
             for (int db = 0; db < 8; ++db) wide_acc[db] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -460,20 +482,42 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
             for (int half = 0; half < 2; ++half)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const uint4 row = widen_fp8x8<EXACT>(tile.v[half][i].x, tile.v[half][i].y, EXACT ? tile.row_value_scale[half][i] : 1.0f);
+                    uint4 row;
+                    if constexpr (FP8) row = widen_fp8x8<EXACT>(tile.v[half][i].x, tile.v[half][i].y, EXACT ? tile.row_value_scale[half][i] : 1.0f);
+                    else row = tile.v[half][i];
                     *reinterpret_cast<uint4*>(staged + (16 * half + 4 * g + i) * kStagedRowBytes + 16 * t) = row;
                 }
             // Scores S^T[key 16 half + row][head]: row = lane % 16 of the A operand is key t of the half.
             f32x4_t s0 = {0.0f, 0.0f, 0.0f, 0.0f}, s1 = {0.0f, 0.0f, 0.0f, 0.0f};
+            if constexpr (FP8) {
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const uint4 a0 = tile.k[0][c >> 1], a1 = tile.k[1][c >> 1];
-                const uint4 first = (c & 1) ? widen_fp8x8<EXACT>(a0.z, a0.w, EXACT ? tile.key_scale[0] : 1.0f)
-                                            : widen_fp8x8<EXACT>(a0.x, a0.y, EXACT ? tile.key_scale[0] : 1.0f);
-                const uint4 second = (c & 1) ? widen_fp8x8<EXACT>(a1.z, a1.w, EXACT ? tile.key_scale[1] : 1.0f)
-                                             : widen_fp8x8<EXACT>(a1.x, a1.y, EXACT ? tile.key_scale[1] : 1.0f);
-                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, first), q[0][c], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, second), q[0][c], s1, 0, 0, 0);
+                for (int c = 0; c < 4; ++c) {
+                    const uint4 a0 = tile.k[0][c >> 1], a1 = tile.k[1][c >> 1];
+                    const uint4 first = (c & 1) ? widen_fp8x8<EXACT>(a0.z, a0.w, EXACT ? tile.key_scale[0] : 1.0f)
+                                                : widen_fp8x8<EXACT>(a0.x, a0.y, EXACT ? tile.key_scale[0] : 1.0f);
+                    const uint4 second = (c & 1) ? widen_fp8x8<EXACT>(a1.z, a1.w, EXACT ? tile.key_scale[1] : 1.0f)
+                                                 : widen_fp8x8<EXACT>(a1.x, a1.y, EXACT ? tile.key_scale[1] : 1.0f);
+                    s0 = score_mma<F16>(first, q[0][c], s0);
+                    s1 = score_mma<F16>(second, q[0][c], s1);
+                }
+            } else {
+                // K rows go to the wave's other buffer as fetched and come back in the operand layout (as in `fold`),
+                // sixteen keys at a time; LDS keeps a wave's accesses in order, so the second half may follow the
+                // first half's reads into the same rows.
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        *reinterpret_cast<uint4*>(key_staging + (4 * g + i) * 256 + ((t ^ (4 * g + i)) << 4)) = tile.k[half][i];
+                    f32x4_t scores = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        const uint4 keys = *reinterpret_cast<const uint4*>(key_staging + t * 256 + (((4 * c + g) ^ t) << 4));
+                        const uint4 mine = *reinterpret_cast<const uint4*>(query_slot + 1024 * c);
+                        scores = score_mma<F16>(keys, __builtin_bit_cast(bf16x8_t, mine), scores);
+                    }
+                    if (half == 0) s0 = scores; else s1 = scores;
+                }
             }
             // Lane (g, t) now holds head t against keys 16 half + 4 g + i.
             float p[8];
@@ -511,7 +555,8 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
                 if constexpr (!EXACT) p[i] *= tile.row_value_scale[i >> 2][i & 3];
             }
             wide_sum += total;
-            const uint4 weights = make_uint4(bf16_pair(p[0], p[1]), bf16_pair(p[2], p[3]), bf16_pair(p[4], p[5]), bf16_pair(p[6], p[7]));
+            const uint4 weights = make_uint4(half_pair<F16>(p[0], p[1]), half_pair<F16>(p[2], p[3]), half_pair<F16>(p[4], p[5]),
+                                             half_pair<F16>(p[6], p[7]));
             // O^T[dim, head] += V^T . P^T: k-slots 8 g + j of the MFMA are keys 4 g + j (j < 4) and
             // 16 + 4 g + j - 4, which is how the two transposing reads of a 16-lane group deliver them.
             typedef short v4i16_t __attribute__((ext_vector_type(4)));
@@ -523,8 +568,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
                 const v4i16_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(patch + 32 * db));
                 const v4i16_t high = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4_t)(patch + 16 * kStagedRowBytes + 32 * db));
                 const v8i16_t both = __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7);
-                wide_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, both), __builtin_bit_cast(bf16x8_t, weights),
-                                                                  wide_acc[db], 0, 0, 0);
+                wide_acc[db] = score_mma<F16>(__builtin_bit_cast(uint4, both), __builtin_bit_cast(bf16x8_t, weights), wide_acc[db]);
             }
         }
     };
@@ -550,13 +594,13 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
                     if (kDim == 128 || 8 * t < static_cast<unsigned int>(kDim))
-                        *reinterpret_cast<uint4*>(staging + wave * kKeyStagingBytes + (16 * half + 4 * g + i) * 256 + ((t ^ (4 * g + i)) << 4)) = tile.k[half][i];
+                        *reinterpret_cast<uint4*>(key_staging + (16 * half + 4 * g + i) * 256 + ((t ^ (4 * g + i)) << 4)) = tile.k[half][i];
         }
 #pragma unroll
         for (int c = 0; c < kDimSteps; ++c) {
             uint4 first, second;
             if constexpr (!FP8) {
-                const unsigned char* row = staging + wave * kKeyStagingBytes + t * 256 + (((4 * c + g) ^ t) << 4);
+                const unsigned char* row = key_staging + t * 256 + (((4 * c + g) ^ t) << 4);
                 first = *reinterpret_cast<const uint4*>(row);
                 second = *reinterpret_cast<const uint4*>(row + 16 * 256);
             }
@@ -743,6 +787,19 @@ SINGE_DECODE_F16_KERNEL(SINGE_DECODE_NAME(singe_paged_decode_f16, _g1_any), 1, f
 SINGE_DECODE_F16_KERNEL(SINGE_DECODE_NAME(singe_paged_decode_f16, _g2_any), 2, false)
 
 #if SINGE_HEAD_DIM == 128
+// bf16 / f16 caches with five to sixteen query heads per kv head: the wide form; a value buffer, a key buffer and Q^T per wave.
+#define SINGE_DECODE_WIDE_HALF_KERNEL(NAME, ALIGNED, F16)                                                               \
+    extern "C" __global__ __launch_bounds__(512) void NAME(DecodeArgs args) {                                            \
+        extern __shared__ unsigned int prefix[];                                                                        \
+        __shared__ __attribute__((aligned(16))) unsigned char staging[8 * (kStagedTileBytes + kKeyStagingBytes / 2 + 4096)]; \
+        paged_decode_body<1, ALIGNED, false, true, true, F16>(args, prefix, staging);                                   \
+    }
+
+SINGE_DECODE_WIDE_HALF_KERNEL(singe_paged_decode_bf16_wide_d128_b16, true, false)
+SINGE_DECODE_WIDE_HALF_KERNEL(singe_paged_decode_bf16_wide_d128_any, false, false)
+SINGE_DECODE_WIDE_HALF_KERNEL(singe_paged_decode_f16_wide_d128_b16, true, true)
+SINGE_DECODE_WIDE_HALF_KERNEL(singe_paged_decode_f16_wide_d128_any, false, true)
+
 #define SINGE_DECODE_WIDE_KERNEL(NAME, ALIGNED, EXACT)                                          \
     extern "C" __global__ __launch_bounds__(512) void NAME(DecodeArgs args) {                    \
         extern __shared__ unsigned int prefix[];                                                \
@@ -769,7 +826,7 @@ SINGE_DEVICE void paged_decode_combine_body(const CombineArgs& a) {
     const unsigned int b = row / a.heads, head = row % a.heads;
     const unsigned int group = a.heads / a.kv_heads;
     const unsigned int kv_head = head / group, in_group = head % group;
-    const unsigned int work = kv_head * a.head_groups + in_group / 8, local = in_group % 8;
+    const unsigned int work = kv_head * a.head_groups + in_group / a.heads_per_wave, local = in_group % a.heads_per_wave;
     const unsigned int share = a.meta[0];
     const unsigned int first_tile = a.meta[2 + b], end_tile = a.meta[3 + b];
     float low = 0.0f, high = 0.0f;  // a sequence with no keys keeps a zero row (cpu/attention.rs:1213-1215)

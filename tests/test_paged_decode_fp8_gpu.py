@@ -59,7 +59,7 @@ def assert_close(got, want, label):
 
 @pytest.mark.parametrize("relaxed", [False, True])
 @pytest.mark.parametrize("heads,kv_heads,block_size", [(64, 8, 16), (8, 2, 16), (8, 1, 16), (6, 2, 32), (16, 1, 16),
-                                                      (8, 2, 7), (8, 1, 1)])
+                                                      (8, 2, 7), (8, 1, 1), (24, 2, 16), (40, 2, 16), (13, 1, 7)])
 def test_fp8_decode_matches_oracle(heads, kv_heads, block_size, relaxed):
     lens = [0, 1, 15, 16, 17, 33, 100, 257, 900, 64, 31, 2048]
     blocks = sum((l + block_size - 1) // block_size for l in lens) + 5

@@ -92,6 +92,31 @@ def test_decode_group_sizes(heads, kv_heads):
     assert_close(got, want, f"{heads}/{kv_heads}")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("block_size", [16, 7, 32, 1])
+@pytest.mark.parametrize("heads,kv_heads", [(40, 8), (64, 8), (7, 1), (24, 2), (48, 3)])
+def test_five_to_sixteen_query_heads_per_kv_head(heads, kv_heads, block_size, dtype):
+    # more than four query heads per kv head: the dense form of the decode kernel at head_dim 128 (every head a
+    # column of one product, values through LDS); sixteen and twelve heads take two waves per kv head
+    lens = [300, 0, 1, 31, 32, 33, 1000, 64, 17, 555]
+    work = synthetic.paged_decode_workload(batch=len(lens), heads=heads, kv_heads=kv_heads, block_size=block_size,
+                                           physical_blocks=max(256, 16 * 2400 // block_size), seq_lens=lens, seed=7 * heads + block_size)
+    if dtype == torch.float16:  # the oracle reads what the kernel reads: bf16 values that f16 holds too
+        work.query, work.key_cache, work.value_cache = (x.to(torch.float16).to(torch.bfloat16)
+                                                        for x in (work.query, work.key_cache, work.value_cache))
+    got, want = run_gpu(work, dtype=dtype), run_oracle(work)
+    assert not got[1].any()
+    assert_close(got, want, f"{heads}/{kv_heads} block {block_size} {dtype}")
+
+
+def test_the_dense_form_steps_aside_for_batches_whose_prefix_sums_do_not_fit():
+    # 1600 sequences: their prefix sums (12.8 KB of LDS) no longer fit beside the dense form's staging
+    rng = np.random.default_rng(12)
+    lens = [int(n) for n in rng.integers(0, 40, 1600)]
+    work = synthetic.paged_decode_workload(batch=len(lens), heads=16, kv_heads=2, physical_blocks=8192, seq_lens=lens, seed=9, fill="used")
+    assert_close(run_gpu(work), run_oracle(work), "1600 sequences, 8 heads per kv head")
+
+
 @pytest.mark.parametrize("block_size", [1, 7, 16, 32, 48, 5])
 @pytest.mark.parametrize("workers", [0, 1, 3, 50, 4096])
 def test_decode_block_sizes_and_splits(block_size, workers):
