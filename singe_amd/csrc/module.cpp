@@ -211,6 +211,8 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_rotary_paged_attention_bf16_d112_i32_p16", "singe_rotary_paged_attention_bf16_d112_i64_p16",
     "singe_paged_decode_bf16_wide_d128_b16", "singe_paged_decode_bf16_wide_d128_any",
     "singe_paged_decode_f16_wide_d128_b16", "singe_paged_decode_f16_wide_d128_any",
+    "singe_paged_decode_combine_many_bf16", "singe_paged_decode_combine_many_f16",
+    "singe_paged_decode_combine_many_bf16_d64", "singe_paged_decode_combine_many_f16_d64",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -243,6 +245,7 @@ constexpr PartRun kPartRuns[] = {
     {20, 10}, {21, 28},           // the head_dim 96 builds
     {22, 10}, {23, 28}, {24, 10}, {25, 28}, {26, 10}, {27, 28}, {28, 10}, {29, 28},  // and those for 16, 48, 80, 112
     {0, 4},                       // the wide decode kernels for bf16 / f16 caches
+    {0, 2}, {13, 2},              // the decode merge for rows with many slots, head_dim 128 and 64
 };
 constexpr int runs_total() {
     int total = 0;

@@ -64,7 +64,9 @@ enum KernelId : int {
     // bf16 / f16 paged decode at head_dim 128 with five to eight query heads per kv head, dense form:
     // + (block size not a multiple of 16) + 2 * f16
     kDecodeWide = kOtherHeadDims + 6 * (10 + (kSplitKReduce - kPagedAttentionI32)),
-    kKernelCount = kDecodeWide + 4
+    // the decode merge for rows with many slots: bf16, f16, then the same for head_dim 64
+    kDecodeCombineMany = kDecodeWide + 4, kDecodeCombineManyF16, kDecodeCombineManyD64, kDecodeCombineManyF16D64,
+    kKernelCount
 };
 
 // The head_dim 64 build of a matrix-core kernel named by its head_dim 128 id.

@@ -298,6 +298,11 @@ int32_t decode(
     combine.workers = plan.workers;
     combine.head_groups = plan.head_groups;
     combine.heads_per_wave = plan.heads_per_wave;
+    // A row has about workers / batch slots: from 32 on, a workgroup of eight waves folds it instead of one wave.
+    if (static_cast<size_t>(plan.workers) >= 32 * c.batch) {
+        const KernelId many = static_cast<KernelId>(kDecodeCombineMany + (f16 ? 1 : 0) + (narrow ? 2 : 0));
+        return launch(many, static_cast<unsigned>(c.batch * c.heads), 1, 1, 512, stream, combine);
+    }
     const KernelId merge = f16 ? kDecodeF16Combine : kDecodeCombine;
     return launch(narrow ? at_head_dim_64(merge) : merge, static_cast<unsigned>((c.batch * c.heads + 3) / 4), 1, 1, 256, stream, combine);
 }

@@ -893,6 +893,109 @@ SINGE_DEVICE void paged_decode_combine_body(const CombineArgs& a) {
     if (holds_values) *reinterpret_cast<unsigned int*>(a.out + static_cast<size_t>(row) * kDim + 2 * lane) = packed;
 }
 
+// The same fold for rows with many slots (few sequences, long contexts: a lone sequence has a slot per worker, 256 of
+// them): a workgroup of eight waves per row, wave w folding the slots of the 16-slot groups w, w + 8, ..., and the first
+// wave folding the eight results, which it finds in LDS.  One wave per row takes a round trip per sixteen slots, 21 us for
+// 256 of them; this takes two.
+constexpr int kCombineWaves = 8;
+
+template <bool F16>
+SINGE_DEVICE void paged_decode_combine_many_body(const CombineArgs& a) {
+    __shared__ float wave_best[kCombineWaves], wave_total[kCombineWaves];
+    __shared__ float2 wave_values[kCombineWaves][64];
+    const unsigned int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned int row = blockIdx.x;  // batch * heads + head
+    const unsigned int b = row / a.heads, head = row % a.heads;
+    const unsigned int group = a.heads / a.kv_heads;
+    const unsigned int kv_head = head / group, in_group = head % group;
+    const unsigned int work = kv_head * a.head_groups + in_group / a.heads_per_wave, local = in_group % a.heads_per_wave;
+    const unsigned int share = a.meta[0];
+    const unsigned int first_tile = a.meta[2 + b], end_tile = a.meta[3 + b];
+    const bool holds_values = 2 * lane < static_cast<unsigned int>(kDim);  // a lane takes two of the row's values
+    float low = 0.0f, high = 0.0f, best = -INFINITY, total = 0.0f;
+    if (end_tile > first_tile) {
+        const unsigned int first_worker = first_tile / share, last_worker = (end_tile - 1) / share;
+        const size_t base = (static_cast<size_t>(work) * (a.workers + a.batch) + first_worker + b) * a.heads_per_wave + local;
+        const unsigned int count = last_worker - first_worker + 1;
+        for (unsigned int first = 16 * wave; first < count; first += 16 * kCombineWaves) {
+            const unsigned int n = count - first < 16 ? count - first : 16;
+            const size_t group_base = base + static_cast<size_t>(first) * a.heads_per_wave;
+            const float mine = lane < n ? a.partial_lse[group_base + static_cast<size_t>(lane) * a.heads_per_wave] : -INFINITY;
+            float2 rows[16];
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                rows[j] = make_float2(0.0f, 0.0f);
+                if (static_cast<unsigned int>(j) < n && holds_values)
+                    rows[j] = *reinterpret_cast<const float2*>(a.partial_out + (group_base + static_cast<size_t>(j) * a.heads_per_wave) * kDim + 2 * lane);
+            }
+            float largest = mine;
+#pragma unroll
+            for (int step = 32; step >= 1; step >>= 1) largest = fmaxf(largest, __shfl_xor(largest, step, 64));
+            largest = fmaxf(largest, best);
+            if (largest == -INFINITY) continue;  // nothing but empty slots so far
+            const float rescale = __expf(best - largest);
+            const float weight = __expf(mine - largest);  // 0 for lanes past n
+            float weights = weight;
+#pragma unroll
+            for (int step = 32; step >= 1; step >>= 1) weights += __shfl_xor(weights, step, 64);
+            total = total * rescale + weights;
+            low *= rescale;
+            high *= rescale;
+            best = largest;
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const float w = __shfl(weight, j, 64);
+                if (static_cast<unsigned int>(j) < n) {
+                    low = fmaf(w, rows[j].x, low);
+                    high = fmaf(w, rows[j].y, high);
+                }
+            }
+        }
+    }
+    if (lane == 0) {
+        wave_best[wave] = best;
+        wave_total[wave] = total;
+    }
+    wave_values[wave][lane] = make_float2(low, high);
+    __syncthreads();
+    if (wave != 0) return;
+    float largest = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kCombineWaves; ++w) largest = fmaxf(largest, wave_best[w]);
+    low = 0.0f;
+    high = 0.0f;
+    total = 0.0f;
+    if (largest != -INFINITY) {
+#pragma unroll
+        for (int w = 0; w < kCombineWaves; ++w) {
+            const float factor = __expf(wave_best[w] - largest);  // 0 for a wave that saw nothing
+            total = fmaf(factor, wave_total[w], total);
+            low = fmaf(factor, wave_values[w][lane].x, low);
+            high = fmaf(factor, wave_values[w][lane].y, high);
+        }
+        if (total > 0.0f) {
+            low /= total;
+            high /= total;
+        }
+    }
+    unsigned int packed;
+    if constexpr (F16) {
+        const f32x2_t both = {low, high};
+        packed = __builtin_bit_cast(unsigned int, __builtin_convertvector(both, f16x2_t));
+    } else {
+        packed = pack_bf16x2(low, high);
+    }
+    if (holds_values) *reinterpret_cast<unsigned int*>(a.out + static_cast<size_t>(row) * kDim + 2 * lane) = packed;
+}
+
+#if SINGE_HEAD_DIM == 128
+extern "C" __global__ __launch_bounds__(512) void singe_paged_decode_combine_many_bf16(CombineArgs a) { paged_decode_combine_many_body<false>(a); }
+extern "C" __global__ __launch_bounds__(512) void singe_paged_decode_combine_many_f16(CombineArgs a) { paged_decode_combine_many_body<true>(a); }
+#else
+extern "C" __global__ __launch_bounds__(512) void SINGE_DECODE_NAME(singe_paged_decode_combine_many_bf16, /**/)(CombineArgs a) { paged_decode_combine_many_body<false>(a); }
+extern "C" __global__ __launch_bounds__(512) void SINGE_DECODE_NAME(singe_paged_decode_combine_many_f16, /**/)(CombineArgs a) { paged_decode_combine_many_body<true>(a); }
+#endif
+
 #if SINGE_HEAD_DIM == 128
 extern "C" __global__ __launch_bounds__(256) void singe_paged_decode_combine_bf16(CombineArgs a) { paged_decode_combine_body<false>(a); }
 extern "C" __global__ __launch_bounds__(256) void singe_paged_decode_combine_f16(CombineArgs a) { paged_decode_combine_body<true>(a); }

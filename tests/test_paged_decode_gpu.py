@@ -109,6 +109,23 @@ def test_five_to_sixteen_query_heads_per_kv_head(heads, kv_heads, block_size, dt
     assert_close(got, want, f"{heads}/{kv_heads} block {block_size} {dtype}")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("head_dim", [128, 64])
+@pytest.mark.parametrize("lens", [[9000], [0, 7777], [33, 5000, 1, 0, 2048], [16] * 3])
+def test_few_sequences_fold_their_many_slots_with_a_workgroup_per_row(lens, head_dim, dtype):
+    # a row of a lone long sequence has a slot per worker: the merge takes a workgroup of eight waves per row then
+    work = synthetic.paged_decode_workload(batch=len(lens), heads=8, kv_heads=2, head_dim=head_dim, physical_blocks=1024,
+                                           seq_lens=lens, seed=len(lens) + head_dim)
+    if dtype == torch.float16:
+        work.query, work.key_cache, work.value_cache = (x.to(torch.float16).to(torch.bfloat16)
+                                                        for x in (work.query, work.key_cache, work.value_cache))
+    got, want = run_gpu(work, dtype=dtype), run_oracle(work)
+    assert_close(got, want, f"lens {lens} head_dim {head_dim} {dtype}")
+    for b, n in enumerate(lens):
+        if n == 0:
+            assert not got[b].any()
+
+
 def test_the_dense_form_steps_aside_for_batches_whose_prefix_sums_do_not_fit():
     # 1600 sequences: their prefix sums (12.8 KB of LDS) no longer fit beside the dense form's staging
     rng = np.random.default_rng(12)
