@@ -20,8 +20,10 @@ bool on_matrix_cores(const SingePagedMlaAttentionProblem& p) {
 
 // Key splits for a problem: the row tiles of a decode step or a short chunk (one workgroup each, one workgroup to a
 // compute unit) leave most of the chip idle, so each tile's keys are shared out until there is about one workgroup
-// per compute unit.  The count of live tiles is not known on the host (it depends on the offsets on the device):
-// every sequence has at least one, and together they hold at least tokens * heads / 128.
+// per compute unit: 64 shares at most (the merge keeps a share's weight per lane), and no more than leave a share
+// four key tiles of a sequence of average length (the page table bounds the keys from above).  The count of live
+// tiles is not known on the host (it depends on the offsets on the device): every sequence has at least one, and
+// together they hold at least tokens * heads / 128.
 // 0 = chosen by problem size (singe_hip_set_paged_mla_attention_splits).
 uint32_t g_latent_splits = 0;
 
@@ -32,8 +34,12 @@ uint32_t latent_splits(const SingePagedMlaAttentionProblem& p) {
     const uint64_t workgroups = packed > static_cast<uint64_t>(p.sequences) ? packed : static_cast<uint64_t>(p.sequences);
     const uint64_t wanted = compute_units();
     if (workgroups >= wanted) return 1;
-    const uint64_t splits = wanted / workgroups;
-    return static_cast<uint32_t>(splits > 16 ? 16 : splits < 1 ? 1 : splits);
+    const uint64_t mean_keys = static_cast<uint64_t>(p.page_table > 0 ? p.page_table : 0) * static_cast<uint64_t>(p.page_size) / static_cast<uint64_t>(p.sequences);
+    const uint64_t worth = mean_keys / (4 * 32);
+    uint64_t splits = wanted / workgroups;
+    if (splits > 64) splits = 64;
+    if (splits > worth) splits = worth;
+    return static_cast<uint32_t>(splits < 1 ? 1 : splits);
 }
 
 size_t latent_scratch_bytes(const SingePagedMlaAttentionProblem& p, uint32_t splits) {
@@ -115,23 +121,29 @@ int32_t paged_mla_attention(void* stream, const void* latent_queries, const void
         // Key splits, when the caller lent scratch for them: the attention kernel leaves partials, a second kernel
         // merges them.
         uint32_t splits = scratch != nullptr ? latent_splits(p) : 1;
-        if (splits > 1 && (scratch_bytes < latent_scratch_bytes(p, splits) || blocks * splits > 0x7fffffffull)) splits = 1;
+        if (splits > 1 && (scratch_bytes < latent_scratch_bytes(p, splits) || blocks * splits > 0x7fffffffull || blocks * 32 > 0x7fffffffull))
+            splits = 1;
         if (splits > 1) {
             if (reinterpret_cast<uintptr_t>(scratch) % 16 != 0) return fail(SINGE_HIP_INVALID_ARGUMENT, "scratch alignment");
             args.splits = splits;
             args.partial_out = static_cast<float*>(scratch);
             args.partial_lse = args.partial_out + static_cast<size_t>(splits) * p.tokens * p.heads * 512;
         }
-        // Units go to the XCDs in bands of neighbours (see the kernel): as wide as leaves every XCD something to do,
-        // 32 (an XCD's compute units, each of which holds one workgroup) at most.  The grid covers whole rounds of eight bands.
-        const uint64_t band = blocks >= 256 ? 32 : (blocks + 7) / 8;
+        // Without splits, units go to the XCDs in bands of neighbours (see the kernel): as wide as leaves every XCD
+        // something to do, 32 (an XCD's compute units, each of which holds one workgroup) at most.  The width follows
+        // the units that are surely live (the count of blocks is an upper bound: up to one per sequence more), and the
+        // grid covers whole rounds of eight bands.  With splits the grid is the units times their shares.
+        const uint64_t surely_live = row_blocks > static_cast<uint64_t>(p.sequences) ? row_blocks : static_cast<uint64_t>(p.sequences);
+        const uint64_t band = surely_live >= 256 ? 32 : (surely_live + 7) / 8;
         const uint64_t rounds = (blocks + 8 * band - 1) / (8 * band);
         args.unit_band = static_cast<uint32_t>(band);
-        if (rounds * 8 * band * splits > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
+        const uint64_t grid = splits > 1 ? blocks * splits : rounds * 8 * band;
+        if (grid > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
         const bool bf16 = p.data_type == SINGE_HIP_BF16;
-        const int32_t launched = launch(bf16 ? kLatentTilesBf16 : kLatentTilesF16, static_cast<unsigned>(rounds * 8 * band * splits), 1, 1, 512, stream, args);
+        const int32_t launched = launch(bf16 ? kLatentTilesBf16 : kLatentTilesF16, static_cast<unsigned>(grid), 1, 1, 512, stream, args);
         if (launched != 0 || splits == 1) return launched;
-        return launch(bf16 ? kLatentCombineBf16 : kLatentCombineF16, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+        // The merge: 32 workgroups of four waves to a unit, a wave to a row.
+        return launch(bf16 ? kLatentCombineBf16 : kLatentCombineF16, static_cast<unsigned>(blocks * 32), 1, 1, 256, stream, args);
     }
     const int kernel = kLatentGeneral + (p.data_type == SINGE_HIP_F32 ? 0 : p.data_type == SINGE_HIP_BF16 ? 1 : 2);
     return launch(static_cast<KernelId>(kernel), static_cast<unsigned>(blocks), 1, 1, 256, stream, args);

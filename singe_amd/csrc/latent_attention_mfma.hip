@@ -144,16 +144,18 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
     const unsigned int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
     const unsigned int column = lane & 15u, g = lane >> 4;  // row of the wave, lane group
     const unsigned int splits = a.splits > 1 ? a.splits : 1u;
-    // Workgroup i runs on XCD i % 8.  Units (row tiles, in sequence order) are dealt to the XCDs in bands of
-    // a.unit_band neighbours, so that the workgroups an XCD runs side by side are row tiles of the same sequence
-    // walking the same keys, and the cache rows one of them brings into the XCD's L2 serve the others.  The splits
-    // of a unit are neighbours.
-    unsigned int split, unit;
-    {
-        const unsigned int xcd = blockIdx.x & 7u;
-        unsigned int within = blockIdx.x >> 3;
-        split = within % splits;
-        within /= splits;
+    // Workgroup i runs on XCD i % 8.  Without key splits, units (row tiles, in sequence order) are dealt to the
+    // XCDs in bands of a.unit_band neighbours, so that the workgroups an XCD runs side by side are row tiles of the
+    // same sequence walking the same keys, and the cache rows one of them brings into the XCD's L2 serve the others.
+    // With key splits the units are few and their shares read different keys: the shares of a unit are neighbouring
+    // workgroups and so go round the XCDs, which keeps every XCD busy however few units there are (and share s of
+    // every unit still meets the same few XCDs when the count of shares is a power of two).
+    unsigned int split = 0, unit;
+    if (splits > 1) {
+        split = blockIdx.x % splits;
+        unit = blockIdx.x / splits;
+    } else {
+        const unsigned int xcd = blockIdx.x & 7u, within = blockIdx.x >> 3;
         unit = ((within / a.unit_band) * 8u + xcd) * a.unit_band + within % a.unit_band;
     }
     unsigned int sequence, row_tile;
@@ -460,48 +462,69 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
 
 // Merges the shares of a row: out = sum_s 2^(lse_s - m) o_s / sum_s 2^(lse_s - m), lse = m + log2 of that sum
 // (the merge of the reference's own split kernels, kernel_plan/source/mla.rs:497-560).  One wave per (token, head)
-// row at a time, lane l dims 8 l .. 8 l + 7; a row whose shares are all empty stays zero with a log-sum-exp of -inf.
+// row, lane l dims 8 l .. 8 l + 7, kCombineBlocks workgroups of four waves to a row tile, so that a tile's 128 rows
+// are merged side by side rather than one after another; a row whose shares are all empty stays zero with a
+// log-sum-exp of -inf.  Lane s holds share s's weight (the host allows 64 shares at most), and the shares' values
+// are asked for four at a time.
+constexpr unsigned int kCombineBlocks = kRows / 4;
+
 template <class Half, int FORM>
 SINGE_DEVICE void latent_combine_rows(const LatentAttentionArgs& a) {
     const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
     // Workgroups map to (sequence, row tile) as in the attention kernel, so only rows that kernel wrote are read.
     unsigned int sequence, row_tile;
-    if (!find_unit<FORM>(a, blockIdx.x, sequence, row_tile)) return;
+    if (!find_unit<FORM>(a, blockIdx.x / kCombineBlocks, sequence, row_tile)) return;
     const SequenceSpan span = load_span<FORM>(sequence, a.query_offsets, a.page_offsets, a.last_page_lengths, nullptr, a.tokens,
                                               a.page_table, a.page_size);
     if (!span.valid) return;  // the attention kernel has reported it
     const unsigned long long rows = static_cast<unsigned long long>(span.queries) * a.heads;
     const size_t rows_total = static_cast<size_t>(a.tokens) * a.heads;
-    const unsigned long long tile_end = static_cast<unsigned long long>(row_tile + 1u) * kRows;
-    for (unsigned long long local = static_cast<unsigned long long>(row_tile) * kRows + wave; local < rows && local < tile_end; local += 4u) {
-        const size_t row = (static_cast<size_t>(span.query_start) + local / a.heads) * a.heads + local % a.heads;
-        float largest = -INFINITY;
-        for (unsigned int s = 0; s < a.splits; ++s) largest = fmaxf(largest, a.partial_lse[s * rows_total + row]);
-        float total = 0.0f, acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
-        if (largest != -INFINITY) {
-            for (unsigned int s = 0; s < a.splits; ++s) {
-                const float mine = a.partial_lse[s * rows_total + row];
-                if (mine == -INFINITY) continue;  // an empty share weighs nothing
-                const float weight = fast_exp2(mine - largest);
-                const float* part = a.partial_out + (s * rows_total + row) * kLatent + 8u * lane;
-                const float4 low = *reinterpret_cast<const float4*>(part), high = *reinterpret_cast<const float4*>(part + 4);
-                total += weight;
-                acc[0] = fmaf(weight, low.x, acc[0]); acc[1] = fmaf(weight, low.y, acc[1]);
-                acc[2] = fmaf(weight, low.z, acc[2]); acc[3] = fmaf(weight, low.w, acc[3]);
-                acc[4] = fmaf(weight, high.x, acc[4]); acc[5] = fmaf(weight, high.y, acc[5]);
-                acc[6] = fmaf(weight, high.z, acc[6]); acc[7] = fmaf(weight, high.w, acc[7]);
-            }
+    const unsigned long long local = static_cast<unsigned long long>(row_tile) * kRows + 4u * (blockIdx.x % kCombineBlocks) + wave;
+    if (local >= rows) return;
+    const size_t row = (static_cast<size_t>(span.query_start) + local / a.heads) * a.heads + local % a.heads;
+    const float mine = lane < a.splits ? a.partial_lse[lane * rows_total + row] : -INFINITY;
+    float largest = mine;
+#pragma unroll
+    for (int step = 32; step >= 1; step >>= 1) largest = fmaxf(largest, __shfl_xor(largest, step, 64));
+    // An empty share weighs nothing (its values are zeros).
+    const float weight = mine == -INFINITY ? 0.0f : fast_exp2(mine - largest);
+    float total = weight;
+#pragma unroll
+    for (int step = 32; step >= 1; step >>= 1) total += __shfl_xor(total, step, 64);
+    float acc[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    const float* part = a.partial_out + row * kLatent + 8u * lane;
+    const size_t share_stride = rows_total * kLatent;
+    auto fold = [&](float w, const float4& low, const float4& high) __attribute__((always_inline)) {
+        acc[0] = fmaf(w, low.x, acc[0]); acc[1] = fmaf(w, low.y, acc[1]);
+        acc[2] = fmaf(w, low.z, acc[2]); acc[3] = fmaf(w, low.w, acc[3]);
+        acc[4] = fmaf(w, high.x, acc[4]); acc[5] = fmaf(w, high.y, acc[5]);
+        acc[6] = fmaf(w, high.z, acc[6]); acc[7] = fmaf(w, high.w, acc[7]);
+    };
+    unsigned int s = 0;
+    for (; s + 4 <= a.splits; s += 4) {
+        float4 low[4], high[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float* from = part + (s + i) * share_stride;
+            low[i] = *reinterpret_cast<const float4*>(from);
+            high[i] = *reinterpret_cast<const float4*>(from + 4);
         }
-        const float inverse = total > 0.0f ? 1.0f / total : 0.0f;
-        const Half half{};
-        uint4 packed;
-        packed.x = pack_pair(half, acc[0] * inverse, acc[1] * inverse);
-        packed.y = pack_pair(half, acc[2] * inverse, acc[3] * inverse);
-        packed.z = pack_pair(half, acc[4] * inverse, acc[5] * inverse);
-        packed.w = pack_pair(half, acc[6] * inverse, acc[7] * inverse);
-        *reinterpret_cast<uint4*>(static_cast<unsigned char*>(a.output) + row * kLatentRowBytes + 16u * lane) = packed;
-        if (a.lse != nullptr && lane == 0) a.lse[row] = total > 0.0f ? largest + fast_log2(total) : -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) fold(__shfl(weight, s + i, 64), low[i], high[i]);
     }
+    for (; s < a.splits; ++s) {
+        const float* from = part + s * share_stride;
+        fold(__shfl(weight, s, 64), *reinterpret_cast<const float4*>(from), *reinterpret_cast<const float4*>(from + 4));
+    }
+    const float inverse = total > 0.0f ? 1.0f / total : 0.0f;
+    const Half half{};
+    uint4 packed;
+    packed.x = pack_pair(half, acc[0] * inverse, acc[1] * inverse);
+    packed.y = pack_pair(half, acc[2] * inverse, acc[3] * inverse);
+    packed.z = pack_pair(half, acc[4] * inverse, acc[5] * inverse);
+    packed.w = pack_pair(half, acc[6] * inverse, acc[7] * inverse);
+    *reinterpret_cast<uint4*>(static_cast<unsigned char*>(a.output) + row * kLatentRowBytes + 16u * lane) = packed;
+    if (a.lse != nullptr && lane == 0) a.lse[row] = total > 0.0f ? largest + fast_log2(total) : -INFINITY;
 }
 
 template <class Half>

@@ -145,6 +145,42 @@ def test_key_splits_match_the_cpu_and_the_unsplit_kernel(splits, causal, dtype):
     assert np.abs(got_lse[~empty] - whole_lse.cpu().numpy()[~empty]).max() <= 2e-3
 
 
+@pytest.mark.parametrize("sequences, heads", [([(1, 9000)], 128), ([(1, 5000), (1, 3000), (1, 16)], 16), ([(2, 4100)] * 5, 40)])
+def test_few_long_sequences_share_their_keys_out_over_the_chip(sequences, heads):
+    """The shares the library picks by itself for a decode step over few, long sequences (up to 64 of them a row
+    tile, spread round the XCDs, merged a wave per row): the scratch it asks for says how many, and the result
+    matches the CPU."""
+    import ctypes
+    from singe_amd import _native
+    page_size = 64
+    query_offsets, page_offsets, last, needed = [0], [0], [], 0
+    for queries, keys in sequences:
+        query_offsets.append(query_offsets[-1] + queries)
+        pages = (keys + page_size - 1) // page_size
+        needed += pages
+        page_offsets.append(needed)
+        last.append(keys - (pages - 1) * page_size)
+    table = [int(page) for page in np.random.default_rng(11).permutation(needed)]
+    tokens = query_offsets[-1]
+    problem = _native.PagedMlaAttentionProblemC(tokens, heads, 512, 64, page_size, len(sequences), needed, needed, 1, 0, 1, 0, 0.0)
+    shares = _native.lib().singe_hip_paged_mla_attention_scratch_bytes(ctypes.byref(problem)) // (tokens * heads * 513 * 4)
+    assert 16 < shares <= 64
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(len(sequences))
+    rand = lambda *shape: torch.randn(shape, generator=gen, device="cuda").to(torch.bfloat16)
+    device = [rand(tokens, heads, 512), rand(tokens, heads, 64), rand(needed, page_size, 512), rand(needed, page_size, 64)]
+    index = lambda entries: torch.tensor(entries, dtype=torch.int32, device="cuda")
+    paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
+    out, lse = neural.paged_mla_attention(*device, paging, neural.AttentionOptions(causal=True))
+    torch.cuda.synchronize()
+    status, want, want_lse = oracle.paged_mla_attention(*[tensor.float().cpu().numpy() for tensor in device], query_offsets, page_offsets, table,
+                                                        last, causal=True, threads=8)
+    assert status == 0
+    gap = np.abs(out.float().cpu().numpy() - want)
+    assert gap.max() <= 2e-2 and gap.mean() <= 2e-3, (gap.max(), gap.mean())
+    assert np.abs(lse.cpu().numpy() - want_lse).max() <= 5e-3
+
+
 @pytest.mark.parametrize("bad_page", [-1, 9])
 def test_matrix_core_kernel_reports_a_bad_page_and_leaves_other_sequences_right(bad_page):
     """A page id outside the cache sets the status word (its keys are read as zeros); the other sequence's rows are
