@@ -16,7 +16,11 @@ using namespace singe_hip;
 
 namespace {
 
-constexpr size_t kWarps = 4, kKeyTile = 64, kMaxShares = 16;
+constexpr size_t kWarps = 4, kKeyTile = 64;
+// Key splits: a row tile's keys go to at most kMaxShares workgroups (the merge kernels keep a share's weight per
+// lane), none with fewer than kShareTiles key tiles where the keys allow it (below that a workgroup's start, its
+// paging loads and its partial rows, outweighs what it folds).
+constexpr size_t kMaxShares = 64, kShareTiles = 8;
 constexpr uint32_t kBuiltMinBlocks = 2;
 
 // 0 = the default (twice the compute units); otherwise split_below_blocks + 1 of the installed parameters.
@@ -159,9 +163,9 @@ namespace singe_hip {
 uint32_t attention_key_splits(uint64_t workgroups, uint64_t keys) {
     const uint64_t installed = g_split_below_plus_one.load(std::memory_order_relaxed);
     const uint64_t below = installed == 0 ? default_split_below() : installed - 1;
-    if (below == 0 || workgroups == 0 || workgroups >= below || keys <= 4 * kKeyTile) return 1;
+    if (below == 0 || workgroups == 0 || workgroups >= below || keys <= kShareTiles * kKeyTile) return 1;
     uint64_t wanted = (2 * below + workgroups - 1) / workgroups;
-    const uint64_t chunks = (keys + 4 * kKeyTile - 1) / (4 * kKeyTile);
+    const uint64_t chunks = (keys + kShareTiles * kKeyTile - 1) / (kShareTiles * kKeyTile);
     wanted = wanted < chunks ? wanted : chunks;
     return static_cast<uint32_t>(wanted > kMaxShares ? kMaxShares : wanted < 1 ? 1 : wanted);
 }

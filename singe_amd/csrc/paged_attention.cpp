@@ -77,8 +77,9 @@ uint32_t paged_attention_splits(const SingePagedAttentionProblem& p) {
     // Workgroups of the unsplit grid that can have work: the list of row tiles, or one per sequence, for every kv head.
     const RowTileGrid tiling = grid_of(static_cast<uint64_t>(p.tokens), static_cast<uint64_t>(p.sequences), groups);
     const uint64_t workgroups = static_cast<uint64_t>(p.kv_heads) * (tiling.compact ? tiling.row_tiles : tiling.row_tiles * static_cast<uint64_t>(p.sequences));
-    // A sequence's key count lives in device memory: the most its pages can hold bounds it.
-    const uint64_t keys = static_cast<uint64_t>(p.page_table > 0 ? p.page_table : 0) * static_cast<uint64_t>(p.page_size);
+    // The sequences' key counts live in device memory: the page table bounds their sum, and shares are sized for
+    // a sequence of average length.
+    const uint64_t keys = static_cast<uint64_t>(p.page_table > 0 ? p.page_table : 0) * static_cast<uint64_t>(p.page_size) / static_cast<uint64_t>(p.sequences);
     return attention_key_splits(workgroups, keys);
 }
 

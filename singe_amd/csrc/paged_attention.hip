@@ -607,13 +607,23 @@ SINGE_DEVICE void combine_body(const PagedAttentionArgs& a, unsigned int shares)
         for (int step = 32; step > 0; step >>= 1) total += __shfl_xor(total, step, 64);
         float2 merged = make_float2(0.0f, 0.0f);
         const bool holds_values = 2u * lane < static_cast<unsigned int>(kHeadDim);
-        for (unsigned int s = 0; s < shares; ++s) {
+        // Four shares' values are asked for together; what a share that weighs nothing holds is not used.
+        const float* mine_of = a.partial_out + flat * kHeadDim + (holds_values ? 2u * lane : 0u);
+        const size_t share_stride = rows_total * kHeadDim;
+        auto fold = [&](unsigned int s, const float2& part) __attribute__((always_inline)) {
             const float w = __shfl(weight, s, 64);
-            if (w == 0.0f || !holds_values) continue;  // a share that weighs nothing was never meant to be read
-            const float2 part = *reinterpret_cast<const float2*>(a.partial_out + (s * rows_total + flat) * kHeadDim + 2u * lane);
-            merged.x = fmaf(w, part.x, merged.x);
-            merged.y = fmaf(w, part.y, merged.y);
+            merged.x = w == 0.0f ? merged.x : fmaf(w, part.x, merged.x);
+            merged.y = w == 0.0f ? merged.y : fmaf(w, part.y, merged.y);
+        };
+        unsigned int s = 0;
+        for (; s + 4 <= shares; s += 4) {
+            float2 part[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) part[i] = *reinterpret_cast<const float2*>(mine_of + (s + i) * share_stride);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) fold(s + i, part[i]);
         }
+        for (; s < shares; ++s) fold(s, *reinterpret_cast<const float2*>(mine_of + s * share_stride));
         const float inverse = total > 0.0f ? 1.0f / total : 0.0f;
         if (holds_values) reinterpret_cast<unsigned int*>(a.output + flat * kHeadDim)[lane] = pack_pair(Half{}, merged.x * inverse, merged.y * inverse);
         if (a.lse != nullptr && lane == 0) a.lse[flat] = total > 0.0f ? largest + fast_log2(total) : -INFINITY;

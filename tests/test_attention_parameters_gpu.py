@@ -68,10 +68,11 @@ def test_every_attention_parameter_matches_the_default():
 
 @pytest.mark.parametrize("dim", [128, 64])
 def test_candidates_agree_where_the_threshold_changes_the_shares(dim):
-    # eight decoding sequences of 2000 to 5000 keys: 16 workgroups unsplit; the candidates' thresholds give 1 to 16 shares
+    # eight decoding sequences of 8000 to 20000 keys: 16 workgroups unsplit; the candidates' thresholds give 1 to 24
+    # shares (a share keeps at least eight key tiles of a sequence of average length)
     gen = torch.Generator(device="cuda")
     gen.manual_seed(dim)
-    lens = [2000, 5000, 3100, 2047, 4096, 2500, 3333, 2049]
+    lens = [8000, 20000, 12400, 8191, 16384, 10000, 13333, 8193]
     pages_of = [(n + 15) // 16 for n in lens]
     page_count = sum(pages_of) + 3
     q = torch.randn((len(lens), 8, dim), generator=gen, device="cuda").to(torch.bfloat16)
