@@ -70,8 +70,8 @@ def traffic(key):
     return entry["FETCH_SIZE"] * FETCH_UNIT_BYTES + entry["WRITE_SIZE"] * WRITE_UNIT_BYTES, entry["source"]
 
 
-SECTIONS = ("decode", "prefill", "chunked_prefill", "fp8_decode", "dense_f32", "latent", "head_dim_64", "mfma_ceiling",
-            "hbm_ceiling")
+SECTIONS = ("decode", "prefill", "chunked_prefill", "fp8_decode", "dense_f32", "latent", "cache_append", "head_dim_64",
+            "mfma_ceiling", "hbm_ceiling")
 
 
 def parse():
@@ -448,6 +448,57 @@ def latent_section():
     return {"decode": decode, "chunked_prefill": chunked}
 
 
+def cache_append_section():
+    """The step before the chunked prefill of the fourth configuration: its 8 x 512 new tokens are normalised (RMS,
+    with a weight, queries and keys), rotated (f32 angles) and the keys and values appended to the paged cache at the
+    cells the page lists name, in one launch (rotary_cache_write): 64 query / 8 KV heads, head_dim 128, page 16, bf16.
+    HBM bound: every operand is read once and every result written once."""
+    import ctypes
+
+    import numpy as np
+    import torch
+
+    from singe_amd import _native, neural, synthetic
+
+    work = synthetic.chunked_prefill_workload(portable=True)
+    tokens, heads, groups, dim = work.query.shape[0], work.heads, work.kv_heads, work.head_dim
+    source = synthetic._PortableSource(synthetic.BASE_SEED, "cuda", "cache_append")
+    key, value = (source.normal(tensor, (tokens, groups, dim)).to(torch.bfloat16) for tensor in ("key", "value"))
+    weights = [source.normal(tensor, (dim,)).to(torch.bfloat16) for tensor in ("query_weight", "key_weight")]
+    # Token j of a sequence is its key prefix + j: angles of that position, the cell its page list gives.
+    position = np.concatenate([prefix + np.arange(work.new_tokens) for prefix in work.prefix]).astype(np.int64)
+    sequence = np.repeat(np.arange(work.sequences), work.new_tokens)
+    pages = np.asarray(work.pages)[np.asarray(work.page_offsets)[sequence] + position // work.page_size].astype(np.int32)
+    slots = (position % work.page_size).astype(np.int32)
+    angle = torch.from_numpy(position).cuda().double()[:, None] * (1e4 ** (-torch.arange(dim // 2, device="cuda").double() / (dim // 2)))[None, :]
+    cos, sin = torch.cos(angle).float().contiguous(), torch.sin(angle).float().contiguous()
+    pages, slots = torch.from_numpy(pages).cuda(), torch.from_numpy(slots).cuda()
+    rotated = torch.empty_like(work.query)
+    status = torch.zeros(1, device="cuda", dtype=torch.int32)
+    problem = _native.RotaryCacheProblemC(tokens, heads, groups, dim, work.key_cache.shape[0], work.page_size,
+                                          neural._DATA_TYPES[torch.bfloat16], neural._DATA_TYPES[torch.float32], 0, 1, 1, 1e-6, 1e-6)
+    stream = int(torch.cuda.current_stream().cuda_stream)
+
+    def launch():
+        _native.check(_native.lib().singe_hip_rotary_cache_write(
+            stream, work.query.data_ptr(), key.data_ptr(), value.data_ptr(), cos.data_ptr(), sin.data_ptr(), pages.data_ptr(),
+            slots.data_ptr(), weights[0].data_ptr(), weights[1].data_ptr(), rotated.data_ptr(), work.key_cache.data_ptr(),
+            work.value_cache.data_ptr(), status.data_ptr(), ctypes.byref(problem)), "rotary_cache_write")
+
+    stats = measure(launch, 4)
+    assert int(status.item()) == 0
+    nbytes = 2 * tokens * (heads + 2 * groups) * dim * 2 + 2 * tokens * (dim // 2) * 4 + 2 * tokens * 4 + 2 * dim * 2
+    gbps = nbytes / (stats["mean_ms"] * 1e-3) / 1e9
+    return {
+        "workload": "rotate and append (rotary_cache_write) for the fourth configuration's 4096 new tokens: 64 query / 8 KV "
+                    "heads, head_dim 128, RMS norm with weights on queries and keys, f32 angles, page 16, bf16",
+        "value": gbps, "unit": "GB/s", "us_per_step": stats["mean_ms"] * 1e3, "us_per_step_median": stats["median_ms"] * 1e3,
+        "algorithmic_bytes": nbytes,
+        "roofline": {"bound": "hbm", "kernel": "singe_rotary_cache_write_chunks_bf16", "achieved": gbps, "peak": HBM_PEAK_GBPS,
+                     "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": None, **timing_fields(stats)},
+    }
+
+
 def dense_f32_section(with_cpu=True):
     """The first benchmark configuration, the f32 accuracy anchor: causal dense attention, batch 1, 8 heads,
     512 x 512, head_dim 64, scale 1/8, tensors [batch, heads, len, dim].  Far too small for a roofline: the
@@ -732,7 +783,7 @@ def main():
     sections = {
         "prefill": lambda: prefill_section(with_cpu), "chunked_prefill": lambda: chunked_prefill_section(with_cpu),
         "fp8_decode": lambda: fp8_decode_section(with_cpu), "dense_f32": lambda: dense_f32_section(with_cpu),
-        "latent": latent_section, "head_dim_64": head_dim_64_section, "mfma_ceiling": mfma_ceiling_section,
+        "latent": latent_section, "cache_append": cache_append_section, "head_dim_64": head_dim_64_section, "mfma_ceiling": mfma_ceiling_section,
         "hbm_ceiling": hbm_ceiling_section,
     }
     if FEW:

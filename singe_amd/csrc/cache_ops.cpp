@@ -1,6 +1,7 @@
 // Host side of the rotate-and-append kernel (singe/src/backend/cuda/kernel_plan/source/rotary_cache.rs:249-427)
 // and of the CSR -> block-table paging conversion (kernel_plan/source/paged_attention.rs:325-398).
 #include <cmath>
+#include <cstdint>
 
 #include "kernel_args.h"
 #include "module.h"
@@ -63,10 +64,30 @@ extern "C" int32_t singe_hip_rotary_cache_write(void* stream, const void* query,
     args.query_eps = p.query_eps;
     args.key_eps = p.key_eps;
     const uint64_t items = static_cast<uint64_t>(p.tokens) * static_cast<uint64_t>(p.query_heads + 2 * p.cache_heads);
+    const int type_index = p.data_type == SINGE_HIP_F32 ? 0 : p.data_type == SINGE_HIP_BF16 ? 1 : 2;
+    // Sixteen bytes at a time where a head is a whole number of chunk pairs (its halves are then whole chunks, and so
+    // are the angles' rows) and every operand starts on a 16-byte boundary; a lane takes one chunk of each half.
+    const uint64_t chunk_elements = p.data_type == SINGE_HIP_F32 ? 4 : 8;
+    args.head_lanes = 0;
+    args.group_lanes = 0;
+    if (static_cast<uint64_t>(p.head_dim) % (2 * chunk_elements) == 0 && static_cast<uint64_t>(p.head_dim) / (2 * chunk_elements) <= 64) {
+        bool aligned = true;
+        const void* operands[] = {query, key, value, cos, sin, args.query_weight, args.key_weight, query_out, key_cache, value_cache};
+        for (const void* operand : operands) aligned = aligned && reinterpret_cast<uintptr_t>(operand) % 16 == 0;
+        if (aligned) {
+            args.head_lanes = static_cast<uint32_t>(static_cast<uint64_t>(p.head_dim) / (2 * chunk_elements));
+            args.group_lanes = 1;
+            while (args.group_lanes < args.head_lanes) args.group_lanes *= 2;
+        }
+    }
+    if (args.group_lanes != 0) {
+        const uint64_t blocks = (items * args.group_lanes + 255) / 256;
+        if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
+        return launch(static_cast<KernelId>(kRotaryCacheChunks + type_index), static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+    }
     const uint64_t blocks = (items + 15) / 16;  // sixteen heads of sixteen lanes per workgroup
     if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
-    const KernelId kernel = p.data_type == SINGE_HIP_F32 ? kRotaryCacheF32 : p.data_type == SINGE_HIP_BF16 ? kRotaryCacheBf16 : kRotaryCacheF16;
-    return launch(kernel, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
+    return launch(static_cast<KernelId>(kRotaryCacheF32 + type_index), static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
 }
 
 extern "C" int32_t singe_hip_paging_indices(void* stream, const void* query_offsets, const void* page_offsets, const void* pages,

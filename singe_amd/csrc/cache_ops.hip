@@ -116,6 +116,155 @@ SINGE_DEVICE void rotary_cache_write_body(const RotaryCacheArgs& a) {
     for (unsigned int dim = part; dim < a.head_dim; dim += 16) to[dim] = from[dim];
 }
 
+// The same step sixteen bytes at a time, for head dimensions that are a whole number of chunk pairs (a multiple of 16
+// elements in a 16-bit type, of 8 in f32) with every operand on a 16-byte boundary.  A head is dealt to a.group_lanes
+// neighbouring lanes (a power of two); lane c < a.head_lanes holds chunk c of the head's first half and chunk c of its
+// second half, which are each other's rotation partners, so a head moves as two loads and two stores per lane and the
+// only lane traffic is the norm's sum of squares.
+template <class E>
+struct Chunk {
+    static constexpr int kCount = 16 / sizeof(typename E::type);
+    float value[kCount];
+    static SINGE_DEVICE Chunk load(const typename E::type* from) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(from);
+        typename E::type lanes[kCount];
+        __builtin_memcpy(lanes, &raw, 16);
+        Chunk chunk;
+#pragma unroll
+        for (int i = 0; i < kCount; ++i) chunk.value[i] = E::load(lanes + i);
+        return chunk;
+    }
+    SINGE_DEVICE void store(typename E::type* to) const {
+        typename E::type lanes[kCount];
+#pragma unroll
+        for (int i = 0; i < kCount; ++i) E::store(lanes + i, value[i]);
+        uint4 raw;
+        __builtin_memcpy(&raw, lanes, 16);
+        *reinterpret_cast<uint4*>(to) = raw;
+    }
+};
+
+// COUNT consecutive angles of a table row, widened to f32.
+template <int COUNT>
+SINGE_DEVICE void table_chunk(float (&out)[COUNT], const void* table, uint32_t table_type, size_t at) {
+    if (table_type == kElementF32) {
+        const float4* from = reinterpret_cast<const float4*>(static_cast<const float*>(table) + at);
+#pragma unroll
+        for (int i = 0; i < COUNT / 4; ++i) {
+            const float4 four = from[i];
+            out[4 * i] = four.x; out[4 * i + 1] = four.y; out[4 * i + 2] = four.z; out[4 * i + 3] = four.w;
+        }
+        return;
+    }
+    unsigned short lanes[COUNT];
+    if constexpr (COUNT == 8) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(static_cast<const unsigned short*>(table) + at);
+        __builtin_memcpy(lanes, &raw, 16);
+    } else {
+        const uint2 raw = *reinterpret_cast<const uint2*>(static_cast<const unsigned short*>(table) + at);
+        __builtin_memcpy(lanes, &raw, 8);
+    }
+#pragma unroll
+    for (int i = 0; i < COUNT; ++i)
+        out[i] = table_type == kElementBf16 ? Element<kElementBf16>::load(lanes + i)
+                                            : Element<kElementF16>::load(reinterpret_cast<const _Float16*>(lanes + i));
+}
+
+template <class E>
+SINGE_DEVICE void rotate_head_chunks(typename E::type* to, const typename E::type* from, const RotaryCacheArgs& a, size_t token,
+                                     unsigned int chunk, bool live, bool has_norm, float eps, const void* weight) {
+    constexpr int kCount = Chunk<E>::kCount;
+    const unsigned int half = a.head_dim / 2, at = chunk * kCount;
+    Chunk<E> first, second;
+    if (live) {
+        first = Chunk<E>::load(from + at);
+        second = Chunk<E>::load(from + half + at);
+    }
+    if (has_norm) {
+        float squares = 0.0f;
+        if (live) {
+#pragma unroll
+            for (int i = 0; i < kCount; ++i) squares += first.value[i] * first.value[i] + second.value[i] * second.value[i];
+        }
+        for (unsigned int step = 1; step < a.group_lanes; step <<= 1) squares += __shfl_xor(squares, step, 64);
+        const float scale = rsqrtf(squares / static_cast<float>(a.head_dim) + eps);
+        if (live) {
+#pragma unroll
+            for (int i = 0; i < kCount; ++i) {
+                first.value[i] *= scale;
+                second.value[i] *= scale;
+            }
+            if (weight != nullptr) {
+                const Chunk<E> low = Chunk<E>::load(static_cast<const typename E::type*>(weight) + at);
+                const Chunk<E> high = Chunk<E>::load(static_cast<const typename E::type*>(weight) + half + at);
+#pragma unroll
+                for (int i = 0; i < kCount; ++i) {
+                    first.value[i] *= low.value[i];
+                    second.value[i] *= high.value[i];
+                }
+            }
+        }
+    }
+    if (!live) return;
+    float cosine[kCount], sine[kCount];
+    table_chunk<kCount>(cosine, a.cos, a.table_type, token * half + at);
+    table_chunk<kCount>(sine, a.sin, a.table_type, token * half + at);
+    Chunk<E> low, high;
+#pragma unroll
+    for (int i = 0; i < kCount; ++i) {
+        low.value[i] = first.value[i] * cosine[i] - second.value[i] * sine[i];
+        high.value[i] = second.value[i] * cosine[i] + first.value[i] * sine[i];
+    }
+    low.store(to + at);
+    high.store(to + half + at);
+}
+
+template <uint32_t ELEMENT>
+SINGE_DEVICE void rotary_cache_write_chunks_body(const RotaryCacheArgs& a) {
+    typedef Element<ELEMENT> E;
+    typedef typename E::type T;
+    constexpr int kCount = Chunk<E>::kCount;
+    // A group of lanes never straddles a wave (its width divides 64), and lanes of a group leave together where a
+    // shuffle follows, so the norm's exchange meets whole groups.
+    const unsigned long long thread = static_cast<unsigned long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    const unsigned long long item = thread / a.group_lanes;
+    const unsigned int chunk = static_cast<unsigned int>(thread % a.group_lanes);
+    const bool live = chunk < a.head_lanes;
+    const unsigned int total_heads = a.query_heads + 2 * a.cache_heads;
+    if (item >= static_cast<unsigned long long>(a.tokens) * total_heads) return;
+    const size_t token = static_cast<size_t>(item / total_heads);
+    const unsigned int local = static_cast<unsigned int>(item % total_heads);
+    if (local < a.query_heads) {
+        const size_t at = (token * a.query_heads + local) * a.head_dim;
+        rotate_head_chunks<E>(static_cast<T*>(a.query_out) + at, static_cast<const T*>(a.query) + at, a, token, chunk, live,
+                              a.has_query_norm != 0, a.query_eps, a.query_weight);
+        return;
+    }
+    long long page = a.wide_index ? static_cast<const long long*>(a.pages)[token] : static_cast<const int*>(a.pages)[token];
+    long long slot = a.wide_index ? static_cast<const long long*>(a.slots)[token] : static_cast<const int*>(a.slots)[token];
+    if (page < 0) page += a.cache_pages;
+    if (slot < 0) slot += a.page_slots;
+    if (page < 0 || page >= static_cast<long long>(a.cache_pages) || slot < 0 || slot >= static_cast<long long>(a.page_slots)) {
+        if (chunk == 0) report_index_error(a.status);
+        return;
+    }
+    const size_t cell = (static_cast<size_t>(page) * a.page_slots + static_cast<size_t>(slot)) * a.cache_heads;
+    if (local < a.query_heads + a.cache_heads) {
+        const unsigned int head = local - a.query_heads;
+        rotate_head_chunks<E>(static_cast<T*>(a.key_cache) + (cell + head) * a.head_dim,
+                              static_cast<const T*>(a.key) + (token * a.cache_heads + head) * a.head_dim, a, token, chunk, live,
+                              a.has_key_norm != 0, a.key_eps, a.key_weight);
+        return;
+    }
+    if (!live) return;
+    const unsigned int head = local - a.query_heads - a.cache_heads, half = a.head_dim / 2;
+    const T* from = static_cast<const T*>(a.value) + (token * a.cache_heads + head) * a.head_dim + chunk * kCount;
+    T* to = static_cast<T*>(a.value_cache) + (cell + head) * a.head_dim + chunk * kCount;
+    const uint4 low = *reinterpret_cast<const uint4*>(from), high = *reinterpret_cast<const uint4*>(from + half);
+    *reinterpret_cast<uint4*>(to) = low;
+    *reinterpret_cast<uint4*>(to + half) = high;
+}
+
 template <bool WIDE>
 SINGE_DEVICE void paging_indices_body(const PagingIndicesArgs& a) {
     constexpr int FORM = WIDE ? kCsrI64 : kCsrI32;
@@ -167,6 +316,15 @@ extern "C" __global__ __launch_bounds__(256) void singe_rotary_cache_write_bf16(
 }
 extern "C" __global__ __launch_bounds__(256) void singe_rotary_cache_write_f16(RotaryCacheArgs args) {
     cache_ops::rotary_cache_write_body<kElementF16>(args);
+}
+extern "C" __global__ __launch_bounds__(256) void singe_rotary_cache_write_chunks_f32(RotaryCacheArgs args) {
+    cache_ops::rotary_cache_write_chunks_body<kElementF32>(args);
+}
+extern "C" __global__ __launch_bounds__(256) void singe_rotary_cache_write_chunks_bf16(RotaryCacheArgs args) {
+    cache_ops::rotary_cache_write_chunks_body<kElementBf16>(args);
+}
+extern "C" __global__ __launch_bounds__(256) void singe_rotary_cache_write_chunks_f16(RotaryCacheArgs args) {
+    cache_ops::rotary_cache_write_chunks_body<kElementF16>(args);
 }
 extern "C" __global__ __launch_bounds__(256) void singe_paging_indices_i32(PagingIndicesArgs args) {
     cache_ops::paging_indices_body<false>(args);

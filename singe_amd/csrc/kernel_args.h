@@ -313,6 +313,9 @@ struct RotaryCacheArgs {
     uint32_t wide_index;
     uint32_t has_query_norm, has_key_norm;
     float query_eps, key_eps;
+    // The 16-byte kernels (singe_rotary_cache_write_chunks_*): a head's lanes that hold data, and the power of two of
+    // neighbouring lanes it is dealt to.
+    uint32_t head_lanes, group_lanes;
 };
 
 // singe_paging_indices_*: FlashInfer CSR paging -> block-table paging.

@@ -213,6 +213,7 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_decode_f16_wide_d128_b16", "singe_paged_decode_f16_wide_d128_any",
     "singe_paged_decode_combine_many_bf16", "singe_paged_decode_combine_many_f16",
     "singe_paged_decode_combine_many_bf16_d64", "singe_paged_decode_combine_many_f16_d64",
+    "singe_rotary_cache_write_chunks_f32", "singe_rotary_cache_write_chunks_bf16", "singe_rotary_cache_write_chunks_f16",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -246,6 +247,7 @@ constexpr PartRun kPartRuns[] = {
     {22, 10}, {23, 28}, {24, 10}, {25, 28}, {26, 10}, {27, 28}, {28, 10}, {29, 28},  // and those for 16, 48, 80, 112
     {0, 4},                       // the wide decode kernels for bf16 / f16 caches
     {0, 2}, {13, 2},              // the decode merge for rows with many slots, head_dim 128 and 64
+    {6, 3},                       // rotate-and-append sixteen bytes at a time
 };
 constexpr int runs_total() {
     int total = 0;

@@ -66,6 +66,8 @@ enum KernelId : int {
     kDecodeWide = kOtherHeadDims + 6 * (10 + (kSplitKReduce - kPagedAttentionI32)),
     // the decode merge for rows with many slots: bf16, f16, then the same for head_dim 64
     kDecodeCombineMany = kDecodeWide + 4, kDecodeCombineManyF16, kDecodeCombineManyD64, kDecodeCombineManyF16D64,
+    // rotate-and-append sixteen bytes at a time: f32, bf16, f16
+    kRotaryCacheChunks, kRotaryCacheChunksBf16, kRotaryCacheChunksF16,
     kKernelCount
 };
 

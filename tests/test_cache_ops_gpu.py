@@ -60,6 +60,40 @@ def test_rotary_cache_write(dtype, table_dtype, index_dtype):
     rotary_case(dtype, table_dtype, index_dtype, tokens=64, heads=4, groups=1, dim=64, pages=8, slots=16, seed=3, with_query=False)
 
 
+@pytest.mark.parametrize("dtype,table_dtype", [(torch.float32, torch.bfloat16), (torch.bfloat16, torch.float32), (torch.float16, torch.float16)])
+def test_rotary_cache_write_sixteen_bytes_at_a_time_and_element_by_element(dtype, table_dtype):
+    """Head dimensions that are a whole number of 16-byte chunk pairs move a chunk of each half per lane (head_dim 96
+    and 80 leave lanes of a head's group idle, 256 and 512 take 16 to 64 lanes a head); 24, 40 and 6 (bf16 / f16; 6 and
+    20 in f32) are not, and go element by element, as do operands off a 16-byte boundary."""
+    for seed, dim in enumerate([96, 256, 512, 32, 16, 24, 40, 6, 20]):
+        rotary_case(dtype, table_dtype, torch.int32, tokens=19, heads=5, groups=2, dim=dim, pages=5, slots=4, seed=20 + seed, norms=seed % 2 == 0)
+    rotary_case(dtype, table_dtype, torch.int32, tokens=700, heads=16, groups=4, dim=128, pages=50, slots=16, seed=31, norms=True)
+
+
+def test_rotary_cache_write_off_a_sixteen_byte_boundary():
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(5)
+    tokens, heads, groups, dim, pages, slots = 9, 4, 2, 64, 3, 4
+    rand = lambda *shape: torch.randn(shape, generator=gen, device="cuda").to(torch.bfloat16)
+    q, k, v = rand(tokens, heads, dim), rand(tokens, groups, dim), rand(tokens, groups, dim)
+    angle = torch.rand((tokens * (dim // 2) + 1,), generator=gen, device="cuda") * 6.28
+    cells = np.random.default_rng(5).permutation(pages * slots)[:tokens]
+    index = lambda values: torch.tensor(values, dtype=torch.int32, device="cuda")
+    results = []
+    for shift in (0, 1):  # the same angles on and off the boundary
+        table = lambda values: torch.cat([values.new_zeros(shift), values[:tokens * (dim // 2)]])[shift:].view(tokens, 1, dim // 2)
+        cos, sin = table(torch.cos(angle)), table(torch.sin(angle))
+        assert cos.data_ptr() % 16 == 4 * shift
+        kc, vc = torch.zeros((pages, slots, groups, dim), dtype=torch.bfloat16, device="cuda"), torch.zeros((pages, slots, groups, dim), dtype=torch.bfloat16, device="cuda")
+        out = neural.rotary_cache_write(q, k, v, cos, sin, index(cells // slots), index(cells % slots), kc, vc,
+                                        key_norm=neural.RotationNorm(1e-5, None))
+        results.append((out, kc, vc))
+    torch.cuda.synchronize()
+    for aligned, shifted in zip(*results):
+        assert (aligned.float() - shifted.float()).abs().max().item() <= 2 ** -6  # one unit in the last place of values below 4
+    assert torch.equal(results[0][2], results[1][2])
+
+
 def test_rotary_cache_write_decode_step_shape():
     """One decode step of the headline shape: 32 tokens, 32 query / 8 KV heads, head_dim 128, block 16."""
     rotary_case(torch.bfloat16, torch.float32, torch.int32, tokens=32, heads=32, groups=8, dim=128, pages=64, slots=16, seed=9,
