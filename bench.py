@@ -382,6 +382,31 @@ def chunked_prefill_section(with_cpu=True):
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": nbytes, "traffic_source": source, **timing_fields(stats)},
     }
+    # The same attention with the query's RMS norm and rotation fused into the kernel (rotary_paged_attention): the
+    # query is normalised, rotated and rounded on its way into the registers, which spares the two-step form's
+    # write and re-read of the rotated query.
+    tokens, half = work.query.shape[0], work.head_dim // 2
+    position = np.concatenate([prefix + np.arange(work.new_tokens) for prefix in work.prefix]).astype(np.float64)
+    angle = torch.from_numpy(position).cuda()[:, None] * (1e4 ** (-torch.arange(half, device="cuda").double() / half))[None, :]
+    cos, sin = torch.cos(angle).float().contiguous(), torch.sin(angle).float().contiguous()
+    weight = synthetic.portable_normal("chunked_prefill.query_weight", (work.head_dim,), torch.bfloat16)
+    rotation = _native.QueryRotationC(neural._DATA_TYPES[torch.float32], 1, 1e-6)
+
+    def launch_fused():
+        _native.check(_native.lib().singe_hip_rotary_paged_attention_bf16(
+            handle, work.query.data_ptr(), work.key_cache.data_ptr(), work.value_cache.data_ptr(),
+            paging.query_offsets.data_ptr(), paging.page_offsets.data_ptr(), paging.pages.data_ptr(),
+            paging.last_page_lengths.data_ptr(), cos.data_ptr(), sin.data_ptr(), weight.data_ptr(), out.data_ptr(), lse.data_ptr(),
+            status.data_ptr(), ctypes.byref(problem), ctypes.byref(rotation)), "rotary_paged_attention")
+
+    fused = measure(launch_fused, 4)
+    assert int(status.item()) == 0
+    result["fused_query_rotation"] = {
+        "workload": "the same attention with the query's RMS norm (with a weight) and rotation (f32 angles) done by the "
+                    "attention kernel (rotary_paged_attention)",
+        "kernel": "singe_rotary_paged_attention_bf16_d128_i32_p16", "ms_per_step": fused["mean_ms"],
+        "ms_per_step_median": fused["median_ms"], "tflops": flops / (fused["mean_ms"] * 1e-3) / 1e12,
+        "over_plain_attention_us": (fused["mean_ms"] - stats["mean_ms"]) * 1e3, **timing_fields(fused)}
     if with_cpu:
         result["cpu_baseline"] = chunked_prefill_cpu_baseline(work)
     return result

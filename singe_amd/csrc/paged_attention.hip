@@ -45,6 +45,31 @@ SINGE_DEVICE float table_value(const void* table, uint32_t table_type, size_t at
     return static_cast<float>(static_cast<const _Float16*>(table)[at]);
 }
 
+// Eight consecutive values of such a table, the index a multiple of eight: as one or two 16-byte loads when the table
+// starts on a 16-byte boundary, one by one otherwise.
+SINGE_DEVICE void table_values8(float (&out)[8], const void* table, uint32_t table_type, size_t at) {
+    if (reinterpret_cast<uintptr_t>(table) % 16 != 0) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) out[i] = table_value(table, table_type, at + i);
+        return;
+    }
+    if (table_type == kElementF32) {
+        const float4* from = reinterpret_cast<const float4*>(static_cast<const float*>(table) + at);
+        const float4 low = from[0], high = from[1];
+        out[0] = low.x; out[1] = low.y; out[2] = low.z; out[3] = low.w;
+        out[4] = high.x; out[5] = high.y; out[6] = high.z; out[7] = high.w;
+        return;
+    }
+    const uint4 raw = *reinterpret_cast<const uint4*>(static_cast<const unsigned short*>(table) + at);
+    const unsigned int words[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const unsigned short bits = static_cast<unsigned short>(words[i / 2] >> (16 * (i % 2)));
+        out[i] = table_type == kElementBf16 ? __builtin_bit_cast(float, static_cast<unsigned int>(bits) << 16)
+                                            : static_cast<float>(__builtin_bit_cast(_Float16, bits));
+    }
+}
+
 constexpr unsigned int kNoPage = 0xFFFFFFFFu;  // a table entry outside the cache: reported, never read through
 
 // Workgroup id -> (unit = sequence * kv_heads + kv head, row tile, key split); false for ids past the units.
@@ -277,27 +302,35 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
             // (Pairs are dims i and i + head_dim / 2, whole steps apart at multiples of 32; the launcher sends the other
             // head dimensions to the two-step form.)
             constexpr int kPairs = kHeadDim / 2, kHalfSteps = kSteps / 2;
+            const bool weighted = a.has_query_norm != 0 && a.query_weight != nullptr;
 #pragma unroll
             for (int s = 0; s < kHalfSteps; ++s) {
                 unsigned int first_words[4] = {bits[s].x, bits[s].y, bits[s].z, bits[s].w};
                 unsigned int second_words[4] = {bits[s + kHalfSteps].x, bits[s + kHalfSteps].y, bits[s + kHalfSteps].z, bits[s + kHalfSteps].w};
+                // The lane's eight pairs of this step are neighbours: their angles and weights come as whole chunks.
+                const unsigned int first_pair = 16u * s + 8u * hi;
+                float cosines[8], sines[8], low_weights[8], high_weights[8];
+                table_values8(cosines, a.cos, a.table_type, token * kPairs + first_pair);
+                table_values8(sines, a.sin, a.table_type, token * kPairs + first_pair);
+                if (weighted) {
+                    table_values8(low_weights, a.query_weight, kElementBf16, first_pair);
+                    table_values8(high_weights, a.query_weight, kElementBf16, first_pair + kPairs);
+                }
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
                     float rotated_first[2], rotated_second[2];
 #pragma unroll
                     for (int upper = 0; upper < 2; ++upper) {
-                        const unsigned int pair = 16u * s + 8u * hi + 2u * w + upper;
                         float first = wide(first_words[w], upper), second = wide(second_words[w], upper);
                         if (a.has_query_norm != 0) {
                             first *= scale;
                             second *= scale;
-                            if (a.query_weight != nullptr) {
-                                first *= __builtin_bit_cast(float, static_cast<unsigned int>(a.query_weight[pair]) << 16);
-                                second *= __builtin_bit_cast(float, static_cast<unsigned int>(a.query_weight[pair + kPairs]) << 16);
+                            if (weighted) {
+                                first *= low_weights[2 * w + upper];
+                                second *= high_weights[2 * w + upper];
                             }
                         }
-                        const float cosine = table_value(a.cos, a.table_type, token * kPairs + pair);
-                        const float sine = table_value(a.sin, a.table_type, token * kPairs + pair);
+                        const float cosine = cosines[2 * w + upper], sine = sines[2 * w + upper];
                         rotated_first[upper] = first * cosine - second * sine;
                         rotated_second[upper] = second * cosine + first * sine;
                     }
