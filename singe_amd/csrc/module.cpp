@@ -214,6 +214,8 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_decode_combine_many_bf16", "singe_paged_decode_combine_many_f16",
     "singe_paged_decode_combine_many_bf16_d64", "singe_paged_decode_combine_many_f16_d64",
     "singe_rotary_cache_write_chunks_f32", "singe_rotary_cache_write_chunks_bf16", "singe_rotary_cache_write_chunks_f16",
+    "singe_paged_decode_combine_few_bf16", "singe_paged_decode_combine_few_f16",
+    "singe_paged_decode_combine_few_bf16_d64", "singe_paged_decode_combine_few_f16_d64",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -248,6 +250,7 @@ constexpr PartRun kPartRuns[] = {
     {0, 4},                       // the wide decode kernels for bf16 / f16 caches
     {0, 2}, {13, 2},              // the decode merge for rows with many slots, head_dim 128 and 64
     {6, 3},                       // rotate-and-append sixteen bytes at a time
+    {0, 2}, {13, 2},              // the decode merge for rows with one or two slots, head_dim 128 and 64
 };
 constexpr int runs_total() {
     int total = 0;

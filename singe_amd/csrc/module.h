@@ -68,6 +68,8 @@ enum KernelId : int {
     kDecodeCombineMany = kDecodeWide + 4, kDecodeCombineManyF16, kDecodeCombineManyD64, kDecodeCombineManyF16D64,
     // rotate-and-append sixteen bytes at a time: f32, bf16, f16
     kRotaryCacheChunks, kRotaryCacheChunksBf16, kRotaryCacheChunksF16,
+    // the decode merge for rows with one or two slots: bf16, f16, then the same for head_dim 64
+    kDecodeCombineFew, kDecodeCombineFewF16, kDecodeCombineFewD64, kDecodeCombineFewF16D64,
     kKernelCount
 };
 

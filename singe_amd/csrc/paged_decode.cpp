@@ -303,6 +303,12 @@ int32_t decode(
         const KernelId many = static_cast<KernelId>(kDecodeCombineMany + (f16 ? 1 : 0) + (narrow ? 2 : 0));
         return launch(many, static_cast<unsigned>(c.batch * c.heads), 1, 1, 512, stream, combine);
     }
+    // With no more workers than sequences a row has one or two slots, and the kernel that fetches four rows at a time
+    // keeps twice the waves in flight.
+    if (static_cast<size_t>(plan.workers) <= c.batch) {
+        const KernelId few = static_cast<KernelId>(kDecodeCombineFew + (f16 ? 1 : 0) + (narrow ? 2 : 0));
+        return launch(few, static_cast<unsigned>((c.batch * c.heads + 3) / 4), 1, 1, 256, stream, combine);
+    }
     const KernelId merge = f16 ? kDecodeF16Combine : kDecodeCombine;
     return launch(narrow ? at_head_dim_64(merge) : merge, static_cast<unsigned>((c.batch * c.heads + 3) / 4), 1, 1, 256, stream, combine);
 }

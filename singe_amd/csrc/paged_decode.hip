@@ -817,8 +817,10 @@ SINGE_DECODE_WIDE_KERNEL(singe_paged_decode_f8kv_wide_relaxed_d128_any, false, f
 // out = sum_s exp(lse_s - max) * partial_s / sum_s exp(lse_s - max)
 // (singe-kernel/src/cpu/attention.rs:2157-2193).  One wave per row.  The kernel is a chain of dependent
 // memory round trips, so it is written to need few of them: lane s fetches the log-sum-exp of slot s
-// (one trip for up to 64 slots), and the slots' rows are fetched sixteen at a time, two dims per lane.
-template <bool F16>
+// (one trip for up to 64 slots), and the slots' rows are fetched FIRST (sixteen) at a time, two dims per lane.  When
+// rows have one or two slots (more sequences than workers) the kernel's time is rounds of waves times its chain of
+// round trips, and the sixteen rows' registers hold it to twelve waves a compute unit: the _few kernels fetch four.
+template <bool F16, int FIRST = 16>
 SINGE_DEVICE void paged_decode_combine_body(const CombineArgs& a) {
     const unsigned int lane = threadIdx.x & 63;
     const unsigned int row = blockIdx.x * 4 + (threadIdx.x >> 6);  // batch * heads + head
@@ -840,12 +842,12 @@ SINGE_DEVICE void paged_decode_combine_body(const CombineArgs& a) {
             const unsigned int n = count - chunk < 64 ? count - chunk : 64;
             const size_t chunk_base = base + static_cast<size_t>(chunk) * a.heads_per_wave;
             const float mine = lane < n ? a.partial_lse[chunk_base + static_cast<size_t>(lane) * a.heads_per_wave] : -INFINITY;
-            // The first sixteen rows are asked for together with the log-sum-exps, before anything waits for those: a
+            // The first FIRST rows are asked for together with the log-sum-exps, before anything waits for those: a
             // sequence rarely has more slots, and the kernel is a chain of memory round trips.
-            float2 rows[16];
+            float2 rows[FIRST];
             auto fetch = [&](unsigned int first) __attribute__((always_inline)) {
 #pragma unroll
-                for (int j = 0; j < 16; ++j) {
+                for (int j = 0; j < FIRST; ++j) {
                     rows[j] = make_float2(0.0f, 0.0f);
                     if (first + j < n && holds_values)
                         rows[j] = *reinterpret_cast<const float2*>(a.partial_out + (chunk_base + static_cast<size_t>(first + j) * a.heads_per_wave) * kDim + 2 * lane);
@@ -866,10 +868,10 @@ SINGE_DEVICE void paged_decode_combine_body(const CombineArgs& a) {
             low *= rescale;
             high *= rescale;
             best = largest;
-            for (unsigned int first = 0; first < n; first += 16) {
+            for (unsigned int first = 0; first < n; first += FIRST) {
                 if (first != 0) fetch(first);
 #pragma unroll
-                for (int j = 0; j < 16; ++j) {
+                for (int j = 0; j < FIRST; ++j) {
                     const float w = __shfl(weight, static_cast<int>(first) + j, 64);
                     if (first + j < n) {
                         low = fmaf(w, rows[j].x, low);
@@ -994,6 +996,14 @@ extern "C" __global__ __launch_bounds__(512) void singe_paged_decode_combine_man
 #else
 extern "C" __global__ __launch_bounds__(512) void SINGE_DECODE_NAME(singe_paged_decode_combine_many_bf16, /**/)(CombineArgs a) { paged_decode_combine_many_body<false>(a); }
 extern "C" __global__ __launch_bounds__(512) void SINGE_DECODE_NAME(singe_paged_decode_combine_many_f16, /**/)(CombineArgs a) { paged_decode_combine_many_body<true>(a); }
+#endif
+
+#if SINGE_HEAD_DIM == 128
+extern "C" __global__ __launch_bounds__(256) void singe_paged_decode_combine_few_bf16(CombineArgs a) { paged_decode_combine_body<false, 4>(a); }
+extern "C" __global__ __launch_bounds__(256) void singe_paged_decode_combine_few_f16(CombineArgs a) { paged_decode_combine_body<true, 4>(a); }
+#else
+extern "C" __global__ __launch_bounds__(256) void SINGE_DECODE_NAME(singe_paged_decode_combine_few_bf16, /**/)(CombineArgs a) { paged_decode_combine_body<false, 4>(a); }
+extern "C" __global__ __launch_bounds__(256) void SINGE_DECODE_NAME(singe_paged_decode_combine_few_f16, /**/)(CombineArgs a) { paged_decode_combine_body<true, 4>(a); }
 #endif
 
 #if SINGE_HEAD_DIM == 128
