@@ -278,6 +278,21 @@ def test_decode_phases_and_scratch_reuse():
             assert torch.equal(both.view(torch.int16), apart.view(torch.int16))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("head_dim", [128, 64])
+def test_no_more_workers_than_sequences_fold_rows_four_slots_at_a_time(head_dim, dtype):
+    """With no more workers than sequences the reduce fetches a row's slots four at a time: most rows have one or two,
+    and the one long sequence here has one in nearly every worker's range."""
+    lens = [3000, 1, 40, 0, 17, 5, 64, 33, 2, 90]
+    work = synthetic.paged_decode_workload(batch=len(lens), heads=8, kv_heads=2, head_dim=head_dim, physical_blocks=256, seq_lens=lens,
+                                           seed=31)
+    for workers in (10, 7):
+        got, want = run_gpu(work, workers, dtype=dtype), run_oracle(work)
+        assert not got[3].any()
+        gap = np.abs(got - want)
+        assert gap.max() <= MAX_ABS and gap.mean() <= MEAN_ABS, (workers, gap.max(), gap.mean())
+
+
 def test_decode_one_long_sequence_spans_more_than_64_ranges():
     """A single sequence cut into more key ranges than a wave has lanes: the reduce walks its slots in
     chunks."""
