@@ -294,6 +294,63 @@ def dense_f32_cpu_baseline(q, k, v):
             "host": host_description()}
 
 
+def latent_cpu_baseline(operands, keys, page, heads, sample=8):
+    """Tensor::paged_mla_attention's CPU form (singe/src/backend/cpu/normalization/attention.rs:540-679, f64
+    arithmetic, serial in the reference) on the first `sample` sequences of the decode workload, each with its pages
+    gathered into a cache of their own: single thread, then the head rows over the host's cores."""
+    import oracle
+
+    latent_queries, positional_queries, latent_cache, positional_cache, table = operands
+    count = (keys + page - 1) // page
+    host = lambda tensor: tensor.float().cpu().numpy()
+    times = {1: 0.0, cpu_threads(): 0.0}
+    for sequence in range(sample):
+        index = table[sequence * count:(sequence + 1) * count]
+        inputs = (host(latent_queries[sequence:sequence + 1]), host(positional_queries[sequence:sequence + 1]), host(latent_cache[index]),
+                  host(positional_cache[index]))
+        for threads in times:
+            start = time.perf_counter()
+            status, _, _ = oracle.paged_mla_attention(*inputs, [0, 1], [0, count], list(range(count)), [keys - (count - 1) * page],
+                                                      causal=True, threads=threads)
+            times[threads] += time.perf_counter() - start
+            assert status == 0
+    nbytes = sample * (keys * 1152 + heads * (576 + 512) * 2)
+    serial, spread = times[1], times[cpu_threads()]
+    return {"value": nbytes / serial / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"the first {sample} of the 256 sequences ({keys} keys, {heads} heads each), single thread ({serial:.1f} s); "
+                      f"bytes counted as for the GPU figure",
+            "row_parallel": {"value": nbytes / spread / 1e9, "unit": "GB/s", "cores": cpu_threads(),
+                             "sample": f"the same sequences, head rows over {cpu_threads()} threads ({spread:.2f} s)"},
+            "host": host_description()}
+
+
+def cache_append_cpu_baseline(query, key, value, cos, sin, weights, page_slots, sample=4096):
+    """The rotate-and-append step (singe/src/backend/cuda/kernel_plan/source/rotary_cache.rs:249-427; norm and rotation
+    rotary_cache.rs:92-185) restated in the oracle, single thread, on the first `sample` tokens of the workload,
+    appended to a cache that holds just their cells."""
+    import numpy as np
+
+    import oracle
+
+    host = lambda tensor: tensor[:sample].float().cpu().numpy()
+    q, k, v, c, s = host(query), host(key), host(value), host(cos), host(sin)
+    groups, dim = k.shape[1:]
+    pages = (sample + page_slots - 1) // page_slots
+    caches = [np.zeros((pages, page_slots, groups, dim), dtype=np.float32) for _ in range(2)]
+    cells = np.random.default_rng(4).permutation(pages * page_slots)[:sample]
+    norms = [(1e-6, weight.float().cpu().numpy()) for weight in weights]
+    start = time.perf_counter()
+    status, _, _, _ = oracle.rotary_cache_write_f32(q, k, v, c, s, cells // page_slots, cells % page_slots, caches[0], caches[1],
+                                                    query_norm=norms[0], key_norm=norms[1], in_place=True)
+    elapsed = time.perf_counter() - start
+    assert status == 0
+    nbytes = 2 * sample * (q.shape[1] + 2 * groups) * dim * 2 + 2 * sample * (dim // 2) * 4 + 2 * sample * 4
+    return {"value": nbytes / elapsed / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"the first {sample} of the workload's {query.shape[0]} tokens, single thread ({elapsed:.2f} s); bytes "
+                      f"counted as for the GPU figure (bf16 operands)",
+            "host": host_description()}
+
+
 # ---- GPU sections ----------------------------------------------------------------------------------------------------
 
 def prefill_section(with_cpu=True, dim=128, key="prefill"):
@@ -412,7 +469,7 @@ def chunked_prefill_section(with_cpu=True):
     return result
 
 
-def latent_section():
+def latent_section(with_cpu=True):
     """Latent (MLA) attention over paged caches at DeepSeek's widths (latent 512, positional 64, 128 heads, bf16,
     page 64), beside the benchmark's configurations: a decode step (256 sequences of 4096 keys; every head reads
     the same 1152 bytes per key, so the step is priced against HBM and the matrix cores both) and a chunked
@@ -445,9 +502,9 @@ def latent_section():
         pairs = sum(sum(min(keys, max(keys - queries + i, 0) + 1) for i in range(queries)) for queries, keys in sequences)
         flops = pairs * heads * (576 + 512) * 2
         cache_bytes = sum(keys for _, keys in sequences) * 1152 + tokens * heads * (576 + 512) * 2
-        return stats, flops, cache_bytes
+        return stats, flops, cache_bytes, (*operands, torch.tensor(table, device="cuda"))
 
-    stats, flops, cache_bytes = case([(1, 4096)] * 256, 4)
+    stats, flops, cache_bytes, decode_operands = case([(1, 4096)] * 256, 4)
     gbps, tflops = cache_bytes / (stats["mean_ms"] * 1e-3) / 1e9, flops / (stats["mean_ms"] * 1e-3) / 1e12
     nbytes, source = traffic("latent_decode")
     decode = {
@@ -458,7 +515,10 @@ def latent_section():
                      "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": nbytes, "traffic_source": source,
                      "mfma_frac": tflops / MFMA_BF16_PEAK_TFLOPS, **timing_fields(stats)},
     }
-    stats, flops, cache_bytes = case([(512, 8192)] * 8, 1)
+    if with_cpu:
+        decode["cpu_baseline"] = latent_cpu_baseline(decode_operands, 4096, 64, 128)
+    del decode_operands
+    stats, flops, cache_bytes, _ = case([(512, 8192)] * 8, 1)
     tflops = flops / (stats["mean_ms"] * 1e-3) / 1e12
     nbytes, source = traffic("latent_chunked_prefill")
     chunked = {
@@ -473,7 +533,7 @@ def latent_section():
     return {"decode": decode, "chunked_prefill": chunked}
 
 
-def cache_append_section():
+def cache_append_section(with_cpu=True):
     """The step before the chunked prefill of the fourth configuration: its 8 x 512 new tokens are normalised (RMS,
     with a weight, queries and keys), rotated (f32 angles) and the keys and values appended to the paged cache at the
     cells the page lists name, in one launch (rotary_cache_write): 64 query / 8 KV heads, head_dim 128, page 16, bf16.
@@ -514,7 +574,7 @@ def cache_append_section():
     assert int(status.item()) == 0
     nbytes = 2 * tokens * (heads + 2 * groups) * dim * 2 + 2 * tokens * (dim // 2) * 4 + 2 * tokens * 4 + 2 * dim * 2
     gbps = nbytes / (stats["mean_ms"] * 1e-3) / 1e9
-    return {
+    result = {
         "workload": "rotate and append (rotary_cache_write) for the fourth configuration's 4096 new tokens: 64 query / 8 KV "
                     "heads, head_dim 128, RMS norm with weights on queries and keys, f32 angles, page 16, bf16",
         "value": gbps, "unit": "GB/s", "us_per_step": stats["mean_ms"] * 1e3, "us_per_step_median": stats["median_ms"] * 1e3,
@@ -522,6 +582,9 @@ def cache_append_section():
         "roofline": {"bound": "hbm", "kernel": "singe_rotary_cache_write_chunks_bf16", "achieved": gbps, "peak": HBM_PEAK_GBPS,
                      "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": None, **timing_fields(stats)},
     }
+    if with_cpu:
+        result["cpu_baseline"] = cache_append_cpu_baseline(work.query, key, value, cos, sin, weights, work.page_size)
+    return result
 
 
 def dense_f32_section(with_cpu=True):
@@ -808,7 +871,8 @@ def main():
     sections = {
         "prefill": lambda: prefill_section(with_cpu), "chunked_prefill": lambda: chunked_prefill_section(with_cpu),
         "fp8_decode": lambda: fp8_decode_section(with_cpu), "dense_f32": lambda: dense_f32_section(with_cpu),
-        "latent": latent_section, "cache_append": cache_append_section, "head_dim_64": head_dim_64_section, "mfma_ceiling": mfma_ceiling_section,
+        "latent": lambda: latent_section(with_cpu), "cache_append": lambda: cache_append_section(with_cpu),
+        "head_dim_64": head_dim_64_section, "mfma_ceiling": mfma_ceiling_section,
         "hbm_ceiling": hbm_ceiling_section,
     }
     if FEW:

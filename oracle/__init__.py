@@ -367,13 +367,16 @@ def rotary_embedding_f32(values, cos, sin):
 
 
 def rotary_cache_write_f32(query, key, value, cos, sin, pages, slots, key_cache, value_cache, *, query_norm=None,
-                           key_norm=None):
+                           key_norm=None, in_place=False):
     """The fused rotate-and-append step (singe/src/backend/cuda/kernel_plan/source/rotary_cache.rs:249-427).
     query [T, H, D] or None, key/value [T, G, D], cos/sin [T, D/2], caches [P, S, G, D] (copied, then the
-    selected cells written); a norm is (eps, weight or None).  Returns (status, query_out, key_cache,
-    value_cache)."""
+    selected cells written; ``in_place`` writes into the caches given, contiguous float32 arrays, instead, for
+    timing); a norm is (eps, weight or None).  Returns (status, query_out, key_cache, value_cache)."""
     key, value, cos, sin = _f32(key), _f32(value), _f32(cos), _f32(sin)
-    key_cache, value_cache = _f32(key_cache).copy(), _f32(value_cache).copy()
+    if in_place:
+        assert all(c.dtype == np.float32 and c.flags["C_CONTIGUOUS"] for c in (key_cache, value_cache))
+    else:
+        key_cache, value_cache = _f32(key_cache).copy(), _f32(value_cache).copy()
     tokens, cache_heads, head_dim = key.shape
     cache_pages, page_slots = key_cache.shape[:2]
     query_heads = 0 if query is None else query.shape[1]
