@@ -59,6 +59,8 @@ COUNTER_TRAFFIC = {
                       "source": "profiles/hbm_traffic_counters.md"},
     "latent_chunked_prefill": {"kernel": "singe_paged_mla_attention_bf16_l512_p64", "FETCH_SIZE": 868387,
                                "WRITE_SIZE": 526766, "source": "profiles/hbm_traffic_counters.md"},
+    "cache_append": {"kernel": "singe_rotary_cache_write_chunks_bf16", "FETCH_SIZE": 44244, "WRITE_SIZE": 81920,
+                     "source": "profiles/hbm_traffic_counters.md"},
 }
 
 
@@ -574,13 +576,15 @@ def cache_append_section(with_cpu=True):
     assert int(status.item()) == 0
     nbytes = 2 * tokens * (heads + 2 * groups) * dim * 2 + 2 * tokens * (dim // 2) * 4 + 2 * tokens * 4 + 2 * dim * 2
     gbps = nbytes / (stats["mean_ms"] * 1e-3) / 1e9
+    counted, source = traffic("cache_append")
     result = {
         "workload": "rotate and append (rotary_cache_write) for the fourth configuration's 4096 new tokens: 64 query / 8 KV "
                     "heads, head_dim 128, RMS norm with weights on queries and keys, f32 angles, page 16, bf16",
         "value": gbps, "unit": "GB/s", "us_per_step": stats["mean_ms"] * 1e3, "us_per_step_median": stats["median_ms"] * 1e3,
         "algorithmic_bytes": nbytes,
         "roofline": {"bound": "hbm", "kernel": "singe_rotary_cache_write_chunks_bf16", "achieved": gbps, "peak": HBM_PEAK_GBPS,
-                     "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": None, **timing_fields(stats)},
+                     "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS, "traffic": counted, "traffic_source": source,
+                     **timing_fields(stats)},
     }
     if with_cpu:
         result["cpu_baseline"] = cache_append_cpu_baseline(work.query, key, value, cos, sin, weights, work.page_size)
