@@ -217,7 +217,10 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
         args.cap_scale = std::fabs(c.scale / options.softcap);
         args.cap_log2e = std::fabs(options.softcap) * 1.4426950408889634074f;
     }
-    const uint64_t rows = (static_cast<uint64_t>(c.batch) * c.heads + 7) / 8 * 8;
+    // A decode step through the dense op (few query rows, grouped heads, no causal mask): the query heads of a kv head
+    // share one tile, so its keys and values are fetched once.
+    args.packed_heads = dense_prefill_packs_heads(c) ? 1u : 0u;
+    const uint64_t rows = (static_cast<uint64_t>(c.batch) * (args.packed_heads ? c.kv_heads : c.heads) + 7) / 8 * 8;
     uint64_t groups = rows * ((args.query_tiles + 1) / 2);  // a workgroup takes a pair of query tiles
     if (groups > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
     // Key splits, when the caller lent scratch for them and the launch is too small to fill the chip.
@@ -245,11 +248,16 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
 
 namespace singe_hip {
 
+bool dense_prefill_packs_heads(const SingeFmhaPrefillConfig& c) {
+    constexpr size_t kTileRows = 32 * kDensePrefillWaves;
+    return !c.causal && c.kv_heads > 0 && c.heads > c.kv_heads && c.heads % c.kv_heads == 0 && c.query_len * (c.heads / c.kv_heads) <= kTileRows;
+}
+
 uint32_t dense_prefill_splits(const SingeFmhaPrefillConfig& c) {
     if (!has_matrix_core_build(static_cast<long long>(c.head_dim)) || c.batch == 0 || c.heads == 0 || c.query_len == 0) return 1;
     constexpr size_t kTileRows = 32 * kDensePrefillWaves;
     const uint64_t query_tiles = (c.query_len + kTileRows - 1) / kTileRows;
-    const uint64_t workgroups = static_cast<uint64_t>(c.batch) * c.heads * ((query_tiles + 1) / 2);
+    const uint64_t workgroups = static_cast<uint64_t>(c.batch) * (dense_prefill_packs_heads(c) ? c.kv_heads : c.heads) * ((query_tiles + 1) / 2);
     return attention_key_splits(workgroups, c.key_len);
 }
 

@@ -42,7 +42,10 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
     const unsigned int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const unsigned int column = lane & 31, hi = lane >> 5;
 
-    const unsigned int batch = bh / a.heads, head = bh % a.heads;
+    // (packed_heads: `bh` counts (batch, kv head) pairs and the rows of the one tile are (query, head of the group) pairs.)
+    const bool packed = a.packed_heads != 0;
+    const unsigned int group = a.heads / a.kv_heads;
+    const unsigned int batch = packed ? bh / a.kv_heads : bh / a.heads;
     // Keys that take part: all of them, or the batch entry's own count (singe/src/backend/cpu/normalization/attention.rs:191-276, key_lengths).
     unsigned int key_len = a.key_len;
     if (a.key_lengths != nullptr) {
@@ -51,10 +54,12 @@ SINGE_DEVICE void fmha_prefill_tile(const PrefillArgs& a, unsigned char* lds, un
         key_len = bound < key_len ? bound : key_len;
     }
     key_len = __builtin_amdgcn_readfirstlane(key_len);
-    const unsigned int kv_head = head / (a.heads / a.kv_heads);
+    const unsigned int kv_head = packed ? bh % a.kv_heads : (bh % a.heads) / group;
 
     const unsigned int first_row = query_tile * kRows + wave * 32u;  // of this wave
-    const unsigned int my_query = first_row + column;
+    const unsigned int my_row = first_row + column;
+    const unsigned int my_query = packed ? my_row / group : my_row;
+    const unsigned int head = packed ? kv_head * group + my_row % group : bh % a.heads;
     const bool query_valid = my_query < a.query_len;
 
     const uint16_t* q_base = a.query + batch * a.query_batch_stride + head * a.query_head_stride;
@@ -384,7 +389,7 @@ SINGE_DEVICE void fmha_prefill_body(const PrefillArgs& a, unsigned char* lds) {
     within /= a.splits;
     const unsigned int pairs = (a.query_tiles + 1u) / 2u;
     const unsigned int bh = (within / pairs) * 8u + xcd;
-    if (bh >= a.batch * a.heads) return;
+    if (bh >= a.batch * (a.packed_heads != 0 ? a.kv_heads : a.heads)) return;
     const unsigned int light = within % pairs, heavy = a.query_tiles - 1u - light;
     fmha_prefill_tile<CAUSAL, Half, WAVES, OPTIONS>(a, lds, bh, heavy, split);
     if (light != heavy) fmha_prefill_tile<CAUSAL, Half, WAVES, OPTIONS>(a, lds, bh, light, split);

@@ -87,6 +87,11 @@ struct PrefillArgs {
     uint32_t splits = 1;
     float* partial_out = nullptr;
     float* partial_lse = nullptr;
+    // Few query rows under grouped heads (a decode step through the dense op, no causal mask): with packed_heads != 0
+    // a workgroup takes a (batch, kv head) pair and its tile's row r is query r / group of head kv_head * group +
+    // r % group (group = heads / kv_heads, query_len * group at most the tile's rows), so the kv head's keys and values
+    // are fetched once for all of its query heads.
+    uint32_t packed_heads = 0;
 };
 
 struct PrefillF32Args {

@@ -42,6 +42,8 @@ int32_t dense_prefill_with_options(void* stream, bool f16, uint16_t* out, size_t
 // scratch they need.
 uint32_t dense_prefill_splits(const SingeFmhaPrefillConfig& config);
 size_t dense_prefill_scratch_bytes(const SingeFmhaPrefillConfig& config, uint32_t splits);
+// Whether the launch gives the query heads of a kv head one tile (few query rows, grouped heads, no causal mask).
+bool dense_prefill_packs_heads(const SingeFmhaPrefillConfig& config);
 
 // attention_parameters.cpp: the shares a launch of `workgroups` workgroups over at most `keys` keys splits its keys
 // into under the installed AttentionParameters (1 = no split).

@@ -149,3 +149,32 @@ def test_dense_key_splits_with_sinks_key_lengths_and_a_mask(dim):
     out = neural.attend(q, k, v, mask, sinks)
     want = oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), mask=host(mask), sinks=host(sinks), threads=8)
     close(host(out), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("heads, kv_heads, query_len", [(8, 2, 1), (32, 8, 4), (16, 1, 8), (16, 2, 16), (16, 2, 17), (6, 3, 5), (64, 8, 16)])
+def test_grouped_heads_of_a_decode_shaped_dense_call_share_a_tile(heads, kv_heads, query_len, dtype):
+    """Without a causal mask, query_len * (heads / kv_heads) rows of at most a tile are packed into one tile per kv head
+    (17 queries under eight heads a kv head are not, nor is anything under a causal mask): with and without key splits,
+    with a mask that differs per head, sinks per head and per-batch key counts, against the oracle."""
+    batch, key_len, dim = 2, 1500, 128
+    q, k, v = tensors((batch, heads, query_len, dim), (batch, kv_heads, key_len, dim), (batch, kv_heads, key_len, dim), dtype, 3 * heads + query_len)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(heads)
+    mask = torch.randn((heads, query_len, key_len), generator=gen, device="cuda").to(dtype)
+    mask[heads - 1, query_len - 1, 100:] = float("-inf")
+    sinks = torch.randn((heads,), generator=gen, device="cuda").to(dtype)
+    lengths = torch.tensor([key_len, 700], dtype=torch.int32, device="cuda")
+    for below in (None, 0):
+        neural.set_attention_parameters(None if below is None else neural.AttentionParameters(split_below_blocks=below))
+        try:
+            plain = neural.attend(q, k, v)
+            with_mask = neural.attend(q, k, v, mask, sinks, neural.AttentionOptions(softcap=20.0))
+            padded = neural.attend_padded(q, k, v, lengths, neural.AttentionOptions(window=900))
+        finally:
+            neural.set_attention_parameters(None)
+        close(host(plain), oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), threads=8), dtype)
+        close(host(with_mask), oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), mask=host(mask), sinks=host(sinks),
+                                                                       softcap=20.0, threads=8), dtype)
+        close(host(padded), oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), key_lengths=[key_len, 700], window=900,
+                                                                    threads=8), dtype)
