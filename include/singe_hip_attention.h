@@ -423,7 +423,12 @@ SINGE_HIP_API int32_t singe_hip_paged_attention_bf16(
  * holds nothing between calls; calls that share it must not overlap.  Results equal the unsplit ones up to
  * the order of summation.  singe_hip_set_paged_attention_splits fixes the number of shares (0 = chosen by
  * problem size, the default), the counterpart of TuningChoice::Explicit
- * (singe-kernel/src/cuda/attention/mod.rs:2364-2380); it changes what ..._scratch_bytes returns. */
+ * (singe-kernel/src/cuda/attention/mod.rs:2364-2380); it changes what ..._scratch_bytes returns.
+ * A decode step (no more tokens than sequences, i32 paging, head_dim 128 or 64, no window or softcap) given
+ * scratch on a 256-byte boundary runs on the block-table decode kernels instead, which cut the keys of all
+ * sequences into equal ranges: a first kernel checks the paging vectors (same status word) and gives each token
+ * its page list and key count, and the scratch then also holds those and the decode kernels' partial rows.  The
+ * result is the same up to the order of summation; a fixed number of shares keeps such a call on the row-tile kernel. */
 SINGE_HIP_API size_t singe_hip_paged_attention_scratch_bytes(const SingePagedAttentionProblem* problem);
 SINGE_HIP_API void singe_hip_set_paged_attention_splits(uint32_t splits);
 SINGE_HIP_API int32_t singe_hip_paged_attention_scratch_bf16(

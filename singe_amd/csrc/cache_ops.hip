@@ -306,6 +306,61 @@ SINGE_DEVICE void paging_indices_body(const PagingIndicesArgs& a) {
     }
 }
 
+// A decode step in FlashInfer form, token by token, for the block-table decode kernels: thread i checks sequence i's
+// paging values (reporting what paged_attention.rs:210-238 refuses), gives token i its row (the page list of the
+// sequence that owns it and the keys it sees: all of them, or under the causal mask those up to its own position,
+// counted from the end as the CPU path does, attention.rs:483), and checks page-table entry i (an id outside the
+// cache is reported when a sequence with queries reads it; the decode kernels themselves mask such keys).
+SINGE_DEVICE void paged_decode_rows_body(const DecodeRowsArgs& a) {
+    constexpr int FORM = kCsrI32;
+    const unsigned long long index = static_cast<unsigned long long>(blockIdx.x) * blockDim.x + threadIdx.x;
+    auto span_of = [&](unsigned int sequence) __attribute__((always_inline)) {
+        return load_span<FORM>(sequence, a.query_offsets, a.page_offsets, a.last_page_lengths, nullptr, a.tokens, a.page_table, a.page_size);
+    };
+    // The last sequence whose offset is at most `value`, by bisection (sequences without queries or pages share an
+    // offset with their successor, and the last of them is the one that holds the value).
+    auto owner_of = [&](const void* offsets, long long value) __attribute__((always_inline)) {
+        unsigned int low = 0, high = a.sequences;  // offsets[low] <= value (or low == 0), offsets[high] > value (or high == sequences)
+        while (high - low > 1) {
+            const unsigned int middle = (low + high) / 2;
+            if (read_index<FORM>(offsets, middle) <= value) low = middle; else high = middle;
+        }
+        return low;
+    };
+    if (index < a.sequences) {
+        if (!span_of(static_cast<unsigned int>(index)).valid) report_index_error(a.status);
+    }
+    if (index < a.tokens) {
+        const long long token = static_cast<long long>(index);
+        unsigned int sequence = static_cast<unsigned int>(index);
+        // One token a sequence, in order, is the usual step: then the owner is found without a search.
+        if (!(index < a.sequences && read_index<FORM>(a.query_offsets, index) == token && read_index<FORM>(a.query_offsets, index + 1) == token + 1))
+            sequence = owner_of(a.query_offsets, token);
+        const SequenceSpan span = span_of(sequence);
+        unsigned int start = 0;
+        long long length = -1;  // no valid sequence owns the token: its row is left alone
+        if (span.valid && token >= span.query_start && token - span.query_start < static_cast<long long>(span.queries)) {
+            start = static_cast<unsigned int>(span.page_start);
+            length = span.keys;
+            if (a.causal != 0 && span.keys != 0) {
+                const long long raw = static_cast<long long>(span.keys) - static_cast<long long>(span.queries) + (token - span.query_start);
+                const long long reach = (raw < 0 ? 0 : raw) + 1;
+                length = reach < static_cast<long long>(span.keys) ? reach : static_cast<long long>(span.keys);
+            }
+        }
+        a.row_starts[index] = start;
+        a.lengths[index] = static_cast<int>(length);
+    }
+    if (index < a.page_table) {
+        const long long page = read_index<FORM>(a.pages, index);
+        if (page < 0 || page >= static_cast<long long>(a.cache_pages)) {
+            const SequenceSpan span = span_of(owner_of(a.page_offsets, static_cast<long long>(index)));
+            const long long entry = static_cast<long long>(index) - span.page_start;
+            if (span.valid && span.queries != 0 && entry >= 0 && entry * a.page_size < static_cast<long long>(span.keys)) report_index_error(a.status);
+        }
+    }
+}
+
 }  // namespace cache_ops
 
 extern "C" __global__ __launch_bounds__(256) void singe_rotary_cache_write_f32(RotaryCacheArgs args) {
@@ -326,6 +381,7 @@ extern "C" __global__ __launch_bounds__(256) void singe_rotary_cache_write_chunk
 extern "C" __global__ __launch_bounds__(256) void singe_rotary_cache_write_chunks_f16(RotaryCacheArgs args) {
     cache_ops::rotary_cache_write_chunks_body<kElementF16>(args);
 }
+extern "C" __global__ __launch_bounds__(256) void singe_paged_decode_rows_i32(DecodeRowsArgs args) { cache_ops::paged_decode_rows_body(args); }
 extern "C" __global__ __launch_bounds__(256) void singe_paging_indices_i32(PagingIndicesArgs args) {
     cache_ops::paging_indices_body<false>(args);
 }

@@ -29,6 +29,9 @@ struct DecodeArgs {
     uint32_t head_groups;           // waves a kv head's query heads are spread over: ceil(group / 8)
     uint32_t heads_per_wave;        // min(group, 8): partial rows per slot
     float scale_log2e;              // scale * log2(e)
+    // Table rows of their own lengths (the paged attention op's page lists): row b starts at entry row_starts[b] of
+    // block_table, which then holds block_table_batch_stride entries in all; null: rows are that stride apart.
+    const uint32_t* row_starts = nullptr;
 };
 
 struct CombineArgs {
@@ -42,6 +45,8 @@ struct CombineArgs {
     uint32_t workers;
     uint32_t head_groups;
     uint32_t heads_per_wave;
+    float* lse = nullptr;           // [batch, heads] base-two log-sum-exp of each row (-inf for a row without keys), or null
+    const int32_t* row_lengths = nullptr;  // non-null: a row whose length is negative belongs to no sequence and is left as it is
 };
 
 // Waves of a dense prefill workgroup (singe_fmha_prefill_*_d128_*), 32 query rows each: host and kernel agree on
@@ -321,6 +326,19 @@ struct RotaryCacheArgs {
     // The 16-byte kernels (singe_rotary_cache_write_chunks_*): a head's lanes that hold data, and the power of two of
     // neighbouring lanes it is dealt to.
     uint32_t head_lanes, group_lanes;
+};
+
+// singe_paged_decode_rows_i32: a decode step given as FlashInfer CSR paging (i32) -> one row per token for the decode
+// kernels: where the token's page list starts in `pages` and how many keys it sees.
+struct DecodeRowsArgs {
+    const void* query_offsets;      // [sequences + 1]
+    const void* page_offsets;       // [sequences + 1]
+    const void* pages;              // [page_table]
+    const void* last_page_lengths;  // [sequences]
+    uint32_t* row_starts;           // [tokens]
+    int32_t* lengths;               // [tokens]: -1 for a token no valid sequence owns
+    uint32_t* status;
+    uint32_t tokens, sequences, page_table, page_size, cache_pages, causal;
 };
 
 // singe_paging_indices_*: FlashInfer CSR paging -> block-table paging.

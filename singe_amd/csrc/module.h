@@ -70,6 +70,8 @@ enum KernelId : int {
     kRotaryCacheChunks, kRotaryCacheChunksBf16, kRotaryCacheChunksF16,
     // the decode merge for rows with one or two slots: bf16, f16, then the same for head_dim 64
     kDecodeCombineFew, kDecodeCombineFewF16, kDecodeCombineFewD64, kDecodeCombineFewF16D64,
+    // a decode step in FlashInfer form -> one row per token for the decode kernels
+    kPagedDecodeRows,
     kKernelCount
 };
 

@@ -83,6 +83,39 @@ uint32_t paged_attention_splits(const SingePagedAttentionProblem& p) {
     return attention_key_splits(workgroups, keys);
 }
 
+// A decode step (no more tokens than sequences: a token a sequence) through this op takes the block-table decode
+// kernels, which cut the keys of all sequences into equal ranges whatever their lengths: a small kernel first turns
+// the paging vectors into one row per token (where its page list starts, how many keys it sees) and checks them.
+// What the host can tell: a matrix-core decode build for the head dimension, i32 paging, no window, cap or fused
+// rotation, and sizes the decode kernels take.
+constexpr size_t kDecodeRowsMost = 8000;
+
+bool decode_rows_config(const SingePagedAttentionProblem& p, SingePagedKvDecodeAttentionConfig* config) {
+    if (g_paged_attention_splits != 0) return false;  // a fixed number of shares asks for the row-tile kernel
+    if ((p.head_dim != 128 && p.head_dim != 64) || p.index_type != SINGE_HIP_INDEX_I32 || p.has_window || p.has_softcap) return false;
+    if (p.tokens <= 0 || p.tokens > p.sequences || static_cast<size_t>(p.tokens) > kDecodeRowsMost || p.page_table <= 0 || p.cache_pages <= 0)
+        return false;
+    if (!fits_i32(static_cast<uint64_t>(p.page_table) * static_cast<uint64_t>(p.page_size))) return false;
+    config->batch = static_cast<size_t>(p.tokens);
+    config->heads = static_cast<size_t>(p.heads);
+    config->kv_heads = static_cast<size_t>(p.kv_heads);
+    config->head_dim = static_cast<size_t>(p.head_dim);
+    config->block_size = static_cast<size_t>(p.page_size);
+    config->physical_blocks = static_cast<size_t>(p.cache_pages);
+    config->block_table_batch_stride = static_cast<size_t>(p.page_table);  // the count of entries: rows have their own lengths
+    config->scale = p.has_scale ? p.scale : 1.0f / std::sqrt(static_cast<float>(p.head_dim));
+    return true;
+}
+
+size_t align256(size_t bytes) { return (bytes + 255) / 256 * 256; }
+
+// Scratch of that route: the tokens' row starts, their lengths, the decode kernels' workspace.
+size_t decode_rows_bytes(const SingePagedAttentionProblem& p) {
+    SingePagedKvDecodeAttentionConfig config;
+    if (!decode_rows_config(p, &config)) return 0;
+    return 2 * align256(static_cast<size_t>(p.tokens) * sizeof(uint32_t)) + paged_decode_workspace_bytes(config);
+}
+
 size_t scratch_bytes_for(const SingePagedAttentionProblem& p, uint32_t splits) {
     if (splits <= 1) return 0;
     return static_cast<size_t>(splits) * static_cast<size_t>(p.tokens) * static_cast<size_t>(p.heads) * (static_cast<size_t>(p.head_dim) + 1) * sizeof(float);
@@ -145,6 +178,45 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
     const uint16_t* value_cache = static_cast<const uint16_t*>(value_cache_any);
     uint16_t* output = static_cast<uint16_t*>(output_any);
 
+    // A decode step with scratch for it: the block-table decode kernels (see decode_rows_config).
+    if (rotation == nullptr && scratch != nullptr && scratch->memory != nullptr && reinterpret_cast<uintptr_t>(scratch->memory) % 256 == 0) {
+        SingePagedKvDecodeAttentionConfig config;
+        const size_t need = decode_rows_bytes(p);
+        if (need != 0 && scratch->bytes >= need && decode_rows_config(p, &config)) {
+            unsigned char* memory = static_cast<unsigned char*>(scratch->memory);
+            const size_t array_bytes = align256(static_cast<size_t>(p.tokens) * sizeof(uint32_t));
+            DecodeRowsArgs rows;
+            rows.query_offsets = query_offsets;
+            rows.page_offsets = page_offsets;
+            rows.pages = pages;
+            rows.last_page_lengths = last_page_lengths;
+            rows.row_starts = reinterpret_cast<uint32_t*>(memory);
+            rows.lengths = reinterpret_cast<int32_t*>(memory + array_bytes);
+            rows.status = status;
+            rows.tokens = static_cast<uint32_t>(p.tokens);
+            rows.sequences = static_cast<uint32_t>(p.sequences);
+            rows.page_table = static_cast<uint32_t>(p.page_table);
+            rows.page_size = static_cast<uint32_t>(p.page_size);
+            rows.cache_pages = static_cast<uint32_t>(p.cache_pages);
+            rows.causal = p.causal ? 1u : 0u;
+            const uint64_t most = static_cast<uint64_t>(p.page_table > p.sequences ? p.page_table : p.sequences);
+            if (int32_t launched = launch(kPagedDecodeRows, static_cast<unsigned>((most + 255) / 256), 1, 1, 256, stream, rows)) return launched;
+            PagedDecodeLaunch decode;
+            decode.stream = stream;
+            decode.out = output;
+            decode.query = query_rows;
+            decode.key_cache = key_cache;
+            decode.value_cache = value_cache;
+            decode.f16 = f16;
+            decode.actual_seq_lens = rows.lengths;
+            decode.block_table = static_cast<const uint32_t*>(pages);
+            decode.workspace = memory + 2 * array_bytes;
+            decode.workspace_bytes = scratch->bytes - 2 * array_bytes;
+            decode.row_starts = rows.row_starts;
+            decode.lse = lse;
+            return launch_paged_decode(config, decode);
+        }
+    }
     const uint64_t groups = static_cast<uint64_t>(p.heads / p.kv_heads);
     PagedAttentionArgs args;
     args.query_rows = query_rows;
@@ -220,7 +292,8 @@ extern "C" void singe_hip_set_paged_attention_splits(uint32_t splits) { g_paged_
 
 extern "C" size_t singe_hip_paged_attention_scratch_bytes(const SingePagedAttentionProblem* problem) {
     if (problem == nullptr) return 0;
-    return scratch_bytes_for(*problem, paged_attention_splits(*problem));
+    const size_t shares = scratch_bytes_for(*problem, paged_attention_splits(*problem)), rows = decode_rows_bytes(*problem);
+    return shares > rows ? shares : rows;
 }
 
 extern "C" int32_t singe_hip_paged_attention_scratch_bf16(void* stream, const uint16_t* query_rows, const uint16_t* key_cache,

@@ -234,6 +234,27 @@ int32_t decode(
                                    c.heads, c.kv_heads, c.head_dim, c.block_size, c.physical_blocks, c.block_table_batch_stride,
                                    false, c.scale);
     }
+    PagedDecodeLaunch launch_of;
+    launch_of.stream = stream, launch_of.out = out, launch_of.query = query, launch_of.key_cache = key_cache, launch_of.value_cache = value_cache;
+    launch_of.key_scales = key_scales, launch_of.value_scales = value_scales, launch_of.fp8 = fp8, launch_of.f16 = f16;
+    launch_of.actual_seq_lens = actual_seq_lens, launch_of.block_table = block_table, launch_of.workspace = workspace;
+    launch_of.workspace_bytes = workspace_bytes, launch_of.phases = phases;
+    return launch_paged_decode(c, launch_of);
+}
+
+}  // namespace
+
+namespace singe_hip {
+
+size_t paged_decode_workspace_bytes(const SingePagedKvDecodeAttentionConfig& c) { return workspace_need(c); }
+
+// The two launches of the matrix-core decode (head_dim 128 or 64), after the entry point's checks.
+int32_t launch_paged_decode(const SingePagedKvDecodeAttentionConfig& c, const PagedDecodeLaunch& l) {
+    void* const stream = l.stream;
+    const bool fp8 = l.fp8, f16 = l.f16;
+    const uint32_t phases = l.phases;
+    void* const workspace = l.workspace;
+    const size_t workspace_bytes = l.workspace_bytes;
     const bool narrow = c.head_dim == 64;  // the head_dim 64 build of the same kernels
     uint64_t reach = static_cast<uint64_t>(c.block_table_batch_stride) * c.block_size;
     if (!fits_i32(reach)) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "block_table_batch_stride * block_size");
@@ -241,7 +262,8 @@ int32_t decode(
     // bf16 caches take the one-hot form, fp8 caches the dense form (see paged_decode.hip); and so do bf16 / f16
     // caches with more than four query heads per kv head at head_dim 128, where the one-hot form would carry two
     // groups per wave, as long as the batch's prefix sums fit beside that form's 132 KiB of staging in LDS.
-    const unsigned prefix_bytes = static_cast<unsigned>((2 * c.batch + 1) * sizeof(uint32_t));
+    // (the kernel keeps the sequences' tile prefix sums and lengths in LDS, and their rows' starts when rows have their own lengths)
+    const unsigned prefix_bytes = static_cast<unsigned>(((l.row_starts != nullptr ? 3 : 2) * c.batch + 1) * sizeof(uint32_t));
     constexpr unsigned kWideStagingBytes = 135168, kLdsBytes = 160 * 1024;
     const bool wide = !fp8 && !narrow && c.heads / c.kv_heads > 4 && kWideStagingBytes + prefix_bytes <= kLdsBytes;
     const Plan plan = make_plan(c, wide || fp8 ? 16 : 8);  // (the dense form of fp8 caches has its Q^T in registers and no such limit)
@@ -251,13 +273,14 @@ int32_t decode(
     unsigned char* scratch = static_cast<unsigned char*>(workspace);
 
     DecodeArgs args;
-    args.query = query;
-    args.key_cache = key_cache;
-    args.value_cache = value_cache;
-    args.key_scales = key_scales;
-    args.value_scales = value_scales;
-    args.actual_seq_lens = actual_seq_lens;
-    args.block_table = block_table;
+    args.query = l.query;
+    args.key_cache = l.key_cache;
+    args.value_cache = l.value_cache;
+    args.key_scales = l.key_scales;
+    args.value_scales = l.value_scales;
+    args.actual_seq_lens = l.actual_seq_lens;
+    args.block_table = l.block_table;
+    args.row_starts = l.row_starts;
     args.meta = reinterpret_cast<uint32_t*>(scratch);
     args.partial_lse = reinterpret_cast<float*>(scratch + plan.lse_offset);
     args.partial_out = reinterpret_cast<float*>(scratch + plan.out_offset);
@@ -288,7 +311,9 @@ int32_t decode(
     if (!(phases & SINGE_HIP_DECODE_REDUCE)) return 0;
 
     CombineArgs combine;
-    combine.out = out;
+    combine.out = l.out;
+    combine.lse = l.lse;
+    combine.row_lengths = l.row_starts != nullptr ? l.actual_seq_lens : nullptr;
     combine.partial_out = args.partial_out;
     combine.partial_lse = args.partial_lse;
     combine.meta = args.meta;
@@ -313,7 +338,7 @@ int32_t decode(
     return launch(narrow ? at_head_dim_64(merge) : merge, static_cast<unsigned>((c.batch * c.heads + 3) / 4), 1, 1, 256, stream, combine);
 }
 
-}  // namespace
+}  // namespace singe_hip
 
 extern "C" {
 

@@ -117,14 +117,15 @@ struct EntryCache {
 };
 
 template <bool FP8>
-SINGE_DEVICE void fill_entries(EntryCache& cache, const DecodeArgs& a, unsigned int sequence, unsigned int first_entry,
+SINGE_DEVICE void fill_entries(EntryCache& cache, const DecodeArgs& a, unsigned int sequence, size_t row_base, unsigned int first_entry,
                                unsigned int kv_head, unsigned int lane) {
     cache.sequence = sequence;
     cache.first_entry = first_entry;
     const unsigned int index = first_entry + lane;
     unsigned int block = 0xffffffffu;
-    if (index < a.block_table_batch_stride)
-        block = a.block_table[static_cast<size_t>(sequence) * a.block_table_batch_stride + index];
+    // (rows of their own lengths: the table holds block_table_batch_stride entries in all)
+    if (a.row_starts != nullptr ? row_base + index < a.block_table_batch_stride : index < a.block_table_batch_stride)
+        block = a.block_table[row_base + index];
     cache.blocks = block;
     if constexpr (FP8) {
         const size_t at = static_cast<size_t>(block < a.physical_blocks ? block : 0) * a.kv_heads + kv_head;
@@ -360,6 +361,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
     // Tiles per sequence, prefix-summed: prefix[b] = tiles of sequences before b; lengths[b] = its keys,
     // clamped to what its table row can address.
     unsigned int* lengths = prefix + a.batch + 1;
+    unsigned int* starts = lengths + a.batch;  // rows of their own lengths: where each begins in the table (the launch then lends a third array)
     if (wave == 0) {
         unsigned int carry = 0;
         for (unsigned int base = 0; base < a.batch; base += 64) {
@@ -378,6 +380,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
             if (base + lane < a.batch) {
                 prefix[base + lane + 1] = carry + scan;
                 lengths[base + lane] = len;
+                if (a.row_starts != nullptr) starts[base + lane] = a.row_starts[base + lane];
             }
             carry += __shfl(scan, 63, 64);
         }
@@ -700,6 +703,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
         if (load_at >= range_end) return;
         while (prefix[load_seq + 1] <= load_at) ++load_seq;  // skips empty sequences
         const unsigned int first_key = (load_at - prefix[load_seq]) * kTile, end = lengths[load_seq];
+        const size_t row_base = a.row_starts != nullptr ? starts[load_seq] : static_cast<size_t>(load_seq) * a.block_table_batch_stride;
         if constexpr (ALIGNED16) {
             // Entries this tile reads: those of its first key and of its last live key (a half past
             // the end re-reads the last key's entry).
@@ -707,10 +711,9 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
             split_key(a, first_key, low, slot);
             split_key(a, (first_key + kTile <= end ? first_key + kTile : end) - 1, high, slot);
             if (entries.sequence != load_seq || low < entries.first_entry || high >= entries.first_entry + 64)
-                fill_entries<FP8>(entries, a, load_seq, low, kv_head, lane);
+                fill_entries<FP8>(entries, a, load_seq, row_base, low, kv_head, lane);
         }
-        load_tile<ALIGNED16>(buffer, a, a.block_table + static_cast<size_t>(load_seq) * a.block_table_batch_stride, entries,
-                             first_key, end, kv_head, g, t);
+        load_tile<ALIGNED16>(buffer, a, a.block_table + row_base, entries, first_key, end, kv_head, g, t);
         ++load_at;
     };
     auto consume = [&](const Tile& buffer) __attribute__((always_inline)) {
@@ -826,18 +829,19 @@ SINGE_DEVICE void paged_decode_combine_body(const CombineArgs& a) {
     const unsigned int row = blockIdx.x * 4 + (threadIdx.x >> 6);  // batch * heads + head
     if (row >= a.batch * a.heads) return;
     const unsigned int b = row / a.heads, head = row % a.heads;
+    if (a.row_lengths != nullptr && a.row_lengths[b] < 0) return;
     const unsigned int group = a.heads / a.kv_heads;
     const unsigned int kv_head = head / group, in_group = head % group;
     const unsigned int work = kv_head * a.head_groups + in_group / a.heads_per_wave, local = in_group % a.heads_per_wave;
     const unsigned int share = a.meta[0];
     const unsigned int first_tile = a.meta[2 + b], end_tile = a.meta[3 + b];
     float low = 0.0f, high = 0.0f;  // a sequence with no keys keeps a zero row (cpu/attention.rs:1213-1215)
+    float best = -INFINITY, total = 0.0f;
     const bool holds_values = 2 * lane < static_cast<unsigned int>(kDim);  // a lane takes two of the row's values
     if (end_tile > first_tile) {
         const unsigned int first_worker = first_tile / share, last_worker = (end_tile - 1) / share;
         const size_t base = (static_cast<size_t>(work) * (a.workers + a.batch) + first_worker + b) * a.heads_per_wave + local;
         const unsigned int count = last_worker - first_worker + 1;
-        float best = -INFINITY, total = 0.0f;
         for (unsigned int chunk = 0; chunk < count; chunk += 64) {
             const unsigned int n = count - chunk < 64 ? count - chunk : 64;
             const size_t chunk_base = base + static_cast<size_t>(chunk) * a.heads_per_wave;
@@ -893,6 +897,8 @@ SINGE_DEVICE void paged_decode_combine_body(const CombineArgs& a) {
         packed = pack_bf16x2(low, high);
     }
     if (holds_values) *reinterpret_cast<unsigned int*>(a.out + static_cast<size_t>(row) * kDim + 2 * lane) = packed;
+    // The row's log-sum-exp in base two, for the paged attention op (the slots hold natural logarithms).
+    if (a.lse != nullptr && lane == 0) a.lse[row] = total > 0.0f ? (best + __logf(total)) * 1.4426950408889634074f : -INFINITY;
 }
 
 // The same fold for rows with many slots (few sequences, long contexts: a lone sequence has a slot per worker, 256 of
@@ -908,6 +914,7 @@ SINGE_DEVICE void paged_decode_combine_many_body(const CombineArgs& a) {
     const unsigned int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const unsigned int row = blockIdx.x;  // batch * heads + head
     const unsigned int b = row / a.heads, head = row % a.heads;
+    if (a.row_lengths != nullptr && a.row_lengths[b] < 0) return;  // (the whole workgroup: it is one row's)
     const unsigned int group = a.heads / a.kv_heads;
     const unsigned int kv_head = head / group, in_group = head % group;
     const unsigned int work = kv_head * a.head_groups + in_group / a.heads_per_wave, local = in_group % a.heads_per_wave;
@@ -988,6 +995,7 @@ SINGE_DEVICE void paged_decode_combine_many_body(const CombineArgs& a) {
         packed = pack_bf16x2(low, high);
     }
     if (holds_values) *reinterpret_cast<unsigned int*>(a.out + static_cast<size_t>(row) * kDim + 2 * lane) = packed;
+    if (a.lse != nullptr && lane == 0) a.lse[row] = total > 0.0f ? (largest + __logf(total)) * 1.4426950408889634074f : -INFINITY;
 }
 
 #if SINGE_HEAD_DIM == 128

@@ -45,6 +45,30 @@ size_t dense_prefill_scratch_bytes(const SingeFmhaPrefillConfig& config, uint32_
 // Whether the launch gives the query heads of a kv head one tile (few query rows, grouped heads, no causal mask).
 bool dense_prefill_packs_heads(const SingeFmhaPrefillConfig& config);
 
+// paged_decode.cpp: the two launches of the matrix-core decode kernels (head_dim 128 or 64) for a config its caller has
+// checked, and the workspace they need.  `row_starts` non-null: the table holds rows of their own lengths (row b
+// starts at entry row_starts[b]; block_table_batch_stride is then the count of entries in all), the way the paged
+// attention op's page lists lie; `lse` non-null: the reduce also leaves each row's base-two log-sum-exp.
+struct PagedDecodeLaunch {
+    void* stream = nullptr;
+    uint16_t* out = nullptr;
+    const uint16_t* query = nullptr;
+    const void* key_cache = nullptr;
+    const void* value_cache = nullptr;
+    const float* key_scales = nullptr;
+    const float* value_scales = nullptr;
+    bool fp8 = false, f16 = false;
+    const int32_t* actual_seq_lens = nullptr;
+    const uint32_t* block_table = nullptr;
+    void* workspace = nullptr;
+    size_t workspace_bytes = 0;
+    uint32_t phases = 3;
+    const uint32_t* row_starts = nullptr;
+    float* lse = nullptr;
+};
+int32_t launch_paged_decode(const SingePagedKvDecodeAttentionConfig& config, const PagedDecodeLaunch& launch);
+size_t paged_decode_workspace_bytes(const SingePagedKvDecodeAttentionConfig& config);
+
 // attention_parameters.cpp: the shares a launch of `workgroups` workgroups over at most `keys` keys splits its keys
 // into under the installed AttentionParameters (1 = no split).
 uint32_t attention_key_splits(uint64_t workgroups, uint64_t keys);

@@ -79,8 +79,10 @@ def test_candidates_agree_where_the_threshold_changes_the_shares(dim):
     kc = torch.randn((page_count, 16, 2, dim), generator=gen, device="cuda").to(torch.bfloat16)
     vc = torch.randn((page_count, 16, 2, dim), generator=gen, device="cuda").to(torch.bfloat16)
     table = np.random.default_rng(3).permutation(page_count)[:sum(pages_of)]
-    paging = neural.Paging(index(list(range(len(lens) + 1))), index(np.concatenate([[0], np.cumsum(pages_of)])), index(table),
-                           index([n - (p - 1) * 16 for n, p in zip(lens, pages_of)]))
+    # (i64 paging: with i32 a decode step like this one would leave the row-tile kernel for the block-table decode kernels)
+    wide = lambda values: index(values, torch.int64)
+    paging = neural.Paging(wide(list(range(len(lens) + 1))), wide(np.concatenate([[0], np.cumsum(pages_of)])), wide(table),
+                           wide([n - (p - 1) * 16 for n, p in zip(lens, pages_of)]))
     problem = neural._problem(q, kc, vc, paging, neural.AttentionOptions(causal=True))
     wanted = set()
     for candidate in neural.attention_candidates():

@@ -266,3 +266,77 @@ def test_a_stream_that_is_not_torchs_current_one_orders_the_fills_and_the_status
         with pytest.raises(error.IndexOutOfBounds):
             neural.paged_attention(q, cache, cache, bad, neural.AttentionOptions(causal=True), stream=side)
     torch.cuda.synchronize()
+
+
+# A decode step (no more tokens than sequences, i32 paging, no window or cap) runs on the block-table decode kernels,
+# token by token: (queries, keys) per sequence.
+DECODE_STEPS = [
+    [(1, 700), (1, 1), (1, 4096), (1, 33), (1, 16)],                      # a token a sequence, ragged
+    [(1, 300), (0, 500), (1, 0), (1, 64), (0, 0), (1, 1500)],             # sequences without a token, a token without keys
+    [(2, 900), (0, 40), (1, 17), (0, 2000)],                              # two tokens of one sequence, as many tokens as sequences
+    [(3, 2), (0, 5), (0, 7), (1, 129)],                                   # more queries than keys
+    [(1, 128 * (b % 5) + b) for b in range(1, 70)],                       # more sequences than a wave has lanes
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("heads, kv_heads, page_size, dim", [(8, 2, 16, 128), (32, 4, 8, 128), (16, 1, 64, 128), (4, 4, 1, 128), (8, 2, 32, 64), (6, 1, 7, 64)])
+@pytest.mark.parametrize("step", range(len(DECODE_STEPS)))
+def test_a_decode_step_through_the_op_matches_the_oracle_and_the_row_tile_kernel(step, heads, kv_heads, page_size, dim, dtype):
+    import ctypes
+    sequences = DECODE_STEPS[step]
+    query_offsets, page_offsets, table, last, page_count = layout(sequences, page_size)
+    tokens = query_offsets[-1]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(100 * step + heads)
+    rand = lambda *shape: torch.randn(shape, generator=gen, device="cuda").to(dtype)
+    q, kc, vc = rand(tokens, heads, dim), rand(page_count, page_size, kv_heads, dim), rand(page_count, page_size, kv_heads, dim)
+    index = lambda values: torch.tensor(values, dtype=torch.int32, device="cuda")
+    paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
+    for options in (neural.AttentionOptions(causal=True), neural.AttentionOptions(scale=0.05)):
+        # the scratch the op asks for covers the decode kernels' rows and partials
+        problem = neural._problem(q, kc, vc, paging, options)
+        assert _native.lib().singe_hip_paged_attention_scratch_bytes(ctypes.byref(problem)) >= 2 * 256 + 4 * tokens * heads * (dim + 1)
+        out, lse = neural.paged_attention(q, kc, vc, paging, options)
+        tiled, tiled_lse = neural.paged_attention(q, kc, vc, paging, options, scratch=False)
+        torch.cuda.synchronize()
+        status, want, want_lse = oracle.paged_attention_f32(q.float().cpu().numpy(), kc.float().cpu().numpy(), vc.float().cpu().numpy(), query_offsets,
+                                                            page_offsets, table, last, scale=options.scale, causal=options.causal, threads=8)
+        assert status == 0
+        got, got_lse = out.float().cpu().numpy(), lse.cpu().numpy()
+        gap = np.abs(got - want)
+        assert gap.max() <= MAX_ABS and gap.mean() <= MEAN_ABS, (gap.max(), gap.mean())
+        empty = np.isneginf(want_lse)
+        assert np.array_equal(np.isneginf(got_lse), empty) and not got[empty].any()
+        assert np.abs(got_lse[~empty] - want_lse[~empty]).max(initial=0.0) <= LSE_ABS
+        assert (out.float() - tiled.float()).abs().max().item() <= 8e-3
+        assert np.array_equal(np.isneginf(tiled_lse.cpu().numpy()), empty)
+
+
+def test_a_decode_step_keeps_the_error_contract_and_leaves_unowned_tokens_alone():
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(4)
+    q = torch.randn((3, 4, 128), generator=gen, device="cuda").to(torch.bfloat16)
+    cache = torch.randn((6, 16, 2, 128), generator=gen, device="cuda").to(torch.bfloat16)
+    index = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
+    options = neural.AttentionOptions(causal=True)
+    good = neural.Paging(index([0, 1, 2, 3]), index([0, 2, 3, 5]), index([4, 1, 0, 2, 5]), index([7, 16, 3]))
+    want, want_lse = neural.paged_attention(q, cache, cache, good, options)
+    for pages, last in (([4, 1, 0, 2, 6], [7, 16, 3]), ([4, 1, 0, -1, 5], [7, 16, 3]), ([4, 1, 0, 2, 5], [7, 16, 17])):
+        bad = neural.Paging(index([0, 1, 2, 3]), index([0, 2, 3, 5]), index(pages), index(last))
+        status = torch.zeros(1, dtype=torch.int32, device="cuda")
+        got, got_lse = neural.paged_attention(q, cache, cache, bad, options, status=status, check=False)
+        assert status.item() == 1
+        assert torch.equal(got[:2], want[:2]) and torch.equal(got_lse[:2], want_lse[:2])  # the sequences with good paging are right
+        with pytest.raises(error.IndexOutOfBounds):
+            neural.paged_attention(q, cache, cache, bad, options)
+    # a page id outside the cache that no sequence with a token reads is not looked at
+    unread = neural.Paging(index([0, 1, 2, 2]), index([0, 2, 3, 5]), index([4, 1, 0, 77, -3]), index([7, 16, 3]))
+    got, _ = neural.paged_attention(q[:2], cache, cache, unread, options)
+    assert torch.equal(got, want[:2])
+    # tokens before the first sequence's and after the last one's belong to nobody: their rows stay as they were
+    edges = neural.Paging(index([1, 2, 2, 2]), index([0, 2, 3, 3]), index([4, 1, 0]), index([7, 16, 0]))
+    got, got_lse = neural.paged_attention(q, cache, cache, edges, options)
+    tiled, tiled_lse = neural.paged_attention(q, cache, cache, edges, options, scratch=False)
+    assert (got[1].float() - tiled[1].float()).abs().max().item() <= 8e-3 and (got_lse[1] - tiled_lse[1]).abs().max().item() <= 2e-3
+    assert not got[0].any() and not got[2].any() and torch.isneginf(got_lse[0]).all() and torch.isneginf(got_lse[2]).all()
