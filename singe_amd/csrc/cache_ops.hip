@@ -311,8 +311,8 @@ SINGE_DEVICE void paging_indices_body(const PagingIndicesArgs& a) {
 // sequence that owns it and the keys it sees: all of them, or under the causal mask those up to its own position,
 // counted from the end as the CPU path does, attention.rs:483), and checks page-table entry i (an id outside the
 // cache is reported when a sequence with queries reads it; the decode kernels themselves mask such keys).
+template <int FORM>
 SINGE_DEVICE void paged_decode_rows_body(const DecodeRowsArgs& a) {
-    constexpr int FORM = kCsrI32;
     const unsigned long long index = static_cast<unsigned long long>(blockIdx.x) * blockDim.x + threadIdx.x;
     auto span_of = [&](unsigned int sequence) __attribute__((always_inline)) {
         return load_span<FORM>(sequence, a.query_offsets, a.page_offsets, a.last_page_lengths, nullptr, a.tokens, a.page_table, a.page_size);
@@ -353,7 +353,9 @@ SINGE_DEVICE void paged_decode_rows_body(const DecodeRowsArgs& a) {
     }
     if (index < a.page_table) {
         const long long page = read_index<FORM>(a.pages, index);
-        if (page < 0 || page >= static_cast<long long>(a.cache_pages)) {
+        const bool outside = page < 0 || page >= static_cast<long long>(a.cache_pages);
+        if (a.pages32 != nullptr) a.pages32[index] = outside ? 0xffffffffu : static_cast<unsigned int>(page);
+        if (outside) {
             const SequenceSpan span = span_of(owner_of(a.page_offsets, static_cast<long long>(index)));
             const long long entry = static_cast<long long>(index) - span.page_start;
             if (span.valid && span.queries != 0 && entry >= 0 && entry * a.page_size < static_cast<long long>(span.keys)) report_index_error(a.status);
@@ -381,7 +383,8 @@ extern "C" __global__ __launch_bounds__(256) void singe_rotary_cache_write_chunk
 extern "C" __global__ __launch_bounds__(256) void singe_rotary_cache_write_chunks_f16(RotaryCacheArgs args) {
     cache_ops::rotary_cache_write_chunks_body<kElementF16>(args);
 }
-extern "C" __global__ __launch_bounds__(256) void singe_paged_decode_rows_i32(DecodeRowsArgs args) { cache_ops::paged_decode_rows_body(args); }
+extern "C" __global__ __launch_bounds__(256) void singe_paged_decode_rows_i32(DecodeRowsArgs args) { cache_ops::paged_decode_rows_body<kCsrI32>(args); }
+extern "C" __global__ __launch_bounds__(256) void singe_paged_decode_rows_i64(DecodeRowsArgs args) { cache_ops::paged_decode_rows_body<kCsrI64>(args); }
 extern "C" __global__ __launch_bounds__(256) void singe_paging_indices_i32(PagingIndicesArgs args) {
     cache_ops::paging_indices_body<false>(args);
 }

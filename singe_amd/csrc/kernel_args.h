@@ -328,8 +328,9 @@ struct RotaryCacheArgs {
     uint32_t head_lanes, group_lanes;
 };
 
-// singe_paged_decode_rows_i32: a decode step given as FlashInfer CSR paging (i32) -> one row per token for the decode
-// kernels: where the token's page list starts in `pages` and how many keys it sees.
+// singe_paged_decode_rows_{i32,i64}: a decode step given as FlashInfer CSR paging -> one row per token for the decode
+// kernels: where the token's page list starts in `pages` and how many keys it sees.  The decode kernels read 32-bit
+// page ids: i64 paging is copied into `pages32` on the way (an id outside the cache as 0xffffffff).
 struct DecodeRowsArgs {
     const void* query_offsets;      // [sequences + 1]
     const void* page_offsets;       // [sequences + 1]
@@ -337,6 +338,7 @@ struct DecodeRowsArgs {
     const void* last_page_lengths;  // [sequences]
     uint32_t* row_starts;           // [tokens]
     int32_t* lengths;               // [tokens]: -1 for a token no valid sequence owns
+    uint32_t* pages32;              // [page_table] (i64 paging), else null
     uint32_t* status;
     uint32_t tokens, sequences, page_table, page_size, cache_pages, causal;
 };

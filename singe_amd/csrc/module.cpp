@@ -216,7 +216,7 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_rotary_cache_write_chunks_f32", "singe_rotary_cache_write_chunks_bf16", "singe_rotary_cache_write_chunks_f16",
     "singe_paged_decode_combine_few_bf16", "singe_paged_decode_combine_few_f16",
     "singe_paged_decode_combine_few_bf16_d64", "singe_paged_decode_combine_few_f16_d64",
-    "singe_paged_decode_rows_i32",
+    "singe_paged_decode_rows_i32", "singe_paged_decode_rows_i64",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -252,7 +252,7 @@ constexpr PartRun kPartRuns[] = {
     {0, 2}, {13, 2},              // the decode merge for rows with many slots, head_dim 128 and 64
     {6, 3},                       // rotate-and-append sixteen bytes at a time
     {0, 2}, {13, 2},              // the decode merge for rows with one or two slots, head_dim 128 and 64
-    {6, 1},                       // a decode step in FlashInfer form -> rows for the decode kernels
+    {6, 2},                       // a decode step in FlashInfer form -> rows for the decode kernels
 };
 constexpr int runs_total() {
     int total = 0;

@@ -71,7 +71,7 @@ enum KernelId : int {
     // the decode merge for rows with one or two slots: bf16, f16, then the same for head_dim 64
     kDecodeCombineFew, kDecodeCombineFewF16, kDecodeCombineFewD64, kDecodeCombineFewF16D64,
     // a decode step in FlashInfer form -> one row per token for the decode kernels
-    kPagedDecodeRows,
+    kPagedDecodeRows, kPagedDecodeRowsI64,
     kKernelCount
 };
 

@@ -86,13 +86,13 @@ uint32_t paged_attention_splits(const SingePagedAttentionProblem& p) {
 // A decode step (no more tokens than sequences: a token a sequence) through this op takes the block-table decode
 // kernels, which cut the keys of all sequences into equal ranges whatever their lengths: a small kernel first turns
 // the paging vectors into one row per token (where its page list starts, how many keys it sees) and checks them.
-// What the host can tell: a matrix-core decode build for the head dimension, i32 paging, no window, cap or fused
-// rotation, and sizes the decode kernels take.
+// What the host can tell: a matrix-core decode build for the head dimension, no window, cap or fused rotation, and
+// sizes the decode kernels take.  (The decode kernels read 32-bit page ids: i64 paging is copied on the way.)
 constexpr size_t kDecodeRowsMost = 8000;
 
 bool decode_rows_config(const SingePagedAttentionProblem& p, SingePagedKvDecodeAttentionConfig* config) {
     if (g_paged_attention_splits != 0) return false;  // a fixed number of shares asks for the row-tile kernel
-    if ((p.head_dim != 128 && p.head_dim != 64) || p.index_type != SINGE_HIP_INDEX_I32 || p.has_window || p.has_softcap) return false;
+    if ((p.head_dim != 128 && p.head_dim != 64) || p.has_window || p.has_softcap) return false;
     if (p.tokens <= 0 || p.tokens > p.sequences || static_cast<size_t>(p.tokens) > kDecodeRowsMost || p.page_table <= 0 || p.cache_pages <= 0)
         return false;
     if (!fits_i32(static_cast<uint64_t>(p.page_table) * static_cast<uint64_t>(p.page_size))) return false;
@@ -109,11 +109,15 @@ bool decode_rows_config(const SingePagedAttentionProblem& p, SingePagedKvDecodeA
 
 size_t align256(size_t bytes) { return (bytes + 255) / 256 * 256; }
 
-// Scratch of that route: the tokens' row starts, their lengths, the decode kernels' workspace.
+size_t decode_rows_page_copy_bytes(const SingePagedAttentionProblem& p) {
+    return p.index_type == SINGE_HIP_INDEX_I64 ? align256(static_cast<size_t>(p.page_table) * sizeof(uint32_t)) : 0;
+}
+
+// Scratch of that route: the tokens' row starts, their lengths, the 32-bit copy of i64 page ids, the decode kernels' workspace.
 size_t decode_rows_bytes(const SingePagedAttentionProblem& p) {
     SingePagedKvDecodeAttentionConfig config;
     if (!decode_rows_config(p, &config)) return 0;
-    return 2 * align256(static_cast<size_t>(p.tokens) * sizeof(uint32_t)) + paged_decode_workspace_bytes(config);
+    return 2 * align256(static_cast<size_t>(p.tokens) * sizeof(uint32_t)) + decode_rows_page_copy_bytes(p) + paged_decode_workspace_bytes(config);
 }
 
 size_t scratch_bytes_for(const SingePagedAttentionProblem& p, uint32_t splits) {
@@ -192,6 +196,8 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
             rows.last_page_lengths = last_page_lengths;
             rows.row_starts = reinterpret_cast<uint32_t*>(memory);
             rows.lengths = reinterpret_cast<int32_t*>(memory + array_bytes);
+            const size_t copy_bytes = decode_rows_page_copy_bytes(p);
+            rows.pages32 = copy_bytes != 0 ? reinterpret_cast<uint32_t*>(memory + 2 * array_bytes) : nullptr;
             rows.status = status;
             rows.tokens = static_cast<uint32_t>(p.tokens);
             rows.sequences = static_cast<uint32_t>(p.sequences);
@@ -200,7 +206,8 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
             rows.cache_pages = static_cast<uint32_t>(p.cache_pages);
             rows.causal = p.causal ? 1u : 0u;
             const uint64_t most = static_cast<uint64_t>(p.page_table > p.sequences ? p.page_table : p.sequences);
-            if (int32_t launched = launch(kPagedDecodeRows, static_cast<unsigned>((most + 255) / 256), 1, 1, 256, stream, rows)) return launched;
+            const KernelId bridge = p.index_type == SINGE_HIP_INDEX_I64 ? kPagedDecodeRowsI64 : kPagedDecodeRows;
+            if (int32_t launched = launch(bridge, static_cast<unsigned>((most + 255) / 256), 1, 1, 256, stream, rows)) return launched;
             PagedDecodeLaunch decode;
             decode.stream = stream;
             decode.out = output;
@@ -209,9 +216,9 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
             decode.value_cache = value_cache;
             decode.f16 = f16;
             decode.actual_seq_lens = rows.lengths;
-            decode.block_table = static_cast<const uint32_t*>(pages);
-            decode.workspace = memory + 2 * array_bytes;
-            decode.workspace_bytes = scratch->bytes - 2 * array_bytes;
+            decode.block_table = rows.pages32 != nullptr ? rows.pages32 : static_cast<const uint32_t*>(pages);
+            decode.workspace = memory + 2 * array_bytes + copy_bytes;
+            decode.workspace_bytes = scratch->bytes - 2 * array_bytes - copy_bytes;
             decode.row_starts = rows.row_starts;
             decode.lse = lse;
             return launch_paged_decode(config, decode);

@@ -79,18 +79,19 @@ def test_candidates_agree_where_the_threshold_changes_the_shares(dim):
     kc = torch.randn((page_count, 16, 2, dim), generator=gen, device="cuda").to(torch.bfloat16)
     vc = torch.randn((page_count, 16, 2, dim), generator=gen, device="cuda").to(torch.bfloat16)
     table = np.random.default_rng(3).permutation(page_count)[:sum(pages_of)]
-    # (i64 paging: with i32 a decode step like this one would leave the row-tile kernel for the block-table decode kernels)
-    wide = lambda values: index(values, torch.int64)
-    paging = neural.Paging(wide(list(range(len(lens) + 1))), wide(np.concatenate([[0], np.cumsum(pages_of)])), wide(table),
-                           wide([n - (p - 1) * 16 for n, p in zip(lens, pages_of)]))
-    problem = neural._problem(q, kc, vc, paging, neural.AttentionOptions(causal=True))
+    paging = neural.Paging(index(list(range(len(lens) + 1))), index(np.concatenate([[0], np.cumsum(pages_of)])), index(table),
+                           index([n - (p - 1) * 16 for n, p in zip(lens, pages_of)]))
+    # (a window wider than any context changes nothing but keeps this decode step on the row-tile kernel, whose shares
+    # the thresholds change; without it the step would run on the block-table decode kernels)
+    options = neural.AttentionOptions(causal=True, window=1 << 20)
+    problem = neural._problem(q, kc, vc, paging, options)
     wanted = set()
     for candidate in neural.attention_candidates():
         neural.set_attention_parameters(candidate)
         wanted.add(int(_native.lib().singe_hip_paged_attention_scratch_bytes(ctypes.byref(problem))))
     neural.set_attention_parameters(None)
     assert 0 in wanted and len(wanted) >= 3  # no split at all, and at least two different numbers of shares
-    every_candidate(lambda: neural.paged_attention(q, kc, vc, paging, neural.AttentionOptions(causal=True)))
+    every_candidate(lambda: neural.paged_attention(q, kc, vc, paging, options))
     q4, k4, v4 = tensors((2, 8, 4, dim), (2, 2, 3000, dim), (2, 2, 3000, dim), torch.bfloat16, 5)
     every_candidate(lambda: (neural.scaled_dot_product_attention(q4, k4, v4, None, True),))
 

@@ -268,7 +268,7 @@ def test_a_stream_that_is_not_torchs_current_one_orders_the_fills_and_the_status
     torch.cuda.synchronize()
 
 
-# A decode step (no more tokens than sequences, i32 paging, no window or cap) runs on the block-table decode kernels,
+# A decode step (no more tokens than sequences, no window or cap) runs on the block-table decode kernels,
 # token by token: (queries, keys) per sequence.
 DECODE_STEPS = [
     [(1, 700), (1, 1), (1, 4096), (1, 33), (1, 16)],                      # a token a sequence, ragged
@@ -282,7 +282,8 @@ DECODE_STEPS = [
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("heads, kv_heads, page_size, dim", [(8, 2, 16, 128), (32, 4, 8, 128), (16, 1, 64, 128), (4, 4, 1, 128), (8, 2, 32, 64), (6, 1, 7, 64)])
 @pytest.mark.parametrize("step", range(len(DECODE_STEPS)))
-def test_a_decode_step_through_the_op_matches_the_oracle_and_the_row_tile_kernel(step, heads, kv_heads, page_size, dim, dtype):
+@pytest.mark.parametrize("index_dtype", [torch.int32, torch.int64])
+def test_a_decode_step_through_the_op_matches_the_oracle_and_the_row_tile_kernel(step, heads, kv_heads, page_size, dim, dtype, index_dtype):
     import ctypes
     sequences = DECODE_STEPS[step]
     query_offsets, page_offsets, table, last, page_count = layout(sequences, page_size)
@@ -291,7 +292,7 @@ def test_a_decode_step_through_the_op_matches_the_oracle_and_the_row_tile_kernel
     gen.manual_seed(100 * step + heads)
     rand = lambda *shape: torch.randn(shape, generator=gen, device="cuda").to(dtype)
     q, kc, vc = rand(tokens, heads, dim), rand(page_count, page_size, kv_heads, dim), rand(page_count, page_size, kv_heads, dim)
-    index = lambda values: torch.tensor(values, dtype=torch.int32, device="cuda")
+    index = lambda values: torch.tensor(values, dtype=index_dtype, device="cuda")
     paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
     for options in (neural.AttentionOptions(causal=True), neural.AttentionOptions(scale=0.05)):
         # the scratch the op asks for covers the decode kernels' rows and partials
@@ -313,12 +314,13 @@ def test_a_decode_step_through_the_op_matches_the_oracle_and_the_row_tile_kernel
         assert np.array_equal(np.isneginf(tiled_lse.cpu().numpy()), empty)
 
 
-def test_a_decode_step_keeps_the_error_contract_and_leaves_unowned_tokens_alone():
+@pytest.mark.parametrize("index_dtype", [torch.int32, torch.int64])
+def test_a_decode_step_keeps_the_error_contract_and_leaves_unowned_tokens_alone(index_dtype):
     gen = torch.Generator(device="cuda")
     gen.manual_seed(4)
     q = torch.randn((3, 4, 128), generator=gen, device="cuda").to(torch.bfloat16)
     cache = torch.randn((6, 16, 2, 128), generator=gen, device="cuda").to(torch.bfloat16)
-    index = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
+    index = lambda v: torch.tensor(v, dtype=index_dtype, device="cuda")
     options = neural.AttentionOptions(causal=True)
     good = neural.Paging(index([0, 1, 2, 3]), index([0, 2, 3, 5]), index([4, 1, 0, 2, 5]), index([7, 16, 3]))
     want, want_lse = neural.paged_attention(q, cache, cache, good, options)
