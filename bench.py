@@ -72,7 +72,7 @@ def traffic(key):
     return entry["FETCH_SIZE"] * FETCH_UNIT_BYTES + entry["WRITE_SIZE"] * WRITE_UNIT_BYTES, entry["source"]
 
 
-SECTIONS = ("decode", "prefill", "chunked_prefill", "fp8_decode", "dense_f32", "latent", "cache_append", "head_dim_64",
+SECTIONS = ("decode", "decode_op", "prefill", "chunked_prefill", "fp8_decode", "dense_f32", "latent", "cache_append", "head_dim_64",
             "mfma_ceiling", "hbm_ceiling")
 
 
@@ -779,6 +779,56 @@ def hbm_ceiling_section():
     return result
 
 
+def decode_op_section():
+    """The headline workload through the paged attention op in FlashInfer form (Operation::PagedAttention, the op a
+    graph of the reference decodes with), its paging vectors i64 as the reference's DecodeStep writes them: one token a
+    sequence, causal.  Given scratch the op checks the vectors, gives every token its page list and key count and runs
+    the block-table decode kernels; with a fixed number of shares it stays on its row-tile kernel, timed beside it."""
+    import ctypes
+
+    import numpy as np
+    import torch
+
+    from singe_amd import _native, neural, synthetic
+
+    work = synthetic.paged_decode_workload(portable=True)
+    counts = (work.seq_lens.astype(np.int64) + work.block_size - 1) // work.block_size
+    pages = np.concatenate([work.block_table[b, :n] for b, n in enumerate(counts)]).astype(np.int64)
+    page_offsets = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
+    last = (work.seq_lens.astype(np.int64) - (counts - 1) * work.block_size)
+    index = lambda values: torch.from_numpy(np.ascontiguousarray(values, dtype=np.int64)).cuda()
+    paging = neural.Paging(index(np.arange(work.batch + 1)), index(page_offsets), index(pages), index(last))
+    options = neural.AttentionOptions(causal=True, scale=work.scale)
+    problem = neural._problem(work.query, work.key_cache, work.value_cache, paging, options)
+    out = torch.empty_like(work.query)
+    lse = torch.empty(work.query.shape[:2], device="cuda", dtype=torch.float32)
+    status = torch.zeros(1, device="cuda", dtype=torch.int32)
+    handle = int(torch.cuda.current_stream().cuda_stream)
+    lib = _native.lib()
+    results = {}
+    for name, shares in (("decode_kernels", 0), ("row_tile_kernel", 4)):
+        lib.singe_hip_set_paged_attention_splits(shares)
+        try:
+            scratch = torch.empty(max(int(lib.singe_hip_paged_attention_scratch_bytes(ctypes.byref(problem))), 256), device="cuda", dtype=torch.uint8)
+
+            def launch():
+                _native.check(lib.singe_hip_paged_attention_scratch_bf16(
+                    handle, work.query.data_ptr(), work.key_cache.data_ptr(), work.value_cache.data_ptr(), paging.query_offsets.data_ptr(),
+                    paging.page_offsets.data_ptr(), paging.pages.data_ptr(), paging.last_page_lengths.data_ptr(), out.data_ptr(),
+                    lse.data_ptr(), status.data_ptr(), scratch.data_ptr(), scratch.numel(), ctypes.byref(problem)), "paged_attention")
+
+            stats = measure(launch, 6)
+        finally:
+            lib.singe_hip_set_paged_attention_splits(0)
+        assert int(status.item()) == 0
+        gbps = DECODE_BYTES / (stats["mean_ms"] * 1e-3) / 1e9
+        results[name] = {"us_per_step": stats["mean_ms"] * 1e3, "us_per_step_median": stats["median_ms"] * 1e3, "value": gbps, "unit": "GB/s",
+                         "pct_hbm_peak": 100.0 * gbps / HBM_PEAK_GBPS, "scratch_bytes": scratch.numel(), **timing_fields(stats)}
+    return {"workload": "the headline decode step (BASELINE config 2) through the paged attention op in FlashInfer form, i64 paging, "
+                        "causal; whole op under HIP events (every launch of it)",
+            "algorithmic_bytes": DECODE_BYTES, **results}
+
+
 def decode_section(args, with_cpu):
     """The headline: --warmup untimed steps (and on to 300 ms), exactly --steps timed steps between two synchronisations,
     then the split kernel alone under HIP events."""
@@ -873,7 +923,7 @@ def main():
     with_cpu = not args.no_cpu_baseline
     FEW = bool(args.few and args.only)
     sections = {
-        "prefill": lambda: prefill_section(with_cpu), "chunked_prefill": lambda: chunked_prefill_section(with_cpu),
+        "decode_op": decode_op_section, "prefill": lambda: prefill_section(with_cpu), "chunked_prefill": lambda: chunked_prefill_section(with_cpu),
         "fp8_decode": lambda: fp8_decode_section(with_cpu), "dense_f32": lambda: dense_f32_section(with_cpu),
         "latent": lambda: latent_section(with_cpu), "cache_append": lambda: cache_append_section(with_cpu),
         "head_dim_64": head_dim_64_section, "mfma_ceiling": mfma_ceiling_section,

@@ -327,16 +327,21 @@ SINGE_DEVICE void paged_decode_rows_body(const DecodeRowsArgs& a) {
         }
         return low;
     };
+    // (every load below is asked for before anything waits: the kernel is a chain of memory round trips)
+    const long long page = index < a.page_table ? read_index<FORM>(a.pages, index) : 0;
+    SequenceSpan own;
+    own.valid = false, own.query_start = 0, own.page_start = 0, own.queries = 0, own.keys = 0;
     if (index < a.sequences) {
-        if (!span_of(static_cast<unsigned int>(index)).valid) report_index_error(a.status);
+        own = span_of(static_cast<unsigned int>(index));
+        if (!own.valid) report_index_error(a.status);
     }
     if (index < a.tokens) {
         const long long token = static_cast<long long>(index);
-        unsigned int sequence = static_cast<unsigned int>(index);
-        // One token a sequence, in order, is the usual step: then the owner is found without a search.
-        if (!(index < a.sequences && read_index<FORM>(a.query_offsets, index) == token && read_index<FORM>(a.query_offsets, index + 1) == token + 1))
-            sequence = owner_of(a.query_offsets, token);
-        const SequenceSpan span = span_of(sequence);
+        // One token a sequence, in order, is the usual step: then the token's owner is the sequence of its own index,
+        // whose values are here already; otherwise the owner is searched for.
+        SequenceSpan span = own;
+        if (!(index < a.sequences && own.valid && own.query_start == token && own.queries == 1u))
+            span = span_of(owner_of(a.query_offsets, token));
         unsigned int start = 0;
         long long length = -1;  // no valid sequence owns the token: its row is left alone
         if (span.valid && token >= span.query_start && token - span.query_start < static_cast<long long>(span.queries)) {
@@ -352,7 +357,6 @@ SINGE_DEVICE void paged_decode_rows_body(const DecodeRowsArgs& a) {
         a.lengths[index] = static_cast<int>(length);
     }
     if (index < a.page_table) {
-        const long long page = read_index<FORM>(a.pages, index);
         const bool outside = page < 0 || page >= static_cast<long long>(a.cache_pages);
         if (a.pages32 != nullptr) a.pages32[index] = outside ? 0xffffffffu : static_cast<unsigned int>(page);
         if (outside) {
