@@ -162,9 +162,19 @@ def test_block_table_prefill_replays():
         assert torch.isfinite(out[:owned].float()).all()
 
 
-def test_paged_attention_with_key_splits_replays():
-    """The FlashInfer-form op in decode shape: the attention kernel leaves partials in caller scratch and a second
-    kernel merges them, both recorded."""
+@pytest.mark.parametrize("shares", [0, 4])
+def test_paged_attention_with_key_splits_replays(shares):
+    """The FlashInfer-form op in decode shape, by itself (the kernel that checks the paging vectors and gives every token
+    its row, then the block-table decode kernels) and held to its row-tile kernel by a fixed number of shares (the
+    attention kernel leaves partials in caller scratch and a second kernel merges them): every launch recorded."""
+    _native.lib().singe_hip_set_paged_attention_splits(shares)
+    try:
+        _paged_attention_replays()
+    finally:
+        _native.lib().singe_hip_set_paged_attention_splits(0)
+
+
+def _paged_attention_replays():
     sequences, heads, kv_heads, dim, page, cache_pages = 5, 32, 8, 128, 16, 640
     rng = np.random.default_rng(31)
     cases = [[900, 16, 2000, 333, 1], [2000, 2000, 2000, 2000, 2000], [17, 1999, 64, 0, 700]]
