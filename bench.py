@@ -520,6 +520,15 @@ def latent_section(with_cpu=True):
     if with_cpu:
         decode["cpu_baseline"] = latent_cpu_baseline(decode_operands, 4096, 64, 128)
     del decode_operands
+    # Fewer sequences than compute units: the op shares each one's keys out over the chip (given scratch) and merges.
+    stats, flops, cache_bytes, _ = case([(1, 8192)] * 32, 4)
+    gbps = cache_bytes / (stats["mean_ms"] * 1e-3) / 1e9
+    few = {
+        "workload": "latent attention decode over few sequences: 32 sequences x 8192 keys, 128 heads, latent 512 + positional 64, "
+                    "page 64, bf16; whole op (the attention kernel on shares of each sequence's keys and its merge)",
+        "value": gbps, "unit": "GB/s", "us_per_step": stats["mean_ms"] * 1e3, "us_per_step_median": stats["median_ms"] * 1e3,
+        "algorithmic_bytes": cache_bytes, "algorithmic_flops": flops, "pct_hbm_peak": 100.0 * gbps / HBM_PEAK_GBPS,
+        "tflops": flops / (stats["mean_ms"] * 1e-3) / 1e12, **timing_fields(stats)}
     stats, flops, cache_bytes, _ = case([(512, 8192)] * 8, 1)
     tflops = flops / (stats["mean_ms"] * 1e-3) / 1e12
     nbytes, source = traffic("latent_chunked_prefill")
@@ -532,7 +541,7 @@ def latent_section(with_cpu=True):
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": nbytes, "traffic_source": source, **timing_fields(stats)},
     }
-    return {"decode": decode, "chunked_prefill": chunked}
+    return {"decode": decode, "decode_few_sequences": few, "chunked_prefill": chunked}
 
 
 def cache_append_section(with_cpu=True):
