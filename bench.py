@@ -476,10 +476,12 @@ def latent_section(with_cpu=True):
     page 64), beside the benchmark's configurations: a decode step (256 sequences of 4096 keys; every head reads
     the same 1152 bytes per key, so the step is priced against HBM and the matrix cores both) and a chunked
     prefill (8 x 512 new tokens on 8192 keys, priced against the dense bf16 MFMA peak).  Synthetic N(0,1) data."""
+    import ctypes
+
     import numpy as np
     import torch
 
-    from singe_amd import neural, synthetic
+    from singe_amd import _native, neural, synthetic
 
     def case(sequences, group, heads=128, page=64):
         query_offsets, page_offsets, last, table, pages = [0], [0], [], [], 0
@@ -499,8 +501,27 @@ def latent_section(with_cpu=True):
             ("latent_cache", (pages, page, 512)), ("positional_cache", (pages, page, 64))))
         index = lambda values: torch.tensor(values, dtype=torch.int32, device="cuda")
         paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
-        options = neural.AttentionOptions(causal=True)
-        stats = measure(lambda: neural.paged_mla_attention(*operands, paging, options, check=False), group)
+        # Through the C ABI with the output, the log-sum-exps, the status word and the scratch for key splits allocated
+        # once, as a caller in a serving loop holds them.
+        problem = _native.PagedMlaAttentionProblemC(tokens, heads, 512, 64, page, len(sequences), pages, len(table),
+                                                    neural._DATA_TYPES[torch.bfloat16], 0, 1, 0, 0.0)
+        out = torch.zeros_like(operands[0])
+        lse = torch.full((tokens, heads), float("-inf"), device="cuda", dtype=torch.float32)
+        status = torch.zeros(1, device="cuda", dtype=torch.int32)
+        lib = _native.lib()
+        scratch = torch.empty(max(int(lib.singe_hip_paged_mla_attention_scratch_bytes(ctypes.byref(problem))), 256), device="cuda",
+                              dtype=torch.uint8)
+        handle = int(torch.cuda.current_stream().cuda_stream)
+
+        def launch():
+            _native.check(lib.singe_hip_paged_mla_attention_scratch(
+                handle, operands[0].data_ptr(), operands[1].data_ptr(), operands[2].data_ptr(), operands[3].data_ptr(),
+                paging.query_offsets.data_ptr(), paging.page_offsets.data_ptr(), paging.pages.data_ptr(), paging.last_page_lengths.data_ptr(),
+                out.data_ptr(), lse.data_ptr(), status.data_ptr(), scratch.data_ptr(), scratch.numel(), ctypes.byref(problem)),
+                "paged_mla_attention")
+
+        stats = measure(launch, group)
+        assert int(status.item()) == 0
         pairs = sum(sum(min(keys, max(keys - queries + i, 0) + 1) for i in range(queries)) for queries, keys in sequences)
         flops = pairs * heads * (576 + 512) * 2
         cache_bytes = sum(keys for _, keys in sequences) * 1152 + tokens * heads * (576 + 512) * 2
