@@ -101,3 +101,57 @@ def test_dense_prefill_random_shapes(seed):
     gap = np.abs(got - want)
     assert gap.max() <= MAX_ABS and gap.mean() <= MEAN_ABS, (case, gap.max())
     assert np.abs(lse.cpu().numpy() - want_lse).max() <= LSE_ABS, case
+
+
+@pytest.mark.parametrize("seed", range(32))
+def test_decode_steps_through_the_op_random_shapes(seed):
+    """Random decode steps (no more tokens than sequences: mostly a token a sequence, some sequences with none, a few
+    with two or three) through the paged attention op, which runs them on the block-table decode kernels: against the
+    oracle, both head dimensions, both index types, bf16 and f16, causal or not, up to 16 query heads a kv head."""
+    rng = np.random.default_rng(5000 + seed)
+    kv_heads = int(rng.choice([1, 2, 4, 8]))
+    heads = kv_heads * int(rng.choice([1, 2, 3, 4, 5, 8, 12, 16]))
+    dim = int(rng.choice([128, 128, 64]))
+    page_size = int(rng.choice([1, 3, 8, 16, 16, 32, 64, 24]))
+    dtype = torch.bfloat16 if rng.integers(0, 3) else torch.float16
+    count = int(rng.choice([1, 2, 5, 17, 70, 130]))
+    sequences, spare = [], 0
+    for _ in range(count):
+        keys = int(rng.choice([0, 1, int(rng.integers(1, 64)), int(rng.integers(64, 700)), int(rng.integers(700, 3000))]))
+        queries = int(rng.choice([1, 1, 1, 1, 0, 2, 3]))
+        if queries > 1 and spare < queries - 1:
+            queries = 1
+        spare += 1 - queries
+        sequences.append((queries, keys))
+    if sum(q for q, _ in sequences) == 0:
+        sequences[0] = (1, sequences[0][1])
+    options = neural.AttentionOptions(causal=bool(rng.integers(0, 2)), scale=None if rng.integers(0, 2) else float(rng.uniform(0.02, 0.2)))
+    index_dtype = torch.int64 if rng.integers(0, 2) else torch.int32
+    query_offsets, page_offsets, last = [0], [0], []
+    for queries, keys in sequences:
+        query_offsets.append(query_offsets[-1] + queries)
+        pages = (keys + page_size - 1) // page_size
+        page_offsets.append(page_offsets[-1] + pages)
+        last.append(0 if keys == 0 else keys - (pages - 1) * page_size)
+    needed = page_offsets[-1]
+    page_count = needed + int(rng.integers(1, 5))
+    table = rng.permutation(page_count)[:needed].tolist()
+    tokens = query_offsets[-1]
+    assert 0 < tokens <= len(sequences)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+    rand = lambda *shape: torch.randn(shape, generator=gen, device="cuda").to(dtype)
+    q, kc, vc = rand(tokens, heads, dim), rand(page_count, page_size, kv_heads, dim), rand(page_count, page_size, kv_heads, dim)
+    index = lambda values: torch.tensor(values, dtype=index_dtype, device="cuda")
+    paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
+    out, lse = neural.paged_attention(q, kc, vc, paging, options)
+    torch.cuda.synchronize()
+    status, want, want_lse = oracle.paged_attention_f32(q.float().cpu().numpy(), kc.float().cpu().numpy(), vc.float().cpu().numpy(), query_offsets,
+                                                        page_offsets, table, last, scale=options.scale, causal=options.causal, threads=8)
+    assert status == 0
+    got, got_lse = out.float().cpu().numpy(), lse.cpu().numpy()
+    gap = np.abs(got - want)
+    assert gap.max() <= MAX_ABS and gap.mean() <= MEAN_ABS, (gap.max(), gap.mean())
+    empty = np.isneginf(want_lse)
+    assert np.array_equal(np.isneginf(got_lse), empty) and not got[empty].any()
+    assert np.abs(got_lse[~empty] - want_lse[~empty]).max(initial=0.0) <= LSE_ABS
