@@ -342,3 +342,28 @@ def test_a_decode_step_keeps_the_error_contract_and_leaves_unowned_tokens_alone(
     tiled, tiled_lse = neural.paged_attention(q, cache, cache, edges, options, scratch=False)
     assert (got[1].float() - tiled[1].float()).abs().max().item() <= 8e-3 and (got_lse[1] - tiled_lse[1]).abs().max().item() <= 2e-3
     assert not got[0].any() and not got[2].any() and torch.isneginf(got_lse[0]).all() and torch.isneginf(got_lse[2]).all()
+
+
+@pytest.mark.parametrize("count, heads, kv_heads", [(7900, 4, 2), (3000, 16, 2), (2300, 16, 2)])
+def test_a_decode_step_of_thousands_of_sequences(count, heads, kv_heads):
+    """The decode kernels keep three words a token in LDS on this route: 7900 tokens fill it beside the one-hot form's
+    staging; with eight heads a kv head 3000 tokens no longer fit beside the dense form's and take the one-hot form, 2300 do."""
+    rng = np.random.default_rng(count)
+    sequences = [(1, int(n)) for n in rng.integers(0, 40, count)]
+    query_offsets, page_offsets, table, last, page_count = layout(sequences, 16)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(count)
+    rand = lambda *shape: torch.randn(shape, generator=gen, device="cuda").to(torch.bfloat16)
+    q, kc, vc = rand(count, heads, 128), rand(page_count, 16, kv_heads, 128), rand(page_count, 16, kv_heads, 128)
+    index = lambda values: torch.tensor(values, dtype=torch.int64, device="cuda")
+    paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
+    out, lse = neural.paged_attention(q, kc, vc, paging, neural.AttentionOptions(causal=True))
+    torch.cuda.synchronize()
+    status, want, want_lse = oracle.paged_attention_f32(q.float().cpu().numpy(), kc.float().cpu().numpy(), vc.float().cpu().numpy(), query_offsets,
+                                                        page_offsets, table, last, causal=True, threads=8)
+    assert status == 0
+    gap = np.abs(out.float().cpu().numpy() - want)
+    assert gap.max() <= MAX_ABS and gap.mean() <= MEAN_ABS, (gap.max(), gap.mean())
+    empty = np.isneginf(want_lse)
+    assert np.array_equal(np.isneginf(lse.cpu().numpy()), empty)
+    assert np.abs(lse.cpu().numpy()[~empty] - want_lse[~empty]).max() <= LSE_ABS
