@@ -342,19 +342,32 @@ SINGE_DEVICE void paged_decode_rows_body(const DecodeRowsArgs& a) {
         SequenceSpan span = own;
         if (!(index < a.sequences && own.valid && own.query_start == token && own.queries == 1u))
             span = span_of(owner_of(a.query_offsets, token));
-        unsigned int start = 0;
+        unsigned int start = 0, begin = 0;
         long long length = -1;  // no valid sequence owns the token: its row is left alone
         if (span.valid && token >= span.query_start && token - span.query_start < static_cast<long long>(span.queries)) {
             start = static_cast<unsigned int>(span.page_start);
             length = span.keys;
-            if (a.causal != 0 && span.keys != 0) {
-                const long long raw = static_cast<long long>(span.keys) - static_cast<long long>(span.queries) + (token - span.query_start);
-                const long long reach = (raw < 0 ? 0 : raw) + 1;
-                length = reach < static_cast<long long>(span.keys) ? reach : static_cast<long long>(span.keys);
+            // The token's position among the keys, counted from the end and held at the first key (attention.rs:483).
+            const long long raw = static_cast<long long>(span.keys) - static_cast<long long>(span.queries) + (token - span.query_start);
+            const long long position = raw < 0 ? 0 : raw;
+            if (a.causal != 0 && span.keys != 0) length = position + 1 < static_cast<long long>(span.keys) ? position + 1 : static_cast<long long>(span.keys);
+            if (a.window >= 0 && length > 0) {
+                // Keys with key + window <= position are hidden: whole pages of them are left out of the row, the rest
+                // of the first page is masked by the decode kernel.
+                const long long first = position + 1 - static_cast<long long>(a.window);
+                if (first >= length) {
+                    length = 0;  // (a window of no keys)
+                } else if (first > 0) {
+                    const long long skipped = first / a.page_size;
+                    start += static_cast<unsigned int>(skipped);
+                    length -= skipped * a.page_size;
+                    begin = static_cast<unsigned int>(first - skipped * a.page_size);
+                }
             }
         }
         a.row_starts[index] = start;
         a.lengths[index] = static_cast<int>(length);
+        if (a.row_begins != nullptr) a.row_begins[index] = begin;
     }
     if (index < a.page_table) {
         const bool outside = page < 0 || page >= static_cast<long long>(a.cache_pages);
@@ -362,7 +375,14 @@ SINGE_DEVICE void paged_decode_rows_body(const DecodeRowsArgs& a) {
         if (outside) {
             const SequenceSpan span = span_of(owner_of(a.page_offsets, static_cast<long long>(index)));
             const long long entry = static_cast<long long>(index) - span.page_start;
-            if (span.valid && span.queries != 0 && entry >= 0 && entry * a.page_size < static_cast<long long>(span.keys)) report_index_error(a.status);
+            // (under a window the pages wholly before the first token's window are read by nobody)
+            long long unread = 0;
+            if (a.window >= 0) {
+                const long long raw = static_cast<long long>(span.keys) - static_cast<long long>(span.queries);
+                const long long first = (raw < 0 ? 0 : raw) + 1 - static_cast<long long>(a.window);
+                unread = first > 0 ? first / a.page_size : 0;
+            }
+            if (span.valid && span.queries != 0 && entry >= unread && entry * a.page_size < static_cast<long long>(span.keys)) report_index_error(a.status);
         }
     }
 }

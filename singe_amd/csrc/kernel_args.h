@@ -32,6 +32,9 @@ struct DecodeArgs {
     // Table rows of their own lengths (the paged attention op's page lists): row b starts at entry row_starts[b] of
     // block_table, which then holds block_table_batch_stride entries in all; null: rows are that stride apart.
     const uint32_t* row_starts = nullptr;
+    // With row_starts: the first row_begins[b] keys of row b are hidden (a sliding window's keys before the page the
+    // row starts in could be left out of the row; those inside that page are masked), or null.
+    const uint32_t* row_begins = nullptr;
 };
 
 struct CombineArgs {
@@ -339,8 +342,10 @@ struct DecodeRowsArgs {
     uint32_t* row_starts;           // [tokens]
     int32_t* lengths;               // [tokens]: -1 for a token no valid sequence owns
     uint32_t* pages32;              // [page_table] (i64 paging), else null
+    uint32_t* row_begins;           // [tokens] (a window), else null: keys of the row's first page that lie before the window
     uint32_t* status;
     uint32_t tokens, sequences, page_table, page_size, cache_pages, causal;
+    int32_t window;                 // a token sees the `window` keys up to its own position; -1: all of them
 };
 
 // singe_paging_indices_*: FlashInfer CSR paging -> block-table paging.

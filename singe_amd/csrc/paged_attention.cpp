@@ -78,22 +78,29 @@ uint32_t paged_attention_splits(const SingePagedAttentionProblem& p) {
     const RowTileGrid tiling = grid_of(static_cast<uint64_t>(p.tokens), static_cast<uint64_t>(p.sequences), groups);
     const uint64_t workgroups = static_cast<uint64_t>(p.kv_heads) * (tiling.compact ? tiling.row_tiles : tiling.row_tiles * static_cast<uint64_t>(p.sequences));
     // The sequences' key counts live in device memory: the page table bounds their sum, and shares are sized for
-    // a sequence of average length.
-    const uint64_t keys = static_cast<uint64_t>(p.page_table > 0 ? p.page_table : 0) * static_cast<uint64_t>(p.page_size) / static_cast<uint64_t>(p.sequences);
+    // a sequence of average length, or for the window when that is shorter (the tiles before it are skipped).
+    uint64_t keys = static_cast<uint64_t>(p.page_table > 0 ? p.page_table : 0) * static_cast<uint64_t>(p.page_size) / static_cast<uint64_t>(p.sequences);
+    if (p.has_window && static_cast<uint64_t>(p.window) < keys) keys = static_cast<uint64_t>(p.window);
     return attention_key_splits(workgroups, keys);
 }
 
 // A decode step (no more tokens than sequences: a token a sequence) through this op takes the block-table decode
 // kernels, which cut the keys of all sequences into equal ranges whatever their lengths: a small kernel first turns
 // the paging vectors into one row per token (where its page list starts, how many keys it sees) and checks them.
-// What the host can tell: a matrix-core decode build for the head dimension, no window, cap or fused rotation, and
+// What the host can tell: a matrix-core decode build for the head dimension, no cap or fused rotation, and
 // sizes the decode kernels take.  (The decode kernels read 32-bit page ids: i64 paging is copied on the way.)
 constexpr size_t kDecodeRowsMost = 8000;
 
 bool decode_rows_config(const SingePagedAttentionProblem& p, SingePagedKvDecodeAttentionConfig* config) {
     if (g_paged_attention_splits != 0) return false;  // a fixed number of shares asks for the row-tile kernel
-    if ((p.head_dim != 128 && p.head_dim != 64) || p.has_window || p.has_softcap) return false;
-    if (p.tokens <= 0 || p.tokens > p.sequences || static_cast<size_t>(p.tokens) > kDecodeRowsMost || p.page_table <= 0 || p.cache_pages <= 0)
+    if ((p.head_dim != 128 && p.head_dim != 64) || p.has_softcap) return false;
+    // Under a short window a token reads few keys, and one workgroup a (sequence, kv head) of the row-tile kernel, which
+    // skips the tiles before the window, is done before the route's two extra launches would be (measured: 32 sequences,
+    // window 128: 12.6 against 15.2 us; window 1024: level; window 4096: 70 against 57 us).
+    if (p.has_window && p.window < 2048) return false;
+    // (the decode kernels keep three words a token in LDS, four under a window)
+    if (p.tokens <= 0 || p.tokens > p.sequences || static_cast<size_t>(p.tokens) > (p.has_window ? kDecodeRowsMost * 3 / 4 : kDecodeRowsMost) ||
+        p.page_table <= 0 || p.cache_pages <= 0)
         return false;
     if (!fits_i32(static_cast<uint64_t>(p.page_table) * static_cast<uint64_t>(p.page_size))) return false;
     config->batch = static_cast<size_t>(p.tokens);
@@ -117,7 +124,8 @@ size_t decode_rows_page_copy_bytes(const SingePagedAttentionProblem& p) {
 size_t decode_rows_bytes(const SingePagedAttentionProblem& p) {
     SingePagedKvDecodeAttentionConfig config;
     if (!decode_rows_config(p, &config)) return 0;
-    return 2 * align256(static_cast<size_t>(p.tokens) * sizeof(uint32_t)) + decode_rows_page_copy_bytes(p) + paged_decode_workspace_bytes(config);
+    return (p.has_window ? 3 : 2) * align256(static_cast<size_t>(p.tokens) * sizeof(uint32_t)) + decode_rows_page_copy_bytes(p) +
+           paged_decode_workspace_bytes(config);
 }
 
 size_t scratch_bytes_for(const SingePagedAttentionProblem& p, uint32_t splits) {
@@ -197,7 +205,10 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
             rows.row_starts = reinterpret_cast<uint32_t*>(memory);
             rows.lengths = reinterpret_cast<int32_t*>(memory + array_bytes);
             const size_t copy_bytes = decode_rows_page_copy_bytes(p);
-            rows.pages32 = copy_bytes != 0 ? reinterpret_cast<uint32_t*>(memory + 2 * array_bytes) : nullptr;
+            const size_t arrays = p.has_window ? 3 : 2;
+            rows.row_begins = p.has_window ? reinterpret_cast<uint32_t*>(memory + 2 * array_bytes) : nullptr;
+            rows.window = !p.has_window ? -1 : p.window > 0x7fffffffll ? 0x7fffffff : static_cast<int32_t>(p.window);  // (positions fit 31 bits)
+            rows.pages32 = copy_bytes != 0 ? reinterpret_cast<uint32_t*>(memory + arrays * array_bytes) : nullptr;
             rows.status = status;
             rows.tokens = static_cast<uint32_t>(p.tokens);
             rows.sequences = static_cast<uint32_t>(p.sequences);
@@ -217,9 +228,10 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
             decode.f16 = f16;
             decode.actual_seq_lens = rows.lengths;
             decode.block_table = rows.pages32 != nullptr ? rows.pages32 : static_cast<const uint32_t*>(pages);
-            decode.workspace = memory + 2 * array_bytes + copy_bytes;
-            decode.workspace_bytes = scratch->bytes - 2 * array_bytes - copy_bytes;
+            decode.workspace = memory + arrays * array_bytes + copy_bytes;
+            decode.workspace_bytes = scratch->bytes - arrays * array_bytes - copy_bytes;
             decode.row_starts = rows.row_starts;
+            decode.row_begins = rows.row_begins;
             decode.lse = lse;
             return launch_paged_decode(config, decode);
         }

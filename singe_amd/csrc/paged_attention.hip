@@ -221,7 +221,8 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     const unsigned int my_token = (row_valid ? my_row : first_row) / groups, my_head = (row_valid ? my_row : first_row) % groups;
     const unsigned int my_position = position_of(row_valid ? my_row : first_row);
     const bool causal = a.causal != 0, windowed = a.window >= 0;
-    const unsigned int window = windowed ? static_cast<unsigned int>(a.window) : 0u;
+    // (positions fit 31 bits: a wider window hides nothing, and is held there so that key + window cannot wrap)
+    const unsigned int window = !windowed ? 0u : a.window > 0x7fffffffll ? 0x7fffffffu : static_cast<unsigned int>(a.window);
 
     // Rows of this wave: none when the wave starts past the sequence's rows.
     const unsigned int wave_first_row = first_row + wave * 32u;

@@ -263,7 +263,7 @@ int32_t launch_paged_decode(const SingePagedKvDecodeAttentionConfig& c, const Pa
     // caches with more than four query heads per kv head at head_dim 128, where the one-hot form would carry two
     // groups per wave, as long as the batch's prefix sums fit beside that form's 132 KiB of staging in LDS.
     // (the kernel keeps the sequences' tile prefix sums and lengths in LDS, and their rows' starts when rows have their own lengths)
-    const unsigned prefix_bytes = static_cast<unsigned>(((l.row_starts != nullptr ? 3 : 2) * c.batch + 1) * sizeof(uint32_t));
+    const unsigned prefix_bytes = static_cast<unsigned>(((l.row_starts == nullptr ? 2 : l.row_begins == nullptr ? 3 : 4) * c.batch + 1) * sizeof(uint32_t));
     constexpr unsigned kWideStagingBytes = 135168, kLdsBytes = 160 * 1024;
     const bool wide = !fp8 && !narrow && c.heads / c.kv_heads > 4 && kWideStagingBytes + prefix_bytes <= kLdsBytes;
     const Plan plan = make_plan(c, wide || fp8 ? 16 : 8);  // (the dense form of fp8 caches has its Q^T in registers and no such limit)
@@ -281,6 +281,7 @@ int32_t launch_paged_decode(const SingePagedKvDecodeAttentionConfig& c, const Pa
     args.actual_seq_lens = l.actual_seq_lens;
     args.block_table = l.block_table;
     args.row_starts = l.row_starts;
+    args.row_begins = l.row_starts != nullptr ? l.row_begins : nullptr;
     args.meta = reinterpret_cast<uint32_t*>(scratch);
     args.partial_lse = reinterpret_cast<float*>(scratch + plan.lse_offset);
     args.partial_out = reinterpret_cast<float*>(scratch + plan.out_offset);

@@ -362,6 +362,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
     // clamped to what its table row can address.
     unsigned int* lengths = prefix + a.batch + 1;
     unsigned int* starts = lengths + a.batch;  // rows of their own lengths: where each begins in the table (the launch then lends a third array)
+    unsigned int* begins = starts + a.batch;   // and, under a window, how many of its first keys are hidden (a fourth)
     if (wave == 0) {
         unsigned int carry = 0;
         for (unsigned int base = 0; base < a.batch; base += 64) {
@@ -381,6 +382,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
                 prefix[base + lane + 1] = carry + scan;
                 lengths[base + lane] = len;
                 if (a.row_starts != nullptr) starts[base + lane] = a.row_starts[base + lane];
+                if (a.row_begins != nullptr) begins[base + lane] = a.row_begins[base + lane];
             }
             carry += __shfl(scan, 63, 64);
         }
@@ -714,6 +716,15 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
                 fill_entries<FP8>(entries, a, load_seq, row_base, low, kv_head, lane);
         }
         load_tile<ALIGNED16>(buffer, a, a.block_table + row_base, entries, first_key, end, kv_head, g, t);
+        if (a.row_begins != nullptr) {
+            // Keys of the row before its window (bit half * 4 + i of `live` is key first_key + 16 half + 4 g + i).
+            const unsigned int begin = begins[load_seq];
+            if (begin > first_key) {
+#pragma unroll
+                for (int bit = 0; bit < 8; ++bit)
+                    if (first_key + 16u * (bit >> 2) + 4u * g + (bit & 3) < begin) buffer.live &= ~(1u << bit);
+            }
+        }
         ++load_at;
     };
     auto consume = [&](const Tile& buffer) __attribute__((always_inline)) {

@@ -64,6 +64,7 @@ struct PagedDecodeLaunch {
     size_t workspace_bytes = 0;
     uint32_t phases = 3;
     const uint32_t* row_starts = nullptr;
+    const uint32_t* row_begins = nullptr;  // with row_starts: keys at the front of each row that a window hides, or null
     float* lse = nullptr;
 };
 int32_t launch_paged_decode(const SingePagedKvDecodeAttentionConfig& config, const PagedDecodeLaunch& launch);

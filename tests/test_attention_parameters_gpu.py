@@ -81,9 +81,9 @@ def test_candidates_agree_where_the_threshold_changes_the_shares(dim):
     table = np.random.default_rng(3).permutation(page_count)[:sum(pages_of)]
     paging = neural.Paging(index(list(range(len(lens) + 1))), index(np.concatenate([[0], np.cumsum(pages_of)])), index(table),
                            index([n - (p - 1) * 16 for n, p in zip(lens, pages_of)]))
-    # (a window wider than any context changes nothing but keeps this decode step on the row-tile kernel, whose shares
-    # the thresholds change; without it the step would run on the block-table decode kernels)
-    options = neural.AttentionOptions(causal=True, window=1 << 20)
+    # (a score cap keeps this decode step on the row-tile kernel, whose shares the thresholds change; without one the
+    # step would run on the block-table decode kernels)
+    options = neural.AttentionOptions(causal=True, softcap=50.0)
     problem = neural._problem(q, kc, vc, paging, options)
     wanted = set()
     for candidate in neural.attention_candidates():

@@ -271,9 +271,9 @@ def test_a_stream_that_is_not_torchs_current_one_orders_the_fills_and_the_status
 # A decode step (no more tokens than sequences, no window or cap) runs on the block-table decode kernels,
 # token by token: (queries, keys) per sequence.
 DECODE_STEPS = [
-    [(1, 700), (1, 1), (1, 4096), (1, 33), (1, 16)],                      # a token a sequence, ragged
+    [(1, 700), (1, 1), (1, 4096), (1, 33), (1, 16), (1, 2049), (1, 5003)], # a token a sequence, ragged
     [(1, 300), (0, 500), (1, 0), (1, 64), (0, 0), (1, 1500)],             # sequences without a token, a token without keys
-    [(2, 900), (0, 40), (1, 17), (0, 2000)],                              # two tokens of one sequence, as many tokens as sequences
+    [(2, 2900), (0, 40), (1, 17), (0, 2000)],                             # two tokens of one sequence, as many tokens as sequences
     [(3, 2), (0, 5), (0, 7), (1, 129)],                                   # more queries than keys
     [(1, 128 * (b % 5) + b) for b in range(1, 70)],                       # more sequences than a wave has lanes
 ]
@@ -294,21 +294,27 @@ def test_a_decode_step_through_the_op_matches_the_oracle_and_the_row_tile_kernel
     q, kc, vc = rand(tokens, heads, dim), rand(page_count, page_size, kv_heads, dim), rand(page_count, page_size, kv_heads, dim)
     index = lambda values: torch.tensor(values, dtype=index_dtype, device="cuda")
     paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
-    for options in (neural.AttentionOptions(causal=True), neural.AttentionOptions(scale=0.05)):
+    # (windows from 2048 keys on take the decode kernels too: whole pages before the window are left out of a token's row,
+    # the keys of its first page before the window are masked; shorter ones stay on the row-tile kernel)
+    windows = (neural.AttentionOptions(causal=True, window=2048), neural.AttentionOptions(causal=True, window=2500), neural.AttentionOptions(window=2077),
+               neural.AttentionOptions(causal=True, window=100), neural.AttentionOptions(causal=True, window=1 << 40))
+    for options in (neural.AttentionOptions(causal=True), neural.AttentionOptions(scale=0.05)) + (windows if dtype == torch.bfloat16 else ()):
         # the scratch the op asks for covers the decode kernels' rows and partials
         problem = neural._problem(q, kc, vc, paging, options)
-        assert _native.lib().singe_hip_paged_attention_scratch_bytes(ctypes.byref(problem)) >= 2 * 256 + 4 * tokens * heads * (dim + 1)
+        if options.window is None or options.window >= 2048:
+            assert _native.lib().singe_hip_paged_attention_scratch_bytes(ctypes.byref(problem)) >= 2 * 256 + 4 * tokens * heads * (dim + 1)
         out, lse = neural.paged_attention(q, kc, vc, paging, options)
         tiled, tiled_lse = neural.paged_attention(q, kc, vc, paging, options, scratch=False)
         torch.cuda.synchronize()
         status, want, want_lse = oracle.paged_attention_f32(q.float().cpu().numpy(), kc.float().cpu().numpy(), vc.float().cpu().numpy(), query_offsets,
-                                                            page_offsets, table, last, scale=options.scale, causal=options.causal, threads=8)
+                                                            page_offsets, table, last, scale=options.scale, causal=options.causal,
+                                                            window=options.window, threads=8)
         assert status == 0
         got, got_lse = out.float().cpu().numpy(), lse.cpu().numpy()
         gap = np.abs(got - want)
-        assert gap.max() <= MAX_ABS and gap.mean() <= MEAN_ABS, (gap.max(), gap.mean())
+        assert gap.max() <= MAX_ABS and gap.mean() <= MEAN_ABS, (options, gap.max(), gap.mean())
         empty = np.isneginf(want_lse)
-        assert np.array_equal(np.isneginf(got_lse), empty) and not got[empty].any()
+        assert np.array_equal(np.isneginf(got_lse), empty) and not got[empty].any(), options
         assert np.abs(got_lse[~empty] - want_lse[~empty]).max(initial=0.0) <= LSE_ABS
         assert (out.float() - tiled.float()).abs().max().item() <= 8e-3
         assert np.array_equal(np.isneginf(tiled_lse.cpu().numpy()), empty)

@@ -107,7 +107,8 @@ def test_dense_prefill_random_shapes(seed):
 def test_decode_steps_through_the_op_random_shapes(seed):
     """Random decode steps (no more tokens than sequences: mostly a token a sequence, some sequences with none, a few
     with two or three) through the paged attention op, which runs them on the block-table decode kernels: against the
-    oracle, both head dimensions, both index types, bf16 and f16, causal or not, up to 16 query heads a kv head."""
+    oracle, both head dimensions, both index types, bf16 and f16, causal or not, with and without a window, up to 16 query
+    heads a kv head."""
     rng = np.random.default_rng(5000 + seed)
     kv_heads = int(rng.choice([1, 2, 4, 8]))
     heads = kv_heads * int(rng.choice([1, 2, 3, 4, 5, 8, 12, 16]))
@@ -117,7 +118,7 @@ def test_decode_steps_through_the_op_random_shapes(seed):
     count = int(rng.choice([1, 2, 5, 17, 70, 130]))
     sequences, spare = [], 0
     for _ in range(count):
-        keys = int(rng.choice([0, 1, int(rng.integers(1, 64)), int(rng.integers(64, 700)), int(rng.integers(700, 3000))]))
+        keys = int(rng.choice([0, 1, int(rng.integers(1, 64)), int(rng.integers(64, 700)), int(rng.integers(700, 3000)), int(rng.integers(2048, 4500))]))
         queries = int(rng.choice([1, 1, 1, 1, 0, 2, 3]))
         if queries > 1 and spare < queries - 1:
             queries = 1
@@ -125,7 +126,8 @@ def test_decode_steps_through_the_op_random_shapes(seed):
         sequences.append((queries, keys))
     if sum(q for q, _ in sequences) == 0:
         sequences[0] = (1, sequences[0][1])
-    options = neural.AttentionOptions(causal=bool(rng.integers(0, 2)), scale=None if rng.integers(0, 2) else float(rng.uniform(0.02, 0.2)))
+    options = neural.AttentionOptions(causal=bool(rng.integers(0, 2)), scale=None if rng.integers(0, 2) else float(rng.uniform(0.02, 0.2)),
+                                      window=None if rng.integers(0, 2) else int(rng.choice([1, 100, 2048, 2300, 2999, 5000])))
     index_dtype = torch.int64 if rng.integers(0, 2) else torch.int32
     query_offsets, page_offsets, last = [0], [0], []
     for queries, keys in sequences:
@@ -147,7 +149,8 @@ def test_decode_steps_through_the_op_random_shapes(seed):
     out, lse = neural.paged_attention(q, kc, vc, paging, options)
     torch.cuda.synchronize()
     status, want, want_lse = oracle.paged_attention_f32(q.float().cpu().numpy(), kc.float().cpu().numpy(), vc.float().cpu().numpy(), query_offsets,
-                                                        page_offsets, table, last, scale=options.scale, causal=options.causal, threads=8)
+                                                        page_offsets, table, last, scale=options.scale, causal=options.causal,
+                                                        window=options.window, threads=8)
     assert status == 0
     got, got_lse = out.float().cpu().numpy(), lse.cpu().numpy()
     gap = np.abs(got - want)
