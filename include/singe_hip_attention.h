@@ -424,7 +424,7 @@ SINGE_HIP_API int32_t singe_hip_paged_attention_bf16(
  * the order of summation.  singe_hip_set_paged_attention_splits fixes the number of shares (0 = chosen by
  * problem size, the default), the counterpart of TuningChoice::Explicit
  * (singe-kernel/src/cuda/attention/mod.rs:2364-2380); it changes what ..._scratch_bytes returns.
- * A decode step (no more tokens than sequences, head_dim 128 or 64, no softcap) given
+ * A decode step (no more tokens than sequences, head_dim 128 or 64, no softcap, no window below 2048 keys) given
  * scratch on a 256-byte boundary runs on the block-table decode kernels instead, which cut the keys of all
  * sequences into equal ranges: a first kernel checks the paging vectors (same status word) and gives each token
  * its page list and key count, and the scratch then also holds those and the decode kernels' partial rows.  The
