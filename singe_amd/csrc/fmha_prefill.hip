@@ -16,7 +16,6 @@
 // XCD i % 8; ids are laid out so the workgroups of one (batch, head) are neighbours on one XCD and walk
 // its keys side by side, which keeps its K/V in that XCD's L2.
 #include "kernel_args.h"
-#define SINGE_WEAVE_FIRST 1  // the dense kernel gains 2 % by it, the paged one loses 1.5 % (prefill_blocks.hip.h)
 #include "prefill_blocks.hip.h"
 
 namespace {

@@ -30,12 +30,6 @@ constexpr int kStagedLdsBytes = (kKeyStages + kValueStages) * kTileBytes;
 
 typedef unsigned int __attribute__((address_space(3))) * lds_words_t;
 
-// Whether a wave goes ahead of the other wave of its SIMD while it turns scores into weights (finish_block): the
-// kernel source that includes this file defines SINGE_WEAVE_FIRST to 1 to ask for it.
-#ifndef SINGE_WEAVE_FIRST
-#define SINGE_WEAVE_FIRST 0
-#endif
-constexpr bool kWeaveFirst = SINGE_WEAVE_FIRST != 0;
 
 // Per-lane LDS read offsets inside a 32-key block, kept as a base and the bits the row's permutation
 // flips so that each read's offset costs one xor-add instead of a register.
@@ -139,10 +133,11 @@ SINGE_DEVICE void finish_block(Half half, RowState& state, f32x16_t& s, float fa
     float total = 0.0f;
     // The two waves of a SIMD belong to different workgroups and drift apart.  While this one turns scores into weights
     // (a dependent chain on the vector unit, with the next block's score products in between) it goes first; during its
-    // value products, which only need the matrix core to be free, the other one does.  Measured on the dense prefill:
-    // 0.580 -> 0.567 ms (the same priority around the value products instead: 0.592 ms; levels 1 to 3 alike); on the
-    // chunked paged prefill 1.232 -> 1.249 ms, so the kernel that includes this file says whether it wants it.
-    if constexpr (kWeaveFirst) __builtin_amdgcn_s_setprio(1);
+    // value products, which only need the matrix core to be free, the other one does.  Together with the priority
+    // around a tile's loads (fold_interior_tile), measured on the dense prefill: 0.580 -> 0.566 ms, on the chunked
+    // paged prefill 1.257 -> 1.249 ms; this one alone: 0.567 ms and, on the paged kernel, a loss (1.232 -> 1.249 ms);
+    // around the value products instead: 0.592 ms; levels 1 to 3 alike.
+    __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int step = 0; step < 8; ++step) {
         if (step == 4) {
@@ -165,7 +160,7 @@ SINGE_DEVICE void finish_block(Half half, RowState& state, f32x16_t& s, float fa
         s[2 * step + 1] = fast_exp2(fmaf(s[2 * step + 1], factor, shift));
         total += s[2 * step] + s[2 * step + 1];
     }
-    if constexpr (kWeaveFirst) __builtin_amdgcn_s_setprio(0);
+    __builtin_amdgcn_s_setprio(0);
     state.running_sum += total;
     // O^T += V^T . P^T, 16 keys per MFMA: registers 8j .. 8j+7 are keys 16j + {0..3, 8..11} + 4hi.
 #pragma unroll
@@ -216,7 +211,10 @@ SINGE_DEVICE void fold_interior_tile(Half half, RowState& state, f32x16_t& score
                                      const unsigned char* __restrict__ next_keys, const unsigned char* __restrict__ values,
                                      unsigned char* __restrict__ key_dest, unsigned char* __restrict__ value_dest, Issue&& issue,
                                      Shape&& shape) {
+    // (the tile's loads and their address arithmetic go out ahead of the other wave's work: see finish_block)
+    __builtin_amdgcn_s_setprio(2);
     issue(key_dest, value_dest);
+    __builtin_amdgcn_s_setprio(0);
     shape(scores, 0u);
     const float shift_even = begin_block(state, scores, hi, factor, false, [](unsigned int) { return false; });
     finish_block<true, AHEAD>(half, state, scores, factor, shift_even, values, offsets, scores, q, keys + kBlockBytes, operand, next_keys);
