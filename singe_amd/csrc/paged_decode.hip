@@ -703,6 +703,9 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
     EntryCache entries;
     auto issue = [&](Tile& buffer) __attribute__((always_inline)) {
         if (load_at >= range_end) return;
+        // A tile's requests (table entries, address arithmetic, loads) go out ahead of the SIMD's other wave's folding:
+        // the split kernel 51.95 -> 51.5 us, the fp8 one 778 -> 767 us (four rounds each way on one box).
+        __builtin_amdgcn_s_setprio(2);
         while (prefix[load_seq + 1] <= load_at) ++load_seq;  // skips empty sequences
         const unsigned int first_key = (load_at - prefix[load_seq]) * kTile, end = lengths[load_seq];
         const size_t row_base = a.row_starts != nullptr ? starts[load_seq] : static_cast<size_t>(load_seq) * a.block_table_batch_stride;
@@ -726,6 +729,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
             }
         }
         ++load_at;
+        __builtin_amdgcn_s_setprio(0);
     };
     auto consume = [&](const Tile& buffer) __attribute__((always_inline)) {
         // Returns false when this was the last tile of the range.
