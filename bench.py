@@ -87,6 +87,9 @@ def parse():
     parser.add_argument("--only", choices=SECTIONS, default=None,
                         help="run one section alone and print it (for profiler and counter runs of its kernel)")
     parser.add_argument("--few", action="store_true", help="with --only: a handful of launches, no warm-up (counter runs)")
+    parser.add_argument("--full", action="store_true", help="print every section's detail as the one line (about 19 KB)")
+    parser.add_argument("--detail", default=os.path.join(ROOT, "gpurun_out", "bench_detail.json"),
+                        help="file that receives every section's detail beside the compact line ('' for none)")
     return parser.parse_args()
 
 
@@ -986,7 +989,98 @@ def main():
     result["roofline"]["frac_of_measured_ceiling"] = result["roofline"]["achieved"] / result["hbm_ceiling"]["decode_sized"]["value"]
     result["fp8_decode"]["roofline"]["frac_of_measured_ceiling"] = (result["fp8_decode"]["roofline"]["achieved"]
                                                                     / result["hbm_ceiling"]["fp8_decode_sized"]["value"])
-    print(json.dumps(result), flush=True)
+    if args.full:
+        print(json.dumps(result), flush=True)
+        return
+    if args.detail:
+        try:
+            os.makedirs(os.path.dirname(os.path.abspath(args.detail)), exist_ok=True)
+            with open(args.detail, "w") as handle:
+                json.dump(result, handle)
+        except OSError as problem:  # the detail file is a convenience; the line below is the result
+            print(f"bench.py: detail file not written: {problem}", file=sys.stderr)
+    print(json.dumps(compact(result), separators=(",", ":")), flush=True)
+
+
+def _rounded(value, digits=4):
+    if isinstance(value, float):
+        return float(f"{value:.{digits}g}")
+    return value
+
+
+def _config_summary(section, ms=None):
+    """The figures of one benchmark configuration that the compact line keeps: the kernel and its time, what it
+    achieved against which peak (and against the ceiling measured in the same run), counter traffic, and the CPU
+    baseline's value and core count."""
+    roofline = section.get("roofline", {})
+    baseline = section.get("cpu_baseline", {})
+    if ms is None:
+        ms = section.get("ms_per_step", section.get("value", 0.0) * 1e-3 if section.get("unit") == "us" else None)
+    summary = {"kernel": roofline.get("kernel", section.get("kernel")), "ms_per_step": ms,
+               "iqr_us": roofline.get("kernel_iqr_us", section.get("kernel_iqr_us")),
+               "achieved": roofline.get("achieved"), "peak": roofline.get("peak"), "unit": roofline.get("unit"),
+               "frac": roofline.get("frac"), "frac_of_measured_ceiling": roofline.get("frac_of_measured_ceiling"),
+               "traffic": roofline.get("traffic"),
+               "cpu_baseline": {"value": baseline.get("value"), "unit": baseline.get("unit"), "cores": baseline.get("cores"),
+                                "row_parallel": baseline.get("row_parallel", {}).get("value"),
+                                "row_parallel_cores": baseline.get("row_parallel", {}).get("cores")}}
+    return {name: _rounded(value) if not isinstance(value, dict) else {k: _rounded(v) for k, v in value.items()}
+            for name, value in summary.items()}
+
+
+def compact(result):
+    """The line the run ends with: the headline's fields as they are, and inside `roofline` one short object per
+    further benchmark configuration (`configs`), the two measured ceilings, the whole decode op beside its dominant
+    kernel, and the fraction of its roofline every other measured kernel reached (`others`).  Everything else is in
+    the --detail file (or the --full line)."""
+    line = {name: result[name] for name in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
+                                            "higher_is_better", "scaling", "vs_baseline", "dtype", "data", "config",
+                                            "tokens_per_s", "pct_hbm_peak")}
+    line["data"] = "synthetic (seeded splitmix64 N(0,1), base seed 0x51A6E)"
+    roofline = {name: _rounded(value, 6) for name, value in result["roofline"].items() if name != "traffic_source"}
+    roofline["whole_op_frac"] = _rounded(result["pct_hbm_peak"] / 100.0)
+    roofline["whole_op_frac_under_events"] = _rounded(result["step_under_events"]["pct_hbm_peak"] / 100.0)
+    roofline["ceilings"] = {
+        "mfma_bf16_register_loop_normal_tflops": _rounded(result["mfma_ceiling"]["normal"]["value"]),
+        "mfma_bf16_register_loop_zeros_tflops": _rounded(result["mfma_ceiling"]["zeros"]["value"]),
+        "hbm_stream_read_decode_sized_gbps": _rounded(result["hbm_ceiling"]["decode_sized"]["value"]),
+        "hbm_stream_read_fp8_decode_sized_gbps": _rounded(result["hbm_ceiling"]["fp8_decode_sized"]["value"])}
+    configs = {}
+    if "unsupported" not in result.get("dense_f32", {"unsupported": 1}):
+        configs["1_dense_f32"] = _config_summary(result["dense_f32"])
+    for label, name in (("3_prefill", "prefill"), ("4_chunked_prefill", "chunked_prefill"), ("5_fp8_decode", "fp8_decode")):
+        if "unsupported" not in result.get(name, {"unsupported": 1}):
+            configs[label] = _config_summary(result[name])
+    if "5_fp8_decode" in configs:
+        configs["5_fp8_decode"]["whole_op_frac"] = _rounded(result["fp8_decode"]["pct_hbm_peak"] / 100.0)
+    roofline["configs"] = configs
+    others = {}
+
+    def note(label, section):
+        inner = section.get("roofline", {})
+        if "frac" in inner:
+            others[label] = _rounded(inner["frac"])
+        elif "pct_hbm_peak" in section:
+            others[label] = _rounded(section["pct_hbm_peak"] / 100.0)
+
+    for name in ("latent", "head_dim_64", "decode_op"):
+        for label, section in result.get(name, {}).items():
+            if isinstance(section, dict):
+                note(f"{name}.{label}", section)
+                if "pct_hbm_peak" in section and "roofline" in section:
+                    others[f"{name}.{label}.whole_op"] = _rounded(section["pct_hbm_peak"] / 100.0)
+    if "roofline" in result.get("cache_append", {}):
+        note("cache_append", result["cache_append"])
+    roofline["others"] = others
+    line["roofline"] = roofline
+    baseline = result.get("cpu_baseline")
+    if baseline:
+        line["cpu_baseline"] = {"value": _rounded(baseline["value"]), "unit": baseline["unit"], "cores": baseline["cores"],
+                                "kind": baseline["kind"], "sample": baseline["sample"],
+                                "row_parallel": {k: _rounded(v) for k, v in baseline.get("row_parallel", {}).items()
+                                                 if k != "sample"},
+                                "host": baseline.get("host")}
+    return line
 
 
 if __name__ == "__main__":

@@ -12,8 +12,9 @@
  * that this library loads with hipModuleLoadData and launches with hipModuleLaunchKernel, in place of
  * the reference's NVRTC -> cuModuleLoadData -> cuLaunchKernelEx path
  * (singe/src/backend/cuda/codegen/compile.rs:43-190, singe-cuda/src/module/mod.rs:2117-2132).
- * The HIP runtime itself is resolved with dlopen on first use, as the reference's sys crates do
- * (singe-loader/src/lib.rs:298-322), so the library has no link-time dependency on ROCm.
+ * The HIP runtime's entry points are resolved with dlopen on first use, as the reference's sys crates do
+ * (singe-loader/src/lib.rs:298-322), from the copy of libamdhip64 the process already holds: the library links that
+ * runtime for the one hipcc-built unit that carries its fixed device scratch, and refuses to run on two copies.
  *
  * Return value of every int32_t function: 0 = success; a positive SingeHipStatus = a validation
  * failure found before launch (mirrors singe-kernel/src/error.rs:12-186); a negative value =
@@ -62,14 +63,27 @@ SINGE_HIP_API const char* singe_hip_status_string(int32_t status);
 
 /* ---- code object management -------------------------------------------------------------------
  * Replaces Context::load_module / Module::function (singe-cuda/src/context.rs:363-385,
- * singe-cuda/src/module/mod.rs:387-410).  An image is a gfx950 code object or a clang offload bundle
- * holding one.  Loading is per process; the module is instantiated lazily on each device that
- * launches.  Without an explicit load the library looks for the parts, singe_attention_gfx950.<part>.hsaco,
- * next to itself and loads a part when a kernel of it is first launched; an image handed to singe_hip_load holds
- * every kernel.  The image bytes are copied.  Launches read their kernel handle without a lock once it has been
- * resolved on their device (the first launch of a kernel there, or singe_hip_prepare, takes a mutex), so load and
- * unload must not run while another thread launches. */
+ * singe-cuda/src/module/mod.rs:387-410) and the kernel cache of CudaRuntime::kernel
+ * (singe/src/backend/cuda/codegen/compile.rs:43-190).  The kernels are built as parts, one gfx950 code object per
+ * kernel source and build (singe_hip_kernel lists which kernel lives in which part).  Loading is per process; a part's
+ * module is instantiated lazily on each device that launches from it.  Without an explicit load the library looks for
+ * singe_attention_gfx950.<part>.hsaco next to itself when a kernel of the part is first launched.  An embedding
+ * caller hands the bytes over instead (they are copied):
+ *   singe_hip_load_part(part, image, bytes)   one part's code object, by the part's name;
+ *   singe_hip_load(image, bytes)              an archive of parts as the build writes it (singe_attention_gfx950.parts:
+ *                                             16 bytes "SINGE_HIP_PARTS\0", u32 version = 1, u32 entries, then per
+ *                                             entry char part[48], u64 offset, u64 bytes; little-endian, offsets from
+ *                                             the archive's first byte), which replaces the parts it lists; any other
+ *                                             image is taken as ONE code object (or clang offload bundle) that holds
+ *                                             every kernel;
+ *   singe_hip_load_file(path)                 the same from a file.
+ * Parts no load has supplied are still looked for next to the library.  A malformed archive changes nothing and returns
+ * SINGE_HIP_INVALID_LENGTH / SINGE_HIP_INVALID_ARGUMENT / SINGE_HIP_LENGTH_TOO_SHORT.  Launches read their kernel handle
+ * without a lock once it has been resolved on their device (the first launch of a kernel there, or singe_hip_prepare,
+ * takes a mutex); a load or unload drops the handles and modules it replaces, so it must not run while another thread
+ * launches, as with cuModuleUnload. */
 SINGE_HIP_API int32_t singe_hip_load(const void* image, size_t bytes);
+SINGE_HIP_API int32_t singe_hip_load_part(const char* part, const void* image, size_t bytes);
 SINGE_HIP_API int32_t singe_hip_load_file(const char* path);
 SINGE_HIP_API void singe_hip_unload(void);
 /* Resolves every kernel of the image on the current device; returns the number found through *count. */
@@ -202,6 +216,25 @@ SINGE_HIP_API int32_t singe_hip_relaxed_numerics(void);
  * (singe-kernel/src/cuda/attention/mod.rs:2364-2380).  Changes what ..._workspace_bytes returns. */
 SINGE_HIP_API void singe_hip_set_decode_workers(uint32_t workers);
 SINGE_HIP_API uint32_t singe_hip_decode_workers(const SingePagedKvDecodeAttentionConfig* config);
+
+/* The same choices for the calling thread alone.  The setters above and below (relaxed numerics, decode workers,
+ * paged / MLA key splits, the installed SingeAttentionParameters) are process-wide defaults; the reference keeps its
+ * numerical policy per thread (thread_local! NUMERICAL_POLICY, singe/src/graph/numerics/mod.rs:44-49) and carries
+ * tuning choices in the call (TuningChoice::Explicit, singe-kernel/src/cuda/attention/mod.rs:2364-2380).  A thread
+ * that installs options reads them in every size query (*_workspace_bytes, *_scratch_bytes, singe_hip_decode_workers)
+ * and every launch it makes afterwards, whatever other threads set meanwhile, so the scratch a thread sized is the
+ * scratch its launch expects.  A field at its "follow" value takes the process-wide setting.  NULL clears the thread's
+ * options.  Returns SINGE_HIP_INVALID_ARGUMENT for relaxed_numerics outside -1 .. 1 or more than 64 splits. */
+typedef struct SingeHipThreadOptions {
+    int32_t relaxed_numerics;             /* -1 = follow; 0 = full; 1 = relaxed */
+    uint32_t decode_workers;              /* 0 = follow; otherwise as singe_hip_set_decode_workers */
+    uint32_t paged_attention_splits;      /* 0 = follow; 1 .. 64 as singe_hip_set_paged_attention_splits */
+    uint32_t paged_mla_attention_splits;  /* 0 = follow; 1 .. 64 as singe_hip_set_paged_mla_attention_splits */
+    uint8_t has_split_below_blocks;       /* 0 = follow the installed SingeAttentionParameters */
+    uint64_t split_below_blocks;          /* AttentionParameters::split_below_blocks for this thread's calls */
+} SingeHipThreadOptions;
+SINGE_HIP_API int32_t singe_hip_set_thread_options(const SingeHipThreadOptions* options);
+SINGE_HIP_API void singe_hip_thread_options(SingeHipThreadOptions* options);
 
 /* ---- singe-kernel surface: paged prefill ----------------------------------------------------------
  * Mirrors PagedKvPrefillAttentionConfig (singe-kernel/src/cuda/attention/mod.rs:92-108). */

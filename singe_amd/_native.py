@@ -116,6 +116,12 @@ class AttentionParametersC(ctypes.Structure):
                 ("has_min_blocks", ctypes.c_uint8), ("min_blocks", ctypes.c_uint32)]
 
 
+class ThreadOptionsC(ctypes.Structure):
+    _fields_ = [("relaxed_numerics", ctypes.c_int32), ("decode_workers", ctypes.c_uint32),
+                ("paged_attention_splits", ctypes.c_uint32), ("paged_mla_attention_splits", ctypes.c_uint32),
+                ("has_split_below_blocks", ctypes.c_uint8), ("split_below_blocks", ctypes.c_uint64)]
+
+
 class QueryRotationC(ctypes.Structure):
     _fields_ = [("table_type", ctypes.c_int32), ("has_norm", ctypes.c_uint8), ("eps", ctypes.c_float)]
 
@@ -141,12 +147,19 @@ _lib = None
 
 def lib() -> ctypes.CDLL:
     global _lib
-    if _lib is not None:
-        return _lib
-    if not os.path.exists(LIBRARY_PATH):
+    if _lib is None:
+        _lib = bind(LIBRARY_PATH)
+    return _lib
+
+
+def bind(path: str) -> ctypes.CDLL:
+    """Opens the C-ABI library at `path` and declares every entry point's argument and result types.  `lib()` is this
+    for the library next to the package; a copy elsewhere (one that finds no code object beside itself and is handed
+    the kernels as bytes, say) binds the same way."""
+    if not os.path.exists(path):
         raise error.KernelNotPrepared(
-            f"{LIBRARY_PATH} is missing: build it with `python -m singe_amd.build` (there is no fallback path)")
-    handle = ctypes.CDLL(LIBRARY_PATH)
+            f"{path} is missing: build it with `python -m singe_amd.build` (there is no fallback path)")
+    handle = ctypes.CDLL(path)
     i32 = ctypes.c_int32
     handle.singe_hip_last_error.argtypes = [ctypes.POINTER(ErrorDetail)]
     handle.singe_hip_last_error.restype = None
@@ -154,6 +167,12 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_status_string.restype = ctypes.c_char_p
     handle.singe_hip_load.argtypes = [c_void, c_size]
     handle.singe_hip_load.restype = i32
+    handle.singe_hip_set_thread_options.argtypes = [ctypes.POINTER(ThreadOptionsC)]
+    handle.singe_hip_set_thread_options.restype = i32
+    handle.singe_hip_thread_options.argtypes = [ctypes.POINTER(ThreadOptionsC)]
+    handle.singe_hip_thread_options.restype = None
+    handle.singe_hip_load_part.argtypes = [ctypes.c_char_p, c_void, c_size]
+    handle.singe_hip_load_part.restype = i32
     handle.singe_hip_load_file.argtypes = [ctypes.c_char_p]
     handle.singe_hip_load_file.restype = i32
     handle.singe_hip_unload.argtypes = []
@@ -309,7 +328,6 @@ def lib() -> ctypes.CDLL:
     handle.singe_hip_rotary_cache_write.restype = i32
     handle.singe_hip_paging_indices.argtypes = [c_void] * 10 + [ctypes.POINTER(PagingIndicesProblemC)]
     handle.singe_hip_paging_indices.restype = i32
-    _lib = handle
     return handle
 
 

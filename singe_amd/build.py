@@ -1,7 +1,9 @@
 """Builds the native artefacts in-tree:
 
 * ``singe_attention_gfx950.<part>.hsaco``: the gfx950 code object, one part per kernel source (hipcc --genco), built
-  side by side, and
+  side by side,
+* ``singe_attention_gfx950.parts``: the same parts in one archive, the image ``singe_hip_load`` takes from a caller
+  that embeds the kernels instead of shipping files, and
 * ``libsinge_hip_attention.so``: the C-ABI launcher (plain g++; it resolves the HIP runtime with dlopen, and
   links it only for the one hipcc-built unit that holds the fixed device scratch).
 
@@ -148,8 +150,39 @@ def build_library() -> str:
     return LIBRARY
 
 
+ARCHIVE = os.path.join(HERE, "singe_attention_gfx950.parts")
+ARCHIVE_MAGIC = b"SINGE_HIP_PARTS\0"
+
+
+def pack_archive(parts=None) -> bytes:
+    """The parts' code objects as one image for ``singe_hip_load`` (what an embedding caller keeps with
+    ``include_bytes!``): the magic, u32 version 1, u32 entries, then per entry the part's name in 48 bytes, u64 offset
+    and u64 size, then the code objects, each at a multiple of 16 bytes.  Little-endian."""
+    import struct
+
+    names = [part for part, _, _ in PARTS if parts is None or part in parts]
+    images = [open(code_object(part), "rb").read() for part in names]
+    offset = 24 + 64 * len(names)
+    table, body = b"", b""
+    for name, image in zip(names, images):
+        offset += -offset % 16
+        table += struct.pack("<48sQQ", name.encode(), offset, len(image))
+        offset += len(image)
+    position = 24 + len(table)
+    for image in images:
+        body += b"\0" * (-(position + len(body)) % 16) + image
+    return ARCHIVE_MAGIC + struct.pack("<II", 1, len(names)) + table + body
+
+
+def write_archive() -> str:
+    with open(ARCHIVE, "wb") as handle:
+        handle.write(pack_archive())
+    return ARCHIVE
+
+
 def build(only_changed: bool = False) -> None:
     build_code_object(only_changed=only_changed)
+    write_archive()
     build_library()
 
 

@@ -10,6 +10,7 @@
 
 #include "module.h"
 #include "singe_hip_attention.h"
+#include "thread_options.h"
 #include "validate.h"
 
 using namespace singe_hip;
@@ -161,8 +162,9 @@ size_t hand_over(const std::string& key, char* buffer, size_t capacity) {
 namespace singe_hip {
 
 uint32_t attention_key_splits(uint64_t workgroups, uint64_t keys) {
+    const SingeHipThreadOptions& own = thread_options();
     const uint64_t installed = g_split_below_plus_one.load(std::memory_order_relaxed);
-    const uint64_t below = installed == 0 ? default_split_below() : installed - 1;
+    const uint64_t below = own.has_split_below_blocks ? own.split_below_blocks : installed == 0 ? default_split_below() : installed - 1;
     if (below == 0 || workgroups == 0 || workgroups >= below || keys <= kShareTiles * kKeyTile) return 1;
     uint64_t wanted = (2 * below + workgroups - 1) / workgroups;
     const uint64_t chunks = (keys + kShareTiles * kKeyTile - 1) / (kShareTiles * kKeyTile);
@@ -215,6 +217,7 @@ void singe_hip_attention_parameters(SingeAttentionParameters* parameters) {
     singe_hip_attention_parameters_default(parameters);
     const uint64_t installed = g_split_below_plus_one.load(std::memory_order_relaxed);
     if (installed != 0) parameters->split_below_blocks = static_cast<size_t>(installed - 1);
+    if (thread_options().has_split_below_blocks) parameters->split_below_blocks = static_cast<size_t>(thread_options().split_below_blocks);
     parameters->stages = static_cast<size_t>(g_stages.load(std::memory_order_relaxed));
     const uint32_t bound = g_min_blocks.load(std::memory_order_relaxed);
     parameters->has_min_blocks = bound != 0;

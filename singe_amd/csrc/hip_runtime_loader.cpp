@@ -4,6 +4,9 @@
 
 #include <mutex>
 
+// The runtime this library is linked against (for the hipcc-built unit that holds the fixed device scratch).
+extern "C" int hipGetDevice(int* device);
+
 namespace singe_hip {
 
 namespace {
@@ -48,6 +51,9 @@ void load() {
     ok &= resolve(handle, "hipEventSynchronize", g_runtime.hipEventSynchronize);
     ok &= resolve(handle, "hipEventElapsedTime", g_runtime.hipEventElapsedTime);
     ok &= resolve(handle, "hipStreamIsCapturing", g_runtime.hipStreamIsCapturing);
+    // Kernel launches go through the table above, the fixed scratch's address comes from the linked runtime: both must
+    // be the one copy, or the address would belong to another runtime's context.
+    ok &= reinterpret_cast<void*>(g_runtime.hipGetDevice) == reinterpret_cast<void*>(&::hipGetDevice);
     g_ready = ok;
 }
 

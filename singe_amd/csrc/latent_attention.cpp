@@ -1,12 +1,14 @@
 // Host side of latent (MLA) attention over paged caches: the shape rules of spec::paged_mla_attention_problem
 // (singe/src/backend/spec/neural/attention.rs:453-497) and the launch, with the kernel's arguments in the order of
 // the reference artifact's ABI (singe/src/backend/cuda/kernel_plan/source/mla.rs:219-230, 260).
+#include <atomic>
 #include <cmath>
 #include <cstdint>
 
 #include "kernel_args.h"
 #include "module.h"
 #include "singe_hip_attention.h"
+#include "thread_options.h"
 #include "validate.h"
 
 using namespace singe_hip;
@@ -25,11 +27,12 @@ bool on_matrix_cores(const SingePagedMlaAttentionProblem& p) {
 // tiles is not known on the host (it depends on the offsets on the device): every sequence has at least one, and
 // together they hold at least tokens * heads / 128.
 // 0 = chosen by problem size (singe_hip_set_paged_mla_attention_splits).
-uint32_t g_latent_splits = 0;
+std::atomic<uint32_t> g_latent_splits{0};
 
 uint32_t latent_splits(const SingePagedMlaAttentionProblem& p) {
     if (!on_matrix_cores(p) || p.tokens <= 0 || p.heads <= 0 || p.sequences <= 0) return 1;
-    if (g_latent_splits != 0) return g_latent_splits;
+    if (const uint32_t fixed = effective_count(thread_options().paged_mla_attention_splits, g_latent_splits.load(std::memory_order_relaxed)))
+        return fixed;
     const uint64_t packed = (static_cast<uint64_t>(p.tokens) * p.heads + 127) / 128;
     const uint64_t workgroups = packed > static_cast<uint64_t>(p.sequences) ? packed : static_cast<uint64_t>(p.sequences);
     const uint64_t wanted = compute_units();
@@ -160,7 +163,9 @@ extern "C" int32_t singe_hip_paged_mla_attention(void* stream, const void* laten
                                pages, last_page_lengths, output, lse, status, nullptr, 0, problem);
 }
 
-extern "C" void singe_hip_set_paged_mla_attention_splits(uint32_t splits) { g_latent_splits = splits > 64 ? 64 : splits; }
+extern "C" void singe_hip_set_paged_mla_attention_splits(uint32_t splits) {
+    g_latent_splits.store(splits > 64 ? 64 : splits, std::memory_order_relaxed);
+}
 
 extern "C" size_t singe_hip_paged_mla_attention_scratch_bytes(const SingePagedMlaAttentionProblem* problem) {
     if (problem == nullptr) return 0;

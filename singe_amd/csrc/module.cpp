@@ -11,6 +11,7 @@
 
 #include "singe_hip_attention.h"
 #include "static_scratch.h"
+#include "thread_options.h"
 
 namespace singe_hip {
 
@@ -287,8 +288,28 @@ struct DeviceModule {
 
 std::mutex g_mutex;                               // guards the images, module loading and the publishing of handles
 std::vector<unsigned char> g_images[kPartCount];  // copies of the code object's parts
-bool g_single_image = false;                      // an image handed to singe_hip_load holds every kernel (in slot 0)
+bool g_single_image = false;                      // one code object handed to singe_hip_load holds every kernel (in slot 0)
 DeviceModule g_devices[kMaxDevices];
+
+// An archive of parts, as singe_amd/build.py writes it (singe_attention_gfx950.parts): the magic, a version and an
+// entry count, then per entry the part's name and where its code object lies in the archive.  All integers little-endian.
+constexpr char kArchiveMagic[16] = {'S', 'I', 'N', 'G', 'E', '_', 'H', 'I', 'P', '_', 'P', 'A', 'R', 'T', 'S', '\0'};
+constexpr uint32_t kArchiveVersion = 1;
+struct ArchiveHeader {
+    char magic[16];
+    uint32_t version, entries;
+};
+struct ArchiveEntry {
+    char part[48];
+    uint64_t offset, bytes;
+};
+static_assert(sizeof(ArchiveHeader) == 24 && sizeof(ArchiveEntry) == 64, "the archive's layout is fixed");
+
+int part_index(const char* name, size_t limit) {
+    for (int part = 0; part < kPartCount; ++part)
+        if (std::strlen(kPartNames[part]) < limit && std::strncmp(kPartNames[part], name, limit) == 0) return part;
+    return -1;
+}
 
 std::string default_image_path(int part) {
     Dl_info info;
@@ -314,16 +335,68 @@ bool read_file(const std::string& path, std::vector<unsigned char>& bytes) {
     return ok;
 }
 
-void drop_modules_locked() {
+// Forgets the handles of one part's kernels (every kernel when part < 0) on every device and unloads the modules.
+void drop_modules_locked(int only_part = -1) {
     const HipRuntime* hip = hip_runtime();
     for (DeviceModule& device : g_devices) {
-        for (std::atomic<hipFunction_t>& function : device.functions) function.store(nullptr, std::memory_order_release);
+        for (int kernel = 0; kernel < kKernelCount; ++kernel)
+            if (only_part < 0 || kernel_part(kernel) == only_part) device.functions[kernel].store(nullptr, std::memory_order_release);
         for (int part = 0; part < kPartCount; ++part) {
+            if (only_part >= 0 && part != only_part) continue;
             if (device.loaded[part] && hip != nullptr) hip->hipModuleUnload(device.modules[part]);
             device.modules[part] = nullptr;
             device.loaded[part] = false;
         }
     }
+}
+
+// A single code object in place of the parts: everything held so far goes.
+void hold_single_image_locked(std::vector<unsigned char>& bytes) {
+    drop_modules_locked();
+    for (std::vector<unsigned char>& held : g_images) held.clear();
+    g_images[0].swap(bytes);
+    g_single_image = true;
+}
+
+// Takes the parts an archive lists; the archive is checked as a whole before anything held changes.
+int32_t hold_archive_locked(const unsigned char* image, size_t bytes) {
+    ArchiveHeader header;
+    if (bytes < sizeof(header)) return fail(SINGE_HIP_INVALID_LENGTH, "parts archive");
+    std::memcpy(&header, image, sizeof(header));
+    if (header.version != kArchiveVersion) return fail(SINGE_HIP_INVALID_ARGUMENT, "parts archive version", kArchiveVersion, header.version);
+    if (header.entries == 0 || header.entries > static_cast<uint32_t>(kPartCount) ||
+        bytes < sizeof(header) + static_cast<size_t>(header.entries) * sizeof(ArchiveEntry))
+        return fail(SINGE_HIP_INVALID_LENGTH, "parts archive entries", 1, header.entries);
+    std::vector<ArchiveEntry> entries(header.entries);
+    std::memcpy(entries.data(), image + sizeof(header), entries.size() * sizeof(ArchiveEntry));
+    int parts[kPartCount];
+    bool seen[kPartCount] = {};
+    for (uint32_t i = 0; i < header.entries; ++i) {
+        const ArchiveEntry& entry = entries[i];
+        const int part = part_index(entry.part, sizeof(entry.part));
+        if (part < 0 || seen[part]) return fail(SINGE_HIP_INVALID_ARGUMENT, "parts archive part name");
+        if (entry.bytes == 0 || entry.offset > bytes || entry.bytes > bytes - entry.offset)
+            return fail(SINGE_HIP_LENGTH_TOO_SHORT, kPartNames[part], entry.offset + entry.bytes, bytes);
+        seen[part] = true;
+        parts[i] = part;
+    }
+    if (g_single_image) {
+        drop_modules_locked();
+        g_images[0].clear();
+        g_single_image = false;
+    }
+    for (uint32_t i = 0; i < header.entries; ++i) {
+        drop_modules_locked(parts[i]);
+        g_images[parts[i]].assign(image + entries[i].offset, image + entries[i].offset + entries[i].bytes);
+    }
+    return 0;
+}
+
+int32_t hold_image_locked(std::vector<unsigned char>& bytes) {
+    if (bytes.size() >= sizeof(kArchiveMagic) && std::memcmp(bytes.data(), kArchiveMagic, sizeof(kArchiveMagic)) == 0)
+        return hold_archive_locked(bytes.data(), bytes.size());
+    hold_single_image_locked(bytes);
+    return 0;
 }
 
 }  // namespace
@@ -339,18 +412,20 @@ int32_t fail(int32_t status, const char* name, uint64_t minimum, uint64_t actual
 int32_t fail_hip(hipError_t error, const char* what) { return fail(-static_cast<int32_t>(error), what); }
 
 unsigned compute_units() {
-    static unsigned cached[kMaxDevices] = {};
+    static std::atomic<unsigned> cached[kMaxDevices] = {};
     const HipRuntime* hip = hip_runtime();
     int device = 0;
     if (hip == nullptr || hip->hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return 256;
-    if (cached[device] == 0) {
+    unsigned known = cached[device].load(std::memory_order_relaxed);
+    if (known == 0) {
         int count = 0;
         constexpr int kMultiprocessorCount = 63;  // hipDeviceAttributeMultiprocessorCount
         if (hip->hipDeviceGetAttribute(&count, kMultiprocessorCount, device) != hipSuccess || count < 1 || count > 4096)
             count = 256;
-        cached[device] = static_cast<unsigned>(count);
+        known = static_cast<unsigned>(count);
+        cached[device].store(known, std::memory_order_relaxed);  // threads that race here store the same value
     }
-    return cached[device];
+    return known;
 }
 
 int32_t kernel_function(KernelId kernel, hipFunction_t* function) {
@@ -383,9 +458,36 @@ int32_t kernel_function(KernelId kernel, hipFunction_t* function) {
 
 }  // namespace singe_hip
 
+namespace {
+thread_local SingeHipThreadOptions t_options = {-1, 0, 0, 0, 0, 0};
+}  // namespace
+
+namespace singe_hip {
+const SingeHipThreadOptions& thread_options() { return t_options; }
+}  // namespace singe_hip
+
 using namespace singe_hip;
 
 extern "C" {
+
+int32_t singe_hip_set_thread_options(const SingeHipThreadOptions* options) {
+    if (options == nullptr) {
+        t_options = SingeHipThreadOptions{-1, 0, 0, 0, 0, 0};
+        return 0;
+    }
+    if (options->relaxed_numerics < -1 || options->relaxed_numerics > 1) return fail(SINGE_HIP_INVALID_ARGUMENT, "relaxed_numerics");
+    if (options->paged_attention_splits > 64) return fail(SINGE_HIP_INVALID_ARGUMENT, "paged_attention_splits", 64, options->paged_attention_splits);
+    if (options->paged_mla_attention_splits > 64)
+        return fail(SINGE_HIP_INVALID_ARGUMENT, "paged_mla_attention_splits", 64, options->paged_mla_attention_splits);
+    t_options = *options;
+    t_options.has_split_below_blocks = options->has_split_below_blocks != 0;
+    return 0;
+}
+
+void singe_hip_thread_options(SingeHipThreadOptions* options) {
+    if (options != nullptr) *options = t_options;
+}
+
 
 void singe_hip_last_error(SingeHipErrorDetail* detail) {
     if (detail != nullptr) *detail = t_error;
@@ -422,11 +524,25 @@ const char* singe_hip_status_string(int32_t status) {
 int32_t singe_hip_load(const void* image, size_t bytes) {
     if (image == nullptr) return fail(SINGE_HIP_NULL_POINTER, "image");
     if (bytes == 0) return fail(SINGE_HIP_INVALID_LENGTH, "image");
+    std::vector<unsigned char> copy(static_cast<const unsigned char*>(image), static_cast<const unsigned char*>(image) + bytes);
     std::lock_guard<std::mutex> lock(g_mutex);
-    drop_modules_locked();
-    for (std::vector<unsigned char>& held : g_images) held.clear();
-    g_images[0].assign(static_cast<const unsigned char*>(image), static_cast<const unsigned char*>(image) + bytes);
-    g_single_image = true;
+    return hold_image_locked(copy);
+}
+
+int32_t singe_hip_load_part(const char* part, const void* image, size_t bytes) {
+    if (part == nullptr) return fail(SINGE_HIP_NULL_POINTER, "part");
+    if (image == nullptr) return fail(SINGE_HIP_NULL_POINTER, "image");
+    if (bytes == 0) return fail(SINGE_HIP_INVALID_LENGTH, "image");
+    const int index = part_index(part, std::strlen(part) + 1);
+    if (index < 0) return fail(SINGE_HIP_INVALID_ARGUMENT, "part name");
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (g_single_image) {  // back from one code object to parts: the other parts are looked for next to the library
+        drop_modules_locked();
+        g_images[0].clear();
+        g_single_image = false;
+    }
+    drop_modules_locked(index);
+    g_images[index].assign(static_cast<const unsigned char*>(image), static_cast<const unsigned char*>(image) + bytes);
     return 0;
 }
 
@@ -435,11 +551,7 @@ int32_t singe_hip_load_file(const char* path) {
     std::vector<unsigned char> bytes;
     if (!read_file(path, bytes)) return fail(SINGE_HIP_KERNEL_NOT_PREPARED, "code object file");
     std::lock_guard<std::mutex> lock(g_mutex);
-    drop_modules_locked();
-    for (std::vector<unsigned char>& held : g_images) held.clear();
-    g_images[0].swap(bytes);
-    g_single_image = true;
-    return 0;
+    return hold_image_locked(bytes);
 }
 
 void singe_hip_unload(void) {

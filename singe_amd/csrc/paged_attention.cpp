@@ -2,11 +2,13 @@
 // (singe/src/backend/spec/neural/attention.rs:337-367, 408-438) and the launch, with the kernel's
 // arguments in the order of the reference artifact's ABI
 // (singe/src/backend/cuda/kernel_plan/source/paged_attention.rs:687-715).
+#include <atomic>
 #include <cmath>
 
 #include "kernel_args.h"
 #include "module.h"
 #include "singe_hip_attention.h"
+#include "thread_options.h"
 #include "validate.h"
 
 using namespace singe_hip;
@@ -66,13 +68,18 @@ RowTileGrid grid_of(uint64_t tokens, uint64_t sequences, uint64_t groups, uint64
 }
 
 // 0 = chosen by problem size (singe_hip_set_paged_attention_splits).
-uint32_t g_paged_attention_splits = 0;
+std::atomic<uint32_t> g_paged_attention_splits{0};
+
+// The count in force on this thread: its own (SingeHipThreadOptions) over the process-wide one.
+uint32_t fixed_paged_attention_splits() {
+    return effective_count(thread_options().paged_attention_splits, g_paged_attention_splits.load(std::memory_order_relaxed));
+}
 
 // Key splits for a problem: enough workgroups to fill the compute units four times over, when the query rows
 // alone do not (decoding, short chunks); one (no split) for other element types and head dimensions.
 uint32_t paged_attention_splits(const SingePagedAttentionProblem& p) {
     if (!has_matrix_core_build(p.head_dim) || p.tokens <= 0 || p.sequences <= 0 || p.kv_heads <= 0 || p.heads <= 0) return 1;
-    if (g_paged_attention_splits != 0) return g_paged_attention_splits;
+    if (const uint32_t fixed = fixed_paged_attention_splits()) return fixed;
     const uint64_t groups = static_cast<uint64_t>(p.heads / p.kv_heads);
     // Workgroups of the unsplit grid that can have work: the list of row tiles, or one per sequence, for every kv head.
     const RowTileGrid tiling = grid_of(static_cast<uint64_t>(p.tokens), static_cast<uint64_t>(p.sequences), groups);
@@ -92,7 +99,7 @@ uint32_t paged_attention_splits(const SingePagedAttentionProblem& p) {
 constexpr size_t kDecodeRowsMost = 8000;
 
 bool decode_rows_config(const SingePagedAttentionProblem& p, SingePagedKvDecodeAttentionConfig* config) {
-    if (g_paged_attention_splits != 0) return false;  // a fixed number of shares asks for the row-tile kernel
+    if (fixed_paged_attention_splits() != 0) return false;  // a fixed number of shares asks for the row-tile kernel
     if ((p.head_dim != 128 && p.head_dim != 64) || p.has_softcap) return false;
     // Under a short window a token reads few keys, and one workgroup a (sequence, kv head) of the row-tile kernel, which
     // skips the tiles before the window, is done before the route's two extra launches would be (measured: 32 sequences,
@@ -307,7 +314,9 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
 
 }  // namespace
 
-extern "C" void singe_hip_set_paged_attention_splits(uint32_t splits) { g_paged_attention_splits = splits > 64 ? 64 : splits; }
+extern "C" void singe_hip_set_paged_attention_splits(uint32_t splits) {
+    g_paged_attention_splits.store(splits > 64 ? 64 : splits, std::memory_order_relaxed);
+}
 
 extern "C" size_t singe_hip_paged_attention_scratch_bytes(const SingePagedAttentionProblem* problem) {
     if (problem == nullptr) return 0;

@@ -8,6 +8,7 @@
 #include "module.h"
 #include "singe_hip_attention.h"
 #include "static_scratch.h"
+#include "thread_options.h"
 #include "validate.h"
 
 using namespace singe_hip;
@@ -54,7 +55,7 @@ Plan make_plan(const SingePagedKvDecodeAttentionConfig& c, size_t span = 8) {
     p.work_per_wg = p.work < kWavesPerWorkgroup ? p.work : kWavesPerWorkgroup;
     p.workers_per_wg = kWavesPerWorkgroup / p.work_per_wg;
     p.grid_y = (p.work + p.work_per_wg - 1) / p.work_per_wg;
-    uint32_t forced = g_forced_workers.load(std::memory_order_relaxed);
+    const uint32_t forced = effective_count(thread_options().decode_workers, g_forced_workers.load(std::memory_order_relaxed));
     if (forced != 0) {
         p.grid_x = (forced + p.workers_per_wg - 1) / p.workers_per_wg;
     } else {
@@ -302,7 +303,7 @@ int32_t launch_paged_decode(const SingePagedKvDecodeAttentionConfig& c, const Pa
     args.scale_log2e = c.scale * 1.4426950408889634074f;
 
     const bool aligned = c.block_size % 16 == 0;
-    const KernelId kernel = fp8    ? static_cast<KernelId>(kDecodeF8Wide + (aligned ? 0 : 1) + (g_relaxed.load(std::memory_order_relaxed) ? 2 : 0))
+    const KernelId kernel = fp8    ? static_cast<KernelId>(kDecodeF8Wide + (aligned ? 0 : 1) + (effective_relaxed(g_relaxed.load(std::memory_order_relaxed)) ? 2 : 0))
                             : wide ? static_cast<KernelId>(kDecodeWide + (aligned ? 0 : 1) + (f16 ? 2 : 0))
                                    : static_cast<KernelId>((f16 ? kDecodeF16 : kDecodeBf16) + (aligned ? 0 : 2) + (plan.groups == 2 ? 1 : 0));
     if (phases & SINGE_HIP_DECODE_SPLIT)
@@ -344,6 +345,6 @@ int32_t launch_paged_decode(const SingePagedKvDecodeAttentionConfig& c, const Pa
 extern "C" {
 
 void singe_hip_set_relaxed_numerics(int32_t relaxed) { g_relaxed.store(relaxed != 0, std::memory_order_relaxed); }
-int32_t singe_hip_relaxed_numerics(void) { return g_relaxed.load(std::memory_order_relaxed) ? 1 : 0; }
+int32_t singe_hip_relaxed_numerics(void) { return effective_relaxed(g_relaxed.load(std::memory_order_relaxed)) ? 1 : 0; }
 
 }  // extern "C"

@@ -3,11 +3,7 @@
 
 #include <stddef.h>
 
-// 16 MiB per GPU: the paged decode scratch of up to 760 sequences at 32 query / 8 KV heads on 256 compute units
-// (the first benchmark decode shape needs 4.7 MB of it).
-#ifndef SINGE_HIP_STATIC_SCRATCH_BYTES
-#define SINGE_HIP_STATIC_SCRATCH_BYTES (16u << 20)
-#endif
+#include "singe_hip_attention.h"  // SINGE_HIP_STATIC_SCRATCH_BYTES: the one place the size is written
 
 namespace singe_hip {
 

@@ -14,6 +14,7 @@
 #include "static_scratch.h"
 
 static __device__ __align__(256) unsigned char scratch[SINGE_HIP_STATIC_SCRATCH_BYTES];
+static_assert(sizeof(scratch) == SINGE_HIP_STATIC_SCRATCH_BYTES, "the size callers are refused by is the array's");
 
 namespace {
 

@@ -8,6 +8,7 @@ is all the reference's DeviceInput/DeviceOutput carry); ``stream`` is a ``torch.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 import math
 from dataclasses import dataclass
@@ -57,13 +58,13 @@ class PagedKvDecodeAttentionConfig:
         """mod.rs:686-709: builds the config and validates it."""
         config = cls(batch, heads, kv_heads, head_dim, block_size, physical_blocks, block_table_batch_stride, scale)
         config.validate()
-        config.reserve_workspace()
         return config
 
     def reserve_workspace(self, device: "torch.device | None" = None) -> None:
-        """Sizes this module's per-device scratch for the config now, so that a decode call without a ``workspace``
-        of its own allocates nothing (the call is then enqueue-only, legal under stream capture, as the reference
-        asks of its launch functions: singe-kernel/src/cuda/mod.rs:3-12).  Without a visible GPU it does nothing."""
+        """Sizes this module's per-device scratch for the config now, so that a later decode call without a
+        ``workspace`` of its own allocates nothing (the call is then enqueue-only, legal under stream capture, as the
+        reference asks of its launch functions: singe-kernel/src/cuda/mod.rs:3-12).  Always an explicit call: building
+        a config touches no device.  Without a visible GPU it does nothing."""
         if not torch.cuda.is_available():
             return
         device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
@@ -94,16 +95,28 @@ class PagedKvDecodeAttentionConfig:
 
 
 class _Workspaces:
-    """One scratch buffer per device, grown on demand.  The C ABI never allocates; this host layer
-    owns the scratch the way the reference's callers own split-KV scratch (mod.rs:2456-2539)."""
+    """Scratch per device for calls that bring none, grown on demand.  The C ABI never allocates; this host layer
+    owns the scratch the way the reference's callers own split-KV scratch (mod.rs:2456-2539).  A buffer that has been
+    handed out may sit in a captured graph or under work in flight on another stream, so growing never frees one:
+    outgrown buffers are kept until the process ends.  Growing is refused while the current stream is being captured
+    (the allocation would not be legal there, and the graph would keep a pointer this layer cannot track): size the
+    scratch beforehand with ``reserve_workspace``, pass ``workspace=``, or take the entry point that allocates nothing."""
 
     def __init__(self):
         self._buffers = {}
+        self._outgrown = []
 
     def get(self, device: torch.device, nbytes: int) -> torch.Tensor:
         key = device.index if device.index is not None else torch.cuda.current_device()
         buffer = self._buffers.get(key)
         if buffer is None or buffer.numel() < nbytes:
+            if torch.cuda.is_current_stream_capturing():
+                raise error.UnsupportedConfiguration(
+                    f"a call under stream capture needs {nbytes} bytes of scratch and the reserved buffer holds "
+                    f"{0 if buffer is None else buffer.numel()}: call reserve_workspace() on the config before the "
+                    "capture, pass workspace=, or use paged_kv_decode_attention_no_alloc_bf16")
+            if buffer is not None:
+                self._outgrown.append(buffer)
             buffer = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=device)
             self._buffers[key] = buffer
         return buffer
@@ -203,6 +216,25 @@ def paged_kv_decode_attention_f8e4m3kv_bf16(stream, out: torch.Tensor, query: to
 def set_relaxed_numerics(relaxed: bool) -> None:
     """NumericalPolicy precision: Full (False, default) or Relaxed (True)."""
     _native.lib().singe_hip_set_relaxed_numerics(1 if relaxed else 0)
+
+
+@contextlib.contextmanager
+def thread_options(relaxed: "bool | None" = None, decode_workers: int = 0, paged_attention_splits: int = 0,
+                   paged_mla_attention_splits: int = 0, split_below_blocks: "int | None" = None):
+    """The calling thread's own settings for the calls inside the block, like NumericalPolicy::scope
+    (singe/src/graph/numerics/mod.rs:44-49) and a TuningChoice::Explicit carried by the call: size queries and
+    launches made by this thread read them whatever other threads or the process-wide setters say; the thread's
+    previous options come back on exit.  None / 0 follow the process-wide setting."""
+    lib = _native.lib()
+    before = _native.ThreadOptionsC()
+    lib.singe_hip_thread_options(ctypes.byref(before))
+    wanted = _native.ThreadOptionsC(-1 if relaxed is None else int(bool(relaxed)), decode_workers, paged_attention_splits,
+                                    paged_mla_attention_splits, split_below_blocks is not None, split_below_blocks or 0)
+    _native.check(lib.singe_hip_set_thread_options(ctypes.byref(wanted)), "thread_options")
+    try:
+        yield
+    finally:
+        lib.singe_hip_set_thread_options(ctypes.byref(before))
 
 
 @dataclass(frozen=True)

@@ -263,3 +263,123 @@ def test_f32_block_table_ops_validate_like_the_bf16_ones():
         short[index] -= 1
         assert run(short) == 2, index
     assert run(sizes, pointer=None) == 6
+
+
+def test_parts_archive_is_checked_before_anything_changes():
+    """singe_hip_load on an archive of parts: the build's own archive is taken; a wrong version, an entry count of
+    zero, a part name the library does not know, a part listed twice and an entry that runs past the image are each
+    refused with the status the header names, without a device."""
+    import struct
+
+    from singe_amd import build
+
+    lib = _native.lib()
+    magic = build.ARCHIVE_MAGIC
+    entry = lambda name, offset, size: struct.pack("<48sQQ", name, offset, size)
+    body = b"\x7fELF" + b"\0" * 60
+    good = magic + struct.pack("<II", 1, 1) + entry(b"hbm_stream", 88, 64) + body
+    try:
+        assert lib.singe_hip_load(good, len(good)) == 0
+        cases = {
+            "version": (magic + struct.pack("<II", 2, 1) + entry(b"hbm_stream", 88, 64) + body, 9),
+            "no entries": (magic + struct.pack("<II", 1, 0), 1),
+            "entries past the image": (magic + struct.pack("<II", 1, 3) + entry(b"hbm_stream", 88, 64) + body, 1),
+            "unknown part": (magic + struct.pack("<II", 1, 1) + entry(b"not_a_part", 88, 64) + body, 9),
+            "part twice": (magic + struct.pack("<II", 1, 2) + entry(b"hbm_stream", 152, 64) + entry(b"hbm_stream", 152, 64) + body, 9),
+            "runs past the end": (magic + struct.pack("<II", 1, 1) + entry(b"hbm_stream", 88, 65) + body, 2),
+            "empty part": (magic + struct.pack("<II", 1, 1) + entry(b"hbm_stream", 88, 0) + body, 2),
+            "header only": (magic + b"\x01", 1),
+        }
+        for name, (image, status) in cases.items():
+            assert lib.singe_hip_load(image, len(image)) == status, name
+        assert lib.singe_hip_load(None, 4) == 6 and lib.singe_hip_load(good, 0) == 1
+        assert lib.singe_hip_load_part(b"hbm_stream", body, len(body)) == 0
+        assert lib.singe_hip_load_part(b"hbm_strea", body, len(body)) == 9
+        assert lib.singe_hip_load_part(b"hbm_stream_", body, len(body)) == 9
+        assert lib.singe_hip_load_part(None, body, len(body)) == 6
+    finally:
+        lib.singe_hip_unload()
+
+
+def test_build_archive_lists_every_part_at_aligned_offsets():
+    import struct
+
+    from singe_amd import build
+
+    image = build.pack_archive()
+    assert image[:16] == build.ARCHIVE_MAGIC
+    version, entries = struct.unpack_from("<II", image, 16)
+    assert version == 1 and entries == len(_native.CODE_OBJECT_PARTS)
+    for index, (part, path) in enumerate(zip(_native.CODE_OBJECT_PARTS, _native.CODE_OBJECT_PATHS)):
+        name, offset, size = struct.unpack_from("<48sQQ", image, 24 + 64 * index)
+        assert name.rstrip(b"\0").decode() == part and offset % 16 == 0
+        assert image[offset:offset + size] == open(path, "rb").read()
+
+
+def test_fixed_scratch_limit_is_where_the_documents_say():
+    """The entry point that allocates nothing refuses a config whose scratch exceeds the fixed array: at 32 query / 8 KV
+    heads (and the 256 compute units the library assumes without a device) that is 759 sequences, not one more."""
+    sized = lambda batch: A.PagedKvDecodeAttentionConfig.contiguous(batch, 32, 8, 128, 16, 16384, 256, 0.1).workspace_bytes()
+    if not (0 < sized(1) < A.STATIC_SCRATCH_BYTES):
+        pytest.skip("the library sees a device with another compute-unit count")
+    text = open(os.path.join(ROOT, "include", "singe_hip_attention.h")).read()
+    assert re.search(r"#define SINGE_HIP_STATIC_SCRATCH_BYTES \(16u << 20\)", text) and A.STATIC_SCRATCH_BYTES == 16 << 20
+    assert sized(759) <= A.STATIC_SCRATCH_BYTES < sized(760)
+    assert sized(32) < 5 << 20  # the headline decode shape uses under a third of it
+
+
+def test_two_threads_hold_different_settings():
+    """Per-thread options: each thread reads its own relaxed-numerics flag, decode workers and split threshold in the
+    size queries it makes, whatever the other thread and the process-wide setters say meanwhile."""
+    import threading
+
+    lib = _native.lib()
+    config = A.PagedKvDecodeAttentionConfig.contiguous(8, 32, 8, 128, 16, 1024, 64, 0.1)
+    c = config._c()
+    default_workers = int(lib.singe_hip_decode_workers(ctypes.byref(c)))
+    default_bytes = config.workspace_bytes()
+    barrier = threading.Barrier(2)
+    seen, failures = {}, []
+
+    def body(name, workers, relaxed, below):
+        try:
+            options = _native.ThreadOptionsC(relaxed, workers, 0, 0, 1, below)
+            assert lib.singe_hip_set_thread_options(ctypes.byref(options)) == 0
+            barrier.wait(timeout=10)
+            if name == "a":  # a process-wide change made while both threads hold their own
+                lib.singe_hip_set_decode_workers(48)
+                lib.singe_hip_set_relaxed_numerics(1 - relaxed)
+            barrier.wait(timeout=10)
+            parameters = _native.AttentionParametersC()
+            for _ in range(200):
+                lib.singe_hip_attention_parameters(ctypes.byref(parameters))
+                seen[name] = (int(lib.singe_hip_decode_workers(ctypes.byref(c))), config.workspace_bytes(),
+                              int(lib.singe_hip_relaxed_numerics()), int(parameters.split_below_blocks))
+                assert seen[name][0] == workers and seen[name][2] == relaxed and seen[name][3] == below
+            barrier.wait(timeout=10)
+            assert lib.singe_hip_set_thread_options(None) == 0
+            cleared = _native.ThreadOptionsC()
+            lib.singe_hip_thread_options(ctypes.byref(cleared))
+            assert (cleared.relaxed_numerics, cleared.decode_workers, cleared.has_split_below_blocks) == (-1, 0, 0)
+            assert int(lib.singe_hip_decode_workers(ctypes.byref(c))) == 48  # back on the process-wide value
+        except Exception as problem:  # noqa: BLE001 - reported by the test's own thread
+            failures.append((name, repr(problem)))
+            barrier.abort()
+
+    try:
+        threads = [threading.Thread(target=body, args=("a", 64, 1, 7)), threading.Thread(target=body, args=("b", 512, 0, 300))]
+        for thread in threads:
+            thread.start()
+        for thread in threads:
+            thread.join(timeout=30)
+        assert not failures, failures
+        assert seen["a"][1] < seen["b"][1]  # more key ranges, more partial rows
+        bad = _native.ThreadOptionsC(2, 0, 0, 0, 0, 0)
+        assert lib.singe_hip_set_thread_options(ctypes.byref(bad)) == 9
+        bad = _native.ThreadOptionsC(-1, 0, 65, 0, 0, 0)
+        assert lib.singe_hip_set_thread_options(ctypes.byref(bad)) == 9
+    finally:
+        lib.singe_hip_set_decode_workers(0)
+        lib.singe_hip_set_relaxed_numerics(0)
+        lib.singe_hip_set_thread_options(None)
+    assert int(lib.singe_hip_decode_workers(ctypes.byref(c))) == default_workers and config.workspace_bytes() == default_bytes

@@ -98,6 +98,59 @@ def test_decode_on_the_fixed_scratch_replays():
     assert gap.max() <= 2e-2 and gap.mean() <= 2e-3, (gap.max(), gap.mean())
 
 
+def test_a_captured_decode_survives_the_module_scratch_growing():
+    """A decode recorded without a workspace of its own holds a pointer to this layer's per-device scratch.  A bigger
+    config that makes that scratch grow afterwards must not free what the graph points at: replays after the growth
+    (and after eager calls on the new buffer) still match eager launches; and growing under capture is refused."""
+    from singe_amd import error
+
+    work, config, lens, table, out, changes, _, _ = _decode_case()
+    config.reserve_workspace()
+    run = lambda stream: A.paged_kv_decode_attention_bf16(stream, out, work.query, work.key_cache, work.value_cache, lens, table, config)
+    changes[0]()
+    run(None)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        run(torch.cuda.current_stream())
+    held = A._workspaces.get(out.device, 1)
+
+    big = synthetic.paged_decode_workload(batch=96, heads=32, kv_heads=8, physical_blocks=1024, seq_lens=[40] * 96, seed=12)
+    big_config = A.PagedKvDecodeAttentionConfig.contiguous(big.batch, big.heads, big.kv_heads, big.head_dim, big.block_size,
+                                                           big.physical_blocks, big.block_table_batch_stride, big.scale)
+    assert big_config.workspace_bytes() > held.numel()
+    big_out = torch.empty((big.batch, big.heads, big.head_dim), device="cuda", dtype=torch.bfloat16)
+    big_lens, big_table = torch.from_numpy(big.seq_lens).cuda(), torch.from_numpy(big.block_table.view(np.int32)).cuda()
+    A.paged_kv_decode_attention_bf16(None, big_out, big.query, big.key_cache, big.value_cache, big_lens, big_table, big_config)
+    torch.cuda.synchronize()
+    grown = A._workspaces.get(out.device, 1)
+    assert grown.data_ptr() != held.data_ptr() and grown.numel() >= big_config.workspace_bytes()
+    filler = [torch.full((held.numel(),), 0xA5, dtype=torch.uint8, device="cuda") for _ in range(4)]  # would land on a freed buffer
+
+    for number, change in enumerate(changes):
+        print(f"graph replay {number} after the scratch grew", flush=True)
+        change()
+        workspace = torch.empty(config.workspace_bytes(), dtype=torch.uint8, device="cuda")
+        out.fill_(float("nan"))
+        A.paged_kv_decode_attention_bf16(None, out, work.query, work.key_cache, work.value_cache, lens, table, config, workspace)
+        torch.cuda.synchronize()
+        want = out.clone()
+        out.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(_bits(want), _bits(out)), f"replay {number} differs from the eager launch"
+    del filler
+
+    huge = A.PagedKvDecodeAttentionConfig.contiguous(400, 32, 8, 128, 16, 1024, 8, 0.1)
+    assert huge.workspace_bytes() > grown.numel()
+    other = torch.cuda.CUDAGraph()
+    with pytest.raises(error.UnsupportedConfiguration):
+        with torch.cuda.graph(other, stream=side):
+            A._workspaces.get(out.device, huge.workspace_bytes())
+
+
 def test_fp8_decode_replays():
     work, config, lens, table, out, changes, _, _ = _decode_case(fp8=True)
     workspace = torch.empty(config.workspace_bytes(), dtype=torch.uint8, device="cuda")

@@ -30,10 +30,17 @@ def _both(work):
     got = torch.full(shape, float("nan"), device="cuda", dtype=torch.bfloat16)
     A.paged_kv_decode_attention_bf16(None, want, work.query, work.key_cache, work.value_cache, lens, table, config)
     torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
+    # A warm first call (the array's address is resolved and the kernels' modules are loaded on first use), then the
+    # call that is held to the device's own free-memory figure: torch's counters would not see a hipMalloc inside the
+    # library, hipMemGetInfo does.
     A.paged_kv_decode_attention_no_alloc_bf16(None, got, work.query, work.key_cache, work.value_cache, lens, table, config)
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    got.fill_(float("nan"))
+    torch.cuda.synchronize()
+    before, reserved = torch.cuda.mem_get_info()[0], torch.cuda.memory_reserved()
+    A.paged_kv_decode_attention_no_alloc_bf16(None, got, work.query, work.key_cache, work.value_cache, lens, table, config)
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == before and torch.cuda.memory_reserved() == reserved
     return want, got
 
 
