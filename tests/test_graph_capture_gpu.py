@@ -116,7 +116,12 @@ def test_a_captured_decode_survives_the_module_scratch_growing():
         run(torch.cuda.current_stream())
     held = A._workspaces.get(out.device, 1)
 
-    big = synthetic.paged_decode_workload(batch=96, heads=32, kv_heads=8, physical_blocks=1024, seq_lens=[40] * 96, seed=12)
+    # (earlier tests may have grown the module's scratch already: the bigger config is sized against what is held now)
+    sized = lambda batch: A.PagedKvDecodeAttentionConfig.contiguous(batch, 32, 8, 128, 16, 4 * batch, 3, 0.1).workspace_bytes()
+    many = 96
+    while sized(many) <= held.numel():
+        many *= 2
+    big = synthetic.paged_decode_workload(batch=many, heads=32, kv_heads=8, physical_blocks=4 * many, seq_lens=[40] * many, seed=12)
     big_config = A.PagedKvDecodeAttentionConfig.contiguous(big.batch, big.heads, big.kv_heads, big.head_dim, big.block_size,
                                                            big.physical_blocks, big.block_table_batch_stride, big.scale)
     assert big_config.workspace_bytes() > held.numel()
@@ -143,12 +148,10 @@ def test_a_captured_decode_survives_the_module_scratch_growing():
         assert torch.equal(_bits(want), _bits(out)), f"replay {number} differs from the eager launch"
     del filler
 
-    huge = A.PagedKvDecodeAttentionConfig.contiguous(400, 32, 8, 128, 16, 1024, 8, 0.1)
-    assert huge.workspace_bytes() > grown.numel()
     other = torch.cuda.CUDAGraph()
     with pytest.raises(error.UnsupportedConfiguration):
         with torch.cuda.graph(other, stream=side):
-            A._workspaces.get(out.device, huge.workspace_bytes())
+            A._workspaces.get(out.device, grown.numel() + 1)
 
 
 def test_fp8_decode_replays():
