@@ -504,9 +504,11 @@ SINGE_HIP_API int32_t singe_hip_paged_attention_scratch_f16(
  * (p, p + head_dim / 2): first = a cos - b sin, second = b cos + a sin, after an optional RMS norm over the head
  * dimension (x * rsqrt(mean(x^2) + eps)) times an optional weight [head_dim] of the query's type; the rotated
  * query is rounded to the query's type before the products, as the reference rounds what it stages.
- * bf16 at head dimension 128 without a softcap; other shapes return SINGE_HIP_UNSUPPORTED_WIDTH or
- * SINGE_HIP_UNSUPPORTED_CONFIGURATION and take singe_hip_rotary_cache_write followed by
- * singe_hip_paged_attention_*, as the reference plans them apart (compiled/plan/group.rs:94-98).
+ * Fused wherever the reference fuses (paged_attention.rs:512-531 with takes_tensor_cores, tensor_core.rs:18-32): bf16
+ * or f16 tensors at a head dimension that is a multiple of 16 up to 128, with or without a softcap, any window.  At odd
+ * multiples of 16 a pair's two dims sit in the two lanes of a query row and change hands with one lane swap per word.
+ * Other head dimensions return SINGE_HIP_UNSUPPORTED_WIDTH and take singe_hip_rotary_cache_write followed by
+ * singe_hip_paged_attention_*, the two-step form the reference plans for them too.
  * `lse` may be null (the reference's fused kernel keeps it in scratch). */
 typedef struct SingeQueryRotation {
     int32_t table_type;   /* SINGE_HIP_F32, SINGE_HIP_BF16 or SINGE_HIP_F16 */
@@ -515,6 +517,25 @@ typedef struct SingeQueryRotation {
 } SingeQueryRotation;
 
 SINGE_HIP_API int32_t singe_hip_rotary_paged_attention_bf16(
+    void* stream,
+    const uint16_t* query_rows,
+    const uint16_t* key_cache,
+    const uint16_t* value_cache,
+    const void* query_offsets,
+    const void* page_offsets,
+    const void* pages,
+    const void* last_page_lengths,
+    const void* cos,
+    const void* sin,
+    const uint16_t* query_weight,
+    uint16_t* output,
+    float* lse,
+    uint32_t* status,
+    const SingePagedAttentionProblem* problem,
+    const SingeQueryRotation* rotation);
+
+/* The same for f16 tensors (query, caches, weight and output are f16 bit patterns). */
+SINGE_HIP_API int32_t singe_hip_rotary_paged_attention_f16(
     void* stream,
     const uint16_t* query_rows,
     const uint16_t* key_cache,

@@ -280,6 +280,8 @@ def bind(path: str) -> ctypes.CDLL:
     handle.singe_hip_rotary_paged_attention_bf16.argtypes = [c_void] * 14 + [ctypes.POINTER(PagedAttentionProblemC),
                                                                              ctypes.POINTER(QueryRotationC)]
     handle.singe_hip_rotary_paged_attention_bf16.restype = i32
+    handle.singe_hip_rotary_paged_attention_f16.argtypes = handle.singe_hip_rotary_paged_attention_bf16.argtypes
+    handle.singe_hip_rotary_paged_attention_f16.restype = i32
     handle.singe_hip_paged_attention_scratch_bf16.argtypes = [c_void] * 12 + [ctypes.c_size_t, ctypes.POINTER(PagedAttentionProblemC)]
     handle.singe_hip_paged_attention_scratch_bf16.restype = i32
     handle.singe_hip_paged_attention_scratch_bytes.argtypes = [ctypes.POINTER(PagedAttentionProblemC)]

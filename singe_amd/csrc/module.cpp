@@ -218,6 +218,56 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_decode_combine_few_bf16", "singe_paged_decode_combine_few_f16",
     "singe_paged_decode_combine_few_bf16_d64", "singe_paged_decode_combine_few_f16_d64",
     "singe_paged_decode_rows_i32", "singe_paged_decode_rows_i64",
+    // the fused query rotation beyond bf16 without a cap: per head dimension (128, 64, 32, 96, 16, 48, 80, 112) bf16 with a
+    // cap, f16, f16 with a cap, four index / page forms each
+    "singe_rotary_paged_attention_bf16_d128_softcap_i32", "singe_rotary_paged_attention_bf16_d128_softcap_i64",
+    "singe_rotary_paged_attention_bf16_d128_softcap_i32_p16", "singe_rotary_paged_attention_bf16_d128_softcap_i64_p16",
+    "singe_rotary_paged_attention_f16_d128_i32", "singe_rotary_paged_attention_f16_d128_i64",
+    "singe_rotary_paged_attention_f16_d128_i32_p16", "singe_rotary_paged_attention_f16_d128_i64_p16",
+    "singe_rotary_paged_attention_f16_d128_softcap_i32", "singe_rotary_paged_attention_f16_d128_softcap_i64",
+    "singe_rotary_paged_attention_f16_d128_softcap_i32_p16", "singe_rotary_paged_attention_f16_d128_softcap_i64_p16",
+    "singe_rotary_paged_attention_bf16_d64_softcap_i32", "singe_rotary_paged_attention_bf16_d64_softcap_i64",
+    "singe_rotary_paged_attention_bf16_d64_softcap_i32_p16", "singe_rotary_paged_attention_bf16_d64_softcap_i64_p16",
+    "singe_rotary_paged_attention_f16_d64_i32", "singe_rotary_paged_attention_f16_d64_i64",
+    "singe_rotary_paged_attention_f16_d64_i32_p16", "singe_rotary_paged_attention_f16_d64_i64_p16",
+    "singe_rotary_paged_attention_f16_d64_softcap_i32", "singe_rotary_paged_attention_f16_d64_softcap_i64",
+    "singe_rotary_paged_attention_f16_d64_softcap_i32_p16", "singe_rotary_paged_attention_f16_d64_softcap_i64_p16",
+    "singe_rotary_paged_attention_bf16_d32_softcap_i32", "singe_rotary_paged_attention_bf16_d32_softcap_i64",
+    "singe_rotary_paged_attention_bf16_d32_softcap_i32_p16", "singe_rotary_paged_attention_bf16_d32_softcap_i64_p16",
+    "singe_rotary_paged_attention_f16_d32_i32", "singe_rotary_paged_attention_f16_d32_i64",
+    "singe_rotary_paged_attention_f16_d32_i32_p16", "singe_rotary_paged_attention_f16_d32_i64_p16",
+    "singe_rotary_paged_attention_f16_d32_softcap_i32", "singe_rotary_paged_attention_f16_d32_softcap_i64",
+    "singe_rotary_paged_attention_f16_d32_softcap_i32_p16", "singe_rotary_paged_attention_f16_d32_softcap_i64_p16",
+    "singe_rotary_paged_attention_bf16_d96_softcap_i32", "singe_rotary_paged_attention_bf16_d96_softcap_i64",
+    "singe_rotary_paged_attention_bf16_d96_softcap_i32_p16", "singe_rotary_paged_attention_bf16_d96_softcap_i64_p16",
+    "singe_rotary_paged_attention_f16_d96_i32", "singe_rotary_paged_attention_f16_d96_i64",
+    "singe_rotary_paged_attention_f16_d96_i32_p16", "singe_rotary_paged_attention_f16_d96_i64_p16",
+    "singe_rotary_paged_attention_f16_d96_softcap_i32", "singe_rotary_paged_attention_f16_d96_softcap_i64",
+    "singe_rotary_paged_attention_f16_d96_softcap_i32_p16", "singe_rotary_paged_attention_f16_d96_softcap_i64_p16",
+    "singe_rotary_paged_attention_bf16_d16_softcap_i32", "singe_rotary_paged_attention_bf16_d16_softcap_i64",
+    "singe_rotary_paged_attention_bf16_d16_softcap_i32_p16", "singe_rotary_paged_attention_bf16_d16_softcap_i64_p16",
+    "singe_rotary_paged_attention_f16_d16_i32", "singe_rotary_paged_attention_f16_d16_i64",
+    "singe_rotary_paged_attention_f16_d16_i32_p16", "singe_rotary_paged_attention_f16_d16_i64_p16",
+    "singe_rotary_paged_attention_f16_d16_softcap_i32", "singe_rotary_paged_attention_f16_d16_softcap_i64",
+    "singe_rotary_paged_attention_f16_d16_softcap_i32_p16", "singe_rotary_paged_attention_f16_d16_softcap_i64_p16",
+    "singe_rotary_paged_attention_bf16_d48_softcap_i32", "singe_rotary_paged_attention_bf16_d48_softcap_i64",
+    "singe_rotary_paged_attention_bf16_d48_softcap_i32_p16", "singe_rotary_paged_attention_bf16_d48_softcap_i64_p16",
+    "singe_rotary_paged_attention_f16_d48_i32", "singe_rotary_paged_attention_f16_d48_i64",
+    "singe_rotary_paged_attention_f16_d48_i32_p16", "singe_rotary_paged_attention_f16_d48_i64_p16",
+    "singe_rotary_paged_attention_f16_d48_softcap_i32", "singe_rotary_paged_attention_f16_d48_softcap_i64",
+    "singe_rotary_paged_attention_f16_d48_softcap_i32_p16", "singe_rotary_paged_attention_f16_d48_softcap_i64_p16",
+    "singe_rotary_paged_attention_bf16_d80_softcap_i32", "singe_rotary_paged_attention_bf16_d80_softcap_i64",
+    "singe_rotary_paged_attention_bf16_d80_softcap_i32_p16", "singe_rotary_paged_attention_bf16_d80_softcap_i64_p16",
+    "singe_rotary_paged_attention_f16_d80_i32", "singe_rotary_paged_attention_f16_d80_i64",
+    "singe_rotary_paged_attention_f16_d80_i32_p16", "singe_rotary_paged_attention_f16_d80_i64_p16",
+    "singe_rotary_paged_attention_f16_d80_softcap_i32", "singe_rotary_paged_attention_f16_d80_softcap_i64",
+    "singe_rotary_paged_attention_f16_d80_softcap_i32_p16", "singe_rotary_paged_attention_f16_d80_softcap_i64_p16",
+    "singe_rotary_paged_attention_bf16_d112_softcap_i32", "singe_rotary_paged_attention_bf16_d112_softcap_i64",
+    "singe_rotary_paged_attention_bf16_d112_softcap_i32_p16", "singe_rotary_paged_attention_bf16_d112_softcap_i64_p16",
+    "singe_rotary_paged_attention_f16_d112_i32", "singe_rotary_paged_attention_f16_d112_i64",
+    "singe_rotary_paged_attention_f16_d112_i32_p16", "singe_rotary_paged_attention_f16_d112_i64_p16",
+    "singe_rotary_paged_attention_f16_d112_softcap_i32", "singe_rotary_paged_attention_f16_d112_softcap_i64",
+    "singe_rotary_paged_attention_f16_d112_softcap_i32_p16", "singe_rotary_paged_attention_f16_d112_softcap_i64_p16",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -254,6 +304,7 @@ constexpr PartRun kPartRuns[] = {
     {6, 3},                       // rotate-and-append sixteen bytes at a time
     {0, 2}, {13, 2},              // the decode merge for rows with one or two slots, head_dim 128 and 64
     {6, 2},                       // a decode step in FlashInfer form -> rows for the decode kernels
+    {3, 12}, {15, 12}, {19, 12}, {21, 12}, {23, 12}, {25, 12}, {27, 12}, {29, 12},  // the further fused-rotation kernels
 };
 constexpr int runs_total() {
     int total = 0;

@@ -72,8 +72,13 @@ enum KernelId : int {
     kDecodeCombineFew, kDecodeCombineFewF16, kDecodeCombineFewD64, kDecodeCombineFewF16D64,
     // a decode step in FlashInfer form -> one row per token for the decode kernels
     kPagedDecodeRows, kPagedDecodeRowsI64,
-    kKernelCount
+    // the fused query rotation beyond bf16 without a cap, twelve kernels per head dimension in the order 128, 64, then
+    // the other multiples of 16 as in kOtherHeadDims: + 4 * (bf16 with a cap, f16, f16 with a cap) + (i64 indices)
+    // + 2 * (page size a power of two of at least 16 keys)
+    kRotaryPagedAttentionMore,
+    kKernelCount = kRotaryPagedAttentionMore + 8 * 12
 };
+
 
 // The head_dim 64 build of a matrix-core kernel named by its head_dim 128 id.
 inline KernelId at_head_dim_64(KernelId kernel) {
@@ -105,6 +110,13 @@ inline KernelId prefill_combine_at(long long head_dim) {
     if (head_dim == 128) return kPrefillCombine;
     if (head_dim == 64) return kPrefillCombineD64;
     return static_cast<KernelId>(other_head_dim_bank(head_dim) + 8);
+}
+
+// The fused-rotation kernel for an element type, a cap and a head dimension, before the index / page form is added.
+inline int rotary_paged_attention_base(bool f16, bool softcap, long long head_dim) {
+    if (!f16 && !softcap) return at_head_dim(kRotaryPagedAttention, head_dim);
+    const int order = head_dim == 128 ? 0 : head_dim == 64 ? 1 : 2 + (other_head_dim_bank(head_dim) - kOtherHeadDims) / (10 + (kSplitKReduce - kPagedAttentionI32));
+    return kRotaryPagedAttentionMore + 12 * order + 4 * ((f16 ? 2 : 0) + (softcap ? 1 : 0) - 1);
 }
 
 extern const char* const kKernelNames[kKernelCount];

@@ -153,12 +153,11 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
         if (table != SINGE_HIP_F32 && table != SINGE_HIP_BF16 && table != SINGE_HIP_F16)
             return fail(SINGE_HIP_INVALID_ARGUMENT, "angle table type");
         if (rotation->attributes->has_norm && !std::isfinite(rotation->attributes->eps)) return fail(SINGE_HIP_INVALID_ARGUMENT, "eps");
-        // The fused form exists for the tensor-core kernel alone and without softcap here; the reference
-        // plans the rotation and the attention apart for the rest (compiled/plan/group.rs:94-98), and so
-        // does a caller of this library (singe_hip_rotary_cache_write, then singe_hip_paged_attention_*).
-        if (data_type != SINGE_HIP_BF16 || !has_matrix_core_build(p.head_dim) || p.head_dim % 32 != 0)  // pairs are whole steps apart
+        // The fused form exists where the reference fuses (paged_attention.rs:512-531, tensor_core.rs:18-32): f16 or
+        // bf16 at a multiple of 16 up to 128, with or without a cap; for the rest the rotation and the attention are
+        // planned apart, and so does a caller of this library (singe_hip_rotary_cache_write, then singe_hip_paged_attention_*).
+        if ((data_type != SINGE_HIP_BF16 && data_type != SINGE_HIP_F16) || !has_matrix_core_build(p.head_dim))
             return fail(SINGE_HIP_UNSUPPORTED_WIDTH, "rotary_paged_attention", static_cast<uint64_t>(p.head_dim));
-        if (p.has_softcap) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "rotary paged attention with a softcap");
     }
     // paged_attention_problem: key_dim == head_dim (one field here), kv_heads > 0 dividing heads, page_size > 0.
     if (p.tokens < 0 || p.heads <= 0 || p.kv_heads <= 0 || p.heads % p.kv_heads != 0 || p.page_size <= 0 || p.head_dim <= 0 ||
@@ -304,8 +303,8 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
         args.table_type = static_cast<uint32_t>(rotation->attributes->table_type);
         args.has_query_norm = rotation->attributes->has_norm ? 1u : 0u;
         args.query_eps = rotation->attributes->eps;
-        const int rotary = kRotaryPagedAttention + (wide ? 1 : 0) + (args.page_shift >= 4 ? 2 : 0);
-        return finish(launch(built(rotary), grid, 1, 1, 256, stream, args));
+        const int rotary = rotary_paged_attention_base(f16, p.has_softcap != 0, head_dim) + (wide ? 1 : 0) + (args.page_shift >= 4 ? 2 : 0);
+        return finish(launch(static_cast<KernelId>(rotary), grid, 1, 1, 256, stream, args));
     }
     const int kernel = (f16 ? kPagedAttentionF16 : kPagedAttentionI32) + (p.has_softcap ? 2 : 0) + (wide ? 1 : 0) +
                        (args.page_shift >= 4 ? 4 : 0);
@@ -355,6 +354,18 @@ extern "C" int32_t singe_hip_rotary_paged_attention_bf16(void* stream, const uin
                                                          const SingeQueryRotation* rotation) {
     const Rotation operands = {cos, sin, query_weight, rotation};
     return paged_attention(SINGE_HIP_BF16, stream, query_rows, key_cache, value_cache, query_offsets, page_offsets, pages,
+                           last_page_lengths, output, lse, status, problem, &operands);
+}
+
+extern "C" int32_t singe_hip_rotary_paged_attention_f16(void* stream, const uint16_t* query_rows, const uint16_t* key_cache,
+                                                        const uint16_t* value_cache, const void* query_offsets,
+                                                        const void* page_offsets, const void* pages,
+                                                        const void* last_page_lengths, const void* cos, const void* sin,
+                                                        const uint16_t* query_weight, uint16_t* output, float* lse,
+                                                        uint32_t* status, const SingePagedAttentionProblem* problem,
+                                                        const SingeQueryRotation* rotation) {
+    const Rotation operands = {cos, sin, query_weight, rotation};
+    return paged_attention(SINGE_HIP_F16, stream, query_rows, key_cache, value_cache, query_offsets, page_offsets, pages,
                            last_page_lengths, output, lse, status, problem, &operands);
 }
 

@@ -267,7 +267,6 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
     // Q^T as the MFMA B operand; a negative scale moves into Q (see fmha_prefill.hip).
     const float factor = SOFTCAP ? 1.0f : fabsf(a.scale_log2e);
     const unsigned int flip = (SOFTCAP ? a.softcap_scale : a.scale_log2e) < 0.0f ? 0x80008000u : 0u;
-    static_assert(!ROTATE || std::is_same<Half, Bf16>::value, "the fused rotation reads bf16 queries");
     const Half half{};
     uint4 q[kSteps];
     {
@@ -281,11 +280,13 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
         if constexpr (ROTATE) {
             // The query arrives before its rotation (paged_attention.rs:881-977): an optional RMS norm over
             // the head dimension with an optional weight, then half-split pairs (p, p + head_dim / 2) turned by the
-            // token's angles, first = a cos - b sin, second = b cos + a sin, rounded to bf16 as the
-            // reference rounds what it stores in its tile.  A lane holds both halves of its pairs (dims
-            // 16 s + 8 hi + j and the same + head_dim / 2); the other half of the row's squares is one swap away.
+            // token's angles, first = a cos - b sin, second = b cos + a sin, rounded to the query's type as the
+            // reference rounds what it stores in its tile.  The other half of the row's squares is one swap away.
+            constexpr bool kF16 = std::is_same<Half, F16>::value;
+            constexpr uint32_t kOwnElement = kF16 ? kElementF16 : kElementBf16;
             auto wide = [](unsigned int pair, int upper) __attribute__((always_inline)) {
-                return __builtin_bit_cast(float, upper ? pair & 0xffff0000u : pair << 16);
+                if constexpr (kF16) return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<unsigned short>(upper ? pair >> 16 : pair & 0xffffu)));
+                else return __builtin_bit_cast(float, upper ? pair & 0xffff0000u : pair << 16);
             };
             float scale = 1.0f;
             if (a.has_query_norm != 0) {
@@ -300,46 +301,75 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
                 scale = rsqrtf(squares / static_cast<float>(kHeadDim) + a.query_eps);
             }
             const size_t token = static_cast<size_t>(query_start) + my_token;
-            // (Pairs are dims i and i + head_dim / 2, whole steps apart at multiples of 32; the launcher sends the other
-            // head dimensions to the two-step form.)
-            constexpr int kPairs = kHeadDim / 2, kHalfSteps = kSteps / 2;
-            const bool weighted = a.has_query_norm != 0 && a.query_weight != nullptr;
-#pragma unroll
-            for (int s = 0; s < kHalfSteps; ++s) {
-                unsigned int first_words[4] = {bits[s].x, bits[s].y, bits[s].z, bits[s].w};
-                unsigned int second_words[4] = {bits[s + kHalfSteps].x, bits[s + kHalfSteps].y, bits[s + kHalfSteps].z, bits[s + kHalfSteps].w};
-                // The lane's eight pairs of this step are neighbours: their angles and weights come as whole chunks.
-                const unsigned int first_pair = 16u * s + 8u * hi;
-                float cosines[8], sines[8], low_weights[8], high_weights[8];
-                table_values8(cosines, a.cos, a.table_type, token * kPairs + first_pair);
-                table_values8(sines, a.sin, a.table_type, token * kPairs + first_pair);
+            constexpr int kPairs = kHeadDim / 2;
+            const bool normed = a.has_query_norm != 0, weighted = normed && a.query_weight != nullptr;
+            // One chunk of eight dims turned against its partner chunk: `mine` holds dims dim0 .. dim0 + 7.
+            auto turn = [&](uint4 mine, uint4 partner, unsigned int dim0, bool mine_is_first) __attribute__((always_inline)) {
+                const unsigned int pair0 = mine_is_first ? dim0 : dim0 - kPairs, partner_dim0 = mine_is_first ? dim0 + kPairs : dim0 - kPairs;
+                float cosines[8], sines[8], own_weights[8], partner_weights[8];
+                table_values8(cosines, a.cos, a.table_type, token * kPairs + pair0);
+                table_values8(sines, a.sin, a.table_type, token * kPairs + pair0);
                 if (weighted) {
-                    table_values8(low_weights, a.query_weight, kElementBf16, first_pair);
-                    table_values8(high_weights, a.query_weight, kElementBf16, first_pair + kPairs);
+                    table_values8(own_weights, a.query_weight, kOwnElement, dim0);
+                    table_values8(partner_weights, a.query_weight, kOwnElement, partner_dim0);
                 }
+                const unsigned int own_words[4] = {mine.x, mine.y, mine.z, mine.w}, partner_words[4] = {partner.x, partner.y, partner.z, partner.w};
+                unsigned int turned[4];
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
-                    float rotated_first[2], rotated_second[2];
+                    float rotated[2];
 #pragma unroll
                     for (int upper = 0; upper < 2; ++upper) {
-                        float first = wide(first_words[w], upper), second = wide(second_words[w], upper);
-                        if (a.has_query_norm != 0) {
-                            first *= scale;
-                            second *= scale;
+                        float own = wide(own_words[w], upper), other = wide(partner_words[w], upper);
+                        if (normed) {
+                            own *= scale;
+                            other *= scale;
                             if (weighted) {
-                                first *= low_weights[2 * w + upper];
-                                second *= high_weights[2 * w + upper];
+                                own *= own_weights[2 * w + upper];
+                                other *= partner_weights[2 * w + upper];
                             }
                         }
                         const float cosine = cosines[2 * w + upper], sine = sines[2 * w + upper];
-                        rotated_first[upper] = first * cosine - second * sine;
-                        rotated_second[upper] = second * cosine + first * sine;
+                        // first = a cos - b sin, second = b cos + a sin
+                        rotated[upper] = mine_is_first ? own * cosine - other * sine : own * cosine + other * sine;
                     }
-                    first_words[w] = row_valid ? pack_pair(rotated_first[0], rotated_first[1]) : 0u;
-                    second_words[w] = row_valid ? pack_pair(rotated_second[0], rotated_second[1]) : 0u;
+                    turned[w] = row_valid ? pack_pair(half, rotated[0], rotated[1]) : 0u;
                 }
-                bits[s] = make_uint4(first_words[0], first_words[1], first_words[2], first_words[3]);
-                bits[s + kHalfSteps] = make_uint4(second_words[0], second_words[1], second_words[2], second_words[3]);
+                return make_uint4(turned[0], turned[1], turned[2], turned[3]);
+            };
+            if constexpr (kSteps % 2 == 0) {
+                // Multiples of 32: a lane holds both halves of its pairs (dims 16 s + 8 hi + j and the same + head_dim / 2),
+                // whole steps apart.
+                constexpr int kHalfSteps = kSteps / 2;
+#pragma unroll
+                for (int s = 0; s < kHalfSteps; ++s) {
+                    const uint4 first = bits[s], second = bits[s + kHalfSteps];
+                    bits[s] = turn(first, second, 16u * s + 8u * hi, true);
+                    bits[s + kHalfSteps] = turn(second, first, 16u * (s + kHalfSteps) + 8u * hi, false);
+                }
+            } else {
+                // Odd multiples of 16: half a head is a whole number of steps and a half, so the partner of a lane's
+                // chunk sits in the row's other lane (lane ^ 32), at another step: chunk (s, hi = 0) pairs with
+                // (s + (kSteps - 1) / 2, hi = 1) and chunk (s, hi = 1) with (s + (kSteps + 1) / 2, hi = 0).  Each lane
+                // hands the other what it asks for at step s, one lane swap per word.
+                constexpr int kLow = (kSteps - 1) / 2, kHigh = (kSteps + 1) / 2;
+                uint4 turned[kSteps];
+#pragma unroll
+                for (int s = 0; s < kSteps; ++s) {
+                    // what the other lane of the row needs from this one at its step s
+                    const int wanted_from_low = s <= kLow - 1 ? s + kHigh : s - kLow;  // asked by hi = 1 of the hi = 0 lane
+                    const int wanted_from_high = s <= kLow ? s + kLow : s - kHigh;     // asked by hi = 0 of the hi = 1 lane
+                    const uint4 give = hi == 0 ? bits[wanted_from_low] : bits[wanted_from_high];
+                    uint4 partner;
+                    partner.x = __shfl_xor(give.x, 32, 64);
+                    partner.y = __shfl_xor(give.y, 32, 64);
+                    partner.z = __shfl_xor(give.z, 32, 64);
+                    partner.w = __shfl_xor(give.w, 32, 64);
+                    const unsigned int dim0 = 16u * s + 8u * hi;
+                    turned[s] = turn(bits[s], partner, dim0, dim0 < static_cast<unsigned int>(kPairs));
+                }
+#pragma unroll
+                for (int s = 0; s < kSteps; ++s) bits[s] = turned[s];
             }
         }
 #pragma unroll
@@ -717,6 +747,18 @@ SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_bf16,
 SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_bf16, _i64), false, kCsrI64, false, true, Bf16)
 SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_bf16, _i32_p16), false, kCsrI32, true, true, Bf16)
 SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_bf16, _i64_p16), false, kCsrI64, true, true, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_bf16, _softcap_i32), true, kCsrI32, false, true, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_bf16, _softcap_i64), true, kCsrI64, false, true, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_bf16, _softcap_i32_p16), true, kCsrI32, true, true, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_bf16, _softcap_i64_p16), true, kCsrI64, true, true, Bf16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_f16, _i32), false, kCsrI32, false, true, F16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_f16, _i64), false, kCsrI64, false, true, F16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_f16, _i32_p16), false, kCsrI32, true, true, F16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_f16, _i64_p16), false, kCsrI64, true, true, F16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_f16, _softcap_i32), true, kCsrI32, false, true, F16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_f16, _softcap_i64), true, kCsrI64, false, true, F16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_f16, _softcap_i32_p16), true, kCsrI32, true, true, F16)
+SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_rotary_paged_attention_f16, _softcap_i64_p16), true, kCsrI64, true, true, F16)
 // f16 operands: the same kernels on v_mfma_f32_32x32x16_f16.
 SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_f16, _i32), false, kCsrI32, false, false, F16)
 SINGE_PAGED_ATTENTION_KERNEL(SINGE_PAGED_NAME(singe_paged_attention_f16, _i64), false, kCsrI64, false, false, F16)

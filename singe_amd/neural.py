@@ -372,15 +372,16 @@ def rotary_paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_c
                            check: bool = True):
     """Paged attention over a query the kernel normalises and rotates itself, the reference's fused
     rotary_paged_attention (singe/src/backend/cuda/kernel_plan/source/paged_attention.rs:533-542, 881-977):
-    ``query`` [tokens, heads, D] bf16 (D = 128 or 64) before its rotation, ``cos`` / ``sin`` [tokens, 1, D / 2] (or [tokens, D / 2]) of
-    f32, bf16 or f16, the same pairs and norm as ``rotary_cache_write``.  Returns (output, lse) like
-    ``paged_attention``.  Other types and head dimensions raise UnsupportedWidth: rotate with
+    ``query`` [tokens, heads, D] bf16 or f16 (D a multiple of 16 up to 128, the set the reference fuses:
+    paged_attention.rs:512-531) before its rotation, ``cos`` / ``sin`` [tokens, 1, D / 2] (or [tokens, D / 2]) of
+    f32, bf16 or f16, the same pairs and norm as ``rotary_cache_write``; a softcap and a window are taken.  Returns
+    (output, lse) like ``paged_attention``.  Other types and head dimensions raise UnsupportedWidth: rotate with
     ``rotary_cache_write`` and attend with ``paged_attention``, as the reference plans them apart."""
     for tensor, name in ((query, "query"), (key_cache, "key_cache"), (value_cache, "value_cache")):
         if not tensor.is_cuda or tensor.dtype != query.dtype or not tensor.is_contiguous():
             raise error.InvalidArgument(f"paged attention {name} must be a contiguous device tensor of the query's type")
-    if query.dtype != torch.bfloat16:
-        raise error.UnsupportedWidth("rotary_paged_attention takes bf16")
+    if query.dtype not in (torch.bfloat16, torch.float16):
+        raise error.UnsupportedWidth("rotary_paged_attention (bf16 or f16 tensors)", 8 * query.element_size())
     for tensor in (paging.query_offsets, paging.page_offsets, paging.pages, paging.last_page_lengths):
         if not tensor.is_cuda or not tensor.is_contiguous():
             raise error.InvalidArgument("paged attention index tensors must be contiguous device tensors")
@@ -401,7 +402,8 @@ def rotary_paged_attention(query: torch.Tensor, key_cache: torch.Tensor, value_c
     if status is None:
         status = torch.zeros(1, device=query.device, dtype=torch.int32)
     handle = int((stream or torch.cuda.current_stream()).cuda_stream)
-    code = _native.lib().singe_hip_rotary_paged_attention_bf16(
+    entry = _native.lib().singe_hip_rotary_paged_attention_bf16 if query.dtype == torch.bfloat16 else _native.lib().singe_hip_rotary_paged_attention_f16
+    code = entry(
         handle, query.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), paging.query_offsets.data_ptr(),
         paging.page_offsets.data_ptr(), paging.pages.data_ptr(), paging.last_page_lengths.data_ptr(), cos.data_ptr(), sin.data_ptr(),
         None if weight is None else weight.data_ptr(), output.data_ptr(), lse.data_ptr(), status.data_ptr(), ctypes.byref(problem),

@@ -150,11 +150,12 @@ def test_rotary_paged_attention_validation():
     good = _native.QueryRotationC(0, 1, 1e-5)
     assert call(None) == 6                                       # no rotation attributes
     assert call(_native.QueryRotationC(7, 0, 0.0)) == 9          # unknown table type
-    assert call(good, head_dim=80) == 5                          # the fused form takes head dimensions 32, 64, 96 and 128
-    assert call(good, head_dim=72) == 5
-    assert call(good, has_softcap=1, softcap=5.0) == 8
+    assert call(good, head_dim=72) == 5                          # the fused form takes the multiples of 16 up to 128
+    assert call(good, head_dim=144) == 5 and call(good, head_dim=8) == 5
+    assert call(good, has_softcap=1, softcap=float("nan")) == 9  # a cap is taken; a cap that is no number is not
     assert call(good, cos=None) == 6
     assert call(good, tokens=0) == 0
+    assert call(good, tokens=0, head_dim=80, has_softcap=1, softcap=5.0) == 0
 
 
 def test_paged_attention_scratch_query_needs_no_device():

@@ -1,7 +1,9 @@
 """Paged attention over a query the kernel normalises and rotates itself (the reference's fused
 rotary_paged_attention, kernel_plan/source/paged_attention.rs:533-542, 881-977) against the CPU oracle: the
-oracle's restatement of the rotation, rounded to bf16 as the reference rounds what it stages, then the paged
-attention oracle.  bf16 outputs within max-abs 2e-2 / mean-abs 2e-3.  The base-two LSE is within 2e-3 for all but
+oracle's restatement of the rotation, rounded to the query's type as the reference rounds what it stages, then the paged
+attention oracle.  bf16 outputs within max-abs 2e-2 / mean-abs 2e-3, f16 outputs within 5e-3 / 5e-4 (the reference's own
+f16 bound, kernel_plan/source/tests.rs:549-553), for bf16 and f16 at every multiple of 16 up to 128, with and without a
+softcap: the set the reference fuses (paged_attention.rs:512-531).  The base-two LSE is within 2e-3 for all but
 a few rows in ten thousand and within 5e-3 for those: the GPU sums the norm's squares in another order than the
 CPU (as the reference's own two rotation kernels do, paged_attention.rs:908-926 against rotary_cache.rs:92-185),
 and a last-place difference in the scale now and then moves a rotated element to the neighbouring bf16 value.
@@ -19,8 +21,8 @@ MAX_ABS, MEAN_ABS, LSE_ABS, LSE_WORST = 2e-2, 2e-3, 2e-3, 5e-3
 DIM = 128
 
 
-def bf16_round(array):
-    return torch.tensor(array, dtype=torch.float32).to(torch.bfloat16).float().numpy()
+def rounded(array, dtype=torch.bfloat16):
+    return torch.tensor(array, dtype=torch.float32).to(dtype).float().numpy()
 
 
 def oracle_rotation(query, cos, sin, norm):
@@ -34,8 +36,9 @@ def oracle_rotation(query, cos, sin, norm):
     return rotated
 
 
-def run_case(sequences, heads, kv_heads, page_size, table_dtype, index_dtype, norm, options, seed, dim=DIM):
+def run_case(sequences, heads, kv_heads, page_size, table_dtype, index_dtype, norm, options, seed, dim=DIM, dtype=torch.bfloat16):
     DIM = dim
+    max_abs, mean_abs = (MAX_ABS, MEAN_ABS) if dtype == torch.bfloat16 else (5e-3, 5e-4)
     gen = torch.Generator(device="cuda")
     gen.manual_seed(seed)
     query_offsets, page_offsets, last, table = [0], [0], [], []
@@ -48,12 +51,12 @@ def run_case(sequences, heads, kv_heads, page_size, table_dtype, index_dtype, no
     page_count = needed + 3
     table = list(np.random.default_rng(seed).permutation(page_count)[:needed])
     tokens = query_offsets[-1]
-    q = torch.randn((tokens, heads, DIM), generator=gen, device="cuda").to(torch.bfloat16)
-    kc = torch.randn((page_count, page_size, kv_heads, DIM), generator=gen, device="cuda").to(torch.bfloat16)
-    vc = torch.randn((page_count, page_size, kv_heads, DIM), generator=gen, device="cuda").to(torch.bfloat16)
+    q = torch.randn((tokens, heads, DIM), generator=gen, device="cuda").to(dtype)
+    kc = torch.randn((page_count, page_size, kv_heads, DIM), generator=gen, device="cuda").to(dtype)
+    vc = torch.randn((page_count, page_size, kv_heads, DIM), generator=gen, device="cuda").to(dtype)
     angle = torch.rand((tokens, 1, DIM // 2), generator=gen, device="cuda") * 6.28
     cos, sin = torch.cos(angle).to(table_dtype), torch.sin(angle).to(table_dtype)
-    weight = torch.randn(DIM, generator=gen, device="cuda").to(torch.bfloat16) if norm == "weighted" else None
+    weight = torch.randn(DIM, generator=gen, device="cuda").to(dtype) if norm == "weighted" else None
     query_norm = None if norm is None else neural.RotationNorm(1e-5, weight)
     index = lambda values: torch.tensor(values, dtype=index_dtype, device="cuda")
     paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
@@ -63,22 +66,23 @@ def run_case(sequences, heads, kv_heads, page_size, table_dtype, index_dtype, no
 
     host = lambda tensor: tensor.float().cpu().numpy()
     oracle_norm = None if norm is None else (1e-5, None if weight is None else host(weight))
-    rotated = bf16_round(oracle_rotation(host(q), host(cos).reshape(tokens, -1), host(sin).reshape(tokens, -1), oracle_norm))
+    rotated = rounded(oracle_rotation(host(q), host(cos).reshape(tokens, -1), host(sin).reshape(tokens, -1), oracle_norm), dtype)
     status, want, want_lse = oracle.paged_attention_f32(rotated, host(kc), host(vc), query_offsets, page_offsets, table, last,
-                                                        scale=options.scale, causal=options.causal, window=options.window, threads=8)
+                                                        scale=options.scale, causal=options.causal, window=options.window,
+                                                        softcap=options.softcap, threads=8)
     assert status == 0
     got, got_lse = host(out), lse.cpu().numpy()
     assert np.isfinite(got).all()
     gap = np.abs(got - want)
-    assert gap.max() <= MAX_ABS and gap.mean() <= MEAN_ABS, (gap.max(), gap.mean())
+    assert gap.max() <= max_abs and gap.mean() <= mean_abs, (gap.max(), gap.mean())
     empty = np.isneginf(want_lse)
     assert np.array_equal(np.isneginf(got_lse), empty)
     lse_gap = np.abs(got_lse[~empty] - want_lse[~empty])
     assert lse_gap.max(initial=0.0) <= LSE_WORST and (lse_gap > LSE_ABS).mean() <= 1e-3, (lse_gap.max(), (lse_gap > LSE_ABS).mean())
 
     # The library's own two-step form: rotate (and round) the query with the append kernel, then attend.
-    scratch_k = torch.zeros((tokens, kv_heads, DIM), device="cuda", dtype=torch.bfloat16)
-    spare_kc, spare_vc = torch.zeros((1, max(tokens, 1), kv_heads, DIM), device="cuda", dtype=torch.bfloat16), None
+    scratch_k = torch.zeros((tokens, kv_heads, DIM), device="cuda", dtype=dtype)
+    spare_kc, spare_vc = torch.zeros((1, max(tokens, 1), kv_heads, DIM), device="cuda", dtype=dtype), None
     spare_vc = torch.zeros_like(spare_kc)
     cells = torch.arange(tokens, device="cuda", dtype=torch.int64)
     rotated_gpu = neural.rotary_cache_write(q, scratch_k, scratch_k, cos, sin, torch.zeros_like(cells), cells, spare_kc, spare_vc,
@@ -108,22 +112,37 @@ def test_fused_rotation_options():
 @pytest.mark.parametrize("norm", [None, "weighted"])
 @pytest.mark.parametrize("heads,kv_heads,page_size,table_dtype,index_dtype", [
     (8, 2, 16, torch.float32, torch.int32), (8, 1, 7, torch.bfloat16, torch.int64)])
-@pytest.mark.parametrize("dim", [64, 32, 96])
+@pytest.mark.parametrize("dim", [64, 32, 96, 16, 48, 80, 112])
 def test_fused_rotation_at_other_head_dims(heads, kv_heads, page_size, table_dtype, index_dtype, norm, dim):
     run_case(SEQUENCES, heads, kv_heads, page_size, table_dtype, index_dtype, norm, neural.AttentionOptions(causal=True),
              seed=heads + page_size, dim=dim)
 
 
+@pytest.mark.parametrize("softcap", [None, 6.0])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dim", [16, 32, 48, 64, 80, 96, 112, 128])
+def test_fused_rotation_over_everything_the_reference_fuses(dim, dtype, softcap):
+    """{bf16, f16} x {16 ... 128} x {cap, no cap} (paged_attention.rs:512-531), norm with a weight, i64 paging on 16-key
+    pages and i32 paging on 7-key pages."""
+    if dtype == torch.bfloat16 and softcap is None and dim != 128:
+        pytest.skip("covered by test_fused_rotation_at_other_head_dims")
+    options = neural.AttentionOptions(causal=True, softcap=softcap)
+    run_case(SEQUENCES, 8, 2, 16, torch.float32, torch.int64, "weighted", options, seed=dim, dim=dim, dtype=dtype)
+    run_case(SEQUENCES, 6, 3, 7, torch.float16, torch.int32, "plain", options, seed=dim + 1, dim=dim, dtype=dtype)
+
+
+def test_fused_rotation_with_a_cap_and_a_window():
+    options = neural.AttentionOptions(causal=True, window=40, softcap=-4.0, scale=0.07)
+    run_case(SEQUENCES, 8, 2, 16, torch.float32, torch.int32, "weighted", options, seed=9, dim=80, dtype=torch.float16)
+    run_case(SEQUENCES, 8, 2, 32, torch.bfloat16, torch.int64, None, options, seed=10, dim=128)
+
+
 def test_fused_rotation_refuses_what_it_does_not_take():
-    q = torch.zeros((2, 2, 80), device="cuda", dtype=torch.bfloat16)
-    cache = torch.zeros((2, 4, 2, 80), device="cuda", dtype=torch.bfloat16)
     index = lambda values: torch.tensor(values, dtype=torch.int32, device="cuda")
     paging = neural.Paging(index([0, 2]), index([0, 1]), index([0]), index([2]))
-    angles = torch.zeros((2, 1, 40), device="cuda")
-    with pytest.raises(error.UnsupportedWidth):
-        neural.rotary_paged_attention(q, cache, cache, paging, angles, angles)
-    q128 = torch.zeros((2, 2, 128), device="cuda", dtype=torch.bfloat16)
-    cache128 = torch.zeros((2, 4, 2, 128), device="cuda", dtype=torch.bfloat16)
-    angles128 = torch.zeros((2, 1, 64), device="cuda")
-    with pytest.raises(error.Error):
-        neural.rotary_paged_attention(q128, cache128, cache128, paging, angles128, angles128, neural.AttentionOptions(softcap=5.0))
+    for dim, dtype in ((72, torch.bfloat16), (256, torch.float16), (128, torch.float32)):
+        q = torch.zeros((2, 2, dim), device="cuda", dtype=dtype)
+        cache = torch.zeros((2, 4, 2, dim), device="cuda", dtype=dtype)
+        angles = torch.zeros((2, 1, dim // 2), device="cuda")
+        with pytest.raises(error.UnsupportedWidth):
+            neural.rotary_paged_attention(q, cache, cache, paging, angles, angles)
