@@ -1070,6 +1070,174 @@ SINGE_HIP_API void singe_hip_synthetic_integers(uint64_t seed, uint64_t first_in
                                                 size_t count);
 SINGE_HIP_API void singe_hip_synthetic_permutation(uint64_t seed, int64_t* out, size_t count);
 
+/* ---- singe-kernel surface: the rest of the dense attention family ---------------------------------------
+ * The launchers of singe-kernel/src/cuda/attention/fmha.rs:193-1036 and paged.rs:36-116, 427-576 that the entry points
+ * above do not cover.  Every one checks its config and lengths in the order of the reference's `validate_lengths` and
+ * then runs on a kernel of this library: the matrix-core prefill kernels where the call is one of their shapes (bf16 /
+ * f16, a head dimension that is a multiple of 16 up to 128, strides in multiples of eight elements, 16-byte aligned
+ * buffers), otherwise the one-wave-per-row kernel that reads every operand through element strides, in f32 arithmetic
+ * whatever the storage type, head dimensions up to 256 (SINGE_HIP_UNSUPPORTED_WIDTH beyond). */
+
+/* softcapped_window_attention_f16 / _bf16 (fmha.rs:295-393; CPU form cpu/attention.rs:1835-1925): the 16-bit forms
+ * of singe_hip_softcapped_window_attention_f32.  A soft cap must be finite and positive (mod.rs:3418-3430). */
+SINGE_HIP_API int32_t singe_hip_softcapped_window_attention_bf16(
+    void* stream, uint16_t* out, size_t out_len, const uint16_t* query, size_t query_len, const uint16_t* key, size_t key_len,
+    const uint16_t* value, size_t value_len, const SingeSoftcappedWindowAttentionConfig* config);
+SINGE_HIP_API int32_t singe_hip_softcapped_window_attention_f16(
+    void* stream, uint16_t* out, size_t out_len, const uint16_t* query, size_t query_len, const uint16_t* key, size_t key_len,
+    const uint16_t* value, size_t value_len, const SingeSoftcappedWindowAttentionConfig* config);
+
+/* Mirrors AttentionSinkPrefillConfig (mod.rs:299-304).  Query q sits at position start_q + q; under the causal mask
+ * later keys are hidden; window w > 0 hides keys before position - (w - 1); every row's softmax also holds its head's
+ * sink logit, which weighs no value (CPU form cpu/attention.rs:2073-2155). */
+typedef struct SingeAttentionSinkPrefillConfig {
+    SingeFmhaPrefillConfig attention;
+    size_t start_q;
+    size_t window;
+} SingeAttentionSinkPrefillConfig;
+
+/* attention_sink_prefill_f32 / _f16 / _bf16 (fmha.rs:193-243, 796-898).  sinks [heads] in the tensors' type. */
+SINGE_HIP_API int32_t singe_hip_attention_sink_prefill_f32(
+    void* stream, float* out, size_t out_len, const float* query, size_t query_len, const float* key, size_t key_len,
+    const float* value, size_t value_len, const float* sinks, size_t sinks_len, const SingeAttentionSinkPrefillConfig* config);
+SINGE_HIP_API int32_t singe_hip_attention_sink_prefill_bf16(
+    void* stream, uint16_t* out, size_t out_len, const uint16_t* query, size_t query_len, const uint16_t* key, size_t key_len,
+    const uint16_t* value, size_t value_len, const uint16_t* sinks, size_t sinks_len, const SingeAttentionSinkPrefillConfig* config);
+SINGE_HIP_API int32_t singe_hip_attention_sink_prefill_f16(
+    void* stream, uint16_t* out, size_t out_len, const uint16_t* query, size_t query_len, const uint16_t* key, size_t key_len,
+    const uint16_t* value, size_t value_len, const uint16_t* sinks, size_t sinks_len, const SingeAttentionSinkPrefillConfig* config);
+
+/* fmha_decode_lse_f32 / _f16 / _bf16 (fmha.rs:395-438, 900-1036): one query per batch item over key_len keys through
+ * the strides of SingeFmhaDecodeConfig; lse [batch, heads] is the natural log-sum-exp of each row's scaled scores
+ * (FmhaDecodeConfig::validate_lengths, mod.rs:2262-2308). */
+SINGE_HIP_API int32_t singe_hip_fmha_decode_lse_f32(
+    void* stream, float* out, size_t out_len, float* lse, size_t lse_len, const float* query, size_t query_len, const float* key,
+    size_t key_len, const float* value, size_t value_len, const SingeFmhaDecodeConfig* config);
+SINGE_HIP_API int32_t singe_hip_fmha_decode_lse_bf16(
+    void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, const uint16_t* query, size_t query_len,
+    const uint16_t* key, size_t key_len, const uint16_t* value, size_t value_len, const SingeFmhaDecodeConfig* config);
+SINGE_HIP_API int32_t singe_hip_fmha_decode_lse_f16(
+    void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, const uint16_t* query, size_t query_len,
+    const uint16_t* key, size_t key_len, const uint16_t* value, size_t value_len, const SingeFmhaDecodeConfig* config);
+
+/* Mirrors SoftcappedWindowDecodeConfig (mod.rs:307-311); soft_cap: Option<f32> as (has_soft_cap, soft_cap).  The query
+ * sits at position key_len - 1; window_size w > 0 hides keys with key + w < that position
+ * (CPU form cpu/attention.rs:1927-1998). */
+typedef struct SingeSoftcappedWindowDecodeConfig {
+    SingeFmhaDecodeConfig decode;
+    size_t window_size;
+    uint8_t has_soft_cap;
+    float soft_cap;
+} SingeSoftcappedWindowDecodeConfig;
+
+/* softcapped_window_decode_lse_f32 / _f16 / _bf16 (fmha.rs:440-582). */
+SINGE_HIP_API int32_t singe_hip_softcapped_window_decode_lse_f32(
+    void* stream, float* out, size_t out_len, float* lse, size_t lse_len, const float* query, size_t query_len, const float* key,
+    size_t key_len, const float* value, size_t value_len, const SingeSoftcappedWindowDecodeConfig* config);
+SINGE_HIP_API int32_t singe_hip_softcapped_window_decode_lse_bf16(
+    void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, const uint16_t* query, size_t query_len,
+    const uint16_t* key, size_t key_len, const uint16_t* value, size_t value_len, const SingeSoftcappedWindowDecodeConfig* config);
+SINGE_HIP_API int32_t singe_hip_softcapped_window_decode_lse_f16(
+    void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, const uint16_t* query, size_t query_len,
+    const uint16_t* key, size_t key_len, const uint16_t* value, size_t value_len, const SingeSoftcappedWindowDecodeConfig* config);
+
+/* Mirrors RaggedKvPrefillAttentionConfig (mod.rs:110-123): query [total_query_tokens, heads, dim] and key / value
+ * [total_kv_tokens, kv_heads, dim] packed by sequence; sequence b owns query tokens actual_seq_offsets[b] .. +
+ * actual_seq_lens_q[b] and keys actual_seq_offsets[b] .. + actual_seq_lens_kv[b]; top-left causal inside a sequence;
+ * lse [total_query_tokens, heads] natural log, -1e20 for a token that sees no key (CPU form
+ * cpu/attention.rs:1343-1420).  Tokens no sequence owns are left as they are; keys past total_kv_tokens are not read. */
+typedef struct SingeRaggedKvPrefillAttentionConfig {
+    size_t batch;
+    size_t total_query_tokens;
+    size_t total_kv_tokens;
+    size_t heads;
+    size_t kv_heads;
+    size_t head_dim;
+    uint8_t causal;
+    float scale;
+} SingeRaggedKvPrefillAttentionConfig;
+
+/* ragged_kv_prefill_attention_f32 / _f16 / _bf16 (paged.rs:427-576). */
+SINGE_HIP_API int32_t singe_hip_ragged_kv_prefill_attention_f32(
+    void* stream, float* out, size_t out_len, float* lse, size_t lse_len, const float* query, size_t query_len, const float* key,
+    size_t key_len, const float* value, size_t value_len, const int32_t* actual_seq_lens_q, size_t actual_seq_lens_q_len,
+    const int32_t* actual_seq_lens_kv, size_t actual_seq_lens_kv_len, const int32_t* actual_seq_offsets,
+    size_t actual_seq_offsets_len, const SingeRaggedKvPrefillAttentionConfig* config);
+SINGE_HIP_API int32_t singe_hip_ragged_kv_prefill_attention_bf16(
+    void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, const uint16_t* query, size_t query_len,
+    const uint16_t* key, size_t key_len, const uint16_t* value, size_t value_len, const int32_t* actual_seq_lens_q,
+    size_t actual_seq_lens_q_len, const int32_t* actual_seq_lens_kv, size_t actual_seq_lens_kv_len,
+    const int32_t* actual_seq_offsets, size_t actual_seq_offsets_len, const SingeRaggedKvPrefillAttentionConfig* config);
+SINGE_HIP_API int32_t singe_hip_ragged_kv_prefill_attention_f16(
+    void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, const uint16_t* query, size_t query_len,
+    const uint16_t* key, size_t key_len, const uint16_t* value, size_t value_len, const int32_t* actual_seq_lens_q,
+    size_t actual_seq_lens_q_len, const int32_t* actual_seq_lens_kv, size_t actual_seq_lens_kv_len,
+    const int32_t* actual_seq_offsets, size_t actual_seq_offsets_len, const SingeRaggedKvPrefillAttentionConfig* config);
+
+/* Mirrors SlidingWindowAttentionConfig (mod.rs:32-56): query q at position query_start + q, key k at key_start + k; a
+ * key is kept when its position is at most the query's and position + window is beyond it; the output is multiplied
+ * by output_scale; a row that sees no key is zero (CPU form cpu/attention.rs:1089-1170).  window 0 is InvalidLength
+ * (mod.rs:3037-3060). */
+typedef struct SingeSlidingWindowAttentionConfig {
+    size_t batch;
+    size_t query_len;
+    size_t key_len;
+    size_t heads;
+    size_t kv_heads;
+    size_t head_dim;
+    size_t query_start;
+    size_t key_start;
+    size_t window;
+    size_t query_batch_stride;
+    size_t key_batch_stride;
+    size_t value_batch_stride;
+    size_t output_batch_stride;
+    size_t query_sequence_stride;
+    size_t key_sequence_stride;
+    size_t value_sequence_stride;
+    size_t output_sequence_stride;
+    size_t query_head_stride;
+    size_t key_head_stride;
+    size_t value_head_stride;
+    size_t output_head_stride;
+    float scale;
+    float output_scale;
+} SingeSlidingWindowAttentionConfig;
+
+/* Mirrors PackedQkvAttentionConfig (mod.rs:59-64): query, key and value are views of one buffer from these offsets on. */
+typedef struct SingePackedQkvAttentionConfig {
+    SingeSlidingWindowAttentionConfig attention;
+    size_t query_offset;
+    size_t key_offset;
+    size_t value_offset;
+} SingePackedQkvAttentionConfig;
+
+/* Mirrors PagedKvAttentionConfig (mod.rs:67-74): key k of batch item b is slot k % block_size of block
+ * block_table[b * block_table_batch_stride + k / block_size], at block * key_cache_block_stride + slot *
+ * key_sequence_stride + kv_head * key_head_stride (the value cache alike); a block id outside the cache hides its keys
+ * (cutile/kernel/attention/local.rs:9150-9330).  The batch strides of key and value are not used. */
+typedef struct SingePagedKvAttentionConfig {
+    SingeSlidingWindowAttentionConfig attention;
+    size_t block_size;
+    size_t physical_blocks;
+    size_t block_table_batch_stride;
+    size_t key_cache_block_stride;
+    size_t value_cache_block_stride;
+} SingePagedKvAttentionConfig;
+
+/* sliding_window_attention_f32 (mod.rs:2812-2855), sliding_window_attention_packed_qkv_f32
+ * (paged.rs:36-50; an offset past the buffer is LengthMismatch there and SINGE_HIP_LENGTH_TOO_SHORT naming "qkv" here)
+ * and sliding_window_attention_paged_kv_f32 (paged.rs:56-116). */
+SINGE_HIP_API int32_t singe_hip_sliding_window_attention_f32(
+    void* stream, float* out, size_t out_len, const float* query, size_t query_len, const float* key, size_t key_len,
+    const float* value, size_t value_len, const SingeSlidingWindowAttentionConfig* config);
+SINGE_HIP_API int32_t singe_hip_sliding_window_attention_packed_qkv_f32(
+    void* stream, float* out, size_t out_len, const float* qkv, size_t qkv_len, const SingePackedQkvAttentionConfig* config);
+SINGE_HIP_API int32_t singe_hip_sliding_window_attention_paged_kv_f32(
+    void* stream, float* out, size_t out_len, const float* query, size_t query_len, const float* key_cache, size_t key_cache_len,
+    const float* value_cache, size_t value_cache_len, const uint32_t* block_table, size_t block_table_len,
+    const SingePagedKvAttentionConfig* config);
+
 #ifdef __cplusplus
 }
 #endif

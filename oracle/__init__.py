@@ -228,6 +228,66 @@ def sliding_window_attention_f32(query, key, value, *, batch, query_len, key_len
     return out
 
 
+def ragged_kv_prefill_attention_f32(query, key, value, lens_q, lens_kv, offsets, *, causal, scale):
+    """singe-kernel/src/cpu/attention.rs:1343-1420: query [T, H, D], key / value [S, G, D] packed by sequence ->
+    (out [T, H, D], lse [T, H] natural log, -1e20 where a token sees no key)."""
+    query, key, value = _f32(query), _f32(key), _f32(value)
+    tokens, heads, head_dim = query.shape
+    kv_heads = key.shape[1]
+    lens_q, lens_kv, offsets = (np.ascontiguousarray(a, dtype=np.int32) for a in (lens_q, lens_kv, offsets))
+    out = np.empty(query.shape, dtype=np.float32)
+    lse = np.empty((tokens, heads), dtype=np.float32)
+    i32 = ctypes.POINTER(ctypes.c_int32)
+    lib().oracle_ragged_kv_prefill_attention_f32(
+        _ptr(out), _ptr(lse), _ptr(query), _ptr(key), _ptr(value), lens_q.ctypes.data_as(i32), lens_kv.ctypes.data_as(i32),
+        offsets.ctypes.data_as(i32), _c_size(len(lens_q)), _c_size(tokens), _c_size(heads), _c_size(kv_heads), _c_size(head_dim),
+        _c_int(bool(causal)), _c_float(scale))
+    return out, lse
+
+
+def softcapped_window_decode_lse_f32(query, key, value, *, scale, window_size=0, soft_cap=None):
+    """singe-kernel/src/cpu/attention.rs:1927-1998: query [B, H, D], key / value [B, G, S, D] -> (out [B, H, D], lse [B, H])."""
+    query, key, value = _f32(query), _f32(key), _f32(value)
+    batch, heads, head_dim = query.shape
+    kv_heads, key_len = key.shape[1], key.shape[2]
+    out = np.empty(query.shape, dtype=np.float32)
+    lse = np.empty((batch, heads), dtype=np.float32)
+    lib().oracle_softcapped_window_decode_lse_f32(
+        _ptr(out), _ptr(lse), _ptr(query), _ptr(key), _ptr(value), _c_size(batch), _c_size(key_len), _c_size(heads), _c_size(kv_heads),
+        _c_size(head_dim), _c_float(scale), _c_size(window_size), _c_int(soft_cap is not None),
+        _c_float(soft_cap if soft_cap is not None else 0.0))
+    return out, lse
+
+
+def attention_sink_prefill_f32(query, key, value, sinks, *, start_q=0, window=0, scale, causal):
+    """singe-kernel/src/cpu/attention.rs:2073-2155: query [B, L, H, D], key / value [B, S, G, D], sinks [H] -> out [B, L, H, D]."""
+    query, key, value, sinks = _f32(query), _f32(key), _f32(value), _f32(sinks)
+    batch, query_len, heads, head_dim = query.shape
+    key_len, kv_heads = key.shape[1], key.shape[2]
+    out = np.empty(query.shape, dtype=np.float32)
+    lib().oracle_attention_sink_prefill_f32(
+        _ptr(out), _ptr(query), _ptr(key), _ptr(value), _ptr(sinks), _c_size(batch), _c_size(query_len), _c_size(key_len), _c_size(heads),
+        _c_size(kv_heads), _c_size(head_dim), _c_size(start_q), _c_size(window), _c_float(scale), _c_int(bool(causal)))
+    return out
+
+
+def sliding_window_attention_paged_kv_f32(query, key_cache, value_cache, block_table, *, key_len, query_start, key_start, window,
+                                          scale, output_scale=1.0):
+    """The reference's sliding_window_attention_paged_kv_f32 kernel (cutile/kernel/attention/local.rs:9150-9330):
+    query [B, L, H, D], caches [P, block, G, D], block_table [B, stride] u32 -> out [B, L, H, D]."""
+    query, key_cache, value_cache = _f32(query), _f32(key_cache), _f32(value_cache)
+    batch, query_len, heads, head_dim = query.shape
+    physical_blocks, block_size, kv_heads, _ = key_cache.shape
+    table = np.ascontiguousarray(block_table, dtype=np.uint32)
+    out = np.empty(query.shape, dtype=np.float32)
+    lib().oracle_sliding_window_attention_paged_kv_f32(
+        _ptr(out), _ptr(query), _ptr(key_cache), _ptr(value_cache), table.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)), _c_size(batch),
+        _c_size(query_len), _c_size(key_len), _c_size(heads), _c_size(kv_heads), _c_size(head_dim), _c_size(query_start),
+        _c_size(key_start), _c_size(window), _c_size(block_size), _c_size(physical_blocks), _c_size(table.shape[1]), _c_float(scale),
+        _c_float(output_scale))
+    return out
+
+
 def splitk_reduce_f32(attn, lse, *, batch, heads, splits, head_dim):
     """singe-kernel/src/cpu/attention.rs:2157-2193."""
     attn, lse = _f32(attn), _f32(lse)

@@ -498,6 +498,180 @@ ORACLE_API void oracle_sliding_window_attention_f32(
     free(scores);
 }
 
+/* singe-kernel/src/cpu/attention.rs:1343-1420  ragged_kv_prefill_attention_f32.
+ * query [tokens, heads, dim], key / value [kv_tokens, kv_heads, dim] packed by
+ * sequence; sequence b owns query tokens offsets[b] .. + lens_q[b] and keys
+ * offsets[b] .. + lens_kv[b]; top-left causal; lse [tokens, heads] natural log,
+ * -1e20 where a token sees no key.  Tokens no sequence owns stay zero. */
+ORACLE_API void oracle_ragged_kv_prefill_attention_f32(
+    float *out, float *lse, const float *query, const float *key, const float *value,
+    const int32_t *lens_q, const int32_t *lens_kv, const int32_t *offsets, size_t batch,
+    size_t total_query_tokens, size_t heads, size_t kv_heads, size_t head_dim, int causal, float scale) {
+    size_t group = heads / kv_heads, features = heads * head_dim, kv_features = kv_heads * head_dim;
+    memset(out, 0, total_query_tokens * features * sizeof(float));
+    memset(lse, 0, total_query_tokens * heads * sizeof(float));
+    for (size_t b = 0; b < batch; ++b) {
+        size_t seq_q = (size_t)lens_q[b], seq_kv = (size_t)lens_kv[b], offset = (size_t)offsets[b];
+        float *scores = (float *)malloc((seq_kv ? seq_kv : 1) * sizeof(float));
+        size_t *kept = (size_t *)malloc((seq_kv ? seq_kv : 1) * sizeof(size_t));
+        for (size_t qi = 0; qi < seq_q; ++qi) {
+            size_t token = offset + qi;
+            for (size_t head = 0; head < heads; ++head) {
+                size_t kv_head = head / group, count = 0;
+                const float *q = query + token * features + head * head_dim;
+                for (size_t j = 0; j < seq_kv; ++j) {
+                    if (causal && j > qi) continue;
+                    scores[count] = dot_fma(q, key + (offset + j) * kv_features + kv_head * head_dim, head_dim) * scale;
+                    kept[count++] = j;
+                }
+                if (count == 0) {
+                    lse[token * heads + head] = -1.0e20f;
+                    continue;
+                }
+                float denom;
+                float largest = normalise(scores, count, &denom);
+                lse[token * heads + head] = largest + logf(denom);
+                float *o = out + token * features + head * head_dim;
+                for (size_t d = 0; d < head_dim; ++d) {
+                    float sum = 0.0f;
+                    for (size_t i = 0; i < count; ++i)
+                        sum = fmaf(scores[i], value[(offset + kept[i]) * kv_features + kv_head * head_dim + d], sum);
+                    o[d] = sum;
+                }
+            }
+        }
+        free(kept);
+        free(scores);
+    }
+}
+
+/* singe-kernel/src/cpu/attention.rs:1927-1998  softcapped_window_decode_lse_f32.
+ * query / out [batch, heads, dim], key / value [batch, kv_heads, key_len, dim]
+ * (BHSD); the query sits at position key_len - 1; window_size w > 0 hides keys
+ * with key + w < that position; lse [batch, heads] natural log. */
+ORACLE_API void oracle_softcapped_window_decode_lse_f32(
+    float *out, float *lse, const float *query, const float *key, const float *value, size_t batch,
+    size_t key_len, size_t heads, size_t kv_heads, size_t head_dim, float scale, size_t window_size,
+    int has_soft_cap, float soft_cap) {
+    size_t key_head_stride = key_len * head_dim, group = heads / kv_heads, position = key_len - 1;
+    float *scores = (float *)malloc((key_len ? key_len : 1) * sizeof(float));
+    size_t *kept = (size_t *)malloc((key_len ? key_len : 1) * sizeof(size_t));
+    for (size_t b = 0; b < batch; ++b)
+        for (size_t head = 0; head < heads; ++head) {
+            size_t kv_head = head / group, count = 0;
+            const float *q = query + b * heads * head_dim + head * head_dim;
+            const float *k = key + b * kv_heads * key_head_stride + kv_head * key_head_stride;
+            const float *v = value + b * kv_heads * key_head_stride + kv_head * key_head_stride;
+            for (size_t j = 0; j < key_len; ++j) {
+                if (window_size > 0 && j + window_size < position) continue;
+                float score = dot_fma(q, k + j * head_dim, head_dim) * scale;
+                if (has_soft_cap) score = tanhf(score / soft_cap) * soft_cap;
+                scores[count] = score;
+                kept[count++] = j;
+            }
+            float denom;
+            float largest = normalise(scores, count, &denom);
+            lse[b * heads + head] = largest + logf(denom);
+            float *o = out + b * heads * head_dim + head * head_dim;
+            for (size_t d = 0; d < head_dim; ++d) {
+                float sum = 0.0f;
+                for (size_t i = 0; i < count; ++i) sum = fmaf(scores[i], v[kept[i] * head_dim + d], sum);
+                o[d] = sum;
+            }
+        }
+    free(kept);
+    free(scores);
+}
+
+/* singe-kernel/src/cpu/attention.rs:2073-2155  attention_sink_prefill_f32.
+ * BSHD; query q sits at start_q + q; causal hides later keys; window w != 0
+ * hides keys before position - (w - 1) (saturating); the head's sink logit
+ * joins the row's maximum and denominator and weighs no value.  The weighted
+ * sum runs key by key over every dim (an fma into the output row). */
+ORACLE_API void oracle_attention_sink_prefill_f32(
+    float *out, const float *query, const float *key, const float *value, const float *sinks,
+    size_t batch, size_t query_len, size_t key_len, size_t heads, size_t kv_heads, size_t head_dim,
+    size_t start_q, size_t window, float scale, int causal) {
+    size_t q_features = heads * head_dim, kv_features = kv_heads * head_dim, group = heads / kv_heads;
+    memset(out, 0, batch * query_len * q_features * sizeof(float));
+    float *scores = (float *)malloc((key_len + 1) * sizeof(float));
+    size_t *kept = (size_t *)malloc((key_len + 1) * sizeof(size_t));
+    for (size_t b = 0; b < batch; ++b)
+        for (size_t qi = 0; qi < query_len; ++qi) {
+            size_t position = start_q + qi;
+            size_t window_start = window == 0 ? 0 : (position >= window - 1 ? position - (window - 1) : 0);
+            for (size_t head = 0; head < heads; ++head) {
+                size_t kv_head = head / group, count = 0;
+                const float *q = query + b * query_len * q_features + qi * q_features + head * head_dim;
+                scores[count++] = sinks[head];
+                for (size_t j = 0; j < key_len; ++j) {
+                    if ((causal && j > position) || (window != 0 && j < window_start)) continue;
+                    kept[count] = j;
+                    scores[count++] = dot_fma(q, key + b * key_len * kv_features + j * kv_features + kv_head * head_dim, head_dim) * scale;
+                }
+                float largest = fold_max(scores, count), denom = 0.0f;
+                for (size_t i = 0; i < count; ++i) {
+                    scores[i] = expf(scores[i] - largest);
+                    denom += scores[i];
+                }
+                float *o = out + b * query_len * q_features + qi * q_features + head * head_dim;
+                for (size_t i = 1; i < count; ++i) {
+                    float weight = scores[i] / denom;
+                    const float *v = value + b * key_len * kv_features + kept[i] * kv_features + kv_head * head_dim;
+                    for (size_t d = 0; d < head_dim; ++d) o[d] = fmaf(weight, v[d], o[d]);
+                }
+            }
+        }
+    free(kept);
+    free(scores);
+}
+
+/* The arithmetic of the reference's sliding_window_attention_paged_kv_f32 kernel
+ * (singe-kernel/src/cuda/cutile/kernel/attention/local.rs:9150-9330; the CPU
+ * module has no paged form): sliding_window_attention_f32 over keys behind a
+ * block table, key j of batch b in slot j % block_size of block
+ * table[b * table_stride + j / block_size]; a block id >= physical_blocks hides
+ * the key.  Caches [physical_blocks, block_size, kv_heads, dim] contiguous,
+ * query / out BSHD contiguous. */
+ORACLE_API void oracle_sliding_window_attention_paged_kv_f32(
+    float *out, const float *query, const float *key_cache, const float *value_cache,
+    const uint32_t *block_table, size_t batch, size_t query_len, size_t key_len, size_t heads,
+    size_t kv_heads, size_t head_dim, size_t query_start, size_t key_start, size_t window,
+    size_t block_size, size_t physical_blocks, size_t table_stride, float scale, float output_scale) {
+    size_t q_features = heads * head_dim, kv_features = kv_heads * head_dim, group = heads / kv_heads;
+    memset(out, 0, batch * query_len * q_features * sizeof(float));
+    float *scores = (float *)malloc((key_len ? key_len : 1) * sizeof(float));
+    size_t *kept = (size_t *)malloc((key_len ? key_len : 1) * sizeof(size_t));
+    for (size_t b = 0; b < batch; ++b)
+        for (size_t qi = 0; qi < query_len; ++qi) {
+            size_t query_abs = query_start + qi;
+            for (size_t head = 0; head < heads; ++head) {
+                size_t kv_head = head / group, count = 0;
+                const float *q = query + b * query_len * q_features + qi * q_features + head * head_dim;
+                for (size_t j = 0; j < key_len; ++j) {
+                    size_t key_abs = key_start + j;
+                    if (key_abs > query_abs || key_abs + window <= query_abs) continue;
+                    size_t block = block_table[b * table_stride + j / block_size];
+                    if (block >= physical_blocks) continue;
+                    size_t row = (block * block_size + j % block_size) * kv_features + kv_head * head_dim;
+                    scores[count] = dot_fma(q, key_cache + row, head_dim) * scale;
+                    kept[count++] = row;
+                }
+                if (count == 0) continue;
+                float denom;
+                normalise(scores, count, &denom);
+                float *o = out + b * query_len * q_features + qi * q_features + head * head_dim;
+                for (size_t d = 0; d < head_dim; ++d) {
+                    float sum = 0.0f;
+                    for (size_t i = 0; i < count; ++i) sum = fmaf(scores[i], value_cache[kept[i] + d], sum);
+                    o[d] = sum * output_scale;
+                }
+            }
+        }
+    free(kept);
+    free(scores);
+}
+
 /* singe-kernel/src/cpu/attention.rs:2157-2193  splitk_reduce_f32.
  * attn [batch, heads, splits, dim], lse [batch, heads, splits] (natural log);
  * out = sum_s exp(lse_s - max) * attn_s / sum_s exp(lse_s - max). */

@@ -53,6 +53,35 @@ class SoftcappedWindowAttentionConfigC(ctypes.Structure):
                 ("soft_cap", ctypes.c_float)]
 
 
+class AttentionSinkPrefillConfigC(ctypes.Structure):
+    _fields_ = [("attention", FmhaPrefillConfigC), ("start_q", c_size), ("window", c_size)]
+
+
+class RaggedKvPrefillAttentionConfigC(ctypes.Structure):
+    _fields_ = [("batch", c_size), ("total_query_tokens", c_size), ("total_kv_tokens", c_size), ("heads", c_size),
+                ("kv_heads", c_size), ("head_dim", c_size), ("causal", ctypes.c_uint8), ("scale", ctypes.c_float)]
+
+
+_SLIDING_FIELDS = ("batch", "query_len", "key_len", "heads", "kv_heads", "head_dim", "query_start", "key_start", "window",
+                   "query_batch_stride", "key_batch_stride", "value_batch_stride", "output_batch_stride",
+                   "query_sequence_stride", "key_sequence_stride", "value_sequence_stride", "output_sequence_stride",
+                   "query_head_stride", "key_head_stride", "value_head_stride", "output_head_stride")
+
+
+class SlidingWindowAttentionConfigC(ctypes.Structure):
+    _fields_ = [(name, c_size) for name in _SLIDING_FIELDS] + [("scale", ctypes.c_float), ("output_scale", ctypes.c_float)]
+
+
+class PackedQkvAttentionConfigC(ctypes.Structure):
+    _fields_ = [("attention", SlidingWindowAttentionConfigC), ("query_offset", c_size), ("key_offset", c_size),
+                ("value_offset", c_size)]
+
+
+class PagedKvAttentionConfigC(ctypes.Structure):
+    _fields_ = [("attention", SlidingWindowAttentionConfigC), ("block_size", c_size), ("physical_blocks", c_size),
+                ("block_table_batch_stride", c_size), ("key_cache_block_stride", c_size), ("value_cache_block_stride", c_size)]
+
+
 class PagedAttentionProblemC(ctypes.Structure):
     _fields_ = [("tokens", ctypes.c_int64), ("heads", ctypes.c_int64), ("kv_heads", ctypes.c_int64),
                 ("head_dim", ctypes.c_int64), ("page_size", ctypes.c_int64), ("sequences", ctypes.c_int64),
@@ -92,6 +121,11 @@ class FmhaDecodeSplitKConfigC(ctypes.Structure):
         "key_batch_stride", "value_batch_stride", "output_batch_stride", "query_head_stride", "key_sequence_stride",
         "value_sequence_stride", "output_head_stride", "output_split_stride", "key_head_stride", "value_head_stride",
         "lse_batch_stride", "lse_head_stride")] + [("scale", ctypes.c_float)]
+
+
+class SoftcappedWindowDecodeConfigC(ctypes.Structure):
+    _fields_ = [("decode", FmhaDecodeConfigC), ("window_size", c_size), ("has_soft_cap", ctypes.c_uint8),
+                ("soft_cap", ctypes.c_float)]
 
 
 class TuneOptionsC(ctypes.Structure):
@@ -326,6 +360,25 @@ def bind(path: str) -> ctypes.CDLL:
     handle.singe_hip_fmha_decode_splitk_reduce_tuned_splits.restype = i32
     handle.singe_hip_clear_tune_cache.argtypes = []
     handle.singe_hip_clear_tune_cache.restype = None
+    pairs4, pairs5 = [c_void, c_size] * 4, [c_void, c_size] * 5
+    for element in ("bf16", "f16"):
+        entry = getattr(handle, f"singe_hip_softcapped_window_attention_{element}")
+        entry.argtypes, entry.restype = [c_void] + pairs4 + [ctypes.POINTER(SoftcappedWindowAttentionConfigC)], i32
+    for element in ("f32", "bf16", "f16"):
+        entry = getattr(handle, f"singe_hip_attention_sink_prefill_{element}")
+        entry.argtypes, entry.restype = [c_void] + pairs5 + [ctypes.POINTER(AttentionSinkPrefillConfigC)], i32
+        entry = getattr(handle, f"singe_hip_fmha_decode_lse_{element}")
+        entry.argtypes, entry.restype = [c_void] + pairs5 + [ctypes.POINTER(FmhaDecodeConfigC)], i32
+        entry = getattr(handle, f"singe_hip_softcapped_window_decode_lse_{element}")
+        entry.argtypes, entry.restype = [c_void] + pairs5 + [ctypes.POINTER(SoftcappedWindowDecodeConfigC)], i32
+        entry = getattr(handle, f"singe_hip_ragged_kv_prefill_attention_{element}")
+        entry.argtypes, entry.restype = [c_void] + [c_void, c_size] * 8 + [ctypes.POINTER(RaggedKvPrefillAttentionConfigC)], i32
+    handle.singe_hip_sliding_window_attention_f32.argtypes = [c_void] + pairs4 + [ctypes.POINTER(SlidingWindowAttentionConfigC)]
+    handle.singe_hip_sliding_window_attention_f32.restype = i32
+    handle.singe_hip_sliding_window_attention_packed_qkv_f32.argtypes = [c_void] + [c_void, c_size] * 2 + [ctypes.POINTER(PackedQkvAttentionConfigC)]
+    handle.singe_hip_sliding_window_attention_packed_qkv_f32.restype = i32
+    handle.singe_hip_sliding_window_attention_paged_kv_f32.argtypes = [c_void] + pairs5 + [ctypes.POINTER(PagedKvAttentionConfigC)]
+    handle.singe_hip_sliding_window_attention_paged_kv_f32.restype = i32
     handle.singe_hip_rotary_cache_write.argtypes = [c_void] * 14 + [ctypes.POINTER(RotaryCacheProblemC)]
     handle.singe_hip_rotary_cache_write.restype = i32
     handle.singe_hip_paging_indices.argtypes = [c_void] * 10 + [ctypes.POINTER(PagingIndicesProblemC)]

@@ -67,7 +67,7 @@ PARTS = [
 ]
 HOST_SOURCES = ["hip_runtime_loader.cpp", "module.cpp", "paged_decode.cpp", "fmha_prefill.cpp", "paged_attention.cpp",
                 "general_attention.cpp", "fmha_decode.cpp", "paged_rows_f32.cpp", "latent_attention.cpp", "cache_ops.cpp",
-                "mfma_ceiling.cpp", "attention_parameters.cpp", "synthetic_inputs.cpp"]
+                "mfma_ceiling.cpp", "attention_parameters.cpp", "synthetic_inputs.cpp", "attention_family.cpp"]
 JOBS = 8
 
 

@@ -268,6 +268,23 @@ size_t dense_prefill_scratch_bytes(const SingeFmhaPrefillConfig& c, uint32_t spl
 
 // The dense op's way into the matrix-core kernel: the public entry points' checks and launch, plus the op's options
 // (general_attention.cpp).
+bool dense_prefill_takes(const SingeFmhaPrefillConfig& c, const void* out, const void* query, const void* key, const void* value) {
+    if (!has_matrix_core_build(static_cast<long long>(c.head_dim))) return false;
+    const size_t strides[] = {c.query_batch_stride, c.key_batch_stride, c.value_batch_stride, c.output_batch_stride,
+                              c.query_sequence_stride, c.key_sequence_stride, c.value_sequence_stride,
+                              c.output_sequence_stride, c.query_head_stride, c.key_head_stride,
+                              c.value_head_stride, c.output_head_stride};
+    for (size_t stride : strides)
+        if (stride % 8 != 0) return false;
+    const uintptr_t addresses[] = {reinterpret_cast<uintptr_t>(out), reinterpret_cast<uintptr_t>(query),
+                                   reinterpret_cast<uintptr_t>(key), reinterpret_cast<uintptr_t>(value)};
+    for (uintptr_t address : addresses)
+        if (address % 16 != 0) return false;
+    const size_t widest = c.key_sequence_stride > c.value_sequence_stride ? c.key_sequence_stride : c.value_sequence_stride;
+    size_t slice_bytes = 0;
+    return checked_mul(c.key_len, widest, &slice_bytes) && checked_mul(slice_bytes, 2, &slice_bytes) && slice_bytes <= 0xffffffffull;
+}
+
 int32_t dense_prefill_with_options(void* stream, bool f16, uint16_t* out, size_t out_len, const uint16_t* query, size_t query_len,
                                    const uint16_t* key, size_t key_len, const uint16_t* value, size_t value_len,
                                    const SingeFmhaPrefillConfig* config, const DenseOptions& options) {

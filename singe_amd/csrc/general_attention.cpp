@@ -163,7 +163,23 @@ int32_t dense_general(int32_t data_type, void* stream, const char* op, const Den
     args.scale = o.scale;
     args.scale_wide = o.scale_wide;
     args.softcap = o.softcap;
-    const uint64_t rows = o.batch * o.heads * o.query_len;
+    args.query_start = o.query_start;
+    args.key_start = o.key_start;
+    args.lookahead = o.lookahead;
+    args.output_scale = o.output_scale;
+    args.empty_lse = o.empty_lse;
+    args.block_table = o.block_table;
+    args.block_size = static_cast<uint32_t>(o.block_size);
+    args.physical_blocks = static_cast<uint32_t>(o.physical_blocks);
+    args.table_stride = static_cast<uint32_t>(o.table_stride);
+    args.key_block_stride = o.key_block_stride;
+    args.value_block_stride = o.value_block_stride;
+    args.ragged = o.ragged ? 1u : 0u;
+    args.total_kv_tokens = static_cast<uint32_t>(o.total_kv_tokens);
+    args.query_lengths = o.query_lengths;
+    args.kv_lengths = o.kv_lengths;
+    args.sequence_offsets = o.sequence_offsets;
+    const uint64_t rows = (o.ragged ? 1 : o.batch) * o.heads * o.query_len;
     const uint64_t blocks = (rows + 3) / 4;
     if (blocks > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
     return launch(kernel, static_cast<unsigned>(blocks), 1, 1, 256, stream, args);

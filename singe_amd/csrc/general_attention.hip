@@ -109,7 +109,7 @@ SINGE_DEVICE void fold_key(LaneState<DMAX, typename E::real>& state, const typen
 // (attention.rs:255-262); pass -inf for none.  Returns max + ln(sum) of the row, -inf when it saw nothing.
 template <class E, int DMAX>
 SINGE_DEVICE typename E::real finish_row(const LaneState<DMAX, typename E::real>& state, typename E::type* out, unsigned int value_dim,
-                                         unsigned int lane, typename E::real sink) {
+                                         unsigned int lane, typename E::real sink, typename E::real output_scale = 1) {
     typedef typename E::real R;
     R row_max = state.largest;
 #pragma unroll
@@ -128,7 +128,7 @@ SINGE_DEVICE typename E::real finish_row(const LaneState<DMAX, typename E::real>
 #pragma unroll
             for (int step = 32; step >= 1; step >>= 1) value += __shfl_xor(value, step, 64);
             // A row that sees no key stays zero (attention.rs:503-515; a key count of zero gives zeros).
-            if (lane == (d & 63)) E::store(out + d, value * inverse);
+            if (lane == (d & 63)) E::store(out + d, output_scale == R(1) ? value * inverse : value * inverse * output_scale);
         }
     }
     return row_sum > 0 ? row_max + real_log(row_sum) : R(-INFINITY);
@@ -141,15 +141,46 @@ SINGE_DEVICE void dense_body(const GeneralAttentionArgs& a, typename Element<ELE
     typedef typename E::real R;
     const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const unsigned long long row = static_cast<unsigned long long>(blockIdx.x) * 4 + wave;
-    const unsigned long long rows = static_cast<unsigned long long>(a.batch) * a.heads * a.query_len;
+    const unsigned long long rows = static_cast<unsigned long long>(a.ragged ? 1u : a.batch) * a.heads * a.query_len;
     if (row >= rows) return;
-    const unsigned int query = static_cast<unsigned int>(row % a.query_len);
-    const unsigned int head = static_cast<unsigned int>((row / a.query_len) % a.heads);
-    const unsigned int batch = static_cast<unsigned int>(row / (static_cast<unsigned long long>(a.query_len) * a.heads));
+    // The row: (batch, head, query) of a dense problem; with ragged sequences (token, head), the token's sequence
+    // found by the lanes (the last sequence that owns it, as the CPU loop's later writes win).
+    unsigned int query, head, batch, key_len = a.key_len;
+    unsigned long long query_at, key_base = 0, lse_at;
+    if (a.ragged) {
+        const unsigned int token = static_cast<unsigned int>(row / a.heads);
+        head = static_cast<unsigned int>(row % a.heads);
+        int owner = -1;
+        for (unsigned int first_sequence = 0; first_sequence < a.batch; first_sequence += 64) {
+            const unsigned int sequence = first_sequence + lane;
+            bool mine = false;
+            if (sequence < a.batch) {
+                const long long offset = a.sequence_offsets[sequence], count = a.query_lengths[sequence];
+                mine = offset >= 0 && count > 0 && static_cast<long long>(token) >= offset && static_cast<long long>(token) < offset + count;
+            }
+            const unsigned long long owners = __ballot(mine);
+            if (owners != 0) owner = static_cast<int>(first_sequence + 63u - static_cast<unsigned int>(__builtin_clzll(owners)));
+        }
+        if (owner < 0) return;
+        batch = 0;
+        const long long offset = a.sequence_offsets[owner], keys = a.kv_lengths[owner];
+        query = token - static_cast<unsigned int>(offset);
+        query_at = token;
+        key_base = static_cast<unsigned long long>(offset);
+        const long long room = static_cast<long long>(a.total_kv_tokens) - offset;
+        key_len = keys <= 0 || room <= 0 ? 0u : static_cast<unsigned int>(keys < room ? keys : room);
+        lse_at = static_cast<unsigned long long>(token) * a.heads + head;
+    } else {
+        query = static_cast<unsigned int>(row % a.query_len);
+        head = static_cast<unsigned int>((row / a.query_len) % a.heads);
+        batch = static_cast<unsigned int>(row / (static_cast<unsigned long long>(a.query_len) * a.heads));
+        query_at = query;
+        lse_at = row;  // (batch * heads + head) * query_len + query
+    }
     const unsigned int kv_head = head / (a.heads / a.kv_heads);
-    const T* q = static_cast<const T*>(a.query) + batch * a.query_strides[0] + head * a.query_strides[1] + query * a.query_strides[2];
-    const T* k = static_cast<const T*>(a.key) + batch * a.key_strides[0] + kv_head * a.key_strides[1];
-    const T* v = static_cast<const T*>(a.value) + batch * a.value_strides[0] + kv_head * a.value_strides[1];
+    const T* q = static_cast<const T*>(a.query) + batch * a.query_strides[0] + head * a.query_strides[1] + query_at * a.query_strides[2];
+    const T* k = static_cast<const T*>(a.key) + batch * a.key_strides[0] + kv_head * a.key_strides[1] + key_base * a.key_strides[2];
+    const T* v = static_cast<const T*>(a.value) + batch * a.value_strides[0] + kv_head * a.value_strides[1] + key_base * a.value_strides[2];
     const T* mask = a.mask == nullptr ? nullptr
                                       : static_cast<const T*>(a.mask) + batch * a.mask_strides[0] + head * a.mask_strides[1] +
                                             query * a.mask_strides[2];
@@ -158,31 +189,39 @@ SINGE_DEVICE void dense_body(const GeneralAttentionArgs& a, typename Element<ELE
     for (unsigned int d = lane; d < a.head_dim; d += 64) q_row[d] = E::load(q + d);
     __builtin_amdgcn_wave_barrier();
 
-    // Keys the row may see (attention.rs:225-246): top-left causal, per-batch key count, and the
-    // window's `key + window <= query` rule.
-    unsigned int first = 0, end = a.key_len;
-    if (a.causal && query + 1 < end) end = query + 1;
+    // Keys the row may see (attention.rs:225-246): top-left causal, per-batch key count, the window's
+    // `key + window <= query` rule and the look-ahead bound, on positions query_start + query and key_start + key.
+    long long first = 0, end = key_len;
+    const long long position = a.query_start + static_cast<long long>(query) - a.key_start;  // of the query, in key indices
+    if (a.causal && position + 1 < end) end = position + 1;
+    if (a.lookahead >= 0 && position + a.lookahead + 1 < end) end = position + a.lookahead + 1;
     if (a.key_lengths != nullptr) {
         const int length = a.key_lengths[batch];
-        const unsigned int bound = length > 0 ? static_cast<unsigned int>(length) : 0u;
+        const long long bound = length > 0 ? length : 0;
         if (bound < end) end = bound;
     }
-    if (a.window >= 0) {
-        const unsigned long long window = static_cast<unsigned long long>(a.window);
-        if (static_cast<unsigned long long>(query) + 1 > window) first = static_cast<unsigned int>(query + 1 - window);
-    }
+    if (a.window >= 0 && position + 1 - a.window > first) first = position + 1 - a.window;
+    if (end < 0) end = 0;
 
     LaneState<DMAX, R> state;
     reset(state);
-    for (unsigned int key = first + lane; key < end; key += 64) {
+    for (long long key = first + lane; key < end; key += 64) {
         const R additive = mask != nullptr ? static_cast<R>(E::load(mask + key * a.mask_strides[3])) : R(0);
-        fold_key<E, DMAX>(state, q_row, k + static_cast<size_t>(key) * a.key_strides[2], v + static_cast<size_t>(key) * a.value_strides[2],
-                          a.head_dim, a.value_dim, own_scale<R>(a), a.has_softcap != 0, a.softcap, additive);
+        const T* k_row = k + static_cast<size_t>(key) * a.key_strides[2];
+        const T* v_row = v + static_cast<size_t>(key) * a.value_strides[2];
+        if (a.block_table != nullptr) {
+            const unsigned long long block = a.block_table[static_cast<size_t>(batch) * a.table_stride + static_cast<size_t>(key) / a.block_size];
+            if (block >= a.physical_blocks) continue;  // a block outside the cache hides its keys
+            const size_t slot = static_cast<size_t>(key) % a.block_size;
+            k_row = static_cast<const T*>(a.key) + block * a.key_block_stride + slot * a.key_strides[2] + kv_head * a.key_strides[1];
+            v_row = static_cast<const T*>(a.value) + block * a.value_block_stride + slot * a.value_strides[2] + kv_head * a.value_strides[1];
+        }
+        fold_key<E, DMAX>(state, q_row, k_row, v_row, a.head_dim, a.value_dim, own_scale<R>(a), a.has_softcap != 0, a.softcap, additive);
     }
     const R sink = a.sinks != nullptr ? static_cast<R>(E::load(static_cast<const T*>(a.sinks) + head)) : R(-INFINITY);
-    T* out = static_cast<T*>(a.out) + batch * a.out_strides[0] + head * a.out_strides[1] + query * a.out_strides[2];
-    const R lse = finish_row<E, DMAX>(state, out, a.value_dim, lane, sink);
-    if (a.lse != nullptr && lane == 0) a.lse[row] = static_cast<float>(lse);  // row = (batch * heads + head) * query_len + query
+    T* out = static_cast<T*>(a.out) + batch * a.out_strides[0] + head * a.out_strides[1] + query_at * a.out_strides[2];
+    const R lse = finish_row<E, DMAX>(state, out, a.value_dim, lane, sink, static_cast<R>(a.output_scale));
+    if (a.lse != nullptr && lane == 0) a.lse[lse_at] = lse == -INFINITY ? a.empty_lse : static_cast<float>(lse);
 }
 
 template <uint32_t ELEMENT, int DMAX, int FORM, bool DECODE = false>

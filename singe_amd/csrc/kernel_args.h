@@ -251,6 +251,26 @@ struct GeneralAttentionArgs {
     uint32_t causal, has_softcap;
     float scale, softcap;
     double scale_wide;              // the scale for f64 tensors: the default 1 / sqrt(head_dim) is taken in f64 there
+    // What the singe-kernel surface's dense family adds (all off by default).  Positions: query q sits at
+    // query_start + q and key k at key_start + k; the causal mask, the window (key + window <= query hidden) and
+    // `lookahead` (key > query + lookahead hidden; -1 = none) compare those.  The output is multiplied by
+    // output_scale; a row that saw no key leaves `empty_lse` as its log-sum-exp.
+    int64_t query_start = 0, key_start = 0, lookahead = -1;
+    float output_scale = 1.0f, empty_lse = -__builtin_inff();
+    // Keys behind a block table (block_table non-null): key k of batch b is slot k % block_size of block
+    // block_table[b * table_stride + k / block_size], at block * key_block_stride (value_block_stride) + slot *
+    // key_strides[2] + kv_head * key_strides[1]; a block id outside the cache hides the key.
+    const uint32_t* block_table = nullptr;
+    uint32_t block_size = 0, physical_blocks = 0, table_stride = 0;
+    uint64_t key_block_stride = 0, value_block_stride = 0;
+    // Ragged sequences (ragged != 0): rows are (token, head) pairs of `batch` sequences packed along the position
+    // axis; sequence s owns query tokens sequence_offsets[s] .. + query_lengths[s] and keys sequence_offsets[s] .. +
+    // kv_lengths[s] of the packed key / value tensors, clamped to total_kv_tokens; query_len is the total token
+    // count, lse is [tokens, heads]; a token no sequence owns is left alone.
+    uint32_t ragged = 0, total_kv_tokens = 0;
+    const int32_t* query_lengths = nullptr;
+    const int32_t* kv_lengths = nullptr;
+    const int32_t* sequence_offsets = nullptr;
 };
 
 // singe_paged_attention_general_*: the paged ops for any element type and head dimension.  `form`: the FlashInfer

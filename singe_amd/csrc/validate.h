@@ -38,6 +38,10 @@ int32_t dense_prefill_with_options(void* stream, bool f16, uint16_t* out, size_t
                                    const uint16_t* key, size_t key_len, const uint16_t* value, size_t value_len,
                                    const SingeFmhaPrefillConfig* config, const DenseOptions& options);
 
+// fmha_prefill.cpp: whether the matrix-core kernels take a call as it lies (a build for the head dimension, strides in
+// multiples of eight elements, 16-byte aligned buffers, a (batch, head) slice of keys within 4 GiB).
+bool dense_prefill_takes(const SingeFmhaPrefillConfig& config, const void* out, const void* query, const void* key, const void* value);
+
 // fmha_prefill.cpp: the shares the matrix-core dense kernel would split this problem's keys into (1 = none) and the
 // scratch they need.
 uint32_t dense_prefill_splits(const SingeFmhaPrefillConfig& config);
@@ -98,6 +102,16 @@ struct DenseGeneralOperands {
     bool causal = false, has_softcap = false;
     float scale = 1.0f, softcap = 0.0f;
     double scale_wide = 1.0;  // for f64 tensors
+    // The additions of the singe-kernel surface's dense family (GeneralAttentionArgs says what each means).
+    long long query_start = 0, key_start = 0, lookahead = -1;
+    float output_scale = 1.0f, empty_lse = -__builtin_inff();
+    const uint32_t* block_table = nullptr;
+    uint64_t block_size = 0, physical_blocks = 0, table_stride = 0, key_block_stride = 0, value_block_stride = 0;
+    bool ragged = false;
+    uint64_t total_kv_tokens = 0;
+    const int32_t* query_lengths = nullptr;
+    const int32_t* kv_lengths = nullptr;
+    const int32_t* sequence_offsets = nullptr;
 };
 int32_t dense_general(int32_t data_type, void* stream, const char* op, const DenseGeneralOperands& operands);
 

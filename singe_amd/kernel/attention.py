@@ -822,3 +822,296 @@ def paged_kv_decode_attention_f16(stream, out: torch.Tensor, query: torch.Tensor
         _ptr(value_cache), value_cache.numel(), _ptr(actual_seq_lens), actual_seq_lens.numel(), _ptr(block_table),
         block_table.numel(), _ptr(workspace), workspace.numel() * workspace.element_size(), ctypes.byref(c))
     _native.check(status, "paged_kv_decode_attention_f16")
+
+
+# ---- the rest of the dense family (fmha.rs:193-1036, paged.rs:36-116, 427-576) --------------------------------------
+
+_ELEMENTS = {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}
+
+
+def _call_family(name: str, dtype: torch.dtype, stream, tensors, config_c) -> None:
+    """Launches singe_hip_<name>_<element>(stream, (pointer, length) of every tensor in order, config)."""
+    element = _ELEMENTS[dtype]
+    arguments = []
+    for tensor in tensors:
+        arguments += [_ptr(tensor), tensor.numel()]
+    status = getattr(_native.lib(), f"singe_hip_{name}_{element}")(_stream_handle(stream), *arguments, ctypes.byref(config_c))
+    _native.check(status, f"{name}_{element}")
+
+
+def _softcapped_window_attention(dtype, stream, out, query, key, value, config: SoftcappedWindowAttentionConfig) -> None:
+    for tensor, name in ((out, "out"), (query, "query"), (key, "key"), (value, "value")):
+        _require(tensor, dtype, name)
+    c = _native.SoftcappedWindowAttentionConfigC(config.attention._c(), config.window_size, 1 if config.soft_cap is not None else 0,
+                                                 config.soft_cap if config.soft_cap is not None else 0.0)
+    _call_family("softcapped_window_attention", dtype, stream, (out, query, key, value), c)
+
+
+def softcapped_window_attention_bf16(stream, out, query, key, value, config: SoftcappedWindowAttentionConfig) -> None:
+    """softcapped_window_attention_bf16 (fmha.rs:345-393)."""
+    _softcapped_window_attention(torch.bfloat16, stream, out, query, key, value, config)
+
+
+def softcapped_window_attention_f16(stream, out, query, key, value, config: SoftcappedWindowAttentionConfig) -> None:
+    """softcapped_window_attention_f16 (fmha.rs:295-343)."""
+    _softcapped_window_attention(torch.float16, stream, out, query, key, value, config)
+
+
+@dataclass(frozen=True)
+class AttentionSinkPrefillConfig:
+    """AttentionSinkPrefillConfig (mod.rs:299-304): prefill whose softmax also holds one sink logit per head; query q
+    sits at position start_q + q; window w > 0 keeps the w keys up to that position."""
+    attention: FmhaPrefillConfig
+    start_q: int = 0
+    window: int = 0
+
+    @classmethod
+    def contiguous(cls, batch, query_len, key_len, heads, kv_heads, head_dim, start_q, window, scale, causal):
+        """mod.rs:1823-1841."""
+        return cls(FmhaPrefillConfig.contiguous(batch, query_len, key_len, heads, kv_heads, head_dim, scale, causal), start_q, window)
+
+    def _c(self):
+        return _native.AttentionSinkPrefillConfigC(self.attention._c(), self.start_q, self.window)
+
+
+def _attention_sink_prefill(dtype, stream, out, query, key, value, sinks, config: AttentionSinkPrefillConfig) -> None:
+    for tensor, name in ((out, "out"), (query, "query"), (key, "key"), (value, "value"), (sinks, "sinks")):
+        _require(tensor, dtype, name)
+    _call_family("attention_sink_prefill", dtype, stream, (out, query, key, value, sinks), config._c())
+
+
+def attention_sink_prefill_f32(stream, out, query, key, value, sinks, config: AttentionSinkPrefillConfig) -> None:
+    """attention_sink_prefill_f32 (fmha.rs:193-243; CPU form cpu/attention.rs:2073-2155)."""
+    _attention_sink_prefill(torch.float32, stream, out, query, key, value, sinks, config)
+
+
+def attention_sink_prefill_bf16(stream, out, query, key, value, sinks, config: AttentionSinkPrefillConfig) -> None:
+    """attention_sink_prefill_bf16 (fmha.rs:848-898)."""
+    _attention_sink_prefill(torch.bfloat16, stream, out, query, key, value, sinks, config)
+
+
+def attention_sink_prefill_f16(stream, out, query, key, value, sinks, config: AttentionSinkPrefillConfig) -> None:
+    """attention_sink_prefill_f16 (fmha.rs:796-846)."""
+    _attention_sink_prefill(torch.float16, stream, out, query, key, value, sinks, config)
+
+
+def _fmha_decode_lse(dtype, stream, out, lse, query, key, value, config: FmhaDecodeConfig) -> None:
+    for tensor, name in ((out, "out"), (query, "query"), (key, "key"), (value, "value")):
+        _require(tensor, dtype, name)
+    _require(lse, torch.float32, "lse")
+    _call_family("fmha_decode_lse", dtype, stream, (out, lse, query, key, value), config._c())
+
+
+def fmha_decode_lse_f32(stream, out, lse, query, key, value, config: FmhaDecodeConfig) -> None:
+    """fmha_decode_lse_f32 (fmha.rs:395-438): one query per batch item, lse [batch, heads] natural log."""
+    _fmha_decode_lse(torch.float32, stream, out, lse, query, key, value, config)
+
+
+def fmha_decode_lse_bf16(stream, out, lse, query, key, value, config: FmhaDecodeConfig) -> None:
+    """fmha_decode_lse_bf16 (fmha.rs:993-1036)."""
+    _fmha_decode_lse(torch.bfloat16, stream, out, lse, query, key, value, config)
+
+
+def fmha_decode_lse_f16(stream, out, lse, query, key, value, config: FmhaDecodeConfig) -> None:
+    """fmha_decode_lse_f16 (fmha.rs:900-943)."""
+    _fmha_decode_lse(torch.float16, stream, out, lse, query, key, value, config)
+
+
+@dataclass(frozen=True)
+class SoftcappedWindowDecodeConfig:
+    """SoftcappedWindowDecodeConfig (mod.rs:307-311): decode whose query sits at position key_len - 1; window_size w > 0
+    keeps the keys with key + w >= that position; optional tanh soft cap."""
+    decode: FmhaDecodeConfig
+    window_size: int = 0
+    soft_cap: float | None = None
+
+    @classmethod
+    def bnsd_contiguous(cls, batch, key_len, heads, kv_heads, head_dim, scale, window_size, soft_cap):
+        """mod.rs:2563-2602: key / value stored [batch, kv_heads, key_len, dim]."""
+        key_head_stride = key_len * head_dim
+        decode = FmhaDecodeConfig(batch, key_len, heads, kv_heads, head_dim, heads * head_dim, kv_heads * key_head_stride,
+                                  kv_heads * key_head_stride, heads * head_dim, head_dim, head_dim, head_dim, head_dim,
+                                  key_head_stride, key_head_stride, scale)
+        return cls(decode, window_size, soft_cap)
+
+    def _c(self):
+        return _native.SoftcappedWindowDecodeConfigC(self.decode._c(), self.window_size, 1 if self.soft_cap is not None else 0,
+                                                     self.soft_cap if self.soft_cap is not None else 0.0)
+
+
+def _softcapped_window_decode_lse(dtype, stream, out, lse, query, key, value, config: SoftcappedWindowDecodeConfig) -> None:
+    for tensor, name in ((out, "out"), (query, "query"), (key, "key"), (value, "value")):
+        _require(tensor, dtype, name)
+    _require(lse, torch.float32, "lse")
+    _call_family("softcapped_window_decode_lse", dtype, stream, (out, lse, query, key, value), config._c())
+
+
+def softcapped_window_decode_lse_f32(stream, out, lse, query, key, value, config: SoftcappedWindowDecodeConfig) -> None:
+    """softcapped_window_decode_lse_f32 (fmha.rs:440-486; CPU form cpu/attention.rs:1927-1998)."""
+    _softcapped_window_decode_lse(torch.float32, stream, out, lse, query, key, value, config)
+
+
+def softcapped_window_decode_lse_bf16(stream, out, lse, query, key, value, config: SoftcappedWindowDecodeConfig) -> None:
+    """softcapped_window_decode_lse_bf16 (fmha.rs:536-582)."""
+    _softcapped_window_decode_lse(torch.bfloat16, stream, out, lse, query, key, value, config)
+
+
+def softcapped_window_decode_lse_f16(stream, out, lse, query, key, value, config: SoftcappedWindowDecodeConfig) -> None:
+    """softcapped_window_decode_lse_f16 (fmha.rs:488-534)."""
+    _softcapped_window_decode_lse(torch.float16, stream, out, lse, query, key, value, config)
+
+
+@dataclass(frozen=True)
+class RaggedKvPrefillAttentionConfig:
+    """RaggedKvPrefillAttentionConfig (mod.rs:110-123): query, key and value tokens packed by sequence; per-batch lengths
+    and offsets describe each ragged segment."""
+    batch: int
+    total_query_tokens: int
+    total_kv_tokens: int
+    heads: int
+    kv_heads: int
+    head_dim: int
+    causal: bool
+    scale: float
+
+    @classmethod
+    def contiguous(cls, batch, total_query_tokens, total_kv_tokens, heads, kv_heads, head_dim, causal, scale):
+        """mod.rs:821-842: builds the config and validates it (validate_ragged_kv_prefill_attention_config, mod.rs:3013-3035)."""
+        config = cls(batch, total_query_tokens, total_kv_tokens, heads, kv_heads, head_dim, causal, scale)
+        extents = (batch, total_query_tokens, total_kv_tokens, heads, kv_heads, head_dim)
+        if any(e <= 0 for e in extents) or heads % kv_heads != 0 or not math.isfinite(scale):
+            raise error.InvalidLength("invalid length")
+        if any(e > I32_MAX for e in extents):
+            raise error.LengthExceedsI32("length exceeds i32")
+        return config
+
+    def _c(self):
+        return _native.RaggedKvPrefillAttentionConfigC(self.batch, self.total_query_tokens, self.total_kv_tokens, self.heads,
+                                                       self.kv_heads, self.head_dim, 1 if self.causal else 0, self.scale)
+
+
+def _ragged_kv_prefill_attention(dtype, stream, out, lse, query, key, value, lens_q, lens_kv, offsets,
+                                 config: RaggedKvPrefillAttentionConfig) -> None:
+    for tensor, name in ((out, "out"), (query, "query"), (key, "key"), (value, "value")):
+        _require(tensor, dtype, name)
+    _require(lse, torch.float32, "lse")
+    for tensor, name in ((lens_q, "actual_seq_lens_q"), (lens_kv, "actual_seq_lens_kv"), (offsets, "actual_seq_offsets")):
+        _require(tensor, torch.int32, name)
+    _call_family("ragged_kv_prefill_attention", dtype, stream, (out, lse, query, key, value, lens_q, lens_kv, offsets), config._c())
+
+
+def ragged_kv_prefill_attention_f32(stream, out, lse, query, key, value, actual_seq_lens_q, actual_seq_lens_kv, actual_seq_offsets,
+                                    config: RaggedKvPrefillAttentionConfig) -> None:
+    """ragged_kv_prefill_attention_f32 (paged.rs:427-477; CPU form cpu/attention.rs:1343-1420)."""
+    _ragged_kv_prefill_attention(torch.float32, stream, out, lse, query, key, value, actual_seq_lens_q, actual_seq_lens_kv,
+                                 actual_seq_offsets, config)
+
+
+def ragged_kv_prefill_attention_bf16(stream, out, lse, query, key, value, actual_seq_lens_q, actual_seq_lens_kv, actual_seq_offsets,
+                                     config: RaggedKvPrefillAttentionConfig) -> None:
+    """ragged_kv_prefill_attention_bf16 (paged.rs:531-576)."""
+    _ragged_kv_prefill_attention(torch.bfloat16, stream, out, lse, query, key, value, actual_seq_lens_q, actual_seq_lens_kv,
+                                 actual_seq_offsets, config)
+
+
+def ragged_kv_prefill_attention_f16(stream, out, lse, query, key, value, actual_seq_lens_q, actual_seq_lens_kv, actual_seq_offsets,
+                                    config: RaggedKvPrefillAttentionConfig) -> None:
+    """ragged_kv_prefill_attention_f16 (paged.rs:479-529)."""
+    _ragged_kv_prefill_attention(torch.float16, stream, out, lse, query, key, value, actual_seq_lens_q, actual_seq_lens_kv,
+                                 actual_seq_offsets, config)
+
+
+@dataclass(frozen=True)
+class SlidingWindowAttentionConfig:
+    """SlidingWindowAttentionConfig (mod.rs:32-56): query q at position query_start + q, key k at key_start + k; a key is
+    kept when its position is at most the query's and position + window is beyond it."""
+    batch: int
+    query_len: int
+    key_len: int
+    heads: int
+    kv_heads: int
+    head_dim: int
+    query_start: int
+    key_start: int
+    window: int
+    query_batch_stride: int
+    key_batch_stride: int
+    value_batch_stride: int
+    output_batch_stride: int
+    query_sequence_stride: int
+    key_sequence_stride: int
+    value_sequence_stride: int
+    output_sequence_stride: int
+    query_head_stride: int
+    key_head_stride: int
+    value_head_stride: int
+    output_head_stride: int
+    scale: float
+    output_scale: float = 1.0
+
+    @classmethod
+    def contiguous(cls, batch, query_len, key_len, heads, kv_heads, head_dim, query_start, key_start, window, scale):
+        """mod.rs:502-541: packed [batch, len, heads, dim] strides, output_scale 1."""
+        q_features, kv_features = heads * head_dim, kv_heads * head_dim
+        return cls(batch, query_len, key_len, heads, kv_heads, head_dim, query_start, key_start, window, query_len * q_features,
+                   key_len * kv_features, key_len * kv_features, query_len * q_features, q_features, kv_features, kv_features,
+                   q_features, head_dim, head_dim, head_dim, head_dim, scale, 1.0)
+
+    def with_output_scale(self, output_scale: float) -> "SlidingWindowAttentionConfig":
+        """mod.rs:543-547."""
+        import dataclasses
+
+        return dataclasses.replace(self, output_scale=output_scale)
+
+    def _c(self):
+        return _native.SlidingWindowAttentionConfigC(*(getattr(self, name) for name in _native._SLIDING_FIELDS), self.scale,
+                                                     self.output_scale)
+
+
+def sliding_window_attention_f32(stream, out, query, key, value, config: SlidingWindowAttentionConfig) -> None:
+    """sliding_window_attention_f32 (mod.rs:2812-2855; CPU form cpu/attention.rs:1089-1170)."""
+    for tensor, name in ((out, "out"), (query, "query"), (key, "key"), (value, "value")):
+        _require(tensor, torch.float32, name)
+    _call_family("sliding_window_attention", torch.float32, stream, (out, query, key, value), config._c())
+
+
+@dataclass(frozen=True)
+class PackedQkvAttentionConfig:
+    """PackedQkvAttentionConfig (mod.rs:59-64): query, key and value are views of one buffer from these offsets on."""
+    attention: SlidingWindowAttentionConfig
+    query_offset: int
+    key_offset: int
+    value_offset: int
+
+
+def sliding_window_attention_packed_qkv_f32(stream, out, qkv, config: PackedQkvAttentionConfig) -> None:
+    """sliding_window_attention_packed_qkv_f32 (paged.rs:36-50)."""
+    _require(out, torch.float32, "out")
+    _require(qkv, torch.float32, "qkv")
+    c = _native.PackedQkvAttentionConfigC(config.attention._c(), config.query_offset, config.key_offset, config.value_offset)
+    status = _native.lib().singe_hip_sliding_window_attention_packed_qkv_f32(_stream_handle(stream), _ptr(out), out.numel(), _ptr(qkv),
+                                                                             qkv.numel(), ctypes.byref(c))
+    _native.check(status, "sliding_window_attention_packed_qkv_f32")
+
+
+@dataclass(frozen=True)
+class PagedKvAttentionConfig:
+    """PagedKvAttentionConfig (mod.rs:67-74): the sliding-window attention's keys and values behind a block table."""
+    attention: SlidingWindowAttentionConfig
+    block_size: int
+    physical_blocks: int
+    block_table_batch_stride: int
+    key_cache_block_stride: int
+    value_cache_block_stride: int
+
+
+def sliding_window_attention_paged_kv_f32(stream, out, query, key_cache, value_cache, block_table, config: PagedKvAttentionConfig) -> None:
+    """sliding_window_attention_paged_kv_f32 (paged.rs:56-116)."""
+    for tensor, name in ((out, "out"), (query, "query"), (key_cache, "key_cache"), (value_cache, "value_cache")):
+        _require(tensor, torch.float32, name)
+    if block_table.dtype not in (torch.int32, torch.uint32):
+        raise error.InvalidArgument(f"block_table must hold 32-bit entries, got {block_table.dtype}")
+    _require(block_table, block_table.dtype, "block_table")
+    c = _native.PagedKvAttentionConfigC(config.attention._c(), config.block_size, config.physical_blocks,
+                                        config.block_table_batch_stride, config.key_cache_block_stride, config.value_cache_block_stride)
+    _call_family("sliding_window_attention_paged_kv", torch.float32, stream, (out, query, key_cache, value_cache, block_table), c)

@@ -384,3 +384,64 @@ def test_two_threads_hold_different_settings():
         lib.singe_hip_set_relaxed_numerics(0)
         lib.singe_hip_set_thread_options(None)
     assert int(lib.singe_hip_decode_workers(ctypes.byref(c))) == default_workers and config.workspace_bytes() == default_bytes
+
+
+def test_dense_family_validation_order_needs_no_device():
+    """The rest of the dense family checks config and lengths in the order of the reference's validate_lengths, before
+    any pointer is read: statuses and the names they carry, on fake pointers."""
+    lib = _native.lib()
+    fake = 0x1000
+    detail = _native.ErrorDetail()
+
+    def named(status):
+        lib.singe_hip_last_error(ctypes.byref(detail))
+        return status, (detail.name or b"").decode()
+
+    prefill = A.FmhaPrefillConfig.contiguous(2, 8, 8, 4, 2, 64, 0.1, True)
+    full = 2 * 8 * 4 * 64
+    sink = _native.AttentionSinkPrefillConfigC(prefill._c(), 3, 2)
+    call = lambda lengths, config=sink: named(lib.singe_hip_attention_sink_prefill_f32(
+        None, fake, lengths[0], fake, lengths[1], fake, lengths[2], fake, lengths[3], fake, lengths[4], ctypes.byref(config)))
+    kv = 2 * 8 * 2 * 64
+    assert call([full, full - 1, kv, kv, 4]) == (2, "query")          # query, key, value, out, then sinks (mod.rs:1843-1858)
+    assert call([full - 1, full, kv - 1, kv, 4]) == (2, "key")
+    assert call([full - 1, full, kv, kv, 4]) == (2, "out")
+    assert call([full, full, kv, kv, 3]) == (2, "sinks")
+    assert call([full, full, kv, kv, 4], _native.AttentionSinkPrefillConfigC(prefill._c(), 1 << 31, 2)) == (3, "start_q")
+    assert named(lib.singe_hip_attention_sink_prefill_f32(None, fake, full, fake, full, fake, kv, fake, kv, None, 4, ctypes.byref(sink))) == (6, "sinks")
+
+    decode = A.FmhaDecodeConfig.contiguous(2, 9, 4, 2, 64, 0.1)
+    capped = _native.SoftcappedWindowDecodeConfigC(decode._c(), 4, 1, 0.0)   # a cap of zero is invalid
+    rows, keys = 2 * 4 * 64, 2 * 9 * 2 * 64
+    windowed = lambda config, lse_len=8: named(lib.singe_hip_softcapped_window_decode_lse_bf16(
+        None, fake, rows, fake, lse_len, fake, rows, fake, keys, fake, keys, ctypes.byref(config)))
+    assert windowed(capped) == (1, "soft_cap")
+    assert windowed(_native.SoftcappedWindowDecodeConfigC(decode._c(), 1 << 31, 0, 0.0)) == (3, "window_size")
+    assert windowed(_native.SoftcappedWindowDecodeConfigC(decode._c(), 4, 1, 2.0), lse_len=7) == (2, "lse")
+    assert named(lib.singe_hip_fmha_decode_lse_f16(None, fake, rows, fake, 8, fake, rows, fake, keys - 1, fake, keys,
+                                                   ctypes.byref(decode._c()))) == (2, "key")
+
+    ragged = A.RaggedKvPrefillAttentionConfig.contiguous(3, 10, 12, 4, 2, 32, True, 0.2)._c()
+    lengths = [10 * 4 * 32, 40, 10 * 4 * 32, 12 * 2 * 32, 12 * 2 * 32, 3, 3, 3]
+    names = ["out", "lse", "query", "key", "value", "actual_seq_lens_q", "actual_seq_lens_kv", "actual_seq_offsets"]
+    for position in reversed(range(8)):   # with every later length good, the first short one is the one reported
+        short = list(lengths)
+        for earlier in range(position, 8):
+            short[earlier] = lengths[earlier] - (1 if earlier == position else 0)
+        arguments = []
+        for length in short:
+            arguments += [fake, length]
+        assert named(lib.singe_hip_ragged_kv_prefill_attention_f32(None, *arguments, ctypes.byref(ragged))) == (2, names[position])
+    with pytest.raises(error.InvalidLength):
+        A.RaggedKvPrefillAttentionConfig.contiguous(3, 10, 12, 4, 3, 32, True, 0.2)   # kv heads must divide heads
+
+    sliding = A.SlidingWindowAttentionConfig.contiguous(2, 5, 13, 4, 2, 16, 8, 0, 4, 0.3)
+    paged = _native.PagedKvAttentionConfigC(sliding._c(), 4, 11, 4, 4 * 2 * 16, 4 * 2 * 16)
+    cache = 11 * 4 * 2 * 16
+    through = lambda table_len, cache_len=cache, config=paged: named(lib.singe_hip_sliding_window_attention_paged_kv_f32(
+        None, fake, 2 * 5 * 4 * 16, fake, 2 * 5 * 4 * 16, fake, cache_len, fake, cache, fake, table_len, ctypes.byref(config)))
+    assert through(7) == (2, "block_table")       # (batch - 1) * stride + ceil(13 / 4) = 8 entries (mod.rs:2893-2900)
+    assert through(8, cache - 1) == (2, "key_cache")
+    assert through(8, cache, _native.PagedKvAttentionConfigC(sliding._c(), 0, 11, 4, 128, 128))[0] == 1
+    packed = _native.PackedQkvAttentionConfigC(sliding._c(), 0, 10, 1 << 40)
+    assert named(lib.singe_hip_sliding_window_attention_packed_qkv_f32(None, fake, 640, fake, 5000, ctypes.byref(packed))) == (2, "qkv")
