@@ -15,10 +15,16 @@ using namespace singe_hip;
 
 namespace {
 
-// Whether the problem runs on the matrix-core kernel (latent width 512, positional width 64, a 16-bit type).
+// Whether the problem runs on a matrix-core kernel: a 16-bit type, a latent width that is a multiple of 32 up to 512
+// and a positional width that is a multiple of 8 and makes the key width a multiple of 16, the widths the reference's
+// tensor-core plan takes (mla.rs:75, 140-146), with a positional part of at most 64 (wider ones, up to the reference's
+// 128, stay on the vector unit: the kernel's LDS rows hold 64).
 bool on_matrix_cores(const SingePagedMlaAttentionProblem& p) {
-    return p.data_type != SINGE_HIP_F32 && p.latent_dim == 512 && p.position_dim == 64;
+    return p.data_type != SINGE_HIP_F32 && p.latent_dim > 0 && p.latent_dim <= 512 && p.latent_dim % 32 == 0 && p.position_dim >= 0 &&
+           p.position_dim <= 64 && p.position_dim % 8 == 0 && (p.latent_dim + p.position_dim) % 16 == 0;
 }
+// The build for exactly latent 512 + positional 64; other widths take the `_any` kernels.
+bool built_shape(const SingePagedMlaAttentionProblem& p) { return p.latent_dim == 512 && p.position_dim == 64; }
 
 // Key splits for a problem: the row tiles of a decode step or a short chunk (one workgroup each, one workgroup to a
 // compute unit) leave most of the chip idle, so each tile's keys are shared out until there is about one workgroup
@@ -100,8 +106,8 @@ int32_t paged_mla_attention(void* stream, const void* latent_queries, const void
     args.sequences = static_cast<uint32_t>(p.sequences);
     args.cache_pages = static_cast<uint32_t>(p.cache_pages);
     args.page_table = static_cast<uint32_t>(p.page_table);
-    // Latent width 512 with positional width 64 in a 16-bit type runs on the matrix cores, 128 (token, head) rows of
-    // a sequence to a workgroup; every other shape on the vector unit, 4 rows to a workgroup.
+    // A 16-bit type at the widths on_matrix_cores names runs on the matrix cores, 128 (token, head) rows of a sequence
+    // to a workgroup; every other shape on the vector unit, 4 rows to a workgroup.
     const bool tiles = on_matrix_cores(p);
     const uint64_t rows_per_block = tiles ? 128 : 4;
     const uint64_t row_blocks = (static_cast<uint64_t>(p.tokens) * p.heads + rows_per_block - 1) / rows_per_block;
@@ -142,11 +148,13 @@ int32_t paged_mla_attention(void* stream, const void* latent_queries, const void
         args.unit_band = static_cast<uint32_t>(band);
         const uint64_t grid = splits > 1 ? blocks * splits : rounds * 8 * band;
         if (grid > 0x7fffffffull) return fail(SINGE_HIP_UNSUPPORTED_CONFIGURATION, "too many workgroups");
-        const bool bf16 = p.data_type == SINGE_HIP_BF16;
-        const int32_t launched = launch(bf16 ? kLatentTilesBf16 : kLatentTilesF16, static_cast<unsigned>(grid), 1, 1, 512, stream, args);
+        const bool bf16 = p.data_type == SINGE_HIP_BF16, built = built_shape(p);
+        const KernelId tiles_kernel = built ? (bf16 ? kLatentTilesBf16 : kLatentTilesF16) : (bf16 ? kLatentTilesAnyBf16 : kLatentTilesAnyF16);
+        const int32_t launched = launch(tiles_kernel, static_cast<unsigned>(grid), 1, 1, 512, stream, args);
         if (launched != 0 || splits == 1) return launched;
         // The merge: 32 workgroups of four waves to a unit, a wave to a row.
-        return launch(bf16 ? kLatentCombineBf16 : kLatentCombineF16, static_cast<unsigned>(blocks * 32), 1, 1, 256, stream, args);
+        const KernelId merge = built ? (bf16 ? kLatentCombineBf16 : kLatentCombineF16) : (bf16 ? kLatentCombineAnyBf16 : kLatentCombineAnyF16);
+        return launch(merge, static_cast<unsigned>(blocks * 32), 1, 1, 256, stream, args);
     }
     const int kernel = kLatentGeneral + (p.data_type == SINGE_HIP_F32 ? 0 : p.data_type == SINGE_HIP_BF16 ? 1 : 2);
     return launch(static_cast<KernelId>(kernel), static_cast<unsigned>(blocks), 1, 1, 256, stream, args);

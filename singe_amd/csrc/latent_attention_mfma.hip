@@ -1,7 +1,11 @@
 // Latent attention over paged caches on the matrix cores: bf16 or f16, latent width 512, positional width 64
 // (DeepSeek's absorbed MLA).  The same op as latent_attention.hip (CPU: singe/src/backend/cpu/normalization/
-// attention.rs:540-679; kernel plan: singe/src/backend/cuda/kernel_plan/source/mla.rs), for the one shape that
-// matters in practice; every other shape stays on the vector-unit kernel.
+// attention.rs:540-679; kernel plan: singe/src/backend/cuda/kernel_plan/source/mla.rs), built for the one shape that
+// matters in practice.  The `_any` kernels (ANY below) run the same loop for every other width the reference's
+// tensor-core plan takes with a positional part of at most 64 (latent a multiple of 32 up to 512, positional a multiple
+// of 8: mla.rs:75, 140-146): rows keep their 512 + 64 places in LDS, a lane whose chunk lies past a row's real width
+// loads nothing and finds the zeros the stages were filled with at the start, Q^T is zero there, and the outputs past
+// the latent width are not stored; narrower shapes pay for the full width's products.
 //
 // Every head of a token attends over the same cache rows, so the rows of a sequence, (query, head) pairs in
 // query-major order, are tiled 128 to a workgroup and the cache is read once per tile of rows instead of once
@@ -139,9 +143,19 @@ struct TilePages {
     RawPage<FORM> positional;
 };
 
-template <class Half, int FORM>
+template <class Half, int FORM, bool ANY>
 SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* lds) {
     const unsigned int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
+    // The widths of a row in global memory: the built shape, or (ANY) whatever the problem says.
+    const unsigned int latent_row_bytes = ANY ? 2u * a.latent_dim : static_cast<unsigned int>(kLatentRowBytes);
+    const unsigned int positional_row_bytes = ANY ? 2u * a.position_dim : static_cast<unsigned int>(kPositionalRowBytes);
+    const unsigned int latent_chunks = ANY ? a.latent_dim / 8u : 64u, positional_chunks = ANY ? a.position_dim / 8u : 8u;
+    if constexpr (ANY) {
+        // Chunks past a row's real width are never loaded: they read as the zeros put here.
+        for (unsigned int at = threadIdx.x * 16u; at < 2u * kStageBytes; at += 64u * kWaves * 16u)
+            *reinterpret_cast<uint4*>(lds + at) = make_uint4(0, 0, 0, 0);
+        __syncthreads();
+    }
     const unsigned int column = lane & 15u, g = lane >> 4;  // row of the wave, lane group
     const unsigned int splits = a.splits > 1 ? a.splits : 1u;
     // Workgroup i runs on XCD i % 8.  Without key splits, units (row tiles, in sequence order) are dealt to the
@@ -218,12 +232,16 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
     uint4 q[kSteps - kParkedSteps];  // steps kParkedSteps and up
     unsigned char* parked = lds + 2 * kStageBytes + wave * (kParkedSteps * 1024) + 16u * lane;
     {
-        const unsigned char* latent_row = static_cast<const unsigned char*>(a.latent_queries) + flat * kLatentRowBytes + 16u * g;
-        const unsigned char* positional_row = static_cast<const unsigned char*>(a.positional_queries) + flat * kPositionalRowBytes + 16u * g;
+        const unsigned char* latent_row = static_cast<const unsigned char*>(a.latent_queries) + flat * latent_row_bytes + 16u * g;
+        const unsigned char* positional_row = static_cast<const unsigned char*>(a.positional_queries) + flat * positional_row_bytes + 16u * g;
 #pragma unroll
         for (int s = 0; s < kSteps; ++s) {
-            uint4 bits = s < kLatentSteps ? *reinterpret_cast<const uint4*>(latent_row + 64 * s)
-                                          : *reinterpret_cast<const uint4*>(positional_row + 64 * (s - kLatentSteps));
+            // (ANY: the lane's chunk of the step, 4 s + g of the latent part or 4 (s - 16) + g of the positional one, may lie past the row)
+            const bool real = !ANY || (s < kLatentSteps ? 4u * s + g < latent_chunks : 4u * (s - kLatentSteps) + g < positional_chunks);
+            uint4 bits = make_uint4(0, 0, 0, 0);
+            if (real)
+                bits = s < kLatentSteps ? *reinterpret_cast<const uint4*>(latent_row + 64 * s)
+                                        : *reinterpret_cast<const uint4*>(positional_row + 64 * (s - kLatentSteps));
             if (!row_valid) bits = make_uint4(0, 0, 0, 0);
             if (s < kParkedSteps)
                 *reinterpret_cast<uint4*>(parked + 1024 * s) = bits;
@@ -271,7 +289,7 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
             unsigned char* dest = stage + row * kLatentRowBytes;
             if (page < static_cast<unsigned long long>(a.cache_pages)) {
                 const size_t slot = static_cast<size_t>(page) * a.page_size + place_of(key_of(tile, row));
-                load_to_lds(latent_cache + slot * kLatentRowBytes, lane_chunk[i & 1], dest);
+                if (!ANY || lane_chunk[i & 1] < 16u * latent_chunks) load_to_lds(latent_cache + slot * latent_row_bytes, lane_chunk[i & 1], dest);
             } else {
                 if (lane == 0) report_index_error(a.status);
                 *reinterpret_cast<uint4*>(dest + 16u * lane) = make_uint4(0, 0, 0, 0);
@@ -285,8 +303,8 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
                 // 64-bit value per lane to keep)
                 unsigned int chunk = positional_chunk;
                 asm volatile("" : "+v"(chunk));
-                const unsigned char* source = positional_cache + (slot * kPositionalRowBytes + chunk);
-                load_to_lds(source, dest);
+                const unsigned char* source = positional_cache + (slot * positional_row_bytes + chunk);
+                if (!ANY || positional_chunk < 16u * positional_chunks) load_to_lds(source, dest);
             } else {
                 report_index_error(a.status);
                 *reinterpret_cast<uint4*>(dest + 16u * lane) = make_uint4(0, 0, 0, 0);
@@ -448,9 +466,10 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
                 make_float4(out[db][0] * inverse, out[db][1] * inverse, out[db][2] * inverse, out[db][3] * inverse);
         if (g == 0) a.partial_lse[slot] = sum > 0.0f ? reference + fast_log2(sum) : -INFINITY;
     } else if (row_valid) {
-        unsigned char* row = static_cast<unsigned char*>(a.output) + flat * kLatentRowBytes + 8u * g;
+        unsigned char* row = static_cast<unsigned char*>(a.output) + flat * latent_row_bytes + 8u * g;
 #pragma unroll
         for (int db = 0; db < kDimBlocks; ++db) {
+            if (ANY && 2u * db >= latent_chunks) break;  // dims past the latent width
             uint2 packed;
             packed.x = pack_pair(half, out[db][0] * inverse, out[db][1] * inverse);
             packed.y = pack_pair(half, out[db][2] * inverse, out[db][3] * inverse);
@@ -468,7 +487,7 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
 // are asked for four at a time.
 constexpr unsigned int kCombineBlocks = kRows / 4;
 
-template <class Half, int FORM>
+template <class Half, int FORM, bool ANY>
 SINGE_DEVICE void latent_combine_rows(const LatentAttentionArgs& a) {
     const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
     // Workgroups map to (sequence, row tile) as in the attention kernel, so only rows that kernel wrote are read.
@@ -523,35 +542,42 @@ SINGE_DEVICE void latent_combine_rows(const LatentAttentionArgs& a) {
     packed.y = pack_pair(half, acc[2] * inverse, acc[3] * inverse);
     packed.z = pack_pair(half, acc[4] * inverse, acc[5] * inverse);
     packed.w = pack_pair(half, acc[6] * inverse, acc[7] * inverse);
-    *reinterpret_cast<uint4*>(static_cast<unsigned char*>(a.output) + row * kLatentRowBytes + 16u * lane) = packed;
+    // (a share's rows are 512 values apart whatever the latent width; the output's rows are as wide as the problem's)
+    if (!ANY || 8u * lane < a.latent_dim)
+        *reinterpret_cast<uint4*>(static_cast<unsigned char*>(a.output) + row * (ANY ? 2u * a.latent_dim : static_cast<unsigned int>(kLatentRowBytes)) + 16u * lane) = packed;
     if (a.lse != nullptr && lane == 0) a.lse[row] = total > 0.0f ? largest + fast_log2(total) : -INFINITY;
 }
 
-template <class Half>
+template <class Half, bool ANY>
 SINGE_DEVICE void latent_tile_body(const LatentAttentionArgs& a, unsigned char* lds) {
     if (a.wide_index)
-        latent_tile_rows<Half, kCsrI64>(a, lds);
+        latent_tile_rows<Half, kCsrI64, ANY>(a, lds);
     else
-        latent_tile_rows<Half, kCsrI32>(a, lds);
+        latent_tile_rows<Half, kCsrI32, ANY>(a, lds);
 }
 
 }  // namespace latent_mfma
 
-#define SINGE_LATENT_MFMA_KERNEL(NAME, HALF)                                                              \
+#define SINGE_LATENT_MFMA_KERNEL(NAME, HALF, ANY)                                                         \
     extern "C" __global__ __launch_bounds__(64 * latent_mfma::kWaves, 2) void NAME(LatentAttentionArgs args) { \
         __shared__ __attribute__((aligned(1024))) unsigned char latent_lds[latent_mfma::kLdsBytes];         \
-        latent_mfma::latent_tile_body<prefill::HALF>(args, latent_lds);                                    \
+        latent_mfma::latent_tile_body<prefill::HALF, ANY>(args, latent_lds);                               \
     }
 
-#define SINGE_LATENT_COMBINE_KERNEL(NAME, HALF)                                                  \
+#define SINGE_LATENT_COMBINE_KERNEL(NAME, HALF, ANY)                                             \
     extern "C" __global__ __launch_bounds__(256) void NAME(LatentAttentionArgs args) {          \
         if (args.wide_index)                                                                    \
-            latent_mfma::latent_combine_rows<prefill::HALF, kCsrI64>(args);                     \
+            latent_mfma::latent_combine_rows<prefill::HALF, kCsrI64, ANY>(args);                \
         else                                                                                    \
-            latent_mfma::latent_combine_rows<prefill::HALF, kCsrI32>(args);                     \
+            latent_mfma::latent_combine_rows<prefill::HALF, kCsrI32, ANY>(args);                \
     }
 
-SINGE_LATENT_COMBINE_KERNEL(singe_paged_mla_attention_combine_bf16, Bf16)
-SINGE_LATENT_COMBINE_KERNEL(singe_paged_mla_attention_combine_f16, F16)
-SINGE_LATENT_MFMA_KERNEL(singe_paged_mla_attention_bf16_l512_p64, Bf16)
-SINGE_LATENT_MFMA_KERNEL(singe_paged_mla_attention_f16_l512_p64, F16)
+SINGE_LATENT_COMBINE_KERNEL(singe_paged_mla_attention_combine_bf16, Bf16, false)
+SINGE_LATENT_COMBINE_KERNEL(singe_paged_mla_attention_combine_f16, F16, false)
+SINGE_LATENT_MFMA_KERNEL(singe_paged_mla_attention_bf16_l512_p64, Bf16, false)
+SINGE_LATENT_MFMA_KERNEL(singe_paged_mla_attention_f16_l512_p64, F16, false)
+// Any latent width that is a multiple of 32 up to 512 with a positional width that is a multiple of 8 up to 64.
+SINGE_LATENT_MFMA_KERNEL(singe_paged_mla_attention_bf16_any, Bf16, true)
+SINGE_LATENT_MFMA_KERNEL(singe_paged_mla_attention_f16_any, F16, true)
+SINGE_LATENT_COMBINE_KERNEL(singe_paged_mla_attention_combine_bf16_any, Bf16, true)
+SINGE_LATENT_COMBINE_KERNEL(singe_paged_mla_attention_combine_f16_any, F16, true)

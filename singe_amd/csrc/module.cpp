@@ -268,6 +268,8 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_rotary_paged_attention_f16_d112_i32_p16", "singe_rotary_paged_attention_f16_d112_i64_p16",
     "singe_rotary_paged_attention_f16_d112_softcap_i32", "singe_rotary_paged_attention_f16_d112_softcap_i64",
     "singe_rotary_paged_attention_f16_d112_softcap_i32_p16", "singe_rotary_paged_attention_f16_d112_softcap_i64_p16",
+    "singe_paged_mla_attention_bf16_any", "singe_paged_mla_attention_f16_any",
+    "singe_paged_mla_attention_combine_bf16_any", "singe_paged_mla_attention_combine_f16_any",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -305,6 +307,7 @@ constexpr PartRun kPartRuns[] = {
     {0, 2}, {13, 2},              // the decode merge for rows with one or two slots, head_dim 128 and 64
     {6, 2},                       // a decode step in FlashInfer form -> rows for the decode kernels
     {3, 12}, {15, 12}, {19, 12}, {21, 12}, {23, 12}, {25, 12}, {27, 12}, {29, 12},  // the further fused-rotation kernels
+    {8, 4},                       // latent attention on the matrix cores at any width it takes
 };
 constexpr int runs_total() {
     int total = 0;

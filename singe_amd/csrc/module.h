@@ -76,7 +76,10 @@ enum KernelId : int {
     // the other multiples of 16 as in kOtherHeadDims: + 4 * (bf16 with a cap, f16, f16 with a cap) + (i64 indices)
     // + 2 * (page size a power of two of at least 16 keys)
     kRotaryPagedAttentionMore,
-    kKernelCount = kRotaryPagedAttentionMore + 8 * 12
+    // latent (MLA) attention on the matrix cores at the other widths (latent a multiple of 32 up to 512, positional a
+    // multiple of 8 up to 64): bf16, f16, then their merges
+    kLatentTilesAnyBf16 = kRotaryPagedAttentionMore + 8 * 12, kLatentTilesAnyF16, kLatentCombineAnyBf16, kLatentCombineAnyF16,
+    kKernelCount
 };
 
 

@@ -100,6 +100,53 @@ def test_matrix_core_shape_on_random_data(heads, page_size, index_dtype, causal,
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("latent,positional", [(128, 32), (256, 64), (384, 16), (32, 16), (96, 32), (480, 48), (512, 32), (256, 0), (64, 64)])
+@pytest.mark.parametrize("splits", [0, 5])
+def test_matrix_cores_at_the_reference_plan_s_other_widths(latent, positional, causal, dtype, splits):
+    """The widths the reference's tensor-core plan takes beside 512 + 64 (latent a multiple of 32 up to 512, positional a
+    multiple of 8 that makes the key width a multiple of 16: mla.rs:75, 140-146; positional parts up to 64 here) run on
+    the matrix cores too, with and without key splits, against the oracle on random data."""
+    import ctypes
+    from singe_amd import _native
+    sequences, heads, page_size = [(1, 700), (37, 37), (20, 333), (3, 0), (9, 4), (1, 65)], 24, 16
+    query_offsets, page_offsets, last, needed = [0], [0], [], 0
+    for queries, keys in sequences:
+        query_offsets.append(query_offsets[-1] + queries)
+        pages = (keys + page_size - 1) // page_size
+        needed += pages
+        page_offsets.append(needed)
+        last.append(0 if keys == 0 else keys - (pages - 1) * page_size)
+    page_count = needed + 2
+    rng = np.random.default_rng(latent + positional)
+    table = [int(page) for page in rng.permutation(page_count)[:needed]]
+    tokens = query_offsets[-1]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(latent)
+    rand = lambda *shape: torch.randn(shape, generator=gen, device="cuda").to(dtype)
+    device = [rand(tokens, heads, latent), rand(tokens, heads, positional), rand(page_count, page_size, latent), rand(page_count, page_size, positional)]
+    index = lambda entries: torch.tensor(entries, dtype=torch.int64, device="cuda")
+    paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
+    _native.lib().singe_hip_set_paged_mla_attention_splits(splits)
+    try:
+        out, lse = neural.paged_mla_attention(*device, paging, neural.AttentionOptions(causal=causal))
+        torch.cuda.synchronize()
+    finally:
+        _native.lib().singe_hip_set_paged_mla_attention_splits(0)
+    status, want, want_lse = oracle.paged_mla_attention(*[tensor.float().cpu().numpy() for tensor in device], query_offsets, page_offsets, table,
+                                                        last, causal=causal, threads=8)
+    assert status == 0
+    got, got_lse = out.float().cpu().numpy(), lse.cpu().numpy()
+    assert np.isfinite(got).all()
+    gap = np.abs(got - want)
+    worst, mean = (2e-2, 2e-3) if dtype == torch.bfloat16 else (5e-3, 5e-4)
+    assert gap.max() <= worst and gap.mean() <= mean, (gap.max(), gap.mean())
+    empty = np.isneginf(want_lse)
+    assert np.array_equal(np.isneginf(got_lse), empty) and not got[empty].any()
+    assert np.abs(got_lse[~empty] - want_lse[~empty]).max() <= 5e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("splits", [2, 3, 16, 64])
 @pytest.mark.parametrize("causal", [False, True])
 def test_key_splits_match_the_cpu_and_the_unsplit_kernel(splits, causal, dtype):
