@@ -64,6 +64,12 @@ PARTS = [
     ("paged_attention_d80", "paged_attention.hip", ["-DSINGE_HEAD_DIM=80"]),
     ("fmha_prefill_d112", "fmha_prefill.hip", ["-DSINGE_HEAD_DIM=112"]),
     ("paged_attention_d112", "paged_attention.hip", ["-DSINGE_HEAD_DIM=112"]),
+    ("paged_decode_d32", "paged_decode.hip", ["-DSINGE_HEAD_DIM=32"]),
+    ("paged_decode_d16", "paged_decode.hip", ["-DSINGE_HEAD_DIM=16"]),
+    ("paged_decode_d48", "paged_decode.hip", ["-DSINGE_HEAD_DIM=48"]),
+    ("paged_decode_d80", "paged_decode.hip", ["-DSINGE_HEAD_DIM=80"]),
+    ("paged_decode_d96", "paged_decode.hip", ["-DSINGE_HEAD_DIM=96"]),
+    ("paged_decode_d112", "paged_decode.hip", ["-DSINGE_HEAD_DIM=112"]),
 ]
 HOST_SOURCES = ["hip_runtime_loader.cpp", "module.cpp", "paged_decode.cpp", "fmha_prefill.cpp", "paged_attention.cpp",
                 "general_attention.cpp", "fmha_decode.cpp", "paged_rows_f32.cpp", "latent_attention.cpp", "cache_ops.cpp",

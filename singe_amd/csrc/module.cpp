@@ -270,6 +270,48 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_rotary_paged_attention_f16_d112_softcap_i32_p16", "singe_rotary_paged_attention_f16_d112_softcap_i64_p16",
     "singe_paged_mla_attention_bf16_any", "singe_paged_mla_attention_f16_any",
     "singe_paged_mla_attention_combine_bf16_any", "singe_paged_mla_attention_combine_f16_any",
+    "singe_paged_decode_bf16_d32_g1_b16", "singe_paged_decode_bf16_d32_g2_b16",
+    "singe_paged_decode_bf16_d32_g1_any", "singe_paged_decode_bf16_d32_g2_any",
+    "singe_paged_decode_combine_bf16_d32", "singe_paged_decode_f16_d32_g1_b16",
+    "singe_paged_decode_f16_d32_g2_b16", "singe_paged_decode_f16_d32_g1_any",
+    "singe_paged_decode_f16_d32_g2_any", "singe_paged_decode_combine_f16_d32",
+    "singe_paged_decode_combine_many_bf16_d32", "singe_paged_decode_combine_many_f16_d32",
+    "singe_paged_decode_combine_few_bf16_d32", "singe_paged_decode_combine_few_f16_d32",
+    "singe_paged_decode_bf16_d16_g1_b16", "singe_paged_decode_bf16_d16_g2_b16",
+    "singe_paged_decode_bf16_d16_g1_any", "singe_paged_decode_bf16_d16_g2_any",
+    "singe_paged_decode_combine_bf16_d16", "singe_paged_decode_f16_d16_g1_b16",
+    "singe_paged_decode_f16_d16_g2_b16", "singe_paged_decode_f16_d16_g1_any",
+    "singe_paged_decode_f16_d16_g2_any", "singe_paged_decode_combine_f16_d16",
+    "singe_paged_decode_combine_many_bf16_d16", "singe_paged_decode_combine_many_f16_d16",
+    "singe_paged_decode_combine_few_bf16_d16", "singe_paged_decode_combine_few_f16_d16",
+    "singe_paged_decode_bf16_d48_g1_b16", "singe_paged_decode_bf16_d48_g2_b16",
+    "singe_paged_decode_bf16_d48_g1_any", "singe_paged_decode_bf16_d48_g2_any",
+    "singe_paged_decode_combine_bf16_d48", "singe_paged_decode_f16_d48_g1_b16",
+    "singe_paged_decode_f16_d48_g2_b16", "singe_paged_decode_f16_d48_g1_any",
+    "singe_paged_decode_f16_d48_g2_any", "singe_paged_decode_combine_f16_d48",
+    "singe_paged_decode_combine_many_bf16_d48", "singe_paged_decode_combine_many_f16_d48",
+    "singe_paged_decode_combine_few_bf16_d48", "singe_paged_decode_combine_few_f16_d48",
+    "singe_paged_decode_bf16_d80_g1_b16", "singe_paged_decode_bf16_d80_g2_b16",
+    "singe_paged_decode_bf16_d80_g1_any", "singe_paged_decode_bf16_d80_g2_any",
+    "singe_paged_decode_combine_bf16_d80", "singe_paged_decode_f16_d80_g1_b16",
+    "singe_paged_decode_f16_d80_g2_b16", "singe_paged_decode_f16_d80_g1_any",
+    "singe_paged_decode_f16_d80_g2_any", "singe_paged_decode_combine_f16_d80",
+    "singe_paged_decode_combine_many_bf16_d80", "singe_paged_decode_combine_many_f16_d80",
+    "singe_paged_decode_combine_few_bf16_d80", "singe_paged_decode_combine_few_f16_d80",
+    "singe_paged_decode_bf16_d96_g1_b16", "singe_paged_decode_bf16_d96_g2_b16",
+    "singe_paged_decode_bf16_d96_g1_any", "singe_paged_decode_bf16_d96_g2_any",
+    "singe_paged_decode_combine_bf16_d96", "singe_paged_decode_f16_d96_g1_b16",
+    "singe_paged_decode_f16_d96_g2_b16", "singe_paged_decode_f16_d96_g1_any",
+    "singe_paged_decode_f16_d96_g2_any", "singe_paged_decode_combine_f16_d96",
+    "singe_paged_decode_combine_many_bf16_d96", "singe_paged_decode_combine_many_f16_d96",
+    "singe_paged_decode_combine_few_bf16_d96", "singe_paged_decode_combine_few_f16_d96",
+    "singe_paged_decode_bf16_d112_g1_b16", "singe_paged_decode_bf16_d112_g2_b16",
+    "singe_paged_decode_bf16_d112_g1_any", "singe_paged_decode_bf16_d112_g2_any",
+    "singe_paged_decode_combine_bf16_d112", "singe_paged_decode_f16_d112_g1_b16",
+    "singe_paged_decode_f16_d112_g2_b16", "singe_paged_decode_f16_d112_g1_any",
+    "singe_paged_decode_f16_d112_g2_any", "singe_paged_decode_combine_f16_d112",
+    "singe_paged_decode_combine_many_bf16_d112", "singe_paged_decode_combine_many_f16_d112",
+    "singe_paged_decode_combine_few_bf16_d112", "singe_paged_decode_combine_few_f16_d112",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -281,7 +323,8 @@ const char* const kPartNames[kPartCount] = {
     "general_attention_f16", "mfma_ceiling", "paged_decode_d64", "fmha_prefill_d64", "paged_attention_d64",
     "general_attention_f64", "hbm_stream", "fmha_prefill_d32", "paged_attention_d32", "fmha_prefill_d96", "paged_attention_d96",
     "fmha_prefill_d16", "paged_attention_d16", "fmha_prefill_d48", "paged_attention_d48", "fmha_prefill_d80", "paged_attention_d80",
-    "fmha_prefill_d112", "paged_attention_d112",
+    "fmha_prefill_d112", "paged_attention_d112", "paged_decode_d32",
+    "paged_decode_d16", "paged_decode_d48", "paged_decode_d80", "paged_decode_d96", "paged_decode_d112",
 };
 
 namespace {
@@ -308,6 +351,7 @@ constexpr PartRun kPartRuns[] = {
     {6, 2},                       // a decode step in FlashInfer form -> rows for the decode kernels
     {3, 12}, {15, 12}, {19, 12}, {21, 12}, {23, 12}, {25, 12}, {27, 12}, {29, 12},  // the further fused-rotation kernels
     {8, 4},                       // latent attention on the matrix cores at any width it takes
+    {30, 14}, {31, 14}, {32, 14}, {33, 14}, {34, 14}, {35, 14},  // the decode kernels and their merges for 32, 16, 48, 80, 96, 112
 };
 constexpr int runs_total() {
     int total = 0;

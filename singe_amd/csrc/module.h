@@ -79,7 +79,11 @@ enum KernelId : int {
     // latent (MLA) attention on the matrix cores at the other widths (latent a multiple of 32 up to 512, positional a
     // multiple of 8 up to 64): bf16, f16, then their merges
     kLatentTilesAnyBf16 = kRotaryPagedAttentionMore + 8 * 12, kLatentTilesAnyF16, kLatentCombineAnyBf16, kLatentCombineAnyF16,
-    kKernelCount
+    // the bf16 / f16 decode kernels built for the other multiples of 16 (32, 16, 48, 80, 96, 112, in that order),
+    // fourteen each: the ten from kDecodeBf16 in their order, then the merges for rows with many slots (bf16, f16)
+    // and with one or two (bf16, f16)
+    kDecodeOtherHeadDims,
+    kKernelCount = kDecodeOtherHeadDims + 6 * 14
 };
 
 
@@ -88,6 +92,29 @@ inline KernelId at_head_dim_64(KernelId kernel) {
     if (kernel < kDecodeF8Wide) return static_cast<KernelId>(kDecodeD64 + kernel);
     if (kernel >= kPrefillCausal && kernel < kPrefillF32D32) return static_cast<KernelId>(kPrefillD64 + (kernel - kPrefillCausal));
     return static_cast<KernelId>(kPagedD64 + (kernel - kPagedAttentionI32));
+}
+
+// Whether the bf16 / f16 decode kernels have a matrix-core build for a head dimension.
+inline bool has_decode_build(long long head_dim) { return head_dim >= 16 && head_dim <= 128 && head_dim % 16 == 0; }
+
+// The bank of the decode builds for a head dimension other than 128 and 64.
+inline int other_decode_bank(long long head_dim) {
+    const int order = head_dim == 32 ? 0 : head_dim == 16 ? 1 : head_dim == 48 ? 2 : head_dim == 80 ? 3 : head_dim == 96 ? 4 : 5;
+    return kDecodeOtherHeadDims + 14 * order;
+}
+
+// That build of a bf16 / f16 decode kernel or of its one-wave merge, named by its head_dim 128 id below kDecodeF8Wide.
+inline KernelId decode_at_head_dim(KernelId kernel, long long head_dim) {
+    if (head_dim == 128) return kernel;
+    return static_cast<KernelId>((head_dim == 64 ? static_cast<int>(kDecodeD64) : other_decode_bank(head_dim)) + kernel);
+}
+
+// The decode merges for rows with many slots (eight waves a row) and with one or two (four rows a fetch): + 1 for f16.
+inline KernelId decode_combine_many_at(long long head_dim) {
+    return head_dim == 128 ? kDecodeCombineMany : head_dim == 64 ? kDecodeCombineManyD64 : static_cast<KernelId>(other_decode_bank(head_dim) + 10);
+}
+inline KernelId decode_combine_few_at(long long head_dim) {
+    return head_dim == 128 ? kDecodeCombineFew : head_dim == 64 ? kDecodeCombineFewD64 : static_cast<KernelId>(other_decode_bank(head_dim) + 12);
 }
 
 // Whether the dense prefill and paged attention kernels have a matrix-core build for a head dimension.
@@ -125,7 +152,7 @@ inline int rotary_paged_attention_base(bool f16, bool softcap, long long head_di
 extern const char* const kKernelNames[kKernelCount];
 
 // Parts of the code object (one file each) and the part a kernel lives in.
-constexpr int kPartCount = 30;
+constexpr int kPartCount = 36;
 extern const char* const kPartNames[kPartCount];
 int kernel_part(int kernel);
 

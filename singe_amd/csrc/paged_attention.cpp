@@ -100,7 +100,7 @@ constexpr size_t kDecodeRowsMost = 8000;
 
 bool decode_rows_config(const SingePagedAttentionProblem& p, SingePagedKvDecodeAttentionConfig* config) {
     if (fixed_paged_attention_splits() != 0) return false;  // a fixed number of shares asks for the row-tile kernel
-    if ((p.head_dim != 128 && p.head_dim != 64) || p.has_softcap) return false;
+    if (!has_decode_build(p.head_dim) || p.has_softcap) return false;
     // Under a short window a token reads few keys, and one workgroup a (sequence, kv head) of the row-tile kernel, which
     // skips the tiles before the window, is done before the route's two extra launches would be (measured: 32 sequences,
     // window 128: 12.6 against 15.2 us; window 1024: level; window 4096: 70 against 57 us).

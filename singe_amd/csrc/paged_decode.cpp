@@ -223,9 +223,10 @@ int32_t decode(
     // What the gfx950 kernels take (the reference's cuTile kernels take head_dim 4..64 only and return
     // UnsupportedWidth otherwise: singe-kernel/src/cuda/cutile/attention/paged.rs:799-810).
     if (fp8 && c.head_dim != 128) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, "paged_kv_decode_attention_f8e4m3kv_bf16", c.head_dim, 0);
-    // The matrix-core kernels are built for head dimensions 128 and 64; the others (the reference's own kernels
-    // take 4 to 64 here, this library up to 256) run on the one-wave-per-row kernel and need no workspace.
-    if (c.head_dim != 128 && c.head_dim != 64) {
+    // The matrix-core kernels are built for the multiples of 16 up to 128 (fp8 caches: 128); the other head dimensions
+    // (the reference's own kernels take 4 to 64 here, this library up to 256) run on the one-wave-per-row kernel and
+    // need no workspace.
+    if (!has_decode_build(c.head_dim)) {
         if (!(phases & SINGE_HIP_DECODE_REDUCE)) return 0;  // nothing is left in the workspace at these widths
         uint64_t reach_keys = static_cast<uint64_t>(c.block_table_batch_stride) * c.block_size;
         if (!fits_i32(reach_keys)) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "block_table_batch_stride * block_size");
@@ -249,14 +250,14 @@ namespace singe_hip {
 
 size_t paged_decode_workspace_bytes(const SingePagedKvDecodeAttentionConfig& c) { return workspace_need(c); }
 
-// The two launches of the matrix-core decode (head_dim 128 or 64), after the entry point's checks.
+// The two launches of the matrix-core decode (a multiple of 16 up to 128), after the entry point's checks.
 int32_t launch_paged_decode(const SingePagedKvDecodeAttentionConfig& c, const PagedDecodeLaunch& l) {
     void* const stream = l.stream;
     const bool fp8 = l.fp8, f16 = l.f16;
     const uint32_t phases = l.phases;
     void* const workspace = l.workspace;
     const size_t workspace_bytes = l.workspace_bytes;
-    const bool narrow = c.head_dim == 64;  // the head_dim 64 build of the same kernels
+    const bool narrow = c.head_dim != 128;  // a narrower build of the same kernels
     uint64_t reach = static_cast<uint64_t>(c.block_table_batch_stride) * c.block_size;
     if (!fits_i32(reach)) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "block_table_batch_stride * block_size");
 
@@ -307,7 +308,7 @@ int32_t launch_paged_decode(const SingePagedKvDecodeAttentionConfig& c, const Pa
                             : wide ? static_cast<KernelId>(kDecodeWide + (aligned ? 0 : 1) + (f16 ? 2 : 0))
                                    : static_cast<KernelId>((f16 ? kDecodeF16 : kDecodeBf16) + (aligned ? 0 : 2) + (plan.groups == 2 ? 1 : 0));
     if (phases & SINGE_HIP_DECODE_SPLIT)
-        if (int32_t status = launch(narrow ? at_head_dim_64(kernel) : kernel, plan.grid_x, plan.grid_y, 1, 64 * kWavesPerWorkgroup, stream, args,
+        if (int32_t status = launch(narrow ? decode_at_head_dim(kernel, c.head_dim) : kernel, plan.grid_x, plan.grid_y, 1, 64 * kWavesPerWorkgroup, stream, args,
                                     prefix_bytes))
             return status;
     if (!(phases & SINGE_HIP_DECODE_REDUCE)) return 0;
@@ -327,17 +328,17 @@ int32_t launch_paged_decode(const SingePagedKvDecodeAttentionConfig& c, const Pa
     combine.heads_per_wave = plan.heads_per_wave;
     // A row has about workers / batch slots: from 32 on, a workgroup of eight waves folds it instead of one wave.
     if (static_cast<size_t>(plan.workers) >= 32 * c.batch) {
-        const KernelId many = static_cast<KernelId>(kDecodeCombineMany + (f16 ? 1 : 0) + (narrow ? 2 : 0));
+        const KernelId many = static_cast<KernelId>(decode_combine_many_at(c.head_dim) + (f16 ? 1 : 0));
         return launch(many, static_cast<unsigned>(c.batch * c.heads), 1, 1, 512, stream, combine);
     }
     // With no more workers than sequences a row has one or two slots, and the kernel that fetches four rows at a time
     // keeps twice the waves in flight.
     if (static_cast<size_t>(plan.workers) <= c.batch) {
-        const KernelId few = static_cast<KernelId>(kDecodeCombineFew + (f16 ? 1 : 0) + (narrow ? 2 : 0));
+        const KernelId few = static_cast<KernelId>(decode_combine_few_at(c.head_dim) + (f16 ? 1 : 0));
         return launch(few, static_cast<unsigned>((c.batch * c.heads + 3) / 4), 1, 1, 256, stream, combine);
     }
     const KernelId merge = f16 ? kDecodeF16Combine : kDecodeCombine;
-    return launch(narrow ? at_head_dim_64(merge) : merge, static_cast<unsigned>((c.batch * c.heads + 3) / 4), 1, 1, 256, stream, combine);
+    return launch(decode_at_head_dim(merge, c.head_dim), static_cast<unsigned>((c.batch * c.heads + 3) / 4), 1, 1, 256, stream, combine);
 }
 
 }  // namespace singe_hip

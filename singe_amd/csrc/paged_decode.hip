@@ -43,16 +43,18 @@
 
 namespace {
 
-// The head dimension a build of these kernels is for: the source is compiled once per value (128, and 64 with
-// -DSINGE_HEAD_DIM=64, bf16 and f16 caches only), each into its own part of the code object.  At 64 the register
-// layouts below stay as they are and only their first half is live: a key's row is eight 16-byte chunks, so lanes
-// t >= 8 fetch no values and the score products run over two 32-dim steps instead of four.
+// The head dimension a build of these kernels is for: the source is compiled once per value (128, and the other
+// multiples of 16 with -DSINGE_HEAD_DIM=, bf16 and f16 caches only), each into its own part of the code object.  Below
+// 128 the register layouts stay as they are and only their front is live: at 64 a key's row is eight 16-byte chunks,
+// so lanes t >= 8 fetch no values and the score products run over two 32-dim steps instead of four; at 32 a row is
+// four chunks and there is one step; where the last step is half a step (16, 48, 80, 112) its upper sixteen
+// dimensions are zeros in both operands.
 #ifndef SINGE_HEAD_DIM
 #define SINGE_HEAD_DIM 128
 #endif
 constexpr int kDim = SINGE_HEAD_DIM;
-static_assert(kDim == 64 || kDim == 128, "head dimensions the decode kernels are built for");
-constexpr int kDimSteps = kDim / 32;  // score products per 16 keys
+static_assert(kDim % 16 == 0 && kDim >= 16 && kDim <= 128, "head dimensions the decode kernels are built for");
+constexpr int kDimSteps = (kDim + 31) / 32;  // score products per 16 keys
 constexpr int kTile = 32;
 constexpr float kReferenceLag = 6.0f;  // doublings a softmax reference point may lag the largest score seen
 
@@ -465,11 +467,12 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
         for (int hg = 0; hg < GROUPS; ++hg) {
             const unsigned int local = 4 * hg + (t >> 2);
             const bool real = local < wave_heads;
-            const uint16_t* qp = a.query + (static_cast<size_t>(b) * a.heads + kv_head * group + head_in_group + (real ? local : 0)) * kDim + dim_lane;
+            const uint16_t* qp = a.query + (static_cast<size_t>(b) * a.heads + kv_head * group + head_in_group + (real ? local : 0)) * kDim;
 #pragma unroll
             for (int c = 0; c < kDimSteps; ++c) {
-                uint4 bits = *reinterpret_cast<const uint4*>(qp + dim_step * c);
-                if (!real) bits = make_uint4(0, 0, 0, 0);
+                const bool within = kDim % 32 == 0 || dim_lane + dim_step * c < static_cast<unsigned int>(kDim);  // (half a last step)
+                uint4 bits = *reinterpret_cast<const uint4*>(qp + (within ? dim_lane + dim_step * c : 0));
+                if (!real || !within) bits = make_uint4(0, 0, 0, 0);
                 q[hg][c] = __builtin_bit_cast(bf16x8_t, bits);
             }
             state[hg].acc[0] = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -613,6 +616,8 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
                 const unsigned char* row = key_staging + t * 256 + (((4 * c + g) ^ t) << 4);
                 first = *reinterpret_cast<const uint4*>(row);
                 second = *reinterpret_cast<const uint4*>(row + 16 * 256);
+                if (kDim % 32 != 0 && 8 * (4 * c + g) >= static_cast<unsigned int>(kDim))  // nobody wrote these chunks
+                    first = second = make_uint4(0, 0, 0, 0);
             }
 #pragma unroll
             for (int hg = 0; hg < GROUPS; ++hg) {

@@ -49,7 +49,7 @@ size_t dense_prefill_scratch_bytes(const SingeFmhaPrefillConfig& config, uint32_
 // Whether the launch gives the query heads of a kv head one tile (few query rows, grouped heads, no causal mask).
 bool dense_prefill_packs_heads(const SingeFmhaPrefillConfig& config);
 
-// paged_decode.cpp: the two launches of the matrix-core decode kernels (head_dim 128 or 64) for a config its caller has
+// paged_decode.cpp: the two launches of the matrix-core decode kernels (head_dim a multiple of 16 up to 128) for a config its caller has
 // checked, and the workspace they need.  `row_starts` non-null: the table holds rows of their own lengths (row b
 // starts at entry row_starts[b]; block_table_batch_stride is then the count of entries in all), the way the paged
 // attention op's page lists lie; `lse` non-null: the reduce also leaves each row's base-two log-sum-exp.

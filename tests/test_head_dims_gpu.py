@@ -5,7 +5,7 @@ The reference's own kernels take head_dim 4 to 64 for block-table decode
 (singe-kernel/src/cuda/attention/fmha.rs:752-755) and every multiple of 16 up to 128 for the tensor-core paged and dense
 kernels (singe/src/backend/cuda/kernel_plan/source/paged_attention.rs:586-592); two of the three shapes of its own
 paged test are head_dim 64 (kernel_plan/source/tests.rs:830-966).  Here every multiple of 16 up to 128 runs on a build
-of the matrix-core dense and paged kernels for that width (decode: 64 and 128), the other widths on the
+of the matrix-core dense, paged and decode kernels for that width, the other widths on the
 one-wave-per-row kernels.  Tolerances as at head_dim 128: bf16 max-abs
 2e-2 / mean-abs 2e-3, log-sum-exp 2e-3."""
 import numpy as np
@@ -88,7 +88,7 @@ def test_block_table_prefill_at_other_head_dims(dim, causal, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("dim", [4, 8, 16, 32, 64])
+@pytest.mark.parametrize("dim", [4, 8, 16, 32, 48, 64, 80, 96, 112])
 @pytest.mark.parametrize("heads,kv_heads,block_size", [(8, 2, 16), (12, 4, 7), (8, 8, 1), (16, 1, 32)])
 def test_block_table_decode_at_the_references_head_dims(dim, heads, kv_heads, block_size, dtype):
     lens = [0, 1, 15, 16, 17, 31, 32, 33, 100, 257, 300, 64]
@@ -101,14 +101,16 @@ def test_block_table_decode_at_the_references_head_dims(dim, heads, kv_heads, bl
     decode.assert_close(got, want, f"d{dim} {heads}/{kv_heads} block {block_size}")
 
 
+@pytest.mark.parametrize("dim", [64, 32, 16, 48, 112])
 @pytest.mark.parametrize("workers", [0, 1, 3, 50, 4096])
-def test_decode_splits_at_head_dim_64(workers):
+def test_decode_splits_at_the_narrow_matrix_core_head_dims(workers, dim):
     lens = [200, 1, 333, 0, 97, 160, 31, 512]
-    work = synthetic.paged_decode_workload(batch=len(lens), heads=8, kv_heads=2, head_dim=64, physical_blocks=128, seq_lens=lens, seed=7)
-    decode.assert_close(decode.run_gpu(work, workers), decode.run_oracle(work), f"split {workers}")
+    work = synthetic.paged_decode_workload(batch=len(lens), heads=8, kv_heads=2, head_dim=dim, physical_blocks=128, seq_lens=lens, seed=7)
+    decode.assert_close(decode.run_gpu(work, workers), decode.run_oracle(work), f"d{dim} split {workers}")
 
 
-def test_decode_at_head_dim_64_full_size_matches_oracle():
-    # the second benchmark configuration at the reference's head dimension
-    work = synthetic.paged_decode_workload(head_dim=64, fill="used")
-    decode.assert_close(decode.run_gpu(work), decode.run_oracle(work), "batch 32, ctx U[512, 4096], head_dim 64")
+@pytest.mark.parametrize("dim", [64, 32, 16, 80])
+def test_decode_at_the_narrow_matrix_core_head_dims_full_size_matches_oracle(dim):
+    # the second benchmark configuration at the reference's head dimensions
+    work = synthetic.paged_decode_workload(head_dim=dim, fill="used")
+    decode.assert_close(decode.run_gpu(work), decode.run_oracle(work), f"batch 32, ctx U[512, 4096], head_dim {dim}")
