@@ -1,5 +1,6 @@
 // Host side of dense prefill: FmhaPrefillConfig validation as the reference does it
 // (singe-kernel/src/cuda/attention/mod.rs:1602-1756, 3369-3398, 3647-3677) and the launch.
+#include <atomic>
 #include <cmath>
 
 #include "kernel_args.h"
@@ -10,6 +11,10 @@
 using namespace singe_hip;
 
 namespace {
+
+// Query rows a wave of the dense bf16 / f16 prefill takes: 0 = chosen by problem size, 32, or 64 where the two-tile
+// kernel takes the call (singe_hip_set_dense_prefill_rows_per_wave).
+std::atomic<uint32_t> g_rows_per_wave{0};
 
 int32_t validate_config(const SingeFmhaPrefillConfig& c) {
     const size_t extents[] = {c.batch, c.query_len, c.key_len, c.heads, c.kv_heads, c.head_dim,
@@ -234,6 +239,21 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
         groups *= splits;
     }
     const long long head_dim = static_cast<long long>(c.head_dim);
+    // Long rows without options at head_dim 128: the kernel that gives a wave two 32-row tiles (256 query rows a
+    // workgroup, one workgroup a compute unit), when every key tile is whole and its launch still fills the chip.
+    {
+        constexpr size_t kPairRows = 256;
+        const uint32_t pair_tiles = static_cast<uint32_t>((c.query_len + kPairRows - 1) / kPairRows);
+        const uint64_t pair_groups = rows * ((pair_tiles + 1) / 2);
+        const uint32_t wanted = g_rows_per_wave.load(std::memory_order_relaxed);
+        const bool eligible = head_dim == 128 && !with_options && options.sinks == nullptr && options.key_lengths == nullptr &&
+                              !args.packed_heads && splits == 1 && c.key_len > 0 && c.key_len % 64 == 0 && c.scale > 0.0f;
+        if (eligible && wanted != 32 && (wanted == 64 || pair_groups >= compute_units())) {
+            args.query_tiles = pair_tiles;
+            const KernelId pair = static_cast<KernelId>(kPrefillPair + (c.causal ? 0 : 1) + (f16 ? 2 : 0));
+            return launch(pair, static_cast<unsigned>(pair_groups), 1, 1, 256, stream, args);
+        }
+    }
     const KernelId kernel = static_cast<KernelId>((f16 ? kPrefillCausalF16 : kPrefillCausal) + (c.causal ? 0 : 1) + (with_options ? 4 : 0));
     if (int32_t status = launch(at_head_dim(kernel, head_dim), static_cast<unsigned>(groups), 1, 1, 64 * kDensePrefillWaves, stream, args))
         return status;
@@ -349,3 +369,5 @@ int32_t singe_hip_fmha_prefill_lse_f16(void* stream, uint16_t* out, size_t out_l
 }
 
 }  // extern "C"
+
+extern "C" void singe_hip_set_dense_prefill_rows_per_wave(uint32_t rows) { g_rows_per_wave.store(rows, std::memory_order_relaxed); }

@@ -312,6 +312,8 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_decode_f16_d112_g2_any", "singe_paged_decode_combine_f16_d112",
     "singe_paged_decode_combine_many_bf16_d112", "singe_paged_decode_combine_many_f16_d112",
     "singe_paged_decode_combine_few_bf16_d112", "singe_paged_decode_combine_few_f16_d112",
+    "singe_fmha_prefill_pair_bf16_d128_causal", "singe_fmha_prefill_pair_bf16_d128_full",
+    "singe_fmha_prefill_pair_f16_d128_causal", "singe_fmha_prefill_pair_f16_d128_full",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -325,6 +327,7 @@ const char* const kPartNames[kPartCount] = {
     "fmha_prefill_d16", "paged_attention_d16", "fmha_prefill_d48", "paged_attention_d48", "fmha_prefill_d80", "paged_attention_d80",
     "fmha_prefill_d112", "paged_attention_d112", "paged_decode_d32",
     "paged_decode_d16", "paged_decode_d48", "paged_decode_d80", "paged_decode_d96", "paged_decode_d112",
+    "fmha_prefill_pair",
 };
 
 namespace {
@@ -352,6 +355,7 @@ constexpr PartRun kPartRuns[] = {
     {3, 12}, {15, 12}, {19, 12}, {21, 12}, {23, 12}, {25, 12}, {27, 12}, {29, 12},  // the further fused-rotation kernels
     {8, 4},                       // latent attention on the matrix cores at any width it takes
     {30, 14}, {31, 14}, {32, 14}, {33, 14}, {34, 14}, {35, 14},  // the decode kernels and their merges for 32, 16, 48, 80, 96, 112
+    {36, 4},                      // the dense prefill with two row tiles a wave
 };
 constexpr int runs_total() {
     int total = 0;

@@ -83,7 +83,9 @@ enum KernelId : int {
     // fourteen each: the ten from kDecodeBf16 in their order, then the merges for rows with many slots (bf16, f16)
     // and with one or two (bf16, f16)
     kDecodeOtherHeadDims,
-    kKernelCount = kDecodeOtherHeadDims + 6 * 14
+    // the dense prefill that gives a wave two 32-row tiles (head_dim 128, no options): + (no causal mask) + 2 * f16
+    kPrefillPair = kDecodeOtherHeadDims + 6 * 14,
+    kKernelCount = kPrefillPair + 4
 };
 
 
@@ -152,7 +154,7 @@ inline int rotary_paged_attention_base(bool f16, bool softcap, long long head_di
 extern const char* const kKernelNames[kKernelCount];
 
 // Parts of the code object (one file each) and the part a kernel lives in.
-constexpr int kPartCount = 36;
+constexpr int kPartCount = 37;
 extern const char* const kPartNames[kPartCount];
 int kernel_part(int kernel);
 

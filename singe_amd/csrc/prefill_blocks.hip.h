@@ -70,6 +70,25 @@ SINGE_DEVICE void score_block(Half half, f32x16_t& scores, const uint4 (&q)[kSte
     scores = s;
 }
 
+// Whether a row's scaled maximum has run too far ahead of the point its weights are scaled by (or the row sees its
+// first key).
+SINGE_DEVICE bool reference_lags(const RowState& state, float largest) {
+    return largest > state.reference + kMaxLag || (state.reference == -INFINITY && largest != -INFINITY);
+}
+
+// Moves the reference point up to the row's maximum and rescales what was summed under the old one.
+SINGE_DEVICE void move_reference(RowState& state, float largest) {
+    const float moved = fmaxf(state.reference, largest);
+    const float base = moved == -INFINITY ? 0.0f : moved;
+    const float rescale = fast_exp2(state.reference - base);
+    state.running_sum *= rescale;
+#pragma unroll
+    for (int db = 0; db < kDimBlocks; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) state.out[db][r] *= rescale;
+    state.reference = moved;
+}
+
 // First half of folding a 32-key block: hides what the mask hides, takes the row maxima and moves the
 // softmax reference point when a row's maximum has run too far ahead of it.  Returns the shift the
 // exponentials take (minus the reference, 0 for rows that have seen nothing).
@@ -89,17 +108,7 @@ SINGE_DEVICE float begin_block(RowState& state, f32x16_t& s, unsigned int hi, fl
     other = max3(other, s[12], s[13]);
     largest = max3(largest, s[14], s[15]);
     largest = swap32_max(max2(largest, other)) * factor;  // both lanes of a query agree from here on
-    if (__any(largest > state.reference + kMaxLag || (state.reference == -INFINITY && largest != -INFINITY))) {
-        const float moved = fmaxf(state.reference, largest);
-        const float base = moved == -INFINITY ? 0.0f : moved;
-        const float rescale = fast_exp2(state.reference - base);
-        state.running_sum *= rescale;
-#pragma unroll
-        for (int db = 0; db < kDimBlocks; ++db)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) state.out[db][r] *= rescale;
-        state.reference = moved;
-    }
+    if (__any(reference_lags(state, largest))) move_reference(state, largest);
     return state.reference == -INFINITY ? 0.0f : -state.reference;
 }
 

@@ -139,3 +139,57 @@ def test_scores_that_keep_outrunning_the_reference_point(magnitude, causal):
     gap = np.abs(got - want)
     assert gap.max() <= 2e-2 and gap.mean() <= 2e-3, (gap.max(), gap.mean())
     assert (np.abs(lse.cpu().numpy() - want_lse) / np.maximum(1.0, np.abs(want_lse))).max() <= 1e-5
+
+
+@pytest.fixture
+def two_tiles_a_wave():
+    """Sends every dense call that has the form to the kernel that gives a wave two 32-row tiles."""
+    from singe_amd import _native
+    _native.lib().singe_hip_set_dense_prefill_rows_per_wave(64)
+    yield
+    _native.lib().singe_hip_set_dense_prefill_rows_per_wave(0)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("batch,query_len,key_len,heads,kv_heads", [
+    (1, 256, 256, 1, 1), (2, 512, 512, 4, 2), (1, 64, 64, 2, 2), (1, 100, 128, 3, 1), (1, 1, 64, 1, 1),
+    (1, 300, 192, 2, 2), (1, 1024, 1024, 8, 8), (1, 640, 1024, 4, 1), (1, 1024, 320, 2, 1), (3, 768, 768, 2, 1),
+])
+def test_two_tiles_a_wave_matches_oracle(two_tiles_a_wave, batch, query_len, key_len, heads, kv_heads, causal):
+    q, k, v = make(batch, query_len, key_len, heads, kv_heads, seed=query_len * 11 + key_len)
+    got, lse, want, want_lse = run(q, k, v, causal)
+    check(got, lse, want, want_lse, f"two tiles: {batch}x{query_len}x{key_len} h{heads}/{kv_heads} causal={causal}")
+
+
+def test_two_tiles_a_wave_negative_scale_and_no_lse(two_tiles_a_wave):
+    q, k, v = make(1, 512, 512, 2, 1, seed=8)
+    got, lse, want, want_lse = run(q, k, v, True, scale=-0.07, with_lse=False)
+    check(got, lse, want, want_lse, "two tiles, negative scale", with_lse=False)
+
+
+def test_two_tiles_a_wave_headline_slice_and_default_choice():
+    # The headline shape fills the chip with 256-row tiles, so the default choice is this kernel: a slice of it against the
+    # oracle, and the whole of it equal to the 32-row kernel's answer within the rounding of the output.
+    from singe_amd import _native
+    q, k, v = make(1, 4096, 4096, 4, 4, seed=99)
+    _native.lib().singe_hip_set_dense_prefill_rows_per_wave(64)
+    try:
+        got, lse, want, want_lse = run(q, k, v, True)
+    finally:
+        _native.lib().singe_hip_set_dense_prefill_rows_per_wave(0)
+    check(got, lse, want, want_lse, "two tiles, seq 4096")
+    batch, seq, heads, dim = 4, 4096, 32, 128
+    q, k, v = make(batch, seq, seq, heads, heads, seed=4)
+    config = A.FmhaPrefillConfig.contiguous(batch, seq, seq, heads, heads, dim, float(dim ** -0.5), True)
+    chosen, narrow = torch.empty_like(q), torch.empty_like(q)
+    lse_chosen = torch.empty((batch, heads, seq), device="cuda", dtype=torch.float32)
+    lse_narrow = torch.empty_like(lse_chosen)
+    A.fmha_prefill_lse_bf16(None, chosen, lse_chosen, q, k, v, config)
+    _native.lib().singe_hip_set_dense_prefill_rows_per_wave(32)
+    try:
+        A.fmha_prefill_lse_bf16(None, narrow, lse_narrow, q, k, v, config)
+    finally:
+        _native.lib().singe_hip_set_dense_prefill_rows_per_wave(0)
+    torch.cuda.synchronize()
+    assert (chosen.float() - narrow.float()).abs().max().item() <= 2 ** -6
+    assert (lse_chosen - lse_narrow).abs().max().item() <= 1e-4
