@@ -82,9 +82,39 @@ SINGE_DEVICE void score_block_pair(Half, f32x16_t& s, const u32x4_t (&q)[kSteps]
     asm volatile("s_nop 7\n\ts_nop 7" : "+v"(s));
 }
 
+// The row maxima of two score tiles, the two chains a statement apart so that no instruction waits for the one before
+// it (the compiler puts an idle slot after every statement whose instruction it does not know): three statements of
+// eight instructions, dealt to three slots of the schedule.
+SINGE_DEVICE void row_maxima_0(const f32x16_t& a, const f32x16_t& b, float& ma, float& na, float& mb, float& nb) {
+    asm volatile(
+        "v_max3_f32 %0, %4, %5, %6\n\tv_max3_f32 %2, %14, %15, %16\n\tv_max3_f32 %1, %7, %8, %9\n\tv_max3_f32 %3, %17, %18, %19\n\t"
+        "v_max3_f32 %0, %0, %10, %11\n\tv_max3_f32 %2, %2, %20, %21\n\tv_max3_f32 %1, %1, %12, %13\n\tv_max3_f32 %3, %3, %22, %23"
+        : "=&v"(ma), "=&v"(na), "=&v"(mb), "=&v"(nb)
+        : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(a[4]), "v"(a[5]), "v"(a[6]), "v"(a[7]), "v"(a[8]), "v"(a[9]), "v"(b[0]), "v"(b[1]),
+          "v"(b[2]), "v"(b[3]), "v"(b[4]), "v"(b[5]), "v"(b[6]), "v"(b[7]), "v"(b[8]), "v"(b[9]));
+}
+SINGE_DEVICE void row_maxima_1(const f32x16_t& a, const f32x16_t& b, float& ma, float& na, float& mb, float& nb) {
+    asm volatile(
+        "v_max3_f32 %0, %0, %4, %5\n\tv_max3_f32 %2, %2, %10, %11\n\tv_max3_f32 %1, %1, %6, %7\n\tv_max3_f32 %3, %3, %12, %13\n\t"
+        "v_max3_f32 %0, %0, %8, %9\n\tv_max3_f32 %2, %2, %14, %15\n\tv_max_f32 %0, %0, %1\n\tv_max_f32 %2, %2, %3"
+        : "+v"(ma), "+v"(na), "+v"(mb), "+v"(nb)
+        : "v"(a[10]), "v"(a[11]), "v"(a[12]), "v"(a[13]), "v"(a[14]), "v"(a[15]), "v"(b[10]), "v"(b[11]), "v"(b[12]), "v"(b[13]), "v"(b[14]),
+          "v"(b[15]));
+}
+// (the two lanes of a query exchange their maxima: see swap32_max)
+SINGE_DEVICE void row_maxima_2(float& ma, float& mb) {
+    float ta, tb;
+    asm volatile(
+        "v_mov_b32 %2, %0\n\tv_mov_b32 %3, %1\n\ts_nop 0\n\tv_permlane32_swap_b32 %0, %2\n\tv_permlane32_swap_b32 %1, %3\n\t"
+        "v_max_f32 %0, %0, %2\n\tv_max_f32 %1, %1, %3"
+        : "+v"(ma), "+v"(mb), "=&v"(ta), "=&v"(tb));
+}
+
 // One 32-key block b for both row tiles.  On entry a_cur / b_cur hold the raw scores of block b (shift_a / shift_b:
 // minus the rows' reference points, which already cover them) and `operand` the K operands of block b + 1; the V^T
-// operands of block b are read from `values` in the block's first slots.  On return a_nxt / b_nxt hold the raw scores
+// operands of block b are read in the block's first half, from value_origin (the first V stage, kept where the
+// compiler cannot fold its address into the offset) + the lane's offsets + `values` (the block's byte offset from
+// there, a constant once inlined: together with the stage's own address it would not fit the instruction's 16 bits).  On return a_nxt / b_nxt hold the raw scores
 // of block b + 1 and largest_a / largest_b their scaled row maxima, `operand` the K operands of block b + 2 (read
 // from keys_after); the rows' sums and O^T have taken block b in.  With LOADS, issue(0 .. 7) is
 // called once each (the tile's eight direct-to-LDS loads of this wave).
@@ -92,228 +122,229 @@ template <bool LOADS, class Half, class Issue>
 SINGE_DEVICE void fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t& a_cur, f32x16_t& b_cur, f32x16_t& a_nxt, f32x16_t& b_nxt,
                                   float factor, float shift_a, float shift_b, float& largest_a_out, float& largest_b_out,
                                   const u32x4_t (&qa)[8], const u32x4_t (&qb)[8], uint4 (&operand)[8], const unsigned char* __restrict__ keys_after,
-                                  const unsigned char* __restrict__ values, const ReadOffsets& offsets, Issue&& issue) {
+                                  const unsigned char* __restrict__ value_origin, unsigned int values, const ReadOffsets& offsets, Issue&& issue) {
     unsigned int wa[2][4], wb[2][4];
     v8i16_t v[2][4];
     float total_a = 0.0f, total_b = 0.0f;
+    float largest_a, other_a, largest_b, other_b;
 #define QK(S, Q, J) score_step<(J) == 0, true, Half>(S, operand[J], Q[J])
 #define PV(X, H, D, WORDS) \
     X.out[D] = mma(half, __builtin_bit_cast(uint4, v[H][D]), make_uint4(WORDS[H][0], WORDS[H][1], WORDS[H][2], WORDS[H][3]), X.out[D])
 #define E(S, I, SHIFT) S[I] = fast_exp2(fmaf(S[I], factor, SHIFT))
 #define T(TOTAL, S, I) TOTAL += S[I]
 #define W(WORDS, S, I) WORDS[(I) / 4][(I) % 4] = pack_pair(half, S[2 * (I)], S[2 * (I) + 1])
+#define ROW_MAXIMA_0 row_maxima_0(a_nxt, b_nxt, largest_a, other_a, largest_b, other_b)
+#define ROW_MAXIMA_1 row_maxima_1(a_nxt, b_nxt, largest_a, other_a, largest_b, other_b)
+#define ROW_MAXIMA_2 row_maxima_2(largest_a, largest_b)
 #define KR(J) operand[J] = *reinterpret_cast<const uint4*>(keys_after + offsets.key(J))
 #define VR(H, D)                                                                                                                        \
     {                                                                                                                                   \
-        const v4i16_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)(values + (16 * (H)) * kRowBytes + offsets.value(D))); \
-        const v4i16_t high = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)(values + (16 * (H) + 8) * kRowBytes + offsets.value(D))); \
+        const v4i16_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)(value_origin + offsets.value(D) + (values + (16 * (H)) * kRowBytes))); \
+        const v4i16_t high = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)(value_origin + offsets.value(D) + (values + (16 * (H) + 8) * kRowBytes))); \
         v[H][D] = __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7);                                                        \
     }
     // slot 0
     QK(a_nxt, qa, 0);
-    VR(0, 0);
     E(a_cur, 0, shift_a);
-    T(total_a, a_cur, 0);
+    E(a_cur, 1, shift_a);
     __builtin_amdgcn_sched_barrier(0);
     // slot 1
     QK(a_nxt, qa, 1);
-    VR(0, 1);
-    E(a_cur, 1, shift_a);
+    T(total_a, a_cur, 0);
+    E(a_cur, 2, shift_a);
     T(total_a, a_cur, 1);
     W(wa, a_cur, 0);
     __builtin_amdgcn_sched_barrier(0);
     // slot 2
     QK(a_nxt, qa, 2);
-    VR(0, 2);
-    E(a_cur, 2, shift_a);
+    E(a_cur, 3, shift_a);
     T(total_a, a_cur, 2);
+    E(a_cur, 4, shift_a);
     __builtin_amdgcn_sched_barrier(0);
     // slot 3
     QK(a_nxt, qa, 3);
-    VR(0, 3);
-    E(a_cur, 3, shift_a);
     T(total_a, a_cur, 3);
+    E(a_cur, 5, shift_a);
+    T(total_a, a_cur, 4);
     W(wa, a_cur, 1);
     __builtin_amdgcn_sched_barrier(0);
     // slot 4
     QK(a_nxt, qa, 4);
-    VR(1, 0);
-    E(a_cur, 4, shift_a);
-    T(total_a, a_cur, 4);
+    E(a_cur, 6, shift_a);
+    T(total_a, a_cur, 5);
+    E(a_cur, 7, shift_a);
     __builtin_amdgcn_sched_barrier(0);
     // slot 5
     QK(a_nxt, qa, 5);
-    VR(1, 1);
-    E(a_cur, 5, shift_a);
-    T(total_a, a_cur, 5);
+    T(total_a, a_cur, 6);
     W(wa, a_cur, 2);
+    T(total_a, a_cur, 7);
+    W(wa, a_cur, 3);
+    E(a_cur, 8, shift_a);
     __builtin_amdgcn_sched_barrier(0);
     // slot 6
     QK(a_nxt, qa, 6);
-    VR(1, 2);
-    E(a_cur, 6, shift_a);
-    T(total_a, a_cur, 6);
+    E(a_cur, 9, shift_a);
+    T(total_a, a_cur, 8);
+    E(a_cur, 10, shift_a);
     __builtin_amdgcn_sched_barrier(0);
     // slot 7
     QK(a_nxt, qa, 7);
-    VR(1, 3);
-    E(a_cur, 7, shift_a);
-    T(total_a, a_cur, 7);
-    W(wa, a_cur, 3);
+    T(total_a, a_cur, 9);
+    E(a_cur, 11, shift_a);
+    T(total_a, a_cur, 10);
+    W(wa, a_cur, 4);
     __builtin_amdgcn_sched_barrier(0);
     // slot 8
     QK(b_nxt, qb, 0);
-    if constexpr (LOADS) issue(0);
-    E(a_cur, 8, shift_a);
-    T(total_a, a_cur, 8);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 9
-    QK(b_nxt, qb, 1);
-    if constexpr (LOADS) issue(1);
-    E(a_cur, 9, shift_a);
-    T(total_a, a_cur, 9);
-    W(wa, a_cur, 4);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 10
-    QK(b_nxt, qb, 2);
-    if constexpr (LOADS) issue(2);
-    E(a_cur, 10, shift_a);
-    T(total_a, a_cur, 10);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 11
-    QK(b_nxt, qb, 3);
-    if constexpr (LOADS) issue(3);
-    E(a_cur, 11, shift_a);
+    VR(0, 0);
+    E(a_cur, 12, shift_a);
     T(total_a, a_cur, 11);
     W(wa, a_cur, 5);
     __builtin_amdgcn_sched_barrier(0);
-    // slot 12
-    QK(b_nxt, qb, 4);
-    if constexpr (LOADS) issue(4);
-    E(a_cur, 12, shift_a);
+    // slot 9
+    QK(b_nxt, qb, 1);
+    VR(0, 1);
+    E(a_cur, 13, shift_a);
     T(total_a, a_cur, 12);
     __builtin_amdgcn_sched_barrier(0);
-    // slot 13
-    QK(b_nxt, qb, 5);
-    if constexpr (LOADS) issue(5);
-    E(a_cur, 13, shift_a);
+    // slot 10
+    QK(b_nxt, qb, 2);
+    VR(0, 2);
+    E(a_cur, 14, shift_a);
     T(total_a, a_cur, 13);
     W(wa, a_cur, 6);
     __builtin_amdgcn_sched_barrier(0);
+    // slot 11
+    QK(b_nxt, qb, 3);
+    VR(0, 3);
+    E(a_cur, 15, shift_a);
+    T(total_a, a_cur, 14);
+    __builtin_amdgcn_sched_barrier(0);
+    // slot 12
+    QK(b_nxt, qb, 4);
+    VR(1, 0);
+    T(total_a, a_cur, 15);
+    W(wa, a_cur, 7);
+    E(b_cur, 0, shift_b);
+    __builtin_amdgcn_sched_barrier(0);
+    // slot 13
+    QK(b_nxt, qb, 5);
+    VR(1, 1);
+    E(b_cur, 1, shift_b);
+    T(total_b, b_cur, 0);
+    __builtin_amdgcn_sched_barrier(0);
     // slot 14
     QK(b_nxt, qb, 6);
-    if constexpr (LOADS) issue(6);
-    E(a_cur, 14, shift_a);
-    T(total_a, a_cur, 14);
+    VR(1, 2);
+    E(b_cur, 2, shift_b);
+    T(total_b, b_cur, 1);
+    W(wb, b_cur, 0);
     __builtin_amdgcn_sched_barrier(0);
     // slot 15
     QK(b_nxt, qb, 7);
-    if constexpr (LOADS) issue(7);
-    E(a_cur, 15, shift_a);
-    T(total_a, a_cur, 15);
-    W(wa, a_cur, 7);
+    VR(1, 3);
+    E(b_cur, 3, shift_b);
+    T(total_b, b_cur, 2);
     __builtin_amdgcn_sched_barrier(0);
     // slot 16
     PV(A, 0, 0, wa);
+    if constexpr (LOADS) issue(0);
     KR(0);
-    E(b_cur, 0, shift_b);
-    E(b_cur, 1, shift_b);
+    E(b_cur, 4, shift_b);
+    T(total_b, b_cur, 3);
     __builtin_amdgcn_sched_barrier(0);
     // slot 17
     PV(A, 0, 1, wa);
+    if constexpr (LOADS) issue(1);
     KR(1);
-    T(total_b, b_cur, 0);
-    E(b_cur, 2, shift_b);
-    T(total_b, b_cur, 1);
-    T(total_b, b_cur, 2);
+    E(b_cur, 5, shift_b);
+    T(total_b, b_cur, 4);
     __builtin_amdgcn_sched_barrier(0);
     // slot 18
     PV(A, 0, 2, wa);
+    if constexpr (LOADS) issue(2);
     KR(2);
-    E(b_cur, 3, shift_b);
-    W(wb, b_cur, 0);
-    T(total_b, b_cur, 3);
     W(wb, b_cur, 1);
+    E(b_cur, 6, shift_b);
     __builtin_amdgcn_sched_barrier(0);
     // slot 19
     PV(A, 0, 3, wa);
+    if constexpr (LOADS) issue(3);
     KR(3);
-    E(b_cur, 4, shift_b);
-    E(b_cur, 5, shift_b);
+    T(total_b, b_cur, 5);
+    E(b_cur, 7, shift_b);
     __builtin_amdgcn_sched_barrier(0);
     // slot 20
     PV(A, 1, 0, wa);
+    if constexpr (LOADS) issue(4);
     KR(4);
-    T(total_b, b_cur, 4);
-    E(b_cur, 6, shift_b);
-    T(total_b, b_cur, 5);
     T(total_b, b_cur, 6);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 21
-    PV(A, 1, 1, wa);
-    KR(5);
-    E(b_cur, 7, shift_b);
     W(wb, b_cur, 2);
     T(total_b, b_cur, 7);
     W(wb, b_cur, 3);
     __builtin_amdgcn_sched_barrier(0);
+    // slot 21
+    PV(A, 1, 1, wa);
+    if constexpr (LOADS) issue(5);
+    KR(5);
+    E(b_cur, 8, shift_b);
+    __builtin_amdgcn_sched_barrier(0);
     // slot 22
     PV(A, 1, 2, wa);
+    if constexpr (LOADS) issue(6);
     KR(6);
-    E(b_cur, 8, shift_b);
     E(b_cur, 9, shift_b);
+    T(total_b, b_cur, 8);
     __builtin_amdgcn_sched_barrier(0);
     // slot 23
     PV(A, 1, 3, wa);
+    if constexpr (LOADS) issue(7);
     KR(7);
-    T(total_b, b_cur, 8);
     E(b_cur, 10, shift_b);
     T(total_b, b_cur, 9);
-    T(total_b, b_cur, 10);
     __builtin_amdgcn_sched_barrier(0);
     // slot 24
     PV(B, 0, 0, wb);
     E(b_cur, 11, shift_b);
+    T(total_b, b_cur, 10);
     W(wb, b_cur, 4);
-    E(b_cur, 12, shift_b);
     __builtin_amdgcn_sched_barrier(0);
     // slot 25
     PV(B, 0, 1, wb);
+    E(b_cur, 12, shift_b);
     T(total_b, b_cur, 11);
     E(b_cur, 13, shift_b);
-    T(total_b, b_cur, 12);
-    W(wb, b_cur, 5);
-    T(total_b, b_cur, 13);
     __builtin_amdgcn_sched_barrier(0);
     // slot 26
     PV(B, 0, 2, wb);
+    T(total_b, b_cur, 12);
+    W(wb, b_cur, 5);
     E(b_cur, 14, shift_b);
-    E(b_cur, 15, shift_b);
-    T(total_b, b_cur, 14);
+    T(total_b, b_cur, 13);
+    W(wb, b_cur, 6);
     __builtin_amdgcn_sched_barrier(0);
     // slot 27
     PV(B, 0, 3, wb);
-    W(wb, b_cur, 6);
-    T(total_b, b_cur, 15);
-    W(wb, b_cur, 7);
-    float largest_a = max3(a_nxt[0], a_nxt[1], a_nxt[2]), largest_a_ = max3(a_nxt[3], a_nxt[4], a_nxt[5]); largest_a = max3(largest_a, a_nxt[6], a_nxt[7]);
+    E(b_cur, 15, shift_b);
+    T(total_b, b_cur, 14);
     __builtin_amdgcn_sched_barrier(0);
     // slot 28
+    W(wb, b_cur, 7);
     PV(B, 1, 0, wb);
-    largest_a_ = max3(largest_a_, a_nxt[8], a_nxt[9]); largest_a = max3(largest_a, a_nxt[10], a_nxt[11]); largest_a_ = max3(largest_a_, a_nxt[12], a_nxt[13]);
-    float largest_b = max3(b_nxt[0], b_nxt[1], b_nxt[2]), largest_b_ = max3(b_nxt[3], b_nxt[4], b_nxt[5]); largest_b = max3(largest_b, b_nxt[6], b_nxt[7]);
+    T(total_b, b_cur, 15);
+    ROW_MAXIMA_0;
     __builtin_amdgcn_sched_barrier(0);
     // slot 29
     PV(B, 1, 1, wb);
-    largest_a = max3(largest_a, a_nxt[14], a_nxt[15]); largest_a = swap32_max(max2(largest_a, largest_a_)) * factor;
+    ROW_MAXIMA_1;
     __builtin_amdgcn_sched_barrier(0);
     // slot 30
     PV(B, 1, 2, wb);
-    largest_b_ = max3(largest_b_, b_nxt[8], b_nxt[9]); largest_b = max3(largest_b, b_nxt[10], b_nxt[11]); largest_b_ = max3(largest_b_, b_nxt[12], b_nxt[13]);
+    ROW_MAXIMA_2;
     __builtin_amdgcn_sched_barrier(0);
     // slot 31
     PV(B, 1, 3, wb);
-    largest_b = max3(largest_b, b_nxt[14], b_nxt[15]); largest_b = swap32_max(max2(largest_b, largest_b_)) * factor;
     __builtin_amdgcn_sched_barrier(0);
 #undef QK
 #undef PV
@@ -321,11 +352,14 @@ SINGE_DEVICE void fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t&
 #undef T
 #undef W
 #undef KR
+#undef ROW_MAXIMA_0
+#undef ROW_MAXIMA_1
+#undef ROW_MAXIMA_2
 #undef VR
     A.running_sum += total_a;
     B.running_sum += total_b;
-    largest_a_out = largest_a;
-    largest_b_out = largest_b;
+    largest_a_out = largest_a * factor;
+    largest_b_out = largest_b * factor;
 }
 
 // One 256-row query tile of (batch, head) pair `bh`.
@@ -422,6 +456,11 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
     if (interior_tiles > 0) {
         uint4 operand[kSteps];
         read_key_operands(operand, lds + kBlockBytes, offsets);
+        // (the V stages start at an offset the compiler must not know, or it folds it into the reads' immediates,
+        // which it then overflows)
+        unsigned int value_base = kPairValueBase;
+        asm volatile("" : "+s"(value_base));
+        const unsigned char* value_origin = lds + value_base;
         float shift_a = begin_block(A, a_even, hi, factor, false, [](unsigned int) { return false; });
         float shift_b = begin_block(B, b_even, hi, factor, false, [](unsigned int) { return false; });
         auto settle = [&](float largest_a, float largest_b) __attribute__((always_inline)) {
@@ -432,13 +471,15 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
             shift_a = A.reference == -INFINITY ? 0.0f : -A.reference;
             shift_b = B.reference == -INFINITY ? 0.0f : -B.reference;
         };
-        for (; tile < interior_tiles; ++tile) {
-            const unsigned int next_stage = stage + 1 == kPairStages ? 0 : stage + 1;
-            const unsigned int spare_stage = next_stage + 1 == kPairStages ? 0 : next_stage + 1;
-            const unsigned char* __restrict__ next_keys = lds + next_stage * kTileBytes;
-            const unsigned char* __restrict__ values = lds + kPairValueBase + stage * kTileBytes;
-            unsigned char* __restrict__ key_dest = lds + spare_stage * kTileBytes;
-            unsigned char* __restrict__ value_dest = lds + kPairValueBase + spare_stage * kTileBytes;
+        // One tile, its stage a constant: the loop below is written out once per stage, so that every LDS address of
+        // the schedule is a register that never changes plus an immediate offset.
+        auto fold_tile = [&](auto stage_constant) __attribute__((always_inline)) {
+            constexpr unsigned int kStage = decltype(stage_constant)::value;
+            constexpr unsigned int kNextStage = (kStage + 1) % kPairStages, kSpareStage = (kStage + 2) % kPairStages;
+            const unsigned char* __restrict__ next_keys = lds + kNextStage * kTileBytes;
+            constexpr unsigned int values = kStage * kTileBytes;
+            unsigned char* __restrict__ key_dest = lds + kSpareStage * kTileBytes;
+            unsigned char* __restrict__ value_dest = lds + kPairValueBase + kSpareStage * kTileBytes;
             // The tile two ahead, or (nobody reads it) the last one again when there is none.
             const unsigned int wanted = tile + 2 < tiles ? tile + 2 : tiles - 1;
             const unsigned char* key_rows = tile_base(k_bytes, key_stride_bytes, wanted);
@@ -449,16 +490,26 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
             };
             float largest_a, largest_b;
             fold_pair_block<true>(half, A, B, a_even, b_even, a_odd, b_odd, factor, shift_a, shift_b, largest_a, largest_b, qa, qb, operand,
-                                  next_keys, values, offsets, issue);
+                                  next_keys, value_origin, values, offsets, issue);
             settle(largest_a, largest_b);
             fold_pair_block<false>(half, A, B, a_odd, b_odd, a_even, b_even, factor, shift_a, shift_b, largest_a, largest_b, qa, qb, operand,
-                                   next_keys + kBlockBytes, values + kBlockBytes, offsets, issue);
+                                   next_keys + kBlockBytes, value_origin, values + kBlockBytes, offsets, issue);
             // (past the wave's last unmasked tile the scores just computed are the diagonal tile's, which the masked path
             // takes as they are, or nobody's)
             if (tile + 1 < interior_tiles) settle(largest_a, largest_b);
             loads_landed();
             __syncthreads();
-            stage = next_stage;
+        };
+        while (tile < interior_tiles) {
+            fold_tile(std::integral_constant<unsigned int, 0>{});
+            stage = 1;
+            if (++tile >= interior_tiles) break;
+            fold_tile(std::integral_constant<unsigned int, 1>{});
+            stage = 2;
+            if (++tile >= interior_tiles) break;
+            fold_tile(std::integral_constant<unsigned int, 2>{});
+            stage = 0;
+            ++tile;
         }
     }
     // The tile on the diagonal: block 2 t holds the keys of tile A's rows (B sees all of it), block 2 t + 1 those of
@@ -524,8 +575,11 @@ SINGE_DEVICE void fmha_prefill_pair_body(const PrefillArgs& a, unsigned char* ld
     const unsigned int bh = (within / pairs) * 8u + xcd;
     if (bh >= a.batch * a.heads) return;
     const unsigned int light = within % pairs, heavy = a.query_tiles - 1u - light;
-    fmha_prefill_pair_tile<CAUSAL, Half>(a, lds, bh, heavy);
-    if (light != heavy) fmha_prefill_pair_tile<CAUSAL, Half>(a, lds, bh, light);
+    // (one copy of the tile's code for both tiles: written out per stage it is long, and two copies of it would not fit
+    // the instruction cache)
+#pragma nounroll
+    for (unsigned int which = 0; which < (light != heavy ? 2u : 1u); ++which)
+        fmha_prefill_pair_tile<CAUSAL, Half>(a, lds, bh, which == 0 ? heavy : light);
 }
 
 }  // namespace
