@@ -22,8 +22,9 @@
 // fmha_prefill.hip.
 //
 // Grid: one workgroup of four waves per (batch, head, pair of 256-row query tiles), tile i from the end and tile i
-// from the start; ids laid out as in fmha_prefill.hip.  LDS: three stages of K and three of V (96 KiB), each tile
-// loaded two tiles ahead, straight from global memory, one barrier per tile.
+// from the start; ids laid out as in fmha_prefill.hip.  LDS: four stages of K and four of V (128 KiB), each tile
+// loaded three tiles ahead, straight from global memory, and waited for a tile after it was asked for (a wave alone
+// on its SIMD has nobody to cover a wait for fresh loads); one barrier per tile.
 #include "kernel_args.h"
 #include "prefill_blocks.hip.h"
 
@@ -34,7 +35,8 @@ static_assert(kHeadDim == 128, "the two-tile kernel is built for head_dim 128");
 
 constexpr int kPairWaves = 4;
 constexpr unsigned int kPairRows = 64u * kPairWaves;  // query rows of a workgroup
-constexpr int kPairStages = 3;
+constexpr int kPairStages = 4;                        // of K and of V: a tile is loaded three tiles ahead
+constexpr int kPairAhead = kPairStages - 1;
 constexpr int kPairValueBase = kPairStages * kTileBytes;
 constexpr int kPairLdsBytes = 2 * kPairStages * kTileBytes;
 
@@ -70,6 +72,8 @@ SINGE_DEVICE u32x4_t load_to_accumulation(const void* address) {
     asm volatile("global_load_dwordx4 %0, %1, off" : "=a"(loaded) : "v"(address) : "memory");
     return loaded;
 }
+// All of this wave's loads but the eight it issued last (a tile's: four of K, four of V) have completed.
+SINGE_DEVICE void older_loads_landed() { __builtin_amdgcn_s_waitcnt(0x0F78); }  // vmcnt(8), other counters left alone
 SINGE_DEVICE void accumulation_loads_landed() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 // The scores of a whole block outside the scheduled loop (the first block, the diagonal tile): the same products, then
@@ -441,14 +445,13 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
     reset(B);
     const ReadOffsets offsets = read_offsets(lane);
 
-    if (tiles > 0) load_tile(0, 0);
-    if (tiles > 1) load_tile(1, 1);
+    for (unsigned int early = 0; early < kPairAhead && early < tiles; ++early) load_tile(early, early);
     loads_landed();
     accumulation_loads_landed();
     __syncthreads();
 
     f32x16_t a_even, b_even, a_odd, b_odd;  // raw scores of the block folded next (even / odd blocks of a tile)
-    unsigned int tile = 0, stage = 0;       // stage = tile % 3
+    unsigned int tile = 0, stage = 0;       // stage = tile % 4
     if (interior_tiles > 0 || has_diagonal) {
         score_block_pair(half, a_even, qa, lds, offsets);
         score_block_pair(half, b_even, qb, lds, offsets);
@@ -475,13 +478,13 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
         // the schedule is a register that never changes plus an immediate offset.
         auto fold_tile = [&](auto stage_constant) __attribute__((always_inline)) {
             constexpr unsigned int kStage = decltype(stage_constant)::value;
-            constexpr unsigned int kNextStage = (kStage + 1) % kPairStages, kSpareStage = (kStage + 2) % kPairStages;
+            constexpr unsigned int kNextStage = (kStage + 1) % kPairStages, kSpareStage = (kStage + kPairAhead) % kPairStages;
             const unsigned char* __restrict__ next_keys = lds + kNextStage * kTileBytes;
             constexpr unsigned int values = kStage * kTileBytes;
             unsigned char* __restrict__ key_dest = lds + kSpareStage * kTileBytes;
             unsigned char* __restrict__ value_dest = lds + kPairValueBase + kSpareStage * kTileBytes;
-            // The tile two ahead, or (nobody reads it) the last one again when there is none.
-            const unsigned int wanted = tile + 2 < tiles ? tile + 2 : tiles - 1;
+            // The tile three ahead, or (nobody reads it) the last one again when there is none.
+            const unsigned int wanted = tile + kPairAhead < tiles ? tile + kPairAhead : tiles - 1;
             const unsigned char* key_rows = tile_base(k_bytes, key_stride_bytes, wanted);
             const unsigned char* value_rows = tile_base(v_bytes, value_stride_bytes, wanted);
             auto issue = [&](unsigned int i) __attribute__((always_inline)) {
@@ -497,7 +500,7 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
             // (past the wave's last unmasked tile the scores just computed are the diagonal tile's, which the masked path
             // takes as they are, or nobody's)
             if (tile + 1 < interior_tiles) settle(largest_a, largest_b);
-            loads_landed();
+            older_loads_landed();  // the next tile's; the eight of this iteration have another tile's time
             __syncthreads();
         };
         while (tile < interior_tiles) {
@@ -508,6 +511,9 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
             stage = 2;
             if (++tile >= interior_tiles) break;
             fold_tile(std::integral_constant<unsigned int, 2>{});
+            stage = 3;
+            if (++tile >= interior_tiles) break;
+            fold_tile(std::integral_constant<unsigned int, 3>{});
             stage = 0;
             ++tile;
         }
@@ -515,11 +521,11 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
     // The tile on the diagonal: block 2 t holds the keys of tile A's rows (B sees all of it), block 2 t + 1 those of
     // tile B's rows (A sees none of it).
     if (has_diagonal) {
-        const unsigned int next_stage = stage + 1 == kPairStages ? 0 : stage + 1;
-        const unsigned int spare_stage = next_stage + 1 == kPairStages ? 0 : next_stage + 1;
+        const unsigned int next_stage = (stage + 1) % kPairStages, spare_stage = (stage + kPairAhead) % kPairStages;
         const unsigned char* keys = lds + stage * kTileBytes;
         const unsigned char* values = lds + kPairValueBase + stage * kTileBytes;
-        if (tile + 2 < tiles) load_tile(tile + 2, spare_stage);
+        const bool loading = tile + kPairAhead < tiles;
+        if (loading) load_tile(tile + kPairAhead, spare_stage);
         const unsigned int key0 = tile * kKeyTile;
         const float edge_a = begin_block(A, a_even, hi, factor, true, [&](unsigned int key_in_block) { return key0 + key_in_block > query_a; });
         finish_block<false>(half, A, a_even, factor, edge_a, values, offsets, a_even, no_query, values);
@@ -528,17 +534,17 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
         score_block_pair(half, b_odd, qb, keys + kBlockBytes, offsets);
         const float edge_b = begin_block(B, b_odd, hi, factor, true, [&](unsigned int key_in_block) { return key0 + 32u + key_in_block > query_b; });
         finish_block<false>(half, B, b_odd, factor, edge_b, values + kBlockBytes, offsets, b_odd, no_query, values);
-        loads_landed();
+        if (loading) older_loads_landed(); else loads_landed();
         __syncthreads();
         stage = next_stage;
         ++tile;
     }
     // The tiles the waves with later rows still work on: this wave's share of their loads, and their barriers.
     for (; tile < tiles; ++tile) {
-        const unsigned int next_stage = stage + 1 == kPairStages ? 0 : stage + 1;
-        const unsigned int spare_stage = next_stage + 1 == kPairStages ? 0 : next_stage + 1;
-        if (tile + 2 < tiles) load_tile(tile + 2, spare_stage);
-        loads_landed();
+        const unsigned int next_stage = (stage + 1) % kPairStages, spare_stage = (stage + kPairAhead) % kPairStages;
+        const bool loading = tile + kPairAhead < tiles;
+        if (loading) load_tile(tile + kPairAhead, spare_stage);
+        if (loading) older_loads_landed(); else loads_landed();
         __syncthreads();
         stage = next_stage;
     }
