@@ -118,12 +118,14 @@ SINGE_DEVICE void row_maxima_2(float& ma, float& mb) {
 // minus the rows' reference points, which already cover them) and `operand` the K operands of block b + 1; the V^T
 // operands of block b are read in the block's first half, from value_origin (the first V stage, kept where the
 // compiler cannot fold its address into the offset) + the lane's offsets + `values` (the block's byte offset from
-// there, a constant once inlined: together with the stage's own address it would not fit the instruction's 16 bits).  On return a_nxt / b_nxt hold the raw scores
-// of block b + 1 and largest_a / largest_b their scaled row maxima, `operand` the K operands of block b + 2 (read
-// from keys_after); the rows' sums and O^T have taken block b in.  With LOADS, issue(0 .. 7) is
-// called once each (the tile's eight direct-to-LDS loads of this wave).
-template <bool LOADS, class Half, class Issue>
-SINGE_DEVICE void fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t& a_cur, f32x16_t& b_cur, f32x16_t& a_nxt, f32x16_t& b_nxt,
+// there, a constant once inlined: together with the stage's own address it would not fit the instruction's 16 bits).
+// On return a_nxt / b_nxt hold the raw scores of block b + 1 and largest_a / largest_b their scaled row maxima,
+// `operand` the K operands of block b + 2 (read from keys_after); the rows' sums and O^T have taken block b in; the
+// return value says whether some row's maximum has run too far ahead of its reference point (the test is part of the
+// schedule; moving the references, which is rare, is the caller's).  issue(0 .. 3) is called once each (four of
+// the tile's eight direct-to-LDS loads of this wave).
+template <class Half, class Issue>
+SINGE_DEVICE bool fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t& a_cur, f32x16_t& b_cur, f32x16_t& a_nxt, f32x16_t& b_nxt,
                                   float factor, float shift_a, float shift_b, float& largest_a_out, float& largest_b_out,
                                   const u32x4_t (&qa)[8], const u32x4_t (&qb)[8], uint4 (&operand)[8], const unsigned char* __restrict__ keys_after,
                                   const unsigned char* __restrict__ value_origin, unsigned int values, const ReadOffsets& offsets, Issue&& issue) {
@@ -131,15 +133,22 @@ SINGE_DEVICE void fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t&
     v8i16_t v[2][4];
     float total_a = 0.0f, total_b = 0.0f;
     float largest_a, other_a, largest_b, other_b;
+    bool lagging;
 #define QK(S, Q, J) score_step<(J) == 0, true, Half>(S, operand[J], Q[J])
 #define PV(X, H, D, WORDS) \
     X.out[D] = mma(half, __builtin_bit_cast(uint4, v[H][D]), make_uint4(WORDS[H][0], WORDS[H][1], WORDS[H][2], WORDS[H][3]), X.out[D])
 #define E(S, I, SHIFT) S[I] = fast_exp2(fmaf(S[I], factor, SHIFT))
-#define T(TOTAL, S, I) TOTAL += S[I]
+// (as a statement the compiler must keep in its place: a plain addition, whose result nothing needs before the block's
+// end, is collected with all the others behind the last matrix instruction)
+#define T(TOTAL, S, I) asm volatile("v_add_f32_e32 %0, %1, %0" : "+v"(TOTAL) : "v"(S[I]))
 #define W(WORDS, S, I) WORDS[(I) / 4][(I) % 4] = pack_pair(half, S[2 * (I)], S[2 * (I) + 1])
 #define ROW_MAXIMA_0 row_maxima_0(a_nxt, b_nxt, largest_a, other_a, largest_b, other_b)
 #define ROW_MAXIMA_1 row_maxima_1(a_nxt, b_nxt, largest_a, other_a, largest_b, other_b)
 #define ROW_MAXIMA_2 row_maxima_2(largest_a, largest_b)
+#define LAG_TEST                             \
+    largest_a *= factor;                     \
+    largest_b *= factor;                     \
+    lagging = __any(reference_lags(A, largest_a) || reference_lags(B, largest_b))
 #define KR(J) operand[J] = *reinterpret_cast<const uint4*>(keys_after + offsets.key(J))
 #define VR(H, D)                                                                                                                        \
     {                                                                                                                                   \
@@ -149,206 +158,235 @@ SINGE_DEVICE void fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t&
     }
     // slot 0
     QK(a_nxt, qa, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    issue(0);
     E(a_cur, 0, shift_a);
-    E(a_cur, 1, shift_a);
     __builtin_amdgcn_sched_barrier(0);
     // slot 1
     QK(a_nxt, qa, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    E(a_cur, 1, shift_a);
     T(total_a, a_cur, 0);
     E(a_cur, 2, shift_a);
-    T(total_a, a_cur, 1);
-    W(wa, a_cur, 0);
     __builtin_amdgcn_sched_barrier(0);
     // slot 2
     QK(a_nxt, qa, 2);
+    __builtin_amdgcn_sched_barrier(0);
+    issue(1);
+    T(total_a, a_cur, 1);
     E(a_cur, 3, shift_a);
-    T(total_a, a_cur, 2);
-    E(a_cur, 4, shift_a);
     __builtin_amdgcn_sched_barrier(0);
     // slot 3
     QK(a_nxt, qa, 3);
+    __builtin_amdgcn_sched_barrier(0);
+    T(total_a, a_cur, 2);
+    W(wa, a_cur, 0);
+    E(a_cur, 4, shift_a);
     T(total_a, a_cur, 3);
-    E(a_cur, 5, shift_a);
-    T(total_a, a_cur, 4);
     W(wa, a_cur, 1);
     __builtin_amdgcn_sched_barrier(0);
     // slot 4
     QK(a_nxt, qa, 4);
+    __builtin_amdgcn_sched_barrier(0);
+    issue(2);
+    E(a_cur, 5, shift_a);
+    T(total_a, a_cur, 4);
+    __builtin_amdgcn_sched_barrier(0);
+    // slot 5
+    QK(a_nxt, qa, 5);
+    __builtin_amdgcn_sched_barrier(0);
     E(a_cur, 6, shift_a);
     T(total_a, a_cur, 5);
     E(a_cur, 7, shift_a);
     __builtin_amdgcn_sched_barrier(0);
-    // slot 5
-    QK(a_nxt, qa, 5);
+    // slot 6
+    QK(a_nxt, qa, 6);
+    __builtin_amdgcn_sched_barrier(0);
+    issue(3);
     T(total_a, a_cur, 6);
     W(wa, a_cur, 2);
     T(total_a, a_cur, 7);
     W(wa, a_cur, 3);
-    E(a_cur, 8, shift_a);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 6
-    QK(a_nxt, qa, 6);
-    E(a_cur, 9, shift_a);
-    T(total_a, a_cur, 8);
-    E(a_cur, 10, shift_a);
     __builtin_amdgcn_sched_barrier(0);
     // slot 7
     QK(a_nxt, qa, 7);
+    __builtin_amdgcn_sched_barrier(0);
+    E(a_cur, 8, shift_a);
+    E(a_cur, 9, shift_a);
+    __builtin_amdgcn_sched_barrier(0);
+    // slot 8
+    QK(b_nxt, qb, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    VR(0, 0);
+    T(total_a, a_cur, 8);
+    E(a_cur, 10, shift_a);
     T(total_a, a_cur, 9);
+    __builtin_amdgcn_sched_barrier(0);
+    // slot 9
+    QK(b_nxt, qb, 1);
+    __builtin_amdgcn_sched_barrier(0);
+    VR(0, 1);
     E(a_cur, 11, shift_a);
     T(total_a, a_cur, 10);
     W(wa, a_cur, 4);
     __builtin_amdgcn_sched_barrier(0);
-    // slot 8
-    QK(b_nxt, qb, 0);
-    VR(0, 0);
+    // slot 10
+    QK(b_nxt, qb, 2);
+    __builtin_amdgcn_sched_barrier(0);
+    VR(0, 2);
     E(a_cur, 12, shift_a);
     T(total_a, a_cur, 11);
     W(wa, a_cur, 5);
     __builtin_amdgcn_sched_barrier(0);
-    // slot 9
-    QK(b_nxt, qb, 1);
-    VR(0, 1);
+    // slot 11
+    QK(b_nxt, qb, 3);
+    __builtin_amdgcn_sched_barrier(0);
+    VR(0, 3);
     E(a_cur, 13, shift_a);
     T(total_a, a_cur, 12);
     __builtin_amdgcn_sched_barrier(0);
-    // slot 10
-    QK(b_nxt, qb, 2);
-    VR(0, 2);
+    // slot 12
+    QK(b_nxt, qb, 4);
+    __builtin_amdgcn_sched_barrier(0);
+    VR(1, 0);
     E(a_cur, 14, shift_a);
     T(total_a, a_cur, 13);
     W(wa, a_cur, 6);
     __builtin_amdgcn_sched_barrier(0);
-    // slot 11
-    QK(b_nxt, qb, 3);
-    VR(0, 3);
+    // slot 13
+    QK(b_nxt, qb, 5);
+    __builtin_amdgcn_sched_barrier(0);
+    VR(1, 1);
     E(a_cur, 15, shift_a);
     T(total_a, a_cur, 14);
     __builtin_amdgcn_sched_barrier(0);
-    // slot 12
-    QK(b_nxt, qb, 4);
-    VR(1, 0);
+    // slot 14
+    QK(b_nxt, qb, 6);
+    __builtin_amdgcn_sched_barrier(0);
+    VR(1, 2);
     T(total_a, a_cur, 15);
     W(wa, a_cur, 7);
     E(b_cur, 0, shift_b);
     __builtin_amdgcn_sched_barrier(0);
-    // slot 13
-    QK(b_nxt, qb, 5);
-    VR(1, 1);
+    // slot 15
+    QK(b_nxt, qb, 7);
+    __builtin_amdgcn_sched_barrier(0);
+    VR(1, 3);
     E(b_cur, 1, shift_b);
     T(total_b, b_cur, 0);
     __builtin_amdgcn_sched_barrier(0);
-    // slot 14
-    QK(b_nxt, qb, 6);
-    VR(1, 2);
+    // slot 16
+    PV(A, 0, 0, wa);
+    __builtin_amdgcn_sched_barrier(0);
+    KR(0);
     E(b_cur, 2, shift_b);
     T(total_b, b_cur, 1);
     W(wb, b_cur, 0);
     __builtin_amdgcn_sched_barrier(0);
-    // slot 15
-    QK(b_nxt, qb, 7);
-    VR(1, 3);
+    // slot 17
+    PV(A, 0, 1, wa);
+    __builtin_amdgcn_sched_barrier(0);
+    KR(1);
     E(b_cur, 3, shift_b);
     T(total_b, b_cur, 2);
     __builtin_amdgcn_sched_barrier(0);
-    // slot 16
-    PV(A, 0, 0, wa);
-    if constexpr (LOADS) issue(0);
-    KR(0);
-    E(b_cur, 4, shift_b);
-    T(total_b, b_cur, 3);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 17
-    PV(A, 0, 1, wa);
-    if constexpr (LOADS) issue(1);
-    KR(1);
-    E(b_cur, 5, shift_b);
-    T(total_b, b_cur, 4);
-    __builtin_amdgcn_sched_barrier(0);
     // slot 18
     PV(A, 0, 2, wa);
-    if constexpr (LOADS) issue(2);
+    __builtin_amdgcn_sched_barrier(0);
     KR(2);
+    E(b_cur, 4, shift_b);
+    T(total_b, b_cur, 3);
     W(wb, b_cur, 1);
-    E(b_cur, 6, shift_b);
     __builtin_amdgcn_sched_barrier(0);
     // slot 19
     PV(A, 0, 3, wa);
-    if constexpr (LOADS) issue(3);
+    __builtin_amdgcn_sched_barrier(0);
     KR(3);
-    T(total_b, b_cur, 5);
-    E(b_cur, 7, shift_b);
+    E(b_cur, 5, shift_b);
+    T(total_b, b_cur, 4);
     __builtin_amdgcn_sched_barrier(0);
     // slot 20
     PV(A, 1, 0, wa);
-    if constexpr (LOADS) issue(4);
+    __builtin_amdgcn_sched_barrier(0);
     KR(4);
-    T(total_b, b_cur, 6);
+    E(b_cur, 6, shift_b);
+    T(total_b, b_cur, 5);
     W(wb, b_cur, 2);
-    T(total_b, b_cur, 7);
-    W(wb, b_cur, 3);
     __builtin_amdgcn_sched_barrier(0);
     // slot 21
     PV(A, 1, 1, wa);
-    if constexpr (LOADS) issue(5);
+    __builtin_amdgcn_sched_barrier(0);
     KR(5);
-    E(b_cur, 8, shift_b);
+    E(b_cur, 7, shift_b);
+    T(total_b, b_cur, 6);
     __builtin_amdgcn_sched_barrier(0);
     // slot 22
     PV(A, 1, 2, wa);
-    if constexpr (LOADS) issue(6);
+    __builtin_amdgcn_sched_barrier(0);
     KR(6);
-    E(b_cur, 9, shift_b);
-    T(total_b, b_cur, 8);
+    T(total_b, b_cur, 7);
+    W(wb, b_cur, 3);
+    E(b_cur, 8, shift_b);
     __builtin_amdgcn_sched_barrier(0);
     // slot 23
     PV(A, 1, 3, wa);
-    if constexpr (LOADS) issue(7);
+    __builtin_amdgcn_sched_barrier(0);
     KR(7);
-    E(b_cur, 10, shift_b);
-    T(total_b, b_cur, 9);
+    E(b_cur, 9, shift_b);
+    T(total_b, b_cur, 8);
     __builtin_amdgcn_sched_barrier(0);
     // slot 24
     PV(B, 0, 0, wb);
+    __builtin_amdgcn_sched_barrier(0);
+    E(b_cur, 10, shift_b);
+    T(total_b, b_cur, 9);
     E(b_cur, 11, shift_b);
-    T(total_b, b_cur, 10);
-    W(wb, b_cur, 4);
     __builtin_amdgcn_sched_barrier(0);
     // slot 25
     PV(B, 0, 1, wb);
+    __builtin_amdgcn_sched_barrier(0);
+    T(total_b, b_cur, 10);
+    W(wb, b_cur, 4);
     E(b_cur, 12, shift_b);
     T(total_b, b_cur, 11);
-    E(b_cur, 13, shift_b);
+    W(wb, b_cur, 5);
     __builtin_amdgcn_sched_barrier(0);
     // slot 26
     PV(B, 0, 2, wb);
+    __builtin_amdgcn_sched_barrier(0);
+    E(b_cur, 13, shift_b);
     T(total_b, b_cur, 12);
-    W(wb, b_cur, 5);
     E(b_cur, 14, shift_b);
-    T(total_b, b_cur, 13);
-    W(wb, b_cur, 6);
     __builtin_amdgcn_sched_barrier(0);
     // slot 27
     PV(B, 0, 3, wb);
+    __builtin_amdgcn_sched_barrier(0);
+    T(total_b, b_cur, 13);
     E(b_cur, 15, shift_b);
     T(total_b, b_cur, 14);
+    W(wb, b_cur, 6);
     __builtin_amdgcn_sched_barrier(0);
     // slot 28
     W(wb, b_cur, 7);
     PV(B, 1, 0, wb);
-    T(total_b, b_cur, 15);
+    __builtin_amdgcn_sched_barrier(0);
     ROW_MAXIMA_0;
     __builtin_amdgcn_sched_barrier(0);
     // slot 29
     PV(B, 1, 1, wb);
+    __builtin_amdgcn_sched_barrier(0);
     ROW_MAXIMA_1;
     __builtin_amdgcn_sched_barrier(0);
     // slot 30
     PV(B, 1, 2, wb);
+    __builtin_amdgcn_sched_barrier(0);
     ROW_MAXIMA_2;
     __builtin_amdgcn_sched_barrier(0);
     // slot 31
     PV(B, 1, 3, wb);
+    __builtin_amdgcn_sched_barrier(0);
+    LAG_TEST;
+    T(total_b, b_cur, 15);
     __builtin_amdgcn_sched_barrier(0);
 #undef QK
 #undef PV
@@ -359,11 +397,13 @@ SINGE_DEVICE void fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t&
 #undef ROW_MAXIMA_0
 #undef ROW_MAXIMA_1
 #undef ROW_MAXIMA_2
+#undef LAG_TEST
 #undef VR
     A.running_sum += total_a;
     B.running_sum += total_b;
-    largest_a_out = largest_a * factor;
-    largest_b_out = largest_b * factor;
+    largest_a_out = largest_a;
+    largest_b_out = largest_b;
+    return lagging;
 }
 
 // One 256-row query tile of (batch, head) pair `bh`.
@@ -467,10 +507,8 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
         float shift_a = begin_block(A, a_even, hi, factor, false, [](unsigned int) { return false; });
         float shift_b = begin_block(B, b_even, hi, factor, false, [](unsigned int) { return false; });
         auto settle = [&](float largest_a, float largest_b) __attribute__((always_inline)) {
-            if (__any(reference_lags(A, largest_a) || reference_lags(B, largest_b))) {
-                move_reference(A, largest_a);
-                move_reference(B, largest_b);
-            }
+            move_reference(A, largest_a);
+            move_reference(B, largest_b);
             shift_a = A.reference == -INFINITY ? 0.0f : -A.reference;
             shift_b = B.reference == -INFINITY ? 0.0f : -B.reference;
         };
@@ -487,19 +525,17 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
             const unsigned int wanted = tile + kPairAhead < tiles ? tile + kPairAhead : tiles - 1;
             const unsigned char* key_rows = tile_base(k_bytes, key_stride_bytes, wanted);
             const unsigned char* value_rows = tile_base(v_bytes, value_stride_bytes, wanted);
-            auto issue = [&](unsigned int i) __attribute__((always_inline)) {
-                if (i < 4) load_part(key_rows, key_stride_bytes, key_lane, i, key_dest);
-                else load_part(value_rows, value_stride_bytes, value_lane, i - 4, value_dest);
-            };
+            auto issue_keys = [&](unsigned int i) __attribute__((always_inline)) { load_part(key_rows, key_stride_bytes, key_lane, i, key_dest); };
+            auto issue_values = [&](unsigned int i) __attribute__((always_inline)) { load_part(value_rows, value_stride_bytes, value_lane, i, value_dest); };
             float largest_a, largest_b;
-            fold_pair_block<true>(half, A, B, a_even, b_even, a_odd, b_odd, factor, shift_a, shift_b, largest_a, largest_b, qa, qb, operand,
-                                  next_keys, value_origin, values, offsets, issue);
-            settle(largest_a, largest_b);
-            fold_pair_block<false>(half, A, B, a_odd, b_odd, a_even, b_even, factor, shift_a, shift_b, largest_a, largest_b, qa, qb, operand,
-                                   next_keys + kBlockBytes, value_origin, values + kBlockBytes, offsets, issue);
+            bool lagging = fold_pair_block(half, A, B, a_even, b_even, a_odd, b_odd, factor, shift_a, shift_b, largest_a, largest_b, qa, qb, operand,
+                                  next_keys, value_origin, values, offsets, issue_keys);
+            if (lagging) settle(largest_a, largest_b);
+            lagging = fold_pair_block(half, A, B, a_odd, b_odd, a_even, b_even, factor, shift_a, shift_b, largest_a, largest_b, qa, qb, operand,
+                                   next_keys + kBlockBytes, value_origin, values + kBlockBytes, offsets, issue_values);
             // (past the wave's last unmasked tile the scores just computed are the diagonal tile's, which the masked path
             // takes as they are, or nobody's)
-            if (tile + 1 < interior_tiles) settle(largest_a, largest_b);
+            if (lagging && tile + 1 < interior_tiles) settle(largest_a, largest_b);
             older_loads_landed();  // the next tile's; the eight of this iteration have another tile's time
             __syncthreads();
         };
