@@ -163,21 +163,21 @@ SINGE_DEVICE bool fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t&
     E(a_cur, 0, shift_a);
     __builtin_amdgcn_sched_barrier(0);
     // slot 1
-    QK(a_nxt, qa, 1);
+    QK(b_nxt, qb, 0);
     __builtin_amdgcn_sched_barrier(0);
     E(a_cur, 1, shift_a);
     T(total_a, a_cur, 0);
     E(a_cur, 2, shift_a);
     __builtin_amdgcn_sched_barrier(0);
     // slot 2
-    QK(a_nxt, qa, 2);
+    QK(a_nxt, qa, 1);
     __builtin_amdgcn_sched_barrier(0);
     issue(1);
     T(total_a, a_cur, 1);
     E(a_cur, 3, shift_a);
     __builtin_amdgcn_sched_barrier(0);
     // slot 3
-    QK(a_nxt, qa, 3);
+    QK(b_nxt, qb, 1);
     __builtin_amdgcn_sched_barrier(0);
     T(total_a, a_cur, 2);
     W(wa, a_cur, 0);
@@ -186,21 +186,21 @@ SINGE_DEVICE bool fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t&
     W(wa, a_cur, 1);
     __builtin_amdgcn_sched_barrier(0);
     // slot 4
-    QK(a_nxt, qa, 4);
+    QK(a_nxt, qa, 2);
     __builtin_amdgcn_sched_barrier(0);
     issue(2);
     E(a_cur, 5, shift_a);
     T(total_a, a_cur, 4);
     __builtin_amdgcn_sched_barrier(0);
     // slot 5
-    QK(a_nxt, qa, 5);
+    QK(b_nxt, qb, 2);
     __builtin_amdgcn_sched_barrier(0);
     E(a_cur, 6, shift_a);
     T(total_a, a_cur, 5);
     E(a_cur, 7, shift_a);
     __builtin_amdgcn_sched_barrier(0);
     // slot 6
-    QK(a_nxt, qa, 6);
+    QK(a_nxt, qa, 3);
     __builtin_amdgcn_sched_barrier(0);
     issue(3);
     T(total_a, a_cur, 6);
@@ -209,13 +209,13 @@ SINGE_DEVICE bool fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t&
     W(wa, a_cur, 3);
     __builtin_amdgcn_sched_barrier(0);
     // slot 7
-    QK(a_nxt, qa, 7);
+    QK(b_nxt, qb, 3);
     __builtin_amdgcn_sched_barrier(0);
     E(a_cur, 8, shift_a);
     E(a_cur, 9, shift_a);
     __builtin_amdgcn_sched_barrier(0);
     // slot 8
-    QK(b_nxt, qb, 0);
+    QK(a_nxt, qa, 4);
     __builtin_amdgcn_sched_barrier(0);
     VR(0, 0);
     T(total_a, a_cur, 8);
@@ -223,7 +223,7 @@ SINGE_DEVICE bool fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t&
     T(total_a, a_cur, 9);
     __builtin_amdgcn_sched_barrier(0);
     // slot 9
-    QK(b_nxt, qb, 1);
+    QK(b_nxt, qb, 4);
     __builtin_amdgcn_sched_barrier(0);
     VR(0, 1);
     E(a_cur, 11, shift_a);
@@ -231,7 +231,7 @@ SINGE_DEVICE bool fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t&
     W(wa, a_cur, 4);
     __builtin_amdgcn_sched_barrier(0);
     // slot 10
-    QK(b_nxt, qb, 2);
+    QK(a_nxt, qa, 5);
     __builtin_amdgcn_sched_barrier(0);
     VR(0, 2);
     E(a_cur, 12, shift_a);
@@ -239,14 +239,14 @@ SINGE_DEVICE bool fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t&
     W(wa, a_cur, 5);
     __builtin_amdgcn_sched_barrier(0);
     // slot 11
-    QK(b_nxt, qb, 3);
+    QK(b_nxt, qb, 5);
     __builtin_amdgcn_sched_barrier(0);
     VR(0, 3);
     E(a_cur, 13, shift_a);
     T(total_a, a_cur, 12);
     __builtin_amdgcn_sched_barrier(0);
     // slot 12
-    QK(b_nxt, qb, 4);
+    QK(a_nxt, qa, 6);
     __builtin_amdgcn_sched_barrier(0);
     VR(1, 0);
     E(a_cur, 14, shift_a);
@@ -254,14 +254,14 @@ SINGE_DEVICE bool fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t&
     W(wa, a_cur, 6);
     __builtin_amdgcn_sched_barrier(0);
     // slot 13
-    QK(b_nxt, qb, 5);
+    QK(b_nxt, qb, 6);
     __builtin_amdgcn_sched_barrier(0);
     VR(1, 1);
     E(a_cur, 15, shift_a);
     T(total_a, a_cur, 14);
     __builtin_amdgcn_sched_barrier(0);
     // slot 14
-    QK(b_nxt, qb, 6);
+    QK(a_nxt, qa, 7);
     __builtin_amdgcn_sched_barrier(0);
     VR(1, 2);
     T(total_a, a_cur, 15);

@@ -193,3 +193,21 @@ def test_two_tiles_a_wave_headline_slice_and_default_choice():
     torch.cuda.synchronize()
     assert (chosen.float() - narrow.float()).abs().max().item() <= 2 ** -6
     assert (lse_chosen - lse_narrow).abs().max().item() <= 1e-4
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_two_tiles_a_wave_f16(two_tiles_a_wave, causal):
+    q, k, v = (t.to(torch.float16) for t in make(2, 600, 576, 4, 2, seed=13))
+    scale = float(1.0 / np.sqrt(np.float32(128)))
+    config = A.FmhaPrefillConfig.contiguous(2, 600, 576, 4, 2, 128, scale, causal)
+    out = torch.full_like(q, float("nan"))
+    lse = torch.full((2, 4, 600), float("nan"), device="cuda")
+    A.fmha_prefill_lse_f16(None, out, lse, q, k, v, config)
+    torch.cuda.synchronize()
+    want, want_lse = oracle.fmha_prefill_lse_f32(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), batch=2,
+                                                 query_len=600, key_len=576, heads=4, kv_heads=2, head_dim=128, scale=scale,
+                                                 causal=causal, threads=8)
+    gap = np.abs(out.float().cpu().numpy() - want)
+    # (f16 carries three more bits than bf16)
+    assert gap.max() <= MAX_ABS / 6 and gap.mean() <= MEAN_ABS / 6, (gap.max(), gap.mean())
+    assert np.abs(lse.cpu().numpy() - want_lse).max() <= LSE_ABS
