@@ -363,9 +363,11 @@ def prefill_section(with_cpu=True, dim=128, key="prefill"):
     head_dim 128)."""
     import torch
 
+    import ctypes
+
     from singe_amd.kernel import attention as A
 
-    from singe_amd import synthetic
+    from singe_amd import _native, synthetic
 
     batch, seq, heads = 4, 4096, 32
     q, k, v = (synthetic.portable_normal(f"{key}.{tensor}", (batch, seq, heads, dim), torch.bfloat16)
@@ -374,6 +376,9 @@ def prefill_section(with_cpu=True, dim=128, key="prefill"):
     scale = float(dim) ** -0.5
     config = A.FmhaPrefillConfig.contiguous(batch, seq, seq, heads, heads, dim, scale, True)
     stats = measure(lambda: A.fmha_prefill_bf16(None, out, q, k, v, config), 5)
+    # (which of the two dense kernels the library gives this shape)
+    rows_per_wave = int(_native.lib().singe_hip_dense_prefill_rows_per_wave(ctypes.byref(config._c())))
+    kernel = f"singe_fmha_prefill_pair_bf16_d{dim}_causal" if rows_per_wave == 64 else f"singe_fmha_prefill_bf16_d{dim}_causal"
     flops = 4 * dim * batch * heads * (seq * (seq + 1) // 2)
     tflops = flops / (stats["mean_ms"] * 1e-3) / 1e12
     nbytes, source = traffic(key)
@@ -383,7 +388,7 @@ def prefill_section(with_cpu=True, dim=128, key="prefill"):
         "value": tflops, "unit": "TFLOP/s", "tokens_per_s": batch * seq / (stats["mean_ms"] * 1e-3),
         "ms_per_step": stats["mean_ms"], "ms_per_step_median": stats["median_ms"], "algorithmic_flops": flops,
         "pct_bf16_mfma_peak": 100.0 * tflops / MFMA_BF16_PEAK_TFLOPS,
-        "roofline": {"bound": "mfma", "kernel": f"singe_fmha_prefill_bf16_d{dim}_causal", "achieved": tflops,
+        "roofline": {"bound": "mfma", "kernel": kernel, "rows_per_wave": rows_per_wave, "achieved": tflops,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": nbytes, "traffic_source": source, **timing_fields(stats)},
     }

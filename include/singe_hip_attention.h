@@ -217,15 +217,6 @@ SINGE_HIP_API int32_t singe_hip_relaxed_numerics(void);
 SINGE_HIP_API void singe_hip_set_decode_workers(uint32_t workers);
 SINGE_HIP_API uint32_t singe_hip_decode_workers(const SingePagedKvDecodeAttentionConfig* config);
 
-/* Tuning knob of the dense bf16 / f16 prefill at head_dim 128: the query rows a wave takes.  32: four waves share a
- * compute unit's SIMDs two by two, 128 rows a workgroup.  64: a wave has a SIMD to itself and folds every key block
- * into two 32-row tiles, 256 rows a workgroup; only calls without options (mask, window, cap, sinks, key lengths, key
- * splits) whose key_len is a multiple of 64 have this form, others keep 32.  0 (the default): 64 where the call has
- * that form and its 256-row tiles still fill the chip.  Results are the same up to the order in which a row's
- * reference point moves.  The counterpart of AttentionParameters::{warps, min_blocks}
- * (singe/src/backend/cuda/kernel_plan/source/parameters.rs:21-57). */
-SINGE_HIP_API void singe_hip_set_dense_prefill_rows_per_wave(uint32_t rows);
-
 /* The same choices for the calling thread alone.  The setters above and below (relaxed numerics, decode workers,
  * paged / MLA key splits, the installed SingeAttentionParameters) are process-wide defaults; the reference keeps its
  * numerical policy per thread (thread_local! NUMERICAL_POLICY, singe/src/graph/numerics/mod.rs:44-49) and carries
@@ -323,6 +314,18 @@ typedef struct SingeFmhaPrefillConfig {
     float scale;
     uint8_t causal;   /* Rust bool: 0 or 1 */
 } SingeFmhaPrefillConfig;
+
+/* Tuning knob of the dense bf16 / f16 prefill at head_dim 128: the query rows a wave takes.  32: four waves share a
+ * compute unit's SIMDs two by two, 128 rows a workgroup.  64: a wave has a SIMD to itself and folds every key block
+ * into two 32-row tiles, 256 rows a workgroup; only calls without options (mask, window, cap, sinks, key lengths, key
+ * splits) whose key_len is a multiple of 64 have this form, others keep 32.  0 (the default): 64 where the call has
+ * that form and its 256-row tiles still fill the chip.  Results are the same up to the order in which a row's
+ * reference point moves.  The counterpart of AttentionParameters::{warps, min_blocks}
+ * (singe/src/backend/cuda/kernel_plan/source/parameters.rs:21-57). */
+SINGE_HIP_API void singe_hip_set_dense_prefill_rows_per_wave(uint32_t rows);
+/* What a bf16 / f16 call of this shape without options takes: 32 or 64 rows a wave, 0 when the head dimension has no
+ * matrix-core build (the one-wave-per-row kernel). */
+SINGE_HIP_API uint32_t singe_hip_dense_prefill_rows_per_wave(const SingeFmhaPrefillConfig* config);
 
 /* validate_fmha_prefill_config (mod.rs:3369-3398). */
 SINGE_HIP_API int32_t singe_hip_fmha_prefill_config_validate(const SingeFmhaPrefillConfig* config);

@@ -144,6 +144,17 @@ int32_t prefill_f32(void* stream, float* out, size_t out_len, float* lse, size_t
     return launch(kernel, static_cast<unsigned>(groups), 1, 1, 256, stream, args);
 }
 
+// Whether a call without options runs on the kernel that gives a wave two 32-row tiles: head_dim 128, every key tile
+// whole, a positive scale, no heads packed into one tile, and (unless the knob says 64) 256-row tiles that still fill
+// the chip.
+bool two_tiles_a_wave(const SingeFmhaPrefillConfig& c) {
+    const uint32_t wanted = g_rows_per_wave.load(std::memory_order_relaxed);
+    if (wanted == 32 || c.head_dim != 128 || c.key_len == 0 || c.key_len % 64 != 0 || !(c.scale > 0.0f) || dense_prefill_packs_heads(c))
+        return false;
+    const uint64_t rows = (static_cast<uint64_t>(c.batch) * c.heads + 7) / 8 * 8, pair_tiles = (c.query_len + 255) / 256;
+    return wanted == 64 || rows * ((pair_tiles + 1) / 2) >= compute_units();
+}
+
 int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, bool with_lse,
                 const uint16_t* query, size_t query_len, const uint16_t* key, size_t key_len, const uint16_t* value,
                 size_t value_len, const SingeFmhaPrefillConfig* config, bool f16 = false, const DenseOptions& options = DenseOptions()) {
@@ -241,18 +252,12 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
     const long long head_dim = static_cast<long long>(c.head_dim);
     // Long rows without options at head_dim 128: the kernel that gives a wave two 32-row tiles (256 query rows a
     // workgroup, one workgroup a compute unit), when every key tile is whole and its launch still fills the chip.
-    {
-        constexpr size_t kPairRows = 256;
-        const uint32_t pair_tiles = static_cast<uint32_t>((c.query_len + kPairRows - 1) / kPairRows);
+    if (!with_options && options.sinks == nullptr && options.key_lengths == nullptr && splits == 1 && two_tiles_a_wave(c)) {
+        const uint32_t pair_tiles = static_cast<uint32_t>((c.query_len + 255) / 256);
         const uint64_t pair_groups = rows * ((pair_tiles + 1) / 2);
-        const uint32_t wanted = g_rows_per_wave.load(std::memory_order_relaxed);
-        const bool eligible = head_dim == 128 && !with_options && options.sinks == nullptr && options.key_lengths == nullptr &&
-                              !args.packed_heads && splits == 1 && c.key_len > 0 && c.key_len % 64 == 0 && c.scale > 0.0f;
-        if (eligible && wanted != 32 && (wanted == 64 || pair_groups >= compute_units())) {
-            args.query_tiles = pair_tiles;
-            const KernelId pair = static_cast<KernelId>(kPrefillPair + (c.causal ? 0 : 1) + (f16 ? 2 : 0));
-            return launch(pair, static_cast<unsigned>(pair_groups), 1, 1, 256, stream, args);
-        }
+        args.query_tiles = pair_tiles;
+        const KernelId pair = static_cast<KernelId>(kPrefillPair + (c.causal ? 0 : 1) + (f16 ? 2 : 0));
+        return launch(pair, static_cast<unsigned>(pair_groups), 1, 1, 256, stream, args);
     }
     const KernelId kernel = static_cast<KernelId>((f16 ? kPrefillCausalF16 : kPrefillCausal) + (c.causal ? 0 : 1) + (with_options ? 4 : 0));
     if (int32_t status = launch(at_head_dim(kernel, head_dim), static_cast<unsigned>(groups), 1, 1, 64 * kDensePrefillWaves, stream, args))
@@ -371,3 +376,8 @@ int32_t singe_hip_fmha_prefill_lse_f16(void* stream, uint16_t* out, size_t out_l
 }  // extern "C"
 
 extern "C" void singe_hip_set_dense_prefill_rows_per_wave(uint32_t rows) { g_rows_per_wave.store(rows, std::memory_order_relaxed); }
+
+extern "C" uint32_t singe_hip_dense_prefill_rows_per_wave(const SingeFmhaPrefillConfig* config) {
+    if (config == nullptr) return 0;
+    return has_matrix_core_build(static_cast<long long>(config->head_dim)) ? (two_tiles_a_wave(*config) ? 64u : 32u) : 0u;
+}

@@ -339,13 +339,43 @@ SINGE_DEVICE void paged_attention_body(const PagedAttentionArgs& a, unsigned cha
             };
             if constexpr (kSteps % 2 == 0) {
                 // Multiples of 32: a lane holds both halves of its pairs (dims 16 s + 8 hi + j and the same + head_dim / 2),
-                // whole steps apart.
+                // whole steps apart, so a step's angles and weights are fetched once for both.
                 constexpr int kHalfSteps = kSteps / 2;
 #pragma unroll
                 for (int s = 0; s < kHalfSteps; ++s) {
-                    const uint4 first = bits[s], second = bits[s + kHalfSteps];
-                    bits[s] = turn(first, second, 16u * s + 8u * hi, true);
-                    bits[s + kHalfSteps] = turn(second, first, 16u * (s + kHalfSteps) + 8u * hi, false);
+                    unsigned int first_words[4] = {bits[s].x, bits[s].y, bits[s].z, bits[s].w};
+                    unsigned int second_words[4] = {bits[s + kHalfSteps].x, bits[s + kHalfSteps].y, bits[s + kHalfSteps].z, bits[s + kHalfSteps].w};
+                    const unsigned int first_pair = 16u * s + 8u * hi;
+                    float cosines[8], sines[8], low_weights[8], high_weights[8];
+                    table_values8(cosines, a.cos, a.table_type, token * kPairs + first_pair);
+                    table_values8(sines, a.sin, a.table_type, token * kPairs + first_pair);
+                    if (weighted) {
+                        table_values8(low_weights, a.query_weight, kOwnElement, first_pair);
+                        table_values8(high_weights, a.query_weight, kOwnElement, first_pair + kPairs);
+                    }
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        float rotated_first[2], rotated_second[2];
+#pragma unroll
+                        for (int upper = 0; upper < 2; ++upper) {
+                            float first = wide(first_words[w], upper), second = wide(second_words[w], upper);
+                            if (normed) {
+                                first *= scale;
+                                second *= scale;
+                                if (weighted) {
+                                    first *= low_weights[2 * w + upper];
+                                    second *= high_weights[2 * w + upper];
+                                }
+                            }
+                            const float cosine = cosines[2 * w + upper], sine = sines[2 * w + upper];
+                            rotated_first[upper] = first * cosine - second * sine;
+                            rotated_second[upper] = second * cosine + first * sine;
+                        }
+                        first_words[w] = row_valid ? pack_pair(half, rotated_first[0], rotated_first[1]) : 0u;
+                        second_words[w] = row_valid ? pack_pair(half, rotated_second[0], rotated_second[1]) : 0u;
+                    }
+                    bits[s] = make_uint4(first_words[0], first_words[1], first_words[2], first_words[3]);
+                    bits[s + kHalfSteps] = make_uint4(second_words[0], second_words[1], second_words[2], second_words[3]);
                 }
             } else {
                 // Odd multiples of 16: half a head is a whole number of steps and a half, so the partner of a lane's
