@@ -469,7 +469,7 @@ SINGE_HIP_API int32_t singe_hip_paged_attention_bf16(
  * the order of summation.  singe_hip_set_paged_attention_splits fixes the number of shares (0 = chosen by
  * problem size, the default), the counterpart of TuningChoice::Explicit
  * (singe-kernel/src/cuda/attention/mod.rs:2364-2380); it changes what ..._scratch_bytes returns.
- * A decode step (no more tokens than sequences, head_dim 128 or 64, no softcap, no window below 2048 keys) given
+ * A decode step (no more tokens than sequences, head_dim a multiple of 16 up to 128, no softcap, no window below 2048 keys) given
  * scratch on a 256-byte boundary runs on the block-table decode kernels instead, which cut the keys of all
  * sequences into equal ranges: a first kernel checks the paging vectors (same status word) and gives each token
  * its page list and key count, and the scratch then also holds those and the decode kernels' partial rows.  The
@@ -662,7 +662,8 @@ SINGE_HIP_API int32_t singe_hip_scaled_dot_product_attention(
 /* The same op with scratch for key splits (the reference's fused_attention plans the same: few blocks and many keys
  * split the keys into chunks attended separately and combined after, singe/src/backend/cuda/kernel_plan/source/
  * attention.rs:283-292, 420-452, 588-654).  A decode-shaped call (few query rows, many keys) has one workgroup per
- * (batch, head) and cannot fill the chip; given scratch, bf16 / f16 calls at head_dim 128 or 64 share the keys of a
+ * (batch, head) and cannot fill the chip; given scratch, bf16 / f16 calls at a head_dim that is a multiple of 16 up to
+ * 128 share the keys of a
  * query tile out over several workgroups, each leaving a normalised f32 partial and its base-two log-sum-exp, and a
  * second kernel merges them (sinks join the first share).  ..._scratch_bytes says how much the problem wants (0: it
  * would not split, by SingeAttentionParameters.split_below_blocks and the key count); with a null or smaller buffer,
