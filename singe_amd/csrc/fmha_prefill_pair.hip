@@ -26,385 +26,11 @@
 // loaded three tiles ahead, straight from global memory, and waited for a tile after it was asked for (a wave alone
 // on its SIMD has nobody to cover a wait for fresh loads); one barrier per tile.
 #include "kernel_args.h"
-#include "prefill_blocks.hip.h"
+#include "prefill_pair.hip.h"
 
 namespace {
 
 using namespace prefill;
-static_assert(kHeadDim == 128, "the two-tile kernel is built for head_dim 128");
-
-constexpr int kPairWaves = 4;
-constexpr unsigned int kPairRows = 64u * kPairWaves;  // query rows of a workgroup
-constexpr int kPairStages = 4;                        // of K and of V: a tile is loaded three tiles ahead
-constexpr int kPairAhead = kPairStages - 1;
-constexpr int kPairValueBase = kPairStages * kTileBytes;
-constexpr int kPairLdsBytes = 2 * kPairStages * kTileBytes;
-
-typedef v4i16_t __attribute__((address_space(3))) * lds_tr_t;
-
-// s (+)= k . q^T with s in vector registers and q in accumulation registers (see the header comment).
-typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
-// SETTLED: the operands were written long ago (the loop: K operands come from LDS reads the compiler waits for, Q^T
-// never changes).  Otherwise two idle issue slots come first, what a matrix instruction needs after a vector
-// instruction wrote one of its operands.
-template <bool FIRST, bool SETTLED, class Half>
-SINGE_DEVICE void score_step(f32x16_t& s, const uint4& k_bits, const u32x4_t& q) {
-    const u32x4_t k = __builtin_bit_cast(u32x4_t, k_bits);
-#define SINGE_SCORE_STEP(OPCODE)                                                                                              \
-    if constexpr (FIRST && SETTLED) asm volatile(OPCODE " %0, %1, %2, 0" : "=&v"(s) : "v"(k), "a"(q));                          \
-    else if constexpr (FIRST) asm volatile("s_nop 1\n\t" OPCODE " %0, %1, %2, 0" : "=&v"(s) : "v"(k), "a"(q));                 \
-    else if constexpr (SETTLED) asm volatile(OPCODE " %0, %1, %2, %0" : "+v"(s) : "v"(k), "a"(q));                             \
-    else asm volatile("s_nop 1\n\t" OPCODE " %0, %1, %2, %0" : "+v"(s) : "v"(k), "a"(q));
-    if constexpr (std::is_same_v<Half, F16>) {
-        SINGE_SCORE_STEP("v_mfma_f32_32x32x16_f16")
-    } else {
-        SINGE_SCORE_STEP("v_mfma_f32_32x32x16_bf16")
-    }
-#undef SINGE_SCORE_STEP
-}
-
-// Sixteen bytes from global memory straight into accumulation registers: Q^T is born there, as a value whose only
-// class is the one the score products read it from, so the register allocator has no vector-register home to copy it
-// back from in front of each use.  The compiler does not know this is a load: accumulation_loads_landed() before
-// the first use.
-SINGE_DEVICE u32x4_t load_to_accumulation(const void* address) {
-    u32x4_t loaded;
-    asm volatile("global_load_dwordx4 %0, %1, off" : "=a"(loaded) : "v"(address) : "memory");
-    return loaded;
-}
-// All of this wave's loads but the eight it issued last (a tile's: four of K, four of V) have completed.
-SINGE_DEVICE void older_loads_landed() { __builtin_amdgcn_s_waitcnt(0x0F78); }  // vmcnt(8), other counters left alone
-SINGE_DEVICE void accumulation_loads_landed() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
-// The scores of a whole block outside the scheduled loop (the first block, the diagonal tile): the same products, then
-// the wait the compiler would have put in front of the first reader had it known what the statements above it are.
-template <class Half>
-SINGE_DEVICE void score_block_pair(Half, f32x16_t& s, const u32x4_t (&q)[kSteps], const unsigned char* keys, const ReadOffsets& offsets) {
-    uint4 operand[kSteps];
-    read_key_operands(operand, keys, offsets);
-    static_for<kSteps>([&](auto step) { score_step<step.value == 0, false, Half>(s, operand[step.value], q[step.value]); });
-    asm volatile("s_nop 7\n\ts_nop 7" : "+v"(s));
-}
-
-// The row maxima of two score tiles, the two chains a statement apart so that no instruction waits for the one before
-// it (the compiler puts an idle slot after every statement whose instruction it does not know): three statements of
-// eight instructions, dealt to three slots of the schedule.
-SINGE_DEVICE void row_maxima_0(const f32x16_t& a, const f32x16_t& b, float& ma, float& na, float& mb, float& nb) {
-    asm volatile(
-        "v_max3_f32 %0, %4, %5, %6\n\tv_max3_f32 %2, %14, %15, %16\n\tv_max3_f32 %1, %7, %8, %9\n\tv_max3_f32 %3, %17, %18, %19\n\t"
-        "v_max3_f32 %0, %0, %10, %11\n\tv_max3_f32 %2, %2, %20, %21\n\tv_max3_f32 %1, %1, %12, %13\n\tv_max3_f32 %3, %3, %22, %23"
-        : "=&v"(ma), "=&v"(na), "=&v"(mb), "=&v"(nb)
-        : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(a[4]), "v"(a[5]), "v"(a[6]), "v"(a[7]), "v"(a[8]), "v"(a[9]), "v"(b[0]), "v"(b[1]),
-          "v"(b[2]), "v"(b[3]), "v"(b[4]), "v"(b[5]), "v"(b[6]), "v"(b[7]), "v"(b[8]), "v"(b[9]));
-}
-SINGE_DEVICE void row_maxima_1(const f32x16_t& a, const f32x16_t& b, float& ma, float& na, float& mb, float& nb) {
-    asm volatile(
-        "v_max3_f32 %0, %0, %4, %5\n\tv_max3_f32 %2, %2, %10, %11\n\tv_max3_f32 %1, %1, %6, %7\n\tv_max3_f32 %3, %3, %12, %13\n\t"
-        "v_max3_f32 %0, %0, %8, %9\n\tv_max3_f32 %2, %2, %14, %15\n\tv_max_f32 %0, %0, %1\n\tv_max_f32 %2, %2, %3"
-        : "+v"(ma), "+v"(na), "+v"(mb), "+v"(nb)
-        : "v"(a[10]), "v"(a[11]), "v"(a[12]), "v"(a[13]), "v"(a[14]), "v"(a[15]), "v"(b[10]), "v"(b[11]), "v"(b[12]), "v"(b[13]), "v"(b[14]),
-          "v"(b[15]));
-}
-// (the two lanes of a query exchange their maxima: see swap32_max)
-SINGE_DEVICE void row_maxima_2(float& ma, float& mb) {
-    float ta, tb;
-    asm volatile(
-        "v_mov_b32 %2, %0\n\tv_mov_b32 %3, %1\n\ts_nop 0\n\tv_permlane32_swap_b32 %0, %2\n\tv_permlane32_swap_b32 %1, %3\n\t"
-        "v_max_f32 %0, %0, %2\n\tv_max_f32 %1, %1, %3"
-        : "+v"(ma), "+v"(mb), "=&v"(ta), "=&v"(tb));
-}
-
-// One 32-key block b for both row tiles.  On entry a_cur / b_cur hold the raw scores of block b (shift_a / shift_b:
-// minus the rows' reference points, which already cover them) and `operand` the K operands of block b + 1; the V^T
-// operands of block b are read in the block's first half, from value_origin (the first V stage, kept where the
-// compiler cannot fold its address into the offset) + the lane's offsets + `values` (the block's byte offset from
-// there, a constant once inlined: together with the stage's own address it would not fit the instruction's 16 bits).
-// On return a_nxt / b_nxt hold the raw scores of block b + 1 and largest_a / largest_b their scaled row maxima,
-// `operand` the K operands of block b + 2 (read from keys_after); the rows' sums and O^T have taken block b in; the
-// return value says whether some row's maximum has run too far ahead of its reference point (the test is part of the
-// schedule; moving the references, which is rare, is the caller's).  issue(0 .. 3) is called once each (four of
-// the tile's eight direct-to-LDS loads of this wave).
-template <class Half, class Issue>
-SINGE_DEVICE bool fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t& a_cur, f32x16_t& b_cur, f32x16_t& a_nxt, f32x16_t& b_nxt,
-                                  float factor, float shift_a, float shift_b, float& largest_a_out, float& largest_b_out,
-                                  const u32x4_t (&qa)[8], const u32x4_t (&qb)[8], uint4 (&operand)[8], const unsigned char* __restrict__ keys_after,
-                                  const unsigned char* __restrict__ value_origin, unsigned int values, const ReadOffsets& offsets, Issue&& issue) {
-    unsigned int wa[2][4], wb[2][4];
-    v8i16_t v[2][4];
-    float total_a = 0.0f, total_b = 0.0f;
-    float largest_a, other_a, largest_b, other_b;
-    bool lagging;
-#define QK(S, Q, J) score_step<(J) == 0, true, Half>(S, operand[J], Q[J])
-#define PV(X, H, D, WORDS) \
-    X.out[D] = mma(half, __builtin_bit_cast(uint4, v[H][D]), make_uint4(WORDS[H][0], WORDS[H][1], WORDS[H][2], WORDS[H][3]), X.out[D])
-#define E(S, I, SHIFT) S[I] = fast_exp2(fmaf(S[I], factor, SHIFT))
-// (as a statement the compiler must keep in its place: a plain addition, whose result nothing needs before the block's
-// end, is collected with all the others behind the last matrix instruction)
-#define T(TOTAL, S, I) asm volatile("v_add_f32_e32 %0, %1, %0" : "+v"(TOTAL) : "v"(S[I]))
-#define W(WORDS, S, I) WORDS[(I) / 4][(I) % 4] = pack_pair(half, S[2 * (I)], S[2 * (I) + 1])
-#define ROW_MAXIMA_0 row_maxima_0(a_nxt, b_nxt, largest_a, other_a, largest_b, other_b)
-#define ROW_MAXIMA_1 row_maxima_1(a_nxt, b_nxt, largest_a, other_a, largest_b, other_b)
-#define ROW_MAXIMA_2 row_maxima_2(largest_a, largest_b)
-#define LAG_TEST                             \
-    largest_a *= factor;                     \
-    largest_b *= factor;                     \
-    lagging = __any(reference_lags(A, largest_a) || reference_lags(B, largest_b))
-#define KR(J) operand[J] = *reinterpret_cast<const uint4*>(keys_after + offsets.key(J))
-#define VR(H, D)                                                                                                                        \
-    {                                                                                                                                   \
-        const v4i16_t low = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)(value_origin + offsets.value(D) + (values + (16 * (H)) * kRowBytes))); \
-        const v4i16_t high = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)(value_origin + offsets.value(D) + (values + (16 * (H) + 8) * kRowBytes))); \
-        v[H][D] = __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7);                                                        \
-    }
-    // slot 0
-    QK(a_nxt, qa, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    issue(0);
-    E(a_cur, 0, shift_a);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 1
-    QK(b_nxt, qb, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    E(a_cur, 1, shift_a);
-    T(total_a, a_cur, 0);
-    E(a_cur, 2, shift_a);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 2
-    QK(a_nxt, qa, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    issue(1);
-    T(total_a, a_cur, 1);
-    E(a_cur, 3, shift_a);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 3
-    QK(b_nxt, qb, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    T(total_a, a_cur, 2);
-    W(wa, a_cur, 0);
-    E(a_cur, 4, shift_a);
-    T(total_a, a_cur, 3);
-    W(wa, a_cur, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 4
-    QK(a_nxt, qa, 2);
-    __builtin_amdgcn_sched_barrier(0);
-    issue(2);
-    E(a_cur, 5, shift_a);
-    T(total_a, a_cur, 4);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 5
-    QK(b_nxt, qb, 2);
-    __builtin_amdgcn_sched_barrier(0);
-    E(a_cur, 6, shift_a);
-    T(total_a, a_cur, 5);
-    E(a_cur, 7, shift_a);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 6
-    QK(a_nxt, qa, 3);
-    __builtin_amdgcn_sched_barrier(0);
-    issue(3);
-    T(total_a, a_cur, 6);
-    W(wa, a_cur, 2);
-    T(total_a, a_cur, 7);
-    W(wa, a_cur, 3);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 7
-    QK(b_nxt, qb, 3);
-    __builtin_amdgcn_sched_barrier(0);
-    E(a_cur, 8, shift_a);
-    E(a_cur, 9, shift_a);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 8
-    QK(a_nxt, qa, 4);
-    __builtin_amdgcn_sched_barrier(0);
-    VR(0, 0);
-    T(total_a, a_cur, 8);
-    E(a_cur, 10, shift_a);
-    T(total_a, a_cur, 9);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 9
-    QK(b_nxt, qb, 4);
-    __builtin_amdgcn_sched_barrier(0);
-    VR(0, 1);
-    E(a_cur, 11, shift_a);
-    T(total_a, a_cur, 10);
-    W(wa, a_cur, 4);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 10
-    QK(a_nxt, qa, 5);
-    __builtin_amdgcn_sched_barrier(0);
-    VR(0, 2);
-    E(a_cur, 12, shift_a);
-    T(total_a, a_cur, 11);
-    W(wa, a_cur, 5);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 11
-    QK(b_nxt, qb, 5);
-    __builtin_amdgcn_sched_barrier(0);
-    VR(0, 3);
-    E(a_cur, 13, shift_a);
-    T(total_a, a_cur, 12);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 12
-    QK(a_nxt, qa, 6);
-    __builtin_amdgcn_sched_barrier(0);
-    VR(1, 0);
-    E(a_cur, 14, shift_a);
-    T(total_a, a_cur, 13);
-    W(wa, a_cur, 6);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 13
-    QK(b_nxt, qb, 6);
-    __builtin_amdgcn_sched_barrier(0);
-    VR(1, 1);
-    E(a_cur, 15, shift_a);
-    T(total_a, a_cur, 14);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 14
-    QK(a_nxt, qa, 7);
-    __builtin_amdgcn_sched_barrier(0);
-    VR(1, 2);
-    T(total_a, a_cur, 15);
-    W(wa, a_cur, 7);
-    E(b_cur, 0, shift_b);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 15
-    QK(b_nxt, qb, 7);
-    __builtin_amdgcn_sched_barrier(0);
-    VR(1, 3);
-    E(b_cur, 1, shift_b);
-    T(total_b, b_cur, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 16
-    PV(A, 0, 0, wa);
-    __builtin_amdgcn_sched_barrier(0);
-    KR(0);
-    E(b_cur, 2, shift_b);
-    T(total_b, b_cur, 1);
-    W(wb, b_cur, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 17
-    PV(A, 0, 1, wa);
-    __builtin_amdgcn_sched_barrier(0);
-    KR(1);
-    E(b_cur, 3, shift_b);
-    T(total_b, b_cur, 2);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 18
-    PV(A, 0, 2, wa);
-    __builtin_amdgcn_sched_barrier(0);
-    KR(2);
-    E(b_cur, 4, shift_b);
-    T(total_b, b_cur, 3);
-    W(wb, b_cur, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 19
-    PV(A, 0, 3, wa);
-    __builtin_amdgcn_sched_barrier(0);
-    KR(3);
-    E(b_cur, 5, shift_b);
-    T(total_b, b_cur, 4);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 20
-    PV(A, 1, 0, wa);
-    __builtin_amdgcn_sched_barrier(0);
-    KR(4);
-    E(b_cur, 6, shift_b);
-    T(total_b, b_cur, 5);
-    W(wb, b_cur, 2);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 21
-    PV(A, 1, 1, wa);
-    __builtin_amdgcn_sched_barrier(0);
-    KR(5);
-    E(b_cur, 7, shift_b);
-    T(total_b, b_cur, 6);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 22
-    PV(A, 1, 2, wa);
-    __builtin_amdgcn_sched_barrier(0);
-    KR(6);
-    T(total_b, b_cur, 7);
-    W(wb, b_cur, 3);
-    E(b_cur, 8, shift_b);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 23
-    PV(A, 1, 3, wa);
-    __builtin_amdgcn_sched_barrier(0);
-    KR(7);
-    E(b_cur, 9, shift_b);
-    T(total_b, b_cur, 8);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 24
-    PV(B, 0, 0, wb);
-    __builtin_amdgcn_sched_barrier(0);
-    E(b_cur, 10, shift_b);
-    T(total_b, b_cur, 9);
-    E(b_cur, 11, shift_b);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 25
-    PV(B, 0, 1, wb);
-    __builtin_amdgcn_sched_barrier(0);
-    T(total_b, b_cur, 10);
-    W(wb, b_cur, 4);
-    E(b_cur, 12, shift_b);
-    T(total_b, b_cur, 11);
-    W(wb, b_cur, 5);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 26
-    PV(B, 0, 2, wb);
-    __builtin_amdgcn_sched_barrier(0);
-    E(b_cur, 13, shift_b);
-    T(total_b, b_cur, 12);
-    E(b_cur, 14, shift_b);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 27
-    PV(B, 0, 3, wb);
-    __builtin_amdgcn_sched_barrier(0);
-    T(total_b, b_cur, 13);
-    E(b_cur, 15, shift_b);
-    T(total_b, b_cur, 14);
-    W(wb, b_cur, 6);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 28
-    W(wb, b_cur, 7);
-    PV(B, 1, 0, wb);
-    __builtin_amdgcn_sched_barrier(0);
-    ROW_MAXIMA_0;
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 29
-    PV(B, 1, 1, wb);
-    __builtin_amdgcn_sched_barrier(0);
-    ROW_MAXIMA_1;
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 30
-    PV(B, 1, 2, wb);
-    __builtin_amdgcn_sched_barrier(0);
-    ROW_MAXIMA_2;
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 31
-    PV(B, 1, 3, wb);
-    __builtin_amdgcn_sched_barrier(0);
-    LAG_TEST;
-    T(total_b, b_cur, 15);
-    __builtin_amdgcn_sched_barrier(0);
-#undef QK
-#undef PV
-#undef E
-#undef T
-#undef W
-#undef KR
-#undef ROW_MAXIMA_0
-#undef ROW_MAXIMA_1
-#undef ROW_MAXIMA_2
-#undef LAG_TEST
-#undef VR
-    A.running_sum += total_a;
-    B.running_sum += total_b;
-    largest_a_out = largest_a;
-    largest_b_out = largest_b;
-    return lagging;
-}
 
 // One 256-row query tile of (batch, head) pair `bh`.
 template <bool CAUSAL, class Half>

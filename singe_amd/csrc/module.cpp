@@ -314,6 +314,8 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_decode_combine_few_bf16_d112", "singe_paged_decode_combine_few_f16_d112",
     "singe_fmha_prefill_pair_bf16_d128_causal", "singe_fmha_prefill_pair_bf16_d128_full",
     "singe_fmha_prefill_pair_f16_d128_causal", "singe_fmha_prefill_pair_f16_d128_full",
+    "singe_paged_attention_pair_bf16_d128_i32", "singe_paged_attention_pair_bf16_d128_i64",
+    "singe_paged_attention_pair_f16_d128_i32", "singe_paged_attention_pair_f16_d128_i64",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -327,7 +329,7 @@ const char* const kPartNames[kPartCount] = {
     "fmha_prefill_d16", "paged_attention_d16", "fmha_prefill_d48", "paged_attention_d48", "fmha_prefill_d80", "paged_attention_d80",
     "fmha_prefill_d112", "paged_attention_d112", "paged_decode_d32",
     "paged_decode_d16", "paged_decode_d48", "paged_decode_d80", "paged_decode_d96", "paged_decode_d112",
-    "fmha_prefill_pair",
+    "fmha_prefill_pair", "paged_attention_pair",
 };
 
 namespace {
@@ -356,6 +358,7 @@ constexpr PartRun kPartRuns[] = {
     {8, 4},                       // latent attention on the matrix cores at any width it takes
     {30, 14}, {31, 14}, {32, 14}, {33, 14}, {34, 14}, {35, 14},  // the decode kernels and their merges for 32, 16, 48, 80, 96, 112
     {36, 4},                      // the dense prefill with two row tiles a wave
+    {37, 4},                      // the paged attention op on the same loop
 };
 constexpr int runs_total() {
     int total = 0;

@@ -85,7 +85,10 @@ enum KernelId : int {
     kDecodeOtherHeadDims,
     // the dense prefill that gives a wave two 32-row tiles (head_dim 128, no options): + (no causal mask) + 2 * f16
     kPrefillPair = kDecodeOtherHeadDims + 6 * 14,
-    kKernelCount = kPrefillPair + 4
+    // the paged attention op on the same two-tile loop (head_dim 128, page sizes that are powers of two from 16, no
+    // options): + (i64 indices) + 2 * f16
+    kPagedPair = kPrefillPair + 4,
+    kKernelCount = kPagedPair + 4
 };
 
 
@@ -154,7 +157,7 @@ inline int rotary_paged_attention_base(bool f16, bool softcap, long long head_di
 extern const char* const kKernelNames[kKernelCount];
 
 // Parts of the code object (one file each) and the part a kernel lives in.
-constexpr int kPartCount = 37;
+constexpr int kPartCount = 38;
 extern const char* const kPartNames[kPartCount];
 int kernel_part(int kernel);
 

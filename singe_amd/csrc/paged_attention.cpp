@@ -39,7 +39,7 @@ struct Scratch {
 // How the grid covers the row tiles (see `locate` in paged_attention.hip).  When no sequence can have more than one
 // row tile the plain form is used: sequences x kv heads workgroups, a sequence found from the workgroup id alone.
 // Otherwise the compact form: every sequence has at least one entry, and the entries of all of them are at most
-// floor(tokens * groups / 128) + sequences.
+// floor(tokens * groups / rows) + sequences (rows: the packed rows of a workgroup, 128, or 256 on the two-tile kernel).
 struct RowTileGrid {
     uint32_t compact;
     uint32_t longest_first;  // the compact list takes the sequences longest first (see `locate`)
@@ -47,9 +47,9 @@ struct RowTileGrid {
     uint64_t blocks;      // workgroups without key splits
 };
 
-RowTileGrid grid_of(uint64_t tokens, uint64_t sequences, uint64_t groups, uint64_t kv_heads = 1) {
+RowTileGrid grid_of(uint64_t tokens, uint64_t sequences, uint64_t groups, uint64_t kv_heads = 1, uint64_t rows = 128) {
     RowTileGrid grid;
-    const uint64_t longest = (groups * tokens + 127) / 128;
+    const uint64_t longest = (groups * tokens + rows - 1) / rows;
     grid.longest_first = 0;
     if (longest <= 1) {
         grid.compact = 0;
@@ -57,10 +57,10 @@ RowTileGrid grid_of(uint64_t tokens, uint64_t sequences, uint64_t groups, uint64
         grid.blocks = (sequences * kv_heads + 7) / 8 * 8 * longest;
     } else {
         grid.compact = 1;
-        grid.row_tiles = groups * tokens / 128 + sequences;
+        grid.row_tiles = groups * tokens / rows + sequences;
         // Longest sequences first where sequences have row tiles to spare (chunks of a prefill): their workgroups run
         // for hundreds of microseconds and the order decides how full the chip's last round is.
-        grid.longest_first = sequences <= 64 && groups * tokens / 128 >= 2 * sequences ? 1u : 0u;
+        grid.longest_first = sequences <= 64 && groups * tokens / rows >= 2 * sequences ? 1u : 0u;
         const uint64_t bands = (grid.row_tiles + 31) / 32;
         grid.blocks = (kv_heads * bands + 7) / 8 * 8 * 32;
     }
@@ -69,6 +69,9 @@ RowTileGrid grid_of(uint64_t tokens, uint64_t sequences, uint64_t groups, uint64
 
 // 0 = chosen by problem size (singe_hip_set_paged_attention_splits).
 std::atomic<uint32_t> g_paged_attention_splits{0};
+// Packed rows a wave of the bf16 / f16 kernels takes: 0 = chosen by problem size, 32, or 64 where the two-tile kernel
+// takes the call (singe_hip_set_paged_attention_rows_per_wave).
+std::atomic<uint32_t> g_paged_rows_per_wave{0};
 
 // The count in force on this thread: its own (SingeHipThreadOptions) over the process-wide one.
 uint32_t fixed_paged_attention_splits() {
@@ -290,6 +293,22 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
         args.partial_out = static_cast<float*>(scratch->memory);
         args.partial_lse = args.partial_out + static_cast<size_t>(splits) * p.tokens * p.heads * p.head_dim;
     }
+    // Prefill-shaped plain calls at head_dim 128 take the kernel that gives a wave two 32-row tiles (256 packed rows a
+    // workgroup, one workgroup a compute unit; paged_attention_pair.hip), when its grid still fills the chip.
+    if (rotation == nullptr && splits == 1 && head_dim == 128 && !p.has_softcap && !p.has_window && args.page_shift >= 4 && scale > 0.0f) {
+        const uint32_t wanted = g_paged_rows_per_wave.load(std::memory_order_relaxed);
+        const RowTileGrid pair = grid_of(static_cast<uint64_t>(p.tokens), static_cast<uint64_t>(p.sequences), groups,
+                                         static_cast<uint64_t>(p.kv_heads), 256);
+        // (workgroups that can have work: a sequence's tiles, or the list's, for every kv head)
+        const uint64_t working = static_cast<uint64_t>(p.kv_heads) * (pair.compact ? groups * static_cast<uint64_t>(p.tokens) / 256 : 0);
+        if (wanted != 32 && pair.blocks <= 0x7fffffffull && pair.row_tiles <= 0xffffffffull && (wanted == 64 || working >= compute_units())) {
+            args.row_tiles = static_cast<uint32_t>(pair.row_tiles);
+            args.compact = pair.compact;
+            args.longest_first = pair.longest_first;
+            const int kernel = kPagedPair + (wide ? 1 : 0) + (f16 ? 2 : 0);
+            return launch(static_cast<KernelId>(kernel), static_cast<unsigned>(pair.blocks), 1, 1, 256, stream, args);
+        }
+    }
     const unsigned grid = static_cast<unsigned>(blocks * splits);
     auto finish = [&](int32_t launched) -> int32_t {
         if (launched != 0 || splits == 1) return launched;
@@ -312,6 +331,8 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
 }
 
 }  // namespace
+
+extern "C" void singe_hip_set_paged_attention_rows_per_wave(uint32_t rows) { g_paged_rows_per_wave.store(rows, std::memory_order_relaxed); }
 
 extern "C" void singe_hip_set_paged_attention_splits(uint32_t splits) {
     g_paged_attention_splits.store(splits > 64 ? 64 : splits, std::memory_order_relaxed);

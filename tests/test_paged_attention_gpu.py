@@ -373,3 +373,42 @@ def test_a_decode_step_of_thousands_of_sequences(count, heads, kv_heads):
     empty = np.isneginf(want_lse)
     assert np.array_equal(np.isneginf(lse.cpu().numpy()), empty)
     assert np.abs(lse.cpu().numpy()[~empty] - want_lse[~empty]).max() <= LSE_ABS
+
+
+@pytest.fixture
+def two_tiles_a_wave():
+    """Sends every paged call that has the form to the kernel that gives a wave two 32-row tiles."""
+    _native.lib().singe_hip_set_paged_attention_rows_per_wave(64)
+    yield
+    _native.lib().singe_hip_set_paged_attention_rows_per_wave(0)
+
+
+@pytest.mark.parametrize("index_dtype", [torch.int32, torch.int64])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("heads,kv_heads,page_size", [(8, 1, 16), (64, 8, 16), (8, 2, 32), (4, 1, 64), (8, 2, 128), (4, 4, 16)])
+def test_two_tiles_a_wave_ragged_sequences_match_oracle(two_tiles_a_wave, heads, kv_heads, page_size, causal, index_dtype):
+    # the shapes of the ragged test (decode, full prefill, chunked prefill, no keys, more queries than keys) and
+    # chunks long enough for several 256-row tiles, several key tiles ahead of the mask and key counts either side of
+    # a tile's and a page's end
+    sequences = [(1, 150), (70, 70), (20, 90), (3, 0), (9, 4), (130, 300), (300, 1000), (257, 513), (64, 1024), (512, 512)]
+    run_case(sequences, heads, kv_heads, page_size, neural.AttentionOptions(causal=causal), index_dtype=index_dtype,
+             seed=heads + page_size + 1)
+
+
+def test_two_tiles_a_wave_equals_the_four_wave_kernel_at_the_chunked_prefill_shape():
+    # The fourth benchmark configuration fills the chip with 256-row tiles, so the default choice is this kernel: its
+    # answer against the 32-row kernel's, within the rounding of the output.
+    from singe_amd import synthetic
+    work = synthetic.chunked_prefill_workload(portable=True)
+    index = lambda values: torch.from_numpy(np.asarray(values, dtype=np.int32)).cuda()
+    paging = neural.Paging(index(work.query_offsets), index(work.page_offsets), index(work.pages), index(work.last_page_lengths))
+    options = neural.AttentionOptions(causal=True)
+    chosen, chosen_lse = neural.paged_attention(work.query, work.key_cache, work.value_cache, paging, options)
+    _native.lib().singe_hip_set_paged_attention_rows_per_wave(32)
+    try:
+        narrow, narrow_lse = neural.paged_attention(work.query, work.key_cache, work.value_cache, paging, options)
+    finally:
+        _native.lib().singe_hip_set_paged_attention_rows_per_wave(0)
+    torch.cuda.synchronize()
+    assert (chosen.float() - narrow.float()).abs().max().item() <= 2 ** -6
+    assert (chosen_lse - narrow_lse).abs().max().item() <= 1e-4

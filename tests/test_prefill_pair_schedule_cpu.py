@@ -1,4 +1,4 @@
-"""The two-tile dense prefill kernel writes its score products as assembly (the compiler would give them
+"""The two-tile prefill kernels (dense and paged) write their score products as assembly (the compiler would give them
 accumulation-register destinations), so the compiler does not know that those statements are matrix instructions and
 keeps no distance between them and what reads their results: the distance is part of the kernel's hand-made schedule.
 This test compiles the kernel to gfx950 assembly and checks, on what the compiler actually emitted (its register
@@ -11,9 +11,11 @@ import re
 import subprocess
 import tempfile
 
+import pytest
+
 from singe_amd import build
 
-SOURCE = os.path.join(os.path.dirname(build.__file__), "csrc", "fmha_prefill_pair.hip")
+SOURCES = [os.path.join(os.path.dirname(build.__file__), "csrc", name) for name in ("fmha_prefill_pair.hip", "paged_attention_pair.hip")]
 WAIT_STATES = 12
 
 
@@ -43,11 +45,12 @@ def instructions(assembly):
         yield stripped.split(";")[0].strip(), inside
 
 
-def test_nothing_touches_a_score_product_before_it_is_done():
+@pytest.mark.parametrize("source", SOURCES, ids=os.path.basename)
+def test_nothing_touches_a_score_product_before_it_is_done(source):
     with tempfile.TemporaryDirectory() as scratch:
         listing = os.path.join(scratch, "pair.s")
         command = [build.hipcc()] + [flag for flag in build.HIPCC_FLAGS if flag != "--genco"] + [
-            "--cuda-device-only", "-S", "-I", os.path.dirname(SOURCE), SOURCE, "-o", listing]
+            "--cuda-device-only", "-S", "-I", os.path.dirname(source), source, "-o", listing]
         subprocess.run(command, check=True, capture_output=True)
         program = list(instructions(open(listing).read()))
     products = 0
