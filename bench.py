@@ -439,7 +439,11 @@ def chunked_prefill_section(with_cpu=True):
     assert int(status.item()) == 0
     flops = work.algorithmic_flops()
     tflops = flops / (stats["mean_ms"] * 1e-3) / 1e12
+    rows_per_wave = int(_native.lib().singe_hip_paged_attention_rows_per_wave(ctypes.byref(problem)))
+    kernel = "singe_paged_attention_pair_bf16_d128_i32" if rows_per_wave == 64 else "singe_paged_attention_bf16_d128_i32_p16"
     nbytes, source = traffic("chunked_prefill")
+    if COUNTER_TRAFFIC["chunked_prefill"]["kernel"] != kernel:
+        nbytes, source = None, None  # the counters were read on the other kernel
     result = {
         "workload": "chunked paged prefill: 8 sequences x 512 new tokens on prefixes U[1024,16384], 64q/8kv heads, "
                     "head_dim 128, page 16, bf16 (BASELINE config 4); whole op (the attention kernel and, where the op "
@@ -447,7 +451,7 @@ def chunked_prefill_section(with_cpu=True):
         "value": tflops, "unit": "TFLOP/s", "tokens_per_s": work.sequences * work.new_tokens / (stats["mean_ms"] * 1e-3),
         "ms_per_step": stats["mean_ms"], "ms_per_step_median": stats["median_ms"], "algorithmic_flops": flops,
         "algorithmic_bytes": work.algorithmic_bytes(), "key_splits_scratch_bytes": scratch_bytes,
-        "roofline": {"bound": "mfma", "kernel": "singe_paged_attention_bf16_d128_i32_p16", "achieved": tflops,
+        "roofline": {"bound": "mfma", "kernel": kernel, "rows_per_wave": rows_per_wave, "achieved": tflops,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": nbytes, "traffic_source": source, **timing_fields(stats)},
     }

@@ -481,6 +481,9 @@ SINGE_HIP_API void singe_hip_set_paged_attention_splits(uint32_t splits);
  * window, key splits or a fused rotation have that form; others keep 32), or 0 (the default): 64 where the call has
  * that form and its 256-row tiles still fill the chip. */
 SINGE_HIP_API void singe_hip_set_paged_attention_rows_per_wave(uint32_t rows);
+/* What a bf16 / f16 call of this problem takes when it is given scratch and has no fused rotation: 32 or 64 rows a wave,
+ * 0 when the head dimension has no matrix-core build. */
+SINGE_HIP_API uint32_t singe_hip_paged_attention_rows_per_wave(const SingePagedAttentionProblem* problem);
 SINGE_HIP_API int32_t singe_hip_paged_attention_scratch_bf16(
     void* stream,
     const uint16_t* query_rows,

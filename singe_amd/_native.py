@@ -277,6 +277,8 @@ def bind(path: str) -> ctypes.CDLL:
     handle.singe_hip_relaxed_numerics.restype = i32
     handle.singe_hip_set_paged_attention_rows_per_wave.argtypes = [ctypes.c_uint32]
     handle.singe_hip_set_paged_attention_rows_per_wave.restype = None
+    handle.singe_hip_paged_attention_rows_per_wave.argtypes = [ctypes.c_void_p]
+    handle.singe_hip_paged_attention_rows_per_wave.restype = ctypes.c_uint32
     handle.singe_hip_set_dense_prefill_rows_per_wave.argtypes = [ctypes.c_uint32]
     handle.singe_hip_set_dense_prefill_rows_per_wave.restype = None
     handle.singe_hip_dense_prefill_rows_per_wave.argtypes = [ctypes.c_void_p]

@@ -78,6 +78,24 @@ uint32_t fixed_paged_attention_splits() {
     return effective_count(thread_options().paged_attention_splits, g_paged_attention_splits.load(std::memory_order_relaxed));
 }
 
+// Whether a bf16 / f16 call without a fused rotation or key splits runs on the kernel that gives a wave two 32-row
+// tiles, and the grid it takes there: head_dim 128, a page size that is a power of two of at least 16 keys, no cap, no
+// window, a positive scale, and (unless the knob says 64) enough 256-row tiles to fill the chip.
+bool two_tiles_a_wave(const SingePagedAttentionProblem& p, RowTileGrid* grid) {
+    const uint32_t wanted = g_paged_rows_per_wave.load(std::memory_order_relaxed);
+    if (wanted == 32 || p.head_dim != 128 || p.has_softcap || p.has_window || p.tokens <= 0 || p.sequences <= 0 || p.kv_heads <= 0 ||
+        p.heads <= 0 || p.page_size < 16 || (p.page_size & (p.page_size - 1)) != 0)
+        return false;
+    const float scale = p.has_scale ? p.scale : 1.0f;
+    if (!(scale > 0.0f)) return false;
+    const uint64_t groups = static_cast<uint64_t>(p.heads / p.kv_heads);
+    *grid = grid_of(static_cast<uint64_t>(p.tokens), static_cast<uint64_t>(p.sequences), groups, static_cast<uint64_t>(p.kv_heads), 256);
+    if (grid->blocks > 0x7fffffffull || grid->row_tiles > 0xffffffffull) return false;
+    // (workgroups that are sure to have work: the whole 256-row tiles of all sequences together, for every kv head)
+    const uint64_t working = static_cast<uint64_t>(p.kv_heads) * (groups * static_cast<uint64_t>(p.tokens) / 256);
+    return wanted == 64 || (grid->compact != 0 && working >= compute_units());
+}
+
 // Key splits for a problem: enough workgroups to fill the compute units four times over, when the query rows
 // alone do not (decoding, short chunks); one (no split) for other element types and head dimensions.
 uint32_t paged_attention_splits(const SingePagedAttentionProblem& p) {
@@ -295,19 +313,13 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
     }
     // Prefill-shaped plain calls at head_dim 128 take the kernel that gives a wave two 32-row tiles (256 packed rows a
     // workgroup, one workgroup a compute unit; paged_attention_pair.hip), when its grid still fills the chip.
-    if (rotation == nullptr && splits == 1 && head_dim == 128 && !p.has_softcap && !p.has_window && args.page_shift >= 4 && scale > 0.0f) {
-        const uint32_t wanted = g_paged_rows_per_wave.load(std::memory_order_relaxed);
-        const RowTileGrid pair = grid_of(static_cast<uint64_t>(p.tokens), static_cast<uint64_t>(p.sequences), groups,
-                                         static_cast<uint64_t>(p.kv_heads), 256);
-        // (workgroups that can have work: a sequence's tiles, or the list's, for every kv head)
-        const uint64_t working = static_cast<uint64_t>(p.kv_heads) * (pair.compact ? groups * static_cast<uint64_t>(p.tokens) / 256 : 0);
-        if (wanted != 32 && pair.blocks <= 0x7fffffffull && pair.row_tiles <= 0xffffffffull && (wanted == 64 || working >= compute_units())) {
-            args.row_tiles = static_cast<uint32_t>(pair.row_tiles);
-            args.compact = pair.compact;
-            args.longest_first = pair.longest_first;
-            const int kernel = kPagedPair + (wide ? 1 : 0) + (f16 ? 2 : 0);
-            return launch(static_cast<KernelId>(kernel), static_cast<unsigned>(pair.blocks), 1, 1, 256, stream, args);
-        }
+    RowTileGrid pair;
+    if (rotation == nullptr && splits == 1 && (data_type == SINGE_HIP_BF16 || f16) && two_tiles_a_wave(p, &pair)) {
+        args.row_tiles = static_cast<uint32_t>(pair.row_tiles);
+        args.compact = pair.compact;
+        args.longest_first = pair.longest_first;
+        const int kernel = kPagedPair + (wide ? 1 : 0) + (f16 ? 2 : 0);
+        return launch(static_cast<KernelId>(kernel), static_cast<unsigned>(pair.blocks), 1, 1, 256, stream, args);
     }
     const unsigned grid = static_cast<unsigned>(blocks * splits);
     auto finish = [&](int32_t launched) -> int32_t {
@@ -333,6 +345,12 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
 }  // namespace
 
 extern "C" void singe_hip_set_paged_attention_rows_per_wave(uint32_t rows) { g_paged_rows_per_wave.store(rows, std::memory_order_relaxed); }
+
+extern "C" uint32_t singe_hip_paged_attention_rows_per_wave(const SingePagedAttentionProblem* problem) {
+    if (problem == nullptr || !has_matrix_core_build(problem->head_dim)) return 0;
+    RowTileGrid grid;
+    return paged_attention_splits(*problem) == 1 && two_tiles_a_wave(*problem, &grid) ? 64u : 32u;
+}
 
 extern "C" void singe_hip_set_paged_attention_splits(uint32_t splits) {
     g_paged_attention_splits.store(splits > 64 ? 64 : splits, std::memory_order_relaxed);
