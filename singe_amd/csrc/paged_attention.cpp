@@ -86,6 +86,8 @@ bool two_tiles_a_wave(const SingePagedAttentionProblem& p, RowTileGrid* grid) {
     if (wanted == 32 || p.head_dim != 128 || p.has_softcap || p.has_window || p.tokens <= 0 || p.sequences <= 0 || p.kv_heads <= 0 ||
         p.heads <= 0 || p.page_size < 16 || (p.page_size & (p.page_size - 1)) != 0)
         return false;
+    // (the kernel works out where a page starts from a 32-bit count of a page's bytes)
+    if (static_cast<uint64_t>(p.page_size) * static_cast<uint64_t>(p.kv_heads) * 256 > 0xffffffffull) return false;
     const float scale = p.has_scale ? p.scale : 1.0f;
     if (!(scale > 0.0f)) return false;
     const uint64_t groups = static_cast<uint64_t>(p.heads / p.kv_heads);

@@ -124,52 +124,69 @@ SINGE_DEVICE void paged_attention_pair_body(const PagedAttentionArgs& a, unsigne
     // group sit in one page (paged_attention.hip, GROUPED).
     const unsigned int load_row = 4u * wave + (lane >> 4), chunk_position = lane & 15u;
     const unsigned int key_chunk = (chunk_position ^ (load_row & 15u)) * 16u, value_chunk = (chunk_position ^ (4u * (load_row & 3u))) * 16u;
-    const size_t page_bytes = static_cast<size_t>(a.page_size) * a.kv_heads * kGlobalRowBytes;
+    const unsigned int page_bytes = a.page_size * a.kv_heads * kGlobalRowBytes;  // (the host sends pages below 4 GiB)
     const unsigned int head_bytes = kv_head * kGlobalRowBytes, slot_bytes = a.kv_heads * kGlobalRowBytes;
     const unsigned char* const key_bytes = reinterpret_cast<const unsigned char*>(a.key_cache);
     const unsigned char* const value_bytes = reinterpret_cast<const unsigned char*>(a.value_cache);
     const unsigned int last_group = tiles > 0 ? (keys - 1u) & ~15u : 0u;  // first key of the sixteen that hold the last one
     const unsigned int key_lane = load_row * slot_bytes + key_chunk, value_lane = load_row * slot_bytes + value_chunk;
+    // Where the four groups of a tile start in either cache, in bytes.
     struct Pages {
-        unsigned int id[4];
+        unsigned long long start[4];
     };
     // First key of the group instruction i of a tile reads: its own, or the last group of the sequence.
     auto group_of = [&](unsigned int tile, unsigned int i) __attribute__((always_inline)) {
         const unsigned int first = tile * kKeyTile + 16u * i;
         return first < last_group ? first : last_group;
     };
-    // The ids of a tile's four groups, one a lane (lane % 4): on their way until the loads before them have landed.
+    // The id of one group of a tile a lane (group lane % 4), on its way until the loads before it have landed, and
+    // where the group starts in its page.  All of this is lane work: the wave is alone on its SIMD, where a scalar
+    // instruction costs the issue slot a vector one does, and four lanes do four groups at once.
+    struct Lookup {
+        RawPage<FORM> raw;
+        unsigned int in_page;
+    };
     auto lookup = [&](unsigned int tile) __attribute__((always_inline)) {
-        return read_raw_page<FORM>(a.pages, static_cast<size_t>(page_start) + (group_of(tile, lane & 3u) >> a.page_shift));
+        const unsigned int group = group_of(tile, lane & 3u);
+        Lookup l;
+        l.raw = read_raw_page<FORM>(a.pages, static_cast<size_t>(page_start) + (group >> a.page_shift));
+        l.in_page = (group & (a.page_size - 1u)) * slot_bytes + head_bytes;
+        return l;
     };
-    auto check = [&](RawPage<FORM> raw, Pages& pages) __attribute__((always_inline)) {
-        const unsigned long long mine = static_cast<unsigned long long>(raw);  // negative ids wrap above any cache
-        const unsigned int low = static_cast<unsigned int>(mine), upper = static_cast<unsigned int>(mine >> 32);
+    auto check = [&](const Lookup& l, Pages& pages) __attribute__((always_inline)) {
+        const unsigned long long mine = static_cast<unsigned long long>(l.raw);  // negative ids wrap above any cache
+        const bool valid = mine < static_cast<unsigned long long>(a.cache_pages);
+        // (an id outside the cache is reported and replaced by page 0: what that holds is not used by a caller that checks)
+        if (__builtin_amdgcn_ballot_w64(!valid) != 0) report_index_error(a.status);
+        const unsigned long long start = static_cast<unsigned long long>(valid ? static_cast<unsigned int>(mine) : 0u) * page_bytes + l.in_page;
+        const unsigned int low = static_cast<unsigned int>(start), upper = static_cast<unsigned int>(start >> 32);
 #pragma unroll
-        for (unsigned int i = 0; i < 4; ++i) {
-            const unsigned long long page = (static_cast<unsigned long long>(__builtin_amdgcn_readlane(upper, i)) << 32) | __builtin_amdgcn_readlane(low, i);
-            const bool valid = page < static_cast<unsigned long long>(a.cache_pages);
-            if (!valid) report_index_error(a.status);
-            pages.id[i] = valid ? static_cast<unsigned int>(page) : 0u;  // (reported; what page 0 holds is not used by a caller that checks)
-        }
+        for (unsigned int i = 0; i < 4; ++i)
+            pages.start[i] = (static_cast<unsigned long long>(static_cast<unsigned int>(__builtin_amdgcn_readlane(upper, i))) << 32) |
+                             static_cast<unsigned int>(__builtin_amdgcn_readlane(low, i));
     };
-    auto load_part = [&](const unsigned char* cache, unsigned int chunk, unsigned int lane_offset, unsigned int tile, const Pages& pages,
+    // `tail`: the tile holds the sequence's last key or lies past it, so some of its rows re-read that key.
+    auto load_part = [&](const unsigned char* cache, unsigned int chunk, unsigned int lane_offset, unsigned int tile, bool tail, const Pages& pages,
                          unsigned int i, unsigned char* stage) __attribute__((always_inline)) {
-        const unsigned int first = tile * kKeyTile + 16u * i, group = group_of(tile, i);
-        const unsigned char* base = cache + (pages.id[i] * page_bytes + ((group & (a.page_size - 1u)) * slot_bytes + head_bytes));
-        // (the group that holds the sequence's last key, or lies past it: rows past that key re-read it)
-        const unsigned int last = keys - 1u - group;
-        unsigned int offset = first + 15u >= keys ? (load_row < last ? load_row : last) * slot_bytes + chunk : lane_offset;
+        const unsigned char* base = cache + pages.start[i];
+        unsigned int offset = lane_offset;
+        if (__builtin_expect(tail, 0)) {
+            const unsigned int last = keys - 1u - group_of(tile, i);
+            offset = (load_row < last ? load_row : last) * slot_bytes + chunk;
+            asm volatile("" : "+v"(offset));  // (keeps the branch a branch)
+        }
         asm("" : "+s"(base));
         asm volatile("" : "+v"(offset));
         __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(base + offset),
                                          (lds_words_t)(stage + (16u * i + 4u * wave) * kRowBytes), 16, 0, 0);
     };
+    auto is_tail = [&](unsigned int tile) __attribute__((always_inline)) { return tile * kKeyTile + kKeyTile > keys; };
     auto load_tile = [&](unsigned int tile, const Pages& pages, unsigned int stage) __attribute__((always_inline)) {
 #pragma unroll
-        for (unsigned int i = 0; i < 4; ++i) load_part(key_bytes, key_chunk, key_lane, tile, pages, i, lds + stage * kTileBytes);
+        for (unsigned int i = 0; i < 4; ++i) load_part(key_bytes, key_chunk, key_lane, tile, is_tail(tile), pages, i, lds + stage * kTileBytes);
 #pragma unroll
-        for (unsigned int i = 0; i < 4; ++i) load_part(value_bytes, value_chunk, value_lane, tile, pages, i, lds + kPairValueBase + stage * kTileBytes);
+        for (unsigned int i = 0; i < 4; ++i)
+            load_part(value_bytes, value_chunk, value_lane, tile, is_tail(tile), pages, i, lds + kPairValueBase + stage * kTileBytes);
     };
 
     RowState A, B;
@@ -181,7 +198,7 @@ SINGE_DEVICE void paged_attention_pair_body(const PagedAttentionArgs& a, unsigne
     // (tile + 3 at the top of tile's iteration; past the last tile, the last tile's again).
     Pages ready = {};
     {
-        RawPage<FORM> raw[kPairAhead + 1];
+        Lookup raw[kPairAhead + 1];
 #pragma unroll
         for (unsigned int early = 0; early <= kPairAhead; ++early)
             if (tiles > 0) raw[early] = lookup(early < tiles ? early : tiles - 1u);
@@ -242,10 +259,11 @@ SINGE_DEVICE void paged_attention_pair_body(const PagedAttentionArgs& a, unsigne
             // after it go out first and are back with the loads that the end of the iteration waits for.
             const unsigned int wanted = tile + kPairAhead < tiles ? tile + kPairAhead : tiles - 1u;
             const unsigned int after = tile + kPairAhead + 1u < tiles ? tile + kPairAhead + 1u : tiles - 1u;
-            const RawPage<FORM> fresh = lookup(after);
+            const Lookup fresh = lookup(after);
+            const bool tail = is_tail(wanted);
             const Pages now = ready;
-            auto issue_keys = [&](unsigned int i) __attribute__((always_inline)) { load_part(key_bytes, key_chunk, key_lane, wanted, now, i, key_dest); };
-            auto issue_values = [&](unsigned int i) __attribute__((always_inline)) { load_part(value_bytes, value_chunk, value_lane, wanted, now, i, value_dest); };
+            auto issue_keys = [&](unsigned int i) __attribute__((always_inline)) { load_part(key_bytes, key_chunk, key_lane, wanted, tail, now, i, key_dest); };
+            auto issue_values = [&](unsigned int i) __attribute__((always_inline)) { load_part(value_bytes, value_chunk, value_lane, wanted, tail, now, i, value_dest); };
             float largest_a, largest_b;
             bool lagging = fold_pair_block(half, A, B, a_even, b_even, a_odd, b_odd, factor, shift_a, shift_b, largest_a, largest_b, qa, qb, operand,
                                            next_keys, value_origin, values, offsets, issue_keys);
@@ -279,7 +297,7 @@ SINGE_DEVICE void paged_attention_pair_body(const PagedAttentionArgs& a, unsigne
     auto plain_tile = [&](auto&& work) __attribute__((always_inline)) {
         const unsigned int next_stage = (stage + 1) % kPairStages, spare_stage = (stage + kPairAhead) % kPairStages;
         const bool loading = tile + kPairAhead < tiles, looking = tile + kPairAhead + 1u < tiles;
-        RawPage<FORM> fresh = {};
+        Lookup fresh = {};
         if (looking) fresh = lookup(tile + kPairAhead + 1u);
         if (loading) load_tile(tile + kPairAhead, ready, spare_stage);
         work(next_stage);

@@ -412,3 +412,41 @@ def test_two_tiles_a_wave_equals_the_four_wave_kernel_at_the_chunked_prefill_sha
     torch.cuda.synchronize()
     assert (chosen.float() - narrow.float()).abs().max().item() <= 2 ** -6
     assert (chosen_lse - narrow_lse).abs().max().item() <= 1e-4
+
+
+@pytest.mark.parametrize("rows_per_wave", [64, 32])
+@pytest.mark.parametrize("index_dtype", [torch.int32, torch.int64])
+def test_pages_beyond_two_and_four_gib_of_a_cache_read_the_same_as_the_first_pages(rows_per_wave, index_dtype):
+    # 150 000 pages of 32 KiB: a page's first byte lies past 2^31 from id 65 536 and past 2^32 from id 131 072.  The
+    # same page contents under small ids in a small cache must give the same bits.
+    heads, kv_heads, page_size, cache_pages = 32, 8, 16, 150_000
+    sequences = [(300, 700), (256, 512)]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(77)
+    page_counts = [-(-keys // page_size) for _, keys in sequences]
+    used = sum(page_counts)
+    high = torch.tensor([65_536 + 3, 131_072 + 5, cache_pages - 1, 70_001, 140_002, 100_000], dtype=torch.int64)
+    ids_high = torch.cat([high, 90_000 + 7 * torch.arange(used - len(high))])
+    ids_low = torch.randperm(used)
+    small_k = torch.randn((used, page_size, kv_heads, 128), generator=gen, device="cuda").to(torch.bfloat16)
+    small_v = torch.randn((used, page_size, kv_heads, 128), generator=gen, device="cuda").to(torch.bfloat16)
+    big_k = torch.zeros((cache_pages, page_size, kv_heads, 128), device="cuda", dtype=torch.bfloat16)
+    big_v = torch.zeros((cache_pages, page_size, kv_heads, 128), device="cuda", dtype=torch.bfloat16)
+    big_k[ids_high.cuda()] = small_k[ids_low.cuda()]
+    big_v[ids_high.cuda()] = small_v[ids_low.cuda()]
+    tokens = sum(queries for queries, _ in sequences)
+    q = torch.randn((tokens, heads, 128), generator=gen, device="cuda").to(torch.bfloat16)
+    query_offsets = np.concatenate([[0], np.cumsum([queries for queries, _ in sequences])])
+    page_offsets = np.concatenate([[0], np.cumsum(page_counts)])
+    last = [keys - (count - 1) * page_size for (_, keys), count in zip(sequences, page_counts)]
+    index = lambda values: torch.as_tensor(np.asarray(values), dtype=index_dtype).cuda()
+    options = neural.AttentionOptions(causal=True)
+    _native.lib().singe_hip_set_paged_attention_rows_per_wave(rows_per_wave)
+    try:
+        far, far_lse = neural.paged_attention(q, big_k, big_v, neural.Paging(index(query_offsets), index(page_offsets), index(ids_high.numpy()), index(last)), options)
+        near, near_lse = neural.paged_attention(q, small_k, small_v, neural.Paging(index(query_offsets), index(page_offsets), index(ids_low.numpy()), index(last)), options)
+    finally:
+        _native.lib().singe_hip_set_paged_attention_rows_per_wave(0)
+    torch.cuda.synchronize()
+    assert torch.equal(far, near) and torch.equal(far_lse, near_lse)
+    assert far.float().abs().max().item() > 0.1
