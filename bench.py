@@ -51,7 +51,7 @@ COUNTER_TRAFFIC = {
                "source": "profiles/hbm_traffic_counters.md"},
     "prefill": {"kernel": "singe_fmha_prefill_pair_bf16_d128_causal", "FETCH_SIZE": 298455, "WRITE_SIZE": 131077,
                 "source": "profiles/hbm_traffic_counters.md"},
-    "chunked_prefill": {"kernel": "singe_paged_attention_bf16_d128_i32_p16", "FETCH_SIZE": 182466, "WRITE_SIZE": 66571,
+    "chunked_prefill": {"kernel": "singe_paged_attention_pair_bf16_d128_i32", "FETCH_SIZE": 182670, "WRITE_SIZE": 66560,
                         "source": "profiles/hbm_traffic_counters.md"},
     "fp8_decode": {"kernel": "singe_paged_decode_f8kv_wide_d128_b16", "FETCH_SIZE": 2129860, "WRITE_SIZE": 8256,
                    "source": "profiles/hbm_traffic_counters.md"},
@@ -394,6 +394,17 @@ def prefill_section(with_cpu=True, dim=128, key="prefill"):
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": nbytes, "traffic_source": source, **timing_fields(stats)},
     }
+    if dim == 128:
+        # The same launch on all-zero tensors: the same instructions in the same order, but matrix-core operands
+        # that never change a bit.  The device holds a higher clock there, so this figure is what the kernel's
+        # instruction stream allows, and its distance to the figure above is what the data's switching costs.
+        blank = torch.zeros_like(q)
+        quiet = measure(lambda: A.fmha_prefill_bf16(None, out, blank, blank, blank, config), 5)
+        quiet_tflops = flops / (quiet["mean_ms"] * 1e-3) / 1e12
+        result["same_kernel_on_zero_inputs"] = {
+            "what": "the same kernel and sizes on all-zero q, k, v (no operand bit changes: the clock is not held back)",
+            "ms_per_step": quiet["mean_ms"], "tflops": quiet_tflops, "frac": quiet_tflops / MFMA_BF16_PEAK_TFLOPS,
+            **timing_fields(quiet)}
     if with_cpu:
         result["cpu_baseline"] = prefill_cpu_baseline(q, k, v, scale)
     return result
@@ -1062,6 +1073,9 @@ def compact(result):
     for label, name in (("3_prefill", "prefill"), ("4_chunked_prefill", "chunked_prefill"), ("5_fp8_decode", "fp8_decode")):
         if "unsupported" not in result.get(name, {"unsupported": 1}):
             configs[label] = _config_summary(result[name])
+    if "same_kernel_on_zero_inputs" in result.get("prefill", {}) and "3_prefill" in configs:
+        # (the same launch on all-zero tensors: what the instruction stream allows where the clock is not held back)
+        configs["3_prefill"]["frac_on_zero_inputs"] = _rounded(result["prefill"]["same_kernel_on_zero_inputs"]["frac"])
     if "5_fp8_decode" in configs:
         configs["5_fp8_decode"]["whole_op_frac"] = _rounded(result["fp8_decode"]["pct_hbm_peak"] / 100.0)
     roofline["configs"] = configs
