@@ -90,8 +90,9 @@ int32_t prefill_f32(void* stream, float* out, size_t out_len, float* lse, size_t
     if (int32_t status = validate_call(c, out, out_len, lse, lse_len, with_lse, query, query_len, key, key_len, value, value_len))
         return status;
     if (c.head_dim > 256) return fail(SINGE_HIP_UNSUPPORTED_WIDTH, op, c.head_dim, 0);
+    // (the cap first, then the window: validate_softcapped_window_attention_config, singe-kernel/src/cuda/attention/mod.rs:3418-3430)
+    if (has_soft_cap && !(std::isfinite(soft_cap) && soft_cap > 0.0f)) return fail(SINGE_HIP_INVALID_LENGTH, "soft_cap");
     if (!fits_i32(window_size)) return fail(SINGE_HIP_LENGTH_EXCEEDS_I32, "window_size");
-    if (has_soft_cap && !(std::isfinite(soft_cap) && soft_cap != 0.0f)) return fail(SINGE_HIP_INVALID_LENGTH, "soft_cap");
     PrefillF32Args args;
     args.query = query;
     args.key = key;
@@ -144,12 +145,11 @@ int32_t prefill_f32(void* stream, float* out, size_t out_len, float* lse, size_t
     return launch(kernel, static_cast<unsigned>(groups), 1, 1, 256, stream, args);
 }
 
-// Whether a call without options runs on the kernel that gives a wave two 32-row tiles: head_dim 128, every key tile
-// whole, a positive scale, no heads packed into one tile, and (unless the knob says 64) 256-row tiles that still fill
-// the chip.
+// Whether a call without options runs on the kernel that gives a wave two 32-row tiles: head_dim 128, a positive
+// scale, no heads packed into one tile, and (unless the knob says 64) 256-row tiles that still fill the chip.
 bool two_tiles_a_wave(const SingeFmhaPrefillConfig& c) {
     const uint32_t wanted = g_rows_per_wave.load(std::memory_order_relaxed);
-    if (wanted == 32 || c.head_dim != 128 || c.key_len == 0 || c.key_len % 64 != 0 || !(c.scale > 0.0f) || dense_prefill_packs_heads(c))
+    if (wanted == 32 || c.head_dim != 128 || c.key_len == 0 || !(c.scale > 0.0f) || dense_prefill_packs_heads(c))
         return false;
     const uint64_t rows = (static_cast<uint64_t>(c.batch) * c.heads + 7) / 8 * 8, pair_tiles = (c.query_len + 255) / 256;
     return wanted == 64 || rows * ((pair_tiles + 1) / 2) >= compute_units();
@@ -251,12 +251,13 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
     }
     const long long head_dim = static_cast<long long>(c.head_dim);
     // Long rows without options at head_dim 128: the kernel that gives a wave two 32-row tiles (256 query rows a
-    // workgroup, one workgroup a compute unit), when every key tile is whole and its launch still fills the chip.
+    // workgroup, one workgroup a compute unit), when its launch still fills the chip; a build of its own where the last
+    // key tile is not whole.
     if (!with_options && options.sinks == nullptr && options.key_lengths == nullptr && splits == 1 && two_tiles_a_wave(c)) {
         const uint32_t pair_tiles = static_cast<uint32_t>((c.query_len + 255) / 256);
         const uint64_t pair_groups = rows * ((pair_tiles + 1) / 2);
         args.query_tiles = pair_tiles;
-        const KernelId pair = static_cast<KernelId>(kPrefillPair + (c.causal ? 0 : 1) + (f16 ? 2 : 0));
+        const KernelId pair = static_cast<KernelId>(kPrefillPair + (c.causal ? 0 : 1) + (f16 ? 2 : 0) + (c.key_len % 64 != 0 ? 4 : 0));
         return launch(pair, static_cast<unsigned>(pair_groups), 1, 1, 256, stream, args);
     }
     const KernelId kernel = static_cast<KernelId>((f16 ? kPrefillCausalF16 : kPrefillCausal) + (c.causal ? 0 : 1) + (with_options ? 4 : 0));

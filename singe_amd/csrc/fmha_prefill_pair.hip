@@ -17,9 +17,9 @@
 //     part of the schedule (at least four slots, some thirty instructions), since the compiler does not see a
 //     matrix instruction there.
 // query/out [batch, query_len, heads, 128], key/value [batch, key_len, kv_heads, 128] with element strides from
-// FmhaPrefillConfig; lse [batch, heads, query_len], natural log.  The host sends calls here whose key_len is a
-// multiple of 64 (every tile whole) and that fill the chip with 256-row tiles; everything else stays on
-// fmha_prefill.hip.
+// FmhaPrefillConfig; lse [batch, heads, query_len], natural log.  The host sends calls here that fill the chip with
+// 256-row tiles; everything else stays on fmha_prefill.hip.  A last tile of fewer than 64 keys re-reads the last key
+// in its spare rows and takes the masked path, like the tile on the causal diagonal.
 //
 // Grid: one workgroup of four waves per (batch, head, pair of 256-row query tiles), tile i from the end and tile i
 // from the start; ids laid out as in fmha_prefill.hip.  LDS: four stages of K and four of V (128 KiB), each tile
@@ -32,8 +32,9 @@ namespace {
 
 using namespace prefill;
 
-// One 256-row query tile of (batch, head) pair `bh`.
-template <bool CAUSAL, class Half>
+// One 256-row query tile of (batch, head) pair `bh`.  RAGGED: key_len is not a multiple of 64 (a build of its own:
+// the extra code of the last tile costs the other build instruction-cache room, 4 % under the causal mask).
+template <bool CAUSAL, bool RAGGED, class Half>
 SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* lds, unsigned int bh, unsigned int query_tile) {
     constexpr unsigned int kLoadRows = 4u * kPairWaves;  // key rows one load instruction of every wave brings in
     const unsigned int tid = threadIdx.x, lane = tid & 63;
@@ -41,7 +42,7 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
     const unsigned int column = lane & 31, hi = lane >> 5;
     const unsigned int group = a.heads / a.kv_heads;
     const unsigned int batch = bh / a.heads, head = bh % a.heads, kv_head = head / group;
-    const unsigned int key_len = a.key_len;  // a multiple of 64 (the host's gate)
+    const unsigned int key_len = a.key_len;  // at least one key, and a multiple of 64 unless RAGGED (the host's gate)
 
     const unsigned int first_row = query_tile * kPairRows + wave * 64u;  // of this wave: tile A, then tile B 32 rows on
     const unsigned int query_a = first_row + column, query_b = query_a + 32u;
@@ -67,17 +68,21 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
     }
     const uint4 no_query[kSteps] = {};  // the masked path's folding functions take a Q^T they do not read
 
-    // Tiles of keys the workgroup visits, and how many of them this wave folds without a mask: under the causal mask
-    // the tile that holds the wave's own rows (index first_row / 64) is its last and takes the masked path.
+    // Tiles of keys the workgroup visits, how many of them this wave folds without a mask, and whether one more takes
+    // the masked path: under the causal mask the tile that holds the wave's own rows (index first_row / 64), and with or
+    // without it a last tile that is not whole.
     unsigned int key_end = key_len;
     if (CAUSAL) {
         const unsigned int reach = query_tile * kPairRows + kPairRows;
         key_end = key_end < reach ? key_end : reach;
     }
-    const unsigned int tiles = key_end / kKeyTile;
-    unsigned int interior_tiles = tiles;
-    if (CAUSAL) interior_tiles = first_row / kKeyTile < tiles ? first_row / kKeyTile : tiles;
-    const bool has_diagonal = CAUSAL && interior_tiles < tiles;
+    const unsigned int tiles = (key_end + kKeyTile - 1) / kKeyTile, whole_tiles = key_end / kKeyTile;
+    unsigned int interior_tiles = whole_tiles;
+    if (CAUSAL) interior_tiles = first_row / kKeyTile < whole_tiles ? first_row / kKeyTile : whole_tiles;
+    const bool has_masked_tile = interior_tiles < tiles;  // (its index is interior_tiles)
+    // The last key tile A and tile B see anything of, as the first key past it.
+    const unsigned int reach_a = CAUSAL && first_row + 32u < key_len ? first_row + 32u : key_len;
+    const unsigned int reach_b = CAUSAL && first_row + 64u < key_len ? first_row + 64u : key_len;
 
     // The loads of a tile, as in fmha_prefill.hip: instruction i of wave w fills rows 16 i + 4 w .. + 3 of the stage.
     const unsigned int key_stride_bytes = static_cast<unsigned int>(a.key_sequence_stride) * 2u;
@@ -85,13 +90,28 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
     const unsigned int load_row = 4u * wave + (lane >> 4), position = lane & 15u;
     const unsigned int key_lane = load_row * key_stride_bytes + (position ^ (load_row & 15u)) * 16u;
     const unsigned int value_lane = load_row * value_stride_bytes + (position ^ (4u * (load_row & 3u))) * 16u;
-    auto load_part = [&](const unsigned char* base, unsigned int stride_bytes, unsigned int lane_offset, unsigned int i,
+    const unsigned int key_chunk = (position ^ (load_row & 15u)) * 16u, value_chunk = (position ^ (4u * (load_row & 3u))) * 16u;
+    // The lane's offsets into a tile, one a load.  A last tile that is not whole has offsets of its own: its rows past
+    // the last key re-read that key (they are masked; what lies behind the last key is not this call's to read).  Both
+    // sets are worked out here, so that a load in the loop picks one with a single select and no branch.
+    unsigned int key_offsets[4], value_offsets[4], key_tail_offsets[4], value_tail_offsets[4];
+#pragma unroll
+    for (unsigned int i = 0; i < 4; ++i) {
+        const unsigned int row = kLoadRows * i + load_row, last = (key_len - 1u) % kKeyTile;
+        const unsigned int kept = row < last ? row : last;
+        key_offsets[i] = key_lane + kLoadRows * i * key_stride_bytes;
+        value_offsets[i] = value_lane + kLoadRows * i * value_stride_bytes;
+        key_tail_offsets[i] = kept * key_stride_bytes + key_chunk;
+        value_tail_offsets[i] = kept * value_stride_bytes + value_chunk;
+    }
+    auto load_part = [&](const unsigned char* base, const unsigned int (&whole)[4], const unsigned int (&tailed)[4], bool tail, unsigned int i,
                          unsigned char* stage) __attribute__((always_inline)) {
-        unsigned int offset = lane_offset + kLoadRows * i * stride_bytes;
+        unsigned int offset = tail ? tailed[i] : whole[i];
         asm volatile("" : "+v"(offset));  // a 32-bit offset next to the load keeps its scalar-base form
         __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(base + offset),
                                          (lds_words_t)(stage + (kLoadRows * i + 4u * wave) * kRowBytes), 16, 0, 0);
     };
+    auto is_tail = [&](unsigned int tile) __attribute__((always_inline)) { return RAGGED && tile * kKeyTile + kKeyTile > key_len; };
     auto tile_base = [&](const unsigned char* rows, unsigned int stride_bytes, unsigned int tile) __attribute__((always_inline)) {
         const unsigned char* base = rows + static_cast<size_t>(tile * kKeyTile) * stride_bytes;
         asm("" : "+s"(base));
@@ -100,10 +120,12 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
     auto load_tile = [&](unsigned int tile, unsigned int stage) __attribute__((always_inline)) {
         const unsigned char* keys = tile_base(k_bytes, key_stride_bytes, tile);
         const unsigned char* values = tile_base(v_bytes, value_stride_bytes, tile);
+        const bool tail = is_tail(tile);
 #pragma unroll
-        for (unsigned int i = 0; i < 4; ++i) load_part(keys, key_stride_bytes, key_lane, i, lds + stage * kTileBytes);
+        for (unsigned int i = 0; i < 4; ++i) load_part(keys, key_offsets, key_tail_offsets, tail, i, lds + stage * kTileBytes);
 #pragma unroll
-        for (unsigned int i = 0; i < 4; ++i) load_part(values, value_stride_bytes, value_lane, i, lds + kPairValueBase + stage * kTileBytes);
+        for (unsigned int i = 0; i < 4; ++i)
+            load_part(values, value_offsets, value_tail_offsets, tail, i, lds + kPairValueBase + stage * kTileBytes);
     };
 
     RowState A, B;
@@ -118,7 +140,7 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
 
     f32x16_t a_even, b_even, a_odd, b_odd;  // raw scores of the block folded next (even / odd blocks of a tile)
     unsigned int tile = 0, stage = 0;       // stage = tile % 4
-    if (interior_tiles > 0 || has_diagonal) {
+    if (interior_tiles > 0 || has_masked_tile) {
         score_block_pair(half, a_even, qa, lds, offsets);
         score_block_pair(half, b_even, qb, lds, offsets);
     }
@@ -151,15 +173,20 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
             const unsigned int wanted = tile + kPairAhead < tiles ? tile + kPairAhead : tiles - 1;
             const unsigned char* key_rows = tile_base(k_bytes, key_stride_bytes, wanted);
             const unsigned char* value_rows = tile_base(v_bytes, value_stride_bytes, wanted);
-            auto issue_keys = [&](unsigned int i) __attribute__((always_inline)) { load_part(key_rows, key_stride_bytes, key_lane, i, key_dest); };
-            auto issue_values = [&](unsigned int i) __attribute__((always_inline)) { load_part(value_rows, value_stride_bytes, value_lane, i, value_dest); };
+            const bool tail = is_tail(wanted);
+            auto issue_keys = [&](unsigned int i) __attribute__((always_inline)) {
+                load_part(key_rows, key_offsets, key_tail_offsets, tail, i, key_dest);
+            };
+            auto issue_values = [&](unsigned int i) __attribute__((always_inline)) {
+                load_part(value_rows, value_offsets, value_tail_offsets, tail, i, value_dest);
+            };
             float largest_a, largest_b;
             bool lagging = fold_pair_block(half, A, B, a_even, b_even, a_odd, b_odd, factor, shift_a, shift_b, largest_a, largest_b, qa, qb, operand,
                                   next_keys, value_origin, values, offsets, issue_keys);
             if (lagging) settle(largest_a, largest_b);
             lagging = fold_pair_block(half, A, B, a_odd, b_odd, a_even, b_even, factor, shift_a, shift_b, largest_a, largest_b, qa, qb, operand,
                                    next_keys + kBlockBytes, value_origin, values + kBlockBytes, offsets, issue_values);
-            // (past the wave's last unmasked tile the scores just computed are the diagonal tile's, which the masked path
+            // (past the wave's last unmasked tile the scores just computed are the masked tile's, which that path
             // takes as they are, or nobody's)
             if (lagging && tile + 1 < interior_tiles) settle(largest_a, largest_b);
             older_loads_landed();  // the next tile's; the eight of this iteration have another tile's time
@@ -180,22 +207,43 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
             ++tile;
         }
     }
-    // The tile on the diagonal: block 2 t holds the keys of tile A's rows (B sees all of it), block 2 t + 1 those of
-    // tile B's rows (A sees none of it).
-    if (has_diagonal) {
+    // The tile a mask touches: on the causal diagonal block 2 t holds the keys of tile A's rows (B sees all of it) and
+    // block 2 t + 1 those of tile B's rows (A sees none of it); a last tile that is not whole ends where the keys end.
+    if (has_masked_tile) {
         const unsigned int next_stage = (stage + 1) % kPairStages, spare_stage = (stage + kPairAhead) % kPairStages;
         const unsigned char* keys = lds + stage * kTileBytes;
         const unsigned char* values = lds + kPairValueBase + stage * kTileBytes;
         const bool loading = tile + kPairAhead < tiles;
         if (loading) load_tile(tile + kPairAhead, spare_stage);
         const unsigned int key0 = tile * kKeyTile;
-        const float edge_a = begin_block(A, a_even, hi, factor, true, [&](unsigned int key_in_block) { return key0 + key_in_block > query_a; });
-        finish_block<false>(half, A, a_even, factor, edge_a, values, offsets, a_even, no_query, values);
-        const float whole_b = begin_block(B, b_even, hi, factor, false, [](unsigned int) { return false; });
-        finish_block<false>(half, B, b_even, factor, whole_b, values, offsets, b_even, no_query, values);
-        score_block_pair(half, b_odd, qb, keys + kBlockBytes, offsets);
-        const float edge_b = begin_block(B, b_odd, hi, factor, true, [&](unsigned int key_in_block) { return key0 + 32u + key_in_block > query_b; });
-        finish_block<false>(half, B, b_odd, factor, edge_b, values + kBlockBytes, offsets, b_odd, no_query, values);
+        if constexpr (!RAGGED) {
+            // (the causal diagonal: A masked, B whole; then B masked)
+            const float edge_a = begin_block(A, a_even, hi, factor, true, [&](unsigned int key_in_block) { return key0 + key_in_block > query_a; });
+            finish_block<false>(half, A, a_even, factor, edge_a, values, offsets, a_even, no_query, values);
+            const float whole_b = begin_block(B, b_even, hi, factor, false, [](unsigned int) { return false; });
+            finish_block<false>(half, B, b_even, factor, whole_b, values, offsets, b_even, no_query, values);
+            score_block_pair(half, b_odd, qb, keys + kBlockBytes, offsets);
+            const float edge_b = begin_block(B, b_odd, hi, factor, true, [&](unsigned int key_in_block) { return key0 + 32u + key_in_block > query_b; });
+            finish_block<false>(half, B, b_odd, factor, edge_b, values + kBlockBytes, offsets, b_odd, no_query, values);
+        } else {
+            // One block of one row tile, masked by the last key each row sees (its own under the causal mask, and never
+            // past the last key there is).
+            auto fold = [&](RowState& state, f32x16_t& s, unsigned int query, unsigned int first_key, const unsigned char* block_values) __attribute__((always_inline)) {
+                const unsigned int last_seen = CAUSAL && query < key_len - 1u ? query : key_len - 1u;
+                const float shift = begin_block(state, s, hi, factor, true, [&](unsigned int key_in_block) { return first_key + key_in_block > last_seen; });
+                finish_block<false>(half, state, s, factor, shift, block_values, offsets, s, no_query, block_values);
+            };
+            if (key0 < reach_a) fold(A, a_even, query_a, key0, values);
+            if (key0 < reach_b) fold(B, b_even, query_b, key0, values);
+            if (key0 + 32u < reach_a) {
+                score_block_pair(half, a_odd, qa, keys + kBlockBytes, offsets);
+                fold(A, a_odd, query_a, key0 + 32u, values + kBlockBytes);
+            }
+            if (key0 + 32u < reach_b) {
+                score_block_pair(half, b_odd, qb, keys + kBlockBytes, offsets);
+                fold(B, b_odd, query_b, key0 + 32u, values + kBlockBytes);
+            }
+        }
         if (loading) older_loads_landed(); else loads_landed();
         __syncthreads();
         stage = next_stage;
@@ -236,7 +284,7 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
 }
 
 // Workgroup id -> (batch * heads + head, pair of query tiles), as in fmha_prefill.hip; query_tiles counts 256-row tiles.
-template <bool CAUSAL, class Half>
+template <bool CAUSAL, bool RAGGED, class Half>
 SINGE_DEVICE void fmha_prefill_pair_body(const PrefillArgs& a, unsigned char* lds) {
     const unsigned int xcd = blockIdx.x & 7u, within = blockIdx.x >> 3;
     const unsigned int pairs = (a.query_tiles + 1u) / 2u;
@@ -247,18 +295,22 @@ SINGE_DEVICE void fmha_prefill_pair_body(const PrefillArgs& a, unsigned char* ld
     // the instruction cache)
 #pragma nounroll
     for (unsigned int which = 0; which < (light != heavy ? 2u : 1u); ++which)
-        fmha_prefill_pair_tile<CAUSAL, Half>(a, lds, bh, which == 0 ? heavy : light);
+        fmha_prefill_pair_tile<CAUSAL, RAGGED, Half>(a, lds, bh, which == 0 ? heavy : light);
 }
 
 }  // namespace
 
-#define SINGE_FMHA_PREFILL_PAIR_KERNEL(NAME, CAUSAL, HALF)                                             \
+#define SINGE_FMHA_PREFILL_PAIR_KERNEL(NAME, CAUSAL, RAGGED, HALF)                                     \
     extern "C" __global__ __launch_bounds__(64 * kPairWaves, 1) void NAME(PrefillArgs args) {          \
         __shared__ __attribute__((aligned(1024))) unsigned char prefill_lds[kPairLdsBytes];            \
-        fmha_prefill_pair_body<CAUSAL, prefill::HALF>(args, prefill_lds);                              \
+        fmha_prefill_pair_body<CAUSAL, RAGGED, prefill::HALF>(args, prefill_lds);                      \
     }
 
-SINGE_FMHA_PREFILL_PAIR_KERNEL(singe_fmha_prefill_pair_bf16_d128_causal, true, Bf16)
-SINGE_FMHA_PREFILL_PAIR_KERNEL(singe_fmha_prefill_pair_bf16_d128_full, false, Bf16)
-SINGE_FMHA_PREFILL_PAIR_KERNEL(singe_fmha_prefill_pair_f16_d128_causal, true, F16)
-SINGE_FMHA_PREFILL_PAIR_KERNEL(singe_fmha_prefill_pair_f16_d128_full, false, F16)
+SINGE_FMHA_PREFILL_PAIR_KERNEL(singe_fmha_prefill_pair_bf16_d128_causal, true, false, Bf16)
+SINGE_FMHA_PREFILL_PAIR_KERNEL(singe_fmha_prefill_pair_bf16_d128_full, false, false, Bf16)
+SINGE_FMHA_PREFILL_PAIR_KERNEL(singe_fmha_prefill_pair_f16_d128_causal, true, false, F16)
+SINGE_FMHA_PREFILL_PAIR_KERNEL(singe_fmha_prefill_pair_f16_d128_full, false, false, F16)
+SINGE_FMHA_PREFILL_PAIR_KERNEL(singe_fmha_prefill_pair_bf16_d128_causal_ragged, true, true, Bf16)
+SINGE_FMHA_PREFILL_PAIR_KERNEL(singe_fmha_prefill_pair_bf16_d128_full_ragged, false, true, Bf16)
+SINGE_FMHA_PREFILL_PAIR_KERNEL(singe_fmha_prefill_pair_f16_d128_causal_ragged, true, true, F16)
+SINGE_FMHA_PREFILL_PAIR_KERNEL(singe_fmha_prefill_pair_f16_d128_full_ragged, false, true, F16)

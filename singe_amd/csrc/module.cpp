@@ -314,6 +314,8 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_decode_combine_few_bf16_d112", "singe_paged_decode_combine_few_f16_d112",
     "singe_fmha_prefill_pair_bf16_d128_causal", "singe_fmha_prefill_pair_bf16_d128_full",
     "singe_fmha_prefill_pair_f16_d128_causal", "singe_fmha_prefill_pair_f16_d128_full",
+    "singe_fmha_prefill_pair_bf16_d128_causal_ragged", "singe_fmha_prefill_pair_bf16_d128_full_ragged",
+    "singe_fmha_prefill_pair_f16_d128_causal_ragged", "singe_fmha_prefill_pair_f16_d128_full_ragged",
     "singe_paged_attention_pair_bf16_d128_i32", "singe_paged_attention_pair_bf16_d128_i64",
     "singe_paged_attention_pair_f16_d128_i32", "singe_paged_attention_pair_f16_d128_i64",
 };
@@ -357,7 +359,7 @@ constexpr PartRun kPartRuns[] = {
     {3, 12}, {15, 12}, {19, 12}, {21, 12}, {23, 12}, {25, 12}, {27, 12}, {29, 12},  // the further fused-rotation kernels
     {8, 4},                       // latent attention on the matrix cores at any width it takes
     {30, 14}, {31, 14}, {32, 14}, {33, 14}, {34, 14}, {35, 14},  // the decode kernels and their merges for 32, 16, 48, 80, 96, 112
-    {36, 4},                      // the dense prefill with two row tiles a wave
+    {36, 8},                      // the dense prefill with two row tiles a wave (whole key tiles, then a last tile that is not)
     {37, 4},                      // the paged attention op on the same loop
 };
 constexpr int runs_total() {

@@ -84,10 +84,11 @@ enum KernelId : int {
     // and with one or two (bf16, f16)
     kDecodeOtherHeadDims,
     // the dense prefill that gives a wave two 32-row tiles (head_dim 128, no options): + (no causal mask) + 2 * f16
+    // + 4 * (key_len not a multiple of 64)
     kPrefillPair = kDecodeOtherHeadDims + 6 * 14,
     // the paged attention op on the same two-tile loop (head_dim 128, page sizes that are powers of two from 16, no
     // options): + (i64 indices) + 2 * f16
-    kPagedPair = kPrefillPair + 4,
+    kPagedPair = kPrefillPair + 8,
     kKernelCount = kPagedPair + 4
 };
 

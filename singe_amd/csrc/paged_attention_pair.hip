@@ -165,16 +165,22 @@ SINGE_DEVICE void paged_attention_pair_body(const PagedAttentionArgs& a, unsigne
             pages.start[i] = (static_cast<unsigned long long>(static_cast<unsigned int>(__builtin_amdgcn_readlane(upper, i))) << 32) |
                              static_cast<unsigned int>(__builtin_amdgcn_readlane(low, i));
     };
-    // `tail`: the tile holds the sequence's last key or lies past it, so some of its rows re-read that key.
-    auto load_part = [&](const unsigned char* cache, unsigned int chunk, unsigned int lane_offset, unsigned int tile, bool tail, const Pages& pages,
+    // The lane's offsets inside a group, for K and for V; the tile that holds the sequence's last key has offsets of its
+    // own, one a group: rows past that key re-read it, and a group that lies past it is the last group again.  Both are
+    // worked out here, so that a load in the loop picks one with a single select and no branch.
+    unsigned int key_tail_lane[4], value_tail_lane[4];
+#pragma unroll
+    for (unsigned int i = 0; i < 4; ++i) {
+        const unsigned int last = tiles > 0 ? keys - 1u - group_of((keys - 1u) / kKeyTile, i) : 0u;
+        const unsigned int kept = load_row < last ? load_row : last;
+        key_tail_lane[i] = kept * slot_bytes + key_chunk;
+        value_tail_lane[i] = kept * slot_bytes + value_chunk;
+    }
+    // `tail`: the tile holds the sequence's last key and is not whole.
+    auto load_part = [&](const unsigned char* cache, unsigned int lane_offset, const unsigned int (&tail_lane)[4], bool tail, const Pages& pages,
                          unsigned int i, unsigned char* stage) __attribute__((always_inline)) {
         const unsigned char* base = cache + pages.start[i];
-        unsigned int offset = lane_offset;
-        if (__builtin_expect(tail, 0)) {
-            const unsigned int last = keys - 1u - group_of(tile, i);
-            offset = (load_row < last ? load_row : last) * slot_bytes + chunk;
-            asm volatile("" : "+v"(offset));  // (keeps the branch a branch)
-        }
+        unsigned int offset = tail ? tail_lane[i] : lane_offset;
         asm("" : "+s"(base));
         asm volatile("" : "+v"(offset));
         __builtin_amdgcn_global_load_lds(reinterpret_cast<const unsigned int*>(base + offset),
@@ -183,10 +189,10 @@ SINGE_DEVICE void paged_attention_pair_body(const PagedAttentionArgs& a, unsigne
     auto is_tail = [&](unsigned int tile) __attribute__((always_inline)) { return tile * kKeyTile + kKeyTile > keys; };
     auto load_tile = [&](unsigned int tile, const Pages& pages, unsigned int stage) __attribute__((always_inline)) {
 #pragma unroll
-        for (unsigned int i = 0; i < 4; ++i) load_part(key_bytes, key_chunk, key_lane, tile, is_tail(tile), pages, i, lds + stage * kTileBytes);
+        for (unsigned int i = 0; i < 4; ++i) load_part(key_bytes, key_lane, key_tail_lane, is_tail(tile), pages, i, lds + stage * kTileBytes);
 #pragma unroll
         for (unsigned int i = 0; i < 4; ++i)
-            load_part(value_bytes, value_chunk, value_lane, tile, is_tail(tile), pages, i, lds + kPairValueBase + stage * kTileBytes);
+            load_part(value_bytes, value_lane, value_tail_lane, is_tail(tile), pages, i, lds + kPairValueBase + stage * kTileBytes);
     };
 
     RowState A, B;
@@ -262,8 +268,8 @@ SINGE_DEVICE void paged_attention_pair_body(const PagedAttentionArgs& a, unsigne
             const Lookup fresh = lookup(after);
             const bool tail = is_tail(wanted);
             const Pages now = ready;
-            auto issue_keys = [&](unsigned int i) __attribute__((always_inline)) { load_part(key_bytes, key_chunk, key_lane, wanted, tail, now, i, key_dest); };
-            auto issue_values = [&](unsigned int i) __attribute__((always_inline)) { load_part(value_bytes, value_chunk, value_lane, wanted, tail, now, i, value_dest); };
+            auto issue_keys = [&](unsigned int i) __attribute__((always_inline)) { load_part(key_bytes, key_lane, key_tail_lane, tail, now, i, key_dest); };
+            auto issue_values = [&](unsigned int i) __attribute__((always_inline)) { load_part(value_bytes, value_lane, value_tail_lane, tail, now, i, value_dest); };
             float largest_a, largest_b;
             bool lagging = fold_pair_block(half, A, B, a_even, b_even, a_odd, b_odd, factor, shift_a, shift_b, largest_a, largest_b, qa, qb, operand,
                                            next_keys, value_origin, values, offsets, issue_keys);

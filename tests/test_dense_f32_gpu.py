@@ -72,3 +72,15 @@ def test_softcapped_window_f32(window, cap):
                                                   query_len=lq, key_len=lk, heads=heads, kv_heads=kv_heads, head_dim=dim,
                                                   scale=0.3, causal=True, window_size=window, soft_cap=cap)
     assert np.abs(out.cpu().numpy() - want).max() <= TOL
+
+
+@pytest.mark.parametrize("cap", [0.0, -2.5, float("inf"), float("nan")])
+def test_softcapped_window_f32_refuses_a_cap_that_is_not_positive_and_finite(cap):
+    # validate_softcapped_window_attention_config: a cap must be finite and above zero, and is looked at before the window
+    from singe_amd import error
+    batch, heads, lq, dim = 1, 2, 8, 32
+    q = torch.zeros((batch, heads, lq, dim), device="cuda")
+    out = torch.zeros_like(q)
+    config = A.bhsd_config(batch, heads, heads, lq, lq, dim, 0.3, True)
+    with pytest.raises(error.InvalidLength):
+        A.softcapped_window_attention_f32(None, out, q, q, q, A.SoftcappedWindowAttentionConfig(config, 2 ** 40, cap))

@@ -154,11 +154,32 @@ def two_tiles_a_wave():
 @pytest.mark.parametrize("batch,query_len,key_len,heads,kv_heads", [
     (1, 256, 256, 1, 1), (2, 512, 512, 4, 2), (1, 64, 64, 2, 2), (1, 100, 128, 3, 1), (1, 1, 64, 1, 1),
     (1, 300, 192, 2, 2), (1, 1024, 1024, 8, 8), (1, 640, 1024, 4, 1), (1, 1024, 320, 2, 1), (3, 768, 768, 2, 1),
+    # key counts that leave a last tile of 1, 63, 33, 32 and 31 keys, fewer keys than a tile, and rows past the last key
+    (1, 257, 257, 2, 1), (1, 1000, 1000, 2, 2), (2, 300, 191, 2, 1), (1, 97, 97, 1, 1), (1, 512, 160, 2, 2), (1, 350, 607, 3, 3),
+    (1, 40, 33, 1, 1), (1, 700, 63, 2, 1), (1, 64, 1, 1, 1),
 ])
 def test_two_tiles_a_wave_matches_oracle(two_tiles_a_wave, batch, query_len, key_len, heads, kv_heads, causal):
     q, k, v = make(batch, query_len, key_len, heads, kv_heads, seed=query_len * 11 + key_len)
     got, lse, want, want_lse = run(q, k, v, causal)
     check(got, lse, want, want_lse, f"two tiles: {batch}x{query_len}x{key_len} h{heads}/{kv_heads} causal={causal}")
+
+
+@pytest.mark.parametrize("rows_per_wave", [64, 32])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("key_len", [1, 63, 65, 250, 1000])
+def test_rows_behind_the_last_key_are_not_read(rows_per_wave, causal, key_len):
+    # keys and values are the front of buffers whose rows behind the last key hold NaN: a last tile that is not whole
+    # must re-read its last key there (a NaN value under a zero weight would still be a NaN)
+    from singe_amd import _native
+    q, k_all, v_all = make(1, 384, key_len + 96, 2, 1, seed=key_len + 5)
+    k_all[:, key_len:] = float("nan")
+    v_all[:, key_len:] = float("nan")
+    _native.lib().singe_hip_set_dense_prefill_rows_per_wave(rows_per_wave)
+    try:
+        got, lse, want, want_lse = run(q, k_all[:, :key_len], v_all[:, :key_len], causal)
+    finally:
+        _native.lib().singe_hip_set_dense_prefill_rows_per_wave(0)
+    check(got, lse, want, want_lse, f"NaN behind key {key_len}, causal={causal}, {rows_per_wave} rows a wave")
 
 
 def test_two_tiles_a_wave_negative_scale_and_no_lse(two_tiles_a_wave):
