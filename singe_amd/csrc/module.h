@@ -89,7 +89,9 @@ enum KernelId : int {
     // the paged attention op on the same two-tile loop (head_dim 128, page sizes that are powers of two from 16, no
     // options): + (i64 indices) + 2 * f16
     kPagedPair = kPrefillPair + 8,
-    kKernelCount = kPagedPair + 4
+    // the head_dim 64 builds of the two-tile dense prefill, in kPrefillPair's order
+    kPrefillPairD64 = kPagedPair + 4,
+    kKernelCount = kPrefillPairD64 + 8
 };
 
 
@@ -158,7 +160,7 @@ inline int rotary_paged_attention_base(bool f16, bool softcap, long long head_di
 extern const char* const kKernelNames[kKernelCount];
 
 // Parts of the code object (one file each) and the part a kernel lives in.
-constexpr int kPartCount = 38;
+constexpr int kPartCount = 39;
 extern const char* const kPartNames[kPartCount];
 int kernel_part(int kernel);
 

@@ -2,14 +2,15 @@
 // (fmha_prefill_pair.hip says why and how; paged_attention_pair.hip is the same loop over a paged cache): the score
 // products as assembly with their register classes spelled out, Q^T loaded straight into accumulation registers, the
 // row maxima of two score tiles in alternating chains, and fold_pair_block, one 32-key block of both tiles with its
-// vector work dealt out over the 32 slots between its matrix instructions.
+// vector work dealt out over the slots between its matrix instructions (32 at head_dim 128, 16 at 64: the text of the
+// block is written by prefill_pair_deal.py).
 #pragma once
 
 #include "prefill_blocks.hip.h"
 
 namespace prefill {
 
-static_assert(kHeadDim == 128, "the two-tile kernel is built for head_dim 128");
+static_assert(kHeadDim == 128 || kHeadDim == 64, "the two-tile kernels are built for head_dim 128 and 64");
 
 constexpr int kPairWaves = 4;
 constexpr unsigned int kPairRows = 64u * kPairWaves;  // query rows of a workgroup
@@ -107,10 +108,10 @@ SINGE_DEVICE void row_maxima_2(float& ma, float& mb) {
 template <class Half, class Issue>
 SINGE_DEVICE bool fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t& a_cur, f32x16_t& b_cur, f32x16_t& a_nxt, f32x16_t& b_nxt,
                                   float factor, float shift_a, float shift_b, float& largest_a_out, float& largest_b_out,
-                                  const u32x4_t (&qa)[8], const u32x4_t (&qb)[8], uint4 (&operand)[8], const unsigned char* __restrict__ keys_after,
+                                  const u32x4_t (&qa)[kSteps], const u32x4_t (&qb)[kSteps], uint4 (&operand)[kSteps], const unsigned char* __restrict__ keys_after,
                                   const unsigned char* __restrict__ value_origin, unsigned int values, const ReadOffsets& offsets, Issue&& issue) {
     unsigned int wa[2][4], wb[2][4];
-    v8i16_t v[2][4];
+    v8i16_t v[2][kDimBlocks];
     float total_a = 0.0f, total_b = 0.0f;
     float largest_a, other_a, largest_b, other_b;
     bool lagging;
@@ -136,238 +137,11 @@ SINGE_DEVICE bool fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t&
         const v4i16_t high = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_t)(value_origin + offsets.value(D) + (values + (16 * (H) + 8) * kRowBytes))); \
         v[H][D] = __builtin_shufflevector(low, high, 0, 1, 2, 3, 4, 5, 6, 7);                                                        \
     }
-    // slot 0
-    QK(a_nxt, qa, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    issue(0);
-    E(a_cur, 0, shift_a);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 1
-    QK(b_nxt, qb, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    E(a_cur, 1, shift_a);
-    T(total_a, a_cur, 0);
-    E(a_cur, 2, shift_a);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 2
-    QK(a_nxt, qa, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    issue(1);
-    T(total_a, a_cur, 1);
-    E(a_cur, 3, shift_a);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 3
-    QK(b_nxt, qb, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    T(total_a, a_cur, 2);
-    W(wa, a_cur, 0);
-    E(a_cur, 4, shift_a);
-    T(total_a, a_cur, 3);
-    W(wa, a_cur, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 4
-    QK(a_nxt, qa, 2);
-    __builtin_amdgcn_sched_barrier(0);
-    issue(2);
-    E(a_cur, 5, shift_a);
-    T(total_a, a_cur, 4);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 5
-    QK(b_nxt, qb, 2);
-    __builtin_amdgcn_sched_barrier(0);
-    E(a_cur, 6, shift_a);
-    T(total_a, a_cur, 5);
-    E(a_cur, 7, shift_a);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 6
-    QK(a_nxt, qa, 3);
-    __builtin_amdgcn_sched_barrier(0);
-    issue(3);
-    T(total_a, a_cur, 6);
-    W(wa, a_cur, 2);
-    T(total_a, a_cur, 7);
-    W(wa, a_cur, 3);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 7
-    QK(b_nxt, qb, 3);
-    __builtin_amdgcn_sched_barrier(0);
-    E(a_cur, 8, shift_a);
-    E(a_cur, 9, shift_a);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 8
-    QK(a_nxt, qa, 4);
-    __builtin_amdgcn_sched_barrier(0);
-    VR(0, 0);
-    T(total_a, a_cur, 8);
-    E(a_cur, 10, shift_a);
-    T(total_a, a_cur, 9);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 9
-    QK(b_nxt, qb, 4);
-    __builtin_amdgcn_sched_barrier(0);
-    VR(0, 1);
-    E(a_cur, 11, shift_a);
-    T(total_a, a_cur, 10);
-    W(wa, a_cur, 4);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 10
-    QK(a_nxt, qa, 5);
-    __builtin_amdgcn_sched_barrier(0);
-    VR(0, 2);
-    E(a_cur, 12, shift_a);
-    T(total_a, a_cur, 11);
-    W(wa, a_cur, 5);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 11
-    QK(b_nxt, qb, 5);
-    __builtin_amdgcn_sched_barrier(0);
-    VR(0, 3);
-    E(a_cur, 13, shift_a);
-    T(total_a, a_cur, 12);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 12
-    QK(a_nxt, qa, 6);
-    __builtin_amdgcn_sched_barrier(0);
-    VR(1, 0);
-    E(a_cur, 14, shift_a);
-    T(total_a, a_cur, 13);
-    W(wa, a_cur, 6);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 13
-    QK(b_nxt, qb, 6);
-    __builtin_amdgcn_sched_barrier(0);
-    VR(1, 1);
-    E(a_cur, 15, shift_a);
-    T(total_a, a_cur, 14);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 14
-    QK(a_nxt, qa, 7);
-    __builtin_amdgcn_sched_barrier(0);
-    VR(1, 2);
-    T(total_a, a_cur, 15);
-    W(wa, a_cur, 7);
-    E(b_cur, 0, shift_b);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 15
-    QK(b_nxt, qb, 7);
-    __builtin_amdgcn_sched_barrier(0);
-    VR(1, 3);
-    E(b_cur, 1, shift_b);
-    T(total_b, b_cur, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 16
-    PV(A, 0, 0, wa);
-    __builtin_amdgcn_sched_barrier(0);
-    KR(0);
-    E(b_cur, 2, shift_b);
-    T(total_b, b_cur, 1);
-    W(wb, b_cur, 0);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 17
-    PV(A, 0, 1, wa);
-    __builtin_amdgcn_sched_barrier(0);
-    KR(1);
-    E(b_cur, 3, shift_b);
-    T(total_b, b_cur, 2);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 18
-    PV(A, 0, 2, wa);
-    __builtin_amdgcn_sched_barrier(0);
-    KR(2);
-    E(b_cur, 4, shift_b);
-    T(total_b, b_cur, 3);
-    W(wb, b_cur, 1);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 19
-    PV(A, 0, 3, wa);
-    __builtin_amdgcn_sched_barrier(0);
-    KR(3);
-    E(b_cur, 5, shift_b);
-    T(total_b, b_cur, 4);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 20
-    PV(A, 1, 0, wa);
-    __builtin_amdgcn_sched_barrier(0);
-    KR(4);
-    E(b_cur, 6, shift_b);
-    T(total_b, b_cur, 5);
-    W(wb, b_cur, 2);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 21
-    PV(A, 1, 1, wa);
-    __builtin_amdgcn_sched_barrier(0);
-    KR(5);
-    E(b_cur, 7, shift_b);
-    T(total_b, b_cur, 6);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 22
-    PV(A, 1, 2, wa);
-    __builtin_amdgcn_sched_barrier(0);
-    KR(6);
-    T(total_b, b_cur, 7);
-    W(wb, b_cur, 3);
-    E(b_cur, 8, shift_b);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 23
-    PV(A, 1, 3, wa);
-    __builtin_amdgcn_sched_barrier(0);
-    KR(7);
-    E(b_cur, 9, shift_b);
-    T(total_b, b_cur, 8);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 24
-    PV(B, 0, 0, wb);
-    __builtin_amdgcn_sched_barrier(0);
-    E(b_cur, 10, shift_b);
-    T(total_b, b_cur, 9);
-    E(b_cur, 11, shift_b);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 25
-    PV(B, 0, 1, wb);
-    __builtin_amdgcn_sched_barrier(0);
-    T(total_b, b_cur, 10);
-    W(wb, b_cur, 4);
-    E(b_cur, 12, shift_b);
-    T(total_b, b_cur, 11);
-    W(wb, b_cur, 5);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 26
-    PV(B, 0, 2, wb);
-    __builtin_amdgcn_sched_barrier(0);
-    E(b_cur, 13, shift_b);
-    T(total_b, b_cur, 12);
-    E(b_cur, 14, shift_b);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 27
-    PV(B, 0, 3, wb);
-    __builtin_amdgcn_sched_barrier(0);
-    T(total_b, b_cur, 13);
-    E(b_cur, 15, shift_b);
-    T(total_b, b_cur, 14);
-    W(wb, b_cur, 6);
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 28
-    W(wb, b_cur, 7);
-    PV(B, 1, 0, wb);
-    __builtin_amdgcn_sched_barrier(0);
-    ROW_MAXIMA_0;
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 29
-    PV(B, 1, 1, wb);
-    __builtin_amdgcn_sched_barrier(0);
-    ROW_MAXIMA_1;
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 30
-    PV(B, 1, 2, wb);
-    __builtin_amdgcn_sched_barrier(0);
-    ROW_MAXIMA_2;
-    __builtin_amdgcn_sched_barrier(0);
-    // slot 31
-    PV(B, 1, 3, wb);
-    __builtin_amdgcn_sched_barrier(0);
-    LAG_TEST;
-    T(total_b, b_cur, 15);
-    __builtin_amdgcn_sched_barrier(0);
+#if SINGE_HEAD_DIM == 128
+#include "prefill_pair_block_d128.inc"
+#else
+#include "prefill_pair_block_d64.inc"
+#endif
 #undef QK
 #undef PV
 #undef E

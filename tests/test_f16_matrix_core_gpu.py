@@ -62,6 +62,19 @@ def test_paged_attention_f16(heads, kv_heads, page_size, index_dtype, options):
     paged_case(SEQUENCES, heads, kv_heads, page_size, options, index_dtype, seed=heads + page_size)
 
 
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("heads,kv_heads,page_size,index_dtype", [(8, 1, 16, torch.int32), (64, 8, 16, torch.int64), (8, 2, 64, torch.int32)])
+def test_paged_attention_f16_two_tiles_a_wave(heads, kv_heads, page_size, index_dtype, causal):
+    # the f16 builds of the kernel that gives a wave two 32-row tiles: chunks of several 256-row tiles, key counts either
+    # side of a tile's end, sequences without keys or with more queries than keys
+    _native.lib().singe_hip_set_paged_attention_rows_per_wave(64)
+    try:
+        paged_case(SEQUENCES + [(300, 1000), (257, 513), (64, 1024)], heads, kv_heads, page_size, neural.AttentionOptions(causal=causal),
+                   index_dtype, seed=heads + page_size + 3)
+    finally:
+        _native.lib().singe_hip_set_paged_attention_rows_per_wave(0)
+
+
 @pytest.mark.parametrize("splits", [3, 16])
 def test_paged_attention_f16_key_splits(splits):
     paged_case([(1, 1500), (1, 40), (5, 700), (2, 0)], 8, 2, 16, neural.AttentionOptions(causal=True), torch.int32, seed=splits,

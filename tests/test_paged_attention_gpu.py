@@ -131,8 +131,18 @@ def test_int64_indices_and_chunked_prefill_shape():
              index_dtype=torch.int64, seed=4)
 
 
-def test_a_bad_page_in_a_large_page_table_is_refused_and_the_rest_is_right():
-    """Page sizes of 16 keys and more look their pages up on the scalar unit: the same error contract."""
+@pytest.mark.parametrize("rows_per_wave", [0, 64])
+def test_a_bad_page_in_a_large_page_table_is_refused_and_the_rest_is_right(rows_per_wave):
+    """Page sizes of 16 keys and more look their pages up on the scalar unit (the two-tile kernel: in the lanes that
+    fetched them): the same error contract."""
+    _native.lib().singe_hip_set_paged_attention_rows_per_wave(rows_per_wave)
+    try:
+        a_bad_page_is_refused_and_the_rest_is_right()
+    finally:
+        _native.lib().singe_hip_set_paged_attention_rows_per_wave(0)
+
+
+def a_bad_page_is_refused_and_the_rest_is_right():
     gen = torch.Generator(device="cuda")
     gen.manual_seed(8)
     q = torch.randn((40, 4, 128), generator=gen, device="cuda").to(torch.bfloat16)

@@ -15,7 +15,9 @@ import pytest
 
 from singe_amd import build
 
-SOURCES = [os.path.join(os.path.dirname(build.__file__), "csrc", name) for name in ("fmha_prefill_pair.hip", "paged_attention_pair.hip")]
+CSRC = os.path.join(os.path.dirname(build.__file__), "csrc")
+# (source, extra flags): every build of the two-tile kernels
+BUILDS = [("fmha_prefill_pair.hip", []), ("paged_attention_pair.hip", []), ("fmha_prefill_pair.hip", ["-DSINGE_HEAD_DIM=64"])]
 WAIT_STATES = 12
 
 
@@ -45,11 +47,13 @@ def instructions(assembly):
         yield stripped.split(";")[0].strip(), inside
 
 
-@pytest.mark.parametrize("source", SOURCES, ids=os.path.basename)
-def test_nothing_touches_a_score_product_before_it_is_done(source):
+@pytest.mark.parametrize("name,flags", BUILDS, ids=lambda value: value if isinstance(value, str) else "".join(value) or "d128")
+def test_nothing_touches_a_score_product_before_it_is_done(name, flags):
+    source = os.path.join(CSRC, name)
+    steps = 4 if flags else 8  # score products a chain
     with tempfile.TemporaryDirectory() as scratch:
         listing = os.path.join(scratch, "pair.s")
-        command = [build.hipcc()] + [flag for flag in build.HIPCC_FLAGS if flag != "--genco"] + [
+        command = [build.hipcc()] + [flag for flag in build.HIPCC_FLAGS if flag != "--genco"] + flags + [
             "--cuda-device-only", "-S", "-I", os.path.dirname(source), source, "-o", listing]
         subprocess.run(command, check=True, capture_output=True)
         program = list(instructions(open(listing).read()))
@@ -87,7 +91,7 @@ def test_nothing_touches_a_score_product_before_it_is_done(source):
             waited += int(nop.group(1)) + 1 if nop else 1
             if later.startswith("v_mfma"):
                 waited += 7  # a matrix instruction holds the issue for its passes
-    assert products >= 4 * 32  # four kernels, two blocks of sixteen score products each
+    assert products >= 4 * 4 * steps  # four kernels at least, two blocks of two chains each
     # Q^T is loaded into accumulation registers by a statement the compiler does not know to be a load: nothing may
     # name those registers before the wait that follows the loads.
     loads = 0
@@ -102,4 +106,4 @@ def test_nothing_touches_a_score_product_before_it_is_done(source):
             if later_inside and later.startswith("global_load_dwordx4 a["):
                 continue
             assert not (registers(later, "a") & loaded), f"{later!r} names what {text!r} is still loading"
-    assert loads >= 4 * 16
+    assert loads >= 4 * 2 * steps
