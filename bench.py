@@ -488,7 +488,8 @@ def chunked_prefill_section(with_cpu=True):
     result["fused_query_rotation"] = {
         "workload": "the same attention with the query's RMS norm (with a weight) and rotation (f32 angles) done by the "
                     "attention kernel (rotary_paged_attention)",
-        "kernel": "singe_rotary_paged_attention_bf16_d128_i32_p16", "ms_per_step": fused["mean_ms"],
+        "kernel": ("singe_rotary_paged_attention_pair_bf16_d128_i32" if rows_per_wave == 64
+                   else "singe_rotary_paged_attention_bf16_d128_i32_p16"), "ms_per_step": fused["mean_ms"],
         "ms_per_step_median": fused["median_ms"], "tflops": flops / (fused["mean_ms"] * 1e-3) / 1e12,
         "over_plain_attention_us": (fused["mean_ms"] - stats["mean_ms"]) * 1e3, **timing_fields(fused)}
     if with_cpu:

@@ -318,6 +318,8 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_fmha_prefill_pair_f16_d128_causal_ragged", "singe_fmha_prefill_pair_f16_d128_full_ragged",
     "singe_paged_attention_pair_bf16_d128_i32", "singe_paged_attention_pair_bf16_d128_i64",
     "singe_paged_attention_pair_f16_d128_i32", "singe_paged_attention_pair_f16_d128_i64",
+    "singe_rotary_paged_attention_pair_bf16_d128_i32", "singe_rotary_paged_attention_pair_bf16_d128_i64",
+    "singe_rotary_paged_attention_pair_f16_d128_i32", "singe_rotary_paged_attention_pair_f16_d128_i64",
     "singe_fmha_prefill_pair_bf16_d64_causal", "singe_fmha_prefill_pair_bf16_d64_full",
     "singe_fmha_prefill_pair_f16_d64_causal", "singe_fmha_prefill_pair_f16_d64_full",
     "singe_fmha_prefill_pair_bf16_d64_causal_ragged", "singe_fmha_prefill_pair_bf16_d64_full_ragged",
@@ -364,7 +366,7 @@ constexpr PartRun kPartRuns[] = {
     {8, 4},                       // latent attention on the matrix cores at any width it takes
     {30, 14}, {31, 14}, {32, 14}, {33, 14}, {34, 14}, {35, 14},  // the decode kernels and their merges for 32, 16, 48, 80, 96, 112
     {36, 8},                      // the dense prefill with two row tiles a wave (whole key tiles, then a last tile that is not)
-    {37, 4},                      // the paged attention op on the same loop
+    {37, 8},                      // the paged attention op on the same loop, then with a fused query rotation
     {38, 8},                      // the two-tile dense prefill at head_dim 64
 };
 constexpr int runs_total() {

@@ -87,10 +87,10 @@ enum KernelId : int {
     // + 4 * (key_len not a multiple of 64)
     kPrefillPair = kDecodeOtherHeadDims + 6 * 14,
     // the paged attention op on the same two-tile loop (head_dim 128, page sizes that are powers of two from 16, no
-    // options): + (i64 indices) + 2 * f16
+    // options): + (i64 indices) + 2 * f16 + 4 * (the query's norm and rotation fused in)
     kPagedPair = kPrefillPair + 8,
     // the head_dim 64 builds of the two-tile dense prefill, in kPrefillPair's order
-    kPrefillPairD64 = kPagedPair + 4,
+    kPrefillPairD64 = kPagedPair + 8,
     kKernelCount = kPrefillPairD64 + 8
 };
 

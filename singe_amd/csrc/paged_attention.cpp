@@ -313,14 +313,23 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
         args.partial_out = static_cast<float*>(scratch->memory);
         args.partial_lse = args.partial_out + static_cast<size_t>(splits) * p.tokens * p.heads * p.head_dim;
     }
-    // Prefill-shaped plain calls at head_dim 128 take the kernel that gives a wave two 32-row tiles (256 packed rows a
-    // workgroup, one workgroup a compute unit; paged_attention_pair.hip), when its grid still fills the chip.
+    if (rotation != nullptr) {
+        args.cos = rotation->cos;
+        args.sin = rotation->sin;
+        args.query_weight = rotation->attributes->has_norm ? static_cast<const uint16_t*>(rotation->weight) : nullptr;
+        args.table_type = static_cast<uint32_t>(rotation->attributes->table_type);
+        args.has_query_norm = rotation->attributes->has_norm ? 1u : 0u;
+        args.query_eps = rotation->attributes->eps;
+    }
+    // Prefill-shaped plain calls at head_dim 128 (with or without the fused query rotation) take the kernel that gives a
+    // wave two 32-row tiles (256 packed rows a workgroup, one workgroup a compute unit; paged_attention_pair.hip), when
+    // its grid still fills the chip.
     RowTileGrid pair;
-    if (rotation == nullptr && splits == 1 && (data_type == SINGE_HIP_BF16 || f16) && two_tiles_a_wave(p, &pair)) {
+    if (splits == 1 && (data_type == SINGE_HIP_BF16 || f16) && two_tiles_a_wave(p, &pair)) {
         args.row_tiles = static_cast<uint32_t>(pair.row_tiles);
         args.compact = pair.compact;
         args.longest_first = pair.longest_first;
-        const int kernel = kPagedPair + (wide ? 1 : 0) + (f16 ? 2 : 0);
+        const int kernel = kPagedPair + (wide ? 1 : 0) + (f16 ? 2 : 0) + (rotation != nullptr ? 4 : 0);
         return launch(static_cast<KernelId>(kernel), static_cast<unsigned>(pair.blocks), 1, 1, 256, stream, args);
     }
     const unsigned grid = static_cast<unsigned>(blocks * splits);
@@ -330,12 +339,6 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
         return launch(built(combine), static_cast<unsigned>(blocks), 1, 1, 256, stream, args);
     };
     if (rotation != nullptr) {
-        args.cos = rotation->cos;
-        args.sin = rotation->sin;
-        args.query_weight = rotation->attributes->has_norm ? static_cast<const uint16_t*>(rotation->weight) : nullptr;
-        args.table_type = static_cast<uint32_t>(rotation->attributes->table_type);
-        args.has_query_norm = rotation->attributes->has_norm ? 1u : 0u;
-        args.query_eps = rotation->attributes->eps;
         const int rotary = rotary_paged_attention_base(f16, p.has_softcap != 0, head_dim) + (wide ? 1 : 0) + (args.page_shift >= 4 ? 2 : 0);
         return finish(launch(static_cast<KernelId>(rotary), grid, 1, 1, 256, stream, args));
     }

@@ -1,6 +1,7 @@
 // Attention of ragged queries over a paged KV cache in FlashInfer form (see paged_attention.hip for the op, its
 // layouts and its paging checks), for the calls that are prefill-shaped and plain: bf16 or f16, head_dim 128, a page
-// size that is a power of two of at least 16 keys, no cap, no window, no key splits, no fused rotation.  The loop is
+// size that is a power of two of at least 16 keys, no cap, no window, no key splits; with or without the fused query
+// rotation of rotary_paged_attention (query_rotation.hip.h).  The loop is
 // the dense two-tile one (fmha_prefill_pair.hip, prefill_pair.hip.h): a wave alone on its SIMD folds every 32-key
 // block into two tiles of 32 packed rows, so a workgroup owns 256 packed rows of one (sequence, kv head) (row r =
 // token r / groups, head r % groups) and a key tile staged in LDS serves all of them.
@@ -17,12 +18,13 @@
 #include "paged_locate.hip.h"
 #include "paging.hip.h"
 #include "prefill_pair.hip.h"
+#include "query_rotation.hip.h"
 
 namespace {
 
 using namespace prefill;
 
-template <int FORM, class Half>
+template <int FORM, bool ROTATE, class Half>
 SINGE_DEVICE void paged_attention_pair_body(const PagedAttentionArgs& a, unsigned char* lds) {
     static_assert(FORM == kCsrI32 || FORM == kCsrI64, "the FlashInfer form");
     const unsigned int tid = threadIdx.x, lane = tid & 63;
@@ -111,12 +113,36 @@ SINGE_DEVICE void paged_attention_pair_body(const PagedAttentionArgs& a, unsigne
         auto row_of = [&](const Tile& t) __attribute__((always_inline)) {
             return a.query_rows + ((static_cast<size_t>(query_start) + t.token) * a.heads + kv_head * groups + t.head) * kHeadDim + 8 * hi;
         };
-        const uint16_t* row_a = row_of(ta);
-        const uint16_t* row_b = row_of(tb);
+        if constexpr (ROTATE) {
+            // The query arrives before its norm and rotation (query_rotation.hip.h): loaded into vector registers, turned
+            // there, parked in LDS (the fourth stage, which nobody loads before the first tile is folded: 8 KiB a wave,
+            // a lane's eight chunks 1 KiB apart) and read back straight into the accumulation registers, so that Q^T is
+            // born in that class here too.
+            unsigned char* const parked = lds + (wave < 2 ? 0 : kPairValueBase) + kPairAhead * kTileBytes + (wave & 1u) * 8192u + lane * 16u;
+            auto turned = [&](const Tile& t, u32x4_t (&q)[kSteps]) __attribute__((always_inline)) {
+                const uint16_t* row = row_of(t);
+                uint4 bits[kSteps];
 #pragma unroll
-        for (int s = 0; s < kSteps; ++s) qa[s] = load_to_accumulation(row_a + 16 * s);
+                for (int s = 0; s < kSteps; ++s) {
+                    bits[s] = *reinterpret_cast<const uint4*>(row + 16 * s);
+                    if (!t.valid) bits[s] = make_uint4(0, 0, 0, 0);
+                }
+                rotate_query(half, bits, a, static_cast<size_t>(query_start) + t.token, t.valid, hi);
 #pragma unroll
-        for (int s = 0; s < kSteps; ++s) qb[s] = load_to_accumulation(row_b + 16 * s);
+                for (int s = 0; s < kSteps; ++s) *reinterpret_cast<uint4*>(parked + 1024 * s) = bits[s];
+#pragma unroll
+                for (int s = 0; s < kSteps; ++s) q[s] = lds_to_accumulation(lds_address(parked + 1024 * s));
+            };
+            turned(ta, qa);
+            turned(tb, qb);
+        } else {
+            const uint16_t* row_a = row_of(ta);
+            const uint16_t* row_b = row_of(tb);
+#pragma unroll
+            for (int s = 0; s < kSteps; ++s) qa[s] = load_to_accumulation(row_a + 16 * s);
+#pragma unroll
+            for (int s = 0; s < kSteps; ++s) qb[s] = load_to_accumulation(row_b + 16 * s);
+        }
     }
     const uint4 no_query[kSteps] = {};  // the masked path's folding functions take a Q^T they do not read
 
@@ -363,13 +389,18 @@ SINGE_DEVICE void paged_attention_pair_body(const PagedAttentionArgs& a, unsigne
 
 }  // namespace
 
-#define SINGE_PAGED_ATTENTION_PAIR_KERNEL(NAME, FORM, HALF)                                         \
+#define SINGE_PAGED_ATTENTION_PAIR_KERNEL(NAME, FORM, ROTATE, HALF)                                 \
     extern "C" __global__ __launch_bounds__(64 * prefill::kPairWaves, 1) void NAME(PagedAttentionArgs args) { \
         __shared__ __attribute__((aligned(1024))) unsigned char paged_lds[prefill::kPairLdsBytes];  \
-        paged_attention_pair_body<FORM, prefill::HALF>(args, paged_lds);                            \
+        paged_attention_pair_body<FORM, ROTATE, prefill::HALF>(args, paged_lds);                    \
     }
 
-SINGE_PAGED_ATTENTION_PAIR_KERNEL(singe_paged_attention_pair_bf16_d128_i32, kCsrI32, Bf16)
-SINGE_PAGED_ATTENTION_PAIR_KERNEL(singe_paged_attention_pair_bf16_d128_i64, kCsrI64, Bf16)
-SINGE_PAGED_ATTENTION_PAIR_KERNEL(singe_paged_attention_pair_f16_d128_i32, kCsrI32, F16)
-SINGE_PAGED_ATTENTION_PAIR_KERNEL(singe_paged_attention_pair_f16_d128_i64, kCsrI64, F16)
+SINGE_PAGED_ATTENTION_PAIR_KERNEL(singe_paged_attention_pair_bf16_d128_i32, kCsrI32, false, Bf16)
+SINGE_PAGED_ATTENTION_PAIR_KERNEL(singe_paged_attention_pair_bf16_d128_i64, kCsrI64, false, Bf16)
+SINGE_PAGED_ATTENTION_PAIR_KERNEL(singe_paged_attention_pair_f16_d128_i32, kCsrI32, false, F16)
+SINGE_PAGED_ATTENTION_PAIR_KERNEL(singe_paged_attention_pair_f16_d128_i64, kCsrI64, false, F16)
+// (with the query's norm and rotation fused in)
+SINGE_PAGED_ATTENTION_PAIR_KERNEL(singe_rotary_paged_attention_pair_bf16_d128_i32, kCsrI32, true, Bf16)
+SINGE_PAGED_ATTENTION_PAIR_KERNEL(singe_rotary_paged_attention_pair_bf16_d128_i64, kCsrI64, true, Bf16)
+SINGE_PAGED_ATTENTION_PAIR_KERNEL(singe_rotary_paged_attention_pair_f16_d128_i32, kCsrI32, true, F16)
+SINGE_PAGED_ATTENTION_PAIR_KERNEL(singe_rotary_paged_attention_pair_f16_d128_i64, kCsrI64, true, F16)

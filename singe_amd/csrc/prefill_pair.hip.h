@@ -53,9 +53,21 @@ SINGE_DEVICE u32x4_t load_to_accumulation(const void* address) {
     asm volatile("global_load_dwordx4 %0, %1, off" : "=a"(loaded) : "v"(address) : "memory");
     return loaded;
 }
+SINGE_DEVICE unsigned int lds_address(const unsigned char* in_lds) {
+    return static_cast<unsigned int>(reinterpret_cast<size_t>((lds_words_t)(in_lds)));
+}
+
+// Sixteen bytes from LDS straight into accumulation registers: the same birth for a Q^T that was worked out in vector
+// registers (a fused rotation) and parked in LDS on its way.  A wave's LDS operations run in order, so the read sees
+// what the same lane wrote just before; accumulation_loads_landed() before the first use.
+SINGE_DEVICE u32x4_t lds_to_accumulation(unsigned int lds_byte_address) {
+    u32x4_t loaded;
+    asm volatile("ds_read_b128 %0, %1" : "=a"(loaded) : "v"(lds_byte_address) : "memory");
+    return loaded;
+}
 // All of this wave's loads but the eight it issued last (a tile's: four of K, four of V) have completed.
 SINGE_DEVICE void older_loads_landed() { __builtin_amdgcn_s_waitcnt(0x0F78); }  // vmcnt(8), other counters left alone
-SINGE_DEVICE void accumulation_loads_landed() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+SINGE_DEVICE void accumulation_loads_landed() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); }
 
 // The scores of a whole block outside the scheduled loop (the first block, the diagonal tile): the same products, then
 // the wait the compiler would have put in front of the first reader had it known what the statements above it are.

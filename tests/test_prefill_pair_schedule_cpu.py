@@ -95,15 +95,16 @@ def test_nothing_touches_a_score_product_before_it_is_done(name, flags):
     # Q^T is loaded into accumulation registers by a statement the compiler does not know to be a load: nothing may
     # name those registers before the wait that follows the loads.
     loads = 0
+    into_accumulation = ("global_load_dwordx4 a[", "ds_read_b128 a[")  # (the second: a Q^T worked out first and parked in LDS)
     for at, (text, inside) in enumerate(program):
-        if not (inside and text.startswith("global_load_dwordx4 a[")):
+        if not (inside and text.startswith(into_accumulation)):
             continue
         loads += 1
-        loaded = registers(text.split(",")[0], "a")
+        loaded = registers(text.split(",")[0].split(" ", 1)[1], "a")
         for later, later_inside in program[at + 1:]:
-            if later_inside and later.startswith("s_waitcnt vmcnt(0)"):
+            if later_inside and later.startswith("s_waitcnt vmcnt(0) lgkmcnt(0)"):
                 break
-            if later_inside and later.startswith("global_load_dwordx4 a["):
+            if later_inside and later.startswith(into_accumulation):
                 continue
             assert not (registers(later, "a") & loaded), f"{later!r} names what {text!r} is still loading"
     assert loads >= 4 * 2 * steps
