@@ -14,26 +14,41 @@ pytestmark = pytest.mark.gpu
 MAX_ABS, MEAN_ABS, LSE_ABS = 2e-2, 2e-3, 2e-3
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_paged_attention_random_shapes_on_the_two_tile_kernel(seed):
+    # plain calls (no window, no cap, no key shares) with page sizes the kernel takes and longer chunks, sent to the kernel
+    # that gives a wave two 32-row tiles whatever their size
+    rng = np.random.default_rng(3000 + seed)
+    _native.lib().singe_hip_set_paged_attention_rows_per_wave(64)
+    try:
+        paged_attention_random_shape(seed, rng, two_tiles=True)
+    finally:
+        _native.lib().singe_hip_set_paged_attention_rows_per_wave(0)
+
+
 @pytest.mark.parametrize("seed", range(24))
 def test_paged_attention_random_shapes(seed):
-    rng = np.random.default_rng(1000 + seed)
+    paged_attention_random_shape(seed, np.random.default_rng(1000 + seed), two_tiles=False)
+
+
+def paged_attention_random_shape(seed, rng, two_tiles):
     kv_heads = int(rng.choice([1, 2, 3, 4, 8]))
     heads = kv_heads * int(rng.choice([1, 2, 4, 5, 8]))
-    page_size = int(rng.choice([1, 2, 3, 8, 16, 16, 32, 64, 128, 24]))
+    page_size = int(rng.choice([16, 16, 32, 64, 128, 256] if two_tiles else [1, 2, 3, 8, 16, 16, 32, 64, 128, 24]))
     count = int(rng.integers(1, 7))
     sequences = []
     for _ in range(count):
         keys = int(rng.choice([0, 1, int(rng.integers(1, 64)), int(rng.integers(64, 700)), int(rng.integers(700, 2500))]))
-        queries = int(rng.choice([0, 1, 1, int(rng.integers(1, 40)), int(rng.integers(40, 300))]))
+        queries = int(rng.choice([0, 1, 1, int(rng.integers(1, 40)), int(rng.integers(40, 900 if two_tiles else 300))]))
         sequences.append((queries, keys))
     if sum(q for q, _ in sequences) == 0:
         sequences[0] = (3, sequences[0][1])
     options = neural.AttentionOptions(causal=bool(rng.integers(0, 2)),
-                                      window=None if rng.integers(0, 3) else int(rng.integers(1, 300)),
-                                      softcap=None if rng.integers(0, 4) else float(rng.uniform(2.0, 40.0)),
+                                      window=None if two_tiles or rng.integers(0, 3) else int(rng.integers(1, 300)),
+                                      softcap=None if two_tiles or rng.integers(0, 4) else float(rng.uniform(2.0, 40.0)),
                                       scale=None if rng.integers(0, 2) else float(rng.uniform(0.02, 0.2)))
     index_dtype = torch.int64 if rng.integers(0, 2) else torch.int32
-    splits = int(rng.choice([0, 0, 1, 2, 5, 16]))
+    splits = 1 if two_tiles else int(rng.choice([0, 0, 1, 2, 5, 16]))
 
     query_offsets, page_offsets, last = [0], [0], []
     for queries, keys in sequences:
@@ -72,31 +87,42 @@ def test_paged_attention_random_shapes(seed):
     assert np.abs(got_lse[~empty] - want_lse[~empty]).max(initial=0.0) <= LSE_ABS, case
 
 
+@pytest.mark.parametrize("rows_per_wave,dim", [(0, 128), (64, 128), (64, 64)])
 @pytest.mark.parametrize("seed", range(12))
-def test_dense_prefill_random_shapes(seed):
-    rng = np.random.default_rng(2000 + seed)
+def test_dense_prefill_random_shapes(seed, rows_per_wave, dim):
+    # (64 rows a wave: the kernel that gives a wave two 32-row tiles, whatever the shape; larger shapes there, so that
+    # several 256-row tiles and key tiles on both sides of the masks are met)
+    rng = np.random.default_rng(2000 + seed + 100 * rows_per_wave + dim)
+    _native.lib().singe_hip_set_dense_prefill_rows_per_wave(rows_per_wave)
+    try:
+        dense_prefill_random_shape(seed, rng, dim, 3 if rows_per_wave else 1)
+    finally:
+        _native.lib().singe_hip_set_dense_prefill_rows_per_wave(0)
+
+
+def dense_prefill_random_shape(seed, rng, dim, stretch):
     batch = int(rng.integers(1, 4))
     kv_heads = int(rng.choice([1, 2, 4]))
     heads = kv_heads * int(rng.choice([1, 2, 4]))
-    query_len = int(rng.choice([1, int(rng.integers(2, 130)), int(rng.integers(130, 700))]))
-    key_len = query_len if rng.integers(0, 2) else int(rng.choice([1, int(rng.integers(2, 130)), int(rng.integers(130, 900))]))
+    query_len = int(rng.choice([1, int(rng.integers(2, 130)), int(rng.integers(130, 700 * stretch))]))
+    key_len = query_len if rng.integers(0, 2) else int(rng.choice([1, int(rng.integers(2, 130)), int(rng.integers(130, 900 * stretch))]))
     causal = bool(rng.integers(0, 2))
     scale = float(rng.uniform(0.03, 0.15)) * (-1.0 if rng.integers(0, 6) == 0 else 1.0)
     gen = torch.Generator(device="cuda")
     gen.manual_seed(seed)
-    q = torch.randn((batch, query_len, heads, 128), generator=gen, device="cuda").to(torch.bfloat16)
-    k = torch.randn((batch, key_len, kv_heads, 128), generator=gen, device="cuda").to(torch.bfloat16)
-    v = torch.randn((batch, key_len, kv_heads, 128), generator=gen, device="cuda").to(torch.bfloat16)
-    config = A.FmhaPrefillConfig.contiguous(batch, query_len, key_len, heads, kv_heads, 128, scale, causal)
+    q = torch.randn((batch, query_len, heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
+    k = torch.randn((batch, key_len, kv_heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
+    v = torch.randn((batch, key_len, kv_heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
+    config = A.FmhaPrefillConfig.contiguous(batch, query_len, key_len, heads, kv_heads, dim, scale, causal)
     out = torch.full_like(q, float("nan"))
     lse = torch.full((batch, heads, query_len), float("nan"), device="cuda", dtype=torch.float32)
     A.fmha_prefill_lse_bf16(None, out, lse, q, k, v, config)
     torch.cuda.synchronize()
     want, want_lse = oracle.fmha_prefill_lse_f32(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), batch=batch,
-                                                 query_len=query_len, key_len=key_len, heads=heads, kv_heads=kv_heads, head_dim=128,
+                                                 query_len=query_len, key_len=key_len, heads=heads, kv_heads=kv_heads, head_dim=dim,
                                                  scale=scale, causal=causal, threads=8)
     got = out.float().cpu().numpy()
-    case = (batch, query_len, key_len, heads, kv_heads, causal, scale)
+    case = (batch, query_len, key_len, heads, kv_heads, causal, scale, dim)
     assert np.isfinite(got).all(), case
     gap = np.abs(got - want)
     assert gap.max() <= MAX_ABS and gap.mean() <= MEAN_ABS, (case, gap.max())
