@@ -283,8 +283,18 @@ def _paged_attention_replays():
     assert np.abs(want_lse.cpu().numpy()[live] - reference_lse[live]).max() <= 2e-3
 
 
-def test_dense_prefill_replays():
-    batch, heads, kv_heads, length, dim = 2, 8, 2, 320, 128
+@pytest.mark.parametrize("rows_per_wave,length", [(0, 320), (64, 320), (64, 417)])
+def test_dense_prefill_replays(rows_per_wave, length):
+    # (64 rows a wave: the kernel that gives a wave two 32-row tiles, with whole key tiles and with a last tile that is not)
+    _native.lib().singe_hip_set_dense_prefill_rows_per_wave(rows_per_wave)
+    try:
+        _dense_prefill_replays(length)
+    finally:
+        _native.lib().singe_hip_set_dense_prefill_rows_per_wave(0)
+
+
+def _dense_prefill_replays(length):
+    batch, heads, kv_heads, dim = 2, 8, 2, 128
     query = torch.empty((batch, length, heads, dim), device="cuda", dtype=torch.bfloat16)
     key = torch.empty((batch, length, kv_heads, dim), device="cuda", dtype=torch.bfloat16)
     value = torch.empty_like(key)
@@ -300,3 +310,55 @@ def test_dense_prefill_replays():
 
     run = lambda stream: A.fmha_prefill_bf16(stream, out, query, key, value, config)
     _replays_equal_eager(run, [change(i) for i in range(3)], [out])
+
+
+def test_prefill_shaped_paged_attention_replays_on_the_two_tile_kernel():
+    """Chunks of new tokens over cached prefixes, on the kernel that gives a wave two 32-row tiles: the page lists, the
+    prefix lengths and the queries change between replays."""
+    sequences, chunk, heads, kv_heads, dim, page, cache_pages = 3, 300, 16, 2, 128, 16, 400
+    rng = np.random.default_rng(37)
+    cases = [[700, 300, 1500], [300, 2000, 301], [1024, 513, 999]]  # keys of each sequence (its chunk included)
+    capacity = 3 * 130
+    query = torch.empty((sequences * chunk, heads, dim), device="cuda", dtype=torch.bfloat16)
+    key_cache = torch.randn((cache_pages, page, kv_heads, dim), device="cuda").to(torch.bfloat16)
+    value_cache = torch.randn((cache_pages, page, kv_heads, dim), device="cuda").to(torch.bfloat16)
+    query_offsets = torch.arange(0, (sequences + 1) * chunk, chunk, dtype=torch.int32, device="cuda")
+    page_offsets = torch.zeros(sequences + 1, dtype=torch.int32, device="cuda")
+    pages = torch.zeros(capacity, dtype=torch.int32, device="cuda")
+    last = torch.zeros(sequences, dtype=torch.int32, device="cuda")
+    paging = neural.Paging(query_offsets, page_offsets, pages, last)
+    problem = neural._problem(query, key_cache, value_cache, paging, neural.AttentionOptions(causal=True))
+    out = torch.empty_like(query)
+    lse = torch.empty((sequences * chunk, heads), device="cuda", dtype=torch.float32)
+    status = torch.zeros(1, device="cuda", dtype=torch.int32)
+
+    def change(i):
+        def apply():
+            counts = [(n + page - 1) // page for n in cases[i]]
+            page_offsets.copy_(torch.tensor(np.concatenate([[0], np.cumsum(counts)]), dtype=torch.int32))
+            listed = np.zeros(capacity, dtype=np.int32)
+            listed[: sum(counts)] = rng.permutation(cache_pages)[: sum(counts)]
+            pages.copy_(torch.from_numpy(listed))
+            last.copy_(torch.tensor([n - (c - 1) * page for n, c in zip(cases[i], counts)], dtype=torch.int32))
+            query.copy_(torch.randn(query.shape, device="cuda", generator=torch.Generator("cuda").manual_seed(90 + i)).to(torch.bfloat16))
+        return apply
+
+    def run(stream):
+        handle = int((stream or torch.cuda.current_stream()).cuda_stream)
+        _native.check(_native.lib().singe_hip_paged_attention_bf16(
+            handle, query.data_ptr(), key_cache.data_ptr(), value_cache.data_ptr(), query_offsets.data_ptr(), page_offsets.data_ptr(),
+            pages.data_ptr(), last.data_ptr(), out.data_ptr(), lse.data_ptr(), status.data_ptr(), ctypes.byref(problem)), "paged_attention")
+
+    _native.lib().singe_hip_set_paged_attention_rows_per_wave(64)
+    try:
+        want_out, want_lse = _replays_equal_eager(run, [change(i) for i in range(len(cases))], [out, lse])
+    finally:
+        _native.lib().singe_hip_set_paged_attention_rows_per_wave(0)
+    assert int(status.item()) == 0
+    code, reference, reference_lse = oracle.paged_attention_f32(
+        query.float().cpu().numpy(), key_cache.float().cpu().numpy(), value_cache.float().cpu().numpy(),
+        query_offsets.cpu().numpy(), page_offsets.cpu().numpy(), pages.cpu().numpy(), last.cpu().numpy(), causal=True, threads=8)
+    assert code == 0
+    gap = np.abs(want_out.float().cpu().numpy() - reference)
+    assert gap.max() <= 2e-2 and gap.mean() <= 2e-3, (gap.max(), gap.mean())
+    assert np.abs(want_lse.cpu().numpy() - reference_lse).max() <= 2e-3
