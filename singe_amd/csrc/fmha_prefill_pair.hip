@@ -8,8 +8,10 @@
 //   * the order of a wave's instructions is the schedule: a block is 32 matrix instructions (8 score products of
 //     the NEXT block for A, 8 for B, 8 value products of this block for A, 8 for B) and the vector work of the block
 //     (exponentials, sums, packing, the next block's row maxima, LDS operand reads, the tile's loads) is dealt out
-//     over the 32 slots between them, at most seven issue cycles a slot, so that each piece is done before the
-//     matrix instruction that needs it is issued and the matrix pipe never waits (fold_pair_block);
+//     evenly over the 32 slots between them, each piece before the matrix instruction that needs it
+//     (fold_pair_block; prefill_pair_deal.py).  A lone wave issues every instruction itself, the matrix ones
+//     included, so the block's instruction count bounds the loop (about 360 issue cycles of four clocks for 256 of
+//     matrix work), and on operands that switch many bits the clock the device holds comes before that;
 //   * the score accumulators must be in ordinary vector registers (the vector unit reads them) while O^T and Q^T
 //     live in the accumulation registers; the compiler gives every matrix instruction of such a kernel an
 //     accumulation-register destination, so the score products are written as assembly with the register classes

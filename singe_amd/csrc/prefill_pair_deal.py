@@ -5,8 +5,10 @@ the block as the text fold_pair_block includes (prefill_pair_block_d128.inc, pre
 
 A block at head_dim D is 2 * D / 16 score products of the NEXT block (tile A's and tile B's chains alternating, so that a
 product never follows the one it accumulates onto) and 4 * ceil(D / 32) value products of this block (A's two 16-key
-halves, then B's).  Behind each product sits a slot of other work: an exponential with its multiply-add (E, 3 issue
-cycles), a running sum (T, 1, at least a slot after its exponential), a rounding of two weights into a word (W, 1, after
+halves, then B's).  Behind each product sits a slot of other work, weighed in nominal issue cycles of four clocks (what
+the dealing needs is an even spread and the right order, not exact costs: measured, a plain vector instruction of a
+lone wave takes 4.5 clocks, an exponential 8, a matrix instruction's own issue 9): an exponential with its multiply-add
+(E, 3), a running sum (T, 1, at least a slot after its exponential), a rounding of two weights into a word (W, 1, after
 both exponentials and before the slot whose product reads the word), four direct-to-LDS loads of the tile (issue, 3 each),
 the V^T operand reads of this block (VR, 2 each, before the value products of their half), the K operand reads of the
 block after next (KR, 1 each, behind the last score product that reads the operand they replace), and in the last four
