@@ -267,3 +267,26 @@ def test_two_tiles_a_wave_head_dim_64_f16_and_nan_behind_the_last_key(two_tiles_
     gap = np.abs(out.float().cpu().numpy() - want)
     assert gap.max() <= MAX_ABS / 6 and gap.mean() <= MEAN_ABS / 6, (gap.max(), gap.mean())
     assert np.abs(lse.cpu().numpy() - want_lse).max() <= LSE_ABS
+
+
+@pytest.mark.parametrize("dim", [128, 64])
+@pytest.mark.parametrize("causal", [True, False])
+def test_two_tiles_a_wave_head_major_layout(two_tiles_a_wave, causal, dim):
+    # tensors stored [batch, heads, len, dim] (strides of their own for every operand), a key count that leaves a last
+    # tile of 21 keys
+    batch, heads, kv_heads, query_len, key_len = 2, 4, 2, 530, 725
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(dim + causal)
+    q = torch.randn((batch, heads, query_len, dim), generator=gen, device="cuda").to(torch.bfloat16)
+    k = torch.randn((batch, kv_heads, key_len, dim), generator=gen, device="cuda").to(torch.bfloat16)
+    v = torch.randn((batch, kv_heads, key_len, dim), generator=gen, device="cuda").to(torch.bfloat16)
+    scale = float(dim) ** -0.5
+    config = A.bhsd_config(batch, heads, kv_heads, query_len, key_len, dim, scale, causal)
+    out = torch.full_like(q, float("nan"))
+    lse = torch.full((batch, heads, query_len), float("nan"), device="cuda", dtype=torch.float32)
+    A.fmha_prefill_lse_bf16(None, out, lse, q, k, v, config)
+    torch.cuda.synchronize()
+    rows = lambda tensor: tensor.float().permute(0, 2, 1, 3).contiguous().cpu().numpy()
+    want, want_lse = oracle.fmha_prefill_lse_f32(rows(q), rows(k), rows(v), batch=batch, query_len=query_len, key_len=key_len,
+                                                 heads=heads, kv_heads=kv_heads, head_dim=dim, scale=scale, causal=causal, threads=8)
+    check(rows(out), lse.cpu().numpy(), want, want_lse, f"two tiles, head-major layout, head_dim {dim}, causal={causal}")
