@@ -253,11 +253,13 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
     // Long rows without options at head_dim 128: the kernel that gives a wave two 32-row tiles (256 query rows a
     // workgroup, one workgroup a compute unit), when its launch still fills the chip; a build of its own where the last
     // key tile is not whole.
-    if (!with_options && options.sinks == nullptr && options.key_lengths == nullptr && splits == 1 && two_tiles_a_wave(c)) {
+    if (!with_options && options.sinks == nullptr && splits == 1 && two_tiles_a_wave(c)) {
         const uint32_t pair_tiles = static_cast<uint32_t>((c.query_len + 255) / 256);
         const uint64_t pair_groups = rows * ((pair_tiles + 1) / 2);
         args.query_tiles = pair_tiles;
-        const KernelId pair = static_cast<KernelId>((c.head_dim == 64 ? kPrefillPairD64 : kPrefillPair) + (c.causal ? 0 : 1) + (f16 ? 2 : 0) + (c.key_len % 64 != 0 ? 4 : 0));
+        // (the builds that take a last tile that is not whole also take a key count of their own for every batch entry)
+        const bool ragged = c.key_len % 64 != 0 || options.key_lengths != nullptr;
+        const KernelId pair = static_cast<KernelId>((c.head_dim == 64 ? kPrefillPairD64 : kPrefillPair) + (c.causal ? 0 : 1) + (f16 ? 2 : 0) + (ragged ? 4 : 0));
         return launch(pair, static_cast<unsigned>(pair_groups), 1, 1, 256, stream, args);
     }
     const KernelId kernel = static_cast<KernelId>((f16 ? kPrefillCausalF16 : kPrefillCausal) + (c.causal ? 0 : 1) + (with_options ? 4 : 0));

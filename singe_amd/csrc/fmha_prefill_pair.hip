@@ -44,7 +44,15 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
     const unsigned int column = lane & 31, hi = lane >> 5;
     const unsigned int group = a.heads / a.kv_heads;
     const unsigned int batch = bh / a.heads, head = bh % a.heads, kv_head = head / group;
-    const unsigned int key_len = a.key_len;  // at least one key, and a multiple of 64 unless RAGGED (the host's gate)
+    // Keys that take part: all of them (at least one, and a multiple of 64 unless RAGGED: the host's gate), or (RAGGED) the
+    // batch entry's own count, which may be none (singe/src/backend/cpu/normalization/attention.rs:191-276, key_lengths).
+    unsigned int key_len = a.key_len;
+    if (RAGGED && a.key_lengths != nullptr) {
+        const int own = a.key_lengths[batch];
+        const unsigned int bound = own > 0 ? static_cast<unsigned int>(own) : 0u;
+        key_len = bound < key_len ? bound : key_len;
+    }
+    key_len = __builtin_amdgcn_readfirstlane(key_len);
 
     const unsigned int first_row = query_tile * kPairRows + wave * 64u;  // of this wave: tile A, then tile B 32 rows on
     const unsigned int query_a = first_row + column, query_b = query_a + 32u;

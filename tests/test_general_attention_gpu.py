@@ -376,3 +376,24 @@ def test_splitk_reduce_validation():
     with pytest.raises(error.LengthTooShort) as caught:
         A.splitk_reduce_f32(None, out, attn, lse, A.SplitKReduceConfig.contiguous(1, 2, 5, 8))
     assert caught.value.name == "out" and caught.value.minimum == 16
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dim", [128, 64])
+@pytest.mark.parametrize("causal", [True, False])
+def test_padded_batches_on_the_two_tile_kernel(causal, dim, dtype):
+    # key counts of their own for every batch entry (none, a few, a last tile that is not whole, all and more than all) on
+    # the dense kernel that gives a wave two 32-row tiles
+    from singe_amd import _native
+    batch, heads, kv_heads, query_len, key_len = 5, 4, 2, 300, 640
+    q, k, v = tensors((batch, heads, query_len, dim), (batch, kv_heads, key_len, dim), (batch, kv_heads, key_len, dim), dtype, 23)
+    counts = [0, 17, 333, 640, 5000]
+    lengths = torch.tensor(counts, dtype=torch.int32, device="cuda")
+    _native.lib().singe_hip_set_dense_prefill_rows_per_wave(64)
+    try:
+        out = neural.attend_padded(q, k, v, lengths, neural.AttentionOptions(causal=causal))
+    finally:
+        _native.lib().singe_hip_set_dense_prefill_rows_per_wave(0)
+    want = oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), causal=causal, key_lengths=counts, threads=8)
+    close(host(out), want, dtype)
+    assert not host(out)[0].any()
