@@ -317,7 +317,7 @@ typedef struct SingeFmhaPrefillConfig {
 
 /* Tuning knob of the dense bf16 / f16 prefill at head_dim 128 and 64: the query rows a wave takes.  32: four waves share a
  * compute unit's SIMDs two by two, 128 rows a workgroup.  64: a wave has a SIMD to itself and folds every key block
- * into two 32-row tiles, 256 rows a workgroup; only calls without options (mask, window, cap, sinks, key splits;
+ * into two 32-row tiles, 256 rows a workgroup; only calls without a mask, a window, a cap or key splits (sinks and
  * key lengths are taken) with a positive scale have this form, others keep 32.  0 (the default): 64 where the call has that form
  * and its 256-row tiles still fill the chip.  Results are the same up to the order in which a row's
  * reference point moves.  The counterpart of AttentionParameters::{warps, min_blocks}

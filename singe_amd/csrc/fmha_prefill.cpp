@@ -253,7 +253,7 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
     // Long rows without options at head_dim 128: the kernel that gives a wave two 32-row tiles (256 query rows a
     // workgroup, one workgroup a compute unit), when its launch still fills the chip; a build of its own where the last
     // key tile is not whole.
-    if (!with_options && options.sinks == nullptr && splits == 1 && two_tiles_a_wave(c)) {
+    if (!with_options && splits == 1 && two_tiles_a_wave(c)) {
         const uint32_t pair_tiles = static_cast<uint32_t>((c.query_len + 255) / 256);
         const uint64_t pair_groups = rows * ((pair_tiles + 1) / 2);
         args.query_tiles = pair_tiles;

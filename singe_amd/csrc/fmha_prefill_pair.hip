@@ -145,6 +145,16 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
     RowState A, B;
     reset(A);
     reset(B);
+    if (a.sinks != nullptr) {
+        // The head's sink: a score that is always there and weighs no value.  A row starts with it as its reference point
+        // and a sum of one (held by one of the row's two lanes), as in fmha_prefill.hip.
+        const uint16_t bits = a.sinks[head];
+        float sink;
+        if constexpr (std::is_same_v<Half, F16>) sink = static_cast<float>(__builtin_bit_cast(_Float16, bits));
+        else sink = __builtin_bit_cast(float, static_cast<unsigned int>(bits) << 16);
+        A.reference = B.reference = sink * kLog2e;
+        A.running_sum = B.running_sum = hi == 0 && A.reference != -INFINITY ? 1.0f : 0.0f;
+    }
     const ReadOffsets offsets = read_offsets(lane);
 
     for (unsigned int early = 0; early < kPairAhead && early < tiles; ++early) load_tile(early, early);

@@ -397,3 +397,27 @@ def test_padded_batches_on_the_two_tile_kernel(causal, dim, dtype):
     want = oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), causal=causal, key_lengths=counts, threads=8)
     close(host(out), want, dtype)
     assert not host(out)[0].any()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dim", [128, 64])
+def test_sinks_on_the_two_tile_kernel(dim, dtype):
+    # a sink per head (one of them so large that it outweighs every key, one absent: -inf) with and without the causal
+    # mask and with padded batches, on the dense kernel that gives a wave two 32-row tiles
+    from singe_amd import _native
+    batch, heads, kv_heads, query_len, key_len = 3, 4, 2, 300, 450
+    q, k, v = tensors((batch, heads, query_len, dim), (batch, kv_heads, key_len, dim), (batch, kv_heads, key_len, dim), dtype, 29)
+    sinks = torch.tensor([0.5, 30.0, float("-inf"), -2.0], device="cuda").to(dtype)
+    counts = [0, 450, 129]
+    lengths = torch.tensor(counts, dtype=torch.int32, device="cuda")
+    _native.lib().singe_hip_set_dense_prefill_rows_per_wave(64)
+    try:
+        for causal in (True, False):
+            out = neural.attend(q, k, v, None, sinks, neural.AttentionOptions(causal=causal))
+            want = oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), causal=causal, sinks=host(sinks), threads=8)
+            close(host(out), want, dtype)
+        out = neural._attend_all(q, k, v, None, sinks, lengths, neural.AttentionOptions(causal=True), None)
+        want = oracle.scaled_dot_product_attention_f32(host(q), host(k), host(v), causal=True, sinks=host(sinks), key_lengths=counts, threads=8)
+        close(host(out), want, dtype)
+    finally:
+        _native.lib().singe_hip_set_dense_prefill_rows_per_wave(0)
