@@ -466,6 +466,18 @@ def chunked_prefill_section(with_cpu=True):
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": tflops / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": nbytes, "traffic_source": source, **timing_fields(stats)},
     }
+    # The same launch on all-zero queries and caches: what the instruction stream allows where no operand bit changes
+    # from one matrix instruction to the next and the clock is not held back (as in the dense prefill section).
+    if rows_per_wave == 64:
+        kept = (work.query, work.key_cache, work.value_cache)
+        work.query, work.key_cache, work.value_cache = (torch.zeros_like(t) for t in kept)
+        quiet = measure(launch, 4)
+        work.query, work.key_cache, work.value_cache = kept
+        quiet_tflops = flops / (quiet["mean_ms"] * 1e-3) / 1e12
+        result["same_kernel_on_zero_inputs"] = {
+            "what": "the same kernel, sizes and page table on all-zero queries and caches",
+            "ms_per_step": quiet["mean_ms"], "tflops": quiet_tflops, "frac": quiet_tflops / MFMA_BF16_PEAK_TFLOPS,
+            **timing_fields(quiet)}
     # The same attention with the query's RMS norm and rotation fused into the kernel (rotary_paged_attention): the
     # query is normalised, rotated and rounded on its way into the registers, which spares the two-step form's
     # write and re-read of the rotated query.
@@ -1077,6 +1089,8 @@ def compact(result):
     if "same_kernel_on_zero_inputs" in result.get("prefill", {}) and "3_prefill" in configs:
         # (the same launch on all-zero tensors: what the instruction stream allows where the clock is not held back)
         configs["3_prefill"]["frac_on_zero_inputs"] = _rounded(result["prefill"]["same_kernel_on_zero_inputs"]["frac"])
+    if "same_kernel_on_zero_inputs" in result.get("chunked_prefill", {}) and "4_chunked_prefill" in configs:
+        configs["4_chunked_prefill"]["frac_on_zero_inputs"] = _rounded(result["chunked_prefill"]["same_kernel_on_zero_inputs"]["frac"])
     if "5_fp8_decode" in configs:
         configs["5_fp8_decode"]["whole_op_frac"] = _rounded(result["fp8_decode"]["pct_hbm_peak"] / 100.0)
     roofline["configs"] = configs
