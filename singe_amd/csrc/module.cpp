@@ -324,6 +324,10 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_fmha_prefill_pair_f16_d64_causal", "singe_fmha_prefill_pair_f16_d64_full",
     "singe_fmha_prefill_pair_bf16_d64_causal_ragged", "singe_fmha_prefill_pair_bf16_d64_full_ragged",
     "singe_fmha_prefill_pair_f16_d64_causal_ragged", "singe_fmha_prefill_pair_f16_d64_full_ragged",
+    "singe_paged_attention_pair_bf16_d64_i32", "singe_paged_attention_pair_bf16_d64_i64",
+    "singe_paged_attention_pair_f16_d64_i32", "singe_paged_attention_pair_f16_d64_i64",
+    "singe_rotary_paged_attention_pair_bf16_d64_i32", "singe_rotary_paged_attention_pair_bf16_d64_i64",
+    "singe_rotary_paged_attention_pair_f16_d64_i32", "singe_rotary_paged_attention_pair_f16_d64_i64",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -337,7 +341,7 @@ const char* const kPartNames[kPartCount] = {
     "fmha_prefill_d16", "paged_attention_d16", "fmha_prefill_d48", "paged_attention_d48", "fmha_prefill_d80", "paged_attention_d80",
     "fmha_prefill_d112", "paged_attention_d112", "paged_decode_d32",
     "paged_decode_d16", "paged_decode_d48", "paged_decode_d80", "paged_decode_d96", "paged_decode_d112",
-    "fmha_prefill_pair", "paged_attention_pair", "fmha_prefill_pair_d64",
+    "fmha_prefill_pair", "paged_attention_pair", "fmha_prefill_pair_d64", "paged_attention_pair_d64",
 };
 
 namespace {
@@ -368,6 +372,7 @@ constexpr PartRun kPartRuns[] = {
     {36, 8},                      // the dense prefill with two row tiles a wave (whole key tiles, then a last tile that is not)
     {37, 8},                      // the paged attention op on the same loop, then with a fused query rotation
     {38, 8},                      // the two-tile dense prefill at head_dim 64
+    {39, 8},                      // the two-tile paged attention at head_dim 64
 };
 constexpr int runs_total() {
     int total = 0;

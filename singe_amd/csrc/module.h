@@ -91,7 +91,9 @@ enum KernelId : int {
     kPagedPair = kPrefillPair + 8,
     // the head_dim 64 builds of the two-tile dense prefill, in kPrefillPair's order
     kPrefillPairD64 = kPagedPair + 8,
-    kKernelCount = kPrefillPairD64 + 8
+    // the head_dim 64 builds of the two-tile paged attention, in kPagedPair's order
+    kPagedPairD64 = kPrefillPairD64 + 8,
+    kKernelCount = kPagedPairD64 + 8
 };
 
 
@@ -160,7 +162,7 @@ inline int rotary_paged_attention_base(bool f16, bool softcap, long long head_di
 extern const char* const kKernelNames[kKernelCount];
 
 // Parts of the code object (one file each) and the part a kernel lives in.
-constexpr int kPartCount = 39;
+constexpr int kPartCount = 40;
 extern const char* const kPartNames[kPartCount];
 int kernel_part(int kernel);
 

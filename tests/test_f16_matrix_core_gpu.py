@@ -15,7 +15,7 @@ pytestmark = pytest.mark.gpu
 MAX_ABS, LSE_ABS = 3e-3, 2e-3
 
 
-def paged_case(sequences, heads, kv_heads, page_size, options, index_dtype, seed, splits=0):
+def paged_case(sequences, heads, kv_heads, page_size, options, index_dtype, seed, splits=0, dim=128):
     query_offsets, page_offsets, last = [0], [0], []
     for queries, keys in sequences:
         query_offsets.append(query_offsets[-1] + queries)
@@ -27,9 +27,9 @@ def paged_case(sequences, heads, kv_heads, page_size, options, index_dtype, seed
     table = np.random.default_rng(seed).permutation(page_count)[:needed].tolist()
     gen = torch.Generator(device="cuda")
     gen.manual_seed(seed)
-    q = torch.randn((query_offsets[-1], heads, 128), generator=gen, device="cuda").to(torch.float16)
-    kc = torch.randn((page_count, page_size, kv_heads, 128), generator=gen, device="cuda").to(torch.float16)
-    vc = torch.randn((page_count, page_size, kv_heads, 128), generator=gen, device="cuda").to(torch.float16)
+    q = torch.randn((query_offsets[-1], heads, dim), generator=gen, device="cuda").to(torch.float16)
+    kc = torch.randn((page_count, page_size, kv_heads, dim), generator=gen, device="cuda").to(torch.float16)
+    vc = torch.randn((page_count, page_size, kv_heads, dim), generator=gen, device="cuda").to(torch.float16)
     index = lambda values: torch.tensor(values, dtype=index_dtype, device="cuda")
     paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
     _native.lib().singe_hip_set_paged_attention_splits(splits)
@@ -63,14 +63,15 @@ def test_paged_attention_f16(heads, kv_heads, page_size, index_dtype, options):
 
 
 @pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("dim", [128, 64])
 @pytest.mark.parametrize("heads,kv_heads,page_size,index_dtype", [(8, 1, 16, torch.int32), (64, 8, 16, torch.int64), (8, 2, 64, torch.int32)])
-def test_paged_attention_f16_two_tiles_a_wave(heads, kv_heads, page_size, index_dtype, causal):
+def test_paged_attention_f16_two_tiles_a_wave(heads, kv_heads, page_size, index_dtype, causal, dim):
     # the f16 builds of the kernel that gives a wave two 32-row tiles: chunks of several 256-row tiles, key counts either
     # side of a tile's end, sequences without keys or with more queries than keys
     _native.lib().singe_hip_set_paged_attention_rows_per_wave(64)
     try:
         paged_case(SEQUENCES + [(300, 1000), (257, 513), (64, 1024)], heads, kv_heads, page_size, neural.AttentionOptions(causal=causal),
-                   index_dtype, seed=heads + page_size + 3)
+                   index_dtype, seed=heads + page_size + 3, dim=dim)
     finally:
         _native.lib().singe_hip_set_paged_attention_rows_per_wave(0)
 

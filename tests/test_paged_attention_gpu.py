@@ -395,14 +395,15 @@ def two_tiles_a_wave():
 
 @pytest.mark.parametrize("index_dtype", [torch.int32, torch.int64])
 @pytest.mark.parametrize("causal", [True, False])
-@pytest.mark.parametrize("heads,kv_heads,page_size", [(8, 1, 16), (64, 8, 16), (8, 2, 32), (4, 1, 64), (8, 2, 128), (4, 4, 16)])
-def test_two_tiles_a_wave_ragged_sequences_match_oracle(two_tiles_a_wave, heads, kv_heads, page_size, causal, index_dtype):
+@pytest.mark.parametrize("heads,kv_heads,page_size,dim", [(8, 1, 16, 128), (64, 8, 16, 128), (8, 2, 32, 128), (4, 1, 64, 128), (8, 2, 128, 128),
+                                                          (4, 4, 16, 128), (8, 1, 16, 64), (64, 8, 16, 64), (8, 2, 64, 64), (4, 4, 32, 64)])
+def test_two_tiles_a_wave_ragged_sequences_match_oracle(two_tiles_a_wave, heads, kv_heads, page_size, dim, causal, index_dtype):
     # the shapes of the ragged test (decode, full prefill, chunked prefill, no keys, more queries than keys) and
     # chunks long enough for several 256-row tiles, several key tiles ahead of the mask and key counts either side of
     # a tile's and a page's end
     sequences = [(1, 150), (70, 70), (20, 90), (3, 0), (9, 4), (130, 300), (300, 1000), (257, 513), (64, 1024), (512, 512)]
     run_case(sequences, heads, kv_heads, page_size, neural.AttentionOptions(causal=causal), index_dtype=index_dtype,
-             seed=heads + page_size + 1)
+             seed=heads + page_size + 1, dim=dim)
 
 
 def test_two_tiles_a_wave_equals_the_four_wave_kernel_at_the_chunked_prefill_shape():

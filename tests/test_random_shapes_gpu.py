@@ -62,9 +62,10 @@ def paged_attention_random_shape(seed, rng, two_tiles):
     tokens = query_offsets[-1]
     gen = torch.Generator(device="cuda")
     gen.manual_seed(seed)
-    q = torch.randn((tokens, heads, 128), generator=gen, device="cuda").to(torch.bfloat16)
-    kc = torch.randn((page_count, page_size, kv_heads, 128), generator=gen, device="cuda").to(torch.bfloat16)
-    vc = torch.randn((page_count, page_size, kv_heads, 128), generator=gen, device="cuda").to(torch.bfloat16)
+    dim = 64 if two_tiles and seed % 2 else 128  # (either build of the two-tile kernel)
+    q = torch.randn((tokens, heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
+    kc = torch.randn((page_count, page_size, kv_heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
+    vc = torch.randn((page_count, page_size, kv_heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
     index = lambda values: torch.tensor(values, dtype=index_dtype, device="cuda")
     paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
     _native.lib().singe_hip_set_paged_attention_splits(splits)

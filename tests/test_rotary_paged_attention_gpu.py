@@ -150,15 +150,16 @@ def test_fused_rotation_refuses_what_it_does_not_take():
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("norm", [None, "plain", "weighted"])
+@pytest.mark.parametrize("dim", [128, 64])
 @pytest.mark.parametrize("heads,kv_heads,page_size,table_dtype,index_dtype,causal", [
     (8, 2, 16, torch.float32, torch.int32, True), (64, 8, 16, torch.bfloat16, torch.int64, True), (8, 1, 64, torch.float16, torch.int32, False)])
-def test_fused_rotation_on_the_two_tile_kernel(heads, kv_heads, page_size, table_dtype, index_dtype, causal, norm, dtype):
+def test_fused_rotation_on_the_two_tile_kernel(heads, kv_heads, page_size, table_dtype, index_dtype, causal, norm, dtype, dim):
     # prefill-shaped calls take the kernel that gives a wave two 32-row tiles: the rotated query is parked in LDS on its
     # way into the accumulation registers there; chunks of several 256-row tiles, empty sequences, more queries than keys
     from singe_amd import _native
     _native.lib().singe_hip_set_paged_attention_rows_per_wave(64)
     try:
         run_case(SEQUENCES + [(300, 1000), (257, 513), (64, 1024)], heads, kv_heads, page_size, table_dtype, index_dtype, norm,
-                 neural.AttentionOptions(causal=causal), seed=heads + page_size + 9, dtype=dtype)
+                 neural.AttentionOptions(causal=causal), seed=heads + page_size + 9, dim=dim, dtype=dtype)
     finally:
         _native.lib().singe_hip_set_paged_attention_rows_per_wave(0)
