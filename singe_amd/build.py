@@ -74,6 +74,8 @@ PARTS = [
     ("paged_attention_pair", "paged_attention_pair.hip", []),
     ("fmha_prefill_pair_d64", "fmha_prefill_pair.hip", ["-DSINGE_HEAD_DIM=64"]),
     ("paged_attention_pair_d64", "paged_attention_pair.hip", ["-DSINGE_HEAD_DIM=64"]),
+    ("fmha_prefill_pair_d96", "fmha_prefill_pair.hip", ["-DSINGE_HEAD_DIM=96"]),
+    ("paged_attention_pair_d96", "paged_attention_pair.hip", ["-DSINGE_HEAD_DIM=96"]),
 ]
 HOST_SOURCES = ["hip_runtime_loader.cpp", "module.cpp", "paged_decode.cpp", "fmha_prefill.cpp", "paged_attention.cpp",
                 "general_attention.cpp", "fmha_decode.cpp", "paged_rows_f32.cpp", "latent_attention.cpp", "cache_ops.cpp",

@@ -1,4 +1,4 @@
-// Dense flash-attention prefill for long rows, bf16 or f16, head_dim 128 (or 64, -DSINGE_HEAD_DIM=64), no options: the same arithmetic and
+// Dense flash-attention prefill for long rows, bf16 or f16, head_dim 128 (or 96, 64: -DSINGE_HEAD_DIM=), no options: the same arithmetic and
 // register layouts as fmha_prefill.hip (S^T = K . Q^T, per-lane softmax, O^T += V^T . P^T; prefill_core.hip.h), with
 // the work laid out the other way round.  There, two waves share a SIMD and each folds keys into 32 query rows;
 // what one wave leaves idle the other uses.  Here ONE wave owns a SIMD (up to 512 registers) and folds every key
@@ -98,12 +98,8 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
     const unsigned int key_stride_bytes = static_cast<unsigned int>(a.key_sequence_stride) * 2u;
     const unsigned int value_stride_bytes = static_cast<unsigned int>(a.value_sequence_stride) * 2u;
     const unsigned int load_row = 4u * wave + (lane >> 4), position = lane & 15u;
-    // (at head_dim 64 a global row has eight chunks and an LDS row still sixteen places: the lanes whose place holds one
-    // of the other eight fetch a chunk of the same row again, which lands where nobody reads, so the load needs no
-    // predicate)
-    constexpr unsigned int kChunkMask = kGlobalRowBytes / 16u - 1u;
-    const unsigned int key_chunk = ((position ^ (load_row & 15u)) & kChunkMask) * 16u;
-    const unsigned int value_chunk = ((position ^ (4u * (load_row & 3u))) & kChunkMask) * 16u;
+    const unsigned int key_chunk = fetched_chunk(position ^ (load_row & 15u)) * 16u;
+    const unsigned int value_chunk = fetched_chunk(position ^ (4u * (load_row & 3u))) * 16u;
     const unsigned int key_lane = load_row * key_stride_bytes + key_chunk, value_lane = load_row * value_stride_bytes + value_chunk;
     // The lane's offsets into a tile, one a load.  A last tile that is not whole has offsets of its own: its rows past
     // the last key re-read that key (they are masked; what lies behind the last key is not this call's to read).  Both
@@ -330,11 +326,7 @@ SINGE_DEVICE void fmha_prefill_pair_body(const PrefillArgs& a, unsigned char* ld
         fmha_prefill_pair_body<CAUSAL, RAGGED, prefill::HALF>(args, prefill_lds);                      \
     }
 
-#if SINGE_HEAD_DIM == 128
-#define SINGE_PAIR_NAME(TYPE, FORM) singe_fmha_prefill_pair_##TYPE##_d128_##FORM
-#else
-#define SINGE_PAIR_NAME(TYPE, FORM) singe_fmha_prefill_pair_##TYPE##_d64_##FORM
-#endif
+#define SINGE_PAIR_NAME(TYPE, FORM) SINGE_PAIR_JOIN(singe_fmha_prefill, pair, TYPE, SINGE_PAIR_DIM, FORM)
 SINGE_FMHA_PREFILL_PAIR_KERNEL(SINGE_PAIR_NAME(bf16, causal), true, false, Bf16)
 SINGE_FMHA_PREFILL_PAIR_KERNEL(SINGE_PAIR_NAME(bf16, full), false, false, Bf16)
 SINGE_FMHA_PREFILL_PAIR_KERNEL(SINGE_PAIR_NAME(f16, causal), true, false, F16)

@@ -328,6 +328,14 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_attention_pair_f16_d64_i32", "singe_paged_attention_pair_f16_d64_i64",
     "singe_rotary_paged_attention_pair_bf16_d64_i32", "singe_rotary_paged_attention_pair_bf16_d64_i64",
     "singe_rotary_paged_attention_pair_f16_d64_i32", "singe_rotary_paged_attention_pair_f16_d64_i64",
+    "singe_fmha_prefill_pair_bf16_d96_causal", "singe_fmha_prefill_pair_bf16_d96_full",
+    "singe_fmha_prefill_pair_f16_d96_causal", "singe_fmha_prefill_pair_f16_d96_full",
+    "singe_fmha_prefill_pair_bf16_d96_causal_ragged", "singe_fmha_prefill_pair_bf16_d96_full_ragged",
+    "singe_fmha_prefill_pair_f16_d96_causal_ragged", "singe_fmha_prefill_pair_f16_d96_full_ragged",
+    "singe_paged_attention_pair_bf16_d96_i32", "singe_paged_attention_pair_bf16_d96_i64",
+    "singe_paged_attention_pair_f16_d96_i32", "singe_paged_attention_pair_f16_d96_i64",
+    "singe_rotary_paged_attention_pair_bf16_d96_i32", "singe_rotary_paged_attention_pair_bf16_d96_i64",
+    "singe_rotary_paged_attention_pair_f16_d96_i32", "singe_rotary_paged_attention_pair_f16_d96_i64",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -342,6 +350,7 @@ const char* const kPartNames[kPartCount] = {
     "fmha_prefill_d112", "paged_attention_d112", "paged_decode_d32",
     "paged_decode_d16", "paged_decode_d48", "paged_decode_d80", "paged_decode_d96", "paged_decode_d112",
     "fmha_prefill_pair", "paged_attention_pair", "fmha_prefill_pair_d64", "paged_attention_pair_d64",
+    "fmha_prefill_pair_d96", "paged_attention_pair_d96",
 };
 
 namespace {
@@ -373,6 +382,7 @@ constexpr PartRun kPartRuns[] = {
     {37, 8},                      // the paged attention op on the same loop, then with a fused query rotation
     {38, 8},                      // the two-tile dense prefill at head_dim 64
     {39, 8},                      // the two-tile paged attention at head_dim 64
+    {40, 8}, {41, 8},             // both at head_dim 96
 };
 constexpr int runs_total() {
     int total = 0;

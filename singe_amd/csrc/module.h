@@ -93,7 +93,10 @@ enum KernelId : int {
     kPrefillPairD64 = kPagedPair + 8,
     // the head_dim 64 builds of the two-tile paged attention, in kPagedPair's order
     kPagedPairD64 = kPrefillPairD64 + 8,
-    kKernelCount = kPagedPairD64 + 8
+    // and the head_dim 96 builds of both
+    kPrefillPairD96 = kPagedPairD64 + 8,
+    kPagedPairD96 = kPrefillPairD96 + 8,
+    kKernelCount = kPagedPairD96 + 8
 };
 
 
@@ -162,7 +165,7 @@ inline int rotary_paged_attention_base(bool f16, bool softcap, long long head_di
 extern const char* const kKernelNames[kKernelCount];
 
 // Parts of the code object (one file each) and the part a kernel lives in.
-constexpr int kPartCount = 40;
+constexpr int kPartCount = 42;
 extern const char* const kPartNames[kPartCount];
 int kernel_part(int kernel);
 

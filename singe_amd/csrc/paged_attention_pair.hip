@@ -1,5 +1,5 @@
 // Attention of ragged queries over a paged KV cache in FlashInfer form (see paged_attention.hip for the op, its
-// layouts and its paging checks), for the calls that are prefill-shaped and plain: bf16 or f16, head_dim 128 (or 64, -DSINGE_HEAD_DIM=64), a page
+// layouts and its paging checks), for the calls that are prefill-shaped and plain: bf16 or f16, head_dim 128 (or 96, 64: -DSINGE_HEAD_DIM=), a page
 // size that is a power of two of at least 16 keys, no cap, no window, no key splits; with or without the fused query
 // rotation of rotary_paged_attention (query_rotation.hip.h).  The loop is
 // the dense two-tile one (fmha_prefill_pair.hip, prefill_pair.hip.h): a wave alone on its SIMD folds every 32-key
@@ -149,11 +149,8 @@ SINGE_DEVICE void paged_attention_pair_body(const PagedAttentionArgs& a, unsigne
     // Loads: instruction i of wave w fills rows 16 i + 4 w .. + 3 of a stage; the sixteen keys of instruction i's
     // group sit in one page (paged_attention.hip, GROUPED).
     const unsigned int load_row = 4u * wave + (lane >> 4), chunk_position = lane & 15u;
-    // (at head_dim 64 a cache row has eight chunks and an LDS row still sixteen places: the lanes whose place holds one of
-    // the other eight fetch a chunk of the same row again, which lands where nobody reads, so the load needs no predicate)
-    constexpr unsigned int kChunkMask = kGlobalRowBytes / 16u - 1u;
-    const unsigned int key_chunk = ((chunk_position ^ (load_row & 15u)) & kChunkMask) * 16u;
-    const unsigned int value_chunk = ((chunk_position ^ (4u * (load_row & 3u))) & kChunkMask) * 16u;
+    const unsigned int key_chunk = fetched_chunk(chunk_position ^ (load_row & 15u)) * 16u;
+    const unsigned int value_chunk = fetched_chunk(chunk_position ^ (4u * (load_row & 3u))) * 16u;
     const unsigned int page_bytes = a.page_size * a.kv_heads * kGlobalRowBytes;  // (the host sends pages below 4 GiB)
     const unsigned int head_bytes = kv_head * kGlobalRowBytes, slot_bytes = a.kv_heads * kGlobalRowBytes;
     const unsigned char* const key_bytes = reinterpret_cast<const unsigned char*>(a.key_cache);
@@ -399,11 +396,7 @@ SINGE_DEVICE void paged_attention_pair_body(const PagedAttentionArgs& a, unsigne
         paged_attention_pair_body<FORM, ROTATE, prefill::HALF>(args, paged_lds);                    \
     }
 
-#if SINGE_HEAD_DIM == 128
-#define SINGE_PAIR_NAME(OP, TYPE, FORM) singe_##OP##_pair_##TYPE##_d128_##FORM
-#else
-#define SINGE_PAIR_NAME(OP, TYPE, FORM) singe_##OP##_pair_##TYPE##_d64_##FORM
-#endif
+#define SINGE_PAIR_NAME(OP, TYPE, FORM) SINGE_PAIR_JOIN(singe_##OP, pair, TYPE, SINGE_PAIR_DIM, FORM)
 SINGE_PAGED_ATTENTION_PAIR_KERNEL(SINGE_PAIR_NAME(paged_attention, bf16, i32), kCsrI32, false, Bf16)
 SINGE_PAGED_ATTENTION_PAIR_KERNEL(SINGE_PAIR_NAME(paged_attention, bf16, i64), kCsrI64, false, Bf16)
 SINGE_PAGED_ATTENTION_PAIR_KERNEL(SINGE_PAIR_NAME(paged_attention, f16, i32), kCsrI32, false, F16)

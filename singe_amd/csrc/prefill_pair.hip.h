@@ -2,7 +2,7 @@
 // (fmha_prefill_pair.hip says why and how; paged_attention_pair.hip is the same loop over a paged cache): the score
 // products as assembly with their register classes spelled out, Q^T loaded straight into accumulation registers, the
 // row maxima of two score tiles in alternating chains, and fold_pair_block, one 32-key block of both tiles with its
-// vector work dealt out over the slots between its matrix instructions (32 at head_dim 128, 16 at 64: the text of the
+// vector work dealt out over the slots between its matrix instructions (32 at head_dim 128, 24 at 96, 16 at 64: the text of the
 // block is written by prefill_pair_deal.py).
 #pragma once
 
@@ -10,7 +10,18 @@
 
 namespace prefill {
 
-static_assert(kHeadDim == 128 || kHeadDim == 64, "the two-tile kernels are built for head_dim 128 and 64");
+static_assert(kHeadDim == 128 || kHeadDim == 96 || kHeadDim == 64, "the two-tile kernels are built for head_dim 128, 96 and 64");
+
+// The kernels' names carry the head dimension they were built for.
+#if SINGE_HEAD_DIM == 128
+#define SINGE_PAIR_DIM d128
+#elif SINGE_HEAD_DIM == 96
+#define SINGE_PAIR_DIM d96
+#else
+#define SINGE_PAIR_DIM d64
+#endif
+#define SINGE_PAIR_JOIN_(A, B, C, D, E) A##_##B##_##C##_##D##_##E
+#define SINGE_PAIR_JOIN(A, B, C, D, E) SINGE_PAIR_JOIN_(A, B, C, D, E)
 
 constexpr int kPairWaves = 4;
 constexpr unsigned int kPairRows = 64u * kPairWaves;  // query rows of a workgroup
@@ -18,6 +29,12 @@ constexpr int kPairStages = 4;                        // of K and of V: a tile i
 constexpr int kPairAhead = kPairStages - 1;
 constexpr int kPairValueBase = kPairStages * kTileBytes;
 constexpr int kPairLdsBytes = 2 * kPairStages * kTileBytes;
+
+// A tile's direct-to-LDS loads fill whole 256-byte LDS rows, sixteen 16-byte places each, from cache rows of
+// kGlobalRowBytes.  Below head_dim 128 some places hold no chunk of the row: their lanes fetch one of the row's chunks
+// again, which lands where nobody reads, so the load needs no predicate (and what the half-used last dim block of an odd
+// multiple of 16 would read there is finite).
+SINGE_DEVICE unsigned int fetched_chunk(unsigned int chunk_of_place) { return chunk_of_place % (kGlobalRowBytes / 16u); }
 
 typedef v4i16_t __attribute__((address_space(3))) * lds_tr_t;
 
@@ -151,6 +168,8 @@ SINGE_DEVICE bool fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t&
     }
 #if SINGE_HEAD_DIM == 128
 #include "prefill_pair_block_d128.inc"
+#elif SINGE_HEAD_DIM == 96
+#include "prefill_pair_block_d96.inc"
 #else
 #include "prefill_pair_block_d64.inc"
 #endif

@@ -1,7 +1,7 @@
 """Deals the work of one 32-key block of two 32-row tiles out over the slots behind its matrix instructions and writes
-the block as the text fold_pair_block includes (prefill_pair_block_d128.inc, prefill_pair_block_d64.inc).
+the block as the text fold_pair_block includes (prefill_pair_block_d128.inc, _d96.inc, _d64.inc).
 
-    python3 singe_amd/csrc/prefill_pair_deal.py          (rewrites both files beside this script)
+    python3 singe_amd/csrc/prefill_pair_deal.py          (rewrites the files beside this script)
 
 A block at head_dim D is 2 * D / 16 score products of the NEXT block (tile A's and tile B's chains alternating, so that a
 product never follows the one it accumulates onto) and 4 * ceil(D / 32) value products of this block (A's two 16-key
@@ -106,7 +106,7 @@ HEADER = """// One 32-key block of two 32-row tiles at head_dim {dim}, slot by s
 
 if __name__ == "__main__":
     here = os.path.dirname(os.path.abspath(__file__))
-    for dim, budget, load_slots in ((128, 7.0, (0, 2, 4, 6)), (64, 14.0, (0, 1, 2, 3))):
+    for dim, budget, load_slots in ((128, 7.0, (0, 2, 4, 6)), (96, 9.0, (0, 2, 4, 5)), (64, 14.0, (0, 1, 2, 3))):
         body, used = deal(dim // 16, (dim + 31) // 32, budget, load_slots)
         with open(os.path.join(here, f"prefill_pair_block_d{dim}.inc"), "w") as out:
             out.write(HEADER.format(dim=dim, used=" ".join(f"{u:.0f}" for u in used)) + body)

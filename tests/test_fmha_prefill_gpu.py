@@ -239,37 +239,39 @@ def test_two_tiles_a_wave_f16(two_tiles_a_wave, causal):
     (1, 256, 256, 1, 1), (2, 512, 512, 4, 2), (1, 100, 128, 3, 1), (1, 1024, 1024, 8, 8), (1, 640, 1024, 4, 1), (1, 1024, 320, 2, 1),
     (1, 257, 257, 2, 1), (1, 1000, 1000, 2, 2), (2, 300, 191, 2, 1), (1, 350, 607, 3, 3), (1, 40, 33, 1, 1), (1, 64, 1, 1, 1),
 ])
-def test_two_tiles_a_wave_head_dim_64(two_tiles_a_wave, batch, query_len, key_len, heads, kv_heads, causal):
-    # the head_dim 64 build of the two-tile kernel: whole key tiles and last tiles that are not
-    q, k, v = make(batch, query_len, key_len, heads, kv_heads, seed=query_len * 13 + key_len, dim=64)
+@pytest.mark.parametrize("dim", [64, 96])
+def test_two_tiles_a_wave_head_dim_64_and_96(two_tiles_a_wave, batch, query_len, key_len, heads, kv_heads, causal, dim):
+    # the head_dim 64 and 96 builds of the two-tile kernel: whole key tiles and last tiles that are not
+    q, k, v = make(batch, query_len, key_len, heads, kv_heads, seed=query_len * 13 + key_len, dim=dim)
     from singe_amd import _native
     import ctypes
-    config = A.FmhaPrefillConfig.contiguous(batch, query_len, key_len, heads, kv_heads, 64, 0.125, causal)
+    config = A.FmhaPrefillConfig.contiguous(batch, query_len, key_len, heads, kv_heads, dim, 0.125, causal)
     assert _native.lib().singe_hip_dense_prefill_rows_per_wave(ctypes.byref(config._c())) == 64
     got, lse, want, want_lse = run(q, k, v, causal)
-    check(got, lse, want, want_lse, f"two tiles, head_dim 64: {batch}x{query_len}x{key_len} h{heads}/{kv_heads} causal={causal}")
+    check(got, lse, want, want_lse, f"two tiles, head_dim {dim}: {batch}x{query_len}x{key_len} h{heads}/{kv_heads} causal={causal}")
 
 
+@pytest.mark.parametrize("dim", [64, 96])
 @pytest.mark.parametrize("causal", [True, False])
-def test_two_tiles_a_wave_head_dim_64_f16_and_nan_behind_the_last_key(two_tiles_a_wave, causal):
-    q, k_all, v_all = (t.to(torch.float16) for t in make(1, 600, 1000 + 96, 4, 2, seed=17, dim=64))
+def test_two_tiles_a_wave_head_dim_64_and_96_f16_and_nan_behind_the_last_key(two_tiles_a_wave, causal, dim):
+    q, k_all, v_all = (t.to(torch.float16) for t in make(1, 600, 1000 + 96, 4, 2, seed=17, dim=dim))
     k_all[:, 1000:] = float("nan")
     v_all[:, 1000:] = float("nan")
     k, v = k_all[:, :1000], v_all[:, :1000]
-    config = A.FmhaPrefillConfig.contiguous(1, 600, 1000, 4, 2, 64, 0.125, causal)
+    config = A.FmhaPrefillConfig.contiguous(1, 600, 1000, 4, 2, dim, 0.125, causal)
     out = torch.full_like(q, float("nan"))
     lse = torch.full((1, 4, 600), float("nan"), device="cuda")
     A.fmha_prefill_lse_f16(None, out, lse, q, k, v, config)
     torch.cuda.synchronize()
     want, want_lse = oracle.fmha_prefill_lse_f32(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy(), batch=1,
-                                                 query_len=600, key_len=1000, heads=4, kv_heads=2, head_dim=64, scale=0.125,
+                                                 query_len=600, key_len=1000, heads=4, kv_heads=2, head_dim=dim, scale=0.125,
                                                  causal=causal, threads=8)
     gap = np.abs(out.float().cpu().numpy() - want)
     assert gap.max() <= MAX_ABS / 6 and gap.mean() <= MEAN_ABS / 6, (gap.max(), gap.mean())
     assert np.abs(lse.cpu().numpy() - want_lse).max() <= LSE_ABS
 
 
-@pytest.mark.parametrize("dim", [128, 64])
+@pytest.mark.parametrize("dim", [128, 64, 96])
 @pytest.mark.parametrize("causal", [True, False])
 def test_two_tiles_a_wave_head_major_layout(two_tiles_a_wave, causal, dim):
     # tensors stored [batch, heads, len, dim] (strides of their own for every operand), a key count that leaves a last

@@ -18,7 +18,8 @@ from singe_amd import build
 CSRC = os.path.join(os.path.dirname(build.__file__), "csrc")
 # (source, extra flags): every build of the two-tile kernels
 BUILDS = [("fmha_prefill_pair.hip", []), ("paged_attention_pair.hip", []), ("fmha_prefill_pair.hip", ["-DSINGE_HEAD_DIM=64"]),
-          ("paged_attention_pair.hip", ["-DSINGE_HEAD_DIM=64"])]
+          ("paged_attention_pair.hip", ["-DSINGE_HEAD_DIM=64"]),
+          ("fmha_prefill_pair.hip", ["-DSINGE_HEAD_DIM=96"]), ("paged_attention_pair.hip", ["-DSINGE_HEAD_DIM=96"])]
 WAIT_STATES = 12
 
 
