@@ -315,11 +315,12 @@ typedef struct SingeFmhaPrefillConfig {
     uint8_t causal;   /* Rust bool: 0 or 1 */
 } SingeFmhaPrefillConfig;
 
-/* Tuning knob of the dense bf16 / f16 prefill at head_dim 128, 96 and 64: the query rows a wave takes.  32: four waves share a
+/* Tuning knob of the dense bf16 / f16 prefill at the multiples of 16 up to 128: the query rows a wave takes.  32: four waves share a
  * compute unit's SIMDs two by two, 128 rows a workgroup.  64: a wave has a SIMD to itself and folds every key block
  * into two 32-row tiles, 256 rows a workgroup; only calls without a mask, a window, a cap or key splits (sinks and
- * key lengths are taken) with a positive scale have this form, others keep 32.  0 (the default): 64 where the call has that form
- * and its 256-row tiles still fill the chip.  Results are the same up to the order in which a row's
+ * key lengths are taken) with a positive scale have this form, others keep 32.  0 (the default): 64 where the call has that form,
+ * its 256-row tiles still fill the chip and the head dimension is one the form is faster at (64 and up; 48 without
+ * the causal mask).  Results are the same up to the order in which a row's
  * reference point moves.  The counterpart of AttentionParameters::{warps, min_blocks}
  * (singe/src/backend/cuda/kernel_plan/source/parameters.rs:21-57). */
 SINGE_HIP_API void singe_hip_set_dense_prefill_rows_per_wave(uint32_t rows);
@@ -477,7 +478,7 @@ SINGE_HIP_API int32_t singe_hip_paged_attention_bf16(
 SINGE_HIP_API size_t singe_hip_paged_attention_scratch_bytes(const SingePagedAttentionProblem* problem);
 SINGE_HIP_API void singe_hip_set_paged_attention_splits(uint32_t splits);
 /* Packed rows a wave of the bf16 / f16 paged attention kernels takes, as singe_hip_set_dense_prefill_rows_per_wave: 32,
- * 64 (only calls at head_dim 128, 96 or 64 with a page size that is a power of two of at least 16 keys and a positive scale,
+ * 64 (only calls at a head_dim that is a multiple of 16 up to 128 with a page size that is a power of two of at least 16 keys and a positive scale,
  * without a softcap, a window or key splits have that form, with or without the fused query rotation; others keep
  * 32), or 0 (the default): 64 where the call has that form and its 256-row tiles still fill the chip. */
 SINGE_HIP_API void singe_hip_set_paged_attention_rows_per_wave(uint32_t rows);

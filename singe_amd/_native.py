@@ -18,7 +18,8 @@ CODE_OBJECT_PARTS = ("paged_decode", "fmha_prefill", "fmha_prefill_f32", "paged_
                      "fmha_prefill_d80", "paged_attention_d80", "fmha_prefill_d112", "paged_attention_d112",
                      "paged_decode_d32", "paged_decode_d16", "paged_decode_d48", "paged_decode_d80", "paged_decode_d96",
                      "paged_decode_d112", "fmha_prefill_pair", "paged_attention_pair", "fmha_prefill_pair_d64", "paged_attention_pair_d64", "fmha_prefill_pair_d96",
-                     "paged_attention_pair_d96")
+                     "paged_attention_pair_d96") + tuple(
+    f"{source}_pair_d{dim}" for dim in (112, 80, 48, 32, 16) for source in ("fmha_prefill", "paged_attention"))
 CODE_OBJECT_PATHS = [os.path.join(_HERE, f"singe_attention_gfx950.{part}.hsaco") for part in CODE_OBJECT_PARTS]
 
 c_size = ctypes.c_size_t

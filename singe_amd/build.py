@@ -76,6 +76,16 @@ PARTS = [
     ("paged_attention_pair_d64", "paged_attention_pair.hip", ["-DSINGE_HEAD_DIM=64"]),
     ("fmha_prefill_pair_d96", "fmha_prefill_pair.hip", ["-DSINGE_HEAD_DIM=96"]),
     ("paged_attention_pair_d96", "paged_attention_pair.hip", ["-DSINGE_HEAD_DIM=96"]),
+    ("fmha_prefill_pair_d112", "fmha_prefill_pair.hip", ["-DSINGE_HEAD_DIM=112"]),
+    ("paged_attention_pair_d112", "paged_attention_pair.hip", ["-DSINGE_HEAD_DIM=112"]),
+    ("fmha_prefill_pair_d80", "fmha_prefill_pair.hip", ["-DSINGE_HEAD_DIM=80"]),
+    ("paged_attention_pair_d80", "paged_attention_pair.hip", ["-DSINGE_HEAD_DIM=80"]),
+    ("fmha_prefill_pair_d48", "fmha_prefill_pair.hip", ["-DSINGE_HEAD_DIM=48"]),
+    ("paged_attention_pair_d48", "paged_attention_pair.hip", ["-DSINGE_HEAD_DIM=48"]),
+    ("fmha_prefill_pair_d32", "fmha_prefill_pair.hip", ["-DSINGE_HEAD_DIM=32"]),
+    ("paged_attention_pair_d32", "paged_attention_pair.hip", ["-DSINGE_HEAD_DIM=32"]),
+    ("fmha_prefill_pair_d16", "fmha_prefill_pair.hip", ["-DSINGE_HEAD_DIM=16"]),
+    ("paged_attention_pair_d16", "paged_attention_pair.hip", ["-DSINGE_HEAD_DIM=16"]),
 ]
 HOST_SOURCES = ["hip_runtime_loader.cpp", "module.cpp", "paged_decode.cpp", "fmha_prefill.cpp", "paged_attention.cpp",
                 "general_attention.cpp", "fmha_decode.cpp", "paged_rows_f32.cpp", "latent_attention.cpp", "cache_ops.cpp",

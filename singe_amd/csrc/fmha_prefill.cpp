@@ -145,14 +145,19 @@ int32_t prefill_f32(void* stream, float* out, size_t out_len, float* lse, size_t
     return launch(kernel, static_cast<unsigned>(groups), 1, 1, 256, stream, args);
 }
 
-// Whether a call without options runs on the kernel that gives a wave two 32-row tiles: head_dim 128, 96 or 64, a positive
+// Whether a call without options runs on the kernel that gives a wave two 32-row tiles: a head_dim that is a multiple of 16 up to 128, a positive
 // scale, no heads packed into one tile, and (unless the knob says 64) 256-row tiles that still fill the chip.
 bool two_tiles_a_wave(const SingeFmhaPrefillConfig& c) {
     const uint32_t wanted = g_rows_per_wave.load(std::memory_order_relaxed);
-    if (wanted == 32 || (c.head_dim != 128 && c.head_dim != 96 && c.head_dim != 64) || c.key_len == 0 || !(c.scale > 0.0f) || dense_prefill_packs_heads(c))
+    if (wanted == 32 || !has_pair_build(static_cast<long long>(c.head_dim)) || c.key_len == 0 || !(c.scale > 0.0f) || dense_prefill_packs_heads(c))
         return false;
     const uint64_t rows = (static_cast<uint64_t>(c.batch) * c.heads + 7) / 8 * 8, pair_tiles = (c.query_len + 255) / 256;
-    return wanted == 64 || rows * ((pair_tiles + 1) / 2) >= compute_units();
+    if (wanted == 64) return true;
+    // Measured against the 32-row kernel at batch 4 x 32 heads x 4096: faster from head_dim 64 up (1.02 - 1.14 x), at 48
+    // without the causal mask only (1.09 x; 0.97 x with it), slower at 32 and 16 under the mask, where the softmax's vector
+    // instructions bound both kernels and two waves a SIMD share them out better than one.
+    if (c.head_dim < 48 || (c.head_dim == 48 && c.causal)) return false;
+    return rows * ((pair_tiles + 1) / 2) >= compute_units();
 }
 
 int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t lse_len, bool with_lse,
@@ -250,7 +255,7 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
         groups *= splits;
     }
     const long long head_dim = static_cast<long long>(c.head_dim);
-    // Long rows without options at head_dim 128, 96 or 64: the kernel that gives a wave two 32-row tiles (256 query rows a
+    // Long rows without options: the kernel that gives a wave two 32-row tiles (256 query rows a
     // workgroup, one workgroup a compute unit), when its launch still fills the chip; a build of its own where the last
     // key tile is not whole.
     if (!with_options && splits == 1 && two_tiles_a_wave(c)) {
@@ -259,7 +264,7 @@ int32_t prefill(void* stream, uint16_t* out, size_t out_len, float* lse, size_t 
         args.query_tiles = pair_tiles;
         // (the builds that take a last tile that is not whole also take a key count of their own for every batch entry)
         const bool ragged = c.key_len % 64 != 0 || options.key_lengths != nullptr;
-        const KernelId pair = static_cast<KernelId>((c.head_dim == 64 ? kPrefillPairD64 : c.head_dim == 96 ? kPrefillPairD96 : kPrefillPair) + (c.causal ? 0 : 1) + (f16 ? 2 : 0) + (ragged ? 4 : 0));
+        const KernelId pair = static_cast<KernelId>(pair_kernels_at(static_cast<long long>(c.head_dim), false) + (c.causal ? 0 : 1) + (f16 ? 2 : 0) + (ragged ? 4 : 0));
         return launch(pair, static_cast<unsigned>(pair_groups), 1, 1, 256, stream, args);
     }
     const KernelId kernel = static_cast<KernelId>((f16 ? kPrefillCausalF16 : kPrefillCausal) + (c.causal ? 0 : 1) + (with_options ? 4 : 0));

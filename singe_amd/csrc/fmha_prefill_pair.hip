@@ -289,6 +289,7 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
         for (int db = 0; db < kDimBlocks; ++db)
 #pragma unroll
             for (int quad = 0; quad < 4; ++quad) {
+                if (32 * db + 8 * quad >= kHeadDim) continue;  // (the last dim block of an odd multiple of 16 is half)
                 uint2 packed;
                 packed.x = pack_pair(half, state.out[db][4 * quad + 0] * inverse, state.out[db][4 * quad + 1] * inverse);
                 packed.y = pack_pair(half, state.out[db][4 * quad + 2] * inverse, state.out[db][4 * quad + 3] * inverse);

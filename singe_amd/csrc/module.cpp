@@ -336,6 +336,46 @@ const char* const kKernelNames[kKernelCount] = {
     "singe_paged_attention_pair_f16_d96_i32", "singe_paged_attention_pair_f16_d96_i64",
     "singe_rotary_paged_attention_pair_bf16_d96_i32", "singe_rotary_paged_attention_pair_bf16_d96_i64",
     "singe_rotary_paged_attention_pair_f16_d96_i32", "singe_rotary_paged_attention_pair_f16_d96_i64",
+    "singe_fmha_prefill_pair_bf16_d112_causal", "singe_fmha_prefill_pair_bf16_d112_full",
+    "singe_fmha_prefill_pair_f16_d112_causal", "singe_fmha_prefill_pair_f16_d112_full",
+    "singe_fmha_prefill_pair_bf16_d112_causal_ragged", "singe_fmha_prefill_pair_bf16_d112_full_ragged",
+    "singe_fmha_prefill_pair_f16_d112_causal_ragged", "singe_fmha_prefill_pair_f16_d112_full_ragged",
+    "singe_paged_attention_pair_bf16_d112_i32", "singe_paged_attention_pair_bf16_d112_i64",
+    "singe_paged_attention_pair_f16_d112_i32", "singe_paged_attention_pair_f16_d112_i64",
+    "singe_rotary_paged_attention_pair_bf16_d112_i32", "singe_rotary_paged_attention_pair_bf16_d112_i64",
+    "singe_rotary_paged_attention_pair_f16_d112_i32", "singe_rotary_paged_attention_pair_f16_d112_i64",
+    "singe_fmha_prefill_pair_bf16_d80_causal", "singe_fmha_prefill_pair_bf16_d80_full",
+    "singe_fmha_prefill_pair_f16_d80_causal", "singe_fmha_prefill_pair_f16_d80_full",
+    "singe_fmha_prefill_pair_bf16_d80_causal_ragged", "singe_fmha_prefill_pair_bf16_d80_full_ragged",
+    "singe_fmha_prefill_pair_f16_d80_causal_ragged", "singe_fmha_prefill_pair_f16_d80_full_ragged",
+    "singe_paged_attention_pair_bf16_d80_i32", "singe_paged_attention_pair_bf16_d80_i64",
+    "singe_paged_attention_pair_f16_d80_i32", "singe_paged_attention_pair_f16_d80_i64",
+    "singe_rotary_paged_attention_pair_bf16_d80_i32", "singe_rotary_paged_attention_pair_bf16_d80_i64",
+    "singe_rotary_paged_attention_pair_f16_d80_i32", "singe_rotary_paged_attention_pair_f16_d80_i64",
+    "singe_fmha_prefill_pair_bf16_d48_causal", "singe_fmha_prefill_pair_bf16_d48_full",
+    "singe_fmha_prefill_pair_f16_d48_causal", "singe_fmha_prefill_pair_f16_d48_full",
+    "singe_fmha_prefill_pair_bf16_d48_causal_ragged", "singe_fmha_prefill_pair_bf16_d48_full_ragged",
+    "singe_fmha_prefill_pair_f16_d48_causal_ragged", "singe_fmha_prefill_pair_f16_d48_full_ragged",
+    "singe_paged_attention_pair_bf16_d48_i32", "singe_paged_attention_pair_bf16_d48_i64",
+    "singe_paged_attention_pair_f16_d48_i32", "singe_paged_attention_pair_f16_d48_i64",
+    "singe_rotary_paged_attention_pair_bf16_d48_i32", "singe_rotary_paged_attention_pair_bf16_d48_i64",
+    "singe_rotary_paged_attention_pair_f16_d48_i32", "singe_rotary_paged_attention_pair_f16_d48_i64",
+    "singe_fmha_prefill_pair_bf16_d32_causal", "singe_fmha_prefill_pair_bf16_d32_full",
+    "singe_fmha_prefill_pair_f16_d32_causal", "singe_fmha_prefill_pair_f16_d32_full",
+    "singe_fmha_prefill_pair_bf16_d32_causal_ragged", "singe_fmha_prefill_pair_bf16_d32_full_ragged",
+    "singe_fmha_prefill_pair_f16_d32_causal_ragged", "singe_fmha_prefill_pair_f16_d32_full_ragged",
+    "singe_paged_attention_pair_bf16_d32_i32", "singe_paged_attention_pair_bf16_d32_i64",
+    "singe_paged_attention_pair_f16_d32_i32", "singe_paged_attention_pair_f16_d32_i64",
+    "singe_rotary_paged_attention_pair_bf16_d32_i32", "singe_rotary_paged_attention_pair_bf16_d32_i64",
+    "singe_rotary_paged_attention_pair_f16_d32_i32", "singe_rotary_paged_attention_pair_f16_d32_i64",
+    "singe_fmha_prefill_pair_bf16_d16_causal", "singe_fmha_prefill_pair_bf16_d16_full",
+    "singe_fmha_prefill_pair_f16_d16_causal", "singe_fmha_prefill_pair_f16_d16_full",
+    "singe_fmha_prefill_pair_bf16_d16_causal_ragged", "singe_fmha_prefill_pair_bf16_d16_full_ragged",
+    "singe_fmha_prefill_pair_f16_d16_causal_ragged", "singe_fmha_prefill_pair_f16_d16_full_ragged",
+    "singe_paged_attention_pair_bf16_d16_i32", "singe_paged_attention_pair_bf16_d16_i64",
+    "singe_paged_attention_pair_f16_d16_i32", "singe_paged_attention_pair_f16_d16_i64",
+    "singe_rotary_paged_attention_pair_bf16_d16_i32", "singe_rotary_paged_attention_pair_bf16_d16_i64",
+    "singe_rotary_paged_attention_pair_f16_d16_i32", "singe_rotary_paged_attention_pair_f16_d16_i64",
 };
 
 // The code object is built in parts, one per kernel source (so they compile side by side and a process loads only
@@ -351,6 +391,11 @@ const char* const kPartNames[kPartCount] = {
     "paged_decode_d16", "paged_decode_d48", "paged_decode_d80", "paged_decode_d96", "paged_decode_d112",
     "fmha_prefill_pair", "paged_attention_pair", "fmha_prefill_pair_d64", "paged_attention_pair_d64",
     "fmha_prefill_pair_d96", "paged_attention_pair_d96",
+    "fmha_prefill_pair_d112", "paged_attention_pair_d112",
+    "fmha_prefill_pair_d80", "paged_attention_pair_d80",
+    "fmha_prefill_pair_d48", "paged_attention_pair_d48",
+    "fmha_prefill_pair_d32", "paged_attention_pair_d32",
+    "fmha_prefill_pair_d16", "paged_attention_pair_d16",
 };
 
 namespace {
@@ -383,6 +428,7 @@ constexpr PartRun kPartRuns[] = {
     {38, 8},                      // the two-tile dense prefill at head_dim 64
     {39, 8},                      // the two-tile paged attention at head_dim 64
     {40, 8}, {41, 8},             // both at head_dim 96
+    {42, 8}, {43, 8}, {44, 8}, {45, 8}, {46, 8}, {47, 8}, {48, 8}, {49, 8}, {50, 8}, {51, 8},  // and at 112, 80, 48, 32, 16
 };
 constexpr int runs_total() {
     int total = 0;

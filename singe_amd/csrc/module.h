@@ -96,8 +96,21 @@ enum KernelId : int {
     // and the head_dim 96 builds of both
     kPrefillPairD96 = kPagedPairD64 + 8,
     kPagedPairD96 = kPrefillPairD96 + 8,
-    kKernelCount = kPagedPairD96 + 8
+    // and those for 112, 80, 48, 32, 16: sixteen each, the dense eight first
+    kPairOtherHeadDims = kPagedPairD96 + 8,
+    kKernelCount = kPairOtherHeadDims + 5 * 16
 };
+
+// The two-tile kernels (fmha_prefill_pair.hip, paged_attention_pair.hip) have a build for every multiple of 16 up to 128.
+inline bool has_pair_build(long long head_dim) { return head_dim >= 16 && head_dim <= 128 && head_dim % 16 == 0; }
+// The first of the eight dense (or paged) two-tile kernels built for a head dimension.
+inline int pair_kernels_at(long long head_dim, bool paged) {
+    if (head_dim == 128) return paged ? kPagedPair : kPrefillPair;
+    if (head_dim == 64) return paged ? kPagedPairD64 : kPrefillPairD64;
+    if (head_dim == 96) return paged ? kPagedPairD96 : kPrefillPairD96;
+    const int order = head_dim == 112 ? 0 : head_dim == 80 ? 1 : head_dim == 48 ? 2 : head_dim == 32 ? 3 : 4;
+    return kPairOtherHeadDims + 16 * order + (paged ? 8 : 0);
+}
 
 
 // The head_dim 64 build of a matrix-core kernel named by its head_dim 128 id.
@@ -165,7 +178,7 @@ inline int rotary_paged_attention_base(bool f16, bool softcap, long long head_di
 extern const char* const kKernelNames[kKernelCount];
 
 // Parts of the code object (one file each) and the part a kernel lives in.
-constexpr int kPartCount = 42;
+constexpr int kPartCount = 52;
 extern const char* const kPartNames[kPartCount];
 int kernel_part(int kernel);
 

@@ -79,11 +79,11 @@ uint32_t fixed_paged_attention_splits() {
 }
 
 // Whether a bf16 / f16 call without a fused rotation or key splits runs on the kernel that gives a wave two 32-row
-// tiles, and the grid it takes there: head_dim 128, 96 or 64, a page size that is a power of two of at least 16 keys, no cap, no
+// tiles, and the grid it takes there: a head_dim that is a multiple of 16 up to 128, a page size that is a power of two of at least 16 keys, no cap, no
 // window, a positive scale, and (unless the knob says 64) enough 256-row tiles to fill the chip.
 bool two_tiles_a_wave(const SingePagedAttentionProblem& p, RowTileGrid* grid) {
     const uint32_t wanted = g_paged_rows_per_wave.load(std::memory_order_relaxed);
-    if (wanted == 32 || (p.head_dim != 128 && p.head_dim != 96 && p.head_dim != 64) || p.has_softcap || p.has_window || p.tokens <= 0 || p.sequences <= 0 || p.kv_heads <= 0 ||
+    if (wanted == 32 || !has_pair_build(p.head_dim) || p.has_softcap || p.has_window || p.tokens <= 0 || p.sequences <= 0 || p.kv_heads <= 0 ||
         p.heads <= 0 || p.page_size < 16 || (p.page_size & (p.page_size - 1)) != 0)
         return false;
     // (the kernel works out where a page starts from a 32-bit count of a page's bytes)
@@ -321,7 +321,7 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
         args.has_query_norm = rotation->attributes->has_norm ? 1u : 0u;
         args.query_eps = rotation->attributes->eps;
     }
-    // Prefill-shaped plain calls at head_dim 128, 96 or 64 (with or without the fused query rotation) take the kernel that gives a
+    // Prefill-shaped plain calls at the matrix-core head dimensions (with or without the fused query rotation) take the kernel that gives a
     // wave two 32-row tiles (256 packed rows a workgroup, one workgroup a compute unit; paged_attention_pair.hip), when
     // its grid still fills the chip.
     RowTileGrid pair;
@@ -329,7 +329,7 @@ int32_t paged_attention(int32_t data_type, void* stream, const void* query_rows_
         args.row_tiles = static_cast<uint32_t>(pair.row_tiles);
         args.compact = pair.compact;
         args.longest_first = pair.longest_first;
-        const int kernel = (p.head_dim == 64 ? kPagedPairD64 : p.head_dim == 96 ? kPagedPairD96 : kPagedPair) + (wide ? 1 : 0) + (f16 ? 2 : 0) + (rotation != nullptr ? 4 : 0);
+        const int kernel = pair_kernels_at(p.head_dim, true) + (wide ? 1 : 0) + (f16 ? 2 : 0) + (rotation != nullptr ? 4 : 0);
         return launch(static_cast<KernelId>(kernel), static_cast<unsigned>(pair.blocks), 1, 1, 256, stream, args);
     }
     const unsigned grid = static_cast<unsigned>(blocks * splits);

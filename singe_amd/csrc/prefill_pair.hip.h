@@ -2,7 +2,7 @@
 // (fmha_prefill_pair.hip says why and how; paged_attention_pair.hip is the same loop over a paged cache): the score
 // products as assembly with their register classes spelled out, Q^T loaded straight into accumulation registers, the
 // row maxima of two score tiles in alternating chains, and fold_pair_block, one 32-key block of both tiles with its
-// vector work dealt out over the slots between its matrix instructions (32 at head_dim 128, 24 at 96, 16 at 64: the text of the
+// vector work dealt out over the slots between its matrix instructions (32 at head_dim 128, 24 at 96, 16 at 64, ...: the text of the
 // block is written by prefill_pair_deal.py).
 #pragma once
 
@@ -10,16 +10,12 @@
 
 namespace prefill {
 
-static_assert(kHeadDim == 128 || kHeadDim == 96 || kHeadDim == 64, "the two-tile kernels are built for head_dim 128, 96 and 64");
+static_assert(kHeadDim % 16 == 0 && kHeadDim >= 16 && kHeadDim <= 128, "the two-tile kernels are built for the multiples of 16 up to 128");
 
 // The kernels' names carry the head dimension they were built for.
-#if SINGE_HEAD_DIM == 128
-#define SINGE_PAIR_DIM d128
-#elif SINGE_HEAD_DIM == 96
-#define SINGE_PAIR_DIM d96
-#else
-#define SINGE_PAIR_DIM d64
-#endif
+#define SINGE_PAIR_DIM_(N) d##N
+#define SINGE_PAIR_DIM_OF(N) SINGE_PAIR_DIM_(N)
+#define SINGE_PAIR_DIM SINGE_PAIR_DIM_OF(SINGE_HEAD_DIM)
 #define SINGE_PAIR_JOIN_(A, B, C, D, E) A##_##B##_##C##_##D##_##E
 #define SINGE_PAIR_JOIN(A, B, C, D, E) SINGE_PAIR_JOIN_(A, B, C, D, E)
 
@@ -168,10 +164,20 @@ SINGE_DEVICE bool fold_pair_block(Half half, RowState& A, RowState& B, f32x16_t&
     }
 #if SINGE_HEAD_DIM == 128
 #include "prefill_pair_block_d128.inc"
+#elif SINGE_HEAD_DIM == 112
+#include "prefill_pair_block_d112.inc"
 #elif SINGE_HEAD_DIM == 96
 #include "prefill_pair_block_d96.inc"
-#else
+#elif SINGE_HEAD_DIM == 80
+#include "prefill_pair_block_d80.inc"
+#elif SINGE_HEAD_DIM == 64
 #include "prefill_pair_block_d64.inc"
+#elif SINGE_HEAD_DIM == 48
+#include "prefill_pair_block_d48.inc"
+#elif SINGE_HEAD_DIM == 32
+#include "prefill_pair_block_d32.inc"
+#else
+#include "prefill_pair_block_d16.inc"
 #endif
 #undef QK
 #undef PV

@@ -1,5 +1,5 @@
 """Deals the work of one 32-key block of two 32-row tiles out over the slots behind its matrix instructions and writes
-the block as the text fold_pair_block includes (prefill_pair_block_d128.inc, _d96.inc, _d64.inc).
+the block as the text fold_pair_block includes (prefill_pair_block_d128.inc and one for every other multiple of 16).
 
     python3 singe_amd/csrc/prefill_pair_deal.py          (rewrites the files beside this script)
 
@@ -106,7 +106,9 @@ HEADER = """// One 32-key block of two 32-row tiles at head_dim {dim}, slot by s
 
 if __name__ == "__main__":
     here = os.path.dirname(os.path.abspath(__file__))
-    for dim, budget, load_slots in ((128, 7.0, (0, 2, 4, 6)), (96, 9.0, (0, 2, 4, 5)), (64, 14.0, (0, 1, 2, 3))):
+    # (the smallest budget the dealing succeeds with, and the slots of the four loads, for every head dimension)
+    for dim, budget, load_slots in ((128, 7.0, (0, 2, 4, 6)), (112, 8.0, (0, 2, 4, 6)), (96, 9.0, (0, 2, 4, 5)), (80, 10.0, (0, 2, 4, 6)),
+                                    (64, 14.0, (0, 1, 2, 3)), (48, 16.0, (0, 1, 2, 3)), (32, 27.0, (0, 1, 2, 3)), (16, 36.0, (0, 1, 2, 3))):
         body, used = deal(dim // 16, (dim + 31) // 32, budget, load_slots)
         with open(os.path.join(here, f"prefill_pair_block_d{dim}.inc"), "w") as out:
             out.write(HEADER.format(dim=dim, used=" ".join(f"{u:.0f}" for u in used)) + body)

@@ -63,7 +63,7 @@ def test_paged_attention_f16(heads, kv_heads, page_size, index_dtype, options):
 
 
 @pytest.mark.parametrize("causal", [True, False])
-@pytest.mark.parametrize("dim", [128, 64, 96])
+@pytest.mark.parametrize("dim", [128, 64, 96, 112, 80, 48, 32, 16])
 @pytest.mark.parametrize("heads,kv_heads,page_size,index_dtype", [(8, 1, 16, torch.int32), (64, 8, 16, torch.int64), (8, 2, 64, torch.int32)])
 def test_paged_attention_f16_two_tiles_a_wave(heads, kv_heads, page_size, index_dtype, causal, dim):
     # the f16 builds of the kernel that gives a wave two 32-row tiles: chunks of several 256-row tiles, key counts either

@@ -239,9 +239,9 @@ def test_two_tiles_a_wave_f16(two_tiles_a_wave, causal):
     (1, 256, 256, 1, 1), (2, 512, 512, 4, 2), (1, 100, 128, 3, 1), (1, 1024, 1024, 8, 8), (1, 640, 1024, 4, 1), (1, 1024, 320, 2, 1),
     (1, 257, 257, 2, 1), (1, 1000, 1000, 2, 2), (2, 300, 191, 2, 1), (1, 350, 607, 3, 3), (1, 40, 33, 1, 1), (1, 64, 1, 1, 1),
 ])
-@pytest.mark.parametrize("dim", [64, 96])
-def test_two_tiles_a_wave_head_dim_64_and_96(two_tiles_a_wave, batch, query_len, key_len, heads, kv_heads, causal, dim):
-    # the head_dim 64 and 96 builds of the two-tile kernel: whole key tiles and last tiles that are not
+@pytest.mark.parametrize("dim", [16, 32, 48, 64, 80, 96, 112])
+def test_two_tiles_a_wave_other_head_dims(two_tiles_a_wave, batch, query_len, key_len, heads, kv_heads, causal, dim):
+    # the other builds of the two-tile kernel: whole key tiles and last tiles that are not
     q, k, v = make(batch, query_len, key_len, heads, kv_heads, seed=query_len * 13 + key_len, dim=dim)
     from singe_amd import _native
     import ctypes
@@ -251,9 +251,9 @@ def test_two_tiles_a_wave_head_dim_64_and_96(two_tiles_a_wave, batch, query_len,
     check(got, lse, want, want_lse, f"two tiles, head_dim {dim}: {batch}x{query_len}x{key_len} h{heads}/{kv_heads} causal={causal}")
 
 
-@pytest.mark.parametrize("dim", [64, 96])
+@pytest.mark.parametrize("dim", [16, 32, 48, 64, 80, 96, 112])
 @pytest.mark.parametrize("causal", [True, False])
-def test_two_tiles_a_wave_head_dim_64_and_96_f16_and_nan_behind_the_last_key(two_tiles_a_wave, causal, dim):
+def test_two_tiles_a_wave_other_head_dims_f16_and_nan_behind_the_last_key(two_tiles_a_wave, causal, dim):
     q, k_all, v_all = (t.to(torch.float16) for t in make(1, 600, 1000 + 96, 4, 2, seed=17, dim=dim))
     k_all[:, 1000:] = float("nan")
     v_all[:, 1000:] = float("nan")
@@ -271,7 +271,7 @@ def test_two_tiles_a_wave_head_dim_64_and_96_f16_and_nan_behind_the_last_key(two
     assert np.abs(lse.cpu().numpy() - want_lse).max() <= LSE_ABS
 
 
-@pytest.mark.parametrize("dim", [128, 64, 96])
+@pytest.mark.parametrize("dim", [128, 64, 96, 80, 48, 16])
 @pytest.mark.parametrize("causal", [True, False])
 def test_two_tiles_a_wave_head_major_layout(two_tiles_a_wave, causal, dim):
     # tensors stored [batch, heads, len, dim] (strides of their own for every operand), a key count that leaves a last

@@ -397,7 +397,9 @@ def two_tiles_a_wave():
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("heads,kv_heads,page_size,dim", [(8, 1, 16, 128), (64, 8, 16, 128), (8, 2, 32, 128), (4, 1, 64, 128), (8, 2, 128, 128),
                                                           (4, 4, 16, 128), (8, 1, 16, 64), (64, 8, 16, 64), (8, 2, 64, 64), (4, 4, 32, 64),
-                                                          (8, 1, 16, 96), (64, 8, 16, 96), (8, 2, 64, 96), (4, 4, 32, 96)])
+                                                          (8, 1, 16, 96), (64, 8, 16, 96), (8, 2, 64, 96), (4, 4, 32, 96),
+                                                          (8, 1, 16, 112), (8, 2, 64, 112), (64, 8, 16, 80), (4, 4, 32, 80), (8, 1, 16, 48),
+                                                          (8, 2, 128, 48), (64, 8, 16, 32), (4, 1, 64, 32), (8, 2, 16, 16), (4, 4, 256, 16)])
 def test_two_tiles_a_wave_ragged_sequences_match_oracle(two_tiles_a_wave, heads, kv_heads, page_size, dim, causal, index_dtype):
     # the shapes of the ragged test (decode, full prefill, chunked prefill, no keys, more queries than keys) and
     # chunks long enough for several 256-row tiles, several key tiles ahead of the mask and key counts either side of

@@ -17,9 +17,8 @@ from singe_amd import build
 
 CSRC = os.path.join(os.path.dirname(build.__file__), "csrc")
 # (source, extra flags): every build of the two-tile kernels
-BUILDS = [("fmha_prefill_pair.hip", []), ("paged_attention_pair.hip", []), ("fmha_prefill_pair.hip", ["-DSINGE_HEAD_DIM=64"]),
-          ("paged_attention_pair.hip", ["-DSINGE_HEAD_DIM=64"]),
-          ("fmha_prefill_pair.hip", ["-DSINGE_HEAD_DIM=96"]), ("paged_attention_pair.hip", ["-DSINGE_HEAD_DIM=96"])]
+BUILDS = [(source, [] if dim == 128 else [f"-DSINGE_HEAD_DIM={dim}"]) for dim in (128, 112, 96, 80, 64, 48, 32, 16)
+          for source in ("fmha_prefill_pair.hip", "paged_attention_pair.hip")]
 WAIT_STATES = 12
 
 
@@ -49,16 +48,29 @@ def instructions(assembly):
         yield stripped.split(";")[0].strip(), inside
 
 
-@pytest.mark.parametrize("name,flags", BUILDS, ids=lambda value: value if isinstance(value, str) else "".join(value) or "d128")
-def test_nothing_touches_a_score_product_before_it_is_done(name, flags):
+def assembly_of(name, flags):
     source = os.path.join(CSRC, name)
-    steps = 4 if flags else 8  # score products a chain
     with tempfile.TemporaryDirectory() as scratch:
         listing = os.path.join(scratch, "pair.s")
         command = [build.hipcc()] + [flag for flag in build.HIPCC_FLAGS if flag != "--genco"] + flags + [
             "--cuda-device-only", "-S", "-I", os.path.dirname(source), source, "-o", listing]
         subprocess.run(command, check=True, capture_output=True)
-        program = list(instructions(open(listing).read()))
+        return open(listing).read()
+
+
+@pytest.fixture(scope="module")
+def listings():
+    """Every build's assembly, compiled side by side (a build takes a quarter of a minute)."""
+    from concurrent.futures import ThreadPoolExecutor
+    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
+        texts = list(pool.map(lambda item: assembly_of(*item), BUILDS))
+    return {(name, tuple(flags)): text for (name, flags), text in zip(BUILDS, texts)}
+
+
+@pytest.mark.parametrize("name,flags", BUILDS, ids=lambda value: value if isinstance(value, str) else "".join(value) or "d128")
+def test_nothing_touches_a_score_product_before_it_is_done(listings, name, flags):
+    steps = int(flags[0].split("=")[1]) // 16 if flags else 8  # score products a chain
+    program = list(instructions(listings[(name, tuple(flags))]))
     products = 0
     for at, (text, inside) in enumerate(program):
         if not (inside and text.startswith("v_mfma")):

@@ -62,7 +62,7 @@ def paged_attention_random_shape(seed, rng, two_tiles):
     tokens = query_offsets[-1]
     gen = torch.Generator(device="cuda")
     gen.manual_seed(seed)
-    dim = (128, 64, 96)[seed % 3] if two_tiles else 128  # (every build of the two-tile kernel)
+    dim = (128, 64, 96, 112, 80, 48, 32, 16)[seed % 8] if two_tiles else 128  # (every build of the two-tile kernel)
     q = torch.randn((tokens, heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
     kc = torch.randn((page_count, page_size, kv_heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
     vc = torch.randn((page_count, page_size, kv_heads, dim), generator=gen, device="cuda").to(torch.bfloat16)
@@ -88,7 +88,7 @@ def paged_attention_random_shape(seed, rng, two_tiles):
     assert np.abs(got_lse[~empty] - want_lse[~empty]).max(initial=0.0) <= LSE_ABS, case
 
 
-@pytest.mark.parametrize("rows_per_wave,dim", [(0, 128), (64, 128), (64, 64), (64, 96)])
+@pytest.mark.parametrize("rows_per_wave,dim", [(0, 128), (64, 128), (64, 64), (64, 96), (64, 112), (64, 80), (64, 48), (64, 32), (64, 16)])
 @pytest.mark.parametrize("seed", range(12))
 def test_dense_prefill_random_shapes(seed, rows_per_wave, dim):
     # (64 rows a wave: the kernel that gives a wave two 32-row tiles, whatever the shape; larger shapes there, so that

@@ -150,7 +150,7 @@ def test_fused_rotation_refuses_what_it_does_not_take():
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("norm", [None, "plain", "weighted"])
-@pytest.mark.parametrize("dim", [128, 64, 96])
+@pytest.mark.parametrize("dim", [128, 64, 96, 112, 80, 48, 32, 16])
 @pytest.mark.parametrize("heads,kv_heads,page_size,table_dtype,index_dtype,causal", [
     (8, 2, 16, torch.float32, torch.int32, True), (64, 8, 16, torch.bfloat16, torch.int64, True), (8, 1, 64, torch.float16, torch.int32, False)])
 def test_fused_rotation_on_the_two_tile_kernel(heads, kv_heads, page_size, table_dtype, index_dtype, causal, norm, dtype, dim):
