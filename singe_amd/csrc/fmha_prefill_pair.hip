@@ -26,7 +26,8 @@
 // Grid: one workgroup of four waves per (batch, head, pair of 256-row query tiles), tile i from the end and tile i
 // from the start; ids laid out as in fmha_prefill.hip.  LDS: four stages of K and four of V (128 KiB), each tile
 // loaded three tiles ahead, straight from global memory, and waited for a tile after it was asked for (a wave alone
-// on its SIMD has nobody to cover a wait for fresh loads); one barrier per tile.
+// on its SIMD has nobody to cover a wait for fresh loads); one barrier per tile.  Behind the stages, 8 KiB a wave that
+// its output rows go through on their way out (32 KiB: all of a compute unit's 160 KiB are in use).
 #include "kernel_args.h"
 #include "prefill_pair.hip.h"
 
@@ -279,27 +280,25 @@ SINGE_DEVICE void fmha_prefill_pair_tile(const PrefillArgs& a, unsigned char* ld
         stage = next_stage;
     }
 
-    // Normalise and store.  Lane (query, hi) holds dims 32db + 8(r / 4) + 4hi + (r % 4).
-    auto store = [&](RowState& state, unsigned int query, bool valid) __attribute__((always_inline)) {
-        const float sum = swap32_sum(state.running_sum);
-        const float inverse = sum > 0.0f ? 1.0f / sum : 0.0f;
-        if (!valid) return;
-        uint16_t* row = a.out + batch * a.output_batch_stride + static_cast<size_t>(query) * a.output_sequence_stride + head * a.output_head_stride;
-#pragma unroll
-        for (int db = 0; db < kDimBlocks; ++db)
-#pragma unroll
-            for (int quad = 0; quad < 4; ++quad) {
-                if (32 * db + 8 * quad >= kHeadDim) continue;  // (the last dim block of an odd multiple of 16 is half)
-                uint2 packed;
-                packed.x = pack_pair(half, state.out[db][4 * quad + 0] * inverse, state.out[db][4 * quad + 1] * inverse);
-                packed.y = pack_pair(half, state.out[db][4 * quad + 2] * inverse, state.out[db][4 * quad + 3] * inverse);
-                *reinterpret_cast<uint2*>(row + 32 * db + 8 * quad + 4 * hi) = packed;
-            }
-        if (a.lse != nullptr && hi == 0)
-            a.lse[(static_cast<size_t>(batch) * a.heads + head) * a.query_len + query] = sum > 0.0f ? (state.reference + fast_log2(sum)) * kLn2 : -INFINITY;
-    };
-    store(A, query_a, valid_a);
-    store(B, query_b, valid_b);
+    // Normalise and store (store_rows).  (Storing as soon as a wave's own last tile is folded, up to three tiles before
+    // the workgroup's under the causal mask, was measured and is no faster: the wave then waits for its stores with the
+    // next tile's loads, and the others wait for it at the barrier.)
+    {
+        uint16_t* const rows = a.out + batch * a.output_batch_stride + head * a.output_head_stride;
+        unsigned char* const staging = lds + kPairLdsBytes + wave * (32u * kRowBytes);
+        auto store = [&](RowState& state, unsigned int tile_first, unsigned int query, bool valid) __attribute__((always_inline)) {
+            const float sum = swap32_sum(state.running_sum);
+            const float inverse = sum > 0.0f ? 1.0f / sum : 0.0f;
+            if (a.lse != nullptr && hi == 0 && valid)
+                a.lse[(static_cast<size_t>(batch) * a.heads + head) * a.query_len + query] = sum > 0.0f ? (state.reference + fast_log2(sum)) * kLn2 : -INFINITY;
+            store_rows(half, state, inverse, lane, staging, [&](unsigned int r) __attribute__((always_inline)) {
+                const unsigned int row = tile_first + r;
+                return row < a.query_len ? rows + static_cast<size_t>(row) * a.output_sequence_stride : nullptr;
+            });
+        };
+        store(A, first_row, query_a, valid_a);
+        store(B, first_row + 32u, query_b, valid_b);
+    }
     // (the next tile of the pair starts by loading into stages this one may still be reading)
     __syncthreads();
 }
@@ -323,7 +322,7 @@ SINGE_DEVICE void fmha_prefill_pair_body(const PrefillArgs& a, unsigned char* ld
 
 #define SINGE_FMHA_PREFILL_PAIR_KERNEL(NAME, CAUSAL, RAGGED, HALF)                                     \
     extern "C" __global__ __launch_bounds__(64 * kPairWaves, 1) void NAME(PrefillArgs args) {          \
-        __shared__ __attribute__((aligned(1024))) unsigned char prefill_lds[kPairLdsBytes];            \
+        __shared__ __attribute__((aligned(1024))) unsigned char prefill_lds[kPairLdsBytes + kPairStoreBytes]; \
         fmha_prefill_pair_body<CAUSAL, RAGGED, prefill::HALF>(args, prefill_lds);                      \
     }
 

@@ -25,6 +25,8 @@ constexpr int kPairStages = 4;                        // of K and of V: a tile i
 constexpr int kPairAhead = kPairStages - 1;
 constexpr int kPairValueBase = kPairStages * kTileBytes;
 constexpr int kPairLdsBytes = 2 * kPairStages * kTileBytes;
+// A tile of 32 output rows a wave, behind the stages of the kernels that store through LDS (store_rows below).
+constexpr int kPairStoreBytes = kPairWaves * 32 * kRowBytes;
 
 // A tile's direct-to-LDS loads fill whole 256-byte LDS rows, sixteen 16-byte places each, from cache rows of
 // kGlobalRowBytes.  Below head_dim 128 some places hold no chunk of the row: their lanes fetch one of the row's chunks
@@ -118,6 +120,38 @@ SINGE_DEVICE void row_maxima_2(float& ma, float& mb) {
         "v_mov_b32 %2, %0\n\tv_mov_b32 %3, %1\n\ts_nop 0\n\tv_permlane32_swap_b32 %0, %2\n\tv_permlane32_swap_b32 %1, %3\n\t"
         "v_max_f32 %0, %0, %2\n\tv_max_f32 %1, %1, %3"
         : "+v"(ma), "+v"(mb), "=&v"(ta), "=&v"(tb));
+}
+
+// Normalises the 32 rows of one tile, rounds them and stores them.  Lane (query, hi) holds dims 32 db + 8 (r / 4) +
+// 4 hi + (r % 4) of its row: stored from there, an instruction would touch 32 rows with sixteen bytes each.  The rows go
+// through the wave's own 8 KiB behind the stages instead (which it may use while other waves still fold their tiles):
+// chunk c of row q sits at place c ^ (q % 16), its halves swapped for q >= 16, so that neither the 8-byte writes nor the
+// 16-byte reads meet in a bank; lane l then takes place l % 16 of row 4 i + l / 16, and an instruction stores four whole
+// rows.  row_address(r): where row r of the tile goes, or null.  A wave's LDS operations run in order, so the next tile's
+// writes come after this one's reads.
+template <class Half, class RowAddress>
+SINGE_DEVICE void store_rows(Half half, const RowState& state, float inverse, unsigned int lane, unsigned char* staging, RowAddress&& row_address) {
+    const unsigned int column = lane & 31u, hi = lane >> 5;
+    unsigned char* const mine = staging + column * kRowBytes + 8u * (hi ^ (column >> 4));
+#pragma unroll
+    for (int db = 0; db < kDimBlocks; ++db)
+#pragma unroll
+        for (int quad = 0; quad < 4; ++quad) {
+            if (32 * db + 8 * quad >= kHeadDim) continue;  // (the last dim block of an odd multiple of 16 is half)
+            uint2 packed;
+            packed.x = pack_pair(half, state.out[db][4 * quad + 0] * inverse, state.out[db][4 * quad + 1] * inverse);
+            packed.y = pack_pair(half, state.out[db][4 * quad + 2] * inverse, state.out[db][4 * quad + 3] * inverse);
+            *reinterpret_cast<uint2*>(mine + 16u * ((4u * db + quad) ^ (column & 15u))) = packed;
+        }
+    const unsigned int row = lane >> 4, place = lane & 15u;
+#pragma unroll
+    for (unsigned int i = 0; i < 8; ++i) {
+        const unsigned int r = 4u * i + row, chunk = place ^ (r & 15u);
+        uint4 bits = *reinterpret_cast<const uint4*>(staging + r * kRowBytes + 16u * place);
+        if (i >= 4) bits = make_uint4(bits.z, bits.w, bits.x, bits.y);
+        uint16_t* const to = row_address(r);
+        if (to != nullptr && chunk < kGlobalRowBytes / 16u) *reinterpret_cast<uint4*>(to + 8u * chunk) = bits;
+    }
 }
 
 // One 32-key block b for both row tiles.  On entry a_cur / b_cur hold the raw scores of block b (shift_a / shift_b:
