@@ -143,7 +143,11 @@ struct TilePages {
     RawPage<FORM> positional;
 };
 
-template <class Half, int FORM, bool ANY>
+// IN_PAGE: the page size is a power of two of at least 32 keys, so the 32 keys of a tile lie in one page: one page id a
+// tile (instead of one a row), no division, and a key's place follows from the tile's.  A wave issues its instructions in
+// order, one every four or five clocks whatever their kind, so the scalar arithmetic of the paging is time the matrix
+// cores do not get from that wave.
+template <class Half, int FORM, bool ANY, bool IN_PAGE>
 SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* lds) {
     const unsigned int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63u;
     // The widths of a row in global memory: the built shape, or (ANY) whatever the problem says.
@@ -267,6 +271,11 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
     };
     auto lookup = [&](unsigned int tile) __attribute__((always_inline)) {
         TilePages<FORM> pages;
+        if constexpr (IN_PAGE) {
+            // (the tile's first key is one of the sequence's: tile < tiles)
+            pages.latent[0] = read_raw_page_uniform<FORM>(a.pages, static_cast<size_t>(span.page_start) + ((tile * kKeys) >> page_shift));
+            return pages;
+        }
 #pragma unroll
         for (int i = 0; i < 4; ++i)
             pages.latent[i] = read_raw_page_uniform<FORM>(a.pages, static_cast<size_t>(span.page_start) + entry_of(key_of(tile, wave + 8u * i)));
@@ -282,6 +291,36 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
     const unsigned int lane_chunk[2] = {16u * (lane ^ chunk_flip(wave & 15u)), 16u * (lane ^ chunk_flip((wave + 8u) & 15u))};
     auto issue_piece = [&](int piece, unsigned int tile, const TilePages<FORM>& pages, unsigned char* __restrict__ stage)
                            __attribute__((always_inline)) {
+        if constexpr (IN_PAGE) {
+            // The tile's page, its first key's slot in the caches, and the last row that holds a key of the sequence
+            // (rows past it re-read it and are masked): all the same for every lane.
+            const unsigned long long page = static_cast<unsigned long long>(pages.latent[0]);
+            const bool good = page < static_cast<unsigned long long>(a.cache_pages);
+            const unsigned int first_key = tile * kKeys, last = keys - 1u - first_key;
+            const size_t slot = static_cast<size_t>(page) * a.page_size + (first_key & (a.page_size - 1u));
+            if (piece < 4) {
+                const unsigned int row = wave + 8u * piece, kept = row < last ? row : last;
+                unsigned char* dest = stage + row * kLatentRowBytes;
+                if (good) {
+                    if (!ANY || lane_chunk[piece & 1] < 16u * latent_chunks)
+                        load_to_lds(latent_cache + (slot + kept) * latent_row_bytes, lane_chunk[piece & 1], dest);
+                } else {
+                    if (lane == 0) report_index_error(a.status);
+                    *reinterpret_cast<uint4*>(dest + 16u * lane) = make_uint4(0, 0, 0, 0);
+                }
+            } else if (wave < 4) {
+                const unsigned int kept = positional_row < last ? positional_row : last;
+                unsigned char* dest = stage + kLatentTileBytes + 8u * wave * kPositionalRowBytes;
+                if (good) {
+                    if (!ANY || positional_chunk < 16u * positional_chunks)
+                        load_to_lds(positional_cache + slot * positional_row_bytes, kept * positional_row_bytes + positional_chunk, dest);
+                } else {
+                    if (lane == 0) report_index_error(a.status);
+                    *reinterpret_cast<uint4*>(dest + 16u * lane) = make_uint4(0, 0, 0, 0);
+                }
+            }
+            return;
+        }
         if (piece < 4) {
             const int i = piece;
             const unsigned int row = wave + 8u * i;
@@ -550,10 +589,14 @@ SINGE_DEVICE void latent_combine_rows(const LatentAttentionArgs& a) {
 
 template <class Half, bool ANY>
 SINGE_DEVICE void latent_tile_body(const LatentAttentionArgs& a, unsigned char* lds) {
-    if (a.wide_index)
-        latent_tile_rows<Half, kCsrI64, ANY>(a, lds);
-    else
-        latent_tile_rows<Half, kCsrI32, ANY>(a, lds);
+    const bool in_page = a.page_shift >= 5;  // a power of two of at least a tile's 32 keys
+    if (a.wide_index) {
+        if (in_page) latent_tile_rows<Half, kCsrI64, ANY, true>(a, lds);
+        else latent_tile_rows<Half, kCsrI64, ANY, false>(a, lds);
+    } else {
+        if (in_page) latent_tile_rows<Half, kCsrI32, ANY, true>(a, lds);
+        else latent_tile_rows<Half, kCsrI32, ANY, false>(a, lds);
+    }
 }
 
 }  // namespace latent_mfma
