@@ -289,35 +289,44 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
     const unsigned int positional_chunk = 16u * ((lane & 7u) ^ (positional_row & 7u));
     // Rows w and w + 16 of a tile permute their chunks alike, and so do w + 8 and w + 24.
     const unsigned int lane_chunk[2] = {16u * (lane ^ chunk_flip(wave & 15u)), 16u * (lane ^ chunk_flip((wave + 8u) & 15u))};
+    // IN_PAGE: where the tile that is being loaded starts in either cache and the last of its rows that holds a key of
+    // the sequence (rows past it re-read it and are masked): the same for every lane, worked out once a tile (locate_tile, from the id that lookup asked for a tile earlier) in scalar arithmetic.
+    struct TileSource {
+        const unsigned char* latent;
+        const unsigned char* positional;
+        unsigned int last;
+    };
+    TileSource source = {};
+    auto locate_tile = [&](unsigned int tile, const TilePages<FORM>& pages) __attribute__((always_inline)) {
+        if constexpr (IN_PAGE) {
+            const unsigned long long page = static_cast<unsigned long long>(pages.latent[0]);
+            unsigned int low = static_cast<unsigned int>(page);
+            // An id outside the cache is reported and replaced by page 0 (what that holds is not used by a caller that
+            // checks the status word), so that the loads need no test of their own.
+            if (static_cast<unsigned int>(page >> 32) != 0u || low >= a.cache_pages) {
+                if (lane == 0) report_index_error(a.status);
+                low = 0u;
+            }
+            const unsigned int first_key = tile * kKeys;
+            const size_t slot = (static_cast<size_t>(low) << page_shift) + (first_key & (a.page_size - 1u));
+            source.last = keys - 1u - first_key;
+            source.latent = latent_cache + slot * latent_row_bytes;
+            source.positional = positional_cache + slot * positional_row_bytes;
+        }
+    };
     auto issue_piece = [&](int piece, unsigned int tile, const TilePages<FORM>& pages, unsigned char* __restrict__ stage)
                            __attribute__((always_inline)) {
         if constexpr (IN_PAGE) {
-            // The tile's page, its first key's slot in the caches, and the last row that holds a key of the sequence
-            // (rows past it re-read it and are masked): all the same for every lane.
-            const unsigned long long page = static_cast<unsigned long long>(pages.latent[0]);
-            const bool good = page < static_cast<unsigned long long>(a.cache_pages);
-            const unsigned int first_key = tile * kKeys, last = keys - 1u - first_key;
-            const size_t slot = static_cast<size_t>(page) * a.page_size + (first_key & (a.page_size - 1u));
+            const TileSource& from = source;
             if (piece < 4) {
-                const unsigned int row = wave + 8u * piece, kept = row < last ? row : last;
-                unsigned char* dest = stage + row * kLatentRowBytes;
-                if (good) {
-                    if (!ANY || lane_chunk[piece & 1] < 16u * latent_chunks)
-                        load_to_lds(latent_cache + (slot + kept) * latent_row_bytes, lane_chunk[piece & 1], dest);
-                } else {
-                    if (lane == 0) report_index_error(a.status);
-                    *reinterpret_cast<uint4*>(dest + 16u * lane) = make_uint4(0, 0, 0, 0);
-                }
+                const unsigned int row = wave + 8u * piece, kept = row < from.last ? row : from.last;
+                if (!ANY || lane_chunk[piece & 1] < 16u * latent_chunks)
+                    load_to_lds(from.latent + kept * latent_row_bytes, lane_chunk[piece & 1], stage + row * kLatentRowBytes);
             } else if (wave < 4) {
-                const unsigned int kept = positional_row < last ? positional_row : last;
-                unsigned char* dest = stage + kLatentTileBytes + 8u * wave * kPositionalRowBytes;
-                if (good) {
-                    if (!ANY || positional_chunk < 16u * positional_chunks)
-                        load_to_lds(positional_cache + slot * positional_row_bytes, kept * positional_row_bytes + positional_chunk, dest);
-                } else {
-                    if (lane == 0) report_index_error(a.status);
-                    *reinterpret_cast<uint4*>(dest + 16u * lane) = make_uint4(0, 0, 0, 0);
-                }
+                const unsigned int kept = positional_row < from.last ? positional_row : from.last;
+                if (!ANY || positional_chunk < 16u * positional_chunks)
+                    load_to_lds(from.positional, kept * positional_row_bytes + positional_chunk,
+                                stage + kLatentTileBytes + 8u * wave * kPositionalRowBytes);
             }
             return;
         }
@@ -352,6 +361,7 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
     };
 
     auto issue = [&](unsigned int tile, const TilePages<FORM>& pages, unsigned char* __restrict__ stage) __attribute__((always_inline)) {
+        locate_tile(tile, pages);
 #pragma unroll
         for (int piece = 0; piece < 5; ++piece) issue_piece(piece, tile, pages, stage);
     };
@@ -477,7 +487,15 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
             // after it once those have been used: address arithmetic in the shadow of the products.
             auto between = [&](int step) __attribute__((always_inline)) {
                 if (step < 5) {
-                    if (tile + 1 < tiles) issue_piece(step, tile + 1, pages, other);
+                    if constexpr (IN_PAGE) {
+                        // (past the last tile: the last one again, into the stage nobody reads any more, so that a piece
+                        // carries no test; `pages` then still holds the last tile's id)
+                        const unsigned int wanted = tile + 1 < tiles ? tile + 1 : tiles - 1u;
+                        if (step == 0) locate_tile(wanted, pages);
+                        issue_piece(step, wanted, pages, other);
+                    } else if (tile + 1 < tiles) {
+                        issue_piece(step, tile + 1, pages, other);
+                    }
                 } else if (step == 6) {
                     if (tile + 2 < tiles) pages = lookup(tile + 2);
                 }
