@@ -93,6 +93,19 @@ SINGE_DEVICE void load_to_lds(const unsigned char* shared_base, unsigned int lan
                  : "=&s"(kept) : "s"(base), "v"(lane_offset), "s"(scalar) : "memory");
 }
 
+// The same with the destination as the byte address in LDS that M0 takes (a pointer into LDS costs a null test and a
+// select on its way there).
+SINGE_DEVICE void load_to_lds(const unsigned char* shared_base, unsigned int lane_offset, unsigned int lds_byte_address) {
+    const unsigned int base = __builtin_amdgcn_readfirstlane(lds_byte_address);
+    const unsigned long long bits = reinterpret_cast<unsigned long long>(shared_base);
+    const unsigned int low_word = __builtin_amdgcn_readfirstlane(static_cast<unsigned int>(bits));
+    const unsigned int high_word = __builtin_amdgcn_readfirstlane(static_cast<unsigned int>(bits >> 32));
+    const unsigned long long scalar = static_cast<unsigned long long>(low_word) | (static_cast<unsigned long long>(high_word) << 32);
+    unsigned int kept;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3\n\ts_mov_b32 m0, %0"
+                 : "=&s"(kept) : "s"(base), "v"(lane_offset), "s"(scalar) : "memory");
+}
+
 // Where the chunk permutation of a latent row puts things: see the header comment.
 SINGE_DEVICE unsigned int chunk_flip(unsigned int key) {
     const unsigned int pair = (key & 3u) | ((((key >> 2) ^ (key >> 3)) & 1u) << 2);
@@ -303,10 +316,9 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
             unsigned int low = static_cast<unsigned int>(page);
             // An id outside the cache is reported and replaced by page 0 (what that holds is not used by a caller that
             // checks the status word), so that the loads need no test of their own.
-            if (static_cast<unsigned int>(page >> 32) != 0u || low >= a.cache_pages) {
-                if (lane == 0) report_index_error(a.status);
-                low = 0u;
-            }
+            const bool outside = static_cast<unsigned int>(page >> 32) != 0u || low >= a.cache_pages;
+            if (outside && lane == 0) report_index_error(a.status);
+            low = __builtin_amdgcn_readfirstlane(outside ? 0u : low);  // (said to be the same for every lane: scalar arithmetic from here on)
             const unsigned int first_key = tile * kKeys;
             const size_t slot = (static_cast<size_t>(low) << page_shift) + (first_key & (a.page_size - 1u));
             source.last = keys - 1u - first_key;
@@ -314,19 +326,21 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
             source.positional = positional_cache + slot * positional_row_bytes;
         }
     };
-    auto issue_piece = [&](int piece, unsigned int tile, const TilePages<FORM>& pages, unsigned char* __restrict__ stage)
+    const unsigned int lds_start = static_cast<unsigned int>(reinterpret_cast<__UINTPTR_TYPE__>((lds_words_t)lds));  // the byte address M0 takes
+    // (stage_at: the stage's byte offset from there)
+    auto issue_piece = [&](int piece, unsigned int tile, const TilePages<FORM>& pages, unsigned char* __restrict__ stage, unsigned int stage_at)
                            __attribute__((always_inline)) {
         if constexpr (IN_PAGE) {
             const TileSource& from = source;
             if (piece < 4) {
                 const unsigned int row = wave + 8u * piece, kept = row < from.last ? row : from.last;
                 if (!ANY || lane_chunk[piece & 1] < 16u * latent_chunks)
-                    load_to_lds(from.latent + kept * latent_row_bytes, lane_chunk[piece & 1], stage + row * kLatentRowBytes);
+                    load_to_lds(from.latent + kept * latent_row_bytes, lane_chunk[piece & 1], lds_start + stage_at + row * kLatentRowBytes);
             } else if (wave < 4) {
                 const unsigned int kept = positional_row < from.last ? positional_row : from.last;
                 if (!ANY || positional_chunk < 16u * positional_chunks)
                     load_to_lds(from.positional, kept * positional_row_bytes + positional_chunk,
-                                stage + kLatentTileBytes + 8u * wave * kPositionalRowBytes);
+                                lds_start + stage_at + kLatentTileBytes + 8u * wave * kPositionalRowBytes);
             }
             return;
         }
@@ -360,10 +374,10 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
         }
     };
 
-    auto issue = [&](unsigned int tile, const TilePages<FORM>& pages, unsigned char* __restrict__ stage) __attribute__((always_inline)) {
+    auto issue = [&](unsigned int tile, const TilePages<FORM>& pages, unsigned char* __restrict__ stage, unsigned int stage_at) __attribute__((always_inline)) {
         locate_tile(tile, pages);
 #pragma unroll
-        for (int piece = 0; piece < 5; ++piece) issue_piece(piece, tile, pages, stage);
+        for (int piece = 0; piece < 5; ++piece) issue_piece(piece, tile, pages, stage, stage_at);
     };
 
     // Read offsets.  Score operand of step s, 16-key half t: row 16 t + column, chunk (4 s + g) ^ flip.  Transposed
@@ -476,13 +490,14 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
 
     if (first_tile < tiles) {
         TilePages<FORM> pages = lookup(first_tile);
-        issue(first_tile, pages, lds + (first_tile & 1u) * kStageBytes);
+        issue(first_tile, pages, lds + (first_tile & 1u) * kStageBytes, (first_tile & 1u) * kStageBytes);
         if (first_tile + 1 < tiles) pages = lookup(first_tile + 1);
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
         for (unsigned int tile = first_tile; tile < tiles; ++tile) {
             unsigned char* stage = lds + (tile & 1u) * kStageBytes;
             unsigned char* other = lds + ((tile & 1u) ^ 1u) * kStageBytes;
+            const unsigned int other_at = ((tile & 1u) ^ 1u) * kStageBytes;
             // The next tile's loads go out one piece after each of the first score steps, the page ids of the tile
             // after it once those have been used: address arithmetic in the shadow of the products.
             auto between = [&](int step) __attribute__((always_inline)) {
@@ -492,9 +507,9 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
                         // carries no test; `pages` then still holds the last tile's id)
                         const unsigned int wanted = tile + 1 < tiles ? tile + 1 : tiles - 1u;
                         if (step == 0) locate_tile(wanted, pages);
-                        issue_piece(step, wanted, pages, other);
+                        issue_piece(step, wanted, pages, other, other_at);
                     } else if (tile + 1 < tiles) {
-                        issue_piece(step, tile + 1, pages, other);
+                        issue_piece(step, tile + 1, pages, other, other_at);
                     }
                 } else if (step == 6) {
                     if (tile + 2 < tiles) pages = lookup(tile + 2);
