@@ -437,14 +437,19 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                float value = s[t][r] * scale_log2e;
-                if (edge) {
+            for (int r = 0; r < 4; ++r) x[4 * t + r] = s[t][r] * scale_log2e;
+        if (edge) {
+            // (a statement the compiler may not run ahead of the test: it would otherwise turn the branch into eight
+            // tests and selects on every tile, and a wave's instruction count is what bounds its time)
+            asm volatile("s_nop 0");
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
                     const unsigned int key = key0 + 16u * t + 4u * g + r;
-                    if (key >= keys || (causal && key > my_position)) value = -INFINITY;
+                    if (key >= keys || (causal && key > my_position)) x[4 * t + r] = -INFINITY;
                 }
-                x[4 * t + r] = value;
-            }
+        }
         float largest = fmaxf(fmaxf(fmaxf(x[0], x[1]), fmaxf(x[2], x[3])), fmaxf(fmaxf(x[4], x[5]), fmaxf(x[6], x[7])));
         largest = across_groups_max(largest);  // the four lanes of a row agree from here on
         if (__any(largest > reference + kMaxLag || (reference == -INFINITY && largest != -INFINITY))) {
