@@ -136,15 +136,42 @@ SINGE_DEVICE void fill_entries(EntryCache& cache, const DecodeArgs& a, unsigned 
     }
 }
 
-template <bool ALIGNED16>
+// LEAN: whole halves take a path of their own (measured: faster for the fp8 kernels, whose vector unit is what bounds
+// them, and for the four-head bf16 / f16 kernels at head_dim 128; slower where the extra code costs the wide bf16 form its
+// last free registers, and at the other head dimensions).
+template <bool ALIGNED16, bool LEAN>
 SINGE_DEVICE HalfRows locate_half(const DecodeArgs& a, const unsigned int* table_row, const EntryCache& cache,
                                   unsigned int base, unsigned int end, unsigned int kv_head, unsigned int g,
                                   unsigned int t) {
     HalfRows rows;
     rows.live = 0;
     if constexpr (ALIGNED16) {
-        // block_size is a multiple of 16, so the 16 keys share one table entry; a half wholly past
-        // the end re-reads the 16-key span that holds the last key.
+        // block_size is a multiple of 16, so the 16 keys share one table entry.
+        if (LEAN && base + 16u <= end) {
+            // All sixteen keys are the sequence's (every half but a sequence's last one or two): the block and the row of
+            // its first key are the same for every lane, and a lane's rows lie whole slots behind it; no key needs a
+            // test of its own.  (The statement below keeps this a branch: as selects, the tests of the general path
+            // would run for every half.)
+            asm volatile("");
+            unsigned int entry, slot0;
+            split_key(a, base, entry, slot0);
+            rows.cache_lane = entry - cache.first_entry;
+            const unsigned int block = __builtin_amdgcn_readlane(cache.blocks, rows.cache_lane);
+            const bool known = block < a.physical_blocks;
+            const unsigned int safe = known ? block : 0;
+            const size_t first_row = cache_row(safe, slot0, a.block_size, a.kv_heads, kv_head);
+            const unsigned int slot_elements = a.kv_heads * static_cast<unsigned int>(kDim);
+            rows.key_block = safe;
+            rows.key_row = first_row + t * slot_elements;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                rows.value_block[i] = safe;
+                rows.value_row[i] = first_row + (4 * g + i) * slot_elements;
+            }
+            rows.live = known ? 0xfu : 0u;
+            return rows;
+        }
+        // A half that holds the sequence's last key, or lies wholly past it and re-reads the 16-key span that holds it.
         unsigned int last_entry, last_slot, entry, slot0;
         split_key(a, end - 1, last_entry, last_slot);
         split_key(a, base < end ? base : ((end - 1) & ~15u), entry, slot0);
@@ -189,7 +216,7 @@ SINGE_DEVICE HalfRows locate_half(const DecodeArgs& a, const unsigned int* table
 }
 
 // Loads the 32 keys from `first` (a multiple of 32) of a sequence of `end` > first keys.
-template <bool ALIGNED16>
+template <bool ALIGNED16, bool LEAN>
 SINGE_DEVICE void load_tile(KeyTileBf16& tile, const DecodeArgs& a, const unsigned int* table_row, const EntryCache& cache,
                             unsigned int first, unsigned int end, unsigned int kv_head, unsigned int g,
                             unsigned int t) {
@@ -198,7 +225,7 @@ SINGE_DEVICE void load_tile(KeyTileBf16& tile, const DecodeArgs& a, const unsign
     const uint16_t* value_cache = static_cast<const uint16_t*>(a.value_cache);
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
-        const HalfRows rows = locate_half<ALIGNED16>(a, table_row, cache, first + half * 16, end, kv_head, g, t);
+        const HalfRows rows = locate_half<ALIGNED16, LEAN>(a, table_row, cache, first + half * 16, end, kv_head, g, t);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             if (kDim == 128 || 8 * t < static_cast<unsigned int>(kDim)) {
@@ -213,7 +240,7 @@ SINGE_DEVICE void load_tile(KeyTileBf16& tile, const DecodeArgs& a, const unsign
     }
 }
 
-template <bool ALIGNED16>
+template <bool ALIGNED16, bool LEAN>
 SINGE_DEVICE void load_tile(KeyTileFp8& tile, const DecodeArgs& a, const unsigned int* table_row, const EntryCache& cache,
                             unsigned int first, unsigned int end, unsigned int kv_head, unsigned int g,
                             unsigned int t) {
@@ -222,7 +249,7 @@ SINGE_DEVICE void load_tile(KeyTileFp8& tile, const DecodeArgs& a, const unsigne
     const uint8_t* value_cache = static_cast<const uint8_t*>(a.value_cache);
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
-        const HalfRows rows = locate_half<ALIGNED16>(a, table_row, cache, first + half * 16, end, kv_head, g, t);
+        const HalfRows rows = locate_half<ALIGNED16, LEAN>(a, table_row, cache, first + half * 16, end, kv_head, g, t);
         const uint8_t* kp = key_cache + rows.key_row + 32 * g;
         tile.k[half][0] = *reinterpret_cast<const uint4*>(kp);
         tile.k[half][1] = *reinterpret_cast<const uint4*>(kp + 16);
@@ -354,6 +381,7 @@ template <int GROUPS, bool ALIGNED16, bool FP8, bool EXACT, bool WIDE = false, b
 SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, unsigned char* staging = nullptr) {
     static_assert((!FP8 || WIDE) && (!WIDE || GROUPS == 1), "fp8 caches take the wide form; the wide form carries one group");
     constexpr bool kQueryInLds = WIDE && !FP8;
+    constexpr bool kLean = FP8 || (!WIDE && GROUPS == 1 && kDim == 128);  // see locate_half
     using Tile = typename std::conditional<FP8, KeyTileFp8, KeyTileBf16>::type;
     constexpr int DEPTH = FP8 ? 3 : 2;  // an fp8 tile is half the bytes, so one more is kept in flight
     const unsigned int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -540,8 +568,17 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
                     first *= tile.row_key_scale[0][i];
                     second *= tile.row_key_scale[1][i];
                 }
-                p[i] = (tile.live >> i) & 1u ? first : -INFINITY;
-                p[4 + i] = (tile.live >> (4 + i)) & 1u ? second : -INFINITY;
+                p[i] = first;
+                p[4 + i] = second;
+            }
+            // Dead keys (past the sequence's end, before its window, behind an entry that is no cache block) leave the
+            // softmax: only a sequence's first and last tiles have any.  (kLean: the statement keeps this a branch that
+            // the other tiles skip; as selects the tests run for every tile.)
+            if (!kLean || __any(tile.live != 0xffu)) {
+                if constexpr (kLean) asm volatile("");
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    if (!((tile.live >> i) & 1u)) p[i] = -INFINITY;
             }
             float largest = fmaxf(fmaxf(fmaxf(p[0], p[1]), fmaxf(p[2], p[3])), fmaxf(fmaxf(p[4], p[5]), fmaxf(p[6], p[7])));
             largest = across_groups_max(largest);
@@ -631,8 +668,15 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
                 const float first = s0[hg][i] * a.scale_log2e, second = s1[hg][i] * a.scale_log2e;
-                p[hg][i] = (tile.live >> i) & 1u ? first : -INFINITY;
-                p[hg][4 + i] = (tile.live >> (4 + i)) & 1u ? second : -INFINITY;
+                p[hg][i] = first;
+                p[hg][4 + i] = second;
+            }
+            // (dead keys leave the softmax: a branch that the tiles without any skip, as in the wide form)
+            if (!kLean || __any(tile.live != 0xffu)) {
+                if constexpr (kLean) asm volatile("");
+#pragma unroll
+                for (int i = 0; i < 8; ++i)
+                    if (!((tile.live >> i) & 1u)) p[hg][i] = -INFINITY;
             }
             float largest = fmaxf(fmaxf(fmaxf(p[hg][0], p[hg][1]), fmaxf(p[hg][2], p[hg][3])),
                                   fmaxf(fmaxf(p[hg][4], p[hg][5]), fmaxf(p[hg][6], p[hg][7])));
@@ -728,7 +772,7 @@ SINGE_DEVICE void paged_decode_body(const DecodeArgs& a, unsigned int* prefix, u
             if (entries.sequence != load_seq || low < entries.first_entry || high >= entries.first_entry + 64)
                 fill_entries<FP8>(entries, a, load_seq, row_base, low, kv_head, lane);
         }
-        load_tile<ALIGNED16>(buffer, a, a.block_table + row_base, entries, first_key, end, kv_head, g, t);
+        load_tile<ALIGNED16, kLean>(buffer, a, a.block_table + row_base, entries, first_key, end, kv_head, g, t);
         if (a.row_begins != nullptr) {
             // Keys of the row before its window (bit half * 4 + i of `live` is key first_key + 16 half + 4 g + i).
             const unsigned int begin = begins[load_seq];
