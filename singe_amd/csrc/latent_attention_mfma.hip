@@ -546,7 +546,9 @@ SINGE_DEVICE void latent_tile_rows(const LatentAttentionArgs& a, unsigned char* 
         unsigned char* row = static_cast<unsigned char*>(a.output) + flat * latent_row_bytes + 8u * g;
 #pragma unroll
         for (int db = 0; db < kDimBlocks; ++db) {
-            if (ANY && 2u * db >= latent_chunks) break;  // dims past the latent width
+            // (a test a dim block, not a way out of the loop: a loop that may end early is not unrolled, and an output
+            // indexed by a variable lives in scratch memory for the whole kernel)
+            if (ANY && 2u * db >= latent_chunks) continue;  // dims past the latent width
             uint2 packed;
             packed.x = pack_pair(half, out[db][0] * inverse, out[db][1] * inverse);
             packed.y = pack_pair(half, out[db][2] * inverse, out[db][3] * inverse);
