@@ -49,16 +49,16 @@ FETCH_UNIT_BYTES, WRITE_UNIT_BYTES = 2048, 1024
 COUNTER_TRAFFIC = {
     "decode": {"kernel": "singe_paged_decode_bf16_d128_g1_b16", "FETCH_SIZE": 150137, "WRITE_SIZE": 4238,
                "source": "profiles/hbm_traffic_counters.md"},
-    "prefill": {"kernel": "singe_fmha_prefill_pair_bf16_d128_causal", "FETCH_SIZE": 298455, "WRITE_SIZE": 131077,
+    "prefill": {"kernel": "singe_fmha_prefill_pair_bf16_d128_causal", "FETCH_SIZE": 300835, "WRITE_SIZE": 131072,
                 "source": "profiles/hbm_traffic_counters.md"},
     "chunked_prefill": {"kernel": "singe_paged_attention_pair_bf16_d128_i32", "FETCH_SIZE": 182670, "WRITE_SIZE": 66560,
                         "source": "profiles/hbm_traffic_counters.md"},
-    "fp8_decode": {"kernel": "singe_paged_decode_f8kv_wide_d128_b16", "FETCH_SIZE": 2129860, "WRITE_SIZE": 8256,
+    "fp8_decode": {"kernel": "singe_paged_decode_f8kv_wide_d128_b16", "FETCH_SIZE": 2118890, "WRITE_SIZE": 8256,
                    "source": "profiles/hbm_traffic_counters.md"},
-    "latent_decode": {"kernel": "singe_paged_mla_attention_bf16_l512_p64", "FETCH_SIZE": 608523, "WRITE_SIZE": 32999,
+    "latent_decode": {"kernel": "singe_paged_mla_attention_bf16_l512_p64", "FETCH_SIZE": 608457, "WRITE_SIZE": 32896,
                       "source": "profiles/hbm_traffic_counters.md"},
-    "latent_chunked_prefill": {"kernel": "singe_paged_mla_attention_bf16_l512_p64", "FETCH_SIZE": 868387,
-                               "WRITE_SIZE": 526766, "source": "profiles/hbm_traffic_counters.md"},
+    "latent_chunked_prefill": {"kernel": "singe_paged_mla_attention_bf16_l512_p64", "FETCH_SIZE": 867638,
+                               "WRITE_SIZE": 526336, "source": "profiles/hbm_traffic_counters.md"},
     "cache_append": {"kernel": "singe_rotary_cache_write_chunks_bf16", "FETCH_SIZE": 44244, "WRITE_SIZE": 81920,
                      "source": "profiles/hbm_traffic_counters.md"},
 }
