@@ -104,11 +104,13 @@ HEADER = """// One 32-key block of two 32-row tiles at head_dim {dim}, slot by s
 // issue cycles: {used}.
 """
 
+# (head dimension, the smallest budget the dealing succeeds with, the slots of the four loads)
+BLOCKS = ((128, 7.0, (0, 2, 4, 6)), (112, 8.0, (0, 2, 4, 6)), (96, 9.0, (0, 2, 4, 5)), (80, 10.0, (0, 2, 4, 6)),
+          (64, 14.0, (0, 1, 2, 3)), (48, 16.0, (0, 1, 2, 3)), (32, 27.0, (0, 1, 2, 3)), (16, 36.0, (0, 1, 2, 3)))
+
 if __name__ == "__main__":
     here = os.path.dirname(os.path.abspath(__file__))
-    # (the smallest budget the dealing succeeds with, and the slots of the four loads, for every head dimension)
-    for dim, budget, load_slots in ((128, 7.0, (0, 2, 4, 6)), (112, 8.0, (0, 2, 4, 6)), (96, 9.0, (0, 2, 4, 5)), (80, 10.0, (0, 2, 4, 6)),
-                                    (64, 14.0, (0, 1, 2, 3)), (48, 16.0, (0, 1, 2, 3)), (32, 27.0, (0, 1, 2, 3)), (16, 36.0, (0, 1, 2, 3))):
+    for dim, budget, load_slots in BLOCKS:
         body, used = deal(dim // 16, (dim + 31) // 32, budget, load_slots)
         with open(os.path.join(here, f"prefill_pair_block_d{dim}.inc"), "w") as out:
             out.write(HEADER.format(dim=dim, used=" ".join(f"{u:.0f}" for u in used)) + body)

@@ -122,3 +122,15 @@ def test_nothing_touches_a_score_product_before_it_is_done(listings, name, flags
                 continue
             assert not (registers(later, "a") & loaded), f"{later!r} names what {text!r} is still loading"
     assert loads >= 4 * 2 * steps
+
+
+def test_the_block_texts_are_what_the_dealing_script_writes():
+    # the .inc files beside the kernels are generated: a hand edit, or a change to the script that was not run, shows here
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("prefill_pair_deal", os.path.join(CSRC, "prefill_pair_deal.py"))
+    dealing = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(dealing)
+    for dim, budget, load_slots in dealing.BLOCKS:
+        body, used = dealing.deal(dim // 16, (dim + 31) // 32, budget, load_slots)
+        text = dealing.HEADER.format(dim=dim, used=" ".join(f"{u:.0f}" for u in used)) + body
+        assert open(os.path.join(CSRC, f"prefill_pair_block_d{dim}.inc")).read() == text, dim
