@@ -341,3 +341,61 @@ def test_shapes_the_op_does_not_take():
         neural.paged_mla_attention(zeros(2, 2, 32), zeros(2, 2, 8), zeros(2, 4, 32), zeros(2, 4, 16), paging)
     with pytest.raises(error.UnsupportedWidth):  # beyond the widths this kernel holds
         neural.paged_mla_attention(zeros(2, 2, 576), zeros(2, 2, 8), zeros(2, 4, 576), zeros(2, 4, 8), paging)
+
+
+def random_latent_case(seed):
+    """Random sequences over pages that hold whole 32-key tiles (the kernel then takes one page id a tile) or do not,
+    at the built widths or others, with or without key shares, against the CPU oracle."""
+    rng = np.random.default_rng(4000 + seed)
+    page_size = int(rng.choice([32, 64, 128, 32, 64, 16, 48]))
+    latent, positional = [(512, 64), (512, 64), (256, 64), (128, 32), (384, 16)][int(rng.integers(0, 5))]
+    heads = int(rng.choice([1, 8, 16, 40, 128]))
+    dtype = torch.bfloat16 if rng.integers(0, 2) else torch.float16
+    index_dtype = torch.int64 if rng.integers(0, 2) else torch.int32
+    causal = bool(rng.integers(0, 2))
+    sequences = []
+    for _ in range(int(rng.integers(1, 6))):
+        keys = int(rng.choice([0, 1, int(rng.integers(1, 33)), int(rng.integers(33, 400)), int(rng.integers(400, 1500))]))
+        queries = int(rng.choice([0, 1, 1, int(rng.integers(1, 30)), int(rng.integers(30, 200))]))
+        sequences.append((queries, keys))
+    if sum(q for q, _ in sequences) == 0:
+        sequences[0] = (2, sequences[0][1])
+    query_offsets, page_offsets, last, needed = [0], [0], [], 0
+    for queries, keys in sequences:
+        query_offsets.append(query_offsets[-1] + queries)
+        pages = (keys + page_size - 1) // page_size
+        needed += pages
+        page_offsets.append(needed)
+        last.append(0 if keys == 0 else keys - (pages - 1) * page_size)
+    page_count = needed + int(rng.integers(1, 4))
+    table = [int(page) for page in rng.permutation(page_count)[:needed]]
+    tokens = query_offsets[-1]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(seed)
+    rand = lambda *shape: torch.randn(shape, generator=gen, device="cuda").to(dtype)
+    device = [rand(tokens, heads, latent), rand(tokens, heads, positional), rand(page_count, page_size, latent), rand(page_count, page_size, positional)]
+    index = lambda entries: torch.tensor(entries, dtype=index_dtype, device="cuda")
+    paging = neural.Paging(index(query_offsets), index(page_offsets), index(table), index(last))
+    from singe_amd import _native
+    splits = int(rng.choice([0, 0, 1, 3, 8]))
+    _native.lib().singe_hip_set_paged_mla_attention_splits(splits)
+    try:
+        out, lse = neural.paged_mla_attention(*device, paging, neural.AttentionOptions(causal=causal))
+        torch.cuda.synchronize()
+    finally:
+        _native.lib().singe_hip_set_paged_mla_attention_splits(0)
+    status, want, want_lse = oracle.paged_mla_attention(*[tensor.float().cpu().numpy() for tensor in device], query_offsets, page_offsets, table,
+                                                        last, causal=causal, threads=8)
+    assert status == 0
+    case = (sequences, heads, latent, positional, page_size, causal, dtype, index_dtype, splits)
+    got, got_lse = out.float().cpu().numpy(), lse.cpu().numpy()
+    gap = np.abs(got - want)
+    assert gap.max(initial=0.0) <= 2e-2 and (gap.size == 0 or gap.mean() <= 2e-3), (case, gap.max(initial=0.0))
+    empty = np.isneginf(want_lse)
+    assert np.array_equal(np.isneginf(got_lse), empty) and not got[empty].any(), case
+    assert np.abs(got_lse[~empty] - want_lse[~empty]).max(initial=0.0) <= 5e-3, case
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes_over_pages_of_whole_tiles_and_others(seed):
+    random_latent_case(seed)
