@@ -333,3 +333,34 @@ def test_decode_peaked_and_flat_softmax(magnitude):
     work.query.mul_(magnitude)
     got, want = run_gpu(work), run_oracle(work)
     assert_close(got, want, f"magnitude {magnitude}")
+
+
+def random_decode_case(seed):
+    """Random batches for the block-table decode kernels, bf16 or f16 or fp8 caches: block sizes whose 16-key halves lie
+    whole in a block (located without per-key tests) and others, lengths that end anywhere in a half, empty sequences,
+    worker counts that cut sequences anywhere."""
+    import test_paged_decode_fp8_gpu as fp8
+    rng = np.random.default_rng(6000 + seed)
+    kv_heads = int(rng.choice([1, 2, 4, 8]))
+    heads = kv_heads * int(rng.choice([1, 2, 4, 4, 8]))
+    block_size = int(rng.choice([16, 16, 32, 64, 48, 7]))
+    lens = [int(rng.choice([0, 1, int(rng.integers(1, 40)), int(rng.integers(40, 700)), int(rng.integers(700, 3000))]))
+            for _ in range(int(rng.integers(1, 12)))]
+    blocks = sum((length + block_size - 1) // block_size for length in lens) + int(rng.integers(1, 9))
+    workers = int(rng.choice([0, 0, 1, 5, 37, 300]))
+    kind = int(rng.integers(0, 3))
+    label = (seed, heads, kv_heads, block_size, lens, workers, kind)
+    if kind == 2:
+        work = synthetic.paged_decode_fp8_workload(batch=len(lens), heads=heads, kv_heads=kv_heads, block_size=block_size,
+                                                   physical_blocks=blocks, seq_lens=lens, seed=seed)
+        fp8.assert_close(fp8.run_gpu(work, False, workers), fp8.run_oracle(work), str(label))
+    else:
+        dtype = torch.bfloat16 if kind == 0 else torch.float16
+        work = synthetic.paged_decode_workload(batch=len(lens), heads=heads, kv_heads=kv_heads, block_size=block_size,
+                                               physical_blocks=blocks, seq_lens=lens, seed=seed)
+        assert_close(run_gpu(work, workers, dtype), run_oracle(work), str(label))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_decode_random_batches(seed):
+    random_decode_case(seed)
